@@ -1,0 +1,171 @@
+/*
+ * lantern_hip.h -- C ABI of the MI355X (gfx950) tensor backend for Lantern.
+ *
+ * One entry point per method of Lantern's `Backend` trait that touches device
+ * data (reference: src/main/scala/lantern/TensorDifferentiation.scala:137-379,
+ * "TD" below), shaped the way the code generator emits calls for the cuBLAS /
+ * cuDNN backend it stands in for ("CUB" = src/main/scala/lantern/
+ * TensorDslCublas.scala, "CDN" = .../TensorDslCudnn.scala, "API" =
+ * .../DslAPI.scala, "CPU" = .../TensorDslCPU.scala).
+ *
+ * Contract
+ *  - Plain pointers and sizes only.  Every `float*` / `int*` is a DEVICE pointer
+ *    unless its name starts with `h_`; shape arrays (`*dims`, `*perm`, `*sizes`)
+ *    and pointer tables are HOST arrays read during the call.
+ *  - Dense row-major fp32, NCHW.  Every `*_grad` / `*_bwd*` entry ACCUMULATES
+ *    (+=) into its gradient outputs unless a `beta` argument says otherwise
+ *    (beta = 1 accumulate, beta = 0 overwrite), as the reference's backends do
+ *    (cuDNN calls with beta = 1: CDN:681, 756, 829, 1106).
+ *  - One caller thread; calls are enqueued on one library-owned stream in
+ *    program order and return without waiting.  lh_d2h and lh_sync wait.
+ *  - Errors: like the reference's CUDA_CALL macros (API:435-451) a failing call
+ *    prints "file:line: message" and exits the process.  A host that prefers
+ *    to handle errors calls lh_set_error_mode(1): the failing entry point then
+ *    returns early and lh_last_error() holds the message.
+ *  - No allocation happens inside an operator: outputs, gradients and scratch
+ *    are caller-provided, normally from the arena below.
+ */
+#ifndef LANTERN_HIP_H
+#define LANTERN_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- operator codes ---------------------------------------------------- */
+enum { LH_ADD = 0, LH_SUB = 1, LH_MUL = 2, LH_DIV = 3 };
+enum { LH_RELU = 0, LH_TANH = 1, LH_SIGMOID = 2, LH_EXP = 3, LH_LOG = 4, LH_SQRT = 5, LH_SQUARE = 6, LH_HARDTANH = 7 };
+
+/* ---- lifetime, errors -------------------------------------------------- */
+/* Backend.setup/cleanup (TD:139-142; CUB:113-131): one device arena of
+ * heap_bytes (the reference hard-codes 8 GiB, API:385; here it is an argument). */
+void lh_setup(size_t heap_bytes);
+void lh_cleanup(void);
+void lh_set_error_mode(int mode);           /* 0 = print and exit (reference), 1 = record and return */
+const char* lh_last_error(void);            /* "" when none; cleared by lh_clear_error */
+void lh_clear_error(void);
+void lh_sync(void);                         /* wait for everything enqueued so far */
+
+/* ---- arena: myGpuMalloc / myGpuFree / getCudaMallocAddr / resetCudaMallocAddr
+ *      (API:453-473, CUB:18-25).  Memory returned by lh_malloc reads as zero,
+ *      the property Tensor.zeros relies on (TD:1075-1076); blocks are 256-byte
+ *      aligned (reference: 16). */
+void*  lh_malloc(size_t bytes);
+void*  lh_malloc_uninit(size_t bytes);      /* same bump pointer, contents unspecified: for outputs an op overwrites */
+void   lh_free_top(size_t bytes);           /* LIFO pop of the most recent block(s) */
+size_t lh_mark(void);
+void   lh_rewind(size_t mark);
+size_t lh_heap_used(void);
+size_t lh_heap_peak(void);
+
+/* ---- transfers: toGPU / toCPU / copyFloatArray (CUB:37-107, 128-131) --- */
+void lh_h2d(void* dst, const void* h_src, size_t bytes);
+void lh_d2h(void* h_dst, const void* src, size_t bytes);   /* waits */
+void lh_d2d(void* dst, const void* src, size_t bytes);
+
+/* ---- timing helpers for the benchmark (HIP events on the library stream) */
+void* lh_event_create(void);
+void  lh_event_record(void* ev);
+float lh_event_elapsed_ms(void* start, void* stop);        /* waits for stop */
+void  lh_event_destroy(void* ev);
+
+/* ---- fill / elementwise ------------------------------------------------ */
+void lh_fill(float* x, float v, int64_t n);                                    /* fill, fillInPlace: CUB:133-151 */
+void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, int64_t inner); /* fillWithBias: CPU:39-62 */
+void lh_clip(float* x, float bound, int64_t n);                                /* clipAt: CUB:157-161 */
+void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t);      /* mask4D: CUB:710-719 */
+/* relu/tanh/sigmoid/hardTanh/exp/log/sqrt/square (TD:319-335; CDN:1349-1429, CUB:733-800).
+ * y may alias x (in place).  lo/hi are used by LH_HARDTANH only. */
+void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi);
+/* inplace != 0: x == y is the activated buffer and dx == dy; the gradient is
+ * zeroed where the activation is flat (mask y > 0 for relu, as CDN:1404-1405). */
+void lh_unary_grad(int op, const float* x, const float* y, const float* dy, float* dx, int64_t n, int inplace, float lo, float hi);
+void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n);       /* tensor (+,-,*,/) scalar: CDN:284-375 */
+/* broadcast binary ops, numpy right-aligned rules, rank <= 4, dims padded with
+ * leading 1s by the caller (TD:997-1016; CDN:153-216) */
+void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const int* bdims, float* out, const int* odims, int rank);
+void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a_is_input,
+                      const float* b, float* bd, const int* bdims, int b_is_input,
+                      const float* outd, const int* odims, int rank);          /* add/minus/mul/div_grad: CPU:246-337 */
+/* a (op)= b with b broadcast, or reduced when a is the smaller one: += -= *= /=,
+ * plusBias, plusEqual and their grads (TD:229-270; CPU:265-296; CDN:476-512, 626-649) */
+void lh_bcast_update(int op, float* a, const int* adims, const float* b, const int* bdims, int rank);
+void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n);   /* geam, no transposes: CPU:342-347 */
+void lh_trans(const float* x, float* y, int rows, int cols);                   /* trans: CUB:361-374 */
+void lh_trans_grad(float* xd, const float* yd, int rows, int cols);
+void lh_permute(const float* x, float* y, const int* dims, const int* perm, int rank);          /* CUB:524-560 */
+void lh_permute_grad(float* xd, const float* yd, const int* dims, const int* perm, int rank);   /* CUB:562-587, accumulates */
+
+/* ---- reductions / loss ------------------------------------------------- */
+void lh_sum_all(const float* x, float* out, int64_t n);                        /* sum: CDN:1579-1581 */
+void lh_mean_all(const float* x, float* out, int64_t n);                       /* mean: CDN:1583-1585 */
+void lh_add_scalar_from(float* dx, const float* dy1, float scale, int64_t n);  /* sum_grad / mean_grad: CDN:1587-1605 */
+void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner);      /* sum(dim): CDN:1607-1621; overwrites y */
+void lh_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner);/* CDN:1623-1636 */
+/* softmax / logSoftmax over the middle axis of an [outer, c, inner] view (CDN:1431-1504) */
+void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner);
+void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int outer, int c, int inner);
+void lh_nll(const float* x, const int* target, float* y, int batch, int stride);          /* nllLoss: CUB:802-807 */
+void lh_nll_grad(float* dx, const int* target, const float* dy, int batch, int stride);   /* nllLoss_grad: CUB:808-813 */
+
+/* ---- dense: dot family and gemm (CUB:173-359, 589-688) ----------------- */
+/* Row-major C[m,n] = alpha * op(A) * op(B) + beta * C; lda/ldb/ldc = row strides. */
+void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, int lda,
+              const float* B, int ldb, float beta, float* C, int ldc);
+void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, const float* x, float beta, float* y);
+void lh_ger(int m, int n, const float* u, const float* v, float* A);           /* A[m,n] += u[m] (x) v[n]  (add_cartesian) */
+void lh_dot_vv(const float* x, const float* y, float* out, int n);
+void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x, int64_t n);   /* y += s[0]*x, s on device (vv-dot grad) */
+
+/* ---- conv2D_batch and its gradient (TD:292-296; CDN:515-880) ----------- */
+/* y[n,k,p,q] = bias[k] + sum_{c,r,s} x[n,c,p*sH-pH+r,q*sW-pW+s] * w[k,c,r,s]; bias may be NULL. */
+void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
+                   int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
+void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
+                        int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
+void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db /* or NULL */, float beta,
+                          int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
+
+/* ---- pooling (TD:298-302; CPU:848-1038; CDN:882-982) ------------------- */
+/* argmax holds the global flat index into x (batch offset included, CPU:908); first maximum wins. */
+void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad);
+void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out);
+void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW);
+void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW);
+
+/* ---- batch norm (TD:304-310; CDN:984-1266).  Spatial: x is [N,C,HW];
+ *      per-activation (batchNorm1D) is the same call with HW = 1.
+ *      save_mean / save_invstd hold mean and 1/sqrt(var+eps); running stats are
+ *      updated as (1-factor)*running + factor*batch (unbiased variance). */
+void lh_bn_infer(const float* x, const float* gamma, const float* beta, const float* run_mean, const float* run_var,
+                 float* y, int N, int C, int HW, float eps);
+void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                     float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor);
+void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+               float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
+
+/* ---- dropout (TD:312-313; CPU:1066-1088).  The mask is drawn from a
+ *      counter-based generator keyed by (seed, offset + element index), so a
+ *      host restatement reproduces it exactly. */
+void lh_dropout_fwd(const float* x, float* y, float* mask, int64_t n, float p, uint64_t seed, uint64_t offset);
+void lh_dropout_bwd(const float* dy, const float* mask, float* dx, int64_t n);
+
+/* ---- concat along one axis of n tensors (TD:369-370; CUB:825-879) ------ */
+void lh_concat(int n, const float* const* h_in_ptrs, const int* sizes, float* out, int outer, int inner);
+void lh_concat_grad(int n, float* const* h_ind_ptrs, const int* sizes, const float* outd, int outer, int inner);
+
+/* ---- optimizers (TD:377-378; NN:255-303; API:652-678) ------------------ */
+void lh_sgd(float* x, float* d, float lr, int64_t n);          /* x -= lr*d; d = 0  (SGD.step = geam + clear_grad, NN:279-285) */
+void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n);
+void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n);
+/* One launch over `count` tensors (pointer tables on the host): the 161-tensor
+ * ResNet-50 update in one kernel instead of one launch per tensor. */
+void lh_multi_momentum(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
+                       float lr, float mu, float clip, int nesterov);
+void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,117 @@
+"""ctypes binding of liblantern_hip.so (the C ABI declared in include/lantern_hip.h).
+
+The library is loaded from lantern_amd/csrc/ (built in-tree).  There is no CPU fallback:
+if the shared object is missing or a symbol does not resolve, loading raises.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "liblantern_hip.so")
+
+P, I, F, L, Z, U64 = C.c_void_p, C.c_int, C.c_float, C.c_int64, C.c_size_t, C.c_uint64
+
+# name -> (restype, argtypes); one line per declaration in include/lantern_hip.h
+SIGNATURES = {
+    "lh_setup": (None, [Z]),
+    "lh_cleanup": (None, []),
+    "lh_set_error_mode": (None, [I]),
+    "lh_last_error": (C.c_char_p, []),
+    "lh_clear_error": (None, []),
+    "lh_sync": (None, []),
+    "lh_malloc": (P, [Z]),
+    "lh_malloc_uninit": (P, [Z]),
+    "lh_free_top": (None, [Z]),
+    "lh_mark": (Z, []),
+    "lh_rewind": (None, [Z]),
+    "lh_heap_used": (Z, []),
+    "lh_heap_peak": (Z, []),
+    "lh_h2d": (None, [P, P, Z]),
+    "lh_d2h": (None, [P, P, Z]),
+    "lh_d2d": (None, [P, P, Z]),
+    "lh_event_create": (P, []),
+    "lh_event_record": (None, [P]),
+    "lh_event_elapsed_ms": (F, [P, P]),
+    "lh_event_destroy": (None, [P]),
+    "lh_fill": (None, [P, F, L]),
+    "lh_fill_with_bias": (None, [P, P, L, L, L]),
+    "lh_clip": (None, [P, F, L]),
+    "lh_mask4d": (None, [P, P, I, I, I, I]),
+    "lh_unary": (None, [I, P, P, L, F, F]),
+    "lh_unary_grad": (None, [I, P, P, P, P, L, I, F, F]),
+    "lh_scalar_op": (None, [I, P, P, F, L]),
+    "lh_bcast_op": (None, [I, P, P, P, P, P, P, I]),
+    "lh_bcast_op_grad": (None, [I, P, P, P, I, P, P, P, I, P, P, I]),
+    "lh_bcast_update": (None, [I, P, P, P, P, I]),
+    "lh_geam": (None, [P, F, P, F, P, L]),
+    "lh_trans": (None, [P, P, I, I]),
+    "lh_trans_grad": (None, [P, P, I, I]),
+    "lh_permute": (None, [P, P, P, P, I]),
+    "lh_permute_grad": (None, [P, P, P, P, I]),
+    "lh_sum_all": (None, [P, P, L]),
+    "lh_mean_all": (None, [P, P, L]),
+    "lh_add_scalar_from": (None, [P, P, F, L]),
+    "lh_sum_dim": (None, [P, P, I, I, I]),
+    "lh_sum_dim_grad": (None, [P, P, I, I, I]),
+    "lh_softmax": (None, [I, P, P, I, I, I]),
+    "lh_softmax_grad": (None, [I, P, P, P, I, I, I]),
+    "lh_nll": (None, [P, P, P, I, I]),
+    "lh_nll_grad": (None, [P, P, P, I, I]),
+    "lh_sgemm": (None, [I, I, I, I, I, F, P, I, P, I, F, P, I]),
+    "lh_sgemv": (None, [I, I, I, F, P, I, P, F, P]),
+    "lh_ger": (None, [I, I, P, P, P]),
+    "lh_dot_vv": (None, [P, P, P, I]),
+    "lh_axpy_dev": (None, [P, P, P, L]),
+    "lh_conv2d_fwd": (None, [P, P, P, P] + [I] * 11),
+    "lh_conv2d_bwd_data": (None, [P, P, P, F] + [I] * 11),
+    "lh_conv2d_bwd_filter": (None, [P, P, P, P, F] + [I] * 11),
+    "lh_maxpool_fwd": (None, [P, P, P] + [I] * 9),
+    "lh_maxpool_bwd": (None, [P, P, P, L]),
+    "lh_avgpool_fwd": (None, [P, P] + [I] * 8),
+    "lh_avgpool_bwd": (None, [P, P] + [I] * 8),
+    "lh_bn_infer": (None, [P, P, P, P, P, P, I, I, I, F]),
+    "lh_bn_train_fwd": (None, [P, P, P, P, P, P, P, P, I, I, I, F, F]),
+    "lh_bn_bwd": (None, [P, P, P, P, P, P, F, P, P, I, I, I]),
+    "lh_dropout_fwd": (None, [P, P, P, L, F, U64, U64]),
+    "lh_dropout_bwd": (None, [P, P, P, L]),
+    "lh_concat": (None, [I, P, P, P, I, I]),
+    "lh_concat_grad": (None, [I, P, P, P, I, I]),
+    "lh_sgd": (None, [P, P, F, L]),
+    "lh_momentum": (None, [P, P, P, F, F, F, I, L]),
+    "lh_adagrad": (None, [P, P, P, F, F, L]),
+    "lh_multi_momentum": (None, [I, P, P, P, P, F, F, F, I]),
+    "lh_multi_sgd": (None, [I, P, P, P, F]),
+}
+
+_lib = None
+
+
+class LanternHipError(RuntimeError):
+    """Raised when an entry point of liblantern_hip reports an error (error mode 1)."""
+
+
+def load():
+    """Load the shared library once and bind every declared symbol; raises if it is absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s not found: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "or `make -C lantern_amd/csrc` (there is no CPU fallback)" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check():
+    """Raise LanternHipError if the last call recorded an error (used with error mode 1)."""
+    msg = _lib.lh_last_error()
+    if msg:
+        text = msg.decode()
+        _lib.lh_clear_error()
+        raise LanternHipError(text)

@@ -1,0 +1,390 @@
+"""Host-side mirror of Lantern's `Backend` trait and its MI355X implementation, BackendHIP.
+
+Reference: src/main/scala/lantern/TensorDifferentiation.scala:137-379 (the trait) and the slot
+BackendCudnn occupies (src/main/scala/lantern/TensorDslCudnn.scala:142-1939).  Method names and
+argument meaning follow the trait; Scala's symbolic methods are spelled out
+(`+` -> add, `-` -> sub, `*` -> mul, `/` -> div, `+=` -> add_inplace, ...).
+
+In the reference these methods run on the JVM at staging time and emit C++ text; here the same
+calls are issued directly, one C-ABI call (include/lantern_hip.h) per emitted call.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+ADD, SUB, MUL, DIV = 0, 1, 2, 3
+RELU, TANH, SIGMOID, EXP, LOG, SQRT, SQUARE, HARDTANH = range(8)
+
+
+class Buf:
+    """A span of backend memory: address, element count (4-byte elements) and an owner to keep alive."""
+    __slots__ = ("ptr", "n", "keep")
+
+    def __init__(self, ptr, n, keep=None):
+        self.ptr = int(ptr)
+        self.n = int(n)
+        self.keep = keep
+
+    def offset(self, k, n=None):
+        """`slice(arr, off)` of the reference (TD:55): same memory, starting k elements in."""
+        return Buf(self.ptr + 4 * int(k), self.n - int(k) if n is None else n, self.keep)
+
+
+def _ints(seq):
+    return (C.c_int * len(seq))(*[int(v) for v in seq])
+
+
+def dim_broadcast(a, b):
+    """Tensor.dimBroadcast (TD:997-1016): right-aligned numpy rules -> (aShape, bShape, resShape)."""
+    a, b = list(a), list(b)
+    r = max(len(a), len(b))
+    a = [1] * (r - len(a)) + a
+    b = [1] * (r - len(b)) + b
+    res = []
+    for x, y in zip(a, b):
+        if not (x == 1 or y == 1 or x == y):
+            raise ValueError("dimensions not compatible for broadcasting %s with %s" % (a, b))
+        res.append(max(x, y))
+    return tuple(a), tuple(b), tuple(res)
+
+
+def conv_size(size, kernel, stride, pad=0):
+    """convSize (TD:34)."""
+    return (size + 2 * pad - kernel) // stride + 1
+
+
+class Backend:
+    """Operator API (TD:137-379).  Tensors are passed as objects with `.data` (Buf) and `.shape`."""
+
+    name = "abstract"
+
+    # -- memory ---------------------------------------------------------------------------
+    def setup(self): raise NotImplementedError
+    def cleanup(self): raise NotImplementedError
+    def mallocArray(self, length, zero=True): raise NotImplementedError     # TD:145
+    def copyFloatArray(self, dest, src, length): raise NotImplementedError  # TD:150
+    def fromHost(self, arr): raise NotImplementedError                      # toGPU (CUB:37-66)
+    def toHost(self, buf, n, dtype=np.float32): raise NotImplementedError   # toCPU (CUB:68-107)
+    def getMallocAddr(self): raise NotImplementedError                      # TD:1782-1784 / CUB:18-20
+    def resetMallocAddr(self, addr): raise NotImplementedError              # TD:1786-1789 / CUB:22-25
+
+
+class BackendHIP(Backend):
+    """The MI355X backend: every method is one or a few calls into liblantern_hip.so.
+
+    Errors raise LanternHipError (the library runs in "record and return" mode under Python;
+    generated C++ hosts keep the reference's print-and-exit behaviour).
+    """
+
+    name = "hip"
+
+    def __init__(self, heap_bytes=8 << 30):
+        self.heap_bytes = int(heap_bytes)
+        self.lib = None
+        self.dropout_seed = 42
+        self.dropout_offset = 0
+
+    # -- lifetime / arena -------------------------------------------------------------------
+    def setup(self):
+        self.lib = _lib.load()
+        self.lib.lh_set_error_mode(1)
+        self.lib.lh_setup(self.heap_bytes)
+        _lib.check()
+
+    def cleanup(self):
+        if self.lib is not None:
+            self.lib.lh_cleanup()
+            self.lib = None
+
+    def sync(self):
+        self.lib.lh_sync(); _lib.check()
+
+    def mallocArray(self, length, zero=True):
+        n = max(int(length), 1)
+        p = (self.lib.lh_malloc if zero else self.lib.lh_malloc_uninit)(4 * n)
+        _lib.check()
+        return Buf(p, n)
+
+    def getMallocAddr(self):
+        return self.lib.lh_mark()
+
+    def resetMallocAddr(self, addr):
+        self.lib.lh_rewind(addr); _lib.check()
+
+    def copyFloatArray(self, dest, src, length):
+        self.lib.lh_d2d(dest.ptr, src.ptr, 4 * int(length)); _lib.check()
+
+    def fromHost(self, arr):
+        arr = np.ascontiguousarray(arr)
+        assert arr.dtype.itemsize == 4, "only 4-byte element types cross the boundary"
+        buf = self.mallocArray(arr.size, zero=False)
+        if arr.size:
+            self.lib.lh_h2d(buf.ptr, arr.ctypes.data, arr.nbytes); _lib.check()
+        return buf
+
+    def toHost(self, buf, n, dtype=np.float32):
+        out = np.empty(int(n), dtype=dtype)
+        if n:
+            self.lib.lh_d2h(out.ctypes.data, buf.ptr, out.nbytes); _lib.check()
+        return out
+
+    def upload(self, buf, arr):
+        arr = np.ascontiguousarray(arr)
+        self.lib.lh_h2d(buf.ptr, arr.ctypes.data, arr.nbytes); _lib.check()
+
+    # -- fills ------------------------------------------------------------------------------
+    def fillInPlace(self, data, n, value):
+        self.lib.lh_fill(data.ptr, value, n); _lib.check()
+
+    def fillWithBias(self, dims, bias, dim):
+        outer = int(np.prod(dims[:dim], dtype=np.int64)); c = dims[dim]; inner = int(np.prod(dims[dim + 1:], dtype=np.int64))
+        res = self.mallocArray(outer * c * inner, zero=False)
+        self.lib.lh_fill_with_bias(res.ptr, bias.ptr, outer, c, inner); _lib.check()
+        return res
+
+    def clipAt(self, data, n, bound):
+        self.lib.lh_clip(data.ptr, bound, n); _lib.check()
+
+    # -- dot family (TD:186-219; CUB:173-282) -----------------------------------------------
+    def vectorVectorDot(self, x, y, n):
+        res = self.mallocArray(1, zero=False)
+        self.lib.lh_dot_vv(x.ptr, y.ptr, res.ptr, n); _lib.check()
+        return res
+
+    def matrixVectorDot(self, x, y, m, n):
+        res = self.mallocArray(m, zero=False)
+        self.lib.lh_sgemv(0, m, n, 1.0, x.ptr, n, y.ptr, 0.0, res.ptr); _lib.check()
+        return res
+
+    def matrixMatrixDot(self, x, y, m, k, n):
+        res = self.mallocArray(m * n, zero=False)
+        self.lib.lh_sgemm(0, 0, m, n, k, 1.0, x.ptr, k, y.ptr, n, 0.0, res.ptr, n); _lib.check()
+        return res
+
+    def addMul_scalar(self, xd, s, y, n):           # x.d.addMul(output.d.data(0), y.x)  (CPU:174-175)
+        self.lib.lh_axpy_dev(xd.ptr, s.ptr, y.ptr, n); _lib.check()
+
+    def add_cartesian(self, xd, y, outd, m, n):     # xd[m,n] += outd[m] (x) y[n]
+        self.lib.lh_ger(m, n, outd.ptr, y.ptr, xd.ptr); _lib.check()
+
+    def add_composition(self, xd, y, outd, m, n):   # xd[n] += y[m,n]^T outd[m]
+        self.lib.lh_sgemv(1, m, n, 1.0, y.ptr, n, outd.ptr, 1.0, xd.ptr); _lib.check()
+
+    def add_dotTrans1(self, xd, y, outd, d1, d2, d3):  # xd[d2,d3] += y[d1,d2]^T outd[d1,d3]
+        self.lib.lh_sgemm(1, 0, d2, d3, d1, 1.0, y.ptr, d2, outd.ptr, d3, 1.0, xd.ptr, d3); _lib.check()
+
+    def add_dotTrans2(self, xd, y, outd, d1, d2, d3):  # xd[d1,d2] += y[d1,d3] outd[d2,d3]^T
+        self.lib.lh_sgemm(0, 1, d1, d2, d3, 1.0, y.ptr, d3, outd.ptr, d3, 1.0, xd.ptr, d2); _lib.check()
+
+    # -- gemm (TD:279-280; CUB:589-688): result [d1,d3], contraction d2 --------------------------
+    def gemm(self, x, tx, y, ty, alpha, d1, d2, d3):
+        res = self.mallocArray(d1 * d3, zero=False)
+        self.lib.lh_sgemm(int(tx), int(ty), d1, d3, d2, alpha, x.ptr, d1 if tx else d2, y.ptr, d2 if ty else d3, 0.0, res.ptr, d3)
+        _lib.check()
+        return res
+
+    def gemm_grad(self, x, xd, x_in, tx, y, yd, y_in, ty, alpha, od, d1, d2, d3):
+        g = self.lib.lh_sgemm
+        if not tx and not ty:
+            if not x_in: g(0, 1, d1, d2, d3, alpha, od.ptr, d3, y.ptr, d3, 1.0, xd.ptr, d2)
+            if not y_in: g(1, 0, d2, d3, d1, alpha, x.ptr, d2, od.ptr, d3, 1.0, yd.ptr, d3)
+        elif not tx and ty:
+            if not x_in: g(0, 0, d1, d2, d3, alpha, od.ptr, d3, y.ptr, d2, 1.0, xd.ptr, d2)
+            if not y_in: g(1, 0, d3, d2, d1, alpha, od.ptr, d3, x.ptr, d2, 1.0, yd.ptr, d2)
+        elif tx and not ty:
+            if not x_in: g(0, 1, d2, d1, d3, alpha, y.ptr, d3, od.ptr, d3, 1.0, xd.ptr, d1)
+            if not y_in: g(0, 0, d2, d3, d1, alpha, x.ptr, d1, od.ptr, d3, 1.0, yd.ptr, d3)
+        else:
+            if not x_in: g(1, 1, d2, d1, d3, alpha, y.ptr, d2, od.ptr, d3, 1.0, xd.ptr, d1)
+            if not y_in: g(1, 1, d3, d2, d1, alpha, od.ptr, d3, x.ptr, d1, 1.0, yd.ptr, d2)
+        _lib.check()
+
+    # -- broadcast arithmetic (TD:222-270) ---------------------------------------------------------
+    def bcast_op(self, op, a, ashape, b, bshape, oshape):
+        n = int(np.prod(oshape, dtype=np.int64))
+        res = self.mallocArray(n, zero=False)
+        self.lib.lh_bcast_op(op, a.ptr, _ints(ashape), b.ptr, _ints(bshape), res.ptr, _ints(oshape), len(oshape)); _lib.check()
+        return res
+
+    def bcast_op_grad(self, op, a, ad, ashape, a_in, b, bd, bshape, b_in, od, oshape):
+        self.lib.lh_bcast_op_grad(op, a.ptr, 0 if a_in else ad.ptr, _ints(ashape), int(a_in), b.ptr, 0 if b_in else bd.ptr, _ints(bshape), int(b_in),
+                                  od.ptr, _ints(oshape), len(oshape)); _lib.check()
+
+    def bcast_update(self, op, a, ashape, b, bshape):
+        self.lib.lh_bcast_update(op, a.ptr, _ints(ashape), b.ptr, _ints(bshape), len(ashape)); _lib.check()
+
+    def scalar_op(self, op, x, s, n, out=None):
+        res = out if out is not None else self.mallocArray(n, zero=False)
+        self.lib.lh_scalar_op(op, x.ptr, res.ptr, s, n); _lib.check()
+        return res
+
+    def geam(self, x, alpha, y, beta, out, n):
+        self.lib.lh_geam(x.ptr, alpha, y.ptr, beta, out.ptr, n); _lib.check()
+
+    def trans(self, x, rows, cols):
+        res = self.mallocArray(rows * cols, zero=False)
+        self.lib.lh_trans(x.ptr, res.ptr, rows, cols); _lib.check()
+        return res
+
+    def trans_grad(self, xd, yd, rows, cols):
+        self.lib.lh_trans_grad(xd.ptr, yd.ptr, rows, cols); _lib.check()
+
+    def permute(self, x, dims, perm):
+        res = self.mallocArray(int(np.prod(dims, dtype=np.int64)), zero=False)
+        self.lib.lh_permute(x.ptr, res.ptr, _ints(dims), _ints(perm), len(dims)); _lib.check()
+        return res
+
+    def permute_grad(self, xd, yd, dims, perm):
+        self.lib.lh_permute_grad(xd.ptr, yd.ptr, _ints(dims), _ints(perm), len(dims)); _lib.check()
+
+    # -- conv / pool / bn ---------------------------------------------------------------------------
+    def conv2D_batch(self, x, w, bias, N, C, H, W, K, R, S, sH, sW, pH, pW):
+        P, Q = conv_size(H, R, sH, pH), conv_size(W, S, sW, pW)
+        y = self.mallocArray(N * K * P * Q, zero=False)
+        self.lib.lh_conv2d_fwd(x.ptr, w.ptr, bias.ptr if bias is not None else 0, y.ptr, N, C, H, W, K, R, S, sH, sW, pH, pW); _lib.check()
+        return y, None      # no im2col buffer is kept (BackendCudnn returns None too, CDN:859-866)
+
+    def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW):
+        if not x_in:
+            self.lib.lh_conv2d_bwd_data(dy.ptr, w.ptr, xd.ptr, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
+        self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
+        _lib.check()
+
+    def maxPool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW, pad):
+        P, Q = conv_size(H, kH, sH, pad), conv_size(W, kW, sW, pad)
+        y = self.mallocArray(N * C * P * Q, zero=False); idx = self.mallocArray(N * C * P * Q, zero=False)
+        self.lib.lh_maxpool_fwd(x.ptr, y.ptr, idx.ptr, N, C, H, W, kH, kW, sH, sW, pad); _lib.check()
+        return y, idx
+
+    def maxPool2D_batch_grad(self, xd, dy, idx, n_out):
+        self.lib.lh_maxpool_bwd(dy.ptr, idx.ptr, xd.ptr, n_out); _lib.check()
+
+    def averagePool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW):
+        P, Q = conv_size(H, kH, sH), conv_size(W, kW, sW)
+        y = self.mallocArray(N * C * P * Q, zero=False)
+        self.lib.lh_avgpool_fwd(x.ptr, y.ptr, N, C, H, W, kH, kW, sH, sW); _lib.check()
+        return y
+
+    def averagePool2D_batch_grad(self, xd, dy, N, C, H, W, kH, kW, sH, sW):
+        self.lib.lh_avgpool_bwd(dy.ptr, xd.ptr, N, C, H, W, kH, kW, sH, sW); _lib.check()
+
+    def batchNormInference(self, x, scale, bias, rmean, rvar, N, C, HW, eps=1e-5):
+        y = self.mallocArray(N * C * HW, zero=False)
+        self.lib.lh_bn_infer(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, N, C, HW, eps); _lib.check()
+        return y
+
+    def batchNormTraining(self, x, scale, bias, rmean, rvar, N, C, HW, eps=1e-5, factor=0.1):
+        y = self.mallocArray(N * C * HW, zero=False)
+        sm = self.mallocArray(C, zero=False); si = self.mallocArray(C, zero=False)
+        self.lib.lh_bn_train_fwd(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
+        return y, sm, si
+
+    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW):
+        self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, 1.0, scaled.ptr, biasd.ptr, N, C, HW); _lib.check()
+
+    # -- dropout ------------------------------------------------------------------------------------
+    def dropout(self, x, n, prob):
+        if not (0.0 <= prob < 1.0):
+            raise ValueError("dropout rate should be [0.0, 1), got %s" % prob)
+        y = self.mallocArray(n, zero=False); mask = self.mallocArray(n, zero=False)
+        self.lib.lh_dropout_fwd(x.ptr, y.ptr, mask.ptr, n, prob, self.dropout_seed, self.dropout_offset); _lib.check()
+        self.dropout_offset += n
+        return y, mask
+
+    def dropout_grad(self, xd, dy, mask, n):
+        self.lib.lh_dropout_bwd(dy.ptr, mask.ptr, xd.ptr, n); _lib.check()
+
+    def mask4D(self, x, lengths, n, c, d, t):
+        self.lib.lh_mask4d(x.ptr, lengths.ptr, n, c, d, t); _lib.check()
+
+    # -- activations ---------------------------------------------------------------------------------
+    def unary(self, op, x, n, inPlace=False, lo=-1.0, hi=1.0):
+        y = x if inPlace else self.mallocArray(n, zero=False)
+        self.lib.lh_unary(op, x.ptr, y.ptr, n, lo, hi); _lib.check()
+        return y
+
+    def unary_grad(self, op, x, y, dy, dx, n, inPlace=False, lo=-1.0, hi=1.0):
+        self.lib.lh_unary_grad(op, x.ptr, y.ptr, dy.ptr, dx.ptr, n, int(inPlace), lo, hi); _lib.check()
+
+    # -- softmax / loss --------------------------------------------------------------------------------
+    def softmax(self, is_log, x, outer, c, inner):
+        y = self.mallocArray(outer * c * inner, zero=False)
+        self.lib.lh_softmax(int(is_log), x.ptr, y.ptr, outer, c, inner); _lib.check()
+        return y
+
+    def softmax_grad(self, is_log, y, dy, dx, outer, c, inner):
+        self.lib.lh_softmax_grad(int(is_log), y.ptr, dy.ptr, dx.ptr, outer, c, inner); _lib.check()
+
+    def nllLoss(self, x, target, batch, stride):
+        y = self.mallocArray(batch, zero=False)
+        self.lib.lh_nll(x.ptr, target.ptr, y.ptr, batch, stride); _lib.check()
+        return y
+
+    def nllLoss_grad(self, dx, target, dy, batch, stride):
+        self.lib.lh_nll_grad(dx.ptr, target.ptr, dy.ptr, batch, stride); _lib.check()
+
+    # -- reductions -------------------------------------------------------------------------------------
+    def sum(self, x, n):
+        y = self.mallocArray(1, zero=False)
+        self.lib.lh_sum_all(x.ptr, y.ptr, n); _lib.check()
+        return y
+
+    def mean(self, x, n):
+        y = self.mallocArray(1, zero=False)
+        self.lib.lh_mean_all(x.ptr, y.ptr, n); _lib.check()
+        return y
+
+    def add_scalar_from(self, dx, dy1, scale, n):       # sum_grad / mean_grad
+        self.lib.lh_add_scalar_from(dx.ptr, dy1.ptr, scale, n); _lib.check()
+
+    def sum_dim(self, x, outer, dim, inner):
+        y = self.mallocArray(outer * inner, zero=False)
+        self.lib.lh_sum_dim(x.ptr, y.ptr, outer, dim, inner); _lib.check()
+        return y
+
+    def sum_dim_grad(self, dx, dy, outer, dim, inner):
+        self.lib.lh_sum_dim_grad(dx.ptr, dy.ptr, outer, dim, inner); _lib.check()
+
+    def concat(self, bufs, sizes, outer, inner):
+        total = outer * inner * sum(sizes)
+        res = self.mallocArray(total, zero=False)
+        ptrs = (C.c_void_p * len(bufs))(*[b.ptr for b in bufs])
+        self.lib.lh_concat(len(bufs), ptrs, _ints(sizes), res.ptr, outer, inner); _lib.check()
+        return res
+
+    def concat_grad(self, dbufs, sizes, outd, outer, inner):
+        ptrs = (C.c_void_p * len(dbufs))(*[(b.ptr if b is not None else 0) for b in dbufs])
+        self.lib.lh_concat_grad(len(dbufs), ptrs, _ints(sizes), outd.ptr, outer, inner); _lib.check()
+
+    # -- optimizers ----------------------------------------------------------------------------------------
+    def sgd_update(self, x, d, lr, n):
+        self.lib.lh_sgd(x.ptr, d.ptr, lr, n); _lib.check()
+
+    def adagrad_update(self, x, d, m, lr, clip, n):
+        self.lib.lh_adagrad(x.ptr, d.ptr, m.ptr, lr, clip, n); _lib.check()
+
+    def momentum_update(self, x, d, v, lr, mu, clip, nesterov, n):
+        self.lib.lh_momentum(x.ptr, d.ptr, v.ptr, lr, mu, clip, int(nesterov), n); _lib.check()
+
+    def multi_momentum_update(self, params, lr, mu, clip, nesterov):
+        """params: list of (x Buf, d Buf, v Buf, n).  One launch for the whole model."""
+        k = len(params)
+        key = tuple((p[0].ptr, p[1].ptr, p[2].ptr, p[3]) for p in params)
+        if getattr(self, "_mt_key", None) != key:
+            self._mt_key = key
+            self._mt = ((C.c_void_p * k)(*[p[0].ptr for p in params]), (C.c_void_p * k)(*[p[1].ptr for p in params]),
+                        (C.c_void_p * k)(*[p[2].ptr for p in params]), (C.c_int64 * k)(*[p[3] for p in params]))
+        xs, ds, vs, ns = self._mt
+        self.lib.lh_multi_momentum(k, xs, ds, vs, ns, lr, mu, clip, int(nesterov)); _lib.check()
+
+    def multi_sgd_update(self, params, lr):
+        k = len(params)
+        key = tuple((p[0].ptr, p[1].ptr, p[2]) for p in params)
+        if getattr(self, "_ms_key", None) != key:
+            self._ms_key = key
+            self._ms = ((C.c_void_p * k)(*[p[0].ptr for p in params]), (C.c_void_p * k)(*[p[1].ptr for p in params]),
+                        (C.c_int64 * k)(*[p[2] for p in params]))
+        xs, ds, ns = self._ms
+        self.lib.lh_multi_sgd(k, xs, ds, ns, lr); _lib.check()

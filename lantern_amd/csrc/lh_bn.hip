@@ -1,0 +1,223 @@
+// Batch normalisation, training forward / backward and inference, for x viewed as [N, C, HW].
+// HBM-bound: the forward reads x twice and writes y (12 B/element), the backward reads x and
+// dy twice and writes dx (20 B/element, 24 when dx accumulates).  Each pass is a 2-D grid
+// (channel, slice of the batch) so that even 64-channel layers fill 256 CUs; per-slice
+// partial statistics go through a small device scratch and are combined (Chan's parallel
+// variance formula, in double) by every block of the second pass.
+#include "lh_common.h"
+using namespace lh;
+
+namespace {
+constexpr int TPB = 256;
+constexpr int MAX_PARTIALS = 1 << 16;           // C * slices upper bound
+__device__ float g_bn_partial[3 * MAX_PARTIALS];
+static float* g_partial_ptr = nullptr;
+
+struct Plan { int slices; int n_per; bool vec4; };
+static Plan make_plan(int N, int C, int HW, bool aligned) {
+  Plan p;
+  int want = (int)cdiv(8 * (int64_t)g_num_cu, C);          // aim at ~8 blocks per CU in total
+  if (want < 1) want = 1;
+  if (want > N) want = N;
+  // keep at least ~4096 elements per block
+  int64_t per_sample = HW;
+  int min_n = (int)cdiv(4096, per_sample);
+  int max_slices = N / (min_n < 1 ? 1 : min_n); if (max_slices < 1) max_slices = 1;
+  if (want > max_slices) want = max_slices;
+  while ((int64_t)want * C > MAX_PARTIALS && want > 1) want--;
+  p.n_per = (int)cdiv(N, want);
+  p.slices = (int)cdiv(N, p.n_per);
+  p.vec4 = (HW % 4) == 0 && aligned;
+  return p;
+}
+
+// Visit the elements of channel c in samples [n0, n1): f4(offset) per aligned group of four
+// when VEC (HW % 4 == 0), else f1(offset) per element.
+template <bool VEC, class F4, class F1>
+__device__ __forceinline__ void bn_foreach(int n0, int n1, int C, int c, int HW, F4 f4, F1 f1) {
+  if (VEC) {
+    const int U = HW >> 2; const int64_t total = (int64_t)(n1 - n0) * U;
+    for (int64_t u = threadIdx.x; u < total; u += TPB) {
+      int dn = (int)(u / U); int q = (int)(u - (int64_t)dn * U);
+      f4(((int64_t)(n0 + dn) * C + c) * HW + 4 * q);
+    }
+  } else {
+    const int64_t total = (int64_t)(n1 - n0) * HW;
+    for (int64_t u = threadIdx.x; u < total; u += TPB) {
+      int dn = (int)(u / HW); int l = (int)(u - (int64_t)dn * HW);
+      f1(((int64_t)(n0 + dn) * C + c) * HW + l);
+    }
+  }
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(TPB) k_bn_stats(const float* __restrict__ x, float* __restrict__ partial, int N, int C, int HW, int n_per) {
+  __shared__ float sm[17];
+  const int c = blockIdx.x, s = blockIdx.y;
+  const int n0 = s * n_per, n1 = min(N, n0 + n_per);
+  const float K = x[((int64_t)n0 * C + c) * HW];      // shift: removes cancellation in sum of squares
+  float s1 = 0.f, s2 = 0.f;
+  bn_foreach<VEC>(n0, n1, C, c, HW,
+    [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off);
+      float a = v.x - K, b = v.y - K, d = v.z - K, e = v.w - K;
+      s1 += (a + b) + (d + e); s2 += (a * a + b * b) + (d * d + e * e); },
+    [&](int64_t off) { float a = x[off] - K; s1 += a; s2 += a * a; });
+  s1 = lh_block_sum(s1, sm);
+  s2 = lh_block_sum(s2, sm);
+  if (threadIdx.x == 0) {
+    float cnt = (float)((int64_t)(n1 - n0) * HW);
+    float* p = partial + 3 * ((int64_t)c * gridDim.y + s);
+    p[0] = K + s1 / cnt;            // slice mean
+    p[1] = s2 - s1 * s1 / cnt;      // slice M2
+    p[2] = cnt;
+  }
+}
+
+__device__ __forceinline__ void combine_stats(const float* partial, int c, int slices, double& mean, double& m2, double& cnt) {
+  cnt = 0.0; double wsum = 0.0;
+  for (int s = 0; s < slices; s++) { const float* p = partial + 3 * ((int64_t)c * slices + s); cnt += p[2]; wsum += (double)p[0] * p[2]; }
+  mean = wsum / cnt; m2 = 0.0;
+  for (int s = 0; s < slices; s++) { const float* p = partial + 3 * ((int64_t)c * slices + s); double d = p[0] - mean; m2 += p[1] + p[2] * d * d; }
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(TPB) k_bn_fwd_apply(const float* __restrict__ x, float* __restrict__ y, const float* __restrict__ partial,
+                                                      const float* gamma, const float* beta, float* run_mean, float* run_var,
+                                                      float* save_mean, float* save_invstd, int N, int C, int HW, int n_per, float eps, float factor) {
+  __shared__ float sh[2];
+  const int c = blockIdx.x, s = blockIdx.y;
+  if (threadIdx.x == 0) {
+    double mean, m2, cnt;
+    combine_stats(partial, c, gridDim.y, mean, m2, cnt);
+    float var = (float)(m2 / cnt);
+    float invstd = 1.0f / sqrtf(var + eps);
+    sh[0] = (float)mean; sh[1] = invstd;
+    if (s == 0) {
+      if (save_mean) save_mean[c] = (float)mean;
+      if (save_invstd) save_invstd[c] = invstd;
+      if (run_mean) run_mean[c] = (1.0f - factor) * run_mean[c] + factor * (float)mean;
+      if (run_var) { float unb = cnt > 1.0 ? (float)(m2 / (cnt - 1.0)) : var; run_var[c] = (1.0f - factor) * run_var[c] + factor * unb; }
+    }
+  }
+  __syncthreads();
+  const float mean = sh[0], invstd = sh[1], g = gamma[c], b = beta[c];
+  const int n0 = s * n_per, n1 = min(N, n0 + n_per);
+  bn_foreach<VEC>(n0, n1, C, c, HW,
+    [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 r;
+      r.x = (v.x - mean) * invstd * g + b; r.y = (v.y - mean) * invstd * g + b;
+      r.z = (v.z - mean) * invstd * g + b; r.w = (v.w - mean) * invstd * g + b;
+      *reinterpret_cast<float4*>(y + off) = r; },
+    [&](int64_t off) { y[off] = (x[off] - mean) * invstd * g + b; });
+}
+
+template <bool VEC>
+__global__ void __launch_bounds__(TPB) k_bn_bwd_stats(const float* __restrict__ x, const float* __restrict__ dy, const float* save_mean, const float* save_invstd,
+                                                      float* __restrict__ partial, int N, int C, int HW, int n_per) {
+  __shared__ float sm[17];
+  const int c = blockIdx.x, s = blockIdx.y;
+  const int n0 = s * n_per, n1 = min(N, n0 + n_per);
+  const float mean = save_mean[c], is = save_invstd[c];
+  float s1 = 0.f, s2 = 0.f;
+  bn_foreach<VEC>(n0, n1, C, c, HW,
+    [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 g = *reinterpret_cast<const float4*>(dy + off);
+      s1 += (g.x + g.y) + (g.z + g.w);
+      s2 += (g.x * ((v.x - mean) * is) + g.y * ((v.y - mean) * is)) + (g.z * ((v.z - mean) * is) + g.w * ((v.w - mean) * is)); },
+    [&](int64_t off) { float g = dy[off]; s1 += g; s2 += g * ((x[off] - mean) * is); });
+  s1 = lh_block_sum(s1, sm);
+  s2 = lh_block_sum(s2, sm);
+  if (threadIdx.x == 0) { float* p = partial + 3 * ((int64_t)c * gridDim.y + s); p[0] = s1; p[1] = s2; }
+}
+
+template <bool VEC, bool ACC>
+__global__ void __launch_bounds__(TPB) k_bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ partial,
+                                                      const float* gamma, const float* save_mean, const float* save_invstd,
+                                                      float* __restrict__ dx, float* dgamma, float* dbeta, int N, int C, int HW, int n_per) {
+  __shared__ float sh[2];
+  const int c = blockIdx.x, s = blockIdx.y;
+  if (threadIdx.x == 0) {
+    double a = 0.0, b = 0.0;
+    for (int t = 0; t < (int)gridDim.y; t++) { const float* p = partial + 3 * ((int64_t)c * gridDim.y + t); a += p[0]; b += p[1]; }
+    double cnt = (double)N * HW;
+    sh[0] = (float)(a / cnt); sh[1] = (float)(b / cnt);
+    if (s == 0) { if (dgamma) dgamma[c] += (float)b; if (dbeta) dbeta[c] += (float)a; }
+  }
+  __syncthreads();
+  if (dx == nullptr) return;
+  const float m1 = sh[0], m2 = sh[1], mean = save_mean[c], is = save_invstd[c], g = gamma[c] * is;
+  const int n0 = s * n_per, n1 = min(N, n0 + n_per);
+  bn_foreach<VEC>(n0, n1, C, c, HW,
+    [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 d = *reinterpret_cast<const float4*>(dy + off); float4 r;
+      r.x = g * (d.x - m1 - (v.x - mean) * is * m2); r.y = g * (d.y - m1 - (v.y - mean) * is * m2);
+      r.z = g * (d.z - m1 - (v.z - mean) * is * m2); r.w = g * (d.w - m1 - (v.w - mean) * is * m2);
+      if (ACC) { float4 o = *reinterpret_cast<const float4*>(dx + off); r.x += o.x; r.y += o.y; r.z += o.z; r.w += o.w; }
+      *reinterpret_cast<float4*>(dx + off) = r; },
+    [&](int64_t off) { float r = g * (dy[off] - m1 - (x[off] - mean) * is * m2); if (ACC) r += dx[off]; dx[off] = r; });
+}
+
+__global__ void __launch_bounds__(TPB) k_bn_infer(const float* __restrict__ x, float* __restrict__ y, const float* gamma, const float* beta,
+                                                  const float* rmean, const float* rvar, int C, int HW, int64_t n, float eps) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    int c = (int)((i / HW) % C);
+    y[i] = (x[i] - rmean[c]) / sqrtf(rvar[c] + eps) * gamma[c] + beta[c];
+  }
+}
+
+static bool get_partial() {
+  if (g_partial_ptr) return true;
+  if (hipGetSymbolAddress((void**)&g_partial_ptr, HIP_SYMBOL(g_bn_partial)) != hipSuccess) { LH_FAIL("bn scratch symbol lookup failed"); return false; }
+  return true;
+}
+}  // namespace
+
+extern "C" {
+
+void lh_bn_infer(const float* x, const float* gamma, const float* beta, const float* run_mean, const float* run_var,
+                 float* y, int N, int C, int HW, float eps) {
+  int64_t n = (int64_t)N * C * HW;
+  if (n <= 0) return;
+  hipLaunchKernelGGL(k_bn_infer, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, gamma, beta, run_mean, run_var, C, HW, n, eps);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                     float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
+  LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_train_fwd: empty shape [%d,%d,%d]", N, C, HW);
+  LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_train_fwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
+  if (!get_partial()) return;
+  Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)y) & 15) == 0);
+  dim3 grid(C, p.slices);
+  if (p.vec4) {
+    hipLaunchKernelGGL((k_bn_stats<true>), grid, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, HW, p.n_per);
+    hipLaunchKernelGGL((k_bn_fwd_apply<true>), grid, dim3(TPB), 0, g_stream, x, y, (const float*)g_partial_ptr, gamma, beta, run_mean, run_var,
+                       save_mean, save_invstd, N, C, HW, p.n_per, eps, factor);
+  } else {
+    hipLaunchKernelGGL((k_bn_stats<false>), grid, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, HW, p.n_per);
+    hipLaunchKernelGGL((k_bn_fwd_apply<false>), grid, dim3(TPB), 0, g_stream, x, y, (const float*)g_partial_ptr, gamma, beta, run_mean, run_var,
+                       save_mean, save_invstd, N, C, HW, p.n_per, eps, factor);
+  }
+  LH_CHECK_LAUNCH();
+}
+
+void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+               float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
+  LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_bwd: empty shape [%d,%d,%d]", N, C, HW);
+  LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_bwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
+  LH_REQUIRE(beta_dx == 0.0f || beta_dx == 1.0f, "lh_bn_bwd: beta must be 0 or 1");
+  if (!get_partial()) return;
+  Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx) & 15) == 0);
+  dim3 grid(C, p.slices);
+  const bool acc = beta_dx != 0.0f;
+#define BWD(V, A) hipLaunchKernelGGL((k_bn_bwd_apply<V, A>), grid, dim3(TPB), 0, g_stream, x, dy, (const float*)g_partial_ptr, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
+  if (p.vec4) {
+    hipLaunchKernelGGL((k_bn_bwd_stats<true>), grid, dim3(TPB), 0, g_stream, x, dy, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per);
+    if (acc) BWD(true, true); else BWD(true, false);
+  } else {
+    hipLaunchKernelGGL((k_bn_bwd_stats<false>), grid, dim3(TPB), 0, g_stream, x, dy, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per);
+    if (acc) BWD(false, true); else BWD(false, false);
+  }
+#undef BWD
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"

@@ -1,0 +1,606 @@
+// Streaming (HBM-bound) operators: fills, activations and their gradients, scalar and
+// broadcast arithmetic, permute, dropout, concat and the optimizer updates.
+// All are grid-stride kernels over float4 where the pointers allow it; each element is
+// read and written once, so the bound is bytes moved / HBM bandwidth.
+#include "lh_common.h"
+using namespace lh;
+
+namespace {
+
+constexpr int TPB = 256;
+
+__global__ void __launch_bounds__(TPB) k_fill(float* __restrict__ y, float v, int64_t n) {
+  // vector body (y 16-byte aligned at its base is required by the caller) + scalar tail
+  int64_t n4 = n >> 2;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n4; j += st) reinterpret_cast<float4*>(y)[j] = make_float4(v, v, v, v);
+  for (int64_t j = 4 * n4 + i; j < n; j += st) y[j] = v;
+}
+__global__ void __launch_bounds__(TPB) k_fill_scalar(float* y, float v, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) y[i] = v;
+}
+__global__ void __launch_bounds__(TPB) k_fill_bias(float* y, const float* bias, int64_t c, int64_t inner, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) y[i] = bias[(i / inner) % c];
+}
+
+static inline bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// ---- generic vectorised elementwise driver: out[i] = f(a[i], b[i], c[i]) --------------
+template <int NIN, class F>
+__global__ void __launch_bounds__(TPB) k_ew_vec(float* __restrict__ out, const float* a, const float* b, const float* c, int64_t n, F f) {
+  int64_t n4 = n >> 2;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n4; j += st) {
+    float4 va = reinterpret_cast<const float4*>(a)[j];
+    float4 vb = NIN > 1 ? reinterpret_cast<const float4*>(b)[j] : va;
+    float4 vc = NIN > 2 ? reinterpret_cast<const float4*>(c)[j] : va;
+    float4 r;
+    r.x = f(va.x, vb.x, vc.x); r.y = f(va.y, vb.y, vc.y); r.z = f(va.z, vb.z, vc.z); r.w = f(va.w, vb.w, vc.w);
+    reinterpret_cast<float4*>(out)[j] = r;
+  }
+  for (int64_t j = 4 * n4 + i; j < n; j += st) out[j] = f(a[j], NIN > 1 ? b[j] : 0.f, NIN > 2 ? c[j] : 0.f);
+}
+template <int NIN, class F>
+__global__ void __launch_bounds__(TPB) k_ew_scalar(float* out, const float* a, const float* b, const float* c, int64_t n, F f) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n; j += st) out[j] = f(a[j], NIN > 1 ? b[j] : 0.f, NIN > 2 ? c[j] : 0.f);
+}
+template <int NIN, class F>
+void ew(float* out, const float* a, const float* b, const float* c, int64_t n, F f) {
+  if (n <= 0) return;
+  bool vec = al16(out) && al16(a) && (NIN < 2 || al16(b)) && (NIN < 3 || al16(c));
+  int grid = stream_grid(n, TPB * 8);
+  if (vec) hipLaunchKernelGGL((k_ew_vec<NIN, F>), dim3(grid), dim3(TPB), 0, g_stream, out, a, b, c, n, f);
+  else hipLaunchKernelGGL((k_ew_scalar<NIN, F>), dim3(grid), dim3(TPB), 0, g_stream, out, a, b, c, n, f);
+}
+
+__device__ __forceinline__ float bop(int op, float a, float b) {
+  switch (op) { case LH_ADD: return a + b; case LH_SUB: return a - b; case LH_MUL: return a * b; default: return a / b; }
+}
+
+struct Dims4 { int d[4]; int64_t sa[4]; int64_t sb[4]; };
+
+}  // namespace
+
+extern "C" {
+
+void lh_fill(float* x, float v, int64_t n) {
+  if (n <= 0) return;
+  if (al16(x)) hipLaunchKernelGGL(k_fill, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, v, n);
+  else hipLaunchKernelGGL(k_fill_scalar, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, v, n);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, int64_t inner) {
+  int64_t n = outer * c * inner;
+  if (n <= 0) return;
+  hipLaunchKernelGGL(k_fill_bias, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, y, bias, c, inner, n);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_clip(float* x, float bound, int64_t n) {
+  ew<1>(x, x, nullptr, nullptr, n, [bound] __device__(float v, float, float) { return v > bound ? bound : (v < -bound ? -bound : v); });
+  LH_CHECK_LAUNCH();
+}
+
+__global__ void k_mask4d(float* x, const int* lengths, int64_t n, int cd, int t) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, st = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += st) {
+    int u = (int)(i % t);
+    int b = (int)(i / ((int64_t)cd * t));
+    if (u >= lengths[b]) x[i] = 0.f;
+  }
+}
+void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t) {
+  int64_t tot = (int64_t)n * c * d * t;
+  if (tot <= 0) return;
+  hipLaunchKernelGGL(k_mask4d, dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, x, lengths, tot, c * d, t);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) {
+  switch (op) {
+    case LH_RELU: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return v < 0.f ? 0.f : v; }); break;
+    case LH_TANH: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return tanhf(v); }); break;
+    case LH_SIGMOID: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return 1.0f / (expf(-v) + 1.0f); }); break;
+    case LH_EXP: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return expf(v); }); break;
+    case LH_LOG: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return logf(v); }); break;
+    case LH_SQRT: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return sqrtf(v); }); break;
+    case LH_SQUARE: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return v * v; }); break;
+    case LH_HARDTANH: ew<1>(y, x, nullptr, nullptr, n, [lo, hi] __device__(float v, float, float) { return v < lo ? lo : (v > hi ? hi : v); }); break;
+    default: LH_FAIL("lh_unary: unknown op %d", op); return;
+  }
+  LH_CHECK_LAUNCH();
+}
+
+void lh_unary_grad(int op, const float* x, const float* y, const float* dy, float* dx, int64_t n, int inplace, float lo, float hi) {
+  // out = dx; inputs (a, b, c) chosen per op.  All forms are dx (+)= g(x|y, dy).
+  switch (op) {
+    case LH_RELU:
+      if (inplace) ew<2>(dx, dx, y, nullptr, n, [] __device__(float d, float yv, float) { return yv > 0.f ? d : 0.f; });
+      else ew<3>(dx, dx, x, dy, n, [] __device__(float d, float xv, float g) { return d + (xv < 0.f ? 0.f : g); });
+      break;
+    case LH_HARDTANH:
+      if (inplace) ew<2>(dx, dx, y, nullptr, n, [lo, hi] __device__(float d, float yv, float) { return (yv > lo && yv < hi) ? d : 0.f; });
+      else ew<3>(dx, dx, x, dy, n, [lo, hi] __device__(float d, float xv, float g) { return d + ((xv < lo || xv > hi) ? 0.f : g); });
+      break;
+    case LH_TANH: ew<3>(dx, dx, y, dy, n, [] __device__(float d, float yv, float g) { return d + (1.0f - yv * yv) * g; }); break;
+    case LH_SIGMOID: ew<3>(dx, dx, y, dy, n, [] __device__(float d, float yv, float g) { return d + ((1.0f - yv) * yv) * g; }); break;
+    case LH_EXP: ew<3>(dx, dx, y, dy, n, [] __device__(float d, float yv, float g) { return d + g * yv; }); break;
+    case LH_LOG: ew<3>(dx, dx, x, dy, n, [] __device__(float d, float xv, float g) { return d + g / xv; }); break;
+    case LH_SQRT: ew<3>(dx, dx, y, dy, n, [] __device__(float d, float yv, float g) { return d + g / yv / 2.0f; }); break;
+    case LH_SQUARE: ew<3>(dx, dx, x, dy, n, [] __device__(float d, float xv, float g) { return d + g * xv * 2.0f; }); break;
+    default: LH_FAIL("lh_unary_grad: unknown op %d", op); return;
+  }
+  LH_CHECK_LAUNCH();
+}
+
+void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) {
+  LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_scalar_op: unknown op %d", op);
+  ew<1>(y, x, nullptr, nullptr, n, [op, s] __device__(float v, float, float) { return bop(op, v, s); });
+  LH_CHECK_LAUNCH();
+}
+
+void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) {
+  ew<2>(out, x, y, nullptr, n, [alpha, beta] __device__(float a, float b, float) { return a * alpha + b * beta; });
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------- broadcast -----------
+namespace {
+
+static bool same_dims(const int* a, const int* b, int rank) { for (int i = 0; i < rank; i++) if (a[i] != b[i]) return false; return true; }
+static int64_t prod(const int* d, int rank) { int64_t p = 1; for (int i = 0; i < rank; i++) p *= d[i]; return p; }
+
+static bool make_dims4(Dims4& D, const int* adims, const int* bdims, const int* odims, int rank) {
+  if (rank < 1 || rank > 4) return false;
+  int pad = 4 - rank;
+  int ad[4] = {1, 1, 1, 1}, bd[4] = {1, 1, 1, 1};
+  for (int i = 0; i < 4; i++) D.d[i] = 1;
+  for (int i = 0; i < rank; i++) { ad[pad + i] = adims[i]; bd[pad + i] = bdims[i]; D.d[pad + i] = odims[i]; }
+  int64_t s = 1; for (int i = 3; i >= 0; i--) { D.sa[i] = ad[i] == 1 ? 0 : s; s *= ad[i]; }
+  s = 1; for (int i = 3; i >= 0; i--) { D.sb[i] = bd[i] == 1 ? 0 : s; s *= bd[i]; }
+  for (int i = 0; i < 4; i++) {
+    if (ad[i] != 1 && ad[i] != D.d[i]) return false;
+    if (bd[i] != 1 && bd[i] != D.d[i]) return false;
+  }
+  return true;
+}
+
+__global__ void __launch_bounds__(TPB) k_bcast_op(int op, const float* a, const float* b, float* out, Dims4 D, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    int64_t r = i;
+    int i3 = (int)(r % D.d[3]); r /= D.d[3];
+    int i2 = (int)(r % D.d[2]); r /= D.d[2];
+    int i1 = (int)(r % D.d[1]); r /= D.d[1];
+    int i0 = (int)r;
+    int64_t ia = i0 * D.sa[0] + i1 * D.sa[1] + i2 * D.sa[2] + i3 * D.sa[3];
+    int64_t ib = i0 * D.sb[0] + i1 * D.sb[1] + i2 * D.sb[2] + i3 * D.sb[3];
+    out[i] = bop(op, a[ia], b[ib]);
+  }
+}
+
+// small[j] (op)= reduce over the broadcast positions of g(...).  One wave per small element.
+// mode 0: value = big[i]                       (bcast_update with reduction, ADD/SUB)
+// mode 1: value = grad wrt operand `which` of out = a op b, with outd = big
+template <int MODE>
+__global__ void __launch_bounds__(TPB) k_bcast_reduce(int op, int which, float* small, const float* a, const float* b, const float* big,
+                                                      Dims4 D /* d = out dims, sa = strides of small, sb = strides of other */,
+                                                      int64_t nsmall, int64_t nred, int rd0, int rd1, int rd2, int rd3) {
+  // rdX = size of the reduced index space along axis X (out dim where small dim == 1, else 1)
+  const int lane = threadIdx.x & 63;
+  int64_t w = ((int64_t)blockIdx.x * TPB + threadIdx.x) >> 6, nw = ((int64_t)gridDim.x * TPB) >> 6;
+  for (; w < nsmall; w += nw) {
+    // decode the kept coordinates of small element w (axes where small dim != 1)
+    int k[4]; int64_t r = w;
+    int kd3 = rd3 == 1 ? D.d[3] : 1, kd2 = rd2 == 1 ? D.d[2] : 1, kd1 = rd1 == 1 ? D.d[1] : 1;
+    k[3] = (int)(r % kd3); r /= kd3; k[2] = (int)(r % kd2); r /= kd2; k[1] = (int)(r % kd1); r /= kd1; k[0] = (int)r;
+    float acc = 0.f;
+    for (int64_t q = lane; q < nred; q += 64) {
+      int64_t t = q; int c[4];
+      c[3] = k[3] + (int)(t % rd3); t /= rd3; c[2] = k[2] + (int)(t % rd2); t /= rd2; c[1] = k[1] + (int)(t % rd1); t /= rd1; c[0] = k[0] + (int)t;
+      int64_t io = ((int64_t)(c[0] * D.d[1] + c[1]) * D.d[2] + c[2]) * D.d[3] + c[3];
+      float v = big[io];
+      if (MODE == 1) {
+        int64_t is = c[0] * D.sa[0] + c[1] * D.sa[1] + c[2] * D.sa[2] + c[3] * D.sa[3];   // index in small's own tensor
+        int64_t it = c[0] * D.sb[0] + c[1] * D.sb[1] + c[2] * D.sb[2] + c[3] * D.sb[3];   // index in the other operand
+        // which == 0: small is `a` (x), other is `b`; which == 1: small is `b`, other is `a`
+        float av = which == 0 ? a[is] : a[it];
+        float bv = which == 0 ? b[it] : b[is];
+        switch (op) {
+          case LH_ADD: break;
+          case LH_SUB: v = which == 0 ? v : 0.0f - v; break;
+          case LH_MUL: v = which == 0 ? v * bv : v * av; break;
+          default: v = which == 0 ? v / bv : -1.0f * av * v / (bv * bv); break;
+        }
+      }
+      acc += v;
+    }
+    acc = lh_wave_sum(acc);
+    if (lane == 0) {
+      if (MODE == 0 && op == LH_SUB) small[w] -= acc; else small[w] += acc;
+    }
+  }
+}
+
+// Elementwise part of a broadcast gradient for an operand that has the full output shape.
+__global__ void __launch_bounds__(TPB) k_bcast_grad_full(int op, int which, float* gd, const float* a, const float* b, const float* od, Dims4 D, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    int64_t r = i;
+    int i3 = (int)(r % D.d[3]); r /= D.d[3];
+    int i2 = (int)(r % D.d[2]); r /= D.d[2];
+    int i1 = (int)(r % D.d[1]); r /= D.d[1];
+    int i0 = (int)r;
+    int64_t ia = i0 * D.sa[0] + i1 * D.sa[1] + i2 * D.sa[2] + i3 * D.sa[3];
+    int64_t ib = i0 * D.sb[0] + i1 * D.sb[1] + i2 * D.sb[2] + i3 * D.sb[3];
+    float c = od[i], g;
+    switch (op) {
+      case LH_ADD: g = c; break;
+      case LH_SUB: g = which == 0 ? c : 0.0f - c; break;
+      case LH_MUL: g = which == 0 ? c * b[ib] : c * a[ia]; break;
+      default: g = which == 0 ? c / b[ib] : -1.0f * a[ia] * c / (b[ib] * b[ib]); break;
+    }
+    gd[i] += g;
+  }
+}
+
+// Launch the reduction of `big`-shaped values into the operand whose dims are sdims.
+template <int MODE>
+void launch_reduce(int op, int which, float* small, const int* sdims4, const float* a, const float* b, const float* big, const Dims4& Dsmall_other) {
+  int rd[4]; int64_t nred = 1, nsmall = 1;
+  for (int i = 0; i < 4; i++) {
+    rd[i] = (sdims4[i] == 1 && Dsmall_other.d[i] > 1) ? Dsmall_other.d[i] : 1;
+    nred *= rd[i];
+    nsmall *= (rd[i] == 1 ? Dsmall_other.d[i] : 1);
+  }
+  int grid = (int)cdiv(nsmall * 64, TPB); if (grid > g_num_cu * 16) grid = g_num_cu * 16; if (grid < 1) grid = 1;
+  hipLaunchKernelGGL((k_bcast_reduce<MODE>), dim3(grid), dim3(TPB), 0, g_stream, op, which, small, a, b, big, Dsmall_other, nsmall, nred, rd[0], rd[1], rd[2], rd[3]);
+}
+
+}  // namespace
+
+extern "C" {
+
+void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const int* bdims, float* out, const int* odims, int rank) {
+  LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_op: unknown op %d", op);
+  int64_t n = prod(odims, rank);
+  if (n <= 0) return;
+  if (same_dims(adims, odims, rank) && same_dims(bdims, odims, rank)) {
+    ew<2>(out, a, b, nullptr, n, [op] __device__(float x, float y, float) { return bop(op, x, y); });
+  } else {
+    Dims4 D;
+    LH_REQUIRE(make_dims4(D, adims, bdims, odims, rank), "lh_bcast_op: shapes do not broadcast (rank %d)", rank);
+    hipLaunchKernelGGL(k_bcast_op, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, op, a, b, out, D, n);
+  }
+  LH_CHECK_LAUNCH();
+}
+
+void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a_is_input,
+                      const float* b, float* bd, const int* bdims, int b_is_input,
+                      const float* outd, const int* odims, int rank) {
+  LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_op_grad: unknown op %d", op);
+  int64_t n = prod(odims, rank);
+  if (n <= 0) return;
+  Dims4 D;
+  LH_REQUIRE(make_dims4(D, adims, bdims, odims, rank), "lh_bcast_op_grad: shapes do not broadcast (rank %d)", rank);
+  int pad = 4 - rank; int a4[4] = {1, 1, 1, 1}, b4[4] = {1, 1, 1, 1};
+  for (int i = 0; i < rank; i++) { a4[pad + i] = adims[i]; b4[pad + i] = bdims[i]; }
+  bool a_full = same_dims(adims, odims, rank), b_full = same_dims(bdims, odims, rank);
+  if (!a_is_input) {
+    if (a_full) {
+      if (b_full && op == LH_ADD) ew<2>(ad, ad, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
+      else if (b_full && op == LH_SUB) ew<2>(ad, ad, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
+      else if (b_full && op == LH_MUL) ew<3>(ad, ad, outd, b, n, [] __device__(float d, float g, float bv) { return d + g * bv; });
+      else hipLaunchKernelGGL(k_bcast_grad_full, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, op, 0, ad, a, b, outd, D, n);
+    } else {
+      launch_reduce<1>(op, 0, ad, a4, a, b, outd, D);
+    }
+  }
+  if (!b_is_input) {
+    if (b_full) {
+      if (a_full && op == LH_ADD) ew<2>(bd, bd, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
+      else if (a_full && op == LH_SUB) ew<2>(bd, bd, outd, nullptr, n, [] __device__(float d, float g, float) { return d + (0.0f - g); });
+      else if (a_full && op == LH_MUL) ew<3>(bd, bd, outd, a, n, [] __device__(float d, float g, float av) { return d + g * av; });
+      else hipLaunchKernelGGL(k_bcast_grad_full, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, op, 1, bd, a, b, outd, D, n);
+    } else {
+      Dims4 Ds = D;  // small = b: swap stride roles so sa = strides of small (b), sb = strides of other (a)
+      for (int i = 0; i < 4; i++) { Ds.sa[i] = D.sb[i]; Ds.sb[i] = D.sa[i]; }
+      launch_reduce<1>(op, 1, bd, b4, a, b, outd, Ds);
+    }
+  }
+  LH_CHECK_LAUNCH();
+}
+
+void lh_bcast_update(int op, float* a, const int* adims, const float* b, const int* bdims, int rank) {
+  LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_update: unknown op %d", op);
+  LH_REQUIRE(rank >= 1 && rank <= 4, "lh_bcast_update: rank %d not in 1..4", rank);
+  int od[4];
+  for (int i = 0; i < rank; i++) od[i] = adims[i] > bdims[i] ? adims[i] : bdims[i];
+  int64_t n = prod(od, rank);
+  if (n <= 0) return;
+  if (same_dims(adims, od, rank)) {  // a has the full shape: a = a op broadcast(b)
+    if (same_dims(bdims, od, rank)) {
+      ew<2>(a, a, b, nullptr, n, [op] __device__(float x, float y, float) { return bop(op, x, y); });
+    } else {
+      Dims4 D;
+      LH_REQUIRE(make_dims4(D, adims, bdims, od, rank), "lh_bcast_update: shapes do not broadcast");
+      hipLaunchKernelGGL(k_bcast_op, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, op, (const float*)a, b, a, D, n);
+    }
+  } else {  // a is the smaller one: reduce b into a (the reference's loop applies op once per broadcast position)
+    LH_REQUIRE(op == LH_ADD || op == LH_SUB, "lh_bcast_update: reducing update supports += and -= only");
+    LH_REQUIRE(same_dims(bdims, od, rank), "lh_bcast_update: reduce source must have the full shape");
+    Dims4 D;
+    LH_REQUIRE(make_dims4(D, adims, bdims, od, rank), "lh_bcast_update: shapes do not broadcast");
+    int pad = 4 - rank; int a4[4] = {1, 1, 1, 1};
+    for (int i = 0; i < rank; i++) a4[pad + i] = adims[i];
+    launch_reduce<0>(op, 0, a, a4, nullptr, nullptr, b, D);
+  }
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------- permute / trans --------
+namespace {
+struct Perm4 { int yd[4]; int64_t sx[4]; };   // y dims and, for each y axis, the stride in x
+
+// 32x32 LDS-tiled transpose of the two fastest axes when the permutation moves x's fastest
+// axis; otherwise a plain gather keeps reads and writes contiguous along the last axis.
+template <bool GRAD>
+__global__ void __launch_bounds__(TPB) k_permute(const float* __restrict__ src, float* __restrict__ dst, Perm4 P, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    int64_t r = i;
+    int i3 = (int)(r % P.yd[3]); r /= P.yd[3];
+    int i2 = (int)(r % P.yd[2]); r /= P.yd[2];
+    int i1 = (int)(r % P.yd[1]); r /= P.yd[1];
+    int i0 = (int)r;
+    int64_t ix = i0 * P.sx[0] + i1 * P.sx[1] + i2 * P.sx[2] + i3 * P.sx[3];
+    if (GRAD) dst[ix] += src[i]; else dst[i] = src[ix];
+  }
+}
+template <bool GRAD>
+__global__ void __launch_bounds__(256) k_trans_tile(const float* __restrict__ src, float* __restrict__ dst, int rows, int cols, int64_t batch_stride) {
+  // !GRAD: dst[c][r] = src[r][c] (src rows x cols).  GRAD: dst is rows x cols, src is cols x rows: dst[r][c] += src[c][r].
+  __shared__ float tile[32][33];
+  const float* s = src + (int64_t)blockIdx.z * batch_stride;
+  float* d = dst + (int64_t)blockIdx.z * batch_stride;
+  int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  if (!GRAD) {
+    for (int j = ty; j < 32; j += 8) { int r = r0 + j, c = c0 + tx; if (r < rows && c < cols) tile[j][tx] = s[(int64_t)r * cols + c]; }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) { int c = c0 + j, r = r0 + tx; if (r < rows && c < cols) d[(int64_t)c * rows + r] = tile[tx][j]; }
+  } else {
+    for (int j = ty; j < 32; j += 8) { int c = c0 + j, r = r0 + tx; if (r < rows && c < cols) tile[tx][j] = s[(int64_t)c * rows + r]; }
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8) { int r = r0 + j, c = c0 + tx; if (r < rows && c < cols) d[(int64_t)r * cols + c] += tile[j][tx]; }
+  }
+}
+static bool make_perm(Perm4& P, const int* dims, const int* perm, int rank) {
+  if (rank < 1 || rank > 4) return false;
+  int pad = 4 - rank; int xd[4] = {1, 1, 1, 1}, pm[4] = {0, 1, 2, 3};
+  for (int i = 0; i < rank; i++) { xd[pad + i] = dims[i]; pm[pad + i] = perm[i] + pad; }
+  bool seen[4] = {false, false, false, false};
+  for (int i = 0; i < 4; i++) { if (pm[i] < 0 || pm[i] > 3 || seen[pm[i]]) return false; seen[pm[i]] = true; }
+  int64_t sx[4]; int64_t s = 1; for (int i = 3; i >= 0; i--) { sx[i] = s; s *= xd[i]; }
+  for (int i = 0; i < 4; i++) { P.yd[i] = xd[pm[i]]; P.sx[i] = sx[pm[i]]; }
+  return true;
+}
+}  // namespace
+
+extern "C" {
+
+void lh_trans(const float* x, float* y, int rows, int cols) {
+  if (rows <= 0 || cols <= 0) return;
+  hipLaunchKernelGGL((k_trans_tile<false>), dim3(cdiv(cols, 32), cdiv(rows, 32), 1), dim3(256), 0, g_stream, x, y, rows, cols, (int64_t)0);
+  LH_CHECK_LAUNCH();
+}
+void lh_trans_grad(float* xd, const float* yd, int rows, int cols) {
+  if (rows <= 0 || cols <= 0) return;
+  hipLaunchKernelGGL((k_trans_tile<true>), dim3(cdiv(cols, 32), cdiv(rows, 32), 1), dim3(256), 0, g_stream, yd, xd, rows, cols, (int64_t)0);
+  LH_CHECK_LAUNCH();
+}
+void lh_permute(const float* x, float* y, const int* dims, const int* perm, int rank) {
+  Perm4 P;
+  LH_REQUIRE(make_perm(P, dims, perm, rank), "lh_permute: bad rank/permutation");
+  int64_t n = 1; for (int i = 0; i < rank; i++) n *= dims[i];
+  if (n <= 0) return;
+  hipLaunchKernelGGL((k_permute<false>), dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, P, n);
+  LH_CHECK_LAUNCH();
+}
+void lh_permute_grad(float* xd, const float* yd, const int* dims, const int* perm, int rank) {
+  Perm4 P;
+  LH_REQUIRE(make_perm(P, dims, perm, rank), "lh_permute_grad: bad rank/permutation");
+  int64_t n = 1; for (int i = 0; i < rank; i++) n *= dims[i];
+  if (n <= 0) return;
+  hipLaunchKernelGGL((k_permute<true>), dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, yd, xd, P, n);
+  LH_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- dropout -------------
+__device__ __forceinline__ float ctr_uniform(uint64_t seed, uint64_t index) {
+  uint64_t z = seed + 0x9E3779B97F4A7C15ULL * (index + 1);
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+  z = z ^ (z >> 31);
+  return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+__global__ void __launch_bounds__(TPB) k_dropout(const float* x, float* y, float* mask, int64_t n, float p, float scale, uint64_t seed, uint64_t offset) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    bool keep = ctr_uniform(seed, offset + (uint64_t)i) > p;
+    y[i] = keep ? x[i] * scale : 0.f;
+    mask[i] = keep ? scale : 0.f;
+  }
+}
+void lh_dropout_fwd(const float* x, float* y, float* mask, int64_t n, float p, uint64_t seed, uint64_t offset) {
+  LH_REQUIRE(p >= 0.f && p < 1.f, "dropout rate should be [0.0, 1), got %f", p);
+  if (n <= 0) return;
+  hipLaunchKernelGGL(k_dropout, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, mask, n, p, 1.0f / (1.0f - p), seed, offset);
+  LH_CHECK_LAUNCH();
+}
+void lh_dropout_bwd(const float* dy, const float* mask, float* dx, int64_t n) {
+  ew<3>(dx, dx, mask, dy, n, [] __device__(float d, float m, float g) { return d + m * g; });
+  LH_CHECK_LAUNCH();
+}
+
+// ---------------------------------------------------------------- concat --------------
+// One launch per input tensor: rows of `st = sizes[t]*inner` floats are copied between a
+// packed source and a strided destination (or accumulated the other way for the gradient).
+}  // extern "C"
+template <bool GRAD>
+__global__ void __launch_bounds__(TPB) k_concat(const float* __restrict__ src, float* __restrict__ dst, int64_t st, int64_t row, int64_t off, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, s = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += s) {
+    int64_t h = i / st, l = i - h * st;
+    int64_t o = h * row + off + l;
+    if (GRAD) dst[i] += src[o]; else dst[o] = src[i];
+  }
+}
+extern "C" {
+void lh_concat(int n, const float* const* h_in, const int* sizes, float* out, int outer, int inner) {
+  int64_t row = 0; for (int t = 0; t < n; t++) row += (int64_t)sizes[t] * inner;
+  int64_t off = 0;
+  for (int t = 0; t < n; t++) {
+    int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
+    if (tot > 0) hipLaunchKernelGGL((k_concat<false>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, h_in[t], out, st, row, off, tot);
+    off += st;
+  }
+  LH_CHECK_LAUNCH();
+}
+void lh_concat_grad(int n, float* const* h_ind, const int* sizes, const float* outd, int outer, int inner) {
+  int64_t row = 0; for (int t = 0; t < n; t++) row += (int64_t)sizes[t] * inner;
+  int64_t off = 0;
+  for (int t = 0; t < n; t++) {
+    int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
+    if (tot > 0 && h_ind[t]) hipLaunchKernelGGL((k_concat<true>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
+    off += st;
+  }
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"
+
+// ---------------------------------------------------------------- optimizers ----------
+namespace {
+__device__ __forceinline__ void momentum_elem(float& x, float& d, float& v, float lr, float mu, float clip, int nesterov) {
+  float t = d;
+  if (t > clip) t = clip;
+  if (t < -clip) t = -clip;
+  float vv = v * mu; vv += t;
+  if (nesterov) t += mu * vv; else t = vv;
+  x -= lr * t; v = vv; d = 0.f;
+}
+__global__ void __launch_bounds__(TPB) k_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) {
+  int64_t n4 = n >> 2;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n4; j += st) {
+    float4 X = reinterpret_cast<float4*>(x)[j], D = reinterpret_cast<float4*>(d)[j], V = reinterpret_cast<float4*>(v)[j];
+    momentum_elem(X.x, D.x, V.x, lr, mu, clip, nesterov); momentum_elem(X.y, D.y, V.y, lr, mu, clip, nesterov);
+    momentum_elem(X.z, D.z, V.z, lr, mu, clip, nesterov); momentum_elem(X.w, D.w, V.w, lr, mu, clip, nesterov);
+    reinterpret_cast<float4*>(x)[j] = X; reinterpret_cast<float4*>(d)[j] = D; reinterpret_cast<float4*>(v)[j] = V;
+  }
+  for (int64_t j = 4 * n4 + i; j < n; j += st) momentum_elem(x[j], d[j], v[j], lr, mu, clip, nesterov);
+}
+__global__ void __launch_bounds__(TPB) k_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    float t = d[i];
+    if (t > clip) t = clip;
+    if (t < -clip) t = -clip;
+    float mm = m[i] + t * t;
+    m[i] = mm;
+    x[i] -= lr * t / sqrtf(mm + 1e-8f);
+    d[i] = 0.f;
+  }
+}
+__global__ void __launch_bounds__(TPB) k_sgd(float* x, float* d, float lr, int64_t n) {
+  int64_t n4 = n >> 2;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n4; j += st) {
+    float4 X = reinterpret_cast<float4*>(x)[j], D = reinterpret_cast<float4*>(d)[j];
+    X.x = X.x * 1.0f + D.x * (-lr); X.y = X.y * 1.0f + D.y * (-lr); X.z = X.z * 1.0f + D.z * (-lr); X.w = X.w * 1.0f + D.w * (-lr);
+    reinterpret_cast<float4*>(x)[j] = X; reinterpret_cast<float4*>(d)[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  for (int64_t j = 4 * n4 + i; j < n; j += st) { x[j] = x[j] * 1.0f + d[j] * (-lr); d[j] = 0.f; }
+}
+
+// Multi-tensor form: a table of (x, d, v, first chunk) per tensor lives in device memory;
+// block b finds its tensor by binary search over chunk starts.  Chunk = 4096 elements.
+constexpr int MT_CHUNK = 4096;
+struct MtEntry { float* x; float* d; float* v; int64_t n; int64_t chunk0; };
+__global__ void __launch_bounds__(TPB) k_multi_update(const MtEntry* tab, int count, int mode, float lr, float mu, float clip, int nesterov) {
+  int64_t b = blockIdx.x;
+  int lo = 0, hi = count - 1;
+  while (lo < hi) { int mid = (lo + hi + 1) >> 1; if (tab[mid].chunk0 <= b) lo = mid; else hi = mid - 1; }
+  MtEntry e = tab[lo];
+  int64_t start = (b - e.chunk0) * MT_CHUNK, end = start + MT_CHUNK; if (end > e.n) end = e.n;
+  for (int64_t j = start + threadIdx.x; j < end; j += TPB) {
+    if (mode == 0) { e.x[j] = e.x[j] * 1.0f + e.d[j] * (-lr); e.d[j] = 0.f; }
+    else momentum_elem(e.x[j], e.d[j], e.v[j], lr, mu, clip, nesterov);
+  }
+}
+// The device-side table is cached per distinct host table (same pointers => same step plan).
+struct MtCache { MtEntry* dev = nullptr; int count = 0; int64_t chunks = 0; uint64_t key = 0; int cap = 0; };
+static MtCache g_mt;
+static void multi_update(int mode, int count, float* const* hx, float* const* hd, float* const* hv, const int64_t* hn,
+                         float lr, float mu, float clip, int nesterov) {
+  if (count <= 0) return;
+  uint64_t key = 1469598103934665603ULL;
+  auto mix = [&key](uint64_t v) { key = (key ^ v) * 1099511628211ULL; };
+  for (int t = 0; t < count; t++) { mix((uint64_t)(uintptr_t)hx[t]); mix((uint64_t)(uintptr_t)hd[t]); mix(hv ? (uint64_t)(uintptr_t)hv[t] : 0); mix((uint64_t)hn[t]); }
+  mix((uint64_t)mode);
+  if (g_mt.dev == nullptr || g_mt.key != key || g_mt.count != count) {
+    MtEntry* host = (MtEntry*)malloc(sizeof(MtEntry) * count);
+    int64_t chunks = 0;
+    for (int t = 0; t < count; t++) { host[t] = {hx[t], hd[t], hv ? hv[t] : nullptr, hn[t], chunks}; chunks += cdiv(hn[t] > 0 ? hn[t] : 1, MT_CHUNK); }
+    if (g_mt.cap < count) {
+      if (g_mt.dev) (void)hipFree(g_mt.dev);
+      if (hipMalloc((void**)&g_mt.dev, sizeof(MtEntry) * count) != hipSuccess) { free(host); LH_FAIL("multi-tensor table allocation failed"); return; }
+      g_mt.cap = count;
+    }
+    hipError_t e = hipMemcpyAsync(g_mt.dev, host, sizeof(MtEntry) * count, hipMemcpyHostToDevice, g_stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_stream);
+    free(host);
+    if (e != hipSuccess) { LH_FAIL("multi-tensor table upload: %s", hipGetErrorString(e)); return; }
+    g_mt.key = key; g_mt.count = count; g_mt.chunks = chunks;
+  }
+  hipLaunchKernelGGL(k_multi_update, dim3((unsigned)g_mt.chunks), dim3(TPB), 0, g_stream, (const MtEntry*)g_mt.dev, count, mode, lr, mu, clip, nesterov);
+}
+}  // namespace
+
+extern "C" {
+void lh_sgd(float* x, float* d, float lr, int64_t n) {
+  if (n <= 0) return;
+  LH_REQUIRE(al16(x) && al16(d), "lh_sgd: pointers must be 16-byte aligned");
+  hipLaunchKernelGGL(k_sgd, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, lr, n);
+  LH_CHECK_LAUNCH();
+}
+void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) {
+  if (n <= 0) return;
+  LH_REQUIRE(al16(x) && al16(d) && al16(v), "lh_momentum: pointers must be 16-byte aligned");
+  hipLaunchKernelGGL(k_momentum, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, v, lr, mu, clip, nesterov, n);
+  LH_CHECK_LAUNCH();
+}
+void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) {
+  if (n <= 0) return;
+  hipLaunchKernelGGL(k_adagrad, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, d, m, lr, clip, n);
+  LH_CHECK_LAUNCH();
+}
+void lh_multi_momentum(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
+                       float lr, float mu, float clip, int nesterov) {
+  multi_update(1, count, h_x, h_d, h_v, h_n, lr, mu, clip, nesterov);
+  if (!failed()) LH_CHECK_LAUNCH();
+}
+void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr) {
+  multi_update(0, count, h_x, h_d, nullptr, h_n, lr, 0.f, 0.f, 0);
+  if (!failed()) LH_CHECK_LAUNCH();
+}
+}  // extern "C"

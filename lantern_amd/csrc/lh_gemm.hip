@@ -1,0 +1,129 @@
+// Dense linear algebra outside convolution: sgemm (all four transpose cases), sgemv, rank-1
+// update and vector dot.  Row-major, fp32.
+#include "lh_common.h"
+using namespace lh;
+
+namespace {
+constexpr int TPB = 256;
+
+// 64x64 output tile per block, 16-deep k slabs through LDS, 4x4 register tile per thread.
+template <bool TA, bool TB>
+__global__ void __launch_bounds__(TPB) k_sgemm_tile(int m, int n, int k, float alpha, const float* __restrict__ A, int lda,
+                                                    const float* __restrict__ B, int ldb, float beta, float* __restrict__ C, int ldc) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Bs[16][64 + 4];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int i0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < k; k0 += 16) {
+    for (int e = threadIdx.x; e < 16 * 64; e += TPB) {
+      int kk, ii;
+      if (TA) { ii = e & 63; kk = e >> 6; } else { kk = e & 15; ii = e >> 4; }
+      int gi = i0 + ii, gk = k0 + kk;
+      As[kk][ii] = (gi < m && gk < k) ? (TA ? A[(int64_t)gk * lda + gi] : A[(int64_t)gi * lda + gk]) : 0.f;
+    }
+    for (int e = threadIdx.x; e < 16 * 64; e += TPB) {
+      int kk, jj;
+      if (TB) { kk = e & 15; jj = e >> 4; } else { jj = e & 63; kk = e >> 6; }
+      int gj = j0 + jj, gk = k0 + kk;
+      Bs[kk][jj] = (gj < n && gk < k) ? (TB ? B[(int64_t)gj * ldb + gk] : B[(int64_t)gk * ldb + gj]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; kk++) {
+      float a[4], b[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) { a[u] = As[kk][ty * 4 + u]; b[u] = Bs[kk][tx * 4 + u]; }
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[u][v] += a[u] * b[v];
+    }
+    __syncthreads();
+  }
+  for (int u = 0; u < 4; u++) {
+    int gi = i0 + ty * 4 + u;
+    if (gi >= m) continue;
+    for (int v = 0; v < 4; v++) {
+      int gj = j0 + tx * 4 + v;
+      if (gj >= n) continue;
+      float* c = C + (int64_t)gi * ldc + gj;
+      *c = alpha * acc[u][v] + (beta == 0.f ? 0.f : beta * *c);
+    }
+  }
+}
+
+// y[m] = alpha * A[m,n] x[n] + beta*y : one wave per row.
+__global__ void __launch_bounds__(TPB) k_sgemv_n(int m, int n, float alpha, const float* __restrict__ A, int lda, const float* __restrict__ x, float beta, float* y) {
+  const int lane = threadIdx.x & 63;
+  int64_t w = ((int64_t)blockIdx.x * TPB + threadIdx.x) >> 6, nw = ((int64_t)gridDim.x * TPB) >> 6;
+  for (; w < m; w += nw) {
+    const float* row = A + w * lda;
+    float acc = 0.f;
+    for (int j = lane; j < n; j += 64) acc += row[j] * x[j];
+    acc = lh_wave_sum(acc);
+    if (lane == 0) y[w] = alpha * acc + (beta == 0.f ? 0.f : beta * y[w]);
+  }
+}
+// y[n] = alpha * A[m,n]^T x[m] + beta*y : thread per column, coalesced along n.
+__global__ void __launch_bounds__(TPB) k_sgemv_t(int m, int n, float alpha, const float* __restrict__ A, int lda, const float* __restrict__ x, float beta, float* y) {
+  int j = blockIdx.x * TPB + threadIdx.x;
+  if (j >= n) return;
+  float acc = 0.f;
+  for (int i = 0; i < m; i++) acc += A[(int64_t)i * lda + j] * x[i];
+  y[j] = alpha * acc + (beta == 0.f ? 0.f : beta * y[j]);
+}
+__global__ void __launch_bounds__(TPB) k_ger(int m, int n, const float* __restrict__ u, const float* __restrict__ v, float* A) {
+  int64_t tot = (int64_t)m * n;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < tot; i += st) { int r = (int)(i / n), c = (int)(i - (int64_t)r * n); A[i] = A[i] + v[c] * u[r]; }
+}
+__global__ void __launch_bounds__(TPB) k_dot(const float* x, const float* y, float* out, int n) {
+  __shared__ float sm[17];
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < n; i += TPB) acc += x[i] * y[i];
+  acc = lh_block_sum(acc, sm);
+  if (threadIdx.x == 0) out[0] = acc;
+}
+__global__ void __launch_bounds__(TPB) k_axpy_dev(float* y, const float* s, const float* x, int64_t n) {
+  float a = s[0];
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) y[i] = y[i] + a * x[i];
+}
+}  // namespace
+
+extern "C" {
+
+void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, int lda,
+              const float* B, int ldb, float beta, float* C, int ldc) {
+  if (m <= 0 || n <= 0) return;
+  LH_REQUIRE(k >= 0, "lh_sgemm: negative k");
+  dim3 grid((unsigned)cdiv(n, 64), (unsigned)cdiv(m, 64));
+  if (!ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<false, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+  else if (!ta && tb) hipLaunchKernelGGL((k_sgemm_tile<false, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+  else if (ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<true, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+  else hipLaunchKernelGGL((k_sgemm_tile<true, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+  LH_CHECK_LAUNCH();
+}
+void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, const float* x, float beta, float* y) {
+  if (m <= 0 || n <= 0) return;
+  if (!trans) hipLaunchKernelGGL(k_sgemv_n, dim3(stream_grid((int64_t)m * 64, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
+  else hipLaunchKernelGGL(k_sgemv_t, dim3((unsigned)cdiv(n, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
+  LH_CHECK_LAUNCH();
+}
+void lh_ger(int m, int n, const float* u, const float* v, float* A) {
+  if (m <= 0 || n <= 0) return;
+  hipLaunchKernelGGL(k_ger, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, m, n, u, v, A);
+  LH_CHECK_LAUNCH();
+}
+void lh_dot_vv(const float* x, const float* y, float* out, int n) {
+  hipLaunchKernelGGL(k_dot, dim3(1), dim3(TPB), 0, g_stream, x, y, out, n);
+  LH_CHECK_LAUNCH();
+}
+void lh_axpy_dev(float* y, const float* s, const float* x, int64_t n) {
+  if (n <= 0) return;
+  hipLaunchKernelGGL(k_axpy_dev, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, y, s, x, n);
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"

@@ -1,0 +1,100 @@
+// Max pooling with argmax and average pooling, forward and backward (HBM-bound streaming).
+// Reference semantics: CPU:848-1038 -- scan kernel rows then columns, strict '>' starting
+// from -FLT_MAX so the first maximum wins; argmax is the global flat index into x.
+#include "lh_common.h"
+using namespace lh;
+
+namespace {
+constexpr int TPB = 256;
+
+__global__ void __launch_bounds__(TPB) k_maxpool_fwd(const float* __restrict__ x, float* __restrict__ y, int* __restrict__ idx,
+                                                     int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t n_out) {
+  int64_t o = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; o < n_out; o += st) {
+    int q = (int)(o % oW); int64_t t = o / oW; int p = (int)(t % oH); int64_t nc = t / oH;
+    const int64_t base = nc * H * W;
+    float best = -3.402823466e+38f; int bi = 0;
+    const int h0 = p * sH - pad, w0 = q * sW - pad;
+    for (int r = 0; r < kH; r++) {
+      int h = h0 + r;
+      if (h < 0 || h >= H) continue;
+      for (int s = 0; s < kW; s++) {
+        int w = w0 + s;
+        if (w < 0 || w >= W) continue;
+        float v = x[base + (int64_t)h * W + w];
+        if (v > best) { best = v; bi = (int)(base + (int64_t)h * W + w); }
+      }
+    }
+    y[o] = best; idx[o] = bi;
+  }
+}
+// Scatter-add.  Windows overlap when stride < kernel, so two outputs may hit the same input:
+// atomic add (the sum has at most a few terms, all orders round the same to ~1 ulp).
+__global__ void __launch_bounds__(TPB) k_maxpool_bwd_atomic(const float* __restrict__ dy, const int* __restrict__ idx, float* dx, int64_t n_out) {
+  int64_t o = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; o < n_out; o += st) atomicAdd(dx + idx[o], dy[o]);
+}
+__global__ void __launch_bounds__(TPB) k_avgpool_fwd(const float* __restrict__ x, float* __restrict__ y, int H, int W, int oH, int oW,
+                                                     int kH, int kW, int sH, int sW, int64_t n_out) {
+  const float ks = (float)(kH * kW);
+  int64_t o = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; o < n_out; o += st) {
+    int q = (int)(o % oW); int64_t t = o / oW; int p = (int)(t % oH); int64_t nc = t / oH;
+    const float* xp = x + nc * H * W + (int64_t)(p * sH) * W + q * sW;
+    float sum = 0.f;
+    for (int r = 0; r < kH; r++) for (int s = 0; s < kW; s++) sum += xp[(int64_t)r * W + s];
+    y[o] = sum / ks;
+  }
+}
+// Gather form of the backward: each input element sums the windows that cover it.
+__global__ void __launch_bounds__(TPB) k_avgpool_bwd(const float* __restrict__ dy, float* dx, int H, int W, int oH, int oW,
+                                                     int kH, int kW, int sH, int sW, int64_t n_in) {
+  const int ks = kH * kW;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n_in; i += st) {
+    int w = (int)(i % W); int64_t t = i / W; int h = (int)(t % H); int64_t nc = t / H;
+    // windows p with p*sH <= h < p*sH + kH
+    int p_lo = h - kH + 1 > 0 ? (h - kH + 1 + sH - 1) / sH : 0, p_hi = min(oH - 1, h / sH);
+    int q_lo = w - kW + 1 > 0 ? (w - kW + 1 + sW - 1) / sW : 0, q_hi = min(oW - 1, w / sW);
+    float acc = 0.f; bool any = false;
+    for (int p = p_lo; p <= p_hi; p++) for (int q = q_lo; q <= q_hi; q++) { acc += dy[(nc * oH + p) * oW + q] / ks; any = true; }
+    if (any) dx[i] += acc;
+  }
+}
+}  // namespace
+
+extern "C" {
+
+void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad) {
+  LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pad >= 0, "lh_maxpool_fwd: kernel/stride must be >= 1 and pad >= 0");
+  LH_REQUIRE(H + 2 * pad >= kH && W + 2 * pad >= kW, "Image too small for maxPool_k: %dx%d | (%d,%d)", H, W, kH, kW);
+  LH_REQUIRE((int64_t)N * C * H * W < 2147483647LL, "lh_maxpool_fwd: input too large for int32 argmax");
+  int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
+  int64_t n_out = (int64_t)N * C * oH * oW;
+  if (n_out <= 0) return;
+  hipLaunchKernelGGL(k_maxpool_fwd, dim3(stream_grid(n_out, TPB * 2)), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, n_out);
+  LH_CHECK_LAUNCH();
+}
+void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out) {
+  if (n_out <= 0) return;
+  hipLaunchKernelGGL(k_maxpool_bwd_atomic, dim3(stream_grid(n_out, TPB * 4)), dim3(TPB), 0, g_stream, dy, argmax, dx, n_out);
+  LH_CHECK_LAUNCH();
+}
+void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {
+  LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW, "lh_avgpool_fwd: bad kernel/stride for %dx%d", H, W);
+  int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
+  int64_t n_out = (int64_t)N * C * oH * oW;
+  if (n_out <= 0) return;
+  hipLaunchKernelGGL(k_avgpool_fwd, dim3(stream_grid(n_out, TPB)), dim3(TPB), 0, g_stream, x, y, H, W, oH, oW, kH, kW, sH, sW, n_out);
+  LH_CHECK_LAUNCH();
+}
+void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {
+  LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW, "lh_avgpool_bwd: bad kernel/stride for %dx%d", H, W);
+  int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
+  int64_t n_in = (int64_t)N * C * H * W;
+  if (n_in <= 0) return;
+  hipLaunchKernelGGL(k_avgpool_bwd, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, dy, dx, H, W, oH, oW, kH, kW, sH, sW, n_in);
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+// Lifetime, error path, device arena, transfers and timing events.
+// Reference behaviour being replaced: CUB:18-25, 113-131 (handles + arena + rewind),
+// API:453-473 (myGpuMalloc / myGpuFree), CUB:37-107 (toGPU / toCPU).
+#include "lh_common.h"
+#include <stdarg.h>
+#include <string.h>
+
+namespace lh {
+hipStream_t g_stream = nullptr;
+int g_error_mode = 0;
+int g_num_cu = 256;
+static char g_err[1024] = "";
+static char* g_heap = nullptr;
+static size_t g_heap_bytes = 0, g_top = 0, g_peak = 0;
+
+bool fail(const char* file, int line, const char* fmt, ...) {
+  char msg[768];
+  va_list ap; va_start(ap, fmt); vsnprintf(msg, sizeof msg, fmt, ap); va_end(ap);
+  const char* base = strrchr(file, '/'); base = base ? base + 1 : file;
+  if (g_error_mode == 0) { fprintf(stderr, "lantern_hip error at %s:%d: %s\n", base, line, msg); fflush(stderr); exit(1); }
+  if (g_err[0] == 0) snprintf(g_err, sizeof g_err, "%s:%d: %s", base, line, msg);
+  return true;
+}
+bool failed() { return g_err[0] != 0; }
+
+__global__ void k_zero16(uint4* p, size_t n16) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, st = (size_t)gridDim.x * blockDim.x;
+  for (; i < n16; i += st) p[i] = make_uint4(0, 0, 0, 0);
+}
+static void zero_async(void* p, size_t bytes) {  // bytes is a multiple of 256
+  size_t n16 = bytes / 16;
+  if (n16 == 0) return;
+  int grid = stream_grid((int64_t)n16, 256 * 4);
+  hipLaunchKernelGGL(k_zero16, dim3(grid), dim3(256), 0, g_stream, (uint4*)p, n16);
+}
+}  // namespace lh
+using namespace lh;
+
+extern "C" {
+
+void lh_set_error_mode(int mode) { g_error_mode = mode; }
+const char* lh_last_error(void) { return g_err; }
+void lh_clear_error(void) { g_err[0] = 0; }
+
+void lh_setup(size_t heap_bytes) {
+  LH_REQUIRE(g_heap == nullptr, "lh_setup called twice without lh_cleanup");
+  LH_REQUIRE(heap_bytes >= 4096, "heap of %zu bytes is too small", heap_bytes);
+  int dev = 0;
+  LH_HIP(hipSetDevice(dev));
+  hipDeviceProp_t prop;
+  LH_HIP(hipGetDeviceProperties(&prop, dev));
+  g_num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  LH_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  heap_bytes = (heap_bytes + 255) & ~(size_t)255;
+  LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
+  g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0;
+}
+
+void lh_cleanup(void) {
+  if (g_stream) (void)hipStreamSynchronize(g_stream);
+  if (g_heap) (void)hipFree(g_heap);
+  if (g_stream) (void)hipStreamDestroy(g_stream);
+  g_heap = nullptr; g_stream = nullptr; g_heap_bytes = g_top = 0;
+}
+
+void lh_sync(void) { LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH(); }
+
+static void* bump(size_t bytes, bool zero) {
+  if (!g_heap) { LH_FAIL("lh_malloc before lh_setup"); return nullptr; }
+  size_t need = (bytes + 255) & ~(size_t)255;
+  if (need == 0) need = 256;
+  if (g_top + need > g_heap_bytes) {
+    // API:462-464 aborts on overflow; here it takes the library's error path.
+    LH_FAIL("device arena exhausted: %zu used + %zu requested > %zu", g_top, need, g_heap_bytes);
+    return nullptr;
+  }
+  void* p = g_heap + g_top;
+  g_top += need;
+  if (g_top > g_peak) g_peak = g_top;
+  if (zero) zero_async(p, need);
+  return p;
+}
+void* lh_malloc(size_t bytes) { return bump(bytes, true); }
+void* lh_malloc_uninit(size_t bytes) { return bump(bytes, false); }
+void lh_free_top(size_t bytes) {
+  size_t need = (bytes + 255) & ~(size_t)255;
+  if (need == 0) need = 256;
+  LH_REQUIRE(need <= g_top, "lh_free_top(%zu) below the arena base", bytes);
+  g_top -= need;
+}
+size_t lh_mark(void) { return g_top; }
+void lh_rewind(size_t mark) {
+  LH_REQUIRE(mark <= g_top && (mark & 255) == 0, "lh_rewind(%zu): not a mark at or below the top (%zu)", mark, g_top);
+  g_top = mark;
+}
+size_t lh_heap_used(void) { return g_top; }
+size_t lh_heap_peak(void) { return g_peak; }
+
+void lh_h2d(void* dst, const void* h_src, size_t bytes) {
+  // Pageable source: the copy is staged before the call returns, so the host buffer may be reused.
+  LH_HIP(hipMemcpyAsync(dst, h_src, bytes, hipMemcpyHostToDevice, g_stream));
+  LH_HIP(hipStreamSynchronize(g_stream));
+}
+void lh_d2h(void* h_dst, const void* src, size_t bytes) {
+  LH_HIP(hipMemcpyAsync(h_dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+  LH_HIP(hipStreamSynchronize(g_stream));
+}
+void lh_d2d(void* dst, const void* src, size_t bytes) {
+  LH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+}
+
+void* lh_event_create(void) {
+  hipEvent_t ev = nullptr;
+  if (hipEventCreate(&ev) != hipSuccess) { LH_FAIL("hipEventCreate failed"); return nullptr; }
+  return (void*)ev;
+}
+void lh_event_record(void* ev) { LH_HIP(hipEventRecord((hipEvent_t)ev, g_stream)); }
+float lh_event_elapsed_ms(void* start, void* stop) {
+  float ms = -1.0f;
+  if (hipEventSynchronize((hipEvent_t)stop) != hipSuccess || hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)stop) != hipSuccess) {
+    LH_FAIL("event timing failed"); return -1.0f;
+  }
+  return ms;
+}
+void lh_event_destroy(void* ev) { (void)hipEventDestroy((hipEvent_t)ev); }
+
+}  // extern "C"
