@@ -1,6 +1,6 @@
 // Dense linear algebra outside convolution: sgemm (all four transpose cases), sgemv, rank-1
 // update and vector dot.  Row-major, fp32.
-#include "lh_common.h"
+#include "lh_igemm.h"
 using namespace lh;
 
 namespace {
@@ -94,10 +94,35 @@ __global__ void __launch_bounds__(TPB) k_axpy_dev(float* y, const float* s, cons
 
 extern "C" {
 
+}  // extern "C"
+// MFMA path for all but tiny products; the 64x64 register-tiled kernel covers those.
+template <class AL, class BL>
+static bool sgemm_mfma(const AL& al, const BL& bl, const EpiRowMajor& ep, int m, int n, int k) {
+  TilePick tp = pick_tile(m, n);
+  if (tp.bm == 128) return igemm_launch<128, 128, 16>(al, bl, ep, m, n, k, 1);
+  if (tp.bn == 128) return igemm_launch<64, 128, 16>(al, bl, ep, m, n, k, 1);
+  return igemm_launch<64, 64, 16>(al, bl, ep, m, n, k, 1);
+}
+
 void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, int lda,
               const float* B, int ldb, float beta, float* C, int ldc) {
   if (m <= 0 || n <= 0) return;
   LH_REQUIRE(k >= 0, "lh_sgemm: negative k");
+  if ((int64_t)m * n * k >= (1 << 18) && m >= 16 && n >= 16) {
+    EpiRowMajor ep; ep.C = C; ep.ldc = ldc; ep.alpha = alpha; ep.beta = beta; ep.atomic = 0;
+    LoadPlainK ak; ak.base = A; ak.ld = lda; ak.vec = (lda % 4 == 0) && (((uintptr_t)A & 15) == 0);
+    LoadPlainT at; at.base = A; at.ld = lda;
+    LoadPlainK bk; bk.base = B; bk.ld = ldb; bk.vec = (ldb % 4 == 0) && (((uintptr_t)B & 15) == 0);
+    LoadPlainT bt; bt.base = B; bt.ld = ldb;
+    bool ok;
+    if (!ta && !tb) ok = sgemm_mfma(ak, bt, ep, m, n, k);
+    else if (!ta && tb) ok = sgemm_mfma(ak, bk, ep, m, n, k);
+    else if (ta && !tb) ok = sgemm_mfma(at, bt, ep, m, n, k);
+    else ok = sgemm_mfma(at, bk, ep, m, n, k);
+    if (!ok) return;
+    LH_CHECK_LAUNCH();
+    return;
+  }
   dim3 grid((unsigned)cdiv(n, 64), (unsigned)cdiv(m, 64));
   if (!ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<false, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
   else if (!ta && tb) hipLaunchKernelGGL((k_sgemm_tile<false, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
@@ -105,6 +130,7 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   else hipLaunchKernelGGL((k_sgemm_tile<true, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
   LH_CHECK_LAUNCH();
 }
+extern "C" {
 void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, const float* x, float beta, float* y) {
   if (m <= 0 || n <= 0) return;
   if (!trans) hipLaunchKernelGGL(k_sgemv_n, dim3(stream_grid((int64_t)m * 64, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);

@@ -1,0 +1,127 @@
+"""conv2D_batch forward / input gradient / filter gradient: HIP (through the C ABI) against
+the CPU oracle on the same seeded inputs.  Tolerance 1e-4 relative (see util.assert_close)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle.backend_cpu import load as load_oracle
+from tests.util import Dev, assert_close, cptr
+
+pytestmark = pytest.mark.gpu
+
+# (N, C, H, W, K, R, S, sH, sW, pH, pW)
+SHAPES = [
+    (2, 3, 9, 9, 8, 3, 3, 1, 1, 1, 1),        # tiny, channels not a multiple of anything
+    (3, 1, 28, 28, 10, 5, 5, 1, 1, 0, 0),     # LeNet conv1
+    (3, 10, 12, 12, 20, 5, 5, 1, 1, 0, 0),    # LeNet conv2
+    (2, 64, 14, 14, 64, 1, 1, 1, 1, 0, 0),    # 1x1 stride 1 (plain GEMM)
+    (2, 64, 14, 14, 128, 1, 1, 2, 2, 0, 0),   # 1x1 stride 2 (ResNet downsample)
+    (2, 32, 14, 14, 48, 3, 3, 1, 1, 1, 1),    # 3x3 pad 1
+    (2, 32, 15, 13, 40, 3, 3, 2, 2, 1, 1),    # 3x3 stride 2, odd non-square input
+    (2, 3, 32, 32, 16, 7, 7, 2, 2, 3, 3),     # 7x7 stride 2 pad 3 (ResNet stem)
+    (4, 16, 7, 7, 24, 3, 3, 1, 1, 1, 1),      # 7x7 maps: P*Q = 49 not a multiple of 4
+    (2, 130, 8, 8, 136, 3, 3, 1, 1, 1, 1),    # M and K just past one 128 tile
+    (1, 1, 41, 30, 8, 11, 5, 2, 2, 0, 0),     # tall DeepSpeech-like kernel, stride (2,2)
+    (1, 4, 21, 30, 6, 5, 3, 2, 1, 2, 1),      # anisotropic stride and pad
+    (2, 96, 16, 16, 16, 1, 1, 1, 1, 0, 0),    # SqueezeNet squeeze (K = 16)
+    (2, 512, 4, 4, 10, 4, 4, 1, 1, 0, 0),     # SqueezeNet head: 4x4 kernel onto 1x1
+    (5, 256, 7, 7, 64, 1, 1, 1, 1, 0, 0),     # long reduction, 49-pixel maps
+]
+
+
+def _oracle_conv(x, w, b, dy, dims, need_dx=True):
+    lc = load_oracle()
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    y = np.zeros((N, K, P, Q), np.float32)
+    fin = np.zeros((N, Cc * R * S, P * Q), np.float32)
+    ints = [C.c_int(v) for v in dims]
+    lc.lc_conv2d_fwd(cptr(x), cptr(w), cptr(b) if b is not None else None, cptr(y), cptr(fin), *ints)
+    dx = np.zeros_like(x); dw = np.zeros_like(w); db = np.zeros(K, np.float32)
+    scratch = np.zeros_like(fin)
+    lc.lc_conv2d_bwd(cptr(fin), cptr(w), cptr(dy), cptr(dx) if need_dx else None, cptr(dw), cptr(db), cptr(scratch), *ints)
+    return y, dx, dw, db
+
+
+@pytest.mark.parametrize("dims", SHAPES, ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("bias", [False, True], ids=["nobias", "bias"])
+def test_conv_fwd_bwd(on_hip, dims, bias):
+    dev = Dev(on_hip)
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    rng = np.random.RandomState(hash(dims) % (2 ** 31))
+    x = rng.randn(N, Cc, H, W).astype(np.float32)
+    w = (rng.randn(K, Cc, R, S) / np.sqrt(Cc * R * S)).astype(np.float32)
+    b = rng.randn(K).astype(np.float32) if bias else None
+    dy = rng.randn(N, K, P, Q).astype(np.float32)
+    y_ref, dx_ref, dw_ref, db_ref = _oracle_conv(x, w, b, dy, dims)
+
+    ints = list(dims)
+    dx_, dw_ = dev.up(x), dev.up(w)
+    db_ = dev.up(b) if bias else None
+    y_ = dev.zeros(y_ref.size)
+    dev.lib.lh_conv2d_fwd(dx_.ptr, dw_.ptr, db_.ptr if bias else 0, y_.ptr, *ints); dev.check()
+    assert_close(dev.down(y_, y_ref.shape), y_ref, what="conv fwd")
+
+    ddy = dev.up(dy)
+    # input gradient: overwrite (beta 0) into garbage, then accumulate (beta 1) on top
+    gdx = dev.up(np.full(x.shape, 7.0, np.float32))
+    dev.lib.lh_conv2d_bwd_data(ddy.ptr, dw_.ptr, gdx.ptr, 0.0, *ints); dev.check()
+    assert_close(dev.down(gdx, x.shape), dx_ref, what="conv bwd_data beta=0")
+    dev.lib.lh_conv2d_bwd_data(ddy.ptr, dw_.ptr, gdx.ptr, 1.0, *ints); dev.check()
+    assert_close(dev.down(gdx, x.shape), 2 * dx_ref, what="conv bwd_data beta=1")
+
+    gdw = dev.up(np.full(w.shape, -3.0, np.float32))
+    gdb = dev.up(np.ones(K, np.float32))
+    dev.lib.lh_conv2d_bwd_filter(dx_.ptr, ddy.ptr, gdw.ptr, gdb.ptr if bias else 0, 0.0, *ints); dev.check()
+    assert_close(dev.down(gdw, w.shape), dw_ref, what="conv bwd_filter beta=0")
+    dev.lib.lh_conv2d_bwd_filter(dx_.ptr, ddy.ptr, gdw.ptr, gdb.ptr if bias else 0, 1.0, *ints); dev.check()
+    assert_close(dev.down(gdw, w.shape), 2 * dw_ref, what="conv bwd_filter beta=1")
+    if bias:
+        assert_close(dev.down(gdb, (K,)), 1 + 2 * db_ref, what="conv bias grad")
+
+
+def test_conv_linearity_at_resnet_shape(on_hip):
+    """Size-independent property at a full ResNet-50 layer shape (too slow for the oracle in a unit
+    test): conv(a*x1 + x2, w) == a*conv(x1, w) + conv(x2, w), and the sum of the output equals
+    the closed form for an all-ones filter on a constant input interior."""
+    dev = Dev(on_hip)
+    dims = (8, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1)
+    N, Cc, H, W, K, R, S = dims[:7]
+    rng = np.random.RandomState(5)
+    x1 = rng.randn(N, Cc, H, W).astype(np.float32); x2 = rng.randn(N, Cc, H, W).astype(np.float32)
+    w = (rng.randn(K, Cc, R, S) / 24).astype(np.float32)
+    dw_ = dev.up(w)
+    outs = []
+    for xin in (x1, x2, (2.5 * x1 + x2).astype(np.float32)):
+        y_ = dev.zeros(N * K * H * W)
+        dev.lib.lh_conv2d_fwd(dev.up(xin).ptr, dw_.ptr, 0, y_.ptr, *dims); dev.check()
+        outs.append(dev.down(y_, (N, K, H, W)))
+    assert_close(outs[2], 2.5 * outs[0] + outs[1], rtol=1e-4, what="linearity")
+    ones_w = dev.up(np.ones((K, Cc, R, S), np.float32))
+    y_ = dev.zeros(N * K * H * W)
+    dev.lib.lh_conv2d_fwd(dev.up(np.ones((N, Cc, H, W), np.float32)).ptr, ones_w.ptr, 0, y_.ptr, *dims); dev.check()
+    y = dev.down(y_, (N, K, H, W))
+    assert (y[:, :, 1:-1, 1:-1] == Cc * 9).all() and (y[:, :, 0, 0] == Cc * 4).all() and (y[:, :, 0, 1:-1] == Cc * 6).all()
+
+
+GEMMS = [(0, 0, 64, 1000, 2048), (0, 1, 64, 1000, 2048), (1, 0, 70, 130, 257), (1, 1, 33, 65, 129),
+         (0, 0, 100, 50, 320), (0, 1, 5, 7, 3), (0, 0, 2, 3, 4), (1, 0, 300, 300, 64)]
+
+
+@pytest.mark.parametrize("ta,tb,m,n,k", GEMMS)
+def test_sgemm(on_hip, ta, tb, m, n, k):
+    dev = Dev(on_hip)
+    lc = load_oracle()
+    rng = np.random.RandomState(m * 131 + n * 7 + k)
+    A = rng.randn(*((k, m) if ta else (m, k))).astype(np.float32)
+    B = rng.randn(*((n, k) if tb else (k, n))).astype(np.float32)
+    Cm = rng.randn(m, n).astype(np.float32)
+    for alpha, beta in ((1.0, 0.0), (0.5, 1.0)):
+        ref = Cm.copy()
+        lc.lc_sgemm(C.c_int(ta), C.c_int(tb), C.c_int(m), C.c_int(n), C.c_int(k), C.c_float(alpha), cptr(A), C.c_int(A.shape[1]),
+                    cptr(B), C.c_int(B.shape[1]), C.c_float(beta), cptr(ref), C.c_int(n))
+        c_ = dev.up(Cm)
+        dev.lib.lh_sgemm(ta, tb, m, n, k, alpha, dev.up(A).ptr, A.shape[1], dev.up(B).ptr, B.shape[1], beta, c_.ptr, n); dev.check()
+        assert_close(dev.down(c_, (m, n)), ref, what="sgemm %d%d a=%g b=%g" % (ta, tb, alpha, beta))
