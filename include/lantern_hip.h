@@ -70,6 +70,14 @@ void  lh_event_record(void* ev);
 float lh_event_elapsed_ms(void* start, void* stop);        /* waits for stop */
 void  lh_event_destroy(void* ev);
 
+/* ---- per-category kernel timing (no counterpart in the reference; a measurement aid for the
+ *      benchmark).  Bit c of `mask` turns on HIP-event timing of category c; lh_prof_collect waits,
+ *      sums elapsed milliseconds and call counts per category since the last collect. */
+enum { LH_CAT_CONV_FWD = 0, LH_CAT_CONV_BWD_DATA, LH_CAT_CONV_BWD_FILTER, LH_CAT_GEMM, LH_CAT_BN_FWD, LH_CAT_BN_BWD,
+       LH_CAT_ELEMENTWISE, LH_CAT_POOL, LH_CAT_REDUCE, LH_CAT_OPTIM, LH_CAT_FILL, LH_CAT_COUNT };
+void lh_prof_enable(unsigned mask);
+void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat);
+
 /* ---- fill / elementwise ------------------------------------------------ */
 void lh_fill(float* x, float v, int64_t n);                                    /* fill, fillInPlace: CUB:133-151 */
 void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, int64_t inner); /* fillWithBias: CPU:39-62 */

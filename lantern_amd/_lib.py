@@ -33,6 +33,8 @@ SIGNATURES = {
     "lh_event_record": (None, [P]),
     "lh_event_elapsed_ms": (F, [P, P]),
     "lh_event_destroy": (None, [P]),
+    "lh_prof_enable": (None, [C.c_uint]),
+    "lh_prof_collect": (None, [P, P, I]),
     "lh_fill": (None, [P, F, L]),
     "lh_fill_with_bias": (None, [P, P, L, L, L]),
     "lh_clip": (None, [P, F, L]),

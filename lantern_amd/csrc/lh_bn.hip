@@ -174,6 +174,7 @@ extern "C" {
 
 void lh_bn_infer(const float* x, const float* gamma, const float* beta, const float* run_mean, const float* run_var,
                  float* y, int N, int C, int HW, float eps) {
+  ProfScope prof_(CAT_BN_FWD);
   int64_t n = (int64_t)N * C * HW;
   if (n <= 0) return;
   hipLaunchKernelGGL(k_bn_infer, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, gamma, beta, run_mean, run_var, C, HW, n, eps);
@@ -182,6 +183,7 @@ void lh_bn_infer(const float* x, const float* gamma, const float* beta, const fl
 
 void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
                      float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
+  ProfScope prof_(CAT_BN_FWD);
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_train_fwd: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_train_fwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   if (!get_partial()) return;
@@ -201,6 +203,7 @@ void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, floa
 
 void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
+  ProfScope prof_(CAT_BN_BWD);
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_bwd: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_bwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   LH_REQUIRE(beta_dx == 0.0f || beta_dx == 1.0f, "lh_bn_bwd: beta must be 0 or 1");

@@ -30,6 +30,20 @@ bool failed();
     if (e_ != hipSuccess) { LH_FAIL("kernel launch: %s", hipGetErrorString(e_)); return; } \
   } while (0)
 
+// ---- per-category timing with HIP events on g_stream (off unless lh_prof_enable was called) ----
+enum {
+  CAT_CONV_FWD = 0, CAT_CONV_BWD_DATA, CAT_CONV_BWD_FILTER, CAT_GEMM, CAT_BN_FWD, CAT_BN_BWD,
+  CAT_ELEMENTWISE, CAT_POOL, CAT_REDUCE, CAT_OPTIM, CAT_FILL, CAT_COUNT
+};
+extern unsigned g_prof_mask;
+void prof_begin(int cat);
+void prof_end(int cat);
+struct ProfScope {
+  int cat; bool on;
+  explicit ProfScope(int c) : cat(c), on((g_prof_mask >> c) & 1u) { if (on) prof_begin(cat); }
+  ~ProfScope() { if (on) prof_end(cat); }
+};
+
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Grid for a grid-stride streaming kernel: enough blocks to cover n at `per_block`

@@ -66,7 +66,7 @@ struct Dims4 { int d[4]; int64_t sa[4]; int64_t sb[4]; };
 
 extern "C" {
 
-void lh_fill(float* x, float v, int64_t n) {
+void lh_fill(float* x, float v, int64_t n) { ProfScope prof_(CAT_FILL);
   if (n <= 0) return;
   if (al16(x)) hipLaunchKernelGGL(k_fill, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, v, n);
   else hipLaunchKernelGGL(k_fill_scalar, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, v, n);
@@ -100,7 +100,7 @@ void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t) {
   LH_CHECK_LAUNCH();
 }
 
-void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) {
+void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) { ProfScope prof_(CAT_ELEMENTWISE);
   switch (op) {
     case LH_RELU: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return v < 0.f ? 0.f : v; }); break;
     case LH_TANH: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return tanhf(v); }); break;
@@ -115,7 +115,7 @@ void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) {
   LH_CHECK_LAUNCH();
 }
 
-void lh_unary_grad(int op, const float* x, const float* y, const float* dy, float* dx, int64_t n, int inplace, float lo, float hi) {
+void lh_unary_grad(int op, const float* x, const float* y, const float* dy, float* dx, int64_t n, int inplace, float lo, float hi) { ProfScope prof_(CAT_ELEMENTWISE);
   // out = dx; inputs (a, b, c) chosen per op.  All forms are dx (+)= g(x|y, dy).
   switch (op) {
     case LH_RELU:
@@ -137,13 +137,13 @@ void lh_unary_grad(int op, const float* x, const float* y, const float* dy, floa
   LH_CHECK_LAUNCH();
 }
 
-void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) {
+void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_scalar_op: unknown op %d", op);
   ew<1>(y, x, nullptr, nullptr, n, [op, s] __device__(float v, float, float) { return bop(op, v, s); });
   LH_CHECK_LAUNCH();
 }
 
-void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) {
+void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
   ew<2>(out, x, y, nullptr, n, [alpha, beta] __device__(float a, float b, float) { return a * alpha + b * beta; });
   LH_CHECK_LAUNCH();
 }
@@ -267,7 +267,7 @@ void launch_reduce(int op, int which, float* small, const int* sdims4, const flo
 
 extern "C" {
 
-void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const int* bdims, float* out, const int* odims, int rank) {
+void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const int* bdims, float* out, const int* odims, int rank) { ProfScope prof_(CAT_ELEMENTWISE);
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_op: unknown op %d", op);
   int64_t n = prod(odims, rank);
   if (n <= 0) return;
@@ -283,7 +283,7 @@ void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const
 
 void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a_is_input,
                       const float* b, float* bd, const int* bdims, int b_is_input,
-                      const float* outd, const int* odims, int rank) {
+                      const float* outd, const int* odims, int rank) { ProfScope prof_(CAT_ELEMENTWISE);
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_op_grad: unknown op %d", op);
   int64_t n = prod(odims, rank);
   if (n <= 0) return;
@@ -317,7 +317,7 @@ void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a
   LH_CHECK_LAUNCH();
 }
 
-void lh_bcast_update(int op, float* a, const int* adims, const float* b, const int* bdims, int rank) {
+void lh_bcast_update(int op, float* a, const int* adims, const float* b, const int* bdims, int rank) { ProfScope prof_(CAT_ELEMENTWISE);
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_update: unknown op %d", op);
   LH_REQUIRE(rank >= 1 && rank <= 4, "lh_bcast_update: rank %d not in 1..4", rank);
   int od[4];
@@ -577,29 +577,29 @@ static void multi_update(int mode, int count, float* const* hx, float* const* hd
 }  // namespace
 
 extern "C" {
-void lh_sgd(float* x, float* d, float lr, int64_t n) {
+void lh_sgd(float* x, float* d, float lr, int64_t n) { ProfScope prof_(CAT_OPTIM);
   if (n <= 0) return;
   LH_REQUIRE(al16(x) && al16(d), "lh_sgd: pointers must be 16-byte aligned");
   hipLaunchKernelGGL(k_sgd, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, lr, n);
   LH_CHECK_LAUNCH();
 }
-void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) {
+void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) { ProfScope prof_(CAT_OPTIM);
   if (n <= 0) return;
   LH_REQUIRE(al16(x) && al16(d) && al16(v), "lh_momentum: pointers must be 16-byte aligned");
   hipLaunchKernelGGL(k_momentum, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, v, lr, mu, clip, nesterov, n);
   LH_CHECK_LAUNCH();
 }
-void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) {
+void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) { ProfScope prof_(CAT_OPTIM);
   if (n <= 0) return;
   hipLaunchKernelGGL(k_adagrad, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, d, m, lr, clip, n);
   LH_CHECK_LAUNCH();
 }
 void lh_multi_momentum(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
-                       float lr, float mu, float clip, int nesterov) {
+                       float lr, float mu, float clip, int nesterov) { ProfScope prof_(CAT_OPTIM);
   multi_update(1, count, h_x, h_d, h_v, h_n, lr, mu, clip, nesterov);
   if (!failed()) LH_CHECK_LAUNCH();
 }
-void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr) {
+void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr) { ProfScope prof_(CAT_OPTIM);
   multi_update(0, count, h_x, h_d, nullptr, h_n, lr, 0.f, 0.f, 0);
   if (!failed()) LH_CHECK_LAUNCH();
 }

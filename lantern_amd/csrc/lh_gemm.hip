@@ -106,6 +106,7 @@ static bool sgemm_mfma(const AL& al, const BL& bl, const EpiRowMajor& ep, int m,
 
 void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, int lda,
               const float* B, int ldb, float beta, float* C, int ldc) {
+  ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
   LH_REQUIRE(k >= 0, "lh_sgemm: negative k");
   if ((int64_t)m * n * k >= (1 << 18) && m >= 16 && n >= 16) {
@@ -132,12 +133,14 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
 }
 extern "C" {
 void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, const float* x, float beta, float* y) {
+  ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
   if (!trans) hipLaunchKernelGGL(k_sgemv_n, dim3(stream_grid((int64_t)m * 64, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
   else hipLaunchKernelGGL(k_sgemv_t, dim3((unsigned)cdiv(n, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
   LH_CHECK_LAUNCH();
 }
 void lh_ger(int m, int n, const float* u, const float* v, float* A) {
+  ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
   hipLaunchKernelGGL(k_ger, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, m, n, u, v, A);
   LH_CHECK_LAUNCH();

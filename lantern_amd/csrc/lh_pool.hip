@@ -66,6 +66,7 @@ __global__ void __launch_bounds__(TPB) k_avgpool_bwd(const float* __restrict__ d
 extern "C" {
 
 void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad) {
+  ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pad >= 0, "lh_maxpool_fwd: kernel/stride must be >= 1 and pad >= 0");
   LH_REQUIRE(H + 2 * pad >= kH && W + 2 * pad >= kW, "Image too small for maxPool_k: %dx%d | (%d,%d)", H, W, kH, kW);
   LH_REQUIRE((int64_t)N * C * H * W < 2147483647LL, "lh_maxpool_fwd: input too large for int32 argmax");
@@ -76,11 +77,13 @@ void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, 
   LH_CHECK_LAUNCH();
 }
 void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out) {
+  ProfScope prof_(CAT_POOL);
   if (n_out <= 0) return;
   hipLaunchKernelGGL(k_maxpool_bwd_atomic, dim3(stream_grid(n_out, TPB * 4)), dim3(TPB), 0, g_stream, dy, argmax, dx, n_out);
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {
+  ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW, "lh_avgpool_fwd: bad kernel/stride for %dx%d", H, W);
   int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
   int64_t n_out = (int64_t)N * C * oH * oW;
@@ -89,6 +92,7 @@ void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {
+  ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW, "lh_avgpool_bwd: bad kernel/stride for %dx%d", H, W);
   int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
   int64_t n_in = (int64_t)N * C * H * W;

@@ -157,31 +157,31 @@ __global__ void k_nll_grad(float* dx, const int* target, const float* dy, int ba
 
 extern "C" {
 
-void lh_sum_all(const float* x, float* out, int64_t n) { sum_impl(x, out, n, 1.0f); if (!failed()) LH_CHECK_LAUNCH(); }
-void lh_mean_all(const float* x, float* out, int64_t n) {
+void lh_sum_all(const float* x, float* out, int64_t n) { ProfScope prof_(CAT_REDUCE); sum_impl(x, out, n, 1.0f); if (!failed()) LH_CHECK_LAUNCH(); }
+void lh_mean_all(const float* x, float* out, int64_t n) { ProfScope prof_(CAT_REDUCE);
   LH_REQUIRE(n > 0, "lh_mean_all of an empty tensor");
   sum_impl(x, out, n, 1.0f / (float)n);
   if (!failed()) LH_CHECK_LAUNCH();
 }
-void lh_add_scalar_from(float* dx, const float* dy1, float scale, int64_t n) {
+void lh_add_scalar_from(float* dx, const float* dy1, float scale, int64_t n) { ProfScope prof_(CAT_REDUCE);
   if (n <= 0) return;
   hipLaunchKernelGGL(k_add_scalar_from, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, dx, dy1, scale, n);
   LH_CHECK_LAUNCH();
 }
-void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner) {
+void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner) { ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * inner <= 0) return;
   if (inner == 1) hipLaunchKernelGGL(k_sum_rows, dim3(stream_grid((int64_t)outer * 64, TPB)), dim3(TPB), 0, g_stream, x, y, outer, dim);
   else hipLaunchKernelGGL(k_sum_dim_inner, dim3(stream_grid((int64_t)outer * inner, TPB)), dim3(TPB), 0, g_stream, x, y, outer, dim, inner);
   LH_CHECK_LAUNCH();
 }
-void lh_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner) {
+void lh_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner) { ProfScope prof_(CAT_REDUCE);
   int64_t n = (int64_t)outer * dim * inner;
   if (n <= 0) return;
   hipLaunchKernelGGL(k_sum_dim_grad, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, dx, dy, n, dim, inner);
   LH_CHECK_LAUNCH();
 }
 
-void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner) {
+void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner) { ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * c * inner <= 0) return;
   if (inner == 1) {
     if (c <= 1024 || outer >= 4 * g_num_cu) {
@@ -199,7 +199,7 @@ void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inne
   }
   LH_CHECK_LAUNCH();
 }
-void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int outer, int c, int inner) {
+void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int outer, int c, int inner) { ProfScope prof_(CAT_REDUCE);
   int64_t groups = (int64_t)outer * inner;
   if (groups * c <= 0) return;
   int grid = stream_grid(groups * 64, TPB);
@@ -207,12 +207,12 @@ void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int
   else hipLaunchKernelGGL((k_softmax_grad_wave<false>), dim3(grid), dim3(TPB), 0, g_stream, y, dy, dx, groups, c, inner);
   LH_CHECK_LAUNCH();
 }
-void lh_nll(const float* x, const int* target, float* y, int batch, int stride) {
+void lh_nll(const float* x, const int* target, float* y, int batch, int stride) { ProfScope prof_(CAT_REDUCE);
   if (batch <= 0) return;
   hipLaunchKernelGGL(k_nll, dim3(cdiv(batch, 64)), dim3(64), 0, g_stream, x, target, y, batch, stride);
   LH_CHECK_LAUNCH();
 }
-void lh_nll_grad(float* dx, const int* target, const float* dy, int batch, int stride) {
+void lh_nll_grad(float* dx, const int* target, const float* dy, int batch, int stride) { ProfScope prof_(CAT_REDUCE);
   if (batch <= 0) return;
   hipLaunchKernelGGL(k_nll_grad, dim3(cdiv(batch, 64)), dim3(64), 0, g_stream, dx, target, dy, batch, stride);
   LH_CHECK_LAUNCH();

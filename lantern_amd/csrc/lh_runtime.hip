@@ -4,6 +4,7 @@
 #include "lh_common.h"
 #include <stdarg.h>
 #include <string.h>
+#include <vector>
 
 namespace lh {
 hipStream_t g_stream = nullptr;
@@ -22,6 +23,32 @@ bool fail(const char* file, int line, const char* fmt, ...) {
   return true;
 }
 bool failed() { return g_err[0] != 0; }
+
+// ---- event profiler ---------------------------------------------------------------------
+unsigned g_prof_mask = 0;
+struct ProfRec { hipEvent_t a, b; int cat; };
+static std::vector<ProfRec> g_prof_recs;
+static std::vector<hipEvent_t> g_prof_pool;
+static hipEvent_t prof_event() {
+  if (!g_prof_pool.empty()) { hipEvent_t e = g_prof_pool.back(); g_prof_pool.pop_back(); return e; }
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) return nullptr;
+  return e;
+}
+void prof_begin(int cat) {
+  ProfRec r; r.a = prof_event(); r.b = nullptr; r.cat = cat;
+  if (r.a) (void)hipEventRecord(r.a, g_stream);
+  g_prof_recs.push_back(r);
+}
+void prof_end(int cat) {
+  for (size_t i = g_prof_recs.size(); i-- > 0;) {
+    if (g_prof_recs[i].cat == cat && g_prof_recs[i].b == nullptr) {
+      g_prof_recs[i].b = prof_event();
+      if (g_prof_recs[i].b) (void)hipEventRecord(g_prof_recs[i].b, g_stream);
+      return;
+    }
+  }
+}
 
 __global__ void k_zero16(uint4* p, size_t n16) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, st = (size_t)gridDim.x * blockDim.x;
@@ -77,7 +104,7 @@ static void* bump(size_t bytes, bool zero) {
   void* p = g_heap + g_top;
   g_top += need;
   if (g_top > g_peak) g_peak = g_top;
-  if (zero) zero_async(p, need);
+  if (zero) { ProfScope prof_(CAT_FILL); zero_async(p, need); }
   return p;
 }
 void* lh_malloc(size_t bytes) { return bump(bytes, true); }
@@ -107,6 +134,19 @@ void lh_d2h(void* h_dst, const void* src, size_t bytes) {
 }
 void lh_d2d(void* dst, const void* src, size_t bytes) {
   LH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+}
+
+void lh_prof_enable(unsigned mask) { g_prof_mask = mask; }
+void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat) {
+  for (int c = 0; c < ncat; c++) { h_ms[c] = 0.0; h_calls[c] = 0; }
+  if (g_stream) (void)hipStreamSynchronize(g_stream);
+  for (auto& r : g_prof_recs) {
+    float ms = 0.f;
+    if (r.a && r.b && hipEventElapsedTime(&ms, r.a, r.b) == hipSuccess && r.cat < ncat) { h_ms[r.cat] += ms; h_calls[r.cat] += 1; }
+    if (r.a) g_prof_pool.push_back(r.a);
+    if (r.b) g_prof_pool.push_back(r.b);
+  }
+  g_prof_recs.clear();
 }
 
 void* lh_event_create(void) {

@@ -1,0 +1,165 @@
+"""Model building blocks and optimizers (reference: src/main/scala/lantern/NNModule.scala).
+
+`Module` keeps an ordered registry of parameters (the reference finds them by JVM reflection,
+NN:20-110); layers follow NN:112-182 (initialisation scales included); optimizers follow
+NN:255-303.  Parameters are TensorR objects living below the arena mark of the training loop.
+"""
+import math
+
+import numpy as np
+
+from .tensor import Tensor, TensorR, get_backend
+
+
+class Module:
+    def __init__(self, name="module"):
+        self.name = name
+        self._params = []        # (name, TensorR)
+        self._children = []
+
+    def param(self, name, t):
+        tr = t if isinstance(t, TensorR) else TensorR(t)
+        self._params.append((name, tr))
+        return tr
+
+    def add(self, m):
+        self._children.append(m)
+        return m
+
+    def namedParameters(self, prefix=""):
+        out = [("%s%s/%s" % (prefix, self.name, n), p) for n, p in self._params]
+        for c in self._children:
+            out += c.namedParameters("%s%s/" % (prefix, self.name))
+        return out
+
+    def parameters(self):
+        return [p for _, p in self.namedParameters()]
+
+    def forEachParameter(self, f):
+        for p in self.parameters():
+            f(p)
+
+
+def _uniform_from(rng, dims, scale):
+    """(U[0,1) - 0.5) * scale: the distribution of Tensor.rand(dims, scale) (CPU:101-110)."""
+    if rng is None:
+        return Tensor.rand(tuple(dims), scale)
+    return Tensor.fromNumpy(((rng.random_sample(tuple(dims)).astype(np.float32) - np.float32(0.5)) * np.float32(scale)))
+
+
+class Linear1D(Module):
+    """y = x . W + b with W of shape [in, out] (NN:112-117)."""
+
+    def __init__(self, inSize, outSize, bias=True, name="linear1d", rng=None):
+        super().__init__(name)
+        scale = 1.0 / math.sqrt(inSize)
+        self.weight = self.param("weight", _uniform_from(rng, (inSize, outSize), scale))
+        self.biasOp = self.param("bias", Tensor.zeros(outSize)) if bias else None
+
+    def __call__(self, x):
+        y = x.dot(self.weight)
+        return y.plusBias(self.biasOp) if self.biasOp is not None else y
+
+
+class Conv2D(Module):
+    """Kaiming-uniform conv (NN:133-146): scale = 2*sqrt(6/fan_in)."""
+
+    def __init__(self, inChannel, outChannel, kernelSize, stride=(1, 1), pad=(0, 0), useBias=True, name="conv2d", rng=None, init=None):
+        super().__init__(name)
+        kh, kw = kernelSize
+        dims = (outChannel, inChannel, kh, kw)
+        if init is not None:
+            k = Tensor.fromNumpy(init(dims))
+        else:
+            k = _uniform_from(rng, dims, 2.0 * math.sqrt(6.0 / (inChannel * kh * kw)))
+        self.kernel = self.param("kernel", k)
+        self.bias = self.param("bias", Tensor.zeros(outChannel)) if useBias else None
+        self.stride, self.pad = tuple(stride), tuple(pad)
+
+    def __call__(self, x):
+        return x.convBBP(self.kernel, self.bias, self.stride, self.pad)
+
+
+class BatchNorm2D(Module):
+    """NN:168-182: scale ones, bias zeros, running mean/var zeros (not parameters)."""
+
+    def __init__(self, num_features, name="batch_norm_2d"):
+        super().__init__(name)
+        self.scale = self.param("scale", Tensor.ones(num_features))
+        self.bias = self.param("bias", Tensor.zeros(num_features))
+        self.runningMean = Tensor.zeros(num_features)
+        self.runningVar = Tensor.zeros(num_features)
+
+    def __call__(self, x):
+        return x.batchNorm(self.scale, self.bias, self.runningMean, self.runningVar)
+
+
+class BatchNorm1D(BatchNorm2D):
+    """NN:158-166: per-activation statistics over the rows of a rank-2 input."""
+
+    def __call__(self, x):
+        assert x.x.rank == 2
+        return x.batchNorm1D(self.scale, self.bias, self.runningMean, self.runningVar)
+
+
+# ---- optimizers (NN:255-303) -------------------------------------------------------------------
+class Optim:
+    def __init__(self, module):
+        self.module = module
+        self.params = module.parameters()
+
+    def zero_grad(self):
+        for p in self.params:
+            p.clear_grad()
+
+
+class SGD(Optim):
+    """x = 1*x + (-lr)*d via geam, then clear_grad (NN:265-287; gradClip is ignored there too).
+    `fused=True` issues the same update for all tensors in one multi-tensor launch."""
+
+    def __init__(self, module, learning_rate, gradClip=1.0, descent=True, fused=True):
+        super().__init__(module)
+        self.lr = learning_rate if descent else -learning_rate
+        self.fused = fused
+
+    def step(self):
+        be = get_backend()
+        if self.fused:
+            be.multi_sgd_update([(p.x.data, p.d.data, p.x.scalarCount) for p in self.params], self.lr)
+        else:
+            for p in self.params:
+                be.sgd_update(p.x.data, p.d.data, self.lr, p.x.scalarCount)
+
+
+class SGD_Momentum(Optim):
+    """NN:296-303 + CPU:1232-1246: clip, v = mu*v + g, (nesterov), x -= lr*g, d = 0."""
+
+    def __init__(self, module, learning_rate, momentum=0.9, gradClip=400.0, nesterov=False, descent=True, fused=True):
+        super().__init__(module)
+        assert descent
+        self.lr, self.mu, self.clip, self.nesterov, self.fused = learning_rate, momentum, gradClip, nesterov, fused
+        self.moment = [Tensor.zeros_like(p.x) for p in self.params]      # enrichParameter (NN:74-84)
+
+    def step(self):
+        be = get_backend()
+        if self.fused:
+            be.multi_momentum_update([(p.x.data, p.d.data, m.data, p.x.scalarCount) for p, m in zip(self.params, self.moment)],
+                                     self.lr, self.mu, self.clip, self.nesterov)
+        else:
+            for p, m in zip(self.params, self.moment):
+                be.momentum_update(p.x.data, p.d.data, m.data, self.lr, self.mu, self.clip, self.nesterov, p.x.scalarCount)
+
+
+class Adagrad(Optim):
+    """NN:289-294 + CPU:1217-1230."""
+
+    def __init__(self, module, learning_rate, gradClip=1.0, descent=True):
+        super().__init__(module)
+        assert descent
+        self.lr, self.clip = learning_rate, gradClip
+        self.moment = [Tensor.zeros_like(p.x) for p in self.params]
+
+    def step(self):
+        be = get_backend()
+        for p, m in zip(self.params, self.moment):
+            be.adagrad_update(p.x.data, p.d.data, m.data, self.lr, self.clip, p.x.scalarCount)
