@@ -19,7 +19,7 @@ static bool make_dims(ConvDims& d, int N, int C, int H, int W, int K, int R, int
   if (N < 1 || C < 1 || H < 1 || W < 1 || K < 1 || R < 1 || S < 1 || sH < 1 || sW < 1 || pH < 0 || pW < 0) return false;
   if (H + 2 * pH < R || W + 2 * pW < S) return false;
   d = {N, C, H, W, K, R, S, sH, sW, pH, pW, (H + 2 * pH - R) / sH + 1, (W + 2 * pW - S) / sW + 1};
-  const int64_t lim = 0x7fffffffLL;
+  const int64_t lim = 0x20000000LL;   // 2 GiB of fp32 per tensor: byte offsets of the buffer loads stay below 2^31
   if ((int64_t)N * C * H * W >= lim || (int64_t)N * K * d.P * d.Q >= lim || (int64_t)K * C * R * S >= lim) return false;
   return true;
 }
@@ -28,25 +28,24 @@ static bool make_dims(ConvDims& d, int N, int C, int H, int W, int K, int R, int
 // column j = (n, p, q) fixed per thread; k = (c, r, s) is uniform across a wavefront.
 struct LoadConvFwdB {
   static constexpr bool ALONG_K = false;
-  const float* x; int C, H, W, sH, sW, pH, pW, HW;
+  static constexpr bool VEC4 = false;
+  const float* base; uint32_t nbytes;
+  int C, H, W, sH, sW, pH, pW, HW;
   FastDiv dPQ, dQ, dRS, dS;
-  struct State { int base, h0, w0; bool valid; };
+  struct State { int pix, h0, w0; bool valid; };     // pix = n*C*H*W + h0*W + w0 (may be negative)
   __device__ __forceinline__ void init(State& s, int j, int ncols) const {
     s.valid = j < ncols;
     uint32_t n, pq, p, q;
     dPQ.divmod(s.valid ? j : 0, n, pq); dQ.divmod(pq, p, q);
-    s.base = (int)n * C * HW; s.h0 = (int)p * sH - pH; s.w0 = (int)q * sW - pW;
+    s.h0 = (int)p * sH - pH; s.w0 = (int)q * sW - pW;
+    s.pix = (int)n * C * HW + s.h0 * W + s.w0;
   }
-  __device__ __forceinline__ float one(const State& s, int k, int kend) const {
-    if (!s.valid || k >= kend) return 0.f;
+  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
     uint32_t c, rs, r, ss;
-    dRS.divmod(k, c, rs); dS.divmod(rs, r, ss);
-    int h = s.h0 + (int)r, w = s.w0 + (int)ss;
-    if ((unsigned)h >= (unsigned)H || (unsigned)w >= (unsigned)W) return 0.f;
-    return x[s.base + ((int)c * H + h) * W + w];
-  }
-  __device__ __forceinline__ float4 load4(const State& s, int k, int kend) const {
-    return make_float4(one(s, k, kend), one(s, k + 1, kend), one(s, k + 2, kend), one(s, k + 3, kend));
+    dRS.divmod(k + e, c, rs); dS.divmod(rs, r, ss);
+    const int tap = ((int)c * H + (int)r) * W + (int)ss;       // wave-uniform
+    const bool ok = s.valid && k + e < kend && (unsigned)(s.h0 + (int)r) < (unsigned)H && (unsigned)(s.w0 + (int)ss) < (unsigned)W;
+    return ok ? (uint32_t)(s.pix + tap) * 4u : LH_OOB;
   }
 };
 
@@ -54,61 +53,55 @@ struct LoadConvFwdB {
 // column j = (n, h, w) of dx fixed per thread; k = (ko, r, s) uniform across a wavefront.
 struct LoadConvBwdDataB {
   static constexpr bool ALONG_K = false;
-  const float* dy; int K, P, Q, PQ;
+  static constexpr bool VEC4 = false;
+  const float* base; uint32_t nbytes;
+  int K, P, Q, PQ;
   FastDiv dHW, dW, dRS, dS, dsH, dsW;
   int pH, pW;
-  struct State { int base, hh, ww; bool valid; };
+  struct State { int nbase, hh, ww; bool valid; };
   __device__ __forceinline__ void init(State& s, int j, int ncols) const {
     s.valid = j < ncols;
     uint32_t n, hw, h, w;
     dHW.divmod(s.valid ? j : 0, n, hw); dW.divmod(hw, h, w);
-    s.base = (int)n * K * PQ; s.hh = (int)h + pH; s.ww = (int)w + pW;
+    s.nbase = (int)n * K * PQ; s.hh = (int)h + pH; s.ww = (int)w + pW;
   }
-  __device__ __forceinline__ float one(const State& s, int k, int kend) const {
-    if (!s.valid || k >= kend) return 0.f;
+  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
     uint32_t ko, rs, r, ss;
-    dRS.divmod(k, ko, rs); dS.divmod(rs, r, ss);
-    int th = s.hh - (int)r, tw = s.ww - (int)ss;
-    if (th < 0 || tw < 0) return 0.f;
+    dRS.divmod(k + e, ko, rs); dS.divmod(rs, r, ss);
+    const int th = s.hh - (int)r, tw = s.ww - (int)ss;
     uint32_t p, ph, q, qw;
-    dsH.divmod(th, p, ph); dsW.divmod(tw, q, qw);
-    if (ph != 0 || qw != 0 || (int)p >= P || (int)q >= Q) return 0.f;
-    return dy[s.base + ((int)ko * P + (int)p) * Q + (int)q];
-  }
-  __device__ __forceinline__ float4 load4(const State& s, int k, int kend) const {
-    return make_float4(one(s, k, kend), one(s, k + 1, kend), one(s, k + 2, kend), one(s, k + 3, kend));
+    dsH.divmod(th < 0 ? 0 : th, p, ph); dsW.divmod(tw < 0 ? 0 : tw, q, qw);
+    const bool ok = s.valid && k + e < kend && th >= 0 && tw >= 0 && ph == 0 && qw == 0 && (int)p < P && (int)q < Q;
+    return ok ? (uint32_t)(s.nbase + ((int)ko * P + (int)p) * Q + (int)q) * 4u : LH_OOB;
   }
 };
 
 // ---- A operand of the filter gradient: dy rows, reduction index (n, p, q) ------------------------------
+template <bool VEC>                      // VEC: PQ % 4 == 0 and dy 16-byte aligned
 struct LoadConvBwdFilterA {
   static constexpr bool ALONG_K = true;
-  const float* dy; int K, PQ, vec;      // vec: PQ % 4 == 0 and dy 16-byte aligned
+  static constexpr bool VEC4 = VEC;
+  const float* base; uint32_t nbytes;
+  int K, PQ;
   FastDiv dPQ;
   struct State { int rowoff; bool valid; };
   __device__ __forceinline__ void init(State& s, int i, int nrows) const { s.valid = i < nrows; s.rowoff = (s.valid ? i : 0) * PQ; }
-  __device__ __forceinline__ float one(const State& s, int kk, int kend) const {
-    if (kk >= kend) return 0.f;
-    uint32_t n, pq; dPQ.divmod(kk, n, pq);
-    return dy[(int64_t)n * K * PQ + s.rowoff + pq];
-  }
-  __device__ __forceinline__ float4 load4(const State& s, int kk, int kend) const {
-    if (!s.valid) return make_float4(0.f, 0.f, 0.f, 0.f);
-    if (vec && kk + 3 < kend) {
-      uint32_t n, pq; dPQ.divmod(kk, n, pq);
-      return *reinterpret_cast<const float4*>(dy + (int64_t)n * K * PQ + s.rowoff + pq);
-    }
-    return make_float4(one(s, kk, kend), one(s, kk + 1, kend), one(s, kk + 2, kend), one(s, kk + 3, kend));
+  __device__ __forceinline__ uint32_t off1(const State& s, int kk, int kend, int e) const {
+    // VEC: the reduction length N*PQ is a multiple of 4 too, so the group at e == 0 is all in or all out
+    uint32_t n, pq; dPQ.divmod(kk + e, n, pq);
+    return (s.valid && kk + e < kend) ? (uint32_t)((int)n * K * PQ + s.rowoff + (int)pq) * 4u : LH_OOB;
   }
 };
 
 // ---- B operand of the filter gradient: gather of x, reduction index (n, p, q) ------------------------------
 // column j = (c, r, s) fixed per thread.
+template <bool ROWVEC>                   // ROWVEC: Q % 4 == 0, the four reduction indices share (n, p)
 struct LoadConvBwdFilterB {
   static constexpr bool ALONG_K = true;
-  const float* x; int C, H, W, sH, sW, pH, pW, CHW;
+  static constexpr bool VEC4 = false;
+  const float* base; uint32_t nbytes;
+  int C, H, W, sH, sW, pH, pW, CHW;
   FastDiv dPQ, dQ, dRS, dS;
-  int rowvec;   // Q % 4 == 0: four consecutive reduction indices share (n, p)
   struct State { int coff, dh, dw; bool valid; };
   __device__ __forceinline__ void init(State& s, int j, int ncols) const {
     s.valid = j < ncols;
@@ -116,30 +109,13 @@ struct LoadConvBwdFilterB {
     dRS.divmod(s.valid ? j : 0, c, rs); dS.divmod(rs, r, ss);
     s.coff = (int)c * H * W; s.dh = (int)r - pH; s.dw = (int)ss - pW;
   }
-  __device__ __forceinline__ float one(const State& s, int kk, int kend) const {
-    if (kk >= kend) return 0.f;
+  __device__ __forceinline__ uint32_t off1(const State& s, int kk, int kend, int e) const {
+    // ROWVEC: the group's four indices share (n, p); decode its first and step along the row
     uint32_t n, pq, p, q;
-    dPQ.divmod(kk, n, pq); dQ.divmod(pq, p, q);
-    int h = (int)p * sH + s.dh, w = (int)q * sW + s.dw;
-    if ((unsigned)h >= (unsigned)H || (unsigned)w >= (unsigned)W) return 0.f;
-    return x[(int64_t)n * CHW + s.coff + h * W + w];
-  }
-  __device__ __forceinline__ float4 load4(const State& s, int kk, int kend) const {
-    if (!s.valid) return make_float4(0.f, 0.f, 0.f, 0.f);
-    if (rowvec && kk + 3 < kend) {
-      uint32_t n, pq, p, q;
-      dPQ.divmod(kk, n, pq); dQ.divmod(pq, p, q);
-      int h = (int)p * sH + s.dh, w = (int)q * sW + s.dw;
-      if ((unsigned)h >= (unsigned)H) return make_float4(0.f, 0.f, 0.f, 0.f);
-      const float* row = x + (int64_t)n * CHW + s.coff + h * W;
-      float4 r;
-      r.x = (unsigned)w < (unsigned)W ? row[w] : 0.f;
-      r.y = (unsigned)(w + sW) < (unsigned)W ? row[w + sW] : 0.f;
-      r.z = (unsigned)(w + 2 * sW) < (unsigned)W ? row[w + 2 * sW] : 0.f;
-      r.w = (unsigned)(w + 3 * sW) < (unsigned)W ? row[w + 3 * sW] : 0.f;
-      return r;
-    }
-    return make_float4(one(s, kk, kend), one(s, kk + 1, kend), one(s, kk + 2, kend), one(s, kk + 3, kend));
+    dPQ.divmod(ROWVEC ? kk : kk + e, n, pq); dQ.divmod(pq, p, q);
+    const int h = (int)p * sH + s.dh, w = ((int)q + (ROWVEC ? e : 0)) * sW + s.dw;
+    const bool ok = s.valid && kk + e < kend && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
+    return ok ? (uint32_t)((int)n * CHW + s.coff + h * W + w) * 4u : LH_OOB;
   }
 };
 
@@ -198,11 +174,15 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_fwd: bad shape N%d C%d H%d W%d K%d R%d S%d s(%d,%d) p(%d,%d)", N, C, H, W, K, R, S, sH, sW, pH, pW);
   const int CRS = C * R * S, PQ = d.P * d.Q;
-  LoadPlainK al; al.base = w; al.ld = CRS; al.vec = (CRS % 4 == 0) && (((uintptr_t)w & 15) == 0);
-  LoadConvFwdB bl; bl.x = x; bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
+  const bool avec = (CRS % 4 == 0) && (((uintptr_t)w & 15) == 0);
+  const uint32_t wbytes = (uint32_t)((size_t)K * CRS * 4);
+  LoadConvFwdB bl; bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * H * W * 4); bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
   bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
   EpiConvOut ep; ep.out = y; ep.bias = bias; ep.chan = K; ep.PIX = PQ; ep.beta = 0.f; ep.dPIX.init(PQ);
-  if (!launch_tiles(al, bl, ep, K, N * PQ, CRS)) return;
+  bool ok;
+  if (avec) { LoadPlainK<true> al; al.base = w; al.nbytes = wbytes; al.ld = CRS; ok = launch_tiles(al, bl, ep, K, N * PQ, CRS); }
+  else { LoadPlainK<false> al; al.base = w; al.nbytes = wbytes; al.ld = CRS; ok = launch_tiles(al, bl, ep, K, N * PQ, CRS); }
+  if (!ok) return;
   LH_CHECK_LAUNCH();
 }
 
@@ -213,12 +193,12 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_data: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_data: beta must be 0 or 1");
   const int RS = R * S, KRS = K * RS, HW = H * W, PQ = d.P * d.Q;
-  LoadConvBwdDataB bl; bl.dy = dy; bl.K = K; bl.P = d.P; bl.Q = d.Q; bl.PQ = PQ; bl.pH = pH; bl.pW = pW;
+  LoadConvBwdDataB bl; bl.base = dy; bl.nbytes = (uint32_t)((size_t)N * K * PQ * 4); bl.K = K; bl.P = d.P; bl.Q = d.Q; bl.PQ = PQ; bl.pH = pH; bl.pW = pW;
   bl.dHW.init(HW); bl.dW.init(W); bl.dRS.init(RS); bl.dS.init(S); bl.dsH.init(sH); bl.dsW.init(sW);
   EpiConvOut ep; ep.out = dx; ep.bias = nullptr; ep.chan = C; ep.PIX = HW; ep.beta = beta; ep.dPIX.init(HW);
   bool ok;
   if (RS == 1) {
-    LoadPlainT al; al.base = w; al.ld = C;          // A[c][k] = w[k][c]
+    LoadPlainT al; al.base = w; al.nbytes = (uint32_t)((size_t)K * C * 4); al.ld = C;          // A[c][k] = w[k][c]
     ok = launch_tiles(al, bl, ep, C, N * HW, KRS);
   } else {
     // transposed filter in scratch taken from the arena top and released again: later
@@ -228,8 +208,8 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
     if (wt == nullptr) return;
     int64_t n = (int64_t)KRS * C;
     hipLaunchKernelGGL(k_filter_transpose, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, RS, n);
-    LoadPlainK al; al.base = wt; al.ld = KRS; al.vec = (KRS % 4 == 0);
-    ok = launch_tiles(al, bl, ep, C, N * HW, KRS);
+    if (KRS % 4 == 0) { LoadPlainK<true> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
+    else { LoadPlainK<false> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
     lh_free_top(bytes);
   }
   if (!ok) return;
@@ -245,9 +225,8 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   const int CRS = C * R * S, PQ = d.P * d.Q;
   const int64_t red = (int64_t)N * PQ;
   LH_REQUIRE(red < 0x7fffffffLL, "lh_conv2d_bwd_filter: reduction length too large");
-  LoadConvBwdFilterA al; al.dy = dy; al.K = K; al.PQ = PQ; al.vec = (PQ % 4 == 0) && (((uintptr_t)dy & 15) == 0); al.dPQ.init(PQ);
-  LoadConvBwdFilterB bl; bl.x = x; bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.CHW = C * H * W;
-  bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S); bl.rowvec = (d.Q % 4 == 0);
+  const bool avec = (PQ % 4 == 0) && (((uintptr_t)dy & 15) == 0);
+  const bool rowvec = (d.Q % 4 == 0);
   // The output is small (K x CRS) and the reduction long (N*P*Q): split it across blocks and
   // combine with fp32 atomic adds.
   TilePick tp = (K >= 128 && CRS >= 128) ? TilePick{128, 128} : (CRS >= 128 ? TilePick{64, 128} : TilePick{64, 64});
@@ -258,10 +237,19 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   if (split < 1) split = 1;
   if (beta == 0.f) lh_fill(dw, 0.f, (int64_t)K * CRS);
   EpiRowMajor ep; ep.C = dw; ep.ldc = CRS; ep.alpha = 1.f; ep.beta = 1.f; ep.atomic = split > 1 ? 1 : 0;
-  bool ok;
-  if (tp.bm == 128) ok = igemm_launch<128, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
-  else if (tp.bn == 128) ok = igemm_launch<64, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
-  else ok = igemm_launch<64, 64, 32>(al, bl, ep, K, CRS, (int)red, split);
+  bool ok = false;
+  auto go = [&](auto al, auto bl) {
+    al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
+    bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * H * W * 4); bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.CHW = C * H * W;
+    bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
+    if (tp.bm == 128) ok = igemm_launch<128, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
+    else if (tp.bn == 128) ok = igemm_launch<64, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
+    else ok = igemm_launch<64, 64, 32>(al, bl, ep, K, CRS, (int)red, split);
+  };
+  if (avec && rowvec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<true>());
+  else if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<false>());
+  else if (rowvec) go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<true>());
+  else go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<false>());
   if (!ok) return;
   if (db) hipLaunchKernelGGL(k_conv_bwd_bias, dim3(K), dim3(TPB), 0, g_stream, dy, db, N, K, PQ);
   LH_CHECK_LAUNCH();

@@ -111,15 +111,22 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   LH_REQUIRE(k >= 0, "lh_sgemm: negative k");
   if ((int64_t)m * n * k >= (1 << 18) && m >= 16 && n >= 16) {
     EpiRowMajor ep; ep.C = C; ep.ldc = ldc; ep.alpha = alpha; ep.beta = beta; ep.atomic = 0;
-    LoadPlainK ak; ak.base = A; ak.ld = lda; ak.vec = (lda % 4 == 0) && (((uintptr_t)A & 15) == 0);
-    LoadPlainT at; at.base = A; at.ld = lda;
-    LoadPlainK bk; bk.base = B; bk.ld = ldb; bk.vec = (ldb % 4 == 0) && (((uintptr_t)B & 15) == 0);
-    LoadPlainT bt; bt.base = B; bt.ld = ldb;
+    const bool av = (lda % 4 == 0) && (((uintptr_t)A & 15) == 0) && (k % 4 == 0);
+    const bool bv = (ldb % 4 == 0) && (((uintptr_t)B & 15) == 0) && (k % 4 == 0);
+    const size_t abytes = (size_t)(ta ? k : m) * lda * 4, bbytes = (size_t)(tb ? n : k) * ldb * 4;
+    LH_REQUIRE(abytes <= 0x80000000ull && bbytes <= 0x80000000ull, "lh_sgemm: operands above 2 GiB are not supported");
+    LoadPlainK<true> akv; akv.base = A; akv.nbytes = (uint32_t)abytes; akv.ld = lda;
+    LoadPlainK<false> aks; aks.base = A; aks.nbytes = (uint32_t)abytes; aks.ld = lda;
+    LoadPlainT at; at.base = A; at.nbytes = (uint32_t)abytes; at.ld = lda;
+    LoadPlainK<true> bkv; bkv.base = B; bkv.nbytes = (uint32_t)bbytes; bkv.ld = ldb;
+    LoadPlainK<false> bks; bks.base = B; bks.nbytes = (uint32_t)bbytes; bks.ld = ldb;
+    LoadPlainT bt; bt.base = B; bt.nbytes = (uint32_t)bbytes; bt.ld = ldb;
     bool ok;
-    if (!ta && !tb) ok = sgemm_mfma(ak, bt, ep, m, n, k);
-    else if (!ta && tb) ok = sgemm_mfma(ak, bk, ep, m, n, k);
+    if (!ta && !tb) ok = av ? sgemm_mfma(akv, bt, ep, m, n, k) : sgemm_mfma(aks, bt, ep, m, n, k);
+    else if (!ta && tb) ok = av ? (bv ? sgemm_mfma(akv, bkv, ep, m, n, k) : sgemm_mfma(akv, bks, ep, m, n, k))
+                                : (bv ? sgemm_mfma(aks, bkv, ep, m, n, k) : sgemm_mfma(aks, bks, ep, m, n, k));
     else if (ta && !tb) ok = sgemm_mfma(at, bt, ep, m, n, k);
-    else ok = sgemm_mfma(at, bk, ep, m, n, k);
+    else ok = bv ? sgemm_mfma(at, bkv, ep, m, n, k) : sgemm_mfma(at, bks, ep, m, n, k);
     if (!ok) return;
     LH_CHECK_LAUNCH();
     return;

@@ -42,40 +42,58 @@ struct GemmShape {
   int total, perXcd;
 };
 
-// ---- plain matrix loaders -------------------------------------------------------------------
-// Element (col, k) at base[col*ld + k]  (k contiguous).
+// ---- operand loaders ---------------------------------------------------------------------------
+// A loader turns (column, k) into BYTE OFFSETS into its tensor; the kernel fetches them with
+// raw buffer loads.  An element outside the matrix (k >= kend, column past the edge, a padding
+// tap of the convolution) gets the offset LH_OOB, which lies beyond the buffer's num_records, so
+// the hardware returns 0 without touching memory: no branches and no selects in the k-loop.
+// Tensors fed through a loader must be at most 2 GiB (checked on the host).
+constexpr uint32_t LH_OOB = 0x80000000u;
+constexpr int LH_RSRC_FLAGS = 0x00020000;    // raw buffer, 32-bit data format
+
+
+// Element (col, k) at base[col*ld + k]  (k contiguous).  VEC: rows are 16-byte aligned and
+// ld % 4 == 0 and K % 4 == 0, so a group of four k is one aligned 16-byte load, all in or all out.
+template <bool VEC>
 struct LoadPlainK {
   static constexpr bool ALONG_K = true;
-  const float* base; int ld; int vec;   // vec: rows are 16-byte aligned and ld % 4 == 0
-  struct State { const float* row; bool valid; };
-  __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.row = base + (int64_t)(s.valid ? col : 0) * ld; }
-  __device__ __forceinline__ float4 load4(const State& s, int k, int kend) const {
-    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (!s.valid) return r;
-    if (vec && k + 3 < kend) return *reinterpret_cast<const float4*>(s.row + k);
-    if (k < kend) r.x = s.row[k];
-    if (k + 1 < kend) r.y = s.row[k + 1];
-    if (k + 2 < kend) r.z = s.row[k + 2];
-    if (k + 3 < kend) r.w = s.row[k + 3];
-    return r;
+  static constexpr bool VEC4 = VEC;
+  const float* base; uint32_t nbytes; int ld;
+  struct State { uint32_t row; bool valid; };
+  __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.row = (uint32_t)(s.valid ? col : 0) * (uint32_t)ld * 4u; }
+  // byte offset of element k + e of the group starting at k (VEC: e == 0 stands for all four)
+  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
+    return (s.valid && k + e < kend) ? s.row + (uint32_t)(k + e) * 4u : LH_OOB;
   }
 };
 // Element (col, k) at base[k*ld + col]  (col contiguous).
 struct LoadPlainT {
   static constexpr bool ALONG_K = false;
-  const float* base; int ld;
-  struct State { const float* colp; bool valid; };
-  __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.colp = base + (s.valid ? col : 0); }
-  __device__ __forceinline__ float4 load4(const State& s, int k, int kend) const {
-    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (!s.valid) return r;
-    if (k < kend) r.x = s.colp[(int64_t)k * ld];
-    if (k + 1 < kend) r.y = s.colp[(int64_t)(k + 1) * ld];
-    if (k + 2 < kend) r.z = s.colp[(int64_t)(k + 2) * ld];
-    if (k + 3 < kend) r.w = s.colp[(int64_t)(k + 3) * ld];
-    return r;
+  static constexpr bool VEC4 = false;
+  const float* base; uint32_t nbytes; int ld;
+  struct State { uint32_t col; bool valid; };
+  __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.col = (uint32_t)(s.valid ? col : 0) * 4u; }
+  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
+    return (s.valid && k + e < kend) ? s.col + (uint32_t)(k + e) * (uint32_t)ld * 4u : LH_OOB;
   }
 };
+
+// Offsets of one group of four k (one offset when the loader is VEC4).
+template <class L> struct LhOff { uint32_t o[4]; };
+template <class L>
+__device__ __forceinline__ float4 lh_fetch4(__amdgpu_buffer_rsrc_t rsrc, const LhOff<L>& f) {
+  if (L::VEC4) {
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)f.o[0], 0, 0);
+    return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+  }
+  float4 r;
+  r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], 0, 0));
+  r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[1], 0, 0));
+  r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[2], 0, 0));
+  r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[3], 0, 0));
+  return r;
+}
 
 // ---- epilogue for row-major C ------------------------------------------------------------------
 // mode 0: C = alpha*acc + beta*C ; mode 1: atomicAdd(C, alpha*acc) (split-K)
@@ -110,6 +128,8 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
   const int m0 = tm * BM, n0 = tn * BN;
   const int kbeg = sp * gs.kPerSplit, kend = min(gs.K, kbeg + gs.kPerSplit);
 
+  const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc((void*)al.base, 0, (int)al.nbytes, LH_RSRC_FLAGS);
+  const __amdgpu_buffer_rsrc_t rsB = __builtin_amdgcn_make_buffer_rsrc((void*)bl.base, 0, (int)bl.nbytes, LH_RSRC_FLAGS);
   const int t = threadIdx.x;
   typename AL::State sa[GA];
   typename BL::State sb[GB];
@@ -137,30 +157,46 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
 
   const int lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
   const int niter = (kend - kbeg + BK - 1) / BK;
+  constexpr int EA = AL::VEC4 ? 1 : 4, EB = BL::VEC4 ? 1 : 4;
+  constexpr int NEL = GA * EA + GB * EB;            // offsets to compute per slab and thread
+  constexpr int NM_PAIR = 4 * MI * NI, NM = (KQ / 2) * NM_PAIR;
   float4 ra[GA], rb[GB];
+  LhOff<AL> oa[GA];
+  LhOff<BL> ob[GB];
+  // e-th offset of the slab starting at k0
+  auto elem = [&](int e, int k0) {
+    if (e < GA * EA) { const int g = e / EA, i = e % EA; oa[g].o[i] = al.off1(sa[g], k0 + 4 * a_kq[g], kend, i); }
+    else { const int f = e - GA * EA, g = f / EB, i = f % EB; ob[g].o[i] = bl.off1(sb[g], k0 + 4 * b_kq[g], kend, i); }
+  };
 
-  if (niter > 0) {
+  // Software pipeline over k-slabs (three slabs in flight):
+  //   the loads of slab t+1 are issued at the top of the iteration from offsets computed one
+  //   iteration earlier and land in LDS after the MFMAs of slab t;
+  //   the offsets of slab t+2 (VALU/SALU only) are computed in small pieces placed between the
+  //   MFMAs of slab t, so they issue while the matrix pipe is busy.
+  // Slabs past kend produce LH_OOB offsets (loads return 0) and LDS stages that are never read.
 #pragma unroll
-    for (int g = 0; g < GA; g++) ra[g] = al.load4(sa[g], kbeg + 4 * a_kq[g], kend);
+  for (int e = 0; e < NEL; e++) elem(e, kbeg);
 #pragma unroll
-    for (int g = 0; g < GB; g++) rb[g] = bl.load4(sb[g], kbeg + 4 * b_kq[g], kend);
+  for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(rsA, oa[g]);
 #pragma unroll
-    for (int g = 0; g < GA; g++) As[a_kq[g] * LDA + a_col[g]] = ra[g];
+  for (int g = 0; g < GB; g++) rb[g] = lh_fetch4<BL>(rsB, ob[g]);
 #pragma unroll
-    for (int g = 0; g < GB; g++) Bs[b_kq[g] * LDB + b_col[g]] = rb[g];
-  }
+  for (int e = 0; e < NEL; e++) elem(e, kbeg + BK);
+#pragma unroll
+  for (int g = 0; g < GA; g++) As[a_kq[g] * LDA + a_col[g]] = ra[g];
+#pragma unroll
+  for (int g = 0; g < GB; g++) Bs[b_kq[g] * LDB + b_col[g]] = rb[g];
   __syncthreads();
 
   for (int it = 0; it < niter; it++) {
     const int st = it & 1;
-    const bool more = it + 1 < niter;
-    if (more) {
-      const int k0 = kbeg + (it + 1) * BK;
+    const int k2 = kbeg + (it + 2) * BK;
 #pragma unroll
-      for (int g = 0; g < GA; g++) ra[g] = al.load4(sa[g], k0 + 4 * a_kq[g], kend);
+    for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(rsA, oa[g]);
 #pragma unroll
-      for (int g = 0; g < GB; g++) rb[g] = bl.load4(sb[g], k0 + 4 * b_kq[g], kend);
-    }
+    for (int g = 0; g < GB; g++) rb[g] = lh_fetch4<BL>(rsB, ob[g]);
+    __builtin_amdgcn_sched_barrier(0);
     const float4* Asc = As + st * KQ * LDA + wm * TM + l32;
     const float4* Bsc = Bs + st * KQ * LDB + wn * TN + l32;
 #pragma unroll
@@ -171,17 +207,25 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
       for (int mi = 0; mi < MI; mi++) a[mi] = Asc[kq * LDA + mi * 32];
 #pragma unroll
       for (int ni = 0; ni < NI; ni++) b[ni] = Bsc[kq * LDB + ni * 32];
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int mi = 0; mi < MI; mi++)
+      for (int m = 0; m < NM_PAIR; m++) {
+        const int c = m / (MI * NI), mi = (m / NI) % MI, ni = m % NI;
+        const float av = c == 0 ? a[mi].x : c == 1 ? a[mi].y : c == 2 ? a[mi].z : a[mi].w;
+        const float bv = c == 0 ? b[ni].x : c == 1 ? b[ni].y : c == 2 ? b[ni].z : b[ni].w;
+        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
+        const int gm = pair * NM_PAIR + m;
+        const int e0 = (gm * NEL) / NM, e1 = ((gm + 1) * NEL) / NM;
+        if (e1 > e0) {
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ni = 0; ni < NI; ni++) {
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi].x, b[ni].x, acc[mi][ni], 0, 0, 0);
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi].y, b[ni].y, acc[mi][ni], 0, 0, 0);
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi].z, b[ni].z, acc[mi][ni], 0, 0, 0);
-          acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi].w, b[ni].w, acc[mi][ni], 0, 0, 0);
+          for (int e = e0; e < e1; e++) elem(e, k2);
+          __builtin_amdgcn_sched_barrier(0);
         }
+      }
     }
-    if (more) {
+    __builtin_amdgcn_sched_barrier(0);
+    {
       const int o = (st ^ 1) * KQ;
 #pragma unroll
       for (int g = 0; g < GA; g++) As[(o + a_kq[g]) * LDA + a_col[g]] = ra[g];
