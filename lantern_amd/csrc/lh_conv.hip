@@ -76,6 +76,60 @@ struct LoadConvBwdDataB {
   }
 };
 
+// ---- fast B operands for channel counts that are a multiple of the k-slab (16) -------------------------
+// The reduction index is ordered tap-major, channel-minor: k = tap*CH + ch.  A 16-wide k-slab
+// then lies inside one filter tap, so the tap decode and the bounds check are done once per
+// slab on wave-uniform values and each element costs an add and a select.  The filter operand
+// is brought into the matching [row][tap][ch] layout by a small transform kernel.
+//
+// Forward: column j = (n, p, q); element = x[n][ch][p*sH - pH + r][q*sW - pW + s], tap = r*S + s.
+struct LoadConvFwdTapB {
+  static constexpr bool ALONG_K = false;
+  static constexpr bool VEC4 = false;
+  const float* base; uint32_t nbytes;
+  int C, H, W, sH, sW, pH, pW, HW;
+  FastDiv dPQ, dQ, dC, dS;
+  struct State { int pix, h0, w0; bool valid; };
+  __device__ __forceinline__ void init(State& s, int j, int ncols) const {
+    s.valid = j < ncols;
+    uint32_t n, pq, p, q;
+    dPQ.divmod(s.valid ? j : 0, n, pq); dQ.divmod(pq, p, q);
+    s.h0 = (int)p * sH - pH; s.w0 = (int)q * sW - pW;
+    s.pix = (int)n * C * HW + s.h0 * W + s.w0;
+  }
+  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
+    uint32_t tap, ch, r, ss;
+    dC.divmod(k, tap, ch); dS.divmod(tap, r, ss);                 // wave-uniform; same tap for e = 0..3
+    const bool ok = s.valid && k < kend && (unsigned)(s.h0 + (int)r) < (unsigned)H && (unsigned)(s.w0 + (int)ss) < (unsigned)W;
+    const int rel = ((int)ch + e) * HW + (int)r * W + (int)ss;   // wave-uniform
+    return ok ? (uint32_t)(s.pix + rel) * 4u : LH_OOB;
+  }
+};
+// Input gradient for one residue class of output pixels (h = aH + sH*h', w = aW + sW*w'): only
+// the taps r = r0 + sH*tr, s = s0 + sW*ts reach it, and on the class grid the gather is a
+// stride-1 correlation:  dy[n][ko][h' + offH - tr][w' + offW - ts],  k = (tr*Sc + ts)*K + ko.
+struct LoadConvBwdDataTapB {
+  static constexpr bool ALONG_K = false;
+  static constexpr bool VEC4 = false;
+  const float* base; uint32_t nbytes;
+  int K, P, Q, PQ, offH, offW;
+  FastDiv dPIX, dWc, dK, dSc;       // class-grid pixels per sample, class-grid width, K, taps per row
+  struct State { int nbase, hq, wq; bool valid; };
+  __device__ __forceinline__ void init(State& s, int j, int ncols) const {
+    s.valid = j < ncols;
+    uint32_t n, pix, h, w;
+    dPIX.divmod(s.valid ? j : 0, n, pix); dWc.divmod(pix, h, w);
+    s.nbase = (int)n * K * PQ; s.hq = (int)h + offH; s.wq = (int)w + offW;
+  }
+  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
+    uint32_t tap, ko, tr, ts;
+    dK.divmod(k, tap, ko); dSc.divmod(tap, tr, ts);               // wave-uniform
+    const int p = s.hq - (int)tr, q = s.wq - (int)ts;
+    const bool ok = s.valid && k < kend && (unsigned)p < (unsigned)P && (unsigned)q < (unsigned)Q;
+    return ok ? (uint32_t)(s.nbase + ((int)ko + e) * PQ + p * Q + q) * 4u : LH_OOB;
+  }
+};
+
 // ---- A operand of the filter gradient: dy rows, reduction index (n, p, q) ------------------------------
 template <bool VEC>                      // VEC: PQ % 4 == 0 and dy 16-byte aligned
 struct LoadConvBwdFilterA {
@@ -119,15 +173,16 @@ struct LoadConvBwdFilterB {
   }
 };
 
-// ---- epilogue writing an NCHW activation: row i = channel, column j = (n, pixel) --------------------------
+// ---- epilogue writing an NCHW activation: row i = channel, column j = (n, u, v) on a grid of
+//      Wc columns; the element lands at out[n][i][aH + eH*u][aW + eW*v] of an image W wide with PIX pixels.
 struct EpiConvOut {
-  float* out; const float* bias; int chan, PIX; float beta;
-  FastDiv dPIX;
+  float* out; const float* bias; int chan, PIX, W, eH, eW, aH, aW; float beta;
+  FastDiv dPIXc, dWc;
   struct Col { int off; bool valid; };
   __device__ __forceinline__ Col col(int j, int N) const {
     Col c; c.valid = j < N;
-    uint32_t n, pix; dPIX.divmod(c.valid ? j : 0, n, pix);
-    c.off = (int)n * chan * PIX + (int)pix;
+    uint32_t n, pix, u, v; dPIXc.divmod(c.valid ? j : 0, n, pix); dWc.divmod(pix, u, v);
+    c.off = (int)n * chan * PIX + (aH + eH * (int)u) * W + aW + eW * (int)v;
     return c;
   }
   __device__ __forceinline__ void store(const Col& c, int i, int M, float v) const {
@@ -137,7 +192,29 @@ struct EpiConvOut {
     *p = beta == 0.f ? v : v + beta * *p;
   }
 };
+static EpiConvOut make_epi(float* out, const float* bias, int chan, int Himg, int Wimg, float beta) {   // dense: grid == image
+  EpiConvOut ep; ep.out = out; ep.bias = bias; ep.chan = chan; ep.PIX = Himg * Wimg; ep.W = Wimg; ep.eH = 1; ep.eW = 1; ep.aH = 0; ep.aW = 0; ep.beta = beta;
+  ep.dPIXc.init(Himg * Wimg); ep.dWc.init(Wimg);
+  return ep;
+}
 
+// w[K][C][RS] -> wt[K][RS][C]   (forward, tap-major reduction order)
+__global__ void __launch_bounds__(TPB) k_filter_to_krsc(const float* __restrict__ w, float* __restrict__ wt, int C, int RS, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    int c = (int)(i % C); int64_t t = i / C; int rs = (int)(t % RS); int64_t k = t / RS;
+    wt[i] = w[(k * C + c) * RS + rs];
+  }
+}
+// w[K][C][R][S] -> wt[C][tr][ts][K] for the taps r = r0 + sH*tr (tr < Rc), s = s0 + sW*ts (ts < Sc)
+__global__ void __launch_bounds__(TPB) k_filter_to_ctk(const float* __restrict__ w, float* __restrict__ wt, int K, int C, int R, int S,
+                                                       int r0, int s0, int sH, int sW, int Rc, int Sc, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n; i += st) {
+    int k = (int)(i % K); int64_t t = i / K; int ts = (int)(t % Sc); t /= Sc; int tr = (int)(t % Rc); int c = (int)(t / Rc);
+    wt[i] = w[(((int64_t)k * C + c) * R + (r0 + sH * tr)) * S + (s0 + sW * ts)];
+  }
+}
 // w[K][C][RS] -> wt[C][K][RS]
 __global__ void __launch_bounds__(TPB) k_filter_transpose(const float* __restrict__ w, float* __restrict__ wt, int K, int C, int RS, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
@@ -173,15 +250,34 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
   ProfScope prof_(CAT_CONV_FWD);
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_fwd: bad shape N%d C%d H%d W%d K%d R%d S%d s(%d,%d) p(%d,%d)", N, C, H, W, K, R, S, sH, sW, pH, pW);
-  const int CRS = C * R * S, PQ = d.P * d.Q;
-  const bool avec = (CRS % 4 == 0) && (((uintptr_t)w & 15) == 0);
-  const uint32_t wbytes = (uint32_t)((size_t)K * CRS * 4);
-  LoadConvFwdB bl; bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * H * W * 4); bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
-  bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
-  EpiConvOut ep; ep.out = y; ep.bias = bias; ep.chan = K; ep.PIX = PQ; ep.beta = 0.f; ep.dPIX.init(PQ);
+  const int RS = R * S, CRS = C * RS, PQ = d.P * d.Q;
+  const uint32_t wbytes = (uint32_t)((size_t)K * CRS * 4), xbytes = (uint32_t)((size_t)N * C * H * W * 4);
+  EpiConvOut ep = make_epi(y, bias, K, d.P, d.Q, 0.f);
   bool ok;
-  if (avec) { LoadPlainK<true> al; al.base = w; al.nbytes = wbytes; al.ld = CRS; ok = launch_tiles(al, bl, ep, K, N * PQ, CRS); }
-  else { LoadPlainK<false> al; al.base = w; al.nbytes = wbytes; al.ld = CRS; ok = launch_tiles(al, bl, ep, K, N * PQ, CRS); }
+  if (C % 16 == 0 && ((uintptr_t)w & 15) == 0) {
+    // tap-major reduction order; a 1x1 filter already has that layout
+    const float* wk = w;
+    size_t scratch = 0;
+    if (RS > 1) {
+      scratch = wbytes;
+      float* wt = (float*)lh_malloc_uninit(scratch);   // released below: stream order keeps it safe
+      if (wt == nullptr) return;
+      int64_t n = (int64_t)K * CRS;
+      hipLaunchKernelGGL(k_filter_to_krsc, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, C, RS, n);
+      wk = wt;
+    }
+    LoadPlainK<true> al; al.base = wk; al.nbytes = wbytes; al.ld = CRS;
+    LoadConvFwdTapB bl; bl.base = x; bl.nbytes = xbytes; bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
+    bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dC.init(C); bl.dS.init(S);
+    ok = launch_tiles(al, bl, ep, K, N * PQ, CRS);
+    if (scratch) lh_free_top(scratch);
+  } else {
+    const bool avec = (CRS % 4 == 0) && (((uintptr_t)w & 15) == 0);
+    LoadConvFwdB bl; bl.base = x; bl.nbytes = xbytes; bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
+    bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(RS); bl.dS.init(S);
+    if (avec) { LoadPlainK<true> al; al.base = w; al.nbytes = wbytes; al.ld = CRS; ok = launch_tiles(al, bl, ep, K, N * PQ, CRS); }
+    else { LoadPlainK<false> al; al.base = w; al.nbytes = wbytes; al.ld = CRS; ok = launch_tiles(al, bl, ep, K, N * PQ, CRS); }
+  }
   if (!ok) return;
   LH_CHECK_LAUNCH();
 }
@@ -193,24 +289,59 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_data: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_data: beta must be 0 or 1");
   const int RS = R * S, KRS = K * RS, HW = H * W, PQ = d.P * d.Q;
-  LoadConvBwdDataB bl; bl.base = dy; bl.nbytes = (uint32_t)((size_t)N * K * PQ * 4); bl.K = K; bl.P = d.P; bl.Q = d.Q; bl.PQ = PQ; bl.pH = pH; bl.pW = pW;
-  bl.dHW.init(HW); bl.dW.init(W); bl.dRS.init(RS); bl.dS.init(S); bl.dsH.init(sH); bl.dsW.init(sW);
-  EpiConvOut ep; ep.out = dx; ep.bias = nullptr; ep.chan = C; ep.PIX = HW; ep.beta = beta; ep.dPIX.init(HW);
-  bool ok;
-  if (RS == 1) {
-    LoadPlainT al; al.base = w; al.nbytes = (uint32_t)((size_t)K * C * 4); al.ld = C;          // A[c][k] = w[k][c]
-    ok = launch_tiles(al, bl, ep, C, N * HW, KRS);
+  const uint32_t dybytes = (uint32_t)((size_t)N * K * PQ * 4);
+  bool ok = true;
+  if (K % 16 == 0) {
+    // One implicit GEMM per residue class (aH, aW) of input pixels modulo the stride: no MFMA
+    // work is spent on taps that cannot reach a pixel.  Stride 1 is the single class (0, 0).
+    bool any_empty = false;
+    for (int aH = 0; aH < sH; aH++) for (int aW = 0; aW < sW; aW++) {
+      int r0 = (aH + pH) % sH, s0 = (aW + pW) % sW;
+      if (r0 >= R || s0 >= S || aH >= H || aW >= W) any_empty = true;
+    }
+    if (beta == 0.f && any_empty) lh_fill(dx, 0.f, (int64_t)N * C * HW);
+    for (int aH = 0; aH < sH && ok; aH++) for (int aW = 0; aW < sW && ok; aW++) {
+      const int r0 = (aH + pH) % sH, s0 = (aW + pW) % sW;
+      if (r0 >= R || s0 >= S || aH >= H || aW >= W) continue;
+      const int Rc = (R - r0 + sH - 1) / sH, Sc = (S - s0 + sW - 1) / sW;
+      const int Hc = (H - aH + sH - 1) / sH, Wc = (W - aW + sW - 1) / sW;
+      const int Kred = Rc * Sc * K;
+      LoadConvBwdDataTapB bl; bl.base = dy; bl.nbytes = dybytes; bl.K = K; bl.P = d.P; bl.Q = d.Q; bl.PQ = PQ;
+      bl.offH = (aH + pH - r0) / sH; bl.offW = (aW + pW - s0) / sW;
+      bl.dPIX.init(Hc * Wc); bl.dWc.init(Wc); bl.dK.init(K); bl.dSc.init(Sc);
+      EpiConvOut ep; ep.out = dx; ep.bias = nullptr; ep.chan = C; ep.PIX = HW; ep.W = W; ep.eH = sH; ep.eW = sW; ep.aH = aH; ep.aW = aW; ep.beta = beta;
+      ep.dPIXc.init(Hc * Wc); ep.dWc.init(Wc);
+      if (RS == 1) {
+        LoadPlainT al; al.base = w; al.nbytes = (uint32_t)((size_t)K * C * 4); al.ld = C;          // A[c][k] = w[k][c]
+        ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred);
+      } else {
+        size_t bytes = (size_t)Kred * C * sizeof(float);
+        float* wt = (float*)lh_malloc_uninit(bytes);     // released below: stream order keeps it safe
+        if (wt == nullptr) return;
+        int64_t n = (int64_t)Kred * C;
+        hipLaunchKernelGGL(k_filter_to_ctk, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, R, S, r0, s0, sH, sW, Rc, Sc, n);
+        LoadPlainK<true> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = Kred;
+        ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred);
+        lh_free_top(bytes);
+      }
+    }
   } else {
-    // transposed filter in scratch taken from the arena top and released again: later
-    // allocations may reuse it, but only by work enqueued after this call on the same stream.
-    size_t bytes = (size_t)KRS * C * sizeof(float);
-    float* wt = (float*)lh_malloc_uninit(bytes);
-    if (wt == nullptr) return;
-    int64_t n = (int64_t)KRS * C;
-    hipLaunchKernelGGL(k_filter_transpose, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, RS, n);
-    if (KRS % 4 == 0) { LoadPlainK<true> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
-    else { LoadPlainK<false> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
-    lh_free_top(bytes);
+    LoadConvBwdDataB bl; bl.base = dy; bl.nbytes = dybytes; bl.K = K; bl.P = d.P; bl.Q = d.Q; bl.PQ = PQ; bl.pH = pH; bl.pW = pW;
+    bl.dHW.init(HW); bl.dW.init(W); bl.dRS.init(RS); bl.dS.init(S); bl.dsH.init(sH); bl.dsW.init(sW);
+    EpiConvOut ep = make_epi(dx, nullptr, C, H, W, beta);
+    if (RS == 1) {
+      LoadPlainT al; al.base = w; al.nbytes = (uint32_t)((size_t)K * C * 4); al.ld = C;
+      ok = launch_tiles(al, bl, ep, C, N * HW, KRS);
+    } else {
+      size_t bytes = (size_t)KRS * C * sizeof(float);
+      float* wt = (float*)lh_malloc_uninit(bytes);
+      if (wt == nullptr) return;
+      int64_t n = (int64_t)KRS * C;
+      hipLaunchKernelGGL(k_filter_transpose, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, RS, n);
+      if (KRS % 4 == 0) { LoadPlainK<true> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
+      else { LoadPlainK<false> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
+      lh_free_top(bytes);
+    }
   }
   if (!ok) return;
   LH_CHECK_LAUNCH();
