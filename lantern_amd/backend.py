@@ -185,20 +185,21 @@ class BackendHIP(Backend):
         _lib.check()
         return res
 
-    def gemm_grad(self, x, xd, x_in, tx, y, yd, y_in, ty, alpha, od, d1, d2, d3):
+    def gemm_grad(self, x, xd, x_in, tx, y, yd, y_in, ty, alpha, od, d1, d2, d3, xbeta=1.0, ybeta=1.0):
+        """CUB:630-688; beta = 0 overwrites a gradient buffer that has no content yet."""
         g = self.lib.lh_sgemm
         if not tx and not ty:
-            if not x_in: g(0, 1, d1, d2, d3, alpha, od.ptr, d3, y.ptr, d3, 1.0, xd.ptr, d2)
-            if not y_in: g(1, 0, d2, d3, d1, alpha, x.ptr, d2, od.ptr, d3, 1.0, yd.ptr, d3)
+            if not x_in: g(0, 1, d1, d2, d3, alpha, od.ptr, d3, y.ptr, d3, xbeta, xd.ptr, d2)
+            if not y_in: g(1, 0, d2, d3, d1, alpha, x.ptr, d2, od.ptr, d3, ybeta, yd.ptr, d3)
         elif not tx and ty:
-            if not x_in: g(0, 0, d1, d2, d3, alpha, od.ptr, d3, y.ptr, d2, 1.0, xd.ptr, d2)
-            if not y_in: g(1, 0, d3, d2, d1, alpha, od.ptr, d3, x.ptr, d2, 1.0, yd.ptr, d2)
+            if not x_in: g(0, 0, d1, d2, d3, alpha, od.ptr, d3, y.ptr, d2, xbeta, xd.ptr, d2)
+            if not y_in: g(1, 0, d3, d2, d1, alpha, od.ptr, d3, x.ptr, d2, ybeta, yd.ptr, d2)
         elif tx and not ty:
-            if not x_in: g(0, 1, d2, d1, d3, alpha, y.ptr, d3, od.ptr, d3, 1.0, xd.ptr, d1)
-            if not y_in: g(0, 0, d2, d3, d1, alpha, x.ptr, d1, od.ptr, d3, 1.0, yd.ptr, d3)
+            if not x_in: g(0, 1, d2, d1, d3, alpha, y.ptr, d3, od.ptr, d3, xbeta, xd.ptr, d1)
+            if not y_in: g(0, 0, d2, d3, d1, alpha, x.ptr, d1, od.ptr, d3, ybeta, yd.ptr, d3)
         else:
-            if not x_in: g(1, 1, d2, d1, d3, alpha, y.ptr, d2, od.ptr, d3, 1.0, xd.ptr, d1)
-            if not y_in: g(1, 1, d3, d2, d1, alpha, od.ptr, d3, x.ptr, d1, 1.0, yd.ptr, d2)
+            if not x_in: g(1, 1, d2, d1, d3, alpha, y.ptr, d2, od.ptr, d3, xbeta, xd.ptr, d1)
+            if not y_in: g(1, 1, d3, d2, d1, alpha, od.ptr, d3, x.ptr, d1, ybeta, yd.ptr, d2)
         _lib.check()
 
     # -- broadcast arithmetic (TD:222-270) ---------------------------------------------------------
@@ -246,9 +247,9 @@ class BackendHIP(Backend):
         self.lib.lh_conv2d_fwd(x.ptr, w.ptr, bias.ptr if bias is not None else 0, y.ptr, N, C, H, W, K, R, S, sH, sW, pH, pW); _lib.check()
         return y, None      # no im2col buffer is kept (BackendCudnn returns None too, CDN:859-866)
 
-    def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW):
+    def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
         if not x_in:
-            self.lib.lh_conv2d_bwd_data(dy.ptr, w.ptr, xd.ptr, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
+            self.lib.lh_conv2d_bwd_data(dy.ptr, w.ptr, xd.ptr, beta_dx, N, C, H, W, K, R, S, sH, sW, pH, pW)
         self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
         _lib.check()
 
@@ -281,8 +282,8 @@ class BackendHIP(Backend):
         self.lib.lh_bn_train_fwd(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
         return y, sm, si
 
-    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW):
-        self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, 1.0, scaled.ptr, biasd.ptr, N, C, HW); _lib.check()
+    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0):
+        self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, beta_dx, scaled.ptr, biasd.ptr, N, C, HW); _lib.check()
 
     # -- dropout ------------------------------------------------------------------------------------
     def dropout(self, x, n, prob):

@@ -234,12 +234,16 @@ __global__ void __launch_bounds__(TPB) k_conv_bwd_bias(const float* __restrict__
   if (threadIdx.x == 0) db[k] += acc;
 }
 
+#ifndef LH_CONV_BK
+#define LH_CONV_BK 16
+#endif
+constexpr int CONV_BK = LH_CONV_BK;      // k-slab of the forward / input-gradient kernels
 template <class AL, class BL, class EP>
 static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K) {
   TilePick tp = pick_tile(M, N);
-  if (tp.bm == 128) return igemm_launch<128, 128, 16>(al, bl, ep, M, N, K, 1);
-  if (tp.bn == 128) return igemm_launch<64, 128, 16>(al, bl, ep, M, N, K, 1);
-  return igemm_launch<64, 64, 16>(al, bl, ep, M, N, K, 1);
+  if (tp.bm == 128) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1);
+  if (tp.bn == 128) return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1);
+  return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1);
 }
 }  // namespace
 
@@ -254,7 +258,7 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
   const uint32_t wbytes = (uint32_t)((size_t)K * CRS * 4), xbytes = (uint32_t)((size_t)N * C * H * W * 4);
   EpiConvOut ep = make_epi(y, bias, K, d.P, d.Q, 0.f);
   bool ok;
-  if (C % 16 == 0 && ((uintptr_t)w & 15) == 0) {
+  if (C % CONV_BK == 0 && ((uintptr_t)w & 15) == 0) {
     // tap-major reduction order; a 1x1 filter already has that layout
     const float* wk = w;
     size_t scratch = 0;
@@ -291,7 +295,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
   const int RS = R * S, KRS = K * RS, HW = H * W, PQ = d.P * d.Q;
   const uint32_t dybytes = (uint32_t)((size_t)N * K * PQ * 4);
   bool ok = true;
-  if (K % 16 == 0) {
+  if (K % CONV_BK == 0) {
     // One implicit GEMM per residue class (aH, aW) of input pixels modulo the stride: no MFMA
     // work is spent on taps that cannot reach a pixel.  Stride 1 is the single class (0, 0).
     bool any_empty = false;

@@ -376,18 +376,44 @@ def int_array(values):
 class TensorR:
     """A value with its gradient (TD:1146-1506).  `d` accumulates; inputs never receive one."""
 
-    def __init__(self, x, d=None, isInput=False):
+    def __init__(self, x, d=None, isInput=False, lazy_grad=False):
+        """`lazy_grad`: the gradient buffer of an intermediate value is created at its first use in
+        the backward pass.  The reference allocates it zero-filled at construction (TD:1509-1514)
+        and every gradient op accumulates; a first writer that can overwrite (beta = 0) makes the
+        zero fill and the read-modify-write unnecessary, with the same result."""
         self.x = x
-        if d is None:
-            d = Tensor.zeros(2) if isInput else Tensor.zeros_like(x)     # TD:1509-1514
-        self.d = d
         self.isInput = isInput
+        self._d = d
+        if d is None and not lazy_grad:
+            self._d = Tensor.zeros(2) if isInput else Tensor.zeros_like(x)     # TD:1509-1514
+
+    @property
+    def d(self):
+        if self._d is None:
+            self._d = Tensor.zeros(2) if self.isInput else Tensor.zeros_like(self.x)
+        return self._d
+
+    @d.setter
+    def d(self, t):
+        self._d = t
+
+    def grad_target(self):
+        """(gradient buffer, beta) for an op that can either overwrite or accumulate."""
+        if self._d is None:
+            self._d = Tensor(get_backend().mallocArray(self.x.scalarCount, zero=False), self.x.shape)
+            return self._d.data, 0.0
+        return self._d.data, 1.0
+
+    @staticmethod
+    def _new(x):
+        """Result of an op: gradient created on demand."""
+        return TensorR(x, lazy_grad=True)
 
     def __call__(self, i): return TensorR(self.x(i), self.d(i))
 
     def resize(self, *dims):
         nd = resize_dim(self.x.scalarCount, dims)
-        return TensorR(Tensor(self.x.data, nd), Tensor(self.d.data, nd), self.isInput)
+        return TensorR(Tensor(self.x.data, nd), Tensor(self.d.data, nd), self.isInput)     # a view: shares x and d
 
     def clip_grad(self, bound): self.d.clipAt(bound)
     def clear_grad(self): self.d.clear()
@@ -414,12 +440,24 @@ class TensorR:
         be = get_backend()
         if isinstance(that, TensorR):
             ya, a, b = self.x._bin(op, that.x)
-            y = TensorR(ya)
-            _tape.append(lambda: be.bcast_op_grad(op, self.x.data, self.d.data, a, self.isInput, that.x.data, that.d.data, b, that.isInput,
-                                                  y.d.data, ya.shape))
+            y = TensorR._new(ya)
+            def back():
+                full = a == ya.shape and b == ya.shape
+                if full and op == B.ADD and self is not that:
+                    # same-shape add: a fresh gradient buffer is written by a copy, not zero + accumulate
+                    for t in (self, that):
+                        if t.isInput: continue
+                        if t._d is None:
+                            buf, _ = t.grad_target()
+                            be.copyFloatArray(buf, y.d.data, ya.scalarCount)
+                        else:
+                            be.bcast_update(B.ADD, t.d.data, ya.shape, y.d.data, ya.shape)
+                    return
+                be.bcast_op_grad(op, self.x.data, self.d.data, a, self.isInput, that.x.data, that.d.data, b, that.isInput, y.d.data, ya.shape)
+            _tape.append(back)
             return y
         s = float(that)
-        y = TensorR(self.x._bin(op, s))
+        y = TensorR._new(self.x._bin(op, s))
         def back():
             if self.isInput: return
             if op in (B.ADD, B.SUB): self.d += y.d                                   # TD:1167-1181
@@ -435,7 +473,7 @@ class TensorR:
 
     def dot(self, that):
         be = get_backend()
-        y = TensorR(self.x.dot(that.x))
+        y = TensorR._new(self.x.dot(that.x))
         def back():                                                                   # dot_grad (CPU:171-184)
             xr, yr = self.x.rank, that.x.rank
             if xr == 1 and yr == 1:
@@ -455,18 +493,21 @@ class TensorR:
     def gemm(self, that, transX, transY, alpha):
         be = get_backend()
         d1, d2, d3 = Tensor._gemm_dims(self.x.shape, transX, that.x.shape, transY)
-        y = TensorR(self.x.gemm(that.x, transX, transY, alpha))
-        _tape.append(lambda: be.gemm_grad(self.x.data, self.d.data, self.isInput, transX, that.x.data, that.d.data, that.isInput, transY,
-                                          float(alpha), y.d.data, d1, d2, d3))
+        y = TensorR._new(self.x.gemm(that.x, transX, transY, alpha))
+        def back():
+            xd, xbeta = (None, 1.0) if self.isInput else self.grad_target()
+            yd, ybeta = (None, 1.0) if that.isInput else that.grad_target()
+            be.gemm_grad(self.x.data, xd, self.isInput, transX, that.x.data, yd, that.isInput, transY, float(alpha), y.d.data, d1, d2, d3, xbeta, ybeta)
+        _tape.append(back)
         return y
 
     def trans(self):
-        y = TensorR(self.x.trans())
+        y = TensorR._new(self.x.trans())
         _tape.append(lambda: get_backend().trans_grad(self.d.data, y.d.data, self.x.shape[0], self.x.shape[1]))
         return y
 
     def permute(self, *dims):
-        y = TensorR(self.x.permute(*dims))
+        y = TensorR._new(self.x.permute(*dims))
         _tape.append(lambda: get_backend().permute_grad(self.d.data, y.d.data, self.x.shape, dims))
         return y
 
@@ -477,7 +518,7 @@ class TensorR:
             self.x._unary(op, True, lo, hi)
             _tape.append(lambda: be.unary_grad(op, self.x.data, self.x.data, self.d.data, self.d.data, self.x.scalarCount, True, lo, hi))
             return self
-        y = TensorR(self.x._unary(op, False, lo, hi))
+        y = TensorR._new(self.x._unary(op, False, lo, hi))
         _tape.append(lambda: be.unary_grad(op, self.x.data, y.x.data, y.d.data, self.d.data, self.x.scalarCount, False, lo, hi))
         return y
 
@@ -501,7 +542,7 @@ class TensorR:
             y = TensorR(self.x.sum(), Tensor.zeros(1))
             _tape.append(lambda: be.add_scalar_from(self.d.data, y.d.data, 1.0, self.x.scalarCount))
             return y
-        y = TensorR(self.x.sum(dim))
+        y = TensorR._new(self.x.sum(dim))
         sh = self.x.shape
         outer, d, inner = _prod(sh[:dim]), sh[dim], _prod(sh[dim + 1:])
         _tape.append(lambda: be.sum_dim_grad(self.d.data, y.d.data, outer, d, inner))
@@ -517,10 +558,12 @@ class TensorR:
     def batchNorm(self, scale, bias, runningMean, runningVar):
         be = get_backend()
         yv, sm, si = self.x.batchNormTraining(scale.x, bias.x, runningMean, runningVar)
-        y = TensorR(yv)
+        y = TensorR._new(yv)
         N, C, HW = self.x._bn_view()
-        _tape.append(lambda: be.batchNorm_grad(self.x.data, None if self.isInput else self.d.data, y.d.data, scale.x.data, scale.d.data,
-                                               bias.d.data, sm.data, si.data, N, C, HW))
+        def back():
+            xd, beta = (None, 1.0) if self.isInput else self.grad_target()
+            be.batchNorm_grad(self.x.data, xd, y.d.data, scale.x.data, scale.d.data, bias.d.data, sm.data, si.data, N, C, HW, beta)
+        _tape.append(back)
         return y
 
     batchNorm1D = batchNorm
@@ -528,21 +571,21 @@ class TensorR:
     def softmax_batch(self, dim=1):
         be = get_backend()
         o, c, i = self.x._softmax_view(dim)
-        y = TensorR(self.x.softmax_batch(dim))
+        y = TensorR._new(self.x.softmax_batch(dim))
         _tape.append(lambda: be.softmax_grad(False, y.x.data, y.d.data, self.d.data, o, c, i))
         return y
 
     def logSoftmaxB(self, dim=1):
         be = get_backend()
         o, c, i = self.x._softmax_view(dim)
-        y = TensorR(self.x.logSoftmaxB(dim))
+        y = TensorR._new(self.x.logSoftmaxB(dim))
         _tape.append(lambda: be.softmax_grad(True, y.x.data, y.d.data, self.d.data, o, c, i))
         return y
 
     def nllLossB(self, target):
         be = get_backend()
         assert self.x.rank == 2, "nllLossB() function only takes tensor of rank 2, got %s" % (self.x.shape,)
-        y = TensorR(self.x.nllLossB(target))
+        y = TensorR._new(self.x.nllLossB(target))
         _tape.append(lambda: be.nllLoss_grad(self.d.data, target, y.d.data, self.x.shape[0], self.x.shape[1]))
         return y
 
@@ -552,30 +595,33 @@ class TensorR:
         assert self.isInput or self.d.scalarCount == self.x.scalarCount, "For convBBP, THIS is either input or intermediate stage"
         assert self.x.rank == 4, "For convBBP, THIS is dim 4: batch, channel, row, col"
         out, finput = self.x.conv2D_batch(kernel.x, bias.x if bias is not None else None, strides, pads)
-        y = TensorR(out)
+        y = TensorR._new(out)
         N, C, H, W = self.x.shape; K, _, R, S = kernel.x.shape
         sH, sW = strides[0], strides[1]; pH, pW = Tensor._pads2(pads)
-        _tape.append(lambda: be.conv2D_batch_grad(self.x.data, self.d.data, self.isInput, finput, kernel.x.data, kernel.d.data, y.d.data,
-                                                  bias.d.data if bias is not None else None, N, C, H, W, K, R, S, sH, sW, pH, pW))
+        def back():
+            xd, beta = (None, 1.0) if self.isInput else self.grad_target()
+            be.conv2D_batch_grad(self.x.data, xd, self.isInput, finput, kernel.x.data, kernel.d.data, y.d.data,
+                                 bias.d.data if bias is not None else None, N, C, H, W, K, R, S, sH, sW, pH, pW, beta)
+        _tape.append(back)
         return y
 
     def maxPoolBK(self, kernels, strides, pads=None):
         be = get_backend()
         yv, idx = self.x.maxPool2D_batch(kernels, strides, pads)
-        y = TensorR(yv)
+        y = TensorR._new(yv)
         _tape.append(lambda: be.maxPool2D_batch_grad(self.d.data, y.d.data, idx, yv.scalarCount))
         return y
 
     def averagePoolBK(self, kernels, strides, pads=None):
         be = get_backend()
-        y = TensorR(self.x.averagePool2D_batch(kernels, strides, pads))
+        y = TensorR._new(self.x.averagePool2D_batch(kernels, strides, pads))
         N, C, H, W = self.x.shape
         _tape.append(lambda: be.averagePool2D_batch_grad(self.d.data, y.d.data, N, C, H, W, kernels[0], kernels[1], strides[0], strides[1]))
         return y
 
     def global_ave_batch(self):
         be = get_backend()
-        y = TensorR(self.x.global_ave_batch())
+        y = TensorR._new(self.x.global_ave_batch())
         n, c, h, w = self.x.shape
         def back():                                  # TD:1454-1479: d += ty.d * (1/HW) broadcast over H,W
             scaled = y.d * (1.0 / (h * w))
@@ -586,7 +632,7 @@ class TensorR:
     def concat(self, dim, *others):
         be = get_backend()
         ts = (self,) + others
-        y = TensorR(self.x.concat(dim, *[t.x for t in others]))
+        y = TensorR._new(self.x.concat(dim, *[t.x for t in others]))
         outer, inner = _prod(self.x.shape[:dim]), _prod(self.x.shape[dim + 1:])
         sizes = [t.x.shape[dim] for t in ts]
         _tape.append(lambda: be.concat_grad([None if t.isInput else t.d.data for t in ts], sizes, y.d.data, outer, inner))
@@ -595,7 +641,7 @@ class TensorR:
     def dropout(self, prob):
         be = get_backend()
         yv, mask = self.x.dropout(prob)
-        y = TensorR(yv)
+        y = TensorR._new(yv)
         _tape.append(lambda: be.dropout_grad(self.d.data, y.d.data, mask, self.x.scalarCount))
         return y
 

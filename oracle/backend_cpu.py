@@ -119,9 +119,10 @@ class BackendCPU(Backend):
         self._c("lc_gemm", I(int(tx)), I(int(ty)), I(d1), I(d2), I(d3), F(alpha), P(x.ptr), P(y.ptr), P(res.ptr))
         return res
 
-    def gemm_grad(self, x, xd, x_in, tx, y, yd, y_in, ty, alpha, od, d1, d2, d3):
-        self._c("lc_gemm_grad", I(int(tx)), I(int(ty)), I(d1), I(d2), I(d3), F(alpha), P(x.ptr), P(xd.ptr), I(int(x_in)),
-                P(y.ptr), P(yd.ptr), I(int(y_in)), P(od.ptr))
+    def gemm_grad(self, x, xd, x_in, tx, y, yd, y_in, ty, alpha, od, d1, d2, d3, xbeta=1.0, ybeta=1.0):
+        # host memory from mallocArray is always zero, so overwrite (beta 0) and accumulate coincide
+        self._c("lc_gemm_grad", I(int(tx)), I(int(ty)), I(d1), I(d2), I(d3), F(alpha), P(x.ptr), P(xd.ptr if xd is not None else 0), I(int(x_in)),
+                P(y.ptr), P(yd.ptr if yd is not None else 0), I(int(y_in)), P(od.ptr))
 
     # -- broadcast -----------------------------------------------------------------------------------
     def bcast_op(self, op, a, ashape, b, bshape, oshape):
@@ -164,7 +165,7 @@ class BackendCPU(Backend):
                 *[I(v) for v in (N, C_, H, W, K, R, S, sH, sW, pH, pW)])
         return y, finput
 
-    def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C_, H, W, K, R, S, sH, sW, pH, pW):
+    def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C_, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
         Pp, Q = conv_size(H, R, sH, pH), conv_size(W, S, sW, pW)
         scratch = None if x_in else self.mallocArray(N * C_ * R * S * Pp * Q)
         self._c("lc_conv2d_bwd", P(finput.ptr), P(w.ptr), P(dy.ptr), P(0 if x_in else xd.ptr), P(wd.ptr), P(bd.ptr if bd is not None else 0),
@@ -197,7 +198,7 @@ class BackendCPU(Backend):
                 I(N), I(C_), I(HW), F(eps), F(factor))
         return y, sm, si
 
-    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C_, HW):
+    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C_, HW, beta_dx=1.0):
         self._c("lc_bn_bwd", P(x.ptr), P(dy.ptr), P(scale.ptr), P(sm.ptr), P(si.ptr), P(xd.ptr if xd is not None else 0),
                 P(scaled.ptr), P(biasd.ptr), I(N), I(C_), I(HW))
 
