@@ -153,6 +153,19 @@ void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, floa
 void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
 
+/* ---- fusions of adjacent trait calls (no single counterpart in the reference; each gives the
+ *      result of the sequence it replaces, in one pass over memory) ------------------------ */
+/* batchNormTraining followed by relu(inPlace = true): y = max(bn(x), 0) */
+void lh_bn_train_fwd_relu(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                          float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor);
+/* relu_grad(inPlace) followed by batchNorm_grad: dy counts only where y > 0 (dy itself is left untouched) */
+void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+                    float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
+/* `+` of two same-shape tensors followed by relu(inPlace = true), and the gradient of that pair:
+ * g = dy where y > 0 else 0;  ad = abeta*ad + g;  bd = bbeta*bd + g  (ad or bd may be NULL) */
+void lh_add_relu(const float* a, const float* b, float* out, int64_t n);
+void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, float* bd, float bbeta, int64_t n);
+
 /* ---- dropout (TD:312-313; CPU:1066-1088).  The mask is drawn from a
  *      counter-based generator keyed by (seed, offset + element index), so a
  *      host restatement reproduces it exactly. */

@@ -74,6 +74,10 @@ SIGNATURES = {
     "lh_bn_infer": (None, [P, P, P, P, P, P, I, I, I, F]),
     "lh_bn_train_fwd": (None, [P, P, P, P, P, P, P, P, I, I, I, F, F]),
     "lh_bn_bwd": (None, [P, P, P, P, P, P, F, P, P, I, I, I]),
+    "lh_bn_train_fwd_relu": (None, [P, P, P, P, P, P, P, P, I, I, I, F, F]),
+    "lh_bn_bwd_relu": (None, [P, P, P, P, P, P, P, F, P, P, I, I, I]),
+    "lh_add_relu": (None, [P, P, P, L]),
+    "lh_add_relu_grad": (None, [P, P, P, F, P, F, L]),
     "lh_dropout_fwd": (None, [P, P, P, L, F, U64, U64]),
     "lh_dropout_bwd": (None, [P, P, P, L]),
     "lh_concat": (None, [I, P, P, P, I, I]),

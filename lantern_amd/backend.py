@@ -70,6 +70,25 @@ class Backend:
     def getMallocAddr(self): raise NotImplementedError                      # TD:1782-1784 / CUB:18-20
     def resetMallocAddr(self, addr): raise NotImplementedError              # TD:1786-1789 / CUB:22-25
 
+    # -- fusable pairs: defaults are the unfused sequences of trait calls ------------------------------
+    def batchNormTraining_into(self, x, scale, bias, rmean, rvar, y, sm, si, N, C, HW, relu, eps=1e-5, factor=0.1):
+        """batchNormTraining writing into caller-provided y / saveMean / saveInvStd, optionally followed by relu(inPlace)."""
+        yy, m, v = self.batchNormTraining(x, scale, bias, rmean, rvar, N, C, HW, eps, factor)
+        self.copyFloatArray(y, yy, N * C * HW); self.copyFloatArray(sm, m, C); self.copyFloatArray(si, v, C)
+        if relu:
+            self.unary(RELU, y, N * C * HW, inPlace=True)
+
+    def add_into(self, a, b, out, n, relu):
+        self.geam(a, 1.0, b, 1.0, out, n)
+        if relu:
+            self.unary(RELU, out, n, inPlace=True)
+
+    def add_relu_grad(self, y, dy, ad, abeta, bd, bbeta, n):
+        self.unary_grad(RELU, y, y, dy, dy, n, inPlace=True)            # masks dy in place (CPU:725-726 with the y > 0 mask)
+        for d in (ad, bd):
+            if d is not None:
+                self.geam(d, 1.0, dy, 1.0, d, n)                        # buffers from mallocArray start at zero
+
 
 class BackendHIP(Backend):
     """The MI355X backend: every method is one or a few calls into liblantern_hip.so.
@@ -282,8 +301,25 @@ class BackendHIP(Backend):
         self.lib.lh_bn_train_fwd(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
         return y, sm, si
 
-    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0):
-        self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, beta_dx, scaled.ptr, biasd.ptr, N, C, HW); _lib.check()
+    def batchNormTraining_into(self, x, scale, bias, rmean, rvar, y, sm, si, N, C, HW, relu, eps=1e-5, factor=0.1):
+        f = self.lib.lh_bn_train_fwd_relu if relu else self.lib.lh_bn_train_fwd
+        f(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
+
+    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0, y_relu=None):
+        xdp = xd.ptr if xd is not None else 0
+        if y_relu is not None:
+            self.lib.lh_bn_bwd_relu(x.ptr, y_relu.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
+        else:
+            self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
+        _lib.check()
+
+    def add_into(self, a, b, out, n, relu):
+        if relu: self.lib.lh_add_relu(a.ptr, b.ptr, out.ptr, n)
+        else: self.lib.lh_geam(a.ptr, 1.0, b.ptr, 1.0, out.ptr, n)
+        _lib.check()
+
+    def add_relu_grad(self, y, dy, ad, abeta, bd, bbeta, n):
+        self.lib.lh_add_relu_grad(y.ptr, dy.ptr, ad.ptr if ad is not None else 0, abeta, bd.ptr if bd is not None else 0, bbeta, n); _lib.check()
 
     # -- dropout ------------------------------------------------------------------------------------
     def dropout(self, x, n, prob):

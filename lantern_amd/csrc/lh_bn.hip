@@ -80,7 +80,7 @@ __device__ __forceinline__ void combine_stats(const float* partial, int c, int s
   for (int s = 0; s < slices; s++) { const float* p = partial + 3 * ((int64_t)c * slices + s); double d = p[0] - mean; m2 += p[1] + p[2] * d * d; }
 }
 
-template <bool VEC>
+template <bool VEC, bool RELU>
 __global__ void __launch_bounds__(TPB) k_bn_fwd_apply(const float* __restrict__ x, float* __restrict__ y, const float* __restrict__ partial,
                                                       const float* gamma, const float* beta, float* run_mean, float* run_var,
                                                       float* save_mean, float* save_invstd, int N, int C, int HW, int n_per, float eps, float factor) {
@@ -106,12 +106,15 @@ __global__ void __launch_bounds__(TPB) k_bn_fwd_apply(const float* __restrict__ 
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 r;
       r.x = (v.x - mean) * invstd * g + b; r.y = (v.y - mean) * invstd * g + b;
       r.z = (v.z - mean) * invstd * g + b; r.w = (v.w - mean) * invstd * g + b;
+      if (RELU) { r.x = r.x < 0.f ? 0.f : r.x; r.y = r.y < 0.f ? 0.f : r.y; r.z = r.z < 0.f ? 0.f : r.z; r.w = r.w < 0.f ? 0.f : r.w; }
       *reinterpret_cast<float4*>(y + off) = r; },
-    [&](int64_t off) { y[off] = (x[off] - mean) * invstd * g + b; });
+    [&](int64_t off) { float r = (x[off] - mean) * invstd * g + b; if (RELU) r = r < 0.f ? 0.f : r; y[off] = r; });
 }
 
-template <bool VEC>
-__global__ void __launch_bounds__(TPB) k_bn_bwd_stats(const float* __restrict__ x, const float* __restrict__ dy, const float* save_mean, const float* save_invstd,
+// RELU: the layer's output y went through an in-place relu; the incoming gradient counts only where y > 0.
+template <bool VEC, bool RELU>
+__global__ void __launch_bounds__(TPB) k_bn_bwd_stats(const float* __restrict__ x, const float* __restrict__ yv, const float* __restrict__ dy,
+                                                      const float* save_mean, const float* save_invstd,
                                                       float* __restrict__ partial, int N, int C, int HW, int n_per) {
   __shared__ float sm[17];
   const int c = blockIdx.x, s = blockIdx.y;
@@ -120,16 +123,18 @@ __global__ void __launch_bounds__(TPB) k_bn_bwd_stats(const float* __restrict__ 
   float s1 = 0.f, s2 = 0.f;
   bn_foreach<VEC>(n0, n1, C, c, HW,
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 g = *reinterpret_cast<const float4*>(dy + off);
+      if (RELU) { float4 m = *reinterpret_cast<const float4*>(yv + off);
+        g.x = m.x > 0.f ? g.x : 0.f; g.y = m.y > 0.f ? g.y : 0.f; g.z = m.z > 0.f ? g.z : 0.f; g.w = m.w > 0.f ? g.w : 0.f; }
       s1 += (g.x + g.y) + (g.z + g.w);
       s2 += (g.x * ((v.x - mean) * is) + g.y * ((v.y - mean) * is)) + (g.z * ((v.z - mean) * is) + g.w * ((v.w - mean) * is)); },
-    [&](int64_t off) { float g = dy[off]; s1 += g; s2 += g * ((x[off] - mean) * is); });
+    [&](int64_t off) { float g = dy[off]; if (RELU) g = yv[off] > 0.f ? g : 0.f; s1 += g; s2 += g * ((x[off] - mean) * is); });
   s1 = lh_block_sum(s1, sm);
   s2 = lh_block_sum(s2, sm);
   if (threadIdx.x == 0) { float* p = partial + 3 * ((int64_t)c * gridDim.y + s); p[0] = s1; p[1] = s2; }
 }
 
-template <bool VEC, bool ACC>
-__global__ void __launch_bounds__(TPB) k_bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ partial,
+template <bool VEC, bool ACC, bool RELU>
+__global__ void __launch_bounds__(TPB) k_bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ yv, const float* __restrict__ dy, const float* __restrict__ partial,
                                                       const float* gamma, const float* save_mean, const float* save_invstd,
                                                       float* __restrict__ dx, float* dgamma, float* dbeta, int N, int C, int HW, int n_per) {
   __shared__ float sh[2];
@@ -147,11 +152,14 @@ __global__ void __launch_bounds__(TPB) k_bn_bwd_apply(const float* __restrict__ 
   const int n0 = s * n_per, n1 = min(N, n0 + n_per);
   bn_foreach<VEC>(n0, n1, C, c, HW,
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 d = *reinterpret_cast<const float4*>(dy + off); float4 r;
+      if (RELU) { float4 m = *reinterpret_cast<const float4*>(yv + off);
+        d.x = m.x > 0.f ? d.x : 0.f; d.y = m.y > 0.f ? d.y : 0.f; d.z = m.z > 0.f ? d.z : 0.f; d.w = m.w > 0.f ? d.w : 0.f; }
       r.x = g * (d.x - m1 - (v.x - mean) * is * m2); r.y = g * (d.y - m1 - (v.y - mean) * is * m2);
       r.z = g * (d.z - m1 - (v.z - mean) * is * m2); r.w = g * (d.w - m1 - (v.w - mean) * is * m2);
       if (ACC) { float4 o = *reinterpret_cast<const float4*>(dx + off); r.x += o.x; r.y += o.y; r.z += o.z; r.w += o.w; }
       *reinterpret_cast<float4*>(dx + off) = r; },
-    [&](int64_t off) { float r = g * (dy[off] - m1 - (x[off] - mean) * is * m2); if (ACC) r += dx[off]; dx[off] = r; });
+    [&](int64_t off) { float d = dy[off]; if (RELU) d = yv[off] > 0.f ? d : 0.f;
+      float r = g * (d - m1 - (x[off] - mean) * is * m2); if (ACC) r += dx[off]; dx[off] = r; });
 }
 
 __global__ void __launch_bounds__(TPB) k_bn_infer(const float* __restrict__ x, float* __restrict__ y, const float* gamma, const float* beta,
@@ -181,46 +189,69 @@ void lh_bn_infer(const float* x, const float* gamma, const float* beta, const fl
   LH_CHECK_LAUNCH();
 }
 
-void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
-                     float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
-  ProfScope prof_(CAT_BN_FWD);
+static void bn_train_fwd_impl(bool relu, const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                              float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_train_fwd: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_train_fwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   if (!get_partial()) return;
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)y) & 15) == 0);
   dim3 grid(C, p.slices);
+#define FWD(V, R) hipLaunchKernelGGL((k_bn_fwd_apply<V, R>), grid, dim3(TPB), 0, g_stream, x, y, (const float*)g_partial_ptr, gamma, beta, run_mean, run_var, \
+                                     save_mean, save_invstd, N, C, HW, p.n_per, eps, factor)
   if (p.vec4) {
     hipLaunchKernelGGL((k_bn_stats<true>), grid, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, HW, p.n_per);
-    hipLaunchKernelGGL((k_bn_fwd_apply<true>), grid, dim3(TPB), 0, g_stream, x, y, (const float*)g_partial_ptr, gamma, beta, run_mean, run_var,
-                       save_mean, save_invstd, N, C, HW, p.n_per, eps, factor);
+    if (relu) FWD(true, true); else FWD(true, false);
   } else {
     hipLaunchKernelGGL((k_bn_stats<false>), grid, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, HW, p.n_per);
-    hipLaunchKernelGGL((k_bn_fwd_apply<false>), grid, dim3(TPB), 0, g_stream, x, y, (const float*)g_partial_ptr, gamma, beta, run_mean, run_var,
-                       save_mean, save_invstd, N, C, HW, p.n_per, eps, factor);
+    if (relu) FWD(false, true); else FWD(false, false);
   }
+#undef FWD
   LH_CHECK_LAUNCH();
 }
 
-void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
-               float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
-  ProfScope prof_(CAT_BN_BWD);
+static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+                        float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_bwd: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_bwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   LH_REQUIRE(beta_dx == 0.0f || beta_dx == 1.0f, "lh_bn_bwd: beta must be 0 or 1");
   if (!get_partial()) return;
-  Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx) & 15) == 0);
+  Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx | (uintptr_t)y_relu) & 15) == 0);
   dim3 grid(C, p.slices);
-  const bool acc = beta_dx != 0.0f;
-#define BWD(V, A) hipLaunchKernelGGL((k_bn_bwd_apply<V, A>), grid, dim3(TPB), 0, g_stream, x, dy, (const float*)g_partial_ptr, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
+  const bool acc = beta_dx != 0.0f, relu = y_relu != nullptr;
+#define STATS(V, R) hipLaunchKernelGGL((k_bn_bwd_stats<V, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per)
+#define APPLY(V, A, R) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, (const float*)g_partial_ptr, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
   if (p.vec4) {
-    hipLaunchKernelGGL((k_bn_bwd_stats<true>), grid, dim3(TPB), 0, g_stream, x, dy, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per);
-    if (acc) BWD(true, true); else BWD(true, false);
+    if (relu) { STATS(true, true); if (acc) APPLY(true, true, true); else APPLY(true, false, true); }
+    else { STATS(true, false); if (acc) APPLY(true, true, false); else APPLY(true, false, false); }
   } else {
-    hipLaunchKernelGGL((k_bn_bwd_stats<false>), grid, dim3(TPB), 0, g_stream, x, dy, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per);
-    if (acc) BWD(false, true); else BWD(false, false);
+    if (relu) { STATS(false, true); if (acc) APPLY(false, true, true); else APPLY(false, false, true); }
+    else { STATS(false, false); if (acc) APPLY(false, true, false); else APPLY(false, false, false); }
   }
-#undef BWD
+#undef STATS
+#undef APPLY
   LH_CHECK_LAUNCH();
+}
+
+void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                     float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
+  ProfScope prof_(CAT_BN_FWD);
+  bn_train_fwd_impl(false, x, gamma, beta, run_mean, run_var, y, save_mean, save_invstd, N, C, HW, eps, factor);
+}
+void lh_bn_train_fwd_relu(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                          float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
+  ProfScope prof_(CAT_BN_FWD);
+  bn_train_fwd_impl(true, x, gamma, beta, run_mean, run_var, y, save_mean, save_invstd, N, C, HW, eps, factor);
+}
+void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+               float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
+  ProfScope prof_(CAT_BN_BWD);
+  bn_bwd_impl(x, nullptr, dy, gamma, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
+}
+void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+                    float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
+  ProfScope prof_(CAT_BN_BWD);
+  LH_REQUIRE(y != nullptr, "lh_bn_bwd_relu: y is required");
+  bn_bwd_impl(x, y, dy, gamma, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
 }
 
 }  // extern "C"

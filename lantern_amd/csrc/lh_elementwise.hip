@@ -143,6 +143,23 @@ void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) { ProfSc
   LH_CHECK_LAUNCH();
 }
 
+void lh_add_relu(const float* a, const float* b, float* out, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+  ew<2>(out, a, b, nullptr, n, [] __device__(float x, float y, float) { float r = x + y; return r < 0.f ? 0.f : r; });
+  LH_CHECK_LAUNCH();
+}
+void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, float* bd, float bbeta, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+  // g = dy where y > 0 else 0 ; ad = abeta*ad + g ; bd = bbeta*bd + g   (either target may be NULL)
+  if (ad) {
+    if (abeta == 0.f) ew<2>(ad, y, dy, nullptr, n, [] __device__(float yv, float g, float) { return yv > 0.f ? g : 0.f; });
+    else ew<3>(ad, ad, y, dy, n, [] __device__(float d, float yv, float g) { return d + (yv > 0.f ? g : 0.f); });
+  }
+  if (bd) {
+    if (bbeta == 0.f) ew<2>(bd, y, dy, nullptr, n, [] __device__(float yv, float g, float) { return yv > 0.f ? g : 0.f; });
+    else ew<3>(bd, bd, y, dy, n, [] __device__(float d, float yv, float g) { return d + (yv > 0.f ? g : 0.f); });
+  }
+  LH_CHECK_LAUNCH();
+}
+
 void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
   ew<2>(out, x, y, nullptr, n, [alpha, beta] __device__(float a, float b, float) { return a * alpha + b * beta; });
   LH_CHECK_LAUNCH();

@@ -27,10 +27,47 @@ def set_backend(b):
     return b
 
 
+# Peephole fusion.  An op whose result is very often consumed by an in-place relu (batchNorm, `+`)
+# does not launch at once: it parks itself here.  If the next op is that relu, one fused kernel
+# runs instead of two; any other op flushes the parked launch first, so program order on the
+# stream is unchanged (at most one launch is ever parked).
+_pending = None
+
+
+class _Pending:
+    def __init__(self, owner, launch):
+        self.owner = owner          # the TensorR whose value is not computed yet
+        self.launch = launch        # launch(relu: bool)
+
+
+def _flush():
+    global _pending
+    if _pending is not None:
+        p, _pending = _pending, None
+        p.launch(False)
+
+
 def get_backend():
     if _backend is None:
         raise RuntimeError("no backend set: call set_backend(BackendHIP(...)) and backend.setup() first")
+    if _pending is not None:
+        _flush()
     return _backend
+
+
+def _park(owner, launch):
+    global _pending
+    _flush()
+    _pending = _Pending(owner, launch)
+
+
+def _take_pending(owner):
+    """The parked launch if it produces `owner`, else None (and nothing is flushed)."""
+    global _pending
+    if _pending is not None and _pending.owner is owner:
+        p, _pending = _pending, None
+        return p
+    return None
 
 
 def _prod(dims):
@@ -438,6 +475,8 @@ class TensorR:
     # -- arithmetic --------------------------------------------------------------------------------
     def _bin(self, op, that):
         be = get_backend()
+        if isinstance(that, TensorR) and op == B.ADD and self.x.shape == that.x.shape and self is not that:
+            return self._add_same_shape(that)
         if isinstance(that, TensorR):
             ya, a, b = self.x._bin(op, that.x)
             y = TensorR._new(ya)
@@ -470,6 +509,36 @@ class TensorR:
     def __sub__(self, t): return self._bin(B.SUB, t)
     def __mul__(self, t): return self._bin(B.MUL, t)
     def __truediv__(self, t): return self._bin(B.DIV, t)
+
+    def _add_same_shape(self, that):
+        """`+` without broadcasting (TD:1171-1176, CPU:299-304), parked so that a following in-place
+        relu fuses with it (the residual join of ResNet)."""
+        be = get_backend()
+        n = self.x.scalarCount
+        ybuf = be.mallocArray(n, zero=False)
+        y = TensorR._new(Tensor(ybuf, self.x.shape))
+        st = {"relu": False}
+
+        def launch(relu):
+            st["relu"] = relu
+            _backend.add_into(self.x.data, that.x.data, ybuf, n, relu)
+        _park(y, launch)
+
+        def back():
+            if st["relu"]:
+                ad, ab = (None, 1.0) if self.isInput else self.grad_target()
+                bd, bb = (None, 1.0) if that.isInput else that.grad_target()
+                be.add_relu_grad(ybuf, y.d.data, ad, ab, bd, bb, n)
+                return
+            for t in (self, that):
+                if t.isInput: continue
+                if t._d is None:            # a fresh gradient buffer is written by a copy, not zero + accumulate
+                    buf, _ = t.grad_target()
+                    be.copyFloatArray(buf, y.d.data, n)
+                else:
+                    be.bcast_update(B.ADD, t.d.data, self.x.shape, y.d.data, self.x.shape)
+        _tape.append(back)
+        return y
 
     def dot(self, that):
         be = get_backend()
@@ -513,6 +582,11 @@ class TensorR:
 
     # -- activations ----------------------------------------------------------------------------------
     def _unary(self, op, inPlace=False, lo=-1.0, hi=1.0):
+        if inPlace and op == B.RELU:
+            p = _take_pending(self)
+            if p is not None:
+                p.launch(True)      # producer + relu in one kernel; its gradient closure applies the mask
+                return self
         be = get_backend()
         if inPlace:
             self.x._unary(op, True, lo, hi)
@@ -557,12 +631,22 @@ class TensorR:
     # -- bn / softmax / loss ----------------------------------------------------------------------------------
     def batchNorm(self, scale, bias, runningMean, runningVar):
         be = get_backend()
-        yv, sm, si = self.x.batchNormTraining(scale.x, bias.x, runningMean, runningVar)
-        y = TensorR._new(yv)
         N, C, HW = self.x._bn_view()
+        n = self.x.scalarCount
+        ybuf = be.mallocArray(n, zero=False)
+        sm, si = be.mallocArray(C, zero=False), be.mallocArray(C, zero=False)
+        y = TensorR._new(Tensor(ybuf, self.x.shape))
+        st = {"relu": False}
+
+        def launch(relu):
+            st["relu"] = relu
+            _backend.batchNormTraining_into(self.x.data, scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, N, C, HW, relu)
+        _park(y, launch)
+
         def back():
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()
-            be.batchNorm_grad(self.x.data, xd, y.d.data, scale.x.data, scale.d.data, bias.d.data, sm.data, si.data, N, C, HW, beta)
+            be.batchNorm_grad(self.x.data, xd, y.d.data, scale.x.data, scale.d.data, bias.d.data, sm, si, N, C, HW, beta,
+                              y_relu=ybuf if st["relu"] else None)
         _tape.append(back)
         return y
 

@@ -198,7 +198,9 @@ class BackendCPU(Backend):
                 I(N), I(C_), I(HW), F(eps), F(factor))
         return y, sm, si
 
-    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C_, HW, beta_dx=1.0):
+    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C_, HW, beta_dx=1.0, y_relu=None):
+        if y_relu is not None:      # the unfused sequence: relu_grad(inPlace) on dy, then batchNorm_grad
+            self.unary_grad(0, y_relu, y_relu, dy, dy, N * C_ * HW, inPlace=True)
         self._c("lc_bn_bwd", P(x.ptr), P(dy.ptr), P(scale.ptr), P(sm.ptr), P(si.ptr), P(xd.ptr if xd is not None else 0),
                 P(scaled.ptr), P(biasd.ptr), I(N), I(C_), I(HW))
 
