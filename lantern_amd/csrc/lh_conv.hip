@@ -185,11 +185,13 @@ struct EpiConvOut {
     c.off = (int)n * chan * PIX + (aH + eH * (int)u) * W + aW + eW * (int)v;
     return c;
   }
-  __device__ __forceinline__ void store(const Col& c, int i, int M, float v) const {
+  // part: 0 = complete sum; 1 = first partial, 2 = later partial (atomic adds onto a prepared output)
+  __device__ __forceinline__ void store(const Col& c, int i, int M, float v, int part) const {
     if (!c.valid || i >= M) return;
     float* p = out + c.off + i * PIX;
-    if (bias) v += bias[i];
-    *p = beta == 0.f ? v : v + beta * *p;
+    if (bias && part < 2) v += bias[i];
+    if (part) atomicAdd(p, v);
+    else *p = beta == 0.f ? v : v + beta * *p;
   }
 };
 static EpiConvOut make_epi(float* out, const float* bias, int chan, int Himg, int Wimg, float beta) {   // dense: grid == image
@@ -238,8 +240,26 @@ __global__ void __launch_bounds__(TPB) k_conv_bwd_bias(const float* __restrict__
 #define LH_CONV_BK 16
 #endif
 constexpr int CONV_BK = LH_CONV_BK;      // k-slab of the forward / input-gradient kernels
+#ifndef LH_BWDF_BK
+#define LH_BWDF_BK 32
+#endif
+constexpr int BWDF_BK = LH_BWDF_BK;      // k-slab of the filter-gradient kernel
+// Forward / input-gradient launch.  A grid with few tiles per CU leaves CUs idle in its last wave
+// of blocks; such shapes run stream-K instead (largest tile, two workers per CU, every worker the
+// same number of k-slabs).  `zero_out`/`zero_n`: the output to clear first when the epilogue
+// overwrites (beta = 0), because shared tiles are completed with atomic adds.
 template <class AL, class BL, class EP>
-static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K) {
+static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out = nullptr, int64_t zero_n = 0, bool prezeroed = false) {
+  const int64_t t128 = cdiv(M, 128) * cdiv(N, 128), t64 = cdiv(M, 64) * cdiv(N, 128);
+  const int workers = 2 * g_num_cu;
+  const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
+  const int64_t slabs = cdiv(K, CONV_BK);
+  // long reductions only: a worker's share must span many slabs for the per-segment set-up to pay off
+  if (few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)workers && (ep.beta == 1.f || zero_out != nullptr || prezeroed)) {
+    if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
+    if (M > 64) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
+    return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
+  }
   TilePick tp = pick_tile(M, N);
   if (tp.bm == 128) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1);
   if (tp.bn == 128) return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1);
@@ -273,7 +293,7 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
     LoadPlainK<true> al; al.base = wk; al.nbytes = wbytes; al.ld = CRS;
     LoadConvFwdTapB bl; bl.base = x; bl.nbytes = xbytes; bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
     bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dC.init(C); bl.dS.init(S);
-    ok = launch_tiles(al, bl, ep, K, N * PQ, CRS);
+    ok = launch_tiles(al, bl, ep, K, N * PQ, CRS, y, (int64_t)N * K * PQ);
     if (scratch) lh_free_top(scratch);
   } else {
     const bool avec = (CRS % 4 == 0) && (((uintptr_t)w & 15) == 0);
@@ -303,7 +323,12 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
       int r0 = (aH + pH) % sH, s0 = (aW + pW) % sW;
       if (r0 >= R || s0 >= S || aH >= H || aW >= W) any_empty = true;
     }
-    if (beta == 0.f && any_empty) lh_fill(dx, 0.f, (int64_t)N * C * HW);
+    // several classes (or an empty one) with beta = 0: clear dx once, then every class may overwrite or add
+    const bool strided = sH * sW > 1;
+    if (beta == 0.f && (any_empty || strided)) lh_fill(dx, 0.f, (int64_t)N * C * HW);
+    float* zo = (beta == 0.f && !strided) ? dx : nullptr;
+    const int64_t zn = (int64_t)N * C * HW;
+    const bool pz = beta == 0.f && strided;
     for (int aH = 0; aH < sH && ok; aH++) for (int aW = 0; aW < sW && ok; aW++) {
       const int r0 = (aH + pH) % sH, s0 = (aW + pW) % sW;
       if (r0 >= R || s0 >= S || aH >= H || aW >= W) continue;
@@ -317,7 +342,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
       ep.dPIXc.init(Hc * Wc); ep.dWc.init(Wc);
       if (RS == 1) {
         LoadPlainT al; al.base = w; al.nbytes = (uint32_t)((size_t)K * C * 4); al.ld = C;          // A[c][k] = w[k][c]
-        ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred);
+        ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred, zo, zn, pz);
       } else {
         size_t bytes = (size_t)Kred * C * sizeof(float);
         float* wt = (float*)lh_malloc_uninit(bytes);     // released below: stream order keeps it safe
@@ -325,7 +350,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
         int64_t n = (int64_t)Kred * C;
         hipLaunchKernelGGL(k_filter_to_ctk, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, R, S, r0, s0, sH, sW, Rc, Sc, n);
         LoadPlainK<true> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = Kred;
-        ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred);
+        ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred, zo, zn, pz);
         lh_free_top(bytes);
       }
     }
@@ -377,9 +402,9 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
     bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * H * W * 4); bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.CHW = C * H * W;
     bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
-    if (tp.bm == 128) ok = igemm_launch<128, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
-    else if (tp.bn == 128) ok = igemm_launch<64, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
-    else ok = igemm_launch<64, 64, 32>(al, bl, ep, K, CRS, (int)red, split);
+    if (tp.bm == 128) ok = igemm_launch<128, 128, 16>(al, bl, ep, K, CRS, (int)red, split);    // measured: the large tile prefers the short slab
+    else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
+    else ok = igemm_launch<64, 64, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
   };
   if (avec && rowvec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<true>());
   else if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<false>());

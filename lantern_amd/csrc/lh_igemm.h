@@ -39,7 +39,10 @@ struct FastDiv {
 struct GemmShape {
   int M, N, K;
   int tilesM, tilesN, splitK, kPerSplit;
-  int total, perXcd;
+  int total, perXcd;          // work items (tiles x k-splits, or stream-K workers) and items per XCD
+  int streamk;                // != 0: `total` workers share tiles*slabsPerTile k-slabs evenly
+  int slabsPerTile;
+  long long units;            // tiles * slabsPerTile
 };
 
 // ---- operand loaders ---------------------------------------------------------------------------
@@ -101,16 +104,18 @@ struct EpiRowMajor {
   float* C; int ldc; float alpha, beta; int atomic;
   struct Col { int j; bool valid; };
   __device__ __forceinline__ Col col(int j, int N) const { Col c; c.j = j; c.valid = j < N; return c; }
-  __device__ __forceinline__ void store(const Col& c, int i, int M, float v) const {
+  // part: 0 = the whole reduction of this element is in v; 1 = first partial sum, 2 = a later one
+  // (partials are combined with atomic adds onto an output the host has prepared)
+  __device__ __forceinline__ void store(const Col& c, int i, int M, float v, int part) const {
     if (!c.valid || i >= M) return;
     float* p = C + (int64_t)i * ldc + c.j;
-    if (atomic) atomicAdd(p, alpha * v);
+    if (atomic || part) atomicAdd(p, alpha * v);
     else *p = alpha * v + (beta == 0.f ? 0.f : beta * *p);
   }
 };
 
 // ---- the kernel ------------------------------------------------------------------------------------
-template <int BM, int BN, int BK, class AL, class BL, class EP>
+template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
 __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const EP ep, const GemmShape gs) {
   constexpr int KQ = BK / 4, PAD = 8 / KQ, LDA = BM + PAD, LDB = BN + PAD;
   constexpr int TM = BM / 2, TN = BN / 2, MI = TM / 32, NI = TN / 32;
@@ -122,30 +127,53 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
 
   const int logical = (blockIdx.x % 8) * gs.perXcd + blockIdx.x / 8;
   if (logical >= gs.total) return;
-  const int tm = logical % gs.tilesM;
-  const int rest = logical / gs.tilesM;
-  const int tn = rest % gs.tilesN, sp = rest / gs.tilesN;
-  const int m0 = tm * BM, n0 = tn * BN;
-  const int kbeg = sp * gs.kPerSplit, kend = min(gs.K, kbeg + gs.kPerSplit);
-
+  // Work of this block: either one (tile, k-split) item, or -- stream-K -- an equal share of all
+  // k-slabs of all tiles, walked tile by tile; a tile whose slabs are shared between two blocks
+  // is completed with atomic adds.
+  long long u = 0, u_end = 1;
+  if (SK) { u = gs.units * logical / gs.total; u_end = gs.units * (logical + 1) / gs.total; }
   const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc((void*)al.base, 0, (int)al.nbytes, LH_RSRC_FLAGS);
   const __amdgpu_buffer_rsrc_t rsB = __builtin_amdgcn_make_buffer_rsrc((void*)bl.base, 0, (int)bl.nbytes, LH_RSRC_FLAGS);
   const int t = threadIdx.x;
-  typename AL::State sa[GA];
-  typename BL::State sb[GB];
   int a_col[GA], a_kq[GA], b_col[GB], b_kq[GB];
 #pragma unroll
   for (int g = 0; g < GA; g++) {
     if (AL::ALONG_K) { a_kq[g] = t % KQ; a_col[g] = t / KQ + g * (256 / KQ); }
     else { a_col[g] = t % BM; a_kq[g] = __builtin_amdgcn_readfirstlane(t / BM) + g * (256 / BM); }
-    al.init(sa[g], m0 + a_col[g], gs.M);
   }
 #pragma unroll
   for (int g = 0; g < GB; g++) {
     if (BL::ALONG_K) { b_kq[g] = t % KQ; b_col[g] = t / KQ + g * (256 / KQ); }
     else { b_col[g] = t % BN; b_kq[g] = __builtin_amdgcn_readfirstlane(t / BN) + g * (256 / BN); }
-    bl.init(sb[g], n0 + b_col[g], gs.N);
   }
+  const int lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
+
+  while (u < u_end) {
+  int tm, tn, kbeg, kend, part = 0;
+  if (SK) {
+    const int tile = (int)(u / gs.slabsPerTile), s0 = (int)(u - (long long)tile * gs.slabsPerTile);
+    const long long left = u_end - u;
+    const int s1 = (int)(left < (long long)(gs.slabsPerTile - s0) ? s0 + left : gs.slabsPerTile);
+    tm = tile % gs.tilesM; tn = tile / gs.tilesM;
+    kbeg = s0 * BK; kend = min(gs.K, s1 * BK);
+    part = (s0 == 0 && s1 == gs.slabsPerTile) ? 0 : (s0 == 0 ? 1 : 2);
+    u += s1 - s0;
+    __syncthreads();            // LDS of the previous segment is free again
+  } else {
+    tm = logical % gs.tilesM;
+    const int rest = logical / gs.tilesM;
+    tn = rest % gs.tilesN;
+    const int sp = rest / gs.tilesN;
+    kbeg = sp * gs.kPerSplit; kend = min(gs.K, kbeg + gs.kPerSplit);
+    u = u_end;
+  }
+  const int m0 = tm * BM, n0 = tn * BN;
+  typename AL::State sa[GA];
+  typename BL::State sb[GB];
+#pragma unroll
+  for (int g = 0; g < GA; g++) al.init(sa[g], m0 + a_col[g], gs.M);
+#pragma unroll
+  for (int g = 0; g < GB; g++) bl.init(sb[g], n0 + b_col[g], gs.N);
 
   f32x16 acc[MI][NI];
 #pragma unroll
@@ -155,7 +183,6 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[mi][ni][v] = 0.f;
 
-  const int lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
   const int niter = (kend - kbeg + BK - 1) / BK;
   constexpr int EA = AL::VEC4 ? 1 : 4, EB = BL::VEC4 ? 1 : 4;
   constexpr int NEL = GA * EA + GB * EB;            // offsets to compute per slab and thread
@@ -243,17 +270,22 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
     for (int mi = 0; mi < MI; mi++) {
       const int ib = m0 + wm * TM + mi * 32 + 4 * half;
 #pragma unroll
-      for (int v = 0; v < 16; v++) ep.store(cs, ib + 8 * (v / 4) + (v % 4), gs.M, acc[mi][ni][v]);
+      for (int v = 0; v < 16; v++) ep.store(cs, ib + 8 * (v / 4) + (v % 4), gs.M, acc[mi][ni][v], part);
     }
   }
+  }  // segments
 }
 
 template <int BM, int BN, int BK>
 constexpr size_t igemm_smem_bytes() { return (size_t)2 * (BK / 4) * ((BM + 8 / (BK / 4)) + (BN + 8 / (BK / 4))) * sizeof(float4); }
 
-// Launch one tile configuration.  splitK > 1 requires an accumulating (atomic) epilogue.
+// Launch one tile configuration.
+//   splitK > 1 : the reduction is cut into splitK pieces per tile (needs an accumulating epilogue).
+//   streamk    : `streamk` workers (about two per CU) share all k-slabs of all tiles evenly, which
+//                removes the idle tail of a grid with few tiles; tiles shared by two workers are
+//                finished with atomic adds, so the caller must have the output hold beta*C.
 template <int BM, int BN, int BK, class AL, class BL, class EP>
-bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, int splitK) {
+bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, int splitK, int streamk = 0) {
   GemmShape gs;
   gs.M = M; gs.N = N; gs.K = K;
   gs.tilesM = (int)cdiv(M, BM); gs.tilesN = (int)cdiv(N, BN);
@@ -262,11 +294,24 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
   if (kper < BK) kper = BK;
   gs.kPerSplit = kper;
   gs.splitK = (int)cdiv(K > 0 ? K : 1, kper);
+  gs.slabsPerTile = (int)cdiv(K > 0 ? K : 1, BK);
+  gs.units = (long long)gs.tilesM * gs.tilesN * gs.slabsPerTile;
+  gs.streamk = 0;
   int64_t total = (int64_t)gs.tilesM * gs.tilesN * gs.splitK;
+  if (streamk > 0) {
+    gs.streamk = 1;
+    total = streamk < gs.units ? streamk : gs.units;
+  }
   if (total <= 0 || total > 0x3fffffff) { LH_FAIL("igemm: tile count %lld out of range", (long long)total); return false; }
   gs.total = (int)total; gs.perXcd = (int)cdiv(total, 8);
   constexpr size_t smem = igemm_smem_bytes<BM, BN, BK>();
-  auto kern = k_igemm<BM, BN, BK, AL, BL, EP>;
+  if (gs.streamk) {
+    if constexpr (smem <= 48 * 1024) {   // stream-K is instantiated for the forward / input-gradient tiles only
+      hipLaunchKernelGGL((k_igemm<BM, BN, BK, AL, BL, EP, true>), dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
+      return true;
+    } else { LH_FAIL("igemm: stream-K is not built for this tile"); return false; }
+  }
+  auto kern = k_igemm<BM, BN, BK, AL, BL, EP, false>;
   static bool attr_done = false;
   if (smem > 48 * 1024 && !attr_done) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
