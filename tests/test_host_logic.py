@@ -1,0 +1,96 @@
+"""Host-side logic that needs no GPU: shape rules, the tape, lazy gradient buffers and the
+relu peephole (run on the CPU oracle backend)."""
+import numpy as np
+import pytest
+
+import lantern_amd as la
+from lantern_amd import Tensor, TensorR, gradR, gradR_loss
+from lantern_amd.backend import dim_broadcast, conv_size
+from lantern_amd.tensor import resize_dim
+import lantern_amd.tensor as T
+
+
+def test_dim_broadcast():  # T/TestBroadcast.scala:14-46 (dimBroadcast cases)
+    assert dim_broadcast((2, 3), (2, 3)) == ((2, 3), (2, 3), (2, 3))
+    assert dim_broadcast((2, 3), (1, 3)) == ((2, 3), (1, 3), (2, 3))
+    assert dim_broadcast((2, 2, 2), (2,)) == ((2, 2, 2), (1, 1, 2), (2, 2, 2))
+    assert dim_broadcast((3,), (4, 1)) == ((1, 3), (4, 1), (4, 3))
+    with pytest.raises(ValueError):
+        dim_broadcast((2, 3), (2, 3, 3)[1:] + (2,))
+
+
+def test_resize_dim_and_conv_size():  # TD:34-49
+    assert resize_dim(320 * 100, (-1, 320)) == (100, 320)
+    assert resize_dim(24, (2, 3, 4)) == (2, 3, 4)
+    with pytest.raises(ValueError):
+        resize_dim(24, (-1, -1))
+    with pytest.raises(ValueError):
+        resize_dim(24, (5, 5))
+    assert conv_size(28, 5, 1) == 24 and conv_size(224, 7, 2, 3) == 112 and conv_size(112, 3, 2, 1) == 56
+
+
+def test_gradients_accumulate_across_uses(on_cpu):
+    # x used twice: d = dL/dx summed over both uses (TD accumulates into d)
+    x = TensorR(Tensor.fromData((3,), 1, 2, 3))
+    gradR_loss(lambda d: (x * x).sum())(Tensor.zeros(1))
+    np.testing.assert_allclose(x.d.toCPU(), [2, 4, 6])
+    gradR_loss(lambda d: (x * 3.0).sum())(Tensor.zeros(1))
+    np.testing.assert_allclose(x.d.toCPU(), [5, 7, 9])         # accumulated on top
+
+
+def test_input_gets_no_gradient(on_cpu):  # TD:1510: inputs carry a 2-element dummy d
+    x = TensorR(Tensor.ones(1, 1, 4, 4), isInput=True)
+    k = TensorR(Tensor.ones(1, 1, 3, 3))
+    gradR_loss(lambda d: x.convBBP(k, None, (1, 1), (0, 0)).sum())(Tensor.zeros(1))
+    assert x.d.scalarCount == 2 and (x.d.toCPU() == 0).all()
+    np.testing.assert_allclose(k.d.toCPU().ravel(), [4] * 9)
+
+
+def test_lazy_gradient_buffer_matches_eager(on_cpu):
+    rng = np.random.RandomState(0)
+    a, b = rng.randn(2, 3, 4, 4).astype(np.float32), rng.randn(2, 3, 4, 4).astype(np.float32)
+
+    def run():
+        x, y = TensorR(Tensor.fromNumpy(a)), TensorR(Tensor.fromNumpy(b))
+        gradR_loss(lambda d: ((x + y).relu(True) + x).sum())(Tensor.zeros(1))
+        return x.d.toCPU(), y.d.toCPU()
+    gx, gy = run()
+    mask = (a + b) > 0
+    np.testing.assert_allclose(gx, mask + 1.0)
+    np.testing.assert_allclose(gy, mask * 1.0)
+
+
+def test_parked_launch_is_flushed_by_any_other_op(on_cpu):
+    """batchNorm parks its launch so a following in-place relu can fuse; anything else must see
+    the finished value."""
+    rng = np.random.RandomState(1)
+    x = TensorR(Tensor.fromNumpy(rng.randn(4, 2, 3, 3).astype(np.float32)))
+    g, b = TensorR(Tensor.ones(2)), TensorR(Tensor.zeros(2))
+    y = x.batchNorm(g, b, Tensor.zeros(2), Tensor.ones(2))
+    assert T._pending is not None and T._pending.owner is y
+    v = y.x.toCPU()                       # toCPU goes through get_backend(): flushes
+    assert T._pending is None
+    xs = x.x.toCPU()
+    ref = (xs - xs.mean(axis=(0, 2, 3), keepdims=True)) / np.sqrt(xs.var(axis=(0, 2, 3), keepdims=True) + 1e-5)
+    np.testing.assert_allclose(v, ref, rtol=1e-4, atol=1e-5)
+    y2 = x.batchNorm(g, b, Tensor.zeros(2), Tensor.ones(2)).relu(True)      # fused path
+    assert T._pending is None
+    np.testing.assert_allclose(y2.x.toCPU(), np.maximum(ref, 0), rtol=1e-4, atol=1e-5)
+    T._tape.clear()
+
+
+def test_fused_and_unfused_relu_gradients_agree(on_cpu):
+    rng = np.random.RandomState(2)
+    xs = rng.randn(4, 3, 5, 5).astype(np.float32)
+
+    def run(fused):
+        x = TensorR(Tensor.fromNumpy(xs)); g = TensorR(Tensor.fromData((3,), 1.5, 0.5, 2.0)); b = TensorR(Tensor.fromData((3,), 0.1, -0.2, 0.0))
+        def f(d):
+            y = x.batchNorm(g, b, Tensor.zeros(3), Tensor.ones(3))
+            if not fused:
+                y.x.toCPU()                 # forces the unfused launch before relu
+            return (y.relu(True) * 2.0).sum()
+        gradR_loss(f)(Tensor.zeros(1))
+        return x.d.toCPU(), g.d.toCPU(), b.d.toCPU()
+    for u, v in zip(run(True), run(False)):
+        np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)

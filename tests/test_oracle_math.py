@@ -1,0 +1,216 @@
+"""Pins the parts of the CPU oracle that the reference's own unit-test vectors leave open
+(tests/test_reference_vectors.py covers the rest): closed forms, brute force on tiny inputs,
+central-difference gradient checks in double, and library routines (torch on the CPU) used as
+an independent textbook implementation at real layer shapes.  A dropped term, a wrong sign, a
+transposed operand or an off-by-one in the oracle fails one of these."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle.backend_cpu import load
+from tests.util import cptr
+
+lc = load()
+I, F, L = C.c_int, C.c_float, C.c_long
+
+
+def conv_ref(x, w, b, sH, sW, pH, pW):
+    """7-loop definition in float64."""
+    N, Cc, H, W = x.shape; K, _, R, S = w.shape
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    y = np.zeros((N, K, P, Q))
+    for n in range(N):
+        for k in range(K):
+            for p in range(P):
+                for q in range(Q):
+                    acc = 0.0 if b is None else float(b[k])
+                    for c in range(Cc):
+                        for r in range(R):
+                            for s in range(S):
+                                h, ww = p * sH - pH + r, q * sW - pW + s
+                                if 0 <= h < H and 0 <= ww < W:
+                                    acc += float(x[n, c, h, ww]) * float(w[k, c, r, s])
+                    y[n, k, p, q] = acc
+    return y
+
+
+def oracle_conv(x, w, b, dims, dy=None):
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    y = np.zeros((N, K, P, Q), np.float32); fin = np.zeros((N, Cc * R * S, P * Q), np.float32)
+    ints = [I(v) for v in dims]
+    lc.lc_conv2d_fwd(cptr(x), cptr(w), cptr(b) if b is not None else None, cptr(y), cptr(fin), *ints)
+    if dy is None:
+        return y
+    dx = np.zeros_like(x); dw = np.zeros_like(w); db = np.zeros(K, np.float32); sc = np.zeros_like(fin)
+    lc.lc_conv2d_bwd(cptr(fin), cptr(w), cptr(dy), cptr(dx), cptr(dw), cptr(db), cptr(sc), *ints)
+    return y, dx, dw, db
+
+
+@pytest.mark.parametrize("dims", [(2, 3, 5, 7, 4, 3, 3, 1, 1, 1, 1), (1, 2, 7, 6, 3, 3, 2, 2, 1, 1, 0), (2, 1, 6, 6, 2, 1, 1, 2, 2, 0, 0),
+                                  (1, 2, 9, 5, 2, 5, 3, 2, 1, 2, 1)])
+def test_conv_forward_against_definition_nonsquare(dims):
+    """Non-square outputs included: the reference's im2col mis-addresses them (CPU:491, outputWidth
+    squared); the oracle follows the mathematical definition."""
+    rng = np.random.RandomState(1)
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    x = rng.randn(N, Cc, H, W).astype(np.float32); w = rng.randn(K, Cc, R, S).astype(np.float32); b = rng.randn(K).astype(np.float32)
+    np.testing.assert_allclose(oracle_conv(x, w, b, dims), conv_ref(x, w, b, sH, sW, pH, pW), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(oracle_conv(x, w, None, dims), conv_ref(x, w, None, sH, sW, pH, pW), rtol=1e-5, atol=1e-5)
+
+
+def test_conv_gradients_by_central_differences():
+    rng = np.random.RandomState(2)
+    dims = (2, 2, 5, 6, 3, 3, 2, 2, 1, 1, 0)
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    x = rng.randn(N, Cc, H, W).astype(np.float32); w = rng.randn(K, Cc, R, S).astype(np.float32); b = rng.randn(K).astype(np.float32)
+    y0 = conv_ref(x, w, b, sH, sW, pH, pW)
+    dy = rng.randn(*y0.shape).astype(np.float32)
+    _, dx, dw, db = oracle_conv(x, w, b, dims, dy)
+    loss = lambda xx, ww, bb: float((conv_ref(xx, ww, bb, sH, sW, pH, pW) * dy).sum())
+    eps = 1e-3
+    for arr, grad in ((x, dx), (w, dw), (b, db)):
+        flat = arr.reshape(-1); g = grad.reshape(-1)
+        for i in rng.choice(flat.size, size=min(12, flat.size), replace=False):
+            old = flat[i]
+            flat[i] = old + eps; lp = loss(x, w, b)
+            flat[i] = old - eps; lm = loss(x, w, b)
+            flat[i] = old
+            assert abs((lp - lm) / (2 * eps) - g[i]) < 2e-2 * max(1.0, abs(g[i])), (i, (lp - lm) / (2 * eps), g[i])
+
+
+def test_conv_pool_bn_against_torch_at_layer_shapes():
+    torch = pytest.importorskip("torch")
+    import torch.nn.functional as Fn
+    rng = np.random.RandomState(3)
+    for dims in [(2, 64, 14, 14, 64, 3, 3, 1, 1, 1, 1), (2, 32, 15, 15, 48, 3, 3, 2, 2, 1, 1), (2, 3, 32, 32, 16, 7, 7, 2, 2, 3, 3), (2, 64, 8, 8, 128, 1, 1, 2, 2, 0, 0)]:
+        N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+        x = rng.randn(N, Cc, H, W).astype(np.float32); w = (rng.randn(K, Cc, R, S) / 8).astype(np.float32)
+        tx = torch.tensor(x, requires_grad=True); tw = torch.tensor(w, requires_grad=True)
+        ty = Fn.conv2d(tx, tw, None, (sH, sW), (pH, pW))
+        dy = rng.randn(*ty.shape).astype(np.float32)
+        ty.backward(torch.tensor(dy))
+        y, dx, dw, _ = oracle_conv(x, w, None, dims, dy)
+        np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-4, atol=1e-4)
+        np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-4, atol=1e-4)
+        np.testing.assert_allclose(dw, tw.grad.numpy(), rtol=1e-3, atol=1e-3)
+    # max pool with padding: values and the argmax as a global flat index, first maximum wins
+    x = rng.randn(3, 4, 9, 9).astype(np.float32)
+    y = np.zeros((3, 4, 5, 5), np.float32); idx = np.zeros((3, 4, 5, 5), np.int32)
+    lc.lc_maxpool_fwd(cptr(x), cptr(y), cptr(idx), I(3), I(4), I(9), I(9), I(3), I(3), I(2), I(2), I(1))
+    ty, tidx = Fn.max_pool2d(torch.tensor(x), 3, 2, 1, return_indices=True)
+    np.testing.assert_array_equal(y, ty.numpy())
+    base = (np.arange(12) * 81).reshape(3, 4, 1, 1)
+    np.testing.assert_array_equal(idx, tidx.numpy() + base)
+    # batch norm (training) forward/backward, running statistics with the unbiased variance
+    x = (rng.randn(4, 6, 5, 5) * 2 + 1).astype(np.float32); g = rng.rand(6).astype(np.float32) + 0.5; b = rng.randn(6).astype(np.float32)
+    rm = np.zeros(6, np.float32); rv = np.ones(6, np.float32)
+    y = np.zeros_like(x); sm = np.zeros(6, np.float32); si = np.zeros(6, np.float32)
+    lc.lc_bn_train_fwd(cptr(x), cptr(g), cptr(b), cptr(rm), cptr(rv), cptr(y), cptr(sm), cptr(si), I(4), I(6), I(25), F(1e-5), F(0.1))
+    tx = torch.tensor(x, requires_grad=True); tg = torch.tensor(g, requires_grad=True); tb = torch.tensor(b, requires_grad=True)
+    trm = torch.zeros(6); trv = torch.ones(6)
+    ty = Fn.batch_norm(tx, trm, trv, tg, tb, True, 0.1, 1e-5)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(rm, trm.numpy(), rtol=1e-5, atol=1e-6); np.testing.assert_allclose(rv, trv.numpy(), rtol=1e-5, atol=1e-6)
+    dy = rng.randn(*x.shape).astype(np.float32)
+    ty.backward(torch.tensor(dy))
+    dx = np.zeros_like(x); dg = np.zeros(6, np.float32); db = np.zeros(6, np.float32)
+    lc.lc_bn_bwd(cptr(x), cptr(dy), cptr(g), cptr(sm), cptr(si), cptr(dx), cptr(dg), cptr(db), I(4), I(6), I(25))
+    np.testing.assert_allclose(dx, tx.grad.numpy(), rtol=1e-3, atol=1e-5)
+    np.testing.assert_allclose(dg, tg.grad.numpy(), rtol=1e-4, atol=1e-4); np.testing.assert_allclose(db, tb.grad.numpy(), rtol=1e-4, atol=1e-4)
+
+
+def test_softmax_invariants_and_gradient():
+    rng = np.random.RandomState(4)
+    x = (rng.randn(5, 7) * 3).astype(np.float32)
+    y = np.zeros_like(x); ly = np.zeros_like(x)
+    lc.lc_softmax(I(0), cptr(x), cptr(y), I(5), I(7)); lc.lc_softmax(I(1), cptr(x), cptr(ly), I(5), I(7))
+    np.testing.assert_allclose(y.sum(1), 1.0, rtol=1e-6)
+    np.testing.assert_allclose(np.exp(ly), y, rtol=1e-5)
+    x64 = x.astype(np.float64); e = np.exp(x64 - x64.max(1, keepdims=True)); ref = e / e.sum(1, keepdims=True)
+    np.testing.assert_allclose(y, ref, rtol=1e-5)
+    dy = rng.randn(5, 7).astype(np.float32)
+    dx = np.zeros_like(x)
+    lc.lc_softmax_grad(I(0), cptr(y), cptr(dy), cptr(dx), I(5), I(7))
+    jac = ref * (dy - (dy * ref).sum(1, keepdims=True))     # J^T dy for softmax
+    np.testing.assert_allclose(dx, jac, rtol=1e-4, atol=1e-6)
+    # [outer, c, inner] view equals the transposed 2-D problem
+    x3 = rng.randn(2, 4, 3).astype(np.float32); y3 = np.zeros_like(x3)
+    lc.lc_softmax3(I(0), cptr(x3), cptr(y3), I(2), I(4), I(3))
+    e3 = np.exp(x3 - x3.max(1, keepdims=True)); np.testing.assert_allclose(y3, e3 / e3.sum(1, keepdims=True), rtol=1e-5)
+
+
+def test_optimizer_recurrences():
+    """SGD (NN:265-287), momentum (CPU:1232-1246) and Adagrad (CPU:1217-1230) against the recurrences in double."""
+    rng = np.random.RandomState(5)
+    n = 33
+    x0 = rng.randn(n).astype(np.float32)
+    for nesterov in (0, 1):
+        x = x0.copy(); v = np.zeros(n, np.float32); xr = x0.astype(np.float64); vr = np.zeros(n)
+        for step in range(4):
+            g = (rng.randn(n) * 300).astype(np.float32)          # some beyond the clip of 400
+            d = g.copy()
+            lc.lc_momentum(cptr(x), cptr(d), cptr(v), F(0.1), F(0.9), F(400.0), I(nesterov), L(n))
+            assert (d == 0).all()
+            gc = np.clip(g.astype(np.float64), -400, 400)
+            vr = 0.9 * vr + gc
+            xr -= 0.1 * ((gc + 0.9 * vr) if nesterov else vr)
+            np.testing.assert_allclose(x, xr, rtol=1e-5, atol=1e-4)
+    x = x0.copy(); m = np.zeros(n, np.float32); xr = x0.astype(np.float64); mr = np.zeros(n)
+    for step in range(4):
+        g = (rng.randn(n) * 2).astype(np.float32); d = g.copy()
+        lc.lc_adagrad(cptr(x), cptr(d), cptr(m), F(0.05), F(1.0), L(n))
+        gc = np.clip(g.astype(np.float64), -1, 1); mr += gc * gc; xr -= 0.05 * gc / np.sqrt(mr + 1e-8)
+        np.testing.assert_allclose(x, xr, rtol=1e-5, atol=1e-6); assert (d == 0).all()
+    x = x0.copy(); d = np.ones(n, np.float32)
+    lc.lc_sgd(cptr(x), cptr(d), F(0.5), L(n))
+    np.testing.assert_allclose(x, x0 - 0.5, rtol=1e-6); assert (d == 0).all()
+
+
+def test_sgemm_all_cases_and_ragged_sizes():
+    rng = np.random.RandomState(6)
+    for (ta, tb, m, n, k) in [(0, 0, 7, 5, 3), (0, 1, 13, 17, 300), (1, 0, 6, 16, 257), (1, 1, 97, 33, 65), (0, 0, 1, 1, 1), (0, 0, 100, 2100, 40)]:
+        A = rng.randn(*((k, m) if ta else (m, k))).astype(np.float32); B = rng.randn(*((n, k) if tb else (k, n))).astype(np.float32)
+        Cm = rng.randn(m, n).astype(np.float32); ref = 0.5 * ((A.T if ta else A).astype(np.float64) @ (B.T if tb else B)) + 2.0 * Cm
+        lc.lc_sgemm(I(ta), I(tb), I(m), I(n), I(k), F(0.5), cptr(A), I(A.shape[1]), cptr(B), I(B.shape[1]), F(2.0), cptr(Cm), I(n))
+        np.testing.assert_allclose(Cm, ref, rtol=1e-4, atol=1e-4)
+
+
+def test_dropout_counter_generator_and_glibc_order():
+    n = 20000
+    x = np.ones(n, np.float32); y = np.zeros(n, np.float32); m = np.zeros(n, np.float32)
+    lc.lc_dropout_ctr(cptr(x), cptr(y), cptr(m), L(n), F(0.5), C.c_uint64(42), C.c_uint64(0))
+    keep = (m > 0).mean()
+    assert abs(keep - 0.5) < 0.02 and set(np.unique(m)) == {0.0, 2.0} and (y == m).all()
+    y2 = np.zeros(n, np.float32); m2 = np.zeros(n, np.float32)
+    lc.lc_dropout_ctr(cptr(x), cptr(y2), cptr(m2), L(n // 2), F(0.5), C.c_uint64(42), C.c_uint64(n // 2))
+    np.testing.assert_array_equal(m2[:n // 2], m[n // 2:])           # keyed by (seed, offset + index)
+    lc.lc_srand(C.c_uint(42))
+    r = np.zeros(8, np.float32); lc.lc_rand_uniform(cptr(r), L(8))
+    lc.lc_srand(C.c_uint(42))
+    lc.lc_dropout_rand(cptr(x), cptr(y), cptr(m), L(8), F(0.5))
+    np.testing.assert_array_equal(m[:8] > 0, (r + 0.5) > 0.5)        # same glibc sequence, keep iff rand > p (CPU:1075)
+
+
+def test_ctc_against_torch():
+    """lc_ctc_loss has no asserted vector in the reference ("parity unpinned" there); the maths is
+    checked against torch's CTC: cost, and gradient w.r.t. the pre-softmax activations / batch."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.RandomState(7)
+    Tn, B, A = 12, 3, 6
+    act = rng.randn(Tn, B, A).astype(np.float32)
+    lens = np.array([3, 2, 4], np.int32); labels = np.array([1, 2, 1, 3, 3, 5, 4, 2, 1], np.int32); ilen = np.array([12, 10, 12], np.int32)
+    ta = torch.tensor(act, requires_grad=True)
+    lp = torch.log_softmax(ta, 2)
+    loss = torch.nn.functional.ctc_loss(lp, torch.tensor(labels.astype(np.int64)), torch.tensor(ilen.astype(np.int64)), torch.tensor(lens.astype(np.int64)),
+                                        blank=0, reduction="none")
+    (loss.sum() / B).backward()
+    probs = torch.softmax(torch.tensor(act), 2).numpy().astype(np.float32)
+    costs = np.zeros(B, np.float32); d = np.zeros_like(probs)
+    lc.lc_ctc_loss(cptr(probs), cptr(d), cptr(labels), cptr(lens), cptr(ilen), cptr(costs), I(Tn), I(B), I(A))
+    np.testing.assert_allclose(costs, loss.detach().numpy(), rtol=1e-4, atol=1e-4)
+    g = ta.grad.numpy().copy()
+    for b in range(B):
+        g[ilen[b]:, b, :] = 0; 
+    np.testing.assert_allclose(d, g, rtol=1e-3, atol=1e-5)
