@@ -109,6 +109,8 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
   LH_REQUIRE(k >= 0, "lh_sgemm: negative k");
+  LH_REQUIRE(lda >= (ta ? m : k) && ldb >= (tb ? k : n) && ldc >= n, "lh_sgemm: leading dimensions (%d,%d,%d) too small for m%d n%d k%d ta%d tb%d", lda, ldb, ldc, m, n, k, ta, tb);
+  LH_REQUIRE(A && B && C, "lh_sgemm: null operand");
   if ((int64_t)m * n * k >= (1 << 18) && m >= 16 && n >= 16) {
     EpiRowMajor ep; ep.C = C; ep.ldc = ldc; ep.alpha = alpha; ep.beta = beta; ep.atomic = 0;
     const bool av = (lda % 4 == 0) && (((uintptr_t)A & 15) == 0) && (k % 4 == 0);

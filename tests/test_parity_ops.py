@@ -1,0 +1,497 @@
+"""Every non-convolution operator of the Backend trait, HIP (through the C ABI) against the CPU
+oracle on the same seeded inputs, at the shapes the five applications use (ResNet-50, LeNet,
+SqueezeNet, TreeLSTM, DeepSpeech2) plus ragged / tiny / empty-ish edge cases.
+
+Bars: bit-exact for integer results (max-pool argmax, dropout mask, nll gather), 1e-4 relative for
+floats (tests/util.assert_close), written at each assert."""
+import numpy as np
+import pytest
+
+import lantern_amd as la
+from lantern_amd import backend as B
+from lantern_amd._lib import LanternHipError
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+class Pair:
+    """Runs one snippet on both backends; `up` uploads the same host array to each."""
+
+    def __init__(self, cpu, hip):
+        self.bes = (cpu, hip)
+
+    def run(self, fn):
+        outs = []
+        for be in self.bes:
+            la.set_backend(be)
+            up = lambda a, be=be: be.fromHost(np.ascontiguousarray(a))
+            down = lambda buf, shape, dtype=np.float32, be=be: be.toHost(buf, int(np.prod(shape)), dtype).reshape(shape)
+            outs.append(fn(be, up, down))
+        return outs
+
+
+@pytest.fixture
+def pair(cpu_backend, on_hip):
+    return Pair(cpu_backend, on_hip)
+
+
+def check_all(outs, rtol=1e-4, exact=()):
+    want, got = outs
+    assert len(want) == len(got)
+    for i, (w, g) in enumerate(zip(want, got)):
+        if i in exact or w.dtype.kind in "iu":
+            np.testing.assert_array_equal(g, w, err_msg="output %d" % i)
+        else:
+            assert_close(g, w, rtol=rtol, what="output %d" % i)
+
+
+# ---- batch norm --------------------------------------------------------------------------------------
+BN_SHAPES = [(64, 64, 56 * 56), (8, 256, 56 * 56), (16, 512, 28 * 28), (32, 2048, 49), (4, 24, 7), (3, 5, 1), (1, 16, 100), (20, 33, 1), (64, 1024, 1)]
+
+
+@pytest.mark.parametrize("shape", BN_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("relu", [False, True], ids=["plain", "relu"])
+def test_batchnorm_training_and_grad(pair, shape, relu):
+    N, Cc, HW = shape
+    rng = np.random.RandomState(11)
+    x = (rng.randn(N, Cc, HW) * 1.7 + rng.randn(1, Cc, 1) * 3).astype(np.float32)   # per-channel offsets: tests the shifted sums
+    g = (rng.rand(Cc) + 0.5).astype(np.float32); b = rng.randn(Cc).astype(np.float32)
+    dy = rng.randn(N, Cc, HW).astype(np.float32)
+    dx0 = rng.randn(N, Cc, HW).astype(np.float32)
+    if N * HW == 1:
+        pytest.skip("variance of one sample is undefined")
+
+    def f(be, up, down):
+        X, G, Bi, rm, rv = up(x), up(g), up(b), up(np.zeros(Cc, np.float32)), up(np.ones(Cc, np.float32))
+        y, sm, si = be.mallocArray(x.size), be.mallocArray(Cc), be.mallocArray(Cc)
+        be.batchNormTraining_into(X, G, Bi, rm, rv, y, sm, si, N, Cc, HW, relu)
+        outs = [down(y, x.shape), down(sm, (Cc,)), down(si, (Cc,)), down(rm, (Cc,)), down(rv, (Cc,))]
+        DY = up(dy); dg, db = be.mallocArray(Cc), be.mallocArray(Cc)
+        if relu:
+            xd = up(dx0)
+            be.batchNorm_grad(X, xd, DY, G, dg, db, sm, si, N, Cc, HW, beta_dx=1.0, y_relu=y) if be.name == "hip" else _cpu_bn_relu_grad(be, X, xd, DY, y, G, dg, db, sm, si, N, Cc, HW)
+        else:
+            xd = up(dx0)
+            be.batchNorm_grad(X, xd, DY, G, dg, db, sm, si, N, Cc, HW)
+        outs += [down(xd, x.shape), down(dg, (Cc,)), down(db, (Cc,))]
+        # beta 0 into garbage must equal (accumulated - initial)
+        if be.name == "hip":
+            xd2 = up(np.full(x.size, 9.0, np.float32)); dg2, db2 = be.mallocArray(Cc), be.mallocArray(Cc)
+            be.batchNorm_grad(X, xd2, up(dy), G, dg2, db2, sm, si, N, Cc, HW, beta_dx=0.0, y_relu=y if relu else None)
+            assert_close(down(xd2, x.shape) + dx0.reshape(x.shape), outs[5], rtol=2e-4, what="beta 0 vs beta 1")
+        return outs
+
+    outs = pair.run(f)
+    if relu:   # elements of y within rounding of zero may land on either side of the mask; compare away from them
+        x64 = x.astype(np.float64); mu = x64.mean((0, 2), keepdims=True); var = x64.var((0, 2), keepdims=True)
+        pre = (x64 - mu) / np.sqrt(var + 1e-5) * g.reshape(1, Cc, 1) + b.reshape(1, Cc, 1)
+        edge = np.abs(pre) < 2e-5
+        assert edge.mean() < 1e-3 or N * Cc * HW < 5000
+        for o in outs:
+            o[0][edge & (np.abs(o[0]) < 2e-5)] = 0.0
+            o[5][edge] = dx0.reshape(x.shape)[edge]
+    check_all(outs, rtol=2e-4 if relu else 1e-4)
+
+
+def _cpu_bn_relu_grad(be, X, xd, DY, y, G, dg, db, sm, si, N, Cc, HW):
+    be.unary_grad(B.RELU, y, y, DY, DY, N * Cc * HW, inPlace=True)
+    be.batchNorm_grad(X, xd, DY, G, dg, db, sm, si, N, Cc, HW)
+
+
+def test_batchnorm_inference(pair):
+    N, Cc, HW = 4, 70, 81
+    rng = np.random.RandomState(12)
+    x = rng.randn(N, Cc, HW).astype(np.float32); g = rng.rand(Cc).astype(np.float32) + .5; b = rng.randn(Cc).astype(np.float32)
+    rm = rng.randn(Cc).astype(np.float32); rv = rng.rand(Cc).astype(np.float32) + .1
+    check_all(pair.run(lambda be, up, down: [down(be.batchNormInference(up(x), up(g), up(b), up(rm), up(rv), N, Cc, HW), x.shape)]))
+
+
+# ---- pooling -----------------------------------------------------------------------------------------
+POOLS = [(64, 64, 112, 112, 3, 3, 2, 2, 1),     # ResNet stem
+         (8, 6, 24, 24, 2, 2, 2, 2, 0),          # LeNet
+         (4, 96, 15, 15, 3, 3, 2, 2, 0),         # SqueezeNet (overlapping windows, no pad)
+         (2, 3, 9, 7, 3, 2, 2, 1, 1), (1, 1, 2, 2, 2, 2, 2, 2, 0), (3, 5, 7, 7, 7, 7, 1, 1, 0)]
+
+
+@pytest.mark.parametrize("p", POOLS, ids=lambda s: "x".join(map(str, s)))
+def test_maxpool_values_argmax_and_grad(pair, p):
+    N, Cc, H, W, kH, kW, sH, sW, pad = p
+    P, Q = B.conv_size(H, kH, sH, pad), B.conv_size(W, kW, sW, pad)
+    rng = np.random.RandomState(13)
+    x = rng.randint(-6, 7, size=(N, Cc, H, W)).astype(np.float32)      # many ties: first maximum in scan order must win
+    dy = rng.randn(N, Cc, P, Q).astype(np.float32)
+
+    def f(be, up, down):
+        y, idx = be.maxPool2D_batch(up(x), N, Cc, H, W, kH, kW, sH, sW, pad)
+        xd = up(np.ones(x.size, np.float32))
+        be.maxPool2D_batch_grad(xd, up(dy), idx, N * Cc * P * Q)
+        return [down(y, dy.shape), down(idx, dy.shape, np.int32), down(xd, x.shape)]
+
+    outs = pair.run(f)
+    check_all(outs, exact=(0, 1), rtol=1e-5)     # values and indices bit-exact; overlapping windows sum in any order
+
+
+@pytest.mark.parametrize("p", [(64, 2048, 7, 7, 7, 7, 1, 1), (4, 10, 13, 13, 13, 13, 1, 1), (2, 3, 8, 6, 2, 3, 2, 3), (2, 3, 9, 9, 3, 3, 2, 2)], ids=lambda s: "x".join(map(str, s)))
+def test_avgpool_and_grad(pair, p):
+    N, Cc, H, W, kH, kW, sH, sW = p
+    P, Q = B.conv_size(H, kH, sH), B.conv_size(W, kW, sW)
+    rng = np.random.RandomState(14)
+    x = rng.randn(N, Cc, H, W).astype(np.float32); dy = rng.randn(N, Cc, P, Q).astype(np.float32)
+
+    def f(be, up, down):
+        y = be.averagePool2D_batch(up(x), N, Cc, H, W, kH, kW, sH, sW)
+        xd = up(np.ones(x.size, np.float32))
+        be.averagePool2D_batch_grad(xd, up(dy), N, Cc, H, W, kH, kW, sH, sW)
+        return [down(y, dy.shape), down(xd, x.shape)]
+
+    check_all(pair.run(f))
+
+
+# ---- element-wise, broadcast, layout -----------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 3, 64, 1000, 64 * 256 * 56 * 56 // 16 + 5])
+def test_unary_ops_and_grads(pair, n):
+    rng = np.random.RandomState(15)
+    x = (rng.randn(n) * 1.5).astype(np.float32)
+    x[np.abs(x) < 1e-3] = 0.5                                   # keep relu / hardTanh away from their kinks
+    xp = np.abs(x) + 0.1
+    dy = rng.randn(n).astype(np.float32)
+
+    def f(be, up, down):
+        outs = []
+        for op, src in ((B.RELU, x), (B.TANH, x), (B.SIGMOID, x), (B.EXP, x), (B.LOG, xp), (B.SQRT, xp), (B.SQUARE, x), (B.HARDTANH, x)):
+            X = up(src); y = be.unary(op, X, n, lo=-0.8, hi=0.9)
+            dx = up(np.full(n, 0.25, np.float32))
+            be.unary_grad(op, X, y, up(dy), dx, n, lo=-0.8, hi=0.9)
+            outs += [down(y, (n,)), down(dx, (n,))]
+        X = up(x); be.unary(B.RELU, X, n, inPlace=True); outs.append(down(X, (n,)))
+        return outs
+
+    check_all(pair.run(f), rtol=2e-4)
+
+
+BCAST = [((64, 256, 7, 7), (64, 256, 7, 7)), ((8, 16, 5, 5), (1, 16, 1, 1)), ((8, 16, 5, 5), (1,)), ((1, 16, 1, 1), (8, 16, 5, 5)),
+         ((100, 150), (150,)), ((100, 1), (1, 150)), ((5,), (5,)), ((3, 1, 4), (1, 6, 1)), ((20, 10), (20, 1)), ((1,), (1,))]
+
+
+@pytest.mark.parametrize("shapes", BCAST, ids=lambda s: "%s_%s" % ("x".join(map(str, s[0])), "x".join(map(str, s[1]))))
+def test_broadcast_ops_grads_and_updates(pair, shapes):
+    sa, sb = shapes
+    A, Bs, O = B.dim_broadcast(sa, sb)
+    rng = np.random.RandomState(16)
+    a = rng.randn(*sa).astype(np.float32); b = (rng.rand(*sb) + 0.5).astype(np.float32) * np.where(rng.rand(*sb) < .5, -1, 1).astype(np.float32)
+    od = rng.randn(*O).astype(np.float32)
+
+    def f(be, up, down):
+        outs = []
+        for op in (B.ADD, B.SUB, B.MUL, B.DIV):
+            Ab, Bb = up(a), up(b)
+            outs.append(down(be.bcast_op(op, Ab, A, Bb, Bs, O), O))
+            ad, bd = up(np.ones(a.size, np.float32)), up(np.ones(b.size, np.float32))
+            be.bcast_op_grad(op, Ab, ad, A, False, Bb, bd, Bs, False, up(od), O)
+            outs += [down(ad, sa), down(bd, sb)]
+            if tuple(A) == tuple(O):                          # in-place update needs the left side to have the result shape
+                be.bcast_update(op, Ab, A, Bb, Bs); outs.append(down(Ab, sa))
+        return outs
+
+    check_all(pair.run(f), rtol=2e-4)
+
+
+def test_scalar_ops_geam_fill_clip(pair):
+    n = 70001
+    rng = np.random.RandomState(17)
+    x = rng.randn(n).astype(np.float32); y = rng.randn(n).astype(np.float32)
+    bias = rng.randn(12).astype(np.float32)
+
+    def f(be, up, down):
+        outs = [down(be.scalar_op(op, up(x), 1.7, n), (n,)) for op in (B.ADD, B.SUB, B.MUL, B.DIV)]
+        o = be.mallocArray(n); be.geam(up(x), 0.3, up(y), -2.0, o, n); outs.append(down(o, (n,)))
+        X = up(x); be.geam(X, 1.0, up(y), 1.0, X, n); outs.append(down(X, (n,)))           # aliasing output with an input
+        X = up(x); be.fillInPlace(X, n, 2.5); outs.append(down(X, (n,)))
+        X = up(x); be.clipAt(X, n, 0.5); outs.append(down(X, (n,)))
+        outs.append(down(be.fillWithBias((3, 12, 5, 7), up(bias), 1), (3, 12, 5, 7)))
+        outs.append(down(be.fillWithBias((4, 12), up(bias), 1), (4, 12)))
+        return outs
+
+    check_all(pair.run(f), rtol=1e-6)
+
+
+@pytest.mark.parametrize("rc", [(1, 1), (3, 5), (64, 64), (100, 257), (2048, 1000), (1, 300)])
+def test_transpose_and_grad(pair, rc):
+    r, c = rc
+    rng = np.random.RandomState(18); x = rng.randn(r, c).astype(np.float32); yd = rng.randn(c, r).astype(np.float32)
+
+    def f(be, up, down):
+        y = be.trans(up(x), r, c); xd = up(np.ones(r * c, np.float32)); be.trans_grad(xd, up(yd), r, c)
+        return [down(y, (c, r)), down(xd, (r, c))]
+
+    outs = pair.run(f)
+    np.testing.assert_array_equal(outs[1][0], x.T)
+    check_all(outs, rtol=1e-6)
+
+
+@pytest.mark.parametrize("case", [((4, 6, 5), (2, 0, 1)), ((3, 32, 21, 50), (3, 0, 1, 2)), ((2, 3, 4, 5), (0, 2, 3, 1)), ((7, 9), (1, 0)), ((2, 3, 4, 5), (3, 2, 1, 0)),
+                                  ((8, 32, 11, 40), (2, 0, 1, 3))], ids=str)
+def test_permute_and_grad(pair, case):
+    dims, perm = case
+    rng = np.random.RandomState(19); x = rng.randn(*dims).astype(np.float32)
+    odims = tuple(dims[p] for p in perm); yd = rng.randn(*odims).astype(np.float32)
+
+    def f(be, up, down):
+        y = be.permute(up(x), dims, perm); xd = up(np.ones(x.size, np.float32)); be.permute_grad(xd, up(yd), dims, perm)
+        return [down(y, odims), down(xd, dims)]
+
+    outs = pair.run(f)
+    np.testing.assert_array_equal(outs[1][0], np.transpose(x, perm))
+    check_all(outs, rtol=1e-6)
+
+
+def test_concat_and_grad(pair):
+    rng = np.random.RandomState(20)
+    for outer, sizes, inner in [(4, (64, 64), 13 * 13), (2, (3, 5, 1), 7), (1, (10,), 1), (3, (2, 2), 1), (5, (128, 128), 1)]:
+        xs = [rng.randn(outer, s, inner).astype(np.float32) for s in sizes]
+        od = rng.randn(outer, sum(sizes), inner).astype(np.float32)
+
+        def f(be, up, down):
+            y = be.concat([up(x) for x in xs], list(sizes), outer, inner)
+            ds = [up(np.ones(x.size, np.float32)) for x in xs]
+            be.concat_grad(ds, list(sizes), up(od), outer, inner)
+            return [down(y, od.shape)] + [down(d, x.shape) for d, x in zip(ds, xs)]
+
+        outs = pair.run(f)
+        np.testing.assert_array_equal(outs[1][0], np.concatenate(xs, 1))
+        check_all(outs, rtol=1e-6)
+
+
+# ---- reductions, softmax, loss -----------------------------------------------------------------------
+@pytest.mark.parametrize("n", [1, 7, 4096, 1000003])
+def test_sum_mean_and_grads(pair, n):
+    rng = np.random.RandomState(21); x = (rng.randn(n) + 0.3).astype(np.float32)
+
+    def f(be, up, down):
+        X = up(x); s, m = be.sum(X, n), be.mean(X, n)
+        dx = up(np.ones(n, np.float32)); be.add_scalar_from(dx, up(np.array([2.5], np.float32)), 1.0 / n, n)
+        return [down(s, (1,)), down(m, (1,)), down(dx, (n,))]
+
+    outs = pair.run(f)
+    assert abs(outs[1][0][0] - x.astype(np.float64).sum()) <= 1e-4 * (np.abs(x).sum())   # device sum against the exact one
+    check_all(outs, rtol=2e-4)
+
+
+@pytest.mark.parametrize("oci", [(64, 49, 1), (1, 5, 1), (8, 3, 20), (100, 1, 7), (3, 1000, 1), (2, 64, 3000)])
+def test_sum_dim_and_grad(pair, oci):
+    o, d, i = oci
+    rng = np.random.RandomState(22); x = rng.randn(o, d, i).astype(np.float32); dy = rng.randn(o, i).astype(np.float32)
+
+    def f(be, up, down):
+        y = be.sum_dim(up(x), o, d, i); dx = up(np.ones(x.size, np.float32)); be.sum_dim_grad(dx, up(dy), o, d, i)
+        return [down(y, (o, i)), down(dx, x.shape)]
+
+    check_all(pair.run(f))
+
+
+@pytest.mark.parametrize("oci", [(64, 1000, 1), (100, 10, 1), (1, 1, 1), (5, 29, 1), (3, 29, 150), (7, 5000, 1), (2, 3, 1)])
+@pytest.mark.parametrize("is_log", [0, 1], ids=["softmax", "logsoftmax"])
+def test_softmax_and_grad(pair, oci, is_log):
+    o, c, i = oci
+    rng = np.random.RandomState(23); x = (rng.randn(o, c, i) * 4).astype(np.float32); dy = rng.randn(o, c, i).astype(np.float32)
+
+    def f(be, up, down):
+        y = be.softmax(is_log, up(x), o, c, i); dx = up(np.ones(x.size, np.float32))
+        be.softmax_grad(is_log, y, up(dy), dx, o, c, i)
+        return [down(y, x.shape), down(dx, x.shape)]
+
+    check_all(pair.run(f), rtol=2e-4)
+
+
+def test_nll_loss_and_grad(pair):
+    rng = np.random.RandomState(24)
+    for batch, classes in [(64, 1000), (100, 10), (1, 5), (7, 1)]:
+        x = rng.randn(batch, classes).astype(np.float32); t = rng.randint(0, classes, size=batch).astype(np.int32)
+        dy = rng.randn(batch).astype(np.float32)
+
+        def f(be, up, down):
+            T = up(t); y = be.nllLoss(up(x), T, batch, classes); dx = up(np.ones(x.size, np.float32))
+            be.nllLoss_grad(dx, T, up(dy), batch, classes)
+            return [down(y, (batch,)), down(dx, x.shape)]
+
+        outs = pair.run(f)
+        np.testing.assert_array_equal(outs[1][0], -x[np.arange(batch), t])           # a gather: exact
+        check_all(outs, rtol=1e-6)
+
+
+# ---- dot family --------------------------------------------------------------------------------------
+def test_dot_family_at_treelstm_and_classifier_shapes(pair):
+    rng = np.random.RandomState(25)
+
+    def f(be, up, down):
+        outs = []
+        for m, n in [(150, 300), (5, 150), (1, 1), (1000, 2048), (33, 7)]:
+            Mx = rng_m[(m, n)]; v = rng_v[n]; w = rng_v2[m]
+            outs.append(down(be.matrixVectorDot(up(Mx), up(v), m, n), (m,)))
+            outs.append(down(be.vectorVectorDot(up(v), up(v[::-1].copy()), n), (1,)))
+            xd = up(np.ones(m * n, np.float32)); be.add_cartesian(xd, up(v), up(w), m, n); outs.append(down(xd, (m, n)))
+            vd = up(np.ones(n, np.float32)); be.add_composition(vd, up(Mx), up(w), m, n); outs.append(down(vd, (n,)))
+            sd = up(np.ones(n, np.float32)); be.addMul_scalar(sd, up(np.array([0.7], np.float32)), up(v), n); outs.append(down(sd, (n,)))
+        for d1, d2, d3 in [(64, 2048, 1000), (100, 320, 50), (3, 4, 5), (20, 1, 7), (1, 33, 1)]:
+            X, Y, O = rng_g[(d1, d2)], rng_g[(d2, d3)], rng_g[(d1, d3)]
+            outs.append(down(be.matrixMatrixDot(up(X), up(Y), d1, d2, d3), (d1, d3)))
+            xd = up(np.ones(d1 * d2, np.float32)); be.add_dotTrans2(xd, up(O), up(Y), d1, d2, d3); outs.append(down(xd, (d1, d2)))
+            yd = up(np.ones(d2 * d3, np.float32)); be.add_dotTrans1(yd, up(X), up(O), d1, d2, d3); outs.append(down(yd, (d2, d3)))
+        return outs
+
+    rng_m = {s: rng.randn(*s).astype(np.float32) for s in [(150, 300), (5, 150), (1, 1), (1000, 2048), (33, 7)]}
+    rng_v = {n: rng.randn(n).astype(np.float32) for n in (300, 150, 1, 2048, 7)}
+    rng_v2 = {m: rng.randn(m).astype(np.float32) for m in (150, 5, 1, 1000, 33)}
+    rng_g = {}
+    for d1, d2, d3 in [(64, 2048, 1000), (100, 320, 50), (3, 4, 5), (20, 1, 7), (1, 33, 1)]:
+        for s in ((d1, d2), (d2, d3), (d1, d3)):
+            rng_g.setdefault(s, rng.randn(*s).astype(np.float32))
+    check_all(pair.run(f))
+
+
+@pytest.mark.parametrize("tx", [False, True])
+@pytest.mark.parametrize("ty", [False, True])
+def test_gemm_and_grad_all_transposes(pair, tx, ty):
+    rng = np.random.RandomState(26)
+    for d1, d2, d3 in [(32, 672, 1024), (5, 7, 3), (64, 100, 29)]:
+        X = rng.randn(*((d2, d1) if tx else (d1, d2))).astype(np.float32); Y = rng.randn(*((d3, d2) if ty else (d2, d3))).astype(np.float32)
+        od = rng.randn(d1, d3).astype(np.float32)
+
+        def f(be, up, down):
+            Xb, Yb = up(X), up(Y)
+            r = be.gemm(Xb, tx, Yb, ty, 0.5, d1, d2, d3)
+            xd, yd = up(np.ones(X.size, np.float32)), up(np.ones(Y.size, np.float32))
+            be.gemm_grad(Xb, xd, False, tx, Yb, yd, False, ty, 0.5, up(od), d1, d2, d3)
+            return [down(r, (d1, d3)), down(xd, X.shape), down(yd, Y.shape)]
+
+        check_all(pair.run(f))
+
+
+# ---- dropout, masks ----------------------------------------------------------------------------------
+def test_dropout_mask_is_bit_exact_and_scaled(pair):
+    n = 100003
+    rng = np.random.RandomState(27); x = rng.randn(n).astype(np.float32); dy = rng.randn(n).astype(np.float32)
+
+    def f(be, up, down):
+        be.dropout_seed, be.dropout_offset = 1234, 77
+        y, mask = be.dropout(up(x), n, 0.3)
+        y2, mask2 = be.dropout(up(x), n, 0.3)                  # the stream advances: a different mask
+        dx = up(np.ones(n, np.float32)); be.dropout_grad(dx, up(dy), mask, n)
+        y0, m0 = be.dropout(up(x), n, 0.0)
+        return [down(mask, (n,)), down(y, (n,)), down(mask2, (n,)), down(dx, (n,)), down(m0, (n,)), down(y0, (n,))]
+
+    outs = pair.run(f)
+    m = outs[1][0]
+    assert abs((m > 0).mean() - 0.7) < 0.01 and not np.array_equal(m, outs[1][2])
+    np.testing.assert_array_equal(outs[1][4], np.ones(n, np.float32))
+    check_all(outs, exact=(0, 2, 4), rtol=1e-6)
+    with pytest.raises(ValueError):
+        pair.bes[1].dropout(None, 4, 1.0)
+
+
+def test_mask4d(pair):
+    n, c, d, t = 4, 3, 5, 17
+    rng = np.random.RandomState(28); x = rng.randn(n, c, d, t).astype(np.float32); lens = np.array([17, 0, 9, 1], np.int32)
+
+    def f(be, up, down):
+        X = up(x); be.mask4D(X, up(lens), n, c, d, t); return [down(X, x.shape)]
+
+    outs = pair.run(f)
+    want = x.copy()
+    for i, l in enumerate(lens):
+        want[i, :, :, l:] = 0
+    np.testing.assert_array_equal(outs[1][0], want)
+    check_all(outs, exact=(0,))
+
+
+# ---- optimizers --------------------------------------------------------------------------------------
+def test_optimizers_single_and_multi_tensor(pair):
+    rng = np.random.RandomState(29)
+    sizes = [1, 7, 64, 1000, 9 * 64 * 64, 2048 * 1000 + 3]
+    xs = [rng.randn(s).astype(np.float32) for s in sizes]; gs = [(rng.randn(s) * 3).astype(np.float32) for s in sizes]
+
+    def f(be, up, down):
+        outs = []
+        for nesterov in (False, True):
+            X, D, V = up(xs[3]), up(gs[3]), be.mallocArray(sizes[3])
+            for _ in range(3):
+                be.momentum_update(X, D, V, 0.1, 0.9, 2.0, nesterov, sizes[3]); be.upload(D, gs[3])
+            outs += [down(X, (sizes[3],)), down(V, (sizes[3],))]
+        X, D, M = up(xs[2]), up(gs[2]), be.mallocArray(sizes[2])
+        be.adagrad_update(X, D, M, 0.05, 1.0, sizes[2]); outs += [down(X, (sizes[2],)), down(M, (sizes[2],)), down(D, (sizes[2],))]
+        X, D = up(xs[4]), up(gs[4]); be.sgd_update(X, D, 0.01, sizes[4]); outs += [down(X, (sizes[4],)), down(D, (sizes[4],))]
+        ps = [(up(x), up(g), be.mallocArray(s), s) for x, g, s in zip(xs, gs, sizes)]
+        for _ in range(2):
+            be.multi_momentum_update(ps, 0.1, 0.9, 400.0, False)
+            for p, g in zip(ps, gs):
+                be.copyFloatArray(p[1], up(g), p[3])
+        for p in ps:
+            outs += [down(p[0], (p[3],)), down(p[2], (p[3],))]
+        ps2 = [(up(x), up(g), s) for x, g, s in zip(xs, gs, sizes)]
+        be.multi_sgd_update(ps2, 0.05)
+        for p in ps2:
+            outs += [down(p[0], (p[2],)), down(p[1], (p[2],))]
+        return outs
+
+    check_all(pair.run(f), rtol=1e-5)
+
+
+# ---- fused pairs against their unfused sequences ----------------------------------------------------
+def test_add_relu_and_its_gradient(pair):
+    n = 64 * 256 * 14 * 14 + 3
+    rng = np.random.RandomState(30)
+    a = rng.randn(n).astype(np.float32); b = rng.randn(n).astype(np.float32); dy = rng.randn(n).astype(np.float32)
+    s = a + b; a[np.abs(s) < 1e-4] += 1.0
+
+    def f(be, up, down):
+        o = be.mallocArray(n); be.add_into(up(a), up(b), o, n, True)
+        ad = be.mallocArray(n, zero=False) if be.name == "hip" else be.mallocArray(n)
+        bd = up(np.ones(n, np.float32))
+        if be.name == "hip":
+            be.add_relu_grad(o, up(dy), ad, 0.0, bd, 1.0, n)         # first writer overwrites, second accumulates
+        else:
+            be.add_relu_grad(o, up(dy), ad, 1.0, bd, 1.0, n)
+        return [down(o, (n,)), down(ad, (n,)), down(bd, (n,))]
+
+    check_all(pair.run(f), rtol=1e-6)
+
+
+# ---- arena and error path (the library's own behaviour; no oracle counterpart) -----------------------
+def test_arena_zeroing_alignment_rewind_and_overflow(on_hip):
+    be = on_hip
+    lib = be.lib
+    mark = be.getMallocAddr()
+    a = be.mallocArray(1000)
+    assert a.ptr % 256 == 0 and not be.toHost(a, 1000).any()
+    be.fillInPlace(a, 1000, 3.0)
+    used = lib.lh_heap_used()
+    b = be.mallocArray(10)
+    assert b.ptr % 256 == 0 and b.ptr >= a.ptr + 4000 and lib.lh_heap_used() > used
+    be.resetMallocAddr(mark)
+    c = be.mallocArray(1000)
+    assert c.ptr == a.ptr and not be.toHost(c, 1000).any()        # memory handed out again starts at zero (CUB:22-25 memset on rewind)
+    be.resetMallocAddr(mark)
+    with pytest.raises(LanternHipError):
+        be.mallocArray(be.heap_bytes)                              # 4x the arena: refused, nothing allocated
+    assert lib.lh_heap_used() <= used                              # nothing was taken by the refused request
+    z = be.mallocArray(4); assert not be.toHost(z, 4).any()        # the library keeps working after an error
+    be.resetMallocAddr(mark)
+
+
+def test_shape_errors_are_reported_not_launched(on_hip):
+    be = on_hip
+    x = be.mallocArray(16)
+    for call in (lambda: be.lib.lh_conv2d_fwd(x.ptr, x.ptr, 0, x.ptr, 1, 1, 2, 2, 1, 3, 3, 1, 1, 0, 0),       # kernel larger than the padded input
+                 lambda: be.lib.lh_conv2d_fwd(x.ptr, x.ptr, 0, x.ptr, 1, 1, 4, 4, 1, 3, 3, 0, 1, 0, 0),       # stride 0
+                 lambda: be.lib.lh_sgemm(0, 0, 4, 4, 4, 1.0, x.ptr, 2, x.ptr, 4, 0.0, x.ptr, 4),              # lda < k
+                 lambda: be.lib.lh_unary(99, x.ptr, x.ptr, 16, 0.0, 0.0),                                     # unknown op code
+                 lambda: be.lib.lh_permute(x.ptr, x.ptr, B._ints((2, 8)), B._ints((0, 0)), 2),                # not a permutation
+                 lambda: be.lib.lh_bcast_op(0, x.ptr, B._ints((2, 8)), x.ptr, B._ints((3, 8)), x.ptr, B._ints((3, 8)), 2),   # 2 against 3 does not broadcast
+                 lambda: be.lib.lh_dropout_fwd(x.ptr, x.ptr, x.ptr, 16, 1.0, 1, 0)):                          # rate outside [0, 1)
+        call()
+        with pytest.raises(LanternHipError):
+            from lantern_amd import _lib
+            _lib.check()
+    be.fillInPlace(x, 16, 1.0)
+    assert (be.toHost(x, 16) == 1.0).all()
