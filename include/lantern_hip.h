@@ -22,8 +22,13 @@
  *    prints "file:line: message" and exits the process.  A host that prefers
  *    to handle errors calls lh_set_error_mode(1): the failing entry point then
  *    returns early and lh_last_error() holds the message.
- *  - No allocation happens inside an operator: outputs, gradients and scratch
- *    are caller-provided, normally from the arena below.
+ *  - Outputs and gradients are caller-provided, normally from the arena below.
+ *    Operators call no hipMalloc: convolution takes its filter-layout scratch
+ *    from the top of the arena and pops it before returning (stream order
+ *    keeps that safe); batch norm uses a fixed device-resident partials
+ *    array.  The one exception is the multi-tensor optimizer entry points,
+ *    which keep a pointer table on the device and re-allocate it when a
+ *    larger model is passed.
  */
 #ifndef LANTERN_HIP_H
 #define LANTERN_HIP_H
