@@ -83,3 +83,20 @@ def test_resnet_imagenet_stem_3_steps(hip_backend, cpu_backend):
     from lantern_amd.apps.resnet50 import ResNet50, Trainer
     _compare(lambda: Trainer(ResNet50(num_classes=20, imagenet_stem=True, layers=(1, 1, 1, 1)), 4, 64, 20, lr=0.005, momentum=0.9),
              hip_backend, cpu_backend, steps=3, per_tensor=2e-2)
+
+
+def test_squeezenet_10_steps(hip_backend, cpu_backend):
+    """All 26 biased convs, 8 concats, 3 max-pools, momentum SGD (the reference's configuration but batch 16)."""
+    from lantern_amd.apps.squeezenet import Trainer
+    _compare(lambda: Trainer(batch=16, lr=0.001), hip_backend, cpu_backend, per_tensor=5e-3)
+
+
+def test_squeezenet_avgpool_head_5_steps(hip_backend, cpu_backend):
+    from lantern_amd.apps.squeezenet import Trainer
+    _compare(lambda: Trainer(batch=8, lr=0.001, avgpool_head=True), hip_backend, cpu_backend, steps=5, per_tensor=5e-3)
+
+
+def test_treelstm_10_trees(hip_backend, cpu_backend):
+    """One Adagrad step per tree over 10 random trees of 5..30 leaves: gemv / rank-1 update / gemv-transposed path."""
+    from lantern_amd.apps.treelstm import Trainer
+    _compare(lambda: Trainer(n_trees=10, vocab=500, max_leaves=30), hip_backend, cpu_backend, steps=10)
