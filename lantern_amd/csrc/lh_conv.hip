@@ -29,6 +29,7 @@ static bool make_dims(ConvDims& d, int N, int C, int H, int W, int K, int R, int
 struct LoadConvFwdB {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
+  static constexpr bool SPLIT = false;
   const float* base; uint32_t nbytes;
   int C, H, W, sH, sW, pH, pW, HW;
   FastDiv dPQ, dQ, dRS, dS;
@@ -54,6 +55,7 @@ struct LoadConvFwdB {
 struct LoadConvBwdDataB {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
+  static constexpr bool SPLIT = false;
   const float* base; uint32_t nbytes;
   int K, P, Q, PQ;
   FastDiv dHW, dW, dRS, dS, dsH, dsW;
@@ -86,6 +88,7 @@ struct LoadConvBwdDataB {
 struct LoadConvFwdTapB {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
+  static constexpr bool SPLIT = true;
   const float* base; uint32_t nbytes;
   int C, H, W, sH, sW, pH, pW, HW;
   FastDiv dPQ, dQ, dC, dS;
@@ -97,12 +100,18 @@ struct LoadConvFwdTapB {
     s.h0 = (int)p * sH - pH; s.w0 = (int)q * sW - pW;
     s.pix = (int)n * C * HW + s.h0 * W + s.w0;
   }
-  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
+  // per-lane part: the pixel under the tap of this group of four k (same tap for all four), or LH_OOB
+  __device__ __forceinline__ uint32_t voff(const State& s, int k, int kend) const {
     uint32_t tap, ch, r, ss;
-    dC.divmod(k, tap, ch); dS.divmod(tap, r, ss);                 // wave-uniform; same tap for e = 0..3
+    dC.divmod(k, tap, ch); dS.divmod(tap, r, ss);                 // wave-uniform
     const bool ok = s.valid && k < kend && (unsigned)(s.h0 + (int)r) < (unsigned)H && (unsigned)(s.w0 + (int)ss) < (unsigned)W;
-    const int rel = ((int)ch + e) * HW + (int)r * W + (int)ss;   // wave-uniform
-    return ok ? (uint32_t)(s.pix + rel) * 4u : LH_OOB;
+    return ok ? (uint32_t)(s.pix + (int)r * W + (int)ss) * 4u : LH_OOB;
+  }
+  // wave-uniform part: the channel plane of element e
+  __device__ __forceinline__ uint32_t soff(int k, int e) const {
+    uint32_t tap, ch;
+    dC.divmod(k, tap, ch);
+    return (uint32_t)(((int)ch + e) * HW) * 4u;
   }
 };
 // Input gradient for one residue class of output pixels (h = aH + sH*h', w = aW + sW*w'): only
@@ -111,6 +120,7 @@ struct LoadConvFwdTapB {
 struct LoadConvBwdDataTapB {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
+  static constexpr bool SPLIT = true;
   const float* base; uint32_t nbytes;
   int K, P, Q, PQ, offH, offW;
   FastDiv dPIX, dWc, dK, dSc;       // class-grid pixels per sample, class-grid width, K, taps per row
@@ -121,12 +131,17 @@ struct LoadConvBwdDataTapB {
     dPIX.divmod(s.valid ? j : 0, n, pix); dWc.divmod(pix, h, w);
     s.nbase = (int)n * K * PQ; s.hq = (int)h + offH; s.wq = (int)w + offW;
   }
-  __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
+  __device__ __forceinline__ uint32_t voff(const State& s, int k, int kend) const {
     uint32_t tap, ko, tr, ts;
     dK.divmod(k, tap, ko); dSc.divmod(tap, tr, ts);               // wave-uniform
     const int p = s.hq - (int)tr, q = s.wq - (int)ts;
     const bool ok = s.valid && k < kend && (unsigned)p < (unsigned)P && (unsigned)q < (unsigned)Q;
-    return ok ? (uint32_t)(s.nbase + ((int)ko + e) * PQ + p * Q + q) * 4u : LH_OOB;
+    return ok ? (uint32_t)(s.nbase + p * Q + q) * 4u : LH_OOB;
+  }
+  __device__ __forceinline__ uint32_t soff(int k, int e) const {
+    uint32_t tap, ko;
+    dK.divmod(k, tap, ko);
+    return (uint32_t)(((int)ko + e) * PQ) * 4u;
   }
 };
 
@@ -135,6 +150,7 @@ template <bool VEC>                      // VEC: PQ % 4 == 0 and dy 16-byte alig
 struct LoadConvBwdFilterA {
   static constexpr bool ALONG_K = true;
   static constexpr bool VEC4 = VEC;
+  static constexpr bool SPLIT = false;
   const float* base; uint32_t nbytes;
   int K, PQ;
   FastDiv dPQ;
@@ -153,6 +169,7 @@ template <bool ROWVEC>                   // ROWVEC: Q % 4 == 0, the four reducti
 struct LoadConvBwdFilterB {
   static constexpr bool ALONG_K = true;
   static constexpr bool VEC4 = false;
+  static constexpr bool SPLIT = false;
   const float* base; uint32_t nbytes;
   int C, H, W, sH, sW, pH, pW, CHW;
   FastDiv dPQ, dQ, dRS, dS;
@@ -248,6 +265,24 @@ constexpr int BWDF_BK = LH_BWDF_BK;      // k-slab of the filter-gradient kernel
 // of blocks; such shapes run stream-K instead (largest tile, two workers per CU, every worker the
 // same number of k-slabs).  `zero_out`/`zero_n`: the output to clear first when the epilogue
 // overwrites (beta = 0), because shared tiles are completed with atomic adds.
+// All blocks of a launch that fit on the chip at once form a round; tiles take about the same
+// time, so a last round with only a few tiles leaves most CUs idle for a whole tile time.  When the
+// tile count is a little above a whole number of rounds, the columns of the surplus tiles are
+// computed by a second launch with smaller tiles, which spreads them over four times as many CUs.
+template <int BM, int BN, int SBM, int SBN, class AL, class BL, class EP>
+static bool launch_rounds(const AL& al, const BL& bl, const EP& ep, int M, int N, int K) {
+  constexpr int rem_div = 3;        // split when the surplus is at most a third of a round
+  const int64_t tm = cdiv(M, BM), tn = cdiv(N, BN), tiles = tm * tn;
+  const int64_t slots = (int64_t)igemm_blocks_per_cu<BM, BN, CONV_BK, AL, BL, EP>() * g_num_cu;
+  const int64_t full = tiles / slots, rem = tiles - full * slots;
+  if (rem_div > 0 && full >= 1 && rem > 0 && rem * rem_div <= slots) {
+    const int col1 = (int)((full * slots / tm) * BN);
+    if (col1 > 0 && col1 < N)
+      return igemm_launch<BM, BN, CONV_BK>(al, bl, ep, M, N, K, 1, 0, 0, col1) && igemm_launch<SBM, SBN, CONV_BK>(al, bl, ep, M, N, K, 1, 0, col1, N);
+  }
+  return igemm_launch<BM, BN, CONV_BK>(al, bl, ep, M, N, K, 1);
+}
+
 template <class AL, class BL, class EP>
 static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out = nullptr, int64_t zero_n = 0, bool prezeroed = false) {
   const int64_t t128 = cdiv(M, 128) * cdiv(N, 128), t64 = cdiv(M, 64) * cdiv(N, 128);
@@ -261,8 +296,8 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
     return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
   }
   TilePick tp = pick_tile(M, N);
-  if (tp.bm == 128) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1);
-  if (tp.bn == 128) return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1);
+  if (tp.bm == 128) return launch_rounds<128, 128, 64, 64>(al, bl, ep, M, N, K);
+  if (tp.bn == 128) return launch_rounds<64, 128, 64, 64>(al, bl, ep, M, N, K);
   return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1);
 }
 }  // namespace
@@ -406,7 +441,19 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
     else ok = igemm_launch<64, 64, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
   };
-  if (avec && rowvec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<true>());
+  // 1x1, stride 1, no padding: the gather of x is a plain [C][N*PQ] matrix with the same layout as dy
+  auto go_plain = [&](auto al, auto bl) {
+    al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
+    bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * PQ * 4); bl.K = C; bl.PQ = PQ; bl.dPQ.init(PQ);
+    if (tp.bm == 128) ok = igemm_launch<128, 128, 16>(al, bl, ep, K, CRS, (int)red, split);
+    else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
+    else ok = igemm_launch<64, 64, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
+  };
+  const bool plain = R == 1 && S == 1 && sH == 1 && sW == 1 && pH == 0 && pW == 0;
+  const bool xvec = (PQ % 4 == 0) && (((uintptr_t)x & 15) == 0);
+  if (plain && avec && xvec) go_plain(LoadConvBwdFilterA<true>(), LoadConvBwdFilterA<true>());
+  else if (plain && !avec && !xvec) go_plain(LoadConvBwdFilterA<false>(), LoadConvBwdFilterA<false>());
+  else if (avec && rowvec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<true>());
   else if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<false>());
   else if (rowvec) go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<true>());
   else go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<false>());

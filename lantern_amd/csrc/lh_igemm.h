@@ -37,7 +37,8 @@ struct FastDiv {
 };
 
 struct GemmShape {
-  int M, N, K;
+  int M, N, K;                // N: end of the column range of this launch
+  int colBase;                // first column of this launch (tiles are counted from here)
   int tilesM, tilesN, splitK, kPerSplit;
   int total, perXcd;          // work items (tiles x k-splits, or stream-K workers) and items per XCD
   int streamk;                // != 0: `total` workers share tiles*slabsPerTile k-slabs evenly
@@ -61,6 +62,7 @@ template <bool VEC>
 struct LoadPlainK {
   static constexpr bool ALONG_K = true;
   static constexpr bool VEC4 = VEC;
+  static constexpr bool SPLIT = false;
   const float* base; uint32_t nbytes; int ld;
   struct State { uint32_t row; bool valid; };
   __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.row = (uint32_t)(s.valid ? col : 0) * (uint32_t)ld * 4u; }
@@ -73,6 +75,7 @@ struct LoadPlainK {
 struct LoadPlainT {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
+  static constexpr bool SPLIT = false;
   const float* base; uint32_t nbytes; int ld;
   struct State { uint32_t col; bool valid; };
   __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.col = (uint32_t)(s.valid ? col : 0) * 4u; }
@@ -81,10 +84,20 @@ struct LoadPlainT {
   }
 };
 
-// Offsets of one group of four k (one offset when the loader is VEC4).
-template <class L> struct LhOff { uint32_t o[4]; };
+// Offsets of one group of four k (one offset when the loader is VEC4).  A SPLIT loader gives one
+// per-lane byte offset for the group (o[0], LH_OOB when the group is out of range for this lane)
+// plus four wave-uniform byte offsets s[i] that go into the scalar-offset operand of the load.
+template <class L> struct LhOff { uint32_t o[4]; uint32_t s[4]; };
 template <class L>
 __device__ __forceinline__ float4 lh_fetch4(__amdgpu_buffer_rsrc_t rsrc, const LhOff<L>& f) {
+  if (L::SPLIT) {
+    float4 r;
+    r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[0], 0));
+    r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[1], 0));
+    r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[2], 0));
+    r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[3], 0));
+    return r;
+  }
   if (L::VEC4) {
     typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
     u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)f.o[0], 0, 0);
@@ -167,7 +180,7 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
     kbeg = sp * gs.kPerSplit; kend = min(gs.K, kbeg + gs.kPerSplit);
     u = u_end;
   }
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * BM, n0 = gs.colBase + tn * BN;
   typename AL::State sa[GA];
   typename BL::State sb[GB];
 #pragma unroll
@@ -187,42 +200,58 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
   constexpr int EA = AL::VEC4 ? 1 : 4, EB = BL::VEC4 ? 1 : 4;
   constexpr int NEL = GA * EA + GB * EB;            // offsets to compute per slab and thread
   constexpr int NM_PAIR = 4 * MI * NI, NM = (KQ / 2) * NM_PAIR;
-  float4 ra[GA], rb[GB];
+  float4 ra0[GA], rb0[GB], ra1[GA], rb1[GB];
   LhOff<AL> oa[GA];
   LhOff<BL> ob[GB];
   // e-th offset of the slab starting at k0
   auto elem = [&](int e, int k0) {
-    if (e < GA * EA) { const int g = e / EA, i = e % EA; oa[g].o[i] = al.off1(sa[g], k0 + 4 * a_kq[g], kend, i); }
-    else { const int f = e - GA * EA, g = f / EB, i = f % EB; ob[g].o[i] = bl.off1(sb[g], k0 + 4 * b_kq[g], kend, i); }
+    if (e < GA * EA) {
+      const int g = e / EA, i = e % EA, k = k0 + 4 * a_kq[g];
+      if constexpr (AL::SPLIT) { if (i == 0) oa[g].o[0] = al.voff(sa[g], k, kend); oa[g].s[i] = al.soff(k, i); }
+      else oa[g].o[i] = al.off1(sa[g], k, kend, i);
+    } else {
+      const int f = e - GA * EA, g = f / EB, i = f % EB, k = k0 + 4 * b_kq[g];
+      if constexpr (BL::SPLIT) { if (i == 0) ob[g].o[0] = bl.voff(sb[g], k, kend); ob[g].s[i] = bl.soff(k, i); }
+      else ob[g].o[i] = bl.off1(sb[g], k, kend, i);
+    }
   };
-
-  // Software pipeline over k-slabs (three slabs in flight):
-  //   the loads of slab t+1 are issued at the top of the iteration from offsets computed one
-  //   iteration earlier and land in LDS after the MFMAs of slab t;
-  //   the offsets of slab t+2 (VALU/SALU only) are computed in small pieces placed between the
-  //   MFMAs of slab t, so they issue while the matrix pipe is busy.
-  // Slabs past kend produce LH_OOB offsets (loads return 0) and LDS stages that are never read.
-#pragma unroll
-  for (int e = 0; e < NEL; e++) elem(e, kbeg);
-#pragma unroll
-  for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(rsA, oa[g]);
-#pragma unroll
-  for (int g = 0; g < GB; g++) rb[g] = lh_fetch4<BL>(rsB, ob[g]);
-#pragma unroll
-  for (int e = 0; e < NEL; e++) elem(e, kbeg + BK);
-#pragma unroll
-  for (int g = 0; g < GA; g++) As[a_kq[g] * LDA + a_col[g]] = ra[g];
-#pragma unroll
-  for (int g = 0; g < GB; g++) Bs[b_kq[g] * LDB + b_col[g]] = rb[g];
-  __syncthreads();
-
-  for (int it = 0; it < niter; it++) {
-    const int st = it & 1;
-    const int k2 = kbeg + (it + 2) * BK;
+  auto fetch = [&](float4 (&ra)[GA], float4 (&rb)[GB]) {
 #pragma unroll
     for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(rsA, oa[g]);
 #pragma unroll
     for (int g = 0; g < GB; g++) rb[g] = lh_fetch4<BL>(rsB, ob[g]);
+  };
+  auto stash = [&](const float4 (&ra)[GA], const float4 (&rb)[GB], int stage) {
+    const int o = stage * KQ;
+#pragma unroll
+    for (int g = 0; g < GA; g++) As[(o + a_kq[g]) * LDA + a_col[g]] = ra[g];
+#pragma unroll
+    for (int g = 0; g < GB; g++) Bs[(o + b_kq[g]) * LDB + b_col[g]] = rb[g];
+  };
+
+  // Software pipeline over k-slabs (four slabs in flight):
+  //   while the MFMAs of slab t run from LDS, slab t+1 is in registers on its way to LDS (its
+  //   loads were issued one iteration earlier), the loads of slab t+2 are issued at the top of the
+  //   iteration into the other register set, and the offsets of slab t+3 (VALU/SALU only) are
+  //   computed in small pieces placed between the MFMAs, so they issue while the matrix pipe is
+  //   busy.  A global load therefore has a whole iteration plus the MFMA time of the next one to
+  //   arrive.  Slabs past kend produce LH_OOB offsets (loads return 0) and LDS stages never read.
+#pragma unroll
+  for (int e = 0; e < NEL; e++) elem(e, kbeg);
+  fetch(ra0, rb0);
+#pragma unroll
+  for (int e = 0; e < NEL; e++) elem(e, kbeg + BK);
+  fetch(ra1, rb1);
+#pragma unroll
+  for (int e = 0; e < NEL; e++) elem(e, kbeg + 2 * BK);
+  stash(ra0, rb0, 0);
+  __syncthreads();
+
+  // one iteration: compute slab `it` from LDS stage st, fetch slab it+2 into (rla, rlb), move slab
+  // it+1 from (rsa, rsb) to LDS stage st^1
+  auto body = [&](int it, int st, float4 (&rla)[GA], float4 (&rlb)[GB], const float4 (&rsa)[GA], const float4 (&rsb)[GB]) {
+    const int k3 = kbeg + (it + 3) * BK;
+    fetch(rla, rlb);
     __builtin_amdgcn_sched_barrier(0);
     const float4* Asc = As + st * KQ * LDA + wm * TM + l32;
     const float4* Bsc = Bs + st * KQ * LDB + wn * TN + l32;
@@ -246,20 +275,19 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
         if (e1 > e0) {
           __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int e = e0; e < e1; e++) elem(e, k2);
+          for (int e = e0; e < e1; e++) elem(e, k3);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    {
-      const int o = (st ^ 1) * KQ;
-#pragma unroll
-      for (int g = 0; g < GA; g++) As[(o + a_kq[g]) * LDA + a_col[g]] = ra[g];
-#pragma unroll
-      for (int g = 0; g < GB; g++) Bs[(o + b_kq[g]) * LDB + b_col[g]] = rb[g];
-    }
+    stash(rsa, rsb, st ^ 1);
     __syncthreads();
+  };
+  // the loop runs an even number of iterations: a trailing slab past kend is all zeros
+  for (int it = 0; it < niter; it += 2) {
+    body(it, 0, ra0, rb0, ra1, rb1);
+    body(it + 1, 1, ra1, rb1, ra0, rb0);
   }
 
   // D layout of a 32x32 block: column = lane % 32, row = 8*(v/4) + 4*(lane/32) + v%4
@@ -284,11 +312,26 @@ constexpr size_t igemm_smem_bytes() { return (size_t)2 * (BK / 4) * ((BM + 8 / (
 //   streamk    : `streamk` workers (about two per CU) share all k-slabs of all tiles evenly, which
 //                removes the idle tail of a grid with few tiles; tiles shared by two workers are
 //                finished with atomic adds, so the caller must have the output hold beta*C.
+// Blocks of one tile configuration that fit on a CU at once (registers and LDS), asked of the runtime once.
 template <int BM, int BN, int BK, class AL, class BL, class EP>
-bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, int splitK, int streamk = 0) {
+int igemm_blocks_per_cu() {
+  static int occ = 0;
+  if (occ == 0) {
+    int v = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, k_igemm<BM, BN, BK, AL, BL, EP, false>, 256, igemm_smem_bytes<BM, BN, BK>()) != hipSuccess || v < 1) v = 2;
+    occ = v;
+  }
+  return occ;
+}
+
+//   [col0, col1) : the columns this launch covers (col1 < 0: up to N); tiles are laid out from col0.
+template <int BM, int BN, int BK, class AL, class BL, class EP>
+bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, int splitK, int streamk = 0, int col0 = 0, int col1 = -1) {
   GemmShape gs;
-  gs.M = M; gs.N = N; gs.K = K;
-  gs.tilesM = (int)cdiv(M, BM); gs.tilesN = (int)cdiv(N, BN);
+  if (col1 < 0 || col1 > N) col1 = N;
+  if (col0 >= col1) return true;
+  gs.M = M; gs.N = col1; gs.K = K; gs.colBase = col0;
+  gs.tilesM = (int)cdiv(M, BM); gs.tilesN = (int)cdiv(col1 - col0, BN);
   if (splitK < 1) splitK = 1;
   int kper = (int)cdiv(cdiv(K, splitK), BK) * BK;
   if (kper < BK) kper = BK;
