@@ -163,9 +163,17 @@ void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float*
 /* batchNormTraining followed by relu(inPlace = true): y = max(bn(x), 0) */
 void lh_bn_train_fwd_relu(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
                           float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor);
-/* relu_grad(inPlace) followed by batchNorm_grad: dy counts only where y > 0 (dy itself is left untouched) */
-void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+/* relu_grad(inPlace) followed by batchNorm_grad: dy counts only where y > 0 (dy itself is left untouched).
+ * With `bias` (the layer's beta, unchanged since the forward call) the mask is recomputed from x as
+ * gamma*(x - mean)*invstd + bias > 0, bit-identical to the y that lh_bn_train_fwd_relu stored, and y
+ * is not read (it may be NULL); with bias == NULL the mask is read from y. */
+void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float* gamma, const float* bias,
+                    const float* save_mean, const float* save_invstd,
                     float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
+/* maxPool2D_batch_grad as a gather: every input pixel sums the dy of the windows whose argmax it is
+ * (no atomics, dx written once); dx = beta*dx + sum.  Same result as lh_maxpool_bwd. */
+void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float beta,
+                          int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad);
 /* `+` of two same-shape tensors followed by relu(inPlace = true), and the gradient of that pair:
  * g = dy where y > 0 else 0;  ad = abeta*ad + g;  bd = bbeta*bd + g  (ad or bd may be NULL) */
 void lh_add_relu(const float* a, const float* b, float* out, int64_t n);

@@ -278,8 +278,14 @@ class BackendHIP(Backend):
         self.lib.lh_maxpool_fwd(x.ptr, y.ptr, idx.ptr, N, C, H, W, kH, kW, sH, sW, pad); _lib.check()
         return y, idx
 
-    def maxPool2D_batch_grad(self, xd, dy, idx, n_out):
-        self.lib.lh_maxpool_bwd(dy.ptr, idx.ptr, xd.ptr, n_out); _lib.check()
+    def maxPool2D_batch_grad(self, xd, dy, idx, n_out, geom=None, beta=1.0):
+        """geom = (N, C, H, W, kH, kW, sH, sW, pad) selects the gather form, which can also overwrite (beta 0)."""
+        if geom is not None:
+            self.lib.lh_maxpool_bwd_dense(dy.ptr, idx.ptr, xd.ptr, beta, *geom)
+        else:
+            assert beta == 1.0
+            self.lib.lh_maxpool_bwd(dy.ptr, idx.ptr, xd.ptr, n_out)
+        _lib.check()
 
     def averagePool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW):
         P, Q = conv_size(H, kH, sH), conv_size(W, kW, sW)
@@ -305,10 +311,13 @@ class BackendHIP(Backend):
         f = self.lib.lh_bn_train_fwd_relu if relu else self.lib.lh_bn_train_fwd
         f(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
 
-    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0, y_relu=None):
+    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0, y_relu=None, bias=None):
+        """y_relu: the layer's output went through a fused in-place relu; `bias` (the layer's beta) lets the
+        kernel rebuild the relu mask from x instead of reading y."""
         xdp = xd.ptr if xd is not None else 0
         if y_relu is not None:
-            self.lib.lh_bn_bwd_relu(x.ptr, y_relu.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
+            self.lib.lh_bn_bwd_relu(x.ptr, y_relu.ptr, dy.ptr, scale.ptr, bias.ptr if bias is not None else 0, sm.ptr, si.ptr, xdp, beta_dx,
+                                    scaled.ptr, biasd.ptr, N, C, HW)
         else:
             self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
         _lib.check()

@@ -50,6 +50,13 @@ __device__ __forceinline__ void bn_foreach(int n0, int n1, int C, int c, int HW,
   }
 }
 
+// y = gamma * (x - mean) * invstd + beta with a fixed operation order (no contraction choices left to
+// the compiler): the backward pass of a fused BN+relu recomputes it to rebuild the relu mask, and
+// must get the forward's value bit for bit.
+__device__ __forceinline__ float bn_affine(float v, float mean, float invstd, float g, float b) {
+  return __fmaf_rn(__fmul_rn(__fsub_rn(v, mean), invstd), g, b);
+}
+
 template <bool VEC>
 __global__ void __launch_bounds__(TPB) k_bn_stats(const float* __restrict__ x, float* __restrict__ partial, int N, int C, int HW, int n_per) {
   __shared__ float sm[17];
@@ -104,38 +111,43 @@ __global__ void __launch_bounds__(TPB) k_bn_fwd_apply(const float* __restrict__ 
   const int n0 = s * n_per, n1 = min(N, n0 + n_per);
   bn_foreach<VEC>(n0, n1, C, c, HW,
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 r;
-      r.x = (v.x - mean) * invstd * g + b; r.y = (v.y - mean) * invstd * g + b;
-      r.z = (v.z - mean) * invstd * g + b; r.w = (v.w - mean) * invstd * g + b;
+      r.x = bn_affine(v.x, mean, invstd, g, b); r.y = bn_affine(v.y, mean, invstd, g, b);
+      r.z = bn_affine(v.z, mean, invstd, g, b); r.w = bn_affine(v.w, mean, invstd, g, b);
       if (RELU) { r.x = r.x < 0.f ? 0.f : r.x; r.y = r.y < 0.f ? 0.f : r.y; r.z = r.z < 0.f ? 0.f : r.z; r.w = r.w < 0.f ? 0.f : r.w; }
       *reinterpret_cast<float4*>(y + off) = r; },
-    [&](int64_t off) { float r = (x[off] - mean) * invstd * g + b; if (RELU) r = r < 0.f ? 0.f : r; y[off] = r; });
+    [&](int64_t off) { float r = bn_affine(x[off], mean, invstd, g, b); if (RELU) r = r < 0.f ? 0.f : r; y[off] = r; });
 }
 
 // RELU: the layer's output y went through an in-place relu; the incoming gradient counts only where y > 0.
-template <bool VEC, bool RELU>
+//   RELU == 1: the mask is read from the stored y;  RELU == 2: it is recomputed from x (y is not read).
+template <bool VEC, int RELU>
 __global__ void __launch_bounds__(TPB) k_bn_bwd_stats(const float* __restrict__ x, const float* __restrict__ yv, const float* __restrict__ dy,
-                                                      const float* save_mean, const float* save_invstd,
+                                                      const float* save_mean, const float* save_invstd, const float* gamma, const float* bias,
                                                       float* __restrict__ partial, int N, int C, int HW, int n_per) {
   __shared__ float sm[17];
   const int c = blockIdx.x, s = blockIdx.y;
   const int n0 = s * n_per, n1 = min(N, n0 + n_per);
   const float mean = save_mean[c], is = save_invstd[c];
+  const float ga = RELU == 2 ? gamma[c] : 0.f, bi = RELU == 2 ? bias[c] : 0.f;
   float s1 = 0.f, s2 = 0.f;
   bn_foreach<VEC>(n0, n1, C, c, HW,
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 g = *reinterpret_cast<const float4*>(dy + off);
-      if (RELU) { float4 m = *reinterpret_cast<const float4*>(yv + off);
+      if (RELU) { float4 m;
+        if (RELU == 1) m = *reinterpret_cast<const float4*>(yv + off);
+        else { m.x = bn_affine(v.x, mean, is, ga, bi); m.y = bn_affine(v.y, mean, is, ga, bi); m.z = bn_affine(v.z, mean, is, ga, bi); m.w = bn_affine(v.w, mean, is, ga, bi); }
         g.x = m.x > 0.f ? g.x : 0.f; g.y = m.y > 0.f ? g.y : 0.f; g.z = m.z > 0.f ? g.z : 0.f; g.w = m.w > 0.f ? g.w : 0.f; }
       s1 += (g.x + g.y) + (g.z + g.w);
       s2 += (g.x * ((v.x - mean) * is) + g.y * ((v.y - mean) * is)) + (g.z * ((v.z - mean) * is) + g.w * ((v.w - mean) * is)); },
-    [&](int64_t off) { float g = dy[off]; if (RELU) g = yv[off] > 0.f ? g : 0.f; s1 += g; s2 += g * ((x[off] - mean) * is); });
+    [&](int64_t off) { float g = dy[off]; if (RELU) { float m = RELU == 1 ? yv[off] : bn_affine(x[off], mean, is, ga, bi); g = m > 0.f ? g : 0.f; }
+      s1 += g; s2 += g * ((x[off] - mean) * is); });
   s1 = lh_block_sum(s1, sm);
   s2 = lh_block_sum(s2, sm);
   if (threadIdx.x == 0) { float* p = partial + 3 * ((int64_t)c * gridDim.y + s); p[0] = s1; p[1] = s2; }
 }
 
-template <bool VEC, bool ACC, bool RELU>
+template <bool VEC, bool ACC, int RELU>
 __global__ void __launch_bounds__(TPB) k_bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ yv, const float* __restrict__ dy, const float* __restrict__ partial,
-                                                      const float* gamma, const float* save_mean, const float* save_invstd,
+                                                      const float* gamma, const float* bias, const float* save_mean, const float* save_invstd,
                                                       float* __restrict__ dx, float* dgamma, float* dbeta, int N, int C, int HW, int n_per) {
   __shared__ float sh[2];
   const int c = blockIdx.x, s = blockIdx.y;
@@ -148,17 +160,20 @@ __global__ void __launch_bounds__(TPB) k_bn_bwd_apply(const float* __restrict__ 
   }
   __syncthreads();
   if (dx == nullptr) return;
-  const float m1 = sh[0], m2 = sh[1], mean = save_mean[c], is = save_invstd[c], g = gamma[c] * is;
+  const float m1 = sh[0], m2 = sh[1], mean = save_mean[c], is = save_invstd[c], ga = gamma[c], g = ga * is;
+  const float bi = RELU == 2 ? bias[c] : 0.f;
   const int n0 = s * n_per, n1 = min(N, n0 + n_per);
   bn_foreach<VEC>(n0, n1, C, c, HW,
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 d = *reinterpret_cast<const float4*>(dy + off); float4 r;
-      if (RELU) { float4 m = *reinterpret_cast<const float4*>(yv + off);
+      if (RELU) { float4 m;
+        if (RELU == 1) m = *reinterpret_cast<const float4*>(yv + off);
+        else { m.x = bn_affine(v.x, mean, is, ga, bi); m.y = bn_affine(v.y, mean, is, ga, bi); m.z = bn_affine(v.z, mean, is, ga, bi); m.w = bn_affine(v.w, mean, is, ga, bi); }
         d.x = m.x > 0.f ? d.x : 0.f; d.y = m.y > 0.f ? d.y : 0.f; d.z = m.z > 0.f ? d.z : 0.f; d.w = m.w > 0.f ? d.w : 0.f; }
       r.x = g * (d.x - m1 - (v.x - mean) * is * m2); r.y = g * (d.y - m1 - (v.y - mean) * is * m2);
       r.z = g * (d.z - m1 - (v.z - mean) * is * m2); r.w = g * (d.w - m1 - (v.w - mean) * is * m2);
       if (ACC) { float4 o = *reinterpret_cast<const float4*>(dx + off); r.x += o.x; r.y += o.y; r.z += o.z; r.w += o.w; }
       *reinterpret_cast<float4*>(dx + off) = r; },
-    [&](int64_t off) { float d = dy[off]; if (RELU) d = yv[off] > 0.f ? d : 0.f;
+    [&](int64_t off) { float d = dy[off]; if (RELU) { float m = RELU == 1 ? yv[off] : bn_affine(x[off], mean, is, ga, bi); d = m > 0.f ? d : 0.f; }
       float r = g * (d - m1 - (x[off] - mean) * is * m2); if (ACC) r += dx[off]; dx[off] = r; });
 }
 
@@ -209,7 +224,8 @@ static void bn_train_fwd_impl(bool relu, const float* x, const float* gamma, con
   LH_CHECK_LAUNCH();
 }
 
-static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, const float* gamma, const float* bias, int relu,
+                        const float* save_mean, const float* save_invstd,
                         float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_bwd: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_bwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
@@ -217,16 +233,13 @@ static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, co
   if (!get_partial()) return;
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx | (uintptr_t)y_relu) & 15) == 0);
   dim3 grid(C, p.slices);
-  const bool acc = beta_dx != 0.0f, relu = y_relu != nullptr;
-#define STATS(V, R) hipLaunchKernelGGL((k_bn_bwd_stats<V, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per)
-#define APPLY(V, A, R) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, (const float*)g_partial_ptr, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
-  if (p.vec4) {
-    if (relu) { STATS(true, true); if (acc) APPLY(true, true, true); else APPLY(true, false, true); }
-    else { STATS(true, false); if (acc) APPLY(true, true, false); else APPLY(true, false, false); }
-  } else {
-    if (relu) { STATS(false, true); if (acc) APPLY(false, true, true); else APPLY(false, false, true); }
-    else { STATS(false, false); if (acc) APPLY(false, true, false); else APPLY(false, false, false); }
-  }
+  const bool acc = beta_dx != 0.0f;
+#define STATS(V, R) hipLaunchKernelGGL((k_bn_bwd_stats<V, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, save_mean, save_invstd, gamma, bias, g_partial_ptr, N, C, HW, p.n_per)
+#define APPLY(V, A, R) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, (const float*)g_partial_ptr, gamma, bias, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
+#define BOTH(V, R) do { STATS(V, R); if (acc) APPLY(V, true, R); else APPLY(V, false, R); } while (0)
+  if (p.vec4) { if (relu == 2) BOTH(true, 2); else if (relu == 1) BOTH(true, 1); else BOTH(true, 0); }
+  else { if (relu == 2) BOTH(false, 2); else if (relu == 1) BOTH(false, 1); else BOTH(false, 0); }
+#undef BOTH
 #undef STATS
 #undef APPLY
   LH_CHECK_LAUNCH();
@@ -245,13 +258,13 @@ void lh_bn_train_fwd_relu(const float* x, const float* gamma, const float* beta,
 void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
   ProfScope prof_(CAT_BN_BWD);
-  bn_bwd_impl(x, nullptr, dy, gamma, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
+  bn_bwd_impl(x, nullptr, dy, gamma, nullptr, 0, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
 }
-void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float* gamma, const float* bias, const float* save_mean, const float* save_invstd,
                     float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
   ProfScope prof_(CAT_BN_BWD);
-  LH_REQUIRE(y != nullptr, "lh_bn_bwd_relu: y is required");
-  bn_bwd_impl(x, y, dy, gamma, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
+  LH_REQUIRE(y != nullptr || bias != nullptr, "lh_bn_bwd_relu: y or the layer's bias is required");
+  bn_bwd_impl(x, bias ? nullptr : y, dy, gamma, bias, bias ? 2 : 1, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
 }
 
 }  // extern "C"

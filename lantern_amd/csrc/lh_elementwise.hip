@@ -47,6 +47,24 @@ __global__ void __launch_bounds__(TPB) k_ew_scalar(float* out, const float* a, c
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
   for (int64_t j = i; j < n; j += st) out[j] = f(a[j], NIN > 1 ? b[j] : 0.f, NIN > 2 ? c[j] : 0.f);
 }
+// g = dy where y > 0 else 0, delivered to two gradient buffers in one pass
+template <bool ACC_A, bool ACC_B>
+__global__ void __launch_bounds__(TPB) k_add_relu_grad2(const float* __restrict__ y, const float* __restrict__ dy, float* __restrict__ ad, float* __restrict__ bd, int64_t n) {
+  int64_t n4 = n >> 2;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n4; j += st) {
+    float4 vy = reinterpret_cast<const float4*>(y)[j], g = reinterpret_cast<const float4*>(dy)[j];
+    g.x = vy.x > 0.f ? g.x : 0.f; g.y = vy.y > 0.f ? g.y : 0.f; g.z = vy.z > 0.f ? g.z : 0.f; g.w = vy.w > 0.f ? g.w : 0.f;
+    float4 ra = g, rb = g;
+    if (ACC_A) { float4 o = reinterpret_cast<const float4*>(ad)[j]; ra.x += o.x; ra.y += o.y; ra.z += o.z; ra.w += o.w; }
+    if (ACC_B) { float4 o = reinterpret_cast<const float4*>(bd)[j]; rb.x += o.x; rb.y += o.y; rb.z += o.z; rb.w += o.w; }
+    reinterpret_cast<float4*>(ad)[j] = ra; reinterpret_cast<float4*>(bd)[j] = rb;
+  }
+  for (int64_t j = 4 * n4 + i; j < n; j += st) {
+    float g = y[j] > 0.f ? dy[j] : 0.f;
+    ad[j] = ACC_A ? ad[j] + g : g; bd[j] = ACC_B ? bd[j] + g : g;
+  }
+}
 template <int NIN, class F>
 void ew(float* out, const float* a, const float* b, const float* c, int64_t n, F f) {
   if (n <= 0) return;
@@ -149,6 +167,17 @@ void lh_add_relu(const float* a, const float* b, float* out, int64_t n) { ProfSc
 }
 void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, float* bd, float bbeta, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
   // g = dy where y > 0 else 0 ; ad = abeta*ad + g ; bd = bbeta*bd + g   (either target may be NULL)
+  if (n <= 0) return;
+  LH_REQUIRE((abeta == 0.f || abeta == 1.f) && (bbeta == 0.f || bbeta == 1.f), "lh_add_relu_grad: beta must be 0 or 1");
+  if (ad && bd && ad != bd && al16(y) && al16(dy) && al16(ad) && al16(bd)) {
+    const int grid = stream_grid(n, TPB * 8);
+#define GO(A, B) hipLaunchKernelGGL((k_add_relu_grad2<A, B>), dim3(grid), dim3(TPB), 0, g_stream, y, dy, ad, bd, n)
+    if (abeta != 0.f) { if (bbeta != 0.f) GO(true, true); else GO(true, false); }
+    else { if (bbeta != 0.f) GO(false, true); else GO(false, false); }
+#undef GO
+    LH_CHECK_LAUNCH();
+    return;
+  }
   if (ad) {
     if (abeta == 0.f) ew<2>(ad, y, dy, nullptr, n, [] __device__(float yv, float g, float) { return yv > 0.f ? g : 0.f; });
     else ew<3>(ad, ad, y, dy, n, [] __device__(float d, float yv, float g) { return d + (yv > 0.f ? g : 0.f); });

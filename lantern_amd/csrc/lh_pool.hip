@@ -34,6 +34,27 @@ __global__ void __launch_bounds__(TPB) k_maxpool_bwd_atomic(const float* __restr
   int64_t o = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
   for (; o < n_out; o += st) atomicAdd(dx + idx[o], dy[o]);
 }
+// Gather form: one thread per input pixel; the windows that contain (h, w) are p in [p_lo, p_hi] x q in
+// [q_lo, q_hi]; a window contributes when its stored argmax is this pixel's flat index.
+template <bool ACC>
+__global__ void __launch_bounds__(TPB) k_maxpool_bwd_dense(const float* __restrict__ dy, const int* __restrict__ idx, float* __restrict__ dx,
+                                                           int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t n_in) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < n_in; i += st) {
+    const int w = (int)(i % W); const int64_t t = i / W; const int h = (int)(t % H); const int64_t nc = t / H;
+    const int hp = h + pad, wp = w + pad;
+    const int p_hi = min(oH - 1, hp / sH), q_hi = min(oW - 1, wp / sW);
+    const int p_lo = hp < kH ? 0 : (hp - kH) / sH + 1, q_lo = wp < kW ? 0 : (wp - kW) / sW + 1;
+    const int64_t ob = nc * oH * oW;
+    float acc = 0.f;
+    for (int p = p_lo; p <= p_hi; p++)
+      for (int q = q_lo; q <= q_hi; q++) {
+        const int64_t o = ob + (int64_t)p * oW + q;
+        if (idx[o] == (int)i) acc += dy[o];
+      }
+    dx[i] = ACC ? dx[i] + acc : acc;
+  }
+}
 __global__ void __launch_bounds__(TPB) k_avgpool_fwd(const float* __restrict__ x, float* __restrict__ y, int H, int W, int oH, int oW,
                                                      int kH, int kW, int sH, int sW, int64_t n_out) {
   const float ks = (float)(kH * kW);
@@ -80,6 +101,21 @@ void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out
   ProfScope prof_(CAT_POOL);
   if (n_out <= 0) return;
   hipLaunchKernelGGL(k_maxpool_bwd_atomic, dim3(stream_grid(n_out, TPB * 4)), dim3(TPB), 0, g_stream, dy, argmax, dx, n_out);
+  LH_CHECK_LAUNCH();
+}
+void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float beta,
+                          int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad) {
+  ProfScope prof_(CAT_POOL);
+  LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pad >= 0, "lh_maxpool_bwd_dense: kernel/stride must be >= 1 and pad >= 0");
+  LH_REQUIRE(H + 2 * pad >= kH && W + 2 * pad >= kW, "lh_maxpool_bwd_dense: image %dx%d too small for (%d,%d)", H, W, kH, kW);
+  LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_maxpool_bwd_dense: beta must be 0 or 1");
+  const int64_t n_in = (int64_t)N * C * H * W;
+  LH_REQUIRE(n_in < 2147483647LL, "lh_maxpool_bwd_dense: input too large for int32 argmax");
+  if (n_in <= 0) return;
+  const int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
+  const int grid = stream_grid(n_in, TPB * 2);
+  if (beta == 0.f) hipLaunchKernelGGL((k_maxpool_bwd_dense<false>), dim3(grid), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, oH, oW, kH, kW, sH, sW, pad, n_in);
+  else hipLaunchKernelGGL((k_maxpool_bwd_dense<true>), dim3(grid), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, oH, oW, kH, kW, sH, sW, pad, n_in);
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {

@@ -646,7 +646,7 @@ class TensorR:
         def back():
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()
             be.batchNorm_grad(self.x.data, xd, y.d.data, scale.x.data, scale.d.data, bias.d.data, sm, si, N, C, HW, beta,
-                              y_relu=ybuf if st["relu"] else None)
+                              y_relu=ybuf if st["relu"] else None, bias=bias.x.data)
         _tape.append(back)
         return y
 
@@ -676,7 +676,7 @@ class TensorR:
     # -- conv / pool ----------------------------------------------------------------------------------------------
     def convBBP(self, kernel, bias, strides, pads):
         be = get_backend()
-        assert self.isInput or self.d.scalarCount == self.x.scalarCount, "For convBBP, THIS is either input or intermediate stage"
+        assert self.isInput or self._d is None or self._d.scalarCount == self.x.scalarCount, "For convBBP, THIS is either input or intermediate stage"
         assert self.x.rank == 4, "For convBBP, THIS is dim 4: batch, channel, row, col"
         out, finput = self.x.conv2D_batch(kernel.x, bias.x if bias is not None else None, strides, pads)
         y = TensorR._new(out)
@@ -693,7 +693,12 @@ class TensorR:
         be = get_backend()
         yv, idx = self.x.maxPool2D_batch(kernels, strides, pads)
         y = TensorR._new(yv)
-        _tape.append(lambda: be.maxPool2D_batch_grad(self.d.data, y.d.data, idx, yv.scalarCount))
+        N, C, H, W = self.x.shape
+        geom = (N, C, H, W, kernels[0], kernels[1], strides[0], strides[1], pads[0] if pads else 0)
+        def back():
+            xd, beta = self.grad_target()
+            be.maxPool2D_batch_grad(xd, y.d.data, idx, yv.scalarCount, geom, beta)
+        _tape.append(back)
         return y
 
     def averagePoolBK(self, kernels, strides, pads=None):

@@ -177,7 +177,7 @@ class BackendCPU(Backend):
         self._c("lc_maxpool_fwd", P(x.ptr), P(y.ptr), P(idx.ptr), *[I(v) for v in (N, C_, H, W, kH, kW, sH, sW, pad)])
         return y, idx
 
-    def maxPool2D_batch_grad(self, xd, dy, idx, n_out): self._c("lc_maxpool_bwd", P(dy.ptr), P(idx.ptr), P(xd.ptr), L(n_out))
+    def maxPool2D_batch_grad(self, xd, dy, idx, n_out, geom=None, beta=1.0): self._c("lc_maxpool_bwd", P(dy.ptr), P(idx.ptr), P(xd.ptr), L(n_out))
 
     def averagePool2D_batch(self, x, N, C_, H, W, kH, kW, sH, sW):
         y = self.mallocArray(N * C_ * conv_size(H, kH, sH) * conv_size(W, kW, sW))
@@ -198,7 +198,7 @@ class BackendCPU(Backend):
                 I(N), I(C_), I(HW), F(eps), F(factor))
         return y, sm, si
 
-    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C_, HW, beta_dx=1.0, y_relu=None):
+    def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C_, HW, beta_dx=1.0, y_relu=None, bias=None):
         if y_relu is not None:      # the unfused sequence: relu_grad(inPlace) on dy, then batchNorm_grad
             self.unary_grad(0, y_relu, y_relu, dy, dy, N * C_ * HW, inPlace=True)
         self._c("lc_bn_bwd", P(x.ptr), P(dy.ptr), P(scale.ptr), P(sm.ptr), P(si.ptr), P(xd.ptr if xd is not None else 0),

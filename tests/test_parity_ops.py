@@ -70,7 +70,14 @@ def test_batchnorm_training_and_grad(pair, shape, relu):
         DY = up(dy); dg, db = be.mallocArray(Cc), be.mallocArray(Cc)
         if relu:
             xd = up(dx0)
-            be.batchNorm_grad(X, xd, DY, G, dg, db, sm, si, N, Cc, HW, beta_dx=1.0, y_relu=y) if be.name == "hip" else _cpu_bn_relu_grad(be, X, xd, DY, y, G, dg, db, sm, si, N, Cc, HW)
+            if be.name == "hip":
+                be.batchNorm_grad(X, xd, DY, G, dg, db, sm, si, N, Cc, HW, beta_dx=1.0, y_relu=y, bias=Bi)      # mask rebuilt from x
+                xd1 = up(dx0); dg1, db1 = be.mallocArray(Cc), be.mallocArray(Cc)
+                be.batchNorm_grad(X, xd1, up(dy), G, dg1, db1, sm, si, N, Cc, HW, beta_dx=1.0, y_relu=y)             # mask read from y
+                for a, b_ in ((xd, xd1), (dg, dg1), (db, db1)):
+                    np.testing.assert_array_equal(be.toHost(a, a.n), be.toHost(b_, b_.n), err_msg="relu mask from x differs from the stored y")
+            else:
+                _cpu_bn_relu_grad(be, X, xd, DY, y, G, dg, db, sm, si, N, Cc, HW)
         else:
             xd = up(dx0)
             be.batchNorm_grad(X, xd, DY, G, dg, db, sm, si, N, Cc, HW)
@@ -126,7 +133,10 @@ def test_maxpool_values_argmax_and_grad(pair, p):
         y, idx = be.maxPool2D_batch(up(x), N, Cc, H, W, kH, kW, sH, sW, pad)
         xd = up(np.ones(x.size, np.float32))
         be.maxPool2D_batch_grad(xd, up(dy), idx, N * Cc * P * Q)
-        return [down(y, dy.shape), down(idx, dy.shape, np.int32), down(xd, x.shape)]
+        geom = (N, Cc, H, W, kH, kW, sH, sW, pad)
+        xg = up(np.ones(x.size, np.float32)); be.maxPool2D_batch_grad(xg, up(dy), idx, N * Cc * P * Q, geom, 1.0)      # gather form, accumulate
+        xo = up(np.full(x.size, 7.0, np.float32)); be.maxPool2D_batch_grad(xo, up(dy), idx, N * Cc * P * Q, geom, 0.0)  # gather form, overwrite
+        return [down(y, dy.shape), down(idx, dy.shape, np.int32), down(xd, x.shape), down(xg, x.shape), down(xo, x.shape) + (7.0 if be.name == "hip" else 0.0)]
 
     outs = pair.run(f)
     check_all(outs, exact=(0, 1), rtol=1e-5)     # values and indices bit-exact; overlapping windows sum in any order
