@@ -22,7 +22,7 @@ if ROOT not in sys.path:
 import numpy as np  # noqa: E402
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
-CATS = ["conv_fwd", "conv_bwd_data", "conv_bwd_filter", "gemm", "bn_fwd", "bn_bwd", "elementwise", "pool", "reduce", "optim", "fill"]
+CATS = ["conv_fwd", "conv_bwd_data", "conv_bwd_filter", "gemm", "bn_fwd", "bn_bwd", "elementwise", "pool", "reduce", "optim", "fill", "rnn"]
 
 
 def conv_flops(model, batch, hw):

@@ -158,6 +158,24 @@ void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, floa
 void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
 
+/* ---- recurrent layer and CTC (DeepSpeech2 path) --------------------------------------------------
+ * RNNBase over cudnnRNNForwardTraining / BackwardData / BackwardWeights (NNModule.scala:332-417,
+ * CDN:1638-1893): one layer, mode 0 = relu, 1 = tanh, optionally bidirectional, zero initial state.
+ *   x [T,B,I];  y [T,B,D*H] (D = 2 when bidirectional: forward half, then reverse half) holds the hidden
+ *   states and is all the backward pass needs besides x;  w = packed parameters, per direction
+ *   W_ih[H,I], W_hh[H,H], b_ih[H], b_hh[H] (NNModule.scala:378-390), forward direction first.
+ * lh_rnn_bwd: dx = beta_dx*dx + ... (dx may be NULL), dw += ...; takes T*B*D*H + D*H*H + ... floats of
+ * scratch from the top of the arena and releases them before returning. */
+void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir);
+void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
+                int T, int B, int I, int H, int bidir);
+/* ctcLoss (TD:349; CDN:1895-1938, cudnnCTCLoss): probs [T,B,A] are softmax outputs, class 0 is the blank;
+ * h_labels (concatenated), h_label_len [B], h_input_len [B] are HOST arrays as in the cuDNN call;
+ * costs[b] = -log p(labels_b | probs).  When dprobs is not NULL the gradient with respect to the
+ * pre-softmax activations (probs - posterior, what cuDNN reports) is ADDED to it, unscaled. */
+void lh_ctc_loss(const float* probs, float* dprobs, const int* h_labels, const int* h_label_len, const int* h_input_len,
+                 float* costs, int T, int B, int A);
+
 /* ---- fusions of adjacent trait calls (no single counterpart in the reference; each gives the
  *      result of the sequence it replaces, in one pass over memory) ------------------------ */
 /* batchNormTraining followed by relu(inPlace = true): y = max(bn(x), 0) */

@@ -404,6 +404,23 @@ class BackendHIP(Backend):
         ptrs = (C.c_void_p * len(dbufs))(*[(b.ptr if b is not None else 0) for b in dbufs])
         self.lib.lh_concat_grad(len(dbufs), ptrs, _ints(sizes), outd.ptr, outer, inner); _lib.check()
 
+    # -- recurrent layer, CTC (CDN:1638-1938) ------------------------------------------------------------
+    def ctcLoss(self, probs, probs_d, input_lengths, labels, label_lengths, T, B, A):
+        """probs [T,B,A] after softmax; lengths and labels are host int arrays; returns per-sample costs [B]."""
+        costs = self.mallocArray(B, zero=False)
+        il = np.ascontiguousarray(input_lengths, np.int32); lb = np.ascontiguousarray(labels, np.int32); ll = np.ascontiguousarray(label_lengths, np.int32)
+        self.lib.lh_ctc_loss(probs.ptr, probs_d.ptr if probs_d is not None else 0, lb.ctypes.data, ll.ctypes.data, il.ctypes.data, costs.ptr, T, B, A)
+        _lib.check()
+        return costs
+
+    def rnn_forward(self, mode, x, w, T, B, I, H, bidir):
+        y = self.mallocArray(T * B * H * (2 if bidir else 1), zero=False)
+        self.lib.lh_rnn_fwd(mode, x.ptr, w.ptr, y.ptr, T, B, I, H, int(bidir)); _lib.check()
+        return y
+
+    def rnn_backward(self, mode, x, y, dy, w, dx, dw, T, B, I, H, bidir, beta_dx=1.0):
+        self.lib.lh_rnn_bwd(mode, x.ptr, y.ptr, dy.ptr, w.ptr, dx.ptr if dx is not None else 0, beta_dx, dw.ptr, T, B, I, H, int(bidir)); _lib.check()
+
     # -- optimizers ----------------------------------------------------------------------------------------
     def sgd_update(self, x, d, lr, n):
         self.lib.lh_sgd(x.ptr, d.ptr, lr, n); _lib.check()

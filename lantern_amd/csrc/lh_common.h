@@ -33,7 +33,7 @@ bool failed();
 // ---- per-category timing with HIP events on g_stream (off unless lh_prof_enable was called) ----
 enum {
   CAT_CONV_FWD = 0, CAT_CONV_BWD_DATA, CAT_CONV_BWD_FILTER, CAT_GEMM, CAT_BN_FWD, CAT_BN_BWD,
-  CAT_ELEMENTWISE, CAT_POOL, CAT_REDUCE, CAT_OPTIM, CAT_FILL, CAT_COUNT
+  CAT_ELEMENTWISE, CAT_POOL, CAT_REDUCE, CAT_OPTIM, CAT_FILL, CAT_RNN, CAT_COUNT
 };
 extern unsigned g_prof_mask;
 void prof_begin(int cat);

@@ -1,0 +1,305 @@
+// Elman RNN layer (tanh / relu, optionally bidirectional) forward and backward, and the CTC loss.
+// Reference behaviour being replaced: RNNBase (NNModule.scala:332-417) over cudnnRNNForwardTraining /
+// cudnnRNNBackwardData / cudnnRNNBackwardWeights (CDN:1638-1893), and cudnnCTCLoss (CDN:1895-1938).
+//
+//   h_t = act(W_ih x_t + b_ih + W_hh h_{t-1} + b_hh),  h_{-1} = 0,   y[t,b,:] = [h_t forward ; h_t reverse]
+//
+// The input projection of all time steps and the three weight/input gradients are large GEMMs
+// (lh_sgemm, MFMA).  Only the recurrence is sequential: one small kernel per time step, both
+// directions in the same launch, each block producing 16 hidden units for the whole batch from
+// W_hh rows held in registers.  The output y doubles as the saved hidden states.
+#include "lh_common.h"
+#include "../../include/lantern_hip.h"
+using namespace lh;
+
+namespace {
+constexpr int TPB = 256;
+constexpr int JT = 16;            // hidden units per block (4 per wavefront)
+constexpr int KMAX = 32;          // K values per lane: supports H up to 64 * 32 = 2048
+
+__device__ __forceinline__ float act_fwd(int mode, float v) { return mode == 1 ? tanhf(v) : (v < 0.f ? 0.f : v); }
+
+// One time step of both directions.
+//   out[b, j] = act(pre[b, j] + bias1[j] + bias2[j] + sum_k prev[b, k] * Wrow[j, k])       (forward)
+// pre/out alias inside y: row stride ld.  dir = blockIdx.y picks the direction's weights and time index.
+struct StepArgs {
+  float* cur[2];              // y + t*B*ld + d*H        (pre-activation in, hidden state out)
+  const float* prev[2];       // y + tp*B*ld + d*H, or nullptr at the first step
+  const float* W[2];          // W_hh of the direction, [H, H] rows = output units
+  const float* b1[2]; const float* b2[2];
+};
+__global__ void __launch_bounds__(TPB) k_rnn_fwd_step(StepArgs a, int B, int H, int ld, int mode) {
+  const int d = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int j0 = blockIdx.x * JT + wave * 4;
+  float* cur = a.cur[d]; const float* prev = a.prev[d]; const float* W = a.W[d];
+  const int nk = (H + 63) >> 6;
+  float w[4][KMAX];
+#pragma unroll
+  for (int c = 0; c < 4; c++)
+#pragma unroll
+    for (int i = 0; i < KMAX; i++) { const int k = lane + 64 * i; w[c][i] = (i < nk && k < H && j0 + c < H && prev) ? W[(int64_t)(j0 + c) * H + k] : 0.f; }
+  for (int b = 0; b < B; b++) {
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    if (prev) {
+#pragma unroll
+      for (int i = 0; i < KMAX; i++) {
+        if (i < nk) {
+          const int k = lane + 64 * i;
+          const float h = k < H ? prev[(int64_t)b * ld + k] : 0.f;
+#pragma unroll
+          for (int c = 0; c < 4; c++) s[c] = fmaf(h, w[c][i], s[c]);
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; c++) s[c] = lh_wave_sum(s[c]);
+    if (lane == 0) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const int j = j0 + c;
+        if (j < H) cur[(int64_t)b * ld + j] = act_fwd(mode, cur[(int64_t)b * ld + j] + a.b1[d][j] + a.b2[d][j] + s[c]);
+      }
+    }
+  }
+}
+
+// One backward time step of both directions:
+//   dpre[b, j]  = (dy[b, j] + dh_in[b, j]) * act'(h[b, j])                 (every block needs all j; it stores only its own 16)
+//   dh_out[b, i] = sum_j dpre[b, j] * Wt[i, j]                             (Wt = W_hh transposed, rows = i)
+struct BwdArgs {
+  const float* dy[2]; const float* h[2]; float* dpre[2];          // time slice t, direction offset applied, row stride ld
+  const float* dh_in[2]; float* dh_out[2];                          // [B, H] dense; dh_in nullptr at the first (last in time) step
+  const float* Wt[2];
+};
+__global__ void __launch_bounds__(TPB) k_rnn_bwd_step(BwdArgs a, int B, int H, int ld, int mode) {
+  const int d = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int i0 = blockIdx.x * JT + wave * 4;
+  const float* Wt = a.Wt[d];
+  const int nk = (H + 63) >> 6;
+  float w[4][KMAX];
+#pragma unroll
+  for (int c = 0; c < 4; c++)
+#pragma unroll
+    for (int i = 0; i < KMAX; i++) { const int k = lane + 64 * i; w[c][i] = (i < nk && k < H && i0 + c < H) ? Wt[(int64_t)(i0 + c) * H + k] : 0.f; }
+  const int jlo = blockIdx.x * JT, jhi = min(H, jlo + JT);
+  for (int b = 0; b < B; b++) {
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < KMAX; i++) {
+      if (i < nk) {
+        const int j = lane + 64 * i;
+        float g = 0.f;
+        if (j < H) {
+          const float hv = a.h[d][(int64_t)b * ld + j];
+          g = a.dy[d][(int64_t)b * ld + j] + (a.dh_in[d] ? a.dh_in[d][(int64_t)b * H + j] : 0.f);
+          g = mode == 1 ? g * (1.0f - hv * hv) : (hv > 0.f ? g : 0.f);
+          if (wave == 0 && j >= jlo && j < jhi) a.dpre[d][(int64_t)b * ld + j] = g;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) s[c] = fmaf(g, w[c][i], s[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; c++) s[c] = lh_wave_sum(s[c]);
+    if (lane == 0) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) if (i0 + c < H) a.dh_out[d][(int64_t)b * H + i0 + c] = s[c];
+    }
+  }
+}
+
+// db1[j] += colsum[j]; db2[j] += colsum[j]
+__global__ void __launch_bounds__(TPB) k_rnn_bias_grad(const float* __restrict__ colsum, float* db1, float* db2, int H) {
+  int j = blockIdx.x * TPB + threadIdx.x;
+  if (j < H) { float v = colsum[j]; db1[j] += v; db2[j] += v; }
+}
+
+static size_t dir_params(int I, int H) { return (size_t)H * I + (size_t)H * H + 2 * (size_t)H; }
+
+// ---- CTC ----------------------------------------------------------------------------------------------
+// One block per sample; threads over the 2L+1 states of the blank-extended label string; time is a loop.
+// Scaled forward-backward in double precision (the per-step normaliser keeps alpha in range).
+constexpr int CTC_TPB = 128;
+__device__ __forceinline__ double block_sum_d(double v, double* sm) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  __syncthreads();
+  if (lane == 0) sm[wave] = v;
+  __syncthreads();
+  double t = 0.0;
+  for (int i = 0; i < (int)(blockDim.x >> 6); i++) t += sm[i];
+  return t;
+}
+__global__ void __launch_bounds__(CTC_TPB) k_ctc(const float* __restrict__ probs, float* dprobs, const int* __restrict__ labels, const int* __restrict__ label_off,
+                                                 const int* __restrict__ label_len, const int* __restrict__ input_len, float* costs,
+                                                 double* alpha_all, double* beta_all, double* cn_all, int T, int B, int A, int Smax) {
+  __shared__ double sm[4];
+  const int b = blockIdx.x;
+  const int L = label_len[b], Tb = input_len[b], S = 2 * L + 1;
+  const int* lab = labels + label_off[b];
+  double* alpha = alpha_all + (size_t)b * T * Smax; double* beta = beta_all + (size_t)b * T * Smax; double* cn = cn_all + (size_t)b * T;
+  auto cls = [&](int s) { return (s & 1) ? lab[s >> 1] : 0; };
+  auto P = [&](int t, int s) { return (double)probs[((size_t)t * B + b) * A + cls(s)]; };
+  double ll = 0.0;
+  for (int t = 0; t < Tb; t++) {
+    double part = 0.0;
+    for (int s = threadIdx.x; s < S; s += CTC_TPB) {
+      double a;
+      if (t == 0) a = s < 2 ? P(0, s) : 0.0;
+      else {
+        const double* ap = alpha + (size_t)(t - 1) * Smax;
+        a = ap[s];
+        if (s >= 1) a += ap[s - 1];
+        if (s >= 2 && (s & 1) && lab[s >> 1] != lab[(s >> 1) - 1]) a += ap[s - 2];
+        a *= P(t, s);
+      }
+      alpha[(size_t)t * Smax + s] = a; part += a;
+    }
+    const double c = block_sum_d(part, sm);
+    if (c > 0.0) for (int s = threadIdx.x; s < S; s += CTC_TPB) alpha[(size_t)t * Smax + s] /= c;
+    if (threadIdx.x == 0) cn[t] = c;
+    ll += log(c);
+    __syncthreads();
+  }
+  for (int s = threadIdx.x; s < S; s += CTC_TPB) beta[(size_t)(Tb - 1) * Smax + s] = (s >= S - 2) ? 1.0 : 0.0;
+  __syncthreads();
+  for (int t = Tb - 2; t >= 0; t--) {
+    const double* bp = beta + (size_t)(t + 1) * Smax; const double c = cn[t + 1];
+    for (int s = threadIdx.x; s < S; s += CTC_TPB) {
+      double v = bp[s] * P(t + 1, s);
+      if (s + 1 < S) v += bp[s + 1] * P(t + 1, s + 1);
+      if (s + 2 < S && ((s + 2) & 1) && lab[(s + 2) >> 1] != lab[s >> 1]) v += bp[s + 2] * P(t + 1, s + 2);
+      beta[(size_t)t * Smax + s] = v / c;
+    }
+    __syncthreads();
+  }
+  const double* al = alpha + (size_t)(Tb - 1) * Smax;
+  const double pfin = al[S - 1] + (S > 1 ? al[S - 2] : 0.0);
+  if (threadIdx.x == 0) costs[b] = (float)(-(ll + log(pfin)));
+  if (dprobs == nullptr) return;
+  // d cost / d activation = probs - posterior(class), the gradient cuDNN reports; accumulated
+  for (int idx = threadIdx.x; idx < Tb * A; idx += CTC_TPB) {
+    const int t = idx / A, k = idx - t * A;
+    double acc = 0.0;
+    for (int s = (k == 0 ? 0 : 1); s < S; s += 2) if (cls(s) == k) acc += alpha[(size_t)t * Smax + s] * beta[(size_t)t * Smax + s];
+    const size_t i = ((size_t)t * B + b) * A + k;
+    dprobs[i] += (float)((double)probs[i] - acc / pfin);
+  }
+}
+}  // namespace
+
+extern "C" {
+
+void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+  LH_REQUIRE(mode == 0 || mode == 1, "lh_rnn_fwd: mode %d (0 = relu, 1 = tanh)", mode);
+  LH_REQUIRE(T >= 1 && B >= 1 && I >= 1 && H >= 1, "lh_rnn_fwd: bad shape T%d B%d I%d H%d", T, B, I, H);
+  LH_REQUIRE(H <= 64 * KMAX, "lh_rnn_fwd: hidden size %d above %d", H, 64 * KMAX);
+  LH_REQUIRE(x && w && y, "lh_rnn_fwd: null operand");
+  const int D = bidir ? 2 : 1, ld = D * H;
+  for (int d = 0; d < D; d++) {          // input projection of every step straight into y
+    const float* Wih = w + d * dir_params(I, H);
+    lh_sgemm(0, 1, T * B, H, I, 1.0f, x, I, Wih, I, 0.0f, y + d * H, ld);
+  }
+  ProfScope prof_(CAT_RNN);
+  for (int step = 0; step < T; step++) {
+    StepArgs a;
+    for (int d = 0; d < 2; d++) {
+      const int dd = d < D ? d : 0;
+      const float* Wih = w + dd * dir_params(I, H); const float* Whh = Wih + (size_t)H * I;
+      const int t = dd == 0 ? step : T - 1 - step, tp = dd == 0 ? t - 1 : t + 1;
+      a.cur[d] = y + (size_t)t * B * ld + dd * H;
+      a.prev[d] = step == 0 ? nullptr : y + (size_t)tp * B * ld + dd * H;
+      a.W[d] = Whh; a.b1[d] = Whh + (size_t)H * H; a.b2[d] = a.b1[d] + H;
+    }
+    hipLaunchKernelGGL(k_rnn_fwd_step, dim3((unsigned)cdiv(H, JT), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode);
+  }
+  LH_CHECK_LAUNCH();
+}
+
+void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
+                int T, int B, int I, int H, int bidir) {
+  LH_REQUIRE(mode == 0 || mode == 1, "lh_rnn_bwd: mode %d (0 = relu, 1 = tanh)", mode);
+  LH_REQUIRE(T >= 1 && B >= 1 && I >= 1 && H >= 1, "lh_rnn_bwd: bad shape T%d B%d I%d H%d", T, B, I, H);
+  LH_REQUIRE(H <= 64 * KMAX, "lh_rnn_bwd: hidden size %d above %d", H, 64 * KMAX);
+  LH_REQUIRE(beta_dx == 0.f || beta_dx == 1.f, "lh_rnn_bwd: beta must be 0 or 1");
+  LH_REQUIRE(x && y && dy && w && dw, "lh_rnn_bwd: null operand");
+  const int D = bidir ? 2 : 1, ld = D * H;
+  // scratch from the top of the arena: dpre [T*B, D*H], W_hh^T per direction, two dh buffers per direction, column sums
+  const size_t n_dpre = (size_t)T * B * ld, n_wt = (size_t)D * H * H, n_dh = (size_t)2 * D * B * H, n_cs = (size_t)ld;
+  const size_t bytes = (n_dpre + n_wt + n_dh + n_cs) * sizeof(float);
+  float* scratch = (float*)lh_malloc_uninit(bytes);
+  if (scratch == nullptr) return;
+  float* dpre = scratch; float* wt = dpre + n_dpre; float* dh = wt + n_wt; float* colsum = dh + n_dh;
+  for (int d = 0; d < D; d++) {
+    const float* Whh = w + d * dir_params(I, H) + (size_t)H * I;
+    lh_trans(Whh, wt + (size_t)d * H * H, H, H);
+  }
+  {
+    ProfScope prof_(CAT_RNN);
+    for (int step = T - 1; step >= 0; step--) {
+      BwdArgs a;
+      const int cur_buf = (T - 1 - step) & 1;
+      for (int d = 0; d < 2; d++) {
+        const int dd = d < D ? d : 0;
+        const int t = dd == 0 ? step : T - 1 - step;
+        const size_t off = (size_t)t * B * ld + dd * H;
+        a.dy[d] = dy + off; a.h[d] = y + off; a.dpre[d] = dpre + off;
+        a.dh_in[d] = step == T - 1 ? nullptr : dh + ((size_t)(cur_buf ^ 1) * D + dd) * B * H;
+        a.dh_out[d] = dh + ((size_t)cur_buf * D + dd) * B * H;
+        a.Wt[d] = wt + (size_t)dd * H * H;
+      }
+      hipLaunchKernelGGL(k_rnn_bwd_step, dim3((unsigned)cdiv(H, JT), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode);
+    }
+  }
+  lh_sum_dim(dpre, colsum, 1, T * B, ld);
+  for (int d = 0; d < D; d++) {
+    const size_t off = d * dir_params(I, H);
+    const float* Wih = w + off;
+    float* dWih = dw + off; float* dWhh = dWih + (size_t)H * I; float* dbih = dWhh + (size_t)H * H; float* dbhh = dbih + H;
+    lh_sgemm(1, 0, H, I, T * B, 1.0f, dpre + d * H, ld, x, I, 1.0f, dWih, I);
+    if (T > 1) {
+      // dW_hh += sum_t dpre_t^T h_{prev(t)}: forward pairs (t, t-1), reverse pairs (t, t+1)
+      const float* A = d == 0 ? dpre + (size_t)B * ld + d * H : dpre + d * H;
+      const float* Bm = d == 0 ? y + d * H : y + (size_t)B * ld + d * H;
+      lh_sgemm(1, 0, H, H, (T - 1) * B, 1.0f, A, ld, Bm, ld, 1.0f, dWhh, H);
+    }
+    hipLaunchKernelGGL(k_rnn_bias_grad, dim3((unsigned)cdiv(H, TPB)), dim3(TPB), 0, g_stream, colsum + d * H, dbih, dbhh, H);
+    if (dx) lh_sgemm(0, 0, T * B, I, H, 1.0f, dpre + d * H, ld, Wih, I, d == 0 ? beta_dx : 1.0f, dx, I);
+  }
+  lh_free_top(bytes);      // stream order: the kernels above run before anything that reuses the space
+  LH_CHECK_LAUNCH();
+}
+
+void lh_ctc_loss(const float* probs, float* dprobs, const int* h_labels, const int* h_label_len, const int* h_input_len,
+                 float* costs, int T, int B, int A) {
+  ProfScope prof_(CAT_REDUCE);
+  LH_REQUIRE(T >= 1 && B >= 1 && A >= 2, "lh_ctc_loss: bad shape T%d B%d A%d", T, B, A);
+  LH_REQUIRE(probs && costs && h_labels && h_label_len && h_input_len, "lh_ctc_loss: null operand");
+  int total = 0, Lmax = 0;
+  int* host = (int*)malloc(sizeof(int) * (size_t)(3 * B));
+  if (!host) { LH_FAIL("lh_ctc_loss: out of host memory"); return; }
+  for (int b = 0; b < B; b++) {
+    const int L = h_label_len[b], Tb = h_input_len[b];
+    if (L < 0 || Tb < 1 || Tb > T || Tb < L) { free(host); LH_FAIL("lh_ctc_loss: sample %d has label length %d and input length %d (T = %d)", b, L, Tb, T); return; }
+    host[b] = total; host[B + b] = L; host[2 * B + b] = Tb;
+    total += L; if (L > Lmax) Lmax = L;
+  }
+  for (int i = 0; i < total; i++) if (h_labels[i] < 1 || h_labels[i] >= A) { free(host); LH_FAIL("lh_ctc_loss: label %d outside 1..%d (0 is the blank)", h_labels[i], A - 1); return; }
+  const int Smax = 2 * Lmax + 1;
+  const size_t n_int = (size_t)3 * B + (size_t)(total > 0 ? total : 1);
+  const size_t int_bytes = ((n_int * sizeof(int)) + 255) & ~(size_t)255;
+  const size_t dbl = ((size_t)2 * B * T * Smax + (size_t)B * T) * sizeof(double);
+  char* scratch = (char*)lh_malloc_uninit(int_bytes + dbl);
+  if (scratch == nullptr) { free(host); return; }
+  int* d_int = (int*)scratch;
+  lh_h2d(d_int, host, sizeof(int) * (size_t)(3 * B));
+  if (total > 0) lh_h2d(d_int + 3 * B, h_labels, sizeof(int) * (size_t)total);
+  free(host);
+  double* alpha = (double*)(scratch + int_bytes); double* beta = alpha + (size_t)B * T * Smax; double* cn = beta + (size_t)B * T * Smax;
+  hipLaunchKernelGGL(k_ctc, dim3(B), dim3(CTC_TPB), 0, g_stream, probs, dprobs, d_int + 3 * B, d_int, d_int + B, d_int + 2 * B, costs, alpha, beta, cn, T, B, A, Smax);
+  lh_free_top(int_bytes + dbl);
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"

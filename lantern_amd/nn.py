@@ -102,6 +102,26 @@ class BatchNorm1D(BatchNorm2D):
         return x.batchNorm1D(self.scale, self.bias, self.runningMean, self.runningVar)
 
 
+class RNNBase(Module):
+    """NN:332-417: one parameter buffer holding, per layer and direction, w_ih [gate, in], w_hh [gate, hidden],
+    b_ih, b_hh (forward direction first), initialised with Tensor.rand(size, 0.01).  Modes: "relu", "tanh"."""
+    MODES = {"relu": 0, "tanh": 1}
+
+    def __init__(self, mode, inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, name="rnn"):
+        super().__init__(name)
+        assert mode in self.MODES, "RNN mode %r is not built (relu and tanh are)" % (mode,)
+        assert inputSize >= 1, "Input size must be at least 1"
+        assert hiddenSize >= 1, "Hidden size must be at least 1"
+        assert numLayers == 1, "one layer per RNNBase (the DeepSpeech program stacks single-layer modules)"
+        assert dropout == 0.0, "dropout between layers is not built"
+        self.mode, self.inputSize, self.hiddenSize, self.bidirectional = self.MODES[mode], inputSize, hiddenSize, bidirectional
+        per_dir = hiddenSize * inputSize + hiddenSize * hiddenSize + 2 * hiddenSize
+        self.parameterBuffer = self.param("parameterBuffer", Tensor.rand((per_dir * (2 if bidirectional else 1),), 0.01))
+
+    def __call__(self, x):
+        return x.rnn(self.mode, self.parameterBuffer, self.hiddenSize, self.bidirectional)
+
+
 # ---- optimizers (NN:255-303) -------------------------------------------------------------------
 class Optim:
     def __init__(self, module):

@@ -727,6 +727,33 @@ class TensorR:
         _tape.append(lambda: be.concat_grad([None if t.isInput else t.d.data for t in ts], sizes, y.d.data, outer, inner))
         return y
 
+    # -- recurrent layer, CTC ----------------------------------------------------------------------------
+    def rnn(self, mode, params, hidden, bidirectional):
+        """RNNBase.apply (NN:392-415): one layer over [seqLength, batch, inputSize], zero initial state;
+        `params` is the packed parameter buffer (a TensorR).  mode 0 = relu, 1 = tanh."""
+        be = get_backend()
+        assert self.x.rank == 3, "RNN input should have rank 3: [seqLength x batchSize x inputSize]"
+        T, Bn, I = self.x.shape
+        D = 2 if bidirectional else 1
+        ybuf = be.rnn_forward(mode, self.x.data, params.x.data, T, Bn, I, hidden, bidirectional)
+        y = TensorR._new(Tensor(ybuf, (T, Bn, D * hidden)))
+        def back():
+            xd, beta = (None, 1.0) if self.isInput else self.grad_target()
+            be.rnn_backward(mode, self.x.data, ybuf, y.d.data, params.x.data, xd, params.d.data, T, Bn, I, hidden, bidirectional, beta)
+        _tape.append(back)
+        return y
+
+    def ctcLoss(self, inputLengths, labels, labelLengths):
+        """TD:1381-1382 + CDN:1895-1938: `self` holds softmax outputs [T, B, A]; the per-sample costs are
+        averaged into the returned 1-element Tensor and the gradient is written into self.d right away
+        (there is no tape entry: the result is a plain Tensor, as in the reference)."""
+        be = get_backend()
+        assert self.x.rank == 3, "Probability tensor should have rank 3: [inputLength, batchSize, alphabetSize]"
+        T, Bn, A = self.x.shape
+        assert Bn <= 256, "'cudnnGetCTCLossWorkspaceSize' requires batch size less than 256, got %d" % Bn
+        costs = be.ctcLoss(self.x.data, self.d.data, inputLengths, labels, labelLengths, T, Bn, A)
+        return Tensor(costs, (Bn,)).mean()
+
     def dropout(self, prob):
         be = get_backend()
         yv, mask = self.x.dropout(prob)

@@ -264,6 +264,23 @@ class BackendCPU(Backend):
         ptrs = (C.c_void_p * len(keep))(*[b.ptr for b in keep])
         self._c("lc_concat_grad", I(len(keep)), ptrs, _ints(sizes), P(outd.ptr), I(outer), I(inner))
 
+    def ctcLoss(self, probs, probs_d, input_lengths, labels, label_lengths, T, B, A):
+        """probs [T,B,A] after softmax; lengths and labels are host int arrays; returns per-sample costs [B]."""
+        costs = self.mallocArray(B)
+        il = np.ascontiguousarray(input_lengths, np.int32); lb = np.ascontiguousarray(labels, np.int32); ll = np.ascontiguousarray(label_lengths, np.int32)
+        self._c("lc_ctc_loss", P(probs.ptr), P(probs_d.ptr if probs_d is not None else 0), P(lb.ctypes.data), P(ll.ctypes.data), P(il.ctypes.data),
+                P(costs.ptr), I(T), I(B), I(A))
+        return costs
+
+    def rnn_forward(self, mode, x, w, T, B, I_, H, bidir):
+        y = self.mallocArray(T * B * H * (2 if bidir else 1))
+        self._c("lc_rnn_fwd", I(mode), P(x.ptr), P(w.ptr), P(y.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))
+        return y
+
+    def rnn_backward(self, mode, x, y, dy, w, dx, dw, T, B, I_, H, bidir, beta_dx=1.0):
+        self._c("lc_rnn_bwd", I(mode), P(x.ptr), P(y.ptr), P(dy.ptr), P(w.ptr), P(dx.ptr if dx is not None else 0), P(dw.ptr),
+                I(T), I(B), I(I_), I(H), I(int(bidir)))
+
     def sgd_update(self, x, d, lr, n): self._c("lc_sgd", P(x.ptr), P(d.ptr), F(lr), L(n))
     def adagrad_update(self, x, d, m, lr, clip, n): self._c("lc_adagrad", P(x.ptr), P(d.ptr), P(m.ptr), F(lr), F(clip), L(n))
     def momentum_update(self, x, d, v, lr, mu, clip, nesterov, n):

@@ -701,8 +701,10 @@ void lc_adagrad(float* x, float* d, float* m, float lr, float clip, long n) { /*
  * cudnnCTCLoss (deterministic) is called at CDN:1895-1938: costs[b] =
  * -log p(labels_b | probs), and the gradient written is with respect to the
  * *pre-softmax activations* (cuDNN's documented output): dact = probs -
- * (1/p(l|x)) * sum_{s: l'_s = k} alpha*beta.  Accumulated into dprobs, scaled
- * by 1/B (the reference takes the mean over the batch afterwards). */
+ * (1/p(l|x)) * sum_{s: l'_s = k} alpha*beta.  Accumulated into dprobs unscaled:
+ * the reference lets cuDNN write this gradient into probs.d during the forward
+ * call and only averages the reported costs (CDN:1930-1937), so training
+ * follows the gradient of the SUM of the per-sample costs. */
 void lc_ctc_loss(const float* probs, float* dprobs, const int* labels, const int* label_len, const int* input_len,
                  float* costs, int T, int B, int A) {
   int loff = 0;
@@ -748,7 +750,7 @@ void lc_ctc_loss(const float* probs, float* dprobs, const int* labels, const int
         for (int k = 0; k < A; k++) {
           size_t i = ((size_t)t * B + b) * A + k;
           double post = acc[k] / pfin; /* alpha,beta scaled: sum_s alpha_t(s)beta_t(s)/pfin = posterior */
-          dprobs[i] += (float)((probs[i] - post) / B);
+          dprobs[i] += (float)(probs[i] - post);
         }
         free(acc);
       }
@@ -756,4 +758,77 @@ void lc_ctc_loss(const float* probs, float* dprobs, const int* labels, const int
     #undef LP
     free(alpha); free(beta); free(cn);
   }
+}
+
+/* ------------------------------------------------------------------- RNN */
+/* parity unpinned against the reference (no CPU implementation, CPU:??? ; the
+ * GPU path is cudnnRNNForwardTraining / BackwardData / BackwardWeights at
+ * CDN:1638-1893).  One layer of an Elman RNN, optionally bidirectional:
+ *   h_t = act(W_ih x_t + b_ih + W_hh h_{t-1} + b_hh),  h_{-1} = 0,
+ * act = tanh (mode 1) or relu (mode 0); y[t,b,:] = [h_t forward ; h_t reverse],
+ * the reverse direction running t = T-1 .. 0.  Packed weights per direction in
+ * the order of NN:378-390: W_ih[H,I], W_hh[H,H], b_ih[H], b_hh[H]; forward
+ * direction first.  Checked against torch.nn.RNN in the tests. */
+static size_t rnn_dir_params(int I, int H) { return (size_t)H * I + (size_t)H * H + 2 * (size_t)H; }
+
+void lc_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+  const int D = bidir ? 2 : 1, DH = D * H;
+  float* pre = (float*)malloc((size_t)T * B * H * sizeof(float));
+  float* hprev = (float*)calloc((size_t)B * H, sizeof(float));
+  float* rec = (float*)malloc((size_t)B * H * sizeof(float));
+  for (int d = 0; d < D; d++) {
+    const float* Wih = w + d * rnn_dir_params(I, H); const float* Whh = Wih + (size_t)H * I;
+    const float* bih = Whh + (size_t)H * H; const float* bhh = bih + H;
+    /* input projection for all steps: pre[T*B, H] = x[T*B, I] * Wih^T */
+    lc_sgemm(0, 1, T * B, H, I, 1.0f, x, I, Wih, I, 0.0f, pre, H);
+    memset(hprev, 0, (size_t)B * H * sizeof(float));
+    for (int step = 0; step < T; step++) {
+      const int t = d == 0 ? step : T - 1 - step;
+      lc_sgemm(0, 1, B, H, H, 1.0f, hprev, H, Whh, H, 0.0f, rec, H);
+      for (int b = 0; b < B; b++)
+        for (int j = 0; j < H; j++) {
+          float v = pre[((size_t)t * B + b) * H + j] + bih[j] + rec[(size_t)b * H + j] + bhh[j];
+          v = mode == 1 ? (float)tanh((double)v) : (v < 0.f ? 0.f : v);
+          y[((size_t)t * B + b) * DH + d * H + j] = v; hprev[(size_t)b * H + j] = v;
+        }
+    }
+  }
+  free(pre); free(hprev); free(rec);
+}
+
+/* dx (may be NULL) and dw accumulate. */
+void lc_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float* dw,
+                int T, int B, int I, int H, int bidir) {
+  const int D = bidir ? 2 : 1, DH = D * H;
+  float* dpre = (float*)malloc((size_t)T * B * H * sizeof(float));
+  float* hs = (float*)malloc((size_t)T * B * H * sizeof(float));      /* h_{t-1} for every step, in time order */
+  float* dh = (float*)malloc((size_t)B * H * sizeof(float));
+  for (int d = 0; d < D; d++) {
+    const size_t off = d * rnn_dir_params(I, H);
+    const float* Wih = w + off; const float* Whh = Wih + (size_t)H * I;
+    float* dWih = dw + off; float* dWhh = dWih + (size_t)H * I; float* dbih = dWhh + (size_t)H * H; float* dbhh = dbih + H;
+    memset(dh, 0, (size_t)B * H * sizeof(float));
+    for (int step = T - 1; step >= 0; step--) {
+      const int t = d == 0 ? step : T - 1 - step;
+      const int tp = d == 0 ? t - 1 : t + 1;                              /* time index of the previous hidden state */
+      for (int b = 0; b < B; b++)
+        for (int j = 0; j < H; j++) {
+          const float h = y[((size_t)t * B + b) * DH + d * H + j];
+          const float g = dy[((size_t)t * B + b) * DH + d * H + j] + dh[(size_t)b * H + j];
+          dpre[((size_t)t * B + b) * H + j] = mode == 1 ? g * (1.0f - h * h) : (h > 0.f ? g : 0.f);
+          hs[((size_t)t * B + b) * H + j] = step == 0 ? 0.f : y[((size_t)tp * B + b) * DH + d * H + j];
+        }
+      /* dh_{prev}[B,H] = dpre_t[B,H] * Whh[H,H] */
+      lc_sgemm(0, 0, B, H, H, 1.0f, dpre + (size_t)t * B * H, H, Whh, H, 0.0f, dh, H);
+    }
+    /* dWih[H,I] += dpre^T x ; dWhh[H,H] += dpre^T hs ; biases += column sums ; dx += dpre Wih */
+    lc_sgemm(1, 0, H, I, T * B, 1.0f, dpre, H, x, I, 1.0f, dWih, I);
+    lc_sgemm(1, 0, H, H, T * B, 1.0f, dpre, H, hs, H, 1.0f, dWhh, H);
+    for (int j = 0; j < H; j++) {
+      double s = 0.0; for (size_t r = 0; r < (size_t)T * B; r++) s += dpre[r * H + j];
+      dbih[j] += (float)s; dbhh[j] += (float)s;
+    }
+    if (dx) lc_sgemm(0, 0, T * B, I, H, 1.0f, dpre, H, Wih, I, 1.0f, dx, I);
+  }
+  free(dpre); free(hs); free(dh);
 }

@@ -205,7 +205,7 @@ def test_ctc_against_torch():
     lp = torch.log_softmax(ta, 2)
     loss = torch.nn.functional.ctc_loss(lp, torch.tensor(labels.astype(np.int64)), torch.tensor(ilen.astype(np.int64)), torch.tensor(lens.astype(np.int64)),
                                         blank=0, reduction="none")
-    (loss.sum() / B).backward()
+    loss.sum().backward()          # the gradient of the SUM of costs (what cuDNN writes), not of their mean
     probs = torch.softmax(torch.tensor(act), 2).numpy().astype(np.float32)
     costs = np.zeros(B, np.float32); d = np.zeros_like(probs)
     lc.lc_ctc_loss(cptr(probs), cptr(d), cptr(labels), cptr(lens), cptr(ilen), cptr(costs), I(Tn), I(B), I(A))
@@ -214,3 +214,38 @@ def test_ctc_against_torch():
     for b in range(B):
         g[ilen[b]:, b, :] = 0; 
     np.testing.assert_allclose(d, g, rtol=1e-3, atol=1e-5)
+
+
+@pytest.mark.parametrize("mode", [0, 1], ids=["relu", "tanh"])
+@pytest.mark.parametrize("bidir", [False, True], ids=["uni", "bi"])
+def test_rnn_against_torch(mode, bidir):
+    """lc_rnn_fwd / lc_rnn_bwd (no counterpart on the reference's CPU side) against torch.nn.RNN: outputs, input
+    gradient and every weight gradient, with the packed weight order W_ih, W_hh, b_ih, b_hh per direction."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.RandomState(8 + mode)
+    T, B, In, H = 7, 3, 5, 6
+    D = 2 if bidir else 1
+    per = H * In + H * H + 2 * H
+    w = (rng.randn(D * per) * 0.4).astype(np.float32)
+    x = rng.randn(T, B, In).astype(np.float32); dy = rng.randn(T, B, D * H).astype(np.float32)
+    rnn = torch.nn.RNN(In, H, 1, nonlinearity="tanh" if mode == 1 else "relu", bidirectional=bidir)
+    names = ["weight_ih_l0", "weight_hh_l0", "bias_ih_l0", "bias_hh_l0"]
+    with torch.no_grad():
+        for d in range(D):
+            o = d * per
+            for nm, size, shape in zip(names, (H * In, H * H, H, H), ((H, In), (H, H), (H,), (H,))):
+                getattr(rnn, nm + ("_reverse" if d else "")).copy_(torch.tensor(w[o:o + size].reshape(shape))); o += size
+    tx = torch.tensor(x, requires_grad=True)
+    ty, _ = rnn(tx)
+    ty.backward(torch.tensor(dy))
+    y = np.zeros((T, B, D * H), np.float32)
+    lc.lc_rnn_fwd(I(mode), cptr(x), cptr(w), cptr(y), I(T), I(B), I(In), I(H), I(int(bidir)))
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-5, atol=1e-6)
+    dx = np.ones_like(x); dw = np.ones_like(w)                    # both accumulate
+    lc.lc_rnn_bwd(I(mode), cptr(x), cptr(y), cptr(dy), cptr(w), cptr(dx), cptr(dw), I(T), I(B), I(In), I(H), I(int(bidir)))
+    np.testing.assert_allclose(dx - 1, tx.grad.numpy(), rtol=1e-4, atol=1e-5)
+    for d in range(D):
+        o = d * per
+        for nm, size in zip(names, (H * In, H * H, H, H)):
+            g = getattr(rnn, nm + ("_reverse" if d else "")).grad.numpy().ravel()
+            np.testing.assert_allclose(dw[o:o + size] - 1, g, rtol=1e-4, atol=1e-5, err_msg=nm + str(d)); o += size

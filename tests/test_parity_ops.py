@@ -505,3 +505,65 @@ def test_shape_errors_are_reported_not_launched(on_hip):
             _lib.check()
     be.fillInPlace(x, 16, 1.0)
     assert (be.toHost(x, 16) == 1.0).all()
+
+
+# ---- recurrent layer and CTC (DeepSpeech2 path) ------------------------------------------------------
+@pytest.mark.parametrize("case", [(1, True, 12, 32, 672, 800), (1, True, 6, 8, 96, 1024), (0, False, 5, 3, 7, 37), (1, False, 1, 2, 5, 16), (0, True, 9, 4, 33, 130)],
+                         ids=lambda c: "mode%d_bi%d_T%d_B%d_I%d_H%d" % c)
+def test_rnn_forward_and_backward(pair, case):
+    mode, bidir, T, Bn, In, H = case
+    D = 2 if bidir else 1
+    rng = np.random.RandomState(31)
+    per = H * In + H * H + 2 * H
+    w = (rng.randn(D * per) * (0.5 / np.sqrt(H))).astype(np.float32)
+    x = rng.randn(T, Bn, In).astype(np.float32); dy = rng.randn(T, Bn, D * H).astype(np.float32)
+    if mode == 0:
+        w[:] = np.abs(w) * np.where(rng.rand(w.size) < 0.3, -1, 1)       # relu: keep most pre-activations away from the kink
+
+    def f(be, up, down):
+        X, W = up(x), up(w)
+        y = be.rnn_forward(mode, X, W, T, Bn, In, H, bidir)
+        dx = up(np.ones(x.size, np.float32)); dw = up(np.ones(w.size, np.float32))
+        be.rnn_backward(mode, X, y, up(dy), W, dx, dw, T, Bn, In, H, bidir, 1.0)
+        outs = [down(y, dy.shape), down(dx, x.shape), down(dw, w.shape)]
+        if be.name == "hip":
+            dx0 = up(np.full(x.size, 5.0, np.float32)); dw0 = up(np.zeros(w.size, np.float32))
+            be.rnn_backward(mode, X, y, up(dy), W, dx0, dw0, T, Bn, In, H, bidir, 0.0)                 # overwrite form
+            assert_close(down(dx0, x.shape) + 1.0, outs[1], rtol=2e-4, what="dx beta 0")
+            be.rnn_backward(mode, X, y, up(dy), W, None, dw0, T, Bn, In, H, bidir, 1.0)                # input layer: no dx
+            assert_close(down(dw0, w.shape) * 0.5 + 1.0, outs[2], rtol=2e-4, what="dw accumulates")
+        return outs
+
+    check_all(pair.run(f), rtol=3e-4)
+
+
+@pytest.mark.parametrize("case", ["ds2", "ragged", "tiny"])
+def test_ctc_loss_and_gradient(pair, case):
+    rng = np.random.RandomState(32)
+    if case == "ds2":
+        T, Bn, A = 185, 32, 29
+        lens = np.full(Bn, 50, np.int32); ilen = np.full(Bn, T, np.int32)
+    elif case == "ragged":
+        T, Bn, A = 40, 7, 11
+        lens = np.array([5, 1, 0, 12, 3, 19, 8], np.int32); ilen = np.array([40, 3, 1, 30, 40, 39, 17], np.int32)
+    else:
+        T, Bn, A = 3, 1, 2
+        lens = np.array([1], np.int32); ilen = np.array([3], np.int32)
+    labels = rng.randint(1, A, size=int(lens.sum())).astype(np.int32)
+    if case == "ragged":
+        labels[5:9] = labels[5]                                   # repeated labels: the skip transition must be closed
+    act = (rng.randn(T, Bn, A) * 2).astype(np.float32)
+    e = np.exp(act - act.max(2, keepdims=True)); probs = (e / e.sum(2, keepdims=True)).astype(np.float32)
+
+    def f(be, up, down):
+        Pb = up(probs); d = up(np.ones(probs.size, np.float32))
+        costs = be.ctcLoss(Pb, d, ilen, labels, lens, T, Bn, A)
+        c2 = be.ctcLoss(Pb, None, ilen, labels, lens, T, Bn, A)       # no gradient requested
+        return [down(costs, (Bn,)), down(d, probs.shape), down(c2, (Bn,))]
+
+    outs = pair.run(f)
+    if case == "tiny":            # one label over three frames: p = sum over the 5 alignments b/l placements
+        p = probs[:, 0, :]; bl, lb = p[:, 0], p[:, 1]
+        want = lb[0] * lb[1] * lb[2] + bl[0] * lb[1] * lb[2] + lb[0] * lb[1] * bl[2] + bl[0] * bl[1] * lb[2] + bl[0] * lb[1] * bl[2] + lb[0] * bl[1] * bl[2]
+        np.testing.assert_allclose(outs[1][0][0], -np.log(want), rtol=1e-5)
+    check_all(outs, rtol=1e-4)

@@ -100,3 +100,11 @@ def test_treelstm_10_trees(hip_backend, cpu_backend):
     """One Adagrad step per tree over 10 random trees of 5..30 leaves: gemv / rank-1 update / gemv-transposed path."""
     from lantern_amd.apps.treelstm import Trainer
     _compare(lambda: Trainer(n_trees=10, vocab=500, max_leaves=30), hip_backend, cpu_backend, steps=10)
+
+
+def test_deepspeech2_5_steps(hip_backend, cpu_backend):
+    """conv(41x11, 21x11 strided) + BN + hardTanh, permute, two bidirectional tanh RNN layers with sequence-wise BN,
+    BatchNorm1D + linear, softmax, CTC; Nesterov momentum.  Reduced sizes so that the oracle finishes in seconds."""
+    from lantern_amd.apps.deepspeech2 import Trainer
+    _compare(lambda: Trainer(batch=4, freq=81, frames=120, hidden=64, layers=2, label_len=8, lr=3e-4), hip_backend, cpu_backend,
+             steps=5, per_tensor=5e-3)
