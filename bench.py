@@ -1,12 +1,14 @@
 #!/usr/bin/env python3
-"""Benchmark: ResNet-50 training step (fwd + bwd + SGD-momentum), fp32, batch 64, 3x224x224,
-1000 classes, synthetic data, on one MI355X through the lantern_hip C ABI.
+"""Benchmark: one training step (fwd + bwd + optimizer), fp32, synthetic data, on one MI355X through
+the lantern_hip C ABI.  Default workload: ResNet-50, batch 64, 3x224x224, 1000 classes (the headline
+configuration); `--workload` selects one of the other four application programs.
 
-Prints ONE JSON line: training samples/s, the MFMA roofline fraction of the convolution kernels
+Prints ONE JSON line: training samples/s, the roofline fraction of the dominant kernel family
 (measured live with HIP events on the library's stream over the timed steps), and the CPU oracle
 timed on the host cores on a bounded sample of the same workload.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64] [--hw 224] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload resnet50|squeezenet|lenet|treelstm|deepspeech2]
+                  [--batch B] [--hw 224] [--no-cpu] [--verbose]
 """
 import argparse
 import ctypes as C
@@ -19,78 +21,66 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-import numpy as np  # noqa: E402
+import numpy as np  # noqa: E402,F401
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
 CATS = ["conv_fwd", "conv_bwd_data", "conv_bwd_filter", "gemm", "bn_fwd", "bn_bwd", "elementwise", "pool", "reduce", "optim", "fill", "rnn"]
 
+DEFAULT_BATCH = {"resnet50": 64, "squeezenet": 64, "lenet": 100, "treelstm": 1, "deepspeech2": 32}
 
-def conv_flops(model, batch, hw):
-    """Algorithmic conv work of one step: 2*N*K*C*R*S*P*Q per direction; every conv has a filter
-    gradient, every conv but the stem an input gradient."""
-    from lantern_amd.nn import Conv2D
-    fwd = 0
-    first = True
-    total = 0
-    shapes = []
 
-    def visit(m, h):
-        return h
-    # walk the network the way __call__ does, tracking spatial size
-    h = hw
-    convs = []
-    c1 = model.conv1
-    def out_hw(h, conv):
-        k = conv.kernel.x.shape
-        return (h + 2 * conv.pad[0] - k[2]) // conv.stride[0] + 1
-    def f(conv, h):
-        k = conv.kernel.x.shape
-        p = out_hw(h, conv)
-        return 2.0 * batch * k[0] * k[1] * k[2] * k[3] * p * p, p
-    fl, h = f(c1, h); convs.append((fl, False))
-    if model.imagenet_stem:
-        h = (h + 2 - 3) // 2 + 1
-    for blk in model.blocks:
-        fl1, h1 = f(blk.conv1, h); convs.append((fl1, True))
-        fl2, h2 = f(blk.conv2, h1); convs.append((fl2, True))
-        fl3, h3 = f(blk.conv3, h2); convs.append((fl3, True))
-        if blk.down is not None:
-            fld, _ = f(blk.down[0], h); convs.append((fld, True))
-        h = h3
-    fwd = sum(c[0] for c in convs)
-    bwd_filter = fwd
-    bwd_data = sum(c[0] for c in convs if c[1])
-    return fwd, bwd_data, bwd_filter
+def make_trainer(args, batch, cpu=False):
+    """(trainer, samples per step, description).  `cpu`: the bounded sample for the oracle."""
+    w = args.workload
+    if w == "resnet50":
+        from lantern_amd.apps.resnet50 import ResNet50, Trainer
+        model = ResNet50(num_classes=args.classes, imagenet_stem=args.hw > 64)
+        return Trainer(model, batch, args.hw, args.classes, lr=0.1, momentum=0.9), batch, \
+            "ResNet-50 training step (configs[3]): batch %d, 3x%dx%d, %d classes, SGD lr 0.1 momentum 0.9, Kaiming-normal init" % (batch, args.hw, args.hw, args.classes)
+    if w == "squeezenet":
+        from lantern_amd.apps.squeezenet import Trainer
+        return Trainer(batch=batch, hw=32, num_classes=10, lr=0.005, momentum=0.9), batch, \
+            "SqueezeNet training step (configs[2]): batch %d, 3x32x32, 10 classes, SGD lr 0.005 momentum 0.9" % batch
+    if w == "lenet":
+        from lantern_amd.apps.lenet import Trainer
+        return Trainer(batch=batch, lr=0.0005), batch, "LeNet-style CNN training step (configs[0]): batch %d, 1x28x28, SGD lr 0.0005, dropout 0.5" % batch
+    if w == "treelstm":
+        from lantern_amd.apps.treelstm import Trainer
+        return Trainer(n_trees=16 if cpu else 64, vocab=20000), 1, \
+            "TreeLSTM sentiment step (configs[1]): one tree of 5-50 leaves per step, hidden 150, embedding 300, Adagrad lr 0.05"
+    if w == "deepspeech2":
+        from lantern_amd.apps.deepspeech2 import Trainer
+        # learning rate 1e-5: the reference program's 3e-4 (DeepSpeech.scala:127) diverges within ten steps on random spectrograms
+        return Trainer(batch=batch, freq=161, frames=args.frames, hidden=args.hidden, layers=3, label_len=50, lr=1e-5), batch, \
+            "DeepSpeech2-style step (configs[4]): batch %d, 1x161x%d, 3 bidirectional tanh RNN layers hidden %d, CTC over 29 symbols, Nesterov SGD lr 1e-5" % (batch, args.frames, args.hidden)
+    raise SystemExit("unknown workload %r" % w)
 
 
 def run_gpu(args):
     import lantern_amd as la
-    from lantern_amd.apps.resnet50 import ResNet50, Trainer
     be = la.BackendHIP(heap_bytes=int(args.heap_gb * (1 << 30)))
     be.setup()
     la.set_backend(be)
-    model = ResNet50(num_classes=args.classes, imagenet_stem=args.hw > 64)
-    tr = Trainer(model, args.batch, args.hw, args.classes, lr=0.1, momentum=0.9)
+    tr, per_step, desc = make_trainer(args, args.batch)
     lib = be.lib
-    losses = []
     for _ in range(args.warmup):
-        l = tr.step(); tr.end_step()
+        tr.step(); tr.end_step()
     be.sync()
-    conv_mask = 0b111
-    lib.lh_prof_enable(conv_mask)
+    lib.lh_prof_enable(0b1111 | (1 << CATS.index("rnn")))        # conv x3, gemm, rnn: the matrix kernels
     ms = (C.c_double * len(CATS))(); calls = (C.c_int64 * len(CATS))()
     lib.lh_prof_collect(ms, calls, len(CATS))       # reset
+    be.work = {}
     be.sync()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        l = tr.step()
-        losses.append(l)
+        tr.step()
         tr.end_step()
     be.sync()
     t1 = time.perf_counter()
     lib.lh_prof_collect(ms, calls, len(CATS))
-    conv_ms = [ms[i] / args.steps for i in range(3)]
-    conv_calls = [int(calls[i]) // args.steps for i in range(3)]
+    timed = {CATS[i]: (ms[i] / args.steps, int(calls[i]) // args.steps) for i in range(len(CATS))}
+    work = {k: v / args.steps for k, v in be.work.items()}
     # a separate, untimed pass with every category instrumented (breakdown for the log)
     lib.lh_prof_enable((1 << len(CATS)) - 1)
     tr.step(); tr.end_step()
@@ -99,33 +89,32 @@ def run_gpu(args):
     lib.lh_prof_enable(0)
     loss_val = float(tr.step().toCPU()[0]); tr.end_step()
     peak_gb = lib.lh_heap_peak() / 2 ** 30
-    fl = conv_flops(model, args.batch, args.hw)
     be.cleanup()
-    return {"sec": t1 - t0, "conv_ms": conv_ms, "conv_calls": conv_calls, "conv_flops": fl, "breakdown": breakdown,
-            "loss": loss_val, "arena_peak_gib": peak_gb}
+    return {"sec": t1 - t0, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "arena_peak_gib": peak_gb,
+            "per_step": per_step, "desc": desc}
 
 
 def run_cpu(args):
     """The oracle (a C restatement of Lantern's BackendCPU: per-sample im2col + own SGEMM) on the
-    host cores, same network and input shape, on a bounded sample: `cpu_batch` images per step."""
+    host cores, same program and input shape, on a bounded sample (a smaller batch, a few steps)."""
     import lantern_amd as la
     from oracle.backend_cpu import BackendCPU
-    from lantern_amd.apps.resnet50 import ResNet50, Trainer
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
     be = BackendCPU(threads=threads)
     be.setup()
     la.set_backend(be)
-    model = ResNet50(num_classes=args.classes, imagenet_stem=args.hw > 64)
-    tr = Trainer(model, args.cpu_batch, args.hw, args.classes, lr=0.1, momentum=0.9)
+    batch = {"resnet50": args.cpu_batch, "squeezenet": 64, "lenet": 100, "treelstm": 1, "deepspeech2": 2}[args.workload]
+    tr, per_step, _ = make_trainer(args, batch, cpu=True)
     tr.step(); tr.end_step()                     # warm-up
+    max_steps = {"resnet50": args.cpu_steps, "squeezenet": 10, "lenet": 50, "treelstm": 32, "deepspeech2": 2}[args.workload]
     t0 = time.perf_counter()
     n = 0
-    while n < args.cpu_steps:
+    while n < max_steps:
         tr.step(); tr.end_step(); n += 1
-        if time.perf_counter() - t0 > 30.0:
+        if time.perf_counter() - t0 > 25.0:
             break
     dt = time.perf_counter() - t0
-    return {"value": args.cpu_batch * n / dt, "cores": threads, "steps": n}
+    return {"value": per_step * n / dt, "cores": threads, "steps": n, "batch": batch}
 
 
 def main():
@@ -133,9 +122,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--workload", default="resnet50", choices=sorted(DEFAULT_BATCH))
+    ap.add_argument("--batch", type=int, default=0)
     ap.add_argument("--hw", type=int, default=224)
     ap.add_argument("--classes", type=int, default=1000)
+    ap.add_argument("--frames", type=int, default=400)
+    ap.add_argument("--hidden", type=int, default=800)
     ap.add_argument("--heap-gb", type=float, default=48.0)
     ap.add_argument("--cpu-batch", type=int, default=4)
     ap.add_argument("--cpu-steps", type=int, default=2)
@@ -144,36 +136,51 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (the reference is single-device; nothing here shards); use --gpus 1")
+    if args.batch <= 0:
+        args.batch = DEFAULT_BATCH[args.workload]
 
     g = run_gpu(args)
     ms_per_step = 1000.0 * g["sec"] / args.steps
-    value = args.batch * args.steps / g["sec"]
-    conv_time_s = sum(g["conv_ms"]) / 1000.0
-    conv_fl = sum(g["conv_flops"])
-    achieved = conv_fl / conv_time_s / 1e12 if conv_time_s > 0 else 0.0
+    value = g["per_step"] * args.steps / g["sec"]
+    timed, work = g["timed"], g["work"]
+    conv_ms = [timed[k][0] for k in ("conv_fwd", "conv_bwd_data", "conv_bwd_filter")]
+    conv_calls = sum(timed[k][1] for k in ("conv_fwd", "conv_bwd_data", "conv_bwd_filter"))
+    if args.workload == "treelstm":
+        # matrix-vector path: the weight matrices are streamed once per product (HBM / launch bound)
+        t = timed["gemm"][0] / 1000.0
+        achieved = work.get("gemv_bytes", 0.0) / t / 1e9 if t > 0 else 0.0
+        roof = {"bound": "hbm", "kernel": "gemv / rank-1 update kernels (%d launches/step; launch-bound at these sizes)" % timed["gemm"][1],
+                "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": None,
+                "bytes_per_step": work.get("gemv_bytes", 0.0), "ms_per_step": round(timed["gemm"][0], 3)}
+    else:
+        conv_fl = work.get("conv_flop", 0.0)
+        conv_t = sum(conv_ms) / 1000.0
+        achieved = conv_fl / conv_t / 1e12 if conv_t > 0 else 0.0
+        roof = {"bound": "mfma", "kernel": "k_igemm (conv fwd + bwd-data + bwd-filter, %d launches/step)" % conv_calls,
+                "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None, "flop_per_step": conv_fl,
+                "ms_per_step": {"fwd": round(conv_ms[0], 3), "bwd_data": round(conv_ms[1], 3), "bwd_filter": round(conv_ms[2], 3)}}
+        if work.get("gemm_flop", 0.0) > 0 and timed["gemm"][0] > 0:
+            roof["gemm"] = {"flop_per_step": work["gemm_flop"], "ms_per_step": round(timed["gemm"][0], 3),
+                            "tflops": round(work["gemm_flop"] / (timed["gemm"][0] / 1000.0) / 1e12, 2)}
+        if timed["rnn"][0] > 0:
+            roof["rnn_recurrence"] = {"flop_per_step": work.get("rnn_flop", 0.0), "ms_per_step": round(timed["rnn"][0], 3), "launches": timed["rnn"][1]}
+    unit = "trees/s" if args.workload == "treelstm" else "samples/s"
     out = {
-        "metric": "train samples/s (fwd+bwd+SGD), ResNet-50 b64 fp32; % of MFMA/HBM roofline",
-        "value": round(value, 2), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": "train samples/s (fwd+bwd+SGD), ResNet-50 b64 fp32; % of MFMA/HBM roofline" if args.workload == "resnet50"
+                  else "train %s (fwd+bwd+optimizer), %s fp32; %% of MFMA/HBM roofline" % (unit, args.workload),
+        "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "ResNet-50 training step (configs[3]): batch %d, 3x%dx%d, %d classes, SGD lr 0.1 momentum 0.9, Kaiming-normal init"
-                               % (args.batch, args.hw, args.hw, args.classes),
-                   "global_batch": args.batch, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2)},
-        "roofline": {"bound": "mfma", "kernel": "k_igemm (conv fwd + bwd-data + bwd-filter, %d launches/step)" % sum(g["conv_calls"]),
-                     "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
-                     "flop_per_step": conv_fl, "ms_per_step": {"fwd": round(g["conv_ms"][0], 3), "bwd_data": round(g["conv_ms"][1], 3),
-                                                               "bwd_filter": round(g["conv_ms"][2], 3)},
-                     "tflops_by_pass": {k: round(f / (m / 1000.0) / 1e12, 2) if m > 0 else None
-                                        for k, f, m in zip(("fwd", "bwd_data", "bwd_filter"), g["conv_flops"], g["conv_ms"])}},
+        "config": {"workload": g["desc"], "global_batch": args.batch, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2)},
+        "roofline": roof,
     }
     if args.verbose:
         print(json.dumps(g["breakdown"], indent=1), file=sys.stderr)
     if not args.no_cpu:
         c = run_cpu(args)
-        out["cpu_baseline"] = {"value": round(c["value"], 3), "unit": "samples/s", "cores": c["cores"], "kind": "port",
-                               "sample": "same network and 3x%dx%d input, %d step(s) of batch %d (bounded sample; own SGEMM, not OpenBLAS)"
-                                         % (args.hw, args.hw, c["steps"], args.cpu_batch)}
+        out["cpu_baseline"] = {"value": round(c["value"], 3), "unit": unit, "cores": c["cores"], "kind": "port",
+                               "sample": "same program and input shape, %d step(s) of batch %d (bounded sample; own SGEMM, not OpenBLAS)" % (c["steps"], c["batch"])}
     print(json.dumps(out))
 
 

@@ -6,7 +6,7 @@
 //
 // The input projection of all time steps and the three weight/input gradients are large GEMMs
 // (lh_sgemm, MFMA).  Only the recurrence is sequential: one small kernel per time step, both
-// directions in the same launch, each block producing 16 hidden units for the whole batch from
+// directions in the same launch, each block producing 4-16 hidden units for the whole batch from
 // W_hh rows held in registers.  The output y doubles as the saved hidden states.
 #include "lh_common.h"
 #include "../../include/lantern_hip.h"
@@ -14,13 +14,50 @@ using namespace lh;
 
 namespace {
 constexpr int TPB = 256;
-constexpr int JT = 16;            // hidden units per block (4 per wavefront)
-constexpr int KMAX = 32;          // K values per lane: supports H up to 64 * 32 = 2048
+constexpr int UB = 4;              // batch rows whose loads are in flight together
 
 __device__ __forceinline__ float act_fwd(int mode, float v) { return mode == 1 ? tanhf(v) : (v < 0.f ? 0.f : v); }
 
+// Shared shape of both step kernels: out[b, j] = sum_k in[b, k] * Wrow[j, k] for the JC rows j0.. of this
+// block and every batch row b.  A lane owns k = lane, lane + 64, ...; the JC x NK weights it needs stay in
+// registers for the whole step.  The four wavefronts of a block take every fourth batch row, UB rows at a
+// time so that UB * NK loads are outstanding before the first use.
+//   in(b, k)        value of the input vector of row b at k          (k < H guaranteed)
+//   done(b, c, s)   called on lane 0 with the finished sum of row b, weight row j0 + c
+template <int NK, int JC, class In, class Done>
+__device__ __forceinline__ void rnn_rows(const float* __restrict__ W, int H, int B, int j0, bool use_w, In in, Done done) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float w[JC][NK];
+#pragma unroll
+  for (int c = 0; c < JC; c++)
+#pragma unroll
+    for (int i = 0; i < NK; i++) { const int k = lane + 64 * i; w[c][i] = (use_w && k < H && j0 + c < H) ? W[(int64_t)(j0 + c) * H + k] : 0.f; }
+  for (int b0 = wave * UB; b0 < B; b0 += 4 * UB) {
+    float h[UB][NK];
+#pragma unroll
+    for (int u = 0; u < UB; u++)
+#pragma unroll
+      for (int i = 0; i < NK; i++) { const int k = lane + 64 * i; h[u][i] = (b0 + u < B && k < H) ? in(b0 + u, k) : 0.f; }
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      float s[JC];
+#pragma unroll
+      for (int c = 0; c < JC; c++) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < NK; i++) t = fmaf(h[u][i], w[c][i], t);
+        s[c] = lh_wave_sum(t);
+      }
+      if (lane == 0 && b0 + u < B) {
+#pragma unroll
+        for (int c = 0; c < JC; c++) if (j0 + c < H) done(b0 + u, c, s[c]);
+      }
+    }
+  }
+}
+
 // One time step of both directions.
-//   out[b, j] = act(pre[b, j] + bias1[j] + bias2[j] + sum_k prev[b, k] * Wrow[j, k])       (forward)
+//   out[b, j] = act(pre[b, j] + bias1[j] + bias2[j] + sum_k prev[b, k] * W_hh[j, k])
 // pre/out alias inside y: row stride ld.  dir = blockIdx.y picks the direction's weights and time index.
 struct StepArgs {
   float* cur[2];              // y + t*B*ld + d*H        (pre-activation in, hidden state out)
@@ -28,84 +65,49 @@ struct StepArgs {
   const float* W[2];          // W_hh of the direction, [H, H] rows = output units
   const float* b1[2]; const float* b2[2];
 };
+template <int NK, int JC>
 __global__ void __launch_bounds__(TPB) k_rnn_fwd_step(StepArgs a, int B, int H, int ld, int mode) {
-  const int d = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int j0 = blockIdx.x * JT + wave * 4;
-  float* cur = a.cur[d]; const float* prev = a.prev[d]; const float* W = a.W[d];
-  const int nk = (H + 63) >> 6;
-  float w[4][KMAX];
-#pragma unroll
-  for (int c = 0; c < 4; c++)
-#pragma unroll
-    for (int i = 0; i < KMAX; i++) { const int k = lane + 64 * i; w[c][i] = (i < nk && k < H && j0 + c < H && prev) ? W[(int64_t)(j0 + c) * H + k] : 0.f; }
-  for (int b = 0; b < B; b++) {
-    float s[4] = {0.f, 0.f, 0.f, 0.f};
-    if (prev) {
-#pragma unroll
-      for (int i = 0; i < KMAX; i++) {
-        if (i < nk) {
-          const int k = lane + 64 * i;
-          const float h = k < H ? prev[(int64_t)b * ld + k] : 0.f;
-#pragma unroll
-          for (int c = 0; c < 4; c++) s[c] = fmaf(h, w[c][i], s[c]);
-        }
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < 4; c++) s[c] = lh_wave_sum(s[c]);
-    if (lane == 0) {
-#pragma unroll
-      for (int c = 0; c < 4; c++) {
-        const int j = j0 + c;
-        if (j < H) cur[(int64_t)b * ld + j] = act_fwd(mode, cur[(int64_t)b * ld + j] + a.b1[d][j] + a.b2[d][j] + s[c]);
-      }
-    }
-  }
+  const int d = blockIdx.y, j0 = blockIdx.x * JC;
+  float* cur = a.cur[d]; const float* prev = a.prev[d]; const float* b1 = a.b1[d]; const float* b2 = a.b2[d];
+  rnn_rows<NK, JC>(a.W[d], H, B, j0, prev != nullptr,
+    [&](int b, int k) { return prev ? prev[(int64_t)b * ld + k] : 0.f; },
+    [&](int b, int c, float s) { const int j = j0 + c; float* p = cur + (int64_t)b * ld + j; *p = act_fwd(mode, *p + b1[j] + b2[j] + s); });
 }
 
 // One backward time step of both directions:
-//   dpre[b, j]  = (dy[b, j] + dh_in[b, j]) * act'(h[b, j])                 (every block needs all j; it stores only its own 16)
+//   dpre[b, j]   = (dy[b, j] + dh_in[b, j]) * act'(h[b, j])                (every block needs all j; block x stores columns with j / JC == x)
 //   dh_out[b, i] = sum_j dpre[b, j] * Wt[i, j]                             (Wt = W_hh transposed, rows = i)
 struct BwdArgs {
   const float* dy[2]; const float* h[2]; float* dpre[2];          // time slice t, direction offset applied, row stride ld
   const float* dh_in[2]; float* dh_out[2];                          // [B, H] dense; dh_in nullptr at the first (last in time) step
   const float* Wt[2];
 };
+template <int NK, int JC>
 __global__ void __launch_bounds__(TPB) k_rnn_bwd_step(BwdArgs a, int B, int H, int ld, int mode) {
-  const int d = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int i0 = blockIdx.x * JT + wave * 4;
-  const float* Wt = a.Wt[d];
-  const int nk = (H + 63) >> 6;
-  float w[4][KMAX];
-#pragma unroll
-  for (int c = 0; c < 4; c++)
-#pragma unroll
-    for (int i = 0; i < KMAX; i++) { const int k = lane + 64 * i; w[c][i] = (i < nk && k < H && i0 + c < H) ? Wt[(int64_t)(i0 + c) * H + k] : 0.f; }
-  const int jlo = blockIdx.x * JT, jhi = min(H, jlo + JT);
-  for (int b = 0; b < B; b++) {
-    float s[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < KMAX; i++) {
-      if (i < nk) {
-        const int j = lane + 64 * i;
-        float g = 0.f;
-        if (j < H) {
-          const float hv = a.h[d][(int64_t)b * ld + j];
-          g = a.dy[d][(int64_t)b * ld + j] + (a.dh_in[d] ? a.dh_in[d][(int64_t)b * H + j] : 0.f);
-          g = mode == 1 ? g * (1.0f - hv * hv) : (hv > 0.f ? g : 0.f);
-          if (wave == 0 && j >= jlo && j < jhi) a.dpre[d][(int64_t)b * ld + j] = g;
-        }
-#pragma unroll
-        for (int c = 0; c < 4; c++) s[c] = fmaf(g, w[c][i], s[c]);
-      }
-    }
-#pragma unroll
-    for (int c = 0; c < 4; c++) s[c] = lh_wave_sum(s[c]);
-    if (lane == 0) {
-#pragma unroll
-      for (int c = 0; c < 4; c++) if (i0 + c < H) a.dh_out[d][(int64_t)b * H + i0 + c] = s[c];
-    }
-  }
+  const int d = blockIdx.y, i0 = blockIdx.x * JC;
+  const float* dy = a.dy[d]; const float* hh = a.h[d]; const float* dh_in = a.dh_in[d]; float* dpre = a.dpre[d]; float* dh_out = a.dh_out[d];
+  rnn_rows<NK, JC>(a.Wt[d], H, B, i0, true,
+    [&](int b, int j) {
+      const float hv = hh[(int64_t)b * ld + j];
+      float g = dy[(int64_t)b * ld + j] + (dh_in ? dh_in[(int64_t)b * H + j] : 0.f);
+      g = mode == 1 ? g * (1.0f - hv * hv) : (hv > 0.f ? g : 0.f);
+      if (j >= i0 && j < i0 + JC) dpre[(int64_t)b * ld + j] = g;
+      return g; },
+    [&](int b, int c, float s) { dh_out[(int64_t)b * H + i0 + c] = s; });
+}
+
+// hidden sizes up to 64 * NK, JC weight rows per block (JC * NK <= 128 registers of weights)
+template <class A>
+static void launch_fwd_step(const A& a, int D, int B, int H, int ld, int mode) {
+#define GO(NK, JC) hipLaunchKernelGGL((k_rnn_fwd_step<NK, JC>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode)
+  if (H <= 256) GO(4, 16); else if (H <= 512) GO(8, 16); else if (H <= 1024) GO(16, 8); else GO(32, 4);
+#undef GO
+}
+template <class A>
+static void launch_bwd_step(const A& a, int D, int B, int H, int ld, int mode) {
+#define GO(NK, JC) hipLaunchKernelGGL((k_rnn_bwd_step<NK, JC>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode)
+  if (H <= 256) GO(4, 16); else if (H <= 512) GO(8, 16); else if (H <= 1024) GO(16, 8); else GO(32, 4);
+#undef GO
 }
 
 // db1[j] += colsum[j]; db2[j] += colsum[j]
@@ -194,7 +196,7 @@ extern "C" {
 void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
   LH_REQUIRE(mode == 0 || mode == 1, "lh_rnn_fwd: mode %d (0 = relu, 1 = tanh)", mode);
   LH_REQUIRE(T >= 1 && B >= 1 && I >= 1 && H >= 1, "lh_rnn_fwd: bad shape T%d B%d I%d H%d", T, B, I, H);
-  LH_REQUIRE(H <= 64 * KMAX, "lh_rnn_fwd: hidden size %d above %d", H, 64 * KMAX);
+  LH_REQUIRE(H <= 2048, "lh_rnn_fwd: hidden size %d above %d", H, 2048);
   LH_REQUIRE(x && w && y, "lh_rnn_fwd: null operand");
   const int D = bidir ? 2 : 1, ld = D * H;
   for (int d = 0; d < D; d++) {          // input projection of every step straight into y
@@ -212,7 +214,7 @@ void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B
       a.prev[d] = step == 0 ? nullptr : y + (size_t)tp * B * ld + dd * H;
       a.W[d] = Whh; a.b1[d] = Whh + (size_t)H * H; a.b2[d] = a.b1[d] + H;
     }
-    hipLaunchKernelGGL(k_rnn_fwd_step, dim3((unsigned)cdiv(H, JT), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode);
+    launch_fwd_step(a, D, B, H, ld, mode);
   }
   LH_CHECK_LAUNCH();
 }
@@ -221,7 +223,7 @@ void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
                 int T, int B, int I, int H, int bidir) {
   LH_REQUIRE(mode == 0 || mode == 1, "lh_rnn_bwd: mode %d (0 = relu, 1 = tanh)", mode);
   LH_REQUIRE(T >= 1 && B >= 1 && I >= 1 && H >= 1, "lh_rnn_bwd: bad shape T%d B%d I%d H%d", T, B, I, H);
-  LH_REQUIRE(H <= 64 * KMAX, "lh_rnn_bwd: hidden size %d above %d", H, 64 * KMAX);
+  LH_REQUIRE(H <= 2048, "lh_rnn_bwd: hidden size %d above %d", H, 2048);
   LH_REQUIRE(beta_dx == 0.f || beta_dx == 1.f, "lh_rnn_bwd: beta must be 0 or 1");
   LH_REQUIRE(x && y && dy && w && dw, "lh_rnn_bwd: null operand");
   const int D = bidir ? 2 : 1, ld = D * H;
@@ -249,7 +251,7 @@ void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
         a.dh_out[d] = dh + ((size_t)cur_buf * D + dd) * B * H;
         a.Wt[d] = wt + (size_t)dd * H * H;
       }
-      hipLaunchKernelGGL(k_rnn_bwd_step, dim3((unsigned)cdiv(H, JT), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode);
+      launch_bwd_step(a, D, B, H, ld, mode);
     }
   }
   lh_sum_dim(dpre, colsum, 1, T * B, ld);
