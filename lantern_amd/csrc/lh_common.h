@@ -44,6 +44,15 @@ struct ProfScope {
   ~ProfScope() { if (on) prof_end(cat); }
 };
 
+// Category the matrix kernels launched below an entry point are timed under: the events then bracket the
+// k_igemm launch itself, not the small layout / fill kernels around it.
+extern int g_kernel_cat;
+struct KernelCat {
+  int saved;
+  explicit KernelCat(int c) : saved(g_kernel_cat) { g_kernel_cat = c; }
+  ~KernelCat() { g_kernel_cat = saved; }
+};
+
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Grid for a grid-stride streaming kernel: enough blocks to cover n at `per_block`

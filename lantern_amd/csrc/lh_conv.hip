@@ -306,7 +306,7 @@ extern "C" {
 
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
-  ProfScope prof_(CAT_CONV_FWD);
+  KernelCat kc_(CAT_CONV_FWD);
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_fwd: bad shape N%d C%d H%d W%d K%d R%d S%d s(%d,%d) p(%d,%d)", N, C, H, W, K, R, S, sH, sW, pH, pW);
   const int RS = R * S, CRS = C * RS, PQ = d.P * d.Q;
@@ -343,7 +343,7 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
 
 void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
                         int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
-  ProfScope prof_(CAT_CONV_BWD_DATA);
+  KernelCat kc_(CAT_CONV_BWD_DATA);
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_data: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_data: beta must be 0 or 1");
@@ -413,7 +413,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
 
 void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db, float beta,
                           int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
-  ProfScope prof_(CAT_CONV_BWD_FILTER);
+  KernelCat kc_(CAT_CONV_BWD_FILTER);
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_filter: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_filter: beta must be 0 or 1");

@@ -106,7 +106,7 @@ static bool sgemm_mfma(const AL& al, const BL& bl, const EpiRowMajor& ep, int m,
 
 void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, int lda,
               const float* B, int ldb, float beta, float* C, int ldc) {
-  ProfScope prof_(CAT_GEMM);
+  KernelCat kc_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
   LH_REQUIRE(k >= 0, "lh_sgemm: negative k");
   LH_REQUIRE(lda >= (ta ? m : k) && ldb >= (tb ? k : n) && ldc >= n, "lh_sgemm: leading dimensions (%d,%d,%d) too small for m%d n%d k%d ta%d tb%d", lda, ldb, ldc, m, n, k, ta, tb);
@@ -133,6 +133,7 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
     LH_CHECK_LAUNCH();
     return;
   }
+  ProfScope prof_(CAT_GEMM);
   dim3 grid((unsigned)cdiv(n, 64), (unsigned)cdiv(m, 64));
   if (!ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<false, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
   else if (!ta && tb) hipLaunchKernelGGL((k_sgemm_tile<false, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);

@@ -350,6 +350,7 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
   constexpr size_t smem = igemm_smem_bytes<BM, BN, BK>();
   if (gs.streamk) {
     if constexpr (smem <= 48 * 1024) {   // stream-K is instantiated for the forward / input-gradient tiles only
+      ProfScope prof_(g_kernel_cat);
       hipLaunchKernelGGL((k_igemm<BM, BN, BK, AL, BL, EP, true>), dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
       return true;
     } else { LH_FAIL("igemm: stream-K is not built for this tile"); return false; }
@@ -362,6 +363,7 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
     }
     attr_done = true;
   }
+  ProfScope prof_(g_kernel_cat);
   hipLaunchKernelGGL(kern, dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
   return true;
 }

@@ -26,6 +26,7 @@ bool failed() { return g_err[0] != 0; }
 
 // ---- event profiler ---------------------------------------------------------------------
 unsigned g_prof_mask = 0;
+int g_kernel_cat = CAT_GEMM;
 struct ProfRec { hipEvent_t a, b; int cat; };
 static std::vector<ProfRec> g_prof_recs;
 static std::vector<hipEvent_t> g_prof_pool;
