@@ -192,6 +192,18 @@ void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float
  * (no atomics, dx written once); dx = beta*dx + sum.  Same result as lh_maxpool_bwd. */
 void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float beta,
                           int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad);
+/* conv2D_batch followed by batchNormTraining of its output: the convolution's epilogue leaves per-channel
+ * partial sums, so the statistics cost no pass over y.  lh_conv2d_fwd_bnstats = lh_conv2d_fwd + the
+ * mean / 1/sqrt(var+eps) / running-statistics part of lh_bn_train_fwd;  lh_bn_apply is the remaining
+ * part (y = gamma*(x-mean)*invstd + beta, then relu when `relu` != 0).  lh_bn_stats computes the same
+ * statistics from a tensor (what lh_conv2d_fwd_bnstats falls back to for shapes without the epilogue). */
+void lh_conv2d_fwd_bnstats(const float* x, const float* w, const float* bias, float* y,
+                           int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW,
+                           float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor);
+void lh_bn_stats(const float* x, float* save_mean, float* save_invstd, float* run_mean, float* run_var,
+                 int N, int C, int HW, float eps, float factor);
+void lh_bn_apply(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd, float* y,
+                 int N, int C, int HW, int relu);
 /* `+` of two same-shape tensors followed by relu(inPlace = true), and the gradient of that pair:
  * g = dy where y > 0 else 0;  ad = abeta*ad + g;  bd = bbeta*bd + g  (ad or bd may be NULL) */
 void lh_add_relu(const float* a, const float* b, float* out, int64_t n);

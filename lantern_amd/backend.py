@@ -83,6 +83,20 @@ class Backend:
         if relu:
             self.unary(RELU, out, n, inPlace=True)
 
+    def conv2D_batch_into(self, x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW):
+        """conv2D_batch writing into a caller-provided y; returns the unfolded input if the backend keeps one (CPU:532-571)."""
+        yy, finput = self.conv2D_batch(x, w, bias, N, C, H, W, K, R, S, sH, sW, pH, pW)
+        self.copyFloatArray(y, yy, N * K * conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW))
+        return finput
+
+    def conv2D_batch_bn_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, ybn, sm, si, relu, eps=1e-5, factor=0.1):
+        """conv2D_batch followed by batchNormTraining of its output (and relu): the unfused sequence."""
+        N, C, H, W, K, R, S, sH, sW, pH, pW = dims
+        finput = self.conv2D_batch_into(x, w, bias, yconv, *dims)
+        HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
+        self.batchNormTraining_into(yconv, scale, bbias, rmean, rvar, ybn, sm, si, N, K, HW, relu, eps, factor)
+        return finput
+
     def add_relu_grad(self, y, dy, ad, abeta, bd, bbeta, n):
         self.unary_grad(RELU, y, y, dy, dy, n, inPlace=True)            # masks dy in place (CPU:725-726 with the y > 0 mask)
         for d in (ad, bd):
@@ -278,6 +292,17 @@ class BackendHIP(Backend):
         self.lib.lh_conv2d_fwd(x.ptr, w.ptr, bias.ptr if bias is not None else 0, y.ptr, N, C, H, W, K, R, S, sH, sW, pH, pW); _lib.check()
         self._count("conv_flop", 2.0 * N * K * C * R * S * P * Q)
         return y, None      # no im2col buffer is kept (BackendCudnn returns None too, CDN:859-866)
+
+    def conv2D_batch_into(self, x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW):
+        self.lib.lh_conv2d_fwd(x.ptr, w.ptr, bias.ptr if bias is not None else 0, y.ptr, N, C, H, W, K, R, S, sH, sW, pH, pW); _lib.check()
+        self._count("conv_flop", 2.0 * N * K * C * R * S * conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW))
+
+    def conv2D_batch_bn_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, ybn, sm, si, relu, eps=1e-5, factor=0.1):
+        N, C, H, W, K, R, S, sH, sW, pH, pW = dims
+        HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
+        self.lib.lh_conv2d_fwd_bnstats(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, eps, factor)
+        self.lib.lh_bn_apply(yconv.ptr, scale.ptr, bbias.ptr, sm.ptr, si.ptr, ybn.ptr, N, K, HW, int(relu)); _lib.check()
+        self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
         if not x_in:

@@ -186,6 +186,76 @@ __global__ void __launch_bounds__(TPB) k_bn_infer(const float* __restrict__ x, f
   }
 }
 
+// Channel statistics from classic per-slice partials (mean, M2, count): one thread per channel.
+__global__ void __launch_bounds__(TPB) k_bn_finalize(const float* __restrict__ partial, int C, int slices, float* save_mean, float* save_invstd,
+                                                     float* run_mean, float* run_var, float eps, float factor) {
+  const int c = blockIdx.x * TPB + threadIdx.x;
+  if (c >= C) return;
+  double mean, m2, cnt;
+  combine_stats(partial, c, slices, mean, m2, cnt);
+  const float var = (float)(m2 / cnt);
+  if (save_mean) save_mean[c] = (float)mean;
+  if (save_invstd) save_invstd[c] = 1.0f / sqrtf(var + eps);
+  if (run_mean) run_mean[c] = (1.0f - factor) * run_mean[c] + factor * (float)mean;
+  if (run_var) { float unb = cnt > 1.0 ? (float)(m2 / (cnt - 1.0)) : var; run_var[c] = (1.0f - factor) * run_var[c] + factor * unb; }
+}
+
+// Channel statistics from the (sum, sum of squares) pieces of a convolution epilogue: one block per channel,
+// each piece turned into (count, mean, M2) and merged with Chan's formula in double.
+__global__ void __launch_bounds__(TPB) k_bn_finalize_conv(const float* __restrict__ partial, int C, int ncols, int col1, int g_main, int slots_main, int g_rem,
+                                                          int slots, float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor) {
+  __shared__ double sc[TPB], sm_[TPB], s2[TPB];
+  const int c = blockIdx.x;
+  double cnt = 0.0, mean = 0.0, m2 = 0.0;
+  for (int s = threadIdx.x; s < slots; s += TPB) {
+    int n;
+    if (s < slots_main) { const int j0 = s * g_main; n = min(g_main, col1 - j0); }
+    else { const int j0 = col1 + (s - slots_main) * g_rem; n = min(g_rem, ncols - j0); }
+    if (n <= 0) continue;
+    const float2 pv = reinterpret_cast<const float2*>(partial)[(size_t)c * slots + s];
+    const double a = pv.x, q = pv.y;
+    const double mb = a / n, m2b = q - a * mb;
+    const double tot = cnt + n, d = mb - mean;
+    mean += d * n / tot; m2 += m2b + d * d * cnt * n / tot; cnt = tot;
+  }
+  sc[threadIdx.x] = cnt; sm_[threadIdx.x] = mean; s2[threadIdx.x] = m2;
+  __syncthreads();
+  for (int off = TPB / 2; off > 0; off >>= 1) {
+    if (threadIdx.x < off) {
+      const double na = sc[threadIdx.x], nb = sc[threadIdx.x + off];
+      if (nb > 0.0) {
+        const double tot = na + nb, d = sm_[threadIdx.x + off] - sm_[threadIdx.x];
+        sm_[threadIdx.x] += d * nb / tot; s2[threadIdx.x] += s2[threadIdx.x + off] + d * d * na * nb / tot; sc[threadIdx.x] = tot;
+      }
+    }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const double n = sc[0], mu = sm_[0], M2 = s2[0] < 0.0 ? 0.0 : s2[0];
+    const float var = (float)(M2 / n);
+    if (save_mean) save_mean[c] = (float)mu;
+    if (save_invstd) save_invstd[c] = 1.0f / sqrtf(var + eps);
+    if (run_mean) run_mean[c] = (1.0f - factor) * run_mean[c] + factor * (float)mu;
+    if (run_var) { float unb = n > 1.0 ? (float)(M2 / (n - 1.0)) : var; run_var[c] = (1.0f - factor) * run_var[c] + factor * unb; }
+  }
+}
+
+// y = gamma * (x - mean) * invstd + beta from given statistics (optionally followed by relu)
+template <bool VEC, bool RELU>
+__global__ void __launch_bounds__(TPB) k_bn_apply(const float* __restrict__ x, float* __restrict__ y, const float* gamma, const float* beta,
+                                                  const float* save_mean, const float* save_invstd, int N, int C, int HW, int n_per) {
+  const int c = blockIdx.x, s = blockIdx.y;
+  const float mean = save_mean[c], invstd = save_invstd[c], g = gamma[c], b = beta[c];
+  const int n0 = s * n_per, n1 = min(N, n0 + n_per);
+  bn_foreach<VEC>(n0, n1, C, c, HW,
+    [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 r;
+      r.x = bn_affine(v.x, mean, invstd, g, b); r.y = bn_affine(v.y, mean, invstd, g, b);
+      r.z = bn_affine(v.z, mean, invstd, g, b); r.w = bn_affine(v.w, mean, invstd, g, b);
+      if (RELU) { r.x = r.x < 0.f ? 0.f : r.x; r.y = r.y < 0.f ? 0.f : r.y; r.z = r.z < 0.f ? 0.f : r.z; r.w = r.w < 0.f ? 0.f : r.w; }
+      *reinterpret_cast<float4*>(y + off) = r; },
+    [&](int64_t off) { float r = bn_affine(x[off], mean, invstd, g, b); if (RELU) r = r < 0.f ? 0.f : r; y[off] = r; });
+}
+
 static bool get_partial() {
   if (g_partial_ptr) return true;
   if (hipGetSymbolAddress((void**)&g_partial_ptr, HIP_SYMBOL(g_bn_partial)) != hipSuccess) { LH_FAIL("bn scratch symbol lookup failed"); return false; }
@@ -193,7 +263,43 @@ static bool get_partial() {
 }
 }  // namespace
 
+namespace lh {
+void bn_finalize_conv_partials(const float* partial, int C, int ncols, int col1, int g_main, int slots_main, int g_rem,
+                               float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor) {
+  const int slots_rem = col1 < ncols ? (int)cdiv(ncols - col1, g_rem) : 0;
+  hipLaunchKernelGGL(k_bn_finalize_conv, dim3(C), dim3(TPB), 0, g_stream, partial, C, ncols, col1, g_main, slots_main, g_rem, slots_main + slots_rem,
+                     save_mean, save_invstd, run_mean, run_var, eps, factor);
+}
+}  // namespace lh
+
 extern "C" {
+
+void lh_bn_stats(const float* x, float* save_mean, float* save_invstd, float* run_mean, float* run_var, int N, int C, int HW, float eps, float factor) {
+  ProfScope prof_(CAT_BN_FWD);
+  LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_stats: empty shape [%d,%d,%d]", N, C, HW);
+  LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_stats: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
+  if (!get_partial()) return;
+  Plan p = make_plan(N, C, HW, ((uintptr_t)x & 15) == 0);
+  dim3 grid(C, p.slices);
+  if (p.vec4) hipLaunchKernelGGL((k_bn_stats<true>), grid, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, HW, p.n_per);
+  else hipLaunchKernelGGL((k_bn_stats<false>), grid, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, HW, p.n_per);
+  hipLaunchKernelGGL(k_bn_finalize, dim3((unsigned)cdiv(C, TPB)), dim3(TPB), 0, g_stream, (const float*)g_partial_ptr, C, p.slices, save_mean, save_invstd,
+                     run_mean, run_var, eps, factor);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_bn_apply(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd, float* y,
+                 int N, int C, int HW, int relu) {
+  ProfScope prof_(CAT_BN_FWD);
+  LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_apply: empty shape [%d,%d,%d]", N, C, HW);
+  Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)y) & 15) == 0);
+  dim3 grid(C, p.slices);
+#define GO(V, R) hipLaunchKernelGGL((k_bn_apply<V, R>), grid, dim3(TPB), 0, g_stream, x, y, gamma, beta, save_mean, save_invstd, N, C, HW, p.n_per)
+  if (p.vec4) { if (relu) GO(true, true); else GO(true, false); }
+  else { if (relu) GO(false, true); else GO(false, false); }
+#undef GO
+  LH_CHECK_LAUNCH();
+}
 
 void lh_bn_infer(const float* x, const float* gamma, const float* beta, const float* run_mean, const float* run_var,
                  float* y, int N, int C, int HW, float eps) {

@@ -53,6 +53,12 @@ struct KernelCat {
   ~KernelCat() { g_kernel_cat = saved; }
 };
 
+// Batch-norm statistics from the per-piece (sum, sum of squares) a convolution epilogue left behind:
+// columns [0, col1) in pieces of g_main columns (slots 0 .. slots_main-1), columns [col1, ncols) in pieces of
+// g_rem columns after them; partial[c][slot] = (sum, sum of squares) as float2.  Writes mean, 1/sqrt(var+eps), updates running stats.
+void bn_finalize_conv_partials(const float* partial, int C, int ncols, int col1, int g_main, int slots_main, int g_rem,
+                               float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor);
+
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Grid for a grid-stride streaming kernel: enough blocks to cover n at `per_block`

@@ -193,6 +193,7 @@ struct LoadConvBwdFilterB {
 // ---- epilogue writing an NCHW activation: row i = channel, column j = (n, u, v) on a grid of
 //      Wc columns; the element lands at out[n][i][aH + eH*u][aW + eW*v] of an image W wide with PIX pixels.
 struct EpiConvOut {
+  static constexpr bool STATS = false;
   float* out; const float* bias; int chan, PIX, W, eH, eW, aH, aW; float beta;
   FastDiv dPIXc, dWc;
   struct Col { int off; bool valid; };
@@ -210,6 +211,11 @@ struct EpiConvOut {
     if (part) atomicAdd(p, v);
     else *p = beta == 0.f ? v : v + beta * *p;
   }
+};
+// The same epilogue, also leaving per-channel (sum, sum of squares) of every 32- or 64-column piece in `partial`.
+struct EpiConvOutStats : EpiConvOut {
+  static constexpr bool STATS = true;
+  float* partial; int slotBase, slotsTotal;      // partial[channel][slot] = (sum, sum of squares)
 };
 static EpiConvOut make_epi(float* out, const float* bias, int chan, int Himg, int Wimg, float beta) {   // dense: grid == image
   EpiConvOut ep; ep.out = out; ep.bias = bias; ep.chan = chan; ep.PIX = Himg * Wimg; ep.W = Wimg; ep.eH = 1; ep.eW = 1; ep.aH = 0; ep.aW = 0; ep.beta = beta;
@@ -300,12 +306,52 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
   if (tp.bn == 128) return launch_rounds<64, 128, 64, 64>(al, bl, ep, M, N, K);
   return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1);
 }
+
+// Where the statistics pieces of a forward launch lie (see bn_finalize_conv_partials).
+struct StatLayout { int col1, g_main, slots_main, g_rem, slots_rem; };
+
+// The tile plan launch_tiles would choose, for a launch that also leaves statistics pieces.  Returns false (and
+// launches nothing) for shapes that take the stream-K path, whose tiles are finished by several blocks.
+template <class AL, class BL>
+static bool plan_tiles_stats(int M, int N, int K, StatLayout& L, int& bm, int& bn) {
+  const int64_t t128 = cdiv(M, 128) * cdiv(N, 128), t64 = cdiv(M, 64) * cdiv(N, 128);
+  const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
+  const int64_t slabs = cdiv(K, CONV_BK);
+  if (few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)(2 * g_num_cu)) return false;
+  TilePick tp = pick_tile(M, N);
+  bm = tp.bm; bn = tp.bn;
+  L.col1 = N; L.g_main = bn / 2; L.g_rem = 32; L.slots_rem = 0;
+  if (bn == 128) {        // the surplus-tile split of launch_rounds
+    const int64_t tm = cdiv(M, bm), tn = cdiv(N, bn), tiles = tm * tn;
+    const int64_t slots = (int64_t)(bm == 128 ? igemm_blocks_per_cu<128, 128, CONV_BK, AL, BL, EpiConvOutStats>()
+                                              : igemm_blocks_per_cu<64, 128, CONV_BK, AL, BL, EpiConvOutStats>()) * g_num_cu;
+    const int64_t full = tiles / slots, rem = tiles - full * slots;
+    if (full >= 1 && rem > 0 && rem * 3 <= slots) {
+      const int c1 = (int)((full * slots / tm) * bn);
+      if (c1 > 0 && c1 < N) L.col1 = c1;
+    }
+  }
+  L.slots_main = (int)cdiv(L.col1, bn) * 2;
+  L.slots_rem = L.col1 < N ? (int)cdiv(N - L.col1, 64) * 2 : 0;
+  return true;
+}
+template <class AL, class BL>
+static bool launch_tiles_stats(const AL& al, const BL& bl, EpiConvOutStats ep, int M, int N, int K, const StatLayout& L, int bm, int bn) {
+  ep.slotBase = 0;
+  bool ok;
+  if (bm == 128) ok = igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, 0, 0, L.col1);
+  else if (bn == 128) ok = igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, 0, 0, L.col1);
+  else ok = igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1, 0, 0, L.col1);
+  if (ok && L.col1 < N) { ep.slotBase = L.slots_main; ok = igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1, 0, L.col1, N); }
+  return ok;
+}
+
+struct BnStatsOut { float* save_mean; float* save_invstd; float* run_mean; float* run_var; float eps, factor; };
 }  // namespace
 
-extern "C" {
-
-void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
-                   int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
+// Forward convolution; with `bn` also the batch-norm statistics of its output channels.
+static void conv_fwd_impl(const float* x, const float* w, const float* bias, float* y,
+                          int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW, const BnStatsOut* bn) {
   KernelCat kc_(CAT_CONV_FWD);
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_fwd: bad shape N%d C%d H%d W%d K%d R%d S%d s(%d,%d) p(%d,%d)", N, C, H, W, K, R, S, sH, sW, pH, pW);
@@ -328,7 +374,19 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
     LoadPlainK<true> al; al.base = wk; al.nbytes = wbytes; al.ld = CRS;
     LoadConvFwdTapB bl; bl.base = x; bl.nbytes = xbytes; bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
     bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dC.init(C); bl.dS.init(S);
-    ok = launch_tiles(al, bl, ep, K, N * PQ, CRS, y, (int64_t)N * K * PQ);
+    StatLayout L; int bm = 0, bn_ = 0;
+    if (bn && bias == nullptr && plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, L, bm, bn_)) {
+      const size_t pbytes = (size_t)(L.slots_main + L.slots_rem) * K * 2 * sizeof(float);
+      float* partial = (float*)lh_malloc_uninit(pbytes);
+      if (partial == nullptr) return;
+      EpiConvOutStats es; static_cast<EpiConvOut&>(es) = ep; es.partial = partial; es.slotBase = 0; es.slotsTotal = L.slots_main + L.slots_rem;
+      ok = launch_tiles_stats(al, bl, es, K, N * PQ, CRS, L, bm, bn_);
+      if (ok) bn_finalize_conv_partials(partial, K, N * PQ, L.col1, L.g_main, L.slots_main, L.g_rem, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, bn->eps, bn->factor);
+      lh_free_top(pbytes);
+      bn = nullptr;      // done
+    } else {
+      ok = launch_tiles(al, bl, ep, K, N * PQ, CRS, y, (int64_t)N * K * PQ);
+    }
     if (scratch) lh_free_top(scratch);
   } else {
     const bool avec = (CRS % 4 == 0) && (((uintptr_t)w & 15) == 0);
@@ -339,6 +397,23 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
   }
   if (!ok) return;
   LH_CHECK_LAUNCH();
+  // shapes whose launch leaves no statistics pieces: one extra pass over y
+  if (bn) lh_bn_stats(y, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, N, K, PQ, bn->eps, bn->factor);
+}
+
+extern "C" {
+
+void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
+                   int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
+  conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, nullptr);
+}
+
+void lh_conv2d_fwd_bnstats(const float* x, const float* w, const float* bias, float* y,
+                           int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW,
+                           float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor) {
+  LH_REQUIRE(save_mean && save_invstd, "lh_conv2d_fwd_bnstats: save_mean and save_invstd are required");
+  BnStatsOut bn{save_mean, save_invstd, run_mean, run_var, eps, factor};
+  conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, &bn);
 }
 
 void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,

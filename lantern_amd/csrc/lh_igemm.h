@@ -114,6 +114,7 @@ __device__ __forceinline__ float4 lh_fetch4(__amdgpu_buffer_rsrc_t rsrc, const L
 // ---- epilogue for row-major C ------------------------------------------------------------------
 // mode 0: C = alpha*acc + beta*C ; mode 1: atomicAdd(C, alpha*acc) (split-K)
 struct EpiRowMajor {
+  static constexpr bool STATS = false;
   float* C; int ldc; float alpha, beta; int atomic;
   struct Col { int j; bool valid; };
   __device__ __forceinline__ Col col(int j, int N) const { Col c; c.j = j; c.valid = j < N; return c; }
@@ -126,6 +127,17 @@ struct EpiRowMajor {
     else *p = alpha * v + (beta == 0.f ? 0.f : beta * *p);
   }
 };
+
+// Sum over the 32 lanes of each half of a wavefront (all 32 lanes get the total): DPP adds inside a
+// row of 16, one swizzle across the two rows.
+__device__ __forceinline__ float lh_half_sum32(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // row_mirror
+  v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));                      // lane ^ 16
+  return v;
+}
 
 // ---- the kernel ------------------------------------------------------------------------------------
 template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
@@ -291,14 +303,34 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
   }
 
   // D layout of a 32x32 block: column = lane % 32, row = 8*(v/4) + 4*(lane/32) + v%4
+  // With EP::STATS the same pass also forms per-row sums of the finished tile (the batch-norm statistics of a
+  // convolution's output rows = channels): every wavefront reduces its TM x TN piece over the columns and
+  // stores (sum, sum of squares) of each row into slot (2*tn + wn) of ep.partial; one writer per slot, no atomics.
+  typename EP::Col cs[NI];
 #pragma unroll
-  for (int ni = 0; ni < NI; ni++) {
-    const typename EP::Col cs = ep.col(n0 + wn * TN + ni * 32 + l32, gs.N);
+  for (int ni = 0; ni < NI; ni++) cs[ni] = ep.col(n0 + wn * TN + ni * 32 + l32, gs.N);
+  bool want_stats = false;
+  if constexpr (EP::STATS && !SK) want_stats = ep.partial != nullptr;
 #pragma unroll
-    for (int mi = 0; mi < MI; mi++) {
-      const int ib = m0 + wm * TM + mi * 32 + 4 * half;
+  for (int mi = 0; mi < MI; mi++) {
+    const int ib = m0 + wm * TM + mi * 32 + 4 * half;
 #pragma unroll
-      for (int v = 0; v < 16; v++) ep.store(cs, ib + 8 * (v / 4) + (v % 4), gs.M, acc[mi][ni][v], part);
+    for (int v = 0; v < 16; v++) {
+      const int row = ib + 8 * (v / 4) + (v % 4);
+      float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+      for (int ni = 0; ni < NI; ni++) {
+        const float val = acc[mi][ni][v];
+        ep.store(cs[ni], row, gs.M, val, part);
+        if constexpr (EP::STATS && !SK) { const float x = cs[ni].valid ? val : 0.f; s1 += x; s2 = fmaf(x, x, s2); }
+      }
+      if constexpr (EP::STATS && !SK) {
+        if (want_stats) {
+          // sums of the accumulators: the host uses this path only for launches without a bias
+          s1 = lh_half_sum32(s1); s2 = lh_half_sum32(s2);
+          if (l32 == 0 && row < gs.M) { float2* p = reinterpret_cast<float2*>(ep.partial) + (size_t)row * ep.slotsTotal + (ep.slotBase + tn * 2 + wn); *p = make_float2(s1, s2); }
+        }
+      }
     }
   }
   }  // segments

@@ -32,12 +32,15 @@ def set_backend(b):
 # runs instead of two; any other op flushes the parked launch first, so program order on the
 # stream is unchanged (at most one launch is ever parked).
 _pending = None
+FUSE_CONV_BN = True       # batchNorm right behind a convolution takes its statistics from the convolution's epilogue
 
 
 class _Pending:
-    def __init__(self, owner, launch):
+    def __init__(self, owner, launch, kind="relu", launch_bn=None):
         self.owner = owner          # the TensorR whose value is not computed yet
         self.launch = launch        # launch(relu: bool)
+        self.kind = kind            # "relu": a following in-place relu can be fused in; "conv": a following batchNorm can
+        self.launch_bn = launch_bn  # kind "conv": launch_bn(scale, bias, rmean, rvar, ybn, sm, si, relu)
 
 
 def _flush():
@@ -55,16 +58,16 @@ def get_backend():
     return _backend
 
 
-def _park(owner, launch):
+def _park(owner, launch, kind="relu", launch_bn=None):
     global _pending
     _flush()
-    _pending = _Pending(owner, launch)
+    _pending = _Pending(owner, launch, kind, launch_bn)
 
 
-def _take_pending(owner):
-    """The parked launch if it produces `owner`, else None (and nothing is flushed)."""
+def _take_pending(owner, kind="relu"):
+    """The parked launch if it produces `owner` and is of `kind`, else None (and nothing is flushed)."""
     global _pending
-    if _pending is not None and _pending.owner is owner:
+    if _pending is not None and _pending.owner is owner and _pending.kind == kind:
         p, _pending = _pending, None
         return p
     return None
@@ -630,6 +633,7 @@ class TensorR:
 
     # -- bn / softmax / loss ----------------------------------------------------------------------------------
     def batchNorm(self, scale, bias, runningMean, runningVar):
+        conv = _take_pending(self, "conv") if FUSE_CONV_BN else None         # before get_backend(), which would flush it
         be = get_backend()
         N, C, HW = self.x._bn_view()
         n = self.x.scalarCount
@@ -640,7 +644,10 @@ class TensorR:
 
         def launch(relu):
             st["relu"] = relu
-            _backend.batchNormTraining_into(self.x.data, scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, N, C, HW, relu)
+            if conv is not None:
+                conv.launch_bn(scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, relu)
+            else:
+                _backend.batchNormTraining_into(self.x.data, scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, N, C, HW, relu)
         _park(y, launch)
 
         def back():
@@ -678,13 +685,23 @@ class TensorR:
         be = get_backend()
         assert self.isInput or self._d is None or self._d.scalarCount == self.x.scalarCount, "For convBBP, THIS is either input or intermediate stage"
         assert self.x.rank == 4, "For convBBP, THIS is dim 4: batch, channel, row, col"
-        out, finput = self.x.conv2D_batch(kernel.x, bias.x if bias is not None else None, strides, pads)
-        y = TensorR._new(out)
+        assert kernel.x.rank == 4 and self.x.shape[1] == kernel.x.shape[1]
         N, C, H, W = self.x.shape; K, _, R, S = kernel.x.shape
         sH, sW = strides[0], strides[1]; pH, pW = Tensor._pads2(pads)
+        dims = (N, C, H, W, K, R, S, sH, sW, pH, pW)
+        kept = {"finput": None}
+        ybuf = be.mallocArray(N * K * conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW), zero=False)
+        y = TensorR._new(Tensor(ybuf, (N, K, conv_size(H, R, sH, pH), conv_size(W, S, sW, pW))))
+        xbuf, wbuf, bbuf = self.x.data, kernel.x.data, (bias.x.data if bias is not None else None)
+        # parked: a batchNorm right behind the convolution takes its statistics from the convolution's epilogue
+        def launch(relu):
+            kept["finput"] = _backend.conv2D_batch_into(xbuf, wbuf, bbuf, ybuf, *dims)
+        def launch_bn(scale, bb, rm, rv, ybn, sm, si, relu):
+            kept["finput"] = _backend.conv2D_batch_bn_into(xbuf, wbuf, bbuf, ybuf, dims, scale, bb, rm, rv, ybn, sm, si, relu)
+        _park(y, launch, "conv", launch_bn)
         def back():
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()
-            be.conv2D_batch_grad(self.x.data, xd, self.isInput, finput, kernel.x.data, kernel.d.data, y.d.data,
+            be.conv2D_batch_grad(self.x.data, xd, self.isInput, kept["finput"], kernel.x.data, kernel.d.data, y.d.data,
                                  bias.d.data if bias is not None else None, N, C, H, W, K, R, S, sH, sW, pH, pW, beta)
         _tape.append(back)
         return y

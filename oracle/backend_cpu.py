@@ -168,6 +168,8 @@ class BackendCPU(Backend):
     def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C_, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
         Pp, Q = conv_size(H, R, sH, pH), conv_size(W, S, sW, pW)
         scratch = None if x_in else self.mallocArray(N * C_ * R * S * Pp * Q)
+        if finput is None:      # the caller kept no unfolded input (the forward wrote into its own buffer): unfold again
+            _, finput = self.conv2D_batch(x, w, None, N, C_, H, W, K, R, S, sH, sW, pH, pW)
         self._c("lc_conv2d_bwd", P(finput.ptr), P(w.ptr), P(dy.ptr), P(0 if x_in else xd.ptr), P(wd.ptr), P(bd.ptr if bd is not None else 0),
                 P(0 if x_in else scratch.ptr), *[I(v) for v in (N, C_, H, W, K, R, S, sH, sW, pH, pW)])
 
