@@ -64,6 +64,22 @@ __global__ void __launch_bounds__(TPB) k_sum_dim_inner(const float* __restrict__
     y[i] = acc;
   }
 }
+// Few outputs, long reduction: a block sums a slice of `dim` for 64 consecutive inner positions (4 threads per
+// position, combined in LDS) and adds its partial sum into y, which the host has zeroed.
+__global__ void __launch_bounds__(TPB) k_sum_dim_split(const float* __restrict__ x, float* y, int dim, int inner, int per_slice) {
+  __shared__ float sm[4][64];
+  const int l = blockIdx.x * 64 + (threadIdx.x & 63), q = threadIdx.x >> 6;
+  const int s0 = blockIdx.y * per_slice, s1 = min(dim, s0 + per_slice);
+  const int64_t h = blockIdx.z;
+  float acc = 0.f;
+  if (l < inner) {
+    const float* p = x + h * dim * inner + l;
+    for (int s = s0 + q; s < s1; s += 4) acc += p[(int64_t)s * inner];
+  }
+  sm[q][threadIdx.x & 63] = acc;
+  __syncthreads();
+  if (q == 0 && l < inner) atomicAdd(y + h * inner + l, (sm[0][threadIdx.x] + sm[1][threadIdx.x]) + (sm[2][threadIdx.x] + sm[3][threadIdx.x]));
+}
 __global__ void __launch_bounds__(TPB) k_sum_rows(const float* __restrict__ x, float* y, int rows, int cols) {
   const int lane = threadIdx.x & 63;
   int64_t w = ((int64_t)blockIdx.x * TPB + threadIdx.x) >> 6, nw = ((int64_t)gridDim.x * TPB) >> 6;
@@ -171,6 +187,16 @@ void lh_add_scalar_from(float* dx, const float* dy1, float scale, int64_t n) { P
 void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner) { ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * inner <= 0) return;
   if (inner == 1) hipLaunchKernelGGL(k_sum_rows, dim3(stream_grid((int64_t)outer * 64, TPB)), dim3(TPB), 0, g_stream, x, y, outer, dim);
+  else if ((int64_t)outer * inner < 64 * (int64_t)g_num_cu && dim >= 512 && outer <= 65535) {
+    const int64_t base = (int64_t)outer * cdiv(inner, 64);
+    int slices = (int)cdiv(4 * (int64_t)g_num_cu, base);
+    if (slices > dim / 64) slices = dim / 64;
+    if (slices < 1) slices = 1;
+    const int per = (int)cdiv(dim, slices);
+    slices = (int)cdiv(dim, per);
+    lh_fill(y, 0.f, (int64_t)outer * inner);
+    hipLaunchKernelGGL(k_sum_dim_split, dim3((unsigned)cdiv(inner, 64), slices, outer), dim3(TPB), 0, g_stream, x, y, dim, inner, per);
+  }
   else hipLaunchKernelGGL(k_sum_dim_inner, dim3(stream_grid((int64_t)outer * inner, TPB)), dim3(TPB), 0, g_stream, x, y, outer, dim, inner);
   LH_CHECK_LAUNCH();
 }

@@ -14,46 +14,69 @@ using namespace lh;
 
 namespace {
 constexpr int TPB = 256;
-constexpr int UB = 4;              // batch rows whose loads are in flight together
 
 __device__ __forceinline__ float act_fwd(int mode, float v) { return mode == 1 ? tanhf(v) : (v < 0.f ? 0.f : v); }
 
 // Shared shape of both step kernels: out[b, j] = sum_k in[b, k] * Wrow[j, k] for the JC rows j0.. of this
 // block and every batch row b.  A lane owns k = lane, lane + 64, ...; the JC x NK weights it needs stay in
-// registers for the whole step.  The four wavefronts of a block take every fourth batch row, UB rows at a
-// time so that UB * NK loads are outstanding before the first use.
+// registers for the whole step.  The four wavefronts of a block take every fourth group of batch rows, a few rows at a
+// time so that several rows of loads are outstanding before the first use.
 //   in(b, k)        value of the input vector of row b at k          (k < H guaranteed)
 //   done(b, c, s)   called on lane 0 with the finished sum of row b, weight row j0 + c
-template <int NK, int JC, class In, class Done>
-__device__ __forceinline__ void rnn_rows(const float* __restrict__ W, int H, int B, int j0, bool use_w, In in, Done done) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  float w[JC][NK];
+template <int NK, int JC>
+__device__ __forceinline__ void rnn_load_w(const float* __restrict__ W, int H, int j0, bool use_w, float (&w)[JC][NK]) {
+  const int lane = threadIdx.x & 63;
 #pragma unroll
   for (int c = 0; c < JC; c++)
 #pragma unroll
     for (int i = 0; i < NK; i++) { const int k = lane + 64 * i; w[c][i] = (use_w && k < H && j0 + c < H) ? W[(int64_t)(j0 + c) * H + k] : 0.f; }
-  for (int b0 = wave * UB; b0 < B; b0 += 4 * UB) {
-    float h[UB][NK];
+}
+// V = (rows per pass) * JC partial sums per lane and pass go through the wavefront's LDS area ([V][65] floats) so that lane L
+// adds up value L % V over one group of lanes; the groups are then combined with xor-shuffles and V lanes
+// finish V outputs in parallel (bias, activation, store).
+constexpr int RED_LD = 65;
+template <int NK, int JC> struct RnnCfg { static constexpr int V = NK >= 32 ? 16 : 32; static constexpr int UBR = V / JC; };
+template <int NK, int JC, class In, class Done>
+__device__ __forceinline__ void rnn_rows_w(const float (&w)[JC][NK], int H, int B, int j0, float* red, In in, Done done) {
+  constexpr int V = RnnCfg<NK, JC>::V, UBR = RnnCfg<NK, JC>::UBR, G = 64 / V;
+  static_assert(UBR >= 1 && UBR * JC == V, "rows per pass times weight rows must be V");
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* my = red + wave * (V * RED_LD);
+  const int v = lane % V, grp = lane / V;
+  for (int b0 = wave * UBR; b0 < B; b0 += 4 * UBR) {
+    float h[UBR][NK];
 #pragma unroll
-    for (int u = 0; u < UB; u++)
+    for (int u = 0; u < UBR; u++)
 #pragma unroll
       for (int i = 0; i < NK; i++) { const int k = lane + 64 * i; h[u][i] = (b0 + u < B && k < H) ? in(b0 + u, k) : 0.f; }
 #pragma unroll
-    for (int u = 0; u < UB; u++) {
-      float s[JC];
+    for (int u = 0; u < UBR; u++)
 #pragma unroll
       for (int c = 0; c < JC; c++) {
         float t = 0.f;
 #pragma unroll
         for (int i = 0; i < NK; i++) t = fmaf(h[u][i], w[c][i], t);
-        s[c] = lh_wave_sum(t);
+        my[(u * JC + c) * RED_LD + lane] = t;
       }
-      if (lane == 0 && b0 + u < B) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float tot = 0.f;
 #pragma unroll
-        for (int c = 0; c < JC; c++) if (j0 + c < H) done(b0 + u, c, s[c]);
-      }
-    }
+    for (int i = 0; i < V; i++) tot += my[v * RED_LD + grp * V + i];
+#pragma unroll
+    for (int m = V; m < 64; m <<= 1) tot += __shfl_xor(tot, m, 64);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();                       // the area is free for the next pass
+    const int u = v / JC, c = v % JC;
+    if (grp == 0 && b0 + u < B && j0 + c < H) done(b0 + u, c, tot);
   }
+}
+template <int NK, int JC, class In, class Done>
+__device__ __forceinline__ void rnn_rows(const float* __restrict__ W, int H, int B, int j0, bool use_w, float* red, In in, Done done) {
+  float w[JC][NK];
+  rnn_load_w<NK, JC>(W, H, j0, use_w, w);
+  rnn_rows_w<NK, JC>(w, H, B, j0, red, in, done);
 }
 
 // One time step of both directions.
@@ -67,33 +90,35 @@ struct StepArgs {
 };
 template <int NK, int JC>
 __global__ void __launch_bounds__(TPB) k_rnn_fwd_step(StepArgs a, int B, int H, int ld, int mode) {
+  __shared__ float red[4 * RnnCfg<NK, JC>::V * RED_LD];
   const int d = blockIdx.y, j0 = blockIdx.x * JC;
   float* cur = a.cur[d]; const float* prev = a.prev[d]; const float* b1 = a.b1[d]; const float* b2 = a.b2[d];
-  rnn_rows<NK, JC>(a.W[d], H, B, j0, prev != nullptr,
+  rnn_rows<NK, JC>(a.W[d], H, B, j0, prev != nullptr, red,
     [&](int b, int k) { return prev ? prev[(int64_t)b * ld + k] : 0.f; },
     [&](int b, int c, float s) { const int j = j0 + c; float* p = cur + (int64_t)b * ld + j; *p = act_fwd(mode, *p + b1[j] + b2[j] + s); });
 }
 
-// One backward time step of both directions:
-//   dpre[b, j]   = (dy[b, j] + dh_in[b, j]) * act'(h[b, j])                (every block needs all j; block x stores columns with j / JC == x)
-//   dh_out[b, i] = sum_j dpre[b, j] * Wt[i, j]                             (Wt = W_hh transposed, rows = i)
+// One backward time step of both directions.  With g_t = dpre of time slice t (already complete):
+//   dh[b, i]       = sum_j g_t[b, j] * Wt[i, j]                               (Wt = W_hh transposed, rows = i)
+//   g_next[b, i]   = (dy_next[b, i] + dh[b, i]) * act'(h_next[b, i])          for the slice the next launch consumes
+// A block reads all of g_t and produces its own columns of g_next, so nothing is computed twice.  cur == nullptr
+// starts the chain: g_next = dy_next * act'(h_next).
 struct BwdArgs {
-  const float* dy[2]; const float* h[2]; float* dpre[2];          // time slice t, direction offset applied, row stride ld
-  const float* dh_in[2]; float* dh_out[2];                          // [B, H] dense; dh_in nullptr at the first (last in time) step
+  const float* cur[2];          // g_t: dpre + t*B*ld + d*H, or nullptr
+  const float* dy[2]; const float* h[2]; float* next[2];          // slice of the next step, direction offset applied
   const float* Wt[2];
 };
 template <int NK, int JC>
 __global__ void __launch_bounds__(TPB) k_rnn_bwd_step(BwdArgs a, int B, int H, int ld, int mode) {
+  __shared__ float red[4 * RnnCfg<NK, JC>::V * RED_LD];
   const int d = blockIdx.y, i0 = blockIdx.x * JC;
-  const float* dy = a.dy[d]; const float* hh = a.h[d]; const float* dh_in = a.dh_in[d]; float* dpre = a.dpre[d]; float* dh_out = a.dh_out[d];
-  rnn_rows<NK, JC>(a.Wt[d], H, B, i0, true,
-    [&](int b, int j) {
-      const float hv = hh[(int64_t)b * ld + j];
-      float g = dy[(int64_t)b * ld + j] + (dh_in ? dh_in[(int64_t)b * H + j] : 0.f);
-      g = mode == 1 ? g * (1.0f - hv * hv) : (hv > 0.f ? g : 0.f);
-      if (j >= i0 && j < i0 + JC) dpre[(int64_t)b * ld + j] = g;
-      return g; },
-    [&](int b, int c, float s) { dh_out[(int64_t)b * H + i0 + c] = s; });
+  const float* cur = a.cur[d]; const float* dy = a.dy[d]; const float* hh = a.h[d]; float* next = a.next[d];
+  rnn_rows<NK, JC>(a.Wt[d], H, B, i0, cur != nullptr, red,
+    [&](int b, int j) { return cur ? cur[(int64_t)b * ld + j] : 0.f; },
+    [&](int b, int c, float s) {
+      const int64_t o = (int64_t)b * ld + i0 + c;
+      const float hv = hh[o], g = dy[o] + s;
+      next[o] = mode == 1 ? g * (1.0f - hv * hv) : (hv > 0.f ? g : 0.f); });
 }
 
 // hidden sizes up to 64 * NK, JC weight rows per block (JC * NK <= 128 registers of weights)
@@ -227,28 +252,28 @@ void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
   LH_REQUIRE(beta_dx == 0.f || beta_dx == 1.f, "lh_rnn_bwd: beta must be 0 or 1");
   LH_REQUIRE(x && y && dy && w && dw, "lh_rnn_bwd: null operand");
   const int D = bidir ? 2 : 1, ld = D * H;
-  // scratch from the top of the arena: dpre [T*B, D*H], W_hh^T per direction, two dh buffers per direction, column sums
-  const size_t n_dpre = (size_t)T * B * ld, n_wt = (size_t)D * H * H, n_dh = (size_t)2 * D * B * H, n_cs = (size_t)ld;
-  const size_t bytes = (n_dpre + n_wt + n_dh + n_cs) * sizeof(float);
+  // scratch from the top of the arena: dpre [T*B, D*H], W_hh^T per direction, column sums
+  const size_t n_dpre = (size_t)T * B * ld, n_wt = (size_t)D * H * H, n_cs = (size_t)ld;
+  const size_t bytes = (n_dpre + n_wt + n_cs) * sizeof(float);
   float* scratch = (float*)lh_malloc_uninit(bytes);
   if (scratch == nullptr) return;
-  float* dpre = scratch; float* wt = dpre + n_dpre; float* dh = wt + n_wt; float* colsum = dh + n_dh;
+  float* dpre = scratch; float* wt = dpre + n_dpre; float* colsum = wt + n_wt;
   for (int d = 0; d < D; d++) {
     const float* Whh = w + d * dir_params(I, H) + (size_t)H * I;
     lh_trans(Whh, wt + (size_t)d * H * H, H, H);
   }
   {
     ProfScope prof_(CAT_RNN);
-    for (int step = T - 1; step >= 0; step--) {
+    // launch k produces dpre of the k-th slice in processing order (forward direction: t = T-1-k, reverse: t = k)
+    for (int k = 0; k < T; k++) {
       BwdArgs a;
-      const int cur_buf = (T - 1 - step) & 1;
       for (int d = 0; d < 2; d++) {
         const int dd = d < D ? d : 0;
-        const int t = dd == 0 ? step : T - 1 - step;
-        const size_t off = (size_t)t * B * ld + dd * H;
-        a.dy[d] = dy + off; a.h[d] = y + off; a.dpre[d] = dpre + off;
-        a.dh_in[d] = step == T - 1 ? nullptr : dh + ((size_t)(cur_buf ^ 1) * D + dd) * B * H;
-        a.dh_out[d] = dh + ((size_t)cur_buf * D + dd) * B * H;
+        const int tn = dd == 0 ? T - 1 - k : k;                 // slice produced
+        const int tc = dd == 0 ? tn + 1 : tn - 1;               // slice consumed (processed just before)
+        const size_t on = (size_t)tn * B * ld + dd * H;
+        a.cur[d] = k == 0 ? nullptr : dpre + (size_t)tc * B * ld + dd * H;
+        a.dy[d] = dy + on; a.h[d] = y + on; a.next[d] = dpre + on;
         a.Wt[d] = wt + (size_t)dd * H * H;
       }
       launch_bwd_step(a, D, B, H, ld, mode);

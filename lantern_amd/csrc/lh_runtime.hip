@@ -91,7 +91,9 @@ void lh_cleanup(void) {
   g_heap = nullptr; g_stream = nullptr; g_heap_bytes = g_top = 0;
 }
 
-void lh_sync(void) { LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH(); }
+void lh_sync(void) {
+  LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH();
+}
 
 static void* bump(size_t bytes, bool zero) {
   if (!g_heap) { LH_FAIL("lh_malloc before lh_setup"); return nullptr; }

@@ -288,7 +288,7 @@ def test_sum_mean_and_grads(pair, n):
     check_all(outs, rtol=2e-4)
 
 
-@pytest.mark.parametrize("oci", [(64, 49, 1), (1, 5, 1), (8, 3, 20), (100, 1, 7), (3, 1000, 1), (2, 64, 3000)])
+@pytest.mark.parametrize("oci", [(64, 49, 1), (1, 5, 1), (8, 3, 20), (100, 1, 7), (3, 1000, 1), (2, 64, 3000), (1, 2000, 300), (3, 700, 100), (1, 5920, 1600)])
 def test_sum_dim_and_grad(pair, oci):
     o, d, i = oci
     rng = np.random.RandomState(22); x = rng.randn(o, d, i).astype(np.float32); dy = rng.randn(o, i).astype(np.float32)
@@ -603,3 +603,40 @@ def test_conv_with_batchnorm_statistics(pair, case, relu):
         for o in outs:
             o[1][edge & (np.abs(o[1]) < 4e-5)] = 0.0
     check_all(outs, rtol=2e-4)
+
+
+# ---- convolution with batch-norm statistics from its epilogue -----------------------------------------
+CONV_BN = [(64, 64, 56, 64, 1, 1, 0, False),      # 64-row GEMM, 64x128 tiles
+           (8, 64, 56, 256, 1, 1, 0, False),      # 128x128 tiles
+           (64, 256, 14, 1024, 1, 1, 0, False),   # 784 tiles: a full round + surplus columns in 64x64 tiles
+           (4, 32, 15, 48, 3, 2, 1, False),       # odd sizes, partial tiles in both directions
+           (2, 16, 9, 24, 3, 1, 1, True),         # with a bias: statistics come from a pass over y
+           (64, 512, 7, 512, 3, 1, 1, False),     # few tiles, long reduction: the shared-tile path, statistics from a pass over y
+           (2, 3, 20, 16, 5, 1, 2, False)]        # channels not a multiple of 16: the general loader, pass over y
+
+
+@pytest.mark.parametrize("case", CONV_BN, ids=lambda c: "N%d_C%d_H%d_K%d_k%d_s%d_p%d_b%d" % c)
+@pytest.mark.parametrize("relu", [False, True], ids=["plain", "relu"])
+def test_conv_with_batchnorm_statistics(pair, case, relu):
+    N, Cc, H, K, k, s, p, with_bias = case
+    P = B.conv_size(H, k, s, p)
+    dims = (N, Cc, H, H, K, k, k, s, s, p, p)
+    rng = np.random.RandomState(33)
+    x = rng.randn(N, Cc, H, H).astype(np.float32); w = (rng.randn(K, Cc, k, k) / np.sqrt(Cc * k * k)).astype(np.float32)
+    bias = (rng.randn(K) * 2).astype(np.float32) if with_bias else None
+    g = (rng.rand(K) + 0.5).astype(np.float32); b = rng.randn(K).astype(np.float32)
+
+    def f(be, up, down):
+        n = N * K * P * P
+        yconv, ybn, sm, si = be.mallocArray(n), be.mallocArray(n), be.mallocArray(K), be.mallocArray(K)
+        rm, rv = up(np.zeros(K, np.float32)), up(np.ones(K, np.float32))
+        be.conv2D_batch_bn_into(up(x), up(w), up(bias) if with_bias else None, yconv, dims, up(g), up(b), rm, rv, ybn, sm, si, relu)
+        return [down(yconv, (N, K, P, P)), down(ybn, (N, K, P, P)), down(sm, (K,)), down(si, (K,)), down(rm, (K,)), down(rv, (K,))]
+
+    outs = pair.run(f)
+    if relu:        # values within rounding of zero may land on either side of the relu
+        edge = np.abs(outs[0][1]) < 2e-5
+        for o in outs:
+            o[1][edge & (np.abs(o[1]) < 4e-5)] = 0.0
+    check_all(outs, rtol=2e-4)
+
