@@ -48,7 +48,7 @@ def make_trainer(args, batch, cpu=False):
         return Trainer(batch=batch, lr=0.0005), batch, "LeNet-style CNN training step (configs[0]): batch %d, 1x28x28, SGD lr 0.0005, dropout 0.5" % batch
     if w == "treelstm":
         from lantern_amd.apps.treelstm import Trainer
-        return Trainer(n_trees=16 if cpu else 64, vocab=20000), 1, \
+        return Trainer(n_trees=64, vocab=20000), 1, \
             "TreeLSTM sentiment step (configs[1]): one tree of 5-50 leaves per step, hidden 150, embedding 300, Adagrad lr 0.05"
     if w == "deepspeech2":
         from lantern_amd.apps.deepspeech2 import Trainer
@@ -110,10 +110,21 @@ def run_cpu(args):
     be = BackendCPU(threads=threads)
     be.setup()
     la.set_backend(be)
-    batch = {"resnet50": args.cpu_batch, "squeezenet": 64, "lenet": 100, "treelstm": 1, "deepspeech2": 2}[args.workload]
+    batch = {"resnet50": args.cpu_batch, "squeezenet": 64, "lenet": 100, "treelstm": 1, "deepspeech2": 4}[args.workload]
     tr, per_step, _ = make_trainer(args, batch, cpu=True)
+    if args.workload == "treelstm":              # the very trees the device run times: W warm-up trees, then the next K, three times over
+        for _ in range(args.warmup):
+            tr.step(); tr.end_step()
+        t0 = time.perf_counter()
+        n = 0
+        for _ in range(3):
+            tr.next = args.warmup
+            for _ in range(args.steps):
+                tr.step(); tr.end_step(); n += 1
+        dt = time.perf_counter() - t0
+        return {"value": per_step * n / dt, "cores": threads, "steps": n, "batch": batch}
     tr.step(); tr.end_step()                     # warm-up
-    max_steps = {"resnet50": args.cpu_steps, "squeezenet": 10, "lenet": 50, "treelstm": 32, "deepspeech2": 2}[args.workload]
+    max_steps = {"resnet50": args.cpu_steps, "squeezenet": 30, "lenet": 200, "deepspeech2": 4}[args.workload]
     t0 = time.perf_counter()
     n = 0
     while n < max_steps:
@@ -136,8 +147,8 @@ def main():
     ap.add_argument("--frames", type=int, default=400)
     ap.add_argument("--hidden", type=int, default=800)
     ap.add_argument("--heap-gb", type=float, default=48.0)
-    ap.add_argument("--cpu-batch", type=int, default=4)
-    ap.add_argument("--cpu-steps", type=int, default=2)
+    ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--cpu-steps", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args()

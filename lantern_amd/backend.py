@@ -32,8 +32,18 @@ class Buf:
         return Buf(self.ptr + 4 * int(k), self.n - int(k) if n is None else n, self.keep)
 
 
+_INTS_CACHE = {}
+
+
 def _ints(seq):
-    return (C.c_int * len(seq))(*[int(v) for v in seq])
+    """A C int array of the values (shape and permutation arguments); the arrays are read-only, so equal tuples share one."""
+    key = tuple(seq)
+    arr = _INTS_CACHE.get(key)
+    if arr is None:
+        arr = (C.c_int * len(key))(*[int(v) for v in key])
+        if len(_INTS_CACHE) < 4096:
+            _INTS_CACHE[key] = arr
+    return arr
 
 
 def dim_broadcast(a, b):

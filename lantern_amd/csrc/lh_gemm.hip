@@ -65,13 +65,30 @@ __global__ void __launch_bounds__(TPB) k_sgemv_n(int m, int n, float alpha, cons
     if (lane == 0) y[w] = alpha * acc + (beta == 0.f ? 0.f : beta * y[w]);
   }
 }
-// y[n] = alpha * A[m,n]^T x[m] + beta*y : thread per column, coalesced along n.
+// y[n] = alpha * A[m,n]^T x[m] + beta*y : a block owns 32 columns; its 8 row groups each sum every 8th row
+// (independent, coalesced loads), and LDS combines the groups.
 __global__ void __launch_bounds__(TPB) k_sgemv_t(int m, int n, float alpha, const float* __restrict__ A, int lda, const float* __restrict__ x, float beta, float* y) {
-  int j = blockIdx.x * TPB + threadIdx.x;
-  if (j >= n) return;
-  float acc = 0.f;
-  for (int i = 0; i < m; i++) acc += A[(int64_t)i * lda + j] * x[i];
-  y[j] = alpha * acc + (beta == 0.f ? 0.f : beta * y[j]);
+  __shared__ float sm[8][33];
+  const int c = threadIdx.x & 31, g = threadIdx.x >> 5;
+  const int j = blockIdx.x * 32 + c;
+  float acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;
+  if (j < n) {
+    const float* a = A + j;
+    int i = g;
+    for (; i + 24 < m; i += 32) {
+      acc0 += a[(int64_t)i * lda] * x[i];
+      acc1 += a[(int64_t)(i + 8) * lda] * x[i + 8];
+      acc2 += a[(int64_t)(i + 16) * lda] * x[i + 16];
+      acc3 += a[(int64_t)(i + 24) * lda] * x[i + 24];
+    }
+    for (; i < m; i += 8) acc0 += a[(int64_t)i * lda] * x[i];
+  }
+  sm[g][c] = (acc0 + acc1) + (acc2 + acc3);
+  __syncthreads();
+  if (g == 0 && j < n) {
+    float acc = ((sm[0][c] + sm[1][c]) + (sm[2][c] + sm[3][c])) + ((sm[4][c] + sm[5][c]) + (sm[6][c] + sm[7][c]));
+    y[j] = alpha * acc + (beta == 0.f ? 0.f : beta * y[j]);
+  }
 }
 __global__ void __launch_bounds__(TPB) k_ger(int m, int n, const float* __restrict__ u, const float* __restrict__ v, float* A) {
   int64_t tot = (int64_t)m * n;
@@ -146,7 +163,7 @@ void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, con
   ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
   if (!trans) hipLaunchKernelGGL(k_sgemv_n, dim3(stream_grid((int64_t)m * 64, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
-  else hipLaunchKernelGGL(k_sgemv_t, dim3((unsigned)cdiv(n, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
+  else hipLaunchKernelGGL(k_sgemv_t, dim3((unsigned)cdiv(n, 32)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
   LH_CHECK_LAUNCH();
 }
 void lh_ger(int m, int n, const float* u, const float* v, float* A) {

@@ -13,6 +13,10 @@ int g_num_cu = 256;
 static char g_err[1024] = "";
 static char* g_heap = nullptr;
 static size_t g_heap_bytes = 0, g_top = 0, g_peak = 0;
+// [g_top, g_zero_end) is known to read zero (when g_zero_end > g_top): small zero-filled blocks are cleared a
+// window at a time, so a run of them costs one fill launch instead of one each.
+static size_t g_zero_end = 0;
+static const size_t ZERO_AHEAD = 1u << 20;
 
 bool fail(const char* file, int line, const char* fmt, ...) {
   char msg[768];
@@ -81,14 +85,14 @@ void lh_setup(size_t heap_bytes) {
   LH_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
   heap_bytes = (heap_bytes + 255) & ~(size_t)255;
   LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
-  g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0;
+  g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0; g_zero_end = 0;
 }
 
 void lh_cleanup(void) {
   if (g_stream) (void)hipStreamSynchronize(g_stream);
   if (g_heap) (void)hipFree(g_heap);
   if (g_stream) (void)hipStreamDestroy(g_stream);
-  g_heap = nullptr; g_stream = nullptr; g_heap_bytes = g_top = 0;
+  g_heap = nullptr; g_stream = nullptr; g_heap_bytes = g_top = g_zero_end = 0;
 }
 
 void lh_sync(void) {
@@ -105,9 +109,16 @@ static void* bump(size_t bytes, bool zero) {
     return nullptr;
   }
   void* p = g_heap + g_top;
+  if (zero && g_top + need > g_zero_end) {
+    const size_t from = g_zero_end > g_top ? g_zero_end : g_top;
+    size_t to = g_top + need;
+    if (need < ZERO_AHEAD) to = g_top + ZERO_AHEAD < g_heap_bytes ? g_top + ZERO_AHEAD : g_heap_bytes;
+    ProfScope prof_(CAT_FILL);
+    zero_async(g_heap + from, to - from);
+    g_zero_end = to;
+  }
   g_top += need;
   if (g_top > g_peak) g_peak = g_top;
-  if (zero) { ProfScope prof_(CAT_FILL); zero_async(p, need); }
   return p;
 }
 void* lh_malloc(size_t bytes) { return bump(bytes, true); }
@@ -117,11 +128,13 @@ void lh_free_top(size_t bytes) {
   if (need == 0) need = 256;
   LH_REQUIRE(need <= g_top, "lh_free_top(%zu) below the arena base", bytes);
   g_top -= need;
+  g_zero_end = g_top;            // what was handed out above the new top may have been written
 }
 size_t lh_mark(void) { return g_top; }
 void lh_rewind(size_t mark) {
   LH_REQUIRE(mark <= g_top && (mark & 255) == 0, "lh_rewind(%zu): not a mark at or below the top (%zu)", mark, g_top);
   g_top = mark;
+  g_zero_end = mark;
 }
 size_t lh_heap_used(void) { return g_top; }
 size_t lh_heap_peak(void) { return g_peak; }

@@ -331,12 +331,15 @@ def test_nll_loss_and_grad(pair):
 
 
 # ---- dot family --------------------------------------------------------------------------------------
+SHAPES_MV = [(150, 300), (5, 150), (1, 1), (1000, 2048), (33, 7), (150, 150), (9, 31), (257, 65), (32, 32)]
+
+
 def test_dot_family_at_treelstm_and_classifier_shapes(pair):
     rng = np.random.RandomState(25)
 
     def f(be, up, down):
         outs = []
-        for m, n in [(150, 300), (5, 150), (1, 1), (1000, 2048), (33, 7)]:
+        for m, n in SHAPES_MV:
             Mx = rng_m[(m, n)]; v = rng_v[n]; w = rng_v2[m]
             outs.append(down(be.matrixVectorDot(up(Mx), up(v), m, n), (m,)))
             outs.append(down(be.vectorVectorDot(up(v), up(v[::-1].copy()), n), (1,)))
@@ -350,9 +353,9 @@ def test_dot_family_at_treelstm_and_classifier_shapes(pair):
             yd = up(np.ones(d2 * d3, np.float32)); be.add_dotTrans1(yd, up(X), up(O), d1, d2, d3); outs.append(down(yd, (d2, d3)))
         return outs
 
-    rng_m = {s: rng.randn(*s).astype(np.float32) for s in [(150, 300), (5, 150), (1, 1), (1000, 2048), (33, 7)]}
-    rng_v = {n: rng.randn(n).astype(np.float32) for n in (300, 150, 1, 2048, 7)}
-    rng_v2 = {m: rng.randn(m).astype(np.float32) for m in (150, 5, 1, 1000, 33)}
+    rng_m = {s: rng.randn(*s).astype(np.float32) for s in SHAPES_MV}
+    rng_v = {n: rng.randn(n).astype(np.float32) for _, n in SHAPES_MV}
+    rng_v2 = {m: rng.randn(m).astype(np.float32) for m, _ in SHAPES_MV}
     rng_g = {}
     for d1, d2, d3 in [(64, 2048, 1000), (100, 320, 50), (3, 4, 5), (20, 1, 7), (1, 33, 1)]:
         for s in ((d1, d2), (d2, d3), (d1, d3)):
@@ -486,6 +489,28 @@ def test_arena_zeroing_alignment_rewind_and_overflow(on_hip):
         be.mallocArray(be.heap_bytes)                              # 4x the arena: refused, nothing allocated
     assert lib.lh_heap_used() <= used                              # nothing was taken by the refused request
     z = be.mallocArray(4); assert not be.toHost(z, 4).any()        # the library keeps working after an error
+    be.resetMallocAddr(mark)
+
+
+def test_arena_small_blocks_read_zero_after_dirty_memory_uninit_blocks_and_pops(on_hip):
+    """Zero-filled blocks are cleared a window at a time; whatever was written there before (a rewound block, an
+    uninitialised block handed out inside the window and popped again) must not show through."""
+    be = on_hip
+    lib = be.lib
+    mark = be.getMallocAddr()
+    big = be.mallocArray(1 << 20, zero=False); be.fillInPlace(big, 1 << 20, 7.0)          # 4 MiB of sevens
+    be.resetMallocAddr(mark)
+    blocks = [be.mallocArray(n) for n in (3, 150, 45000, 1, 300000, 64, 150)]            # crosses several windows
+    for blk, n in zip(blocks, (3, 150, 45000, 1, 300000, 64, 150)):
+        assert not be.toHost(blk, n).any()
+        be.fillInPlace(blk, n, 5.0)
+    top = lib.lh_heap_used()
+    s = be.mallocArray(5000, zero=False); be.fillInPlace(s, 5000, 9.0)                    # scratch inside the cleared window
+    lib.lh_free_top(5000 * 4)
+    assert lib.lh_heap_used() == top
+    z = be.mallocArray(5000); assert z.ptr == s.ptr and not be.toHost(z, 5000).any()
+    u = be.mallocArray(100, zero=False); be.fillInPlace(u, 100, 2.0)
+    z2 = be.mallocArray(100); assert not be.toHost(z2, 100).any() and (be.toHost(u, 100) == 2.0).all()
     be.resetMallocAddr(mark)
 
 
