@@ -113,12 +113,32 @@ extern "C" {
 
 }  // extern "C"
 // MFMA path for all but tiny products; the 64x64 register-tiled kernel covers those.
+struct SgemmPlan { TilePick tp; int split; };
+// Few output tiles and a long reduction (weight gradients over many rows): the reduction is cut into `split`
+// slices whose blocks add into C with fp32 atomics; C is scaled by beta beforehand.
+static SgemmPlan sgemm_plan(int m, int n, int k) {
+  SgemmPlan p; p.tp = pick_tile(m, n); p.split = 1;
+  const int64_t tiles = cdiv(m, p.tp.bm) * cdiv(n, p.tp.bn);
+  if (k >= 1024 && 2 * tiles <= 3 * (int64_t)g_num_cu) {
+    TilePick big = (m >= 128 && n >= 128) ? TilePick{128, 128} : (n >= 128 ? TilePick{64, 128} : TilePick{64, 64});
+    const int64_t bt = cdiv(m, big.bm) * cdiv(n, big.bn);
+    int split = (int)cdiv(3 * (int64_t)g_num_cu, bt);
+    const int max_split = k / 256;
+    if (split > max_split) split = max_split;
+    if (split > 1) { p.tp = big; p.split = split; }
+  }
+  return p;
+}
+__global__ void __launch_bounds__(TPB) k_scale_rows(float* C, int ldc, int m, int n, float beta) {
+  const int64_t tot = (int64_t)m * n;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < tot; i += st) { const int r = (int)(i / n), c = (int)(i - (int64_t)r * n); float* p = C + (int64_t)r * ldc + c; *p = beta == 0.f ? 0.f : beta * *p; }
+}
 template <class AL, class BL>
-static bool sgemm_mfma(const AL& al, const BL& bl, const EpiRowMajor& ep, int m, int n, int k) {
-  TilePick tp = pick_tile(m, n);
-  if (tp.bm == 128) return igemm_launch<128, 128, 16>(al, bl, ep, m, n, k, 1);
-  if (tp.bn == 128) return igemm_launch<64, 128, 16>(al, bl, ep, m, n, k, 1);
-  return igemm_launch<64, 64, 16>(al, bl, ep, m, n, k, 1);
+static bool sgemm_mfma(const AL& al, const BL& bl, const EpiRowMajor& ep, int m, int n, int k, const SgemmPlan& pl) {
+  if (pl.tp.bm == 128) return igemm_launch<128, 128, 16>(al, bl, ep, m, n, k, pl.split);
+  if (pl.tp.bn == 128) return igemm_launch<64, 128, 16>(al, bl, ep, m, n, k, pl.split);
+  return igemm_launch<64, 64, 16>(al, bl, ep, m, n, k, pl.split);
 }
 
 void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, int lda,
@@ -130,6 +150,11 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   LH_REQUIRE(A && B && C, "lh_sgemm: null operand");
   if ((int64_t)m * n * k >= (1 << 18) && m >= 16 && n >= 16) {
     EpiRowMajor ep; ep.C = C; ep.ldc = ldc; ep.alpha = alpha; ep.beta = beta; ep.atomic = 0;
+    const SgemmPlan pl = sgemm_plan(m, n, k);
+    if (pl.split > 1) {
+      if (beta != 1.f) { hipLaunchKernelGGL(k_scale_rows, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, C, ldc, m, n, beta); LH_CHECK_LAUNCH(); }
+      ep.atomic = 1; ep.beta = 1.f;
+    }
     const bool av = (lda % 4 == 0) && (((uintptr_t)A & 15) == 0) && (k % 4 == 0);
     const bool bv = (ldb % 4 == 0) && (((uintptr_t)B & 15) == 0) && (k % 4 == 0);
     const size_t abytes = (size_t)(ta ? k : m) * lda * 4, bbytes = (size_t)(tb ? n : k) * ldb * 4;
@@ -141,11 +166,11 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
     LoadPlainK<false> bks; bks.base = B; bks.nbytes = (uint32_t)bbytes; bks.ld = ldb;
     LoadPlainT bt; bt.base = B; bt.nbytes = (uint32_t)bbytes; bt.ld = ldb;
     bool ok;
-    if (!ta && !tb) ok = av ? sgemm_mfma(akv, bt, ep, m, n, k) : sgemm_mfma(aks, bt, ep, m, n, k);
-    else if (!ta && tb) ok = av ? (bv ? sgemm_mfma(akv, bkv, ep, m, n, k) : sgemm_mfma(akv, bks, ep, m, n, k))
-                                : (bv ? sgemm_mfma(aks, bkv, ep, m, n, k) : sgemm_mfma(aks, bks, ep, m, n, k));
-    else if (ta && !tb) ok = sgemm_mfma(at, bt, ep, m, n, k);
-    else ok = bv ? sgemm_mfma(at, bkv, ep, m, n, k) : sgemm_mfma(at, bks, ep, m, n, k);
+    if (!ta && !tb) ok = av ? sgemm_mfma(akv, bt, ep, m, n, k, pl) : sgemm_mfma(aks, bt, ep, m, n, k, pl);
+    else if (!ta && tb) ok = av ? (bv ? sgemm_mfma(akv, bkv, ep, m, n, k, pl) : sgemm_mfma(akv, bks, ep, m, n, k, pl))
+                                : (bv ? sgemm_mfma(aks, bkv, ep, m, n, k, pl) : sgemm_mfma(aks, bks, ep, m, n, k, pl));
+    else if (ta && !tb) ok = sgemm_mfma(at, bt, ep, m, n, k, pl);
+    else ok = bv ? sgemm_mfma(at, bkv, ep, m, n, k, pl) : sgemm_mfma(at, bks, ep, m, n, k, pl);
     if (!ok) return;
     LH_CHECK_LAUNCH();
     return;

@@ -18,46 +18,74 @@ constexpr int TPB = 256;
 __device__ __forceinline__ float act_fwd(int mode, float v) { return mode == 1 ? tanhf(v) : (v < 0.f ? 0.f : v); }
 
 // Shared shape of both step kernels: out[b, j] = sum_k in[b, k] * Wrow[j, k] for the JC rows j0.. of this
-// block and every batch row b.  A lane owns k = lane, lane + 64, ...; the JC x NK weights it needs stay in
-// registers for the whole step.  The four wavefronts of a block take every fourth group of batch rows, a few rows at a
-// time so that several rows of loads are outstanding before the first use.
-//   in(b, k)        value of the input vector of row b at k          (k < H guaranteed)
-//   done(b, c, s)   called on lane 0 with the finished sum of row b, weight row j0 + c
-template <int NK, int JC>
-__device__ __forceinline__ void rnn_load_w(const float* __restrict__ W, int H, int j0, bool use_w, float (&w)[JC][NK]) {
+// block and every batch row b.  A lane owns NK values of k (V4: groups of four consecutive ones, k = 256 q + 4 lane + r,
+// fetched as one 16-byte load; otherwise k = lane + 64 i); the JC x NK weights it needs stay in registers for the
+// whole step.  The four wavefronts of a block take every fourth group of batch rows, a few rows at a time, and the
+// loads of the next group are issued before the sums of the current one are reduced.
+template <int NK, bool V4>
+__device__ __forceinline__ void rnn_load_row(const float* __restrict__ row, int H, bool use, float (&r)[NK]) {
   const int lane = threadIdx.x & 63;
+  if (V4) {
 #pragma unroll
-  for (int c = 0; c < JC; c++)
+    for (int q = 0; q < NK / 4; q++) {
+      const int k = 256 * q + 4 * lane;
+      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (use && k < H) t = *reinterpret_cast<const float4*>(row + k);      // H % 4 == 0: the whole group is inside the row
+      r[4 * q] = t.x; r[4 * q + 1] = t.y; r[4 * q + 2] = t.z; r[4 * q + 3] = t.w;
+    }
+  } else {
 #pragma unroll
-    for (int i = 0; i < NK; i++) { const int k = lane + 64 * i; w[c][i] = (use_w && k < H && j0 + c < H) ? W[(int64_t)(j0 + c) * H + k] : 0.f; }
+    for (int i = 0; i < NK; i++) { const int k = lane + 64 * i; r[i] = (use && k < H) ? row[k] : 0.f; }
+  }
+}
+template <int NK, int JC, bool V4>
+__device__ __forceinline__ void rnn_load_w(const float* __restrict__ W, int H, int j0, bool use_w, float (&w)[JC][NK]) {
+#pragma unroll
+  for (int c = 0; c < JC; c++) rnn_load_row<NK, V4>(W + (int64_t)(j0 + c < H ? j0 + c : 0) * H, H, use_w && j0 + c < H, w[c]);
 }
 // V = (rows per pass) * JC partial sums per lane and pass go through the wavefront's LDS area ([V][65] floats) so that lane L
 // adds up value L % V over one group of lanes; the groups are then combined with xor-shuffles and V lanes
 // finish V outputs in parallel (bias, activation, store).
+//   in, ld, use_in   input vectors: row b starts at in + b * ld (read only when use_in)
+//   pre(b, c)        called on a finishing lane before the sums: fetches what done() will need (so that those
+//                    loads are in flight during the arithmetic)
+//   done(b, c, s, f) called on the same lane with the finished sum of row b, weight row j0 + c
+struct RnnPre { float a, b, c; };
 constexpr int RED_LD = 65;
 template <int NK, int JC> struct RnnCfg { static constexpr int V = NK >= 32 ? 16 : 32; static constexpr int UBR = V / JC; };
-template <int NK, int JC, class In, class Done>
-__device__ __forceinline__ void rnn_rows_w(const float (&w)[JC][NK], int H, int B, int j0, float* red, In in, Done done) {
-  constexpr int V = RnnCfg<NK, JC>::V, UBR = RnnCfg<NK, JC>::UBR, G = 64 / V;
+template <int NK, int JC, bool V4, class Pre, class Done>
+__device__ __forceinline__ void rnn_rows_w(const float (&w)[JC][NK], const float* __restrict__ in, int ld, bool use_in, int H, int B, int j0, float* red,
+                                           Pre pre, Done done) {
+  constexpr int V = RnnCfg<NK, JC>::V, UBR = RnnCfg<NK, JC>::UBR;
   static_assert(UBR >= 1 && UBR * JC == V, "rows per pass times weight rows must be V");
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float* my = red + wave * (V * RED_LD);
   const int v = lane % V, grp = lane / V;
-  for (int b0 = wave * UBR; b0 < B; b0 += 4 * UBR) {
-    float h[UBR][NK];
+  const int fu = v / JC, fc = v % JC;                      // the output this lane finishes in every pass
+  float h[UBR][NK];
+  auto fetch = [&](int b0) {
 #pragma unroll
-    for (int u = 0; u < UBR; u++)
-#pragma unroll
-      for (int i = 0; i < NK; i++) { const int k = lane + 64 * i; h[u][i] = (b0 + u < B && k < H) ? in(b0 + u, k) : 0.f; }
+    for (int u = 0; u < UBR; u++) rnn_load_row<NK, V4>(in + (int64_t)(b0 + u < B ? b0 + u : 0) * ld, H, use_in && b0 + u < B, h[u]);
+  };
+  int b0 = wave * UBR;
+  if (b0 < B) fetch(b0);
+  for (; b0 < B; b0 += 4 * UBR) {
+    const bool fin = grp == 0 && b0 + fu < B && j0 + fc < H;
+    RnnPre f = {0.f, 0.f, 0.f};
+    if (fin) f = pre(b0 + fu, fc);
+    float t[UBR * JC];
 #pragma unroll
     for (int u = 0; u < UBR; u++)
 #pragma unroll
       for (int c = 0; c < JC; c++) {
-        float t = 0.f;
+        float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < NK; i++) t = fmaf(h[u][i], w[c][i], t);
-        my[(u * JC + c) * RED_LD + lane] = t;
+        for (int i = 0; i < NK; i++) acc = fmaf(h[u][i], w[c][i], acc);
+        t[u * JC + c] = acc;
       }
+    if (b0 + 4 * UBR < B) fetch(b0 + 4 * UBR);            // next group's loads overlap the reduction below
+#pragma unroll
+    for (int i = 0; i < UBR * JC; i++) my[i * RED_LD + lane] = t[i];
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -68,15 +96,15 @@ __device__ __forceinline__ void rnn_rows_w(const float (&w)[JC][NK], int H, int 
     for (int m = V; m < 64; m <<= 1) tot += __shfl_xor(tot, m, 64);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();                       // the area is free for the next pass
-    const int u = v / JC, c = v % JC;
-    if (grp == 0 && b0 + u < B && j0 + c < H) done(b0 + u, c, tot);
+    if (fin) done(b0 + fu, fc, tot, f);
   }
 }
-template <int NK, int JC, class In, class Done>
-__device__ __forceinline__ void rnn_rows(const float* __restrict__ W, int H, int B, int j0, bool use_w, float* red, In in, Done done) {
+template <int NK, int JC, bool V4, class Pre, class Done>
+__device__ __forceinline__ void rnn_rows(const float* __restrict__ W, const float* __restrict__ in, int ld, bool use_in, int H, int B, int j0, float* red,
+                                         Pre pre, Done done) {
   float w[JC][NK];
-  rnn_load_w<NK, JC>(W, H, j0, use_w, w);
-  rnn_rows_w<NK, JC>(w, H, B, j0, red, in, done);
+  rnn_load_w<NK, JC, V4>(W, H, j0, use_in, w);
+  rnn_rows_w<NK, JC, V4>(w, in, ld, use_in, H, B, j0, red, pre, done);
 }
 
 // One time step of both directions.
@@ -88,14 +116,14 @@ struct StepArgs {
   const float* W[2];          // W_hh of the direction, [H, H] rows = output units
   const float* b1[2]; const float* b2[2];
 };
-template <int NK, int JC>
+template <int NK, int JC, bool V4>
 __global__ void __launch_bounds__(TPB) k_rnn_fwd_step(StepArgs a, int B, int H, int ld, int mode) {
   __shared__ float red[4 * RnnCfg<NK, JC>::V * RED_LD];
   const int d = blockIdx.y, j0 = blockIdx.x * JC;
   float* cur = a.cur[d]; const float* prev = a.prev[d]; const float* b1 = a.b1[d]; const float* b2 = a.b2[d];
-  rnn_rows<NK, JC>(a.W[d], H, B, j0, prev != nullptr, red,
-    [&](int b, int k) { return prev ? prev[(int64_t)b * ld + k] : 0.f; },
-    [&](int b, int c, float s) { const int j = j0 + c; float* p = cur + (int64_t)b * ld + j; *p = act_fwd(mode, *p + b1[j] + b2[j] + s); });
+  rnn_rows<NK, JC, V4>(a.W[d], prev, ld, prev != nullptr, H, B, j0, red,
+    [&](int b, int c) { const int j = j0 + c; RnnPre f = {cur[(int64_t)b * ld + j], b1[j], b2[j]}; return f; },
+    [&](int b, int c, float s, const RnnPre& f) { cur[(int64_t)b * ld + j0 + c] = act_fwd(mode, f.a + f.b + f.c + s); });
 }
 
 // One backward time step of both directions.  With g_t = dpre of time slice t (already complete):
@@ -108,29 +136,32 @@ struct BwdArgs {
   const float* dy[2]; const float* h[2]; float* next[2];          // slice of the next step, direction offset applied
   const float* Wt[2];
 };
-template <int NK, int JC>
+template <int NK, int JC, bool V4>
 __global__ void __launch_bounds__(TPB) k_rnn_bwd_step(BwdArgs a, int B, int H, int ld, int mode) {
   __shared__ float red[4 * RnnCfg<NK, JC>::V * RED_LD];
   const int d = blockIdx.y, i0 = blockIdx.x * JC;
   const float* cur = a.cur[d]; const float* dy = a.dy[d]; const float* hh = a.h[d]; float* next = a.next[d];
-  rnn_rows<NK, JC>(a.Wt[d], H, B, i0, cur != nullptr, red,
-    [&](int b, int j) { return cur ? cur[(int64_t)b * ld + j] : 0.f; },
-    [&](int b, int c, float s) {
-      const int64_t o = (int64_t)b * ld + i0 + c;
-      const float hv = hh[o], g = dy[o] + s;
-      next[o] = mode == 1 ? g * (1.0f - hv * hv) : (hv > 0.f ? g : 0.f); });
+  rnn_rows<NK, JC, V4>(a.Wt[d], cur, ld, cur != nullptr, H, B, i0, red,
+    [&](int b, int c) { const int64_t o = (int64_t)b * ld + i0 + c; RnnPre f = {hh[o], dy[o], 0.f}; return f; },
+    [&](int b, int c, float s, const RnnPre& f) {
+      const float g = f.b + s;
+      next[(int64_t)b * ld + i0 + c] = mode == 1 ? g * (1.0f - f.a * f.a) : (f.a > 0.f ? g : 0.f); });
 }
 
-// hidden sizes up to 64 * NK, JC weight rows per block (JC * NK <= 128 registers of weights)
+// hidden sizes up to 64 * NK, JC weight rows per block (JC * NK <= 128 registers of weights).  v4: every row the
+// kernel reads starts on a 16-byte boundary and H is a multiple of 4.
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 template <class A>
-static void launch_fwd_step(const A& a, int D, int B, int H, int ld, int mode) {
-#define GO(NK, JC) hipLaunchKernelGGL((k_rnn_fwd_step<NK, JC>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode)
+static void launch_fwd_step(const A& a, int D, int B, int H, int ld, int mode, bool v4) {
+#define GO(NK, JC) do { if (v4) hipLaunchKernelGGL((k_rnn_fwd_step<NK, JC, true>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode); \
+                        else hipLaunchKernelGGL((k_rnn_fwd_step<NK, JC, false>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode); } while (0)
   if (H <= 256) GO(4, 16); else if (H <= 512) GO(8, 16); else if (H <= 1024) GO(16, 8); else GO(32, 4);
 #undef GO
 }
 template <class A>
-static void launch_bwd_step(const A& a, int D, int B, int H, int ld, int mode) {
-#define GO(NK, JC) hipLaunchKernelGGL((k_rnn_bwd_step<NK, JC>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode)
+static void launch_bwd_step(const A& a, int D, int B, int H, int ld, int mode, bool v4) {
+#define GO(NK, JC) do { if (v4) hipLaunchKernelGGL((k_rnn_bwd_step<NK, JC, true>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode); \
+                        else hipLaunchKernelGGL((k_rnn_bwd_step<NK, JC, false>), dim3((unsigned)cdiv(H, JC), D), dim3(TPB), 0, g_stream, a, B, H, ld, mode); } while (0)
   if (H <= 256) GO(4, 16); else if (H <= 512) GO(8, 16); else if (H <= 1024) GO(16, 8); else GO(32, 4);
 #undef GO
 }
@@ -214,6 +245,98 @@ __global__ void __launch_bounds__(CTC_TPB) k_ctc(const float* __restrict__ probs
     dprobs[i] += (float)((double)probs[i] - acc / pfin);
   }
 }
+
+// Label strings of at most 63 symbols (2L+1 <= 127 states): one wavefront per recursion, lane l holding the blank state
+// 2l and the label state 2l+1, so a time step needs no block barrier: neighbours come through one lane shift and the
+// normaliser through a wavefront sum.  Wavefront 0 runs the forward recursion while wavefront 1 runs the backward one,
+// each with its own per-step normaliser (the posterior alpha*beta / sum_s alpha*beta does not depend on either scale).
+// Then both wavefronts turn rows of alpha*beta into class posteriors through a small LDS table.
+constexpr int CTC_ROW = 128;                      // doubles per (sample, time) row of alpha and of beta
+__device__ __forceinline__ double wave_sum_d(double v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__global__ void __launch_bounds__(128) k_ctc_wave(const float* __restrict__ probs, float* dprobs, const int* __restrict__ labels, const int* __restrict__ label_off,
+                                                  const int* __restrict__ label_len, const int* __restrict__ input_len, float* costs,
+                                                  double* alpha_all, double* beta_all, int T, int B, int A) {
+  extern __shared__ double hist_all[];             // [2][A]
+  __shared__ double s_pfin;
+  const int b = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int L = label_len[b], Tb = input_len[b];
+  const int* lab = labels + label_off[b];
+  const bool has_e = lane <= L, has_o = lane < L;
+  const int my = has_o ? lab[lane] : 0;
+  double2* arow = reinterpret_cast<double2*>(alpha_all + (size_t)b * T * CTC_ROW) + lane;      // row t: arow[t * 64]
+  double2* brow = reinterpret_cast<double2*>(beta_all + (size_t)b * T * CTC_ROW) + lane;
+  auto pe_at = [&](int t) { return (double)probs[((size_t)t * B + b) * A]; };
+  auto po_at = [&](int t) { return has_o ? (double)probs[((size_t)t * B + b) * A + my] : 0.0; };
+  if (wave == 0) {
+    const bool skip = has_o && lane >= 1 && lab[lane - 1] != my;        // label state may be entered from the previous label
+    double e = 0.0, o = 0.0, ll = 0.0;
+    double pe_n = pe_at(0), po_n = po_at(0);
+    for (int t = 0; t < Tb; t++) {
+      const double pe = pe_n, po = po_n;
+      if (t + 1 < Tb) { pe_n = pe_at(t + 1); po_n = po_at(t + 1); }
+      if (t == 0) { e = lane == 0 ? pe : 0.0; o = lane == 0 ? po : 0.0; }
+      else {
+        double up = __shfl_up(o, 1, 64);
+        if (lane == 0) up = 0.0;
+        const double ne = has_e ? (e + up) * pe : 0.0;
+        const double no = has_o ? (o + e + (skip ? up : 0.0)) * po : 0.0;
+        e = ne; o = no;
+      }
+      const double c = wave_sum_d(e + o);
+      if (c > 0.0) { const double r = 1.0 / c; e *= r; o *= r; }
+      ll += log(c);
+      arow[(size_t)t * 64] = make_double2(e, o);
+    }
+    const double pf = wave_sum_d((lane == L ? e : 0.0) + (lane == L - 1 ? o : 0.0));
+    if (lane == 0) { costs[b] = (float)(-(ll + log(pf))); s_pfin = pf; }
+  } else {
+    const bool skip = lane + 1 < L && lab[lane + 1] != my;               // label state may jump to the next label
+    double e = lane == L ? 1.0 : 0.0, o = lane == L - 1 ? 1.0 : 0.0;
+    brow[(size_t)(Tb - 1) * 64] = make_double2(e, o);
+    double pe_n = Tb >= 2 ? pe_at(Tb - 1) : 0.0, po_n = Tb >= 2 ? po_at(Tb - 1) : 0.0;
+    for (int t = Tb - 2; t >= 0; t--) {
+      const double pe = pe_n, po = po_n;                                   // emissions of time t + 1
+      if (t >= 1) { pe_n = pe_at(t); po_n = po_at(t); }
+      const double qe = e * pe, qo = o * po;
+      double dn_e = __shfl_down(qe, 1, 64), dn_o = __shfl_down(qo, 1, 64);
+      if (lane == 63) { dn_e = 0.0; dn_o = 0.0; }
+      const double ne = has_e ? qe + qo : 0.0;
+      const double no = has_o ? qo + dn_e + (skip ? dn_o : 0.0) : 0.0;
+      const double c = wave_sum_d(ne + no);
+      const double r = c > 0.0 ? 1.0 / c : 1.0;
+      e = ne * r; o = no * r;
+      brow[(size_t)t * 64] = make_double2(e, o);
+    }
+  }
+  __syncthreads();
+  if (dprobs == nullptr) return;
+  // d cost / d activation = probs - posterior(class), the gradient cuDNN reports; accumulated
+  double* hist = hist_all + (size_t)wave * A;
+  for (int t = wave; t < Tb; t += 2) {
+    const double2 al = arow[(size_t)t * 64], be = brow[(size_t)t * 64];
+    const double ge = al.x * be.x, go = al.y * be.y;
+    const double z = wave_sum_d(ge + go), blank = wave_sum_d(ge);
+    for (int k = lane; k < A; k += 64) hist[k] = 0.0;
+    wave_lds_sync();
+    if (has_o) atomicAdd(&hist[my], go);
+    wave_lds_sync();
+    for (int k = lane; k < A; k += 64) {
+      const size_t i = ((size_t)t * B + b) * A + k;
+      const double post = (k == 0 ? blank : hist[k]) / z;
+      dprobs[i] += (float)((double)probs[i] - post);
+    }
+    wave_lds_sync();
+  }
+}
 }  // namespace
 
 extern "C" {
@@ -239,7 +362,7 @@ void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B
       a.prev[d] = step == 0 ? nullptr : y + (size_t)tp * B * ld + dd * H;
       a.W[d] = Whh; a.b1[d] = Whh + (size_t)H * H; a.b2[d] = a.b1[d] + H;
     }
-    launch_fwd_step(a, D, B, H, ld, mode);
+    launch_fwd_step(a, D, B, H, ld, mode, (H & 3) == 0 && aligned16(y) && aligned16(w));
   }
   LH_CHECK_LAUNCH();
 }
@@ -276,7 +399,7 @@ void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
         a.dy[d] = dy + on; a.h[d] = y + on; a.next[d] = dpre + on;
         a.Wt[d] = wt + (size_t)dd * H * H;
       }
-      launch_bwd_step(a, D, B, H, ld, mode);
+      launch_bwd_step(a, D, B, H, ld, mode, (H & 3) == 0 && aligned16(dpre) && aligned16(wt) && aligned16(dy) && aligned16(y));
     }
   }
   lh_sum_dim(dpre, colsum, 1, T * B, ld);
@@ -314,17 +437,20 @@ void lh_ctc_loss(const float* probs, float* dprobs, const int* h_labels, const i
   }
   for (int i = 0; i < total; i++) if (h_labels[i] < 1 || h_labels[i] >= A) { free(host); LH_FAIL("lh_ctc_loss: label %d outside 1..%d (0 is the blank)", h_labels[i], A - 1); return; }
   const int Smax = 2 * Lmax + 1;
+  const bool one_wave = Lmax <= 63 && A <= 2048;       // 2L+1 states fit a wavefront's lane pairs; the class table fits LDS
   const size_t n_int = (size_t)3 * B + (size_t)(total > 0 ? total : 1);
   const size_t int_bytes = ((n_int * sizeof(int)) + 255) & ~(size_t)255;
-  const size_t dbl = ((size_t)2 * B * T * Smax + (size_t)B * T) * sizeof(double);
+  const size_t row = one_wave ? (size_t)CTC_ROW : (size_t)Smax;
+  const size_t dbl = ((size_t)2 * B * T * row + (size_t)B * T) * sizeof(double);
   char* scratch = (char*)lh_malloc_uninit(int_bytes + dbl);
   if (scratch == nullptr) { free(host); return; }
   int* d_int = (int*)scratch;
   lh_h2d(d_int, host, sizeof(int) * (size_t)(3 * B));
   if (total > 0) lh_h2d(d_int + 3 * B, h_labels, sizeof(int) * (size_t)total);
   free(host);
-  double* alpha = (double*)(scratch + int_bytes); double* beta = alpha + (size_t)B * T * Smax; double* cn = beta + (size_t)B * T * Smax;
-  hipLaunchKernelGGL(k_ctc, dim3(B), dim3(CTC_TPB), 0, g_stream, probs, dprobs, d_int + 3 * B, d_int, d_int + B, d_int + 2 * B, costs, alpha, beta, cn, T, B, A, Smax);
+  double* alpha = (double*)(scratch + int_bytes); double* beta = alpha + (size_t)B * T * row; double* cn = beta + (size_t)B * T * row;
+  if (one_wave) hipLaunchKernelGGL(k_ctc_wave, dim3(B), dim3(128), 2 * (size_t)A * sizeof(double), g_stream, probs, dprobs, d_int + 3 * B, d_int, d_int + B, d_int + 2 * B, costs, alpha, beta, T, B, A);
+  else hipLaunchKernelGGL(k_ctc, dim3(B), dim3(CTC_TPB), 0, g_stream, probs, dprobs, d_int + 3 * B, d_int, d_int + B, d_int + 2 * B, costs, alpha, beta, cn, T, B, A, Smax);
   lh_free_top(int_bytes + dbl);
   LH_CHECK_LAUNCH();
 }

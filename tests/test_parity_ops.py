@@ -470,6 +470,27 @@ def test_add_relu_and_its_gradient(pair):
     check_all(pair.run(f), rtol=1e-6)
 
 
+@pytest.mark.parametrize("beta", [0.0, 1.0, 0.5])
+@pytest.mark.parametrize("tt", [(1, 0), (0, 1), (0, 0), (1, 1)], ids=lambda t: "ta%d_tb%d" % t)
+def test_sgemm_few_tiles_long_reduction_with_row_stride(on_hip, tt, beta):
+    """Weight-gradient shape: a small output over thousands of rows (the reduction is split over blocks and combined
+    with atomic adds onto beta*C); C has a row stride larger than n and the padding must stay untouched."""
+    be = on_hip
+    ta, tb = tt
+    m, n, k, ldc = 200, 136, 3000, 144
+    rng = np.random.RandomState(41)
+    A = rng.randn(*((k, m) if ta else (m, k))).astype(np.float32); Bm = rng.randn(*((n, k) if tb else (k, n))).astype(np.float32)
+    C0 = rng.randn(m, ldc).astype(np.float32)
+    a, b, c = be.fromHost(A), be.fromHost(Bm), be.fromHost(C0)
+    be.lib.lh_sgemm(ta, tb, m, n, k, 0.75, a.ptr, A.shape[1], b.ptr, Bm.shape[1], beta, c.ptr, ldc)
+    from lantern_amd import _lib
+    _lib.check()
+    got = be.toHost(c, m * ldc).reshape(m, ldc)
+    want = 0.75 * ((A.T if ta else A).astype(np.float64) @ (Bm.T if tb else Bm).astype(np.float64)) + beta * C0[:, :n]
+    assert_close(got[:, :n], want.astype(np.float32), rtol=1e-4, what="sgemm split")
+    np.testing.assert_array_equal(got[:, n:], C0[:, n:])
+
+
 # ---- arena and error path (the library's own behaviour; no oracle counterpart) -----------------------
 def test_arena_zeroing_alignment_rewind_and_overflow(on_hip):
     be = on_hip
@@ -533,7 +554,7 @@ def test_shape_errors_are_reported_not_launched(on_hip):
 
 
 # ---- recurrent layer and CTC (DeepSpeech2 path) ------------------------------------------------------
-@pytest.mark.parametrize("case", [(1, True, 12, 32, 672, 800), (1, True, 6, 8, 96, 1024), (0, False, 5, 3, 7, 37), (1, False, 1, 2, 5, 16), (0, True, 9, 4, 33, 130)],
+@pytest.mark.parametrize("case", [(1, True, 12, 32, 672, 800), (1, True, 6, 8, 96, 1024), (0, False, 5, 3, 7, 37), (1, False, 1, 2, 5, 16), (0, True, 9, 4, 33, 130), (1, True, 4, 5, 20, 300), (0, True, 3, 6, 16, 1100), (1, False, 3, 33, 10, 1030), (1, True, 3, 70, 24, 64)],
                          ids=lambda c: "mode%d_bi%d_T%d_B%d_I%d_H%d" % c)
 def test_rnn_forward_and_backward(pair, case):
     mode, bidir, T, Bn, In, H = case
@@ -562,7 +583,7 @@ def test_rnn_forward_and_backward(pair, case):
     check_all(pair.run(f), rtol=3e-4)
 
 
-@pytest.mark.parametrize("case", ["ds2", "ragged", "tiny"])
+@pytest.mark.parametrize("case", ["ds2", "ragged", "tiny", "long_labels", "lane_limit"])
 def test_ctc_loss_and_gradient(pair, case):
     rng = np.random.RandomState(32)
     if case == "ds2":
@@ -571,6 +592,12 @@ def test_ctc_loss_and_gradient(pair, case):
     elif case == "ragged":
         T, Bn, A = 40, 7, 11
         lens = np.array([5, 1, 0, 12, 3, 19, 8], np.int32); ilen = np.array([40, 3, 1, 30, 40, 39, 17], np.int32)
+    elif case == "long_labels":          # more than 63 symbols: the block-per-sample kernel with states in a loop
+        T, Bn, A = 150, 3, 6
+        lens = np.array([70, 64, 10], np.int32); ilen = np.array([150, 149, 30], np.int32)
+    elif case == "lane_limit":           # 63 symbols = 127 states: the last lane pair of the one-wavefront kernel
+        T, Bn, A = 130, 2, 40
+        lens = np.array([63, 62], np.int32); ilen = np.array([130, 128], np.int32)
     else:
         T, Bn, A = 3, 1, 2
         lens = np.array([1], np.int32); ilen = np.array([3], np.int32)
