@@ -81,6 +81,20 @@ void  lh_event_destroy(void* ev);
 enum { LH_CAT_CONV_FWD = 0, LH_CAT_CONV_BWD_DATA, LH_CAT_CONV_BWD_FILTER, LH_CAT_GEMM, LH_CAT_BN_FWD, LH_CAT_BN_BWD,
        LH_CAT_ELEMENTWISE, LH_CAT_POOL, LH_CAT_REDUCE, LH_CAT_OPTIM, LH_CAT_FILL, LH_CAT_COUNT };
 void lh_prof_enable(unsigned mask);
+
+/* Command list for launch-bound programs (the sentiment TreeLSTM, SentimentTreeLSTM.scala:242-318, issues about
+ * 5000 operator calls on 150-element vectors per tree; the reference pays one cuBLAS / kernel launch for each,
+ * CUB:171-560).  Between lh_cmdlist_begin and lh_cmdlist_end every entry point of this header whose operands are
+ * small (element-wise up to 65536 elements, matrix-vector up to 131072 matrix elements: fill, copy, geam, scalar and
+ * same-shape broadcast arithmetic with gradients, unary ops with gradients, sgemv, ger, dot_vv, axpy_dev, softmax and
+ * nll with gradients over rows, adagrad, sgd, and the arena's zero fill) is recorded instead of launched; recorded
+ * commands run in order on one workgroup, and are handed to the device whenever any other entry point is called, when
+ * 256 are pending, and at lh_cmdlist_end / lh_sync / lh_d2h.  Results equal those of the stand-alone kernels up to
+ * summation order in the reductions.  Generated code calls lh_cmdlist_begin() once after lh_setup(). */
+void lh_cmdlist_begin(void);
+void lh_cmdlist_end(void);
+/* Commands recorded and interpreter launches since lh_setup (either pointer may be NULL). */
+void lh_cmdlist_stats(int64_t* recorded, int64_t* launches);
 void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat);
 
 /* ---- fill / elementwise ------------------------------------------------ */

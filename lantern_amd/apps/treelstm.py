@@ -125,8 +125,13 @@ class TreeNet(Module):
 
 class Trainer:
     def __init__(self, n_trees=8, vocab=2000, emb=300, hidden=150, classes=5, lr=0.05, seed=42, min_leaves=5, max_leaves=50, trees=None,
-                 reference_binding=True):
+                 reference_binding=True, batch_small_ops=True):
         be = get_backend()
+        # ~5000 operator calls on 150-element vectors per tree: let the backend run them from a command list
+        # instead of one launch each, where it can (BackendHIP.batchSmallOps; `close()` switches it off again)
+        self.batching = bool(batch_small_ops) and hasattr(be, "batchSmallOps")
+        if self.batching:
+            be.batchSmallOps(True)
         rng = np.random.RandomState(seed)
         Tensor.randseed(seed)
         self.model = TreeNet(emb, hidden, classes, reference_binding)
@@ -149,3 +154,8 @@ class Trainer:
 
     def end_step(self):
         get_backend().resetMallocAddr(self.mark)
+
+    def close(self):
+        if self.batching:
+            get_backend().batchSmallOps(False)
+            self.batching = False

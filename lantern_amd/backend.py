@@ -148,6 +148,15 @@ class BackendHIP(Backend):
     def sync(self):
         self.lib.lh_sync(); _lib.check()
 
+    def batchSmallOps(self, on=True):
+        """Record small operations into the library's command list instead of launching each (launch-bound programs)."""
+        (self.lib.lh_cmdlist_begin if on else self.lib.lh_cmdlist_end)(); _lib.check()
+
+    def cmdlistStats(self):
+        rec, launches = C.c_int64(0), C.c_int64(0)
+        self.lib.lh_cmdlist_stats(C.byref(rec), C.byref(launches))
+        return rec.value, launches.value
+
     def mallocArray(self, length, zero=True):
         n = max(int(length), 1)
         p = (self.lib.lh_malloc if zero else self.lib.lh_malloc_uninit)(4 * n)

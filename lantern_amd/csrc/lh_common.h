@@ -8,7 +8,14 @@
 
 namespace lh {
 
-extern hipStream_t g_stream;     // every kernel is enqueued here
+extern hipStream_t g_stream_raw;  // the library's stream
+// Small operations recorded by the command list (lh_cmdlist.hip) but not launched yet.  Anything that is about to use
+// the stream goes through `g_stream`, which launches the recorded commands first, so program order is kept.
+extern int g_rec_pending;
+void rec_flush();
+void cmdlist_release();           // frees the command buffers (lh_cleanup)
+static inline hipStream_t ordered_stream() { if (g_rec_pending) rec_flush(); return g_stream_raw; }
+#define g_stream (::lh::ordered_stream())     // every kernel is enqueued here
 extern int g_error_mode;         // 0 = print and exit, 1 = record and return
 extern int g_num_cu;             // compute units of the device in use
 
@@ -33,7 +40,7 @@ bool failed();
 // ---- per-category timing with HIP events on g_stream (off unless lh_prof_enable was called) ----
 enum {
   CAT_CONV_FWD = 0, CAT_CONV_BWD_DATA, CAT_CONV_BWD_FILTER, CAT_GEMM, CAT_BN_FWD, CAT_BN_BWD,
-  CAT_ELEMENTWISE, CAT_POOL, CAT_REDUCE, CAT_OPTIM, CAT_FILL, CAT_RNN, CAT_COUNT
+  CAT_ELEMENTWISE, CAT_POOL, CAT_REDUCE, CAT_OPTIM, CAT_FILL, CAT_RNN, CAT_CMDLIST, CAT_COUNT
 };
 extern unsigned g_prof_mask;
 void prof_begin(int cat);
@@ -60,6 +67,28 @@ void bn_finalize_conv_partials(const float* partial, int C, int ncols, int col1,
                                float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor);
 
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- command list: small operations recorded on the host and executed in order by one workgroup -------------
+// While recording is on (lh_cmdlist_begin), an entry point whose operands are small enough appends a command instead
+// of launching a kernel; a tree-structured model of 150-element vectors issues thousands of such operations per
+// step, and the host's launch rate is what bounds it.
+enum {
+  CL_ZERO16 = 0, CL_FILL, CL_COPY, CL_GEAM, CL_SCALAR, CL_BIN, CL_ACC, CL_ACCNEG, CL_ACCMUL, CL_UNARY, CL_UNARY_GRAD,
+  CL_GEMV_N, CL_GEMV_T, CL_GER, CL_DOT, CL_AXPY_DEV, CL_SOFTMAX, CL_SOFTMAX_GRAD, CL_NLL, CL_NLL_GRAD, CL_ADAGRAD, CL_SGD
+};
+struct LhCmd { int32_t op, i0, i1, i2; float f0, f1, f2, f3; void* p0; void* p1; void* p2; void* p3; };   // 64 bytes
+constexpr int64_t REC_MAX_ELEMS = 1 << 16;        // element-wise operands up to this many elements are recorded
+constexpr int64_t REC_MAX_MATRIX = 1 << 17;       // matrix-vector operands up to this many matrix elements
+extern int g_rec_on;
+LhCmd* rec_next();                                 // the slot of the next command (launches a full buffer first); nullptr on error
+static inline bool rec_ok(int64_t n, int64_t limit = REC_MAX_ELEMS) { return g_rec_on && n <= limit; }
+static inline LhCmd* rec_cmd(int op, int i0, int i1, int i2, float f0, float f1, float f2, float f3,
+                             const void* p0, const void* p1, const void* p2, const void* p3) {
+  LhCmd* c = rec_next();
+  if (c) { c->op = op; c->i0 = i0; c->i1 = i1; c->i2 = i2; c->f0 = f0; c->f1 = f1; c->f2 = f2; c->f3 = f3;
+           c->p0 = (void*)p0; c->p1 = (void*)p1; c->p2 = (void*)p2; c->p3 = (void*)p3; }
+  return c;
+}
 
 // Grid for a grid-stride streaming kernel: enough blocks to cover n at `per_block`
 // elements each, capped at a few waves of blocks per CU.

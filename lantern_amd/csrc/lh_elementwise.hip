@@ -85,6 +85,7 @@ struct Dims4 { int d[4]; int64_t sa[4]; int64_t sb[4]; };
 extern "C" {
 
 void lh_fill(float* x, float v, int64_t n) { ProfScope prof_(CAT_FILL);
+  if (n > 0 && rec_ok(n)) { rec_cmd(CL_FILL, (int)n, 0, 0, v, 0.f, 0.f, 0.f, x, nullptr, nullptr, nullptr); return; }
   if (n <= 0) return;
   if (al16(x)) hipLaunchKernelGGL(k_fill, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, v, n);
   else hipLaunchKernelGGL(k_fill_scalar, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, v, n);
@@ -119,6 +120,7 @@ void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t) {
 }
 
 void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) { ProfScope prof_(CAT_ELEMENTWISE);
+  if (n > 0 && op >= LH_RELU && op <= LH_HARDTANH && rec_ok(n)) { rec_cmd(CL_UNARY, (int)n, op, 0, lo, hi, 0.f, 0.f, y, x, nullptr, nullptr); return; }
   switch (op) {
     case LH_RELU: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return v < 0.f ? 0.f : v; }); break;
     case LH_TANH: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return tanhf(v); }); break;
@@ -134,6 +136,7 @@ void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) {
 }
 
 void lh_unary_grad(int op, const float* x, const float* y, const float* dy, float* dx, int64_t n, int inplace, float lo, float hi) { ProfScope prof_(CAT_ELEMENTWISE);
+  if (n > 0 && op >= LH_RELU && op <= LH_HARDTANH && rec_ok(n)) { rec_cmd(CL_UNARY_GRAD, (int)n, op, inplace ? 1 : 0, lo, hi, 0.f, 0.f, dx, x, y, dy); return; }
   // out = dx; inputs (a, b, c) chosen per op.  All forms are dx (+)= g(x|y, dy).
   switch (op) {
     case LH_RELU:
@@ -157,6 +160,7 @@ void lh_unary_grad(int op, const float* x, const float* y, const float* dy, floa
 
 void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_scalar_op: unknown op %d", op);
+  if (n > 0 && rec_ok(n)) { rec_cmd(CL_SCALAR, (int)n, op, 0, s, 0.f, 0.f, 0.f, y, x, nullptr, nullptr); return; }
   ew<1>(y, x, nullptr, nullptr, n, [op, s] __device__(float v, float, float) { return bop(op, v, s); });
   LH_CHECK_LAUNCH();
 }
@@ -190,6 +194,7 @@ void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, f
 }
 
 void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+  if (n > 0 && rec_ok(n)) { rec_cmd(CL_GEAM, (int)n, 0, 0, alpha, beta, 0.f, 0.f, out, x, y, nullptr); return; }
   ew<2>(out, x, y, nullptr, n, [alpha, beta] __device__(float a, float b, float) { return a * alpha + b * beta; });
   LH_CHECK_LAUNCH();
 }
@@ -318,6 +323,7 @@ void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const
   int64_t n = prod(odims, rank);
   if (n <= 0) return;
   if (same_dims(adims, odims, rank) && same_dims(bdims, odims, rank)) {
+    if (rec_ok(n)) { rec_cmd(CL_BIN, (int)n, op, 0, 0.f, 0.f, 0.f, 0.f, out, a, b, nullptr); return; }
     ew<2>(out, a, b, nullptr, n, [op] __device__(float x, float y, float) { return bop(op, x, y); });
   } else {
     Dims4 D;
@@ -338,6 +344,11 @@ void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a
   int pad = 4 - rank; int a4[4] = {1, 1, 1, 1}, b4[4] = {1, 1, 1, 1};
   for (int i = 0; i < rank; i++) { a4[pad + i] = adims[i]; b4[pad + i] = bdims[i]; }
   bool a_full = same_dims(adims, odims, rank), b_full = same_dims(bdims, odims, rank);
+  if (a_full && b_full && op != LH_DIV && rec_ok(n)) {       // same shapes: d += g, d += -g or d += g * other
+    if (!a_is_input) rec_cmd(op == LH_MUL ? CL_ACCMUL : CL_ACC, (int)n, 0, 0, 0.f, 0.f, 0.f, 0.f, ad, outd, b, nullptr);
+    if (!b_is_input) rec_cmd(op == LH_MUL ? CL_ACCMUL : (op == LH_SUB ? CL_ACCNEG : CL_ACC), (int)n, 0, 0, 0.f, 0.f, 0.f, 0.f, bd, outd, a, nullptr);
+    return;
+  }
   if (!a_is_input) {
     if (a_full) {
       if (b_full && op == LH_ADD) ew<2>(ad, ad, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
@@ -372,6 +383,7 @@ void lh_bcast_update(int op, float* a, const int* adims, const float* b, const i
   if (n <= 0) return;
   if (same_dims(adims, od, rank)) {  // a has the full shape: a = a op broadcast(b)
     if (same_dims(bdims, od, rank)) {
+      if (rec_ok(n)) { rec_cmd(CL_BIN, (int)n, op, 0, 0.f, 0.f, 0.f, 0.f, a, a, b, nullptr); return; }
       ew<2>(a, a, b, nullptr, n, [op] __device__(float x, float y, float) { return bop(op, x, y); });
     } else {
       Dims4 D;
@@ -626,6 +638,7 @@ extern "C" {
 void lh_sgd(float* x, float* d, float lr, int64_t n) { ProfScope prof_(CAT_OPTIM);
   if (n <= 0) return;
   LH_REQUIRE(al16(x) && al16(d), "lh_sgd: pointers must be 16-byte aligned");
+  if (rec_ok(n)) { rec_cmd(CL_SGD, (int)n, 0, 0, lr, 0.f, 0.f, 0.f, x, d, nullptr, nullptr); return; }
   hipLaunchKernelGGL(k_sgd, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, lr, n);
   LH_CHECK_LAUNCH();
 }
@@ -637,6 +650,7 @@ void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, i
 }
 void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) { ProfScope prof_(CAT_OPTIM);
   if (n <= 0) return;
+  if (rec_ok(n)) { rec_cmd(CL_ADAGRAD, (int)n, 0, 0, lr, clip, 0.f, 0.f, x, d, m, nullptr); return; }
   hipLaunchKernelGGL(k_adagrad, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, d, m, lr, clip, n);
   LH_CHECK_LAUNCH();
 }

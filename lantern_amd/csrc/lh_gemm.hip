@@ -187,6 +187,7 @@ extern "C" {
 void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, const float* x, float beta, float* y) {
   ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
+  if (rec_ok((int64_t)m * n, REC_MAX_MATRIX)) { rec_cmd(trans ? CL_GEMV_T : CL_GEMV_N, m, n, lda, alpha, beta, 0.f, 0.f, y, A, x, nullptr); return; }
   if (!trans) hipLaunchKernelGGL(k_sgemv_n, dim3(stream_grid((int64_t)m * 64, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
   else hipLaunchKernelGGL(k_sgemv_t, dim3((unsigned)cdiv(n, 32)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
   LH_CHECK_LAUNCH();
@@ -194,15 +195,18 @@ void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, con
 void lh_ger(int m, int n, const float* u, const float* v, float* A) {
   ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
+  if (rec_ok((int64_t)m * n, REC_MAX_MATRIX)) { rec_cmd(CL_GER, m, n, 0, 0.f, 0.f, 0.f, 0.f, A, u, v, nullptr); return; }
   hipLaunchKernelGGL(k_ger, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, m, n, u, v, A);
   LH_CHECK_LAUNCH();
 }
 void lh_dot_vv(const float* x, const float* y, float* out, int n) {
+  if (rec_ok(n)) { rec_cmd(CL_DOT, n, 0, 0, 0.f, 0.f, 0.f, 0.f, out, x, y, nullptr); return; }
   hipLaunchKernelGGL(k_dot, dim3(1), dim3(TPB), 0, g_stream, x, y, out, n);
   LH_CHECK_LAUNCH();
 }
 void lh_axpy_dev(float* y, const float* s, const float* x, int64_t n) {
   if (n <= 0) return;
+  if (rec_ok(n)) { rec_cmd(CL_AXPY_DEV, (int)n, 0, 0, 0.f, 0.f, 0.f, 0.f, y, s, x, nullptr); return; }
   hipLaunchKernelGGL(k_axpy_dev, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, y, s, x, n);
   LH_CHECK_LAUNCH();
 }

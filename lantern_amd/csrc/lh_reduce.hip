@@ -209,6 +209,7 @@ void lh_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner) 
 
 void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner) { ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * c * inner <= 0) return;
+  if (inner == 1 && rec_ok((int64_t)outer * c)) { rec_cmd(CL_SOFTMAX, outer, c, is_log ? 1 : 0, 0.f, 0.f, 0.f, 0.f, y, x, nullptr, nullptr); return; }
   if (inner == 1) {
     if (c <= 1024 || outer >= 4 * g_num_cu) {
       int grid = stream_grid((int64_t)outer * 64, TPB);
@@ -228,6 +229,7 @@ void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inne
 void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int outer, int c, int inner) { ProfScope prof_(CAT_REDUCE);
   int64_t groups = (int64_t)outer * inner;
   if (groups * c <= 0) return;
+  if (inner == 1 && rec_ok(groups * c)) { rec_cmd(CL_SOFTMAX_GRAD, outer, c, is_log ? 1 : 0, 0.f, 0.f, 0.f, 0.f, dx, y, dy, nullptr); return; }
   int grid = stream_grid(groups * 64, TPB);
   if (is_log) hipLaunchKernelGGL((k_softmax_grad_wave<true>), dim3(grid), dim3(TPB), 0, g_stream, y, dy, dx, groups, c, inner);
   else hipLaunchKernelGGL((k_softmax_grad_wave<false>), dim3(grid), dim3(TPB), 0, g_stream, y, dy, dx, groups, c, inner);
@@ -235,11 +237,13 @@ void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int
 }
 void lh_nll(const float* x, const int* target, float* y, int batch, int stride) { ProfScope prof_(CAT_REDUCE);
   if (batch <= 0) return;
+  if (rec_ok(batch)) { rec_cmd(CL_NLL, batch, stride, 0, 0.f, 0.f, 0.f, 0.f, y, x, target, nullptr); return; }
   hipLaunchKernelGGL(k_nll, dim3(cdiv(batch, 64)), dim3(64), 0, g_stream, x, target, y, batch, stride);
   LH_CHECK_LAUNCH();
 }
 void lh_nll_grad(float* dx, const int* target, const float* dy, int batch, int stride) { ProfScope prof_(CAT_REDUCE);
   if (batch <= 0) return;
+  if (rec_ok(batch)) { rec_cmd(CL_NLL_GRAD, batch, stride, 0, 0.f, 0.f, 0.f, 0.f, dx, dy, target, nullptr); return; }
   hipLaunchKernelGGL(k_nll_grad, dim3(cdiv(batch, 64)), dim3(64), 0, g_stream, dx, target, dy, batch, stride);
   LH_CHECK_LAUNCH();
 }

@@ -7,7 +7,7 @@
 #include <vector>
 
 namespace lh {
-hipStream_t g_stream = nullptr;
+hipStream_t g_stream_raw = nullptr;
 int g_error_mode = 0;
 int g_num_cu = 256;
 static char g_err[1024] = "";
@@ -62,6 +62,7 @@ __global__ void k_zero16(uint4* p, size_t n16) {
 static void zero_async(void* p, size_t bytes) {  // bytes is a multiple of 256
   size_t n16 = bytes / 16;
   if (n16 == 0) return;
+  if (rec_ok((int64_t)n16)) { rec_cmd(CL_ZERO16, (int)n16, 0, 0, 0.f, 0.f, 0.f, 0.f, p, nullptr, nullptr, nullptr); return; }
   int grid = stream_grid((int64_t)n16, 256 * 4);
   hipLaunchKernelGGL(k_zero16, dim3(grid), dim3(256), 0, g_stream, (uint4*)p, n16);
 }
@@ -82,17 +83,18 @@ void lh_setup(size_t heap_bytes) {
   hipDeviceProp_t prop;
   LH_HIP(hipGetDeviceProperties(&prop, dev));
   g_num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-  LH_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+  LH_HIP(hipStreamCreateWithFlags(&g_stream_raw, hipStreamNonBlocking));
   heap_bytes = (heap_bytes + 255) & ~(size_t)255;
   LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
   g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0; g_zero_end = 0;
 }
 
 void lh_cleanup(void) {
-  if (g_stream) (void)hipStreamSynchronize(g_stream);
+  if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
+  cmdlist_release();
   if (g_heap) (void)hipFree(g_heap);
-  if (g_stream) (void)hipStreamDestroy(g_stream);
-  g_heap = nullptr; g_stream = nullptr; g_heap_bytes = g_top = g_zero_end = 0;
+  if (g_stream_raw) (void)hipStreamDestroy(g_stream_raw);
+  g_heap = nullptr; g_stream_raw = nullptr; g_heap_bytes = g_top = g_zero_end = 0;
 }
 
 void lh_sync(void) {
@@ -149,13 +151,14 @@ void lh_d2h(void* h_dst, const void* src, size_t bytes) {
   LH_HIP(hipStreamSynchronize(g_stream));
 }
 void lh_d2d(void* dst, const void* src, size_t bytes) {
+  if ((bytes & 3) == 0 && bytes > 0 && rec_ok((int64_t)(bytes / 4))) { rec_cmd(CL_COPY, (int)(bytes / 4), 0, 0, 0.f, 0.f, 0.f, 0.f, dst, src, nullptr, nullptr); return; }
   LH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
 }
 
 void lh_prof_enable(unsigned mask) { g_prof_mask = mask; }
 void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat) {
   for (int c = 0; c < ncat; c++) { h_ms[c] = 0.0; h_calls[c] = 0; }
-  if (g_stream) (void)hipStreamSynchronize(g_stream);
+  if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
   for (auto& r : g_prof_recs) {
     float ms = 0.f;
     if (r.a && r.b && hipEventElapsedTime(&ms, r.a, r.b) == hipSuccess && r.cat < ncat) { h_ms[r.cat] += ms; h_calls[r.cat] += 1; }

@@ -47,6 +47,7 @@ def on_hip(hip_backend):
     la.set_backend(hip_backend)
     mark = hip_backend.getMallocAddr()
     yield hip_backend
+    hip_backend.batchSmallOps(False)
     hip_backend.sync()
     hip_backend.resetMallocAddr(mark)
 

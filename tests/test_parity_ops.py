@@ -692,3 +692,90 @@ def test_conv_with_batchnorm_statistics(pair, case, relu):
             o[1][edge & (np.abs(o[1]) < 4e-5)] = 0.0
     check_all(outs, rtol=2e-4)
 
+
+
+# ---- command list: small operators recorded and run in order by one workgroup --------------------------
+def _small_op_program(be, rng_seed=50):
+    """A chain of dependent small operators covering every recordable entry point; returns host copies of all results."""
+    rng = np.random.RandomState(rng_seed)
+    n, m = 150, 37
+    up = lambda a: be.fromHost(np.ascontiguousarray(a, np.float32))
+    W = up(rng.randn(m, n) * 0.1); x = up(rng.randn(n)); bias = up(rng.randn(m)); gy = up(rng.randn(m))
+    lib = be.lib
+    outs = []
+    h = be.matrixVectorDot(W, x, m, n)                                        # gemv
+    lib.lh_bcast_update(B.ADD, h.ptr, B._ints((m,)), bias.ptr, B._ints((m,)), 1)   # += bias
+    s = be.unary(B.SIGMOID, h, m); t = be.unary(B.TANH, h, m)
+    prod = be.bcast_op(B.MUL, s, (m,), t, (m,), (m,))
+    diff = be.bcast_op(B.SUB, prod, (m,), bias, (m,), (m,))
+    sc = be.scalar_op(B.MUL, diff, 0.5, m)
+    ge = be.mallocArray(m, zero=False); be.geam(sc, 2.0, t, -1.0, ge, m)
+    dotv = be.vectorVectorDot(ge, gy, m)
+    outs += [(h, m), (s, m), (prod, m), (diff, m), (sc, m), (ge, m), (dotv, 1)]
+    # gradients back through the chain
+    dprod = be.mallocArray(m); dbias = be.mallocArray(m); ds = be.mallocArray(m); dt = be.mallocArray(m); dh = be.mallocArray(m)
+    be.bcast_op_grad(B.SUB, prod, dprod, (m,), False, bias, dbias, (m,), False, gy, (m,))
+    be.bcast_op_grad(B.MUL, s, ds, (m,), False, t, dt, (m,), False, dprod, (m,))
+    be.unary_grad(B.SIGMOID, h, s, ds, dh, m); be.unary_grad(B.TANH, h, t, dt, dh, m)
+    dW = be.mallocArray(m * n); dx = be.mallocArray(n)
+    be.add_cartesian(dW, x, dh, m, n); be.add_composition(dx, W, dh, m, n)
+    be.addMul_scalar(dx, dotv, x, n)                                           # dx += dotv[0] * x
+    outs += [(dprod, m), (dbias, m), (ds, m), (dt, m), (dh, m), (dW, m * n), (dx, n)]
+    # classifier head: rows of 5 classes
+    logits = be.mallocArray(3 * 5, zero=False); be.copyFloatArray(logits, h, 15)
+    lsm = be.softmax(1, logits, 3, 5, 1); sm = be.softmax(0, logits, 3, 5, 1)
+    tgt = be.fromHost(np.array([4, 0, 2], np.int32))
+    loss = be.nllLoss(lsm, tgt, 3, 5)
+    dl = be.mallocArray(15); dlog = be.mallocArray(15)
+    be.nllLoss_grad(dl, tgt, up(np.ones(3)), 3, 5)
+    be.softmax_grad(1, lsm, dl, dlog, 3, 5, 1); be.softmax_grad(0, sm, dl, dlog, 3, 5, 1)
+    outs += [(lsm, 15), (sm, 15), (loss, 3), (dl, 15), (dlog, 15)]
+    # optimizers consume and clear the gradient
+    cache = be.mallocArray(m * n)
+    lib.lh_adagrad(W.ptr, dW.ptr, cache.ptr, 0.05, 1.0, m * n)
+    lib.lh_sgd(x.ptr, dx.ptr, 0.1, n)
+    outs += [(W, m * n), (cache, m * n), (x, n), (dW, m * n)]
+    return [be.toHost(buf, cnt).copy() for buf, cnt in outs]
+
+
+def test_command_list_matches_one_launch_per_operator(on_hip):
+    be = on_hip
+    direct = _small_op_program(be)
+    rec0, launches0 = be.cmdlistStats()
+    be.batchSmallOps(True)
+    try:
+        listed = _small_op_program(be)
+    finally:
+        be.batchSmallOps(False)
+    rec, launches = be.cmdlistStats()
+    assert rec - rec0 >= 25 and 0 < launches - launches0 <= 30, (rec - rec0, launches - launches0)
+    for i, (a, b_) in enumerate(zip(listed, direct)):
+        assert_close(a, b_, rtol=2e-6, what="result %d" % i)
+
+
+def test_command_list_keeps_program_order_around_other_kernels_and_wraps_its_buffers(on_hip):
+    """Recorded commands, kernels too large to record and copies interleave in program order; more commands than the
+    pinned buffers hold in total go through without loss."""
+    be = on_hip
+    lib = be.lib
+    big_n = 1 << 20                                                             # above the recording limit: a normal launch
+    big = be.mallocArray(big_n, zero=False); small = be.mallocArray(64); one = be.fromHost(np.ones(64, np.float32))
+    be.batchSmallOps(True)
+    try:
+        lib.lh_fill(small.ptr, 3.0, 64)                                         # recorded
+        lib.lh_fill(big.ptr, 2.0, big_n)                                        # launched: the recorded fill must land first
+        lib.lh_geam(small.ptr, 1.0, big.ptr, 1.0, small.ptr, 64)                # recorded: reads what the big fill wrote -> 5
+        lib.lh_scalar_op(B.MUL, big.ptr, big.ptr, 0.5, big_n)                   # launched after the recorded read
+        lib.lh_geam(small.ptr, 1.0, big.ptr, 1.0, small.ptr, 64)                # 5 + 1 = 6
+        assert (be.toHost(small, 64) == 6.0).all()
+        z = be.mallocArray(300)                                                 # the arena's zero fill is recorded too
+        lib.lh_bcast_update(B.ADD, z.ptr, B._ints((64,)), small.ptr, B._ints((64,)), 1)
+        assert (be.toHost(z, 300)[:64] == 6.0).all() and not be.toHost(z, 300)[64:].any()
+        cnt = be.mallocArray(64)
+        for _ in range(10000):                                                  # 10000 dependent commands: five buffers' worth
+            lib.lh_bcast_update(B.ADD, cnt.ptr, B._ints((64,)), one.ptr, B._ints((64,)), 1)
+        assert (be.toHost(cnt, 64) == 10000.0).all()
+    finally:
+        be.batchSmallOps(False)
+    from lantern_amd import _lib
+    _lib.check()

@@ -20,6 +20,8 @@ def _run(make_trainer, backend, steps):
         losses.append(float(tr.step().toCPU()[0]))
         tr.end_step()
     params = [(n, p.x.toCPU().copy()) for n, p in tr.model.namedParameters()]
+    if hasattr(tr, "close"):
+        tr.close()
     if hasattr(backend, "sync"):
         backend.sync()
     backend.resetMallocAddr(mark)
@@ -96,10 +98,15 @@ def test_squeezenet_avgpool_head_5_steps(hip_backend, cpu_backend):
     _compare(lambda: Trainer(batch=8, lr=0.001, avgpool_head=True), hip_backend, cpu_backend, steps=5, per_tensor=5e-3)
 
 
-def test_treelstm_10_trees(hip_backend, cpu_backend):
-    """One Adagrad step per tree over 10 random trees of 5..30 leaves: gemv / rank-1 update / gemv-transposed path."""
+@pytest.mark.parametrize("batching", [False, True], ids=["one_launch_per_op", "command_list"])
+def test_treelstm_10_trees(hip_backend, cpu_backend, batching):
+    """One Adagrad step per tree over 10 random trees of 5..30 leaves: gemv / rank-1 update / gemv-transposed path,
+    with one kernel launch per operator and with the small operators run from the library's command list."""
     from lantern_amd.apps.treelstm import Trainer
-    _compare(lambda: Trainer(n_trees=10, vocab=500, max_leaves=30), hip_backend, cpu_backend, steps=10)
+    rec0 = hip_backend.cmdlistStats()[0]
+    _compare(lambda: Trainer(n_trees=10, vocab=500, max_leaves=30, batch_small_ops=batching), hip_backend, cpu_backend, steps=10)
+    rec = hip_backend.cmdlistStats()[0] - rec0
+    assert (rec > 10000) if batching else (rec == 0), "commands recorded: %d" % rec
 
 
 def test_deepspeech2_5_steps(hip_backend, cpu_backend):
