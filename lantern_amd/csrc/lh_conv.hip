@@ -8,9 +8,18 @@
 //
 // Algorithmic work of each: 2*N*K*C*R*S*P*Q flop.
 #include "lh_igemm.h"
+#include <map>
+#include <tuple>
 using namespace lh;
 
 namespace {
+// Slices of the filter-gradient reduction that measured fastest, per convolution shape (filled on first use).
+struct BwdfKey {
+  int v[11];
+  bool operator<(const BwdfKey& o) const { for (int i = 0; i < 11; i++) if (v[i] != o.v[i]) return v[i] < o.v[i]; return false; }
+};
+static std::map<BwdfKey, int> g_bwdf_split;
+static const bool g_bwdf_tune = getenv("LH_NO_TUNE") == nullptr;
 constexpr int TPB = 256;
 
 struct ConvDims { int N, C, H, W, K, R, S, sH, sW, pH, pW, P, Q; };
@@ -146,7 +155,10 @@ struct LoadConvBwdDataTapB {
 };
 
 // ---- A operand of the filter gradient: dy rows, reduction index (n, p, q) ------------------------------
-template <bool VEC>                      // VEC: PQ % 4 == 0 and dy 16-byte aligned
+// VEC: PQ % 4 == 0 and dy 16-byte aligned (one 16-byte load per group of four reduction indices).
+// CARRY (PQ >= 4): the group's first index is decoded once and the other three follow by stepping with at most one carry
+// into the next sample, instead of one division each.
+template <bool VEC, bool CARRY = false>
 struct LoadConvBwdFilterA {
   static constexpr bool ALONG_K = true;
   static constexpr bool VEC4 = VEC;
@@ -158,20 +170,29 @@ struct LoadConvBwdFilterA {
   __device__ __forceinline__ void init(State& s, int i, int nrows) const { s.valid = i < nrows; s.rowoff = (s.valid ? i : 0) * PQ; }
   __device__ __forceinline__ uint32_t off1(const State& s, int kk, int kend, int e) const {
     // VEC: the reduction length N*PQ is a multiple of 4 too, so the group at e == 0 is all in or all out
-    uint32_t n, pq; dPQ.divmod(kk + e, n, pq);
+    uint32_t n, pq;
+    if (CARRY && !VEC) {
+      dPQ.divmod(kk, n, pq);
+      pq += (uint32_t)e;
+      if (pq >= (uint32_t)PQ) { pq -= (uint32_t)PQ; n += 1; }
+    } else {
+      dPQ.divmod(kk + e, n, pq);
+    }
     return (s.valid && kk + e < kend) ? (uint32_t)((int)n * K * PQ + s.rowoff + (int)pq) * 4u : LH_OOB;
   }
 };
 
 // ---- B operand of the filter gradient: gather of x, reduction index (n, p, q) ------------------------------
-// column j = (c, r, s) fixed per thread.
-template <bool ROWVEC>                   // ROWVEC: Q % 4 == 0, the four reduction indices share (n, p)
+// column j = (c, r, s) fixed per thread.  MODE 1: Q % 4 == 0, the four reduction indices of a group share (n, p).
+// MODE 2 (Q >= 4): the group's first index is decoded once, the others step along the row with at most one carry
+// into the next row / sample.  MODE 0: one decode per index (maps narrower than 4).
+template <int MODE>
 struct LoadConvBwdFilterB {
   static constexpr bool ALONG_K = true;
   static constexpr bool VEC4 = false;
   static constexpr bool SPLIT = false;
   const float* base; uint32_t nbytes;
-  int C, H, W, sH, sW, pH, pW, CHW;
+  int C, H, W, sH, sW, pH, pW, CHW, P, Q;
   FastDiv dPQ, dQ, dRS, dS;
   struct State { int coff, dh, dw; bool valid; };
   __device__ __forceinline__ void init(State& s, int j, int ncols) const {
@@ -181,10 +202,14 @@ struct LoadConvBwdFilterB {
     s.coff = (int)c * H * W; s.dh = (int)r - pH; s.dw = (int)ss - pW;
   }
   __device__ __forceinline__ uint32_t off1(const State& s, int kk, int kend, int e) const {
-    // ROWVEC: the group's four indices share (n, p); decode its first and step along the row
     uint32_t n, pq, p, q;
-    dPQ.divmod(ROWVEC ? kk : kk + e, n, pq); dQ.divmod(pq, p, q);
-    const int h = (int)p * sH + s.dh, w = ((int)q + (ROWVEC ? e : 0)) * sW + s.dw;
+    dPQ.divmod(MODE == 0 ? kk + e : kk, n, pq); dQ.divmod(pq, p, q);
+    if (MODE != 0) q += (uint32_t)e;
+    if (MODE == 2 && q >= (uint32_t)Q) {
+      q -= (uint32_t)Q; p += 1;
+      if (p >= (uint32_t)P) { p = 0; n += 1; }
+    }
+    const int h = (int)p * sH + s.dh, w = (int)q * sW + s.dw;
     const bool ok = s.valid && kk + e < kend && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
     return ok ? (uint32_t)((int)n * CHW + s.coff + h * W + w) * 4u : LH_OOB;
   }
@@ -275,6 +300,14 @@ constexpr int BWDF_BK = LH_BWDF_BK;      // k-slab of the filter-gradient kernel
 // time, so a last round with only a few tiles leaves most CUs idle for a whole tile time.  When the
 // tile count is a little above a whole number of rounds, the columns of the surplus tiles are
 // computed by a second launch with smaller tiles, which spreads them over four times as many CUs.
+// Tile choice of the forward / input-gradient launches.  With a reduction of at most 512 (1x1 filters over up to 512
+// channels) a tile is finished after at most 32 slabs, and the fixed cost per tile (pipeline fill, epilogue) and the
+// low occupancy of the 128-wide tiles weigh more than their better operand reuse: measured over the ResNet-50 layers,
+// 64x64 tiles are 4-17 % faster there and equal or slower for longer reductions.
+static inline TilePick pick_tile_conv(int M, int N, int K) {
+  if (K <= 512) return {64, 64};
+  return pick_tile(M, N);
+}
 template <int BM, int BN, int SBM, int SBN, class AL, class BL, class EP>
 static bool launch_rounds(const AL& al, const BL& bl, const EP& ep, int M, int N, int K) {
   constexpr int rem_div = 3;        // split when the surplus is at most a third of a round
@@ -301,7 +334,7 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
     if (M > 64) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
     return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
   }
-  TilePick tp = pick_tile(M, N);
+  TilePick tp = pick_tile_conv(M, N, K);
   if (tp.bm == 128) return launch_rounds<128, 128, 64, 64>(al, bl, ep, M, N, K);
   if (tp.bn == 128) return launch_rounds<64, 128, 64, 64>(al, bl, ep, M, N, K);
   return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1);
@@ -318,7 +351,7 @@ static bool plan_tiles_stats(int M, int N, int K, StatLayout& L, int& bm, int& b
   const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
   const int64_t slabs = cdiv(K, CONV_BK);
   if (few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)(2 * g_num_cu)) return false;
-  TilePick tp = pick_tile(M, N);
+  TilePick tp = pick_tile_conv(M, N, K);
   bm = tp.bm; bn = tp.bn;
   L.col1 = N; L.g_main = bn / 2; L.g_rem = 32; L.slots_rem = 0;
   if (bn == 128) {        // the surplus-tile split of launch_rounds
@@ -501,17 +534,25 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   // combine with fp32 atomic adds.
   TilePick tp = (K >= 128 && CRS >= 128) ? TilePick{128, 128} : (CRS >= 128 ? TilePick{64, 128} : TilePick{64, 64});
   int64_t tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
-  int split = (int)cdiv(3 * (int64_t)g_num_cu, tiles);
   int max_split = (int)cdiv(red, 256); if (max_split < 1) max_split = 1;
-  if (split > max_split) split = max_split;
-  if (split < 1) split = 1;
+  auto clamp_split = [&](int64_t v) { return (int)(v < 1 ? 1 : (v > max_split ? max_split : v)); };
+  int split = clamp_split(cdiv(3 * (int64_t)g_num_cu, tiles));
+  // How many slices pays best depends on how tiles x slices fall onto the resident block slots and on how short the
+  // per-block reduction gets; it is measured once per shape (a few candidates on a scratch output) and remembered.
+  const BwdfKey key = {{N, C, H, W, K, R, S, sH, sW, pH, pW}};
+  const bool tunable = g_bwdf_tune && max_split > 1 && 2.0 * K * CRS * (double)red >= 2e8;
+  bool tune_now = false;
+  if (tunable) {
+    auto it = g_bwdf_split.find(key);
+    if (it != g_bwdf_split.end()) split = clamp_split(it->second); else tune_now = true;
+  }
   if (beta == 0.f) lh_fill(dw, 0.f, (int64_t)K * CRS);
   EpiRowMajor ep; ep.C = dw; ep.ldc = CRS; ep.alpha = 1.f; ep.beta = 1.f; ep.atomic = split > 1 ? 1 : 0;
   bool ok = false;
   auto go = [&](auto al, auto bl) {
     al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
     bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * H * W * 4); bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.CHW = C * H * W;
-    bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
+    bl.P = d.P; bl.Q = d.Q; bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
     if (tp.bm == 128) ok = igemm_launch<128, 128, 16>(al, bl, ep, K, CRS, (int)red, split);    // measured: the large tile prefers the short slab
     else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
     else ok = igemm_launch<64, 64, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
@@ -526,12 +567,55 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   };
   const bool plain = R == 1 && S == 1 && sH == 1 && sW == 1 && pH == 0 && pW == 0;
   const bool xvec = (PQ % 4 == 0) && (((uintptr_t)x & 15) == 0);
-  if (plain && avec && xvec) go_plain(LoadConvBwdFilterA<true>(), LoadConvBwdFilterA<true>());
-  else if (plain && !avec && !xvec) go_plain(LoadConvBwdFilterA<false>(), LoadConvBwdFilterA<false>());
-  else if (avec && rowvec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<true>());
-  else if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<false>());
-  else if (rowvec) go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<true>());
-  else go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<false>());
+  const bool narrow = PQ < 4 || d.Q < 4;        // the stepping loaders assume at most one carry inside a group of four
+  auto dispatch = [&]() {
+    ep.atomic = split > 1 ? 1 : 0;
+    if (plain && avec && xvec) go_plain(LoadConvBwdFilterA<true>(), LoadConvBwdFilterA<true>());
+    else if (plain && !avec && !xvec && !narrow) go_plain(LoadConvBwdFilterA<false, true>(), LoadConvBwdFilterA<false, true>());
+    else if (plain && !avec && !xvec) go_plain(LoadConvBwdFilterA<false>(), LoadConvBwdFilterA<false>());
+    else if (narrow) { if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<0>()); else go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<0>()); }
+    else if (avec && rowvec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<1>());
+    else if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<2>());
+    else go(LoadConvBwdFilterA<false, true>(), LoadConvBwdFilterB<2>());
+  };
+  if (tune_now) {
+    const size_t sbytes = (size_t)K * CRS * sizeof(float);
+    float* scratch = (float*)lh_malloc_uninit(sbytes);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (scratch && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+      const double targets[] = {1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 5.0, 6.0};
+      int cand[10]; int nc = 0;
+      auto add = [&](int v) { for (int i = 0; i < nc; i++) if (cand[i] == v) return; cand[nc++] = v; };
+      add(split);
+      add(clamp_split((3 * (int64_t)g_num_cu) / tiles));
+      for (double t : targets) add(clamp_split((int64_t)(t * g_num_cu) / tiles));
+      float* const real_out = ep.C;
+      ep.C = scratch;
+      int best = split; float best_ms = 3.0e38f;
+      for (int i = 0; i < nc && !failed(); i++) {
+        split = cand[i];
+        float ms_min = 3.0e38f;
+        for (int rep = 0; rep < 3; rep++) {           // first repetition warms the caches
+          (void)hipEventRecord(e0, g_stream);
+          dispatch();
+          (void)hipEventRecord(e1, g_stream);
+          (void)hipEventSynchronize(e1);
+          float ms = 0.f;
+          if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
+        }
+        if (ms_min < best_ms) { best_ms = ms_min; best = cand[i]; }
+      }
+      ep.C = real_out;
+      split = best;
+      g_bwdf_split[key] = best;
+      if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: %lld tiles, split %d (%.3f ms)\n", N, C, H, K, R, sH, (long long)tiles, best, best_ms);
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (scratch) lh_free_top(sbytes);
+    if (failed()) return;
+  }
+  dispatch();
   if (!ok) return;
   if (db) hipLaunchKernelGGL(k_conv_bwd_bias, dim3(K), dim3(TPB), 0, g_stream, dy, db, N, K, PQ);
   LH_CHECK_LAUNCH();
