@@ -218,6 +218,18 @@ void lh_bn_stats(const float* x, float* save_mean, float* save_invstd, float* ru
                  int N, int C, int HW, float eps, float factor);
 void lh_bn_apply(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd, float* y,
                  int N, int C, int HW, int relu);
+
+/* The residual join behind a batch norm (ResNet's bn3 -> Add -> Relu; the reference runs cudnnBatchNormalizationForwardTraining,
+ * an element-wise add kernel (CUB:397-420) and cudnnActivationForward, CDN:1025-1068, 1380-1400, as three passes):
+ *   out = relu(gamma * (x - mean) * invstd + beta + shortcut)     with the statistics in save_mean / save_invstd
+ * (from lh_conv2d_fwd_bnstats or lh_bn_stats), one pass.  Its backward, given dout = d loss / d out:
+ *   g = dout where out > 0 else 0;   ds = beta_ds * ds + g;   dx = beta_dx * dx + batch-norm backward of g;
+ *   dgamma += sum g * xhat;  dbeta += sum g.
+ * When ds accumulates (beta_ds = 1) or is NULL, dout is overwritten with g.  dx may be NULL (no input gradient). */
+void lh_bn_apply_add_relu(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd,
+                          const float* shortcut, float* out, int N, int C, int HW);
+void lh_bn_bwd_add_relu(const float* x, const float* out, float* dout, const float* gamma, const float* save_mean, const float* save_invstd,
+                        float* dx, float beta_dx, float* ds, float beta_ds, float* dgamma, float* dbeta, int N, int C, int HW);
 /* `+` of two same-shape tensors followed by relu(inPlace = true), and the gradient of that pair:
  * g = dy where y > 0 else 0;  ad = abeta*ad + g;  bd = bbeta*bd + g  (ad or bd may be NULL) */
 void lh_add_relu(const float* a, const float* b, float* out, int64_t n);

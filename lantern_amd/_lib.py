@@ -82,6 +82,8 @@ SIGNATURES = {
     "lh_conv2d_fwd_bnstats": (None, [P, P, P, P] + [I] * 11 + [P, P, P, P, F, F]),
     "lh_bn_stats": (None, [P, P, P, P, P, I, I, I, F, F]),
     "lh_bn_apply": (None, [P, P, P, P, P, P, I, I, I, I]),
+    "lh_bn_apply_add_relu": (None, [P, P, P, P, P, P, P, I, I, I]),
+    "lh_bn_bwd_add_relu": (None, [P, P, P, P, P, P, P, F, P, F, P, P, I, I, I]),
     "lh_rnn_fwd": (None, [I, P, P, P, I, I, I, I, I]),
     "lh_rnn_bwd": (None, [I, P, P, P, P, P, F, P, I, I, I, I, I]),
     "lh_ctc_loss": (None, [P, P, P, P, P, P, I, I, I]),

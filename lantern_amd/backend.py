@@ -93,6 +93,28 @@ class Backend:
         if relu:
             self.unary(RELU, out, n, inPlace=True)
 
+    # out = relu(batchNorm(x) + shortcut): the unfused sequence batchNorm -> + -> relu(inPlace)
+    def batchNormTraining_add_relu_into(self, x, scale, bias, rmean, rvar, shortcut, out, sm, si, N, C, HW, eps=1e-5, factor=0.1):
+        self.batchNormTraining_into(x, scale, bias, rmean, rvar, out, sm, si, N, C, HW, False, eps, factor)
+        self.add_into(out, shortcut, out, N * C * HW, True)
+
+    def conv2D_batch_bn_add_relu_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, shortcut, out, sm, si, eps=1e-5, factor=0.1):
+        N, C, H, W, K, R, S, sH, sW, pH, pW = dims
+        finput = self.conv2D_batch_into(x, w, bias, yconv, *dims)
+        HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
+        self.batchNormTraining_add_relu_into(yconv, scale, bbias, rmean, rvar, shortcut, out, sm, si, N, K, HW, eps, factor)
+        return finput
+
+    def batchNorm_add_relu_grad(self, x, xd, beta_dx, out, dout, scale, scaled, biasd, sm, si, sd, beta_sd, N, C, HW):
+        """Backward of out = relu(batchNorm(x) + shortcut): relu_grad(inPlace) masks dout, the shortcut's gradient takes it,
+        batchNorm_grad does the rest.  dout is overwritten."""
+        n = N * C * HW
+        self.unary_grad(RELU, out, out, dout, dout, n, inPlace=True)
+        if sd is not None:
+            if beta_sd == 0.0: self.copyFloatArray(sd, dout, n)
+            else: self.geam(sd, 1.0, dout, 1.0, sd, n)
+        self.batchNorm_grad(x, xd, dout, scale, scaled, biasd, sm, si, N, C, HW, beta_dx)
+
     def conv2D_batch_into(self, x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW):
         """conv2D_batch writing into a caller-provided y; returns the unfolded input if the backend keeps one (CPU:532-571)."""
         yy, finput = self.conv2D_batch(x, w, bias, N, C, H, W, K, R, S, sH, sW, pH, pW)
@@ -380,6 +402,21 @@ class BackendHIP(Backend):
         else:
             self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
         _lib.check()
+
+    def batchNormTraining_add_relu_into(self, x, scale, bias, rmean, rvar, shortcut, out, sm, si, N, C, HW, eps=1e-5, factor=0.1):
+        self.lib.lh_bn_stats(x.ptr, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, N, C, HW, eps, factor)
+        self.lib.lh_bn_apply_add_relu(x.ptr, scale.ptr, bias.ptr, sm.ptr, si.ptr, shortcut.ptr, out.ptr, N, C, HW); _lib.check()
+
+    def conv2D_batch_bn_add_relu_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, shortcut, out, sm, si, eps=1e-5, factor=0.1):
+        N, C, H, W, K, R, S, sH, sW, pH, pW = dims
+        HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
+        self.lib.lh_conv2d_fwd_bnstats(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, eps, factor)
+        self.lib.lh_bn_apply_add_relu(yconv.ptr, scale.ptr, bbias.ptr, sm.ptr, si.ptr, shortcut.ptr, out.ptr, N, K, HW); _lib.check()
+        self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
+
+    def batchNorm_add_relu_grad(self, x, xd, beta_dx, out, dout, scale, scaled, biasd, sm, si, sd, beta_sd, N, C, HW):
+        self.lib.lh_bn_bwd_add_relu(x.ptr, out.ptr, dout.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, beta_dx,
+                                    sd.ptr if sd is not None else 0, beta_sd, scaled.ptr, biasd.ptr, N, C, HW); _lib.check()
 
     def add_into(self, a, b, out, n, relu):
         if relu: self.lib.lh_add_relu(a.ptr, b.ptr, out.ptr, n)

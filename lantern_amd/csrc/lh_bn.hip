@@ -256,6 +256,54 @@ __global__ void __launch_bounds__(TPB) k_bn_apply(const float* __restrict__ x, f
     [&](int64_t off) { float r = bn_affine(x[off], mean, invstd, g, b); if (RELU) r = r < 0.f ? 0.f : r; y[off] = r; });
 }
 
+// out = relu(gamma * (x - mean) * invstd + beta + shortcut): the residual join behind a batch norm, one read of x and of
+// the shortcut and one write.
+template <bool VEC>
+__global__ void __launch_bounds__(TPB) k_bn_apply_add_relu(const float* __restrict__ x, const float* __restrict__ sc, float* __restrict__ y, const float* gamma, const float* beta,
+                                                           const float* save_mean, const float* save_invstd, int N, int C, int HW, int n_per) {
+  const int c = blockIdx.x, s = blockIdx.y;
+  const float mean = save_mean[c], invstd = save_invstd[c], g = gamma[c], b = beta[c];
+  const int n0 = s * n_per, n1 = min(N, n0 + n_per);
+  bn_foreach<VEC>(n0, n1, C, c, HW,
+    [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 a = *reinterpret_cast<const float4*>(sc + off); float4 r;
+      r.x = __fadd_rn(bn_affine(v.x, mean, invstd, g, b), a.x); r.y = __fadd_rn(bn_affine(v.y, mean, invstd, g, b), a.y);
+      r.z = __fadd_rn(bn_affine(v.z, mean, invstd, g, b), a.z); r.w = __fadd_rn(bn_affine(v.w, mean, invstd, g, b), a.w);
+      r.x = r.x < 0.f ? 0.f : r.x; r.y = r.y < 0.f ? 0.f : r.y; r.z = r.z < 0.f ? 0.f : r.z; r.w = r.w < 0.f ? 0.f : r.w;
+      *reinterpret_cast<float4*>(y + off) = r; },
+    [&](int64_t off) { float r = __fadd_rn(bn_affine(x[off], mean, invstd, g, b), sc[off]); y[off] = r < 0.f ? 0.f : r; });
+}
+
+// First pass of the backward of out = relu(bn(x) + shortcut): g = dout where out > 0 else 0; per-slice sums of g and
+// of g * xhat; g goes to the shortcut's gradient.  INPLACE: ds accumulates (or is absent), so g is also written over
+// dout, where the second pass reads it; otherwise ds = g and the second pass reads ds.
+template <bool VEC, bool INPLACE, bool HAS_DS>
+__global__ void __launch_bounds__(TPB) k_bn_bwd_stats_add(const float* __restrict__ x, const float* __restrict__ out, float* dout, float* ds,
+                                                          const float* save_mean, const float* save_invstd, float* __restrict__ partial, int N, int C, int HW, int n_per) {
+  __shared__ float sm[17];
+  const int c = blockIdx.x, s = blockIdx.y;
+  const int n0 = s * n_per, n1 = min(N, n0 + n_per);
+  const float mean = save_mean[c], is = save_invstd[c];
+  float s1 = 0.f, s2 = 0.f;
+  bn_foreach<VEC>(n0, n1, C, c, HW,
+    [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 g = *reinterpret_cast<const float4*>(dout + off);
+      const float4 m = *reinterpret_cast<const float4*>(out + off);
+      g.x = m.x > 0.f ? g.x : 0.f; g.y = m.y > 0.f ? g.y : 0.f; g.z = m.z > 0.f ? g.z : 0.f; g.w = m.w > 0.f ? g.w : 0.f;
+      if (INPLACE) {
+        *reinterpret_cast<float4*>(dout + off) = g;
+        if (HAS_DS) { float4 o = *reinterpret_cast<const float4*>(ds + off); o.x += g.x; o.y += g.y; o.z += g.z; o.w += g.w; *reinterpret_cast<float4*>(ds + off) = o; }
+      } else {
+        *reinterpret_cast<float4*>(ds + off) = g;
+      }
+      s1 += (g.x + g.y) + (g.z + g.w);
+      s2 += (g.x * ((v.x - mean) * is) + g.y * ((v.y - mean) * is)) + (g.z * ((v.z - mean) * is) + g.w * ((v.w - mean) * is)); },
+    [&](int64_t off) { float g = out[off] > 0.f ? dout[off] : 0.f;
+      if (INPLACE) { dout[off] = g; if (HAS_DS) ds[off] += g; } else ds[off] = g;
+      s1 += g; s2 += g * ((x[off] - mean) * is); });
+  s1 = lh_block_sum(s1, sm);
+  s2 = lh_block_sum(s2, sm);
+  if (threadIdx.x == 0) { float* p = partial + 3 * ((int64_t)c * gridDim.y + s); p[0] = s1; p[1] = s2; }
+}
+
 static bool get_partial() {
   if (g_partial_ptr) return true;
   if (hipGetSymbolAddress((void**)&g_partial_ptr, HIP_SYMBOL(g_bn_partial)) != hipSuccess) { LH_FAIL("bn scratch symbol lookup failed"); return false; }
@@ -371,6 +419,45 @@ void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float
   ProfScope prof_(CAT_BN_BWD);
   LH_REQUIRE(y != nullptr || bias != nullptr, "lh_bn_bwd_relu: y or the layer's bias is required");
   bn_bwd_impl(x, bias ? nullptr : y, dy, gamma, bias, bias ? 2 : 1, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
+}
+
+void lh_bn_apply_add_relu(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd,
+                          const float* shortcut, float* out, int N, int C, int HW) {
+  ProfScope prof_(CAT_BN_FWD);
+  LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_apply_add_relu: empty shape [%d,%d,%d]", N, C, HW);
+  LH_REQUIRE(x && shortcut && out && gamma && beta && save_mean && save_invstd, "lh_bn_apply_add_relu: null operand");
+  Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)out | (uintptr_t)shortcut) & 15) == 0);
+  dim3 grid(C, p.slices);
+  if (p.vec4) hipLaunchKernelGGL((k_bn_apply_add_relu<true>), grid, dim3(TPB), 0, g_stream, x, shortcut, out, gamma, beta, save_mean, save_invstd, N, C, HW, p.n_per);
+  else hipLaunchKernelGGL((k_bn_apply_add_relu<false>), grid, dim3(TPB), 0, g_stream, x, shortcut, out, gamma, beta, save_mean, save_invstd, N, C, HW, p.n_per);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_bn_bwd_add_relu(const float* x, const float* out, float* dout, const float* gamma, const float* save_mean, const float* save_invstd,
+                        float* dx, float beta_dx, float* ds, float beta_ds, float* dgamma, float* dbeta, int N, int C, int HW) {
+  ProfScope prof_(CAT_BN_BWD);
+  LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_bwd_add_relu: empty shape [%d,%d,%d]", N, C, HW);
+  LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_bwd_add_relu: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
+  LH_REQUIRE((beta_dx == 0.0f || beta_dx == 1.0f) && (beta_ds == 0.0f || beta_ds == 1.0f), "lh_bn_bwd_add_relu: beta must be 0 or 1");
+  LH_REQUIRE(x && out && dout && gamma && save_mean && save_invstd, "lh_bn_bwd_add_relu: null operand");
+  LH_REQUIRE(ds != dout && dx != dout, "lh_bn_bwd_add_relu: dout may not alias a gradient output");
+  if (!get_partial()) return;
+  Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dx | (uintptr_t)ds) & 15) == 0);
+  dim3 grid(C, p.slices);
+  const bool inplace = ds == nullptr || beta_ds != 0.0f, acc = beta_dx != 0.0f;
+  const float* g = inplace ? dout : ds;            // where the masked gradient lies after the first pass
+#define STATS(V, I, H) hipLaunchKernelGGL((k_bn_bwd_stats_add<V, I, H>), grid, dim3(TPB), 0, g_stream, x, out, dout, ds, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per)
+#define APPLY(V, A) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, 0>), grid, dim3(TPB), 0, g_stream, x, (const float*)nullptr, g, (const float*)g_partial_ptr, gamma, (const float*)nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
+  if (p.vec4) {
+    if (!inplace) STATS(true, false, true); else if (ds) STATS(true, true, true); else STATS(true, true, false);
+    if (acc) APPLY(true, true); else APPLY(true, false);
+  } else {
+    if (!inplace) STATS(false, false, true); else if (ds) STATS(false, true, true); else STATS(false, true, false);
+    if (acc) APPLY(false, true); else APPLY(false, false);
+  }
+#undef STATS
+#undef APPLY
+  LH_CHECK_LAUNCH();
 }
 
 }  // extern "C"

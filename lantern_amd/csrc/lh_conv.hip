@@ -18,7 +18,8 @@ struct BwdfKey {
   int v[11];
   bool operator<(const BwdfKey& o) const { for (int i = 0; i < 11; i++) if (v[i] != o.v[i]) return v[i] < o.v[i]; return false; }
 };
-static std::map<BwdfKey, int> g_bwdf_split;
+struct BwdfPlan { int bm, bn, split; };
+static std::map<BwdfKey, BwdfPlan> g_bwdf_split;
 static const bool g_bwdf_tune = getenv("LH_NO_TUNE") == nullptr;
 constexpr int TPB = 256;
 
@@ -544,7 +545,8 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   bool tune_now = false;
   if (tunable) {
     auto it = g_bwdf_split.find(key);
-    if (it != g_bwdf_split.end()) split = clamp_split(it->second); else tune_now = true;
+    if (it != g_bwdf_split.end()) { tp = TilePick{it->second.bm, it->second.bn}; tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn); split = clamp_split(it->second.split); }
+    else tune_now = true;
   }
   if (beta == 0.f) lh_fill(dw, 0.f, (int64_t)K * CRS);
   EpiRowMajor ep; ep.C = dw; ep.ldc = CRS; ep.alpha = 1.f; ep.beta = 1.f; ep.atomic = split > 1 ? 1 : 0;
@@ -584,31 +586,38 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (scratch && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
       const double targets[] = {1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 5.0, 6.0};
-      int cand[10]; int nc = 0;
-      auto add = [&](int v) { for (int i = 0; i < nc; i++) if (cand[i] == v) return; cand[nc++] = v; };
-      add(split);
-      add(clamp_split((3 * (int64_t)g_num_cu) / tiles));
-      for (double t : targets) add(clamp_split((int64_t)(t * g_num_cu) / tiles));
+      const TilePick shapes[3] = {{128, 128}, {64, 128}, {64, 64}};
       float* const real_out = ep.C;
       ep.C = scratch;
-      int best = split; float best_ms = 3.0e38f;
-      for (int i = 0; i < nc && !failed(); i++) {
-        split = cand[i];
-        float ms_min = 3.0e38f;
-        for (int rep = 0; rep < 3; rep++) {           // first repetition warms the caches
-          (void)hipEventRecord(e0, g_stream);
-          dispatch();
-          (void)hipEventRecord(e1, g_stream);
-          (void)hipEventSynchronize(e1);
-          float ms = 0.f;
-          if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
+      BwdfPlan best = {tp.bm, tp.bn, split}; float best_ms = 3.0e38f;
+      for (int sh = 0; sh < 3 && !failed(); sh++) {
+        if ((shapes[sh].bm == 128 && K < 128) || (shapes[sh].bn == 128 && CRS < 128)) continue;
+        tp = shapes[sh];
+        tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
+        int cand[10]; int nc = 0;
+        auto add = [&](int v) { for (int i = 0; i < nc; i++) if (cand[i] == v) return; cand[nc++] = v; };
+        add(clamp_split((3 * (int64_t)g_num_cu) / tiles));
+        for (double t : targets) add(clamp_split((int64_t)(t * g_num_cu) / tiles));
+        for (int i = 0; i < nc && !failed(); i++) {
+          split = cand[i];
+          float ms_min = 3.0e38f;
+          for (int rep = 0; rep < 3; rep++) {           // first repetition warms the caches
+            (void)hipEventRecord(e0, g_stream);
+            dispatch();
+            (void)hipEventRecord(e1, g_stream);
+            (void)hipEventSynchronize(e1);
+            float ms = 0.f;
+            if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
+          }
+          if (ms_min < best_ms) { best_ms = ms_min; best = BwdfPlan{tp.bm, tp.bn, cand[i]}; }
         }
-        if (ms_min < best_ms) { best_ms = ms_min; best = cand[i]; }
       }
       ep.C = real_out;
-      split = best;
+      tp = TilePick{best.bm, best.bn};
+      tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
+      split = best.split;
       g_bwdf_split[key] = best;
-      if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: %lld tiles, split %d (%.3f ms)\n", N, C, H, K, R, sH, (long long)tiles, best, best_ms);
+      if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: tile %dx%d, %lld tiles, split %d (%.3f ms)\n", N, C, H, K, R, sH, tp.bm, tp.bn, (long long)tiles, split, best_ms);
     }
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);

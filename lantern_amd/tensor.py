@@ -33,6 +33,7 @@ def set_backend(b):
 # stream is unchanged (at most one launch is ever parked).
 _pending = None
 FUSE_CONV_BN = True       # batchNorm right behind a convolution takes its statistics from the convolution's epilogue
+FUSE_BN_ADD_RELU = True   # batchNorm -> + -> relu(inPlace), the residual join, runs as one pass forward and one fused backward
 
 
 class _Pending:
@@ -40,7 +41,8 @@ class _Pending:
         self.owner = owner          # the TensorR whose value is not computed yet
         self.launch = launch        # launch(relu: bool)
         self.kind = kind            # "relu": a following in-place relu can be fused in; "conv": a following batchNorm can
-        self.launch_bn = launch_bn  # kind "conv": launch_bn(scale, bias, rmean, rvar, ybn, sm, si, relu)
+        self.launch_bn = launch_bn  # kind "conv": launch_bn(scale, bias, rmean, rvar, ybn, sm, si, relu, shortcut=None)
+        self.bn = None              # a parked batchNorm describes itself here so that a following `+` can absorb it
 
 
 def _flush():
@@ -477,9 +479,9 @@ class TensorR:
 
     # -- arithmetic --------------------------------------------------------------------------------
     def _bin(self, op, that):
-        be = get_backend()
         if isinstance(that, TensorR) and op == B.ADD and self.x.shape == that.x.shape and self is not that:
-            return self._add_same_shape(that)
+            return self._add_same_shape(that)      # before get_backend(): a parked batchNorm may be absorbed
+        be = get_backend()
         if isinstance(that, TensorR):
             ya, a, b = self.x._bin(op, that.x)
             y = TensorR._new(ya)
@@ -516,18 +518,39 @@ class TensorR:
     def _add_same_shape(self, that):
         """`+` without broadcasting (TD:1171-1176, CPU:299-304), parked so that a following in-place
         relu fuses with it (the residual join of ResNet)."""
+        global _pending
+        bnp = None                       # a parked batchNorm producing one of the operands: absorbed if a relu follows
+        if FUSE_BN_ADD_RELU and _pending is not None and _pending.bn is not None and (_pending.owner is self or _pending.owner is that):
+            bnp, _pending = _pending, None
         be = get_backend()
         n = self.x.scalarCount
         ybuf = be.mallocArray(n, zero=False)
         y = TensorR._new(Tensor(ybuf, self.x.shape))
-        st = {"relu": False}
+        st = {"relu": False, "joined": False}
+        other = None if bnp is None else (that if bnp.owner is self else self)
 
         def launch(relu):
             st["relu"] = relu
+            if bnp is not None and relu:
+                st["joined"] = True
+                bnp.launch(True, other.x.data, ybuf)
+                bnp.owner.x = None        # the batchNorm's own output is never materialised: a later read must fail, not see garbage
+                return
+            if bnp is not None:
+                bnp.launch(False)
             _backend.add_into(self.x.data, that.x.data, ybuf, n, relu)
         _park(y, launch)
 
         def back():
+            if st["joined"]:
+                info = bnp.bn
+                xin = info["xin"]
+                xd, xbeta = (None, 1.0) if xin.isInput else xin.grad_target()
+                sd, sbeta = (None, 1.0) if other.isInput else other.grad_target()
+                be.batchNorm_add_relu_grad(xin.x.data, xd, xbeta, ybuf, y.d.data, info["scale"].x.data, info["scale"].d.data, info["bias"].d.data,
+                                           info["sm"], info["si"], sd, sbeta, info["N"], info["C"], info["HW"])
+                info["st"]["joined"] = True
+                return
             if st["relu"]:
                 ad, ab = (None, 1.0) if self.isInput else self.grad_target()
                 bd, bb = (None, 1.0) if that.isInput else that.grad_target()
@@ -642,15 +665,23 @@ class TensorR:
         y = TensorR._new(Tensor(ybuf, self.x.shape))
         st = {"relu": False}
 
-        def launch(relu):
+        def launch(relu, shortcut=None, out=None):
             st["relu"] = relu
-            if conv is not None:
+            if shortcut is not None:          # absorbed by a following `+` and relu: out = relu(bn(x) + shortcut)
+                if conv is not None:
+                    conv.launch_bn(scale.x.data, bias.x.data, runningMean.data, runningVar.data, out, sm, si, True, shortcut)
+                else:
+                    _backend.batchNormTraining_add_relu_into(self.x.data, scale.x.data, bias.x.data, runningMean.data, runningVar.data, shortcut, out, sm, si, N, C, HW)
+            elif conv is not None:
                 conv.launch_bn(scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, relu)
             else:
                 _backend.batchNormTraining_into(self.x.data, scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, N, C, HW, relu)
         _park(y, launch)
+        _pending.bn = {"xin": self, "scale": scale, "bias": bias, "sm": sm, "si": si, "N": N, "C": C, "HW": HW, "st": st}
 
         def back():
+            if st.get("joined"):              # the residual join's backward has done this layer's part
+                return
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()
             be.batchNorm_grad(self.x.data, xd, y.d.data, scale.x.data, scale.d.data, bias.d.data, sm, si, N, C, HW, beta,
                               y_relu=ybuf if st["relu"] else None, bias=bias.x.data)
@@ -696,8 +727,11 @@ class TensorR:
         # parked: a batchNorm right behind the convolution takes its statistics from the convolution's epilogue
         def launch(relu):
             kept["finput"] = _backend.conv2D_batch_into(xbuf, wbuf, bbuf, ybuf, *dims)
-        def launch_bn(scale, bb, rm, rv, ybn, sm, si, relu):
-            kept["finput"] = _backend.conv2D_batch_bn_into(xbuf, wbuf, bbuf, ybuf, dims, scale, bb, rm, rv, ybn, sm, si, relu)
+        def launch_bn(scale, bb, rm, rv, ybn, sm, si, relu, shortcut=None):
+            if shortcut is not None:
+                kept["finput"] = _backend.conv2D_batch_bn_add_relu_into(xbuf, wbuf, bbuf, ybuf, dims, scale, bb, rm, rv, shortcut, ybn, sm, si)
+            else:
+                kept["finput"] = _backend.conv2D_batch_bn_into(xbuf, wbuf, bbuf, ybuf, dims, scale, bb, rm, rv, ybn, sm, si, relu)
         _park(y, launch, "conv", launch_bn)
         def back():
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()

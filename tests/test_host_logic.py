@@ -94,3 +94,50 @@ def test_fused_and_unfused_relu_gradients_agree(on_cpu):
         return x.d.toCPU(), g.d.toCPU(), b.d.toCPU()
     for u, v in zip(run(True), run(False)):
         np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("bn_side", ["left", "right"])
+def test_residual_join_absorbs_the_batchnorm_and_matches_the_unfused_program(on_cpu, bn_side):
+    """conv -> batchNorm -> + shortcut -> relu(inPlace): with the join fused the batchNorm is absorbed by the `+`
+    (either operand) and its own output is never materialised; values and every gradient equal the unfused program."""
+    rng = np.random.RandomState(3)
+    xs = rng.randn(2, 4, 6, 6).astype(np.float32); ws = (rng.randn(4, 4, 3, 3) * 0.2).astype(np.float32)
+
+    def run(fused):
+        T.FUSE_BN_ADD_RELU = fused
+        try:
+            x = TensorR(Tensor.fromNumpy(xs)); w = TensorR(Tensor.fromNumpy(ws))
+            g = TensorR(Tensor.fromData((4,), 1.5, 0.5, 2.0, 1.0)); b = TensorR(Tensor.fromData((4,), 0.1, -0.2, 0.0, 0.3))
+            kept = {}
+            def f(d):
+                h = (x * 1.5)                                     # the shortcut has a gradient of its own
+                y = h.convBBP(w, None, (1, 1), (1, 1)).batchNorm(g, b, Tensor.zeros(4), Tensor.ones(4))
+                kept["bn"] = y
+                z = (y + h) if bn_side == "left" else (h + y)
+                assert (T._pending is not None and T._pending.owner is z)
+                out = z.relu(True)
+                kept["out"] = out.x.toCPU().copy()
+                return (out * out).sum()
+            gradR_loss(f)(Tensor.zeros(1))
+            return kept, [kept["out"], x.d.toCPU(), w.d.toCPU(), g.d.toCPU(), b.d.toCPU()]
+        finally:
+            T.FUSE_BN_ADD_RELU = True
+    kf, fused = run(True)
+    ku, plain = run(False)
+    assert kf["bn"].x is None and ku["bn"].x is not None          # absorbed: reading the batchNorm's output later fails loudly
+    for u, v in zip(fused, plain):
+        np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)
+
+
+def test_batchnorm_followed_by_add_without_relu_runs_unfused(on_cpu):
+    rng = np.random.RandomState(4)
+    xs = rng.randn(3, 2, 4, 4).astype(np.float32)
+    x = TensorR(Tensor.fromNumpy(xs)); g, b = TensorR(Tensor.ones(2)), TensorR(Tensor.zeros(2))
+    s = TensorR(Tensor.fromNumpy(rng.randn(3, 2, 4, 4).astype(np.float32)))
+    y = x.batchNorm(g, b, Tensor.zeros(2), Tensor.ones(2))
+    z = y + s
+    v = z.x.toCPU()                                                   # no relu follows: batchNorm, then the add
+    ref = (xs - xs.mean(axis=(0, 2, 3), keepdims=True)) / np.sqrt(xs.var(axis=(0, 2, 3), keepdims=True) + 1e-5)
+    np.testing.assert_allclose(v, ref + s.x.toCPU(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(y.x.toCPU(), ref, rtol=1e-4, atol=1e-5)      # and the batchNorm's output exists
+    T._tape.clear()

@@ -779,3 +779,34 @@ def test_command_list_keeps_program_order_around_other_kernels_and_wraps_its_buf
         be.batchSmallOps(False)
     from lantern_amd import _lib
     _lib.check()
+
+
+# ---- residual join behind a batch norm: out = relu(bn(x) + shortcut) -----------------------------------
+@pytest.mark.parametrize("shape", [(8, 16, 28, 28), (3, 5, 7, 7), (4, 32, 1, 1)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("beta_sd", [0.0, 1.0, None], ids=["shortcut_grad_fresh", "shortcut_grad_accumulates", "shortcut_is_input"])
+def test_batchnorm_add_relu_join_forward_and_backward(pair, shape, beta_sd):
+    N, Cc, H, W = shape
+    HW, n = H * W, N * Cc * H * W
+    rng = np.random.RandomState(60)
+    x = rng.randn(*shape).astype(np.float32); s = rng.randn(*shape).astype(np.float32); dout = rng.randn(*shape).astype(np.float32)
+    g = (rng.rand(Cc) + 0.5).astype(np.float32); b = (rng.randn(Cc) * 0.3).astype(np.float32)
+
+    pre = (x.astype(np.float64) - x.mean((0, 2, 3), keepdims=True)) / np.sqrt(x.var((0, 2, 3), keepdims=True) + 1e-5) * g.reshape(1, -1, 1, 1) + b.reshape(1, -1, 1, 1) + s
+    s[np.abs(pre) < 1e-4] += 0.01               # keep every element away from the relu's kink: a flipped mask changes the whole channel
+
+    def f(be, up, down):
+        X, S, G, Bb = up(x), up(s), up(g), up(b)
+        rm, rv = up(np.zeros(Cc, np.float32)), up(np.ones(Cc, np.float32))
+        out = be.mallocArray(n, zero=False); sm = be.mallocArray(Cc, zero=False); si = be.mallocArray(Cc, zero=False)
+        be.batchNormTraining_add_relu_into(X, G, Bb, rm, rv, S, out, sm, si, N, Cc, HW)
+        dx = up(np.full(n, 2.0, np.float32)); dg = up(np.ones(Cc, np.float32)); db = up(np.ones(Cc, np.float32))
+        sd = None if beta_sd is None else up(np.full(n, 3.0, np.float32))
+        D = up(dout)
+        be.batchNorm_add_relu_grad(X, dx, 1.0, out, D, G, dg, db, sm, si, sd, beta_sd if beta_sd is not None else 1.0, N, Cc, HW)
+        outs = [down(out, shape), down(dx, shape), down(dg, (Cc,)), down(db, (Cc,)), down(rm, (Cc,)), down(rv, (Cc,))]
+        if sd is not None:
+            outs.append(down(sd, shape))
+        return outs
+
+    outs = pair.run(f)
+    check_all(outs, rtol=2e-4)
