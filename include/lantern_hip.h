@@ -146,7 +146,10 @@ void lh_dot_vv(const float* x, const float* y, float* out, int n);
 void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x, int64_t n);   /* y += s[0]*x, s on device (vv-dot grad) */
 
 /* ---- conv2D_batch and its gradient (TD:292-296; CDN:515-880) ----------- */
-/* y[n,k,p,q] = bias[k] + sum_{c,r,s} x[n,c,p*sH-pH+r,q*sW-pW+s] * w[k,c,r,s]; bias may be NULL. */
+/* y[n,k,p,q] = bias[k] + sum_{c,r,s} x[n,c,p*sH-pH+r,q*sW-pW+s] * w[k,c,r,s]; bias may be NULL.
+ * The filter gradient cuts its long reduction (N*P*Q) into slices combined with atomic adds; tile shape and slice count are
+ * measured once per convolution shape on first use (a few dozen timed launches on scratch memory, then remembered for the
+ * life of the process).  Environment: LH_NO_TUNE=1 keeps the built-in rule, LH_TUNE_VERBOSE=1 prints each choice to stderr. */
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
 void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,

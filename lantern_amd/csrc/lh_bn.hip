@@ -200,38 +200,31 @@ __global__ void __launch_bounds__(TPB) k_bn_finalize(const float* __restrict__ p
   if (run_var) { float unb = cnt > 1.0 ? (float)(m2 / (cnt - 1.0)) : var; run_var[c] = (1.0f - factor) * run_var[c] + factor * unb; }
 }
 
-// Channel statistics from the (sum, sum of squares) pieces of a convolution epilogue: one block per channel,
-// each piece turned into (count, mean, M2) and merged with Chan's formula in double.
+// Channel statistics from the (sum, sum of squares) pieces of a convolution epilogue: one block per channel adds the
+// pieces up in double (they are fp32 sums of at most 64 values each, so double carries them exactly enough:
+// M2 = sum q - (sum a)^2 / n loses about log2(n mean^2 / M2) of 53 bits) and finishes the channel.
 __global__ void __launch_bounds__(TPB) k_bn_finalize_conv(const float* __restrict__ partial, int C, int ncols, int col1, int g_main, int slots_main, int g_rem,
                                                           int slots, float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor) {
-  __shared__ double sc[TPB], sm_[TPB], s2[TPB];
+  __shared__ double sa_[TPB], sq_[TPB];
   const int c = blockIdx.x;
-  double cnt = 0.0, mean = 0.0, m2 = 0.0;
+  const float2* pc = reinterpret_cast<const float2*>(partial) + (size_t)c * slots;
+  double sa = 0.0, sq = 0.0;
   for (int s = threadIdx.x; s < slots; s += TPB) {
-    int n;
-    if (s < slots_main) { const int j0 = s * g_main; n = min(g_main, col1 - j0); }
-    else { const int j0 = col1 + (s - slots_main) * g_rem; n = min(g_rem, ncols - j0); }
-    if (n <= 0) continue;
-    const float2 pv = reinterpret_cast<const float2*>(partial)[(size_t)c * slots + s];
-    const double a = pv.x, q = pv.y;
-    const double mb = a / n, m2b = q - a * mb;
-    const double tot = cnt + n, d = mb - mean;
-    mean += d * n / tot; m2 += m2b + d * d * cnt * n / tot; cnt = tot;
+    const int j0 = s < slots_main ? s * g_main : col1 + (s - slots_main) * g_rem;
+    const int n = s < slots_main ? min(g_main, col1 - j0) : min(g_rem, ncols - j0);
+    if (n <= 0) continue;                       // a slot behind the last column holds nothing
+    const float2 pv = pc[s];
+    sa += (double)pv.x; sq += (double)pv.y;
   }
-  sc[threadIdx.x] = cnt; sm_[threadIdx.x] = mean; s2[threadIdx.x] = m2;
+  sa_[threadIdx.x] = sa; sq_[threadIdx.x] = sq;
   __syncthreads();
   for (int off = TPB / 2; off > 0; off >>= 1) {
-    if (threadIdx.x < off) {
-      const double na = sc[threadIdx.x], nb = sc[threadIdx.x + off];
-      if (nb > 0.0) {
-        const double tot = na + nb, d = sm_[threadIdx.x + off] - sm_[threadIdx.x];
-        sm_[threadIdx.x] += d * nb / tot; s2[threadIdx.x] += s2[threadIdx.x + off] + d * d * na * nb / tot; sc[threadIdx.x] = tot;
-      }
-    }
+    if (threadIdx.x < off) { sa_[threadIdx.x] += sa_[threadIdx.x + off]; sq_[threadIdx.x] += sq_[threadIdx.x + off]; }
     __syncthreads();
   }
   if (threadIdx.x == 0) {
-    const double n = sc[0], mu = sm_[0], M2 = s2[0] < 0.0 ? 0.0 : s2[0];
+    const double n = (double)ncols, mu = sa_[0] / n;
+    double M2 = sq_[0] - sa_[0] * mu; if (M2 < 0.0) M2 = 0.0;
     const float var = (float)(M2 / n);
     if (save_mean) save_mean[c] = (float)mu;
     if (save_invstd) save_invstd[c] = 1.0f / sqrtf(var + eps);

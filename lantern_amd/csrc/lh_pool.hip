@@ -7,12 +7,14 @@ using namespace lh;
 namespace {
 constexpr int TPB = 256;
 
+// IT: uint32_t when every flat index fits 32 bits (a 64-bit division costs several times a 32-bit one)
+template <class IT>
 __global__ void __launch_bounds__(TPB) k_maxpool_fwd(const float* __restrict__ x, float* __restrict__ y, int* __restrict__ idx,
                                                      int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t n_out) {
-  int64_t o = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
-  for (; o < n_out; o += st) {
-    int q = (int)(o % oW); int64_t t = o / oW; int p = (int)(t % oH); int64_t nc = t / oH;
-    const int64_t base = nc * H * W;
+  IT o = (IT)blockIdx.x * TPB + threadIdx.x; const IT st = (IT)gridDim.x * TPB;
+  for (; o < (IT)n_out; o += st) {
+    int q = (int)(o % (IT)oW); IT t = o / (IT)oW; int p = (int)(t % (IT)oH); IT nc = t / (IT)oH;
+    const int64_t base = (int64_t)nc * H * W;
     float best = -3.402823466e+38f; int bi = 0;
     const int h0 = p * sH - pad, w0 = q * sW - pad;
     for (int r = 0; r < kH; r++) {
@@ -39,9 +41,10 @@ __global__ void __launch_bounds__(TPB) k_maxpool_bwd_atomic(const float* __restr
 template <bool ACC>
 __global__ void __launch_bounds__(TPB) k_maxpool_bwd_dense(const float* __restrict__ dy, const int* __restrict__ idx, float* __restrict__ dx,
                                                            int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t n_in) {
-  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
-  for (; i < n_in; i += st) {
-    const int w = (int)(i % W); const int64_t t = i / W; const int h = (int)(t % H); const int64_t nc = t / H;
+  // n_in < 2^31 (the argmax is an int32 flat index): 32-bit index arithmetic
+  uint32_t i = blockIdx.x * TPB + threadIdx.x; const uint32_t st = gridDim.x * TPB;
+  for (; i < (uint32_t)n_in; i += st) {
+    const int w = (int)(i % (uint32_t)W); const uint32_t t = i / (uint32_t)W; const int h = (int)(t % (uint32_t)H); const int64_t nc = t / (uint32_t)H;
     const int hp = h + pad, wp = w + pad;
     const int p_hi = min(oH - 1, hp / sH), q_hi = min(oW - 1, wp / sW);
     const int p_lo = hp < kH ? 0 : (hp - kH) / sH + 1, q_lo = wp < kW ? 0 : (wp - kW) / sW + 1;
@@ -94,7 +97,8 @@ void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, 
   int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
   int64_t n_out = (int64_t)N * C * oH * oW;
   if (n_out <= 0) return;
-  hipLaunchKernelGGL(k_maxpool_fwd, dim3(stream_grid(n_out, TPB * 2)), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, n_out);
+  if (n_out < 0x7fffffffLL) hipLaunchKernelGGL((k_maxpool_fwd<uint32_t>), dim3(stream_grid(n_out, TPB * 2)), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, n_out);
+  else hipLaunchKernelGGL((k_maxpool_fwd<int64_t>), dim3(stream_grid(n_out, TPB * 2)), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, n_out);
   LH_CHECK_LAUNCH();
 }
 void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out) {
