@@ -147,9 +147,11 @@ void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x,
 
 /* ---- conv2D_batch and its gradient (TD:292-296; CDN:515-880) ----------- */
 /* y[n,k,p,q] = bias[k] + sum_{c,r,s} x[n,c,p*sH-pH+r,q*sW-pW+s] * w[k,c,r,s]; bias may be NULL.
- * The filter gradient cuts its long reduction (N*P*Q) into slices combined with atomic adds; tile shape and slice count are
- * measured once per convolution shape on first use (a few dozen timed launches on scratch memory, then remembered for the
- * life of the process).  Environment: LH_NO_TUNE=1 keeps the built-in rule, LH_TUNE_VERBOSE=1 prints each choice to stderr. */
+ * Launch plans are measured once per convolution shape on first use and remembered for the life of the process: the
+ * filter gradient (tile shape and number of slices of its long reduction N*P*Q, timed on scratch memory) and, on calls
+ * whose result overwrites its output, the forward and input-gradient products (tile shape, stream-K workers; a few timed
+ * repetitions of the launch itself).  Environment: LH_NO_TUNE=1 keeps the built-in rules, LH_TUNE_VERBOSE=1 prints each
+ * choice to stderr. */
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
 void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,

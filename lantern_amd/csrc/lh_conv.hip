@@ -323,8 +323,28 @@ static bool launch_rounds(const AL& al, const BL& bl, const EP& ep, int M, int N
   return igemm_launch<BM, BN, CONV_BK>(al, bl, ep, M, N, K, 1);
 }
 
+// The launch plans of a forward / input-gradient product.  0: the built-in rule (stream-K for few tiles over a long
+// reduction, else the tile pick_tile_conv names).  1-3: plain tiles 128x128, 64x128, 64x64.  4-7: stream-K over
+// 128x128 / 64x128 tiles with two or three workers per CU.
+constexpr int N_PLANS = 8;
 template <class AL, class BL, class EP>
-static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out = nullptr, int64_t zero_n = 0, bool prezeroed = false) {
+static bool plan_valid(int plan, const EP& ep, int M, int K, bool can_zero) {
+  if (plan == 0) return true;
+  if ((plan == 1 || plan == 4 || plan == 6) && M <= 64) return false;
+  if (plan >= 4) return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= 16;
+  return true;
+}
+template <class AL, class BL, class EP>
+static bool launch_plan(int plan, const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out, int64_t zero_n, bool prezeroed) {
+  if (plan >= 4) {
+    const int workers = (plan >= 6 ? 3 : 2) * g_num_cu;
+    if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
+    if (plan == 4 || plan == 6) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
+    return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
+  }
+  if (plan == 1) return launch_rounds<128, 128, 64, 64>(al, bl, ep, M, N, K);
+  if (plan == 2) return launch_rounds<64, 128, 64, 64>(al, bl, ep, M, N, K);
+  if (plan == 3) return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1);
   const int64_t t128 = cdiv(M, 128) * cdiv(N, 128), t64 = cdiv(M, 64) * cdiv(N, 128);
   const int workers = 2 * g_num_cu;
   const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
@@ -341,18 +361,67 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
   return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1);
 }
 
+// Which plan is fastest depends on how the tiles fall onto the chip, on the length of the reduction and on the
+// gather; it is measured once per shape, on a call whose epilogue overwrites (so that repeating the launch is
+// harmless), and remembered per loader / epilogue combination.
+struct PlanKey {
+  int v[7];
+  bool operator<(const PlanKey& o) const { for (int i = 0; i < 7; i++) if (v[i] != o.v[i]) return v[i] < o.v[i]; return false; }
+};
+template <class AL, class BL, class EP>
+static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out = nullptr, int64_t zero_n = 0, bool prezeroed = false) {
+  static std::map<PlanKey, int> chosen;
+  const bool can_zero = zero_out != nullptr || prezeroed;
+  if (!g_bwdf_tune || 2.0 * M * N * (double)K < 2e8) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  const PlanKey key = {{M, N, K, ep.eH, ep.eW, ep.W, ep.PIX}};
+  auto it = chosen.find(key);
+  if (it != chosen.end()) {
+    const int plan = plan_valid<AL, BL, EP>(it->second, ep, M, K, can_zero) ? it->second : 0;
+    return launch_plan(plan, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  }
+  // tuned only on a call that may be repeated: an overwriting epilogue onto an output this launch alone writes
+  if (ep.beta != 0.f || prezeroed) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+    if (e0) (void)hipEventDestroy(e0);
+    return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  }
+  int best = 0; float best_ms = 3.0e38f, base_ms = 0.f;
+  bool ok = true;
+  for (int plan = 0; plan < N_PLANS && ok; plan++) {
+    if (!plan_valid<AL, BL, EP>(plan, ep, M, K, can_zero)) continue;
+    float ms_min = 3.0e38f;
+    for (int rep = 0; rep < 3 && ok; rep++) {             // the first repetition warms the caches
+      (void)hipEventRecord(e0, g_stream);
+      ok = launch_plan(plan, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+      (void)hipEventRecord(e1, g_stream);
+      (void)hipEventSynchronize(e1);
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
+    }
+    if (plan == 0) base_ms = ms_min;
+    if (ms_min < best_ms * 0.98f) { best_ms = ms_min; best = plan; }      // a later plan must win by 2 % to displace an earlier one
+  }
+  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+  if (!ok || failed()) return false;
+  chosen[key] = best;
+  if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv product M%d N%d K%d (stride %d,%d): plan %d, %.3f ms (built-in rule %.3f ms)\n", M, N, K, ep.eH, ep.eW, best, best_ms, base_ms);
+  return true;                                               // the timed launches have produced the result
+}
+
 // Where the statistics pieces of a forward launch lie (see bn_finalize_conv_partials).
 struct StatLayout { int col1, g_main, slots_main, g_rem, slots_rem; };
 
 // The tile plan launch_tiles would choose, for a launch that also leaves statistics pieces.  Returns false (and
 // launches nothing) for shapes that take the stream-K path, whose tiles are finished by several blocks.
 template <class AL, class BL>
-static bool plan_tiles_stats(int M, int N, int K, StatLayout& L, int& bm, int& bn) {
+static bool plan_tiles_stats(int M, int N, int K, StatLayout& L, int& bm, int& bn, int force = 0 /* 1-3: the tile of launch plan 1-3 */) {
   const int64_t t128 = cdiv(M, 128) * cdiv(N, 128), t64 = cdiv(M, 64) * cdiv(N, 128);
   const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
   const int64_t slabs = cdiv(K, CONV_BK);
   if (few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)(2 * g_num_cu)) return false;
   TilePick tp = pick_tile_conv(M, N, K);
+  if (force == 1 && M > 64) tp = {128, 128}; else if (force == 2) tp = {64, 128}; else if (force == 3) tp = {64, 64};
   bm = tp.bm; bn = tp.bn;
   L.col1 = N; L.g_main = bn / 2; L.g_rem = 32; L.slots_rem = 0;
   if (bn == 128) {        // the surplus-tile split of launch_rounds
@@ -410,6 +479,54 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
     bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dC.init(C); bl.dS.init(S);
     StatLayout L; int bm = 0, bn_ = 0;
     if (bn && bias == nullptr && plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, L, bm, bn_)) {
+      // the tile shape of this launch is measured once per shape (the launch overwrites y and its statistics pieces, so
+      // repeating it is harmless) and remembered
+      static std::map<PlanKey, int> chosen;
+      const PlanKey key = {{K, N * PQ, CRS, H, W, sH, R}};
+      const bool tunable = g_bwdf_tune && 2.0 * K * CRS * (double)N * PQ >= 2e8;
+      int force = 0;
+      auto run = [&](int f) {
+        StatLayout Lf; int bmf = 0, bnf = 0;
+        if (!plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, Lf, bmf, bnf, f)) return false;
+        const size_t pbytes = (size_t)(Lf.slots_main + Lf.slots_rem) * K * 2 * sizeof(float);
+        float* partial = (float*)lh_malloc_uninit(pbytes);
+        if (partial == nullptr) return false;
+        EpiConvOutStats es; static_cast<EpiConvOut&>(es) = ep; es.partial = partial; es.slotBase = 0; es.slotsTotal = Lf.slots_main + Lf.slots_rem;
+        bool good = launch_tiles_stats(al, bl, es, K, N * PQ, CRS, Lf, bmf, bnf);
+        if (good) bn_finalize_conv_partials(partial, K, N * PQ, Lf.col1, Lf.g_main, Lf.slots_main, Lf.g_rem, bn->save_mean, bn->save_invstd, nullptr, nullptr, bn->eps, bn->factor);
+        lh_free_top(pbytes);
+        return good;
+      };
+      if (tunable) {
+        auto it = chosen.find(key);
+        if (it != chosen.end()) force = it->second;
+        else {
+          hipEvent_t e0 = nullptr, e1 = nullptr;
+          if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+            float best_ms = 3.0e38f, base_ms = 0.f; int best = 0;
+            for (int f = 0; f <= 3 && !failed(); f++) {
+              if (f == 1 && K <= 64) continue;
+              float ms_min = 3.0e38f;
+              for (int rep = 0; rep < 3; rep++) {
+                (void)hipEventRecord(e0, g_stream);
+                if (!run(f)) break;
+                (void)hipEventRecord(e1, g_stream);
+                (void)hipEventSynchronize(e1);
+                float ms = 0.f;
+                if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
+              }
+              if (f == 0) base_ms = ms_min;
+              if (ms_min < best_ms * 0.98f) { best_ms = ms_min; best = f; }
+            }
+            chosen[key] = best; force = best;
+            if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv fwd+stats K%d N%d CRS%d H%d: tile plan %d, %.3f ms (built-in rule %.3f ms)\n", K, N * PQ, CRS, H, best, best_ms, base_ms);
+          }
+          if (e0) (void)hipEventDestroy(e0);
+          if (e1) (void)hipEventDestroy(e1);
+          if (failed()) return;
+        }
+      }
+      plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, L, bm, bn_, force);
       const size_t pbytes = (size_t)(L.slots_main + L.slots_rem) * K * 2 * sizeof(float);
       float* partial = (float*)lh_malloc_uninit(pbytes);
       if (partial == nullptr) return;
