@@ -151,7 +151,9 @@ void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x,
  * filter gradient (tile shape and number of slices of its long reduction N*P*Q, timed on scratch memory) and, on calls
  * whose result overwrites its output, the forward and input-gradient products (tile shape, stream-K workers; a few timed
  * repetitions of the launch itself).  Environment: LH_NO_TUNE=1 keeps the built-in rules, LH_TUNE_VERBOSE=1 prints each
- * choice to stderr. */
+ * choice to stderr.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
+ * remembered and are used again after lh_set_tuning(1)). */
+void lh_set_tuning(int on);
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
 void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,

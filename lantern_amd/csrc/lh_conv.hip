@@ -20,7 +20,30 @@ struct BwdfKey {
 };
 struct BwdfPlan { int bm, bn, split; };
 static std::map<BwdfKey, BwdfPlan> g_bwdf_split;
-static const bool g_bwdf_tune = getenv("LH_NO_TUNE") == nullptr;
+static bool g_bwdf_tune = getenv("LH_NO_TUNE") == nullptr;      // lh_set_tuning
+
+// Times `launch` (a callable returning false on failure) on the library's stream: three repetitions, the first warms
+// the caches, the smaller of the other two counts.  Returns a negative number when a launch or the timer failed.
+struct LaunchTimer {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  bool ok;
+  LaunchTimer() { ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess; }
+  ~LaunchTimer() { if (e0) (void)hipEventDestroy(e0); if (e1) (void)hipEventDestroy(e1); }
+  template <class F>
+  float ms(F launch) {
+    float best = 3.0e38f;
+    for (int rep = 0; rep < 3; rep++) {
+      (void)hipEventRecord(e0, g_stream);
+      if (!launch()) return -1.f;
+      (void)hipEventRecord(e1, g_stream);
+      if (hipEventSynchronize(e1) != hipSuccess) return -1.f;
+      float t = 0.f;
+      if (hipEventElapsedTime(&t, e0, e1) != hipSuccess) return -1.f;
+      if (rep > 0 && t < best) best = t;
+    }
+    return best;
+  }
+};
 constexpr int TPB = 256;
 
 struct ConvDims { int N, C, H, W, K, R, S, sH, sW, pH, pW, P, Q; };
@@ -381,29 +404,16 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
   }
   // tuned only on a call that may be repeated: an overwriting epilogue onto an output this launch alone writes
   if (ep.beta != 0.f || prezeroed) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
-  hipEvent_t e0 = nullptr, e1 = nullptr;
-  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
-    if (e0) (void)hipEventDestroy(e0);
-    return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
-  }
+  LaunchTimer timer;
+  if (!timer.ok) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   int best = 0; float best_ms = 3.0e38f, base_ms = 0.f;
-  bool ok = true;
-  for (int plan = 0; plan < N_PLANS && ok; plan++) {
+  for (int plan = 0; plan < N_PLANS; plan++) {
     if (!plan_valid<AL, BL, EP>(plan, ep, M, K, can_zero)) continue;
-    float ms_min = 3.0e38f;
-    for (int rep = 0; rep < 3 && ok; rep++) {             // the first repetition warms the caches
-      (void)hipEventRecord(e0, g_stream);
-      ok = launch_plan(plan, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
-      (void)hipEventRecord(e1, g_stream);
-      (void)hipEventSynchronize(e1);
-      float ms = 0.f;
-      if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
-    }
-    if (plan == 0) base_ms = ms_min;
-    if (ms_min < best_ms * 0.98f) { best_ms = ms_min; best = plan; }      // a later plan must win by 2 % to displace an earlier one
+    const float ms = timer.ms([&]() { return launch_plan(plan, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed); });
+    if (ms < 0.f || failed()) return false;
+    if (plan == 0) base_ms = ms;
+    if (ms < best_ms * 0.98f) { best_ms = ms; best = plan; }      // a later plan must win by 2 % to displace an earlier one
   }
-  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
-  if (!ok || failed()) return false;
   chosen[key] = best;
   if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv product M%d N%d K%d (stride %d,%d): plan %d, %.3f ms (built-in rule %.3f ms)\n", M, N, K, ep.eH, ep.eW, best, best_ms, base_ms);
   return true;                                               // the timed launches have produced the result
@@ -501,29 +511,19 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
         auto it = chosen.find(key);
         if (it != chosen.end()) force = it->second;
         else {
-          hipEvent_t e0 = nullptr, e1 = nullptr;
-          if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+          LaunchTimer timer;
+          if (timer.ok) {
             float best_ms = 3.0e38f, base_ms = 0.f; int best = 0;
-            for (int f = 0; f <= 3 && !failed(); f++) {
+            for (int f = 0; f <= 3; f++) {
               if (f == 1 && K <= 64) continue;
-              float ms_min = 3.0e38f;
-              for (int rep = 0; rep < 3; rep++) {
-                (void)hipEventRecord(e0, g_stream);
-                if (!run(f)) break;
-                (void)hipEventRecord(e1, g_stream);
-                (void)hipEventSynchronize(e1);
-                float ms = 0.f;
-                if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
-              }
-              if (f == 0) base_ms = ms_min;
-              if (ms_min < best_ms * 0.98f) { best_ms = ms_min; best = f; }
+              const float ms = timer.ms([&]() { return run(f); });
+              if (ms < 0.f || failed()) return;
+              if (f == 0) base_ms = ms;
+              if (ms < best_ms * 0.98f) { best_ms = ms; best = f; }
             }
             chosen[key] = best; force = best;
             if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv fwd+stats K%d N%d CRS%d H%d: tile plan %d, %.3f ms (built-in rule %.3f ms)\n", K, N * PQ, CRS, H, best, best_ms, base_ms);
           }
-          if (e0) (void)hipEventDestroy(e0);
-          if (e1) (void)hipEventDestroy(e1);
-          if (failed()) return;
         }
       }
       plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, L, bm, bn_, force);
@@ -553,6 +553,8 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
 }
 
 extern "C" {
+
+void lh_set_tuning(int on) { g_bwdf_tune = on != 0; }
 
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
@@ -700,8 +702,8 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   if (tune_now) {
     const size_t sbytes = (size_t)K * CRS * sizeof(float);
     float* scratch = (float*)lh_malloc_uninit(sbytes);
-    hipEvent_t e0 = nullptr, e1 = nullptr;
-    if (scratch && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+    LaunchTimer timer;
+    if (scratch && timer.ok) {
       const double targets[] = {1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 5.0, 6.0};
       const TilePick shapes[3] = {{128, 128}, {64, 128}, {64, 64}};
       float* const real_out = ep.C;
@@ -717,15 +719,8 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
         for (double t : targets) add(clamp_split((int64_t)(t * g_num_cu) / tiles));
         for (int i = 0; i < nc && !failed(); i++) {
           split = cand[i];
-          float ms_min = 3.0e38f;
-          for (int rep = 0; rep < 3; rep++) {           // first repetition warms the caches
-            (void)hipEventRecord(e0, g_stream);
-            dispatch();
-            (void)hipEventRecord(e1, g_stream);
-            (void)hipEventSynchronize(e1);
-            float ms = 0.f;
-            if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess && rep > 0 && ms < ms_min) ms_min = ms;
-          }
+          const float ms_min = timer.ms([&]() { dispatch(); return ok; });
+          if (ms_min < 0.f) break;
           if (ms_min < best_ms) { best_ms = ms_min; best = BwdfPlan{tp.bm, tp.bn, cand[i]}; }
         }
       }
@@ -736,8 +731,6 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
       g_bwdf_split[key] = best;
       if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: tile %dx%d, %lld tiles, split %d (%.3f ms)\n", N, C, H, K, R, sH, tp.bm, tp.bn, (long long)tiles, split, best_ms);
     }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
     if (scratch) lh_free_top(sbytes);
     if (failed()) return;
   }

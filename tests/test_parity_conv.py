@@ -125,3 +125,54 @@ def test_sgemm(on_hip, ta, tb, m, n, k):
         c_ = dev.up(Cm)
         dev.lib.lh_sgemm(ta, tb, m, n, k, alpha, dev.up(A).ptr, A.shape[1], dev.up(B).ptr, B.shape[1], beta, c_.ptr, n); dev.check()
         assert_close(dev.down(c_, (m, n)), ref, what="sgemm %d%d a=%g b=%g" % (ta, tb, alpha, beta))
+
+
+# Shapes large enough for the launch plans to be measured on first use (>= 2e8 flop) and small enough for the oracle.
+TUNED_SHAPES = [
+    (8, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),      # tap path, 64-row product
+    (4, 256, 14, 14, 256, 3, 3, 1, 1, 1, 1),    # few tiles over a long reduction: the stream-K plans compete
+    (16, 128, 14, 14, 512, 1, 1, 1, 1, 0, 0),   # 1x1: the plain filter-gradient loaders
+    (8, 64, 28, 28, 128, 3, 3, 2, 2, 1, 1),     # stride 2: four residue classes share a pre-zeroed dx (never timed)
+    (6, 96, 15, 15, 160, 3, 3, 1, 1, 1, 1),     # odd map, partial tiles everywhere
+]
+
+
+@pytest.mark.parametrize("dims", TUNED_SHAPES, ids=lambda d: "x".join(map(str, d)))
+def test_conv_measured_launch_plans_and_their_reuse(on_hip, dims):
+    """First calls time several launch plans (repeating the launch), later calls reuse the remembered plan, also with an
+    accumulating epilogue; every call must give the oracle's result, with the tuner on and off."""
+    dev = Dev(on_hip)
+    lib = on_hip.lib
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    rng = np.random.RandomState(77)
+    x = rng.randn(N, Cc, H, W).astype(np.float32)
+    w = (rng.randn(K, Cc, R, S) / np.sqrt(Cc * R * S)).astype(np.float32)
+    dy = rng.randn(N, K, P, Q).astype(np.float32)
+    y_ref, dx_ref, dw_ref, _ = _oracle_conv(x, w, None, dy, dims)
+    mean_ref = y_ref.astype(np.float64).mean((0, 2, 3)); var_ref = y_ref.astype(np.float64).var((0, 2, 3))
+    ints = list(dims)
+    xd, wd, dyd = dev.up(x), dev.up(w), dev.up(dy)
+    try:
+        for tuning in (1, 1, 0, 1):                     # measures, reuses, built-in rule, reuses again
+            lib.lh_set_tuning(tuning)
+            y = dev.zeros(y_ref.size); lib.lh_conv2d_fwd(xd.ptr, wd.ptr, 0, y.ptr, *ints)
+            assert_close(dev.down(y, y_ref.shape), y_ref, what="fwd (tuning %d)" % tuning)
+            y2 = dev.zeros(y_ref.size); sm = dev.zeros(K); si = dev.zeros(K); rm = dev.zeros(K); rv = dev.up(np.ones(K, np.float32))
+            lib.lh_conv2d_fwd_bnstats(xd.ptr, wd.ptr, 0, y2.ptr, *ints, sm.ptr, si.ptr, rm.ptr, rv.ptr, 1e-5, 0.1)
+            assert_close(dev.down(y2, y_ref.shape), y_ref, what="fwd with statistics (tuning %d)" % tuning)
+            np.testing.assert_allclose(dev.down(sm, (K,)), mean_ref, rtol=1e-4, atol=1e-5)
+            np.testing.assert_allclose(dev.down(si, (K,)), 1.0 / np.sqrt(var_ref + 1e-5), rtol=2e-4)
+            np.testing.assert_allclose(dev.down(rm, (K,)), 0.1 * mean_ref, rtol=1e-4, atol=1e-5)      # running statistics updated exactly once
+            dx0 = dev.up(np.full(x.size, 9.0, np.float32)); lib.lh_conv2d_bwd_data(dyd.ptr, wd.ptr, dx0.ptr, 0.0, *ints)
+            assert_close(dev.down(dx0, x.shape), dx_ref, what="dx, overwriting (tuning %d)" % tuning)
+            dx1 = dev.up(np.ones(x.size, np.float32)); lib.lh_conv2d_bwd_data(dyd.ptr, wd.ptr, dx1.ptr, 1.0, *ints)
+            assert_close(dev.down(dx1, x.shape) - 1.0, dx_ref, what="dx, accumulating (tuning %d)" % tuning)
+            dw1 = dev.zeros(w.size)
+            lib.lh_conv2d_bwd_filter(xd.ptr, dyd.ptr, dw1.ptr, 0, 1.0, *ints); lib.lh_conv2d_bwd_filter(xd.ptr, dyd.ptr, dw1.ptr, 0, 1.0, *ints)
+            assert_close(dev.down(dw1, w.shape) * 0.5, dw_ref, what="dw, accumulated twice (tuning %d)" % tuning)
+            dw0 = dev.up(np.full(w.size, 5.0, np.float32)); lib.lh_conv2d_bwd_filter(xd.ptr, dyd.ptr, dw0.ptr, 0, 0.0, *ints)
+            assert_close(dev.down(dw0, w.shape), dw_ref, what="dw, overwriting (tuning %d)" % tuning)
+    finally:
+        lib.lh_set_tuning(1)
+    dev.check()
