@@ -244,6 +244,8 @@ struct LoadConvBwdFilterB {
 struct EpiConvOut {
   static constexpr bool STATS = false;
   float* out; const float* bias; int chan, PIX, W, eH, eW, aH, aW; float beta;
+  int zfill2 = 0;           // the grid is every second pixel of every second row of an image with even sides (a 1x1 filter, stride 2):
+                            // the element is stored together with the three zeros of its 2x2 cell, so the output needs no clearing
   FastDiv dPIXc, dWc;
   struct Col { int off; bool valid; };
   __device__ __forceinline__ Col col(int j, int N) const {
@@ -257,6 +259,11 @@ struct EpiConvOut {
     if (!c.valid || i >= M) return;
     float* p = out + c.off + i * PIX;
     if (bias && part < 2) v += bias[i];
+    if (zfill2) {             // only set for overwriting, complete sums (host side)
+      *reinterpret_cast<float2*>(p) = make_float2(v, 0.f);
+      *reinterpret_cast<float2*>(p + W) = make_float2(0.f, 0.f);
+      return;
+    }
     if (part) atomicAdd(p, v);
     else *p = beta == 0.f ? v : v + beta * *p;
   }
@@ -586,12 +593,91 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
       int r0 = (aH + pH) % sH, s0 = (aW + pW) % sW;
       if (r0 >= R || s0 >= S || aH >= H || aW >= W) any_empty = true;
     }
+    // Stride > 1 with a filter wider than one tap: the residue classes are independent products with disjoint outputs
+    // and different reduction lengths; they run as one grouped launch (longest reduction first), so the chip is
+    // filled once instead of up to sH*sW times with a quarter of the columns each.
+    if (sH * sW > 1 && RS > 1) {
+      struct Cls { int aH, aW, r0, s0, Rc, Sc, Hc, Wc, Kred; };
+      Cls cls[IGEMM_MAX_GROUPS]; int ng = 0; bool fits = true;
+      for (int aH = 0; aH < sH; aH++) for (int aW = 0; aW < sW; aW++) {
+        const int r0 = (aH + pH) % sH, s0 = (aW + pW) % sW;
+        if (r0 >= R || s0 >= S || aH >= H || aW >= W) continue;
+        if (ng == IGEMM_MAX_GROUPS) { fits = false; continue; }
+        Cls c; c.aH = aH; c.aW = aW; c.r0 = r0; c.s0 = s0;
+        c.Rc = (R - r0 + sH - 1) / sH; c.Sc = (S - s0 + sW - 1) / sW; c.Hc = (H - aH + sH - 1) / sH; c.Wc = (W - aW + sW - 1) / sW;
+        c.Kred = c.Rc * c.Sc * K;
+        cls[ng++] = c;
+      }
+      if (fits && ng >= 2) {
+        for (int i = 1; i < ng; i++) for (int j = i; j > 0 && cls[j].Kred > cls[j - 1].Kred; j--) { Cls t = cls[j]; cls[j] = cls[j - 1]; cls[j - 1] = t; }
+        if (beta == 0.f && any_empty) lh_fill(dx, 0.f, (int64_t)N * C * HW);       // pixels no class reaches
+        size_t bytes = 0;
+        for (int i = 0; i < ng; i++) bytes += (((size_t)cls[i].Kred * C * sizeof(float)) + 255) & ~(size_t)255;
+        char* scratch = (char*)lh_malloc_uninit(bytes);
+        if (scratch == nullptr) return;
+        LoadPlainK<true> al[IGEMM_MAX_GROUPS]; LoadConvBwdDataTapB bl[IGEMM_MAX_GROUPS]; EpiConvOut ep[IGEMM_MAX_GROUPS];
+        int Ms[IGEMM_MAX_GROUPS], Ns[IGEMM_MAX_GROUPS], Ks[IGEMM_MAX_GROUPS];
+        size_t off = 0; int64_t ntot = 0; int kmax = 0;
+        for (int i = 0; i < ng; i++) {
+          const Cls& c = cls[i];
+          float* wt = (float*)(scratch + off);
+          const size_t wbytes = (size_t)c.Kred * C * sizeof(float);
+          off += (wbytes + 255) & ~(size_t)255;
+          const int64_t n = (int64_t)c.Kred * C;
+          hipLaunchKernelGGL(k_filter_to_ctk, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, R, S, c.r0, c.s0, sH, sW, c.Rc, c.Sc, n);
+          al[i].base = wt; al[i].nbytes = (uint32_t)wbytes; al[i].ld = c.Kred;
+          LoadConvBwdDataTapB& b = bl[i];
+          b.base = dy; b.nbytes = dybytes; b.K = K; b.P = d.P; b.Q = d.Q; b.PQ = PQ;
+          b.offH = (c.aH + pH - c.r0) / sH; b.offW = (c.aW + pW - c.s0) / sW;
+          b.dPIX.init(c.Hc * c.Wc); b.dWc.init(c.Wc); b.dK.init(K); b.dSc.init(c.Sc);
+          EpiConvOut& e = ep[i];
+          e.out = dx; e.bias = nullptr; e.chan = C; e.PIX = HW; e.W = W; e.eH = sH; e.eW = sW; e.aH = c.aH; e.aW = c.aW; e.beta = beta;
+          e.dPIXc.init(c.Hc * c.Wc); e.dWc.init(c.Wc);
+          Ms[i] = C; Ns[i] = N * c.Hc * c.Wc; Ks[i] = c.Kred;
+          ntot += Ns[i]; if (c.Kred > kmax) kmax = c.Kred;
+        }
+        auto run = [&](int tile) {           // 1: 128x128, 2: 64x128, 3: 64x64
+          if (tile == 1) return igemm_launch_grouped<128, 128, CONV_BK>(ng, al, bl, ep, Ms, Ns, Ks);
+          if (tile == 2) return igemm_launch_grouped<64, 128, CONV_BK>(ng, al, bl, ep, Ms, Ns, Ks);
+          return igemm_launch_grouped<64, 64, CONV_BK>(ng, al, bl, ep, Ms, Ns, Ks);
+        };
+        // tile shape: measured once per shape on an overwriting call (every pixel of a class is written by one block, so
+        // repeating the launch is harmless), else the remembered one, else by the total tile count
+        static std::map<PlanKey, int> chosen;
+        const PlanKey key = {{N, C, H, W, K, R * 100 + S, sH * 100 + sW}};
+        TilePick tp = pick_tile(C, (int)(ntot < 0x7fffffff ? ntot : 0x7fffffff));
+        int tile = tp.bm == 128 ? 1 : (tp.bn == 128 ? 2 : 3);
+        auto it = chosen.find(key);
+        if (it != chosen.end()) tile = it->second;
+        else if (g_bwdf_tune && beta == 0.f && 2.0 * C * (double)ntot * kmax >= 2e8) {
+          LaunchTimer timer;
+          if (timer.ok) {
+            float best_ms = 3.0e38f; int best = tile;
+            for (int tcand = 1; tcand <= 3; tcand++) {
+              if (tcand == 1 && C <= 64) continue;
+              const float ms = timer.ms([&]() { return run(tcand); });
+              if (ms < 0.f || failed()) { lh_free_top(bytes); return; }
+              if (ms < best_ms * 0.98f) { best_ms = ms; best = tcand; }
+            }
+            chosen[key] = best; tile = best;
+            if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv input gradient, stride (%d,%d), C%d H%d K%d k%d: %d classes in one launch, tile plan %d, %.3f ms\n", sH, sW, C, H, K, R, ng, best, best_ms);
+          }
+        }
+        ok = run(tile);
+        lh_free_top(bytes);
+        if (!ok) return;
+        LH_CHECK_LAUNCH();
+        return;
+      }
+    }
     // several classes (or an empty one) with beta = 0: clear dx once, then every class may overwrite or add
     const bool strided = sH * sW > 1;
-    if (beta == 0.f && (any_empty || strided)) lh_fill(dx, 0.f, (int64_t)N * C * HW);
+    // 1x1 filter, stride 2, no padding, even image: the one class that has a tap writes whole 2x2 cells
+    const bool cells = beta == 0.f && RS == 1 && sH == 2 && sW == 2 && pH == 0 && pW == 0 && (H % 2) == 0 && (W % 2) == 0 && (((uintptr_t)dx & 7) == 0);
+    if (beta == 0.f && (any_empty || strided) && !cells) lh_fill(dx, 0.f, (int64_t)N * C * HW);
     float* zo = (beta == 0.f && !strided) ? dx : nullptr;
     const int64_t zn = (int64_t)N * C * HW;
-    const bool pz = beta == 0.f && strided;
+    const bool pz = beta == 0.f && strided && !cells;
     for (int aH = 0; aH < sH && ok; aH++) for (int aW = 0; aW < sW && ok; aW++) {
       const int r0 = (aH + pH) % sH, s0 = (aW + pW) % sW;
       if (r0 >= R || s0 >= S || aH >= H || aW >= W) continue;
@@ -603,6 +689,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
       bl.dPIX.init(Hc * Wc); bl.dWc.init(Wc); bl.dK.init(K); bl.dSc.init(Sc);
       EpiConvOut ep; ep.out = dx; ep.bias = nullptr; ep.chan = C; ep.PIX = HW; ep.W = W; ep.eH = sH; ep.eW = sW; ep.aH = aH; ep.aW = aW; ep.beta = beta;
       ep.dPIXc.init(Hc * Wc); ep.dWc.init(Wc);
+      ep.zfill2 = cells ? 1 : 0;
       if (RS == 1) {
         LoadPlainT al; al.base = w; al.nbytes = (uint32_t)((size_t)K * C * 4); al.ld = C;          // A[c][k] = w[k][c]
         ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred, zo, zn, pz);

@@ -140,8 +140,9 @@ __device__ __forceinline__ float lh_half_sum32(float v) {
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------
+// The work of one block; `block` is its index within the launch (or within its group of a grouped launch).
 template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
-__global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const EP ep, const GemmShape gs) {
+__device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP& ep, const GemmShape& gs, const int block) {
   constexpr int KQ = BK / 4, PAD = 8 / KQ, LDA = BM + PAD, LDB = BN + PAD;
   constexpr int TM = BM / 2, TN = BN / 2, MI = TM / 32, NI = TN / 32;
   constexpr int GA = BM * KQ / 256, GB = BN * KQ / 256;
@@ -150,7 +151,7 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
   float4* As = lh_smem;
   float4* Bs = lh_smem + 2 * KQ * LDA;
 
-  const int logical = (blockIdx.x % 8) * gs.perXcd + blockIdx.x / 8;
+  const int logical = (block % 8) * gs.perXcd + block / 8;
   if (logical >= gs.total) return;
   // Work of this block: either one (tile, k-split) item, or -- stream-K -- an equal share of all
   // k-slabs of all tiles, walked tile by tile; a tile whose slabs are shared between two blocks
@@ -336,6 +337,25 @@ __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const E
   }  // segments
 }
 
+template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
+__global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const EP ep, const GemmShape gs) {
+  igemm_block<BM, BN, BK, AL, BL, EP, SK>(al, bl, ep, gs, (int)blockIdx.x);
+}
+
+// Up to four products in one launch (the residue classes of a strided input gradient: same loaders and tile, their own
+// operands, reduction lengths and output maps).  Blocks [first[g], first[g+1]) belong to group g; the longest first.
+constexpr int IGEMM_MAX_GROUPS = 4;
+template <class AL, class BL, class EP>
+struct IgemmGroups { AL al[IGEMM_MAX_GROUPS]; BL bl[IGEMM_MAX_GROUPS]; EP ep[IGEMM_MAX_GROUPS]; GemmShape gs[IGEMM_MAX_GROUPS]; int first[IGEMM_MAX_GROUPS + 1]; };
+template <int BM, int BN, int BK, class AL, class BL, class EP>
+__global__ void __launch_bounds__(256) k_igemm_grouped(const IgemmGroups<AL, BL, EP> g) {
+  const int b = (int)blockIdx.x;
+  int gi = 0;
+#pragma unroll
+  for (int i = 1; i < IGEMM_MAX_GROUPS; i++) if (b >= g.first[i]) gi = i;
+  igemm_block<BM, BN, BK, AL, BL, EP, false>(g.al[gi], g.bl[gi], g.ep[gi], g.gs[gi], b - g.first[gi]);
+}
+
 template <int BM, int BN, int BK>
 constexpr size_t igemm_smem_bytes() { return (size_t)2 * (BK / 4) * ((BM + 8 / (BK / 4)) + (BN + 8 / (BK / 4))) * sizeof(float4); }
 
@@ -397,6 +417,44 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
   }
   ProfScope prof_(g_kernel_cat);
   hipLaunchKernelGGL(kern, dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
+  return true;
+}
+
+// One launch for up to IGEMM_MAX_GROUPS products that share loaders and tile shape (plain tiles: no k-split, no stream-K).
+template <int BM, int BN, int BK, class AL, class BL, class EP>
+bool igemm_launch_grouped(int ngroups, const AL* al, const BL* bl, const EP* ep, const int* M, const int* N, const int* K) {
+  if (ngroups < 1 || ngroups > IGEMM_MAX_GROUPS) { LH_FAIL("igemm: %d groups", ngroups); return false; }
+  IgemmGroups<AL, BL, EP> g;
+  int64_t first = 0;
+  for (int i = 0; i < IGEMM_MAX_GROUPS; i++) {
+    const int j = i < ngroups ? i : 0;                      // unused slots repeat group 0 behind the last block
+    g.al[i] = al[j]; g.bl[i] = bl[j]; g.ep[i] = ep[j];
+    GemmShape& gs = g.gs[i];
+    gs.M = M[j]; gs.N = N[j]; gs.K = K[j]; gs.colBase = 0;
+    gs.tilesM = (int)cdiv(M[j], BM); gs.tilesN = (int)cdiv(N[j], BN);
+    int kper = (int)cdiv(K[j] > 0 ? K[j] : 1, BK) * BK;
+    gs.kPerSplit = kper; gs.splitK = 1;
+    gs.slabsPerTile = (int)cdiv(K[j] > 0 ? K[j] : 1, BK);
+    gs.units = (long long)gs.tilesM * gs.tilesN * gs.slabsPerTile;
+    gs.streamk = 0;
+    const int64_t total = (int64_t)gs.tilesM * gs.tilesN;
+    gs.total = (int)total; gs.perXcd = (int)cdiv(total, 8);
+    g.first[i] = (int)first;
+    if (i < ngroups) first += 8 * (int64_t)gs.perXcd;
+    if (first <= 0 || first > 0x3fffffff) { LH_FAIL("igemm: grouped tile count %lld out of range", (long long)first); return false; }
+  }
+  g.first[IGEMM_MAX_GROUPS] = (int)first;
+  constexpr size_t smem = igemm_smem_bytes<BM, BN, BK>();
+  auto kern = k_igemm_grouped<BM, BN, BK, AL, BL, EP>;
+  static bool attr_done = false;
+  if (smem > 48 * 1024 && !attr_done) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+      LH_FAIL("igemm: cannot reserve %zu bytes of LDS", smem); return false;
+    }
+    attr_done = true;
+  }
+  ProfScope prof_(g_kernel_cat);
+  hipLaunchKernelGGL(kern, dim3((unsigned)first), dim3(256), smem, g_stream, g);
   return true;
 }
 
