@@ -7,27 +7,48 @@ using namespace lh;
 namespace {
 constexpr int TPB = 256;
 
-// IT: uint32_t when every flat index fits 32 bits (a 64-bit division costs several times a 32-bit one)
-template <class IT>
+// One block row-slot per output row (n*C + c, p); threads run along q, so the only division is one per row.
+// S2: stride (2,2), the common case, with the stride folded into shifts.
+// K3: a 3x3 window, unrolled so that its nine loads are in flight together (with run-time bounds the loop serialises them).
+template <bool S2, bool K3>
 __global__ void __launch_bounds__(TPB) k_maxpool_fwd(const float* __restrict__ x, float* __restrict__ y, int* __restrict__ idx,
-                                                     int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t n_out) {
-  IT o = (IT)blockIdx.x * TPB + threadIdx.x; const IT st = (IT)gridDim.x * TPB;
-  for (; o < (IT)n_out; o += st) {
-    int q = (int)(o % (IT)oW); IT t = o / (IT)oW; int p = (int)(t % (IT)oH); IT nc = t / (IT)oH;
-    const int64_t base = (int64_t)nc * H * W;
-    float best = -3.402823466e+38f; int bi = 0;
-    const int h0 = p * sH - pad, w0 = q * sW - pad;
-    for (int r = 0; r < kH; r++) {
-      int h = h0 + r;
-      if (h < 0 || h >= H) continue;
-      for (int s = 0; s < kW; s++) {
-        int w = w0 + s;
-        if (w < 0 || w >= W) continue;
-        float v = x[base + (int64_t)h * W + w];
-        if (v > best) { best = v; bi = (int)(base + (int64_t)h * W + w); }
+                                                     int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t rows) {
+  const int ry = threadIdx.x / 64, lane = threadIdx.x & 63;            // four rows per block, a wavefront each
+  for (int64_t row = (int64_t)blockIdx.x * 4 + ry; row < rows; row += (int64_t)gridDim.x * 4) {
+    const int p = (int)(row % oH); const int64_t nc = row / oH;
+    const int64_t base = nc * H * W;
+    const int h0 = (S2 ? 2 * p : p * sH) - pad;
+    for (int q = lane; q < oW; q += 64) {
+      const int w0 = (S2 ? 2 * q : q * sW) - pad;
+      float best = -3.402823466e+38f; int bi = 0;
+      if (K3) {
+        float v[9]; bool in[9];
+#pragma unroll
+        for (int r = 0; r < 3; r++)
+#pragma unroll
+          for (int t = 0; t < 3; t++) {
+            const int h = h0 + r, w = w0 + t;
+            in[r * 3 + t] = h >= 0 && h < H && w >= 0 && w < W;
+            v[r * 3 + t] = in[r * 3 + t] ? x[base + (int64_t)h * W + w] : 0.f;
+          }
+#pragma unroll
+        for (int e = 0; e < 9; e++)          // same visiting order and strict comparison as the loop below
+          if (in[e] && v[e] > best) { best = v[e]; bi = (int)(base + (int64_t)(h0 + e / 3) * W + w0 + e % 3); }
+      } else {
+        for (int r = 0; r < kH; r++) {
+          const int h = h0 + r;
+          if (h < 0 || h >= H) continue;
+          for (int t = 0; t < kW; t++) {
+            const int w = w0 + t;
+            if (w < 0 || w >= W) continue;
+            const float v = x[base + (int64_t)h * W + w];
+            if (v > best) { best = v; bi = (int)(base + (int64_t)h * W + w); }
+          }
+        }
       }
+      const int64_t o = row * oW + q;
+      y[o] = best; idx[o] = bi;
     }
-    y[o] = best; idx[o] = bi;
   }
 }
 // Scatter-add.  Windows overlap when stride < kernel, so two outputs may hit the same input:
@@ -38,24 +59,44 @@ __global__ void __launch_bounds__(TPB) k_maxpool_bwd_atomic(const float* __restr
 }
 // Gather form: one thread per input pixel; the windows that contain (h, w) are p in [p_lo, p_hi] x q in
 // [q_lo, q_hi]; a window contributes when its stored argmax is this pixel's flat index.
-template <bool ACC>
+// W2: at most two windows per direction cover a pixel (kernel <= 2 * stride): the four candidates are fetched together.
+template <bool ACC, bool S2, bool W2>
 __global__ void __launch_bounds__(TPB) k_maxpool_bwd_dense(const float* __restrict__ dy, const int* __restrict__ idx, float* __restrict__ dx,
-                                                           int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t n_in) {
-  // n_in < 2^31 (the argmax is an int32 flat index): 32-bit index arithmetic
-  uint32_t i = blockIdx.x * TPB + threadIdx.x; const uint32_t st = gridDim.x * TPB;
-  for (; i < (uint32_t)n_in; i += st) {
-    const int w = (int)(i % (uint32_t)W); const uint32_t t = i / (uint32_t)W; const int h = (int)(t % (uint32_t)H); const int64_t nc = t / (uint32_t)H;
-    const int hp = h + pad, wp = w + pad;
-    const int p_hi = min(oH - 1, hp / sH), q_hi = min(oW - 1, wp / sW);
-    const int p_lo = hp < kH ? 0 : (hp - kH) / sH + 1, q_lo = wp < kW ? 0 : (wp - kW) / sW + 1;
+                                                           int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t rows) {
+  // a wavefront per input row (n*C + c, h), lanes along w: one division per row; S2 folds stride (2,2) into shifts
+  const int ry = threadIdx.x / 64, lane = threadIdx.x & 63;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + ry; row < rows; row += (int64_t)gridDim.x * 4) {
+    const int h = (int)(row % H); const int64_t nc = row / H;
+    const int hp = h + pad;
+    const int p_hi = min(oH - 1, S2 ? hp >> 1 : hp / sH);
+    const int p_lo = hp < kH ? 0 : (S2 ? (hp - kH) >> 1 : (hp - kH) / sH) + 1;
     const int64_t ob = nc * oH * oW;
-    float acc = 0.f;
-    for (int p = p_lo; p <= p_hi; p++)
-      for (int q = q_lo; q <= q_hi; q++) {
-        const int64_t o = ob + (int64_t)p * oW + q;
-        if (idx[o] == (int)i) acc += dy[o];
+    for (int w = lane; w < W; w += 64) {
+      const int wp = w + pad;
+      const int q_hi = min(oW - 1, S2 ? wp >> 1 : wp / sW);
+      const int q_lo = wp < kW ? 0 : (S2 ? (wp - kW) >> 1 : (wp - kW) / sW) + 1;
+      const int64_t i = row * W + w;
+      float acc = 0.f;
+      if (W2) {
+        int id[4]; float g[4]; bool in[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int p = p_lo + (e >> 1), q = q_lo + (e & 1);
+          in[e] = p <= p_hi && q <= q_hi;
+          const int64_t o = ob + (int64_t)(in[e] ? p : p_hi) * oW + (in[e] ? q : q_hi);      // p_hi, q_hi are always valid windows
+          id[e] = idx[o]; g[e] = dy[o];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) if (in[e] && id[e] == (int)i) acc += g[e];        // same order as the loops below
+      } else {
+        for (int p = p_lo; p <= p_hi; p++)
+          for (int q = q_lo; q <= q_hi; q++) {
+            const int64_t o = ob + (int64_t)p * oW + q;
+            if (idx[o] == (int)i) acc += dy[o];
+          }
       }
-    dx[i] = ACC ? dx[i] + acc : acc;
+      dx[i] = ACC ? dx[i] + acc : acc;
+    }
   }
 }
 __global__ void __launch_bounds__(TPB) k_avgpool_fwd(const float* __restrict__ x, float* __restrict__ y, int H, int W, int oH, int oW,
@@ -97,8 +138,13 @@ void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, 
   int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
   int64_t n_out = (int64_t)N * C * oH * oW;
   if (n_out <= 0) return;
-  if (n_out < 0x7fffffffLL) hipLaunchKernelGGL((k_maxpool_fwd<uint32_t>), dim3(stream_grid(n_out, TPB * 2)), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, n_out);
-  else hipLaunchKernelGGL((k_maxpool_fwd<int64_t>), dim3(stream_grid(n_out, TPB * 2)), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, n_out);
+  const int64_t rows = (int64_t)N * C * oH;
+  const int grid = stream_grid(rows, 4);
+#define GO(S, K) hipLaunchKernelGGL((k_maxpool_fwd<S, K>), dim3(grid), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, rows)
+  const bool k3 = kH == 3 && kW == 3;
+  if (sH == 2 && sW == 2) { if (k3) GO(true, true); else GO(true, false); }
+  else { if (k3) GO(false, true); else GO(false, false); }
+#undef GO
   LH_CHECK_LAUNCH();
 }
 void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out) {
@@ -117,9 +163,15 @@ void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float b
   LH_REQUIRE(n_in < 2147483647LL, "lh_maxpool_bwd_dense: input too large for int32 argmax");
   if (n_in <= 0) return;
   const int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
-  const int grid = stream_grid(n_in, TPB * 2);
-  if (beta == 0.f) hipLaunchKernelGGL((k_maxpool_bwd_dense<false>), dim3(grid), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, oH, oW, kH, kW, sH, sW, pad, n_in);
-  else hipLaunchKernelGGL((k_maxpool_bwd_dense<true>), dim3(grid), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, oH, oW, kH, kW, sH, sW, pad, n_in);
+  const int64_t rows = (int64_t)N * C * H;
+  const int grid = stream_grid(rows, 4);
+  const bool s2 = sH == 2 && sW == 2;
+  const bool w2 = kH <= 2 * sH && kW <= 2 * sW;
+#define GO(A, S, T) hipLaunchKernelGGL((k_maxpool_bwd_dense<A, S, T>), dim3(grid), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, oH, oW, kH, kW, sH, sW, pad, rows)
+#define GO2(A) do { if (s2) { if (w2) GO(A, true, true); else GO(A, true, false); } else { if (w2) GO(A, false, true); else GO(A, false, false); } } while (0)
+  if (beta == 0.f) GO2(false); else GO2(true);
+#undef GO2
+#undef GO
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {

@@ -118,7 +118,11 @@ def test_batchnorm_inference(pair):
 POOLS = [(64, 64, 112, 112, 3, 3, 2, 2, 1),     # ResNet stem
          (8, 6, 24, 24, 2, 2, 2, 2, 0),          # LeNet
          (4, 96, 15, 15, 3, 3, 2, 2, 0),         # SqueezeNet (overlapping windows, no pad)
-         (2, 3, 9, 7, 3, 2, 2, 1, 1), (1, 1, 2, 2, 2, 2, 2, 2, 0), (3, 5, 7, 7, 7, 7, 1, 1, 0)]
+         (2, 3, 9, 7, 3, 2, 2, 1, 1), (1, 1, 2, 2, 2, 2, 2, 2, 0), (3, 5, 7, 7, 7, 7, 1, 1, 0),
+         (2, 3, 10, 10, 2, 2, 3, 3, 0),          # stride above the window: pixels no window covers
+         (2, 4, 9, 9, 3, 3, 1, 1, 1),            # 3x3 stride 1: three windows per direction over a pixel
+         (1, 2, 11, 11, 5, 5, 2, 2, 2),          # 5x5 stride 2
+         (2, 2, 70, 70, 3, 3, 2, 2, 1)]          # rows wider than a wavefront
 
 
 @pytest.mark.parametrize("p", POOLS, ids=lambda s: "x".join(map(str, s)))
