@@ -502,7 +502,12 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
       const PlanKey key = {{K, N * PQ, CRS, H, W, sH, R}};
       const bool tunable = g_bwdf_tune && 2.0 * K * CRS * (double)N * PQ >= 2e8;
       int force = 0;
-      auto run = [&](int f) {
+      auto run = [&](int f) {           // 0: the rule's tile, 1-3: a forced tile, 4: unfused (any launch plan, then a pass over y)
+        if (f == 4) {
+          if (!launch_tiles(al, bl, ep, K, N * PQ, CRS, y, (int64_t)N * K * PQ)) return false;
+          lh_bn_stats(y, bn->save_mean, bn->save_invstd, nullptr, nullptr, N, K, PQ, bn->eps, bn->factor);
+          return !failed();
+        }
         StatLayout Lf; int bmf = 0, bnf = 0;
         if (!plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, Lf, bmf, bnf, f)) return false;
         const size_t pbytes = (size_t)(Lf.slots_main + Lf.slots_rem) * K * 2 * sizeof(float);
@@ -521,7 +526,7 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
           LaunchTimer timer;
           if (timer.ok) {
             float best_ms = 3.0e38f, base_ms = 0.f; int best = 0;
-            for (int f = 0; f <= 3; f++) {
+            for (int f = 0; f <= 4; f++) {
               if (f == 1 && K <= 64) continue;
               const float ms = timer.ms([&]() { return run(f); });
               if (ms < 0.f || failed()) return;
@@ -533,15 +538,19 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
           }
         }
       }
-      plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, L, bm, bn_, force);
-      const size_t pbytes = (size_t)(L.slots_main + L.slots_rem) * K * 2 * sizeof(float);
-      float* partial = (float*)lh_malloc_uninit(pbytes);
-      if (partial == nullptr) return;
-      EpiConvOutStats es; static_cast<EpiConvOut&>(es) = ep; es.partial = partial; es.slotBase = 0; es.slotsTotal = L.slots_main + L.slots_rem;
-      ok = launch_tiles_stats(al, bl, es, K, N * PQ, CRS, L, bm, bn_);
-      if (ok) bn_finalize_conv_partials(partial, K, N * PQ, L.col1, L.g_main, L.slots_main, L.g_rem, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, bn->eps, bn->factor);
-      lh_free_top(pbytes);
-      bn = nullptr;      // done
+      if (force == 4) {           // measured: better without the statistics epilogue (stream-K or another plan, then lh_bn_stats below)
+        ok = launch_tiles(al, bl, ep, K, N * PQ, CRS, y, (int64_t)N * K * PQ);
+      } else {
+        plan_tiles_stats<LoadPlainK<true>, LoadConvFwdTapB>(K, N * PQ, CRS, L, bm, bn_, force);
+        const size_t pbytes = (size_t)(L.slots_main + L.slots_rem) * K * 2 * sizeof(float);
+        float* partial = (float*)lh_malloc_uninit(pbytes);
+        if (partial == nullptr) return;
+        EpiConvOutStats es; static_cast<EpiConvOut&>(es) = ep; es.partial = partial; es.slotBase = 0; es.slotsTotal = L.slots_main + L.slots_rem;
+        ok = launch_tiles_stats(al, bl, es, K, N * PQ, CRS, L, bm, bn_);
+        if (ok) bn_finalize_conv_partials(partial, K, N * PQ, L.col1, L.g_main, L.slots_main, L.g_rem, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, bn->eps, bn->factor);
+        lh_free_top(pbytes);
+        bn = nullptr;      // done
+      }
     } else {
       ok = launch_tiles(al, bl, ep, K, N * PQ, CRS, y, (int64_t)N * K * PQ);
     }

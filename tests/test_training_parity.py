@@ -28,12 +28,12 @@ def _run(make_trainer, backend, steps):
     return np.array(losses), params
 
 
-def _compare(make_trainer, hip_backend, cpu_backend, steps=10, tol=1e-3, per_tensor=1e-3):
+def _compare(make_trainer, hip_backend, cpu_backend, steps=10, tol=1e-3, per_tensor=1e-3, loss_late=None):
     """Tracking criteria.  fp32 summation order differs between the two backends, and a relu (or a
     max-pool argmax) is discontinuous at 0: on the ResNet program one mask flip in 10^6 elements
     after the first step already moves that layer's gradient by 4e-4 of its norm (measured), and SGD
     with momentum compounds such events.  Hence:
-      - loss of every step within 2*tol relative;
+      - loss of every step within 2*tol relative (with `loss_late`: the first half of the steps, and `loss_late` for the rest);
       - the whole parameter vector within tol (relative L2);
       - every tensor that is not tiny (rms >= 1e-2: filters, matrices, BN scales) within `per_tensor`
         (relative L2): 1e-3 for LeNet; 2e-2 for the batch-normalised ResNet programs, where the
@@ -44,7 +44,12 @@ def _compare(make_trainer, hip_backend, cpu_backend, steps=10, tol=1e-3, per_ten
     l_ref, p_ref = _run(make_trainer, cpu_backend, steps)
     l_hip, p_hip = _run(make_trainer, hip_backend, steps)
     assert np.isfinite(l_ref).all() and np.isfinite(l_hip).all()
-    np.testing.assert_allclose(l_hip, l_ref, rtol=2 * tol, atol=1e-6, err_msg="loss trajectory")
+    if loss_late is None:
+        np.testing.assert_allclose(l_hip, l_ref, rtol=2 * tol, atol=1e-6, err_msg="loss trajectory")
+    else:       # a trajectory that amplifies rounding differences: tight over the first half, `loss_late` afterwards
+        h = steps // 2
+        np.testing.assert_allclose(l_hip[:h], l_ref[:h], rtol=2 * tol, atol=1e-6, err_msg="loss trajectory, first half")
+        np.testing.assert_allclose(l_hip[h:], l_ref[h:], rtol=loss_late, atol=1e-6, err_msg="loss trajectory, second half")
     assert l_ref[-1] != l_ref[0], "training did not move the loss"
     A = np.concatenate([a.ravel() for _, a in p_hip]).astype(np.float64)
     B = np.concatenate([b.ravel() for _, b in p_ref]).astype(np.float64)
@@ -90,7 +95,10 @@ def test_resnet_imagenet_stem_3_steps(hip_backend, cpu_backend):
 def test_squeezenet_10_steps(hip_backend, cpu_backend):
     """All 26 biased convs, 8 concats, 3 max-pools, momentum SGD (the reference's configuration but batch 16)."""
     from lantern_amd.apps.squeezenet import Trainer
-    _compare(lambda: Trainer(batch=16, lr=0.001), hip_backend, cpu_backend, per_tensor=5e-3)
+    # The device's filter gradients and stream-K tiles are combined with fp32 atomic adds, so two device runs differ by
+    # rounding; this program (relu and max-pool argmax flips, momentum) amplifies that about threefold per step: the loss
+    # of step 1 agrees to 3e-7, and ten device runs against the oracle ended between 2e-5 and 2.7e-3 at step 10.
+    _compare(lambda: Trainer(batch=16, lr=0.001), hip_backend, cpu_backend, per_tensor=5e-3, loss_late=1e-2)
 
 
 def test_squeezenet_avgpool_head_5_steps(hip_backend, cpu_backend):
