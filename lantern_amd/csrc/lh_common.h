@@ -18,6 +18,7 @@ static inline hipStream_t ordered_stream() { if (g_rec_pending) rec_flush(); ret
 #define g_stream (::lh::ordered_stream())     // every kernel is enqueued here
 extern int g_error_mode;         // 0 = print and exit, 1 = record and return
 extern int g_num_cu;             // compute units of the device in use
+extern bool g_tune;              // launch plans are measured on first use (lh_set_tuning; off with LH_NO_TUNE in the environment)
 
 // Records (mode 1) or prints and exits (mode 0).  Returns true so callers can `return` on it.
 bool fail(const char* file, int line, const char* fmt, ...);

@@ -20,30 +20,7 @@ struct BwdfKey {
 };
 struct BwdfPlan { int bm, bn, split; };
 static std::map<BwdfKey, BwdfPlan> g_bwdf_split;
-static bool g_bwdf_tune = getenv("LH_NO_TUNE") == nullptr;      // lh_set_tuning
 
-// Times `launch` (a callable returning false on failure) on the library's stream: three repetitions, the first warms
-// the caches, the smaller of the other two counts.  Returns a negative number when a launch or the timer failed.
-struct LaunchTimer {
-  hipEvent_t e0 = nullptr, e1 = nullptr;
-  bool ok;
-  LaunchTimer() { ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess; }
-  ~LaunchTimer() { if (e0) (void)hipEventDestroy(e0); if (e1) (void)hipEventDestroy(e1); }
-  template <class F>
-  float ms(F launch) {
-    float best = 3.0e38f;
-    for (int rep = 0; rep < 3; rep++) {
-      (void)hipEventRecord(e0, g_stream);
-      if (!launch()) return -1.f;
-      (void)hipEventRecord(e1, g_stream);
-      if (hipEventSynchronize(e1) != hipSuccess) return -1.f;
-      float t = 0.f;
-      if (hipEventElapsedTime(&t, e0, e1) != hipSuccess) return -1.f;
-      if (rep > 0 && t < best) best = t;
-    }
-    return best;
-  }
-};
 constexpr int TPB = 256;
 
 struct ConvDims { int N, C, H, W, K, R, S, sH, sW, pH, pW, P, Q; };
@@ -402,7 +379,7 @@ template <class AL, class BL, class EP>
 static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out = nullptr, int64_t zero_n = 0, bool prezeroed = false) {
   static std::map<PlanKey, int> chosen;
   const bool can_zero = zero_out != nullptr || prezeroed;
-  if (!g_bwdf_tune || 2.0 * M * N * (double)K < 2e8) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  if (!g_tune || 2.0 * M * N * (double)K < 2e8) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   const PlanKey key = {{M, N, K, ep.eH, ep.eW, ep.W, ep.PIX}};
   auto it = chosen.find(key);
   if (it != chosen.end()) {
@@ -500,7 +477,7 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
       // repeating it is harmless) and remembered
       static std::map<PlanKey, int> chosen;
       const PlanKey key = {{K, N * PQ, CRS, H, W, sH, R}};
-      const bool tunable = g_bwdf_tune && 2.0 * K * CRS * (double)N * PQ >= 2e8;
+      const bool tunable = g_tune && 2.0 * K * CRS * (double)N * PQ >= 2e8;
       int force = 0;
       auto run = [&](int f) {           // 0: the rule's tile, 1-3: a forced tile, 4: unfused (any launch plan, then a pass over y)
         if (f == 4) {
@@ -569,8 +546,6 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
 }
 
 extern "C" {
-
-void lh_set_tuning(int on) { g_bwdf_tune = on != 0; }
 
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
@@ -658,7 +633,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
         int tile = tp.bm == 128 ? 1 : (tp.bn == 128 ? 2 : 3);
         auto it = chosen.find(key);
         if (it != chosen.end()) tile = it->second;
-        else if (g_bwdf_tune && beta == 0.f && 2.0 * C * (double)ntot * kmax >= 2e8) {
+        else if (g_tune && beta == 0.f && 2.0 * C * (double)ntot * kmax >= 2e8) {
           LaunchTimer timer;
           if (timer.ok) {
             float best_ms = 3.0e38f; int best = tile;
@@ -756,7 +731,7 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   // How many slices pays best depends on how tiles x slices fall onto the resident block slots and on how short the
   // per-block reduction gets; it is measured once per shape (a few candidates on a scratch output) and remembered.
   const BwdfKey key = {{N, C, H, W, K, R, S, sH, sW, pH, pW}};
-  const bool tunable = g_bwdf_tune && max_split > 1 && 2.0 * K * CRS * (double)red >= 2e8;
+  const bool tunable = g_tune && max_split > 1 && 2.0 * K * CRS * (double)red >= 2e8;
   bool tune_now = false;
   if (tunable) {
     auto it = g_bwdf_split.find(key);

@@ -1,6 +1,8 @@
 // Dense linear algebra outside convolution: sgemm (all four transpose cases), sgemv, rank-1
 // update and vector dot.  Row-major, fp32.
 #include "lh_igemm.h"
+#include <array>
+#include <map>
 using namespace lh;
 
 namespace {
@@ -149,12 +151,6 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   LH_REQUIRE(lda >= (ta ? m : k) && ldb >= (tb ? k : n) && ldc >= n, "lh_sgemm: leading dimensions (%d,%d,%d) too small for m%d n%d k%d ta%d tb%d", lda, ldb, ldc, m, n, k, ta, tb);
   LH_REQUIRE(A && B && C, "lh_sgemm: null operand");
   if ((int64_t)m * n * k >= (1 << 18) && m >= 16 && n >= 16) {
-    EpiRowMajor ep; ep.C = C; ep.ldc = ldc; ep.alpha = alpha; ep.beta = beta; ep.atomic = 0;
-    const SgemmPlan pl = sgemm_plan(m, n, k);
-    if (pl.split > 1) {
-      if (beta != 1.f) { hipLaunchKernelGGL(k_scale_rows, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, C, ldc, m, n, beta); LH_CHECK_LAUNCH(); }
-      ep.atomic = 1; ep.beta = 1.f;
-    }
     const bool av = (lda % 4 == 0) && (((uintptr_t)A & 15) == 0) && (k % 4 == 0);
     const bool bv = (ldb % 4 == 0) && (((uintptr_t)B & 15) == 0) && (k % 4 == 0);
     const size_t abytes = (size_t)(ta ? k : m) * lda * 4, bbytes = (size_t)(tb ? n : k) * ldb * 4;
@@ -165,12 +161,61 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
     LoadPlainK<true> bkv; bkv.base = B; bkv.nbytes = (uint32_t)bbytes; bkv.ld = ldb;
     LoadPlainK<false> bks; bks.base = B; bks.nbytes = (uint32_t)bbytes; bks.ld = ldb;
     LoadPlainT bt; bt.base = B; bt.nbytes = (uint32_t)bbytes; bt.ld = ldb;
-    bool ok;
-    if (!ta && !tb) ok = av ? sgemm_mfma(akv, bt, ep, m, n, k, pl) : sgemm_mfma(aks, bt, ep, m, n, k, pl);
-    else if (!ta && tb) ok = av ? (bv ? sgemm_mfma(akv, bkv, ep, m, n, k, pl) : sgemm_mfma(akv, bks, ep, m, n, k, pl))
-                                : (bv ? sgemm_mfma(aks, bkv, ep, m, n, k, pl) : sgemm_mfma(aks, bks, ep, m, n, k, pl));
-    else if (ta && !tb) ok = sgemm_mfma(at, bt, ep, m, n, k, pl);
-    else ok = bv ? sgemm_mfma(at, bkv, ep, m, n, k, pl) : sgemm_mfma(at, bks, ep, m, n, k, pl);
+    // one product under plan `pl` into Cout (row stride ldo) with the given beta
+    auto run = [&](const SgemmPlan& pl, float* Cout, int ldo, float be) -> bool {
+      EpiRowMajor e; e.C = Cout; e.ldc = ldo; e.alpha = alpha; e.beta = be; e.atomic = 0;
+      if (pl.split > 1) {
+        if (be != 1.f) { hipLaunchKernelGGL(k_scale_rows, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, Cout, ldo, m, n, be); }
+        e.atomic = 1; e.beta = 1.f;
+      }
+      if (!ta && !tb) return av ? sgemm_mfma(akv, bt, e, m, n, k, pl) : sgemm_mfma(aks, bt, e, m, n, k, pl);
+      if (!ta && tb) return av ? (bv ? sgemm_mfma(akv, bkv, e, m, n, k, pl) : sgemm_mfma(akv, bks, e, m, n, k, pl))
+                               : (bv ? sgemm_mfma(aks, bkv, e, m, n, k, pl) : sgemm_mfma(aks, bks, e, m, n, k, pl));
+      if (ta && !tb) return sgemm_mfma(at, bt, e, m, n, k, pl);
+      return bv ? sgemm_mfma(at, bkv, e, m, n, k, pl) : sgemm_mfma(at, bks, e, m, n, k, pl);
+    };
+    SgemmPlan pl = sgemm_plan(m, n, k);
+    // Tile shape and reduction slices are measured once per (transposes, m, n, k) on a scratch output and remembered.
+    static std::map<std::array<int, 7>, SgemmPlan> chosen;
+    if (g_tune && 2.0 * m * n * (double)k >= 2e8) {
+      const std::array<int, 7> key = {ta, tb, m, n, k, (int)av, (int)bv};
+      auto it = chosen.find(key);
+      if (it != chosen.end()) pl = it->second;
+      else {
+        const size_t sbytes = (size_t)m * n * sizeof(float);
+        float* scratch = (float*)lh_malloc_uninit(sbytes);
+        LaunchTimer timer;
+        if (scratch && timer.ok) {
+          const TilePick shapes[3] = {{128, 128}, {64, 128}, {64, 64}};
+          const double targets[] = {1.5, 3.0, 4.5};
+          float best_ms = timer.ms([&]() { return run(pl, scratch, n, 0.f); });
+          SgemmPlan best = pl;
+          for (int sh = 0; sh < 3 && best_ms >= 0.f && !failed(); sh++) {
+            if ((shapes[sh].bm == 128 && m <= 64) || (shapes[sh].bn == 128 && n <= 64)) continue;
+            const int64_t tiles = cdiv(m, shapes[sh].bm) * cdiv(n, shapes[sh].bn);
+            int cand[4] = {1, 0, 0, 0}; int nc = 1;
+            for (double tg : targets) {
+              int sp = (int)((int64_t)(tg * g_num_cu) / tiles);
+              if (sp > k / 256) sp = k / 256;
+              bool dup = sp <= 1;
+              for (int i = 0; i < nc; i++) dup = dup || cand[i] == sp;
+              if (!dup) cand[nc++] = sp;
+            }
+            for (int i = 0; i < nc; i++) {
+              SgemmPlan c; c.tp = shapes[sh]; c.split = cand[i];
+              const float ms = timer.ms([&]() { return run(c, scratch, n, 0.f); });
+              if (ms < 0.f) { best_ms = -1.f; break; }
+              if (ms < best_ms * 0.98f) { best_ms = ms; best = c; }
+            }
+          }
+          if (best_ms >= 0.f && !failed()) { chosen[key] = best; pl = best; }
+          if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "sgemm ta%d tb%d %dx%dx%d: tile %dx%d, %d slice(s), %.3f ms\n", ta, tb, m, n, k, best.tp.bm, best.tp.bn, best.split, best_ms);
+        }
+        if (scratch) lh_free_top(sbytes);
+        if (failed()) return;
+      }
+    }
+    const bool ok = run(pl, C, ldc, beta);
     if (!ok) return;
     LH_CHECK_LAUNCH();
     return;

@@ -420,6 +420,29 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
   return true;
 }
 
+// Times `launch` (a callable returning false on failure) on the library's stream: three repetitions, the first warms
+// the caches, the smaller of the other two counts.  Returns a negative number when a launch or the timer failed.
+struct LaunchTimer {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  bool ok;
+  LaunchTimer() { ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess; }
+  ~LaunchTimer() { if (e0) (void)hipEventDestroy(e0); if (e1) (void)hipEventDestroy(e1); }
+  template <class F>
+  float ms(F launch) {
+    float best = 3.0e38f;
+    for (int rep = 0; rep < 3; rep++) {
+      (void)hipEventRecord(e0, g_stream);
+      if (!launch()) return -1.f;
+      (void)hipEventRecord(e1, g_stream);
+      if (hipEventSynchronize(e1) != hipSuccess) return -1.f;
+      float t = 0.f;
+      if (hipEventElapsedTime(&t, e0, e1) != hipSuccess) return -1.f;
+      if (rep > 0 && t < best) best = t;
+    }
+    return best;
+  }
+};
+
 // One launch for up to IGEMM_MAX_GROUPS products that share loaders and tile shape (plain tiles: no k-split, no stream-K).
 template <int BM, int BN, int BK, class AL, class BL, class EP>
 bool igemm_launch_grouped(int ngroups, const AL* al, const BL* bl, const EP* ep, const int* M, const int* N, const int* K) {

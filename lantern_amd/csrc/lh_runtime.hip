@@ -8,6 +8,7 @@
 
 namespace lh {
 hipStream_t g_stream_raw = nullptr;
+bool g_tune = getenv("LH_NO_TUNE") == nullptr;
 int g_error_mode = 0;
 int g_num_cu = 256;
 static char g_err[1024] = "";
@@ -72,6 +73,7 @@ using namespace lh;
 extern "C" {
 
 void lh_set_error_mode(int mode) { g_error_mode = mode; }
+void lh_set_tuning(int on) { g_tune = on != 0; }
 const char* lh_last_error(void) { return g_err; }
 void lh_clear_error(void) { g_err[0] = 0; }
 
