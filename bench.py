@@ -181,7 +181,7 @@ def main():
                 "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
                 # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this workload (see profiles/), not measured live
-                "traffic": 160.1e6 if args.workload == "resnet50" and args.batch == 64 and args.hw == 224 else None, "flop_per_step": conv_fl,
+                "traffic": 150.8e6 if args.workload == "resnet50" and args.batch == 64 and args.hw == 224 else None, "flop_per_step": conv_fl,
                 "ms_per_step": {"fwd": round(conv_ms[0], 3), "bwd_data": round(conv_ms[1], 3), "bwd_filter": round(conv_ms[2], 3)}}
         if work.get("gemm_flop", 0.0) > 0 and timed["gemm"][0] > 0:
             roof["gemm"] = {"flop_per_step": work["gemm_flop"], "ms_per_step": round(timed["gemm"][0], 3),
