@@ -281,15 +281,17 @@ __global__ void __launch_bounds__(TPB) k_filter_transpose(const float* __restric
     wt[i] = w[((int64_t)k * C + c) * RS + rs];
   }
 }
-// db[k] += sum over n, p, q of dy: one block per k
-__global__ void __launch_bounds__(TPB) k_conv_bwd_bias(const float* __restrict__ dy, float* db, int N, int K, int PQ) {
+// db[k] += sum over n, p, q of dy: block (k, slice of the batch); slices add their sums atomically
+__global__ void __launch_bounds__(TPB) k_conv_bwd_bias(const float* __restrict__ dy, float* db, int N, int K, int PQ, int n_per) {
   __shared__ float sm[17];
-  int k = blockIdx.x;
+  const int k = blockIdx.x, n0 = blockIdx.y * n_per, n1 = min(N, n0 + n_per);
   float acc = 0.f;
-  int64_t tot = (int64_t)N * PQ;
-  for (int64_t j = threadIdx.x; j < tot; j += TPB) { int n = (int)(j / PQ); int l = (int)(j - (int64_t)n * PQ); acc += dy[((int64_t)n * K + k) * PQ + l]; }
+  for (int n = n0; n < n1; n++) {
+    const float* p = dy + ((int64_t)n * K + k) * PQ;
+    for (int l = threadIdx.x; l < PQ; l += TPB) acc += p[l];
+  }
   acc = lh_block_sum(acc, sm);
-  if (threadIdx.x == 0) db[k] += acc;
+  if (threadIdx.x == 0) atomicAdd(db + k, acc);
 }
 
 #ifndef LH_CONV_BK
@@ -807,7 +809,13 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   }
   dispatch();
   if (!ok) return;
-  if (db) hipLaunchKernelGGL(k_conv_bwd_bias, dim3(K), dim3(TPB), 0, g_stream, dy, db, N, K, PQ);
+  if (db) {
+    int slices = (int)cdiv(2 * (int64_t)g_num_cu, K);
+    if (slices > N) slices = N;
+    if (slices < 1) slices = 1;
+    const int n_per = (int)cdiv(N, slices);
+    hipLaunchKernelGGL(k_conv_bwd_bias, dim3(K, (unsigned)cdiv(N, n_per)), dim3(TPB), 0, g_stream, dy, db, N, K, PQ, n_per);
+  }
   LH_CHECK_LAUNCH();
 }
 
