@@ -68,13 +68,24 @@ def run_gpu(args):
     for _ in range(args.warmup):
         tr.step(); tr.end_step()
     be.sync()
-    # the timed region: exactly `steps` steps, nothing else on the stream
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        tr.step()
-        tr.end_step()
-    be.sync()
-    t1 = time.perf_counter()
+    if args.graph:
+        # the step recorded once (after the warm-up measured the launch plans) and replayed: one host call per step
+        g = la.StepGraph(tr, eager_steps=0)
+        g.launch(); be.sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            g.launch()
+        be.sync()
+        t1 = time.perf_counter()
+        g.close()
+    else:
+        # the timed region: exactly `steps` steps, nothing else on the stream
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            tr.step()
+            tr.end_step()
+        be.sync()
+        t1 = time.perf_counter()
     # the same `steps` steps again with a HIP event pair around every matrix-kernel launch (conv x3, gemm, rnn).
     # Kept out of the timed region: an event between two launches drains the pipeline and costs about 1 ms per step.
     # (a program that runs from the command list times only the interpreter launches: an event elsewhere would cut the list short)
@@ -151,6 +162,7 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="time replays of the step recorded into a HIP graph (fixed-shape workloads)")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -195,7 +207,8 @@ def main():
         "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": g["desc"], "global_batch": args.batch, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2)},
+        "config": {"workload": g["desc"], "global_batch": args.batch, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
+                   "launch": "hip graph replay" if args.graph else "one launch per kernel"},
         "roofline": roof,
     }
     if args.verbose:

@@ -82,6 +82,19 @@ enum { LH_CAT_CONV_FWD = 0, LH_CAT_CONV_BWD_DATA, LH_CAT_CONV_BWD_FILTER, LH_CAT
        LH_CAT_ELEMENTWISE, LH_CAT_POOL, LH_CAT_REDUCE, LH_CAT_OPTIM, LH_CAT_FILL, LH_CAT_COUNT };
 void lh_prof_enable(unsigned mask);
 
+/* HIP graph of a whole step, for programs whose kernels are shorter than their launches (LeNet, SqueezeNet on 32x32
+ * images: several hundred launches of a few microseconds per step; the reference pays a launch per operator, CUB:171-560).
+ * lh_capture_begin() switches the library's stream to capture: every entry point called until lh_capture_end() is
+ * recorded instead of run (entry points that wait for the device -- lh_sync, lh_h2d, lh_d2h -- are errors there, and
+ * launch plans are not measured, so run the step a few times first).  lh_capture_end() returns a handle;
+ * lh_graph_launch(handle) enqueues the recorded step again.  The step must be replayable as recorded: the same arena
+ * addresses (rewind to the same mark before capturing and after), inputs refreshed in place, parameters updated in place
+ * by the recorded optimizer.  No memset nodes are recorded: the library clears memory with kernels. */
+void lh_capture_begin(void);
+int lh_capture_end(void);
+void lh_graph_launch(int graph);
+void lh_graph_destroy(int graph);
+
 /* Command list for launch-bound programs (the sentiment TreeLSTM, SentimentTreeLSTM.scala:242-318, issues about
  * 5000 operator calls on 150-element vectors per tree; the reference pays one cuBLAS / kernel launch for each,
  * CUB:171-560).  Between lh_cmdlist_begin and lh_cmdlist_end every entry point of this header whose operands are

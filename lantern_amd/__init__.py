@@ -7,3 +7,4 @@ written against, with the names of the reference's TensorDifferentiation.scala.
 from .backend import BackendHIP, Backend, Buf                      # noqa: F401
 from .tensor import (Tensor, TensorR, Random, gradR, gradR_loss,  # noqa: F401
                      set_backend, get_backend, int_array)
+from .graph import StepGraph                                       # noqa: F401

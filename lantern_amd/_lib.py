@@ -35,6 +35,10 @@ SIGNATURES = {
     "lh_event_destroy": (None, [P]),
     "lh_prof_enable": (None, [C.c_uint]),
     "lh_set_tuning": (None, [I]),
+    "lh_capture_begin": (None, []),
+    "lh_capture_end": (I, []),
+    "lh_graph_launch": (None, [I]),
+    "lh_graph_destroy": (None, [I]),
     "lh_cmdlist_begin": (None, []),
     "lh_cmdlist_end": (None, []),
     "lh_cmdlist_stats": (None, [C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),

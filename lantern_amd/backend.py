@@ -170,6 +170,20 @@ class BackendHIP(Backend):
     def sync(self):
         self.lib.lh_sync(); _lib.check()
 
+    def captureBegin(self):
+        """Record everything issued until captureEnd() into a HIP graph instead of running it."""
+        self.lib.lh_capture_begin(); _lib.check()
+
+    def captureEnd(self):
+        g = self.lib.lh_capture_end(); _lib.check()
+        return g
+
+    def graphLaunch(self, g):
+        self.lib.lh_graph_launch(g); _lib.check()
+
+    def graphDestroy(self, g):
+        self.lib.lh_graph_destroy(g); _lib.check()
+
     def batchSmallOps(self, on=True):
         """Record small operations into the library's command list instead of launching each (launch-bound programs)."""
         (self.lib.lh_cmdlist_begin if on else self.lib.lh_cmdlist_end)(); _lib.check()

@@ -304,6 +304,7 @@ void cmdlist_release() {
 extern "C" {
 void lh_cmdlist_begin(void) {
   LH_REQUIRE(g_stream_raw != nullptr, "lh_cmdlist_begin before lh_setup");
+  LH_REQUIRE(!g_capturing, "lh_cmdlist_begin: a graph is being recorded (the command buffers cannot be replayed)");
   if (!ring_init()) return;
   g_rec_on = 1;
 }

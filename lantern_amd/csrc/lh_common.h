@@ -18,7 +18,16 @@ static inline hipStream_t ordered_stream() { if (g_rec_pending) rec_flush(); ret
 #define g_stream (::lh::ordered_stream())     // every kernel is enqueued here
 extern int g_error_mode;         // 0 = print and exit, 1 = record and return
 extern int g_num_cu;             // compute units of the device in use
-extern bool g_tune;              // launch plans are measured on first use (lh_set_tuning; off with LH_NO_TUNE in the environment)
+extern bool g_tune_enabled;      // launch plans are measured on first use (lh_set_tuning; off with LH_NO_TUNE in the environment)
+extern bool g_capturing;         // between lh_capture_begin and lh_capture_end: work is recorded into a HIP graph, nothing may wait on the stream
+#define g_tune (::lh::g_tune_enabled && !::lh::g_capturing)
+// Dropout draws from a counter-based stream whose position the caller passes per launch.  A replayed graph repeats its
+// launch arguments, so a captured dropout adds *g_capture_advance (device memory; 0 for the first replay, advanced at the
+// end of every replay by the g_capture_drawn positions the recorded step used) to the position it was recorded with.
+// Entry points that wait for the device refuse to run while a graph is recorded (the wait would invalidate the capture).
+#define LH_NOT_CAPTURING(what) LH_REQUIRE(!::lh::g_capturing, "%s waits for the device, which a graph being recorded cannot do (lh_capture_end first)", what)
+extern unsigned long long* g_capture_advance;
+extern unsigned long long g_capture_drawn;
 
 // Records (mode 1) or prints and exits (mode 0).  Returns true so callers can `return` on it.
 bool fail(const char* file, int line, const char* fmt, ...);

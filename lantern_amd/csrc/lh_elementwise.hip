@@ -490,7 +490,9 @@ __device__ __forceinline__ float ctr_uniform(uint64_t seed, uint64_t index) {
   z = z ^ (z >> 31);
   return (float)(z >> 40) * (1.0f / 16777216.0f);
 }
-__global__ void __launch_bounds__(TPB) k_dropout(const float* x, float* y, float* mask, int64_t n, float p, float scale, uint64_t seed, uint64_t offset) {
+__global__ void __launch_bounds__(TPB) k_dropout(const float* x, float* y, float* mask, int64_t n, float p, float scale, uint64_t seed, uint64_t offset,
+                                                 const unsigned long long* advance) {
+  if (advance) offset += *advance;      // a replayed graph: positions move on by what the earlier replays drew
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
   for (; i < n; i += st) {
     bool keep = ctr_uniform(seed, offset + (uint64_t)i) > p;
@@ -501,7 +503,9 @@ __global__ void __launch_bounds__(TPB) k_dropout(const float* x, float* y, float
 void lh_dropout_fwd(const float* x, float* y, float* mask, int64_t n, float p, uint64_t seed, uint64_t offset) {
   LH_REQUIRE(p >= 0.f && p < 1.f, "dropout rate should be [0.0, 1), got %f", p);
   if (n <= 0) return;
-  hipLaunchKernelGGL(k_dropout, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, mask, n, p, 1.0f / (1.0f - p), seed, offset);
+  hipLaunchKernelGGL(k_dropout, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, mask, n, p, 1.0f / (1.0f - p), seed, offset,
+                     g_capturing ? (const unsigned long long*)g_capture_advance : (const unsigned long long*)nullptr);
+  if (g_capturing) g_capture_drawn += (unsigned long long)n;
   LH_CHECK_LAUNCH();
 }
 void lh_dropout_bwd(const float* dy, const float* mask, float* dx, int64_t n) {
@@ -616,6 +620,7 @@ static void multi_update(int mode, int count, float* const* hx, float* const* hd
   for (int t = 0; t < count; t++) { mix((uint64_t)(uintptr_t)hx[t]); mix((uint64_t)(uintptr_t)hd[t]); mix(hv ? (uint64_t)(uintptr_t)hv[t] : 0); mix((uint64_t)hn[t]); }
   mix((uint64_t)mode);
   if (g_mt.dev == nullptr || g_mt.key != key || g_mt.count != count) {
+    LH_NOT_CAPTURING("the first multi-tensor update of a parameter set (its table is uploaded)");
     MtEntry* host = (MtEntry*)malloc(sizeof(MtEntry) * count);
     int64_t chunks = 0;
     for (int t = 0; t < count; t++) { host[t] = {hx[t], hd[t], hv ? hv[t] : nullptr, hn[t], chunks}; chunks += cdiv(hn[t] > 0 ? hn[t] : 1, MT_CHUNK); }

@@ -8,7 +8,12 @@
 
 namespace lh {
 hipStream_t g_stream_raw = nullptr;
-bool g_tune = getenv("LH_NO_TUNE") == nullptr;
+bool g_tune_enabled = getenv("LH_NO_TUNE") == nullptr;
+bool g_capturing = false;
+unsigned long long* g_capture_advance = nullptr;
+unsigned long long g_capture_drawn = 0;
+static unsigned long long* g_advance_pool = nullptr;   // one counter per graph
+constexpr int MAX_GRAPHS = 256;
 int g_error_mode = 0;
 int g_num_cu = 256;
 static char g_err[1024] = "";
@@ -56,6 +61,8 @@ void prof_end(int cat) {
   }
 }
 
+static std::vector<hipGraphExec_t> g_graphs;
+__global__ void k_set_u64(unsigned long long* p, unsigned long long keep, unsigned long long add) { *p = (keep ? *p : 0ull) + add; }
 __global__ void k_zero16(uint4* p, size_t n16) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, st = (size_t)gridDim.x * blockDim.x;
   for (; i < n16; i += st) p[i] = make_uint4(0, 0, 0, 0);
@@ -73,7 +80,7 @@ using namespace lh;
 extern "C" {
 
 void lh_set_error_mode(int mode) { g_error_mode = mode; }
-void lh_set_tuning(int on) { g_tune = on != 0; }
+void lh_set_tuning(int on) { g_tune_enabled = on != 0; }
 const char* lh_last_error(void) { return g_err; }
 void lh_clear_error(void) { g_err[0] = 0; }
 
@@ -89,17 +96,23 @@ void lh_setup(size_t heap_bytes) {
   heap_bytes = (heap_bytes + 255) & ~(size_t)255;
   LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
   g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0; g_zero_end = 0;
+  LH_HIP(hipMalloc((void**)&g_advance_pool, MAX_GRAPHS * sizeof(unsigned long long)));
 }
 
 void lh_cleanup(void) {
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
   cmdlist_release();
+  for (auto& e : g_graphs) if (e) { (void)hipGraphExecDestroy(e); e = nullptr; }
+  g_graphs.clear(); g_capturing = false;
+  if (g_advance_pool) (void)hipFree(g_advance_pool);
+  g_advance_pool = nullptr; g_capture_advance = nullptr;
   if (g_heap) (void)hipFree(g_heap);
   if (g_stream_raw) (void)hipStreamDestroy(g_stream_raw);
   g_heap = nullptr; g_stream_raw = nullptr; g_heap_bytes = g_top = g_zero_end = 0;
 }
 
 void lh_sync(void) {
+  LH_NOT_CAPTURING("lh_sync");
   LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH();
 }
 
@@ -145,16 +158,61 @@ size_t lh_heap_peak(void) { return g_peak; }
 
 void lh_h2d(void* dst, const void* h_src, size_t bytes) {
   // Pageable source: the copy is staged before the call returns, so the host buffer may be reused.
+  LH_NOT_CAPTURING("lh_h2d");
   LH_HIP(hipMemcpyAsync(dst, h_src, bytes, hipMemcpyHostToDevice, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
 }
 void lh_d2h(void* h_dst, const void* src, size_t bytes) {
+  LH_NOT_CAPTURING("lh_d2h");
   LH_HIP(hipMemcpyAsync(h_dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
 }
 void lh_d2d(void* dst, const void* src, size_t bytes) {
   if ((bytes & 3) == 0 && bytes > 0 && rec_ok((int64_t)(bytes / 4))) { rec_cmd(CL_COPY, (int)(bytes / 4), 0, 0, 0.f, 0.f, 0.f, 0.f, dst, src, nullptr, nullptr); return; }
   LH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+}
+
+// ---- HIP graphs: a launch-bound step recorded once and replayed ----------------------------------------------
+void lh_capture_begin(void) {
+  LH_REQUIRE(g_stream_raw != nullptr, "lh_capture_begin before lh_setup");
+  LH_REQUIRE(!g_capturing, "lh_capture_begin: already capturing");
+  LH_REQUIRE(!g_rec_on, "lh_capture_begin: the command list is recording (its buffers cannot be replayed)");
+  LH_REQUIRE(g_prof_mask == 0, "lh_capture_begin: per-category timing is on");
+  LH_REQUIRE((int)g_graphs.size() < MAX_GRAPHS, "lh_capture_begin: %d graphs exist already", MAX_GRAPHS);
+  g_capture_advance = g_advance_pool + g_graphs.size(); g_capture_drawn = 0;
+  hipLaunchKernelGGL(k_set_u64, dim3(1), dim3(1), 0, g_stream, g_capture_advance, 0ull, 0ull);
+  LH_CHECK_LAUNCH();
+  LH_HIP(hipStreamBeginCapture(g_stream_raw, hipStreamCaptureModeThreadLocal));
+  g_capturing = true;
+}
+int lh_capture_end(void) {
+  if (!g_capturing) { LH_FAIL("lh_capture_end without lh_capture_begin"); return -1; }
+  if (g_capture_drawn) hipLaunchKernelGGL(k_set_u64, dim3(1), dim3(1), 0, g_stream_raw, g_capture_advance, 1ull, g_capture_drawn);
+  g_capturing = false;
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(g_stream_raw, &graph);
+  if (e != hipSuccess || graph == nullptr) {
+    (void)hipGetLastError();      // the capture is over; its error must not be reported by the next launch
+    LH_FAIL("hipStreamEndCapture: %s (an entry point that waits for the device was called during capture?); lh_cleanup and lh_setup give a fresh stream", hipGetErrorString(e));
+    return -1;
+  }
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) { LH_FAIL("hipGraphInstantiate: %s", hipGetErrorString(e)); return -1; }
+  g_graphs.push_back(exec);
+  return (int)g_graphs.size() - 1;
+}
+void lh_graph_launch(int id) {
+  LH_REQUIRE(id >= 0 && id < (int)g_graphs.size() && g_graphs[id] != nullptr, "lh_graph_launch: no graph %d", id);
+  LH_HIP(hipGraphLaunch(g_graphs[id], g_stream));
+}
+void lh_graph_destroy(int id) {
+  LH_REQUIRE(id >= 0 && id < (int)g_graphs.size() && g_graphs[id] != nullptr, "lh_graph_destroy: no graph %d", id);
+  LH_NOT_CAPTURING("lh_graph_destroy");
+  (void)hipStreamSynchronize(g_stream);
+  (void)hipGraphExecDestroy(g_graphs[id]);
+  g_graphs[id] = nullptr;
 }
 
 void lh_prof_enable(unsigned mask) { g_prof_mask = mask; }
@@ -178,6 +236,7 @@ void* lh_event_create(void) {
 void lh_event_record(void* ev) { LH_HIP(hipEventRecord((hipEvent_t)ev, g_stream)); }
 float lh_event_elapsed_ms(void* start, void* stop) {
   float ms = -1.0f;
+  if (g_capturing) { LH_FAIL("lh_event_elapsed_ms waits for the device, which a graph being recorded cannot do"); return ms; }
   if (hipEventSynchronize((hipEvent_t)stop) != hipSuccess || hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)stop) != hipSuccess) {
     LH_FAIL("event timing failed"); return -1.0f;
   }
