@@ -47,7 +47,11 @@ def _oracle_conv(x, w, b, dy, dims, need_dx=True):
 @pytest.mark.parametrize("dims", SHAPES, ids=lambda d: "x".join(map(str, d)))
 @pytest.mark.parametrize("bias", [False, True], ids=["nobias", "bias"])
 def test_conv_fwd_bwd(on_hip, dims, bias):
-    dev = Dev(on_hip)
+    check_conv(Dev(on_hip), dims, bias)
+
+
+def check_conv(dev, dims, bias):
+    """Forward, input gradient and filter (+ bias) gradient of one geometry against the oracle, overwrite and accumulate forms."""
     N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
     P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
     rng = np.random.RandomState(hash(dims) % (2 ** 31))

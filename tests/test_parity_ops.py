@@ -36,6 +36,29 @@ def pair(cpu_backend, on_hip):
     return Pair(cpu_backend, on_hip)
 
 
+def _random_cases(seed, n, gen):
+    """Seeded random geometries appended to the hand-picked tables below: the named cases say which paths the kernels
+    take, these look for the ones nobody thought of (the ids in the test report give the geometry)."""
+    rng = np.random.RandomState(seed)
+    return [gen(rng) for _ in range(n)]
+
+
+def _ri(rng, lo, hi): return int(rng.randint(lo, hi + 1))
+def _pick(rng, xs): return xs[int(rng.randint(len(xs)))]
+
+
+def _gen_pool(rng):
+    kH, kW = _ri(rng, 2, 5), _ri(rng, 2, 5)
+    if rng.rand() < 0.6: kW = kH
+    pad = _ri(rng, 0, min(kH, kW) // 2)
+    return (_ri(rng, 1, 4), _ri(rng, 1, 9), _ri(rng, kH, 40), _ri(rng, kW, 40), kH, kW, _ri(rng, 1, 3), _ri(rng, 1, 3), pad)
+
+
+def _gen_perm(rng):
+    rank = _ri(rng, 2, 4)
+    return (tuple(_ri(rng, 1, 9) for _ in range(rank)), tuple(int(v) for v in rng.permutation(rank)))
+
+
 def check_all(outs, rtol=1e-4, exact=()):
     want, got = outs
     assert len(want) == len(got)
@@ -48,6 +71,7 @@ def check_all(outs, rtol=1e-4, exact=()):
 
 # ---- batch norm --------------------------------------------------------------------------------------
 BN_SHAPES = [(64, 64, 56 * 56), (8, 256, 56 * 56), (16, 512, 28 * 28), (32, 2048, 49), (4, 24, 7), (3, 5, 1), (1, 16, 100), (20, 33, 1), (64, 1024, 1)]
+BN_SHAPES += _random_cases(101, 10, lambda r: (_ri(r, 2, 20), _ri(r, 1, 70), _pick(r, [1, 2, 7, 49, 100, 196, 333, 1023])))
 
 
 @pytest.mark.parametrize("shape", BN_SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -125,6 +149,9 @@ POOLS = [(64, 64, 112, 112, 3, 3, 2, 2, 1),     # ResNet stem
          (2, 2, 70, 70, 3, 3, 2, 2, 1)]          # rows wider than a wavefront
 
 
+POOLS += _random_cases(102, 16, _gen_pool)
+
+
 @pytest.mark.parametrize("p", POOLS, ids=lambda s: "x".join(map(str, s)))
 def test_maxpool_values_argmax_and_grad(pair, p):
     N, Cc, H, W, kH, kW, sH, sW, pad = p
@@ -146,7 +173,8 @@ def test_maxpool_values_argmax_and_grad(pair, p):
     check_all(outs, exact=(0, 1), rtol=1e-5)     # values and indices bit-exact; overlapping windows sum in any order
 
 
-@pytest.mark.parametrize("p", [(64, 2048, 7, 7, 7, 7, 1, 1), (4, 10, 13, 13, 13, 13, 1, 1), (2, 3, 8, 6, 2, 3, 2, 3), (2, 3, 9, 9, 3, 3, 2, 2)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("p", [(64, 2048, 7, 7, 7, 7, 1, 1), (4, 10, 13, 13, 13, 13, 1, 1), (2, 3, 8, 6, 2, 3, 2, 3), (2, 3, 9, 9, 3, 3, 2, 2)]
+                         + [c[:8] for c in _random_cases(103, 8, _gen_pool)], ids=lambda s: "x".join(map(str, s)))
 def test_avgpool_and_grad(pair, p):
     N, Cc, H, W, kH, kW, sH, sW = p
     P, Q = B.conv_size(H, kH, sH), B.conv_size(W, kW, sW)
@@ -245,7 +273,7 @@ def test_transpose_and_grad(pair, rc):
 
 
 @pytest.mark.parametrize("case", [((4, 6, 5), (2, 0, 1)), ((3, 32, 21, 50), (3, 0, 1, 2)), ((2, 3, 4, 5), (0, 2, 3, 1)), ((7, 9), (1, 0)), ((2, 3, 4, 5), (3, 2, 1, 0)),
-                                  ((8, 32, 11, 40), (2, 0, 1, 3))], ids=str)
+                                  ((8, 32, 11, 40), (2, 0, 1, 3))] + _random_cases(104, 8, _gen_perm), ids=str)
 def test_permute_and_grad(pair, case):
     dims, perm = case
     rng = np.random.RandomState(19); x = rng.randn(*dims).astype(np.float32)
@@ -292,7 +320,8 @@ def test_sum_mean_and_grads(pair, n):
     check_all(outs, rtol=2e-4)
 
 
-@pytest.mark.parametrize("oci", [(64, 49, 1), (1, 5, 1), (8, 3, 20), (100, 1, 7), (3, 1000, 1), (2, 64, 3000), (1, 2000, 300), (3, 700, 100), (1, 5920, 1600)])
+@pytest.mark.parametrize("oci", [(64, 49, 1), (1, 5, 1), (8, 3, 20), (100, 1, 7), (3, 1000, 1), (2, 64, 3000), (1, 2000, 300), (3, 700, 100), (1, 5920, 1600)]
+                         + _random_cases(105, 8, lambda r: (_ri(r, 1, 9), _ri(r, 1, 300), _ri(r, 1, 50))))
 def test_sum_dim_and_grad(pair, oci):
     o, d, i = oci
     rng = np.random.RandomState(22); x = rng.randn(o, d, i).astype(np.float32); dy = rng.randn(o, i).astype(np.float32)
@@ -304,7 +333,8 @@ def test_sum_dim_and_grad(pair, oci):
     check_all(pair.run(f))
 
 
-@pytest.mark.parametrize("oci", [(64, 1000, 1), (100, 10, 1), (1, 1, 1), (5, 29, 1), (3, 29, 150), (7, 5000, 1), (2, 3, 1)])
+@pytest.mark.parametrize("oci", [(64, 1000, 1), (100, 10, 1), (1, 1, 1), (5, 29, 1), (3, 29, 150), (7, 5000, 1), (2, 3, 1)]
+                         + _random_cases(106, 6, lambda r: (_ri(r, 1, 40), _ri(r, 1, 600), _pick(r, [1, 1, 1, 7, 33]))))
 @pytest.mark.parametrize("is_log", [0, 1], ids=["softmax", "logsoftmax"])
 def test_softmax_and_grad(pair, oci, is_log):
     o, c, i = oci
@@ -558,7 +588,8 @@ def test_shape_errors_are_reported_not_launched(on_hip):
 
 
 # ---- recurrent layer and CTC (DeepSpeech2 path) ------------------------------------------------------
-@pytest.mark.parametrize("case", [(1, True, 12, 32, 672, 800), (1, True, 6, 8, 96, 1024), (0, False, 5, 3, 7, 37), (1, False, 1, 2, 5, 16), (0, True, 9, 4, 33, 130), (1, True, 4, 5, 20, 300), (0, True, 3, 6, 16, 1100), (1, False, 3, 33, 10, 1030), (1, True, 3, 70, 24, 64)],
+@pytest.mark.parametrize("case", [(1, True, 12, 32, 672, 800), (1, True, 6, 8, 96, 1024), (0, False, 5, 3, 7, 37), (1, False, 1, 2, 5, 16), (0, True, 9, 4, 33, 130), (1, True, 4, 5, 20, 300), (0, True, 3, 6, 16, 1100), (1, False, 3, 33, 10, 1030), (1, True, 3, 70, 24, 64)]
+                         + _random_cases(107, 6, lambda r: (_ri(r, 0, 1), bool(r.rand() < 0.5), _ri(r, 1, 8), _ri(r, 1, 9), _ri(r, 1, 40), _pick(r, [5, 16, 37, 64, 130, 300]))),
                          ids=lambda c: "mode%d_bi%d_T%d_B%d_I%d_H%d" % c)
 def test_rnn_forward_and_backward(pair, case):
     mode, bidir, T, Bn, In, H = case
@@ -623,42 +654,6 @@ def test_ctc_loss_and_gradient(pair, case):
         want = lb[0] * lb[1] * lb[2] + bl[0] * lb[1] * lb[2] + lb[0] * lb[1] * bl[2] + bl[0] * bl[1] * lb[2] + bl[0] * lb[1] * bl[2] + lb[0] * bl[1] * bl[2]
         np.testing.assert_allclose(outs[1][0][0], -np.log(want), rtol=1e-5)
     check_all(outs, rtol=1e-4)
-
-
-# ---- convolution with batch-norm statistics from its epilogue -----------------------------------------
-CONV_BN = [(64, 64, 56, 64, 1, 1, 0, False),      # 64-row GEMM, 64x128 tiles
-           (8, 64, 56, 256, 1, 1, 0, False),      # 128x128 tiles
-           (64, 256, 14, 1024, 1, 1, 0, False),   # 784 tiles: a full round + surplus columns in 64x64 tiles
-           (4, 32, 15, 48, 3, 2, 1, False),       # odd sizes, partial tiles in both directions
-           (2, 16, 9, 24, 3, 1, 1, True),         # with a bias: statistics come from a pass over y
-           (64, 512, 7, 512, 3, 1, 1, False),     # few tiles, long reduction: the shared-tile path, statistics from a pass over y
-           (2, 3, 20, 16, 5, 1, 2, False)]        # channels not a multiple of 16: the general loader, pass over y
-
-
-@pytest.mark.parametrize("case", CONV_BN, ids=lambda c: "N%d_C%d_H%d_K%d_k%d_s%d_p%d_b%d" % c)
-@pytest.mark.parametrize("relu", [False, True], ids=["plain", "relu"])
-def test_conv_with_batchnorm_statistics(pair, case, relu):
-    N, Cc, H, K, k, s, p, with_bias = case
-    P = B.conv_size(H, k, s, p)
-    dims = (N, Cc, H, H, K, k, k, s, s, p, p)
-    rng = np.random.RandomState(33)
-    x = rng.randn(N, Cc, H, H).astype(np.float32); w = (rng.randn(K, Cc, k, k) / np.sqrt(Cc * k * k)).astype(np.float32)
-    bias = (rng.randn(K) * 2).astype(np.float32) if with_bias else None
-    g = (rng.rand(K) + 0.5).astype(np.float32); b = rng.randn(K).astype(np.float32)
-
-    def f(be, up, down):
-        n = N * K * P * P
-        yconv, ybn, sm, si = be.mallocArray(n), be.mallocArray(n), be.mallocArray(K), be.mallocArray(K)
-        rm, rv = up(np.zeros(K, np.float32)), up(np.ones(K, np.float32))
-        be.conv2D_batch_bn_into(up(x), up(w), up(bias) if with_bias else None, yconv, dims, up(g), up(b), rm, rv, ybn, sm, si, relu)
-        return [down(yconv, (N, K, P, P)), down(ybn, (N, K, P, P)), down(sm, (K,)), down(si, (K,)), down(rm, (K,)), down(rv, (K,))]
-
-    outs = pair.run(f)
-    if relu:        # values within rounding of zero may land on either side of the relu
-        edge = np.abs(outs[0][1]) < 2e-5
-        for o in outs:
-            o[1][edge & (np.abs(o[1]) < 4e-5)] = 0.0
-    check_all(outs, rtol=2e-4)
 
 
 # ---- convolution with batch-norm statistics from its epilogue -----------------------------------------

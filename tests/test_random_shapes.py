@@ -1,0 +1,66 @@
+"""Seeded random geometries against the CPU oracle: the hand-picked cases of the other parity files name the paths the
+kernels take; these sweeps look for the ones nobody thought of (partial tiles, odd strides and pads, windows hanging over
+the border, reductions shorter than a tile).  Every case is printed before it runs so that a failure names its geometry."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+from oracle.backend_cpu import load as load_oracle
+from tests.test_parity_conv import check_conv
+from tests.util import Dev, assert_close, cptr
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True); sys.stdout.flush()
+
+
+def _conv_case(rng):
+    R, S = [int(rng.choice([1, 1, 2, 3, 3, 4, 5, 7])) for _ in range(2)]
+    if rng.rand() < 0.6: S = R
+    sH, sW = [int(rng.choice([1, 1, 1, 2, 2, 3])) for _ in range(2)]
+    pH, pW = int(rng.randint(0, R)), int(rng.randint(0, S))             # pad < kernel, as the reference's programs use
+    H = int(rng.randint(max(1, R - 2 * pH), 26)); W = int(rng.randint(max(1, S - 2 * pW), 26))
+    N = int(rng.randint(1, 6)); Cc = int(rng.choice([1, 2, 3, 4, 7, 8, 16, 17, 32, 40, 64, 96])); K = int(rng.choice([1, 2, 5, 8, 16, 24, 33, 64, 70, 130]))
+    return (N, Cc, H, W, K, R, S, sH, sW, pH, pW)
+
+
+@pytest.mark.parametrize("group", range(8))
+def test_random_conv_geometries(on_hip, group):
+    dev = Dev(on_hip)
+    rng = np.random.RandomState(1000 + group)
+    for i in range(8):
+        dims = _conv_case(rng); bias = bool(rng.rand() < 0.5)
+        _say("conv group %d case %d dims %s bias %s" % (group, i, dims, bias))
+        mark = on_hip.getMallocAddr()
+        check_conv(dev, dims, bias)
+        on_hip.sync(); on_hip.resetMallocAddr(mark)
+
+
+@pytest.mark.parametrize("group", range(4))
+def test_random_sgemm_shapes_with_row_strides(on_hip, group):
+    """All four transpose forms, leading dimensions larger than the rows (views into wider matrices), alpha/beta."""
+    dev = Dev(on_hip); lc = load_oracle()
+    rng = np.random.RandomState(2000 + group)
+    for i in range(10):
+        ta, tb = int(rng.randint(2)), int(rng.randint(2))
+        m, n, k = [int(rng.choice([1, 2, 3, 7, 16, 31, 64, 65, 100, 129, 200, 257])) for _ in range(3)]
+        pa, pb, pc = [int(rng.choice([0, 0, 1, 4, 13])) for _ in range(3)]
+        alpha, beta = float(rng.choice([1.0, 0.5, -2.0])), float(rng.choice([0.0, 1.0, 0.25]))
+        _say("sgemm group %d case %d ta%d tb%d m%d n%d k%d pads %d %d %d alpha %g beta %g" % (group, i, ta, tb, m, n, k, pa, pb, pc, alpha, beta))
+        ash = (k, m) if ta else (m, k); bsh = (n, k) if tb else (k, n)
+        A = rng.randn(ash[0], ash[1] + pa).astype(np.float32); Bm = rng.randn(bsh[0], bsh[1] + pb).astype(np.float32)
+        Cm = rng.randn(m, n + pc).astype(np.float32)
+        ref = Cm.copy()
+        lc.lc_sgemm(C.c_int(ta), C.c_int(tb), C.c_int(m), C.c_int(n), C.c_int(k), C.c_float(alpha), cptr(A), C.c_int(A.shape[1]),
+                    cptr(Bm), C.c_int(Bm.shape[1]), C.c_float(beta), cptr(ref), C.c_int(Cm.shape[1]))
+        mark = on_hip.getMallocAddr()
+        c_ = dev.up(Cm)
+        dev.lib.lh_sgemm(ta, tb, m, n, k, alpha, dev.up(A).ptr, A.shape[1], dev.up(Bm).ptr, Bm.shape[1], beta, c_.ptr, Cm.shape[1]); dev.check()
+        got = dev.down(c_, Cm.shape)
+        assert_close(got[:, :n], ref[:, :n], what="sgemm values")
+        np.testing.assert_array_equal(got[:, n:], Cm[:, n:], err_msg="columns beyond n were written")
+        on_hip.sync(); on_hip.resetMallocAddr(mark)
