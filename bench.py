@@ -65,6 +65,8 @@ def run_gpu(args):
     la.set_backend(be)
     tr, per_step, desc = make_trainer(args, args.batch)
     lib = be.lib
+    if args.no_side_stream:
+        lib.lh_set_side_stream(0)
     for _ in range(args.warmup):
         tr.step(); tr.end_step()
     be.sync()
@@ -162,6 +164,7 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-side-stream", action="store_true", help="filter gradients in line on the main stream (kernel profiles: no two kernels overlap)")
     ap.add_argument("--graph", action="store_true", help="time replays of the step recorded into a HIP graph (fixed-shape workloads)")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args()
@@ -193,7 +196,7 @@ def main():
                 "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
                 # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this workload (see profiles/), not measured live
-                "traffic": 150.8e6 if args.workload == "resnet50" and args.batch == 64 and args.hw == 224 else None, "flop_per_step": conv_fl,
+                "traffic": 151.1e6 if args.workload == "resnet50" and args.batch == 64 and args.hw == 224 else None, "flop_per_step": conv_fl,
                 "ms_per_step": {"fwd": round(conv_ms[0], 3), "bwd_data": round(conv_ms[1], 3), "bwd_filter": round(conv_ms[2], 3)}}
         if work.get("gemm_flop", 0.0) > 0 and timed["gemm"][0] > 0:
             roof["gemm"] = {"flop_per_step": work["gemm_flop"], "ms_per_step": round(timed["gemm"][0], 3),
@@ -208,7 +211,8 @@ def main():
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": g["desc"], "global_batch": args.batch, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
-                   "launch": "hip graph replay" if args.graph else "one launch per kernel"},
+                   "launch": "hip graph replay" if args.graph else "one launch per kernel",
+                   "filter_gradients": "in line" if args.no_side_stream else "side stream"},
         "roofline": roof,
     }
     if args.verbose:

@@ -82,6 +82,24 @@ enum { LH_CAT_CONV_FWD = 0, LH_CAT_CONV_BWD_DATA, LH_CAT_CONV_BWD_FILTER, LH_CAT
        LH_CAT_ELEMENTWISE, LH_CAT_POOL, LH_CAT_REDUCE, LH_CAT_OPTIM, LH_CAT_FILL, LH_CAT_COUNT };
 void lh_prof_enable(unsigned mask);
 
+/* Side stream: work whose results nothing needs for a while runs beside the main chain of kernels instead of in it.
+ * The reference issues every operator on one stream (CUB:171-560), so the filter gradient of a convolution, which only
+ * the optimizer reads, delays the input gradient the next backward operator is waiting for.  Entry points called
+ * between lh_side_begin() and lh_side_end() are enqueued on a second stream (same priority) that first waits for
+ * everything issued before lh_side_begin(); work issued after lh_side_end() does NOT wait for them.  The caller
+ * guarantees that, until the next join, later calls neither touch what the side work writes nor write what it reads
+ * (for filter gradients: x and dy are dead or read-only for the rest of the backward pass, dw and db are read by the
+ * optimizer only).  Joins (the main stream waits for the side work): lh_side_join(), and implicitly lh_sync, lh_h2d,
+ * lh_d2h, lh_rewind, lh_clip and every optimizer entry point (lh_sgd, lh_momentum, lh_adagrad, lh_multi_*).
+ * lh_malloc is refused on the side stream.  The side stream is bypassed (calls run in line) while per-category timing,
+ * the command list or a graph recording is on, after lh_set_side_stream(0), or with LH_NO_SIDE_STREAM in the
+ * environment.  lh_side_forks() counts the lh_side_begin() calls that did switch streams. */
+void lh_side_begin(void);
+void lh_side_end(void);
+void lh_side_join(void);
+void lh_set_side_stream(int on);
+int64_t lh_side_forks(void);
+
 /* HIP graph of a whole step, for programs whose kernels are shorter than their launches (LeNet, SqueezeNet on 32x32
  * images: several hundred launches of a few microseconds per step; the reference pays a launch per operator, CUB:171-560).
  * lh_capture_begin() switches the library's stream to capture: every entry point called until lh_capture_end() is

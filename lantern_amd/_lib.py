@@ -35,6 +35,11 @@ SIGNATURES = {
     "lh_event_destroy": (None, [P]),
     "lh_prof_enable": (None, [C.c_uint]),
     "lh_set_tuning": (None, [I]),
+    "lh_side_begin": (None, []),
+    "lh_side_end": (None, []),
+    "lh_side_join": (None, []),
+    "lh_set_side_stream": (None, [I]),
+    "lh_side_forks": (L, []),
     "lh_capture_begin": (None, []),
     "lh_capture_end": (I, []),
     "lh_graph_launch": (None, [I]),

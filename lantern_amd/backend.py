@@ -9,6 +9,7 @@ In the reference these methods run on the JVM at staging time and emit C++ text;
 calls are issued directly, one C-ABI call (include/lantern_hip.h) per emitted call.
 """
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -69,6 +70,7 @@ class Backend:
     """Operator API (TD:137-379).  Tensors are passed as objects with `.data` (Buf) and `.shape`."""
 
     name = "abstract"
+    ops_left = 0      # set by the tape before a convolution's backward: how many backward operators follow it
 
     # -- memory ---------------------------------------------------------------------------
     def setup(self): raise NotImplementedError
@@ -149,6 +151,8 @@ class BackendHIP(Backend):
         self.heap_bytes = int(heap_bytes)
         self.lib = None
         self.dropout_seed = 42
+        self.side_order = int(os.environ.get("LH_SIDE_ORDER", "1"))
+        self.side_min_ops = int(os.environ.get("LH_SIDE_MIN_OPS", "6"))
         self.dropout_offset = 0
         self.work = {}            # algorithmic flop / bytes issued, by kind (read by the benchmark; a few adds per call)
 
@@ -360,9 +364,22 @@ class BackendHIP(Backend):
         self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
+        # The filter gradient is read by the optimizer only: it goes to the side stream, where it runs beside the
+        # rest of the backward pass (x and dy stay untouched until the optimizer joins).  The input gradient, which
+        # the next backward operator waits for, is issued first and stays on the main stream.
+        so = self.side_order
+        if x_in or self.ops_left < self.side_min_ops:
+            so = 0      # (almost) nothing left to run beside it: the optimizer's join would only add the cross-stream hand-over
+        if so == 2:
+            self.lib.lh_side_begin()
+            self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
+            self.lib.lh_side_end()
         if not x_in:
             self.lib.lh_conv2d_bwd_data(dy.ptr, w.ptr, xd.ptr, beta_dx, N, C, H, W, K, R, S, sH, sW, pH, pW)
-        self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
+        if so != 2:
+            if so: self.lib.lh_side_begin()
+            self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
+            if so: self.lib.lh_side_end()
         _lib.check()
         P, Q = conv_size(H, R, sH, pH), conv_size(W, S, sW, pW)
         self._count("conv_flop", 2.0 * N * K * C * R * S * P * Q * (1 if x_in else 2))

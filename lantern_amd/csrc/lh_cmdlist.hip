@@ -305,6 +305,7 @@ extern "C" {
 void lh_cmdlist_begin(void) {
   LH_REQUIRE(g_stream_raw != nullptr, "lh_cmdlist_begin before lh_setup");
   LH_REQUIRE(!g_capturing, "lh_cmdlist_begin: a graph is being recorded (the command buffers cannot be replayed)");
+  LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_cmdlist_begin on the side stream");
   if (!ring_init()) return;
   g_rec_on = 1;
 }

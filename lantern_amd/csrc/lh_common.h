@@ -9,12 +9,16 @@
 namespace lh {
 
 extern hipStream_t g_stream_raw;  // the library's stream
+// Where entry points enqueue now: g_stream_raw, or the side stream between lh_side_begin and lh_side_end.
+extern hipStream_t g_stream_cur;
+void side_join();                 // the main stream waits for what the side stream was given (no-op when it is idle)
+void quiet_other_stream();        // host-side wait for the stream that is NOT current, so that a timing run has the device to itself
 // Small operations recorded by the command list (lh_cmdlist.hip) but not launched yet.  Anything that is about to use
 // the stream goes through `g_stream`, which launches the recorded commands first, so program order is kept.
 extern int g_rec_pending;
 void rec_flush();
 void cmdlist_release();           // frees the command buffers (lh_cleanup)
-static inline hipStream_t ordered_stream() { if (g_rec_pending) rec_flush(); return g_stream_raw; }
+static inline hipStream_t ordered_stream() { if (g_rec_pending) rec_flush(); return g_stream_cur; }
 #define g_stream (::lh::ordered_stream())     // every kernel is enqueued here
 extern int g_error_mode;         // 0 = print and exit, 1 = record and return
 extern int g_num_cu;             // compute units of the device in use

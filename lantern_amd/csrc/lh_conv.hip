@@ -718,6 +718,8 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_filter: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_filter: beta must be 0 or 1");
+  // A filter gradient issued in line must not overtake one of the same filter that is still on the side stream.
+  if (g_stream_cur == g_stream_raw) side_join();
   const int CRS = C * R * S, PQ = d.P * d.Q;
   const int64_t red = (int64_t)N * PQ;
   LH_REQUIRE(red < 0x7fffffffLL, "lh_conv2d_bwd_filter: reduction length too large");

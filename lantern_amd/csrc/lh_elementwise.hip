@@ -100,6 +100,7 @@ void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, in
 }
 
 void lh_clip(float* x, float bound, int64_t n) {
+  side_join();      // clips gradients, which may still be in flight on the side stream
   ew<1>(x, x, nullptr, nullptr, n, [bound] __device__(float v, float, float) { return v > bound ? bound : (v < -bound ? -bound : v); });
   LH_CHECK_LAUNCH();
 }
@@ -641,6 +642,7 @@ static void multi_update(int mode, int count, float* const* hx, float* const* hd
 
 extern "C" {
 void lh_sgd(float* x, float* d, float lr, int64_t n) { ProfScope prof_(CAT_OPTIM);
+  side_join();      // parameter gradients may still be in flight on the side stream
   if (n <= 0) return;
   LH_REQUIRE(al16(x) && al16(d), "lh_sgd: pointers must be 16-byte aligned");
   if (rec_ok(n)) { rec_cmd(CL_SGD, (int)n, 0, 0, lr, 0.f, 0.f, 0.f, x, d, nullptr, nullptr); return; }
@@ -648,12 +650,14 @@ void lh_sgd(float* x, float* d, float lr, int64_t n) { ProfScope prof_(CAT_OPTIM
   LH_CHECK_LAUNCH();
 }
 void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) { ProfScope prof_(CAT_OPTIM);
+  side_join();      // parameter gradients may still be in flight on the side stream
   if (n <= 0) return;
   LH_REQUIRE(al16(x) && al16(d) && al16(v), "lh_momentum: pointers must be 16-byte aligned");
   hipLaunchKernelGGL(k_momentum, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, v, lr, mu, clip, nesterov, n);
   LH_CHECK_LAUNCH();
 }
 void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) { ProfScope prof_(CAT_OPTIM);
+  side_join();      // parameter gradients may still be in flight on the side stream
   if (n <= 0) return;
   if (rec_ok(n)) { rec_cmd(CL_ADAGRAD, (int)n, 0, 0, lr, clip, 0.f, 0.f, x, d, m, nullptr); return; }
   hipLaunchKernelGGL(k_adagrad, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, d, m, lr, clip, n);
@@ -661,10 +665,12 @@ void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) {
 }
 void lh_multi_momentum(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
                        float lr, float mu, float clip, int nesterov) { ProfScope prof_(CAT_OPTIM);
+  side_join();      // parameter gradients may still be in flight on the side stream
   multi_update(1, count, h_x, h_d, h_v, h_n, lr, mu, clip, nesterov);
   if (!failed()) LH_CHECK_LAUNCH();
 }
 void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr) { ProfScope prof_(CAT_OPTIM);
+  side_join();      // parameter gradients may still be in flight on the side stream
   multi_update(0, count, h_x, h_d, nullptr, h_n, lr, 0.f, 0.f, 0);
   if (!failed()) LH_CHECK_LAUNCH();
 }

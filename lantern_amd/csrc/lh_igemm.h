@@ -425,7 +425,7 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
 struct LaunchTimer {
   hipEvent_t e0 = nullptr, e1 = nullptr;
   bool ok;
-  LaunchTimer() { ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess; }
+  LaunchTimer() { ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess; quiet_other_stream(); }
   ~LaunchTimer() { if (e0) (void)hipEventDestroy(e0); if (e1) (void)hipEventDestroy(e1); }
   template <class F>
   float ms(F launch) {

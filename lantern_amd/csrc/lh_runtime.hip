@@ -8,6 +8,27 @@
 
 namespace lh {
 hipStream_t g_stream_raw = nullptr;
+hipStream_t g_stream_cur = nullptr;
+// Side stream: work whose results nothing needs before the optimizer (filter gradients) runs beside the main chain.
+static hipStream_t g_side_stream = nullptr;
+static bool g_side_dirty = false;            // the side stream holds work the main stream has not waited for
+static int g_side_enabled = getenv("LH_NO_SIDE_STREAM") == nullptr;
+constexpr int SIDE_EVENTS = 16;              // fork and join events, used round-robin
+static hipEvent_t g_side_ev[SIDE_EVENTS];
+static unsigned g_side_ev_next = 0;
+static int64_t g_side_forks = 0;
+static hipEvent_t side_event() { return g_side_ev[g_side_ev_next++ % SIDE_EVENTS]; }
+void quiet_other_stream() {
+  if (g_stream_cur == g_stream_raw) { if (g_side_dirty) (void)hipStreamSynchronize(g_side_stream); }
+  else (void)hipStreamSynchronize(g_stream_raw);
+}
+void side_join() {
+  if (!g_side_dirty) return;
+  g_side_dirty = false;
+  hipEvent_t ev = side_event();
+  LH_HIP(hipEventRecord(ev, g_side_stream));
+  LH_HIP(hipStreamWaitEvent(g_stream_raw, ev, 0));
+}
 bool g_tune_enabled = getenv("LH_NO_TUNE") == nullptr;
 bool g_capturing = false;
 unsigned long long* g_capture_advance = nullptr;
@@ -93,6 +114,9 @@ void lh_setup(size_t heap_bytes) {
   LH_HIP(hipGetDeviceProperties(&prop, dev));
   g_num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   LH_HIP(hipStreamCreateWithFlags(&g_stream_raw, hipStreamNonBlocking));
+  LH_HIP(hipStreamCreateWithFlags(&g_side_stream, hipStreamNonBlocking));     // same (default) priority as the main stream
+  for (auto& e : g_side_ev) LH_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+  g_stream_cur = g_stream_raw; g_side_dirty = false;
   heap_bytes = (heap_bytes + 255) & ~(size_t)255;
   LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
   g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0; g_zero_end = 0;
@@ -100,6 +124,9 @@ void lh_setup(size_t heap_bytes) {
 }
 
 void lh_cleanup(void) {
+  g_stream_cur = g_stream_raw;
+  if (g_side_stream) { (void)hipStreamSynchronize(g_side_stream); (void)hipStreamDestroy(g_side_stream); for (auto& e : g_side_ev) (void)hipEventDestroy(e); }
+  g_side_stream = nullptr; g_side_dirty = false;
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
   cmdlist_release();
   for (auto& e : g_graphs) if (e) { (void)hipGraphExecDestroy(e); e = nullptr; }
@@ -108,16 +135,18 @@ void lh_cleanup(void) {
   g_advance_pool = nullptr; g_capture_advance = nullptr;
   if (g_heap) (void)hipFree(g_heap);
   if (g_stream_raw) (void)hipStreamDestroy(g_stream_raw);
-  g_heap = nullptr; g_stream_raw = nullptr; g_heap_bytes = g_top = g_zero_end = 0;
+  g_heap = nullptr; g_stream_raw = nullptr; g_stream_cur = nullptr; g_heap_bytes = g_top = g_zero_end = 0;
 }
 
 void lh_sync(void) {
   LH_NOT_CAPTURING("lh_sync");
+  side_join();
   LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH();
 }
 
 static void* bump(size_t bytes, bool zero) {
   if (!g_heap) { LH_FAIL("lh_malloc before lh_setup"); return nullptr; }
+  if (zero && g_stream_cur != g_stream_raw) { LH_FAIL("lh_malloc between lh_side_begin and lh_side_end: zeroed memory is handed out in main-stream order only"); return nullptr; }
   size_t need = (bytes + 255) & ~(size_t)255;
   if (need == 0) need = 256;
   if (g_top + need > g_heap_bytes) {
@@ -150,6 +179,7 @@ void lh_free_top(size_t bytes) {
 size_t lh_mark(void) { return g_top; }
 void lh_rewind(size_t mark) {
   LH_REQUIRE(mark <= g_top && (mark & 255) == 0, "lh_rewind(%zu): not a mark at or below the top (%zu)", mark, g_top);
+  side_join();      // what is handed out again must not be in use on the side stream
   g_top = mark;
   g_zero_end = mark;
 }
@@ -159,11 +189,13 @@ size_t lh_heap_peak(void) { return g_peak; }
 void lh_h2d(void* dst, const void* h_src, size_t bytes) {
   // Pageable source: the copy is staged before the call returns, so the host buffer may be reused.
   LH_NOT_CAPTURING("lh_h2d");
+  side_join();
   LH_HIP(hipMemcpyAsync(dst, h_src, bytes, hipMemcpyHostToDevice, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
 }
 void lh_d2h(void* h_dst, const void* src, size_t bytes) {
   LH_NOT_CAPTURING("lh_d2h");
+  side_join();
   LH_HIP(hipMemcpyAsync(h_dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
 }
@@ -173,7 +205,24 @@ void lh_d2d(void* dst, const void* src, size_t bytes) {
 }
 
 // ---- HIP graphs: a launch-bound step recorded once and replayed ----------------------------------------------
+// ---- side stream ---------------------------------------------------------------------------------------------
+void lh_side_begin(void) {
+  LH_REQUIRE(g_stream_raw != nullptr, "lh_side_begin before lh_setup");
+  LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_side_begin: already on the side stream");
+  // In line (no concurrency) when switched off, while kernels are timed one by one, or while the stream is recorded.
+  if (!g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on) return;
+  hipEvent_t ev = side_event();
+  LH_HIP(hipEventRecord(ev, g_stream));              // (flushes recorded commands first)
+  LH_HIP(hipStreamWaitEvent(g_side_stream, ev, 0));
+  g_stream_cur = g_side_stream; g_side_dirty = true; g_side_forks++;
+}
+void lh_side_end(void) { g_stream_cur = g_stream_raw; }
+void lh_side_join(void) { LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_side_join between lh_side_begin and lh_side_end"); side_join(); }
+void lh_set_side_stream(int on) { g_side_enabled = on != 0; }
+int64_t lh_side_forks(void) { return g_side_forks; }
+
 void lh_capture_begin(void) {
+  side_join();
   LH_REQUIRE(g_stream_raw != nullptr, "lh_capture_begin before lh_setup");
   LH_REQUIRE(!g_capturing, "lh_capture_begin: already capturing");
   LH_REQUIRE(!g_rec_on, "lh_capture_begin: the command list is recording (its buffers cannot be replayed)");
@@ -215,7 +264,7 @@ void lh_graph_destroy(int id) {
   g_graphs[id] = nullptr;
 }
 
-void lh_prof_enable(unsigned mask) { g_prof_mask = mask; }
+void lh_prof_enable(unsigned mask) { side_join(); g_prof_mask = mask; }
 void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat) {
   for (int c = 0; c < ncat; c++) { h_ms[c] = 0.0; h_calls[c] = 0; }
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);

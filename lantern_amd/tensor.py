@@ -735,6 +735,7 @@ class TensorR:
         _park(y, launch, "conv", launch_bn)
         def back():
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()
+            be.ops_left = len(_tape)        # backward operators still to come (a backend may run the filter gradient beside them)
             be.conv2D_batch_grad(self.x.data, xd, self.isInput, kept["finput"], kernel.x.data, kernel.d.data, y.d.data,
                                  bias.d.data if bias is not None else None, N, C, H, W, K, R, S, sH, sW, pH, pW, beta)
         _tape.append(back)

@@ -809,3 +809,71 @@ def test_batchnorm_add_relu_join_forward_and_backward(pair, shape, beta_sd):
 
     outs = pair.run(f)
     check_all(outs, rtol=2e-4)
+
+
+# ---- side stream: filter gradients beside the main chain of kernels -------------------------------------
+def test_side_stream_filter_gradients_match_in_line_and_wait_for_their_inputs(on_hip):
+    """Through the C ABI: dy is produced on the main stream right before the fork (the side work must wait for it),
+    main-stream work that does not touch the operands follows, the optimizer-style join comes last.  Accumulating twice
+    into one dw from the side stream, then once in line, must give three times the in-line gradient."""
+    be, lib = on_hip, on_hip.lib
+    dims = (8, 32, 20, 20, 48, 3, 3, 1, 1, 1, 1)
+    N, Cc, H, W, K = dims[:5]
+    rng = np.random.RandomState(71)
+    x = be.fromHost(rng.randn(N * Cc * H * W).astype(np.float32)); dy0 = be.fromHost(rng.randn(N * K * H * W).astype(np.float32))
+    n_dy = N * K * H * W; n_w = K * Cc * 9
+
+    def grads(side):
+        lib.lh_set_side_stream(1 if side else 0)
+        forks0 = lib.lh_side_forks()
+        dy = be.mallocArray(n_dy, zero=False); dw = be.mallocArray(n_w); db = be.mallocArray(K); other = be.mallocArray(1 << 20, zero=False)
+        lib.lh_scalar_op(B.MUL, dy0.ptr, dy.ptr, 1.0, n_dy)      # dy written on the main stream just before
+        for rep in range(2):
+            lib.lh_side_begin()
+            lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, dw.ptr, db.ptr, 1.0, *dims)
+            lib.lh_side_end()
+            for _ in range(4):                                   # unrelated main-stream work meanwhile
+                lib.lh_fill(other.ptr, float(rep), 1 << 20)
+        lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, dw.ptr, db.ptr, 1.0, *dims)     # in line: joins first
+        from lantern_amd import _lib
+        _lib.check()
+        out = (be.toHost(dw, n_w).copy(), be.toHost(db, K).copy())              # the read-back joins too
+        lib.lh_set_side_stream(1)
+        return out, lib.lh_side_forks() - forks0
+
+    (dw_a, db_a), forks_a = grads(False)
+    (dw_b, db_b), forks_b = grads(True)
+    assert forks_a == 0 and forks_b == 2
+    assert_close(dw_b, dw_a, rtol=1e-5, what="filter gradient from the side stream")
+    assert_close(db_b, db_a, rtol=1e-5, what="bias gradient from the side stream")
+    assert np.abs(dw_a).max() > 1.0
+
+
+def test_convolution_applied_twice_accumulates_one_filter_gradient_across_streams(pair):
+    """One Conv2D module used deep in the network (its filter gradient goes to the side stream) and again on the
+    network input (in line): both accumulate into the same gradient buffer."""
+    from lantern_amd.nn import Conv2D
+    rng = np.random.RandomState(72)
+    x = rng.randn(4, 8, 12, 12).astype(np.float32)
+    w0 = (rng.randn(8, 8, 3, 3) * 0.2).astype(np.float32)
+
+    def f(be, up, down):
+        conv = Conv2D(8, 8, (3, 3), pad=(1, 1), useBias=True, init=lambda dims: w0)
+        xin = la.TensorR(la.Tensor.fromNumpy(x), isInput=True)
+
+        def loss(dummy):
+            h = conv(xin).tanh()
+            for _ in range(7):
+                h = (h * h).tanh()
+            h = conv(h)                       # the deep use
+            for _ in range(7):
+                h = (h * h).tanh()
+            return h.sum()
+        forks0 = be.lib.lh_side_forks() if be.name == "hip" else 0
+        lval = la.gradR_loss(loss)(la.Tensor.zeros(1))
+        if be.name == "hip":
+            assert be.lib.lh_side_forks() - forks0 == 1
+        return [lval.toCPU().copy(), conv.kernel.d.toCPU().copy(), conv.bias.d.toCPU().copy()]
+
+    outs = pair.run(f)
+    check_all(outs, rtol=1e-4)
