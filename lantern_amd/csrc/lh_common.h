@@ -25,6 +25,7 @@ extern int g_num_cu;             // compute units of the device in use
 extern bool g_tune_enabled;      // launch plans are measured on first use (lh_set_tuning; off with LH_NO_TUNE in the environment)
 extern bool g_capturing;         // between lh_capture_begin and lh_capture_end: work is recorded into a HIP graph, nothing may wait on the stream
 #define g_tune (::lh::g_tune_enabled && !::lh::g_capturing)
+extern double g_tune_min_flop;   // products below this many flop keep the built-in launch rule (a timing run costs more than it can win)
 // Dropout draws from a counter-based stream whose position the caller passes per launch.  A replayed graph repeats its
 // launch arguments, so a captured dropout adds *g_capture_advance (device memory; 0 for the first replay, advanced at the
 // end of every replay by the g_capture_drawn positions the recorded step used) to the position it was recorded with.

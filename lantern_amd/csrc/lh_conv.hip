@@ -381,7 +381,7 @@ template <class AL, class BL, class EP>
 static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out = nullptr, int64_t zero_n = 0, bool prezeroed = false) {
   static std::map<PlanKey, int> chosen;
   const bool can_zero = zero_out != nullptr || prezeroed;
-  if (!g_tune || 2.0 * M * N * (double)K < 2e8) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  if (!g_tune || 2.0 * M * N * (double)K < g_tune_min_flop) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   const PlanKey key = {{M, N, K, ep.eH, ep.eW, ep.W, ep.PIX}};
   auto it = chosen.find(key);
   if (it != chosen.end()) {
@@ -479,7 +479,7 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
       // repeating it is harmless) and remembered
       static std::map<PlanKey, int> chosen;
       const PlanKey key = {{K, N * PQ, CRS, H, W, sH, R}};
-      const bool tunable = g_tune && 2.0 * K * CRS * (double)N * PQ >= 2e8;
+      const bool tunable = g_tune && 2.0 * K * CRS * (double)N * PQ >= g_tune_min_flop;
       int force = 0;
       auto run = [&](int f) {           // 0: the rule's tile, 1-3: a forced tile, 4: unfused (any launch plan, then a pass over y)
         if (f == 4) {
@@ -635,7 +635,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
         int tile = tp.bm == 128 ? 1 : (tp.bn == 128 ? 2 : 3);
         auto it = chosen.find(key);
         if (it != chosen.end()) tile = it->second;
-        else if (g_tune && beta == 0.f && 2.0 * C * (double)ntot * kmax >= 2e8) {
+        else if (g_tune && beta == 0.f && 2.0 * C * (double)ntot * kmax >= g_tune_min_flop) {
           LaunchTimer timer;
           if (timer.ok) {
             float best_ms = 3.0e38f; int best = tile;
@@ -735,7 +735,7 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   // How many slices pays best depends on how tiles x slices fall onto the resident block slots and on how short the
   // per-block reduction gets; it is measured once per shape (a few candidates on a scratch output) and remembered.
   const BwdfKey key = {{N, C, H, W, K, R, S, sH, sW, pH, pW}};
-  const bool tunable = g_tune && max_split > 1 && 2.0 * K * CRS * (double)red >= 2e8;
+  const bool tunable = g_tune && max_split > 1 && 2.0 * K * CRS * (double)red >= g_tune_min_flop;
   bool tune_now = false;
   if (tunable) {
     auto it = g_bwdf_split.find(key);

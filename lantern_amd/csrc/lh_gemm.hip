@@ -8,31 +8,43 @@ using namespace lh;
 namespace {
 constexpr int TPB = 256;
 
-// 64x64 output tile per block, 16-deep k slabs through LDS, 4x4 register tile per thread.
+// Small products (below the MFMA path's sizes): 64x64 output tile per block, 64-deep k slabs through LDS, 4x4 register tile
+// per thread.  These launches are latency-bound (one or a few blocks), so a slab is deep: all of a thread's 32 loads of
+// a slab are independent and in flight together, and k = 100 takes two round trips to memory instead of seven.
+constexpr int SMALL_KS = 64;
 template <bool TA, bool TB>
 __global__ void __launch_bounds__(TPB) k_sgemm_tile(int m, int n, int k, float alpha, const float* __restrict__ A, int lda,
                                                     const float* __restrict__ B, int ldb, float beta, float* __restrict__ C, int ldc) {
-  __shared__ float As[16][64 + 4];
-  __shared__ float Bs[16][64 + 4];
+  __shared__ float As[SMALL_KS][64 + 4];
+  __shared__ float Bs[SMALL_KS][64 + 4];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
   const int i0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
   float acc[4][4] = {};
-  for (int k0 = 0; k0 < k; k0 += 16) {
-    for (int e = threadIdx.x; e < 16 * 64; e += TPB) {
+  for (int k0 = 0; k0 < k; k0 += SMALL_KS) {
+    const int kn = k - k0 < SMALL_KS ? k - k0 : SMALL_KS;
+    float ra[SMALL_KS * 64 / TPB], rb[SMALL_KS * 64 / TPB];
+#pragma unroll
+    for (int r = 0; r < SMALL_KS * 64 / TPB; r++) {
+      const int e = threadIdx.x + r * TPB;
       int kk, ii;
-      if (TA) { ii = e & 63; kk = e >> 6; } else { kk = e & 15; ii = e >> 4; }
-      int gi = i0 + ii, gk = k0 + kk;
-      As[kk][ii] = (gi < m && gk < k) ? (TA ? A[(int64_t)gk * lda + gi] : A[(int64_t)gi * lda + gk]) : 0.f;
+      if (TA) { ii = e & 63; kk = e >> 6; } else { kk = e & (SMALL_KS - 1); ii = e / SMALL_KS; }
+      const int gi = i0 + ii, gk = k0 + kk;
+      ra[r] = (gi < m && kk < kn) ? (TA ? A[(int64_t)gk * lda + gi] : A[(int64_t)gi * lda + gk]) : 0.f;
+      int jj;
+      if (TB) { kk = e & (SMALL_KS - 1); jj = e / SMALL_KS; } else { jj = e & 63; kk = e >> 6; }
+      const int gj = j0 + jj; const int gk2 = k0 + kk;
+      rb[r] = (gj < n && kk < kn) ? (TB ? B[(int64_t)gj * ldb + gk2] : B[(int64_t)gk2 * ldb + gj]) : 0.f;
     }
-    for (int e = threadIdx.x; e < 16 * 64; e += TPB) {
-      int kk, jj;
-      if (TB) { kk = e & 15; jj = e >> 4; } else { jj = e & 63; kk = e >> 6; }
-      int gj = j0 + jj, gk = k0 + kk;
-      Bs[kk][jj] = (gj < n && gk < k) ? (TB ? B[(int64_t)gj * ldb + gk] : B[(int64_t)gk * ldb + gj]) : 0.f;
+#pragma unroll
+    for (int r = 0; r < SMALL_KS * 64 / TPB; r++) {
+      const int e = threadIdx.x + r * TPB;
+      if (TA) As[e >> 6][e & 63] = ra[r]; else As[e & (SMALL_KS - 1)][e / SMALL_KS] = ra[r];
+      if (TB) Bs[e & (SMALL_KS - 1)][e / SMALL_KS] = rb[r]; else Bs[e >> 6][e & 63] = rb[r];
     }
     __syncthreads();
-#pragma unroll
-    for (int kk = 0; kk < 16; kk++) {
+    const int kn8 = (kn + 7) & ~7;          // rows kn.. of the slab hold zeros
+#pragma unroll 8
+    for (int kk = 0; kk < kn8; kk++) {
       float a[4], b[4];
 #pragma unroll
       for (int u = 0; u < 4; u++) { a[u] = As[kk][ty * 4 + u]; b[u] = Bs[kk][tx * 4 + u]; }
@@ -177,7 +189,7 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
     SgemmPlan pl = sgemm_plan(m, n, k);
     // Tile shape and reduction slices are measured once per (transposes, m, n, k) on a scratch output and remembered.
     static std::map<std::array<int, 7>, SgemmPlan> chosen;
-    if (g_tune && 2.0 * m * n * (double)k >= 2e8) {
+    if (g_tune && 2.0 * m * n * (double)k >= g_tune_min_flop) {
       const std::array<int, 7> key = {ta, tb, m, n, k, (int)av, (int)bv};
       auto it = chosen.find(key);
       if (it != chosen.end()) pl = it->second;

@@ -31,6 +31,7 @@ void side_join() {
 }
 bool g_tune_enabled = getenv("LH_NO_TUNE") == nullptr;
 bool g_capturing = false;
+double g_tune_min_flop = getenv("LH_TUNE_MIN_FLOP") ? atof(getenv("LH_TUNE_MIN_FLOP")) : 1e7;
 unsigned long long* g_capture_advance = nullptr;
 unsigned long long g_capture_drawn = 0;
 static unsigned long long* g_advance_pool = nullptr;   // one counter per graph

@@ -131,7 +131,7 @@ def test_sgemm(on_hip, ta, tb, m, n, k):
         assert_close(dev.down(c_, (m, n)), ref, what="sgemm %d%d a=%g b=%g" % (ta, tb, alpha, beta))
 
 
-# Shapes large enough for the launch plans to be measured on first use (>= 2e8 flop) and small enough for the oracle.
+# Shapes large enough for the launch plans to be measured on first use (well above the 1e7-flop floor) and small enough for the oracle.
 TUNED_SHAPES = [
     (8, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),      # tap path, 64-row product
     (4, 256, 14, 14, 256, 3, 3, 1, 1, 1, 1),    # few tiles over a long reduction: the stream-K plans compete
