@@ -132,14 +132,22 @@ def load():
         fn = getattr(lib, name)  # AttributeError if the symbol is missing
         fn.restype = res
         fn.argtypes = args
+    # The error text lives in one static buffer: its first byte says whether an error is recorded, and reading that byte
+    # costs a third of a foreign call (check() runs after every operator).
+    global _err_flag
+    lib.lh_last_error.restype = C.c_void_p
+    _err_flag = C.c_ubyte.from_address(lib.lh_last_error())
+    lib.lh_last_error.restype = C.c_char_p
     _lib = lib
     return lib
 
 
+_err_flag = None
+
+
 def check():
     """Raise LanternHipError if the last call recorded an error (used with error mode 1)."""
-    msg = _lib.lh_last_error()
-    if msg:
-        text = msg.decode()
+    if _err_flag.value:
+        text = _lib.lh_last_error().decode()
         _lib.lh_clear_error()
         raise LanternHipError(text)

@@ -198,7 +198,7 @@ class BackendHIP(Backend):
         return rec.value, launches.value
 
     def mallocArray(self, length, zero=True):
-        n = max(int(length), 1)
+        n = int(length) if length > 0 else 1
         p = (self.lib.lh_malloc if zero else self.lib.lh_malloc_uninit)(4 * n)
         _lib.check()
         return Buf(p, n)

@@ -112,13 +112,19 @@ class Tensor:
 
     def __init__(self, data, dims):
         self.data = data
-        self.shape = tuple(int(d) for d in dims)
-        self.scalarCount = _prod(self.shape)
+        if type(dims) is not tuple:
+            dims = tuple(dims)
+        n = 1
+        for d in dims:
+            n *= d
+        if type(n) is not int:              # numpy integers in the shape: normalise once
+            dims = tuple(int(d) for d in dims)
+            n = int(n)
+        self.shape = dims
+        self.scalarCount = n
+        self.rank = len(dims)
 
     # -- shape helpers ----------------------------------------------------------------------
-    @property
-    def rank(self): return len(self.shape)
-
     @property
     def strides(self):
         st, s = [], 1
@@ -144,7 +150,7 @@ class Tensor:
 
     @staticmethod
     def zeros_like(t):
-        return Tensor.zeros(*t.shape)
+        return Tensor(get_backend().mallocArray(t.scalarCount), t.shape)
 
     @staticmethod
     def fill(dims, value):
@@ -229,9 +235,12 @@ class Tensor:
     def _ibin(self, op, that):
         be = get_backend()
         if isinstance(that, Tensor):
-            r = max(self.rank, that.rank)
-            a = (1,) * (r - self.rank) + self.shape
-            b = (1,) * (r - that.rank) + that.shape
+            if self.shape == that.shape:
+                a = b = self.shape
+            else:
+                r = max(self.rank, that.rank)
+                a = (1,) * (r - self.rank) + self.shape
+                b = (1,) * (r - that.rank) + that.shape
             be.bcast_update(op, self.data, a, that.data, b)
         else:
             be.scalar_op(op, self.data, float(that), self.scalarCount, out=self.data)
