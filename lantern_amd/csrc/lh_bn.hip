@@ -148,9 +148,12 @@ __global__ void __launch_bounds__(TPB) k_bn_bwd_stats(const float* __restrict__ 
 template <bool VEC, bool ACC, int RELU>
 __global__ void __launch_bounds__(TPB) k_bn_bwd_apply(const float* __restrict__ x, const float* __restrict__ yv, const float* __restrict__ dy, const float* __restrict__ partial,
                                                       const float* gamma, const float* bias, const float* save_mean, const float* save_invstd,
-                                                      float* __restrict__ dx, float* dgamma, float* dbeta, int N, int C, int HW, int n_per) {
+                                                      float* __restrict__ dx, float* dgamma, float* dbeta, int N, int C, int HW, int n_per, int from_end) {
   __shared__ float sh[2];
-  const int c = blockIdx.x, s = blockIdx.y;
+  // from_end: blocks walk the tensor from its end.  The statistics pass that ran just before read it front to back, so on
+  // tensors beyond the last-level cache the part touched last is the part still there (measured: 5 % on 2 x 206 MB,
+  // a loss on tensors that fit, hence the switch).
+  const int c = from_end ? gridDim.x - 1 - blockIdx.x : blockIdx.x, s = from_end ? gridDim.y - 1 - blockIdx.y : blockIdx.y;
   if (threadIdx.x == 0) {
     double a = 0.0, b = 0.0;
     for (int t = 0; t < (int)gridDim.y; t++) { const float* p = partial + 3 * ((int64_t)c * gridDim.y + t); a += p[0]; b += p[1]; }
@@ -381,8 +384,9 @@ static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, co
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx | (uintptr_t)y_relu) & 15) == 0);
   dim3 grid(C, p.slices);
   const bool acc = beta_dx != 0.0f;
+  const int from_end = 8.0 * N * C * (double)HW > 192e6;      // x and dy together beyond most of the 256 MB last-level cache
 #define STATS(V, R) hipLaunchKernelGGL((k_bn_bwd_stats<V, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, save_mean, save_invstd, gamma, bias, g_partial_ptr, N, C, HW, p.n_per)
-#define APPLY(V, A, R) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, (const float*)g_partial_ptr, gamma, bias, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
+#define APPLY(V, A, R) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, R>), grid, dim3(TPB), 0, g_stream, x, y_relu, dy, (const float*)g_partial_ptr, gamma, bias, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per, from_end)
 #define BOTH(V, R) do { STATS(V, R); if (acc) APPLY(V, true, R); else APPLY(V, false, R); } while (0)
   if (p.vec4) { if (relu == 2) BOTH(true, 2); else if (relu == 1) BOTH(true, 1); else BOTH(true, 0); }
   else { if (relu == 2) BOTH(false, 2); else if (relu == 1) BOTH(false, 1); else BOTH(false, 0); }
@@ -439,8 +443,9 @@ void lh_bn_bwd_add_relu(const float* x, const float* out, float* dout, const flo
   dim3 grid(C, p.slices);
   const bool inplace = ds == nullptr || beta_ds != 0.0f, acc = beta_dx != 0.0f;
   const float* g = inplace ? dout : ds;            // where the masked gradient lies after the first pass
+  const int from_end = 8.0 * N * C * (double)HW > 192e6;
 #define STATS(V, I, H) hipLaunchKernelGGL((k_bn_bwd_stats_add<V, I, H>), grid, dim3(TPB), 0, g_stream, x, out, dout, ds, save_mean, save_invstd, g_partial_ptr, N, C, HW, p.n_per)
-#define APPLY(V, A) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, 0>), grid, dim3(TPB), 0, g_stream, x, (const float*)nullptr, g, (const float*)g_partial_ptr, gamma, (const float*)nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per)
+#define APPLY(V, A) hipLaunchKernelGGL((k_bn_bwd_apply<V, A, 0>), grid, dim3(TPB), 0, g_stream, x, (const float*)nullptr, g, (const float*)g_partial_ptr, gamma, (const float*)nullptr, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW, p.n_per, from_end)
   if (p.vec4) {
     if (!inplace) STATS(true, false, true); else if (ds) STATS(true, true, true); else STATS(true, true, false);
     if (acc) APPLY(true, true); else APPLY(true, false);

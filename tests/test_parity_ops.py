@@ -70,7 +70,8 @@ def check_all(outs, rtol=1e-4, exact=()):
 
 
 # ---- batch norm --------------------------------------------------------------------------------------
-BN_SHAPES = [(64, 64, 56 * 56), (8, 256, 56 * 56), (16, 512, 28 * 28), (32, 2048, 49), (4, 24, 7), (3, 5, 1), (1, 16, 100), (20, 33, 1), (64, 1024, 1)]
+BN_SHAPES = [(64, 64, 56 * 56), (8, 256, 56 * 56), (16, 128, 112 * 112),      # the third: x and dy beyond the last-level cache, walked from the end
+             (16, 512, 28 * 28), (32, 2048, 49), (4, 24, 7), (3, 5, 1), (1, 16, 100), (20, 33, 1), (64, 1024, 1)]
 BN_SHAPES += _random_cases(101, 10, lambda r: (_ri(r, 2, 20), _ri(r, 1, 70), _pick(r, [1, 2, 7, 49, 100, 196, 333, 1023])))
 
 
@@ -781,7 +782,7 @@ def test_command_list_keeps_program_order_around_other_kernels_and_wraps_its_buf
 
 
 # ---- residual join behind a batch norm: out = relu(bn(x) + shortcut) -----------------------------------
-@pytest.mark.parametrize("shape", [(8, 16, 28, 28), (3, 5, 7, 7), (4, 32, 1, 1)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", [(8, 16, 28, 28), (3, 5, 7, 7), (4, 32, 1, 1), (16, 128, 112, 112)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("beta_sd", [0.0, 1.0, None], ids=["shortcut_grad_fresh", "shortcut_grad_accumulates", "shortcut_is_input"])
 def test_batchnorm_add_relu_join_forward_and_backward(pair, shape, beta_sd):
     N, Cc, H, W = shape
