@@ -282,6 +282,9 @@ void lh_dropout_bwd(const float* dy, const float* mask, float* dx, int64_t n);
 /* ---- concat along one axis of n tensors (TD:369-370; CUB:825-879) ------ */
 void lh_concat(int n, const float* const* h_in_ptrs, const int* sizes, float* out, int outer, int inner);
 void lh_concat_grad(int n, float* const* h_ind_ptrs, const int* sizes, const float* outd, int outer, int inner);
+/* The same with a host array of n betas: input t's gradient is overwritten (beta 0: a buffer no other consumer has written,
+ * which then needs no zero fill) or accumulated (beta 1, what the reference does for all of them); h_beta NULL = all 1. */
+void lh_concat_grad_beta(int n, float* const* h_ind_ptrs, const float* h_beta, const int* sizes, const float* outd, int outer, int inner);
 
 /* ---- optimizers (TD:377-378; NN:255-303; API:652-678) ------------------ */
 void lh_sgd(float* x, float* d, float lr, int64_t n);          /* x -= lr*d; d = 0  (SGD.step = geam + clear_grad, NN:279-285) */

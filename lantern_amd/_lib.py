@@ -104,6 +104,7 @@ SIGNATURES = {
     "lh_dropout_bwd": (None, [P, P, P, L]),
     "lh_concat": (None, [I, P, P, P, I, I]),
     "lh_concat_grad": (None, [I, P, P, P, I, I]),
+    "lh_concat_grad_beta": (None, [I, P, P, P, P, I, I]),
     "lh_sgd": (None, [P, P, F, L]),
     "lh_momentum": (None, [P, P, P, F, F, F, I, L]),
     "lh_adagrad": (None, [P, P, P, F, F, L]),

@@ -527,9 +527,13 @@ class BackendHIP(Backend):
         self.lib.lh_concat(len(bufs), ptrs, _ints(sizes), res.ptr, outer, inner); _lib.check()
         return res
 
-    def concat_grad(self, dbufs, sizes, outd, outer, inner):
+    def concat_grad(self, dbufs, sizes, outd, outer, inner, betas=None):
         ptrs = (C.c_void_p * len(dbufs))(*[(b.ptr if b is not None else 0) for b in dbufs])
-        self.lib.lh_concat_grad(len(dbufs), ptrs, _ints(sizes), outd.ptr, outer, inner); _lib.check()
+        if betas is None:
+            self.lib.lh_concat_grad(len(dbufs), ptrs, _ints(sizes), outd.ptr, outer, inner)
+        else:
+            self.lib.lh_concat_grad_beta(len(dbufs), ptrs, (C.c_float * len(betas))(*betas), _ints(sizes), outd.ptr, outer, inner)
+        _lib.check()
 
     # -- recurrent layer, CTC (CDN:1638-1938) ------------------------------------------------------------
     def ctcLoss(self, probs, probs_d, input_lengths, labels, label_lengths, T, B, A):

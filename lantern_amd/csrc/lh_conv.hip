@@ -285,10 +285,14 @@ __global__ void __launch_bounds__(TPB) k_filter_transpose(const float* __restric
 __global__ void __launch_bounds__(TPB) k_conv_bwd_bias(const float* __restrict__ dy, float* db, int N, int K, int PQ, int n_per) {
   __shared__ float sm[17];
   const int k = blockIdx.x, n0 = blockIdx.y * n_per, n1 = min(N, n0 + n_per);
+  // (sample, pixel) pairs flattened over the threads: small maps (PQ below the block size) keep every lane busy and
+  // the loads of one thread do not wait for each other
   float acc = 0.f;
-  for (int n = n0; n < n1; n++) {
-    const float* p = dy + ((int64_t)n * K + k) * PQ;
-    for (int l = threadIdx.x; l < PQ; l += TPB) acc += p[l];
+  const int total = (n1 - n0) * PQ;
+#pragma unroll 4
+  for (int i = threadIdx.x; i < total; i += TPB) {
+    const int dn = i / PQ, l = i - dn * PQ;
+    acc += dy[((int64_t)(n0 + dn) * K + k) * PQ + l];
   }
   acc = lh_block_sum(acc, sm);
   if (threadIdx.x == 0) atomicAdd(db + k, acc);

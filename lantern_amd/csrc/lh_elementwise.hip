@@ -518,13 +518,14 @@ void lh_dropout_bwd(const float* dy, const float* mask, float* dx, int64_t n) {
 // One launch per input tensor: rows of `st = sizes[t]*inner` floats are copied between a
 // packed source and a strided destination (or accumulated the other way for the gradient).
 }  // extern "C"
-template <bool GRAD>
+// GRAD: 0 = forward copy into the strided destination, 1 = gradient accumulated into the packed one, 2 = gradient overwriting it
+template <int GRAD>
 __global__ void __launch_bounds__(TPB) k_concat(const float* __restrict__ src, float* __restrict__ dst, int64_t st, int64_t row, int64_t off, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, s = (int64_t)gridDim.x * TPB;
   for (; i < n; i += s) {
     int64_t h = i / st, l = i - h * st;
     int64_t o = h * row + off + l;
-    if (GRAD) dst[i] += src[o]; else dst[o] = src[i];
+    if (GRAD == 1) dst[i] += src[o]; else if (GRAD == 2) dst[i] = src[o]; else dst[o] = src[i];
   }
 }
 extern "C" {
@@ -533,20 +534,27 @@ void lh_concat(int n, const float* const* h_in, const int* sizes, float* out, in
   int64_t off = 0;
   for (int t = 0; t < n; t++) {
     int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
-    if (tot > 0) hipLaunchKernelGGL((k_concat<false>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, h_in[t], out, st, row, off, tot);
+    if (tot > 0) hipLaunchKernelGGL((k_concat<0>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, h_in[t], out, st, row, off, tot);
+    off += st;
+  }
+  LH_CHECK_LAUNCH();
+}
+void lh_concat_grad_beta(int n, float* const* h_ind, const float* h_beta, const int* sizes, const float* outd, int outer, int inner) {
+  int64_t row = 0; for (int t = 0; t < n; t++) row += (int64_t)sizes[t] * inner;
+  for (int t = 0; t < n && h_beta; t++) LH_REQUIRE(h_beta[t] == 0.f || h_beta[t] == 1.f, "lh_concat_grad_beta: beta must be 0 or 1");
+  int64_t off = 0;
+  for (int t = 0; t < n; t++) {
+    int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
+    if (tot > 0 && h_ind[t]) {
+      if (h_beta && h_beta[t] == 0.f) hipLaunchKernelGGL((k_concat<2>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
+      else hipLaunchKernelGGL((k_concat<1>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
+    }
     off += st;
   }
   LH_CHECK_LAUNCH();
 }
 void lh_concat_grad(int n, float* const* h_ind, const int* sizes, const float* outd, int outer, int inner) {
-  int64_t row = 0; for (int t = 0; t < n; t++) row += (int64_t)sizes[t] * inner;
-  int64_t off = 0;
-  for (int t = 0; t < n; t++) {
-    int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
-    if (tot > 0 && h_ind[t]) hipLaunchKernelGGL((k_concat<true>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
-    off += st;
-  }
-  LH_CHECK_LAUNCH();
+  lh_concat_grad_beta(n, h_ind, nullptr, sizes, outd, outer, inner);
 }
 
 }  // extern "C"

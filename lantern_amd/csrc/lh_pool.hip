@@ -13,12 +13,18 @@ constexpr int TPB = 256;
 template <bool S2, bool K3>
 __global__ void __launch_bounds__(TPB) k_maxpool_fwd(const float* __restrict__ x, float* __restrict__ y, int* __restrict__ idx,
                                                      int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t rows) {
-  const int ry = threadIdx.x / 64, lane = threadIdx.x & 63;            // four rows per block, a wavefront each
-  for (int64_t row = (int64_t)blockIdx.x * 4 + ry; row < rows; row += (int64_t)gridDim.x * 4) {
+  // A wavefront per output row; rows narrower than half a wavefront share one (G rows side by side), so that the
+  // 16x16 and 8x8 maps of small networks still fill the lanes.
+  const int ry = threadIdx.x / 64, lane = threadIdx.x & 63;
+  const int G = oW > 32 ? 1 : 64 / oW;
+  const int lr = G > 1 ? lane / oW : 0, lq = G > 1 ? lane - lr * oW : lane;
+  for (int64_t row0 = ((int64_t)blockIdx.x * 4 + ry) * G; row0 < rows; row0 += (int64_t)gridDim.x * 4 * G) {
+    const int64_t row = row0 + lr;
+    if (lr >= G || row >= rows) continue;
     const int p = (int)(row % oH); const int64_t nc = row / oH;
     const int64_t base = nc * H * W;
     const int h0 = (S2 ? 2 * p : p * sH) - pad;
-    for (int q = lane; q < oW; q += 64) {
+    for (int q = lq; q < oW; q += 64) {
       const int w0 = (S2 ? 2 * q : q * sW) - pad;
       float best = -3.402823466e+38f; int bi = 0;
       if (K3) {
@@ -65,13 +71,17 @@ __global__ void __launch_bounds__(TPB) k_maxpool_bwd_dense(const float* __restri
                                                            int H, int W, int oH, int oW, int kH, int kW, int sH, int sW, int pad, int64_t rows) {
   // a wavefront per input row (n*C + c, h), lanes along w: one division per row; S2 folds stride (2,2) into shifts
   const int ry = threadIdx.x / 64, lane = threadIdx.x & 63;
-  for (int64_t row = (int64_t)blockIdx.x * 4 + ry; row < rows; row += (int64_t)gridDim.x * 4) {
+  const int G = W > 32 ? 1 : 64 / W;                      // narrow rows share a wavefront, as in the forward kernel
+  const int lr = G > 1 ? lane / W : 0, lw = G > 1 ? lane - lr * W : lane;
+  for (int64_t row0 = ((int64_t)blockIdx.x * 4 + ry) * G; row0 < rows; row0 += (int64_t)gridDim.x * 4 * G) {
+    const int64_t row = row0 + lr;
+    if (lr >= G || row >= rows) continue;
     const int h = (int)(row % H); const int64_t nc = row / H;
     const int hp = h + pad;
     const int p_hi = min(oH - 1, S2 ? hp >> 1 : hp / sH);
     const int p_lo = hp < kH ? 0 : (S2 ? (hp - kH) >> 1 : (hp - kH) / sH) + 1;
     const int64_t ob = nc * oH * oW;
-    for (int w = lane; w < W; w += 64) {
+    for (int w = lw; w < W; w += 64) {
       const int wp = w + pad;
       const int q_hi = min(oW - 1, S2 ? wp >> 1 : wp / sW);
       const int q_lo = wp < kW ? 0 : (S2 ? (wp - kW) >> 1 : (wp - kW) / sW) + 1;
@@ -139,7 +149,7 @@ void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, 
   int64_t n_out = (int64_t)N * C * oH * oW;
   if (n_out <= 0) return;
   const int64_t rows = (int64_t)N * C * oH;
-  const int grid = stream_grid(rows, 4);
+  const int grid = stream_grid(rows, 4 * (oW > 32 ? 1 : 64 / oW));
 #define GO(S, K) hipLaunchKernelGGL((k_maxpool_fwd<S, K>), dim3(grid), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, rows)
   const bool k3 = kH == 3 && kW == 3;
   if (sH == 2 && sW == 2) { if (k3) GO(true, true); else GO(true, false); }
@@ -164,7 +174,7 @@ void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float b
   if (n_in <= 0) return;
   const int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
   const int64_t rows = (int64_t)N * C * H;
-  const int grid = stream_grid(rows, 4);
+  const int grid = stream_grid(rows, 4 * (W > 32 ? 1 : 64 / W));
   const bool s2 = sH == 2 && sW == 2;
   const bool w2 = kH <= 2 * sH && kW <= 2 * sW;
 #define GO(A, S, T) hipLaunchKernelGGL((k_maxpool_bwd_dense<A, S, T>), dim3(grid), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, oH, oW, kH, kW, sH, sW, pad, rows)

@@ -785,7 +785,11 @@ class TensorR:
         y = TensorR._new(self.x.concat(dim, *[t.x for t in others]))
         outer, inner = _prod(self.x.shape[:dim]), _prod(self.x.shape[dim + 1:])
         sizes = [t.x.shape[dim] for t in ts]
-        _tape.append(lambda: be.concat_grad([None if t.isInput else t.d.data for t in ts], sizes, y.d.data, outer, inner))
+        def back():
+            # an input whose gradient nobody has written yet is overwritten (its buffer then needs no zero fill)
+            tg = [(None, 1.0) if t.isInput else t.grad_target() for t in ts]
+            be.concat_grad([b for b, _ in tg], sizes, y.d.data, outer, inner, [bt for _, bt in tg])
+        _tape.append(back)
         return y
 
     # -- recurrent layer, CTC ----------------------------------------------------------------------------

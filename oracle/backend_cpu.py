@@ -260,7 +260,7 @@ class BackendCPU(Backend):
         self._c("lc_concat", I(len(bufs)), ptrs, _ints(sizes), P(res.ptr), I(outer), I(inner))
         return res
 
-    def concat_grad(self, dbufs, sizes, outd, outer, inner):
+    def concat_grad(self, dbufs, sizes, outd, outer, inner, betas=None):      # host memory starts at zero: overwrite = accumulate
         # the oracle has no isInput skip: give inputs a throw-away gradient
         keep = [b if b is not None else self.mallocArray(outer * inner * s) for b, s in zip(dbufs, sizes)]
         ptrs = (C.c_void_p * len(keep))(*[b.ptr for b in keep])

@@ -299,7 +299,14 @@ def test_concat_and_grad(pair):
             y = be.concat([up(x) for x in xs], list(sizes), outer, inner)
             ds = [up(np.ones(x.size, np.float32)) for x in xs]
             be.concat_grad(ds, list(sizes), up(od), outer, inner)
-            return [down(y, od.shape)] + [down(d, x.shape) for d, x in zip(ds, xs)]
+            outs = [down(y, od.shape)] + [down(d, x.shape) for d, x in zip(ds, xs)]
+            if be.name == "hip":      # overwrite form: first input into garbage with beta 0, the others accumulate
+                ds2 = [up(np.full(x.size, 9.0 if t == 0 else 1.0, np.float32)) for t, x in enumerate(xs)]
+                be.concat_grad(ds2, list(sizes), up(od), outer, inner, [0.0] + [1.0] * (len(xs) - 1))
+                np.testing.assert_array_equal(down(ds2[0], xs[0].shape) + 1.0, outs[1])
+                for t in range(1, len(xs)):
+                    np.testing.assert_array_equal(down(ds2[t], xs[t].shape), outs[1 + t])
+            return outs
 
         outs = pair.run(f)
         np.testing.assert_array_equal(outs[1][0], np.concatenate(xs, 1))
