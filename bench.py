@@ -94,7 +94,7 @@ def run_gpu(args):
     lib.lh_prof_enable((1 << CATS.index("cmdlist")) if getattr(tr, "batching", False) else (0b1111 | (1 << CATS.index("rnn"))))
     ms = (C.c_double * len(CATS))(); calls = (C.c_int64 * len(CATS))()
     lib.lh_prof_collect(ms, calls, len(CATS))       # reset
-    be.work = {}
+    be.work = {}; be.count_work = True
     for _ in range(args.steps):
         tr.step()
         tr.end_step()
@@ -102,6 +102,7 @@ def run_gpu(args):
     lib.lh_prof_collect(ms, calls, len(CATS))
     timed = {CATS[i]: (ms[i] / args.steps, int(calls[i]) // args.steps) for i in range(len(CATS))}
     work = {k: v / args.steps for k, v in be.work.items()}
+    be.count_work = False
     # a separate, untimed pass with every category instrumented (breakdown for the log)
     lib.lh_prof_enable((1 << CATS.index("cmdlist")) if getattr(tr, "batching", False) else (1 << len(CATS)) - 1)
     tr.step(); tr.end_step()

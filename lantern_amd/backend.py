@@ -154,7 +154,8 @@ class BackendHIP(Backend):
         self.side_order = int(os.environ.get("LH_SIDE_ORDER", "1"))
         self.side_min_ops = int(os.environ.get("LH_SIDE_MIN_OPS", "6"))
         self.dropout_offset = 0
-        self.work = {}            # algorithmic flop / bytes issued, by kind (read by the benchmark; a few adds per call)
+        self.work = {}            # algorithmic flop / bytes issued, by kind, while count_work is on (the benchmark's profiled pass)
+        self.count_work = False
 
     def _count(self, kind, amount):
         self.work[kind] = self.work.get(kind, 0.0) + amount
@@ -165,6 +166,7 @@ class BackendHIP(Backend):
         self.lib.lh_set_error_mode(1)
         self.lib.lh_setup(self.heap_bytes)
         _lib.check()
+        self._chunk_ptr, self._chunk_left = 0, 0
 
     def cleanup(self):
         if self.lib is not None:
@@ -199,14 +201,32 @@ class BackendHIP(Backend):
 
     def mallocArray(self, length, zero=True):
         n = int(length) if length > 0 else 1
+        nb = (4 * n + 255) & -256
+        if nb <= self.SMALL_BLOCK:
+            # Small blocks are cut from a zero-filled 1 MiB block of the arena on this side of the boundary: a TreeLSTM
+            # tree asks for ~1900 blocks of a few hundred bytes, and a foreign call costs more than everything else
+            # this method does.  Generated C++ calls lh_malloc directly.
+            if nb > self._chunk_left:
+                self._chunk_ptr = self.lib.lh_malloc(self.CHUNK)
+                _lib.check()
+                self._chunk_left = self.CHUNK
+            p = self._chunk_ptr
+            self._chunk_ptr = p + nb
+            self._chunk_left -= nb
+            return Buf(p, n)
         p = (self.lib.lh_malloc if zero else self.lib.lh_malloc_uninit)(4 * n)
         _lib.check()
         return Buf(p, n)
 
+    SMALL_BLOCK = 1 << 16
+    CHUNK = 1 << 20
+
     def getMallocAddr(self):
+        self._chunk_left = 0        # what is handed out from here on lies above the mark
         return self.lib.lh_mark()
 
     def resetMallocAddr(self, addr):
+        self._chunk_left = 0
         self.lib.lh_rewind(addr); _lib.check()
 
     def copyFloatArray(self, dest, src, length):
@@ -252,13 +272,13 @@ class BackendHIP(Backend):
     def matrixVectorDot(self, x, y, m, n):
         res = self.mallocArray(m, zero=False)
         self.lib.lh_sgemv(0, m, n, 1.0, x.ptr, n, y.ptr, 0.0, res.ptr); _lib.check()
-        self._count("gemv_flop", 2.0 * m * n); self._count("gemv_bytes", 4.0 * m * n)
+        if self.count_work: self._count("gemv_flop", 2.0 * m * n); self._count("gemv_bytes", 4.0 * m * n)
         return res
 
     def matrixMatrixDot(self, x, y, m, k, n):
         res = self.mallocArray(m * n, zero=False)
         self.lib.lh_sgemm(0, 0, m, n, k, 1.0, x.ptr, k, y.ptr, n, 0.0, res.ptr, n); _lib.check()
-        self._count("gemm_flop", 2.0 * m * n * k)
+        if self.count_work: self._count("gemm_flop", 2.0 * m * n * k)
         return res
 
     def addMul_scalar(self, xd, s, y, n):           # x.d.addMul(output.d.data(0), y.x)  (CPU:174-175)
@@ -266,26 +286,26 @@ class BackendHIP(Backend):
 
     def add_cartesian(self, xd, y, outd, m, n):     # xd[m,n] += outd[m] (x) y[n]
         self.lib.lh_ger(m, n, outd.ptr, y.ptr, xd.ptr); _lib.check()
-        self._count("gemv_flop", 2.0 * m * n); self._count("gemv_bytes", 8.0 * m * n)
+        if self.count_work: self._count("gemv_flop", 2.0 * m * n); self._count("gemv_bytes", 8.0 * m * n)
 
     def add_composition(self, xd, y, outd, m, n):   # xd[n] += y[m,n]^T outd[m]
         self.lib.lh_sgemv(1, m, n, 1.0, y.ptr, n, outd.ptr, 1.0, xd.ptr); _lib.check()
-        self._count("gemv_flop", 2.0 * m * n); self._count("gemv_bytes", 4.0 * m * n)
+        if self.count_work: self._count("gemv_flop", 2.0 * m * n); self._count("gemv_bytes", 4.0 * m * n)
 
     def add_dotTrans1(self, xd, y, outd, d1, d2, d3):  # xd[d2,d3] += y[d1,d2]^T outd[d1,d3]
         self.lib.lh_sgemm(1, 0, d2, d3, d1, 1.0, y.ptr, d2, outd.ptr, d3, 1.0, xd.ptr, d3); _lib.check()
-        self._count("gemm_flop", 2.0 * d1 * d2 * d3)
+        if self.count_work: self._count("gemm_flop", 2.0 * d1 * d2 * d3)
 
     def add_dotTrans2(self, xd, y, outd, d1, d2, d3):  # xd[d1,d2] += y[d1,d3] outd[d2,d3]^T
         self.lib.lh_sgemm(0, 1, d1, d2, d3, 1.0, y.ptr, d3, outd.ptr, d3, 1.0, xd.ptr, d2); _lib.check()
-        self._count("gemm_flop", 2.0 * d1 * d2 * d3)
+        if self.count_work: self._count("gemm_flop", 2.0 * d1 * d2 * d3)
 
     # -- gemm (TD:279-280; CUB:589-688): result [d1,d3], contraction d2 --------------------------
     def gemm(self, x, tx, y, ty, alpha, d1, d2, d3):
         res = self.mallocArray(d1 * d3, zero=False)
         self.lib.lh_sgemm(int(tx), int(ty), d1, d3, d2, alpha, x.ptr, d1 if tx else d2, y.ptr, d2 if ty else d3, 0.0, res.ptr, d3)
         _lib.check()
-        self._count("gemm_flop", 2.0 * d1 * d2 * d3)
+        if self.count_work: self._count("gemm_flop", 2.0 * d1 * d2 * d3)
         return res
 
     def gemm_grad(self, x, xd, x_in, tx, y, yd, y_in, ty, alpha, od, d1, d2, d3, xbeta=1.0, ybeta=1.0):
@@ -304,7 +324,7 @@ class BackendHIP(Backend):
             if not x_in: g(1, 1, d2, d1, d3, alpha, y.ptr, d2, od.ptr, d3, xbeta, xd.ptr, d1)
             if not y_in: g(1, 1, d3, d2, d1, alpha, od.ptr, d3, x.ptr, d1, ybeta, yd.ptr, d2)
         _lib.check()
-        self._count("gemm_flop", 2.0 * d1 * d2 * d3 * ((not x_in) + (not y_in)))
+        if self.count_work: self._count("gemm_flop", 2.0 * d1 * d2 * d3 * ((not x_in) + (not y_in)))
 
     # -- broadcast arithmetic (TD:222-270) ---------------------------------------------------------
     def bcast_op(self, op, a, ashape, b, bshape, oshape):
@@ -349,19 +369,19 @@ class BackendHIP(Backend):
         P, Q = conv_size(H, R, sH, pH), conv_size(W, S, sW, pW)
         y = self.mallocArray(N * K * P * Q, zero=False)
         self.lib.lh_conv2d_fwd(x.ptr, w.ptr, bias.ptr if bias is not None else 0, y.ptr, N, C, H, W, K, R, S, sH, sW, pH, pW); _lib.check()
-        self._count("conv_flop", 2.0 * N * K * C * R * S * P * Q)
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * P * Q)
         return y, None      # no im2col buffer is kept (BackendCudnn returns None too, CDN:859-866)
 
     def conv2D_batch_into(self, x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW):
         self.lib.lh_conv2d_fwd(x.ptr, w.ptr, bias.ptr if bias is not None else 0, y.ptr, N, C, H, W, K, R, S, sH, sW, pH, pW); _lib.check()
-        self._count("conv_flop", 2.0 * N * K * C * R * S * conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW))
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW))
 
     def conv2D_batch_bn_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, ybn, sm, si, relu, eps=1e-5, factor=0.1):
         N, C, H, W, K, R, S, sH, sW, pH, pW = dims
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
         self.lib.lh_conv2d_fwd_bnstats(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, eps, factor)
         self.lib.lh_bn_apply(yconv.ptr, scale.ptr, bbias.ptr, sm.ptr, si.ptr, ybn.ptr, N, K, HW, int(relu)); _lib.check()
-        self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
         # The filter gradient is read by the optimizer only: it goes to the side stream, where it runs beside the
@@ -382,7 +402,7 @@ class BackendHIP(Backend):
             if so: self.lib.lh_side_end()
         _lib.check()
         P, Q = conv_size(H, R, sH, pH), conv_size(W, S, sW, pW)
-        self._count("conv_flop", 2.0 * N * K * C * R * S * P * Q * (1 if x_in else 2))
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * P * Q * (1 if x_in else 2))
 
     def maxPool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW, pad):
         P, Q = conv_size(H, kH, sH, pad), conv_size(W, kW, sW, pad)
@@ -443,7 +463,7 @@ class BackendHIP(Backend):
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
         self.lib.lh_conv2d_fwd_bnstats(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, eps, factor)
         self.lib.lh_bn_apply_add_relu(yconv.ptr, scale.ptr, bbias.ptr, sm.ptr, si.ptr, shortcut.ptr, out.ptr, N, K, HW); _lib.check()
-        self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def batchNorm_add_relu_grad(self, x, xd, beta_dx, out, dout, scale, scaled, biasd, sm, si, sd, beta_sd, N, C, HW):
         self.lib.lh_bn_bwd_add_relu(x.ptr, out.ptr, dout.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, beta_dx,
@@ -547,13 +567,13 @@ class BackendHIP(Backend):
     def rnn_forward(self, mode, x, w, T, B, I, H, bidir):
         y = self.mallocArray(T * B * H * (2 if bidir else 1), zero=False)
         self.lib.lh_rnn_fwd(mode, x.ptr, w.ptr, y.ptr, T, B, I, H, int(bidir)); _lib.check()
-        self._count("gemm_flop", 2.0 * T * B * H * I * (2 if bidir else 1)); self._count("rnn_flop", 2.0 * T * B * H * H * (2 if bidir else 1))
+        if self.count_work: self._count("gemm_flop", 2.0 * T * B * H * I * (2 if bidir else 1)); self._count("rnn_flop", 2.0 * T * B * H * H * (2 if bidir else 1))
         return y
 
     def rnn_backward(self, mode, x, y, dy, w, dx, dw, T, B, I, H, bidir, beta_dx=1.0):
         self.lib.lh_rnn_bwd(mode, x.ptr, y.ptr, dy.ptr, w.ptr, dx.ptr if dx is not None else 0, beta_dx, dw.ptr, T, B, I, H, int(bidir)); _lib.check()
         D = 2 if bidir else 1
-        self._count("gemm_flop", 2.0 * T * B * H * D * (I * (2 if dx is not None else 1) + H)); self._count("rnn_flop", 2.0 * T * B * H * H * D)
+        if self.count_work: self._count("gemm_flop", 2.0 * T * B * H * D * (I * (2 if dx is not None else 1) + H)); self._count("rnn_flop", 2.0 * T * B * H * H * D)
 
     # -- optimizers ----------------------------------------------------------------------------------------
     def sgd_update(self, x, d, lr, n):

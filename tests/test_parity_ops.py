@@ -534,24 +534,32 @@ def test_sgemm_few_tiles_long_reduction_with_row_stride(on_hip, tt, beta):
 
 
 # ---- arena and error path (the library's own behaviour; no oracle counterpart) -----------------------
+def _arena_block(be, n, zero=True):
+    """A block straight from the library's arena (BackendHIP.mallocArray cuts small blocks from larger ones itself)."""
+    from lantern_amd import _lib
+    p = (be.lib.lh_malloc if zero else be.lib.lh_malloc_uninit)(4 * n)
+    _lib.check()
+    return B.Buf(p, n)
+
+
 def test_arena_zeroing_alignment_rewind_and_overflow(on_hip):
     be = on_hip
     lib = be.lib
     mark = be.getMallocAddr()
-    a = be.mallocArray(1000)
+    a = _arena_block(be, 1000)
     assert a.ptr % 256 == 0 and not be.toHost(a, 1000).any()
     be.fillInPlace(a, 1000, 3.0)
     used = lib.lh_heap_used()
-    b = be.mallocArray(10)
+    b = _arena_block(be, 10)
     assert b.ptr % 256 == 0 and b.ptr >= a.ptr + 4000 and lib.lh_heap_used() > used
     be.resetMallocAddr(mark)
-    c = be.mallocArray(1000)
+    c = _arena_block(be, 1000)
     assert c.ptr == a.ptr and not be.toHost(c, 1000).any()        # memory handed out again starts at zero (CUB:22-25 memset on rewind)
     be.resetMallocAddr(mark)
     with pytest.raises(LanternHipError):
         be.mallocArray(be.heap_bytes)                              # 4x the arena: refused, nothing allocated
     assert lib.lh_heap_used() <= used                              # nothing was taken by the refused request
-    z = be.mallocArray(4); assert not be.toHost(z, 4).any()        # the library keeps working after an error
+    z = _arena_block(be, 4); assert not be.toHost(z, 4).any()      # the library keeps working after an error
     be.resetMallocAddr(mark)
 
 
@@ -561,19 +569,45 @@ def test_arena_small_blocks_read_zero_after_dirty_memory_uninit_blocks_and_pops(
     be = on_hip
     lib = be.lib
     mark = be.getMallocAddr()
-    big = be.mallocArray(1 << 20, zero=False); be.fillInPlace(big, 1 << 20, 7.0)          # 4 MiB of sevens
+    big = _arena_block(be, 1 << 20, zero=False); be.fillInPlace(big, 1 << 20, 7.0)          # 4 MiB of sevens
     be.resetMallocAddr(mark)
-    blocks = [be.mallocArray(n) for n in (3, 150, 45000, 1, 300000, 64, 150)]            # crosses several windows
+    blocks = [_arena_block(be, n) for n in (3, 150, 45000, 1, 300000, 64, 150)]            # crosses several windows
     for blk, n in zip(blocks, (3, 150, 45000, 1, 300000, 64, 150)):
         assert not be.toHost(blk, n).any()
         be.fillInPlace(blk, n, 5.0)
     top = lib.lh_heap_used()
-    s = be.mallocArray(5000, zero=False); be.fillInPlace(s, 5000, 9.0)                    # scratch inside the cleared window
+    s = _arena_block(be, 5000, zero=False); be.fillInPlace(s, 5000, 9.0)                    # scratch inside the cleared window
     lib.lh_free_top(5000 * 4)
     assert lib.lh_heap_used() == top
-    z = be.mallocArray(5000); assert z.ptr == s.ptr and not be.toHost(z, 5000).any()
-    u = be.mallocArray(100, zero=False); be.fillInPlace(u, 100, 2.0)
-    z2 = be.mallocArray(100); assert not be.toHost(z2, 100).any() and (be.toHost(u, 100) == 2.0).all()
+    z = _arena_block(be, 5000); assert z.ptr == s.ptr and not be.toHost(z, 5000).any()
+    u = _arena_block(be, 100, zero=False); be.fillInPlace(u, 100, 2.0)
+    z2 = _arena_block(be, 100); assert not be.toHost(z2, 100).any() and (be.toHost(u, 100) == 2.0).all()
+    be.resetMallocAddr(mark)
+
+
+def test_mirror_cuts_small_blocks_from_zeroed_arena_blocks_and_drops_them_at_marks(on_hip):
+    """BackendHIP.mallocArray: small blocks come 256-byte aligned out of one 1 MiB arena block, read zero even after the
+    memory was dirty, never straddle a mark, and large blocks still come straight from the arena."""
+    be = on_hip
+    mark = be.getMallocAddr()
+    dirty = _arena_block(be, 1 << 19, zero=False); be.fillInPlace(dirty, 1 << 19, 4.0)      # 2 MiB of fours
+    be.resetMallocAddr(mark)
+    used0 = be.lib.lh_heap_used()
+    a = be.mallocArray(150); b = be.mallocArray(1, zero=False); c = be.mallocArray(16000)
+    assert be.lib.lh_heap_used() == used0 + be.CHUNK
+    assert a.ptr % 256 == 0 and b.ptr == a.ptr + 768 and c.ptr == b.ptr + 256
+    for blk, n in ((a, 150), (b, 1), (c, 16000)):
+        assert not be.toHost(blk, n).any()
+    be.fillInPlace(c, 16000, 1.0)
+    m2 = be.getMallocAddr()
+    d = be.mallocArray(150)
+    assert d.ptr == a.ptr + be.CHUNK and not be.toHost(d, 150).any()                        # a fresh block above the mark
+    big = be.mallocArray(1 << 18)
+    assert big.ptr == d.ptr + be.CHUNK and not be.toHost(big, 1 << 18).any()
+    be.resetMallocAddr(m2)
+    e = be.mallocArray(150)
+    assert e.ptr == d.ptr and not be.toHost(e, 150).any()
+    assert (be.toHost(c, 16000) == 1.0).all()
     be.resetMallocAddr(mark)
 
 
