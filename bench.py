@@ -48,6 +48,10 @@ def make_trainer(args, batch, cpu=False):
         return Trainer(batch=batch, lr=0.0005), batch, "LeNet-style CNN training step (configs[0]): batch %d, 1x28x28, SGD lr 0.0005, dropout 0.5" % batch
     if w == "treelstm":
         from lantern_amd.apps.treelstm import Trainer
+        if args.tree_file:
+            from lantern_amd.apps.treelstm import read_trees
+            return Trainer(vocab=20000, trees=read_trees(args.tree_file)), 1, \
+                "TreeLSTM sentiment step (configs[1]): one tree of %s per step, hidden 150, embedding 300, Adagrad lr 0.05" % os.path.basename(args.tree_file)
         return Trainer(n_trees=64, vocab=20000), 1, \
             "TreeLSTM sentiment step (configs[1]): one tree of 5-50 leaves per step, hidden 150, embedding 300, Adagrad lr 0.05"
     if w == "deepspeech2":
@@ -165,6 +169,7 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--tree-file", default=None, help="treelstm: trees in the reference's array_tree.txt format instead of random ones (tests/golden/array_tree_first24.txt)")
     ap.add_argument("--no-side-stream", action="store_true", help="filter gradients in line on the main stream (kernel profiles: no two kernels overlap)")
     ap.add_argument("--graph", action="store_true", help="time replays of the step recorded into a HIP graph (fixed-shape workloads)")
     ap.add_argument("--verbose", action="store_true")

@@ -121,6 +121,16 @@ def test_treelstm_10_trees(hip_backend, cpu_backend, batching):
     assert (rec > 10000) if batching else (rec == 0), "commands recorded: %d" % rec
 
 
+def test_treelstm_reference_tree_shapes(hip_backend, cpu_backend):
+    """The first trees of the reference's own evaluation set (tests/golden/array_tree_first24.txt: 8 to 34 leaves, the
+    real left/right structure and labels; word ids folded into a synthetic embedding table), command list on."""
+    import os
+    from lantern_amd.apps.treelstm import Trainer, read_trees
+    trees = read_trees(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "array_tree_first24.txt"))
+    assert len(trees) == 24 and [len(t[0]) for t in trees[:3]] == [25, 25, 47]
+    _compare(lambda: Trainer(vocab=500, trees=trees[:8]), hip_backend, cpu_backend, steps=8)
+
+
 def test_deepspeech2_5_steps(hip_backend, cpu_backend):
     """conv(41x11, 21x11 strided) + BN + hardTanh, permute, two bidirectional tanh RNN layers with sequence-wise BN,
     BatchNorm1D + linear, softmax, CTC; Nesterov momentum.  Reduced sizes so that the oracle finishes in seconds."""
