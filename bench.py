@@ -74,6 +74,7 @@ def run_gpu(args):
     for _ in range(args.warmup):
         tr.step(); tr.end_step()
     be.sync()
+    t_issued = None
     if args.graph:
         # the step recorded once (after the warm-up measured the launch plans) and replayed: one host call per step
         g = la.StepGraph(tr, eager_steps=0)
@@ -90,6 +91,7 @@ def run_gpu(args):
         for _ in range(args.steps):
             tr.step()
             tr.end_step()
+        t_issued = time.perf_counter()      # the host has enqueued everything; the device may still be working
         be.sync()
         t1 = time.perf_counter()
     # the same `steps` steps again with a HIP event pair around every matrix-kernel launch (conv x3, gemm, rnn).
@@ -116,7 +118,7 @@ def run_gpu(args):
     loss_val = float(tr.step().toCPU()[0]); tr.end_step()
     peak_gb = lib.lh_heap_peak() / 2 ** 30
     be.cleanup()
-    return {"sec": t1 - t0, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "arena_peak_gib": peak_gb,
+    return {"sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "arena_peak_gib": peak_gb,
             "per_step": per_step, "desc": desc}
 
 
@@ -218,6 +220,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": g["desc"], "global_batch": args.batch, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
                    "launch": "hip graph replay" if args.graph else "one launch per kernel",
+                   "host_issue_ms_per_step": round(1000.0 * g["issue_sec"] / args.steps, 3) if g["issue_sec"] is not None else None,
                    "filter_gradients": "in line" if args.no_side_stream else "side stream"},
         "roofline": roof,
     }

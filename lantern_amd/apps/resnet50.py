@@ -56,7 +56,7 @@ class ResNet50(Module):
         self.imagenet_stem = imagenet_stem
         if imagenet_stem:
             self.conv1 = self.add(Conv2D(3, 64, (7, 7), (2, 2), (3, 3), useBias=False, name="conv1", init=ini))
-        else:   # the reference's CIFAR variant: 3x3 stride-1 stem (resnet50.py:101-103)
+        else:   # the reference's CIFAR variant: 3x3 stride-1 stem and a 2x2 max-pool (resnet50.py:101-104)
             self.conv1 = self.add(Conv2D(3, 64, (3, 3), (1, 1), (1, 1), useBias=False, name="conv1", init=ini))
         self.bn1 = self.add(BatchNorm2D(64, "bn1"))
         self.blocks = []
@@ -75,6 +75,8 @@ class ResNet50(Module):
         h = self.bn1(self.conv1(x)).relu(True)
         if self.imagenet_stem:
             h = h.maxPoolBK((3, 3), (2, 2), (1, 1, 1, 1))
+        else:                       # resnet50.py:104: MaxPool2d(2, 2), 32x32 -> 16x16 before layer1
+            h = h.maxPoolBK((2, 2), (2, 2), None)
         for blk in self.blocks:
             h = blk(h)
         hw = h.x.shape[2]

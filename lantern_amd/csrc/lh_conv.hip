@@ -338,8 +338,9 @@ static bool launch_rounds(const AL& al, const BL& bl, const EP& ep, int M, int N
 
 // The launch plans of a forward / input-gradient product.  0: the built-in rule (stream-K for few tiles over a long
 // reduction, else the tile pick_tile_conv names).  1-3: plain tiles 128x128, 64x128, 64x64.  4-7: stream-K over
-// 128x128 / 64x128 tiles with two or three workers per CU.
-constexpr int N_PLANS = 8;
+// 128x128 / 64x128 tiles with two or three workers per CU.  8-9: stream-K over 64x64 tiles with four or eight workers per
+// CU, for products so small that even their 64x64 tiles leave most CUs with one block whose loads nothing hides.
+constexpr int N_PLANS = 10;
 template <class AL, class BL, class EP>
 static bool plan_valid(int plan, const EP& ep, int M, int K, bool can_zero) {
   if (plan == 0) return true;
@@ -350,8 +351,9 @@ static bool plan_valid(int plan, const EP& ep, int M, int K, bool can_zero) {
 template <class AL, class BL, class EP>
 static bool launch_plan(int plan, const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out, int64_t zero_n, bool prezeroed) {
   if (plan >= 4) {
-    const int workers = (plan >= 6 ? 3 : 2) * g_num_cu;
+    const int workers = (plan >= 8 ? (plan == 8 ? 4 : 8) : (plan >= 6 ? 3 : 2)) * g_num_cu;
     if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
+    if (plan >= 8) return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
     if (plan == 4 || plan == 6) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
     return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
   }

@@ -85,8 +85,10 @@ def test_resnet_bottlenecks_10_steps(hip_backend, cpu_backend):
     """The ResNet-50 program (reference's 32x32 variant, one bottleneck per stage to keep the oracle
     fast; every op kind of the headline network, momentum SGD)."""
     from lantern_amd.apps.resnet50 import ResNet50, Trainer
+    # 16 images are memorised within ten steps (loss 2.36 -> 0.03), and the last stage normalises over 16 x 2 x 2 values per
+    # channel: the two backends stay within 2e-4 absolute of each other, which is 6e-3 of the late, small losses.
     _compare(lambda: Trainer(ResNet50(num_classes=10, imagenet_stem=False, layers=(1, 1, 1, 1)), 16, 32, 10, lr=0.005, momentum=0.9),
-             hip_backend, cpu_backend, per_tensor=2e-2)
+             hip_backend, cpu_backend, per_tensor=2e-2, loss_late=1e-2)
 
 
 def test_resnet_imagenet_stem_3_steps(hip_backend, cpu_backend):
