@@ -109,6 +109,72 @@ __global__ void __launch_bounds__(TPB) k_maxpool_bwd_dense(const float* __restri
     }
   }
 }
+// The 3x3 / stride 2 / pad 1 pool of the ResNet stem, for even H and W % 4 == 0 (so oH = H/2, oW = W/2): a thread produces
+// two neighbouring outputs from one 16-byte load and one scalar load per window row (input columns 4j-1 .. 4j+3) instead
+// of nine strided scalar loads each.  Same scan order and strict comparison as the general kernel: the first maximum wins.
+__global__ void __launch_bounds__(TPB) k_maxpool_fwd_k3s2p1(const float* __restrict__ x, float* __restrict__ y, int* __restrict__ idx,
+                                                            int H, int W, int64_t total /* N*C*oH*(oW/2) */) {
+  const int oW = W >> 1, oH = H >> 1, half = oW >> 1;
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < total; i += (int64_t)gridDim.x * TPB) {
+    const int j = (int)(i % half); const int64_t row = i / half;
+    const int p = (int)(row % oH); const int64_t nc = row / oH;
+    const int64_t base = nc * H * W;
+    float v[3][5]; bool in[3];
+#pragma unroll
+    for (int r = 0; r < 3; r++) {
+      const int h = 2 * p - 1 + r;
+      in[r] = h >= 0 && h < H;
+      const int64_t o = base + (int64_t)(in[r] ? h : 0) * W + 4 * j;
+      const float4 t = *reinterpret_cast<const float4*>(x + o);
+      v[r][0] = j > 0 ? x[o - 1] : 0.f; v[r][1] = t.x; v[r][2] = t.y; v[r][3] = t.z; v[r][4] = t.w;
+    }
+    float b0 = -3.402823466e+38f, b1 = -3.402823466e+38f; int i0 = 0, i1 = 0;
+#pragma unroll
+    for (int r = 0; r < 3; r++) {
+      if (!in[r]) continue;
+      const int rowbase = (int)(base + (int64_t)(2 * p - 1 + r) * W + 4 * j);
+#pragma unroll
+      for (int t = 0; t < 3; t++) {
+        if ((t > 0 || j > 0) && v[r][t] > b0) { b0 = v[r][t]; i0 = rowbase + t - 1; }       // output 2j: columns 4j-1 .. 4j+1
+        if (v[r][t + 2] > b1) { b1 = v[r][t + 2]; i1 = rowbase + t + 1; }                     // output 2j+1: columns 4j+1 .. 4j+3
+      }
+    }
+    const int64_t o = row * oW + 2 * j;
+    *reinterpret_cast<float2*>(y + o) = make_float2(b0, b1);
+    *reinterpret_cast<int2*>(idx + o) = make_int2(i0, i1);
+  }
+}
+// Its backward as a gather: a thread owns the 2x2 input cell (2i..2i+1, 2j..2j+1), which only the windows (i..i+1, j..j+1)
+// cover -- (2i,2j) lies in window (i,j) alone, (2i,2j+1) in (i,j),(i,j+1), (2i+1,2j) in (i,j),(i+1,j), the last pixel in all
+// four -- so four (argmax, dy) pairs serve four pixels.  Sums run in window order, as in the general kernel.
+template <bool ACC>
+__global__ void __launch_bounds__(TPB) k_maxpool_bwd_k3s2p1(const float* __restrict__ dy, const int* __restrict__ idx, float* __restrict__ dx,
+                                                            int H, int W, int64_t total /* N*C*(H/2)*(W/2) */) {
+  const int oW = W >> 1, oH = H >> 1;
+  for (int64_t t = (int64_t)blockIdx.x * TPB + threadIdx.x; t < total; t += (int64_t)gridDim.x * TPB) {
+    const int j = (int)(t % oW); const int64_t r = t / oW;
+    const int i = (int)(r % oH); const int64_t nc = r / oH;
+    const int64_t ob = nc * oH * oW, ib = nc * H * W;
+    const bool pd = i + 1 < oH, qd = j + 1 < oW;
+    const int64_t o00 = ob + (int64_t)i * oW + j, o01 = qd ? o00 + 1 : o00, o10 = pd ? o00 + oW : o00, o11 = pd ? o01 + oW : o01;
+    const int a00 = idx[o00], a01 = idx[o01], a10 = idx[o10], a11 = idx[o11];
+    const float g00 = dy[o00], g01 = dy[o01], g10 = dy[o10], g11 = dy[o11];
+    const int e00 = (int)(ib + (int64_t)(2 * i) * W + 2 * j), e01 = e00 + 1, e10 = e00 + W, e11 = e10 + 1;
+    float s00 = 0.f, s01 = 0.f, s10 = 0.f, s11 = 0.f;
+    if (a00 == e00) s00 += g00;
+    if (a00 == e01) s01 += g00;
+    if (qd && a01 == e01) s01 += g01;
+    if (a00 == e10) s10 += g00;
+    if (pd && a10 == e10) s10 += g10;
+    if (a00 == e11) s11 += g00;
+    if (qd && a01 == e11) s11 += g01;
+    if (pd && a10 == e11) s11 += g10;
+    if (pd && qd && a11 == e11) s11 += g11;
+    float2* d0 = reinterpret_cast<float2*>(dx + e00); float2* d1 = reinterpret_cast<float2*>(dx + e10);
+    if (ACC) { const float2 u0 = *d0, u1 = *d1; s00 += u0.x; s01 += u0.y; s10 += u1.x; s11 += u1.y; }
+    *d0 = make_float2(s00, s01); *d1 = make_float2(s10, s11);
+  }
+}
 __global__ void __launch_bounds__(TPB) k_avgpool_fwd(const float* __restrict__ x, float* __restrict__ y, int H, int W, int oH, int oW,
                                                      int kH, int kW, int sH, int sW, int64_t n_out) {
   const float ks = (float)(kH * kW);
@@ -136,6 +202,23 @@ __global__ void __launch_bounds__(TPB) k_avgpool_bwd(const float* __restrict__ d
     if (any) dx[i] += acc;
   }
 }
+// Global average pooling (the window is the whole map, one output per channel image): a wavefront per image with
+// coalesced loads; the general kernel would walk each image with one thread.
+__global__ void __launch_bounds__(TPB) k_avgpool_global_fwd(const float* __restrict__ x, float* __restrict__ y, int HW, int64_t rows) {
+  const int lane = threadIdx.x & 63;
+  const float ks = (float)HW;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); row < rows; row += (int64_t)gridDim.x * 4) {
+    const float* xp = x + row * HW;
+    float a = 0.f;
+    for (int l = lane; l < HW; l += 64) a += xp[l];
+    a = lh_wave_sum(a);
+    if (lane == 0) y[row] = a / ks;
+  }
+}
+__global__ void __launch_bounds__(TPB) k_avgpool_global_bwd(const float* __restrict__ dy, float* dx, int HW, int64_t n_in) {
+  const float ks = (float)HW;
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n_in; i += (int64_t)gridDim.x * TPB) dx[i] += dy[i / HW] / ks;
+}
 }  // namespace
 
 extern "C" {
@@ -148,6 +231,12 @@ void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, 
   int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
   int64_t n_out = (int64_t)N * C * oH * oW;
   if (n_out <= 0) return;
+  if (kH == 3 && kW == 3 && sH == 2 && sW == 2 && pad == 1 && (H & 1) == 0 && (W & 3) == 0 && ((((uintptr_t)x | (uintptr_t)y | (uintptr_t)argmax) & 15) == 0)) {
+    const int64_t total = (int64_t)N * C * oH * (oW / 2);
+    hipLaunchKernelGGL(k_maxpool_fwd_k3s2p1, dim3(stream_grid(total, TPB)), dim3(TPB), 0, g_stream, x, y, argmax, H, W, total);
+    LH_CHECK_LAUNCH();
+    return;
+  }
   const int64_t rows = (int64_t)N * C * oH;
   const int grid = stream_grid(rows, 4 * (oW > 32 ? 1 : 64 / oW));
 #define GO(S, K) hipLaunchKernelGGL((k_maxpool_fwd<S, K>), dim3(grid), dim3(TPB), 0, g_stream, x, y, argmax, H, W, oH, oW, kH, kW, sH, sW, pad, rows)
@@ -173,6 +262,13 @@ void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float b
   LH_REQUIRE(n_in < 2147483647LL, "lh_maxpool_bwd_dense: input too large for int32 argmax");
   if (n_in <= 0) return;
   const int oH = (H + 2 * pad - kH) / sH + 1, oW = (W + 2 * pad - kW) / sW + 1;
+  if (kH == 3 && kW == 3 && sH == 2 && sW == 2 && pad == 1 && (H & 1) == 0 && (W & 1) == 0 && (((uintptr_t)dx & 7) == 0)) {
+    const int64_t total = (int64_t)N * C * (H / 2) * (W / 2);
+    if (beta == 0.f) hipLaunchKernelGGL((k_maxpool_bwd_k3s2p1<false>), dim3(stream_grid(total, TPB)), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, total);
+    else hipLaunchKernelGGL((k_maxpool_bwd_k3s2p1<true>), dim3(stream_grid(total, TPB)), dim3(TPB), 0, g_stream, dy, argmax, dx, H, W, total);
+    LH_CHECK_LAUNCH();
+    return;
+  }
   const int64_t rows = (int64_t)N * C * H;
   const int grid = stream_grid(rows, 4 * (W > 32 ? 1 : 64 / W));
   const bool s2 = sH == 2 && sW == 2;
@@ -190,7 +286,8 @@ void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH
   int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
   int64_t n_out = (int64_t)N * C * oH * oW;
   if (n_out <= 0) return;
-  hipLaunchKernelGGL(k_avgpool_fwd, dim3(stream_grid(n_out, TPB)), dim3(TPB), 0, g_stream, x, y, H, W, oH, oW, kH, kW, sH, sW, n_out);
+  if (kH == H && kW == W) hipLaunchKernelGGL(k_avgpool_global_fwd, dim3(stream_grid(n_out, 4)), dim3(TPB), 0, g_stream, x, y, H * W, n_out);
+  else hipLaunchKernelGGL(k_avgpool_fwd, dim3(stream_grid(n_out, TPB)), dim3(TPB), 0, g_stream, x, y, H, W, oH, oW, kH, kW, sH, sW, n_out);
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {
@@ -199,7 +296,8 @@ void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int 
   int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
   int64_t n_in = (int64_t)N * C * H * W;
   if (n_in <= 0) return;
-  hipLaunchKernelGGL(k_avgpool_bwd, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, dy, dx, H, W, oH, oW, kH, kW, sH, sW, n_in);
+  if (kH == H && kW == W) hipLaunchKernelGGL(k_avgpool_global_bwd, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, dy, dx, H * W, n_in);
+  else hipLaunchKernelGGL(k_avgpool_bwd, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, dy, dx, H, W, oH, oW, kH, kW, sH, sW, n_in);
   LH_CHECK_LAUNCH();
 }
 

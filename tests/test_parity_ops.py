@@ -147,7 +147,8 @@ POOLS = [(64, 64, 112, 112, 3, 3, 2, 2, 1),     # ResNet stem
          (2, 3, 10, 10, 2, 2, 3, 3, 0),          # stride above the window: pixels no window covers
          (2, 4, 9, 9, 3, 3, 1, 1, 1),            # 3x3 stride 1: three windows per direction over a pixel
          (1, 2, 11, 11, 5, 5, 2, 2, 2),          # 5x5 stride 2
-         (2, 2, 70, 70, 3, 3, 2, 2, 1)]          # rows wider than a wavefront
+         (2, 2, 70, 70, 3, 3, 2, 2, 1),          # rows wider than a wavefront
+         (2, 3, 8, 12, 3, 3, 2, 2, 1), (1, 2, 6, 4, 3, 3, 2, 2, 1), (3, 5, 30, 36, 3, 3, 2, 2, 1)]      # 3x3/2 pad 1 on even maps: the paired-output kernels (as the ResNet stem)
 
 
 POOLS += _random_cases(102, 16, _gen_pool)
