@@ -256,6 +256,14 @@ void lh_bn_stats(const float* x, float* save_mean, float* save_invstd, float* ru
                  int N, int C, int HW, float eps, float factor);
 void lh_bn_apply(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd, float* y,
                  int N, int C, int HW, int relu);
+/* Both in one call: y = conv(x, w) and out = bn(y) with relu when `relu` != 0, or, with a shortcut, the residual join
+ * out = relu(bn(y) + shortcut).  Same results as lh_conv2d_fwd_bnstats followed by lh_bn_apply / lh_bn_apply_add_relu (bit for
+ * bit wherever two launches of the convolution itself agree bit for bit); where the convolution's epilogue leaves the partial sums, the normalisation pass adds them up itself (every block for
+ * its channel), so no statistics kernel runs between the two. */
+void lh_conv2d_fwd_bn_apply(const float* x, const float* w, const float* bias, float* y,
+                            int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW,
+                            const float* gamma, const float* beta, float* save_mean, float* save_invstd, float* run_mean, float* run_var,
+                            float eps, float factor, const float* shortcut, float* out, int relu);
 
 /* The residual join behind a batch norm (ResNet's bn3 -> Add -> Relu; the reference runs cudnnBatchNormalizationForwardTraining,
  * an element-wise add kernel (CUB:397-420) and cudnnActivationForward, CDN:1025-1068, 1380-1400, as three passes):

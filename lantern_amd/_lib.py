@@ -90,6 +90,7 @@ SIGNATURES = {
     "lh_bn_train_fwd_relu": (None, [P, P, P, P, P, P, P, P, I, I, I, F, F]),
     "lh_bn_bwd_relu": (None, [P, P, P, P, P, P, P, P, F, P, P, I, I, I]),
     "lh_conv2d_fwd_bnstats": (None, [P, P, P, P] + [I] * 11 + [P, P, P, P, F, F]),
+    "lh_conv2d_fwd_bn_apply": (None, [P, P, P, P] + [I] * 11 + [P, P, P, P, P, P, F, F, P, P, I]),
     "lh_bn_stats": (None, [P, P, P, P, P, I, I, I, F, F]),
     "lh_bn_apply": (None, [P, P, P, P, P, P, I, I, I, I]),
     "lh_bn_apply_add_relu": (None, [P, P, P, P, P, P, P, I, I, I]),

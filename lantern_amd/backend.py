@@ -379,8 +379,8 @@ class BackendHIP(Backend):
     def conv2D_batch_bn_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, ybn, sm, si, relu, eps=1e-5, factor=0.1):
         N, C, H, W, K, R, S, sH, sW, pH, pW = dims
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
-        self.lib.lh_conv2d_fwd_bnstats(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, eps, factor)
-        self.lib.lh_bn_apply(yconv.ptr, scale.ptr, bbias.ptr, sm.ptr, si.ptr, ybn.ptr, N, K, HW, int(relu)); _lib.check()
+        self.lib.lh_conv2d_fwd_bn_apply(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, scale.ptr, bbias.ptr, sm.ptr, si.ptr,
+                                        rmean.ptr, rvar.ptr, eps, factor, 0, ybn.ptr, int(relu)); _lib.check()
         if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
@@ -461,8 +461,8 @@ class BackendHIP(Backend):
     def conv2D_batch_bn_add_relu_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, shortcut, out, sm, si, eps=1e-5, factor=0.1):
         N, C, H, W, K, R, S, sH, sW, pH, pW = dims
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
-        self.lib.lh_conv2d_fwd_bnstats(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, eps, factor)
-        self.lib.lh_bn_apply_add_relu(yconv.ptr, scale.ptr, bbias.ptr, sm.ptr, si.ptr, shortcut.ptr, out.ptr, N, K, HW); _lib.check()
+        self.lib.lh_conv2d_fwd_bn_apply(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, scale.ptr, bbias.ptr, sm.ptr, si.ptr,
+                                        rmean.ptr, rvar.ptr, eps, factor, shortcut.ptr, out.ptr, 1); _lib.check()
         if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def batchNorm_add_relu_grad(self, x, xd, beta_dx, out, dout, scale, scaled, biasd, sm, si, sd, beta_sd, N, C, HW):

@@ -236,12 +236,53 @@ __global__ void __launch_bounds__(TPB) k_bn_finalize_conv(const float* __restric
   }
 }
 
-// y = gamma * (x - mean) * invstd + beta from given statistics (optionally followed by relu)
-template <bool VEC, bool RELU>
+// Mean and 1/sqrt(var + eps) of channel c from the pieces a convolution epilogue left, computed by the whole block exactly as
+// k_bn_finalize_conv does (same partition over threads, same tree), so every block of a channel gets the same bits; the
+// owner block also stores the saved and running statistics.
+__device__ __forceinline__ void bn_stats_from_pieces(const ConvPieces& P, int c, bool owner, float& mean_out, float& invstd_out) {
+  __shared__ double sa_[TPB], sq_[TPB];
+  __shared__ float res_[2];
+  const float2* pc = reinterpret_cast<const float2*>(P.partial) + (size_t)c * P.slots;
+  double sa = 0.0, sq = 0.0;
+  for (int s = threadIdx.x; s < P.slots; s += TPB) {
+    const int j0 = s < P.slots_main ? s * P.g_main : P.col1 + (s - P.slots_main) * P.g_rem;
+    const int n = s < P.slots_main ? min(P.g_main, P.col1 - j0) : min(P.g_rem, P.ncols - j0);
+    if (n <= 0) continue;
+    const float2 pv = pc[s];
+    sa += (double)pv.x; sq += (double)pv.y;
+  }
+  sa_[threadIdx.x] = sa; sq_[threadIdx.x] = sq;
+  __syncthreads();
+  for (int off = TPB / 2; off > 0; off >>= 1) {
+    if (threadIdx.x < off) { sa_[threadIdx.x] += sa_[threadIdx.x + off]; sq_[threadIdx.x] += sq_[threadIdx.x + off]; }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const double n = (double)P.ncols, mu = sa_[0] / n;
+    double M2 = sq_[0] - sa_[0] * mu; if (M2 < 0.0) M2 = 0.0;
+    const float var = (float)(M2 / n);
+    const float is = 1.0f / sqrtf(var + P.eps);
+    res_[0] = (float)mu; res_[1] = is;
+    if (owner) {
+      if (P.save_mean) P.save_mean[c] = (float)mu;
+      if (P.save_invstd) P.save_invstd[c] = is;
+      if (P.run_mean) P.run_mean[c] = (1.0f - P.factor) * P.run_mean[c] + P.factor * (float)mu;
+      if (P.run_var) { float unb = n > 1.0 ? (float)(M2 / (n - 1.0)) : var; P.run_var[c] = (1.0f - P.factor) * P.run_var[c] + P.factor * unb; }
+    }
+  }
+  __syncthreads();
+  mean_out = res_[0]; invstd_out = res_[1];
+}
+
+// y = gamma * (x - mean) * invstd + beta from given statistics (optionally followed by relu); PIECES: the statistics come
+// from a convolution's pieces instead of save_mean / save_invstd
+template <bool VEC, bool RELU, bool PIECES = false>
 __global__ void __launch_bounds__(TPB) k_bn_apply(const float* __restrict__ x, float* __restrict__ y, const float* gamma, const float* beta,
-                                                  const float* save_mean, const float* save_invstd, int N, int C, int HW, int n_per) {
+                                                  const float* save_mean, const float* save_invstd, int N, int C, int HW, int n_per, ConvPieces P = ConvPieces()) {
   const int c = blockIdx.x, s = blockIdx.y;
-  const float mean = save_mean[c], invstd = save_invstd[c], g = gamma[c], b = beta[c];
+  float mean, invstd;
+  if (PIECES) bn_stats_from_pieces(P, c, s == 0, mean, invstd); else { mean = save_mean[c]; invstd = save_invstd[c]; }
+  const float g = gamma[c], b = beta[c];
   const int n0 = s * n_per, n1 = min(N, n0 + n_per);
   bn_foreach<VEC>(n0, n1, C, c, HW,
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 r;
@@ -254,11 +295,13 @@ __global__ void __launch_bounds__(TPB) k_bn_apply(const float* __restrict__ x, f
 
 // out = relu(gamma * (x - mean) * invstd + beta + shortcut): the residual join behind a batch norm, one read of x and of
 // the shortcut and one write.
-template <bool VEC>
+template <bool VEC, bool PIECES = false>
 __global__ void __launch_bounds__(TPB) k_bn_apply_add_relu(const float* __restrict__ x, const float* __restrict__ sc, float* __restrict__ y, const float* gamma, const float* beta,
-                                                           const float* save_mean, const float* save_invstd, int N, int C, int HW, int n_per) {
+                                                           const float* save_mean, const float* save_invstd, int N, int C, int HW, int n_per, ConvPieces P = ConvPieces()) {
   const int c = blockIdx.x, s = blockIdx.y;
-  const float mean = save_mean[c], invstd = save_invstd[c], g = gamma[c], b = beta[c];
+  float mean, invstd;
+  if (PIECES) bn_stats_from_pieces(P, c, s == 0, mean, invstd); else { mean = save_mean[c]; invstd = save_invstd[c]; }
+  const float g = gamma[c], b = beta[c];
   const int n0 = s * n_per, n1 = min(N, n0 + n_per);
   bn_foreach<VEC>(n0, n1, C, c, HW,
     [&](int64_t off) { float4 v = *reinterpret_cast<const float4*>(x + off); float4 a = *reinterpret_cast<const float4*>(sc + off); float4 r;
@@ -313,6 +356,22 @@ void bn_finalize_conv_partials(const float* partial, int C, int ncols, int col1,
   const int slots_rem = col1 < ncols ? (int)cdiv(ncols - col1, g_rem) : 0;
   hipLaunchKernelGGL(k_bn_finalize_conv, dim3(C), dim3(TPB), 0, g_stream, partial, C, ncols, col1, g_main, slots_main, g_rem, slots_main + slots_rem,
                      save_mean, save_invstd, run_mean, run_var, eps, factor);
+}
+void bn_apply_from_pieces(const float* y, const ConvPieces& pieces, const float* gamma, const float* beta, const float* shortcut, float* out, int relu,
+                          int N, int C, int HW) {
+  ProfScope prof_(CAT_BN_FWD);
+  Plan p = make_plan(N, C, HW, (((uintptr_t)y | (uintptr_t)out | (uintptr_t)shortcut) & 15) == 0);
+  dim3 grid(C, p.slices);
+  const float* none = nullptr;
+  if (shortcut) {
+    if (p.vec4) hipLaunchKernelGGL((k_bn_apply_add_relu<true, true>), grid, dim3(TPB), 0, g_stream, y, shortcut, out, gamma, beta, none, none, N, C, HW, p.n_per, pieces);
+    else hipLaunchKernelGGL((k_bn_apply_add_relu<false, true>), grid, dim3(TPB), 0, g_stream, y, shortcut, out, gamma, beta, none, none, N, C, HW, p.n_per, pieces);
+  } else {
+#define GO(V, R) hipLaunchKernelGGL((k_bn_apply<V, R, true>), grid, dim3(TPB), 0, g_stream, y, out, gamma, beta, none, none, N, C, HW, p.n_per, pieces)
+    if (p.vec4) { if (relu) GO(true, true); else GO(true, false); }
+    else { if (relu) GO(false, true); else GO(false, false); }
+#undef GO
+  }
 }
 }  // namespace lh
 

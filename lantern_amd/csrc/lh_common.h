@@ -80,6 +80,12 @@ struct KernelCat {
 // g_rem columns after them; partial[c][slot] = (sum, sum of squares) as float2.  Writes mean, 1/sqrt(var+eps), updates running stats.
 void bn_finalize_conv_partials(const float* partial, int C, int ncols, int col1, int g_main, int slots_main, int g_rem,
                                float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor);
+// The same pieces consumed by the normalisation itself: every block of the apply pass adds up its channel's pieces (as
+// k_bn_finalize_conv does), so the separate statistics launch between the convolution and the apply pass disappears.
+// out = bn(y) [relu] or relu(bn(y) + shortcut); the block of batch slice 0 stores the saved and running statistics.
+struct ConvPieces { const float* partial; int ncols, col1, g_main, slots_main, g_rem, slots; float eps, factor; float* save_mean; float* save_invstd; float* run_mean; float* run_var; };
+void bn_apply_from_pieces(const float* y, const ConvPieces& pieces, const float* gamma, const float* beta, const float* shortcut, float* out, int relu,
+                          int N, int C, int HW);
 
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

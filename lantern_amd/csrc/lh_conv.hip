@@ -451,12 +451,17 @@ static bool launch_tiles_stats(const AL& al, const BL& bl, EpiConvOutStats ep, i
   return ok;
 }
 
-struct BnStatsOut { float* save_mean; float* save_invstd; float* run_mean; float* run_var; float eps, factor; };
+struct BnStatsOut {
+  float* save_mean; float* save_invstd; float* run_mean; float* run_var; float eps, factor;
+  // optional: the normalisation itself (out = bn(y) [relu] or relu(bn(y) + shortcut)); when the launch left statistics pieces the
+  // apply pass consumes them directly and `applied` is set, otherwise the caller runs it from the saved statistics
+  const float* gamma = nullptr; const float* beta = nullptr; const float* shortcut = nullptr; float* out = nullptr; int relu = 0; bool applied = false;
+};
 }  // namespace
 
 // Forward convolution; with `bn` also the batch-norm statistics of its output channels.
 static void conv_fwd_impl(const float* x, const float* w, const float* bias, float* y,
-                          int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW, const BnStatsOut* bn) {
+                          int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW, BnStatsOut* bn) {
   KernelCat kc_(CAT_CONV_FWD);
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_fwd: bad shape N%d C%d H%d W%d K%d R%d S%d s(%d,%d) p(%d,%d)", N, C, H, W, K, R, S, sH, sW, pH, pW);
@@ -532,7 +537,13 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
         if (partial == nullptr) return;
         EpiConvOutStats es; static_cast<EpiConvOut&>(es) = ep; es.partial = partial; es.slotBase = 0; es.slotsTotal = L.slots_main + L.slots_rem;
         ok = launch_tiles_stats(al, bl, es, K, N * PQ, CRS, L, bm, bn_);
-        if (ok) bn_finalize_conv_partials(partial, K, N * PQ, L.col1, L.g_main, L.slots_main, L.g_rem, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, bn->eps, bn->factor);
+        if (ok && bn->out != nullptr) {
+          ConvPieces cp{partial, N * PQ, L.col1, L.g_main, L.slots_main, L.g_rem, L.slots_main + L.slots_rem, bn->eps, bn->factor, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var};
+          bn_apply_from_pieces(y, cp, bn->gamma, bn->beta, bn->shortcut, bn->out, bn->relu, N, K, PQ);
+          bn->applied = true;
+        } else if (ok) {
+          bn_finalize_conv_partials(partial, K, N * PQ, L.col1, L.g_main, L.slots_main, L.g_rem, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, bn->eps, bn->factor);
+        }
         lh_free_top(pbytes);
         bn = nullptr;      // done
       }
@@ -566,6 +577,22 @@ void lh_conv2d_fwd_bnstats(const float* x, const float* w, const float* bias, fl
   LH_REQUIRE(save_mean && save_invstd, "lh_conv2d_fwd_bnstats: save_mean and save_invstd are required");
   BnStatsOut bn{save_mean, save_invstd, run_mean, run_var, eps, factor};
   conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, &bn);
+}
+
+void lh_conv2d_fwd_bn_apply(const float* x, const float* w, const float* bias, float* y,
+                            int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW,
+                            const float* gamma, const float* beta, float* save_mean, float* save_invstd, float* run_mean, float* run_var,
+                            float eps, float factor, const float* shortcut, float* out, int relu) {
+  LH_REQUIRE(save_mean && save_invstd && gamma && beta && out, "lh_conv2d_fwd_bn_apply: gamma, beta, save_mean, save_invstd and out are required");
+  LH_REQUIRE(shortcut == nullptr || relu, "lh_conv2d_fwd_bn_apply: the residual join is relu(bn(y) + shortcut)");
+  BnStatsOut bn{save_mean, save_invstd, run_mean, run_var, eps, factor};
+  bn.gamma = gamma; bn.beta = beta; bn.shortcut = shortcut; bn.out = out; bn.relu = relu;
+  conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, &bn);
+  if (failed() || bn.applied) return;
+  ConvDims d;
+  if (!make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW)) return;
+  if (shortcut) lh_bn_apply_add_relu(y, gamma, beta, save_mean, save_invstd, shortcut, out, N, K, d.P * d.Q);
+  else lh_bn_apply(y, gamma, beta, save_mean, save_invstd, out, N, K, d.P * d.Q, relu);
 }
 
 void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
