@@ -561,7 +561,13 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
   if (!ok) return;
   LH_CHECK_LAUNCH();
   // shapes whose launch leaves no statistics pieces: one extra pass over y
-  if (bn) lh_bn_stats(y, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, N, K, PQ, bn->eps, bn->factor);
+  if (bn && bn->out != nullptr && bn->shortcut == nullptr) {       // statistics pass + apply pass that combines the partial sums itself
+    if (bn->relu) lh_bn_train_fwd_relu(y, bn->gamma, bn->beta, bn->run_mean, bn->run_var, bn->out, bn->save_mean, bn->save_invstd, N, K, PQ, bn->eps, bn->factor);
+    else lh_bn_train_fwd(y, bn->gamma, bn->beta, bn->run_mean, bn->run_var, bn->out, bn->save_mean, bn->save_invstd, N, K, PQ, bn->eps, bn->factor);
+    bn->applied = true;
+  } else if (bn) {
+    lh_bn_stats(y, bn->save_mean, bn->save_invstd, bn->run_mean, bn->run_var, N, K, PQ, bn->eps, bn->factor);
+  }
 }
 
 extern "C" {
