@@ -936,3 +936,28 @@ def test_convolution_applied_twice_accumulates_one_filter_gradient_across_stream
 
     outs = pair.run(f)
     check_all(outs, rtol=1e-4)
+
+
+def test_side_stream_contract_errors_are_reported_and_leave_the_library_usable(on_hip):
+    """Nested forks, a join or a zero-filled allocation between lh_side_begin and lh_side_end are refused with a message;
+    with the side stream switched off the same calls run in line."""
+    be, lib = on_hip, on_hip.lib
+    from lantern_amd import _lib
+    lib.lh_set_side_stream(1)
+    lib.lh_side_begin(); _lib.check()
+    for call, text in ((lambda: lib.lh_side_begin(), "already on the side stream"),
+                       (lambda: lib.lh_side_join(), "lh_side_join between"),
+                       (lambda: lib.lh_malloc(1024), "main-stream order only")):
+        call()
+        with pytest.raises(LanternHipError, match=text):
+            _lib.check()
+    u = lib.lh_malloc_uninit(1024); _lib.check()             # scratch without a zero fill is allowed there
+    assert u
+    lib.lh_fill(u, 3.0, 256); _lib.check()                    # runs on the side stream
+    lib.lh_side_end(); _lib.check()
+    assert (be.toHost(B.Buf(u, 256), 256) == 3.0).all()       # the read-back joins first
+    forks = lib.lh_side_forks()
+    lib.lh_set_side_stream(0)
+    lib.lh_side_begin(); lib.lh_fill(u, 4.0, 256); lib.lh_side_end(); _lib.check()      # in line
+    assert lib.lh_side_forks() == forks and (be.toHost(B.Buf(u, 256), 256) == 4.0).all()
+    lib.lh_set_side_stream(1)
