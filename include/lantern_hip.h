@@ -182,7 +182,8 @@ void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x,
  * filter gradient (tile shape and number of slices of its long reduction N*P*Q, timed on scratch memory) and, on calls
  * whose result overwrites its output, the forward and input-gradient products (tile shape, stream-K workers; a few timed
  * repetitions of the launch itself).  Products below 1e7 flop (LH_TUNE_MIN_FLOP) keep the built-in rule.  Environment:
- * LH_NO_TUNE=1 keeps the built-in rules everywhere, LH_TUNE_VERBOSE=1 prints each choice to stderr.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
+ * LH_NO_TUNE=1 keeps the built-in rules everywhere, LH_TUNE_VERBOSE=1 prints each choice to stderr, LH_FORCE_M32=1 (a test
+ * switch) sends every product of at most 32 rows to the 32-row tile whatever was measured.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
  * remembered and are used again after lh_set_tuning(1)). */
 void lh_set_tuning(int on);
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,

@@ -340,16 +340,22 @@ static bool launch_rounds(const AL& al, const BL& bl, const EP& ep, int M, int N
 // reduction, else the tile pick_tile_conv names).  1-3: plain tiles 128x128, 64x128, 64x64.  4-7: stream-K over
 // 128x128 / 64x128 tiles with two or three workers per CU.  8-9: stream-K over 64x64 tiles with four or eight workers per
 // CU, for products so small that even their 64x64 tiles leave most CUs with one block whose loads nothing hides.
-constexpr int N_PLANS = 10;
+// 10: 32x128 tiles (32-deep slabs) for products of at most 32 rows, whose 64-row tiles would be half empty.
+constexpr int N_PLANS = 11;
+// LH_FORCE_M32 in the environment: products of at most 32 rows always take the 32-row tile (for tests of that tile; the
+// measured choice may well be another one).
+static inline bool force_m32() { return getenv("LH_FORCE_M32") != nullptr; }
 template <class AL, class BL, class EP>
 static bool plan_valid(int plan, const EP& ep, int M, int K, bool can_zero) {
   if (plan == 0) return true;
+  if (plan == 10) return M <= 32;
   if ((plan == 1 || plan == 4 || plan == 6) && M <= 64) return false;
-  if (plan >= 4) return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= 16;
+  if (plan >= 4 && plan <= 9) return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= 16;
   return true;
 }
 template <class AL, class BL, class EP>
 static bool launch_plan(int plan, const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out, int64_t zero_n, bool prezeroed) {
+  if (plan == 10) return igemm_launch<32, 128, 32>(al, bl, ep, M, N, K, 1);
   if (plan >= 4) {
     const int workers = (plan >= 8 ? (plan == 8 ? 4 : 8) : (plan >= 6 ? 3 : 2)) * g_num_cu;
     if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
@@ -387,6 +393,7 @@ template <class AL, class BL, class EP>
 static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out = nullptr, int64_t zero_n = 0, bool prezeroed = false) {
   static std::map<PlanKey, int> chosen;
   const bool can_zero = zero_out != nullptr || prezeroed;
+  if (M <= 32 && force_m32()) return launch_plan(10, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   if (!g_tune || 2.0 * M * N * (double)K < g_tune_min_flop) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   const PlanKey key = {{M, N, K, ep.eH, ep.eW, ep.W, ep.PIX}};
   auto it = chosen.find(key);
@@ -661,7 +668,8 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
           Ms[i] = C; Ns[i] = N * c.Hc * c.Wc; Ks[i] = c.Kred;
           ntot += Ns[i]; if (c.Kred > kmax) kmax = c.Kred;
         }
-        auto run = [&](int tile) {           // 1: 128x128, 2: 64x128, 3: 64x64
+        auto run = [&](int tile) {           // 1: 128x128, 2: 64x128, 3: 64x64, 4: 32x128 (at most 32 input channels)
+          if (tile == 4) return igemm_launch_grouped<32, 128, 32>(ng, al, bl, ep, Ms, Ns, Ks);
           if (tile == 1) return igemm_launch_grouped<128, 128, CONV_BK>(ng, al, bl, ep, Ms, Ns, Ks);
           if (tile == 2) return igemm_launch_grouped<64, 128, CONV_BK>(ng, al, bl, ep, Ms, Ns, Ks);
           return igemm_launch_grouped<64, 64, CONV_BK>(ng, al, bl, ep, Ms, Ns, Ks);
@@ -673,13 +681,15 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
         TilePick tp = pick_tile(C, (int)(ntot < 0x7fffffff ? ntot : 0x7fffffff));
         int tile = tp.bm == 128 ? 1 : (tp.bn == 128 ? 2 : 3);
         auto it = chosen.find(key);
-        if (it != chosen.end()) tile = it->second;
+        if (C <= 32 && force_m32()) tile = 4;
+        else if (it != chosen.end()) tile = it->second;
         else if (g_tune && beta == 0.f && 2.0 * C * (double)ntot * kmax >= g_tune_min_flop) {
           LaunchTimer timer;
           if (timer.ok) {
             float best_ms = 3.0e38f; int best = tile;
-            for (int tcand = 1; tcand <= 3; tcand++) {
+            for (int tcand = 1; tcand <= 4; tcand++) {
               if (tcand == 1 && C <= 64) continue;
+              if (tcand == 4 && C > 32) continue;
               const float ms = timer.ms([&]() { return run(tcand); });
               if (ms < 0.f || failed()) { lh_free_top(bytes); return; }
               if (ms < best_ms * 0.98f) { best_ms = ms; best = tcand; }
@@ -781,6 +791,7 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     if (it != g_bwdf_split.end()) { tp = TilePick{it->second.bm, it->second.bn}; tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn); split = clamp_split(it->second.split); }
     else tune_now = true;
   }
+  if (K <= 32 && force_m32()) { tp = TilePick{32, 128}; tiles = cdiv(K, 32) * cdiv(CRS, 128); split = clamp_split(cdiv(3 * (int64_t)g_num_cu, tiles)); tune_now = false; }
   if (beta == 0.f) lh_fill(dw, 0.f, (int64_t)K * CRS);
   EpiRowMajor ep; ep.C = dw; ep.ldc = CRS; ep.alpha = 1.f; ep.beta = 1.f; ep.atomic = split > 1 ? 1 : 0;
   bool ok = false;
@@ -789,6 +800,7 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * H * W * 4); bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.CHW = C * H * W;
     bl.P = d.P; bl.Q = d.Q; bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
     if (tp.bm == 128) ok = igemm_launch<128, 128, 16>(al, bl, ep, K, CRS, (int)red, split);    // measured: the large tile prefers the short slab
+    else if (tp.bm == 32) ok = igemm_launch<32, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
     else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
     else ok = igemm_launch<64, 64, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
   };
@@ -797,6 +809,7 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
     bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * PQ * 4); bl.K = C; bl.PQ = PQ; bl.dPQ.init(PQ);
     if (tp.bm == 128) ok = igemm_launch<128, 128, 16>(al, bl, ep, K, CRS, (int)red, split);
+    else if (tp.bm == 32) ok = igemm_launch<32, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
     else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
     else ok = igemm_launch<64, 64, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
   };
@@ -819,12 +832,12 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     LaunchTimer timer;
     if (scratch && timer.ok) {
       const double targets[] = {1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 5.0, 6.0};
-      const TilePick shapes[3] = {{128, 128}, {64, 128}, {64, 64}};
+      const TilePick shapes[4] = {{128, 128}, {64, 128}, {64, 64}, {32, 128}};      // the last for layers of at most 32 output channels
       float* const real_out = ep.C;
       ep.C = scratch;
       BwdfPlan best = {tp.bm, tp.bn, split}; float best_ms = 3.0e38f;
-      for (int sh = 0; sh < 3 && !failed(); sh++) {
-        if ((shapes[sh].bm == 128 && K < 128) || (shapes[sh].bn == 128 && CRS < 128)) continue;
+      for (int sh = 0; sh < 4 && !failed(); sh++) {
+        if ((shapes[sh].bm == 128 && K < 128) || (shapes[sh].bn == 128 && CRS < 128) || (shapes[sh].bm == 32 && K > 32)) continue;
         tp = shapes[sh];
         tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
         int cand[10]; int nc = 0;

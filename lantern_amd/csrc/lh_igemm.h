@@ -144,7 +144,11 @@ __device__ __forceinline__ float lh_half_sum32(float v) {
 template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
 __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP& ep, const GemmShape& gs, const int block) {
   constexpr int KQ = BK / 4, PAD = 8 / KQ, LDA = BM + PAD, LDB = BN + PAD;
-  constexpr int TM = BM / 2, TN = BN / 2, MI = TM / 32, NI = TN / 32;
+  // The four wavefronts form a 2 x 2 grid over the tile, or, for a 32-row tile (products with at most 32 rows: layers with
+  // few channels), a 1 x 4 grid, so that no matrix instruction is spent on rows beyond the 32.
+  constexpr int WM = BM >= 64 ? 2 : 1, WN = 4 / WM;
+  constexpr int TM = BM / WM, TN = BN / WN, MI = TM / 32, NI = TN / 32;
+  static_assert(WM == 2 || !EP::STATS, "the statistics epilogue assumes two wavefronts along the columns");
   constexpr int GA = BM * KQ / 256, GB = BN * KQ / 256;
   static_assert(GA >= 1 && GB >= 1 && MI >= 1 && NI >= 1, "tile too small for 256 threads");
   extern __shared__ float4 lh_smem[];
@@ -165,14 +169,14 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
 #pragma unroll
   for (int g = 0; g < GA; g++) {
     if (AL::ALONG_K) { a_kq[g] = t % KQ; a_col[g] = t / KQ + g * (256 / KQ); }
-    else { a_col[g] = t % BM; a_kq[g] = __builtin_amdgcn_readfirstlane(t / BM) + g * (256 / BM); }
+    else { a_col[g] = t % BM; a_kq[g] = (BM >= 64 ? __builtin_amdgcn_readfirstlane(t / BM) : t / BM) + g * (256 / BM); }   // uniform per wavefront from 64 rows on
   }
 #pragma unroll
   for (int g = 0; g < GB; g++) {
     if (BL::ALONG_K) { b_kq[g] = t % KQ; b_col[g] = t / KQ + g * (256 / KQ); }
     else { b_col[g] = t % BN; b_kq[g] = __builtin_amdgcn_readfirstlane(t / BN) + g * (256 / BN); }
   }
-  const int lane = t & 63, wave = t >> 6, wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
+  const int lane = t & 63, wave = t >> 6, wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave, half = lane >> 5, l32 = lane & 31;
 
   while (u < u_end) {
   int tm, tn, kbeg, kend, part = 0;

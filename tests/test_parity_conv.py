@@ -138,6 +138,9 @@ TUNED_SHAPES = [
     (16, 128, 14, 14, 512, 1, 1, 1, 1, 0, 0),   # 1x1: the plain filter-gradient loaders
     (8, 64, 28, 28, 128, 3, 3, 2, 2, 1, 1),     # stride 2: four residue classes share a pre-zeroed dx (never timed)
     (6, 96, 15, 15, 160, 3, 3, 1, 1, 1, 1),     # odd map, partial tiles everywhere
+    (16, 32, 28, 28, 32, 3, 3, 1, 1, 1, 1),     # 32 channels in and out: the 32-row tiles compete in forward and input gradient (tap path)
+    (50, 10, 12, 12, 20, 5, 5, 1, 1, 0, 0),     # LeNet's second convolution: 20- and 10-row products through the general loaders
+    (8, 1, 41, 60, 32, 11, 5, 2, 2, 0, 0),      # one input channel, tall filter, stride 2 (DeepSpeech2's first layer in small)
 ]
 
 
@@ -180,3 +183,17 @@ def test_conv_measured_launch_plans_and_their_reuse(on_hip, dims):
     finally:
         lib.lh_set_tuning(1)
     dev.check()
+
+
+M32_SHAPES = [(16, 32, 28, 28, 32, 3, 3, 1, 1, 1, 1), (50, 10, 12, 12, 20, 5, 5, 1, 1, 0, 0), (8, 1, 41, 60, 32, 11, 5, 2, 2, 0, 0),
+              (4, 32, 21, 30, 32, 5, 3, 2, 1, 2, 1),     # stride (2,1): the residue classes of the input gradient in one grouped launch
+              (3, 7, 9, 9, 5, 3, 3, 1, 1, 1, 1), (2, 32, 16, 16, 16, 1, 1, 1, 1, 0, 0)]
+
+
+@pytest.mark.parametrize("dims", M32_SHAPES, ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("bias", [False, True], ids=["nobias", "bias"])
+def test_conv_32_row_tiles(on_hip, dims, bias, monkeypatch):
+    """Layers with at most 32 output (forward, filter gradient) or input (input gradient) channels on the 32 x 128 tile,
+    forced through the library's test switch (the measured launch plan may be another one)."""
+    monkeypatch.setenv("LH_FORCE_M32", "1")
+    check_conv(Dev(on_hip), dims, bias)

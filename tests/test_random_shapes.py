@@ -40,6 +40,23 @@ def test_random_conv_geometries(on_hip, group):
         on_hip.sync(); on_hip.resetMallocAddr(mark)
 
 
+@pytest.mark.parametrize("group", range(3))
+def test_random_conv_geometries_on_32_row_tiles(on_hip, group, monkeypatch):
+    """The same sweep with at most 32 channels on either side and the library's test switch that sends every product of at
+    most 32 rows to the 32 x 128 tile (forward, input gradient with its strided residue classes, filter gradient)."""
+    monkeypatch.setenv("LH_FORCE_M32", "1")
+    dev = Dev(on_hip)
+    rng = np.random.RandomState(3000 + group)
+    for i in range(8):
+        d = list(_conv_case(rng))
+        d[1] = int(rng.choice([1, 3, 4, 8, 16, 20, 32])); d[4] = int(rng.choice([1, 5, 10, 16, 20, 32]))
+        dims = tuple(d); bias = bool(rng.rand() < 0.5)
+        _say("conv (32-row tiles) group %d case %d dims %s bias %s" % (group, i, dims, bias))
+        mark = on_hip.getMallocAddr()
+        check_conv(dev, dims, bias)
+        on_hip.sync(); on_hip.resetMallocAddr(mark)
+
+
 @pytest.mark.parametrize("group", range(4))
 def test_random_sgemm_shapes_with_row_strides(on_hip, group):
     """All four transpose forms, leading dimensions larger than the rows (views into wider matrices), alpha/beta."""
