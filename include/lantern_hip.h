@@ -65,6 +65,9 @@ size_t lh_heap_used(void);
 size_t lh_heap_peak(void);
 
 /* ---- transfers: toGPU / toCPU / copyFloatArray (CUB:37-107, 128-131) --- */
+/* The host buffer may be reused as soon as lh_h2d returns.  Up to 64 KiB it is copied into a pinned staging slot and the
+ * transfer is only enqueued (no wait for the device; the stream orders it before later calls); larger uploads wait for
+ * the device as the reference's cudaMemcpy does. */
 void lh_h2d(void* dst, const void* h_src, size_t bytes);
 void lh_d2h(void* h_dst, const void* src, size_t bytes);   /* waits */
 void lh_d2d(void* dst, const void* src, size_t bytes);

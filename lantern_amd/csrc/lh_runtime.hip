@@ -124,12 +124,14 @@ void lh_setup(size_t heap_bytes) {
   LH_HIP(hipMalloc((void**)&g_advance_pool, MAX_GRAPHS * sizeof(unsigned long long)));
 }
 
+static void stage_release();
 void lh_cleanup(void) {
   g_stream_cur = g_stream_raw;
   if (g_side_stream) { (void)hipStreamSynchronize(g_side_stream); (void)hipStreamDestroy(g_side_stream); for (auto& e : g_side_ev) (void)hipEventDestroy(e); }
   g_side_stream = nullptr; g_side_dirty = false;
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
   cmdlist_release();
+  stage_release();
   for (auto& e : g_graphs) if (e) { (void)hipGraphExecDestroy(e); e = nullptr; }
   g_graphs.clear(); g_capturing = false;
   if (g_advance_pool) (void)hipFree(g_advance_pool);
@@ -187,10 +189,46 @@ void lh_rewind(size_t mark) {
 size_t lh_heap_used(void) { return g_top; }
 size_t lh_heap_peak(void) { return g_peak; }
 
+// Small uploads (a tree's labels, a batch's targets) go through a ring of pinned staging slots and do not wait for the
+// device: the caller's buffer is free again when the call returns (it was copied into the slot), and the stream orders
+// the transfer before everything issued afterwards.  A slot is reused after the event recorded behind its transfer.
+constexpr size_t STAGE_BYTES = 64 << 10;
+constexpr int STAGE_SLOTS = 32;
+static char* g_stage = nullptr;                 // STAGE_SLOTS * STAGE_BYTES of pinned host memory
+static hipEvent_t g_stage_ev[STAGE_SLOTS];
+static bool g_stage_used[STAGE_SLOTS];
+static unsigned g_stage_next = 0;
+static bool stage_init() {
+  if (g_stage) return true;
+  if (hipHostMalloc((void**)&g_stage, STAGE_SLOTS * STAGE_BYTES, hipHostMallocDefault) != hipSuccess) { g_stage = nullptr; (void)hipGetLastError(); return false; }
+  for (int i = 0; i < STAGE_SLOTS; i++) {
+    g_stage_used[i] = false;
+    if (hipEventCreateWithFlags(&g_stage_ev[i], hipEventDisableTiming) != hipSuccess) { (void)hipHostFree(g_stage); g_stage = nullptr; return false; }
+  }
+  return true;
+}
+static void stage_release() {
+  if (!g_stage) return;
+  for (int i = 0; i < STAGE_SLOTS; i++) (void)hipEventDestroy(g_stage_ev[i]);
+  (void)hipHostFree(g_stage);
+  g_stage = nullptr;
+}
+
 void lh_h2d(void* dst, const void* h_src, size_t bytes) {
-  // Pageable source: the copy is staged before the call returns, so the host buffer may be reused.
   LH_NOT_CAPTURING("lh_h2d");
   side_join();
+  if (bytes == 0) return;
+  if (bytes <= STAGE_BYTES && stage_init()) {
+    const int slot = (int)(g_stage_next++ % STAGE_SLOTS);
+    if (g_stage_used[slot]) LH_HIP(hipEventSynchronize(g_stage_ev[slot]));       // long since complete unless 32 uploads are in flight
+    char* buf = g_stage + (size_t)slot * STAGE_BYTES;
+    memcpy(buf, h_src, bytes);
+    LH_HIP(hipMemcpyAsync(dst, buf, bytes, hipMemcpyHostToDevice, g_stream));
+    LH_HIP(hipEventRecord(g_stage_ev[slot], g_stream));
+    g_stage_used[slot] = true;
+    return;
+  }
+  // Pageable source: the copy is staged before the call returns, so the host buffer may be reused.
   LH_HIP(hipMemcpyAsync(dst, h_src, bytes, hipMemcpyHostToDevice, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
 }
