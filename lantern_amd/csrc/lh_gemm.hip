@@ -14,14 +14,17 @@ constexpr int TPB = 256;
 constexpr int SMALL_KS = 64;
 template <bool TA, bool TB>
 __global__ void __launch_bounds__(TPB) k_sgemm_tile(int m, int n, int k, float alpha, const float* __restrict__ A, int lda,
-                                                    const float* __restrict__ B, int ldb, float beta, float* __restrict__ C, int ldc) {
+                                                    const float* __restrict__ B, int ldb, float beta, float* __restrict__ C, int ldc, int kper) {
+  // kper < k: blockIdx.z takes the slice [z * kper, (z + 1) * kper) of the reduction and adds its part to C atomically (C holds beta*C)
   __shared__ float As[SMALL_KS][64 + 4];
   __shared__ float Bs[SMALL_KS][64 + 4];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
   const int i0 = blockIdx.y * 64, j0 = blockIdx.x * 64;
   float acc[4][4] = {};
-  for (int k0 = 0; k0 < k; k0 += SMALL_KS) {
-    const int kn = k - k0 < SMALL_KS ? k - k0 : SMALL_KS;
+  const bool sliced = kper < k;
+  const int kbeg = sliced ? (int)blockIdx.z * kper : 0, kend = sliced ? min(k, kbeg + kper) : k;
+  for (int k0 = kbeg; k0 < kend; k0 += SMALL_KS) {
+    const int kn = kend - k0 < SMALL_KS ? kend - k0 : SMALL_KS;
     float ra[SMALL_KS * 64 / TPB], rb[SMALL_KS * 64 / TPB];
 #pragma unroll
     for (int r = 0; r < SMALL_KS * 64 / TPB; r++) {
@@ -62,7 +65,8 @@ __global__ void __launch_bounds__(TPB) k_sgemm_tile(int m, int n, int k, float a
       int gj = j0 + tx * 4 + v;
       if (gj >= n) continue;
       float* c = C + (int64_t)gi * ldc + gj;
-      *c = alpha * acc[u][v] + (beta == 0.f ? 0.f : beta * *c);
+      if (sliced) atomicAdd(c, alpha * acc[u][v]);
+      else *c = alpha * acc[u][v] + (beta == 0.f ? 0.f : beta * *c);
     }
   }
 }
@@ -234,10 +238,20 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   }
   ProfScope prof_(CAT_GEMM);
   dim3 grid((unsigned)cdiv(n, 64), (unsigned)cdiv(m, 64));
-  if (!ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<false, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
-  else if (!ta && tb) hipLaunchKernelGGL((k_sgemm_tile<false, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
-  else if (ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<true, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
-  else hipLaunchKernelGGL((k_sgemm_tile<true, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+  // A few tiles over a long reduction (a classifier with ten outputs behind 2048 features: one block walking 32 slabs took
+  // 194 us): the reduction is cut into slices of at least 128 that add into beta*C.
+  int kper = k;
+  if (k >= 512 && (int64_t)grid.x * grid.y <= 64) {
+    int slices = k / 128; if (slices > 32) slices = 32;
+    kper = (int)cdiv(cdiv(k, slices), SMALL_KS) * SMALL_KS;
+    grid.z = (unsigned)cdiv(k, kper);
+    if (grid.z > 1 && beta != 1.f) hipLaunchKernelGGL(k_scale_rows, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, C, ldc, m, n, beta);
+    if (grid.z <= 1) kper = k;
+  }
+  if (!ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<false, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kper);
+  else if (!ta && tb) hipLaunchKernelGGL((k_sgemm_tile<false, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kper);
+  else if (ta && !tb) hipLaunchKernelGGL((k_sgemm_tile<true, false>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kper);
+  else hipLaunchKernelGGL((k_sgemm_tile<true, true>), grid, dim3(TPB), 0, g_stream, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, kper);
   LH_CHECK_LAUNCH();
 }
 extern "C" {

@@ -111,7 +111,8 @@ def test_conv_linearity_at_resnet_shape(on_hip):
 
 
 GEMMS = [(0, 0, 64, 1000, 2048), (0, 1, 64, 1000, 2048), (1, 0, 70, 130, 257), (1, 1, 33, 65, 129),
-         (0, 0, 100, 50, 320), (0, 1, 5, 7, 3), (0, 0, 2, 3, 4), (1, 0, 300, 300, 64)]
+         (0, 0, 100, 50, 320), (0, 1, 5, 7, 3), (0, 0, 2, 3, 4), (1, 0, 300, 300, 64),
+         (0, 1, 64, 10, 2048), (1, 0, 12, 7, 1500), (0, 0, 5, 3, 700), (1, 1, 9, 15, 513)]      # few outputs over a long reduction: the sliced small kernel
 
 
 @pytest.mark.parametrize("ta,tb,m,n,k", GEMMS)
