@@ -71,8 +71,12 @@ def run_gpu(args):
     lib = be.lib
     if args.no_side_stream:
         lib.lh_set_side_stream(0)
-    for _ in range(args.warmup):
-        tr.step(); tr.end_step()
+    loss_first = None
+    for i in range(args.warmup):
+        l = tr.step()
+        if i == 0:
+            loss_first = float(l.toCPU()[0])      # before any update: ln(classes) for a freshly initialised classifier
+        tr.end_step()
     be.sync()
     t_issued = None
     if args.graph:
@@ -118,7 +122,7 @@ def run_gpu(args):
     loss_val = float(tr.step().toCPU()[0]); tr.end_step()
     peak_gb = lib.lh_heap_peak() / 2 ** 30
     be.cleanup()
-    return {"sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "arena_peak_gib": peak_gb,
+    return {"sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
             "per_step": per_step, "desc": desc}
 
 
@@ -218,7 +222,7 @@ def main():
         "value": round(value, 2), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": g["desc"], "global_batch": args.batch, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
+        "config": {"workload": g["desc"], "global_batch": args.batch, "loss_first_step": round(g["loss_first"], 5) if g["loss_first"] is not None else None, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
                    "launch": "hip graph replay" if args.graph else "one launch per kernel",
                    "host_issue_ms_per_step": round(1000.0 * g["issue_sec"] / args.steps, 3) if g["issue_sec"] is not None else None,
                    "filter_gradients": "in line" if args.no_side_stream else "side stream"},
