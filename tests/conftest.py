@@ -20,7 +20,7 @@ def _gpu_present():
 def hip_backend():
     """One BackendHIP for the whole session (the library owns one arena); fails loudly if the .so is missing."""
     import lantern_amd as la
-    be = la.BackendHIP(heap_bytes=int(os.environ.get("LANTERN_TEST_HEAP", 6 << 30)))
+    be = la.BackendHIP(heap_bytes=int(os.environ.get("LANTERN_TEST_HEAP", 16 << 30)))      # the headline step at full size needs 12.4 GiB
     be.setup()
     yield be
     be.cleanup()

@@ -206,3 +206,40 @@ def test_capture_rejects_waiting_entry_points(hip_backend):
     be.graphDestroy(g)
     assert float((t + t).sum().toCPU()[0]) == 256.0
     be.resetMallocAddr(mark)
+
+
+def test_resnet50_headline_step_invariants_at_full_size(hip_backend):
+    """The headline configuration itself (batch 64, 3x224x224, 1000 classes) is far too large for the oracle; what its
+    mathematics fixes is checked instead, after one forward + backward pass at full size:
+      - the loss of a freshly initialised 1000-way classifier is ln(1000) plus the spread of its random logits;
+      - a softmax cross-entropy gradient sums to zero over the classes, so the classifier's bias gradient sums to zero;
+      - batch norm makes the loss invariant to the scale of each output channel of the convolution in front of it, so the
+        gradient of every filter is orthogonal to the filter, channel by channel (up to eps / variance).  All 53 convolutions
+        are followed by a batch norm: this involves every forward kernel, every input gradient, every batch-norm backward,
+        the residual joins, the pooling layers and all 53 filter gradients (which run on the side stream)."""
+    from lantern_amd.apps.resnet50 import ResNet50, Trainer
+    from lantern_amd.tensor import Tensor, TensorR, gradR_loss
+    be = hip_backend
+    la.set_backend(be)
+    mark = be.getMallocAddr()
+    tr = Trainer(ResNet50(num_classes=1000, imagenet_stem=True), 64, 224, 1000, lr=0.1, momentum=0.9)
+    xin = TensorR(tr.x, isInput=True)
+    loss = gradR_loss(lambda dummy: tr.model(xin).logSoftmaxB().nllLossB(tr.target).mean())(Tensor.zeros(1))
+    l0 = float(loss.toCPU()[0])
+    assert 6.5 < l0 < 7.8, l0
+    params = dict(tr.model.namedParameters())
+    db = [p for n, p in params.items() if n.endswith("fc_bias")][0].d.toCPU().astype(np.float64)
+    assert np.abs(db).sum() > 1e-4 and abs(db.sum()) <= 1e-4 * np.abs(db).sum(), (db.sum(), np.abs(db).sum())
+    worst, n_filters = 0.0, 0
+    for name, p in params.items():
+        if not name.endswith("/kernel"):
+            continue
+        w = p.x.toCPU().astype(np.float64); dw = p.d.toCPU().astype(np.float64)
+        w = w.reshape(w.shape[0], -1); dw = dw.reshape(dw.shape[0], -1)
+        assert np.isfinite(dw).all() and np.abs(dw).max() > 0, name
+        cos = np.abs((w * dw).sum(1)) / (np.linalg.norm(w, axis=1) * np.linalg.norm(dw, axis=1) + 1e-300)
+        worst = max(worst, float(cos.max())); n_filters += 1
+        assert cos.max() < 3e-4, "%s: a filter gradient is not orthogonal to its filter (|cos| %.3g)" % (name, cos.max())
+    assert n_filters == 53
+    print("loss %.4f, classifier bias gradient sum %.3g of %.3g, largest |cos(filter, gradient)| %.3g" % (l0, db.sum(), np.abs(db).sum(), worst))
+    be.sync(); be.resetMallocAddr(mark)
