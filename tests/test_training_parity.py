@@ -222,24 +222,27 @@ def test_resnet50_headline_step_invariants_at_full_size(hip_backend):
     be = hip_backend
     la.set_backend(be)
     mark = be.getMallocAddr()
-    tr = Trainer(ResNet50(num_classes=1000, imagenet_stem=True), 64, 224, 1000, lr=0.1, momentum=0.9)
-    xin = TensorR(tr.x, isInput=True)
-    loss = gradR_loss(lambda dummy: tr.model(xin).logSoftmaxB().nllLossB(tr.target).mean())(Tensor.zeros(1))
-    l0 = float(loss.toCPU()[0])
-    assert 6.5 < l0 < 7.8, l0
+    tr = Trainer(ResNet50(num_classes=1000, imagenet_stem=True), 64, 224, 1000, lr=0.01, momentum=0.9)
     params = dict(tr.model.namedParameters())
-    db = [p for n, p in params.items() if n.endswith("fc_bias")][0].d.toCPU().astype(np.float64)
-    assert np.abs(db).sum() > 1e-4 and abs(db.sum()) <= 1e-4 * np.abs(db).sum(), (db.sum(), np.abs(db).sum())
-    worst, n_filters = 0.0, 0
-    for name, p in params.items():
-        if not name.endswith("/kernel"):
-            continue
-        w = p.x.toCPU().astype(np.float64); dw = p.d.toCPU().astype(np.float64)
-        w = w.reshape(w.shape[0], -1); dw = dw.reshape(dw.shape[0], -1)
-        assert np.isfinite(dw).all() and np.abs(dw).max() > 0, name
-        cos = np.abs((w * dw).sum(1)) / (np.linalg.norm(w, axis=1) * np.linalg.norm(dw, axis=1) + 1e-300)
-        worst = max(worst, float(cos.max())); n_filters += 1
-        assert cos.max() < 3e-4, "%s: a filter gradient is not orthogonal to its filter (|cos| %.3g)" % (name, cos.max())
-    assert n_filters == 53
-    print("loss %.4f, classifier bias gradient sum %.3g of %.3g, largest |cos(filter, gradient)| %.3g" % (l0, db.sum(), np.abs(db).sum(), worst))
+    for step in range(3):       # the first pass measures launch plans; the later ones run the remembered plans, filter gradients beside the chain
+        xin = TensorR(tr.x, isInput=True)
+        loss = gradR_loss(lambda dummy: tr.model(xin).logSoftmaxB().nllLossB(tr.target).mean())(Tensor.zeros(1))
+        l0 = float(loss.toCPU()[0])
+        assert (6.5 < l0 < 7.8) if step == 0 else (0.0 < l0 < 12.0), l0
+        db = [p for n, p in params.items() if n.endswith("fc_bias")][0].d.toCPU().astype(np.float64)
+        assert np.abs(db).sum() > 1e-4 and abs(db.sum()) <= 1e-4 * np.abs(db).sum(), (db.sum(), np.abs(db).sum())
+        worst, n_filters = 0.0, 0
+        for name, p in params.items():
+            if not name.endswith("/kernel"):
+                continue
+            w = p.x.toCPU().astype(np.float64); dw = p.d.toCPU().astype(np.float64)
+            w = w.reshape(w.shape[0], -1); dw = dw.reshape(dw.shape[0], -1)
+            assert np.isfinite(dw).all() and np.abs(dw).max() > 0, name
+            cos = np.abs((w * dw).sum(1)) / (np.linalg.norm(w, axis=1) * np.linalg.norm(dw, axis=1) + 1e-300)
+            worst = max(worst, float(cos.max())); n_filters += 1
+            assert cos.max() < 3e-4, "step %d, %s: a filter gradient is not orthogonal to its filter (|cos| %.3g)" % (step, name, cos.max())
+        assert n_filters == 53
+        print("step %d: loss %.4f, classifier bias gradient sum %.3g of %.3g, largest |cos(filter, gradient)| %.3g" % (step, l0, db.sum(), np.abs(db).sum(), worst))
+        tr.opt.step()           # updates the parameters and clears the gradients
+        tr.end_step()
     be.sync(); be.resetMallocAddr(mark)
