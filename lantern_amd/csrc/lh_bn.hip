@@ -189,6 +189,123 @@ __global__ void __launch_bounds__(TPB) k_bn_infer(const float* __restrict__ x, f
   }
 }
 
+// ---- HW == 1 (BatchNorm1D over [rows, C]): the elements of a channel lie C floats apart, so the (channel, slice) blocks
+// above would touch one cache line per element.  Here a block takes 64 neighbouring channels (a 256-byte row segment per
+// load, coalesced) times a slice of the rows; four row lanes per channel are combined through LDS.  The partial sums have
+// the layout of the kernels above, so statistics finalisation and the other passes are shared.
+constexpr int C1 = 64;                          // channels per block
+struct Plan1 { int slices, rows_per; };
+static Plan1 make_plan1(int N, int C) {
+  const int colb = (int)cdiv(C, C1);
+  int want = (int)cdiv(2 * (int64_t)g_num_cu, colb);
+  if (want > 16) want = 16;                  // every thread of the second pass walks the slices' partial sums
+  int max_slices = N / 32; if (max_slices < 1) max_slices = 1;         // at least 32 rows per block
+  if (want > max_slices) want = max_slices;
+  if (want < 1) want = 1;
+  while ((int64_t)want * C > MAX_PARTIALS && want > 1) want--;
+  Plan1 p; p.rows_per = (int)cdiv(N, want); p.slices = (int)cdiv(N, p.rows_per);
+  return p;
+}
+__global__ void __launch_bounds__(TPB) k_bn1d_stats(const float* __restrict__ x, float* __restrict__ partial, int N, int C, int rows_per) {
+  __shared__ float sh[2][4][C1];
+  const int cx = threadIdx.x & (C1 - 1), ry = threadIdx.x >> 6;
+  const int c = blockIdx.x * C1 + cx, s = blockIdx.y;
+  const int n0 = s * rows_per, n1 = min(N, n0 + rows_per);
+  const bool ok = c < C;
+  const float K = ok ? x[(int64_t)n0 * C + c] : 0.f;          // shift, as k_bn_stats
+  float s1 = 0.f, s2 = 0.f;
+  float t1 = 0.f, t2 = 0.f;                     // two independent chains: the loads of neighbouring iterations overlap
+  if (ok) {
+    int n = n0 + ry;
+    for (; n + 4 < n1; n += 8) {
+      const float a = x[(int64_t)n * C + c] - K, b = x[(int64_t)(n + 4) * C + c] - K;
+      s1 += a; s2 += a * a; t1 += b; t2 += b * b;
+    }
+    if (n < n1) { const float a = x[(int64_t)n * C + c] - K; s1 += a; s2 += a * a; }
+    s1 += t1; s2 += t2;
+  }
+  sh[0][ry][cx] = s1; sh[1][ry][cx] = s2;
+  __syncthreads();
+  if (ry == 0 && ok) {
+    s1 = (sh[0][0][cx] + sh[0][1][cx]) + (sh[0][2][cx] + sh[0][3][cx]);
+    s2 = (sh[1][0][cx] + sh[1][1][cx]) + (sh[1][2][cx] + sh[1][3][cx]);
+    const float cnt = (float)(n1 - n0);
+    float* p = partial + 3 * ((int64_t)c * gridDim.y + s);
+    p[0] = K + s1 / cnt; p[1] = s2 - s1 * s1 / cnt; p[2] = cnt;
+  }
+}
+__global__ void __launch_bounds__(TPB) k_bn1d_fwd_apply(const float* __restrict__ x, float* __restrict__ y, const float* __restrict__ partial,
+                                                        const float* gamma, const float* beta, float* run_mean, float* run_var,
+                                                        float* save_mean, float* save_invstd, int N, int C, int rows_per, float eps, float factor) {
+  const int cx = threadIdx.x & (C1 - 1), ry = threadIdx.x >> 6;
+  const int c = blockIdx.x * C1 + cx, s = blockIdx.y;
+  if (c >= C) return;
+  double mean, m2, cnt;
+  combine_stats(partial, c, gridDim.y, mean, m2, cnt);        // every row lane of a channel gets the same bits
+  const float var = (float)(m2 / cnt), invstd = 1.0f / sqrtf(var + eps), mu = (float)mean;
+  if (s == 0 && ry == 0) {
+    if (save_mean) save_mean[c] = mu;
+    if (save_invstd) save_invstd[c] = invstd;
+    if (run_mean) run_mean[c] = (1.0f - factor) * run_mean[c] + factor * mu;
+    if (run_var) { float unb = cnt > 1.0 ? (float)(m2 / (cnt - 1.0)) : var; run_var[c] = (1.0f - factor) * run_var[c] + factor * unb; }
+  }
+  const float g = gamma[c], b = beta[c];
+  const int n0 = s * rows_per, n1 = min(N, n0 + rows_per);
+#pragma unroll 4
+  for (int n = n0 + ry; n < n1; n += 4) { const int64_t o = (int64_t)n * C + c; y[o] = bn_affine(x[o], mu, invstd, g, b); }
+}
+__global__ void __launch_bounds__(TPB) k_bn1d_bwd_stats(const float* __restrict__ x, const float* __restrict__ dy, const float* save_mean, const float* save_invstd,
+                                                        float* __restrict__ partial, int N, int C, int rows_per) {
+  __shared__ float sh[2][4][C1];
+  const int cx = threadIdx.x & (C1 - 1), ry = threadIdx.x >> 6;
+  const int c = blockIdx.x * C1 + cx, s = blockIdx.y;
+  const int n0 = s * rows_per, n1 = min(N, n0 + rows_per);
+  const bool ok = c < C;
+  const float mean = ok ? save_mean[c] : 0.f, is = ok ? save_invstd[c] : 0.f;
+  float s1 = 0.f, s2 = 0.f;
+  float t1 = 0.f, t2 = 0.f;
+  if (ok) {
+    int n = n0 + ry;
+    for (; n + 4 < n1; n += 8) {
+      const int64_t o = (int64_t)n * C + c, o2 = (int64_t)(n + 4) * C + c;
+      const float g = dy[o], g2 = dy[o2], xa = x[o], xb = x[o2];
+      s1 += g; s2 += g * ((xa - mean) * is); t1 += g2; t2 += g2 * ((xb - mean) * is);
+    }
+    if (n < n1) { const int64_t o = (int64_t)n * C + c; const float g = dy[o]; s1 += g; s2 += g * ((x[o] - mean) * is); }
+    s1 += t1; s2 += t2;
+  }
+  sh[0][ry][cx] = s1; sh[1][ry][cx] = s2;
+  __syncthreads();
+  if (ry == 0 && ok) {
+    float* p = partial + 3 * ((int64_t)c * gridDim.y + s);
+    p[0] = (sh[0][0][cx] + sh[0][1][cx]) + (sh[0][2][cx] + sh[0][3][cx]);
+    p[1] = (sh[1][0][cx] + sh[1][1][cx]) + (sh[1][2][cx] + sh[1][3][cx]);
+  }
+}
+template <bool ACC>
+__global__ void __launch_bounds__(TPB) k_bn1d_bwd_apply(const float* __restrict__ x, const float* __restrict__ dy, const float* __restrict__ partial,
+                                                        const float* gamma, const float* save_mean, const float* save_invstd,
+                                                        float* __restrict__ dx, float* dgamma, float* dbeta, int N, int C, int rows_per) {
+  const int cx = threadIdx.x & (C1 - 1), ry = threadIdx.x >> 6;
+  const int c = blockIdx.x * C1 + cx, s = blockIdx.y;
+  if (c >= C) return;
+  double a = 0.0, b = 0.0;
+  for (int t = 0; t < (int)gridDim.y; t++) { const float* p = partial + 3 * ((int64_t)c * gridDim.y + t); a += p[0]; b += p[1]; }
+  const double cnt = (double)N;
+  const float m1 = (float)(a / cnt), m2 = (float)(b / cnt);
+  if (s == 0 && ry == 0) { if (dgamma) dgamma[c] += (float)b; if (dbeta) dbeta[c] += (float)a; }
+  if (dx == nullptr) return;
+  const float mean = save_mean[c], is = save_invstd[c], g = gamma[c] * is;
+  const int n0 = s * rows_per, n1 = min(N, n0 + rows_per);
+#pragma unroll 4
+  for (int n = n0 + ry; n < n1; n += 4) {
+    const int64_t o = (int64_t)n * C + c;
+    float r = g * (dy[o] - m1 - (x[o] - mean) * is * m2);
+    if (ACC) r += dx[o];
+    dx[o] = r;
+  }
+}
+
 // Channel statistics from classic per-slice partials (mean, M2, count): one thread per channel.
 __global__ void __launch_bounds__(TPB) k_bn_finalize(const float* __restrict__ partial, int C, int slices, float* save_mean, float* save_invstd,
                                                      float* run_mean, float* run_var, float eps, float factor) {
@@ -418,6 +535,15 @@ static void bn_train_fwd_impl(bool relu, const float* x, const float* gamma, con
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_train_fwd: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_train_fwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   if (!get_partial()) return;
+  if (HW == 1 && !relu && C >= 32) {          // rows of channels: the column kernels
+    const Plan1 p1 = make_plan1(N, C);
+    dim3 g1((unsigned)cdiv(C, C1), p1.slices);
+    hipLaunchKernelGGL(k_bn1d_stats, g1, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, p1.rows_per);
+    hipLaunchKernelGGL(k_bn1d_fwd_apply, g1, dim3(TPB), 0, g_stream, x, y, (const float*)g_partial_ptr, gamma, beta, run_mean, run_var,
+                       save_mean, save_invstd, N, C, p1.rows_per, eps, factor);
+    LH_CHECK_LAUNCH();
+    return;
+  }
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)y) & 15) == 0);
   dim3 grid(C, p.slices);
 #define FWD(V, R) hipLaunchKernelGGL((k_bn_fwd_apply<V, R>), grid, dim3(TPB), 0, g_stream, x, y, (const float*)g_partial_ptr, gamma, beta, run_mean, run_var, \
@@ -440,6 +566,15 @@ static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, co
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_bwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   LH_REQUIRE(beta_dx == 0.0f || beta_dx == 1.0f, "lh_bn_bwd: beta must be 0 or 1");
   if (!get_partial()) return;
+  if (HW == 1 && relu == 0 && C >= 32) {
+    const Plan1 p1 = make_plan1(N, C);
+    dim3 g1((unsigned)cdiv(C, C1), p1.slices);
+    hipLaunchKernelGGL(k_bn1d_bwd_stats, g1, dim3(TPB), 0, g_stream, x, dy, save_mean, save_invstd, g_partial_ptr, N, C, p1.rows_per);
+    if (beta_dx != 0.0f) hipLaunchKernelGGL((k_bn1d_bwd_apply<true>), g1, dim3(TPB), 0, g_stream, x, dy, (const float*)g_partial_ptr, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, p1.rows_per);
+    else hipLaunchKernelGGL((k_bn1d_bwd_apply<false>), g1, dim3(TPB), 0, g_stream, x, dy, (const float*)g_partial_ptr, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, p1.rows_per);
+    LH_CHECK_LAUNCH();
+    return;
+  }
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx | (uintptr_t)y_relu) & 15) == 0);
   dim3 grid(C, p.slices);
   const bool acc = beta_dx != 0.0f;
