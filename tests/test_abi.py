@@ -70,3 +70,40 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(ImportError):
         _lib.load()
+
+
+HOST_C = os.path.join(ROOT, "tests", "host_c")
+HOST_BIN = os.path.join(HOST_C, "_build", "lenet_step")
+
+
+def test_header_is_plain_c99(tmp_path):
+    """The boundary is a C header: a C99 translation unit that only includes it compiles without warnings."""
+    src = tmp_path / "only_header.c"
+    src.write_text('#include "lantern_hip.h"\nint main(void) { return 0; }\n')
+    subprocess.check_call(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I",
+                           os.path.join(ROOT, "include"), str(src)])
+
+
+def _build_host_program():
+    subprocess.check_call(["make", "-C", HOST_C], stdout=subprocess.DEVNULL)
+    return HOST_BIN
+
+
+def test_c_host_program_links_without_python_or_torch():
+    """A plain-C program written against the header links to the library and loads it (no device call is made)."""
+    exe = _build_host_program()
+    out = subprocess.run([exe], env=dict(os.environ, LENET_STEP_LINK_ONLY="1"), capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0 and out.stdout.strip() == "linked", out.stdout + out.stderr
+    deps = subprocess.run(["ldd", exe], capture_output=True, text=True).stdout
+    assert "liblantern_hip.so" in deps and "torch" not in deps and "python" not in deps, deps
+
+
+@pytest.mark.gpu
+def test_c_host_program_trains_lenet_like_the_oracle():
+    """Five SGD steps of the MNIST CNN issued from C through the C-ABI, against the oracle in the same process:
+    losses within 1e-4 relative, parameters within 1e-3 of the largest one (the program's own exit code)."""
+    exe = HOST_BIN if os.path.exists(HOST_BIN) else _build_host_program()
+    env = {k: v for k, v in os.environ.items() if k != "LENET_STEP_LINK_ONLY"}
+    out = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=110)
+    print(out.stdout, out.stderr)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
