@@ -136,6 +136,10 @@ void lh_fill(float* x, float v, int64_t n);                                    /
 void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, int64_t inner); /* fillWithBias: CPU:39-62 */
 void lh_clip(float* x, float bound, int64_t n);                                /* clipAt: CUB:157-161 */
 void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t);      /* mask4D: CUB:710-719 */
+/* Cifar10DataLoader's decode (src/main/scala/lantern/TensorDataLoader.scala:109-127) on the device: n records of one label
+ * byte + count pixel bytes -> x[n, count] = (float)byte / 255.0f (correctly rounded, the host loop's bits), y[n] = (int)byte.
+ * records need no alignment; x and y must not overlap records. */
+void lh_cifar_decode(const unsigned char* records, float* x, int* y, int n, int count);
 /* relu/tanh/sigmoid/hardTanh/exp/log/sqrt/square (TD:319-335; CDN:1349-1429, CUB:733-800).
  * y may alias x (in place).  lo/hi are used by LH_HARDTANH only. */
 void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi);

@@ -56,3 +56,55 @@ class Trainer:
 
     def end_step(self):
         get_backend().resetMallocAddr(self.mark)
+
+
+def train_from_files(result_path, root="../data/bin", nbEpoch=4, batchSize=100, lr=0.0005, seed=42, out=print):
+    """The reference program's main loop on dataset files (MnistCNN.scala:60-115): load and normalize `mnist_train.bin`,
+    train nbEpoch epochs of full batches, print the progress lines, write the result file.  Returns the per-epoch losses."""
+    import time
+    from ..data import DataLoader, write_result_file
+    be = get_backend()
+    t0 = time.time()
+    model = MNIST(seed)
+    opt = SGD(model, lr, gradClip=1000.0)
+    train = DataLoader("mnist", True, 0.1307, 0.3081, (1, 28, 28), root=root)
+    train.normalize()
+    prepare = time.time() - t0
+    out("Data normalized (all prepare time) in %f sec" % prepare)
+    loss_save = []
+    addr = be.getMallocAddr()
+    for epoch in range(nbEpoch):
+        state = {"img": 0, "loss": 0.0}
+        out("Start training epoch %d" % (epoch + 1))
+        t1 = time.time()
+
+        def batch(batchIndex, x, target):
+            state["img"] += batchSize
+            xin = TensorR(Tensor.fromNumpy(np.ascontiguousarray(x)), isInput=True)
+            tgt = int_array(np.ascontiguousarray(target))
+            loss = gradR_loss(lambda dummy: model(xin).logSoftmaxB(1).nllLossB(tgt).sum())(Tensor.zeros(4))
+            state["loss"] += float(loss.toCPU()[0])
+            opt.step()
+            if train.length >= 10 and state["img"] % (train.length // 10) == 0:
+                out("Train epoch %d: [%d/%d (%.0f%%)]\tAverage Loss: %.6f" % (epoch, state["img"], train.length,
+                                                                           100.0 * state["img"] / train.length, state["loss"] / state["img"]))
+            be.resetMallocAddr(addr)
+
+        train.foreachBatch(batchSize, batch)
+        delta = (time.time() - t1) * 1e6
+        out("Training completed in %dms (%d us/images)" % (delta // 1000, delta // max(train.length, 1)))
+        loss_save.append(state["loss"] / max(train.length, 1))
+    total = time.time() - t0
+    write_result_file(result_path, loss_save, prepare, (total - prepare) / max(nbEpoch, 1))
+    return loss_save
+
+
+if __name__ == "__main__":
+    import sys
+    from .. import BackendHIP, set_backend
+    hip = BackendHIP()
+    hip.setup()
+    set_backend(hip)
+    train_from_files(sys.argv[1] if len(sys.argv) > 1 else "result_Lantern.txt", *(sys.argv[2:3]))
+    hip.cleanup()
+

@@ -492,6 +492,20 @@ class BackendHIP(Backend):
     def mask4D(self, x, lengths, n, c, d, t):
         self.lib.lh_mask4d(x.ptr, lengths.ptr, n, c, d, t); _lib.check()
 
+    def cifar_decode(self, records, count):
+        """records: uint8 host array [n, count + 1] (label byte, then pixels).  Uploads the bytes and decodes them on the
+        device; returns (x float32 [n, count], y int32 [n]) in arena memory (TensorDataLoader.scala:109-127)."""
+        records = np.ascontiguousarray(records, dtype=np.uint8)
+        n = int(records.shape[0])
+        assert records.ndim == 2 and records.shape[1] == count + 1, "records must be [n, count + 1] bytes"
+        raw = self.mallocArray((records.nbytes + 3) // 4, zero=False)
+        x = self.mallocArray(n * count, zero=False)
+        y = self.mallocArray(n, zero=False)
+        if n:
+            self.lib.lh_h2d(raw.ptr, records.ctypes.data, records.nbytes); _lib.check()
+            self.lib.lh_cifar_decode(raw.ptr, x.ptr, y.ptr, n, count); _lib.check()
+        return x, y
+
     # -- activations ---------------------------------------------------------------------------------
     def unary(self, op, x, n, inPlace=False, lo=-1.0, hi=1.0):
         y = x if inPlace else self.mallocArray(n, zero=False)

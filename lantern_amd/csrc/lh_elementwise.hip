@@ -82,6 +82,29 @@ struct Dims4 { int d[4]; int64_t sa[4]; int64_t sb[4]; };
 
 }  // namespace
 
+// Records of one label byte and `count` pixel bytes (CIFAR-10's .bin layout) -> x[n, count] = byte / 255.0f, y[n] = byte.
+// A thread turns 4 consecutive pixels into one 16-byte store; a wave reads 256 consecutive record bytes.  The division
+// is the correctly rounded one, so the floats carry the bits the host loop `(float)(unsigned char)b / 255.0f` gives.
+template <int V>
+__global__ void k_cifar_decode(const unsigned char* __restrict__ rec, float* __restrict__ x, int* __restrict__ y,
+                               int64_t n_groups, int count) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, st = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n_groups; i += st) {
+    const int64_t e = i * V, r = e / count;
+    const int j = (int)(e - r * count);
+    const unsigned char* src = rec + r * ((int64_t)count + 1) + 1 + j;
+    if (j == 0) y[r] = (int)src[-1];
+    if constexpr (V == 4) {
+      float4 o;
+      o.x = __fdiv_rn((float)src[0], 255.0f); o.y = __fdiv_rn((float)src[1], 255.0f);
+      o.z = __fdiv_rn((float)src[2], 255.0f); o.w = __fdiv_rn((float)src[3], 255.0f);
+      *reinterpret_cast<float4*>(x + e) = o;
+    } else {
+      x[e] = __fdiv_rn((float)src[0], 255.0f);
+    }
+  }
+}
+
 extern "C" {
 
 void lh_fill(float* x, float v, int64_t n) { ProfScope prof_(CAT_FILL);
@@ -117,6 +140,18 @@ void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t) {
   int64_t tot = (int64_t)n * c * d * t;
   if (tot <= 0) return;
   hipLaunchKernelGGL(k_mask4d, dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, x, lengths, tot, c * d, t);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_cifar_decode(const unsigned char* records, float* x, int* y, int n, int count) {
+  if (n < 0 || count <= 0) { LH_FAIL("lh_cifar_decode: n %d, count %d", n, count); return; }
+  if (n == 0) return;
+  const int64_t tot = (int64_t)n * count;
+  if (count % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    hipLaunchKernelGGL(k_cifar_decode<4>, dim3(stream_grid(tot / 4, TPB)), dim3(TPB), 0, g_stream, records, x, y, tot / 4, count);
+  } else {
+    hipLaunchKernelGGL(k_cifar_decode<1>, dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, records, x, y, tot, count);
+  }
   LH_CHECK_LAUNCH();
 }
 
