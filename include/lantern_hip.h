@@ -229,6 +229,17 @@ void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float*
 void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir);
 void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
                 int T, int B, int I, int H, int bidir);
+/* The LSTM and GRU modes of RNNBase (NNModule.scala:324-330 over the same cuDNN calls): mode 2 = LSTM (gates i, f, g, o;
+ * c' = f*c + i*g, h' = o*tanh(c')), 3 = GRU (gates r, z, n; n = tanh(W_in x + b_in + r*(W_hn h + b_hn)), h' = (1-z)*n + z*h),
+ * cuDNN's gate order and formulas.  One layer, zero initial state; x, y, w, dx, dw as for lh_rnn_fwd / lh_rnn_bwd with
+ * W_ih[G,I], W_hh[G,H], b_ih[G], b_hh[G] per direction, G = 4H or 3H.  `reserve` (cuDNN's reserve space) is caller memory of
+ * lh_rnn_gated_reserve_floats(...) floats that the forward call fills and the backward call consumes (it is overwritten:
+ * one backward call per forward call).  Both calls take a few [B, G] blocks (the GRU backward: T*B*G floats) from the top
+ * of the arena and release them before returning. */
+int64_t lh_rnn_gated_reserve_floats(int mode, int T, int B, int H, int bidir);
+void lh_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, float* reserve, int T, int B, int I, int H, int bidir);
+void lh_rnn_gated_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* reserve, float* dx, float beta_dx,
+                      float* dw, int T, int B, int I, int H, int bidir);
 /* ctcLoss (TD:349; CDN:1895-1938, cudnnCTCLoss): probs [T,B,A] are softmax outputs, class 0 is the blank;
  * h_labels (concatenated), h_label_len [B], h_input_len [B] are HOST arrays as in the cuDNN call;
  * costs[b] = -log p(labels_b | probs).  When dprobs is not NULL the gradient with respect to the

@@ -1,0 +1,214 @@
+// LSTM and GRU layers (RNNBase with LstmMode / GruMode: src/main/scala/lantern/NNModule.scala:324-417 over
+// cudnnRNNForwardTraining / BackwardData / BackwardWeights, src/main/scala/lantern/TensorDslCudnn.scala:1638-1893).
+//
+// Gate order and formulas are cuDNN's: LSTM i, f, g, o with c' = f*c + i*g, h' = o*tanh(c'); GRU r, z, n with
+// n = tanh(W_in x + b_in + r*(W_hn h + b_hn)), h' = (1 - z)*n + z*h.  One layer, zero initial state, optionally
+// bidirectional (y = forward half, then reverse half).  Parameters per direction: W_ih[G, I], W_hh[G, H], b_ih[G],
+// b_hh[G] with G = 4H or 3H (NNModule.scala:378-390).
+//
+// Everything that is not sequential is one matrix product over all time steps (lh_sgemm on MFMA): the input projection,
+// both weight gradients, the input gradient.  A time step is one [B, H] x [H, G] product with the previous state and one
+// element-wise kernel over [B, H].  The forward pass leaves the gate activations and the cell state (GRU: W_hn h + b_hn)
+// of every step in `reserve`; the backward pass turns the activations into pre-activation gradients in place.
+#include "lh_common.h"
+#include "../../include/lantern_hip.h"
+using namespace lh;
+
+namespace {
+
+constexpr int TPB = 256;
+
+__device__ __forceinline__ float sigm(float v) { return 1.0f / (1.0f + expf(-v)); }
+
+// act [B, 4H]: input projection of this step on entry, gate activations on exit.  gh [B, 4H] = h_prev W_hh^T or null.
+__global__ void __launch_bounds__(TPB) k_lstm_fwd_point(float* __restrict__ act, const float* __restrict__ gh, const float* __restrict__ b_ih,
+                                                        const float* __restrict__ b_hh, const float* __restrict__ c_prev, float* __restrict__ c,
+                                                        float* __restrict__ h, int B, int H, int ldh) {
+  const int idx = blockIdx.x * TPB + threadIdx.x;
+  if (idx >= B * H) return;
+  const int b = idx / H, j = idx - b * H;
+  float* a = act + (size_t)b * 4 * H + j;
+  float p[4];
+#pragma unroll
+  for (int g = 0; g < 4; g++) p[g] = a[g * H] + b_ih[g * H + j] + b_hh[g * H + j] + (gh ? gh[(size_t)b * 4 * H + g * H + j] : 0.f);
+  const float ig = sigm(p[0]), fg = sigm(p[1]), gg = tanhf(p[2]), og = sigm(p[3]);
+  const float cn = fg * (c_prev ? c_prev[idx] : 0.f) + ig * gg;
+  a[0] = ig; a[H] = fg; a[2 * H] = gg; a[3 * H] = og;
+  c[idx] = cn;
+  h[(size_t)b * ldh + j] = og * tanhf(cn);
+}
+
+// act [B, 4H]: activations on entry, pre-activation gradients on exit.  dh_rec / dc hold what flows in from the step
+// processed before (null / ignored on the first processed step); dc is rewritten with the cell gradient passed on.
+__global__ void __launch_bounds__(TPB) k_lstm_bwd_point(float* __restrict__ act, const float* __restrict__ c, const float* __restrict__ c_prev,
+                                                        const float* __restrict__ dy, const float* __restrict__ dh_rec, float* __restrict__ dc,
+                                                        int first, int B, int H, int ldh) {
+  const int idx = blockIdx.x * TPB + threadIdx.x;
+  if (idx >= B * H) return;
+  const int b = idx / H, j = idx - b * H;
+  float* a = act + (size_t)b * 4 * H + j;
+  const float ig = a[0], fg = a[H], gg = a[2 * H], og = a[3 * H];
+  const float dh = dy[(size_t)b * ldh + j] + (dh_rec ? dh_rec[idx] : 0.f);
+  const float tc = tanhf(c[idx]);
+  const float dcc = dh * og * (1.f - tc * tc) + (first ? 0.f : dc[idx]);
+  const float cp = c_prev ? c_prev[idx] : 0.f;
+  a[0] = dcc * gg * ig * (1.f - ig);
+  a[H] = dcc * cp * fg * (1.f - fg);
+  a[2 * H] = dcc * ig * (1.f - gg * gg);
+  a[3 * H] = dh * tc * og * (1.f - og);
+  dc[idx] = dcc * fg;
+}
+
+// act [B, 3H]: input projection on entry, r, z, n on exit.  gh [B, 3H] = h_prev W_hh^T or null.  q [B, H] = W_hn h + b_hn.
+__global__ void __launch_bounds__(TPB) k_gru_fwd_point(float* __restrict__ act, const float* __restrict__ gh, const float* __restrict__ b_ih,
+                                                       const float* __restrict__ b_hh, const float* __restrict__ h_prev, float* __restrict__ q,
+                                                       float* __restrict__ h, int B, int H, int ldh) {
+  const int idx = blockIdx.x * TPB + threadIdx.x;
+  if (idx >= B * H) return;
+  const int b = idx / H, j = idx - b * H;
+  float* a = act + (size_t)b * 3 * H + j;
+  const float* g = gh ? gh + (size_t)b * 3 * H + j : nullptr;
+  const float r = sigm(a[0] + b_ih[j] + b_hh[j] + (g ? g[0] : 0.f));
+  const float z = sigm(a[H] + b_ih[H + j] + b_hh[H + j] + (g ? g[H] : 0.f));
+  const float qq = (g ? g[2 * H] : 0.f) + b_hh[2 * H + j];
+  const float n = tanhf(a[2 * H] + b_ih[2 * H + j] + r * qq);
+  const float hp = h_prev ? h_prev[(size_t)b * ldh + j] : 0.f;
+  a[0] = r; a[H] = z; a[2 * H] = n;
+  q[idx] = qq;
+  h[(size_t)b * ldh + j] = (1.f - z) * n + z * hp;
+}
+
+// act [B, 3H]: r, z, n on entry, gradients of the input-side pre-activations on exit; dgh [B, 3H] receives those of the
+// hidden side (the n column scaled by r).  carry [B, H]: the recurrent gradient on entry (ignored when first), dh * z on
+// exit; the caller adds dgh W_hh to it.
+__global__ void __launch_bounds__(TPB) k_gru_bwd_point(float* __restrict__ act, float* __restrict__ dgh, const float* __restrict__ q,
+                                                       const float* __restrict__ h_prev, const float* __restrict__ dy, float* __restrict__ carry,
+                                                       int first, int B, int H, int ldh) {
+  const int idx = blockIdx.x * TPB + threadIdx.x;
+  if (idx >= B * H) return;
+  const int b = idx / H, j = idx - b * H;
+  float* a = act + (size_t)b * 3 * H + j;
+  float* g = dgh + (size_t)b * 3 * H + j;
+  const float r = a[0], z = a[H], n = a[2 * H];
+  const float dh = dy[(size_t)b * ldh + j] + (first ? 0.f : carry[idx]);
+  const float hp = h_prev ? h_prev[(size_t)b * ldh + j] : 0.f;
+  const float dn = dh * (1.f - z) * (1.f - n * n);
+  const float dz = dh * (hp - n) * z * (1.f - z);
+  const float dr = dn * q[idx] * r * (1.f - r);
+  a[0] = dr; a[H] = dz; a[2 * H] = dn;
+  g[0] = dr; g[H] = dz; g[2 * H] = dn * r;
+  carry[idx] = dh * z;
+}
+
+__global__ void __launch_bounds__(TPB) k_add_into(float* __restrict__ dst, const float* __restrict__ src, int n) {
+  const int i = blockIdx.x * TPB + threadIdx.x;
+  if (i < n) dst[i] += src[i];
+}
+
+int gates_of(int mode) { return mode == 2 ? 4 : 3; }
+size_t dir_params(int mode, int I, int H) { const size_t G = (size_t)gates_of(mode) * H; return G * I + G * H + 2 * G; }
+size_t dir_reserve(int mode, int T, int B, int H) { return (size_t)T * B * (gates_of(mode) + 1) * H; }
+unsigned point_grid(int B, int H) { return (unsigned)cdiv((int64_t)B * H, TPB); }
+
+bool check_shape(const char* who, int mode, int T, int B, int I, int H) {
+  if (mode != 2 && mode != 3) { LH_FAIL("%s: mode %d (2 = LSTM, 3 = GRU)", who, mode); return false; }
+  if (T < 1 || B < 1 || I < 1 || H < 1) { LH_FAIL("%s: bad shape T%d B%d I%d H%d", who, T, B, I, H); return false; }
+  if ((int64_t)T * B * 4 * H > INT32_MAX || (int64_t)B * 4 * H > (1 << 28)) { LH_FAIL("%s: T%d B%d H%d too large", who, T, B, H); return false; }
+  return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t lh_rnn_gated_reserve_floats(int mode, int T, int B, int H, int bidir) {
+  if ((mode != 2 && mode != 3) || T < 1 || B < 1 || H < 1) return 0;
+  return (int64_t)((bidir ? 2 : 1) * dir_reserve(mode, T, B, H));
+}
+
+void lh_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, float* reserve, int T, int B, int I, int H, int bidir) {
+  if (!check_shape("lh_rnn_gated_fwd", mode, T, B, I, H)) return;
+  LH_REQUIRE(x && w && y && reserve, "lh_rnn_gated_fwd: null operand");
+  const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
+  const size_t gh_bytes = (size_t)B * G * sizeof(float);
+  float* gh = (float*)lh_malloc_uninit(gh_bytes);
+  if (gh == nullptr) return;
+  for (int d = 0; d < D; d++) {
+    const float* Wih = w + d * dir_params(mode, I, H);
+    const float* Whh = Wih + (size_t)G * I; const float* bih = Whh + (size_t)G * H; const float* bhh = bih + G;
+    float* act = reserve + d * dir_reserve(mode, T, B, H);
+    float* aux = act + (size_t)T * B * G;
+    lh_sgemm(0, 1, T * B, G, I, 1.0f, x, I, Wih, I, 0.0f, act, G);          // input projection of every step
+    for (int step = 0; step < T; step++) {
+      const int t = d == 0 ? step : T - 1 - step, tp = d == 0 ? t - 1 : t + 1;
+      float* h = y + (size_t)t * B * ldh + d * H;
+      const float* hp = step == 0 ? nullptr : y + (size_t)tp * B * ldh + d * H;
+      if (hp) lh_sgemm(0, 1, B, G, H, 1.0f, hp, ldh, Whh, H, 0.0f, gh, G);
+      float* a = act + (size_t)t * B * G;
+      if (mode == 2)
+        hipLaunchKernelGGL(k_lstm_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh,
+                           hp ? aux + (size_t)tp * B * H : nullptr, aux + (size_t)t * B * H, h, B, H, ldh);
+      else
+        hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh, hp,
+                           aux + (size_t)t * B * H, h, B, H, ldh);
+    }
+  }
+  lh_free_top(gh_bytes);       // stream order: the kernels above run before anything that reuses the space
+  LH_CHECK_LAUNCH();
+}
+
+void lh_rnn_gated_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* reserve, float* dx, float beta_dx,
+                      float* dw, int T, int B, int I, int H, int bidir) {
+  if (!check_shape("lh_rnn_gated_bwd", mode, T, B, I, H)) return;
+  LH_REQUIRE(beta_dx == 0.f || beta_dx == 1.f, "lh_rnn_gated_bwd: beta must be 0 or 1");
+  LH_REQUIRE(x && y && dy && w && reserve && dw, "lh_rnn_gated_bwd: null operand");
+  const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
+  // scratch from the top of the arena: recurrent gradient [B, H], cell gradient [B, H], column sums [2G],
+  // and for the GRU the hidden-side pre-activation gradients of every step [T, B, G]
+  const size_t n_bh = (size_t)B * H, n_dgh = mode == 3 ? (size_t)T * B * G : 0;
+  const size_t bytes = (2 * n_bh + 2 * (size_t)G + n_dgh) * sizeof(float);
+  float* scratch = (float*)lh_malloc_uninit(bytes);
+  if (scratch == nullptr) return;
+  float* carry = scratch; float* dc = carry + n_bh; float* colsum = dc + n_bh; float* dgh = colsum + 2 * (size_t)G;
+  for (int d = 0; d < D; d++) {
+    const size_t off = d * dir_params(mode, I, H);
+    const float* Wih = w + off; const float* Whh = Wih + (size_t)G * I;
+    float* dWih = dw + off; float* dWhh = dWih + (size_t)G * I; float* dbih = dWhh + (size_t)G * H; float* dbhh = dbih + G;
+    float* act = reserve + d * dir_reserve(mode, T, B, H);
+    const float* aux = act + (size_t)T * B * G;
+    for (int k = 0; k < T; k++) {
+      const int t = d == 0 ? T - 1 - k : k;                        // reverse of the forward processing order
+      const int tp = d == 0 ? t - 1 : t + 1;                       // the step whose state this one consumed
+      const bool has_prev = d == 0 ? t > 0 : t < T - 1;
+      float* a = act + (size_t)t * B * G;
+      const float* dyt = dy + (size_t)t * B * ldh + d * H;
+      if (mode == 2) {
+        hipLaunchKernelGGL(k_lstm_bwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, aux + (size_t)t * B * H,
+                           has_prev ? aux + (size_t)tp * B * H : nullptr, dyt, k == 0 ? nullptr : carry, dc, k == 0 ? 1 : 0, B, H, ldh);
+        if (has_prev) lh_sgemm(0, 0, B, H, G, 1.0f, a, G, Whh, H, 0.0f, carry, H);
+      } else {
+        float* g = dgh + (size_t)t * B * G;
+        hipLaunchKernelGGL(k_gru_bwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, g, aux + (size_t)t * B * H,
+                           has_prev ? y + (size_t)tp * B * ldh + d * H : nullptr, dyt, carry, k == 0 ? 1 : 0, B, H, ldh);
+        if (has_prev) lh_sgemm(0, 0, B, H, G, 1.0f, g, G, Whh, H, 1.0f, carry, H);
+      }
+    }
+    const float* hid = mode == 2 ? act : dgh;                       // gradients of the hidden-side pre-activations
+    lh_sgemm(1, 0, G, I, T * B, 1.0f, act, G, x, I, 1.0f, dWih, I);
+    if (T > 1) {
+      // dW_hh += sum_t hid_t^T h_{prev(t)}: forward pairs (t, t-1), reverse pairs (t, t+1)
+      const float* A = d == 0 ? hid + (size_t)B * G : hid;
+      const float* Bm = d == 0 ? y + d * H : y + (size_t)B * ldh + d * H;
+      lh_sgemm(1, 0, G, H, (T - 1) * B, 1.0f, A, G, Bm, ldh, 1.0f, dWhh, H);
+    }
+    lh_sum_dim(act, colsum, 1, T * B, G);
+    hipLaunchKernelGGL(k_add_into, dim3((unsigned)cdiv(G, TPB)), dim3(TPB), 0, g_stream, dbih, colsum, G);
+    if (mode == 3) lh_sum_dim(dgh, colsum + G, 1, T * B, G);
+    hipLaunchKernelGGL(k_add_into, dim3((unsigned)cdiv(G, TPB)), dim3(TPB), 0, g_stream, dbhh, mode == 3 ? colsum + G : colsum, G);
+    if (dx) lh_sgemm(0, 0, T * B, I, G, 1.0f, act, G, Wih, I, d == 0 ? beta_dx : 1.0f, dx, I);
+  }
+  lh_free_top(bytes);
+  LH_CHECK_LAUNCH();
+}
+
+}  // extern "C"

@@ -104,22 +104,58 @@ class BatchNorm1D(BatchNorm2D):
 
 class RNNBase(Module):
     """NN:332-417: one parameter buffer holding, per layer and direction, w_ih [gate, in], w_hh [gate, hidden],
-    b_ih, b_hh (forward direction first), initialised with Tensor.rand(size, 0.01).  Modes: "relu", "tanh"."""
-    MODES = {"relu": 0, "tanh": 1}
+    b_ih, b_hh (forward direction first), initialised with Tensor.rand(size, 0.01).  Modes "relu", "tanh", "lstm", "gru"
+    (1, 1, 4 and 3 gates of hiddenSize rows each).  Layers after the first read the previous layer's output, which is
+    numDirections * hiddenSize wide (what cuDNN expects; the reference's size formula, NN:357, leaves the factor out and
+    so only works for one direction).  Zero initial state; no dropout between layers."""
+    MODES = {"relu": (0, 1), "tanh": (1, 1), "lstm": (2, 4), "gru": (3, 3)}
 
     def __init__(self, mode, inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, name="rnn"):
         super().__init__(name)
-        assert mode in self.MODES, "RNN mode %r is not built (relu and tanh are)" % (mode,)
+        assert mode in self.MODES, "RNN mode %r (relu, tanh, lstm, gru)" % (mode,)
         assert inputSize >= 1, "Input size must be at least 1"
         assert hiddenSize >= 1, "Hidden size must be at least 1"
-        assert numLayers == 1, "one layer per RNNBase (the DeepSpeech program stacks single-layer modules)"
+        assert numLayers >= 1, "Number of layers must be at least 1"
         assert dropout == 0.0, "dropout between layers is not built"
-        self.mode, self.inputSize, self.hiddenSize, self.bidirectional = self.MODES[mode], inputSize, hiddenSize, bidirectional
-        per_dir = hiddenSize * inputSize + hiddenSize * hiddenSize + 2 * hiddenSize
-        self.parameterBuffer = self.param("parameterBuffer", Tensor.rand((per_dir * (2 if bidirectional else 1),), 0.01))
+        self.mode, self.numGates = self.MODES[mode]
+        self.inputSize, self.hiddenSize, self.numLayers, self.bidirectional = inputSize, hiddenSize, numLayers, bidirectional
+        self.numDirections = 2 if bidirectional else 1
+        self.gateSize = hiddenSize * self.numGates
+        self.offsets, total = [], 0
+        for layer in range(numLayers):
+            self.offsets.append(total)
+            total += self.numDirections * self._dir_size(self._layer_input(layer))
+        self.parameterBuffer = self.param("parameterBuffer", Tensor.rand((total,), 0.01))
+
+    def _layer_input(self, layer):
+        return self.inputSize if layer == 0 else self.hiddenSize * self.numDirections
+
+    def _dir_size(self, layerInputSize):
+        return self.gateSize * layerInputSize + self.gateSize * self.hiddenSize + 2 * self.gateSize
+
+    def getParameterSize(self):
+        return self.parameterBuffer.x.scalarCount
 
     def __call__(self, x):
-        return x.rnn(self.mode, self.parameterBuffer, self.hiddenSize, self.bidirectional)
+        for layer in range(self.numLayers):
+            x = x.rnn(self.mode, self.parameterBuffer, self.hiddenSize, self.bidirectional, offset=self.offsets[layer])
+        return x
+
+
+def RNNRelu(inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, name="rnn_relu"):      # NN:316-330
+    return RNNBase("relu", inputSize, hiddenSize, numLayers, dropout, bidirectional, name)
+
+
+def RNNTanh(inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, name="rnn_tanh"):
+    return RNNBase("tanh", inputSize, hiddenSize, numLayers, dropout, bidirectional, name)
+
+
+def LSTM(inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, name="lstm"):
+    return RNNBase("lstm", inputSize, hiddenSize, numLayers, dropout, bidirectional, name)
+
+
+def GRU(inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, name="gru"):
+    return RNNBase("gru", inputSize, hiddenSize, numLayers, dropout, bidirectional, name)
 
 
 # ---- optimizers (NN:255-303) -------------------------------------------------------------------

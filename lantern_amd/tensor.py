@@ -796,18 +796,26 @@ class TensorR:
         return y
 
     # -- recurrent layer, CTC ----------------------------------------------------------------------------
-    def rnn(self, mode, params, hidden, bidirectional):
+    def rnn(self, mode, params, hidden, bidirectional, offset=0):
         """RNNBase.apply (NN:392-415): one layer over [seqLength, batch, inputSize], zero initial state;
-        `params` is the packed parameter buffer (a TensorR).  mode 0 = relu, 1 = tanh."""
+        `params` is the packed parameter buffer (a TensorR), this layer's parameters starting `offset` elements in.
+        mode 0 = relu, 1 = tanh, 2 = LSTM, 3 = GRU (cuDNN's numbering)."""
         be = get_backend()
         assert self.x.rank == 3, "RNN input should have rank 3: [seqLength x batchSize x inputSize]"
         T, Bn, I = self.x.shape
         D = 2 if bidirectional else 1
-        ybuf = be.rnn_forward(mode, self.x.data, params.x.data, T, Bn, I, hidden, bidirectional)
+        w, dw = (params.x.data, params.d.data) if offset == 0 else (params.x.data.offset(offset), params.d.data.offset(offset))
+        if mode >= 2:
+            ybuf, reserve = be.rnn_gated_forward(mode, self.x.data, w, T, Bn, I, hidden, bidirectional)
+        else:
+            ybuf = be.rnn_forward(mode, self.x.data, w, T, Bn, I, hidden, bidirectional)
         y = TensorR._new(Tensor(ybuf, (T, Bn, D * hidden)))
         def back():
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()
-            be.rnn_backward(mode, self.x.data, ybuf, y.d.data, params.x.data, xd, params.d.data, T, Bn, I, hidden, bidirectional, beta)
+            if mode >= 2:
+                be.rnn_gated_backward(mode, self.x.data, ybuf, y.d.data, w, reserve, xd, dw, T, Bn, I, hidden, bidirectional, beta)
+            else:
+                be.rnn_backward(mode, self.x.data, ybuf, y.d.data, w, xd, dw, T, Bn, I, hidden, bidirectional, beta)
         _tape.append(back)
         return y
 

@@ -283,6 +283,15 @@ class BackendCPU(Backend):
         self._c("lc_rnn_bwd", I(mode), P(x.ptr), P(y.ptr), P(dy.ptr), P(w.ptr), P(dx.ptr if dx is not None else 0), P(dw.ptr),
                 I(T), I(B), I(I_), I(H), I(int(bidir)))
 
+    def rnn_gated_forward(self, mode, x, w, T, B, I_, H, bidir):
+        y = self.mallocArray(T * B * H * (2 if bidir else 1))
+        self._c("lc_rnn_gated_fwd", I(mode), P(x.ptr), P(w.ptr), P(y.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))
+        return y, None
+
+    def rnn_gated_backward(self, mode, x, y, dy, w, reserve, dx, dw, T, B, I_, H, bidir, beta_dx=1.0):
+        self._c("lc_rnn_gated_bwd", I(mode), P(x.ptr), P(dy.ptr), P(w.ptr), P(dx.ptr if dx is not None else 0), P(dw.ptr),
+                I(T), I(B), I(I_), I(H), I(int(bidir)))
+
     def sgd_update(self, x, d, lr, n): self._c("lc_sgd", P(x.ptr), P(d.ptr), F(lr), L(n))
     def adagrad_update(self, x, d, m, lr, clip, n): self._c("lc_adagrad", P(x.ptr), P(d.ptr), P(m.ptr), F(lr), F(clip), L(n))
     def momentum_update(self, x, d, v, lr, mu, clip, nesterov, n):

@@ -832,3 +832,140 @@ void lc_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
   }
   free(dpre); free(hs); free(dh);
 }
+
+/* ---------------------------------------------------------- LSTM and GRU
+ * parity unpinned against the reference (no CPU implementation and no asserted vector; the GPU path is the same cuDNN
+ * calls as above with CUDNN_LSTM / CUDNN_GRU, NN:324-330).  cuDNN's documented formulas, gates in its order:
+ *   LSTM: i, f, o = sigmoid, g = tanh of (W x + b_i + R h + b_h), order i f g o;  c' = f c + i g;  h' = o tanh(c')
+ *   GRU:  r, z = sigmoid(W x + b_i + R h + b_h);  n = tanh(W_n x + b_in + r (R_n h + b_hn));  h' = (1 - z) n + z h
+ * Packed weights per direction as NN:378-390 with G = 4H / 3H rows.  Written per sample and per step with double
+ * accumulation; the backward pass keeps no state from the forward one (it recomputes it) and adds each step's outer
+ * products into dw as it goes.  Checked against torch.nn.LSTM / torch.nn.GRU (CPU) in the tests. */
+static int gated_ng(int mode) { return mode == 2 ? 4 : 3; }
+static size_t gated_dir_params(int mode, int I, int H) { size_t G = (size_t)gated_ng(mode) * H; return G * I + G * H + 2 * G; }
+static double sigm_d(double v) { return 1.0 / (1.0 + exp(-v)); }
+
+/* One direction of one sample, forward; fills (when not NULL) per-step records for the backward pass:
+ * gate[T][G] activations, cell[T][H] (LSTM: c_t; GRU: q_t = R_n h + b_hn), hid[T][H] = h_t. */
+static void gated_forward_sample(int mode, const float* x, size_t xs, const float* Wih, const float* Whh, const float* bih, const float* bhh,
+                                 int T, int I, int H, int reverse, double* gate, double* cell, double* hid) {
+  const int ng = gated_ng(mode), G = ng * H;
+  double* h = (double*)calloc((size_t)H, sizeof(double));
+  double* c = (double*)calloc((size_t)H, sizeof(double));
+  double* px = (double*)malloc((size_t)G * sizeof(double));
+  double* ph = (double*)malloc((size_t)G * sizeof(double));
+  for (int step = 0; step < T; step++) {
+    const int t = reverse ? T - 1 - step : step;
+    const float* xt = x + (size_t)t * xs;
+    for (int g = 0; g < G; g++) {
+      double a = 0.0, r = 0.0;
+      for (int k = 0; k < I; k++) a += (double)Wih[(size_t)g * I + k] * xt[k];
+      for (int k = 0; k < H; k++) r += (double)Whh[(size_t)g * H + k] * h[k];
+      px[g] = a + bih[g]; ph[g] = r + bhh[g];
+    }
+    double* gt = gate + (size_t)t * G;
+    for (int j = 0; j < H; j++) {
+      if (mode == 2) {
+        const double ig = sigm_d(px[j] + ph[j]), fg = sigm_d(px[H + j] + ph[H + j]);
+        const double gg = tanh(px[2 * H + j] + ph[2 * H + j]), og = sigm_d(px[3 * H + j] + ph[3 * H + j]);
+        c[j] = fg * c[j] + ig * gg;
+        gt[j] = ig; gt[H + j] = fg; gt[2 * H + j] = gg; gt[3 * H + j] = og;
+        cell[(size_t)t * H + j] = c[j];
+        hid[(size_t)t * H + j] = og * tanh(c[j]);
+      } else {
+        const double r = sigm_d(px[j] + ph[j]), z = sigm_d(px[H + j] + ph[H + j]);
+        const double n = tanh(px[2 * H + j] + r * ph[2 * H + j]);
+        gt[j] = r; gt[H + j] = z; gt[2 * H + j] = n;
+        cell[(size_t)t * H + j] = ph[2 * H + j];
+        hid[(size_t)t * H + j] = (1.0 - z) * n + z * h[j];
+      }
+    }
+    for (int j = 0; j < H; j++) h[j] = hid[(size_t)t * H + j];
+  }
+  free(h); free(c); free(px); free(ph);
+}
+
+void lc_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+  const int D = bidir ? 2 : 1, G = gated_ng(mode) * H;
+  double* gate = (double*)malloc((size_t)T * G * sizeof(double));
+  double* cell = (double*)malloc((size_t)T * H * sizeof(double));
+  double* hid = (double*)malloc((size_t)T * H * sizeof(double));
+  for (int d = 0; d < D; d++) {
+    const float* Wih = w + d * gated_dir_params(mode, I, H); const float* Whh = Wih + (size_t)G * I;
+    const float* bih = Whh + (size_t)G * H; const float* bhh = bih + G;
+    for (int b = 0; b < B; b++) {
+      gated_forward_sample(mode, x + (size_t)b * I, (size_t)B * I, Wih, Whh, bih, bhh, T, I, H, d, gate, cell, hid);
+      for (int t = 0; t < T; t++)
+        for (int j = 0; j < H; j++) y[((size_t)t * B + b) * D * H + (size_t)d * H + j] = (float)hid[(size_t)t * H + j];
+    }
+  }
+  free(gate); free(cell); free(hid);
+}
+
+/* dx (may be NULL) and dw accumulate. */
+void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w, float* dx, float* dw, int T, int B, int I, int H, int bidir) {
+  const int D = bidir ? 2 : 1, ng = gated_ng(mode), G = ng * H;
+  double* gate = (double*)malloc((size_t)T * G * sizeof(double));
+  double* cell = (double*)malloc((size_t)T * H * sizeof(double));
+  double* hid = (double*)malloc((size_t)T * H * sizeof(double));
+  double* dh = (double*)malloc((size_t)H * sizeof(double));
+  double* dc = (double*)malloc((size_t)H * sizeof(double));
+  double* gx = (double*)malloc((size_t)G * sizeof(double));       /* gradient of the input-side pre-activations */
+  double* gh = (double*)malloc((size_t)G * sizeof(double));       /* ... of the hidden-side ones */
+  const size_t np = gated_dir_params(mode, I, H);
+  double* acc = (double*)calloc(np, sizeof(double));
+  for (int d = 0; d < D; d++) {
+    const size_t off = d * np;
+    const float* Wih = w + off; const float* Whh = Wih + (size_t)G * I; const float* bih = Whh + (size_t)G * H; const float* bhh = bih + G;
+    double* aWih = acc; double* aWhh = aWih + (size_t)G * I; double* abih = aWhh + (size_t)G * H; double* abhh = abih + G;
+    memset(acc, 0, np * sizeof(double));
+    for (int b = 0; b < B; b++) {
+      gated_forward_sample(mode, x + (size_t)b * I, (size_t)B * I, Wih, Whh, bih, bhh, T, I, H, d, gate, cell, hid);
+      for (int j = 0; j < H; j++) dh[j] = dc[j] = 0.0;
+      for (int step = T - 1; step >= 0; step--) {
+        const int t = d ? T - 1 - step : step;
+        const int tp = d ? t + 1 : t - 1;
+        const double* gt = gate + (size_t)t * G;
+        const double* hp = step == 0 ? NULL : hid + (size_t)tp * H;
+        for (int j = 0; j < H; j++) {
+          const double g = dh[j] + dy[((size_t)t * B + b) * D * H + (size_t)d * H + j];
+          if (mode == 2) {
+            const double ig = gt[j], fg = gt[H + j], gg = gt[2 * H + j], og = gt[3 * H + j];
+            const double tc = tanh(cell[(size_t)t * H + j]);
+            const double cp = step == 0 ? 0.0 : cell[(size_t)tp * H + j];
+            const double dcell = dc[j] + g * og * (1.0 - tc * tc);
+            gx[j] = dcell * gg * ig * (1.0 - ig);
+            gx[H + j] = dcell * cp * fg * (1.0 - fg);
+            gx[2 * H + j] = dcell * ig * (1.0 - gg * gg);
+            gx[3 * H + j] = g * tc * og * (1.0 - og);
+            gh[j] = gx[j]; gh[H + j] = gx[H + j]; gh[2 * H + j] = gx[2 * H + j]; gh[3 * H + j] = gx[3 * H + j];
+            dc[j] = dcell * fg;
+            dh[j] = 0.0;
+          } else {
+            const double r = gt[j], z = gt[H + j], n = gt[2 * H + j], q = cell[(size_t)t * H + j];
+            const double hprev = hp ? hp[j] : 0.0;
+            const double dn = g * (1.0 - z) * (1.0 - n * n);
+            gx[j] = dn * q * r * (1.0 - r);
+            gx[H + j] = g * (hprev - n) * z * (1.0 - z);
+            gx[2 * H + j] = dn;
+            gh[j] = gx[j]; gh[H + j] = gx[H + j]; gh[2 * H + j] = dn * r;
+            dh[j] = g * z;
+          }
+        }
+        const float* xt = x + ((size_t)t * B + b) * I;
+        for (int g = 0; g < G; g++) {
+          for (int k = 0; k < I; k++) aWih[(size_t)g * I + k] += gx[g] * xt[k];
+          if (hp) for (int k = 0; k < H; k++) aWhh[(size_t)g * H + k] += gh[g] * hp[k];
+          abih[g] += gx[g]; abhh[g] += gh[g];
+        }
+        for (int k = 0; k < H; k++) { double s = 0.0; for (int g = 0; g < G; g++) s += gh[g] * Whh[(size_t)g * H + k]; dh[k] += s; }
+        if (dx) for (int k = 0; k < I; k++) {
+          double s = 0.0; for (int g = 0; g < G; g++) s += gx[g] * Wih[(size_t)g * I + k];
+          dx[((size_t)t * B + b) * I + k] += (float)s;
+        }
+      }
+    }
+    for (size_t i = 0; i < np; i++) dw[off + i] += (float)acc[i];
+  }
+  free(gate); free(cell); free(hid); free(dh); free(dc); free(gx); free(gh); free(acc);
+}

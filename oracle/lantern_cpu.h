@@ -18,7 +18,7 @@
  * Pinning status of each function (what independent evidence fixes it) is
  * listed in tests/test_oracle_golden.py; functions without a reference
  * vector are marked "parity unpinned" there and below.
- *   parity unpinned: lc_ctc_loss, lc_rnn_fwd, lc_rnn_bwd (no asserted vector and no CPU implementation in the
+ *   parity unpinned: lc_ctc_loss, lc_rnn_fwd, lc_rnn_bwd, lc_rnn_gated_fwd, lc_rnn_gated_bwd (no asserted vector and no CPU implementation in the
  *   reference; both are checked against torch's CPU routines in tests/test_oracle_math.py).
  */
 #ifndef LANTERN_CPU_ORACLE_H
@@ -139,6 +139,9 @@ void lc_adagrad(float* x, float* d, float* m, float lr, float clip, long n);
 void lc_ctc_loss(const float* probs, float* dprobs, const int* labels, const int* label_len, const int* input_len,
                  float* costs, int T, int B, int A);
 void lc_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir);
+/* LSTM (mode 2) / GRU (mode 3), cuDNN formulas; parity unpinned against the reference, checked against torch.nn.LSTM / GRU */
+void lc_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir);
+void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w, float* dx, float* dw, int T, int B, int I, int H, int bidir);
 void lc_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float* dw,
                 int T, int B, int I, int H, int bidir);
 

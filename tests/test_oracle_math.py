@@ -249,3 +249,41 @@ def test_rnn_against_torch(mode, bidir):
         for nm, size in zip(names, (H * In, H * H, H, H)):
             g = getattr(rnn, nm + ("_reverse" if d else "")).grad.numpy().ravel()
             np.testing.assert_allclose(dw[o:o + size] - 1, g, rtol=1e-4, atol=1e-5, err_msg=nm + str(d)); o += size
+
+
+@pytest.mark.parametrize("mode", [2, 3], ids=["lstm", "gru"])
+@pytest.mark.parametrize("bidir", [False, True], ids=["uni", "bi"])
+def test_gated_rnn_against_torch(mode, bidir):
+    """lc_rnn_gated_fwd / lc_rnn_gated_bwd (cuDNN's LSTM / GRU formulas; nothing on the reference's CPU side) against
+    torch.nn.LSTM / torch.nn.GRU, which use the same gate order (i f g o; r z n) and the same reset-after-product GRU:
+    outputs, input gradient and every weight gradient, packed W_ih, W_hh, b_ih, b_hh per direction.  A swapped gate, a
+    reset gate applied before the product or a bias on the wrong side of it changes the output or one of the bias gradients."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.RandomState(20 + mode)
+    T, B, In, H = 6, 3, 5, 4
+    D, G = (2 if bidir else 1), (4 if mode == 2 else 3) * H
+    per = G * In + G * H + 2 * G
+    w = (rng.randn(D * per) * 0.5).astype(np.float32)
+    x = rng.randn(T, B, In).astype(np.float32); dy = rng.randn(T, B, D * H).astype(np.float32)
+    net = (torch.nn.LSTM if mode == 2 else torch.nn.GRU)(In, H, 1, bidirectional=bidir)
+    names = ["weight_ih_l0", "weight_hh_l0", "bias_ih_l0", "bias_hh_l0"]
+    sizes, shapes = (G * In, G * H, G, G), ((G, In), (G, H), (G,), (G,))
+    with torch.no_grad():
+        for d in range(D):
+            o = d * per
+            for nm, size, shape in zip(names, sizes, shapes):
+                getattr(net, nm + ("_reverse" if d else "")).copy_(torch.tensor(w[o:o + size].reshape(shape))); o += size
+    tx = torch.tensor(x, requires_grad=True)
+    ty, _ = net(tx)
+    ty.backward(torch.tensor(dy))
+    y = np.zeros((T, B, D * H), np.float32)
+    lc.lc_rnn_gated_fwd(I(mode), cptr(x), cptr(w), cptr(y), I(T), I(B), I(In), I(H), I(int(bidir)))
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-5, atol=1e-6)
+    dx = np.ones_like(x); dw = np.ones_like(w)                    # both accumulate
+    lc.lc_rnn_gated_bwd(I(mode), cptr(x), cptr(dy), cptr(w), cptr(dx), cptr(dw), I(T), I(B), I(In), I(H), I(int(bidir)))
+    np.testing.assert_allclose(dx - 1, tx.grad.numpy(), rtol=1e-4, atol=1e-5)
+    for d in range(D):
+        o = d * per
+        for nm, size in zip(names, sizes):
+            g = getattr(net, nm + ("_reverse" if d else "")).grad.numpy().ravel()
+            np.testing.assert_allclose(dw[o:o + size] - 1, g, rtol=1e-4, atol=1e-5, err_msg=nm + str(d)); o += size

@@ -661,6 +661,55 @@ def test_rnn_forward_and_backward(pair, case):
     check_all(pair.run(f), rtol=3e-4)
 
 
+@pytest.mark.parametrize("case", [(2, True, 7, 5, 20, 48), (3, True, 7, 5, 20, 48), (2, False, 1, 2, 5, 16), (3, False, 1, 2, 5, 16), (2, False, 9, 33, 7, 37),
+                                  (3, True, 4, 3, 33, 130), (2, True, 3, 4, 161, 96), (3, False, 12, 8, 64, 256)]
+                         + _random_cases(108, 6, lambda r: (_ri(r, 2, 3), bool(r.rand() < 0.5), _ri(r, 1, 8), _ri(r, 1, 9), _ri(r, 1, 40), _pick(r, [5, 16, 37, 64, 130]))),
+                         ids=lambda c: "mode%d_bi%d_T%d_B%d_I%d_H%d" % c)
+def test_gated_rnn_forward_and_backward(pair, case):
+    """LSTM (mode 2) and GRU (mode 3) layers against the oracle: outputs, input gradient (accumulate, overwrite, none)
+    and the packed weight gradient."""
+    mode, bidir, T, Bn, In, H = case
+    D, G = (2 if bidir else 1), (4 if mode == 2 else 3) * H
+    rng = np.random.RandomState(41)
+    per = G * In + G * H + 2 * G
+    w = (rng.randn(D * per) * (0.7 / np.sqrt(H))).astype(np.float32)
+    x = rng.randn(T, Bn, In).astype(np.float32); dy = rng.randn(T, Bn, D * H).astype(np.float32)
+
+    def f(be, up, down):
+        X, W = up(x), up(w)
+        y, reserve = be.rnn_gated_forward(mode, X, W, T, Bn, In, H, bidir)
+        dx = up(np.ones(x.size, np.float32)); dw = up(np.ones(w.size, np.float32))
+        be.rnn_gated_backward(mode, X, y, up(dy), W, reserve, dx, dw, T, Bn, In, H, bidir, 1.0)
+        outs = [down(y, dy.shape), down(dx, x.shape), down(dw, w.shape)]
+        if be.name == "hip":
+            y2, reserve2 = be.rnn_gated_forward(mode, X, W, T, Bn, In, H, bidir)                        # the reserve is used up: run forward again
+            dx0 = up(np.full(x.size, 5.0, np.float32)); dw0 = up(np.zeros(w.size, np.float32))
+            be.rnn_gated_backward(mode, X, y2, up(dy), W, reserve2, dx0, dw0, T, Bn, In, H, bidir, 0.0)  # overwrite form
+            assert_close(down(dx0, x.shape) + 1.0, outs[1], rtol=2e-4, what="dx beta 0")
+            y3, reserve3 = be.rnn_gated_forward(mode, X, W, T, Bn, In, H, bidir)
+            be.rnn_gated_backward(mode, X, y3, up(dy), W, reserve3, None, dw0, T, Bn, In, H, bidir, 1.0)  # input layer: no dx
+            assert_close(down(dw0, w.shape) * 0.5 + 1.0, outs[2], rtol=2e-4, what="dw accumulates")
+            assert np.array_equal(down(y2, dy.shape), outs[0]) and np.array_equal(down(y3, dy.shape), outs[0])
+        return outs
+
+    check_all(pair.run(f), rtol=3e-4)
+
+
+@pytest.mark.gpu
+def test_gated_rnn_rejects_bad_arguments(hip_backend):
+    be = hip_backend
+    from lantern_amd import _lib
+    mark = be.getMallocAddr()
+    x = be.mallocArray(8)
+    assert be.lib.lh_rnn_gated_reserve_floats(2, 3, 2, 4, 1) == 2 * 3 * 2 * 5 * 4 and be.lib.lh_rnn_gated_reserve_floats(3, 3, 2, 4, 0) == 3 * 2 * 4 * 4
+    assert be.lib.lh_rnn_gated_reserve_floats(1, 3, 2, 4, 0) == 0
+    with pytest.raises(LanternHipError, match="mode"):
+        be.rnn_gated_forward(1, x, x, 1, 1, 1, 1, False)
+    with pytest.raises(LanternHipError, match="shape"):
+        be.lib.lh_rnn_gated_fwd(2, x.ptr, x.ptr, x.ptr, x.ptr, 0, 1, 1, 1, 0); _lib.check()
+    be.resetMallocAddr(mark)
+
+
 @pytest.mark.parametrize("case", ["ds2", "ragged", "tiny", "long_labels", "lane_limit"])
 def test_ctc_loss_and_gradient(pair, case):
     rng = np.random.RandomState(32)

@@ -246,3 +246,49 @@ def test_resnet50_headline_step_invariants_at_full_size(hip_backend):
         tr.opt.step()           # updates the parameters and clears the gradients
         tr.end_step()
     be.sync(); be.resetMallocAddr(mark)
+
+
+class _SeqClassifier:
+    """[T, B, I] -> stacked LSTM / GRU module -> last time step's features -> Linear1D -> logSoftmax -> nll, SGD."""
+
+    def __init__(self, kind, bidirectional, numLayers):
+        from lantern_amd.nn import Module, Linear1D, LSTM, GRU, SGD
+        from lantern_amd.tensor import Tensor, int_array
+        T, B, I, H, C = 6, 4, 10, 12, 5
+        Tensor.randseed(7)
+        rng = np.random.RandomState(7)
+
+        class Net(Module):
+            def __init__(self):
+                super().__init__("seq")
+                self.rnn = self.add((LSTM if kind == "lstm" else GRU)(I, H, numLayers, bidirectional=bidirectional))
+                self.fc = self.add(Linear1D(T * H * (2 if bidirectional else 1), C, name="fc"))
+
+            def __call__(self, x):
+                return self.fc(self.rnn(x).permute(1, 0, 2).resize(B, -1))
+
+        self.model = Net()
+        # Tensor.rand(size, 0.01) of the reference leaves the gates near 0.5 / 0: scale the packed buffer up so every gate matters
+        be = la.get_backend()
+        buf = self.model.rnn.parameterBuffer
+        be.upload(buf.x.data, (rng.randn(buf.x.scalarCount) * 0.4).astype(np.float32))
+        self.opt = SGD(self.model, 0.05)
+        self.x = Tensor.fromNumpy(rng.randn(T, B, I).astype(np.float32))
+        self.target = int_array(rng.randint(0, C, size=B))
+        self.mark = be.getMallocAddr()
+
+    def step(self):
+        from lantern_amd.tensor import Tensor, TensorR, gradR_loss
+        xin = TensorR(self.x, isInput=True)
+        loss = gradR_loss(lambda dummy: self.model(xin).logSoftmaxB(1).nllLossB(self.target).sum())(Tensor.zeros(1))
+        self.opt.step()
+        return loss
+
+    def end_step(self):
+        la.get_backend().resetMallocAddr(self.mark)
+
+
+@pytest.mark.parametrize("kind,bidirectional,numLayers", [("lstm", False, 1), ("lstm", True, 2), ("gru", False, 2), ("gru", True, 1)])
+def test_lstm_gru_modules_10_steps(hip_backend, cpu_backend, kind, bidirectional, numLayers):
+    """The LSTM / GRU modes of RNNBase (NNModule.scala:324-330), stacked and bidirectional, trained for ten steps."""
+    _compare(lambda: _SeqClassifier(kind, bidirectional, numLayers), hip_backend, cpu_backend)
