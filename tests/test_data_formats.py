@@ -185,3 +185,40 @@ def test_mnist_program_from_files_matches_the_oracle_run(hip_backend, cpu_backen
     text = runs["hip"][2]
     assert text[0] == "unit: 1 epoch" and len(text) == 4 and text[3].startswith("run time: ")
     assert [float(v) for v in text[1:3]] == pytest.approx(lh, abs=1e-6)
+
+
+@pytest.mark.gpu
+def test_cifar_program_from_file_matches_the_oracle_run(hip_backend, cpu_backend, tmp_path):
+    """The CIFAR training loop of the reference's SqueezeNet program (squeezenetFromOnnx.scala:115-187) on a synthetic record
+    file: per-epoch losses on the device against the oracle's (2e-3 relative for the first epoch of ten steps), with the records decoded on the device and on
+    the host; progress lines and the result file in the reference's layout."""
+    import lantern_amd as la
+    from lantern_amd.apps.cifar_loop import train_from_file
+    from lantern_amd.apps.squeezenet import SqueezeNet
+    path, rec = _cifar_file(tmp_path, 85, 3072, seed=5)
+    runs = {}
+    for name, be, dev in (("cpu", cpu_backend, False), ("hip", hip_backend, True), ("hip_host_decode", hip_backend, False)):
+        la.set_backend(be)
+        be.dropout_seed, be.dropout_offset = 42, 0
+        mark = be.getMallocAddr()
+        lines = []
+        losses = train_from_file(SqueezeNet(10), str(tmp_path / (name + ".txt")), path, nbEpoch=2, batchSize=8, learning_rate=0.005,
+                                 out=lines.append, device_decode=dev)
+        be.resetMallocAddr(mark)
+        runs[name] = (losses, lines, (tmp_path / (name + ".txt")).read_text().splitlines())
+    lc, lh, lhh = runs["cpu"][0], runs["hip"][0], runs["hip_host_decode"][0]
+    assert len(lh) == 2 and all(np.isfinite(lh))
+    np.testing.assert_allclose(lh[0], lc[0], rtol=2e-3)          # mean over the first ten steps
+    np.testing.assert_allclose(lh[1], lc[1], rtol=1e-2)          # steps 11-20: rounding differences grown through relu / max-pool flips (2e-3 measured)
+    # two device runs do not repeat to the last bit (fp32 atomic adds in the split reductions arrive in any order, and ten SGD
+    # steps through relu / max-pool amplify that to ~3e-4 of the epoch mean, measured): the first batches must agree as printed
+    np.testing.assert_allclose(lh, lhh, rtol=1e-2)
+    first = [[float(l.split()[-1]) for l in runs[k][1] if l.startswith("Train epoch 0")][1:4] for k in ("hip", "hip_host_decode")]
+    np.testing.assert_allclose(first[0][:1], first[1][:1], rtol=1e-5)        # same input bits: the first two losses agree
+    np.testing.assert_allclose(first[0], first[1], rtol=1e-3)
+    progress = [l for l in runs["hip"][1] if l.startswith("Train epoch")]
+    assert len(progress) == 2 * 10 and progress[0].startswith("Train epoch 0: [0/85 (0%)] Average Loss: inf")   # 85 / 8 / 10 = 1: every batch reports
+    assert progress[1].startswith("Train epoch 0: [8/85 (9%)] Average Loss: ")
+    text = runs["hip"][2]
+    assert text[0] == "unit: 1 epoch" and len(text) == 4 and text[3].startswith("run time: ")
+    assert [float(v) for v in text[1:3]] == pytest.approx(lh, abs=1e-6)
