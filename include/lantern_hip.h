@@ -206,6 +206,11 @@ void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, 
 void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out);
 void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW);
 void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW);
+/* averagePool2D_batch with padding (CDN:975-982: CUDNN_POOLING_AVERAGE_COUNT_EXCLUDE_PADDING; the reference's CPU backend has
+ * no implementation, CPU:1003-1005, 1035-1037): windows over the zero-padded image, divided by the number of elements inside the
+ * image; pad < kernel.  lh_avgpool_pad_bwd adds into dx. */
+void lh_avgpool_pad_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW);
+void lh_avgpool_pad_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW);
 
 /* ---- batch norm (TD:304-310; CDN:984-1266).  Spatial: x is [N,C,HW];
  *      per-activation (batchNorm1D) is the same call with HW = 1.

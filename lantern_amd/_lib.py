@@ -85,6 +85,8 @@ SIGNATURES = {
     "lh_maxpool_bwd": (None, [P, P, P, L]),
     "lh_avgpool_fwd": (None, [P, P] + [I] * 8),
     "lh_avgpool_bwd": (None, [P, P] + [I] * 8),
+    "lh_avgpool_pad_fwd": (None, [P, P] + [I] * 10),
+    "lh_avgpool_pad_bwd": (None, [P, P] + [I] * 10),
     "lh_bn_infer": (None, [P, P, P, P, P, P, I, I, I, F]),
     "lh_bn_train_fwd": (None, [P, P, P, P, P, P, P, P, I, I, I, F, F]),
     "lh_bn_bwd": (None, [P, P, P, P, P, P, F, P, P, I, I, I]),

@@ -419,14 +419,18 @@ class BackendHIP(Backend):
             self.lib.lh_maxpool_bwd(dy.ptr, idx.ptr, xd.ptr, n_out)
         _lib.check()
 
-    def averagePool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW):
-        P, Q = conv_size(H, kH, sH), conv_size(W, kW, sW)
+    def averagePool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW, pH=0, pW=0):
+        P, Q = conv_size(H, kH, sH, pH), conv_size(W, kW, sW, pW)
         y = self.mallocArray(N * C * P * Q, zero=False)
-        self.lib.lh_avgpool_fwd(x.ptr, y.ptr, N, C, H, W, kH, kW, sH, sW); _lib.check()
+        if pH or pW: self.lib.lh_avgpool_pad_fwd(x.ptr, y.ptr, N, C, H, W, kH, kW, sH, sW, pH, pW)
+        else: self.lib.lh_avgpool_fwd(x.ptr, y.ptr, N, C, H, W, kH, kW, sH, sW)
+        _lib.check()
         return y
 
-    def averagePool2D_batch_grad(self, xd, dy, N, C, H, W, kH, kW, sH, sW):
-        self.lib.lh_avgpool_bwd(dy.ptr, xd.ptr, N, C, H, W, kH, kW, sH, sW); _lib.check()
+    def averagePool2D_batch_grad(self, xd, dy, N, C, H, W, kH, kW, sH, sW, pH=0, pW=0):
+        if pH or pW: self.lib.lh_avgpool_pad_bwd(dy.ptr, xd.ptr, N, C, H, W, kH, kW, sH, sW, pH, pW)
+        else: self.lib.lh_avgpool_bwd(dy.ptr, xd.ptr, N, C, H, W, kH, kW, sH, sW)
+        _lib.check()
 
     def batchNormInference(self, x, scale, bias, rmean, rvar, N, C, HW, eps=1e-5):
         y = self.mallocArray(N * C * HW, zero=False)

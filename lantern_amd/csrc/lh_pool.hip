@@ -221,6 +221,45 @@ __global__ void __launch_bounds__(TPB) k_avgpool_global_bwd(const float* __restr
 }
 }  // namespace
 
+// Average pooling with zero padding, the divisor counting only the elements inside the image (the reference's cuDNN backend
+// asks for CUDNN_POOLING_AVERAGE_COUNT_EXCLUDE_PADDING, TensorDslCudnn.scala:975-978).  One thread per output; the
+// backward kernel gathers, one thread per input element over the windows that cover it, so nothing needs an atomic.
+__global__ void __launch_bounds__(256) k_avgpool_pad_fwd(const float* __restrict__ x, float* __restrict__ y, int H, int W, int oH, int oW,
+                                                         int kH, int kW, int sH, int sW, int pH, int pW, int64_t n_out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, st = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n_out; i += st) {
+    const int ow = (int)(i % oW), oh = (int)((i / oW) % oH);
+    const int64_t nc = i / ((int64_t)oW * oH);
+    const int h0 = max(oh * sH - pH, 0), h1 = min(oh * sH - pH + kH, H), w0 = max(ow * sW - pW, 0), w1 = min(ow * sW - pW + kW, W);
+    const float* p = x + nc * H * W;
+    float sum = 0.f;
+    for (int h = h0; h < h1; h++) for (int w = w0; w < w1; w++) sum += p[h * W + w];
+    const int cnt = (h1 - h0) * (w1 - w0);
+    y[i] = cnt > 0 ? sum / (float)cnt : 0.f;
+  }
+}
+__global__ void __launch_bounds__(256) k_avgpool_pad_bwd(const float* __restrict__ dy, float* __restrict__ dx, int H, int W, int oH, int oW,
+                                                         int kH, int kW, int sH, int sW, int pH, int pW, int64_t n_in) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, st = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n_in; i += st) {
+    const int w = (int)(i % W), h = (int)((i / W) % H);
+    const int64_t nc = i / ((int64_t)W * H);
+    const int a0 = h + pH - kH + 1, b0 = w + pW - kW + 1;
+    const int oh0 = a0 <= 0 ? 0 : (a0 + sH - 1) / sH, oh1 = min((h + pH) / sH, oH - 1);
+    const int ow0 = b0 <= 0 ? 0 : (b0 + sW - 1) / sW, ow1 = min((w + pW) / sW, oW - 1);
+    const float* g = dy + nc * oH * oW;
+    float acc = 0.f;
+    for (int oh = oh0; oh <= oh1; oh++) {
+      const int ch = min(oh * sH - pH + kH, H) - max(oh * sH - pH, 0);
+      for (int ow = ow0; ow <= ow1; ow++) {
+        const int cw = min(ow * sW - pW + kW, W) - max(ow * sW - pW, 0);
+        acc += g[oh * oW + ow] / (float)(ch * cw);
+      }
+    }
+    dx[i] += acc;
+  }
+}
+
 extern "C" {
 
 void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad) {
@@ -298,6 +337,27 @@ void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int 
   if (n_in <= 0) return;
   if (kH == H && kW == W) hipLaunchKernelGGL(k_avgpool_global_bwd, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, dy, dx, H * W, n_in);
   else hipLaunchKernelGGL(k_avgpool_bwd, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, dy, dx, H, W, oH, oW, kH, kW, sH, sW, n_in);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_avgpool_pad_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW) {
+  ProfScope prof_(CAT_POOL);
+  LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pH >= 0 && pW >= 0 && pH < kH && pW < kW, "lh_avgpool_pad_fwd: kernel (%d,%d) stride (%d,%d) pad (%d,%d)", kH, kW, sH, sW, pH, pW);
+  LH_REQUIRE(H + 2 * pH >= kH && W + 2 * pW >= kW, "lh_avgpool_pad_fwd: image %dx%d too small for (%d,%d)", H, W, kH, kW);
+  const int oH = (H + 2 * pH - kH) / sH + 1, oW = (W + 2 * pW - kW) / sW + 1;
+  const int64_t n_out = (int64_t)N * C * oH * oW;
+  if (n_out <= 0) return;
+  hipLaunchKernelGGL(k_avgpool_pad_fwd, dim3(stream_grid(n_out, 256)), dim3(256), 0, g_stream, x, y, H, W, oH, oW, kH, kW, sH, sW, pH, pW, n_out);
+  LH_CHECK_LAUNCH();
+}
+void lh_avgpool_pad_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW) {
+  ProfScope prof_(CAT_POOL);
+  LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pH >= 0 && pW >= 0 && pH < kH && pW < kW, "lh_avgpool_pad_bwd: kernel (%d,%d) stride (%d,%d) pad (%d,%d)", kH, kW, sH, sW, pH, pW);
+  LH_REQUIRE(H + 2 * pH >= kH && W + 2 * pW >= kW, "lh_avgpool_pad_bwd: image %dx%d too small for (%d,%d)", H, W, kH, kW);
+  const int oH = (H + 2 * pH - kH) / sH + 1, oW = (W + 2 * pW - kW) / sW + 1;
+  const int64_t n_in = (int64_t)N * C * H * W;
+  if (n_in <= 0) return;
+  hipLaunchKernelGGL(k_avgpool_pad_bwd, dim3(stream_grid(n_in, 256)), dim3(256), 0, g_stream, dy, dx, H, W, oH, oW, kH, kW, sH, sW, pH, pW, n_in);
   LH_CHECK_LAUNCH();
 }
 

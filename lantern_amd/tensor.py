@@ -374,12 +374,13 @@ class Tensor:
         return Tensor(y, (N, C, conv_size(H, kernels[0], strides[0], pad), conv_size(W, kernels[1], strides[1], pad))), idx
 
     def averagePool2D_batch(self, kernels, strides, pads=None):
+        """pads = (top, bottom, left, right) as ONNX orders them; the vertical pad is pads[0] and the horizontal one pads[2]
+        (CDN:884-889), the divisor counts only elements inside the image (CDN:975-978)."""
         assert self.rank == 4
-        if pads is not None and any(p != 0 for p in pads):
-            raise NotImplementedError("averagePool2D_batch with padding (the reference's CPU backend has ??? here, CPU:1003-1005)")
+        pH, pW = _avg_pads(pads)
         N, C, H, W = self.shape
-        y = get_backend().averagePool2D_batch(self.data, N, C, H, W, kernels[0], kernels[1], strides[0], strides[1])
-        return Tensor(y, (N, C, conv_size(H, kernels[0], strides[0]), conv_size(W, kernels[1], strides[1])))
+        y = get_backend().averagePool2D_batch(self.data, N, C, H, W, kernels[0], kernels[1], strides[0], strides[1], pH, pW)
+        return Tensor(y, (N, C, conv_size(H, kernels[0], strides[0], pH), conv_size(W, kernels[1], strides[1], pW)))
 
     def _bn_view(self):
         if self.rank == 4: return self.shape[0], self.shape[1], self.shape[2] * self.shape[3]
@@ -420,6 +421,14 @@ class Tensor:
         s = Tensor(get_backend().sum_dim(self.data, n * c, h * w, 1), (n, c))
         s *= 1.0 / (h * w)
         return s
+
+
+def _avg_pads(pads):
+    if pads is None:
+        return 0, 0
+    assert len(pads) == 4, "paddings should be size 4"
+    assert pads[0] == pads[1] and pads[2] == pads[3] and min(pads) >= 0, "pads must be symmetric"
+    return int(pads[0]), int(pads[2])
 
 
 def int_array(values):
@@ -769,7 +778,8 @@ class TensorR:
         be = get_backend()
         y = TensorR._new(self.x.averagePool2D_batch(kernels, strides, pads))
         N, C, H, W = self.x.shape
-        _tape.append(lambda: be.averagePool2D_batch_grad(self.d.data, y.d.data, N, C, H, W, kernels[0], kernels[1], strides[0], strides[1]))
+        pH, pW = _avg_pads(pads)
+        _tape.append(lambda: be.averagePool2D_batch_grad(self.d.data, y.d.data, N, C, H, W, kernels[0], kernels[1], strides[0], strides[1], pH, pW))
         return y
 
     def global_ave_batch(self):

@@ -181,13 +181,15 @@ class BackendCPU(Backend):
 
     def maxPool2D_batch_grad(self, xd, dy, idx, n_out, geom=None, beta=1.0): self._c("lc_maxpool_bwd", P(dy.ptr), P(idx.ptr), P(xd.ptr), L(n_out))
 
-    def averagePool2D_batch(self, x, N, C_, H, W, kH, kW, sH, sW):
-        y = self.mallocArray(N * C_ * conv_size(H, kH, sH) * conv_size(W, kW, sW))
-        self._c("lc_avgpool_fwd", P(x.ptr), P(y.ptr), *[I(v) for v in (N, C_, H, W, kH, kW, sH, sW)])
+    def averagePool2D_batch(self, x, N, C_, H, W, kH, kW, sH, sW, pH=0, pW=0):
+        y = self.mallocArray(N * C_ * conv_size(H, kH, sH, pH) * conv_size(W, kW, sW, pW))
+        if pH or pW: self._c("lc_avgpool_pad_fwd", P(x.ptr), P(y.ptr), *[I(v) for v in (N, C_, H, W, kH, kW, sH, sW, pH, pW)])
+        else: self._c("lc_avgpool_fwd", P(x.ptr), P(y.ptr), *[I(v) for v in (N, C_, H, W, kH, kW, sH, sW)])
         return y
 
-    def averagePool2D_batch_grad(self, xd, dy, N, C_, H, W, kH, kW, sH, sW):
-        self._c("lc_avgpool_bwd", P(dy.ptr), P(xd.ptr), *[I(v) for v in (N, C_, H, W, kH, kW, sH, sW)])
+    def averagePool2D_batch_grad(self, xd, dy, N, C_, H, W, kH, kW, sH, sW, pH=0, pW=0):
+        if pH or pW: self._c("lc_avgpool_pad_bwd", P(dy.ptr), P(xd.ptr), *[I(v) for v in (N, C_, H, W, kH, kW, sH, sW, pH, pW)])
+        else: self._c("lc_avgpool_bwd", P(dy.ptr), P(xd.ptr), *[I(v) for v in (N, C_, H, W, kH, kW, sH, sW)])
 
     def batchNormInference(self, x, scale, bias, rmean, rvar, N, C_, HW, eps=1e-5):
         y = self.mallocArray(N * C_ * HW)

@@ -969,3 +969,43 @@ void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w,
   }
   free(gate); free(cell); free(hid); free(dh); free(dc); free(gx); free(gh); free(acc);
 }
+
+/* ------------------------------------------ average pooling with padding
+ * parity unpinned against the reference (CPU:1003-1005 and 1035-1037 are ???; the GPU path is cudnnPoolingForward /
+ * Backward with CUDNN_POOLING_AVERAGE_COUNT_EXCLUDE_PADDING, CDN:975-982): each output is the mean of the window's
+ * elements that lie inside the image.  The backward pass scatters from the outputs.  Checked against
+ * torch.nn.functional.avg_pool2d(count_include_pad=False) forward and autograd in the tests. */
+void lc_avgpool_pad_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW) {
+  const int oH = (H + 2 * pH - kH) / sH + 1, oW = (W + 2 * pW - kW) / sW + 1;
+  for (long nc = 0; nc < (long)N * C; nc++)
+    for (int oh = 0; oh < oH; oh++)
+      for (int ow = 0; ow < oW; ow++) {
+        float sum = 0.0f; int cnt = 0;
+        for (int r = 0; r < kH; r++)
+          for (int q = 0; q < kW; q++) {
+            const int h = oh * sH - pH + r, w = ow * sW - pW + q;
+            if (h >= 0 && h < H && w >= 0 && w < W) { sum += x[(nc * H + h) * W + w]; cnt++; }
+          }
+        y[(nc * oH + oh) * oW + ow] = cnt ? sum / (float)cnt : 0.0f;
+      }
+}
+void lc_avgpool_pad_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW) {
+  const int oH = (H + 2 * pH - kH) / sH + 1, oW = (W + 2 * pW - kW) / sW + 1;
+  for (long nc = 0; nc < (long)N * C; nc++)
+    for (int oh = 0; oh < oH; oh++)
+      for (int ow = 0; ow < oW; ow++) {
+        int cnt = 0;
+        for (int r = 0; r < kH; r++)
+          for (int q = 0; q < kW; q++) {
+            const int h = oh * sH - pH + r, w = ow * sW - pW + q;
+            if (h >= 0 && h < H && w >= 0 && w < W) cnt++;
+          }
+        if (!cnt) continue;
+        const float g = dy[(nc * oH + oh) * oW + ow] / (float)cnt;
+        for (int r = 0; r < kH; r++)
+          for (int q = 0; q < kW; q++) {
+            const int h = oh * sH - pH + r, w = ow * sW - pW + q;
+            if (h >= 0 && h < H && w >= 0 && w < W) dx[(nc * H + h) * W + w] += g;
+          }
+      }
+}

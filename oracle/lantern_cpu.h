@@ -18,7 +18,7 @@
  * Pinning status of each function (what independent evidence fixes it) is
  * listed in tests/test_oracle_golden.py; functions without a reference
  * vector are marked "parity unpinned" there and below.
- *   parity unpinned: lc_ctc_loss, lc_rnn_fwd, lc_rnn_bwd, lc_rnn_gated_fwd, lc_rnn_gated_bwd (no asserted vector and no CPU implementation in the
+ *   parity unpinned: lc_ctc_loss, lc_rnn_fwd, lc_rnn_bwd, lc_rnn_gated_fwd, lc_rnn_gated_bwd, lc_avgpool_pad_fwd, lc_avgpool_pad_bwd (no asserted vector and no CPU implementation in the
  *   reference; both are checked against torch's CPU routines in tests/test_oracle_math.py).
  */
 #ifndef LANTERN_CPU_ORACLE_H
@@ -98,6 +98,9 @@ void lc_nll_grad(float* dx, const int* target, const float* dy, int batch, int s
 void lc_maxpool_fwd(const float* x, float* y, int* idx, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad);
 void lc_maxpool_bwd(const float* dy, const int* idx, float* dx, long n_out);
 void lc_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW);
+/* padded, divisor = elements inside the image (CDN:975-982); parity unpinned against the reference, checked against torch */
+void lc_avgpool_pad_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW);
+void lc_avgpool_pad_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW);
 void lc_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW);
 
 /* batch norm: forward formula CPU:1040-1056; statistics/backward semantics CDN:1025-1131 */

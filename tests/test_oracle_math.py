@@ -287,3 +287,27 @@ def test_gated_rnn_against_torch(mode, bidir):
         for nm, size in zip(names, sizes):
             g = getattr(net, nm + ("_reverse" if d else "")).grad.numpy().ravel()
             np.testing.assert_allclose(dw[o:o + size] - 1, g, rtol=1e-4, atol=1e-5, err_msg=nm + str(d)); o += size
+
+
+@pytest.mark.parametrize("p", [(2, 3, 8, 8, 3, 3, 1, 1, 1, 1), (1, 2, 5, 9, 2, 4, 2, 3, 1, 2), (2, 2, 13, 13, 3, 3, 2, 2, 0, 1), (1, 1, 4, 4, 4, 4, 3, 3, 3, 3)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_padded_avgpool_against_torch(p):
+    """lc_avgpool_pad_fwd / _bwd (the reference's CPU backend has nothing here) against torch's avg_pool2d with
+    count_include_pad=False, values and autograd; a divisor that counts the padding fails on every border output."""
+    torch = pytest.importorskip("torch")
+    N, C, H, W, kH, kW, sH, sW, pH, pW = p
+    if pH > kH // 2 or pW > kW // 2:
+        pytest.skip("torch limits the pad to half the kernel")
+    rng = np.random.RandomState(33)
+    x = rng.randn(N, C, H, W).astype(np.float32)
+    tx = torch.tensor(x, requires_grad=True)
+    ty = torch.nn.functional.avg_pool2d(tx, (kH, kW), (sH, sW), (pH, pW), count_include_pad=False)
+    dy = rng.randn(*ty.shape).astype(np.float32)
+    ty.backward(torch.tensor(dy))
+    y = np.zeros(ty.shape, np.float32)
+    args = [I(v) for v in (N, C, H, W, kH, kW, sH, sW, pH, pW)]
+    lc.lc_avgpool_pad_fwd(cptr(x), cptr(y), *args)
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-5, atol=1e-6)
+    dx = np.ones_like(x)
+    lc.lc_avgpool_pad_bwd(cptr(dy), cptr(dx), *args)
+    np.testing.assert_allclose(dx - 1, tx.grad.numpy(), rtol=1e-5, atol=1e-6)

@@ -192,6 +192,48 @@ def test_avgpool_and_grad(pair, p):
     check_all(pair.run(f))
 
 
+def _gen_avgpad(r):
+    kH, kW = _ri(r, 1, 5), _ri(r, 1, 5)
+    pH, pW = _ri(r, 0, kH - 1), _ri(r, 0, kW - 1)
+    if pH == 0 and pW == 0: pH = kH - 1 if kH > 1 else 0; pW = 0 if pH else max(kW - 1, 0)
+    H, W = _ri(r, max(1, kH - 2 * pH), 20), _ri(r, max(1, kW - 2 * pW), 20)
+    return (_ri(r, 1, 4), _ri(r, 1, 9), H, W, kH, kW, _ri(r, 1, 3), _ri(r, 1, 3), pH, pW)
+
+
+@pytest.mark.parametrize("p", [(2, 3, 8, 8, 3, 3, 1, 1, 1, 1), (4, 16, 7, 7, 3, 3, 2, 2, 1, 1), (1, 2, 5, 9, 2, 4, 2, 3, 1, 2), (2, 2, 13, 13, 3, 3, 2, 2, 0, 1),
+                               (1, 1, 1, 1, 3, 3, 1, 1, 2, 2), (8, 64, 28, 28, 3, 3, 1, 1, 1, 1)]
+                         + [c for c in _random_cases(109, 8, _gen_avgpad) if c[8] or c[9]], ids=lambda s: "x".join(map(str, s)))
+def test_avgpool_with_padding_and_grad(pair, p):
+    """averagePool2D_batch with pads (CDN:975-982, divisor = elements inside the image): values and the accumulated input gradient."""
+    N, Cc, H, W, kH, kW, sH, sW, pH, pW = p
+    P, Q = B.conv_size(H, kH, sH, pH), B.conv_size(W, kW, sW, pW)
+    rng = np.random.RandomState(16)
+    x = rng.randn(N, Cc, H, W).astype(np.float32); dy = rng.randn(N, Cc, P, Q).astype(np.float32)
+
+    def f(be, up, down):
+        y = be.averagePool2D_batch(up(x), N, Cc, H, W, kH, kW, sH, sW, pH, pW)
+        xd = up(np.ones(x.size, np.float32))
+        be.averagePool2D_batch_grad(xd, up(dy), N, Cc, H, W, kH, kW, sH, sW, pH, pW)
+        return [down(y, dy.shape), down(xd, x.shape)]
+
+    check_all(pair.run(f))
+
+
+def test_avgpool_with_padding_through_the_tape(be):
+    """TensorR.averagePoolBK with ONNX-ordered pads: a constant image averages to itself whatever the padding, and the
+    gradient of the sum of outputs is the number-weighted coverage of each pixel (every pixel's shares add up to the
+    number of outputs when summed over the image)."""
+    from lantern_amd.tensor import Tensor, TensorR, gradR
+    x = Tensor.fromNumpy(np.full((2, 3, 6, 5), 2.5, np.float32))
+    g = gradR(lambda t: t.averagePoolBK((3, 3), (2, 2), (1, 1, 1, 1)).sum())(x)
+    y = x.averagePool2D_batch((3, 3), (2, 2), (1, 1, 1, 1))
+    assert y.shape == (2, 3, 3, 3) and np.allclose(y.toCPU(), 2.5)
+    gx = g.toCPU().reshape(2, 3, 6, 5)
+    assert np.allclose(gx.sum(axis=(2, 3)), 9.0, rtol=1e-5)
+    with pytest.raises(AssertionError):
+        x.averagePool2D_batch((3, 3), (2, 2), (1, 0, 1, 1))
+
+
 # ---- element-wise, broadcast, layout -----------------------------------------------------------------
 @pytest.mark.parametrize("n", [1, 3, 64, 1000, 64 * 256 * 56 * 56 // 16 + 5])
 def test_unary_ops_and_grads(pair, n):
