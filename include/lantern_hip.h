@@ -136,6 +136,12 @@ void lh_fill(float* x, float v, int64_t n);                                    /
 void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, int64_t inner); /* fillWithBias: CPU:39-62 */
 void lh_clip(float* x, float bound, int64_t n);                                /* clipAt: CUB:157-161 */
 void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t);      /* mask4D: CUB:710-719 */
+/* repeat0 / repeat0_grad (TD:1446-1451; CDN:378-399 with the repeat0 / shift0 kernels of API:625-650): in [rows, inner] ->
+ * out [rows - context, context + 1, inner] with out[i0, i1, :] = in[i0 + i1, :] (the Lookahead layer's sliding window).
+ * lh_repeat0_grad adds every window's gradient into ind, all rows included (the reference leaves out the last `context` rows,
+ * which its only caller fills with zero padding that has no use for a gradient). */
+void lh_repeat0(const float* in, float* out, int rows, int context, int64_t inner);
+void lh_repeat0_grad(float* ind, const float* outd, int rows, int context, int64_t inner);
 /* Cifar10DataLoader's decode (src/main/scala/lantern/TensorDataLoader.scala:109-127) on the device: n records of one label
  * byte + count pixel bytes -> x[n, count] = (float)byte / 255.0f (correctly rounded, the host loop's bits), y[n] = (int)byte.
  * records need no alignment; x and y must not overlap records. */

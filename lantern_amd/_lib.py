@@ -53,6 +53,8 @@ SIGNATURES = {
     "lh_clip": (None, [P, F, L]),
     "lh_mask4d": (None, [P, P, I, I, I, I]),
     "lh_cifar_decode": (None, [P, P, P, I, I]),
+    "lh_repeat0": (None, [P, P, I, I, L]),
+    "lh_repeat0_grad": (None, [P, P, I, I, L]),
     "lh_unary": (None, [I, P, P, L, F, F]),
     "lh_unary_grad": (None, [I, P, P, P, P, L, I, F, F]),
     "lh_scalar_op": (None, [I, P, P, F, L]),

@@ -12,7 +12,7 @@ deepspeech.pytorch model it cites normalises, and so does the default here).
 """
 import numpy as np
 
-from ..nn import Module, Conv2D, BatchNorm2D, BatchNorm1D, Linear1D, RNNBase, SGD_Momentum
+from ..nn import Module, Conv2D, BatchNorm2D, BatchNorm1D, Linear1D, RNNBase, Lookahead, SGD_Momentum
 from ..tensor import Tensor, TensorR, gradR_loss, get_backend
 
 
@@ -34,7 +34,8 @@ class BatchRNN(Module):
 
 
 class DeepSpeech(Module):
-    def __init__(self, labels="_'ABCDEFGHIJKLMNOPQRSTUVWXYZ ", rnnHiddenSize=1024, numLayers=3, freq=161, mode="tanh", rnn_batch_norm=True, seed=42):
+    def __init__(self, labels="_'ABCDEFGHIJKLMNOPQRSTUVWXYZ ", rnnHiddenSize=1024, numLayers=3, freq=161, mode="tanh", rnn_batch_norm=True, seed=42,
+                 bidirectional=True, context=20):
         super().__init__("deepspeech")
         Tensor.randseed(seed)
         rng = np.random.RandomState(seed)
@@ -46,8 +47,10 @@ class DeepSpeech(Module):
         d = (freq - 41) // 2 + 1
         d = (d - 21) // 2 + 1
         self.rnnInputSize = 32 * d
-        self.rnns = [self.add(BatchRNN(self.rnnInputSize if i == 0 else rnnHiddenSize, rnnHiddenSize, mode, True,
+        self.rnns = [self.add(BatchRNN(self.rnnInputSize if i == 0 else rnnHiddenSize, rnnHiddenSize, mode, bidirectional,
                                        useBatchNorm=rnn_batch_norm and i > 0, name="batch_rnn%d" % i)) for i in range(numLayers)]
+        # one-directional model: a look-ahead convolution over `context` future steps, then hardTanh (DeepSpeech.scala:108, 140)
+        self.lookahead = None if bidirectional else self.add(Lookahead(rnnHiddenSize, context))
         self.fc_bn = self.add(BatchNorm1D(rnnHiddenSize, "fc_bn"))
         self.fc = self.add(Linear1D(rnnHiddenSize, self.numClasses, bias=False, name="fc", rng=rng))
 
@@ -58,16 +61,20 @@ class DeepSpeech(Module):
         h = h.resize(Bn, C * Dd, T).permute(2, 0, 1)          # [T, B, C*D]
         for r in self.rnns:
             h = r(h)
+        if self.lookahead is not None:
+            h = self.lookahead(h).hardTanh(0.0, 20.0, True)
         T, Bn, Hd = h.x.shape
         out = self.fc(self.fc_bn(h.resize(T * Bn, Hd)))
         return out.resize(T, Bn, self.numClasses)
 
 
 class Trainer:
-    def __init__(self, batch=32, freq=161, frames=400, hidden=1024, layers=3, label_len=50, lr=3e-4, seed=42, rnn_batch_norm=True):
+    def __init__(self, batch=32, freq=161, frames=400, hidden=1024, layers=3, label_len=50, lr=3e-4, seed=42, rnn_batch_norm=True,
+                 bidirectional=True, context=20):
         be = get_backend()
         rng = np.random.RandomState(seed + 1)
-        self.model = DeepSpeech(rnnHiddenSize=hidden, numLayers=layers, freq=freq, rnn_batch_norm=rnn_batch_norm, seed=seed)
+        self.model = DeepSpeech(rnnHiddenSize=hidden, numLayers=layers, freq=freq, rnn_batch_norm=rnn_batch_norm, seed=seed,
+                                bidirectional=bidirectional, context=context)
         self.opt = SGD_Momentum(self.model, lr, 0.9, gradClip=400.0, nesterov=True)
         self.x = Tensor.fromNumpy(np.exp(rng.standard_normal((batch, 1, freq, frames))).astype(np.float32))
         self.labels = rng.randint(1, self.model.numClasses, size=batch * label_len).astype(np.int32)

@@ -496,6 +496,14 @@ class BackendHIP(Backend):
     def mask4D(self, x, lengths, n, c, d, t):
         self.lib.lh_mask4d(x.ptr, lengths.ptr, n, c, d, t); _lib.check()
 
+    def repeat0(self, x, rows, context, inner):
+        y = self.mallocArray((rows - context) * (context + 1) * inner, zero=False)
+        self.lib.lh_repeat0(x.ptr, y.ptr, rows, context, inner); _lib.check()
+        return y
+
+    def repeat0_grad(self, xd, yd, rows, context, inner):
+        self.lib.lh_repeat0_grad(xd.ptr, yd.ptr, rows, context, inner); _lib.check()
+
     def cifar_decode(self, records, count):
         """records: uint8 host array [n, count + 1] (label byte, then pixels).  Uploads the bytes and decodes them on the
         device; returns (x float32 [n, count], y int32 [n]) in arena memory (TensorDataLoader.scala:109-127)."""

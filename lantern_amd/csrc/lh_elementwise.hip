@@ -105,6 +105,29 @@ __global__ void k_cifar_decode(const unsigned char* __restrict__ rec, float* __r
   }
 }
 
+// repeat0 (the sliding window of the Lookahead layer): out[i0, i1, j] = in[i0 + i1, j] for i0 < rows - context, i1 <= context.
+__global__ void k_repeat0(const float* __restrict__ in, float* __restrict__ out, int c1, int64_t inner, int64_t n_out) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, st = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n_out; i += st) {
+    const int64_t j = i % inner, r = i / inner;
+    const int64_t i0 = r / c1, i1 = r - i0 * c1;
+    out[i] = in[(i0 + i1) * inner + j];
+  }
+}
+// ind[r, j] += sum over the windows that hold row r: outd[r - i1, i1, j] for 0 <= i1 <= context, 0 <= r - i1 < out_rows (a gather)
+__global__ void k_repeat0_grad(float* __restrict__ ind, const float* __restrict__ outd, int c1, int64_t out_rows, int64_t inner, int64_t n_in) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, st = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n_in; i += st) {
+    const int64_t j = i % inner, r = i / inner;
+    float acc = 0.f;
+    for (int i1 = 0; i1 < c1; i1++) {
+      const int64_t i0 = r - i1;
+      if (i0 >= 0 && i0 < out_rows) acc += outd[(i0 * c1 + i1) * inner + j];
+    }
+    ind[i] += acc;
+  }
+}
+
 extern "C" {
 
 void lh_fill(float* x, float v, int64_t n) { ProfScope prof_(CAT_FILL);
@@ -140,6 +163,19 @@ void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t) {
   int64_t tot = (int64_t)n * c * d * t;
   if (tot <= 0) return;
   hipLaunchKernelGGL(k_mask4d, dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, x, lengths, tot, c * d, t);
+  LH_CHECK_LAUNCH();
+}
+
+void lh_repeat0(const float* in, float* out, int rows, int context, int64_t inner) {
+  if (rows < 1 || context < 0 || context >= rows || inner < 1) { LH_FAIL("lh_repeat0: rows %d, context %d, inner %lld", rows, context, (long long)inner); return; }
+  const int64_t n_out = (int64_t)(rows - context) * (context + 1) * inner;
+  hipLaunchKernelGGL(k_repeat0, dim3(stream_grid(n_out, TPB * 4)), dim3(TPB), 0, g_stream, in, out, context + 1, inner, n_out);
+  LH_CHECK_LAUNCH();
+}
+void lh_repeat0_grad(float* ind, const float* outd, int rows, int context, int64_t inner) {
+  if (rows < 1 || context < 0 || context >= rows || inner < 1) { LH_FAIL("lh_repeat0_grad: rows %d, context %d, inner %lld", rows, context, (long long)inner); return; }
+  const int64_t n_in = (int64_t)rows * inner;
+  hipLaunchKernelGGL(k_repeat0_grad, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, ind, outd, context + 1, (int64_t)(rows - context), inner, n_in);
   LH_CHECK_LAUNCH();
 }
 

@@ -158,6 +158,23 @@ def GRU(inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, na
     return RNNBase("gru", inputSize, hiddenSize, numLayers, dropout, bidirectional, name)
 
 
+class Lookahead(Module):
+    """The look-ahead convolution of the one-directional DeepSpeech model (src/main/scala/lantern/PLDI19APP/DeepSpeech.scala:54-66):
+    y[t, b, f] = sum_{k <= context} x[t + k, b, f] * weight[f, k], the sequence padded with `context` zero steps.  Built from
+    concat, repeat0, permute, a broadcast product and a sum over the last axis, as the reference builds it."""
+
+    def __init__(self, numFeatures, context, name="lookahead"):
+        super().__init__(name)
+        assert context >= 1, "Context size must be at least 1"
+        self.numFeatures, self.context = numFeatures, context
+        self.weight = self.param("weight", Tensor.rand((numFeatures, context + 1), math.sqrt(context + 1)))
+
+    def __call__(self, x):
+        padding = TensorR(Tensor.zeros(self.context, *x.x.shape[1:]), isInput=True)
+        xs = x.concat(0, padding).repeat0(self.context).permute(0, 2, 3, 1)
+        return (xs * self.weight).sum(3)
+
+
 # ---- optimizers (NN:255-303) -------------------------------------------------------------------
 class Optim:
     def __init__(self, module):

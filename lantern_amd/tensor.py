@@ -410,6 +410,13 @@ class Tensor:
         res_shape = self.shape[:dim] + (sum(sizes),) + self.shape[dim + 1:]
         return Tensor(get_backend().concat([t.data for t in ts], sizes, outer, inner), res_shape)
 
+    def repeat0(self, context):
+        """TD:1446-1451 / CDN:378-386: [rows, ...] -> [rows - context, context + 1, ...], out[i0, i1] = in[i0 + i1]."""
+        assert self.rank <= 3, "only support input with no more than 3D, got %d" % self.rank
+        rows, inner = self.shape[0], _prod(self.shape[1:])
+        assert 0 <= context < rows, "context must be smaller than the first dimension"
+        return Tensor(get_backend().repeat0(self.data, rows, context, inner), (rows - context, context + 1) + tuple(self.shape[1:]))
+
     def mask4D(self, lengths):
         assert self.rank == 4
         get_backend().mask4D(self.data, lengths, *self.shape)
@@ -839,6 +846,15 @@ class TensorR:
         assert Bn <= 256, "'cudnnGetCTCLossWorkspaceSize' requires batch size less than 256, got %d" % Bn
         costs = be.ctcLoss(self.x.data, self.d.data, inputLengths, labels, labelLengths, T, Bn, A)
         return Tensor(costs, (Bn,)).mean()
+
+    def repeat0(self, context):
+        be = get_backend()
+        y = TensorR._new(self.x.repeat0(context))
+        rows, inner = self.x.shape[0], _prod(self.x.shape[1:])
+        def back():
+            if not self.isInput: be.repeat0_grad(self.d.data, y.d.data, rows, context, inner)
+        _tape.append(back)
+        return y
 
     def dropout(self, prob):
         be = get_backend()

@@ -285,6 +285,14 @@ class BackendCPU(Backend):
         self._c("lc_rnn_bwd", I(mode), P(x.ptr), P(y.ptr), P(dy.ptr), P(w.ptr), P(dx.ptr if dx is not None else 0), P(dw.ptr),
                 I(T), I(B), I(I_), I(H), I(int(bidir)))
 
+    def repeat0(self, x, rows, context, inner):
+        y = self.mallocArray((rows - context) * (context + 1) * inner)
+        self._c("lc_repeat0", P(x.ptr), P(y.ptr), I(rows), I(context), L(inner))
+        return y
+
+    def repeat0_grad(self, xd, yd, rows, context, inner):
+        self._c("lc_repeat0_grad", P(xd.ptr), P(yd.ptr), I(rows), I(context), L(inner))
+
     def rnn_gated_forward(self, mode, x, w, T, B, I_, H, bidir):
         y = self.mallocArray(T * B * H * (2 if bidir else 1))
         self._c("lc_rnn_gated_fwd", I(mode), P(x.ptr), P(w.ptr), P(y.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))

@@ -1009,3 +1009,19 @@ void lc_avgpool_pad_bwd(const float* dy, float* dx, int N, int C, int H, int W, 
           }
       }
 }
+
+/* ------------------------------------------------------------- repeat0
+ * TD:1446-1451; the reference's CPU backend has ??? (CPU:1214-1215), its GPU backend the repeat0 / shift0 kernels
+ * (API:625-650, CDN:378-399): out[i0][i1][:] = in[i0 + i1][:].  The gradient scatters every window back, all rows
+ * included.  Pinned by what the definition fixes: against numpy's sliding windows and a finite-difference-free identity
+ * (the gradient of sum(out * g) with respect to in is the scatter of g) in the tests. */
+void lc_repeat0(const float* in, float* out, int rows, int context, long inner) {
+  for (long i0 = 0; i0 < rows - context; i0++)
+    for (long i1 = 0; i1 <= context; i1++)
+      memcpy(out + (i0 * (context + 1) + i1) * inner, in + (i0 + i1) * inner, (size_t)inner * sizeof(float));
+}
+void lc_repeat0_grad(float* ind, const float* outd, int rows, int context, long inner) {
+  for (long i0 = 0; i0 < rows - context; i0++)
+    for (long i1 = 0; i1 <= context; i1++)
+      for (long j = 0; j < inner; j++) ind[(i0 + i1) * inner + j] += outd[(i0 * (context + 1) + i1) * inner + j];
+}

@@ -73,6 +73,9 @@ void lc_scalar_op(int op, const float* x, float* y, float s, long n);           
 void lc_geam(const float* x, float alpha, const float* y, float beta, float* out, long n); /* CPU:342-347 */
 void lc_trans(const float* x, float* y, int rows, int cols);                        /* CPU:349-362 */
 void lc_trans_grad(float* xd, const float* yd, int rows, int cols);                 /* CPU:364-374 */
+/* repeat0 (TD:1446-1451; CPU ??? 1214-1215; API:625-650) */
+void lc_repeat0(const float* in, float* out, int rows, int context, long inner);
+void lc_repeat0_grad(float* ind, const float* outd, int rows, int context, long inner);
 void lc_permute(const float* x, float* y, const int* dims, const int* perm, int rank);      /* math; CPU ??? 376 */
 void lc_permute_grad(float* xd, const float* yd, const int* dims, const int* perm, int rank);
 

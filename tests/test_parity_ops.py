@@ -1052,3 +1052,58 @@ def test_side_stream_contract_errors_are_reported_and_leave_the_library_usable(o
     lib.lh_side_begin(); lib.lh_fill(u, 4.0, 256); lib.lh_side_end(); _lib.check()      # in line
     assert lib.lh_side_forks() == forks and (be.toHost(B.Buf(u, 256), 256) == 4.0).all()
     lib.lh_set_side_stream(1)
+
+
+@pytest.mark.parametrize("shape,context", [((7, 3, 5), 2), ((5, 4), 4), ((9,), 1), ((30, 2, 16), 20), ((4, 1, 1), 0)], ids=str)
+def test_repeat0_and_grad(pair, shape, context):
+    """repeat0 (TD:1446-1451): values against numpy's sliding windows bit for bit, gradient against the scatter the
+    definition fixes (every window's slice added back to the rows it was cut from)."""
+    rng = np.random.RandomState(51)
+    x = rng.randn(*shape).astype(np.float32)
+    rows, inner = shape[0], int(np.prod(shape[1:]))
+    oshape = (rows - context, context + 1) + tuple(shape[1:])
+    dy = rng.randn(*oshape).astype(np.float32)
+    want_y = np.stack([x[i:i + context + 1] for i in range(rows - context)])
+    want_dx = np.ones_like(x)
+    for i0 in range(rows - context):
+        for i1 in range(context + 1):
+            want_dx[i0 + i1] += dy[i0, i1]
+
+    def f(be, up, down):
+        y = be.repeat0(up(x), rows, context, inner)
+        xd = up(np.ones(x.size, np.float32))
+        be.repeat0_grad(xd, up(dy), rows, context, inner)
+        return [down(y, oshape), down(xd, x.shape)]
+
+    outs = pair.run(f)
+    check_all(outs, exact=(0,), rtol=1e-5)
+    for o in outs:
+        assert np.array_equal(o[0], want_y)
+        np.testing.assert_allclose(o[1], want_dx, rtol=1e-5, atol=1e-6)
+
+
+def test_lookahead_module_forward_and_gradient(be):
+    """Lookahead (DeepSpeech.scala:54-66) through the tape: y[t, b, f] = sum_k x[t + k, b, f] w[f, k] with zero padding, and the
+    gradients of sum(y * g) with respect to x and w, against numpy."""
+    from lantern_amd.nn import Lookahead
+    from lantern_amd.tensor import Tensor, TensorR, _tape, _run_tape
+    rng = np.random.RandomState(52)
+    T, Bn, F, ctx = 6, 2, 5, 3
+    x = rng.randn(T, Bn, F).astype(np.float32); g = rng.randn(T, Bn, F).astype(np.float32)
+    Tensor.randseed(3)
+    la_mod = Lookahead(F, ctx)
+    w = la_mod.weight.x.toCPU().reshape(F, ctx + 1)
+    xr = TensorR(Tensor.fromNumpy(x))
+    start = len(_tape)
+    y = la_mod(xr)
+    be.upload(y.d.data, g)
+    _run_tape(start)
+    xp = np.concatenate([x, np.zeros((ctx, Bn, F), np.float32)])
+    want = sum(xp[k:k + T] * w[:, k] for k in range(ctx + 1))
+    np.testing.assert_allclose(y.x.toCPU().reshape(T, Bn, F), want, rtol=1e-5, atol=1e-6)
+    want_dx = np.zeros_like(xp)
+    for k in range(ctx + 1):
+        want_dx[k:k + T] += g * w[:, k]
+    np.testing.assert_allclose(xr.d.toCPU().reshape(T, Bn, F), want_dx[:T], rtol=1e-5, atol=1e-6)
+    want_dw = np.stack([(g * xp[k:k + T]).sum(axis=(0, 1)) for k in range(ctx + 1)], axis=1)
+    np.testing.assert_allclose(la_mod.weight.d.toCPU().reshape(F, ctx + 1), want_dw, rtol=1e-4, atol=1e-5)

@@ -141,6 +141,14 @@ def test_deepspeech2_5_steps(hip_backend, cpu_backend):
              steps=5, per_tensor=5e-3)
 
 
+def test_deepspeech2_one_directional_with_lookahead_5_steps(hip_backend, cpu_backend):
+    """The one-directional variant (DeepSpeech.scala:108, 140): forward-only RNN layers, then the look-ahead convolution over the
+    next `context` steps (concat with zero padding, repeat0, permute, broadcast product, sum) and hardTanh."""
+    from lantern_amd.apps.deepspeech2 import Trainer
+    _compare(lambda: Trainer(batch=4, freq=81, frames=120, hidden=64, layers=2, label_len=8, lr=3e-4, bidirectional=False, context=5),
+             hip_backend, cpu_backend, steps=5, per_tensor=5e-3)
+
+
 def _graph_against_eager(make_trainer, be, eager_steps, replays, tol, per_tensor):
     """Steps eager_steps .. eager_steps+replays-1 run as replays of one recorded step must give the losses and the
     parameters of the same steps run eagerly.  Between replays the program does eager work of its own on the same
