@@ -4,6 +4,7 @@
   python -m lantern_amd.microbench conv   [fwd|bwd_data|bwd_filter|all]   every distinct convolution of ResNet-50 (batch 64, 224x224), TFLOP/s
   python -m lantern_amd.microbench stream                                  batch norm, relu, add, fill, copy at ResNet-50 tensor sizes, TB/s
   python -m lantern_amd.microbench gemm                                    sgemm at a few sizes, TFLOP/s
+  python -m lantern_amd.microbench rnn_gated                               LSTM / GRU layer forward + backward at T 185, B 32, I = H = 800
   python -m lantern_amd.microbench copy   [MiB]                            one out-of-place element-wise pass over MiB of input: the
                                                                            known-size kernel the HBM byte counters are calibrated with
 
@@ -115,6 +116,30 @@ def gemm(be):
         be.resetMallocAddr(mark)
 
 
+def rnn_gated(be, T=185, B=32, I=800, H=800):
+    """LSTM / GRU layer, forward + backward, at the DeepSpeech2 layer shape (HIP events around three calls)."""
+    lib, t = be.lib, timer(be.lib)
+    rng = np.random.RandomState(0)
+    for mode, name in ((2, "lstm"), (3, "gru")):
+        for bidir in (False, True):
+            D, G = (2 if bidir else 1), (4 if mode == 2 else 3) * H
+            mark = be.getMallocAddr()
+            w = be.fromHost((rng.randn(D * (G * I + G * H + 2 * G)) * 0.03).astype(np.float32))
+            x = be.fromHost(rng.randn(T * B * I).astype(np.float32)); dy = be.fromHost(rng.randn(T * B * D * H).astype(np.float32))
+            dx = be.mallocArray(T * B * I); dw = be.mallocArray(D * (G * I + G * H + 2 * G))
+            inner = be.getMallocAddr()
+
+            def step():
+                y, r = be.rnn_gated_forward(mode, x, w, T, B, I, H, bidir)
+                be.rnn_gated_backward(mode, x, y, dy, w, r, dx, dw, T, B, I, H, bidir, 0.0)
+                be.resetMallocAddr(inner)
+
+            ms = t(step, reps=3)
+            flop = 3 * 2.0 * T * B * G * (I + H) * D
+            print("%s %s T%d B%d I%d H%d: forward + backward %.2f ms, %.1f TFLOP/s" % (name, "bidirectional" if bidir else "one direction", T, B, I, H, ms, flop / ms / 1e9), flush=True)
+            be.resetMallocAddr(mark)
+
+
 def copy(be, mib=256):
     n = int(mib) * (1 << 20) // 4
     x = be.mallocArray(n, zero=False); y = be.mallocArray(n, zero=False)
@@ -133,6 +158,7 @@ def main():
     if what == "conv": conv(be, sys.argv[2] if len(sys.argv) > 2 else "all")
     elif what == "stream": stream(be)
     elif what == "gemm": gemm(be)
+    elif what == "rnn_gated": rnn_gated(be)
     elif what == "copy": copy(be, sys.argv[2] if len(sys.argv) > 2 else 256)
     else: sys.exit(__doc__)
     be.cleanup()
