@@ -33,7 +33,6 @@ void lc_fill_with_bias(float* y, const float* bias, long outer, long c, long inn
 void lc_srand(unsigned seed) { srand(seed); }
 /* ref emits "(float)rand()/RAND_MAX" (TD:66-69) */
 static inline float ref_rand(void) { return (float)rand() / RAND_MAX; }
-void lc_randinit(float* x, long n, float scale) { for (long i = 0; i < n; i++) x[i] = (ref_rand() - 0.5f) * scale; }
 void lc_rand_uniform(float* x, long n) { for (long i = 0; i < n; i++) x[i] = (ref_rand() - 0.5f) * 1.0f; }
 
 void lc_clip(float* x, float bound, long n) {
@@ -524,14 +523,6 @@ void lc_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int 
 }
 
 /* ------------------------------------------------------------ batch norm */
-void lc_batchnorm_av(const float* x, float* out, int N, int C, int HW) { /* TD:523-538 */
-  float base = (float)N * HW * 1.0f;
-  for (int c = 0; c < C; c++) out[c] = 0.0f;
-  for (int n = 0; n < N; n++)
-    for (int c = 0; c < C; c++)
-      for (int l = 0; l < HW; l++) out[c] = out[c] + x[((size_t)n * C + c) * HW + l];
-  for (int c = 0; c < C; c++) out[c] = out[c] / base;
-}
 void lc_bn_infer(const float* x, const float* gamma, const float* beta, const float* rmean, const float* rvar,
                  float* y, int N, int C, int HW, float eps) { /* CPU:1040-1045 */
   for (int n = 0; n < N; n++)
@@ -636,14 +627,6 @@ void lc_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner) 
   for (int h = 0; h < outer; h++)
     for (int s = 0; s < dim; s++)
       for (int l = 0; l < inner; l++) dx[((size_t)h * dim + s) * inner + l] += dy[(size_t)h * inner + l];
-}
-void lc_global_ave(const float* x, float* y, int N, int C, int HW) { /* TD:880-906 */
-  float scale = 1.0f / HW;
-  for (int i = 0; i < N * C; i++) { float s = 0.0f; for (int l = 0; l < HW; l++) s += x[(size_t)i * HW + l]; y[i] = s * scale; }
-}
-void lc_global_ave_grad(float* dx, const float* dy, int N, int C, int HW) { /* TD:1454-1479 */
-  float scale = 1.0f / HW;
-  for (int i = 0; i < N * C; i++) for (int l = 0; l < HW; l++) dx[(size_t)i * HW + l] += dy[i] * scale;
 }
 
 /* ---------------------------------------------------------------- concat */

@@ -16,7 +16,8 @@
  * *_grad function accumulates (+=) into the gradient buffers.
  *
  * Pinning status of each function (what independent evidence fixes it) is
- * listed in tests/test_oracle_golden.py; functions without a reference
+ * given by tests/test_reference_vectors.py (the reference's own vectors) and
+ * tests/test_oracle_math.py (closed forms, brute force, library routines); functions without a reference
  * vector are marked "parity unpinned" there and below.
  *   parity unpinned: lc_ctc_loss, lc_rnn_fwd, lc_rnn_bwd, lc_rnn_gated_fwd, lc_rnn_gated_bwd, lc_avgpool_pad_fwd, lc_avgpool_pad_bwd (no asserted vector and no CPU implementation in the
  *   reference; both are checked against torch's CPU routines in tests/test_oracle_math.py).
@@ -39,7 +40,6 @@ int  lc_get_threads(void);
 void lc_fill(float* x, float v, long n);                                           /* CPU:26-37 */
 void lc_fill_with_bias(float* y, const float* bias, long outer, long c, long inner);/* CPU:39-62 */
 void lc_srand(unsigned seed);                                                      /* TD:66-69 */
-void lc_randinit(float* x, long n, float scale);                                   /* CPU:101-110 */
 void lc_rand_uniform(float* x, long n);                                            /* Tensor.rand: TD Random.rand */
 void lc_clip(float* x, float bound, long n);                                       /* CPU:112-119 */
 
@@ -113,7 +113,6 @@ void lc_bn_train_fwd(const float* x, const float* gamma, const float* beta, floa
                      float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor);
 void lc_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                float* dx, float* dgamma, float* dbeta, int N, int C, int HW);
-void lc_batchnorm_av(const float* x, float* out, int N, int C, int HW);                     /* TD:523-538 */
 
 /* dropout: CPU:1066-1088 (glibc rand order) and the counter-based variant the device uses */
 void lc_dropout_rand(const float* x, float* y, float* mask, long n, float p);
@@ -127,8 +126,6 @@ void lc_mean_all(const float* x, float* out, long n);
 void lc_add_scalar_from(float* dx, const float* dy1, float scale, long n);          /* sum_grad / mean_grad */
 void lc_sum_dim(const float* x, float* y, int outer, int dim, int inner);
 void lc_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner);
-void lc_global_ave(const float* x, float* y, int N, int C, int HW);                 /* TD:880-906 */
-void lc_global_ave_grad(float* dx, const float* dy, int N, int C, int HW);          /* TD:1454-1479 */
 
 /* concat along dim of n tensors: CPU:1166-1212 */
 void lc_concat(int n, const float* const* in, const int* sizes, float* out, int outer, int inner);

@@ -311,3 +311,33 @@ def test_padded_avgpool_against_torch(p):
     dx = np.ones_like(x)
     lc.lc_avgpool_pad_bwd(cptr(dy), cptr(dx), *args)
     np.testing.assert_allclose(dx - 1, tx.grad.numpy(), rtol=1e-5, atol=1e-6)
+
+
+def test_mean_clip_bias_fill_and_sgemv_literals():
+    """Literal answers for the one-liners that no reference vector reaches: mean (CPU:1115-1124: sum, then one division by the
+    count), clipAt (CPU:112-119: symmetric clamp, values inside untouched), fillWithBias (CPU:39-62: the bias runs along the middle
+    of outer x c x inner) and the matrix-vector kernel behind the dot family (both orientations, alpha and beta)."""
+    x = np.array([1, 2, 3, 6], np.float32); out = np.full(1, -7, np.float32)
+    lc.lc_mean_all(cptr(x), cptr(out), L(4))
+    assert out[0] == 3.0
+    x = np.array([0.5, -1.5, 4.0], np.float32); lc.lc_mean_all(cptr(x), cptr(out), L(3))
+    assert out[0] == 1.0                                   # not the sum (3), not divided by n-1 (1.5)
+
+    v = np.array([-2.0, 0.3, 2.0, -0.5, 0.5, -0.25], np.float32)
+    lc.lc_clip(cptr(v), F(0.5), L(6))
+    np.testing.assert_array_equal(v, np.array([-0.5, 0.3, 0.5, -0.5, 0.5, -0.25], np.float32))
+    v = np.array([3.0, -3.0, 9.0], np.float32); lc.lc_clip(cptr(v), F(1.0), L(2))          # the count bounds it
+    np.testing.assert_array_equal(v, np.array([1.0, -1.0, 9.0], np.float32))
+
+    y = np.full((2, 3, 2), -1, np.float32); bias = np.array([10, 20, 30], np.float32)
+    lc.lc_fill_with_bias(cptr(y), cptr(bias), L(2), L(3), L(2))
+    np.testing.assert_array_equal(y, np.array([[[10, 10], [20, 20], [30, 30]]] * 2, np.float32))
+    y = np.zeros((4, 3), np.float32); lc.lc_fill_with_bias(cptr(y), cptr(bias), L(4), L(3), L(1))   # the linear layers' [batch, out] case
+    np.testing.assert_array_equal(y, np.tile(bias, (4, 1)))
+
+    A = np.array([[1, 2, 3], [4, 5, 6]], np.float32); xv = np.array([1, -1, 2], np.float32); yv = np.array([100, 200], np.float32)
+    lc.lc_sgemv(I(0), I(2), I(3), F(2.0), cptr(A), I(3), cptr(xv), F(0.5), cptr(yv))      # y = 2*A x + 0.5*y
+    np.testing.assert_array_equal(yv, np.array([2 * 5 + 50, 2 * 11 + 100], np.float32))
+    tv = np.array([1, -1], np.float32); zv = np.array([1, 1, 1], np.float32)
+    lc.lc_sgemv(I(1), I(2), I(3), F(1.0), cptr(A), I(3), cptr(tv), F(1.0), cptr(zv))      # z += A^T t
+    np.testing.assert_array_equal(zv, np.array([1 - 3, 1 - 3, 1 - 3], np.float32))
