@@ -26,9 +26,8 @@
  *    Operators call no hipMalloc: convolution takes its filter-layout scratch
  *    from the top of the arena and pops it before returning (stream order
  *    keeps that safe); batch norm uses a fixed device-resident partials
- *    array.  The one exception is the multi-tensor optimizer entry points,
- *    which keep a pointer table on the device and re-allocate it when a
- *    larger model is passed.
+ *    array; the multi-tensor optimizer entry points keep their pointer
+ *    table (up to 65536 tensors) in memory that lh_setup reserved.
  */
 #ifndef LANTERN_HIP_H
 #define LANTERN_HIP_H

@@ -18,6 +18,8 @@ void quiet_other_stream();        // host-side wait for the stream that is NOT c
 extern int g_rec_pending;
 void rec_flush();
 void cmdlist_release();           // frees the command buffers (lh_cleanup)
+bool multi_tensor_setup();        // the multi-tensor optimizers' device table: reserved by lh_setup, freed by lh_cleanup
+void multi_tensor_release();
 static inline hipStream_t ordered_stream() { if (g_rec_pending) rec_flush(); return g_stream_cur; }
 #define g_stream (::lh::ordered_stream())     // every kernel is enqueued here
 extern int g_error_mode;         // 0 = print and exit, 1 = record and return

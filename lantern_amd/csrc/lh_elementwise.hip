@@ -689,35 +689,49 @@ __global__ void __launch_bounds__(TPB) k_multi_update(const MtEntry* tab, int co
     else momentum_elem(e.x[j], e.d[j], e.v[j], lr, mu, clip, nesterov);
   }
 }
-// The device-side table is cached per distinct host table (same pointers => same step plan).
-struct MtCache { MtEntry* dev = nullptr; int count = 0; int64_t chunks = 0; uint64_t key = 0; int cap = 0; };
+// The device-side table is cached per distinct host table (same pointers => same step plan).  Its memory is reserved by
+// lh_setup (MT_TABLE_MAX entries), so no operator call allocates.
+constexpr int MT_TABLE_MAX = 65536;
+struct MtCache { MtEntry* dev = nullptr; int count = 0; int64_t chunks = 0; uint64_t key = 0; };
 static MtCache g_mt;
-static void multi_update(int mode, int count, float* const* hx, float* const* hd, float* const* hv, const int64_t* hn,
-                         float lr, float mu, float clip, int nesterov) {
-  if (count <= 0) return;
+static uint64_t mt_key(int mode, int count, float* const* hx, float* const* hd, float* const* hv, const int64_t* hn) {
   uint64_t key = 1469598103934665603ULL;
   auto mix = [&key](uint64_t v) { key = (key ^ v) * 1099511628211ULL; };
   for (int t = 0; t < count; t++) { mix((uint64_t)(uintptr_t)hx[t]); mix((uint64_t)(uintptr_t)hd[t]); mix(hv ? (uint64_t)(uintptr_t)hv[t] : 0); mix((uint64_t)hn[t]); }
   mix((uint64_t)mode);
-  if (g_mt.dev == nullptr || g_mt.key != key || g_mt.count != count) {
+  return key;
+}
+static void multi_update(int mode, int count, float* const* hx, float* const* hd, float* const* hv, const int64_t* hn,
+                         float lr, float mu, float clip, int nesterov) {
+  if (count <= 0) return;
+  LH_REQUIRE(g_mt.dev != nullptr, "multi-tensor update before lh_setup");
+  LH_REQUIRE(count <= MT_TABLE_MAX, "multi-tensor update over %d tensors (at most %d)", count, MT_TABLE_MAX);
+  const uint64_t key = mt_key(mode, count, hx, hd, hv, hn);
+  if (g_mt.count == 0 || g_mt.key != key || g_mt.count != count) {
     LH_NOT_CAPTURING("the first multi-tensor update of a parameter set (its table is uploaded)");
     MtEntry* host = (MtEntry*)malloc(sizeof(MtEntry) * count);
+    LH_REQUIRE(host != nullptr, "multi-tensor table: out of host memory");
     int64_t chunks = 0;
     for (int t = 0; t < count; t++) { host[t] = {hx[t], hd[t], hv ? hv[t] : nullptr, hn[t], chunks}; chunks += cdiv(hn[t] > 0 ? hn[t] : 1, MT_CHUNK); }
-    if (g_mt.cap < count) {
-      if (g_mt.dev) (void)hipFree(g_mt.dev);
-      if (hipMalloc((void**)&g_mt.dev, sizeof(MtEntry) * count) != hipSuccess) { free(host); LH_FAIL("multi-tensor table allocation failed"); return; }
-      g_mt.cap = count;
-    }
     hipError_t e = hipMemcpyAsync(g_mt.dev, host, sizeof(MtEntry) * count, hipMemcpyHostToDevice, g_stream);
     if (e == hipSuccess) e = hipStreamSynchronize(g_stream);
     free(host);
     if (e != hipSuccess) { LH_FAIL("multi-tensor table upload: %s", hipGetErrorString(e)); return; }
     g_mt.key = key; g_mt.count = count; g_mt.chunks = chunks;
   }
+  LH_REQUIRE(g_mt.chunks > 0 && g_mt.chunks < 0x7fffffffLL, "multi-tensor update: %lld chunks", (long long)g_mt.chunks);
   hipLaunchKernelGGL(k_multi_update, dim3((unsigned)g_mt.chunks), dim3(TPB), 0, g_stream, (const MtEntry*)g_mt.dev, count, mode, lr, mu, clip, nesterov);
 }
 }  // namespace
+
+namespace lh {
+bool multi_tensor_setup() {
+  g_mt = MtCache();
+  if (hipMalloc((void**)&g_mt.dev, sizeof(MtEntry) * MT_TABLE_MAX) != hipSuccess) { g_mt.dev = nullptr; LH_FAIL("multi-tensor table allocation failed"); return false; }
+  return true;
+}
+void multi_tensor_release() { if (g_mt.dev) (void)hipFree(g_mt.dev); g_mt = MtCache(); }
+}  // namespace lh
 
 extern "C" {
 void lh_sgd(float* x, float* d, float lr, int64_t n) { ProfScope prof_(CAT_OPTIM);

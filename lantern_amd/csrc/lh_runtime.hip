@@ -122,6 +122,7 @@ void lh_setup(size_t heap_bytes) {
   LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
   g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0; g_zero_end = 0;
   LH_HIP(hipMalloc((void**)&g_advance_pool, MAX_GRAPHS * sizeof(unsigned long long)));
+  if (!multi_tensor_setup()) return;
 }
 
 static void stage_release();
@@ -132,6 +133,7 @@ void lh_cleanup(void) {
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
   cmdlist_release();
   stage_release();
+  multi_tensor_release();
   for (auto& e : g_graphs) if (e) { (void)hipGraphExecDestroy(e); e = nullptr; }
   g_graphs.clear(); g_capturing = false;
   if (g_advance_pool) (void)hipFree(g_advance_pool);
