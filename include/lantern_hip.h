@@ -332,6 +332,14 @@ void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n);
 void lh_multi_momentum(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
                        float lr, float mu, float clip, int nesterov);
 void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr);
+/* lh_multi_momentum for callers that cannot allocate or wait: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  No counterpart in the reference.  Same arguments and the same results, bit for bit.  The pointer
+ * table goes into a fixed 160 KiB device array (at most 4096 tensors per call; more is an error) and is written by kernels
+ * that carry the entries as launch arguments, so the call allocates nothing, copies nothing from the host and never waits for
+ * the device; it may be recorded into a graph.  Every call on a GPU shares that GPU's array: calls that overlap on one GPU
+ * (two host threads, two streams) race. */
+void lh_multi_momentum_static(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
+                              float lr, float mu, float clip, int nesterov);
 
 #ifdef __cplusplus
 }

@@ -119,6 +119,7 @@ SIGNATURES = {
     "lh_adagrad": (None, [P, P, P, F, F, L]),
     "lh_multi_momentum": (None, [I, P, P, P, P, F, F, F, I]),
     "lh_multi_sgd": (None, [I, P, P, P, F]),
+    "lh_multi_momentum_static": (None, [I, P, P, P, P, F, F, F, I]),
 }
 
 _lib = None

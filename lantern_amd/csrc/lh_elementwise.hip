@@ -722,13 +722,41 @@ static void multi_update(int mode, int count, float* const* hx, float* const* hd
   LH_REQUIRE(g_mt.chunks > 0 && g_mt.chunks < 0x7fffffffLL, "multi-tensor update: %lld chunks", (long long)g_mt.chunks);
   hipLaunchKernelGGL(k_multi_update, dim3((unsigned)g_mt.chunks), dim3(TPB), 0, g_stream, (const MtEntry*)g_mt.dev, count, mode, lr, mu, clip, nesterov);
 }
+// ---- the same update for callers that cannot allocate ----------------------------------------------------------
+// The table lives in a fixed device array; it is written by small kernels that receive the entries as launch
+// arguments (no host-to-device copy, so nothing waits for the device and nothing is staged).
+constexpr int MT_STATIC_MAX = 4096;                 // tensors per call
+constexpr int MT_ARGS = 64;                         // table entries one writer launch carries
+static __device__ __align__(256) unsigned char scratch[MT_STATIC_MAX * sizeof(MtEntry)];   // 160 KiB per GPU, held until the process ends
+struct MtArgs { MtEntry e[MT_ARGS]; };
+__global__ void __launch_bounds__(MT_ARGS) k_mt_table_write(MtEntry* tab, const MtArgs a, int first, int n) {
+  const int i = threadIdx.x;
+  if (i < n) tab[first + i] = a.e[i];
+}
+constexpr int MT_MAX_DEVICES = 16;
+struct MtStatic { MtEntry* ptr = nullptr; int count = 0; int64_t chunks = 0; uint64_t key = 0; };
+static MtStatic g_mt_static[MT_MAX_DEVICES];
+// The array's address on the current device (looked up once per device: every GPU holds its own copy).
+static MtStatic* mt_static_state() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MT_MAX_DEVICES) { LH_FAIL("lh_multi_momentum_static: no current device below %d", MT_MAX_DEVICES); return nullptr; }
+  MtStatic* st = &g_mt_static[dev];
+  if (st->ptr == nullptr) {
+    void* p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) { LH_FAIL("lh_multi_momentum_static: address of the table array: %s", hipGetErrorString(e)); return nullptr; }
+    st->ptr = (MtEntry*)p;
+  }
+  return st;
+}
 }  // namespace
 
 namespace lh {
 bool multi_tensor_setup() {
   g_mt = MtCache();
   if (hipMalloc((void**)&g_mt.dev, sizeof(MtEntry) * MT_TABLE_MAX) != hipSuccess) { g_mt.dev = nullptr; LH_FAIL("multi-tensor table allocation failed"); return false; }
-  return true;
+  for (auto& st : g_mt_static) st = MtStatic();       // a fresh stream after lh_setup: no table written on it yet
+  return mt_static_state() != nullptr;                // the fixed table's address on this device
 }
 void multi_tensor_release() { if (g_mt.dev) (void)hipFree(g_mt.dev); g_mt = MtCache(); }
 }  // namespace lh
@@ -761,6 +789,41 @@ void lh_multi_momentum(int count, float* const* h_x, float* const* h_d, float* c
   side_join();      // parameter gradients may still be in flight on the side stream
   multi_update(1, count, h_x, h_d, h_v, h_n, lr, mu, clip, nesterov);
   if (!failed()) LH_CHECK_LAUNCH();
+}
+void lh_multi_momentum_static(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
+                              float lr, float mu, float clip, int nesterov) { ProfScope prof_(CAT_OPTIM);
+  side_join();      // parameter gradients may still be in flight on the side stream
+  if (count <= 0) return;
+  LH_REQUIRE(count <= MT_STATIC_MAX, "lh_multi_momentum_static: %d tensors, the fixed table holds at most %d (lh_multi_momentum has no such limit)", count, MT_STATIC_MAX);
+  LH_REQUIRE(h_x && h_d && h_v && h_n, "lh_multi_momentum_static: null pointer table");
+  int64_t chunks = 0;
+  for (int t = 0; t < count; t++) {
+    LH_REQUIRE(h_n[t] >= 0 && (h_n[t] == 0 || (h_x[t] && h_d[t] && h_v[t])), "lh_multi_momentum_static: tensor %d has a null pointer or a negative size", t);
+    chunks += cdiv(h_n[t] > 0 ? h_n[t] : 1, MT_CHUNK);
+  }
+  LH_REQUIRE(chunks < 0x7fffffffLL, "lh_multi_momentum_static: %lld chunks of %d elements exceed one launch", (long long)chunks, MT_CHUNK);
+  MtStatic* st = mt_static_state();
+  if (st == nullptr) return;
+  const uint64_t key = mt_key(1, count, h_x, h_d, h_v, h_n);
+  if (st->count != count || st->key != key) {
+    // (re)write the table: entries beyond `count` left by an earlier, larger call are never read
+    st->count = 0;
+    int64_t c0 = 0;
+    for (int first = 0; first < count; first += MT_ARGS) {
+      MtArgs a;
+      const int n = count - first < MT_ARGS ? count - first : MT_ARGS;
+      for (int i = 0; i < MT_ARGS; i++) {
+        if (i < n) { const int t = first + i; a.e[i] = {h_x[t], h_d[t], h_v[t], h_n[t], c0}; c0 += cdiv(h_n[t] > 0 ? h_n[t] : 1, MT_CHUNK); }
+        else a.e[i] = {nullptr, nullptr, nullptr, 0, 0};
+      }
+      hipLaunchKernelGGL(k_mt_table_write, dim3(1), dim3(MT_ARGS), 0, g_stream, st->ptr, a, first, n);
+    }
+    LH_CHECK_LAUNCH();
+    // A graph being recorded holds these writer launches; outside it the table would be stale, so it is not remembered.
+    if (!g_capturing) { st->count = count; st->key = key; st->chunks = chunks; }
+  }
+  hipLaunchKernelGGL(k_multi_update, dim3((unsigned)chunks), dim3(TPB), 0, g_stream, (const MtEntry*)st->ptr, count, 1, lr, mu, clip, nesterov);
+  LH_CHECK_LAUNCH();
 }
 void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr) { ProfScope prof_(CAT_OPTIM);
   side_join();      // parameter gradients may still be in flight on the side stream
