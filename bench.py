@@ -71,6 +71,8 @@ def run_gpu(args):
     lib = be.lib
     if args.no_side_stream:
         lib.lh_set_side_stream(0)
+    if args.deterministic:
+        be.setDeterministic(True)
     loss_first = None
     for i in range(args.warmup):
         l = tr.step()
@@ -177,6 +179,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--tree-file", default=None, help="treelstm: trees in the reference's array_tree.txt format instead of random ones (tests/golden/array_tree_first24.txt)")
     ap.add_argument("--no-side-stream", action="store_true", help="filter gradients in line on the main stream (kernel profiles: no two kernels overlap)")
+    ap.add_argument("--deterministic", action="store_true", help="fixed-order reductions and rule-chosen launch plans (lh_set_deterministic): what run-to-run bit equality costs")
     ap.add_argument("--graph", action="store_true", help="time replays of the step recorded into a HIP graph (fixed-shape workloads)")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args()
@@ -225,7 +228,8 @@ def main():
         "config": {"workload": g["desc"], "global_batch": args.batch, "loss_first_step": round(g["loss_first"], 5) if g["loss_first"] is not None else None, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
                    "launch": "hip graph replay" if args.graph else "one launch per kernel",
                    "host_issue_ms_per_step": round(1000.0 * g["issue_sec"] / args.steps, 3) if g["issue_sec"] is not None else None,
-                   "filter_gradients": "in line" if args.no_side_stream else "side stream"},
+                   "filter_gradients": "in line" if (args.no_side_stream or args.deterministic) else "side stream",
+                   "reductions": "deterministic (two-pass, rule-chosen plans)" if args.deterministic else "atomic combine, measured plans"},
         "roofline": roof,
     }
     if args.verbose:

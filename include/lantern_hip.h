@@ -198,6 +198,20 @@ void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x,
  * switch) sends every product of at most 32 rows to the 32-row tile whatever was measured.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
  * remembered and are used again after lh_set_tuning(1)). */
 void lh_set_tuning(int on);
+/* How many launch plans have been measured so far, and how many launches have used a remembered plan (either pointer may be
+ * NULL).  While a graph is recorded nothing is measured, but remembered plans are what gets recorded. */
+void lh_tune_counters(int64_t* measured, int64_t* remembered);
+/* Deterministic mode (no counterpart in the reference, whose CPU backend accumulates in one fixed order: CPU:589-620).  By
+ * default, reductions that are cut across blocks (filter gradients, long matrix products with few tiles, stream-K tiles,
+ * convolution bias gradients, sums over a long middle axis) combine their pieces with fp32 atomic adds, so two runs on the
+ * same inputs differ in the last bits.  With lh_set_deterministic(1) (or LH_DETERMINISTIC=1 in the environment) every such
+ * reduction writes its pieces to arena scratch and a second kernel adds them in a fixed order; stream-K and all measured
+ * launch plans are off (the built-in rules decide tile shapes and slice counts, so nothing depends on a timing), and the side
+ * stream runs in line.  Two runs of the same calls on the same inputs then give the same bits.  Outside the guarantee:
+ * lh_maxpool_bwd (the scatter form: three or more overlapping windows add in any order; lh_maxpool_bwd_dense is exact)
+ * and lh_ctc_loss (fp64 sums rounded to fp32 once). */
+void lh_set_deterministic(int on);
+int lh_get_deterministic(void);
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
 void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,

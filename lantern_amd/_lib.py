@@ -35,6 +35,9 @@ SIGNATURES = {
     "lh_event_destroy": (None, [P]),
     "lh_prof_enable": (None, [C.c_uint]),
     "lh_set_tuning": (None, [I]),
+    "lh_tune_counters": (None, [P, P]),
+    "lh_set_deterministic": (None, [I]),
+    "lh_get_deterministic": (I, []),
     "lh_side_begin": (None, []),
     "lh_side_end": (None, []),
     "lh_side_join": (None, []),

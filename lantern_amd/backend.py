@@ -176,6 +176,10 @@ class BackendHIP(Backend):
     def sync(self):
         self.lib.lh_sync(); _lib.check()
 
+    def setDeterministic(self, on=True):
+        """Fixed-order reductions and rule-chosen launch plans: two runs of the same program give the same bits."""
+        self.lib.lh_set_deterministic(1 if on else 0); _lib.check()
+
     def captureBegin(self):
         """Record everything issued until captureEnd() into a HIP graph instead of running it."""
         self.lib.lh_capture_begin(); _lib.check()

@@ -632,6 +632,7 @@ void lh_bn_bwd_add_relu(const float* x, const float* out, float* dout, const flo
   LH_REQUIRE((beta_dx == 0.0f || beta_dx == 1.0f) && (beta_ds == 0.0f || beta_ds == 1.0f), "lh_bn_bwd_add_relu: beta must be 0 or 1");
   LH_REQUIRE(x && out && dout && gamma && save_mean && save_invstd, "lh_bn_bwd_add_relu: null operand");
   LH_REQUIRE(ds != dout && dx != dout, "lh_bn_bwd_add_relu: dout may not alias a gradient output");
+  LH_REQUIRE(dx == nullptr || dx != ds, "lh_bn_bwd_add_relu: dx and ds are the same buffer (a batch norm whose input is also the shortcut): the first pass would add into what the second overwrites; run lh_add_relu_grad and lh_bn_bwd instead");
   if (!get_partial()) return;
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dx | (uintptr_t)ds) & 15) == 0);
   dim3 grid(C, p.slices);

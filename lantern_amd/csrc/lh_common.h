@@ -26,7 +26,19 @@ extern int g_error_mode;         // 0 = print and exit, 1 = record and return
 extern int g_num_cu;             // compute units of the device in use
 extern bool g_tune_enabled;      // launch plans are measured on first use (lh_set_tuning; off with LH_NO_TUNE in the environment)
 extern bool g_capturing;         // between lh_capture_begin and lh_capture_end: work is recorded into a HIP graph, nothing may wait on the stream
-#define g_tune (::lh::g_tune_enabled && !::lh::g_capturing)
+// Deterministic mode (lh_set_deterministic): no result depends on the order in which blocks finish or on a measured launch
+// plan.  Reductions that are cut across blocks write their partial sums to scratch memory and a second kernel adds them in a
+// fixed order (instead of fp32 atomic adds); stream-K and every measured plan are off (the built-in rules decide), and the
+// side stream runs in line.
+extern bool g_deterministic;
+// A remembered launch plan may be used / a plan may be measured now.  While a graph is recorded nothing can be timed, but
+// what was measured before is still what gets launched.
+extern int64_t g_plans_measured, g_plans_remembered;     // launch plans timed so far / launches that used a remembered plan (lh_tune_counters)
+#define g_tune_lookup (::lh::g_tune_enabled && !::lh::g_deterministic)
+#define g_tune_measure (g_tune_lookup && !::lh::g_capturing)
+// C[m,n] (row stride ldc) = beta*C + partial[0] + partial[1] + ... + partial[slices-1], each partial a dense [m,n] block,
+// added in that order by one thread per element.
+void reduce_slices(float* C, int ldc, int m, int n, const float* partial, int slices, float beta);
 extern double g_tune_min_flop;   // products below this many flop keep the built-in launch rule (a timing run costs more than it can win)
 // Dropout draws from a counter-based stream whose position the caller passes per launch.  A replayed graph repeats its
 // launch arguments, so a captured dropout adds *g_capture_advance (device memory; 0 for the first replay, advanced at the

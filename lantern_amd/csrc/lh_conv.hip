@@ -220,6 +220,7 @@ struct LoadConvBwdFilterB {
 //      Wc columns; the element lands at out[n][i][aH + eH*u][aW + eW*v] of an image W wide with PIX pixels.
 struct EpiConvOut {
   static constexpr bool STATS = false;
+  static constexpr bool SLICED = false;
   float* out; const float* bias; int chan, PIX, W, eH, eW, aH, aW; float beta;
   int zfill2 = 0;           // the grid is every second pixel of every second row of an image with even sides (a 1x1 filter, stride 2):
                             // the element is stored together with the three zeros of its 2x2 cell, so the output needs no clearing
@@ -371,7 +372,7 @@ static bool launch_plan(int plan, const AL& al, const BL& bl, const EP& ep, int 
   const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
   const int64_t slabs = cdiv(K, CONV_BK);
   // long reductions only: a worker's share must span many slabs for the per-segment set-up to pay off
-  if (few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)workers && (ep.beta == 1.f || zero_out != nullptr || prezeroed)) {
+  if (!g_deterministic && few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)workers && (ep.beta == 1.f || zero_out != nullptr || prezeroed)) {
     if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
     if (M > 64) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
     return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
@@ -394,15 +395,16 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
   static std::map<PlanKey, int> chosen;
   const bool can_zero = zero_out != nullptr || prezeroed;
   if (M <= 32 && force_m32()) return launch_plan(10, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
-  if (!g_tune || 2.0 * M * N * (double)K < g_tune_min_flop) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  if (!g_tune_lookup || 2.0 * M * N * (double)K < g_tune_min_flop) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   const PlanKey key = {{M, N, K, ep.eH, ep.eW, ep.W, ep.PIX}};
   auto it = chosen.find(key);
   if (it != chosen.end()) {
+    g_plans_remembered++;
     const int plan = plan_valid<AL, BL, EP>(it->second, ep, M, K, can_zero) ? it->second : 0;
     return launch_plan(plan, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   }
   // tuned only on a call that may be repeated: an overwriting epilogue onto an output this launch alone writes
-  if (ep.beta != 0.f || prezeroed) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  if (!g_tune_measure || ep.beta != 0.f || prezeroed) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   LaunchTimer timer;
   if (!timer.ok) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   int best = 0; float best_ms = 3.0e38f, base_ms = 0.f;
@@ -413,7 +415,7 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
     if (plan == 0) base_ms = ms;
     if (ms < best_ms * 0.98f) { best_ms = ms; best = plan; }      // a later plan must win by 2 % to displace an earlier one
   }
-  chosen[key] = best;
+  chosen[key] = best; g_plans_measured++;
   if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv product M%d N%d K%d (stride %d,%d): plan %d, %.3f ms (built-in rule %.3f ms)\n", M, N, K, ep.eH, ep.eW, best, best_ms, base_ms);
   return true;                                               // the timed launches have produced the result
 }
@@ -428,7 +430,7 @@ static bool plan_tiles_stats(int M, int N, int K, StatLayout& L, int& bm, int& b
   const int64_t t128 = cdiv(M, 128) * cdiv(N, 128), t64 = cdiv(M, 64) * cdiv(N, 128);
   const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
   const int64_t slabs = cdiv(K, CONV_BK);
-  if (few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)(2 * g_num_cu)) return false;
+  if (!g_deterministic && few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)(2 * g_num_cu)) return false;
   TilePick tp = pick_tile_conv(M, N, K);
   if (force == 1 && M > 64) tp = {128, 128}; else if (force == 2) tp = {64, 128}; else if (force == 3) tp = {64, 64};
   bm = tp.bm; bn = tp.bn;
@@ -497,7 +499,7 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
       // repeating it is harmless) and remembered
       static std::map<PlanKey, int> chosen;
       const PlanKey key = {{K, N * PQ, CRS, H, W, sH, R}};
-      const bool tunable = g_tune && 2.0 * K * CRS * (double)N * PQ >= g_tune_min_flop;
+      const bool tunable = g_tune_lookup && 2.0 * K * CRS * (double)N * PQ >= g_tune_min_flop;
       int force = 0;
       auto run = [&](int f) {           // 0: the rule's tile, 1-3: a forced tile, 4: unfused (any launch plan, then a pass over y)
         if (f == 4) {
@@ -518,8 +520,8 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
       };
       if (tunable) {
         auto it = chosen.find(key);
-        if (it != chosen.end()) force = it->second;
-        else {
+        if (it != chosen.end()) { force = it->second; g_plans_remembered++; }
+        else if (g_tune_measure) {
           LaunchTimer timer;
           if (timer.ok) {
             float best_ms = 3.0e38f, base_ms = 0.f; int best = 0;
@@ -530,7 +532,7 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
               if (f == 0) base_ms = ms;
               if (ms < best_ms * 0.98f) { best_ms = ms; best = f; }
             }
-            chosen[key] = best; force = best;
+            chosen[key] = best; force = best; g_plans_measured++;
             if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv fwd+stats K%d N%d CRS%d H%d: tile plan %d, %.3f ms (built-in rule %.3f ms)\n", K, N * PQ, CRS, H, best, best_ms, base_ms);
           }
         }
@@ -682,8 +684,8 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
         int tile = tp.bm == 128 ? 1 : (tp.bn == 128 ? 2 : 3);
         auto it = chosen.find(key);
         if (C <= 32 && force_m32()) tile = 4;
-        else if (it != chosen.end()) tile = it->second;
-        else if (g_tune && beta == 0.f && 2.0 * C * (double)ntot * kmax >= g_tune_min_flop) {
+        else if (it != chosen.end() && g_tune_lookup) { tile = it->second; g_plans_remembered++; }
+        else if (it == chosen.end() && g_tune_measure && beta == 0.f && 2.0 * C * (double)ntot * kmax >= g_tune_min_flop) {
           LaunchTimer timer;
           if (timer.ok) {
             float best_ms = 3.0e38f; int best = tile;
@@ -694,7 +696,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
               if (ms < 0.f || failed()) { lh_free_top(bytes); return; }
               if (ms < best_ms * 0.98f) { best_ms = ms; best = tcand; }
             }
-            chosen[key] = best; tile = best;
+            chosen[key] = best; tile = best; g_plans_measured++;
             if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "conv input gradient, stride (%d,%d), C%d H%d K%d k%d: %d classes in one launch, tile plan %d, %.3f ms\n", sH, sW, C, H, K, R, ng, best, best_ms);
           }
         }
@@ -784,16 +786,30 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   // How many slices pays best depends on how tiles x slices fall onto the resident block slots and on how short the
   // per-block reduction gets; it is measured once per shape (a few candidates on a scratch output) and remembered.
   const BwdfKey key = {{N, C, H, W, K, R, S, sH, sW, pH, pW}};
-  const bool tunable = g_tune && max_split > 1 && 2.0 * K * CRS * (double)red >= g_tune_min_flop;
+  const bool tunable = g_tune_lookup && max_split > 1 && 2.0 * K * CRS * (double)red >= g_tune_min_flop;
   bool tune_now = false;
   if (tunable) {
     auto it = g_bwdf_split.find(key);
-    if (it != g_bwdf_split.end()) { tp = TilePick{it->second.bm, it->second.bn}; tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn); split = clamp_split(it->second.split); }
-    else tune_now = true;
+    if (it != g_bwdf_split.end()) { g_plans_remembered++; tp = TilePick{it->second.bm, it->second.bn}; tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn); split = clamp_split(it->second.split); }
+    else tune_now = g_tune_measure;
   }
   if (K <= 32 && force_m32()) { tp = TilePick{32, 128}; tiles = cdiv(K, 32) * cdiv(CRS, 128); split = clamp_split(cdiv(3 * (int64_t)g_num_cu, tiles)); tune_now = false; }
-  if (beta == 0.f) lh_fill(dw, 0.f, (int64_t)K * CRS);
+  // Deterministic mode: every slice of the reduction writes its own [K, CRS] block of scratch memory (no atomics), and a
+  // second kernel adds the blocks onto beta*dw in slice order.
+  float* partial = nullptr; size_t partial_bytes = 0; int slices = 1;
+  if (g_deterministic && split > 1) {
+    const int bk = tp.bm == 128 ? 16 : (tp.bm == 32 ? 32 : BWDF_BK);
+    int64_t kper = cdiv(cdiv(red, split), bk) * bk; if (kper < bk) kper = bk;
+    slices = (int)cdiv(red, kper);                                    // what igemm_launch will make of `split`
+    if (slices > 1) {
+      partial_bytes = (size_t)slices * K * CRS * sizeof(float);
+      partial = (float*)lh_malloc_uninit(partial_bytes);
+      if (partial == nullptr) return;
+    }
+  }
+  if (beta == 0.f && partial == nullptr) lh_fill(dw, 0.f, (int64_t)K * CRS);
   EpiRowMajor ep; ep.C = dw; ep.ldc = CRS; ep.alpha = 1.f; ep.beta = 1.f; ep.atomic = split > 1 ? 1 : 0;
+  if (partial) { ep.C = partial; ep.sliceStride = (long long)K * CRS; ep.beta = 0.f; }
   bool ok = false;
   auto go = [&](auto al, auto bl) {
     al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
@@ -817,7 +833,7 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   const bool xvec = (PQ % 4 == 0) && (((uintptr_t)x & 15) == 0);
   const bool narrow = PQ < 4 || d.Q < 4;        // the stepping loaders assume at most one carry inside a group of four
   auto dispatch = [&]() {
-    ep.atomic = split > 1 ? 1 : 0;
+    ep.atomic = (split > 1 && ep.sliceStride == 0) ? 1 : 0;
     if (plain && avec && xvec) go_plain(LoadConvBwdFilterA<true>(), LoadConvBwdFilterA<true>());
     else if (plain && !avec && !xvec && !narrow) go_plain(LoadConvBwdFilterA<false, true>(), LoadConvBwdFilterA<false, true>());
     else if (plain && !avec && !xvec) go_plain(LoadConvBwdFilterA<false>(), LoadConvBwdFilterA<false>());
@@ -855,19 +871,23 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
       tp = TilePick{best.bm, best.bn};
       tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
       split = best.split;
-      g_bwdf_split[key] = best;
+      g_bwdf_split[key] = best; g_plans_measured++;
       if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: tile %dx%d, %lld tiles, split %d (%.3f ms)\n", N, C, H, K, R, sH, tp.bm, tp.bn, (long long)tiles, split, best_ms);
     }
     if (scratch) lh_free_top(sbytes);
     if (failed()) return;
   }
   dispatch();
+  if (partial) {
+    if (ok) reduce_slices(dw, CRS, K, CRS, partial, slices, beta);
+    lh_free_top(partial_bytes);
+  }
   if (!ok) return;
   if (db) {
-    int slices = (int)cdiv(2 * (int64_t)g_num_cu, K);
-    if (slices > N) slices = N;
-    if (slices < 1) slices = 1;
-    const int n_per = (int)cdiv(N, slices);
+    int bslices = g_deterministic ? 1 : (int)cdiv(2 * (int64_t)g_num_cu, K);     // slices of the batch add atomically: one slice when the order must be fixed
+    if (bslices > N) bslices = N;
+    if (bslices < 1) bslices = 1;
+    const int n_per = (int)cdiv(N, bslices);
     hipLaunchKernelGGL(k_conv_bwd_bias, dim3(K, (unsigned)cdiv(N, n_per)), dim3(TPB), 0, g_stream, dy, db, N, K, PQ, n_per);
   }
   LH_CHECK_LAUNCH();

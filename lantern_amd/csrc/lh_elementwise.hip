@@ -29,7 +29,7 @@ static inline bool al16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 // ---- generic vectorised elementwise driver: out[i] = f(a[i], b[i], c[i]) --------------
 template <int NIN, class F>
-__global__ void __launch_bounds__(TPB) k_ew_vec(float* __restrict__ out, const float* a, const float* b, const float* c, int64_t n, F f) {
+__global__ void __launch_bounds__(TPB) k_ew_vec(float* out /* may be one of the inputs (in-place forms): no restrict */, const float* a, const float* b, const float* c, int64_t n, F f) {
   int64_t n4 = n >> 2;
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
   for (int64_t j = i; j < n4; j += st) {

@@ -152,12 +152,30 @@ __global__ void __launch_bounds__(TPB) k_scale_rows(float* C, int ldc, int m, in
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
   for (; i < tot; i += st) { const int r = (int)(i / n), c = (int)(i - (int64_t)r * n); float* p = C + (int64_t)r * ldc + c; *p = beta == 0.f ? 0.f : beta * *p; }
 }
+// C = beta*C + sum of the slices' partial products, in slice order (the deterministic stand-in for atomic adds)
+__global__ void __launch_bounds__(TPB) k_reduce_slices(float* C, int ldc, int m, int n, const float* __restrict__ partial, int slices, float beta) {
+  const int64_t tot = (int64_t)m * n;
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+  for (; i < tot; i += st) {
+    const int r = (int)(i / n), c = (int)(i - (int64_t)r * n);
+    float* p = C + (int64_t)r * ldc + c;
+    float acc = beta == 0.f ? 0.f : beta * *p;
+    for (int s = 0; s < slices; s++) acc += partial[(int64_t)s * tot + i];
+    *p = acc;
+  }
+}
 template <class AL, class BL>
 static bool sgemm_mfma(const AL& al, const BL& bl, const EpiRowMajor& ep, int m, int n, int k, const SgemmPlan& pl) {
   if (pl.tp.bm == 128) return igemm_launch<128, 128, 16>(al, bl, ep, m, n, k, pl.split);
   if (pl.tp.bn == 128) return igemm_launch<64, 128, 16>(al, bl, ep, m, n, k, pl.split);
   return igemm_launch<64, 64, 16>(al, bl, ep, m, n, k, pl.split);
 }
+
+namespace lh {
+void reduce_slices(float* C, int ldc, int m, int n, const float* partial, int slices, float beta) {
+  hipLaunchKernelGGL(k_reduce_slices, dim3(stream_grid((int64_t)m * n, TPB * 2)), dim3(TPB), 0, g_stream, C, ldc, m, n, partial, slices, beta);
+}
+}  // namespace lh
 
 void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, int lda,
               const float* B, int ldb, float beta, float* C, int ldc) {
@@ -180,24 +198,38 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
     // one product under plan `pl` into Cout (row stride ldo) with the given beta
     auto run = [&](const SgemmPlan& pl, float* Cout, int ldo, float be) -> bool {
       EpiRowMajor e; e.C = Cout; e.ldc = ldo; e.alpha = alpha; e.beta = be; e.atomic = 0;
-      if (pl.split > 1) {
+      float* partial = nullptr; size_t pbytes = 0; int slices = 1;
+      if (pl.split > 1 && g_deterministic) {            // slices into scratch blocks, added in order afterwards
+        int64_t kper = cdiv(cdiv(k, pl.split), 16) * 16; if (kper < 16) kper = 16;
+        slices = (int)cdiv(k, kper);
+        pbytes = (size_t)slices * m * n * sizeof(float);
+        partial = (float*)lh_malloc_uninit(pbytes);
+        if (partial == nullptr) return false;
+        e.C = partial; e.ldc = n; e.beta = 0.f; e.sliceStride = (long long)m * n;
+      } else if (pl.split > 1) {
         if (be != 1.f) { hipLaunchKernelGGL(k_scale_rows, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, Cout, ldo, m, n, be); }
         e.atomic = 1; e.beta = 1.f;
       }
-      if (!ta && !tb) return av ? sgemm_mfma(akv, bt, e, m, n, k, pl) : sgemm_mfma(aks, bt, e, m, n, k, pl);
-      if (!ta && tb) return av ? (bv ? sgemm_mfma(akv, bkv, e, m, n, k, pl) : sgemm_mfma(akv, bks, e, m, n, k, pl))
-                               : (bv ? sgemm_mfma(aks, bkv, e, m, n, k, pl) : sgemm_mfma(aks, bks, e, m, n, k, pl));
-      if (ta && !tb) return sgemm_mfma(at, bt, e, m, n, k, pl);
-      return bv ? sgemm_mfma(at, bkv, e, m, n, k, pl) : sgemm_mfma(at, bks, e, m, n, k, pl);
+      bool good;
+      if (!ta && !tb) good = av ? sgemm_mfma(akv, bt, e, m, n, k, pl) : sgemm_mfma(aks, bt, e, m, n, k, pl);
+      else if (!ta && tb) good = av ? (bv ? sgemm_mfma(akv, bkv, e, m, n, k, pl) : sgemm_mfma(akv, bks, e, m, n, k, pl))
+                                    : (bv ? sgemm_mfma(aks, bkv, e, m, n, k, pl) : sgemm_mfma(aks, bks, e, m, n, k, pl));
+      else if (ta && !tb) good = sgemm_mfma(at, bt, e, m, n, k, pl);
+      else good = bv ? sgemm_mfma(at, bkv, e, m, n, k, pl) : sgemm_mfma(at, bks, e, m, n, k, pl);
+      if (partial) {
+        if (good) reduce_slices(Cout, ldo, m, n, partial, slices, be);
+        lh_free_top(pbytes);
+      }
+      return good;
     };
     SgemmPlan pl = sgemm_plan(m, n, k);
     // Tile shape and reduction slices are measured once per (transposes, m, n, k) on a scratch output and remembered.
     static std::map<std::array<int, 7>, SgemmPlan> chosen;
-    if (g_tune && 2.0 * m * n * (double)k >= g_tune_min_flop) {
+    if (g_tune_lookup && 2.0 * m * n * (double)k >= g_tune_min_flop) {
       const std::array<int, 7> key = {ta, tb, m, n, k, (int)av, (int)bv};
       auto it = chosen.find(key);
-      if (it != chosen.end()) pl = it->second;
-      else {
+      if (it != chosen.end()) { pl = it->second; g_plans_remembered++; }
+      else if (g_tune_measure) {
         const size_t sbytes = (size_t)m * n * sizeof(float);
         float* scratch = (float*)lh_malloc_uninit(sbytes);
         LaunchTimer timer;
@@ -224,7 +256,7 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
               if (ms < best_ms * 0.98f) { best_ms = ms; best = c; }
             }
           }
-          if (best_ms >= 0.f && !failed()) { chosen[key] = best; pl = best; }
+          if (best_ms >= 0.f && !failed()) { chosen[key] = best; pl = best; g_plans_measured++; }
           if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "sgemm ta%d tb%d %dx%dx%d: tile %dx%d, %d slice(s), %.3f ms\n", ta, tb, m, n, k, best.tp.bm, best.tp.bn, best.split, best_ms);
         }
         if (scratch) lh_free_top(sbytes);
@@ -241,7 +273,7 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   // A few tiles over a long reduction (a classifier with ten outputs behind 2048 features: one block walking 32 slabs took
   // 194 us): the reduction is cut into slices of at least 128 that add into beta*C.
   int kper = k;
-  if (k >= 512 && (int64_t)grid.x * grid.y <= 64) {
+  if (k >= 512 && (int64_t)grid.x * grid.y <= 64 && !g_deterministic) {
     int slices = k / 128; if (slices > 32) slices = 32;
     kper = (int)cdiv(cdiv(k, slices), SMALL_KS) * SMALL_KS;
     grid.z = (unsigned)cdiv(k, kper);

@@ -16,6 +16,7 @@
 // 8 XCDs (own L2 each) works on a contiguous range of tiles, M-tiles of one N-column first.
 #pragma once
 #include "lh_common.h"
+#include <type_traits>
 
 namespace lh {
 
@@ -115,7 +116,10 @@ __device__ __forceinline__ float4 lh_fetch4(__amdgpu_buffer_rsrc_t rsrc, const L
 // mode 0: C = alpha*acc + beta*C ; mode 1: atomicAdd(C, alpha*acc) (split-K)
 struct EpiRowMajor {
   static constexpr bool STATS = false;
+  static constexpr bool SLICED = true;
   float* C; int ldc; float alpha, beta; int atomic;
+  long long sliceStride = 0;       // != 0: slice sp of a cut reduction writes its own block C + sp*sliceStride (no atomics; added up afterwards)
+  __device__ __forceinline__ void slice(int sp) { C += (long long)sp * sliceStride; }
   struct Col { int j; bool valid; };
   __device__ __forceinline__ Col col(int j, int N) const { Col c; c.j = j; c.valid = j < N; return c; }
   // part: 0 = the whole reduction of this element is in v; 1 = first partial sum, 2 = a later one
@@ -142,7 +146,8 @@ __device__ __forceinline__ float lh_half_sum32(float v) {
 // ---- the kernel ------------------------------------------------------------------------------------
 // The work of one block; `block` is its index within the launch (or within its group of a grouped launch).
 template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
-__device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP& ep, const GemmShape& gs, const int block) {
+__device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP& ep_in, const GemmShape& gs, const int block) {
+  typename std::conditional<EP::SLICED, EP, const EP&>::type ep = ep_in;      // a sliced epilogue is a private copy that slice() moves
   constexpr int KQ = BK / 4, PAD = 8 / KQ, LDA = BM + PAD, LDB = BN + PAD;
   // The four wavefronts form a 2 x 2 grid over the tile, or, for a 32-row tile (products with at most 32 rows: layers with
   // few channels), a 1 x 4 grid, so that no matrix instruction is spent on rows beyond the 32.
@@ -195,6 +200,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
     tn = rest % gs.tilesN;
     const int sp = rest / gs.tilesN;
     kbeg = sp * gs.kPerSplit; kend = min(gs.K, kbeg + gs.kPerSplit);
+    if constexpr (EP::SLICED) ep.slice(sp);
     u = u_end;
   }
   const int m0 = tm * BM, n0 = gs.colBase + tn * BN;

@@ -187,7 +187,7 @@ void lh_add_scalar_from(float* dx, const float* dy1, float scale, int64_t n) { P
 void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner) { ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * inner <= 0) return;
   if (inner == 1) hipLaunchKernelGGL(k_sum_rows, dim3(stream_grid((int64_t)outer * 64, TPB)), dim3(TPB), 0, g_stream, x, y, outer, dim);
-  else if ((int64_t)outer * inner < 64 * (int64_t)g_num_cu && dim >= 512 && outer <= 65535) {
+  else if (!g_deterministic && (int64_t)outer * inner < 64 * (int64_t)g_num_cu && dim >= 512 && outer <= 65535) {      // slices add atomically
     const int64_t base = (int64_t)outer * cdiv(inner, 64);
     int slices = (int)cdiv(4 * (int64_t)g_num_cu, base);
     if (slices > dim / 64) slices = dim / 64;

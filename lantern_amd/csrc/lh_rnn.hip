@@ -424,6 +424,7 @@ void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
 void lh_ctc_loss(const float* probs, float* dprobs, const int* h_labels, const int* h_label_len, const int* h_input_len,
                  float* costs, int T, int B, int A) {
   ProfScope prof_(CAT_REDUCE);
+  LH_NOT_CAPTURING("lh_ctc_loss (it uploads its label and length arrays)");
   LH_REQUIRE(T >= 1 && B >= 1 && A >= 2, "lh_ctc_loss: bad shape T%d B%d A%d", T, B, A);
   LH_REQUIRE(probs && costs && h_labels && h_label_len && h_input_len, "lh_ctc_loss: null operand");
   int total = 0, Lmax = 0;
@@ -446,8 +447,9 @@ void lh_ctc_loss(const float* probs, float* dprobs, const int* h_labels, const i
   if (scratch == nullptr) { free(host); return; }
   int* d_int = (int*)scratch;
   lh_h2d(d_int, host, sizeof(int) * (size_t)(3 * B));
-  if (total > 0) lh_h2d(d_int + 3 * B, h_labels, sizeof(int) * (size_t)total);
+  if (total > 0 && !failed()) lh_h2d(d_int + 3 * B, h_labels, sizeof(int) * (size_t)total);
   free(host);
+  if (failed()) { lh_free_top(int_bytes + dbl); return; }       // nothing is launched on lengths and labels that were not uploaded
   double* alpha = (double*)(scratch + int_bytes); double* beta = alpha + (size_t)B * T * row; double* cn = beta + (size_t)B * T * row;
   if (one_wave) hipLaunchKernelGGL(k_ctc_wave, dim3(B), dim3(128), 2 * (size_t)A * sizeof(double), g_stream, probs, dprobs, d_int + 3 * B, d_int, d_int + B, d_int + 2 * B, costs, alpha, beta, T, B, A);
   else hipLaunchKernelGGL(k_ctc, dim3(B), dim3(CTC_TPB), 0, g_stream, probs, dprobs, d_int + 3 * B, d_int, d_int + B, d_int + 2 * B, costs, alpha, beta, cn, T, B, A, Smax);

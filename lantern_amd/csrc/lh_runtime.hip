@@ -31,6 +31,8 @@ void side_join() {
 }
 bool g_tune_enabled = getenv("LH_NO_TUNE") == nullptr;
 bool g_capturing = false;
+int64_t g_plans_measured = 0, g_plans_remembered = 0;
+bool g_deterministic = getenv("LH_DETERMINISTIC") != nullptr;
 double g_tune_min_flop = getenv("LH_TUNE_MIN_FLOP") ? atof(getenv("LH_TUNE_MIN_FLOP")) : 1e7;
 unsigned long long* g_capture_advance = nullptr;
 unsigned long long g_capture_drawn = 0;
@@ -103,6 +105,9 @@ extern "C" {
 
 void lh_set_error_mode(int mode) { g_error_mode = mode; }
 void lh_set_tuning(int on) { g_tune_enabled = on != 0; }
+void lh_tune_counters(int64_t* measured, int64_t* remembered) { if (measured) *measured = g_plans_measured; if (remembered) *remembered = g_plans_remembered; }
+void lh_set_deterministic(int on) { side_join(); g_deterministic = on != 0; }
+int lh_get_deterministic(void) { return g_deterministic ? 1 : 0; }
 const char* lh_last_error(void) { return g_err; }
 void lh_clear_error(void) { g_err[0] = 0; }
 
@@ -251,7 +256,7 @@ void lh_side_begin(void) {
   LH_REQUIRE(g_stream_raw != nullptr, "lh_side_begin before lh_setup");
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_side_begin: already on the side stream");
   // In line (no concurrency) when switched off, while kernels are timed one by one, or while the stream is recorded.
-  if (!g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on) return;
+  if (!g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on || g_deterministic) return;
   hipEvent_t ev = side_event();
   LH_HIP(hipEventRecord(ev, g_stream));              // (flushes recorded commands first)
   LH_HIP(hipStreamWaitEvent(g_side_stream, ev, 0));
@@ -274,11 +279,13 @@ void lh_capture_begin(void) {
   LH_CHECK_LAUNCH();
   LH_HIP(hipStreamBeginCapture(g_stream_raw, hipStreamCaptureModeThreadLocal));
   g_capturing = true;
+  g_zero_end = g_top;       // a zero fill done eagerly says nothing about replays: every block handed out while recording records its own fill
 }
 int lh_capture_end(void) {
   if (!g_capturing) { LH_FAIL("lh_capture_end without lh_capture_begin"); return -1; }
   if (g_capture_drawn) hipLaunchKernelGGL(k_set_u64, dim3(1), dim3(1), 0, g_stream_raw, g_capture_advance, 1ull, g_capture_drawn);
   g_capturing = false;
+  g_zero_end = g_top;       // fills recorded into the graph have not run
   hipGraph_t graph = nullptr;
   hipError_t e = hipStreamEndCapture(g_stream_raw, &graph);
   if (e != hipSuccess || graph == nullptr) {

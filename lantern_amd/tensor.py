@@ -550,6 +550,11 @@ class TensorR:
         bnp = None                       # a parked batchNorm producing one of the operands: absorbed if a relu follows
         if FUSE_BN_ADD_RELU and _pending is not None and _pending.bn is not None and (_pending.owner is self or _pending.owner is that):
             bnp, _pending = _pending, None
+            if bnp.bn["xin"] is (that if bnp.owner is self else self):
+                # relu(bn(h) + h): the batch norm's input is also the shortcut, so both gradients of the fused backward would be
+                # one buffer (its first pass adds into what its second overwrites); this join runs unfused
+                bnp.launch(False)
+                bnp = None
         be = get_backend()
         n = self.x.scalarCount
         ybuf = be.mallocArray(n, zero=False)

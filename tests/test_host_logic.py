@@ -141,3 +141,39 @@ def test_batchnorm_followed_by_add_without_relu_runs_unfused(on_cpu):
     np.testing.assert_allclose(v, ref + s.x.toCPU(), rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(y.x.toCPU(), ref, rtol=1e-4, atol=1e-5)      # and the batchNorm's output exists
     T._tape.clear()
+
+
+def test_join_whose_shortcut_is_the_batchnorms_own_input(be):
+    """relu(bn(h) + h): the batch norm's input is also the shortcut, so the fused backward would be handed one buffer for both of
+    its gradient outputs (its first pass adds the masked gradient into what its second pass overwrites, losing the shortcut's
+    share).  The mirror runs this join unfused; values and gradients equal the program with the fusion switched off."""
+    rng = np.random.RandomState(5)
+    xs = rng.randn(4, 3, 5, 5).astype(np.float32)
+
+    def run(fused):
+        T.FUSE_BN_ADD_RELU = fused
+        try:
+            x = TensorR(Tensor.fromNumpy(xs)); g = TensorR(Tensor.fromData((3,), 1.5, 0.5, 2.0)); b = TensorR(Tensor.fromData((3,), 0.1, -0.2, 0.3))
+            kept = {}
+            def f(d):
+                h = x * 1.5
+                out = (h.batchNorm(g, b, Tensor.zeros(3), Tensor.ones(3)) + h).relu(True)
+                kept["out"] = out.x.toCPU().copy()
+                return (out * out).sum()
+            gradR_loss(f)(Tensor.zeros(1))
+            return [kept["out"], x.d.toCPU(), g.d.toCPU(), b.d.toCPU()]
+        finally:
+            T.FUSE_BN_ADD_RELU = True
+    fused, plain = run(True), run(False)
+    for u, v in zip(fused, plain):
+        np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)
+    # and against the definition: d/dh [relu(bn(h) + h)] has the identity term of the shortcut
+    h = 1.5 * xs.astype(np.float64)
+    mu = h.mean((0, 2, 3), keepdims=True); var = h.var((0, 2, 3), keepdims=True); xhat = (h - mu) / np.sqrt(var + 1e-5)
+    gam = np.array([1.5, 0.5, 2.0]).reshape(1, 3, 1, 1); bet = np.array([0.1, -0.2, 0.3]).reshape(1, 3, 1, 1)
+    out = np.maximum(gam * xhat + bet + h, 0)
+    np.testing.assert_allclose(fused[0], out, rtol=1e-4, atol=1e-5)
+    dz = 2 * out * (out > 0)
+    dxhat = dz * gam
+    dh = (dxhat - dxhat.mean((0, 2, 3), keepdims=True) - xhat * (dxhat * xhat).mean((0, 2, 3), keepdims=True)) / np.sqrt(var + 1e-5) + dz
+    np.testing.assert_allclose(fused[1], 1.5 * dh, rtol=2e-4, atol=2e-4)

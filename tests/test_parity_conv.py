@@ -198,3 +198,35 @@ def test_conv_32_row_tiles(on_hip, dims, bias, monkeypatch):
     forced through the library's test switch (the measured launch plan may be another one)."""
     monkeypatch.setenv("LH_FORCE_M32", "1")
     check_conv(Dev(on_hip), dims, bias)
+
+
+@pytest.mark.parametrize("dims", [(8, 64, 28, 28, 64, 3, 3, 1, 1, 1, 1),      # filter gradient cut into 25 slices
+                                  (4, 32, 15, 13, 40, 3, 3, 2, 2, 1, 1),      # strided, odd maps, with bias
+                                  (16, 256, 7, 7, 512, 3, 3, 1, 1, 1, 1),     # few tiles over a long reduction (stream-K by default)
+                                  (3, 10, 12, 12, 20, 5, 5, 1, 1, 0, 0)], ids=lambda d: "x".join(map(str, d)))
+def test_conv_deterministic_mode(on_hip, dims):
+    """lh_set_deterministic(1): the same results against the oracle (slices of a reduction added by a second kernel in a fixed
+    order instead of by atomic adds, no stream-K), and two calls give the same bits."""
+    dev = Dev(on_hip)
+    on_hip.setDeterministic(True)
+    try:
+        assert dev.lib.lh_get_deterministic() == 1
+        check_conv(dev, dims, bias=True)
+        N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+        P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+        rng = np.random.RandomState(11)
+        x = dev.up(rng.randn(N, Cc, H, W).astype(np.float32)); dy = dev.up(rng.randn(N, K, P, Q).astype(np.float32))
+        w = dev.up((rng.randn(K, Cc, R, S) / np.sqrt(Cc * R * S)).astype(np.float32))
+        runs = []
+        for _ in range(2):
+            gdw = dev.up(np.full((K, Cc, R, S), 0.5, np.float32)); gdb = dev.up(np.ones(K, np.float32)); gdx = dev.zeros(N * Cc * H * W)
+            y = dev.zeros(N * K * P * Q)
+            dev.lib.lh_conv2d_fwd(x.ptr, w.ptr, 0, y.ptr, *dims)
+            dev.lib.lh_conv2d_bwd_data(dy.ptr, w.ptr, gdx.ptr, 0.0, *dims)
+            dev.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, gdw.ptr, gdb.ptr, 1.0, *dims); dev.check()
+            runs.append([dev.down(y, (N, K, P, Q)), dev.down(gdx, (N, Cc, H, W)), dev.down(gdw, (K, Cc, R, S)), dev.down(gdb, (K,))])
+        for a, b, what in zip(runs[0], runs[1], ("y", "dx", "dw", "db")):
+            np.testing.assert_array_equal(a, b, err_msg=what)
+    finally:
+        on_hip.setDeterministic(False)
+    assert dev.lib.lh_get_deterministic() == 0

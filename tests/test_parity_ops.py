@@ -576,6 +576,37 @@ def test_sgemm_few_tiles_long_reduction_with_row_stride(on_hip, tt, beta):
     np.testing.assert_array_equal(got[:, n:], C0[:, n:])
 
 
+@pytest.mark.parametrize("beta", [0.0, 1.0, 0.5])
+def test_deterministic_mode_sgemm_slices_and_axis_sums(on_hip, beta):
+    """lh_set_deterministic(1): a product whose reduction is cut into slices (each into its own scratch block, added in slice
+    order onto beta*C), the 10-output classifier shape of the small-product kernel, and a sum over a long middle axis give
+    the right values and the same bits on a second call; padding columns of a strided C stay untouched."""
+    be = on_hip
+    from lantern_amd import _lib
+    rng = np.random.RandomState(43)
+    be.setDeterministic(True)
+    try:
+        for (ta, tb, m, n, k, ldc) in ((1, 0, 200, 136, 3000, 144), (0, 1, 64, 10, 2048, 10), (0, 0, 800, 800, 5920, 800)):
+            A = rng.randn(*((k, m) if ta else (m, k))).astype(np.float32); Bm = rng.randn(*((n, k) if tb else (k, n))).astype(np.float32)
+            C0 = rng.randn(m, ldc).astype(np.float32)
+            a, b = be.fromHost(A), be.fromHost(Bm)
+            outs = []
+            for _ in range(2):
+                c = be.fromHost(C0)
+                be.lib.lh_sgemm(ta, tb, m, n, k, 0.75, a.ptr, A.shape[1], b.ptr, Bm.shape[1], beta, c.ptr, ldc); _lib.check()
+                outs.append(be.toHost(c, m * ldc).reshape(m, ldc))
+            want = 0.75 * ((A.T if ta else A).astype(np.float64) @ (Bm.T if tb else Bm).astype(np.float64)) + beta * C0[:, :n]
+            assert_close(outs[0][:, :n], want.astype(np.float32), rtol=1e-4, what="deterministic sgemm %dx%dx%d" % (m, n, k))
+            np.testing.assert_array_equal(outs[0], outs[1])
+            np.testing.assert_array_equal(outs[0][:, n:], C0[:, n:])
+        x = rng.randn(2, 5920, 1600).astype(np.float32); xd = be.fromHost(x)
+        ys = [be.toHost(be.sum_dim(xd, 2, 5920, 1600), 2 * 1600) for _ in range(2)]
+        assert_close(ys[0].reshape(2, 1600), x.astype(np.float64).sum(1).astype(np.float32), rtol=1e-4, what="deterministic sum over the middle axis")
+        np.testing.assert_array_equal(ys[0], ys[1])
+    finally:
+        be.setDeterministic(False)
+
+
 # ---- arena and error path (the library's own behaviour; no oracle counterpart) -----------------------
 def _arena_block(be, n, zero=True):
     """A block straight from the library's arena (BackendHIP.mallocArray cuts small blocks from larger ones itself)."""
