@@ -26,6 +26,8 @@ import numpy as np  # noqa: E402,F401
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# conv kernels of the headline step under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/resnet50_b64_hbm_traffic_and_mfma_counters.md)
+PROFILED_TRAFFIC = {"bytes_per_launch": 151.1e6, "launches_per_step": 158}
 CATS = ["conv_fwd", "conv_bwd_data", "conv_bwd_filter", "gemm", "bn_fwd", "bn_bwd", "elementwise", "pool", "reduce", "optim", "fill", "rnn", "cmdlist"]
 
 DEFAULT_BATCH = {"resnet50": 64, "squeezenet": 64, "lenet": 100, "treelstm": 1, "deepspeech2": 32}
@@ -37,7 +39,7 @@ def make_trainer(args, batch, cpu=False):
     if w == "resnet50":
         from lantern_amd.apps.resnet50 import ResNet50, Trainer
         model = ResNet50(num_classes=args.classes, imagenet_stem=args.hw > 64)
-        return Trainer(model, batch, args.hw, args.classes, lr=0.1, momentum=0.9), batch, \
+        return Trainer(model, batch, args.hw, args.classes, lr=0.1, momentum=0.9, streamed=not cpu and not args.resident and not args.graph), batch, \
             "ResNet-50 training step (configs[3]): batch %d, 3x%dx%d, %d classes, SGD lr 0.1 momentum 0.9, Kaiming-normal init" % (batch, args.hw, args.hw, args.classes)
     if w == "squeezenet":
         from lantern_amd.apps.squeezenet import Trainer
@@ -73,6 +75,7 @@ def run_gpu(args):
         lib.lh_set_side_stream(0)
     if args.deterministic:
         be.setDeterministic(True)
+    streamed = bool(getattr(tr, "streamed", False))
     loss_first = None
     for i in range(args.warmup):
         l = tr.step()
@@ -80,7 +83,18 @@ def run_gpu(args):
             loss_first = float(l.toCPU()[0])      # before any update: ln(classes) for a freshly initialised classifier
         tr.end_step()
     be.sync()
+    if streamed:
+        # The host link's clock ramps up under sustained traffic (the first ~0.5 s of per-step uploads run 2-4 % slower than the
+        # steady state an epoch of thousands of steps sees): about a second of untimed uploads into a scratch buffer first.
+        scratch = be.mallocArray(tr.hx[0].size, zero=False)
+        t_w = time.perf_counter()
+        while time.perf_counter() - t_w < 1.0:
+            for _ in range(32):
+                be.uploadAsync(scratch, tr.hx[1])
+            be.sync()
+        tr.end_step()
     t_issued = None
+    resident_sec = None
     if args.graph:
         # the step recorded once (after the warm-up measured the launch plans) and replayed: one host call per step
         g = la.StepGraph(tr, eager_steps=0)
@@ -92,7 +106,8 @@ def run_gpu(args):
         t1 = time.perf_counter()
         g.close()
     else:
-        # the timed region: exactly `steps` steps, nothing else on the stream
+        # the timed region: exactly `steps` steps, nothing else on the stream.  Streamed (the headline program): every step
+        # uploads its batch from pinned host memory and reads its loss back, as the reference's loop does.
         t0 = time.perf_counter()
         for _ in range(args.steps):
             tr.step()
@@ -100,6 +115,17 @@ def run_gpu(args):
         t_issued = time.perf_counter()      # the host has enqueued everything; the device may still be working
         be.sync()
         t1 = time.perf_counter()
+        if streamed:
+            assert np.isfinite(tr.losses()[-min(args.steps, tr.LOSS_RING):]).all(), "a streamed step's loss did not arrive"
+            # the same steps on a resident batch, no upload and no read-back (second figure; not the metric)
+            tr.streamed = False
+            tr.step(); tr.end_step(); be.sync()
+            r0 = time.perf_counter()
+            for _ in range(args.steps):
+                tr.step()
+                tr.end_step()
+            be.sync()
+            resident_sec = time.perf_counter() - r0
     # the same `steps` steps again with a HIP event pair around every matrix-kernel launch (conv x3, gemm, rnn).
     # Kept out of the timed region: an event between two launches drains the pipeline and costs about 1 ms per step.
     # (a program that runs from the command list times only the interpreter launches: an event elsewhere would cut the list short)
@@ -115,6 +141,18 @@ def run_gpu(args):
     timed = {CATS[i]: (ms[i] / args.steps, int(calls[i]) // args.steps) for i in range(len(CATS))}
     work = {k: v / args.steps for k, v in be.work.items()}
     be.count_work = False
+    # the same again around the HBM-bound families (batch norm forward / backward, element-wise, pooling, optimizer)
+    hbm_cats = ("bn_fwd", "bn_bwd", "elementwise", "pool", "optim")
+    timed_hbm = {}
+    if not getattr(tr, "batching", False):
+        lib.lh_prof_enable(sum(1 << CATS.index(c) for c in hbm_cats))
+        lib.lh_prof_collect(ms, calls, len(CATS))
+        for _ in range(args.steps):
+            tr.step()
+            tr.end_step()
+        be.sync()
+        lib.lh_prof_collect(ms, calls, len(CATS))
+        timed_hbm = {c: (ms[CATS.index(c)] / args.steps, int(calls[CATS.index(c)]) // args.steps) for c in hbm_cats}
     # a separate, untimed pass with every category instrumented (breakdown for the log)
     lib.lh_prof_enable((1 << CATS.index("cmdlist")) if getattr(tr, "batching", False) else (1 << len(CATS)) - 1)
     tr.step(); tr.end_step()
@@ -124,7 +162,7 @@ def run_gpu(args):
     loss_val = float(tr.step().toCPU()[0]); tr.end_step()
     peak_gb = lib.lh_heap_peak() / 2 ** 30
     be.cleanup()
-    return {"sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
+    return {"streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
             "per_step": per_step, "desc": desc}
 
 
@@ -179,6 +217,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--tree-file", default=None, help="treelstm: trees in the reference's array_tree.txt format instead of random ones (tests/golden/array_tree_first24.txt)")
     ap.add_argument("--no-side-stream", action="store_true", help="filter gradients in line on the main stream (kernel profiles: no two kernels overlap)")
+    ap.add_argument("--resident", action="store_true", help="resnet50: keep one batch resident on the device (no per-step upload, no loss read-back)")
     ap.add_argument("--deterministic", action="store_true", help="fixed-order reductions and rule-chosen launch plans (lh_set_deterministic): what run-to-run bit equality costs")
     ap.add_argument("--graph", action="store_true", help="time replays of the step recorded into a HIP graph (fixed-shape workloads)")
     ap.add_argument("--verbose", action="store_true")
@@ -210,9 +249,25 @@ def main():
         roof = {"bound": "mfma", "kernel": "k_igemm (conv fwd + bwd-data + bwd-filter, %d launches/step)" % conv_calls,
                 "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this workload (see profiles/), not measured live
-                "traffic": 151.1e6 if args.workload == "resnet50" and args.batch == 64 and args.hw == 224 else None, "flop_per_step": conv_fl,
+                # HBM bytes per launch come from separate rocprofv3 FETCH_SIZE / WRITE_SIZE runs (profiles/), which this process cannot
+                # make; the profiled figure is reported only when this run launched the kernel as often per step as the profiled run
+                "traffic": PROFILED_TRAFFIC["bytes_per_launch"] if (args.workload == "resnet50" and args.batch == 64 and args.hw == 224 and not args.deterministic
+                                                                    and conv_calls == PROFILED_TRAFFIC["launches_per_step"]) else None,
+                "flop_per_step": conv_fl,
                 "ms_per_step": {"fwd": round(conv_ms[0], 3), "bwd_data": round(conv_ms[1], 3), "bwd_filter": round(conv_ms[2], 3)}}
+        # the HBM-bound families against the 8 TB/s peak: algorithmic bytes of what was issued / event-timed kernel time
+        th = g["timed_hbm"]
+        hbm = {}
+        for fam, key in (("bn_fwd", "bn_fwd_bytes"), ("bn_bwd", "bn_bwd_bytes"), ("elementwise", "elementwise_bytes")):
+            if fam in th and th[fam][0] > 0 and work.get(key, 0.0) > 0:
+                gbs = work[key] / (th[fam][0] / 1000.0) / 1e9
+                hbm[fam] = {"bytes_per_step": work[key], "ms_per_step": round(th[fam][0], 3), "launches": th[fam][1], "achieved": round(gbs, 1),
+                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
+        for fam in ("pool", "optim"):
+            if fam in th and th[fam][0] > 0:
+                hbm[fam] = {"ms_per_step": round(th[fam][0], 3), "launches": th[fam][1]}
+        if hbm:
+            roof["hbm"] = hbm
         if work.get("gemm_flop", 0.0) > 0 and timed["gemm"][0] > 0:
             roof["gemm"] = {"flop_per_step": work["gemm_flop"], "ms_per_step": round(timed["gemm"][0], 3),
                             "tflops": round(work["gemm_flop"] / (timed["gemm"][0] / 1000.0) / 1e12, 2)}
@@ -228,10 +283,15 @@ def main():
         "config": {"workload": g["desc"], "global_batch": args.batch, "loss_first_step": round(g["loss_first"], 5) if g["loss_first"] is not None else None, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
                    "launch": "hip graph replay" if args.graph else "one launch per kernel",
                    "host_issue_ms_per_step": round(1000.0 * g["issue_sec"] / args.steps, 3) if g["issue_sec"] is not None else None,
+                   "h2d": ("included: the batch (%.1f MB) is uploaded from pinned host memory for every step on a copy stream, beside the previous step; "
+                           "the loss is read back every step without a wait" % (args.batch * 3 * args.hw * args.hw * 4 / 1e6)) if g["streamed"] else "not included: inputs resident on the device",
                    "filter_gradients": "in line" if (args.no_side_stream or args.deterministic) else "side stream",
                    "reductions": "deterministic (two-pass, rule-chosen plans)" if args.deterministic else "atomic combine, measured plans"},
         "roofline": roof,
     }
+    if g["resident_sec"] is not None:
+        out["resident_input"] = {"value": round(g["per_step"] * args.steps / g["resident_sec"], 2), "ms_per_step": round(1000.0 * g["resident_sec"] / args.steps, 3),
+                                 "note": "the same steps with the batch resident on the device: no upload, no loss read-back"}
     if args.verbose:
         print(json.dumps(g["breakdown"], indent=1), file=sys.stderr)
     if not args.no_cpu:

@@ -70,6 +70,21 @@ size_t lh_heap_peak(void);
 void lh_h2d(void* dst, const void* h_src, size_t bytes);
 void lh_d2h(void* h_dst, const void* src, size_t bytes);   /* waits */
 void lh_d2d(void* dst, const void* src, size_t bytes);
+/* Transfers that do not stall the step.  The reference's training loop uploads every batch with a blocking cudaMemcpy and
+ * reads the loss back with another (GPUOPS:64-65; resnet50FromOnnx.scala:172-176): the device idles during the upload and
+ * the host cannot issue the next step until the loss has arrived.  Same data movement, overlapped:
+ *   lh_host_alloc / lh_host_free   pinned host memory (what the two calls below need on the host side);
+ *   lh_h2d_async   the upload runs on a copy stream, after everything issued so far (so the last reader of dst is done)
+ *                  and beside everything issued afterwards; dst must not be touched until lh_copy_join(), which makes the
+ *                  main stream wait for the uploads issued so far (lh_sync and lh_cleanup join too).  With two device
+ *                  buffers the batch of step i+1 travels while step i computes;
+ *   lh_d2h_async   enqueues the read-back and returns; the value is in h_dst after the next lh_sync (or any later lh_d2h).
+ * None of them can be recorded into a graph. */
+void* lh_host_alloc(size_t bytes);
+void  lh_host_free(void* p);
+void  lh_h2d_async(void* dst, const void* h_src_pinned, size_t bytes);
+void  lh_copy_join(void);
+void  lh_d2h_async(void* h_dst_pinned, const void* src, size_t bytes);
 
 /* ---- timing helpers for the benchmark (HIP events on the library stream) */
 void* lh_event_create(void);

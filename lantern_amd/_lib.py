@@ -28,6 +28,11 @@ SIGNATURES = {
     "lh_heap_peak": (Z, []),
     "lh_h2d": (None, [P, P, Z]),
     "lh_d2h": (None, [P, P, Z]),
+    "lh_host_alloc": (P, [Z]),
+    "lh_host_free": (None, [P]),
+    "lh_h2d_async": (None, [P, P, Z]),
+    "lh_copy_join": (None, []),
+    "lh_d2h_async": (None, [P, P, Z]),
     "lh_d2d": (None, [P, P, Z]),
     "lh_event_create": (P, []),
     "lh_event_record": (None, [P]),

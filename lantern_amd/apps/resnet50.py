@@ -87,26 +87,65 @@ class ResNet50(Module):
 
 class Trainer:
     """One emitted training loop: parameters and the batch live below the arena mark; everything a
-    step allocates is released by rewinding to it (resnet50FromOnnx.scala:162-191)."""
+    step allocates is released by rewinding to it (resnet50FromOnnx.scala:162-191).
 
-    def __init__(self, model, batch, hw, num_classes, lr=0.1, momentum=0.9, seed=42):
+    `streamed`: the loop body as the reference's program runs it, with a fresh batch uploaded from the host for every step
+    and the loss read back after every step (resnet50FromOnnx.scala:172-176), but without the two stalls: batches alternate
+    between two device buffers, the upload of batch i+1 runs on the copy stream while step i computes, and the loss is read
+    back into a ring of pinned host slots that the host looks at later (`losses()`)."""
+
+    LOSS_RING = 64
+
+    def __init__(self, model, batch, hw, num_classes, lr=0.1, momentum=0.9, seed=42, streamed=False):
         be = get_backend()
         rng = np.random.RandomState(seed + 1)
         self.model = model
         self.opt = SGD_Momentum(model, lr, momentum)
         self.x_host = rng.standard_normal((batch, 3, hw, hw)).astype(np.float32)
         self.y_host = rng.randint(0, num_classes, size=batch).astype(np.int32)
-        self.x = Tensor.fromNumpy(self.x_host)
-        self.target = int_array(self.y_host)
+        self.streamed = streamed
+        if streamed:
+            shape = (batch, 3, hw, hw)
+            self.hx = [be.hostArray(shape), be.hostArray(shape)]
+            self.hy = [be.hostArray((batch,), np.int32), be.hostArray((batch,), np.int32)]
+            self.hx[0][...] = self.x_host; self.hy[0][...] = self.y_host
+            self.hx[1][...] = rng.standard_normal(shape).astype(np.float32); self.hy[1][...] = rng.randint(0, num_classes, size=batch)
+            self.dx = [Tensor(be.mallocArray(self.x_host.size, zero=False), shape) for _ in range(2)]
+            self.dt = [be.mallocArray(batch, zero=False) for _ in range(2)]
+            self.hloss = be.hostArray((self.LOSS_RING,))
+            self.hloss[...] = np.nan
+            self.i = 0
+            be.uploadAsync(self.dx[0].data, self.hx[0]); be.uploadAsync(self.dt[0], self.hy[0])
+            self.x, self.target = self.dx[0], self.dt[0]
+        else:
+            self.x = Tensor.fromNumpy(self.x_host)
+            self.target = int_array(self.y_host)
         self.mark = be.getMallocAddr()
 
     def step(self):
         be = get_backend()
+        if self.streamed:
+            k = self.i % 2
+            be.copyJoin()                     # batch i has arrived (its upload was issued during step i-1)
+            self.x, self.target = self.dx[k], self.dt[k]
+            # batch i+1 travels while this step computes: the last reader of its buffer, step i-1, has been issued already
+            be.uploadAsync(self.dx[1 - k].data, self.hx[1 - k]); be.uploadAsync(self.dt[1 - k], self.hy[1 - k])
         xin = TensorR(self.x, isInput=True)
-        loss = gradR_loss(lambda dummy: self.model(xin).logSoftmaxB().nllLossB(self.target).mean())(Tensor.zeros(1))
+        target = self.target
+        loss = gradR_loss(lambda dummy: self.model(xin).logSoftmaxB().nllLossB(target).mean())(Tensor.zeros(1))
+        if self.streamed:
+            slot = self.i % self.LOSS_RING
+            be.downloadAsync(self.hloss[slot:slot + 1], loss.data)
+            self.i += 1
         self.opt.step()
         self.last_loss = loss
         return loss
+
+    def losses(self):
+        """The losses of the last LOSS_RING streamed steps, oldest first (waits for the device)."""
+        get_backend().sync()
+        n = min(self.i, self.LOSS_RING)
+        return np.array([self.hloss[(self.i - n + j) % self.LOSS_RING] for j in range(n)], np.float32)
 
     def end_step(self):
         get_backend().resetMallocAddr(self.mark)

@@ -171,6 +171,9 @@ class BackendHIP(Backend):
     def cleanup(self):
         if self.lib is not None:
             self.lib.lh_cleanup()
+            for p in getattr(self, "_pinned", []):
+                self.lib.lh_host_free(p)
+            self._pinned = []
             self.lib = None
 
     def sync(self):
@@ -253,6 +256,26 @@ class BackendHIP(Backend):
     def upload(self, buf, arr):
         arr = np.ascontiguousarray(arr)
         self.lib.lh_h2d(buf.ptr, arr.ctypes.data, arr.nbytes); _lib.check()
+
+    # -- transfers that do not stall the step (pinned host memory, copy stream, deferred read-back) ----------
+    def hostArray(self, shape, dtype=np.float32):
+        """A numpy array over pinned host memory (freed by cleanup())."""
+        n = int(np.prod(shape, dtype=np.int64)) * np.dtype(dtype).itemsize
+        p = self.lib.lh_host_alloc(n); _lib.check()
+        self._pinned = getattr(self, "_pinned", [])
+        self._pinned.append(p)
+        return np.ctypeslib.as_array((C.c_byte * n).from_address(p)).view(dtype).reshape(shape)
+
+    def uploadAsync(self, buf, pinned_arr):
+        """Upload on the copy stream: after everything issued so far, beside everything issued from now on (copyJoin before use)."""
+        self.lib.lh_h2d_async(buf.ptr, pinned_arr.ctypes.data, pinned_arr.nbytes); _lib.check()
+
+    def copyJoin(self):
+        self.lib.lh_copy_join(); _lib.check()
+
+    def downloadAsync(self, pinned_arr, buf):
+        """Read-back that returns at once; the values are there after the next sync()."""
+        self.lib.lh_d2h_async(pinned_arr.ctypes.data, buf.ptr, pinned_arr.nbytes); _lib.check()
 
     # -- fills ------------------------------------------------------------------------------
     def fillInPlace(self, data, n, value):
@@ -385,7 +408,7 @@ class BackendHIP(Backend):
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
         self.lib.lh_conv2d_fwd_bn_apply(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, scale.ptr, bbias.ptr, sm.ptr, si.ptr,
                                         rmean.ptr, rvar.ptr, eps, factor, 0, ybn.ptr, int(relu)); _lib.check()
-        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW); self._count("bn_fwd_bytes", 8.0 * N * K * HW)    # statistics from the conv epilogue: one read, one write
 
     def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
         # The filter gradient is read by the optimizer only: it goes to the side stream, where it runs beside the
@@ -445,11 +468,13 @@ class BackendHIP(Backend):
         y = self.mallocArray(N * C * HW, zero=False)
         sm = self.mallocArray(C, zero=False); si = self.mallocArray(C, zero=False)
         self.lib.lh_bn_train_fwd(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
+        if self.count_work: self._count("bn_fwd_bytes", 12.0 * N * C * HW)       # x read for the statistics, read again, y written
         return y, sm, si
 
     def batchNormTraining_into(self, x, scale, bias, rmean, rvar, y, sm, si, N, C, HW, relu, eps=1e-5, factor=0.1):
         f = self.lib.lh_bn_train_fwd_relu if relu else self.lib.lh_bn_train_fwd
         f(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
+        if self.count_work: self._count("bn_fwd_bytes", 12.0 * N * C * HW)
 
     def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0, y_relu=None, bias=None):
         """y_relu: the layer's output went through a fused in-place relu; `bias` (the layer's beta) lets the
@@ -461,29 +486,38 @@ class BackendHIP(Backend):
         else:
             self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
         _lib.check()
+        # x and dy read for the two sums, read again, dx written (and read first when it accumulates)
+        if self.count_work: self._count("bn_bwd_bytes", (20.0 + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0)) * N * C * HW)
 
     def batchNormTraining_add_relu_into(self, x, scale, bias, rmean, rvar, shortcut, out, sm, si, N, C, HW, eps=1e-5, factor=0.1):
         self.lib.lh_bn_stats(x.ptr, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, N, C, HW, eps, factor)
         self.lib.lh_bn_apply_add_relu(x.ptr, scale.ptr, bias.ptr, sm.ptr, si.ptr, shortcut.ptr, out.ptr, N, C, HW); _lib.check()
+        if self.count_work: self._count("bn_fwd_bytes", 16.0 * N * C * HW)       # statistics pass, then x and the shortcut read, out written
 
     def conv2D_batch_bn_add_relu_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, shortcut, out, sm, si, eps=1e-5, factor=0.1):
         N, C, H, W, K, R, S, sH, sW, pH, pW = dims
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
         self.lib.lh_conv2d_fwd_bn_apply(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, scale.ptr, bbias.ptr, sm.ptr, si.ptr,
                                         rmean.ptr, rvar.ptr, eps, factor, shortcut.ptr, out.ptr, 1); _lib.check()
-        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW); self._count("bn_fwd_bytes", 12.0 * N * K * HW)   # y and the shortcut read, out written
 
     def batchNorm_add_relu_grad(self, x, xd, beta_dx, out, dout, scale, scaled, biasd, sm, si, sd, beta_sd, N, C, HW):
         self.lib.lh_bn_bwd_add_relu(x.ptr, out.ptr, dout.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, beta_dx,
                                     sd.ptr if sd is not None else 0, beta_sd, scaled.ptr, biasd.ptr, N, C, HW); _lib.check()
+        # pass 1 reads x, out, dout and writes the masked gradient (to the shortcut's buffer, or over dout); pass 2 reads x and the
+        # masked gradient and writes dx: 28 B per element, plus a read for each output that accumulates
+        if self.count_work:
+            self._count("bn_bwd_bytes", (28.0 + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0) + (8.0 if (sd is not None and beta_sd != 0.0) else 0.0)) * N * C * HW)
 
     def add_into(self, a, b, out, n, relu):
         if relu: self.lib.lh_add_relu(a.ptr, b.ptr, out.ptr, n)
         else: self.lib.lh_geam(a.ptr, 1.0, b.ptr, 1.0, out.ptr, n)
         _lib.check()
+        if self.count_work: self._count("elementwise_bytes", 12.0 * n)
 
     def add_relu_grad(self, y, dy, ad, abeta, bd, bbeta, n):
         self.lib.lh_add_relu_grad(y.ptr, dy.ptr, ad.ptr if ad is not None else 0, abeta, bd.ptr if bd is not None else 0, bbeta, n); _lib.check()
+        if self.count_work: self._count("elementwise_bytes", (8.0 + (0 if ad is None else 4.0 + 4.0 * (abeta != 0.0)) + (0 if bd is None else 4.0 + 4.0 * (bbeta != 0.0))) * n)
 
     # -- dropout ------------------------------------------------------------------------------------
     def dropout(self, x, n, prob):

@@ -131,6 +131,7 @@ void lh_setup(size_t heap_bytes) {
 }
 
 static void stage_release();
+static void copy_release();
 void lh_cleanup(void) {
   g_stream_cur = g_stream_raw;
   if (g_side_stream) { (void)hipStreamSynchronize(g_side_stream); (void)hipStreamDestroy(g_side_stream); for (auto& e : g_side_ev) (void)hipEventDestroy(e); }
@@ -138,6 +139,7 @@ void lh_cleanup(void) {
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
   cmdlist_release();
   stage_release();
+  copy_release();
   multi_tensor_release();
   for (auto& e : g_graphs) if (e) { (void)hipGraphExecDestroy(e); e = nullptr; }
   g_graphs.clear(); g_capturing = false;
@@ -151,6 +153,7 @@ void lh_cleanup(void) {
 void lh_sync(void) {
   LH_NOT_CAPTURING("lh_sync");
   side_join();
+  lh_copy_join();
   LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH();
 }
 
@@ -245,6 +248,56 @@ void lh_d2h(void* h_dst, const void* src, size_t bytes) {
   LH_HIP(hipMemcpyAsync(h_dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
 }
+// ---- transfers that do not stall the step: pinned host memory, a copy stream for uploads, read-backs without a wait ----
+static hipStream_t g_copy_stream = nullptr;
+static hipEvent_t g_copy_ev[4];
+static unsigned g_copy_ev_next = 0;
+static bool g_copy_dirty = false;              // the copy stream holds uploads the main stream has not waited for
+static bool copy_init() {
+  if (g_copy_stream) return true;
+  if (hipStreamCreateWithFlags(&g_copy_stream, hipStreamNonBlocking) != hipSuccess) { g_copy_stream = nullptr; return false; }   // default priority
+  for (auto& e : g_copy_ev) if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) return false;
+  return true;
+}
+static void copy_release() {
+  if (!g_copy_stream) return;
+  (void)hipStreamSynchronize(g_copy_stream);
+  for (auto& e : g_copy_ev) (void)hipEventDestroy(e);
+  (void)hipStreamDestroy(g_copy_stream);
+  g_copy_stream = nullptr; g_copy_dirty = false;
+}
+void* lh_host_alloc(size_t bytes) {
+  void* p = nullptr;
+  if (hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocDefault) != hipSuccess) { (void)hipGetLastError(); LH_FAIL("lh_host_alloc(%zu): no pinned host memory", bytes); return nullptr; }
+  return p;
+}
+void lh_host_free(void* p) { if (p) (void)hipHostFree(p); }
+void lh_h2d_async(void* dst, const void* h_src_pinned, size_t bytes) {
+  LH_NOT_CAPTURING("lh_h2d_async");
+  LH_REQUIRE(g_stream_raw != nullptr, "lh_h2d_async before lh_setup");
+  LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_h2d_async between lh_side_begin and lh_side_end");
+  if (bytes == 0) return;
+  LH_REQUIRE(copy_init(), "lh_h2d_async: cannot create the copy stream");
+  // after everything issued so far (the last reader of dst), beside everything issued from now on
+  hipEvent_t ev = g_copy_ev[g_copy_ev_next++ % 4];
+  LH_HIP(hipEventRecord(ev, g_stream));
+  LH_HIP(hipStreamWaitEvent(g_copy_stream, ev, 0));
+  LH_HIP(hipMemcpyAsync(dst, h_src_pinned, bytes, hipMemcpyHostToDevice, g_copy_stream));
+  g_copy_dirty = true;
+}
+void lh_copy_join(void) {
+  if (!g_copy_dirty) return;
+  g_copy_dirty = false;
+  hipEvent_t ev = g_copy_ev[g_copy_ev_next++ % 4];
+  LH_HIP(hipEventRecord(ev, g_copy_stream));
+  LH_HIP(hipStreamWaitEvent(g_stream_raw, ev, 0));
+}
+void lh_d2h_async(void* h_dst_pinned, const void* src, size_t bytes) {
+  LH_NOT_CAPTURING("lh_d2h_async");
+  if (bytes == 0) return;
+  LH_HIP(hipMemcpyAsync(h_dst_pinned, src, bytes, hipMemcpyDeviceToHost, g_stream));
+}
+
 void lh_d2d(void* dst, const void* src, size_t bytes) {
   if ((bytes & 3) == 0 && bytes > 0 && rec_ok((int64_t)(bytes / 4))) { rec_cmd(CL_COPY, (int)(bytes / 4), 0, 0, 0.f, 0.f, 0.f, 0.f, dst, src, nullptr, nullptr); return; }
   LH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));

@@ -270,6 +270,42 @@ def test_capture_rejects_waiting_entry_points(hip_backend):
     be.resetMallocAddr(mark)
 
 
+def test_streamed_batches_and_deferred_loss_give_the_resident_trajectory(hip_backend):
+    """The loop body with a batch uploaded for every step on the copy stream (two device buffers, the upload of batch i+1 beside
+    step i) and the loss read back without a wait: with the same data in both host buffers it must reproduce, bit for bit in
+    deterministic mode, the trajectory of the trainer whose batch is resident; with different data in the second buffer the
+    odd steps must differ (the upload really is what the step reads)."""
+    from lantern_amd.apps.resnet50 import ResNet50, Trainer
+    be = hip_backend
+    la.set_backend(be)
+    mk = lambda streamed: Trainer(ResNet50(num_classes=10, imagenet_stem=False, layers=(1, 1, 1, 1)), 8, 32, 10, lr=0.005, momentum=0.9, streamed=streamed)
+    be.setDeterministic(True)
+    try:
+        mark = be.getMallocAddr()
+        tr = mk(False)
+        want = []
+        for _ in range(6):
+            want.append(float(tr.step().toCPU()[0])); tr.end_step()
+        be.sync(); be.resetMallocAddr(mark)
+
+        tr = mk(True)
+        tr.hx[1][...] = tr.hx[0]; tr.hy[1][...] = tr.hy[0]
+        for _ in range(6):
+            tr.step(); tr.end_step()
+        got = tr.losses()
+        be.resetMallocAddr(mark)
+        np.testing.assert_array_equal(got, np.array(want, np.float32))
+
+        tr = mk(True)                       # the second host buffer holds another batch
+        for _ in range(6):
+            tr.step(); tr.end_step()
+        other = tr.losses()
+        be.resetMallocAddr(mark)
+        assert other[0] == got[0] and other[1] != got[1] and np.isfinite(other).all()
+    finally:
+        be.setDeterministic(False)
+
+
 def test_recorded_graph_launches_the_remembered_plans(hip_backend):
     """While a graph is recorded nothing can be timed, but the plans measured before are what gets recorded: the counter of
     launches that used a remembered plan moves during the recording, the counter of measurements does not, and the replay
