@@ -6,7 +6,10 @@ logSoftmax, plain SGD `x -= lr * d` followed by clear_grad, a progress line ever
 every batch, and a result file holding the per-epoch losses and the median epoch time.  With `device_decode` the raw records
 are uploaded and decoded on the device (same floats, a quarter of the copy); otherwise the host decodes as the reference does.
 
-    python -m lantern_amd.apps.cifar_loop squeezenet|resnet50 result.txt path/to/data_batch_1.bin
+    python -m lantern_amd.apps.cifar_loop squeezenet|resnet50|path/to/model.onnx result.txt path/to/data_batch_1.bin
+
+With a `.onnx` path the network comes from the file through lantern_amd.onnx (readONNX + training_func, as the reference's programs
+build theirs: resnet50FromOnnx.scala:150-157), its float initialisers being the parameters.
 """
 import time
 
@@ -69,7 +72,10 @@ def main(argv):
     hip = BackendHIP()
     hip.setup()
     set_backend(hip)
-    if which == "squeezenet":
+    if which.endswith(".onnx"):
+        from ..onnx import OnnxModel
+        model = OnnxModel(which)
+    elif which == "squeezenet":
         from .squeezenet import SqueezeNet
         model = SqueezeNet(10)
     else:
