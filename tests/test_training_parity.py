@@ -484,3 +484,71 @@ class _SeqClassifier:
 def test_lstm_gru_modules_10_steps(hip_backend, cpu_backend, kind, bidirectional, numLayers):
     """The LSTM / GRU modes of RNNBase (NNModule.scala:324-330), stacked and bidirectional, trained for ten steps."""
     _compare(lambda: _SeqClassifier(kind, bidirectional, numLayers), hip_backend, cpu_backend)
+
+
+# ---- the other configurations at their full sizes -----------------------------------------------------------------------------
+def test_squeezenet_full_batch_5_steps(hip_backend):
+    """SqueezeNet exactly as configured for the throughput figure (batch 64, 3x32x32, learning rate 0.005, momentum 0.9)
+    against the oracle on all host cores.  At this learning rate the trajectory is unstable (the loss rises after the first
+    step), so a rounding-sized difference grows quickly: five steps, and per-tensor bounds calibrated by the oracle's own
+    response to a one-ulp nudge."""
+    from oracle.backend_cpu import BackendCPU
+    from lantern_amd.apps.squeezenet import Trainer
+    cpu = BackendCPU(threads=8); cpu.setup()
+    _compare(lambda: Trainer(batch=64, lr=0.005, momentum=0.9), hip_backend, cpu, steps=5, self_calibrate=True)
+
+
+def test_treelstm_50_leaf_trees_against_the_oracle(hip_backend, cpu_backend):
+    """The largest trees of the configuration (50 leaves, 99 nodes, ~9000 operator calls each) over the full 20000-word table,
+    one Adagrad step per tree, small operators from the command list."""
+    from lantern_amd.apps.treelstm import Trainer
+    _compare(lambda: Trainer(n_trees=3, vocab=20000, min_leaves=50, max_leaves=50), hip_backend, cpu_backend, steps=3)
+
+
+def test_deepspeech2_full_size_invariants(hip_backend):
+    """DeepSpeech2 as configured for the throughput figure (batch 32, 161 x 400 spectrograms, three bidirectional layers of 800
+    units, 50 labels per utterance) is far beyond the oracle's reach; checked after a forward and backward pass at full size:
+      - the CTC cost of every utterance is positive and finite (it is -log of a probability), and the reported loss is their mean;
+      - both convolutions are followed by a batch norm, so each filter's gradient is orthogonal to the filter;
+      - the classifier has no bias and feeds a softmax: the gradient with respect to its logits sums to zero over the classes at
+        every frame, hence every row of the [800, 29] weight gradient (one input feature against all classes) sums to zero;
+      - gradients of all parameters are finite and not all zero (the recurrence, sequence-wise batch norms and permutes are between
+        the loss and the convolutions)."""
+    from lantern_amd.apps.deepspeech2 import Trainer
+    from lantern_amd.tensor import Tensor, TensorR, gradR_loss
+    be = hip_backend
+    la.set_backend(be)
+    mark = be.getMallocAddr()
+    tr = Trainer(batch=32, freq=161, frames=400, hidden=800, layers=3, label_len=50, lr=1e-5)
+    params = dict(tr.model.namedParameters())
+    for step in range(2):            # the second pass runs the remembered launch plans
+        xin = TensorR(tr.x, isInput=True)
+        seen = {}
+
+        def loss_fun(dummy):
+            probs = tr.model(xin).softmax_batch(2)
+            seen["T"] = probs.x.shape[0]
+            out_len = (tr.percent * probs.x.shape[0]).astype(np.int32)
+            return TensorR(probs.ctcLoss(out_len, tr.labels, tr.label_lengths))
+        loss = float(gradR_loss(loss_fun)(Tensor.zeros(1)).toCPU()[0])
+        assert seen["T"] == 185
+        # a uniform guess over 29 symbols for 185 frames costs 185*ln(29) = 623; a fresh network is near it, never below the 50-label floor
+        assert np.isfinite(loss) and 50.0 < loss < 2000.0, loss
+        for name in ("conv1", "conv2"):
+            p = [q for n, q in params.items() if n.endswith(name + "/kernel")][0]
+            w = p.x.toCPU().astype(np.float64); dw = p.d.toCPU().astype(np.float64)
+            w = w.reshape(w.shape[0], -1); dw = dw.reshape(dw.shape[0], -1)
+            assert np.isfinite(dw).all() and np.abs(dw).max() > 0
+            cos = np.abs((w * dw).sum(1)) / (np.linalg.norm(w, axis=1) * np.linalg.norm(dw, axis=1) + 1e-300)
+            assert cos.max() < 1e-3, "step %d, %s: |cos(filter, gradient)| %.3g" % (step, name, cos.max())
+        fcw = [q for n, q in params.items() if "fc" in n and "bn" not in n and q.x.shape[-1] == 29][0]
+        dfc = fcw.d.toCPU().astype(np.float64)
+        rows = np.abs(dfc.sum(1)); scale = np.abs(dfc).sum(1)
+        assert scale.max() > 0 and (rows <= 1e-3 * scale + 1e-7).all(), float((rows / (scale + 1e-30)).max())
+        for n, p in params.items():
+            d = p.d.toCPU()
+            assert np.isfinite(d).all() and np.abs(d).max() > 0, n
+        print("step %d: loss %.3f; classifier gradient row sums at most %.3g of their absolute sums" % (step, loss, float((rows / (scale + 1e-30)).max())))
+        tr.opt.step()
+        tr.end_step()
+    be.sync(); be.resetMallocAddr(mark)
