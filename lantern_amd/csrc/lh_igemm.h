@@ -278,20 +278,29 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
     __builtin_amdgcn_sched_barrier(0);
     const float4* Asc = As + st * KQ * LDA + wm * TM + l32;
     const float4* Bsc = Bs + st * KQ * LDB + wn * TN + l32;
+    // operands of the next pair of k-quads are read from LDS before the matrix instructions of the current pair are
+    // issued, so a wavefront does not stand still for the LDS latency between pairs
+    float4 a[2][MI], b[2][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; mi++) a[0][mi] = Asc[half * LDA + mi * 32];
+#pragma unroll
+    for (int ni = 0; ni < NI; ni++) b[0][ni] = Bsc[half * LDB + ni * 32];
 #pragma unroll
     for (int pair = 0; pair < KQ / 2; pair++) {
-      const int kq = 2 * pair + half;
-      float4 a[MI], b[NI];
+      const int cur = pair & 1, nxt = cur ^ 1;
+      if (pair + 1 < KQ / 2) {
+        const int kq = 2 * (pair + 1) + half;
 #pragma unroll
-      for (int mi = 0; mi < MI; mi++) a[mi] = Asc[kq * LDA + mi * 32];
+        for (int mi = 0; mi < MI; mi++) a[nxt][mi] = Asc[kq * LDA + mi * 32];
 #pragma unroll
-      for (int ni = 0; ni < NI; ni++) b[ni] = Bsc[kq * LDB + ni * 32];
+        for (int ni = 0; ni < NI; ni++) b[nxt][ni] = Bsc[kq * LDB + ni * 32];
+      }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int m = 0; m < NM_PAIR; m++) {
         const int c = m / (MI * NI), mi = (m / NI) % MI, ni = m % NI;
-        const float av = c == 0 ? a[mi].x : c == 1 ? a[mi].y : c == 2 ? a[mi].z : a[mi].w;
-        const float bv = c == 0 ? b[ni].x : c == 1 ? b[ni].y : c == 2 ? b[ni].z : b[ni].w;
+        const float av = c == 0 ? a[cur][mi].x : c == 1 ? a[cur][mi].y : c == 2 ? a[cur][mi].z : a[cur][mi].w;
+        const float bv = c == 0 ? b[cur][ni].x : c == 1 ? b[cur][ni].y : c == 2 ? b[cur][ni].z : b[cur][ni].w;
         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
         const int gm = pair * NM_PAIR + m;
         const int e0 = (gm * NEL) / NM, e1 = ((gm + 1) * NEL) / NM;
