@@ -279,6 +279,16 @@ int64_t lh_rnn_gated_reserve_floats(int mode, int T, int B, int H, int bidir);
 void lh_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, float* reserve, int T, int B, int I, int H, int bidir);
 void lh_rnn_gated_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* reserve, float* dx, float beta_dx,
                       float* dw, int T, int B, int I, int H, int bidir);
+/* The same four calls with the initial states of RNNBase.apply(input, hx, cx) (NNModule.scala:392-409; hxData / cxData at
+ * CDN:1832-1833): hx [D,B,H] and, for the LSTM, cx [D,B,H] of this layer (NULL = zeros, which is what the calls above pass).
+ * They are values only: the reference passes NULL for dhx / dcx (CDN:1843-1844), so no gradient is produced for them. */
+void lh_rnn_fwd_init(int mode, const float* x, const float* hx, const float* w, float* y, int T, int B, int I, int H, int bidir);
+void lh_rnn_bwd_init(int mode, const float* x, const float* hx, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
+                     int T, int B, int I, int H, int bidir);
+void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const float* cx, const float* w, float* y, float* reserve,
+                           int T, int B, int I, int H, int bidir);
+void lh_rnn_gated_bwd_init(int mode, const float* x, const float* hx, const float* cx, const float* y, const float* dy, const float* w,
+                           float* reserve, float* dx, float beta_dx, float* dw, int T, int B, int I, int H, int bidir);
 /* ctcLoss (TD:349; CDN:1895-1938, cudnnCTCLoss): probs [T,B,A] are softmax outputs, class 0 is the blank;
  * h_labels (concatenated), h_label_len [B], h_input_len [B] are HOST arrays as in the cuDNN call;
  * costs[b] = -log p(labels_b | probs).  When dprobs is not NULL the gradient with respect to the

@@ -113,6 +113,10 @@ SIGNATURES = {
     "lh_rnn_gated_reserve_floats": (L, [I, I, I, I, I]),
     "lh_rnn_gated_fwd": (None, [I, P, P, P, P, I, I, I, I, I]),
     "lh_rnn_gated_bwd": (None, [I, P, P, P, P, P, P, F, P, I, I, I, I, I]),
+    "lh_rnn_fwd_init": (None, [I, P, P, P, P, I, I, I, I, I]),
+    "lh_rnn_bwd_init": (None, [I, P, P, P, P, P, P, F, P, I, I, I, I, I]),
+    "lh_rnn_gated_fwd_init": (None, [I, P, P, P, P, P, P, I, I, I, I, I]),
+    "lh_rnn_gated_bwd_init": (None, [I, P, P, P, P, P, P, P, P, F, P, I, I, I, I, I]),
     "lh_ctc_loss": (None, [P, P, P, P, P, P, I, I, I]),
     "lh_maxpool_bwd_dense": (None, [P, P, P, F, I, I, I, I, I, I, I, I, I]),
     "lh_add_relu": (None, [P, P, P, L]),

@@ -628,30 +628,32 @@ class BackendHIP(Backend):
         _lib.check()
         return costs
 
-    def rnn_forward(self, mode, x, w, T, B, I, H, bidir):
+    def rnn_forward(self, mode, x, w, T, B, I, H, bidir, hx=None):
         y = self.mallocArray(T * B * H * (2 if bidir else 1), zero=False)
-        self.lib.lh_rnn_fwd(mode, x.ptr, w.ptr, y.ptr, T, B, I, H, int(bidir)); _lib.check()
+        self.lib.lh_rnn_fwd_init(mode, x.ptr, hx.ptr if hx is not None else 0, w.ptr, y.ptr, T, B, I, H, int(bidir)); _lib.check()
         if self.count_work: self._count("gemm_flop", 2.0 * T * B * H * I * (2 if bidir else 1)); self._count("rnn_flop", 2.0 * T * B * H * H * (2 if bidir else 1))
         return y
 
-    def rnn_backward(self, mode, x, y, dy, w, dx, dw, T, B, I, H, bidir, beta_dx=1.0):
-        self.lib.lh_rnn_bwd(mode, x.ptr, y.ptr, dy.ptr, w.ptr, dx.ptr if dx is not None else 0, beta_dx, dw.ptr, T, B, I, H, int(bidir)); _lib.check()
+    def rnn_backward(self, mode, x, y, dy, w, dx, dw, T, B, I, H, bidir, beta_dx=1.0, hx=None):
+        self.lib.lh_rnn_bwd_init(mode, x.ptr, hx.ptr if hx is not None else 0, y.ptr, dy.ptr, w.ptr, dx.ptr if dx is not None else 0, beta_dx, dw.ptr,
+                                 T, B, I, H, int(bidir)); _lib.check()
         D = 2 if bidir else 1
         if self.count_work: self._count("gemm_flop", 2.0 * T * B * H * D * (I * (2 if dx is not None else 1) + H)); self._count("rnn_flop", 2.0 * T * B * H * H * D)
 
-    def rnn_gated_forward(self, mode, x, w, T, B, I, H, bidir):
+    def rnn_gated_forward(self, mode, x, w, T, B, I, H, bidir, hx=None, cx=None):
         """LSTM (mode 2) / GRU (mode 3): returns (y, reserve); the reserve goes to rnn_gated_backward, once."""
         D = 2 if bidir else 1
         y = self.mallocArray(T * B * H * D, zero=False)
         reserve = self.mallocArray(self.lib.lh_rnn_gated_reserve_floats(mode, T, B, H, int(bidir)), zero=False)
-        self.lib.lh_rnn_gated_fwd(mode, x.ptr, w.ptr, y.ptr, reserve.ptr, T, B, I, H, int(bidir)); _lib.check()
+        self.lib.lh_rnn_gated_fwd_init(mode, x.ptr, hx.ptr if hx is not None else 0, cx.ptr if cx is not None else 0, w.ptr, y.ptr, reserve.ptr,
+                                       T, B, I, H, int(bidir)); _lib.check()
         G = (4 if mode == 2 else 3) * H
         if self.count_work: self._count("gemm_flop", 2.0 * T * B * G * (I + H) * D)
         return y, reserve
 
-    def rnn_gated_backward(self, mode, x, y, dy, w, reserve, dx, dw, T, B, I, H, bidir, beta_dx=1.0):
-        self.lib.lh_rnn_gated_bwd(mode, x.ptr, y.ptr, dy.ptr, w.ptr, reserve.ptr, dx.ptr if dx is not None else 0, beta_dx, dw.ptr,
-                                  T, B, I, H, int(bidir)); _lib.check()
+    def rnn_gated_backward(self, mode, x, y, dy, w, reserve, dx, dw, T, B, I, H, bidir, beta_dx=1.0, hx=None, cx=None):
+        self.lib.lh_rnn_gated_bwd_init(mode, x.ptr, hx.ptr if hx is not None else 0, cx.ptr if cx is not None else 0, y.ptr, dy.ptr, w.ptr, reserve.ptr,
+                                       dx.ptr if dx is not None else 0, beta_dx, dw.ptr, T, B, I, H, int(bidir)); _lib.check()
         G = (4 if mode == 2 else 3) * H
         if self.count_work: self._count("gemm_flop", 2.0 * T * B * G * (I * (2 if dx is not None else 1) + 2 * H) * (2 if bidir else 1))
 

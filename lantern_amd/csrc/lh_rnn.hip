@@ -342,6 +342,14 @@ __global__ void __launch_bounds__(128) k_ctc_wave(const float* __restrict__ prob
 extern "C" {
 
 void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+  lh_rnn_fwd_init(mode, x, nullptr, w, y, T, B, I, H, bidir);
+}
+void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
+                int T, int B, int I, int H, int bidir) {
+  lh_rnn_bwd_init(mode, x, nullptr, y, dy, w, dx, beta_dx, dw, T, B, I, H, bidir);
+}
+
+void lh_rnn_fwd_init(int mode, const float* x, const float* hx, const float* w, float* y, int T, int B, int I, int H, int bidir) {
   LH_REQUIRE(mode == 0 || mode == 1, "lh_rnn_fwd: mode %d (0 = relu, 1 = tanh)", mode);
   LH_REQUIRE(T >= 1 && B >= 1 && I >= 1 && H >= 1, "lh_rnn_fwd: bad shape T%d B%d I%d H%d", T, B, I, H);
   LH_REQUIRE(H <= 2048, "lh_rnn_fwd: hidden size %d above %d", H, 2048);
@@ -350,6 +358,9 @@ void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B
   for (int d = 0; d < D; d++) {          // input projection of every step straight into y
     const float* Wih = w + d * dir_params(I, H);
     lh_sgemm(0, 1, T * B, H, I, 1.0f, x, I, Wih, I, 0.0f, y + d * H, ld);
+    // an initial state enters the first processed step as one more product added to that step's input projection
+    // (the step kernel then sees no previous step, as with a zero state)
+    if (hx) lh_sgemm(0, 1, B, H, H, 1.0f, hx + (size_t)d * B * H, H, Wih + (size_t)H * I, H, 1.0f, y + (size_t)(d == 0 ? 0 : T - 1) * B * ld + d * H, ld);
   }
   ProfScope prof_(CAT_RNN);
   for (int step = 0; step < T; step++) {
@@ -367,8 +378,8 @@ void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B
   LH_CHECK_LAUNCH();
 }
 
-void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
-                int T, int B, int I, int H, int bidir) {
+void lh_rnn_bwd_init(int mode, const float* x, const float* hx, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
+                     int T, int B, int I, int H, int bidir) {
   LH_REQUIRE(mode == 0 || mode == 1, "lh_rnn_bwd: mode %d (0 = relu, 1 = tanh)", mode);
   LH_REQUIRE(T >= 1 && B >= 1 && I >= 1 && H >= 1, "lh_rnn_bwd: bad shape T%d B%d I%d H%d", T, B, I, H);
   LH_REQUIRE(H <= 2048, "lh_rnn_bwd: hidden size %d above %d", H, 2048);
@@ -414,6 +425,8 @@ void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
       const float* Bm = d == 0 ? y + d * H : y + (size_t)B * ld + d * H;
       lh_sgemm(1, 0, H, H, (T - 1) * B, 1.0f, A, ld, Bm, ld, 1.0f, dWhh, H);
     }
+    // the first processed step's pair is (dpre of that step, the initial state)
+    if (hx) lh_sgemm(1, 0, H, H, B, 1.0f, dpre + (size_t)(d == 0 ? 0 : T - 1) * B * ld + d * H, ld, hx + (size_t)d * B * H, H, 1.0f, dWhh, H);
     hipLaunchKernelGGL(k_rnn_bias_grad, dim3((unsigned)cdiv(H, TPB)), dim3(TPB), 0, g_stream, colsum + d * H, dbih, dbhh, H);
     if (dx) lh_sgemm(0, 0, T * B, I, H, 1.0f, dpre + d * H, ld, Wih, I, d == 0 ? beta_dx : 1.0f, dx, I);
   }

@@ -2,7 +2,7 @@
 // cudnnRNNForwardTraining / BackwardData / BackwardWeights, src/main/scala/lantern/TensorDslCudnn.scala:1638-1893).
 //
 // Gate order and formulas are cuDNN's: LSTM i, f, g, o with c' = f*c + i*g, h' = o*tanh(c'); GRU r, z, n with
-// n = tanh(W_in x + b_in + r*(W_hn h + b_hn)), h' = (1 - z)*n + z*h.  One layer, zero initial state, optionally
+// n = tanh(W_in x + b_in + r*(W_hn h + b_hn)), h' = (1 - z)*n + z*h.  One layer, optional initial state (values only, no gradient), optionally
 // bidirectional (y = forward half, then reverse half).  Parameters per direction: W_ih[G, I], W_hh[G, H], b_ih[G],
 // b_hh[G] with G = 4H or 3H (NNModule.scala:378-390).
 //
@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(TPB) k_lstm_bwd_point(float* __restrict__ act,
 
 // act [B, 3H]: input projection on entry, r, z, n on exit.  gh [B, 3H] = h_prev W_hh^T or null.  q [B, H] = W_hn h + b_hn.
 __global__ void __launch_bounds__(TPB) k_gru_fwd_point(float* __restrict__ act, const float* __restrict__ gh, const float* __restrict__ b_ih,
-                                                       const float* __restrict__ b_hh, const float* __restrict__ h_prev, float* __restrict__ q,
+                                                       const float* __restrict__ b_hh, const float* __restrict__ h_prev, int ldp, float* __restrict__ q,
                                                        float* __restrict__ h, int B, int H, int ldh) {
   const int idx = blockIdx.x * TPB + threadIdx.x;
   if (idx >= B * H) return;
@@ -72,7 +72,7 @@ __global__ void __launch_bounds__(TPB) k_gru_fwd_point(float* __restrict__ act, 
   const float z = sigm(a[H] + b_ih[H + j] + b_hh[H + j] + (g ? g[H] : 0.f));
   const float qq = (g ? g[2 * H] : 0.f) + b_hh[2 * H + j];
   const float n = tanhf(a[2 * H] + b_ih[2 * H + j] + r * qq);
-  const float hp = h_prev ? h_prev[(size_t)b * ldh + j] : 0.f;
+  const float hp = h_prev ? h_prev[(size_t)b * ldp + j] : 0.f;      // ldp: row stride of h_prev (an initial state is [B, H])
   a[0] = r; a[H] = z; a[2 * H] = n;
   q[idx] = qq;
   h[(size_t)b * ldh + j] = (1.f - z) * n + z * hp;
@@ -82,7 +82,7 @@ __global__ void __launch_bounds__(TPB) k_gru_fwd_point(float* __restrict__ act, 
 // hidden side (the n column scaled by r).  carry [B, H]: the recurrent gradient on entry (ignored when first), dh * z on
 // exit; the caller adds dgh W_hh to it.
 __global__ void __launch_bounds__(TPB) k_gru_bwd_point(float* __restrict__ act, float* __restrict__ dgh, const float* __restrict__ q,
-                                                       const float* __restrict__ h_prev, const float* __restrict__ dy, float* __restrict__ carry,
+                                                       const float* __restrict__ h_prev, int ldp, const float* __restrict__ dy, float* __restrict__ carry,
                                                        int first, int B, int H, int ldh) {
   const int idx = blockIdx.x * TPB + threadIdx.x;
   if (idx >= B * H) return;
@@ -91,7 +91,7 @@ __global__ void __launch_bounds__(TPB) k_gru_bwd_point(float* __restrict__ act, 
   float* g = dgh + (size_t)b * 3 * H + j;
   const float r = a[0], z = a[H], n = a[2 * H];
   const float dh = dy[(size_t)b * ldh + j] + (first ? 0.f : carry[idx]);
-  const float hp = h_prev ? h_prev[(size_t)b * ldh + j] : 0.f;
+  const float hp = h_prev ? h_prev[(size_t)b * ldp + j] : 0.f;
   const float dn = dh * (1.f - z) * (1.f - n * n);
   const float dz = dh * (hp - n) * z * (1.f - z);
   const float dr = dn * q[idx] * r * (1.f - r);
@@ -127,7 +127,17 @@ int64_t lh_rnn_gated_reserve_floats(int mode, int T, int B, int H, int bidir) {
 }
 
 void lh_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, float* reserve, int T, int B, int I, int H, int bidir) {
+  lh_rnn_gated_fwd_init(mode, x, nullptr, nullptr, w, y, reserve, T, B, I, H, bidir);
+}
+void lh_rnn_gated_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* reserve, float* dx, float beta_dx,
+                      float* dw, int T, int B, int I, int H, int bidir) {
+  lh_rnn_gated_bwd_init(mode, x, nullptr, nullptr, y, dy, w, reserve, dx, beta_dx, dw, T, B, I, H, bidir);
+}
+
+void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const float* cx, const float* w, float* y, float* reserve,
+                           int T, int B, int I, int H, int bidir) {
   if (!check_shape("lh_rnn_gated_fwd", mode, T, B, I, H)) return;
+  LH_REQUIRE(cx == nullptr || mode == 2, "lh_rnn_gated_fwd: only the LSTM has a cell state");
   LH_REQUIRE(x && w && y && reserve, "lh_rnn_gated_fwd: null operand");
   const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
   const size_t gh_bytes = (size_t)B * G * sizeof(float);
@@ -142,14 +152,17 @@ void lh_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, float*
     for (int step = 0; step < T; step++) {
       const int t = d == 0 ? step : T - 1 - step, tp = d == 0 ? t - 1 : t + 1;
       float* h = y + (size_t)t * B * ldh + d * H;
-      const float* hp = step == 0 ? nullptr : y + (size_t)tp * B * ldh + d * H;
-      if (hp) lh_sgemm(0, 1, B, G, H, 1.0f, hp, ldh, Whh, H, 0.0f, gh, G);
+      // previous state: the step processed before, or the caller's initial state ([B, H] rows), or none (zeros)
+      const float* hp = step == 0 ? (hx ? hx + (size_t)d * B * H : nullptr) : y + (size_t)tp * B * ldh + d * H;
+      const int ldp = step == 0 ? H : ldh;
+      const float* cp = step == 0 ? (cx ? cx + (size_t)d * B * H : nullptr) : aux + (size_t)tp * B * H;
+      if (hp) lh_sgemm(0, 1, B, G, H, 1.0f, hp, ldp, Whh, H, 0.0f, gh, G);
       float* a = act + (size_t)t * B * G;
       if (mode == 2)
         hipLaunchKernelGGL(k_lstm_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh,
-                           hp ? aux + (size_t)tp * B * H : nullptr, aux + (size_t)t * B * H, h, B, H, ldh);
+                           cp, aux + (size_t)t * B * H, h, B, H, ldh);
       else
-        hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh, hp,
+        hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh, hp, ldp,
                            aux + (size_t)t * B * H, h, B, H, ldh);
     }
   }
@@ -157,9 +170,10 @@ void lh_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, float*
   LH_CHECK_LAUNCH();
 }
 
-void lh_rnn_gated_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* reserve, float* dx, float beta_dx,
-                      float* dw, int T, int B, int I, int H, int bidir) {
+void lh_rnn_gated_bwd_init(int mode, const float* x, const float* hx, const float* cx, const float* y, const float* dy, const float* w,
+                           float* reserve, float* dx, float beta_dx, float* dw, int T, int B, int I, int H, int bidir) {
   if (!check_shape("lh_rnn_gated_bwd", mode, T, B, I, H)) return;
+  LH_REQUIRE(cx == nullptr || mode == 2, "lh_rnn_gated_bwd: only the LSTM has a cell state");
   LH_REQUIRE(beta_dx == 0.f || beta_dx == 1.f, "lh_rnn_gated_bwd: beta must be 0 or 1");
   LH_REQUIRE(x && y && dy && w && reserve && dw, "lh_rnn_gated_bwd: null operand");
   const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
@@ -180,16 +194,18 @@ void lh_rnn_gated_bwd(int mode, const float* x, const float* y, const float* dy,
       const int t = d == 0 ? T - 1 - k : k;                        // reverse of the forward processing order
       const int tp = d == 0 ? t - 1 : t + 1;                       // the step whose state this one consumed
       const bool has_prev = d == 0 ? t > 0 : t < T - 1;
+      const float* h0 = hx ? hx + (size_t)d * B * H : nullptr;      // read only by the step the forward pass processed first
+      const float* c0 = cx ? cx + (size_t)d * B * H : nullptr;
       float* a = act + (size_t)t * B * G;
       const float* dyt = dy + (size_t)t * B * ldh + d * H;
       if (mode == 2) {
         hipLaunchKernelGGL(k_lstm_bwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, aux + (size_t)t * B * H,
-                           has_prev ? aux + (size_t)tp * B * H : nullptr, dyt, k == 0 ? nullptr : carry, dc, k == 0 ? 1 : 0, B, H, ldh);
+                           has_prev ? aux + (size_t)tp * B * H : c0, dyt, k == 0 ? nullptr : carry, dc, k == 0 ? 1 : 0, B, H, ldh);
         if (has_prev) lh_sgemm(0, 0, B, H, G, 1.0f, a, G, Whh, H, 0.0f, carry, H);
       } else {
         float* g = dgh + (size_t)t * B * G;
         hipLaunchKernelGGL(k_gru_bwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, g, aux + (size_t)t * B * H,
-                           has_prev ? y + (size_t)tp * B * ldh + d * H : nullptr, dyt, carry, k == 0 ? 1 : 0, B, H, ldh);
+                           has_prev ? y + (size_t)tp * B * ldh + d * H : h0, has_prev ? ldh : H, dyt, carry, k == 0 ? 1 : 0, B, H, ldh);
         if (has_prev) lh_sgemm(0, 0, B, H, G, 1.0f, g, G, Whh, H, 1.0f, carry, H);
       }
     }
@@ -201,6 +217,8 @@ void lh_rnn_gated_bwd(int mode, const float* x, const float* y, const float* dy,
       const float* Bm = d == 0 ? y + d * H : y + (size_t)B * ldh + d * H;
       lh_sgemm(1, 0, G, H, (T - 1) * B, 1.0f, A, G, Bm, ldh, 1.0f, dWhh, H);
     }
+    // the first processed step's pair is (its hidden-side gradients, the initial state)
+    if (hx) lh_sgemm(1, 0, G, H, B, 1.0f, hid + (size_t)(d == 0 ? 0 : T - 1) * B * G, G, hx + (size_t)d * B * H, H, 1.0f, dWhh, H);
     lh_sum_dim(act, colsum, 1, T * B, G);
     hipLaunchKernelGGL(k_add_into, dim3((unsigned)cdiv(G, TPB)), dim3(TPB), 0, g_stream, dbih, colsum, G);
     if (mode == 3) lh_sum_dim(dgh, colsum + G, 1, T * B, G);

@@ -107,7 +107,10 @@ class RNNBase(Module):
     b_ih, b_hh (forward direction first), initialised with Tensor.rand(size, 0.01).  Modes "relu", "tanh", "lstm", "gru"
     (1, 1, 4 and 3 gates of hiddenSize rows each).  Layers after the first read the previous layer's output, which is
     numDirections * hiddenSize wide (what cuDNN expects; the reference's size formula, NN:357, leaves the factor out and
-    so only works for one direction).  Zero initial state; no dropout between layers."""
+    so only works for one direction).  `apply(input, hx, cx)`: optional initial hidden / cell states
+    [numLayers * numDirections, batch, hidden] (TensorR or Tensor; values only, no gradient: CDN:1843-1844 pass NULL for
+    dhx / dcx).  `dropout`: applied to the output of every layer but the last, as cuDNN does, with the backend's own
+    dropout operator (cuDNN's generator is its own; the masks are not comparable, their statistics are)."""
     MODES = {"relu": (0, 1), "tanh": (1, 1), "lstm": (2, 4), "gru": (3, 3)}
 
     def __init__(self, mode, inputSize, hiddenSize, numLayers=1, dropout=0.0, bidirectional=False, name="rnn"):
@@ -116,7 +119,8 @@ class RNNBase(Module):
         assert inputSize >= 1, "Input size must be at least 1"
         assert hiddenSize >= 1, "Hidden size must be at least 1"
         assert numLayers >= 1, "Number of layers must be at least 1"
-        assert dropout == 0.0, "dropout between layers is not built"
+        assert 0.0 <= dropout <= 1.0, "Dropout must be between 0 and 1"
+        self.dropout = float(dropout)
         self.mode, self.numGates = self.MODES[mode]
         self.inputSize, self.hiddenSize, self.numLayers, self.bidirectional = inputSize, hiddenSize, numLayers, bidirectional
         self.numDirections = 2 if bidirectional else 1
@@ -136,9 +140,22 @@ class RNNBase(Module):
     def getParameterSize(self):
         return self.parameterBuffer.x.scalarCount
 
-    def __call__(self, x):
+    def __call__(self, x, hx=None, cx=None):
+        assert x.x.rank == 3, "RNN input should have rank 3: [seqLength x batchSize x inputSize]"
+        D, Bn, H = self.numDirections, x.x.shape[1], self.hiddenSize
+        states = []
+        for name, s in (("hidden", hx), ("cell", cx)):
+            t = s.x if isinstance(s, TensorR) else s
+            if t is not None:
+                assert t.rank == 3, "RNN %s state should have rank 3: [numLayers * numDirections x batchSize x hiddenSize]" % name
+                assert t.shape[1] == Bn, "RNN %s state second dimension should equal input second dimension (batch size)" % name
+                assert t.shape[0] == self.numLayers * D and t.shape[2] == H, "RNN %s state should be [%d, %d, %d]" % (name, self.numLayers * D, Bn, H)
+            states.append(t)
         for layer in range(self.numLayers):
-            x = x.rnn(self.mode, self.parameterBuffer, self.hiddenSize, self.bidirectional, offset=self.offsets[layer])
+            h0, c0 = [None if t is None else t.data.offset(layer * D * Bn * H) if layer else t.data for t in states]
+            x = x.rnn(self.mode, self.parameterBuffer, self.hiddenSize, self.bidirectional, offset=self.offsets[layer], hx=h0, cx=c0)
+            if self.dropout > 0.0 and layer + 1 < self.numLayers:
+                x = x.dropout(self.dropout)
         return x
 
 

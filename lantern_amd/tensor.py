@@ -818,26 +818,28 @@ class TensorR:
         return y
 
     # -- recurrent layer, CTC ----------------------------------------------------------------------------
-    def rnn(self, mode, params, hidden, bidirectional, offset=0):
-        """RNNBase.apply (NN:392-415): one layer over [seqLength, batch, inputSize], zero initial state;
+    def rnn(self, mode, params, hidden, bidirectional, offset=0, hx=None, cx=None):
+        """RNNBase.apply (NN:392-415): one layer over [seqLength, batch, inputSize];
         `params` is the packed parameter buffer (a TensorR), this layer's parameters starting `offset` elements in.
-        mode 0 = relu, 1 = tanh, 2 = LSTM, 3 = GRU (cuDNN's numbering)."""
+        mode 0 = relu, 1 = tanh, 2 = LSTM, 3 = GRU (cuDNN's numbering).  `hx`, `cx`: this layer's initial hidden and cell
+        state as plain data [numDirections, batch, hidden] (None = zeros); they receive no gradient (CDN:1843-1844 pass NULL)."""
         be = get_backend()
         assert self.x.rank == 3, "RNN input should have rank 3: [seqLength x batchSize x inputSize]"
         T, Bn, I = self.x.shape
         D = 2 if bidirectional else 1
         w, dw = (params.x.data, params.d.data) if offset == 0 else (params.x.data.offset(offset), params.d.data.offset(offset))
+        assert cx is None or mode == 2, "only the LSTM has a cell state"
         if mode >= 2:
-            ybuf, reserve = be.rnn_gated_forward(mode, self.x.data, w, T, Bn, I, hidden, bidirectional)
+            ybuf, reserve = be.rnn_gated_forward(mode, self.x.data, w, T, Bn, I, hidden, bidirectional, hx=hx, cx=cx)
         else:
-            ybuf = be.rnn_forward(mode, self.x.data, w, T, Bn, I, hidden, bidirectional)
+            ybuf = be.rnn_forward(mode, self.x.data, w, T, Bn, I, hidden, bidirectional, hx=hx)
         y = TensorR._new(Tensor(ybuf, (T, Bn, D * hidden)))
         def back():
             xd, beta = (None, 1.0) if self.isInput else self.grad_target()
             if mode >= 2:
-                be.rnn_gated_backward(mode, self.x.data, ybuf, y.d.data, w, reserve, xd, dw, T, Bn, I, hidden, bidirectional, beta)
+                be.rnn_gated_backward(mode, self.x.data, ybuf, y.d.data, w, reserve, xd, dw, T, Bn, I, hidden, bidirectional, beta, hx=hx, cx=cx)
             else:
-                be.rnn_backward(mode, self.x.data, ybuf, y.d.data, w, xd, dw, T, Bn, I, hidden, bidirectional, beta)
+                be.rnn_backward(mode, self.x.data, ybuf, y.d.data, w, xd, dw, T, Bn, I, hidden, bidirectional, beta, hx=hx)
         _tape.append(back)
         return y
 

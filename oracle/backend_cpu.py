@@ -276,14 +276,14 @@ class BackendCPU(Backend):
                 P(costs.ptr), I(T), I(B), I(A))
         return costs
 
-    def rnn_forward(self, mode, x, w, T, B, I_, H, bidir):
+    def rnn_forward(self, mode, x, w, T, B, I_, H, bidir, hx=None):
         y = self.mallocArray(T * B * H * (2 if bidir else 1))
-        self._c("lc_rnn_fwd", I(mode), P(x.ptr), P(w.ptr), P(y.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))
+        self._c("lc_rnn_fwd_init", I(mode), P(x.ptr), P(hx.ptr if hx is not None else 0), P(w.ptr), P(y.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))
         return y
 
-    def rnn_backward(self, mode, x, y, dy, w, dx, dw, T, B, I_, H, bidir, beta_dx=1.0):
-        self._c("lc_rnn_bwd", I(mode), P(x.ptr), P(y.ptr), P(dy.ptr), P(w.ptr), P(dx.ptr if dx is not None else 0), P(dw.ptr),
-                I(T), I(B), I(I_), I(H), I(int(bidir)))
+    def rnn_backward(self, mode, x, y, dy, w, dx, dw, T, B, I_, H, bidir, beta_dx=1.0, hx=None):
+        self._c("lc_rnn_bwd_init", I(mode), P(x.ptr), P(hx.ptr if hx is not None else 0), P(y.ptr), P(dy.ptr), P(w.ptr), P(dx.ptr if dx is not None else 0),
+                P(dw.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))
 
     def repeat0(self, x, rows, context, inner):
         y = self.mallocArray((rows - context) * (context + 1) * inner)
@@ -293,14 +293,15 @@ class BackendCPU(Backend):
     def repeat0_grad(self, xd, yd, rows, context, inner):
         self._c("lc_repeat0_grad", P(xd.ptr), P(yd.ptr), I(rows), I(context), L(inner))
 
-    def rnn_gated_forward(self, mode, x, w, T, B, I_, H, bidir):
+    def rnn_gated_forward(self, mode, x, w, T, B, I_, H, bidir, hx=None, cx=None):
         y = self.mallocArray(T * B * H * (2 if bidir else 1))
-        self._c("lc_rnn_gated_fwd", I(mode), P(x.ptr), P(w.ptr), P(y.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))
+        self._c("lc_rnn_gated_fwd_init", I(mode), P(x.ptr), P(hx.ptr if hx is not None else 0), P(cx.ptr if cx is not None else 0), P(w.ptr), P(y.ptr),
+                I(T), I(B), I(I_), I(H), I(int(bidir)))
         return y, None
 
-    def rnn_gated_backward(self, mode, x, y, dy, w, reserve, dx, dw, T, B, I_, H, bidir, beta_dx=1.0):
-        self._c("lc_rnn_gated_bwd", I(mode), P(x.ptr), P(dy.ptr), P(w.ptr), P(dx.ptr if dx is not None else 0), P(dw.ptr),
-                I(T), I(B), I(I_), I(H), I(int(bidir)))
+    def rnn_gated_backward(self, mode, x, y, dy, w, reserve, dx, dw, T, B, I_, H, bidir, beta_dx=1.0, hx=None, cx=None):
+        self._c("lc_rnn_gated_bwd_init", I(mode), P(x.ptr), P(hx.ptr if hx is not None else 0), P(cx.ptr if cx is not None else 0), P(dy.ptr), P(w.ptr),
+                P(dx.ptr if dx is not None else 0), P(dw.ptr), I(T), I(B), I(I_), I(H), I(int(bidir)))
 
     def sgd_update(self, x, d, lr, n): self._c("lc_sgd", P(x.ptr), P(d.ptr), F(lr), L(n))
     def adagrad_update(self, x, d, m, lr, clip, n): self._c("lc_adagrad", P(x.ptr), P(d.ptr), P(m.ptr), F(lr), F(clip), L(n))

@@ -754,7 +754,9 @@ void lc_ctc_loss(const float* probs, float* dprobs, const int* labels, const int
  * direction first.  Checked against torch.nn.RNN in the tests. */
 static size_t rnn_dir_params(int I, int H) { return (size_t)H * I + (size_t)H * H + 2 * (size_t)H; }
 
-void lc_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+/* hx (may be NULL = zeros): initial hidden state [D, B, H], the `hx` of RNNBase.apply (NN:392) as cudnnRNNForwardTraining takes
+ * it (CDN:1796); it receives no gradient (dhx is NULL at CDN:1843-1844). */
+void lc_rnn_fwd_init(int mode, const float* x, const float* hx, const float* w, float* y, int T, int B, int I, int H, int bidir) {
   const int D = bidir ? 2 : 1, DH = D * H;
   float* pre = (float*)malloc((size_t)T * B * H * sizeof(float));
   float* hprev = (float*)calloc((size_t)B * H, sizeof(float));
@@ -764,7 +766,8 @@ void lc_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B
     const float* bih = Whh + (size_t)H * H; const float* bhh = bih + H;
     /* input projection for all steps: pre[T*B, H] = x[T*B, I] * Wih^T */
     lc_sgemm(0, 1, T * B, H, I, 1.0f, x, I, Wih, I, 0.0f, pre, H);
-    memset(hprev, 0, (size_t)B * H * sizeof(float));
+    if (hx) memcpy(hprev, hx + (size_t)d * B * H, (size_t)B * H * sizeof(float));
+    else memset(hprev, 0, (size_t)B * H * sizeof(float));
     for (int step = 0; step < T; step++) {
       const int t = d == 0 ? step : T - 1 - step;
       lc_sgemm(0, 1, B, H, H, 1.0f, hprev, H, Whh, H, 0.0f, rec, H);
@@ -778,10 +781,13 @@ void lc_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B
   }
   free(pre); free(hprev); free(rec);
 }
+void lc_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+  lc_rnn_fwd_init(mode, x, NULL, w, y, T, B, I, H, bidir);
+}
 
 /* dx (may be NULL) and dw accumulate. */
-void lc_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float* dw,
-                int T, int B, int I, int H, int bidir) {
+void lc_rnn_bwd_init(int mode, const float* x, const float* hx, const float* y, const float* dy, const float* w, float* dx, float* dw,
+                     int T, int B, int I, int H, int bidir) {
   const int D = bidir ? 2 : 1, DH = D * H;
   float* dpre = (float*)malloc((size_t)T * B * H * sizeof(float));
   float* hs = (float*)malloc((size_t)T * B * H * sizeof(float));      /* h_{t-1} for every step, in time order */
@@ -799,7 +805,7 @@ void lc_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
           const float h = y[((size_t)t * B + b) * DH + d * H + j];
           const float g = dy[((size_t)t * B + b) * DH + d * H + j] + dh[(size_t)b * H + j];
           dpre[((size_t)t * B + b) * H + j] = mode == 1 ? g * (1.0f - h * h) : (h > 0.f ? g : 0.f);
-          hs[((size_t)t * B + b) * H + j] = step == 0 ? 0.f : y[((size_t)tp * B + b) * DH + d * H + j];
+          hs[((size_t)t * B + b) * H + j] = step == 0 ? (hx ? hx[((size_t)d * B + b) * H + j] : 0.f) : y[((size_t)tp * B + b) * DH + d * H + j];
         }
       /* dh_{prev}[B,H] = dpre_t[B,H] * Whh[H,H] */
       lc_sgemm(0, 0, B, H, H, 1.0f, dpre + (size_t)t * B * H, H, Whh, H, 0.0f, dh, H);
@@ -814,6 +820,10 @@ void lc_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const
     if (dx) lc_sgemm(0, 0, T * B, I, H, 1.0f, dpre, H, Wih, I, 1.0f, dx, I);
   }
   free(dpre); free(hs); free(dh);
+}
+void lc_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float* dw,
+                int T, int B, int I, int H, int bidir) {
+  lc_rnn_bwd_init(mode, x, NULL, y, dy, w, dx, dw, T, B, I, H, bidir);
 }
 
 /* ---------------------------------------------------------- LSTM and GRU
@@ -831,10 +841,11 @@ static double sigm_d(double v) { return 1.0 / (1.0 + exp(-v)); }
 /* One direction of one sample, forward; fills (when not NULL) per-step records for the backward pass:
  * gate[T][G] activations, cell[T][H] (LSTM: c_t; GRU: q_t = R_n h + b_hn), hid[T][H] = h_t. */
 static void gated_forward_sample(int mode, const float* x, size_t xs, const float* Wih, const float* Whh, const float* bih, const float* bhh,
-                                 int T, int I, int H, int reverse, double* gate, double* cell, double* hid) {
+                                 int T, int I, int H, int reverse, double* gate, double* cell, double* hid, const float* h0, const float* c0) {
   const int ng = gated_ng(mode), G = ng * H;
   double* h = (double*)calloc((size_t)H, sizeof(double));
   double* c = (double*)calloc((size_t)H, sizeof(double));
+  for (int j = 0; j < H; j++) { if (h0) h[j] = h0[j]; if (c0) c[j] = c0[j]; }    /* initial state of this sample and direction */
   double* px = (double*)malloc((size_t)G * sizeof(double));
   double* ph = (double*)malloc((size_t)G * sizeof(double));
   for (int step = 0; step < T; step++) {
@@ -868,7 +879,8 @@ static void gated_forward_sample(int mode, const float* x, size_t xs, const floa
   free(h); free(c); free(px); free(ph);
 }
 
-void lc_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+/* hx, cx (each may be NULL = zeros): initial hidden and cell state [D, B, H] (cx: LSTM only); no gradient flows to them. */
+void lc_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const float* cx, const float* w, float* y, int T, int B, int I, int H, int bidir) {
   const int D = bidir ? 2 : 1, G = gated_ng(mode) * H;
   double* gate = (double*)malloc((size_t)T * G * sizeof(double));
   double* cell = (double*)malloc((size_t)T * H * sizeof(double));
@@ -877,16 +889,21 @@ void lc_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, int T,
     const float* Wih = w + d * gated_dir_params(mode, I, H); const float* Whh = Wih + (size_t)G * I;
     const float* bih = Whh + (size_t)G * H; const float* bhh = bih + G;
     for (int b = 0; b < B; b++) {
-      gated_forward_sample(mode, x + (size_t)b * I, (size_t)B * I, Wih, Whh, bih, bhh, T, I, H, d, gate, cell, hid);
+      gated_forward_sample(mode, x + (size_t)b * I, (size_t)B * I, Wih, Whh, bih, bhh, T, I, H, d, gate, cell, hid,
+                           hx ? hx + ((size_t)d * B + b) * H : NULL, cx ? cx + ((size_t)d * B + b) * H : NULL);
       for (int t = 0; t < T; t++)
         for (int j = 0; j < H; j++) y[((size_t)t * B + b) * D * H + (size_t)d * H + j] = (float)hid[(size_t)t * H + j];
     }
   }
   free(gate); free(cell); free(hid);
 }
+void lc_rnn_gated_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir) {
+  lc_rnn_gated_fwd_init(mode, x, NULL, NULL, w, y, T, B, I, H, bidir);
+}
 
 /* dx (may be NULL) and dw accumulate. */
-void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w, float* dx, float* dw, int T, int B, int I, int H, int bidir) {
+void lc_rnn_gated_bwd_init(int mode, const float* x, const float* hx, const float* cx, const float* dy, const float* w, float* dx, float* dw,
+                           int T, int B, int I, int H, int bidir) {
   const int D = bidir ? 2 : 1, ng = gated_ng(mode), G = ng * H;
   double* gate = (double*)malloc((size_t)T * G * sizeof(double));
   double* cell = (double*)malloc((size_t)T * H * sizeof(double));
@@ -895,6 +912,7 @@ void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w,
   double* dc = (double*)malloc((size_t)H * sizeof(double));
   double* gx = (double*)malloc((size_t)G * sizeof(double));       /* gradient of the input-side pre-activations */
   double* gh = (double*)malloc((size_t)G * sizeof(double));       /* ... of the hidden-side ones */
+  double* h0d = (double*)malloc((size_t)H * sizeof(double));      /* the initial hidden state of the current sample */
   const size_t np = gated_dir_params(mode, I, H);
   double* acc = (double*)calloc(np, sizeof(double));
   for (int d = 0; d < D; d++) {
@@ -903,19 +921,22 @@ void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w,
     double* aWih = acc; double* aWhh = aWih + (size_t)G * I; double* abih = aWhh + (size_t)G * H; double* abhh = abih + G;
     memset(acc, 0, np * sizeof(double));
     for (int b = 0; b < B; b++) {
-      gated_forward_sample(mode, x + (size_t)b * I, (size_t)B * I, Wih, Whh, bih, bhh, T, I, H, d, gate, cell, hid);
+      const float* h0 = hx ? hx + ((size_t)d * B + b) * H : NULL;
+      const float* c0 = cx ? cx + ((size_t)d * B + b) * H : NULL;
+      gated_forward_sample(mode, x + (size_t)b * I, (size_t)B * I, Wih, Whh, bih, bhh, T, I, H, d, gate, cell, hid, h0, c0);
       for (int j = 0; j < H; j++) dh[j] = dc[j] = 0.0;
       for (int step = T - 1; step >= 0; step--) {
         const int t = d ? T - 1 - step : step;
         const int tp = d ? t + 1 : t - 1;
         const double* gt = gate + (size_t)t * G;
         const double* hp = step == 0 ? NULL : hid + (size_t)tp * H;
+        if (step == 0 && h0) { for (int j = 0; j < H; j++) h0d[j] = h0[j]; hp = h0d; }
         for (int j = 0; j < H; j++) {
           const double g = dh[j] + dy[((size_t)t * B + b) * D * H + (size_t)d * H + j];
           if (mode == 2) {
             const double ig = gt[j], fg = gt[H + j], gg = gt[2 * H + j], og = gt[3 * H + j];
             const double tc = tanh(cell[(size_t)t * H + j]);
-            const double cp = step == 0 ? 0.0 : cell[(size_t)tp * H + j];
+            const double cp = step == 0 ? (c0 ? (double)c0[j] : 0.0) : cell[(size_t)tp * H + j];
             const double dcell = dc[j] + g * og * (1.0 - tc * tc);
             gx[j] = dcell * gg * ig * (1.0 - ig);
             gx[H + j] = dcell * cp * fg * (1.0 - fg);
@@ -950,7 +971,10 @@ void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w,
     }
     for (size_t i = 0; i < np; i++) dw[off + i] += (float)acc[i];
   }
-  free(gate); free(cell); free(hid); free(dh); free(dc); free(gx); free(gh); free(acc);
+  free(gate); free(cell); free(hid); free(dh); free(dc); free(gx); free(gh); free(acc); free(h0d);
+}
+void lc_rnn_gated_bwd(int mode, const float* x, const float* dy, const float* w, float* dx, float* dw, int T, int B, int I, int H, int bidir) {
+  lc_rnn_gated_bwd_init(mode, x, NULL, NULL, dy, w, dx, dw, T, B, I, H, bidir);
 }
 
 /* ------------------------------------------ average pooling with padding

@@ -595,30 +595,69 @@ trait TensorDslHIP extends TensorDslCPU with GPUOps {
 
     // ---- recurrent layers (CDN:1638-1893; called by RNNBase, NNModule.scala:392-416).  One layer, zero initial states, no dropout;
     //      RNNBase stacks layers itself when numLayers > 1.  The weight buffer has cuDNN's layout (NNModule.scala:378-390) -----------
+    // One library call per layer (the library's layer = cuDNN's with numLayers = 1); a stack is a loop at staging time over the
+    // packed parameter buffer (per layer: forward direction W_ih, W_hh, b_ih, b_hh, then the reverse direction; NN:378-390),
+    // with the backend's dropout between layers (cuDNN applies its own to every layer's output but the last) and the initial
+    // states cut per layer ([numLayers * numDirections, batch, hidden], CDN:1823).  What the backward pass needs of the
+    // layers in between is kept here at staging time under the call's counter.
+    case class RnnLayerRecord(input: TensorR, output: TensorR, reserve: Rep[Array[Float]], mask: Option[Rep[Array[Float]]], wOffset: Int)
+    val rnnRecords = scala.collection.mutable.HashMap[Int, Seq[RnnLayerRecord]]()
+    var rnnCounter = 0
     def rnnForwardTraining(mode: RnnMode, x: Tensor, hx: Option[Tensor] = None, cx: Option[Tensor] = None, w: Tensor, numLayers: Int, hiddenSize: Int,
                            dropout: Float = 0f, bidirectional: Boolean = false): (Tensor, Option[Tensor], Rep[Array[Float]], Rep[Int], Int) = {
       assert(x.rank == 3, "RNN input should have rank 3: [seqLength x batchSize x inputSize]")
-      assert(numLayers == 1 && hx.isEmpty && cx.isEmpty && dropout == 0.0f, "lh_rnn_fwd: one layer per call, zero initial state, no dropout")
-      val (t, b, i) = (x.shape(0), x.shape(1), x.shape(2)); val d = if (bidirectional) 2 else 1
-      val res = Tensor(mallocArray[Float](t * b * d * hiddenSize), t, b, d * hiddenSize)
-      if (mode == LstmMode || mode == GruMode) {                 // the gate activations of every step go to a reserve, as with cuDNN
-        val reserveSize = t * b * (mode.numGates + 1) * hiddenSize * d                  // = lh_rnn_gated_reserve_floats(mode, T, B, H, bidirectional)
-        val reserve = mallocArray[Float](reserveSize)
-        hip("lh_rnn_gated_fwd", mode.id, x.data, w.data, res.data, reserve, t, b, i, hiddenSize, bidirectional)
-        (res, None, reserve, reserveSize, 0)
-      } else {                                                    // the output doubles as the saved hidden states: no reserve space
-        hip("lh_rnn_fwd", mode.id, x.data, w.data, res.data, t, b, i, hiddenSize, bidirectional)
-        (res, None, unchecked[Array[Float]]("(float*)0"), unit(0), 0)
+      assert(cx.isEmpty || mode == LstmMode, "only the LSTM has a cell state")
+      val (t, b) = (x.shape(0), x.shape(1)); val d = if (bidirectional) 2 else 1
+      val gated = mode == LstmMode || mode == GruMode
+      val gateSize = mode.numGates * hiddenSize
+      val records = scala.collection.mutable.ArrayBuffer[RnnLayerRecord]()
+      var layerIn = new TensorR(x, x)                             // the first layer's gradient target is the caller's (rnnBackward)
+      var wOffset = 0
+      for (layer <- 0 until numLayers) {
+        val i = layerIn.x.shape(2)
+        val res = Tensor(mallocArray[Float](t * b * d * hiddenSize), t, b, d * hiddenSize)
+        val stateOffset = layer * d * b * hiddenSize
+        val h0: Any = hx.map(h => slice(h.data, stateOffset): Any).getOrElse(nullFloats)
+        val c0: Any = cx.map(c => slice(c.data, stateOffset): Any).getOrElse(nullFloats)
+        val wl = slice(w.data, wOffset)
+        val reserve = if (gated) mallocArray[Float](t * b * (mode.numGates + 1) * hiddenSize * d) else unchecked[Array[Float]]("(float*)0")
+        if (gated) hip("lh_rnn_gated_fwd_init", mode.id, layerIn.x.data, h0, c0, wl, res.data, reserve, t, b, i, hiddenSize, bidirectional)
+        else hip("lh_rnn_fwd_init", mode.id, layerIn.x.data, h0, wl, res.data, t, b, i, hiddenSize, bidirectional)
+        val out = TensorR(res)
+        val last = layer == numLayers - 1
+        val (next, mask) = if (dropout > 0f && !last) { val (y, m, _) = this.dropout(res, dropout); (TensorR(y), Some(m)) } else (out, None)
+        records += RnnLayerRecord(layerIn, out, reserve, mask, wOffset)
+        if (mask.isDefined) records += RnnLayerRecord(out, next, reserve, mask, -1)          // the dropout between two layers
+        wOffset += d * (gateSize * i + gateSize * hiddenSize + 2 * gateSize)
+        layerIn = next
       }
+      rnnCounter += 1
+      rnnRecords(rnnCounter) = records.toSeq
+      (layerIn.x, None, records.last.reserve, unit(0), rnnCounter)
     }
     def rnnBackward(mode: RnnMode, input: TensorR, hx: Option[Tensor], cx: Option[Tensor], w: TensorR, output: TensorR, numLayers: Int, hiddenSize: Int,
                     dropout: Float = 0f, bidirectional: Boolean = false, reserve: Rep[Array[Float]], reserveSize: Rep[Int], counter: Int): Unit = {
-      val (t, b, i) = (input.x.shape(0), input.x.shape(1), input.x.shape(2))
-      val dx: Any = if (input.isInput) nullFloats else input.d.data           // cudnnRNNBackwardData is skipped for inputs (CDN:1889-1890)
-      if (mode == LstmMode || mode == GruMode)
-        hip("lh_rnn_gated_bwd", mode.id, input.x.data, output.x.data, output.d.data, w.x.data, reserve, dx, 1.0f, w.d.data, t, b, i, hiddenSize, bidirectional)
-      else
-        hip("lh_rnn_bwd", mode.id, input.x.data, output.x.data, output.d.data, w.x.data, dx, 1.0f, w.d.data, t, b, i, hiddenSize, bidirectional)
+      val (t, b) = (input.x.shape(0), input.x.shape(1)); val d = if (bidirectional) 2 else 1
+      val gated = mode == LstmMode || mode == GruMode
+      val records = rnnRecords(counter)
+      var layer = numLayers
+      records.zipWithIndex.reverse.foreach { case (r, idx) =>
+        val outR = if (idx == records.size - 1) output else r.output       // the caller's TensorR carries the gradient of the last layer
+        if (r.wOffset < 0) dropout_grad(r.input, outR, dropout, r.mask.get, r.input.x.scalarCount)
+        else {
+          layer -= 1
+          val inR = if (idx == 0) input else r.input
+          val i = inR.x.shape(2)
+          val stateOffset = layer * d * b * hiddenSize
+          val h0: Any = hx.map(h => slice(h.data, stateOffset): Any).getOrElse(nullFloats)
+          val c0: Any = cx.map(c => slice(c.data, stateOffset): Any).getOrElse(nullFloats)
+          val dx: Any = if (inR.isInput) nullFloats else inR.d.data       // cudnnRNNBackwardData is skipped for inputs (CDN:1889-1890)
+          val (wl, dwl) = (slice(w.x.data, r.wOffset), slice(w.d.data, r.wOffset))
+          if (gated) hip("lh_rnn_gated_bwd_init", mode.id, inR.x.data, h0, c0, outR.x.data, outR.d.data, wl, r.reserve, dx, 1.0f, dwl, t, b, i, hiddenSize, bidirectional)
+          else hip("lh_rnn_bwd_init", mode.id, inR.x.data, h0, outR.x.data, outR.d.data, wl, dx, 1.0f, dwl, t, b, i, hiddenSize, bidirectional)
+        }
+      }
+      rnnRecords -= counter
     }
     // the names RNNBase calls (NNModule.scala:407-416)
     def cudnnRNNForwardTraining(mode: RnnMode, x: Tensor, hx: Option[Tensor] = None, cx: Option[Tensor] = None, w: Tensor, numLayers: Int, hiddenSize: Int,
@@ -677,8 +716,10 @@ trait NNModuleHIP extends NNModule with TensorDslHIP {
   case class SGD(override val module: Module, learning_rate: Float, gradClip: Float = 1.0f, descent: Boolean = true) extends Optim {
     def step_func = { case (tr, _) => backend.asInstanceOf[BackendHIP].sgd_update(tr, learning_rate, descent) }
   }
-  // RNNBase itself (NNModule.scala:332-417) is reused with `BackendCudnn()` read as `BackendHIP()`: same parameter buffer layout,
-  // same calls (cudnnRNNForwardTraining / cudnnRNNBackward above).
+  // RNNBase itself (NNModule.scala:332-417) is reused with `BackendCudnn()` read as `BackendHIP()`: same calls
+  // (cudnnRNNForwardTraining / cudnnRNNBackward above, initial states and dropout included).  One difference: layers after the
+  // first of a bidirectional stack read 2 * hiddenSize features, which getParameterSize (NN:357) leaves out ("// * numDirections");
+  // the buffer must be gateSize * inputSize + (numLayers - 1) * gateSize * hiddenSize * numDirections long per direction.
 }
 
 // ---- the driver the applications extend (DslAPI.scala:1064-1077) -------------------------------------------------------------------

@@ -289,6 +289,54 @@ def test_gated_rnn_against_torch(mode, bidir):
             np.testing.assert_allclose(dw[o:o + size] - 1, g, rtol=1e-4, atol=1e-5, err_msg=nm + str(d)); o += size
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2, 3], ids=["relu", "tanh", "lstm", "gru"])
+@pytest.mark.parametrize("bidir", [False, True], ids=["uni", "bi"])
+def test_rnn_initial_states_against_torch(mode, bidir):
+    """The *_init forms (initial hidden state, and cell state for the LSTM, as values without a gradient) against torch's
+    h_0 / c_0: outputs, input gradient and weight gradients.  A state handed to the wrong direction, used as a zero in the
+    backward pass (the W_hh gradient of the first step would miss its term) or a cell state read as hidden state fails."""
+    torch = pytest.importorskip("torch")
+    rng = np.random.RandomState(50 + mode)
+    T, B, In, H = 5, 3, 4, 6
+    ng = {0: 1, 1: 1, 2: 4, 3: 3}[mode]
+    D, G = (2 if bidir else 1), ng * H
+    per = G * In + G * H + 2 * G
+    w = (rng.randn(D * per) * 0.5).astype(np.float32)
+    x = rng.randn(T, B, In).astype(np.float32); dy = rng.randn(T, B, D * H).astype(np.float32)
+    hx = rng.randn(D, B, H).astype(np.float32); cx = rng.randn(D, B, H).astype(np.float32)
+    if mode < 2:
+        net = torch.nn.RNN(In, H, 1, nonlinearity="tanh" if mode == 1 else "relu", bidirectional=bidir)
+    else:
+        net = (torch.nn.LSTM if mode == 2 else torch.nn.GRU)(In, H, 1, bidirectional=bidir)
+    names = ["weight_ih_l0", "weight_hh_l0", "bias_ih_l0", "bias_hh_l0"]
+    sizes, shapes = (G * In, G * H, G, G), ((G, In), (G, H), (G,), (G,))
+    with torch.no_grad():
+        for d in range(D):
+            o = d * per
+            for nm, size, shape in zip(names, sizes, shapes):
+                getattr(net, nm + ("_reverse" if d else "")).copy_(torch.tensor(w[o:o + size].reshape(shape))); o += size
+    tx = torch.tensor(x, requires_grad=True)
+    state = (torch.tensor(hx), torch.tensor(cx)) if mode == 2 else torch.tensor(hx)
+    ty, _ = net(tx, state)
+    ty.backward(torch.tensor(dy))
+    y = np.zeros((T, B, D * H), np.float32)
+    dx = np.ones_like(x); dw = np.ones_like(w)
+    if mode < 2:
+        lc.lc_rnn_fwd_init(I(mode), cptr(x), cptr(hx), cptr(w), cptr(y), I(T), I(B), I(In), I(H), I(int(bidir)))
+        lc.lc_rnn_bwd_init(I(mode), cptr(x), cptr(hx), cptr(y), cptr(dy), cptr(w), cptr(dx), cptr(dw), I(T), I(B), I(In), I(H), I(int(bidir)))
+    else:
+        c0 = cptr(cx) if mode == 2 else None
+        lc.lc_rnn_gated_fwd_init(I(mode), cptr(x), cptr(hx), c0, cptr(w), cptr(y), I(T), I(B), I(In), I(H), I(int(bidir)))
+        lc.lc_rnn_gated_bwd_init(I(mode), cptr(x), cptr(hx), c0, cptr(dy), cptr(w), cptr(dx), cptr(dw), I(T), I(B), I(In), I(H), I(int(bidir)))
+    np.testing.assert_allclose(y, ty.detach().numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(dx - 1, tx.grad.numpy(), rtol=1e-4, atol=1e-5)
+    for d in range(D):
+        o = d * per
+        for nm, size in zip(names, sizes):
+            g = getattr(net, nm + ("_reverse" if d else "")).grad.numpy().ravel()
+            np.testing.assert_allclose(dw[o:o + size] - 1, g, rtol=1e-4, atol=1e-5, err_msg=nm + str(d)); o += size
+
+
 @pytest.mark.parametrize("p", [(2, 3, 8, 8, 3, 3, 1, 1, 1, 1), (1, 2, 5, 9, 2, 4, 2, 3, 1, 2), (2, 2, 13, 13, 3, 3, 2, 2, 0, 1), (1, 1, 4, 4, 4, 4, 3, 3, 3, 3)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_padded_avgpool_against_torch(p):

@@ -768,6 +768,40 @@ def test_gated_rnn_forward_and_backward(pair, case):
     check_all(pair.run(f), rtol=3e-4)
 
 
+@pytest.mark.parametrize("case", [(0, True, 5, 3, 7, 37), (1, False, 4, 5, 20, 64), (1, True, 6, 32, 96, 800), (2, True, 7, 5, 20, 48), (2, False, 1, 2, 5, 16),
+                                  (3, True, 4, 3, 33, 130), (3, False, 6, 8, 64, 256)], ids=lambda c: "mode%d_bi%d_T%d_B%d_I%d_H%d" % c)
+def test_rnn_with_initial_states(pair, case):
+    """RNNBase.apply(input, hx, cx): a layer started from a given hidden (and, for the LSTM, cell) state; outputs, input
+    gradient and weight gradients.  The states themselves receive no gradient (CDN:1843-1844)."""
+    mode, bidir, T, Bn, In, H = case
+    ng = {0: 1, 1: 1, 2: 4, 3: 3}[mode]
+    D, G = (2 if bidir else 1), ng * H
+    rng = np.random.RandomState(51)
+    per = G * In + G * H + 2 * G
+    w = (rng.randn(D * per) * (0.5 / np.sqrt(H))).astype(np.float32)
+    if mode == 0:
+        w[:] = np.abs(w) * np.where(rng.rand(w.size) < 0.3, -1, 1)
+    x = rng.randn(T, Bn, In).astype(np.float32); dy = rng.randn(T, Bn, D * H).astype(np.float32)
+    hx = rng.randn(D, Bn, H).astype(np.float32); cx = rng.randn(D, Bn, H).astype(np.float32)
+
+    def f(be, up, down):
+        X, W, HX = up(x), up(w), up(hx)
+        CX = up(cx) if mode == 2 else None
+        dx = up(np.ones(x.size, np.float32)); dw = up(np.ones(w.size, np.float32))
+        if mode < 2:
+            y = be.rnn_forward(mode, X, W, T, Bn, In, H, bidir, hx=HX)
+            be.rnn_backward(mode, X, y, up(dy), W, dx, dw, T, Bn, In, H, bidir, 1.0, hx=HX)
+            y0 = be.rnn_forward(mode, X, W, T, Bn, In, H, bidir)
+        else:
+            y, reserve = be.rnn_gated_forward(mode, X, W, T, Bn, In, H, bidir, hx=HX, cx=CX)
+            be.rnn_gated_backward(mode, X, y, up(dy), W, reserve, dx, dw, T, Bn, In, H, bidir, 1.0, hx=HX, cx=CX)
+            y0, _ = be.rnn_gated_forward(mode, X, W, T, Bn, In, H, bidir)
+        assert np.abs(down(y, dy.shape) - down(y0, dy.shape)).max() > 1e-3, "the initial state changed nothing"
+        return [down(y, dy.shape), down(dx, x.shape), down(dw, w.shape)]
+
+    check_all(pair.run(f), rtol=3e-4)
+
+
 @pytest.mark.gpu
 def test_gated_rnn_rejects_bad_arguments(hip_backend):
     be = hip_backend

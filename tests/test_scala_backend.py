@@ -120,6 +120,8 @@ NOT_CALLED = {
     "lh_bn_train_fwd_relu", "lh_conv2d_fwd_bnstats", "lh_concat_grad_beta",
     # superseded within the trait mapping: padded average pooling covers pad 0; the dense max-pool gradient replaces the scatter form
     "lh_avgpool_fwd", "lh_avgpool_bwd", "lh_maxpool_bwd",
+    # the zero-state forms: the backend always calls the *_init forms, with NULL for a state it was not given
+    "lh_rnn_fwd", "lh_rnn_bwd", "lh_rnn_gated_fwd", "lh_rnn_gated_bwd",
     # the reserve size is a staging-time product in Scala (same formula, checked in tests/test_parity_ops.py against the call)
     "lh_rnn_gated_reserve_floats",
     # data loader side, not the trait

@@ -443,8 +443,10 @@ def test_resnet50_headline_step_invariants_at_full_size(hip_backend):
 class _SeqClassifier:
     """[T, B, I] -> stacked LSTM / GRU module -> last time step's features -> Linear1D -> logSoftmax -> nll, SGD."""
 
-    def __init__(self, kind, bidirectional, numLayers):
+    def __init__(self, kind, bidirectional, numLayers, dropout=0.0):
         from lantern_amd.nn import Module, Linear1D, LSTM, GRU, SGD
+        self.hx = self.cx = None
+        outer = self
         from lantern_amd.tensor import Tensor, int_array
         T, B, I, H, C = 6, 4, 10, 12, 5
         Tensor.randseed(7)
@@ -453,11 +455,11 @@ class _SeqClassifier:
         class Net(Module):
             def __init__(self):
                 super().__init__("seq")
-                self.rnn = self.add((LSTM if kind == "lstm" else GRU)(I, H, numLayers, bidirectional=bidirectional))
+                self.rnn = self.add((LSTM if kind == "lstm" else GRU)(I, H, numLayers, dropout=dropout, bidirectional=bidirectional))
                 self.fc = self.add(Linear1D(T * H * (2 if bidirectional else 1), C, name="fc"))
 
             def __call__(self, x):
-                return self.fc(self.rnn(x).permute(1, 0, 2).resize(B, -1))
+                return self.fc(self.rnn(x, outer.hx, outer.cx).permute(1, 0, 2).resize(B, -1))
 
         self.model = Net()
         # Tensor.rand(size, 0.01) of the reference leaves the gates near 0.5 / 0: scale the packed buffer up so every gate matters
@@ -478,6 +480,19 @@ class _SeqClassifier:
 
     def end_step(self):
         la.get_backend().resetMallocAddr(self.mark)
+
+
+def test_stacked_lstm_with_initial_states_and_dropout_10_steps(hip_backend, cpu_backend):
+    """RNNBase(LstmMode, numLayers = 2, dropout = 0.3, bidirectional) called with hx and cx (NN:392-409): the states are cut
+    per layer, dropout sits between the layers (the same counter-based mask on both backends)."""
+    def make():
+        tr = _SeqClassifier("lstm", True, 2, dropout=0.3)
+        rng = np.random.RandomState(11)
+        tr.hx = la.Tensor.fromNumpy(rng.randn(4, 4, 12).astype(np.float32))
+        tr.cx = la.Tensor.fromNumpy(rng.randn(4, 4, 12).astype(np.float32))
+        tr.mark = la.get_backend().getMallocAddr()
+        return tr
+    _compare(make, hip_backend, cpu_backend)
 
 
 @pytest.mark.parametrize("kind,bidirectional,numLayers", [("lstm", False, 1), ("lstm", True, 2), ("gru", False, 2), ("gru", True, 1)])
