@@ -107,3 +107,75 @@ def test_c_host_program_trains_lenet_like_the_oracle():
     out = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=110)
     print(out.stdout, out.stderr)
     assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
+
+
+# ---- the TreeLSTM loop from C ---------------------------------------------------------------------------------------------
+TREE_BIN = os.path.join(HOST_C, "_build", "treelstm_step")
+
+
+def write_treelstm_inputs(tmp_path, trainer, trees):
+    """The C program's two input files from a freshly built mirror trainer (tests and bench.py use the same writer)."""
+    import numpy as np
+    model = trainer.model
+    params = [p for _, p in model.namedParameters()]
+    names = [n.split("/", 1)[1] for n, _ in model.namedParameters()]
+    assert names == ["leaf/Wi", "leaf/bi", "leaf/Wo", "leaf/bo", "leaf/Wu", "leaf/bu"] + ["node/" + n for n in type(model.node).NAMES] + ["output/Why", "output/by"], names
+    emb = trainer.embedding.toCPU()
+    vocab, e = emb.shape
+    hidden, classes = params[1].x.shape[0], params[-1].x.shape[0]
+    with open(tmp_path / "params.bin", "wb") as f:
+        np.array([vocab, e, hidden, classes], np.int32).tofile(f)
+        emb.astype(np.float32).tofile(f)
+        for p in params:
+            p.x.toCPU().astype(np.float32).tofile(f)
+    with open(tmp_path / "trees.txt", "w") as f:
+        f.write("%d\n" % len(trees))
+        for t in trees:
+            f.write("%d\n" % len(t[0]))
+            for arr in t:
+                f.write(" ".join(str(int(v)) for v in arr) + "\n")
+    return params
+
+
+def test_c_treelstm_program_links():
+    exe = _build_host_program() and TREE_BIN
+    out = subprocess.run([exe], env=dict(os.environ, TREELSTM_STEP_LINK_ONLY="1"), capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0 and out.stdout.strip() == "linked", out.stdout + out.stderr
+    deps = subprocess.run(["ldd", exe], capture_output=True, text=True).stdout
+    assert "liblantern_hip.so" in deps and "torch" not in deps and "python" not in deps and "lantern_cpu" not in deps, deps
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cmdlist", [0, 1], ids=["one_launch_per_op", "command_list"])
+def test_c_treelstm_program_tracks_the_oracle(tmp_path, cpu_backend, cmdlist):
+    """The recursion over the tree arrays written in C against the C-ABI (tests/host_c/treelstm_step.c), one Adagrad step per tree
+    over the first eight trees of the reference's own evaluation set (tests/golden/array_tree_first24.txt: 8 to 34 leaves), against
+    the same trees run through the host mirror on the CPU oracle from the same initial parameters: every loss within 1e-4
+    relative, every parameter tensor within 1e-3 (relative L2)."""
+    import numpy as np
+    import lantern_amd as la
+    from lantern_amd.apps.treelstm import Trainer, read_trees
+    exe = TREE_BIN if os.path.exists(TREE_BIN) else (_build_host_program() and TREE_BIN)
+    la.set_backend(cpu_backend)
+    mark = cpu_backend.getMallocAddr()
+    trees = read_trees(os.path.join(ROOT, "tests", "golden", "array_tree_first24.txt"))[:8]
+    tr = Trainer(vocab=500, trees=trees)
+    params = write_treelstm_inputs(tmp_path, tr, tr.trees)
+    want_losses = []
+    for _ in range(len(trees)):
+        want_losses.append(float(tr.step().toCPU()[0])); tr.end_step()
+    want = [p.x.toCPU().copy() for p in params]
+    tr.close(); cpu_backend.resetMallocAddr(mark)
+    out = subprocess.run([exe, str(tmp_path / "params.bin"), str(tmp_path / "trees.txt"), str(tmp_path / "out.bin"), str(len(trees)), "0", str(cmdlist)],
+                         capture_output=True, text=True, timeout=110)
+    print(out.stdout, out.stderr)
+    assert out.returncode == 0 and out.stdout.startswith("trees_per_s"), out.stdout + out.stderr
+    got = np.fromfile(tmp_path / "out.bin", np.float32)
+    assert got.size == len(trees) + sum(w.size for w in want)
+    np.testing.assert_allclose(got[:len(trees)], want_losses, rtol=1e-4)
+    assert want_losses[0] != want_losses[-1]
+    pos = len(trees)
+    for w in want:
+        g = got[pos:pos + w.size].reshape(w.shape); pos += w.size
+        err = np.linalg.norm(g.astype(np.float64) - w) / max(np.linalg.norm(w.astype(np.float64)), 1e-30)
+        assert err <= 1e-3 or np.abs(g - w).max() <= 1e-5, err
