@@ -1,12 +1,19 @@
-// Command list: small operations recorded on the host and executed, in order, by one 1024-thread workgroup.
+// Command list: small operations recorded on the host and executed by one 1024-thread workgroup.
 //
-// A model built from 150-element vectors (the sentiment TreeLSTM: ~5000 operator calls per tree) is bound by the
+// A model built from 150-element vectors (the sentiment TreeLSTM: ~7000 operator calls per tree) is bound by the
 // host's kernel-launch rate (about 3 us per launch), not by the device.  Between lh_cmdlist_begin() and
-// lh_cmdlist_end() every entry point whose operands are small appends a 64-byte command to a pinned host buffer
-// instead of launching; the buffer is handed to k_cmdlist when it is full, when recording ends, or when any other
-// entry point is about to use the stream (lh::ordered_stream), so the program order of all operations is kept.
-// One workgroup runs the commands one after the other with a block barrier between them: every command sees the
-// global-memory results of the ones before it (same compute unit, same L1), and no other kernel runs in between.
+// lh_cmdlist_end() every entry point whose operands are small appends a 64-byte command instead of launching; the
+// commands of a buffer are handed to k_cmdlist when the buffer is full, when recording ends, or when any other entry
+// point is about to use the stream (lh::ordered_stream), so the program order of all operations is kept.
+//
+// One workgroup pays a full memory round trip (load, store, barrier) per dependent command, about 1 us, whatever the
+// command's size.  So the host works out, per buffer, which commands depend on which (byte ranges read and written: a
+// command that writes a range comes after every earlier command that touches it, one that reads it after every earlier
+// writer) and gives each command a LEVEL, one more than the highest level it depends on.  The buffer is executed level
+// by level: commands of one level have no dependence on each other, run without a barrier between them, and are spread
+// over the workgroup's 16 wavefronts (each command carries a rotation of the thread index), so their round trips overlap;
+// one block barrier per level makes a level's stores visible to the next.  Independent work of a program (the ten gate
+// products of a tree node, the two subtrees of a node) thus runs side by side without the program saying so.
 // The arithmetic of each command follows the stand-alone kernel of the same operation.
 #include "lh_common.h"
 using namespace lh;
@@ -19,13 +26,24 @@ int g_rec_pending = 0;
 namespace {
 constexpr int CL_THREADS = 1024;
 constexpr int CL_CHUNK = 256;                 // commands staged in LDS at a time
-constexpr int CL_BUF_CMDS = 256;              // commands per host buffer: a full buffer is launched while the host records the next
+constexpr int CL_BUF_CMDS = 2048;              // commands per host buffer: a full buffer is launched while the host records the next
 constexpr int CL_NBUF = 32;
+constexpr int CL_OP_MASK = 0xff;              // LhCmd::op as the kernel sees it: operation | barrier flag | rotation << 12
+constexpr int CL_BARRIER = 0x100;             // first command of a level: a block barrier comes before it
+constexpr int CL_ROT_SHIFT = 12;              // 12 bits: where the command's work starts (a wavefront 0..15 of the owner, or, for a
+                                              // command split over all workgroups, one of their wavefronts taken together)
+constexpr int CL_OWNER_SHIFT = 24;            // the workgroup (0..255) that runs a command which is not split over all of them
+constexpr int CL_MAX_GROUPS = 64;
+constexpr long CL_SPIN_LIMIT = 40000000L;     // polls of a grid barrier before a workgroup gives up (far beyond any real wait)
 
 struct Ring {
   LhCmd* host[CL_NBUF]; LhCmd* dev[CL_NBUF]; hipEvent_t done[CL_NBUF]; bool busy[CL_NBUF];
   int cur; bool ready;
-  int64_t recorded, launches;
+  int64_t recorded, launches, levels;
+  unsigned long long* sync;          // device: [0] arrivals at grid barriers, [1] a workgroup gave up waiting
+  unsigned long long sync_base;      // arrivals once everything launched so far has run
+  int groups;                        // workgroups per launch
+  unsigned* host_flag; unsigned* host_flag_dev;       // pinned word a workgroup sets when its barrier wait ran out
 };
 static Ring g_ring = {};
 
@@ -68,12 +86,46 @@ __device__ __forceinline__ float cl_wave_max_all(float v) {
   return v;
 }
 
+// Matrix operands are read and written through buffer descriptors: a 32-bit byte offset per lane instead of a 64-bit
+// address computed per element (one workgroup's vector ALUs, not memory, bound these commands), constant column steps folded
+// into the instruction, and anything past the operand's last byte reads as zero or is not stored, so rows past the matrix
+// need no test.  The descriptor's base must be wave-uniform: the pointer comes out of LDS and is made so explicitly.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t cl_rsrc(const void* p, int64_t bytes) {
+  const uint64_t a = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return __builtin_amdgcn_make_buffer_rsrc((void*)(((uint64_t)hi << 32) | lo), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float cl_ld(__amdgpu_buffer_rsrc_t r, uint32_t off) { return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0)); }
+__device__ __forceinline__ void cl_st(__amdgpu_buffer_rsrc_t r, uint32_t off, float v) { __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, (int)off, 0, 0); }
+constexpr uint32_t CL_OOB = 0x80000000u;       // an offset no operand reaches (operands are far below 2 GiB)
+// Sum over the 64 lanes, the same value in every lane: DPP inside rows of 16, one swizzle, two lane reads.
+__device__ __forceinline__ float cl_wave_sum_dpp(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // row_mirror
+  v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));                      // lane ^ 16
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+}
+
 // Data pointers carry no __restrict__ and no const: a command may read what the command before it wrote.
-__device__ void cl_run(const LhCmd& c, float* red /* [4][257] */) {
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+// `rot`: the wavefront that takes the command's first elements (commands of one level start on different wavefronts).
+// `grp` of `ngrp` workgroups: the matrix commands are cut by rows over all workgroups (one compute unit draws only some
+// 25 GB/s from memory, whatever its wavefronts do; the rows of a 150 x 150 matrix spread over 16 units take one memory
+// round trip); every other command is run by the one workgroup its `owner` field names.
+__device__ void cl_run(const LhCmd& c, const int rot, float* red /* [16][257] */, const int grp, const int ngrp) {
   constexpr int NT = CL_THREADS, NW = CL_THREADS / 64;
+  const int opc = c.op & CL_OP_MASK;
+  const bool split = ngrp > 1 && (opc == CL_GEMV_N || opc == CL_GER || (opc == CL_GEMV_T && c.f1 == 1.0f));
+  if (!split && ngrp > 1 && ((c.op >> CL_OWNER_SHIFT) & 0xff) != grp) return;
+  const int lane = threadIdx.x & 63, wave = split ? (int)(threadIdx.x >> 6) : (int)(((threadIdx.x >> 6) + NW - (rot & (NW - 1))) & (NW - 1)), t = wave * 64 + lane;
   float* p0 = (float*)c.p0; float* p1 = (float*)c.p1; float* p2 = (float*)c.p2; float* p3 = (float*)c.p3;
-  switch (c.op) {
+  // A matrix command is cut into pieces of a few rows; piece k goes to wavefront (rot + k) mod GW of all GW wavefronts that share
+  // the command (neighbouring ones in different workgroups).  The pieces of the commands of one level follow each other round the
+  // wavefronts, so a wavefront rarely holds pieces of two of them and their memory round trips overlap instead of queueing.
+  const int GW = split ? ngrp * NW : NW;
+  const int gw = split ? (wave * ngrp + grp + GW - rot % GW) % GW : wave;
+  switch (opc) {
     case CL_ZERO16: { uint4* p = (uint4*)c.p0; const int n = c.i0; for (int i = t; i < n; i += NT) p[i] = make_uint4(0, 0, 0, 0); break; }
     case CL_FILL: { const int n = c.i0; const float v = c.f0; for (int i = t; i < n; i += NT) p0[i] = v; break; }
     case CL_COPY: { const int n = c.i0; for (int i = t; i < n; i += NT) p0[i] = p1[i]; break; }
@@ -93,65 +145,108 @@ __device__ void cl_run(const LhCmd& c, float* red /* [4][257] */) {
         p0[i] = cl_unary_grad(op, inplace, p0[i], need_x ? p1[i] : 0.f, need_y ? p2[i] : 0.f, need_g ? p3[i] : 0.f, lo, hi);
       break;
     }
-    case CL_GEMV_N: {            // y[m] = alpha * A[m,n] x[n] + beta * y   (p0 = y, p1 = A, p2 = x; i2 = lda): a wavefront per row,
-      // four rows at a time so that their loads are in flight together (a store to y ends a batch, not every row)
+    case CL_GEMV_N: {            // y[m] = alpha * A[m,n] x[n] + beta * y   (p0 = y, p1 = A, p2 = x; i2 = lda): a wavefront takes
+      // up to ten rows at a time and a lane four columns of each, all loads issued before the first product
       const int m = c.i0, n = c.i1, lda = c.i2; const float al = c.f0, be = c.f1;
-      for (int r0 = wave * 4; r0 < m; r0 += NW * 4) {
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int j = lane; j < n; j += 64) {
-          const float xv = p2[j];
+      const __amdgpu_buffer_rsrc_t rA = cl_rsrc(p1, ((int64_t)(m - 1) * lda + n) * 4), rX = cl_rsrc(p2, (int64_t)n * 4);
+      constexpr int RB = 10;
+      for (int r0 = gw * RB; r0 < m; r0 += GW * RB) {
+        float acc[RB];
 #pragma unroll
-          for (int u = 0; u < 4; u++) acc[u] += (r0 + u < m ? p1[(int64_t)(r0 + u) * lda + j] : 0.f) * xv;
-        }
+        for (int u = 0; u < RB; u++) acc[u] = 0.f;
+        for (int j0 = 0; j0 < n; j0 += 256) {
+          float xv[4], av[RB][4];
+          const uint32_t co = (uint32_t)(j0 + lane) * 4u;
 #pragma unroll
-        for (int u = 0; u < 4; u++) acc[u] = cl_wave_sum_all(acc[u]);
-        if (lane < 4 && r0 + lane < m) {
-          const float s = lane == 0 ? acc[0] : (lane == 1 ? acc[1] : (lane == 2 ? acc[2] : acc[3]));
-          p0[r0 + lane] = al * s + (be == 0.f ? 0.f : be * p0[r0 + lane]);
-        }
-      }
-      break;
-    }
-    case CL_GEMV_T: {            // y[n] = alpha * A[m,n]^T x[m] + beta * y  (p0 = y, p1 = A, p2 = x): 256 columns x 4 row groups per pass
-      const int m = c.i0, n = c.i1, lda = c.i2; const float al = c.f0, be = c.f1;
-      const int col = t & 255, g = t >> 8;
-      for (int j0 = 0; j0 < n; j0 += 256) {
-        const int j = j0 + col;
-        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-        if (j < n) {
-          int i = g;
-          for (; i + 12 < m; i += 16) {
-            a0 += p1[(int64_t)i * lda + j] * p2[i];
-            a1 += p1[(int64_t)(i + 4) * lda + j] * p2[i + 4];
-            a2 += p1[(int64_t)(i + 8) * lda + j] * p2[i + 8];
-            a3 += p1[(int64_t)(i + 12) * lda + j] * p2[i + 12];
+          for (int q = 0; q < 4; q++) xv[q] = cl_ld(rX, co + q * 256u);                  // zero past n
+#pragma unroll
+          for (int u = 0; u < RB; u++) {
+            const uint32_t ro = (uint32_t)(r0 + u) * (uint32_t)lda * 4u + co;            // rows past m lie past the operand's end
+#pragma unroll
+            for (int q = 0; q < 4; q++) av[u][q] = cl_ld(rA, ro + q * 256u);
           }
-          for (; i < m; i += 4) a0 += p1[(int64_t)i * lda + j] * p2[i];
+          if (j0 + 256 > n) {                                                            // columns past n hold the next row's values
+#pragma unroll
+            for (int q = 0; q < 4; q++) if (j0 + q * 64 + lane >= n) {
+#pragma unroll
+              for (int u = 0; u < RB; u++) av[u][q] = 0.f;
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < RB; u++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) acc[u] += av[u][q] * xv[q];
         }
-        red[g * 257 + col] = (a0 + a1) + (a2 + a3);
+        float sv = 0.f;
+#pragma unroll
+        for (int u = 0; u < RB; u++) { const float tot = cl_wave_sum_dpp(acc[u]); sv = lane == u ? tot : sv; }
+        if (lane < RB && r0 + lane < m) p0[r0 + lane] = al * sv + (be == 0.f ? 0.f : be * p0[r0 + lane]);
+      }
+      break;
+    }
+    case CL_GEMV_T: {            // y[n] = alpha * A[m,n]^T x[m] + beta * y  (p0 = y, p1 = A, p2 = x): a wavefront takes five rows
+      // at a time, a lane four columns of each, all loads in flight together; the wavefronts' partial sums meet in LDS
+      const int m = c.i0, n = c.i1, lda = c.i2; const float al = c.f0, be = c.f1;
+      const __amdgpu_buffer_rsrc_t rA = cl_rsrc(p1, ((int64_t)(m - 1) * lda + n) * 4), rX = cl_rsrc(p2, (int64_t)m * 4);
+      for (int j0 = 0; j0 < n; j0 += 256) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        uint32_t co[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) { const int j = j0 + q * 64 + lane; co[q] = j < n ? (uint32_t)j * 4u : CL_OOB; }
+        for (int i0 = gw * 5; i0 < m; i0 += 5 * GW) {
+          float xv[5], av[5][4];
+#pragma unroll
+          for (int u = 0; u < 5; u++) {
+            const uint32_t i = (uint32_t)(i0 + u);
+            xv[u] = cl_ld(rX, i * 4u);                                                   // zero past m
+            const uint32_t ro = i * (uint32_t)lda * 4u;
+#pragma unroll
+            for (int q = 0; q < 4; q++) av[u][q] = cl_ld(rA, ro + co[q]);
+          }
+#pragma unroll
+          for (int u = 0; u < 5; u++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) acc[q] += av[u][q] * xv[u];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) red[wave * 257 + q * 64 + lane] = acc[q];
         __syncthreads();
-        if (g == 0 && j < n) {
-          const float s = (red[col] + red[257 + col]) + (red[2 * 257 + col] + red[3 * 257 + col]);
-          p0[j] = al * s + (be == 0.f ? 0.f : be * p0[j]);
+        if (t < 256 && j0 + t < n) {
+          float sv = 0.f;
+#pragma unroll
+          for (int w = 0; w < NW; w++) sv += red[w * 257 + t];
+          if (split) atomicAdd(p0 + j0 + t, al * sv);          // beta is 1: every workgroup adds the sum over its rows
+          else p0[j0 + t] = al * sv + (be == 0.f ? 0.f : be * p0[j0 + t]);
         }
         __syncthreads();
       }
       break;
     }
-    case CL_GER: {               // A[m,n] += u[m] (x) v[n]   (p0 = A, p1 = u, p2 = v): four elements per thread and pass, loads first
-      const int m = c.i0, n = c.i1, tot = m * n;
-      for (int i0 = t; i0 < tot; i0 += 4 * NT) {
-        float a[4], w[4];
+    case CL_GER: {               // A[m,n] += u[m] (x) v[n]   (p0 = A, p1 = u, p2 = v): a wavefront takes five rows at a time, a lane
+      // four columns of each, all loads in flight together
+      const int m = c.i0, n = c.i1;
+      const __amdgpu_buffer_rsrc_t rA = cl_rsrc(p0, (int64_t)m * n * 4), rU = cl_rsrc(p1, (int64_t)m * 4), rV = cl_rsrc(p2, (int64_t)n * 4);
+      for (int j0 = 0; j0 < n; j0 += 256) {
+        float vv[4]; uint32_t co[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-          const int i = i0 + u * NT;
-          const bool ok = i < tot;
-          const int r = ok ? i / n : 0, cc = ok ? i - r * n : 0;
-          a[u] = ok ? p0[i] : 0.f;
-          w[u] = p2[cc] * p1[r];
+        for (int q = 0; q < 4; q++) { const int j = j0 + q * 64 + lane; co[q] = j < n ? (uint32_t)j * 4u : CL_OOB; vv[q] = cl_ld(rV, co[q]); }
+        for (int i0 = gw * 5; i0 < m; i0 += 5 * GW) {
+          float uu[5], av[5][4];
+#pragma unroll
+          for (int u = 0; u < 5; u++) {
+            const uint32_t i = (uint32_t)(i0 + u);
+            uu[u] = cl_ld(rU, i * 4u);
+            const uint32_t ro = i * (uint32_t)n * 4u;
+#pragma unroll
+            for (int q = 0; q < 4; q++) av[u][q] = cl_ld(rA, ro + co[q]);
+          }
+#pragma unroll
+          for (int u = 0; u < 5; u++) {
+            const uint32_t ro = (uint32_t)(i0 + u) * (uint32_t)n * 4u;
+#pragma unroll
+            for (int q = 0; q < 4; q++) cl_st(rA, ro + co[q], av[u][q] + vv[q] * uu[u]);   // nothing is stored past the operand or the row
+          }
         }
-#pragma unroll
-        for (int u = 0; u < 4; u++) { const int i = i0 + u * NT; if (i < tot) p0[i] = a[u] + w[u]; }
       }
       break;
     }
@@ -163,6 +258,7 @@ __device__ void cl_run(const LhCmd& c, float* red /* [4][257] */) {
       if (lane == 0) red[wave] = acc;
       __syncthreads();
       if (wave == 0) { float v = lane < NW ? red[lane] : 0.f; v = cl_wave_sum_all(v); if (lane == 0) p0[0] = v; }
+      __syncthreads();           // `red` is free again: the next command of the level may follow without a barrier
       break;
     }
     case CL_AXPY_DEV: {          // y += s[0] * x   (p0 = y, p1 = s, p2 = x)
@@ -232,13 +328,43 @@ __device__ void cl_run(const LhCmd& c, float* red /* [4][257] */) {
   }
 }
 
-// cmds: pinned host memory (read over the host link, a chunk at a time, the next chunk fetched while the current one runs).
-__global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const LhCmd* cmds, int n) {
+// One barrier over all workgroups of the launch: everything a workgroup stored before it is visible to every workgroup
+// after it (release and acquire at device scope: the workgroups sit on different XCDs with their own L2).  `sync[0]` counts
+// arrivals over the life of the library (64 bits; `target` is the count this barrier completes at), `sync[1]` is set by a
+// workgroup whose wait ran out, which makes every workgroup leave the kernel: a lost workgroup cannot hang the device.
+__device__ __forceinline__ bool cl_grid_barrier(unsigned long long* sync, unsigned long long target, int* lds_flag, unsigned* host_flag) {
+  __syncthreads();                                       // every wavefront's stores are issued before wavefront 0 releases them
+  if (threadIdx.x == 0) {
+    __hip_atomic_fetch_add(sync, 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    long spins = 0;
+    int gave_up = 0;
+    while (__hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      if (++spins > CL_SPIN_LIMIT || __hip_atomic_load(sync + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0ull) {
+        __hip_atomic_store(sync + 1, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *(volatile unsigned*)host_flag = 1u;              // pinned host memory: the host sees it without waiting for the stream
+        gave_up = 1;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    *lds_flag = gave_up;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   // the caches this workgroup reads through drop what other workgroups have since replaced
+  }
+  __syncthreads();
+  return *lds_flag == 0;
+}
+
+// cmds: pinned host memory (read over the host link, a chunk at a time, the next chunk fetched while the current one runs),
+// in execution order: level by level, the first command of every level but the first flagged CL_BARRIER.  Every workgroup of
+// the launch walks the whole list.
+__global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const LhCmd* cmds, int n, unsigned long long* sync, unsigned long long sync_base, unsigned* host_flag) {
   __shared__ uint4 stage[CL_CHUNK * 4];                 // 256 commands of 64 bytes
-  __shared__ float red[4 * 257];
-  const int t = threadIdx.x;
+  __shared__ float red[(CL_THREADS / 64) * 257];
+  __shared__ int gave_up;
+  const int t = threadIdx.x, grp = blockIdx.x, ngrp = gridDim.x;
   const uint4* src = reinterpret_cast<const uint4*>(cmds);
   const int total16 = n * 4;
+  unsigned long long arrived = sync_base;
   uint4 next = make_uint4(0, 0, 0, 0);
   if (t < total16) next = src[t];
   for (int base = 0; base < n; base += CL_CHUNK) {
@@ -249,9 +375,14 @@ __global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const LhCmd* cmds, int n
     const int cnt = n - base < CL_CHUNK ? n - base : CL_CHUNK;
     const LhCmd* list = reinterpret_cast<const LhCmd*>(stage);
     for (int i = 0; i < cnt; i++) {
-      cl_run(list[i], red);
-      __syncthreads();
+      const int op = list[i].op;                        // uniform: every thread reads the same LDS word
+      if (op & CL_BARRIER) {                            // the level before is complete and its stores are visible
+        if (ngrp == 1) __syncthreads();
+        else { arrived += (unsigned long long)ngrp; if (!cl_grid_barrier(sync, arrived, &gave_up, host_flag)) return; }
+      }
+      cl_run(list[i], (op >> CL_ROT_SHIFT) & 0xfff, red, grp, ngrp);
     }
+    __syncthreads();                                    // the staged commands are no longer read
   }
 }
 
@@ -263,19 +394,194 @@ static bool ring_init() {
     if (hipEventCreateWithFlags(&g_ring.done[i], hipEventDisableTiming) != hipSuccess) { LH_FAIL("command list: event creation failed"); return false; }
     g_ring.busy[i] = false;
   }
+  if (hipMalloc((void**)&g_ring.sync, 2 * sizeof(unsigned long long)) != hipSuccess || hipMemset(g_ring.sync, 0, 2 * sizeof(unsigned long long)) != hipSuccess) {
+    LH_FAIL("command list: cannot allocate the barrier words"); return false;
+  }
+  g_ring.sync_base = 0;
+  if (hipHostMalloc((void**)&g_ring.host_flag, 64, hipHostMallocDefault) != hipSuccess || hipHostGetDevicePointer((void**)&g_ring.host_flag_dev, g_ring.host_flag, 0) != hipSuccess) {
+    LH_FAIL("command list: cannot allocate the pinned flag"); return false;
+  }
+  *g_ring.host_flag = 0;
+  // Workgroups per launch: 16 compute units draw the matrices of a level in about one memory round trip, and a barrier over
+  // 16 costs 3.5 us against 2.5 us for one workgroup's own device-scope fences (6 us over 32).  LH_CMDLIST_GROUPS overrides.
+  int groups = 16;
+  if (const char* e = getenv("LH_CMDLIST_GROUPS")) groups = atoi(e);
+  if (groups < 1) groups = 1;
+  if (groups > CL_MAX_GROUPS) groups = CL_MAX_GROUPS;
+  if (groups > g_num_cu / 4) groups = g_num_cu / 4 > 0 ? g_num_cu / 4 : 1;       // all workgroups of a launch must be resident together
+  g_ring.groups = groups;
   g_ring.cur = 0; g_ring.ready = true;
   return true;
 }
 }  // namespace
 
+// ---- dependence levels of the commands in the buffer being recorded ------------------------------------------------------------
+namespace {
+struct Extent { uintptr_t s, e; bool w; };            // a byte range a command reads (w = false) or writes / updates (w = true)
+
+// The byte ranges a command touches.  Returns how many of o[0..3] are filled.
+static int cmd_extents(const LhCmd& c, Extent* o) {
+  int k = 0;
+  auto add = [&](const void* p, int64_t bytes, bool w) { if (p && bytes > 0) { o[k].s = (uintptr_t)p; o[k].e = (uintptr_t)p + (uintptr_t)bytes; o[k].w = w; k++; } };
+  const int64_t n4 = (int64_t)c.i0 * 4;
+  switch (c.op) {
+    case CL_ZERO16: add(c.p0, (int64_t)c.i0 * 16, true); break;
+    case CL_FILL: add(c.p0, n4, true); break;
+    case CL_COPY: case CL_SCALAR: case CL_UNARY: add(c.p0, n4, true); add(c.p1, n4, false); break;
+    case CL_GEAM: case CL_BIN: case CL_ACC: case CL_ACCNEG: case CL_ACCMUL: add(c.p0, n4, true); add(c.p1, n4, false); add(c.p2, n4, false); break;
+    case CL_UNARY_GRAD: add(c.p0, n4, true); add(c.p1, n4, false); add(c.p2, n4, false); add(c.p3, n4, false); break;
+    case CL_GEMV_N: add(c.p0, n4, true); add(c.p1, ((int64_t)(c.i0 - 1) * c.i2 + c.i1) * 4, false); add(c.p2, (int64_t)c.i1 * 4, false); break;
+    case CL_GEMV_T: add(c.p0, (int64_t)c.i1 * 4, true); add(c.p1, ((int64_t)(c.i0 - 1) * c.i2 + c.i1) * 4, false); add(c.p2, n4, false); break;
+    case CL_GER: add(c.p0, (int64_t)c.i0 * c.i1 * 4, true); add(c.p1, n4, false); add(c.p2, (int64_t)c.i1 * 4, false); break;
+    case CL_DOT: add(c.p0, 4, true); add(c.p1, n4, false); add(c.p2, n4, false); break;
+    case CL_AXPY_DEV: add(c.p0, n4, true); add(c.p1, 4, false); add(c.p2, n4, false); break;
+    case CL_SOFTMAX: add(c.p0, n4 * c.i1, true); add(c.p1, n4 * c.i1, false); break;
+    case CL_SOFTMAX_GRAD: add(c.p0, n4 * c.i1, true); add(c.p1, n4 * c.i1, false); add(c.p2, n4 * c.i1, false); break;
+    case CL_NLL: add(c.p0, n4, true); add(c.p1, n4 * c.i1, false); add(c.p2, n4, false); break;
+    case CL_NLL_GRAD: add(c.p0, n4 * c.i1, true); add(c.p1, n4, false); add(c.p2, n4, false); break;
+    case CL_ADAGRAD: add(c.p0, n4, true); add(c.p1, n4, true); add(c.p2, n4, true); break;
+    case CL_SGD: add(c.p0, n4, true); add(c.p1, n4, true); break;
+    default: break;
+  }
+  return k;
+}
+// How many wavefronts of work a command is (where the next command of its level should start).
+static bool cmd_splits(const LhCmd& c) { return c.op == CL_GEMV_N || c.op == CL_GER || (c.op == CL_GEMV_T && c.f1 == 1.0f); }
+static int cmd_waves(const LhCmd& c) {
+  switch (c.op) {
+    case CL_GEMV_N: return (c.i0 + 9) / 10;
+    case CL_GEMV_T: case CL_GER: return (c.i0 + 4) / 5;
+    case CL_SOFTMAX: case CL_SOFTMAX_GRAD: return c.i0;
+    default: return (c.i0 + 63) / 64;
+  }
+}
+
+// Ranges of up to SMALL_BYTES are tracked per 256-byte block in a hash table (arena blocks are 256-byte aligned, so two
+// buffers share a block only when one lies inside the other's allocation: then the dependence is real or harmless);
+// larger ranges (matrices, zero fills) in a short table of distinct ranges.  A level is a uint16: 1 + highest level touched.
+constexpr uintptr_t SMALL_BYTES = 4096;
+constexpr int HASH_N = 65536, BIG_N = 96;
+struct Window {
+  LhCmd cmd[CL_BUF_CMDS]; uint16_t level[CL_BUF_CMDS]; int n; int top;       // top: highest level handed out
+  struct Slot { uintptr_t key; uint32_t epoch; uint16_t w, r; } slot[HASH_N]; uint32_t epoch;
+  struct Big { uintptr_t s, e; uint16_t w, r; } big[BIG_N]; int nbig;
+  struct Small { uintptr_t s, e; uint16_t level; bool w; } small[CL_BUF_CMDS * 4]; int nsmall;
+  uintptr_t small_lo, small_hi;                                               // bounding box of the small ranges
+};
+static Window* g_win = nullptr;
+
+static void window_reset(Window& W) {
+  W.n = 0; W.top = 0; W.nbig = 0; W.nsmall = 0; W.small_lo = ~(uintptr_t)0; W.small_hi = 0;
+  if (++W.epoch == 0) { for (int i = 0; i < HASH_N; i++) W.slot[i].epoch = 0; W.epoch = 1; }
+}
+static inline Window::Slot* slot_of(Window& W, uintptr_t block, bool create) {
+  uint32_t h = (uint32_t)((block * 0x9E3779B97F4A7C15ull) >> 48) & (HASH_N - 1);
+  for (int probe = 0; probe < HASH_N; probe++, h = (h + 1) & (HASH_N - 1)) {
+    Window::Slot& sl = W.slot[h];
+    if (sl.epoch != W.epoch) { if (!create) return nullptr; sl.key = block; sl.epoch = W.epoch; sl.w = sl.r = 0; return &sl; }
+    if (sl.key == block) return &sl;
+  }
+  return nullptr;
+}
+// The highest level among earlier commands of the window that `x` must come after.
+static int conflict_level(Window& W, const Extent& x) {
+  int lv = 0;
+  for (int i = 0; i < W.nbig; i++) {
+    const Window::Big& b = W.big[i];
+    if (b.s < x.e && x.s < b.e) { const int v = x.w ? (b.w > b.r ? b.w : b.r) : b.w; if (v > lv) lv = v; }
+  }
+  if (x.e - x.s <= SMALL_BYTES) {
+    for (uintptr_t blk = x.s >> 8; blk <= (x.e - 1) >> 8; blk++) {
+      const Window::Slot* sl = slot_of(W, blk, false);
+      if (sl) { const int v = x.w ? (sl->w > sl->r ? sl->w : sl->r) : sl->w; if (v > lv) lv = v; }
+    }
+  } else if (x.s < W.small_hi && W.small_lo < x.e) {         // a large range over memory that small ranges of this window touch: rare
+    for (int i = 0; i < W.nsmall; i++) {
+      const Window::Small& m = W.small[i];
+      if (m.s < x.e && x.s < m.e && (x.w || m.w) && m.level > lv) lv = m.level;
+    }
+  }
+  return lv;
+}
+static bool note_extent(Window& W, const Extent& x, int level) {
+  if (x.e - x.s <= SMALL_BYTES) {
+    for (uintptr_t blk = x.s >> 8; blk <= (x.e - 1) >> 8; blk++) {
+      Window::Slot* sl = slot_of(W, blk, true);
+      if (!sl) return false;
+      if (x.w) { if (level > sl->w) sl->w = (uint16_t)level; } else if (level > sl->r) sl->r = (uint16_t)level;
+    }
+    Window::Small& m = W.small[W.nsmall++];
+    m.s = x.s; m.e = x.e; m.level = (uint16_t)level; m.w = x.w;
+    if (x.s < W.small_lo) W.small_lo = x.s;
+    if (x.e > W.small_hi) W.small_hi = x.e;
+    return true;
+  }
+  for (int i = 0; i < W.nbig; i++) {
+    Window::Big& b = W.big[i];
+    if (b.s == x.s && b.e == x.e) { if (x.w) { if (level > b.w) b.w = (uint16_t)level; } else if (level > b.r) b.r = (uint16_t)level; return true; }
+  }
+  if (W.nbig == BIG_N) return false;
+  Window::Big& b = W.big[W.nbig++];
+  b.s = x.s; b.e = x.e; b.w = x.w ? (uint16_t)level : 0; b.r = x.w ? 0 : (uint16_t)level;
+  return true;
+}
+}  // namespace
+
 namespace lh {
+static unsigned long long g_tsc_push = 0, g_tsc_flush = 0, g_tsc_wait = 0;      // host cycles spent recording (LH_CMDLIST_VERBOSE prints them)
+// Hands the recorded buffer to the device: commands in level order (recording order within a level), the first of each
+// level flagged for a barrier, each with the wavefront its elements start on.
 void rec_flush() {
-  const int n = g_rec_pending;
-  if (n <= 0) return;
+  if (g_rec_pending <= 0 || g_win == nullptr) return;
+  const unsigned long long f0 = __builtin_ia32_rdtsc();
+  Window& W = *g_win;
+  const int n = W.n;
   g_rec_pending = 0;                                  // before any use of the stream below
   Ring& r = g_ring;
+  if (*(volatile unsigned*)r.host_flag != 0) {        // an earlier launch left its barrier: its results are incomplete
+    (void)hipStreamSynchronize(g_stream_raw);
+    (void)hipMemset(r.sync, 0, 2 * sizeof(unsigned long long));
+    *r.host_flag = 0; r.sync_base = 0;
+    window_reset(W);
+    LH_FAIL("command list: a barrier between workgroups timed out; the commands of that buffer did not all run");
+    return;
+  }
+  LhCmd* out = r.host[r.cur];
+  static int start[CL_BUF_CMDS + 2];
+  for (int l = 0; l <= W.top + 1; l++) start[l] = 0;
+  for (int i = 0; i < n; i++) start[W.level[i] + 1]++;
+  for (int l = 1; l <= W.top + 1; l++) start[l] += start[l - 1];
+  static int rot_of_level[CL_BUF_CMDS + 2], owner_of_level[CL_BUF_CMDS + 2], split_of_level[CL_BUF_CMDS + 2];
+  static bool seen[CL_BUF_CMDS + 2];
+  for (int l = 0; l <= W.top; l++) { rot_of_level[l] = 0; owner_of_level[l] = 0; split_of_level[l] = 0; seen[l] = false; }
+  for (int i = 0; i < n; i++) {
+    const int l = W.level[i];
+    LhCmd& d = out[start[l]++];
+    d = W.cmd[i];
+    // a command that one workgroup runs alone goes to the next workgroup in turn; its first elements to wavefront `rot`
+    // a command that one workgroup runs alone goes to the next workgroup in turn, its first elements to the next free wavefront
+    // there; the pieces of a command split over all workgroups start where those of the level's previous split command ended
+    const int groups = g_deterministic ? 1 : r.groups;      // one workgroup adds in a fixed order; several combine transposed products with atomic adds
+    int owner = 0, start;
+    if (groups > 1 && cmd_splits(W.cmd[i])) {
+      start = split_of_level[l] % (groups * (CL_THREADS / 64));
+      split_of_level[l] += cmd_waves(W.cmd[i]);
+    } else {
+      owner = owner_of_level[l] % groups;
+      start = rot_of_level[l] & 15;
+      owner_of_level[l]++;
+      if (owner_of_level[l] % groups == 0) rot_of_level[l] = (rot_of_level[l] + cmd_waves(W.cmd[i])) & 15;
+    }
+    d.op = W.cmd[i].op | ((seen[l] || l == 1) ? 0 : CL_BARRIER) | (start << CL_ROT_SHIFT) | (owner << CL_OWNER_SHIFT);
+    seen[l] = true;
+  }
+  const int groups = g_deterministic ? 1 : r.groups;
+  const int barriers = W.top > 1 ? W.top - 1 : 0;
+  g_ring.levels += W.top;
+  window_reset(W);
   ProfScope prof_(CAT_CMDLIST);
-  hipLaunchKernelGGL(k_cmdlist, dim3(1), dim3(CL_THREADS), 0, g_stream_raw, (const LhCmd*)r.dev[r.cur], n);
+  hipLaunchKernelGGL(k_cmdlist, dim3(groups), dim3(CL_THREADS), 0, g_stream_raw, (const LhCmd*)r.dev[r.cur], n, r.sync, r.sync_base, r.host_flag_dev);
+  if (groups > 1) r.sync_base += (unsigned long long)barriers * (unsigned long long)groups;
   hipError_t e = hipGetLastError();
   if (e == hipSuccess) e = hipEventRecord(r.done[r.cur], g_stream_raw);
   if (e != hipSuccess) { LH_FAIL("command list launch: %s", hipGetErrorString(e)); return; }
@@ -283,20 +589,45 @@ void rec_flush() {
   r.launches++;
   r.cur = (r.cur + 1) % CL_NBUF;
   if (r.busy[r.cur]) {                                // the buffer about to be refilled must have been consumed
+    const unsigned long long w0 = __builtin_ia32_rdtsc();
     (void)hipEventSynchronize(r.done[r.cur]);
+    g_tsc_wait += __builtin_ia32_rdtsc() - w0;
     r.busy[r.cur] = false;
   }
+  g_tsc_flush += __builtin_ia32_rdtsc() - f0;
 }
-LhCmd* rec_next() {
-  if (!g_ring.ready) return nullptr;
-  if (g_rec_pending == CL_BUF_CMDS) { rec_flush(); if (failed()) return nullptr; }
-  g_ring.recorded++;
-  return &g_ring.host[g_ring.cur][g_rec_pending++];
+// Appends a command: works out its level from the ranges it touches, then notes those ranges.
+bool rec_push(const LhCmd& c) {
+  if (!g_ring.ready || g_win == nullptr) return false;
+  const unsigned long long tsc0 = __builtin_ia32_rdtsc();
+  struct Acc { unsigned long long t0; ~Acc() { g_tsc_push += __builtin_ia32_rdtsc() - t0; } } acc_{tsc0};
+  Window& W = *g_win;
+  Extent x[4];
+  const int k = cmd_extents(c, x);
+  for (int attempt = 0; attempt < 2; attempt++) {
+    if (W.n == CL_BUF_CMDS) { rec_flush(); if (failed()) return false; }
+    int lv = 0;
+    for (int i = 0; i < k; i++) { const int v = conflict_level(W, x[i]); if (v > lv) lv = v; }
+    lv += 1;
+    bool ok = true;
+    for (int i = 0; i < k && ok; i++) ok = note_extent(W, x[i], lv);
+    if (!ok) { rec_flush(); if (failed()) return false; continue; }       // a table is full: start a new buffer (which begins with a barrier)
+    W.cmd[W.n] = c; W.level[W.n] = (uint16_t)lv; W.n++;
+    if (lv > W.top) W.top = lv;
+    g_rec_pending = W.n;
+    g_ring.recorded++;
+    return true;
+  }
+  LH_FAIL("command list: a single command overflows the dependence tables");
+  return false;
 }
 void cmdlist_release() {
   g_rec_on = 0; g_rec_pending = 0;
+  delete g_win; g_win = nullptr;
   if (!g_ring.ready) return;
   for (int i = 0; i < CL_NBUF; i++) { (void)hipEventDestroy(g_ring.done[i]); (void)hipHostFree(g_ring.host[i]); }
+  if (g_ring.sync) (void)hipFree(g_ring.sync);
+  if (g_ring.host_flag) (void)hipHostFree(g_ring.host_flag);
   g_ring = Ring{};
 }
 }  // namespace lh
@@ -307,11 +638,14 @@ void lh_cmdlist_begin(void) {
   LH_REQUIRE(!g_capturing, "lh_cmdlist_begin: a graph is being recorded (the command buffers cannot be replayed)");
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_cmdlist_begin on the side stream");
   if (!ring_init()) return;
+  if (g_win == nullptr) { g_win = new Window(); for (int i = 0; i < HASH_N; i++) g_win->slot[i].epoch = 0; g_win->epoch = 0; window_reset(*g_win); }
   g_rec_on = 1;
 }
 void lh_cmdlist_end(void) {
   rec_flush();
   g_rec_on = 0;
+  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld commands in %lld levels, %lld launches\n", (long long)g_ring.recorded, (long long)g_ring.levels, (long long)g_ring.launches);
+  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list host cycles: push %.1f M (flush inside %.1f M, of which waiting for a free buffer %.1f M)\n", g_tsc_push * 1e-6, g_tsc_flush * 1e-6, g_tsc_wait * 1e-6);
 }
 void lh_cmdlist_stats(int64_t* recorded, int64_t* launches) {
   if (recorded) *recorded = g_ring.recorded;

@@ -115,14 +115,14 @@ struct LhCmd { int32_t op, i0, i1, i2; float f0, f1, f2, f3; void* p0; void* p1;
 constexpr int64_t REC_MAX_ELEMS = 1 << 16;        // element-wise operands up to this many elements are recorded
 constexpr int64_t REC_MAX_MATRIX = 1 << 17;       // matrix-vector operands up to this many matrix elements
 extern int g_rec_on;
-LhCmd* rec_next();                                 // the slot of the next command (launches a full buffer first); nullptr on error
+bool rec_push(const LhCmd& c);                     // appends a command (launches a full buffer first); false on error
 static inline bool rec_ok(int64_t n, int64_t limit = REC_MAX_ELEMS) { return g_rec_on && n <= limit; }
-static inline LhCmd* rec_cmd(int op, int i0, int i1, int i2, float f0, float f1, float f2, float f3,
+static inline bool rec_cmd(int op, int i0, int i1, int i2, float f0, float f1, float f2, float f3,
                              const void* p0, const void* p1, const void* p2, const void* p3) {
-  LhCmd* c = rec_next();
-  if (c) { c->op = op; c->i0 = i0; c->i1 = i1; c->i2 = i2; c->f0 = f0; c->f1 = f1; c->f2 = f2; c->f3 = f3;
-           c->p0 = (void*)p0; c->p1 = (void*)p1; c->p2 = (void*)p2; c->p3 = (void*)p3; }
-  return c;
+  LhCmd c;
+  c.op = op; c.i0 = i0; c.i1 = i1; c.i2 = i2; c.f0 = f0; c.f1 = f1; c.f2 = f2; c.f3 = f3;
+  c.p0 = (void*)p0; c.p1 = (void*)p1; c.p2 = (void*)p2; c.p3 = (void*)p3;
+  return rec_push(c);
 }
 
 // Grid for a grid-stride streaming kernel: enough blocks to cover n at `per_block`

@@ -995,6 +995,60 @@ def test_command_list_keeps_program_order_around_other_kernels_and_wraps_its_buf
     _lib.check()
 
 
+def test_command_list_reordering_keeps_every_dependence(on_hip):
+    """The command list runs independent commands of a buffer side by side and dependent ones in order.  A random program of
+    several hundred small operations over a few buffers and their sub-ranges (reads after writes, writes after reads, writes
+    after writes; vectors inside a matrix another command updates as a whole; a scalar one command leaves for the next) must
+    give the bits of the same program issued one launch per operator, whose order is the program's."""
+    be = on_hip
+    lib = be.lib
+    rng = np.random.RandomState(77)
+    n_vec, vlen, m = 12, 150, 24
+
+    def program():
+        mark = be.getMallocAddr()
+        r = np.random.RandomState(5)
+        vecs = [be.fromHost((r.rand(vlen) + 0.5).astype(np.float32)) for _ in range(n_vec)]
+        mat = be.fromHost((r.rand(m * vlen) * 0.1).astype(np.float32))
+        scal = be.mallocArray(1)
+        ops = np.random.RandomState(9)
+        for step in range(600):
+            k = ops.randint(0, 9)
+            a, b_, c = (int(v) for v in ops.randint(0, n_vec, 3))
+            row = int(ops.randint(0, m))
+            if k == 0: lib.lh_geam(vecs[a].ptr, 0.5, vecs[b_].ptr, 0.5, vecs[c].ptr, vlen)                      # c = (a + b) / 2
+            elif k == 1: lib.lh_unary(B.TANH, vecs[a].ptr, vecs[c].ptr, vlen, -1.0, 1.0)
+            elif k == 2: lib.lh_geam(vecs[a].ptr, 1.0, mat.ptr + 4 * row * vlen, 0.25, vecs[a].ptr, vlen)          # reads a row of the matrix
+            elif k == 3: lib.lh_ger(m, vlen, vecs[a].ptr, vecs[b_].ptr, mat.ptr) if a != b_ else None               # updates the whole matrix (u = first m of a)
+            elif k == 4: lib.lh_sgemv(0, m, vlen, 0.01, mat.ptr, vlen, vecs[a].ptr, 0.0, vecs[c].ptr)                # first m elements of c
+            elif k == 5: lib.lh_sgemv(1, m, vlen, 0.01, mat.ptr, vlen, vecs[a].ptr, 1.0, vecs[c].ptr) if a != c else None
+            elif k == 6: lib.lh_fill(mat.ptr + 4 * row * vlen, 0.02 * (step % 7), vlen)                               # overwrites one row
+            elif k == 7:
+                lib.lh_dot_vv(vecs[a].ptr, vecs[b_].ptr, scal.ptr, vlen)
+                lib.lh_scalar_op(B.MUL, scal.ptr, scal.ptr, 1e-3, 1)
+                lib.lh_axpy_dev(vecs[c].ptr, scal.ptr, vecs[a].ptr, vlen) if a != c else None
+            else: lib.lh_geam(vecs[a].ptr, 1.0, vecs[b_].ptr + 4 * 50, -0.5, vecs[a].ptr, 64)                        # a[:64] -= b[50:114] / 2
+            # keep the values bounded: the matrix is halved after an update, a vector that was added to goes through tanh (in place)
+            if k == 3 and a != b_: lib.lh_scalar_op(B.MUL, mat.ptr, mat.ptr, 0.5, m * vlen)
+            if k in (2, 8): lib.lh_unary(B.TANH, vecs[a].ptr, vecs[a].ptr, vlen, -1.0, 1.0)
+            if k in (5, 7) and a != c: lib.lh_unary(B.TANH, vecs[c].ptr, vecs[c].ptr, vlen, -1.0, 1.0)
+        from lantern_amd import _lib
+        _lib.check()
+        out = [be.toHost(v, vlen).copy() for v in vecs] + [be.toHost(mat, m * vlen).copy()]
+        be.resetMallocAddr(mark)
+        return out
+
+    direct = program()
+    be.batchSmallOps(True)
+    try:
+        listed = program()
+    finally:
+        be.batchSmallOps(False)
+    assert all(np.isfinite(a).all() for a in direct)
+    for i, (a, b_) in enumerate(zip(listed, direct)):
+        assert_close(a, b_, rtol=2e-5, what="buffer %d" % i)
+
+
 # ---- residual join behind a batch norm: out = relu(bn(x) + shortcut) -----------------------------------
 @pytest.mark.parametrize("shape", [(8, 16, 28, 28), (3, 5, 7, 7), (4, 32, 1, 1), (16, 128, 112, 112)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("beta_sd", [0.0, 1.0, None], ids=["shortcut_grad_fresh", "shortcut_grad_accumulates", "shortcut_is_input"])
