@@ -30,6 +30,7 @@ PEAK_HBM_GBS = 8000.0
 PROFILED_TRAFFIC = {"bytes_per_launch": 151.1e6, "launches_per_step": 158}
 CATS = ["conv_fwd", "conv_bwd_data", "conv_bwd_filter", "gemm", "bn_fwd", "bn_bwd", "elementwise", "pool", "reduce", "optim", "fill", "rnn", "cmdlist"]
 
+TREE_C_PROGRAM = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "host_c", "_build", "treelstm_step")
 DEFAULT_BATCH = {"resnet50": 64, "squeezenet": 64, "lenet": 100, "treelstm": 1, "deepspeech2": 32}
 
 
@@ -161,8 +162,32 @@ def run_gpu(args):
     lib.lh_prof_enable(0)
     loss_val = float(tr.step().toCPU()[0]); tr.end_step()
     peak_gb = lib.lh_heap_peak() / 2 ** 30
+    c_host = None
+    c_dir = None
+    if args.workload == "treelstm" and os.path.exists(TREE_C_PROGRAM):
+        # the same loop as a plain-C host program over the C-ABI (what the reference's generated code is): fresh parameters of the
+        # same distribution, the same trees; it runs after this process has released the device
+        import tempfile
+        from lantern_amd.apps.treelstm import write_c_program_inputs
+        c_dir = tempfile.mkdtemp(prefix="lantern_treelstm_")
+        tr.close(); tr.end_step()
+        tr2, _, _ = make_trainer(args, args.batch)
+        write_c_program_inputs(c_dir, tr2)
+        tr2.close()
     be.cleanup()
-    return {"streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
+    if c_dir is not None:
+        import subprocess
+        r = subprocess.run([TREE_C_PROGRAM, os.path.join(c_dir, "params.bin"), os.path.join(c_dir, "trees.txt"), os.path.join(c_dir, "out.bin"),
+                            str(args.steps), str(args.warmup), "1"], capture_output=True, text=True, timeout=600)
+        if r.returncode != 0 or not r.stdout.startswith("trees_per_s"):
+            sys.exit("bench.py: the C host program failed: " + r.stdout + r.stderr)
+        f = r.stdout.split()
+        c_host = {"trees_per_s": float(f[1]), "ms_per_tree": float(f[3]), "host_issue_ms_per_tree": float(f[7])}
+        losses = np.fromfile(os.path.join(c_dir, "out.bin"), np.float32, count=args.steps)
+        assert np.isfinite(losses).all() and (losses > 0).all(), "the C host program's losses"
+        import shutil
+        shutil.rmtree(c_dir, ignore_errors=True)
+    return {"c_host": c_host, "streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
             "per_step": per_step, "desc": desc}
 
 
@@ -230,6 +255,13 @@ def main():
     g = run_gpu(args)
     ms_per_step = 1000.0 * g["sec"] / args.steps
     value = g["per_step"] * args.steps / g["sec"]
+    python_host = None
+    if g.get("c_host"):
+        # TreeLSTM issues ~7000 operator calls per tree: from Python the host is the bound, so the figure of the library is the
+        # one measured from the C host program; the Python mirror's is kept beside it
+        python_host = {"value": round(value, 2), "ms_per_step": round(ms_per_step, 3), "host_issue_ms_per_step": round(1000.0 * g["issue_sec"] / args.steps, 3)}
+        value, ms_per_step = g["c_host"]["trees_per_s"], g["c_host"]["ms_per_tree"]
+        g["issue_sec"] = g["c_host"]["host_issue_ms_per_tree"] * args.steps / 1000.0
     timed, work = g["timed"], g["work"]
     conv_ms = [timed[k][0] for k in ("conv_fwd", "conv_bwd_data", "conv_bwd_filter")]
     conv_calls = sum(timed[k][1] for k in ("conv_fwd", "conv_bwd_data", "conv_bwd_filter"))
@@ -238,8 +270,8 @@ def main():
         # list (one workgroup interpreting ~90 small operations per node), so the step is latency-bound, not HBM-bound
         t = timed["cmdlist"][0] / 1000.0
         achieved = work.get("gemv_bytes", 0.0) / t / 1e9 if t > 0 else 0.0
-        roof = {"bound": "hbm", "kernel": "k_cmdlist (%d interpreter launches/step running the gemv / rank-1 update / element-wise commands; "
-                                          "one workgroup, latency-bound at these sizes)" % timed["cmdlist"][1],
+        roof = {"bound": "hbm", "kernel": "k_cmdlist (%d interpreter launches/step running the gemv / rank-1 update / element-wise commands level by level "
+                                          "over 16 workgroups; bound by memory round trips and the barrier per level at these sizes; timed under the Python mirror)" % timed["cmdlist"][1],
                 "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": None,
                 "bytes_per_step": work.get("gemv_bytes", 0.0), "ms_per_step": round(timed["cmdlist"][0], 3)}
     else:
@@ -289,6 +321,9 @@ def main():
                    "reductions": "deterministic (two-pass, rule-chosen plans)" if args.deterministic else "atomic combine, measured plans"},
         "roofline": roof,
     }
+    if python_host is not None:
+        out["config"]["host"] = "plain-C host program over the C-ABI (tests/host_c/treelstm_step.c): the reference's generated-code shape, command list on"
+        out["python_mirror_host"] = python_host
     if g["resident_sec"] is not None:
         out["resident_input"] = {"value": round(g["per_step"] * args.steps / g["resident_sec"], 2), "ms_per_step": round(1000.0 * g["resident_sec"] / args.steps, 3),
                                  "note": "the same steps with the batch resident on the device: no upload, no loss read-back"}

@@ -159,3 +159,30 @@ class Trainer:
         if self.batching:
             get_backend().batchSmallOps(False)
             self.batching = False
+
+
+def write_c_program_inputs(directory, trainer):
+    """The two input files of the plain-C host program of this training loop (tests/host_c/treelstm_step.c) from a freshly
+    built Trainer: params.bin (sizes, embedding table, the 22 parameter tensors in creation order) and trees.txt (the
+    reference's array_tree.txt layout).  Returns the parameter TensorRs in file order."""
+    import os
+    model = trainer.model
+    named = model.namedParameters()
+    names = [n.split("/", 1)[1] for n, _ in named]
+    assert names == ["leaf/Wi", "leaf/bi", "leaf/Wo", "leaf/bo", "leaf/Wu", "leaf/bu"] + ["node/" + n for n in Node.NAMES] + ["output/Why", "output/by"], names
+    params = [p for _, p in named]
+    emb = trainer.embedding.toCPU()
+    vocab, e = emb.shape
+    hidden, classes = params[1].x.shape[0], params[-1].x.shape[0]
+    with open(os.path.join(str(directory), "params.bin"), "wb") as f:
+        np.array([vocab, e, hidden, classes], np.int32).tofile(f)
+        emb.astype(np.float32).tofile(f)
+        for p in params:
+            p.x.toCPU().astype(np.float32).tofile(f)
+    with open(os.path.join(str(directory), "trees.txt"), "w") as f:
+        f.write("%d\n" % len(trainer.trees))
+        for t in trainer.trees:
+            f.write("%d\n" % len(t[0]))
+            for arr in t:
+                f.write(" ".join(str(int(v)) for v in arr) + "\n")
+    return params

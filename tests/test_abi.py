@@ -114,27 +114,9 @@ TREE_BIN = os.path.join(HOST_C, "_build", "treelstm_step")
 
 
 def write_treelstm_inputs(tmp_path, trainer, trees):
-    """The C program's two input files from a freshly built mirror trainer (tests and bench.py use the same writer)."""
-    import numpy as np
-    model = trainer.model
-    params = [p for _, p in model.namedParameters()]
-    names = [n.split("/", 1)[1] for n, _ in model.namedParameters()]
-    assert names == ["leaf/Wi", "leaf/bi", "leaf/Wo", "leaf/bo", "leaf/Wu", "leaf/bu"] + ["node/" + n for n in type(model.node).NAMES] + ["output/Why", "output/by"], names
-    emb = trainer.embedding.toCPU()
-    vocab, e = emb.shape
-    hidden, classes = params[1].x.shape[0], params[-1].x.shape[0]
-    with open(tmp_path / "params.bin", "wb") as f:
-        np.array([vocab, e, hidden, classes], np.int32).tofile(f)
-        emb.astype(np.float32).tofile(f)
-        for p in params:
-            p.x.toCPU().astype(np.float32).tofile(f)
-    with open(tmp_path / "trees.txt", "w") as f:
-        f.write("%d\n" % len(trees))
-        for t in trees:
-            f.write("%d\n" % len(t[0]))
-            for arr in t:
-                f.write(" ".join(str(int(v)) for v in arr) + "\n")
-    return params
+    from lantern_amd.apps.treelstm import write_c_program_inputs
+    assert trees is trainer.trees
+    return write_c_program_inputs(tmp_path, trainer)
 
 
 def test_c_treelstm_program_links():
