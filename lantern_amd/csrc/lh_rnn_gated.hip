@@ -140,10 +140,13 @@ void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const floa
   LH_REQUIRE(cx == nullptr || mode == 2, "lh_rnn_gated_fwd: only the LSTM has a cell state");
   LH_REQUIRE(x && w && y && reserve, "lh_rnn_gated_fwd: null operand");
   const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
-  const size_t gh_bytes = (size_t)B * G * sizeof(float);
-  float* gh = (float*)lh_malloc_uninit(gh_bytes);
-  if (gh == nullptr) return;
-  for (int d = 0; d < D; d++) {
+  const size_t gh_bytes = (size_t)D * B * G * sizeof(float);
+  float* gh_all = (float*)lh_malloc_uninit(gh_bytes);
+  if (gh_all == nullptr) return;
+  // The two directions of a bidirectional layer share nothing but the input: the reverse one runs on the library's second
+  // stream beside the forward one (in line when that stream is off, while a graph is recorded or in deterministic mode).
+  auto run_direction = [&](int d) {
+    float* gh = gh_all + (size_t)d * B * G;
     const float* Wih = w + d * dir_params(mode, I, H);
     const float* Whh = Wih + (size_t)G * I; const float* bih = Whh + (size_t)G * H; const float* bhh = bih + G;
     float* act = reserve + d * dir_reserve(mode, T, B, H);
@@ -165,7 +168,10 @@ void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const floa
         hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh, hp, ldp,
                            aux + (size_t)t * B * H, h, B, H, ldh);
     }
-  }
+  };
+  const bool fork = D == 2 && g_stream_cur == g_stream_raw;
+  if (fork) { lh_side_begin(); run_direction(1); lh_side_end(); run_direction(0); lh_side_join(); }
+  else for (int d = 0; d < D; d++) run_direction(d);
   lh_free_top(gh_bytes);       // stream order: the kernels above run before anything that reuses the space
   LH_CHECK_LAUNCH();
 }
@@ -180,11 +186,14 @@ void lh_rnn_gated_bwd_init(int mode, const float* x, const float* hx, const floa
   // scratch from the top of the arena: recurrent gradient [B, H], cell gradient [B, H], column sums [2G],
   // and for the GRU the hidden-side pre-activation gradients of every step [T, B, G]
   const size_t n_bh = (size_t)B * H, n_dgh = mode == 3 ? (size_t)T * B * G : 0;
-  const size_t bytes = (2 * n_bh + 2 * (size_t)G + n_dgh) * sizeof(float);
+  const size_t per_dir = 2 * n_bh + 2 * (size_t)G + n_dgh;
+  const size_t bytes = (size_t)D * per_dir * sizeof(float);
   float* scratch = (float*)lh_malloc_uninit(bytes);
   if (scratch == nullptr) return;
-  float* carry = scratch; float* dc = carry + n_bh; float* colsum = dc + n_bh; float* dgh = colsum + 2 * (size_t)G;
-  for (int d = 0; d < D; d++) {
+  // each direction has its own scratch and its own part of dw, and runs on its own stream (see the forward pass); the input
+  // gradient, to which both add, is formed afterwards on the caller's stream
+  auto run_direction = [&](int d) {
+    float* carry = scratch + (size_t)d * per_dir; float* dc = carry + n_bh; float* colsum = dc + n_bh; float* dgh = colsum + 2 * (size_t)G;
     const size_t off = d * dir_params(mode, I, H);
     const float* Wih = w + off; const float* Whh = Wih + (size_t)G * I;
     float* dWih = dw + off; float* dWhh = dWih + (size_t)G * I; float* dbih = dWhh + (size_t)G * H; float* dbhh = dbih + G;
@@ -223,8 +232,13 @@ void lh_rnn_gated_bwd_init(int mode, const float* x, const float* hx, const floa
     hipLaunchKernelGGL(k_add_into, dim3((unsigned)cdiv(G, TPB)), dim3(TPB), 0, g_stream, dbih, colsum, G);
     if (mode == 3) lh_sum_dim(dgh, colsum + G, 1, T * B, G);
     hipLaunchKernelGGL(k_add_into, dim3((unsigned)cdiv(G, TPB)), dim3(TPB), 0, g_stream, dbhh, mode == 3 ? colsum + G : colsum, G);
-    if (dx) lh_sgemm(0, 0, T * B, I, G, 1.0f, act, G, Wih, I, d == 0 ? beta_dx : 1.0f, dx, I);
-  }
+  };
+  const bool fork = D == 2 && g_stream_cur == g_stream_raw;
+  if (fork) { lh_side_begin(); run_direction(1); lh_side_end(); run_direction(0); lh_side_join(); }
+  else for (int d = 0; d < D; d++) run_direction(d);
+  if (dx)
+    for (int d = 0; d < D; d++)
+      lh_sgemm(0, 0, T * B, I, G, 1.0f, reserve + d * dir_reserve(mode, T, B, H), G, w + d * dir_params(mode, I, H), I, d == 0 ? beta_dx : 1.0f, dx, I);
   lh_free_top(bytes);
   LH_CHECK_LAUNCH();
 }
