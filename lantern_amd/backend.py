@@ -464,17 +464,25 @@ class BackendHIP(Backend):
         self.lib.lh_bn_infer(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, N, C, HW, eps); _lib.check()
         return y
 
+    @staticmethod
+    def _bn_one_pass(N, C, HW):
+        """The library's rule for running a batch norm as one launch with a channel per block (lh_bn.hip: small_fits): the
+        channel's N*HW elements fit one block's registers and there are enough channels for the chip.  The tensor is then
+        read once, not twice (the byte counts below are what the kernels that run must move)."""
+        units = N * (HW // 4) if HW % 4 == 0 else N * HW
+        return units <= 16 * 256 and C >= 128
+
     def batchNormTraining(self, x, scale, bias, rmean, rvar, N, C, HW, eps=1e-5, factor=0.1):
         y = self.mallocArray(N * C * HW, zero=False)
         sm = self.mallocArray(C, zero=False); si = self.mallocArray(C, zero=False)
         self.lib.lh_bn_train_fwd(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
-        if self.count_work: self._count("bn_fwd_bytes", 12.0 * N * C * HW)       # x read for the statistics, read again, y written
+        if self.count_work: self._count("bn_fwd_bytes", (8.0 if self._bn_one_pass(N, C, HW) else 12.0) * N * C * HW)       # x read for the statistics, read again, y written
         return y, sm, si
 
     def batchNormTraining_into(self, x, scale, bias, rmean, rvar, y, sm, si, N, C, HW, relu, eps=1e-5, factor=0.1):
         f = self.lib.lh_bn_train_fwd_relu if relu else self.lib.lh_bn_train_fwd
         f(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
-        if self.count_work: self._count("bn_fwd_bytes", 12.0 * N * C * HW)
+        if self.count_work: self._count("bn_fwd_bytes", (8.0 if self._bn_one_pass(N, C, HW) else 12.0) * N * C * HW)
 
     def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0, y_relu=None, bias=None):
         """y_relu: the layer's output went through a fused in-place relu; `bias` (the layer's beta) lets the
@@ -487,7 +495,7 @@ class BackendHIP(Backend):
             self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
         _lib.check()
         # x and dy read for the two sums, read again, dx written (and read first when it accumulates)
-        if self.count_work: self._count("bn_bwd_bytes", (20.0 + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0)) * N * C * HW)
+        if self.count_work: self._count("bn_bwd_bytes", ((12.0 if self._bn_one_pass(N, C, HW) else 20.0) + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0)) * N * C * HW)
 
     def batchNormTraining_add_relu_into(self, x, scale, bias, rmean, rvar, shortcut, out, sm, si, N, C, HW, eps=1e-5, factor=0.1):
         self.lib.lh_bn_stats(x.ptr, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, N, C, HW, eps, factor)
@@ -507,7 +515,10 @@ class BackendHIP(Backend):
         # pass 1 reads x, out, dout and writes the masked gradient (to the shortcut's buffer, or over dout); pass 2 reads x and the
         # masked gradient and writes dx: 28 B per element, plus a read for each output that accumulates
         if self.count_work:
-            self._count("bn_bwd_bytes", (28.0 + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0) + (8.0 if (sd is not None and beta_sd != 0.0) else 0.0)) * N * C * HW)
+            if self._bn_one_pass(N, C, HW):      # x, out, dout read once; the shortcut's gradient and dx written (each read first when it accumulates)
+                self._count("bn_bwd_bytes", (16.0 + (4.0 if sd is not None else 0.0) + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0) + (4.0 if (sd is not None and beta_sd != 0.0) else 0.0)) * N * C * HW)
+            else:
+                self._count("bn_bwd_bytes", (28.0 + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0) + (8.0 if (sd is not None and beta_sd != 0.0) else 0.0)) * N * C * HW)
 
     def add_into(self, a, b, out, n, relu):
         if relu: self.lib.lh_add_relu(a.ptr, b.ptr, out.ptr, n)

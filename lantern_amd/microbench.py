@@ -81,10 +81,11 @@ def stream(be, N=64):
         g = be.mallocArray(Cc); b = be.mallocArray(Cc); sm = be.mallocArray(Cc); si = be.mallocArray(Cc); dg = be.mallocArray(Cc); db = be.mallocArray(Cc)
         lib.lh_fill(g.ptr, 1.0, Cc)
         lib.lh_bn_train_fwd_relu(x.ptr, g.ptr, b.ptr, 0, 0, y.ptr, sm.ptr, si.ptr, N, Cc, HW, 1e-5, 0.1)
+        one = be._bn_one_pass(N, Cc, HW)      # a channel fits one block: the tensor is read once (forward 8, backward 12 bytes per element)
         ops = {      # name: (callable, algorithmic bytes per element)
-            "bn_fwd+relu": (lambda: lib.lh_bn_train_fwd_relu(x.ptr, g.ptr, b.ptr, 0, 0, y.ptr, sm.ptr, si.ptr, N, Cc, HW, 1e-5, 0.1), 12),
-            "bn_bwd+relu": (lambda: lib.lh_bn_bwd_relu(x.ptr, y.ptr, dy.ptr, g.ptr, b.ptr, sm.ptr, si.ptr, dx.ptr, 0.0, dg.ptr, db.ptr, N, Cc, HW), 20),
-            "bn_bwd": (lambda: lib.lh_bn_bwd(x.ptr, dy.ptr, g.ptr, sm.ptr, si.ptr, dx.ptr, 0.0, dg.ptr, db.ptr, N, Cc, HW), 20),
+            "bn_fwd+relu": (lambda: lib.lh_bn_train_fwd_relu(x.ptr, g.ptr, b.ptr, 0, 0, y.ptr, sm.ptr, si.ptr, N, Cc, HW, 1e-5, 0.1), 8 if one else 12),
+            "bn_bwd+relu": (lambda: lib.lh_bn_bwd_relu(x.ptr, y.ptr, dy.ptr, g.ptr, b.ptr, sm.ptr, si.ptr, dx.ptr, 0.0, dg.ptr, db.ptr, N, Cc, HW), 12 if one else 20),
+            "bn_bwd": (lambda: lib.lh_bn_bwd(x.ptr, dy.ptr, g.ptr, sm.ptr, si.ptr, dx.ptr, 0.0, dg.ptr, db.ptr, N, Cc, HW), 12 if one else 20),
             "add+relu": (lambda: lib.lh_add_relu(x.ptr, dy.ptr, y.ptr, n), 12),
             "add+relu grad": (lambda: lib.lh_add_relu_grad(y.ptr, dy.ptr, dx.ptr, 0.0, d2.ptr, 0.0, n), 16),
             "relu": (lambda: lib.lh_unary(0, x.ptr, x.ptr, n, 0.0, 0.0), 8),
