@@ -27,7 +27,7 @@ import numpy as np  # noqa: E402,F401
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 # conv kernels of the headline step under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/resnet50_b64_hbm_traffic_and_mfma_counters.md)
-PROFILED_TRAFFIC = {"bytes_per_launch": 151.1e6, "launches_per_step": 158}
+PROFILED_TRAFFIC = {"bytes_per_launch": 152.3e6, "launches_per_step": 158}
 CATS = ["conv_fwd", "conv_bwd_data", "conv_bwd_filter", "gemm", "bn_fwd", "bn_bwd", "elementwise", "pool", "reduce", "optim", "fill", "rnn", "cmdlist"]
 
 TREE_C_PROGRAM = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "host_c", "_build", "treelstm_step")
