@@ -36,6 +36,7 @@ constexpr int CL_OWNER_SHIFT = 24;            // the workgroup (0..255) that run
 constexpr int CL_MAX_GROUPS = 64;
 constexpr long CL_SPIN_LIMIT = 40000000L;     // polls of a grid barrier before a workgroup gives up (far beyond any real wait)
 
+static bool g_chains = true;          // LH_CMDLIST_CHAINS=0 in the environment: every dependent command opens a new level
 struct Ring {
   LhCmd* host[CL_NBUF]; LhCmd* dev[CL_NBUF]; hipEvent_t done[CL_NBUF]; bool busy[CL_NBUF];
   int cur; bool ready;
@@ -406,6 +407,7 @@ static bool ring_init() {
   // 16 costs 3.5 us against 2.5 us for one workgroup's own device-scope fences (6 us over 32).  LH_CMDLIST_GROUPS overrides.
   int groups = 16;
   if (const char* e = getenv("LH_CMDLIST_GROUPS")) groups = atoi(e);
+  if (const char* e = getenv("LH_CMDLIST_CHAINS")) g_chains = atoi(e) != 0;
   if (groups < 1) groups = 1;
   if (groups > CL_MAX_GROUPS) groups = CL_MAX_GROUPS;
   if (groups > g_num_cu / 4) groups = g_num_cu / 4 > 0 ? g_num_cu / 4 : 1;       // all workgroups of a launch must be resident together
@@ -446,6 +448,14 @@ static int cmd_extents(const LhCmd& c, Extent* o) {
   return k;
 }
 // How many wavefronts of work a command is (where the next command of its level should start).
+// Element i of every operand is handled by lane i mod 1024 (see "Chains" below).
+static bool cmd_lanewise(const LhCmd& c) {
+  switch (c.op) {
+    case CL_FILL: case CL_COPY: case CL_GEAM: case CL_SCALAR: case CL_BIN: case CL_ACC: case CL_ACCNEG: case CL_ACCMUL:
+    case CL_UNARY: case CL_UNARY_GRAD: case CL_ADAGRAD: case CL_SGD: return true;
+    default: return false;
+  }
+}
 static bool cmd_splits(const LhCmd& c) { return c.op == CL_GEMV_N || c.op == CL_GER || (c.op == CL_GEMV_T && c.f1 == 1.0f); }
 static int cmd_waves(const LhCmd& c) {
   switch (c.op) {
@@ -461,9 +471,15 @@ static int cmd_waves(const LhCmd& c) {
 // larger ranges (matrices, zero fills) in a short table of distinct ranges.  A level is a uint16: 1 + highest level touched.
 constexpr uintptr_t SMALL_BYTES = 4096;
 constexpr int HASH_N = 65536, BIG_N = 96;
+// Chains.  An element-wise command gives element i of every operand to the same lane (thread i mod 1024 of the workgroup and
+// wavefront rotation it runs on).  If everything such a command must follow at the highest level L is ONE chain of element-wise
+// commands, through ranges that start at the very addresses this command's operands start at, then each lane only ever needs what
+// it read or wrote itself, program order within the lane is enough, and the command joins that chain AT level L (same workgroup,
+// same rotation, recording order) instead of opening level L + 1: bias add, second product's add and activation of a gate are one
+// level, not three.
 struct Window {
-  LhCmd cmd[CL_BUF_CMDS]; uint16_t level[CL_BUF_CMDS]; int n; int top;       // top: highest level handed out
-  struct Slot { uintptr_t key; uint32_t epoch; uint16_t w, r; } slot[HASH_N]; uint32_t epoch;
+  LhCmd cmd[CL_BUF_CMDS]; uint16_t level[CL_BUF_CMDS]; int16_t chain[CL_BUF_CMDS]; int n; int top, nchains;       // top: highest level handed out
+  struct Slot { uintptr_t key, wbase, rbase; uint32_t epoch; uint16_t w, r; int16_t wchain, rchain; } slot[HASH_N]; uint32_t epoch;
   struct Big { uintptr_t s, e; uint16_t w, r; } big[BIG_N]; int nbig;
   struct Small { uintptr_t s, e; uint16_t level; bool w; } small[CL_BUF_CMDS * 4]; int nsmall;
   uintptr_t small_lo, small_hi;                                               // bounding box of the small ranges
@@ -471,44 +487,59 @@ struct Window {
 static Window* g_win = nullptr;
 
 static void window_reset(Window& W) {
-  W.n = 0; W.top = 0; W.nbig = 0; W.nsmall = 0; W.small_lo = ~(uintptr_t)0; W.small_hi = 0;
+  W.n = 0; W.top = 0; W.nchains = 0; W.nbig = 0; W.nsmall = 0; W.small_lo = ~(uintptr_t)0; W.small_hi = 0;
   if (++W.epoch == 0) { for (int i = 0; i < HASH_N; i++) W.slot[i].epoch = 0; W.epoch = 1; }
 }
 static inline Window::Slot* slot_of(Window& W, uintptr_t block, bool create) {
   uint32_t h = (uint32_t)((block * 0x9E3779B97F4A7C15ull) >> 48) & (HASH_N - 1);
   for (int probe = 0; probe < HASH_N; probe++, h = (h + 1) & (HASH_N - 1)) {
     Window::Slot& sl = W.slot[h];
-    if (sl.epoch != W.epoch) { if (!create) return nullptr; sl.key = block; sl.epoch = W.epoch; sl.w = sl.r = 0; return &sl; }
+    if (sl.epoch != W.epoch) { if (!create) return nullptr; sl.key = block; sl.epoch = W.epoch; sl.w = sl.r = 0; sl.wchain = sl.rchain = -1; sl.wbase = sl.rbase = 0; return &sl; }
     if (sl.key == block) return &sl;
   }
   return nullptr;
 }
-// The highest level among earlier commands of the window that `x` must come after.
-static int conflict_level(Window& W, const Extent& x) {
-  int lv = 0;
+// What a command must follow: the highest level among the earlier commands of the window it conflicts with, and whether all of
+// its conflicts AT that level are with one chain through identically based ranges (then it may join that chain).
+struct Conflict {
+  int lv = 0, chain = -1; bool one_chain = false;
+  void see(int v, int ch, bool same_base) {
+    if (v <= 0) return;
+    if (v > lv) { lv = v; chain = ch; one_chain = same_base && ch >= 0; }
+    else if (v == lv && (!same_base || ch != chain)) one_chain = false;
+  }
+};
+static void conflicts_of(Window& W, const Extent& x, Conflict& c) {
   for (int i = 0; i < W.nbig; i++) {
     const Window::Big& b = W.big[i];
-    if (b.s < x.e && x.s < b.e) { const int v = x.w ? (b.w > b.r ? b.w : b.r) : b.w; if (v > lv) lv = v; }
+    if (b.s < x.e && x.s < b.e) c.see(x.w ? (b.w > b.r ? b.w : b.r) : b.w, -1, false);
   }
   if (x.e - x.s <= SMALL_BYTES) {
     for (uintptr_t blk = x.s >> 8; blk <= (x.e - 1) >> 8; blk++) {
       const Window::Slot* sl = slot_of(W, blk, false);
-      if (sl) { const int v = x.w ? (sl->w > sl->r ? sl->w : sl->r) : sl->w; if (v > lv) lv = v; }
+      if (!sl) continue;
+      c.see(sl->w, sl->wchain, sl->wbase == x.s);
+      if (x.w) c.see(sl->r, sl->rchain, sl->rbase == x.s);
     }
   } else if (x.s < W.small_hi && W.small_lo < x.e) {         // a large range over memory that small ranges of this window touch: rare
     for (int i = 0; i < W.nsmall; i++) {
       const Window::Small& m = W.small[i];
-      if (m.s < x.e && x.s < m.e && (x.w || m.w) && m.level > lv) lv = m.level;
+      if (m.s < x.e && x.s < m.e && (x.w || m.w)) c.see(m.level, -1, false);
     }
   }
-  return lv;
 }
-static bool note_extent(Window& W, const Extent& x, int level) {
+static bool note_extent(Window& W, const Extent& x, int level, int chain) {
   if (x.e - x.s <= SMALL_BYTES) {
     for (uintptr_t blk = x.s >> 8; blk <= (x.e - 1) >> 8; blk++) {
       Window::Slot* sl = slot_of(W, blk, true);
       if (!sl) return false;
-      if (x.w) { if (level > sl->w) sl->w = (uint16_t)level; } else if (level > sl->r) sl->r = (uint16_t)level;
+      if (x.w) {
+        if (level > sl->w) { sl->w = (uint16_t)level; sl->wchain = (int16_t)chain; sl->wbase = x.s; }
+        else if (level == sl->w && (sl->wchain != chain || sl->wbase != x.s)) sl->wchain = -1;       // two chains (or two alignments) at one level
+      } else {
+        if (level > sl->r) { sl->r = (uint16_t)level; sl->rchain = (int16_t)chain; sl->rbase = x.s; }
+        else if (level == sl->r && (sl->rchain != chain || sl->rbase != x.s)) sl->rchain = -1;
+      }
     }
     Window::Small& m = W.small[W.nsmall++];
     m.s = x.s; m.e = x.e; m.level = (uint16_t)level; m.w = x.w;
@@ -554,6 +585,8 @@ void rec_flush() {
   static int rot_of_level[CL_BUF_CMDS + 2], owner_of_level[CL_BUF_CMDS + 2], split_of_level[CL_BUF_CMDS + 2];
   static bool seen[CL_BUF_CMDS + 2];
   for (int l = 0; l <= W.top; l++) { rot_of_level[l] = 0; owner_of_level[l] = 0; split_of_level[l] = 0; seen[l] = false; }
+  static int chain_place[CL_BUF_CMDS + 1];
+  for (int ch = 0; ch < W.nchains; ch++) chain_place[ch] = -1;
   for (int i = 0; i < n; i++) {
     const int l = W.level[i];
     LhCmd& d = out[start[l]++];
@@ -566,11 +599,14 @@ void rec_flush() {
     if (groups > 1 && cmd_splits(W.cmd[i])) {
       start = split_of_level[l] % (groups * (CL_THREADS / 64));
       split_of_level[l] += cmd_waves(W.cmd[i]);
+    } else if (W.chain[i] >= 0 && chain_place[W.chain[i]] >= 0) {          // a later command of a chain: where its first one runs
+      owner = chain_place[W.chain[i]] >> 4; start = chain_place[W.chain[i]] & 15;
     } else {
       owner = owner_of_level[l] % groups;
       start = rot_of_level[l] & 15;
       owner_of_level[l]++;
       if (owner_of_level[l] % groups == 0) rot_of_level[l] = (rot_of_level[l] + cmd_waves(W.cmd[i])) & 15;
+      if (W.chain[i] >= 0) chain_place[W.chain[i]] = (owner << 4) | start;
     }
     d.op = W.cmd[i].op | ((seen[l] || l == 1) ? 0 : CL_BARRIER) | (start << CL_ROT_SHIFT) | (owner << CL_OWNER_SHIFT);
     seen[l] = true;
@@ -606,13 +642,16 @@ bool rec_push(const LhCmd& c) {
   const int k = cmd_extents(c, x);
   for (int attempt = 0; attempt < 2; attempt++) {
     if (W.n == CL_BUF_CMDS) { rec_flush(); if (failed()) return false; }
-    int lv = 0;
-    for (int i = 0; i < k; i++) { const int v = conflict_level(W, x[i]); if (v > lv) lv = v; }
-    lv += 1;
+    Conflict cf;
+    for (int i = 0; i < k; i++) conflicts_of(W, x[i], cf);
+    const bool lanewise = cmd_lanewise(c);
+    int lv, chain;
+    if (lanewise && cf.one_chain && g_chains) { lv = cf.lv; chain = cf.chain; }                    // joins the chain it follows
+    else { lv = cf.lv + 1; chain = lanewise ? W.nchains++ : -1; }
     bool ok = true;
-    for (int i = 0; i < k && ok; i++) ok = note_extent(W, x[i], lv);
+    for (int i = 0; i < k && ok; i++) ok = note_extent(W, x[i], lv, chain);
     if (!ok) { rec_flush(); if (failed()) return false; continue; }       // a table is full: start a new buffer (which begins with a barrier)
-    W.cmd[W.n] = c; W.level[W.n] = (uint16_t)lv; W.n++;
+    W.cmd[W.n] = c; W.level[W.n] = (uint16_t)lv; W.chain[W.n] = (int16_t)chain; W.n++;
     if (lv > W.top) W.top = lv;
     g_rec_pending = W.n;
     g_ring.recorded++;
