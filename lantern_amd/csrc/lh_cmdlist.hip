@@ -28,17 +28,24 @@ constexpr int CL_THREADS = 1024;
 constexpr int CL_CHUNK = 256;                 // commands staged in LDS at a time
 constexpr int CL_BUF_CMDS = 2048;              // commands per host buffer: a full buffer is launched while the host records the next
 constexpr int CL_NBUF = 32;
-constexpr int CL_OP_MASK = 0xff;              // LhCmd::op as the kernel sees it: operation | barrier flag | rotation << 12
-constexpr int CL_BARRIER = 0x100;             // first command of a level: a block barrier comes before it
-constexpr int CL_ROT_SHIFT = 12;              // 12 bits: where the command's work starts (a wavefront 0..15 of the owner, or, for a
-                                              // command split over all workgroups, one of their wavefronts taken together)
-constexpr int CL_OWNER_SHIFT = 24;            // the workgroup (0..255) that runs a command which is not split over all of them
+// Two op words per command.  Word 0: operation | flags | start << 12; word 1: owner | pieces << 8.
+constexpr int CL_OP_MASK = 0xff;
+constexpr int CL_BARRIER = 0x100;             // first command of a level: a barrier comes before it
+constexpr int CL_SPLIT = 0x200;               // a matrix command: its pieces are dealt round the wavefronts of all workgroups
+constexpr int CL_START_SHIFT = 12;            // where the command's work starts: a wavefront 0..15 of the owner or, for a split command,
+                                              // one of the wavefronts of all workgroups taken together
+constexpr int CL_PIECES_SHIFT = 8;            // word 1: how many wavefronts, counted from `start`, have work (a DOT needs them all)
 constexpr int CL_MAX_GROUPS = 64;
 constexpr long CL_SPIN_LIMIT = 40000000L;     // polls of a grid barrier before a workgroup gives up (far beyond any real wait)
 
 static bool g_chains = true;          // LH_CMDLIST_CHAINS=0 in the environment: every dependent command opens a new level
+// A buffer is CL_BUF_CMDS + 16 pairs of op words, then the commands.
+constexpr size_t CL_OPS_BYTES = (size_t)(CL_BUF_CMDS + 16) * sizeof(uint2);
+constexpr size_t CL_BUF_BYTES = CL_OPS_BYTES + sizeof(LhCmd) * CL_BUF_CMDS;
+static_assert(CL_OPS_BYTES % 64 == 0, "the commands start on a 64-byte boundary");
 struct Ring {
-  LhCmd* host[CL_NBUF]; LhCmd* dev[CL_NBUF]; hipEvent_t done[CL_NBUF]; bool busy[CL_NBUF];
+  char* host[CL_NBUF]; hipEvent_t done[CL_NBUF]; bool busy[CL_NBUF];
+  char* mirror;                      // device copy of the buffer being executed (launches are in stream order: one is enough)
   int cur; bool ready;
   int64_t recorded, launches, levels;
   unsigned long long* sync;          // device: [0] arrivals at grid barriers, [1] a workgroup gave up waiting
@@ -110,22 +117,16 @@ __device__ __forceinline__ float cl_wave_sum_dpp(float v) {
 }
 
 // Data pointers carry no __restrict__ and no const: a command may read what the command before it wrote.
-// `rot`: the wavefront that takes the command's first elements (commands of one level start on different wavefronts).
-// `grp` of `ngrp` workgroups: the matrix commands are cut by rows over all workgroups (one compute unit draws only some
-// 25 GB/s from memory, whatever its wavefronts do; the rows of a 150 x 150 matrix spread over 16 units take one memory
-// round trip); every other command is run by the one workgroup its `owner` field names.
-__device__ void cl_run(const LhCmd& c, const int rot, float* red /* [16][257] */, const int grp, const int ngrp) {
+// `gw` of `GW`: which of the wavefronts that share the command this one is.  An element-wise command belongs to one workgroup
+// (GW = 16, gw counted from the wavefront the host let it start on); the matrix commands are cut into pieces over the wavefronts
+// of all workgroups (one compute unit draws only some 25 GB/s from memory, whatever its wavefronts do; a 150 x 150 matrix spread
+// over 16 units takes one memory round trip): piece k goes to wavefront (start + k) mod GW, neighbouring wavefronts sit in
+// different workgroups, and the pieces of the commands of one level follow each other round the wavefronts, so a wavefront
+// rarely holds pieces of two of them and their memory round trips overlap instead of queueing.
+__device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int gw, const int GW) {
   constexpr int NT = CL_THREADS, NW = CL_THREADS / 64;
-  const int opc = c.op & CL_OP_MASK;
-  const bool split = ngrp > 1 && (opc == CL_GEMV_N || opc == CL_GER || (opc == CL_GEMV_T && c.f1 == 1.0f));
-  if (!split && ngrp > 1 && ((c.op >> CL_OWNER_SHIFT) & 0xff) != grp) return;
-  const int lane = threadIdx.x & 63, wave = split ? (int)(threadIdx.x >> 6) : (int)(((threadIdx.x >> 6) + NW - (rot & (NW - 1))) & (NW - 1)), t = wave * 64 + lane;
+  const int lane = threadIdx.x & 63, wave = gw, t = wave * 64 + lane;
   float* p0 = (float*)c.p0; float* p1 = (float*)c.p1; float* p2 = (float*)c.p2; float* p3 = (float*)c.p3;
-  // A matrix command is cut into pieces of a few rows; piece k goes to wavefront (rot + k) mod GW of all GW wavefronts that share
-  // the command (neighbouring ones in different workgroups).  The pieces of the commands of one level follow each other round the
-  // wavefronts, so a wavefront rarely holds pieces of two of them and their memory round trips overlap instead of queueing.
-  const int GW = split ? ngrp * NW : NW;
-  const int gw = split ? (wave * ngrp + grp + GW - rot % GW) % GW : wave;
   switch (opc) {
     case CL_ZERO16: { uint4* p = (uint4*)c.p0; const int n = c.i0; for (int i = t; i < n; i += NT) p[i] = make_uint4(0, 0, 0, 0); break; }
     case CL_FILL: { const int n = c.i0; const float v = c.f0; for (int i = t; i < n; i += NT) p0[i] = v; break; }
@@ -185,41 +186,31 @@ __device__ void cl_run(const LhCmd& c, const int rot, float* red /* [16][257] */
       }
       break;
     }
-    case CL_GEMV_T: {            // y[n] = alpha * A[m,n]^T x[m] + beta * y  (p0 = y, p1 = A, p2 = x): a wavefront takes five rows
-      // at a time, a lane four columns of each, all loads in flight together; the wavefronts' partial sums meet in LDS
+    case CL_GEMV_T: {            // y[n] = alpha * A[m,n]^T x[m] + beta * y  (p0 = y, p1 = A, p2 = x): a wavefront takes 16 columns
+      // (64 bytes of every row); lane l holds column l mod 16 of the rows congruent to l / 16 mod 4, up to 20 of them in flight
+      // together.  The four row classes meet by lane exchange: no LDS, no atomics, and the order of the sum is fixed.
       const int m = c.i0, n = c.i1, lda = c.i2; const float al = c.f0, be = c.f1;
       const __amdgpu_buffer_rsrc_t rA = cl_rsrc(p1, ((int64_t)(m - 1) * lda + n) * 4), rX = cl_rsrc(p2, (int64_t)m * 4);
-      for (int j0 = 0; j0 < n; j0 += 256) {
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        uint32_t co[4];
+      const int cj = lane & 15, rg = lane >> 4;
+      constexpr int RU = 20;
+      for (int j0 = gw * 16; j0 < n; j0 += GW * 16) {
+        const int j = j0 + cj;
+        const uint32_t co = j < n ? (uint32_t)j * 4u : CL_OOB;
+        float acc = 0.f;
+        for (int i0 = 0; i0 < m; i0 += 4 * RU) {
+          float xv[RU], av[RU];
 #pragma unroll
-        for (int q = 0; q < 4; q++) { const int j = j0 + q * 64 + lane; co[q] = j < n ? (uint32_t)j * 4u : CL_OOB; }
-        for (int i0 = gw * 5; i0 < m; i0 += 5 * GW) {
-          float xv[5], av[5][4];
-#pragma unroll
-          for (int u = 0; u < 5; u++) {
-            const uint32_t i = (uint32_t)(i0 + u);
+          for (int u = 0; u < RU; u++) {
+            const uint32_t i = (uint32_t)(i0 + u * 4 + rg);
             xv[u] = cl_ld(rX, i * 4u);                                                   // zero past m
-            const uint32_t ro = i * (uint32_t)lda * 4u;
-#pragma unroll
-            for (int q = 0; q < 4; q++) av[u][q] = cl_ld(rA, ro + co[q]);
+            av[u] = cl_ld(rA, i * (uint32_t)lda * 4u + co);                              // rows past m lie past the operand's end
           }
 #pragma unroll
-          for (int u = 0; u < 5; u++)
-#pragma unroll
-            for (int q = 0; q < 4; q++) acc[q] += av[u][q] * xv[u];
+          for (int u = 0; u < RU; u++) acc += av[u] * xv[u];
         }
-#pragma unroll
-        for (int q = 0; q < 4; q++) red[wave * 257 + q * 64 + lane] = acc[q];
-        __syncthreads();
-        if (t < 256 && j0 + t < n) {
-          float sv = 0.f;
-#pragma unroll
-          for (int w = 0; w < NW; w++) sv += red[w * 257 + t];
-          if (split) atomicAdd(p0 + j0 + t, al * sv);          // beta is 1: every workgroup adds the sum over its rows
-          else p0[j0 + t] = al * sv + (be == 0.f ? 0.f : be * p0[j0 + t]);
-        }
-        __syncthreads();
+        acc += __shfl_xor(acc, 16, 64);
+        acc += __shfl_xor(acc, 32, 64);
+        if (rg == 0 && j < n) p0[j] = al * acc + (be == 0.f ? 0.f : be * p0[j]);
       }
       break;
     }
@@ -256,6 +247,7 @@ __device__ void cl_run(const LhCmd& c, const int rot, float* red /* [16][257] */
       float acc = 0.f;
       for (int i = t; i < n; i += NT) acc += p1[i] * p2[i];
       acc = cl_wave_sum_all(acc);
+      __shared__ float red[NW];
       if (lane == 0) red[wave] = acc;
       __syncthreads();
       if (wave == 0) { float v = lane < NW ? red[lane] : 0.f; v = cl_wave_sum_all(v); if (lane == 0) p0[0] = v; }
@@ -355,33 +347,59 @@ __device__ __forceinline__ bool cl_grid_barrier(unsigned long long* sync, unsign
   return *lds_flag == 0;
 }
 
-// cmds: pinned host memory (read over the host link, a chunk at a time, the next chunk fetched while the current one runs),
-// in execution order: level by level, the first command of every level but the first flagged CL_BARRIER.  Every workgroup of
-// the launch walks the whole list.
-__global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const LhCmd* cmds, int n, unsigned long long* sync, unsigned long long sync_base, unsigned* host_flag) {
+// ops, cmds: the device copy of a buffer, in execution order: level by level, the first command of every level but the first
+// flagged CL_BARRIER.  The buffer is staged in LDS 256 commands at a time (the next chunk is fetched while the current one runs).
+// Every wavefront of every workgroup walks the op words (8 bytes a command, read one ahead and made wave-uniform, so the walk is
+// scalar work) and reads the 64-byte command only when it has a part in it: the op words say which workgroup owns the command or,
+// for a matrix command, at which wavefront of the launch its pieces start, and how many wavefronts have work.  A command that is
+// somebody else's costs a few scalar instructions.
+__global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const uint2* ops, const LhCmd* cmds, int n, unsigned long long* sync, unsigned long long sync_base,
+                                                        unsigned* host_flag) {
   __shared__ uint4 stage[CL_CHUNK * 4];                 // 256 commands of 64 bytes
-  __shared__ float red[(CL_THREADS / 64) * 257];
+  __shared__ uint2 sop[CL_CHUNK + 1];
   __shared__ int gave_up;
+  constexpr int NW = CL_THREADS / 64;
   const int t = threadIdx.x, grp = blockIdx.x, ngrp = gridDim.x;
+  const int w0 = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int all_w = ngrp * NW, my_w = w0 * ngrp + grp;  // this wavefront among all of the launch: neighbours sit in different workgroups
   const uint4* src = reinterpret_cast<const uint4*>(cmds);
   const int total16 = n * 4;
   unsigned long long arrived = sync_base;
   uint4 next = make_uint4(0, 0, 0, 0);
+  uint2 next_op = make_uint2(0, 0);
   if (t < total16) next = src[t];
+  if (t < CL_CHUNK) next_op = ops[t];                   // the op words are allocated past the last command
   for (int base = 0; base < n; base += CL_CHUNK) {
     stage[t] = next;
+    if (t < CL_CHUNK) sop[t] = next_op;
     const int nb = base + CL_CHUNK;
-    if (nb < n && nb * 4 + t < total16) next = src[nb * 4 + t];
+    if (nb < n) {
+      if (nb * 4 + t < total16) next = src[nb * 4 + t];
+      if (t < CL_CHUNK) next_op = ops[nb + t];
+    }
     __syncthreads();
     const int cnt = n - base < CL_CHUNK ? n - base : CL_CHUNK;
     const LhCmd* list = reinterpret_cast<const LhCmd*>(stage);
+    uint2 ahead = sop[0];
     for (int i = 0; i < cnt; i++) {
-      const int op = list[i].op;                        // uniform: every thread reads the same LDS word
+      const uint32_t op = __builtin_amdgcn_readfirstlane(ahead.x), who = __builtin_amdgcn_readfirstlane(ahead.y);
+      ahead = sop[i + 1];
       if (op & CL_BARRIER) {                            // the level before is complete and its stores are visible
         if (ngrp == 1) __syncthreads();
         else { arrived += (unsigned long long)ngrp; if (!cl_grid_barrier(sync, arrived, &gave_up, host_flag)) return; }
       }
-      cl_run(list[i], (op >> CL_ROT_SHIFT) & 0xfff, red, grp, ngrp);
+      const int start = (int)(op >> CL_START_SHIFT), pieces = (int)(who >> CL_PIECES_SHIFT);
+      int gw, GW;
+      if (op & CL_SPLIT) {
+        gw = my_w - start; if (gw < 0) gw += all_w;
+        GW = all_w;
+      } else {
+        if ((int)(who & 0xff) != grp) continue;
+        gw = (w0 + NW - start) & (NW - 1);
+        GW = NW;
+      }
+      if (gw >= pieces) continue;                       // no part of this command falls to this wavefront
+      cl_run(list[i], (int)(op & CL_OP_MASK), gw, GW);
     }
     __syncthreads();                                    // the staged commands are no longer read
   }
@@ -390,11 +408,11 @@ __global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const LhCmd* cmds, int n
 static bool ring_init() {
   if (g_ring.ready) return true;
   for (int i = 0; i < CL_NBUF; i++) {
-    if (hipHostMalloc((void**)&g_ring.host[i], sizeof(LhCmd) * CL_BUF_CMDS, hipHostMallocDefault) != hipSuccess) { LH_FAIL("command list: pinned buffer allocation failed"); return false; }
-    if (hipHostGetDevicePointer((void**)&g_ring.dev[i], g_ring.host[i], 0) != hipSuccess) { LH_FAIL("command list: pinned buffer has no device address"); return false; }
+    if (hipHostMalloc((void**)&g_ring.host[i], CL_BUF_BYTES, hipHostMallocDefault) != hipSuccess) { LH_FAIL("command list: pinned buffer allocation failed"); return false; }
     if (hipEventCreateWithFlags(&g_ring.done[i], hipEventDisableTiming) != hipSuccess) { LH_FAIL("command list: event creation failed"); return false; }
     g_ring.busy[i] = false;
   }
+  if (hipMalloc((void**)&g_ring.mirror, CL_BUF_BYTES) != hipSuccess) { LH_FAIL("command list: cannot allocate the device copy of a buffer"); return false; }
   if (hipMalloc((void**)&g_ring.sync, 2 * sizeof(unsigned long long)) != hipSuccess || hipMemset(g_ring.sync, 0, 2 * sizeof(unsigned long long)) != hipSuccess) {
     LH_FAIL("command list: cannot allocate the barrier words"); return false;
   }
@@ -456,11 +474,12 @@ static bool cmd_lanewise(const LhCmd& c) {
     default: return false;
   }
 }
-static bool cmd_splits(const LhCmd& c) { return c.op == CL_GEMV_N || c.op == CL_GER || (c.op == CL_GEMV_T && c.f1 == 1.0f); }
+static bool cmd_splits(const LhCmd& c) { return c.op == CL_GEMV_N || c.op == CL_GER || c.op == CL_GEMV_T; }
 static int cmd_waves(const LhCmd& c) {
   switch (c.op) {
     case CL_GEMV_N: return (c.i0 + 9) / 10;
-    case CL_GEMV_T: case CL_GER: return (c.i0 + 4) / 5;
+    case CL_GEMV_T: return (c.i1 + 15) / 16;
+    case CL_GER: return (c.i0 + 4) / 5;
     case CL_SOFTMAX: case CL_SOFTMAX_GRAD: return c.i0;
     default: return (c.i0 + 63) / 64;
   }
@@ -577,7 +596,8 @@ void rec_flush() {
     LH_FAIL("command list: a barrier between workgroups timed out; the commands of that buffer did not all run");
     return;
   }
-  LhCmd* out = r.host[r.cur];
+  uint2* ops = reinterpret_cast<uint2*>(r.host[r.cur]);
+  LhCmd* out = reinterpret_cast<LhCmd*>(r.host[r.cur] + CL_OPS_BYTES);
   static int start[CL_BUF_CMDS + 2];
   for (int l = 0; l <= W.top + 1; l++) start[l] = 0;
   for (int i = 0; i < n; i++) start[W.level[i] + 1]++;
@@ -589,14 +609,14 @@ void rec_flush() {
   for (int ch = 0; ch < W.nchains; ch++) chain_place[ch] = -1;
   for (int i = 0; i < n; i++) {
     const int l = W.level[i];
-    LhCmd& d = out[start[l]++];
-    d = W.cmd[i];
-    // a command that one workgroup runs alone goes to the next workgroup in turn; its first elements to wavefront `rot`
+    const int at = start[l]++;
+    out[at] = W.cmd[i];
     // a command that one workgroup runs alone goes to the next workgroup in turn, its first elements to the next free wavefront
     // there; the pieces of a command split over all workgroups start where those of the level's previous split command ended
-    const int groups = g_deterministic ? 1 : r.groups;      // one workgroup adds in a fixed order; several combine transposed products with atomic adds
+    const int groups = r.groups;
     int owner = 0, start;
-    if (groups > 1 && cmd_splits(W.cmd[i])) {
+    const bool split = cmd_splits(W.cmd[i]);
+    if (split) {
       start = split_of_level[l] % (groups * (CL_THREADS / 64));
       split_of_level[l] += cmd_waves(W.cmd[i]);
     } else if (W.chain[i] >= 0 && chain_place[W.chain[i]] >= 0) {          // a later command of a chain: where its first one runs
@@ -608,17 +628,23 @@ void rec_flush() {
       if (owner_of_level[l] % groups == 0) rot_of_level[l] = (rot_of_level[l] + cmd_waves(W.cmd[i])) & 15;
       if (W.chain[i] >= 0) chain_place[W.chain[i]] = (owner << 4) | start;
     }
-    d.op = W.cmd[i].op | ((seen[l] || l == 1) ? 0 : CL_BARRIER) | (start << CL_ROT_SHIFT) | (owner << CL_OWNER_SHIFT);
+    const int waves = W.cmd[i].op == CL_DOT ? 0xffff : (cmd_waves(W.cmd[i]) < 0xffff ? cmd_waves(W.cmd[i]) : 0xffff);
+    ops[at].x = (uint32_t)W.cmd[i].op | ((seen[l] || l == 1) ? 0u : (uint32_t)CL_BARRIER) | (split ? (uint32_t)CL_SPLIT : 0u) | ((uint32_t)start << CL_START_SHIFT);
+    ops[at].y = (uint32_t)owner | ((uint32_t)waves << CL_PIECES_SHIFT);
     seen[l] = true;
   }
-  const int groups = g_deterministic ? 1 : r.groups;
+  ops[n] = make_uint2(0, 0);
+  const int groups = r.groups;
   const int barriers = W.top > 1 ? W.top - 1 : 0;
   g_ring.levels += W.top;
   window_reset(W);
   ProfScope prof_(CAT_CMDLIST);
-  hipLaunchKernelGGL(k_cmdlist, dim3(groups), dim3(CL_THREADS), 0, g_stream_raw, (const LhCmd*)r.dev[r.cur], n, r.sync, r.sync_base, r.host_flag_dev);
+  hipError_t e = hipMemcpyAsync(r.mirror, r.host[r.cur], CL_OPS_BYTES + sizeof(LhCmd) * (size_t)n, hipMemcpyHostToDevice, g_stream_raw);
+  if (e != hipSuccess) { LH_FAIL("command list copy: %s", hipGetErrorString(e)); return; }
+  hipLaunchKernelGGL(k_cmdlist, dim3(groups), dim3(CL_THREADS), 0, g_stream_raw, reinterpret_cast<const uint2*>(r.mirror),
+                     reinterpret_cast<const LhCmd*>(r.mirror + CL_OPS_BYTES), n, r.sync, r.sync_base, r.host_flag_dev);
   if (groups > 1) r.sync_base += (unsigned long long)barriers * (unsigned long long)groups;
-  hipError_t e = hipGetLastError();
+  e = hipGetLastError();
   if (e == hipSuccess) e = hipEventRecord(r.done[r.cur], g_stream_raw);
   if (e != hipSuccess) { LH_FAIL("command list launch: %s", hipGetErrorString(e)); return; }
   r.busy[r.cur] = true;
@@ -666,6 +692,7 @@ void cmdlist_release() {
   if (!g_ring.ready) return;
   for (int i = 0; i < CL_NBUF; i++) { (void)hipEventDestroy(g_ring.done[i]); (void)hipHostFree(g_ring.host[i]); }
   if (g_ring.sync) (void)hipFree(g_ring.sync);
+  if (g_ring.mirror) (void)hipFree(g_ring.mirror);
   if (g_ring.host_flag) (void)hipHostFree(g_ring.host_flag);
   g_ring = Ring{};
 }
