@@ -27,22 +27,26 @@ namespace {
 constexpr int CL_THREADS = 1024;
 constexpr int CL_CHUNK = 256;                 // commands staged in LDS at a time
 constexpr int CL_BUF_CMDS = 2048;              // commands per host buffer: a full buffer is launched while the host records the next
-constexpr int CL_NBUF = 32;
-// Two op words per command.  Word 0: operation | flags | start << 12; word 1: owner | pieces << 8.
-constexpr int CL_OP_MASK = 0xff;
-constexpr int CL_BARRIER = 0x100;             // first command of a level: a barrier comes before it
-constexpr int CL_SPLIT = 0x200;               // a matrix command: its pieces are dealt round the wavefronts of all workgroups
-constexpr int CL_START_SHIFT = 12;            // where the command's work starts: a wavefront 0..15 of the owner or, for a split command,
-                                              // one of the wavefronts of all workgroups taken together
-constexpr int CL_PIECES_SHIFT = 8;            // word 1: how many wavefronts, counted from `start`, have work (a DOT needs them all)
+constexpr int CL_NBUF = 16;
 constexpr int CL_MAX_GROUPS = 64;
+// Two op words per entry of a workgroup's list.  Word 0: operation | CL_SPLIT | start << 12 | barriers << 24; word 1: pieces.
+constexpr int CL_OP_MASK = 0xff;
+constexpr int CL_NOP = 0xff;                  // an entry that only carries barriers (a workgroup with nothing to do in some levels)
+constexpr int CL_SPLIT = 0x200;               // a matrix command: its pieces are dealt round the wavefronts of all workgroups
+constexpr int CL_START_SHIFT = 12;            // 12 bits: where the command's work starts: a wavefront 0..15 of the workgroup or, for a split
+                                              // command, one of the wavefronts of all workgroups taken together
+constexpr int CL_BARRIERS_SHIFT = 24;         // 8 bits: barriers over all workgroups to pass before the entry (levels completed since the last one)
+constexpr int CL_WBLOCK = 4;                  // wavefronts of all workgroups are numbered in blocks of 4 of one workgroup, the blocks dealt
+                                              // round the workgroups: the pieces of a 150-row product fall to 4 workgroups, not to 15
 constexpr long CL_SPIN_LIMIT = 40000000L;     // polls of a grid barrier before a workgroup gives up (far beyond any real wait)
 
 static bool g_chains = true;          // LH_CMDLIST_CHAINS=0 in the environment: every dependent command opens a new level
-// A buffer is CL_BUF_CMDS + 16 pairs of op words, then the commands.
-constexpr size_t CL_OPS_BYTES = (size_t)(CL_BUF_CMDS + 16) * sizeof(uint2);
-constexpr size_t CL_BUF_BYTES = CL_OPS_BYTES + sizeof(LhCmd) * CL_BUF_CMDS;
-static_assert(CL_OPS_BYTES % 64 == 0, "the commands start on a 64-byte boundary");
+// A buffer as the device sees it: a directory (first entry and number of entries of each workgroup's list), the lists' commands
+// (64 bytes an entry; a command is copied into the list of every workgroup that has a part in it), then their op words.
+constexpr int CL_CAP = 4 * CL_BUF_CMDS;       // entries a buffer holds
+constexpr size_t CL_DIR_BYTES = CL_MAX_GROUPS * sizeof(uint2);
+constexpr size_t CL_BUF_BYTES = CL_DIR_BYTES + (sizeof(LhCmd) + sizeof(uint2)) * (size_t)(CL_CAP + CL_CHUNK);
+static_assert(CL_DIR_BYTES % 64 == 0, "the commands start on a 64-byte boundary");
 struct Ring {
   char* host[CL_NBUF]; hipEvent_t done[CL_NBUF]; bool busy[CL_NBUF];
   char* mirror;                      // device copy of the buffer being executed (launches are in stream order: one is enough)
@@ -347,28 +351,33 @@ __device__ __forceinline__ bool cl_grid_barrier(unsigned long long* sync, unsign
   return *lds_flag == 0;
 }
 
-// ops, cmds: the device copy of a buffer, in execution order: level by level, the first command of every level but the first
-// flagged CL_BARRIER.  The buffer is staged in LDS 256 commands at a time (the next chunk is fetched while the current one runs).
-// Every wavefront of every workgroup walks the op words (8 bytes a command, read one ahead and made wave-uniform, so the walk is
-// scalar work) and reads the 64-byte command only when it has a part in it: the op words say which workgroup owns the command or,
-// for a matrix command, at which wavefront of the launch its pieces start, and how many wavefronts have work.  A command that is
-// somebody else's costs a few scalar instructions.
-__global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const uint2* ops, const LhCmd* cmds, int n, unsigned long long* sync, unsigned long long sync_base,
-                                                        unsigned* host_flag) {
+// dir, ops, cmds: the device copy of a buffer.  Each workgroup has its own list, in execution order: level by level, an entry saying
+// how many barriers over all workgroups come before it (every list passes the same number of barriers in all).  A list is staged
+// in LDS 256 entries at a time (the next chunk is fetched while the current one runs).  Every wavefront of the workgroup walks the
+// op words (8 bytes an entry, read one ahead and made wave-uniform: the walk is scalar work, and the one scalar unit of a compute
+// unit serves all 16 wavefronts, which is why a list holds only what its workgroup has a part in) and reads the 64-byte command
+// only when a piece of it is its own.
+__global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const uint2* dir, const uint2* ops_all, const LhCmd* cmds_all, unsigned long long* sync,
+                                                        unsigned long long sync_base, unsigned* host_flag, unsigned long long* trace) {
   __shared__ uint4 stage[CL_CHUNK * 4];                 // 256 commands of 64 bytes
   __shared__ uint2 sop[CL_CHUNK + 1];
   __shared__ int gave_up;
   constexpr int NW = CL_THREADS / 64;
   const int t = threadIdx.x, grp = blockIdx.x, ngrp = gridDim.x;
   const int w0 = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int all_w = ngrp * NW, my_w = w0 * ngrp + grp;  // this wavefront among all of the launch: neighbours sit in different workgroups
-  const uint4* src = reinterpret_cast<const uint4*>(cmds);
+  const int all_w = ngrp * NW, my_w = ((w0 / CL_WBLOCK) * ngrp + grp) * CL_WBLOCK + w0 % CL_WBLOCK;      // this wavefront among all of the launch
+  const uint32_t first = __builtin_amdgcn_readfirstlane(dir[grp].x);
+  const int n = __builtin_amdgcn_readfirstlane((int)dir[grp].y);
+  const uint2* ops = ops_all + first;
+  const uint4* src = reinterpret_cast<const uint4*>(cmds_all + first);
   const int total16 = n * 4;
   unsigned long long arrived = sync_base;
+  int tr_k = 0;
+  if (trace && grp == 0 && t == 0) trace[tr_k++] = wall_clock64();
   uint4 next = make_uint4(0, 0, 0, 0);
   uint2 next_op = make_uint2(0, 0);
   if (t < total16) next = src[t];
-  if (t < CL_CHUNK) next_op = ops[t];                   // the op words are allocated past the last command
+  if (t < CL_CHUNK) next_op = ops[t];                   // op words are allocated a chunk past the last list
   for (int base = 0; base < n; base += CL_CHUNK) {
     stage[t] = next;
     if (t < CL_CHUNK) sop[t] = next_op;
@@ -382,19 +391,20 @@ __global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const uint2* ops, const 
     const LhCmd* list = reinterpret_cast<const LhCmd*>(stage);
     uint2 ahead = sop[0];
     for (int i = 0; i < cnt; i++) {
-      const uint32_t op = __builtin_amdgcn_readfirstlane(ahead.x), who = __builtin_amdgcn_readfirstlane(ahead.y);
+      const uint32_t op = __builtin_amdgcn_readfirstlane(ahead.x);
+      const int pieces = (int)__builtin_amdgcn_readfirstlane(ahead.y);
       ahead = sop[i + 1];
-      if (op & CL_BARRIER) {                            // the level before is complete and its stores are visible
+      for (int b = (int)(op >> CL_BARRIERS_SHIFT); b > 0; b--) {      // levels completed: their stores become visible
         if (ngrp == 1) __syncthreads();
         else { arrived += (unsigned long long)ngrp; if (!cl_grid_barrier(sync, arrived, &gave_up, host_flag)) return; }
+        if (trace && grp == 0 && t == 0) trace[tr_k++] = wall_clock64();
       }
-      const int start = (int)(op >> CL_START_SHIFT), pieces = (int)(who >> CL_PIECES_SHIFT);
+      const int start = (int)(op >> CL_START_SHIFT) & 0xfff;
       int gw, GW;
       if (op & CL_SPLIT) {
         gw = my_w - start; if (gw < 0) gw += all_w;
         GW = all_w;
       } else {
-        if ((int)(who & 0xff) != grp) continue;
         gw = (w0 + NW - start) & (NW - 1);
         GW = NW;
       }
@@ -403,6 +413,7 @@ __global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const uint2* ops, const 
     }
     __syncthreads();                                    // the staged commands are no longer read
   }
+  if (trace && grp == 0 && t == 0) trace[tr_k++] = wall_clock64();
 }
 
 static bool ring_init() {
@@ -489,7 +500,7 @@ static int cmd_waves(const LhCmd& c) {
 // buffers share a block only when one lies inside the other's allocation: then the dependence is real or harmless);
 // larger ranges (matrices, zero fills) in a short table of distinct ranges.  A level is a uint16: 1 + highest level touched.
 constexpr uintptr_t SMALL_BYTES = 4096;
-constexpr int HASH_N = 65536, BIG_N = 96;
+constexpr int HASH_N = 65536, BIG_N = 96, PAGE_N = 16384, PAGE_SCAN_MAX = 512;
 // Chains.  An element-wise command gives element i of every operand to the same lane (thread i mod 1024 of the workgroup and
 // wavefront rotation it runs on).  If everything such a command must follow at the highest level L is ONE chain of element-wise
 // commands, through ranges that start at the very addresses this command's operands start at, then each lane only ever needs what
@@ -498,16 +509,19 @@ constexpr int HASH_N = 65536, BIG_N = 96;
 // level, not three.
 struct Window {
   LhCmd cmd[CL_BUF_CMDS]; uint16_t level[CL_BUF_CMDS]; int16_t chain[CL_BUF_CMDS]; int n; int top, nchains;       // top: highest level handed out
+  int entries;                                                                // upper bound of the entries the workgroups' lists will hold
   struct Slot { uintptr_t key, wbase, rbase; uint32_t epoch; uint16_t w, r; int16_t wchain, rchain; } slot[HASH_N]; uint32_t epoch;
-  struct Big { uintptr_t s, e; uint16_t w, r; } big[BIG_N]; int nbig;
-  struct Small { uintptr_t s, e; uint16_t level; bool w; } small[CL_BUF_CMDS * 4]; int nsmall;
+  struct Big { uintptr_t s, e; uint16_t w, r; } big[BIG_N]; int nbig; bool big_anywhere;
+  // the distinct small ranges, each on the list of the one or two 4 KiB pages it touches: what a LARGE range is checked against
+  struct Small { uintptr_t s, e, page0; uint16_t w, r; int next[2]; } small[CL_BUF_CMDS * 4]; int nsmall;
+  struct Page { uintptr_t key; uint32_t epoch; int head; bool big; } page[PAGE_N];       // big: some large range touches the page
   uintptr_t small_lo, small_hi;                                               // bounding box of the small ranges
 };
 static Window* g_win = nullptr;
 
 static void window_reset(Window& W) {
-  W.n = 0; W.top = 0; W.nchains = 0; W.nbig = 0; W.nsmall = 0; W.small_lo = ~(uintptr_t)0; W.small_hi = 0;
-  if (++W.epoch == 0) { for (int i = 0; i < HASH_N; i++) W.slot[i].epoch = 0; W.epoch = 1; }
+  W.n = 0; W.entries = 0; W.top = 0; W.nchains = 0; W.nbig = 0; W.big_anywhere = false; W.nsmall = 0; W.small_lo = ~(uintptr_t)0; W.small_hi = 0;
+  if (++W.epoch == 0) { for (int i = 0; i < HASH_N; i++) W.slot[i].epoch = 0; for (int i = 0; i < PAGE_N; i++) W.page[i].epoch = 0; W.epoch = 1; }
 }
 static inline Window::Slot* slot_of(Window& W, uintptr_t block, bool create) {
   uint32_t h = (uint32_t)((block * 0x9E3779B97F4A7C15ull) >> 48) & (HASH_N - 1);
@@ -515,6 +529,15 @@ static inline Window::Slot* slot_of(Window& W, uintptr_t block, bool create) {
     Window::Slot& sl = W.slot[h];
     if (sl.epoch != W.epoch) { if (!create) return nullptr; sl.key = block; sl.epoch = W.epoch; sl.w = sl.r = 0; sl.wchain = sl.rchain = -1; sl.wbase = sl.rbase = 0; return &sl; }
     if (sl.key == block) return &sl;
+  }
+  return nullptr;
+}
+static inline Window::Page* page_of(Window& W, uintptr_t pg, bool create) {
+  uint32_t h = (uint32_t)((pg * 0x9E3779B97F4A7C15ull) >> 50) & (PAGE_N - 1);
+  for (int probe = 0; probe < PAGE_N; probe++, h = (h + 1) & (PAGE_N - 1)) {
+    Window::Page& pe = W.page[h];
+    if (pe.epoch != W.epoch) { if (!create) return nullptr; pe.key = pg; pe.epoch = W.epoch; pe.head = -1; pe.big = false; return &pe; }
+    if (pe.key == pg) return &pe;
   }
   return nullptr;
 }
@@ -529,22 +552,35 @@ struct Conflict {
   }
 };
 static void conflicts_of(Window& W, const Extent& x, Conflict& c) {
-  for (int i = 0; i < W.nbig; i++) {
-    const Window::Big& b = W.big[i];
-    if (b.s < x.e && x.s < b.e) c.see(x.w ? (b.w > b.r ? b.w : b.r) : b.w, -1, false);
+  const bool small = x.e - x.s <= SMALL_BYTES;
+  bool scan_big = !small || W.big_anywhere;
+  if (!scan_big && W.nbig > 0) {                              // a small range meets a large one only on a page a large one touches
+    const Window::Page* pa = page_of(W, x.s >> 12, false);
+    scan_big = pa && pa->big;
+    if (!scan_big && ((x.e - 1) >> 12) != (x.s >> 12)) { const Window::Page* pb = page_of(W, (x.e - 1) >> 12, false); scan_big = pb && pb->big; }
   }
-  if (x.e - x.s <= SMALL_BYTES) {
+  if (scan_big)
+    for (int i = 0; i < W.nbig; i++) {
+      const Window::Big& b = W.big[i];
+      if (b.s < x.e && x.s < b.e) c.see(x.w ? (b.w > b.r ? b.w : b.r) : b.w, -1, false);
+    }
+  if (small) {
     for (uintptr_t blk = x.s >> 8; blk <= (x.e - 1) >> 8; blk++) {
       const Window::Slot* sl = slot_of(W, blk, false);
       if (!sl) continue;
       c.see(sl->w, sl->wchain, sl->wbase == x.s);
       if (x.w) c.see(sl->r, sl->rchain, sl->rbase == x.s);
     }
-  } else if (x.s < W.small_hi && W.small_lo < x.e) {         // a large range over memory that small ranges of this window touch: rare
-    for (int i = 0; i < W.nsmall; i++) {
-      const Window::Small& m = W.small[i];
-      if (m.s < x.e && x.s < m.e && (x.w || m.w)) c.see(m.level, -1, false);
-    }
+  } else if (x.s < W.small_hi && W.small_lo < x.e) {         // a large range over memory that small ranges of this window touch
+    auto meet = [&](const Window::Small& m) { if (m.s < x.e && x.s < m.e) c.see(x.w ? (m.w > m.r ? m.w : m.r) : m.w, -1, false); };
+    const uintptr_t pa = (x.s > W.small_lo ? x.s : W.small_lo) >> 12, pb = ((x.e < W.small_hi ? x.e : W.small_hi) - 1) >> 12;
+    if (pb - pa >= (uintptr_t)PAGE_SCAN_MAX) { for (int i = 0; i < W.nsmall; i++) meet(W.small[i]); }
+    else
+      for (uintptr_t pg = pa; pg <= pb; pg++) {
+        const Window::Page* pe = page_of(W, pg, false);
+        if (!pe) continue;
+        for (int i = pe->head; i >= 0;) { const Window::Small& m = W.small[i]; meet(m); i = m.next[m.page0 == pg ? 0 : 1]; }
+      }
   }
 }
 static bool note_extent(Window& W, const Extent& x, int level, int chain) {
@@ -560,8 +596,22 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
         else if (level == sl->r && (sl->rchain != chain || sl->rbase != x.s)) sl->rchain = -1;
       }
     }
-    Window::Small& m = W.small[W.nsmall++];
-    m.s = x.s; m.e = x.e; m.level = (uint16_t)level; m.w = x.w;
+    const uintptr_t pa = x.s >> 12, pb = (x.e - 1) >> 12;
+    Window::Page* pe = page_of(W, pa, true);
+    if (!pe) return false;
+    int at = pe->head;
+    while (at >= 0 && !(W.small[at].s == x.s && W.small[at].e == x.e)) at = W.small[at].next[W.small[at].page0 == pa ? 0 : 1];
+    if (at < 0) {                                             // a range not seen in this window: on the list of each page it touches
+      Window::Page* pf = pb != pa ? page_of(W, pb, true) : nullptr;
+      if (pb != pa && !pf) return false;
+      at = W.nsmall++;
+      Window::Small& m = W.small[at];
+      m.s = x.s; m.e = x.e; m.page0 = pa; m.w = m.r = 0; m.next[0] = pe->head; m.next[1] = -1;
+      pe->head = at;
+      if (pf) { m.next[1] = pf->head; pf->head = at; }
+    }
+    Window::Small& m = W.small[at];
+    if (x.w) { if (level > m.w) m.w = (uint16_t)level; } else if (level > m.r) m.r = (uint16_t)level;
     if (x.s < W.small_lo) W.small_lo = x.s;
     if (x.e > W.small_hi) W.small_hi = x.e;
     return true;
@@ -571,6 +621,9 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
     if (b.s == x.s && b.e == x.e) { if (x.w) { if (level > b.w) b.w = (uint16_t)level; } else if (level > b.r) b.r = (uint16_t)level; return true; }
   }
   if (W.nbig == BIG_N) return false;
+  const uintptr_t pa = x.s >> 12, pb = (x.e - 1) >> 12;
+  if (pb - pa >= (uintptr_t)PAGE_SCAN_MAX) W.big_anywhere = true;
+  else for (uintptr_t pg = pa; pg <= pb; pg++) { Window::Page* pe = page_of(W, pg, true); if (!pe) return false; pe->big = true; }
   Window::Big& b = W.big[W.nbig++];
   b.s = x.s; b.e = x.e; b.w = x.w ? (uint16_t)level : 0; b.r = x.w ? 0 : (uint16_t)level;
   return true;
@@ -578,7 +631,7 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
 }  // namespace
 
 namespace lh {
-static unsigned long long g_tsc_push = 0, g_tsc_flush = 0, g_tsc_wait = 0;      // host cycles spent recording (LH_CMDLIST_VERBOSE prints them)
+static unsigned long long g_tsc_push = 0, g_tsc_flush = 0, g_tsc_wait = 0, g_tsc_conf = 0, g_tsc_note = 0;      // host cycles spent recording (LH_CMDLIST_VERBOSE prints them)
 // Hands the recorded buffer to the device: commands in level order (recording order within a level), the first of each
 // level flagged for a barrier, each with the wavefront its elements start on.
 void rec_flush() {
@@ -596,53 +649,100 @@ void rec_flush() {
     LH_FAIL("command list: a barrier between workgroups timed out; the commands of that buffer did not all run");
     return;
   }
-  uint2* ops = reinterpret_cast<uint2*>(r.host[r.cur]);
-  LhCmd* out = reinterpret_cast<LhCmd*>(r.host[r.cur] + CL_OPS_BYTES);
-  static int start[CL_BUF_CMDS + 2];
+  const int groups = r.groups, all_w = groups * (CL_THREADS / 64);
+  static int start[CL_BUF_CMDS + 2], order[CL_BUF_CMDS];
   for (int l = 0; l <= W.top + 1; l++) start[l] = 0;
   for (int i = 0; i < n; i++) start[W.level[i] + 1]++;
   for (int l = 1; l <= W.top + 1; l++) start[l] += start[l - 1];
+  for (int i = 0; i < n; i++) order[start[W.level[i]]++] = i;
   static int rot_of_level[CL_BUF_CMDS + 2], owner_of_level[CL_BUF_CMDS + 2], split_of_level[CL_BUF_CMDS + 2];
-  static bool seen[CL_BUF_CMDS + 2];
-  for (int l = 0; l <= W.top; l++) { rot_of_level[l] = 0; owner_of_level[l] = 0; split_of_level[l] = 0; seen[l] = false; }
+  for (int l = 0; l <= W.top; l++) { rot_of_level[l] = 0; owner_of_level[l] = 0; split_of_level[l] = 0; }
   static int chain_place[CL_BUF_CMDS + 1];
   for (int ch = 0; ch < W.nchains; ch++) chain_place[ch] = -1;
-  for (int i = 0; i < n; i++) {
-    const int l = W.level[i];
-    const int at = start[l]++;
-    out[at] = W.cmd[i];
+  // Pass 1: where each command runs, and how long each workgroup's list gets.
+  struct Place { uint32_t op, pieces; int g0, gn; };
+  static Place place[CL_BUF_CMDS];
+  int entries[CL_MAX_GROUPS], passed[CL_MAX_GROUPS];
+  for (int g = 0; g < groups; g++) entries[g] = passed[g] = 0;
+  auto entries_for = [](int need) { return 1 + (need > 255 ? (need - 1) / 255 : 0); };      // an entry carries up to 255 barriers
+  for (int k = 0; k < n; k++) {
+    const int i = order[k], l = W.level[i];
+    const LhCmd& c = W.cmd[i];
     // a command that one workgroup runs alone goes to the next workgroup in turn, its first elements to the next free wavefront
-    // there; the pieces of a command split over all workgroups start where those of the level's previous split command ended
-    const int groups = r.groups;
-    int owner = 0, start;
-    const bool split = cmd_splits(W.cmd[i]);
+    // there; the pieces of a split command start where those of the level's previous split command ended
+    int owner = 0, at;
+    const bool split = cmd_splits(c);
+    const int waves = c.op == CL_DOT ? 0xffff : (cmd_waves(c) < 0xffff ? cmd_waves(c) : 0xffff);
     if (split) {
-      start = split_of_level[l] % (groups * (CL_THREADS / 64));
-      split_of_level[l] += cmd_waves(W.cmd[i]);
+      at = split_of_level[l] % all_w;
+      split_of_level[l] += waves;
     } else if (W.chain[i] >= 0 && chain_place[W.chain[i]] >= 0) {          // a later command of a chain: where its first one runs
-      owner = chain_place[W.chain[i]] >> 4; start = chain_place[W.chain[i]] & 15;
+      owner = chain_place[W.chain[i]] >> 4; at = chain_place[W.chain[i]] & 15;
     } else {
       owner = owner_of_level[l] % groups;
-      start = rot_of_level[l] & 15;
+      at = rot_of_level[l] & 15;
       owner_of_level[l]++;
-      if (owner_of_level[l] % groups == 0) rot_of_level[l] = (rot_of_level[l] + cmd_waves(W.cmd[i])) & 15;
-      if (W.chain[i] >= 0) chain_place[W.chain[i]] = (owner << 4) | start;
+      if (owner_of_level[l] % groups == 0) rot_of_level[l] = (rot_of_level[l] + waves) & 15;
+      if (W.chain[i] >= 0) chain_place[W.chain[i]] = (owner << 4) | at;
     }
-    const int waves = W.cmd[i].op == CL_DOT ? 0xffff : (cmd_waves(W.cmd[i]) < 0xffff ? cmd_waves(W.cmd[i]) : 0xffff);
-    ops[at].x = (uint32_t)W.cmd[i].op | ((seen[l] || l == 1) ? 0u : (uint32_t)CL_BARRIER) | (split ? (uint32_t)CL_SPLIT : 0u) | ((uint32_t)start << CL_START_SHIFT);
-    ops[at].y = (uint32_t)owner | ((uint32_t)waves << CL_PIECES_SHIFT);
-    seen[l] = true;
+    Place& pl = place[k];
+    pl.op = (uint32_t)c.op | (split ? (uint32_t)CL_SPLIT : 0u) | ((uint32_t)at << CL_START_SHIFT);
+    pl.pieces = (uint32_t)waves;
+    if (split) {
+      const int span = waves < all_w ? waves : all_w, b0 = at / CL_WBLOCK, b1 = (at + span - 1) / CL_WBLOCK;
+      pl.g0 = b0 % groups; pl.gn = b1 - b0 + 1 < groups ? b1 - b0 + 1 : groups;
+    } else { pl.g0 = owner; pl.gn = 1; }
+    for (int j = 0; j < pl.gn; j++) { const int g = (pl.g0 + j) % groups; entries[g] += entries_for(l - 1 - passed[g]); passed[g] = l - 1; }
   }
-  ops[n] = make_uint2(0, 0);
-  const int groups = r.groups;
   const int barriers = W.top > 1 ? W.top - 1 : 0;
+  for (int g = 0; g < groups; g++) if (passed[g] < barriers) entries[g] += entries_for(barriers - passed[g]);
+  // Pass 2: the lists, one after the other.
+  uint2* dir = reinterpret_cast<uint2*>(r.host[r.cur]);
+  LhCmd* out = reinterpret_cast<LhCmd*>(r.host[r.cur] + CL_DIR_BYTES);
+  int first[CL_MAX_GROUPS], total = 0;
+  for (int g = 0; g < groups; g++) { first[g] = total; dir[g] = make_uint2((uint32_t)total, (uint32_t)entries[g]); total += entries[g]; passed[g] = 0; }
+  if (total > CL_CAP) { window_reset(W); LH_FAIL("command list: %d entries exceed a buffer (%d)", total, CL_CAP); return; }
+  uint2* ops = reinterpret_cast<uint2*>(out + total);
+  auto put = [&](int g, uint32_t op, uint32_t pieces, const LhCmd* c, int need) {
+    for (; need > 255; need -= 255) { ops[first[g]] = make_uint2((uint32_t)CL_NOP | (255u << CL_BARRIERS_SHIFT), 0u); first[g]++; }
+    ops[first[g]] = make_uint2(op | ((uint32_t)need << CL_BARRIERS_SHIFT), pieces);
+    if (c) out[first[g]] = *c;
+    first[g]++;
+  };
+  for (int k = 0; k < n; k++) {
+    const int i = order[k], l = W.level[i];
+    const Place& pl = place[k];
+    for (int j = 0; j < pl.gn; j++) { const int g = (pl.g0 + j) % groups; put(g, pl.op, pl.pieces, &W.cmd[i], l - 1 - passed[g]); passed[g] = l - 1; }
+  }
+  for (int g = 0; g < groups; g++) if (passed[g] < barriers) put(g, (uint32_t)CL_NOP, 0u, nullptr, barriers - passed[g]);
   g_ring.levels += W.top;
+  static unsigned long long* trace_buf = nullptr; static int trace_from = -1;
+  if (trace_from == -1) { const char* e = getenv("LH_CMDLIST_TRACE"); trace_from = e ? atoi(e) : -2; if (e) (void)hipHostMalloc((void**)&trace_buf, 8 * 4096, hipHostMallocDefault); }
+  const bool tracing = trace_from >= 0 && r.launches >= trace_from && r.launches < trace_from + 2;
+  static int tr_counts[CL_BUF_CMDS / 8][7]; int tr_levels = 0; static int tr_len[CL_BUF_CMDS + 1];
+  if (tracing) {
+    tr_levels = W.top < CL_BUF_CMDS / 8 ? W.top : CL_BUF_CMDS / 8 - 1;
+    for (int l = 0; l <= tr_levels; l++) for (int k = 0; k < 7; k++) tr_counts[l][k] = 0;
+    for (int c = 0; c <= W.nchains; c++) tr_len[c] = 0;
+    static int tr_hist[CL_BUF_CMDS / 8][24]; static long tr_zero[CL_BUF_CMDS / 8];
+    for (int l = 0; l <= tr_levels; l++) { for (int k = 0; k < 24; k++) tr_hist[l][k] = 0; tr_zero[l] = 0; }
+    for (int i = 0; i < n; i++) if (W.level[i] <= tr_levels) { tr_hist[W.level[i]][W.cmd[i].op % 24]++; if (W.cmd[i].op == CL_ZERO16) tr_zero[W.level[i]] += (long)W.cmd[i].i0 * 16; }
+    if (getenv("LH_CMDLIST_TRACE_HIST")) for (int l = 1; l <= tr_levels; l++) { fprintf(stderr, "  hist level %d:", l); for (int k = 0; k < 24; k++) if (tr_hist[l][k]) fprintf(stderr, " op%d x%d", k, tr_hist[l][k]); fprintf(stderr, " zero bytes %ld\n", tr_zero[l]); }
+    for (int i = 0; i < n; i++) if (W.chain[i] >= 0 && W.level[i] <= tr_levels) { const int L = ++tr_len[W.chain[i]]; if (L == 1) tr_counts[W.level[i]][5]++; if (L > tr_counts[W.level[i]][6]) tr_counts[W.level[i]][6] = L; }
+    for (int i = 0; i < n; i++) { const int l = W.level[i]; if (l > tr_levels) continue; const int o = W.cmd[i].op; tr_counts[l][o == CL_GEMV_N ? 1 : o == CL_GEMV_T ? 2 : o == CL_GER ? 3 : cmd_lanewise(W.cmd[i]) ? 0 : 4]++; }
+  }
   window_reset(W);
   ProfScope prof_(CAT_CMDLIST);
-  hipError_t e = hipMemcpyAsync(r.mirror, r.host[r.cur], CL_OPS_BYTES + sizeof(LhCmd) * (size_t)n, hipMemcpyHostToDevice, g_stream_raw);
+  hipError_t e = hipMemcpyAsync(r.mirror, r.host[r.cur], CL_DIR_BYTES + (sizeof(LhCmd) + sizeof(uint2)) * (size_t)total, hipMemcpyHostToDevice, g_stream_raw);
   if (e != hipSuccess) { LH_FAIL("command list copy: %s", hipGetErrorString(e)); return; }
   hipLaunchKernelGGL(k_cmdlist, dim3(groups), dim3(CL_THREADS), 0, g_stream_raw, reinterpret_cast<const uint2*>(r.mirror),
-                     reinterpret_cast<const LhCmd*>(r.mirror + CL_OPS_BYTES), n, r.sync, r.sync_base, r.host_flag_dev);
+                     reinterpret_cast<const uint2*>(r.mirror + CL_DIR_BYTES + sizeof(LhCmd) * (size_t)total), reinterpret_cast<const LhCmd*>(r.mirror + CL_DIR_BYTES),
+                     r.sync, r.sync_base, r.host_flag_dev, tracing ? trace_buf : nullptr);
+  if (tracing) {
+    (void)hipStreamSynchronize(g_stream_raw);
+    fprintf(stderr, "trace launch %lld: %d commands, %d levels, total %.1f us\n", (long long)r.launches, n, tr_levels, (trace_buf[tr_levels + 1 > 1 ? tr_levels : 1] - trace_buf[0]) * 0.01);
+    for (int l = 1; l <= tr_levels; l++) fprintf(stderr, "  level %3d: %6.2f us  ew %3d gemv %3d gemv_t %3d ger %3d other %3d chains %3d longest %3d\n", l, (trace_buf[l] - trace_buf[l - 1]) * 0.01, tr_counts[l][0], tr_counts[l][1], tr_counts[l][2], tr_counts[l][3], tr_counts[l][4], tr_counts[l][5], tr_counts[l][6]);
+  }
   if (groups > 1) r.sync_base += (unsigned long long)barriers * (unsigned long long)groups;
   e = hipGetLastError();
   if (e == hipSuccess) e = hipEventRecord(r.done[r.cur], g_stream_raw);
@@ -666,18 +766,30 @@ bool rec_push(const LhCmd& c) {
   Window& W = *g_win;
   Extent x[4];
   const int k = cmd_extents(c, x);
+  // the lists of how many workgroups the command goes on (an upper bound; the barrier-only entries are allowed for below)
+  int copies = 1;
+  if (cmd_splits(c)) {
+    const int all_w = g_ring.groups * (CL_THREADS / 64), span = cmd_waves(c) < all_w ? cmd_waves(c) : all_w;
+    copies = (span + CL_WBLOCK - 2) / CL_WBLOCK + 1;
+    if (copies > g_ring.groups) copies = g_ring.groups;
+  }
   for (int attempt = 0; attempt < 2; attempt++) {
-    if (W.n == CL_BUF_CMDS) { rec_flush(); if (failed()) return false; }
+    if (W.n == CL_BUF_CMDS || W.entries + copies + g_ring.groups * 10 > CL_CAP) { rec_flush(); if (failed()) return false; }
     Conflict cf;
+    const unsigned long long q0 = __builtin_ia32_rdtsc();
     for (int i = 0; i < k; i++) conflicts_of(W, x[i], cf);
+    g_tsc_conf += __builtin_ia32_rdtsc() - q0;
     const bool lanewise = cmd_lanewise(c);
     int lv, chain;
     if (lanewise && cf.one_chain && g_chains) { lv = cf.lv; chain = cf.chain; }                    // joins the chain it follows
     else { lv = cf.lv + 1; chain = lanewise ? W.nchains++ : -1; }
     bool ok = true;
+    const unsigned long long q1 = __builtin_ia32_rdtsc();
     for (int i = 0; i < k && ok; i++) ok = note_extent(W, x[i], lv, chain);
+    g_tsc_note += __builtin_ia32_rdtsc() - q1;
     if (!ok) { rec_flush(); if (failed()) return false; continue; }       // a table is full: start a new buffer (which begins with a barrier)
     W.cmd[W.n] = c; W.level[W.n] = (uint16_t)lv; W.chain[W.n] = (int16_t)chain; W.n++;
+    W.entries += copies;
     if (lv > W.top) W.top = lv;
     g_rec_pending = W.n;
     g_ring.recorded++;
@@ -704,14 +816,14 @@ void lh_cmdlist_begin(void) {
   LH_REQUIRE(!g_capturing, "lh_cmdlist_begin: a graph is being recorded (the command buffers cannot be replayed)");
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_cmdlist_begin on the side stream");
   if (!ring_init()) return;
-  if (g_win == nullptr) { g_win = new Window(); for (int i = 0; i < HASH_N; i++) g_win->slot[i].epoch = 0; g_win->epoch = 0; window_reset(*g_win); }
+  if (g_win == nullptr) { g_win = new Window(); for (int i = 0; i < HASH_N; i++) g_win->slot[i].epoch = 0; for (int i = 0; i < PAGE_N; i++) g_win->page[i].epoch = 0; g_win->epoch = 0; window_reset(*g_win); }
   g_rec_on = 1;
 }
 void lh_cmdlist_end(void) {
   rec_flush();
   g_rec_on = 0;
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld commands in %lld levels, %lld launches\n", (long long)g_ring.recorded, (long long)g_ring.levels, (long long)g_ring.launches);
-  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list host cycles: push %.1f M (flush inside %.1f M, of which waiting for a free buffer %.1f M)\n", g_tsc_push * 1e-6, g_tsc_flush * 1e-6, g_tsc_wait * 1e-6);
+  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list host cycles: push %.1f M (flush inside %.1f M, of which waiting for a free buffer %.1f M), conflicts %.1f M, notes %.1f M\n", g_tsc_push * 1e-6, g_tsc_flush * 1e-6, g_tsc_wait * 1e-6, g_tsc_conf * 1e-6, g_tsc_note * 1e-6);
 }
 void lh_cmdlist_stats(int64_t* recorded, int64_t* launches) {
   if (recorded) *recorded = g_ring.recorded;
