@@ -131,7 +131,7 @@ void lh_graph_launch(int graph);
 void lh_graph_destroy(int graph);
 
 /* Command list for launch-bound programs (the sentiment TreeLSTM, SentimentTreeLSTM.scala:242-318, issues about
- * 7000 operator calls on 150-element vectors per tree; the reference pays one cuBLAS / kernel launch for each,
+ * 3600 operator calls on 150-element vectors per tree; the reference pays one cuBLAS / kernel launch for each,
  * CUB:171-560).  Between lh_cmdlist_begin and lh_cmdlist_end every entry point of this header whose operands are
  * small (element-wise up to 65536 elements, matrix-vector up to 131072 matrix elements: fill, copy, geam, scalar and
  * same-shape broadcast arithmetic with gradients, unary ops with gradients, sgemv, ger, dot_vv, axpy_dev, softmax and
@@ -139,12 +139,13 @@ void lh_graph_destroy(int graph);
  * commands are handed to the device whenever any other entry point is called, when 2048 are pending, and at
  * lh_cmdlist_end / lh_sync / lh_d2h, so program order holds between recorded and launched work.  Within a buffer the
  * library works out from the byte ranges each command reads and writes which commands depend on which, and runs the buffer
- * level by level: commands that do not depend on each other side by side (the matrix commands cut by rows over 16
- * workgroups, LH_CMDLIST_GROUPS in the environment overrides), a barrier over the workgroups between levels.  The barrier's
- * wait is bounded: if a workgroup never arrives the kernel ends, and the next call that touches the command list reports it.
- * Results equal those of the stand-alone kernels up to summation order in the reductions (a transposed matrix-vector product
- * that accumulates is combined over the workgroups with atomic adds; in deterministic mode one workgroup runs the list and the
- * order is fixed).  Generated code calls lh_cmdlist_begin() once after lh_setup(). */
+ * level by level: commands that do not depend on each other side by side (element-wise commands dealt over 24 workgroups,
+ * LH_CMDLIST_GROUPS in the environment overrides; the matrix commands cut by rows or columns over the wavefronts of all of
+ * them), a barrier over the workgroups between levels.  The barrier's wait is bounded: if a workgroup never arrives the
+ * kernel ends, and the next call that touches the command list reports it.  Results equal those of the stand-alone kernels
+ * up to summation order in the reductions; no command uses atomic adds and every sum has a fixed order, so two runs give the
+ * same bits whatever the number of workgroups.  LH_CMDLIST_TRACE=<launch> prints, for that launch and the next, how long each
+ * level took and what it held.  Generated code calls lh_cmdlist_begin() once after lh_setup(). */
 void lh_cmdlist_begin(void);
 void lh_cmdlist_end(void);
 /* Commands recorded and interpreter launches since lh_setup (either pointer may be NULL). */

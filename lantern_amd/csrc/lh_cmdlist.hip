@@ -1,20 +1,22 @@
-// Command list: small operations recorded on the host and executed by one 1024-thread workgroup.
+// Command list: small operations recorded on the host and executed by a few 1024-thread workgroups in one launch per buffer.
 //
-// A model built from 150-element vectors (the sentiment TreeLSTM: ~7000 operator calls per tree) is bound by the
-// host's kernel-launch rate (about 3 us per launch), not by the device.  Between lh_cmdlist_begin() and
-// lh_cmdlist_end() every entry point whose operands are small appends a 64-byte command instead of launching; the
-// commands of a buffer are handed to k_cmdlist when the buffer is full, when recording ends, or when any other entry
-// point is about to use the stream (lh::ordered_stream), so the program order of all operations is kept.
+// A model built from 150-element vectors (the sentiment TreeLSTM: ~3600 operator calls per tree) is bound by the host's
+// kernel-launch rate (about 3 us per launch), not by the device.  Between lh_cmdlist_begin() and lh_cmdlist_end() every entry
+// point whose operands are small appends a 64-byte command instead of launching; the commands of a buffer are handed to
+// k_cmdlist when the buffer is full, when recording ends, or when any other entry point is about to use the stream
+// (lh::ordered_stream), so the program order of all operations is kept.
 //
-// One workgroup pays a full memory round trip (load, store, barrier) per dependent command, about 1 us, whatever the
-// command's size.  So the host works out, per buffer, which commands depend on which (byte ranges read and written: a
-// command that writes a range comes after every earlier command that touches it, one that reads it after every earlier
-// writer) and gives each command a LEVEL, one more than the highest level it depends on.  The buffer is executed level
-// by level: commands of one level have no dependence on each other, run without a barrier between them, and are spread
-// over the workgroup's 16 wavefronts (each command carries a rotation of the thread index), so their round trips overlap;
-// one block barrier per level makes a level's stores visible to the next.  Independent work of a program (the ten gate
-// products of a tree node, the two subtrees of a node) thus runs side by side without the program saying so.
-// The arithmetic of each command follows the stand-alone kernel of the same operation.
+// A dependent command costs a memory round trip (load, store, visibility), a microsecond or more, whatever its size.  So the host
+// works out, per buffer, which commands depend on which (byte ranges read and written: a command that writes a range comes after
+// every earlier command that touches it, one that reads it after every earlier writer) and gives each command a LEVEL, one more
+// than the highest level it depends on.  The buffer is executed level by level: commands of one level have no dependence on each
+// other and are spread over the workgroups and their wavefronts, so their round trips overlap; one barrier over all workgroups
+// per level makes a level's stores visible to the next.  Independent work of a program (the ten gate products of a tree node, the
+// two subtrees of a node) thus runs side by side without the program saying so.  Element-wise commands that depend only on each
+// other, lane by lane, share a level (a chain).  Each workgroup gets its own list of the commands it has a part in: the walk over
+// a list is scalar work, and a compute unit has one scalar unit for its 16 wavefronts.
+// The arithmetic of each command follows the stand-alone kernel of the same operation; no command uses atomics, so the result does
+// not depend on how many workgroups run it.
 #include "lh_common.h"
 using namespace lh;
 
@@ -432,9 +434,10 @@ static bool ring_init() {
     LH_FAIL("command list: cannot allocate the pinned flag"); return false;
   }
   *g_ring.host_flag = 0;
-  // Workgroups per launch: 16 compute units draw the matrices of a level in about one memory round trip, and a barrier over
-  // 16 costs 3.5 us against 2.5 us for one workgroup's own device-scope fences (6 us over 32).  LH_CMDLIST_GROUPS overrides.
-  int groups = 16;
+  // Workgroups per launch.  More of them draw a level's matrices faster (a compute unit gets some 25 GB/s) and make the barrier
+  // dearer; on the sentiment TreeLSTM 4 / 8 / 16 / 24 / 32 workgroups give 573 / 732 / 842 / 870 / 871 trees a second.
+  // LH_CMDLIST_GROUPS overrides.
+  int groups = 24;
   if (const char* e = getenv("LH_CMDLIST_GROUPS")) groups = atoi(e);
   if (const char* e = getenv("LH_CMDLIST_CHAINS")) g_chains = atoi(e) != 0;
   if (groups < 1) groups = 1;
@@ -716,20 +719,21 @@ void rec_flush() {
   }
   for (int g = 0; g < groups; g++) if (passed[g] < barriers) put(g, (uint32_t)CL_NOP, 0u, nullptr, barriers - passed[g]);
   g_ring.levels += W.top;
+  // LH_CMDLIST_TRACE=<launch>: workgroup 0 notes the time of every barrier of that launch and the next one; the host prints how long
+  // each level took and what it held (a diagnostic: the launch is waited for)
   static unsigned long long* trace_buf = nullptr; static int trace_from = -1;
-  if (trace_from == -1) { const char* e = getenv("LH_CMDLIST_TRACE"); trace_from = e ? atoi(e) : -2; if (e) (void)hipHostMalloc((void**)&trace_buf, 8 * 4096, hipHostMallocDefault); }
+  if (trace_from == -1) { const char* e = getenv("LH_CMDLIST_TRACE"); trace_from = e ? atoi(e) : -2; if (e && hipHostMalloc((void**)&trace_buf, 8 * (CL_BUF_CMDS + 2), hipHostMallocDefault) != hipSuccess) trace_from = -2; }
   const bool tracing = trace_from >= 0 && r.launches >= trace_from && r.launches < trace_from + 2;
-  static int tr_counts[CL_BUF_CMDS / 8][7]; int tr_levels = 0; static int tr_len[CL_BUF_CMDS + 1];
+  static int tr_counts[CL_BUF_CMDS + 1][7], tr_len[CL_BUF_CMDS + 1];       // per level: element-wise, gemv, gemv_t, ger, other, chains, longest chain
+  const int tr_levels = W.top;
   if (tracing) {
-    tr_levels = W.top < CL_BUF_CMDS / 8 ? W.top : CL_BUF_CMDS / 8 - 1;
     for (int l = 0; l <= tr_levels; l++) for (int k = 0; k < 7; k++) tr_counts[l][k] = 0;
     for (int c = 0; c <= W.nchains; c++) tr_len[c] = 0;
-    static int tr_hist[CL_BUF_CMDS / 8][24]; static long tr_zero[CL_BUF_CMDS / 8];
-    for (int l = 0; l <= tr_levels; l++) { for (int k = 0; k < 24; k++) tr_hist[l][k] = 0; tr_zero[l] = 0; }
-    for (int i = 0; i < n; i++) if (W.level[i] <= tr_levels) { tr_hist[W.level[i]][W.cmd[i].op % 24]++; if (W.cmd[i].op == CL_ZERO16) tr_zero[W.level[i]] += (long)W.cmd[i].i0 * 16; }
-    if (getenv("LH_CMDLIST_TRACE_HIST")) for (int l = 1; l <= tr_levels; l++) { fprintf(stderr, "  hist level %d:", l); for (int k = 0; k < 24; k++) if (tr_hist[l][k]) fprintf(stderr, " op%d x%d", k, tr_hist[l][k]); fprintf(stderr, " zero bytes %ld\n", tr_zero[l]); }
-    for (int i = 0; i < n; i++) if (W.chain[i] >= 0 && W.level[i] <= tr_levels) { const int L = ++tr_len[W.chain[i]]; if (L == 1) tr_counts[W.level[i]][5]++; if (L > tr_counts[W.level[i]][6]) tr_counts[W.level[i]][6] = L; }
-    for (int i = 0; i < n; i++) { const int l = W.level[i]; if (l > tr_levels) continue; const int o = W.cmd[i].op; tr_counts[l][o == CL_GEMV_N ? 1 : o == CL_GEMV_T ? 2 : o == CL_GER ? 3 : cmd_lanewise(W.cmd[i]) ? 0 : 4]++; }
+    for (int i = 0; i < n; i++) {
+      const int l = W.level[i], o = W.cmd[i].op;
+      tr_counts[l][o == CL_GEMV_N ? 1 : o == CL_GEMV_T ? 2 : o == CL_GER ? 3 : cmd_lanewise(W.cmd[i]) ? 0 : 4]++;
+      if (W.chain[i] >= 0) { const int L = ++tr_len[W.chain[i]]; if (L == 1) tr_counts[l][5]++; if (L > tr_counts[l][6]) tr_counts[l][6] = L; }
+    }
   }
   window_reset(W);
   ProfScope prof_(CAT_CMDLIST);
@@ -740,8 +744,10 @@ void rec_flush() {
                      r.sync, r.sync_base, r.host_flag_dev, tracing ? trace_buf : nullptr);
   if (tracing) {
     (void)hipStreamSynchronize(g_stream_raw);
-    fprintf(stderr, "trace launch %lld: %d commands, %d levels, total %.1f us\n", (long long)r.launches, n, tr_levels, (trace_buf[tr_levels + 1 > 1 ? tr_levels : 1] - trace_buf[0]) * 0.01);
-    for (int l = 1; l <= tr_levels; l++) fprintf(stderr, "  level %3d: %6.2f us  ew %3d gemv %3d gemv_t %3d ger %3d other %3d chains %3d longest %3d\n", l, (trace_buf[l] - trace_buf[l - 1]) * 0.01, tr_counts[l][0], tr_counts[l][1], tr_counts[l][2], tr_counts[l][3], tr_counts[l][4], tr_counts[l][5], tr_counts[l][6]);
+    fprintf(stderr, "command list launch %lld: %d commands, %d levels, %.1f us\n", (long long)r.launches, n, tr_levels, (trace_buf[tr_levels + 1] - trace_buf[0]) * 0.01);
+    for (int l = 1; l <= tr_levels; l++)
+      fprintf(stderr, "  level %3d: %6.2f us  element-wise %3d gemv %3d gemv_t %3d ger %3d other %3d chains %3d longest %3d\n", l, (trace_buf[l] - trace_buf[l - 1]) * 0.01,
+              tr_counts[l][0], tr_counts[l][1], tr_counts[l][2], tr_counts[l][3], tr_counts[l][4], tr_counts[l][5], tr_counts[l][6]);
   }
   if (groups > 1) r.sync_base += (unsigned long long)barriers * (unsigned long long)groups;
   e = hipGetLastError();

@@ -161,3 +161,29 @@ def test_c_treelstm_program_tracks_the_oracle(tmp_path, cpu_backend, cmdlist):
         g = got[pos:pos + w.size].reshape(w.shape); pos += w.size
         err = np.linalg.norm(g.astype(np.float64) - w) / max(np.linalg.norm(w.astype(np.float64)), 1e-30)
         assert err <= 1e-3 or np.abs(g - w).max() <= 1e-5, err
+
+
+@pytest.mark.gpu
+def test_c_treelstm_command_list_gives_the_same_bits_on_any_number_of_workgroups(tmp_path, cpu_backend):
+    """No command of the list combines partial results with atomic adds and every sum has a fixed order, so eight training steps
+    of the C program end in the same bits whether 1, 5 or 24 workgroups share the commands (LH_CMDLIST_GROUPS), and twice over."""
+    import numpy as np
+    import lantern_amd as la
+    from lantern_amd.apps.treelstm import Trainer, read_trees
+    exe = TREE_BIN if os.path.exists(TREE_BIN) else (_build_host_program() and TREE_BIN)
+    la.set_backend(cpu_backend)
+    mark = cpu_backend.getMallocAddr()
+    trees = read_trees(os.path.join(ROOT, "tests", "golden", "array_tree_first24.txt"))[:8]
+    tr = Trainer(vocab=500, trees=trees)
+    write_treelstm_inputs(tmp_path, tr, tr.trees)
+    tr.close(); cpu_backend.resetMallocAddr(mark)
+    results = []
+    for groups in ("1", "5", "24", "24"):
+        out_file = tmp_path / ("out_%d.bin" % len(results))
+        out = subprocess.run([exe, str(tmp_path / "params.bin"), str(tmp_path / "trees.txt"), str(out_file), str(len(trees)), "0", "1"],
+                             capture_output=True, text=True, timeout=110, env=dict(os.environ, LH_CMDLIST_GROUPS=groups))
+        assert out.returncode == 0 and out.stdout.startswith("trees_per_s"), out.stdout + out.stderr
+        results.append(np.fromfile(out_file, np.uint32))
+    assert results[0].size > len(trees) and np.isfinite(results[0].view(np.float32)).all()
+    for r in results[1:]:
+        assert np.array_equal(results[0], r)
