@@ -192,28 +192,30 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
       }
       break;
     }
-    case CL_GEMV_T: {            // y[n] = alpha * A[m,n]^T x[m] + beta * y  (p0 = y, p1 = A, p2 = x): a wavefront takes 16 columns
-      // (64 bytes of every row); lane l holds column l mod 16 of the rows congruent to l / 16 mod 4, up to 20 of them in flight
-      // together.  The four row classes meet by lane exchange: no LDS, no atomics, and the order of the sum is fixed.
+    case CL_GEMV_T: {            // y[n] = alpha * A[m,n]^T x[m] + beta * y  (p0 = y, p1 = A, p2 = x): a wavefront takes 8 columns
+      // (the four wavefronts of a block, side by side in one compute unit, a 128-byte line of every row); lane l holds column
+      // l mod 8 of the rows congruent to l / 8 mod 8, up to 20 of them in flight together: 160 rows in one memory round trip.  The
+      // eight row classes meet by lane exchange: no LDS, no atomics, and the order of the sum is fixed.
       const int m = c.i0, n = c.i1, lda = c.i2; const float al = c.f0, be = c.f1;
       const __amdgpu_buffer_rsrc_t rA = cl_rsrc(p1, ((int64_t)(m - 1) * lda + n) * 4), rX = cl_rsrc(p2, (int64_t)m * 4);
-      const int cj = lane & 15, rg = lane >> 4;
+      const int cj = lane & 7, rg = lane >> 3;
       constexpr int RU = 20;
-      for (int j0 = gw * 16; j0 < n; j0 += GW * 16) {
+      for (int j0 = gw * 8; j0 < n; j0 += GW * 8) {
         const int j = j0 + cj;
         const uint32_t co = j < n ? (uint32_t)j * 4u : CL_OOB;
         float acc = 0.f;
-        for (int i0 = 0; i0 < m; i0 += 4 * RU) {
+        for (int i0 = 0; i0 < m; i0 += 8 * RU) {
           float xv[RU], av[RU];
 #pragma unroll
           for (int u = 0; u < RU; u++) {
-            const uint32_t i = (uint32_t)(i0 + u * 4 + rg);
+            const uint32_t i = (uint32_t)(i0 + u * 8 + rg);
             xv[u] = cl_ld(rX, i * 4u);                                                   // zero past m
             av[u] = cl_ld(rA, i * (uint32_t)lda * 4u + co);                              // rows past m lie past the operand's end
           }
 #pragma unroll
           for (int u = 0; u < RU; u++) acc += av[u] * xv[u];
         }
+        acc += __shfl_xor(acc, 8, 64);
         acc += __shfl_xor(acc, 16, 64);
         acc += __shfl_xor(acc, 32, 64);
         if (rg == 0 && j < n) p0[j] = al * acc + (be == 0.f ? 0.f : be * p0[j]);
@@ -488,11 +490,18 @@ static bool cmd_lanewise(const LhCmd& c) {
     default: return false;
   }
 }
+// How a command maps what it writes onto wavefronts: 1 element-wise (element i: thread i mod 1024), 2 rows of a matrix-vector
+// product (ten to a wavefront), 3 columns of a transposed product (eight to a wavefront), 4 rows of a rank-1 update (five to a
+// wavefront); 0: none of these.
+static int cmd_class(const LhCmd& c) {
+  if (cmd_lanewise(c)) return 1;
+  return c.op == CL_GEMV_N ? 2 : c.op == CL_GEMV_T ? 3 : c.op == CL_GER ? 4 : 0;
+}
 static bool cmd_splits(const LhCmd& c) { return c.op == CL_GEMV_N || c.op == CL_GER || c.op == CL_GEMV_T; }
 static int cmd_waves(const LhCmd& c) {
   switch (c.op) {
     case CL_GEMV_N: return (c.i0 + 9) / 10;
-    case CL_GEMV_T: return (c.i1 + 15) / 16;
+    case CL_GEMV_T: return (c.i1 + 7) / 8;
     case CL_GER: return (c.i0 + 4) / 5;
     case CL_SOFTMAX: case CL_SOFTMAX_GRAD: return c.i0;
     default: return (c.i0 + 63) / 64;
@@ -510,11 +519,15 @@ constexpr int HASH_N = 65536, BIG_N = 96, PAGE_N = 16384, PAGE_SCAN_MAX = 512;
 // it read or wrote itself, program order within the lane is enough, and the command joins that chain AT level L (same workgroup,
 // same rotation, recording order) instead of opening level L + 1: bias add, second product's add and activation of a gate are one
 // level, not three.
+// The matrix commands chain the same way through what they WRITE: a wavefront owns the same rows (or columns) of the result in every
+// command of the chain, so five transposed products that add into one gradient vector, or the rank-1 updates of one weight
+// gradient, are one level (the same wavefronts take them in recording order) instead of five.  What a matrix command READS is
+// needed whole by every wavefront: a conflict through an input at the highest level always opens a new level.
 struct Window {
-  LhCmd cmd[CL_BUF_CMDS]; uint16_t level[CL_BUF_CMDS]; int16_t chain[CL_BUF_CMDS]; int n; int top, nchains;       // top: highest level handed out
+  LhCmd cmd[CL_BUF_CMDS]; uint16_t level[CL_BUF_CMDS]; int16_t chain[CL_BUF_CMDS]; uint8_t chain_class[CL_BUF_CMDS + 1]; int32_t chain_row[CL_BUF_CMDS + 1]; int n; int top, nchains;       // top: highest level handed out
   int entries;                                                                // upper bound of the entries the workgroups' lists will hold
   struct Slot { uintptr_t key, wbase, rbase; uint32_t epoch; uint16_t w, r; int16_t wchain, rchain; } slot[HASH_N]; uint32_t epoch;
-  struct Big { uintptr_t s, e; uint16_t w, r; } big[BIG_N]; int nbig; bool big_anywhere;
+  struct Big { uintptr_t s, e; uint16_t w, r; int16_t wchain, rchain; } big[BIG_N]; int nbig; bool big_anywhere;
   // the distinct small ranges, each on the list of the one or two 4 KiB pages it touches: what a LARGE range is checked against
   struct Small { uintptr_t s, e, page0; uint16_t w, r; int next[2]; } small[CL_BUF_CMDS * 4]; int nsmall;
   struct Page { uintptr_t key; uint32_t epoch; int head; bool big; } page[PAGE_N];       // big: some large range touches the page
@@ -565,7 +578,11 @@ static void conflicts_of(Window& W, const Extent& x, Conflict& c) {
   if (scan_big)
     for (int i = 0; i < W.nbig; i++) {
       const Window::Big& b = W.big[i];
-      if (b.s < x.e && x.s < b.e) c.see(x.w ? (b.w > b.r ? b.w : b.r) : b.w, -1, false);
+      if (b.s < x.e && x.s < b.e) {
+        const bool same = b.s == x.s && b.e == x.e;
+        c.see(b.w, b.wchain, same);
+        if (x.w) c.see(b.r, b.rchain, same);
+      }
     }
   if (small) {
     for (uintptr_t blk = x.s >> 8; blk <= (x.e - 1) >> 8; blk++) {
@@ -621,7 +638,11 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
   }
   for (int i = 0; i < W.nbig; i++) {
     Window::Big& b = W.big[i];
-    if (b.s == x.s && b.e == x.e) { if (x.w) { if (level > b.w) b.w = (uint16_t)level; } else if (level > b.r) b.r = (uint16_t)level; return true; }
+    if (b.s == x.s && b.e == x.e) {
+      if (x.w) { if (level > b.w) { b.w = (uint16_t)level; b.wchain = (int16_t)chain; } else if (level == b.w && b.wchain != chain) b.wchain = -1; }
+      else { if (level > b.r) { b.r = (uint16_t)level; b.rchain = (int16_t)chain; } else if (level == b.r && b.rchain != chain) b.rchain = -1; }
+      return true;
+    }
   }
   if (W.nbig == BIG_N) return false;
   const uintptr_t pa = x.s >> 12, pb = (x.e - 1) >> 12;
@@ -629,6 +650,7 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
   else for (uintptr_t pg = pa; pg <= pb; pg++) { Window::Page* pe = page_of(W, pg, true); if (!pe) return false; pe->big = true; }
   Window::Big& b = W.big[W.nbig++];
   b.s = x.s; b.e = x.e; b.w = x.w ? (uint16_t)level : 0; b.r = x.w ? 0 : (uint16_t)level;
+  b.wchain = x.w ? (int16_t)chain : -1; b.rchain = x.w ? -1 : (int16_t)chain;
   return true;
 }
 }  // namespace
@@ -676,9 +698,12 @@ void rec_flush() {
     int owner = 0, at;
     const bool split = cmd_splits(c);
     const int waves = c.op == CL_DOT ? 0xffff : (cmd_waves(c) < 0xffff ? cmd_waves(c) : 0xffff);
-    if (split) {
+    if (split && W.chain[i] >= 0 && chain_place[W.chain[i]] >= 0) {     // a later matrix command of a chain: the wavefronts of its first one
+      at = chain_place[W.chain[i]];
+    } else if (split) {
       at = split_of_level[l] % all_w;
       split_of_level[l] += waves;
+      if (W.chain[i] >= 0) chain_place[W.chain[i]] = at;
     } else if (W.chain[i] >= 0 && chain_place[W.chain[i]] >= 0) {          // a later command of a chain: where its first one runs
       owner = chain_place[W.chain[i]] >> 4; at = chain_place[W.chain[i]] & 15;
     } else {
@@ -781,17 +806,20 @@ bool rec_push(const LhCmd& c) {
   }
   for (int attempt = 0; attempt < 2; attempt++) {
     if (W.n == CL_BUF_CMDS || W.entries + copies + g_ring.groups * 10 > CL_CAP) { rec_flush(); if (failed()) return false; }
-    Conflict cf;
+    // cf: what the command must follow through operands that map onto wavefronts as the chain's do (all operands of an element-wise
+    // command; what a matrix command writes, which cmd_extents lists first); cf_in: through what a matrix command reads
+    Conflict cf, cf_in;
+    const int cls = cmd_class(c);
     const unsigned long long q0 = __builtin_ia32_rdtsc();
-    for (int i = 0; i < k; i++) conflicts_of(W, x[i], cf);
+    for (int i = 0; i < k; i++) conflicts_of(W, x[i], (cls >= 2 && i > 0) ? cf_in : cf);
     g_tsc_conf += __builtin_ia32_rdtsc() - q0;
-    const bool lanewise = cmd_lanewise(c);
     int lv, chain;
-    if (lanewise && cf.one_chain && g_chains) { lv = cf.lv; chain = cf.chain; }                    // joins the chain it follows
-    else { lv = cf.lv + 1; chain = lanewise ? W.nchains++ : -1; }
+    const int row = cls == 4 ? c.i1 : 0;             // rank-1 updates own rows: the same buffer cut into rows of another length is another mapping
+    if (cls && g_chains && cf.one_chain && W.chain_class[cf.chain] == cls && W.chain_row[cf.chain] == row && cf_in.lv < cf.lv) { lv = cf.lv; chain = cf.chain; }      // joins the chain it follows
+    else { lv = (cf.lv > cf_in.lv ? cf.lv : cf_in.lv) + 1; chain = -1; if (cls) { chain = W.nchains++; W.chain_class[chain] = (uint8_t)cls; W.chain_row[chain] = row; } }
     bool ok = true;
     const unsigned long long q1 = __builtin_ia32_rdtsc();
-    for (int i = 0; i < k && ok; i++) ok = note_extent(W, x[i], lv, chain);
+    for (int i = 0; i < k && ok; i++) ok = note_extent(W, x[i], lv, (cls >= 2 && i > 0) ? -1 : chain);
     g_tsc_note += __builtin_ia32_rdtsc() - q1;
     if (!ok) { rec_flush(); if (failed()) return false; continue; }       // a table is full: start a new buffer (which begins with a barrier)
     W.cmd[W.n] = c; W.level[W.n] = (uint16_t)lv; W.chain[W.n] = (int16_t)chain; W.n++;
