@@ -169,7 +169,8 @@ def run_gpu(args):
         # same distribution, the same trees; it runs after this process has released the device
         import tempfile
         from lantern_amd.apps.treelstm import write_c_program_inputs
-        c_dir = tempfile.mkdtemp(prefix="lantern_treelstm_")
+        c_dir = args.keep_c_inputs or tempfile.mkdtemp(prefix="lantern_treelstm_")
+        os.makedirs(c_dir, exist_ok=True)
         tr.close(); tr.end_step()
         tr2, _, _ = make_trainer(args, args.batch)
         write_c_program_inputs(c_dir, tr2)
@@ -185,8 +186,9 @@ def run_gpu(args):
         c_host = {"trees_per_s": float(f[1]), "ms_per_tree": float(f[3]), "host_issue_ms_per_tree": float(f[7])}
         losses = np.fromfile(os.path.join(c_dir, "out.bin"), np.float32, count=args.steps)
         assert np.isfinite(losses).all() and (losses > 0).all(), "the C host program's losses"
-        import shutil
-        shutil.rmtree(c_dir, ignore_errors=True)
+        if not args.keep_c_inputs:
+            import shutil
+            shutil.rmtree(c_dir, ignore_errors=True)
     return {"c_host": c_host, "streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
             "per_step": per_step, "desc": desc}
 
@@ -240,6 +242,7 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--keep-c-inputs", default=None, help="treelstm: write the C host program's input files (params.bin, trees.txt) into this directory and leave them there")
     ap.add_argument("--tree-file", default=None, help="treelstm: trees in the reference's array_tree.txt format instead of random ones (tests/golden/array_tree_first24.txt)")
     ap.add_argument("--no-side-stream", action="store_true", help="filter gradients in line on the main stream (kernel profiles: no two kernels overlap)")
     ap.add_argument("--resident", action="store_true", help="resnet50: keep one batch resident on the device (no per-step upload, no loss read-back)")

@@ -139,7 +139,7 @@ void lh_graph_destroy(int graph);
  * commands are handed to the device whenever any other entry point is called, when 2048 are pending, and at
  * lh_cmdlist_end / lh_sync / lh_d2h, so program order holds between recorded and launched work.  Within a buffer the
  * library works out from the byte ranges each command reads and writes which commands depend on which, and runs the buffer
- * level by level: commands that do not depend on each other side by side (element-wise commands dealt over 24 workgroups,
+ * level by level: commands that do not depend on each other side by side (element-wise commands dealt over 32 workgroups,
  * LH_CMDLIST_GROUPS in the environment overrides; the matrix commands cut by rows or columns over the wavefronts of all of
  * them), a barrier over the workgroups between levels.  The barrier's wait is bounded: if a workgroup never arrives the
  * kernel ends, and the next call that touches the command list reports it.  Results equal those of the stand-alone kernels

@@ -130,26 +130,27 @@ __device__ __forceinline__ float cl_wave_sum_dpp(float v) {
 // different workgroups, and the pieces of the commands of one level follow each other round the wavefronts, so a wavefront
 // rarely holds pieces of two of them and their memory round trips overlap instead of queueing.
 __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int gw, const int GW) {
-  constexpr int NT = CL_THREADS, NW = CL_THREADS / 64;
+  constexpr int NW = CL_THREADS / 64;
   const int lane = threadIdx.x & 63, wave = gw, t = wave * 64 + lane;
+  const int ST = GW * 64;                               // threads that share the command
   float* p0 = (float*)c.p0; float* p1 = (float*)c.p1; float* p2 = (float*)c.p2; float* p3 = (float*)c.p3;
   switch (opc) {
-    case CL_ZERO16: { uint4* p = (uint4*)c.p0; const int n = c.i0; for (int i = t; i < n; i += NT) p[i] = make_uint4(0, 0, 0, 0); break; }
-    case CL_FILL: { const int n = c.i0; const float v = c.f0; for (int i = t; i < n; i += NT) p0[i] = v; break; }
-    case CL_COPY: { const int n = c.i0; for (int i = t; i < n; i += NT) p0[i] = p1[i]; break; }
-    case CL_GEAM: { const int n = c.i0; const float al = c.f0, be = c.f1; for (int i = t; i < n; i += NT) p0[i] = p1[i] * al + p2[i] * be; break; }
-    case CL_SCALAR: { const int n = c.i0, op = c.i1; const float s = c.f0; for (int i = t; i < n; i += NT) p0[i] = cl_bop(op, p1[i], s); break; }
-    case CL_BIN: { const int n = c.i0, op = c.i1; for (int i = t; i < n; i += NT) p0[i] = cl_bop(op, p1[i], p2[i]); break; }
-    case CL_ACC: { const int n = c.i0; for (int i = t; i < n; i += NT) p0[i] = p0[i] + p1[i]; break; }
-    case CL_ACCNEG: { const int n = c.i0; for (int i = t; i < n; i += NT) p0[i] = p0[i] + (0.0f - p1[i]); break; }
-    case CL_ACCMUL: { const int n = c.i0; for (int i = t; i < n; i += NT) p0[i] = p0[i] + p1[i] * p2[i]; break; }
-    case CL_UNARY: { const int n = c.i0, op = c.i1; const float lo = c.f0, hi = c.f1; for (int i = t; i < n; i += NT) p0[i] = cl_unary(op, p1[i], lo, hi); break; }
+    case CL_ZERO16: { uint4* p = (uint4*)c.p0; const int n = c.i0; for (int i = t; i < n; i += ST) p[i] = make_uint4(0, 0, 0, 0); break; }
+    case CL_FILL: { const int n = c.i0; const float v = c.f0; for (int i = t; i < n; i += ST) p0[i] = v; break; }
+    case CL_COPY: { const int n = c.i0; for (int i = t; i < n; i += ST) p0[i] = p1[i]; break; }
+    case CL_GEAM: { const int n = c.i0; const float al = c.f0, be = c.f1; for (int i = t; i < n; i += ST) p0[i] = p1[i] * al + p2[i] * be; break; }
+    case CL_SCALAR: { const int n = c.i0, op = c.i1; const float s = c.f0; for (int i = t; i < n; i += ST) p0[i] = cl_bop(op, p1[i], s); break; }
+    case CL_BIN: { const int n = c.i0, op = c.i1; for (int i = t; i < n; i += ST) p0[i] = cl_bop(op, p1[i], p2[i]); break; }
+    case CL_ACC: { const int n = c.i0; for (int i = t; i < n; i += ST) p0[i] = p0[i] + p1[i]; break; }
+    case CL_ACCNEG: { const int n = c.i0; for (int i = t; i < n; i += ST) p0[i] = p0[i] + (0.0f - p1[i]); break; }
+    case CL_ACCMUL: { const int n = c.i0; for (int i = t; i < n; i += ST) p0[i] = p0[i] + p1[i] * p2[i]; break; }
+    case CL_UNARY: { const int n = c.i0, op = c.i1; const float lo = c.f0, hi = c.f1; for (int i = t; i < n; i += ST) p0[i] = cl_unary(op, p1[i], lo, hi); break; }
     case CL_UNARY_GRAD: {        // p0 = dx, p1 = x, p2 = y, p3 = dy
       const int n = c.i0, op = c.i1, inplace = c.i2; const float lo = c.f0, hi = c.f1;
       const bool need_x = (op == LH_RELU || op == LH_HARDTANH) ? !inplace : (op == LH_LOG || op == LH_SQUARE);
       const bool need_y = (op == LH_RELU || op == LH_HARDTANH) ? inplace != 0 : !(op == LH_LOG || op == LH_SQUARE);
       const bool need_g = !((op == LH_RELU || op == LH_HARDTANH) && inplace);
-      for (int i = t; i < n; i += NT)
+      for (int i = t; i < n; i += ST)
         p0[i] = cl_unary_grad(op, inplace, p0[i], need_x ? p1[i] : 0.f, need_y ? p2[i] : 0.f, need_g ? p3[i] : 0.f, lo, hi);
       break;
     }
@@ -162,6 +163,7 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
         float acc[RB];
 #pragma unroll
         for (int u = 0; u < RB; u++) acc[u] = 0.f;
+        const float yold = (be != 0.f && lane < RB && r0 + lane < m) ? p0[r0 + lane] : 0.f;  // asked for with the matrix, not after it
         for (int j0 = 0; j0 < n; j0 += 256) {
           float xv[4], av[RB][4];
           const uint32_t co = (uint32_t)(j0 + lane) * 4u;
@@ -188,7 +190,7 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
         float sv = 0.f;
 #pragma unroll
         for (int u = 0; u < RB; u++) { const float tot = cl_wave_sum_dpp(acc[u]); sv = lane == u ? tot : sv; }
-        if (lane < RB && r0 + lane < m) p0[r0 + lane] = al * sv + (be == 0.f ? 0.f : be * p0[r0 + lane]);
+        if (lane < RB && r0 + lane < m) p0[r0 + lane] = al * sv + (be == 0.f ? 0.f : be * yold);
       }
       break;
     }
@@ -203,6 +205,7 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
       for (int j0 = gw * 8; j0 < n; j0 += GW * 8) {
         const int j = j0 + cj;
         const uint32_t co = j < n ? (uint32_t)j * 4u : CL_OOB;
+        const float yold = (be != 0.f && rg == 0 && j < n) ? p0[j] : 0.f;               // asked for with the matrix, not after it
         float acc = 0.f;
         for (int i0 = 0; i0 < m; i0 += 8 * RU) {
           float xv[RU], av[RU];
@@ -218,7 +221,7 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
         acc += __shfl_xor(acc, 8, 64);
         acc += __shfl_xor(acc, 16, 64);
         acc += __shfl_xor(acc, 32, 64);
-        if (rg == 0 && j < n) p0[j] = al * acc + (be == 0.f ? 0.f : be * p0[j]);
+        if (rg == 0 && j < n) p0[j] = al * acc + (be == 0.f ? 0.f : be * yold);
       }
       break;
     }
@@ -253,7 +256,7 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
     case CL_DOT: {               // out[0] = x . y   (p0 = out, p1 = x, p2 = y)
       const int n = c.i0;
       float acc = 0.f;
-      for (int i = t; i < n; i += NT) acc += p1[i] * p2[i];
+      for (int i = t; i < n; i += ST) acc += p1[i] * p2[i];
       acc = cl_wave_sum_all(acc);
       __shared__ float red[NW];
       if (lane == 0) red[wave] = acc;
@@ -265,7 +268,7 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
     case CL_AXPY_DEV: {          // y += s[0] * x   (p0 = y, p1 = s, p2 = x)
       const int n = c.i0;
       const float a = *(volatile float*)p1;                 // written by an earlier command: a vector load, not the scalar cache
-      for (int i = t; i < n; i += NT) p0[i] = p0[i] + a * p2[i];
+      for (int i = t; i < n; i += ST) p0[i] = p0[i] + a * p2[i];
       break;
     }
     case CL_SOFTMAX: {           // rows of length cc, a wavefront per row   (p0 = y, p1 = x; i2 = log form)
@@ -299,17 +302,17 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
     }
     case CL_NLL: {               // y[b] = -x[b*stride + target[b]]   (p0 = y, p1 = x, p2 = target)
       const int batch = c.i0, stride = c.i1; const int* tg = (const int*)c.p2;
-      for (int b = t; b < batch; b += NT) p0[b] = -1.0f * p1[(int64_t)b * stride + tg[b]];
+      for (int b = t; b < batch; b += ST) p0[b] = -1.0f * p1[(int64_t)b * stride + tg[b]];
       break;
     }
     case CL_NLL_GRAD: {          // dx[b*stride + target[b]] += -dy[b]   (p0 = dx, p1 = dy, p2 = target)
       const int batch = c.i0, stride = c.i1; const int* tg = (const int*)c.p2;
-      for (int b = t; b < batch; b += NT) p0[(int64_t)b * stride + tg[b]] += -1.0f * p1[b];
+      for (int b = t; b < batch; b += ST) p0[(int64_t)b * stride + tg[b]] += -1.0f * p1[b];
       break;
     }
     case CL_ADAGRAD: {           // p0 = x, p1 = d, p2 = m
       const int n = c.i0; const float lr = c.f0, clip = c.f1;
-      for (int i = t; i < n; i += NT) {
+      for (int i = t; i < n; i += ST) {
         float g = p1[i];
         if (g > clip) g = clip;
         if (g < -clip) g = -clip;
@@ -322,7 +325,7 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
     }
     case CL_SGD: {               // p0 = x, p1 = d
       const int n = c.i0; const float lr = c.f0;
-      for (int i = t; i < n; i += NT) { p0[i] = p0[i] * 1.0f + p1[i] * (-lr); p1[i] = 0.f; }
+      for (int i = t; i < n; i += ST) { p0[i] = p0[i] * 1.0f + p1[i] * (-lr); p1[i] = 0.f; }
       break;
     }
     default: break;
@@ -437,9 +440,9 @@ static bool ring_init() {
   }
   *g_ring.host_flag = 0;
   // Workgroups per launch.  More of them draw a level's matrices faster (a compute unit gets some 25 GB/s) and make the barrier
-  // dearer; on the sentiment TreeLSTM 4 / 8 / 16 / 24 / 32 workgroups give 573 / 732 / 842 / 870 / 871 trees a second.
-  // LH_CMDLIST_GROUPS overrides.
-  int groups = 24;
+  // dearer; on the sentiment TreeLSTM 4 / 8 / 16 / 24 / 32 / 48 / 64 workgroups give 593 / 803 / 981 / 1058 / 1105 / 1114 / 1095
+  // trees a second.  LH_CMDLIST_GROUPS overrides.
+  int groups = 32;
   if (const char* e = getenv("LH_CMDLIST_GROUPS")) groups = atoi(e);
   if (const char* e = getenv("LH_CMDLIST_CHAINS")) g_chains = atoi(e) != 0;
   if (groups < 1) groups = 1;
@@ -492,12 +495,16 @@ static bool cmd_lanewise(const LhCmd& c) {
 }
 // How a command maps what it writes onto wavefronts: 1 element-wise (element i: thread i mod 1024), 2 rows of a matrix-vector
 // product (ten to a wavefront), 3 columns of a transposed product (eight to a wavefront), 4 rows of a rank-1 update (five to a
-// wavefront); 0: none of these.
+// wavefront), 5 element-wise over the wavefronts of all workgroups (a parameter update over a whole weight matrix: one compute unit
+// alone would draw it at 25 GB/s); 0: none of these.
+constexpr int WIDE_ELEMS = 4096;          // element-wise commands from this size on are shared by the wavefronts of all workgroups
 static int cmd_class(const LhCmd& c) {
-  if (cmd_lanewise(c)) return 1;
+  if (cmd_lanewise(c)) return c.i0 >= WIDE_ELEMS ? 5 : 1;
   return c.op == CL_GEMV_N ? 2 : c.op == CL_GEMV_T ? 3 : c.op == CL_GER ? 4 : 0;
 }
-static bool cmd_splits(const LhCmd& c) { return c.op == CL_GEMV_N || c.op == CL_GER || c.op == CL_GEMV_T; }
+static bool cmd_splits(const LhCmd& c) {
+  return c.op == CL_GEMV_N || c.op == CL_GER || c.op == CL_GEMV_T || (cmd_lanewise(c) && c.i0 >= WIDE_ELEMS) || (c.op == CL_ZERO16 && c.i0 >= WIDE_ELEMS / 4);
+}
 static int cmd_waves(const LhCmd& c) {
   switch (c.op) {
     case CL_GEMV_N: return (c.i0 + 9) / 10;
@@ -769,7 +776,7 @@ void rec_flush() {
                      r.sync, r.sync_base, r.host_flag_dev, tracing ? trace_buf : nullptr);
   if (tracing) {
     (void)hipStreamSynchronize(g_stream_raw);
-    fprintf(stderr, "command list launch %lld: %d commands, %d levels, %.1f us\n", (long long)r.launches, n, tr_levels, (trace_buf[tr_levels + 1] - trace_buf[0]) * 0.01);
+    fprintf(stderr, "command list launch %lld: %d commands, %d levels, %.1f us\n", (long long)r.launches, n, tr_levels, (trace_buf[tr_levels] - trace_buf[0]) * 0.01);
     for (int l = 1; l <= tr_levels; l++)
       fprintf(stderr, "  level %3d: %6.2f us  element-wise %3d gemv %3d gemv_t %3d ger %3d other %3d chains %3d longest %3d\n", l, (trace_buf[l] - trace_buf[l - 1]) * 0.01,
               tr_counts[l][0], tr_counts[l][1], tr_counts[l][2], tr_counts[l][3], tr_counts[l][4], tr_counts[l][5], tr_counts[l][6]);
