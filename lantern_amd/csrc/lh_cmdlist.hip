@@ -33,6 +33,11 @@ constexpr int CL_NBUF = 16;
 constexpr int CL_MAX_GROUPS = 64;
 // Two op words per entry of a workgroup's list.  Word 0: operation | CL_SPLIT | start << 12 | barriers << 24; word 1: pieces.
 constexpr int CL_OP_MASK = 0xff;
+constexpr int CL_SYNC = 0xfe;                 // the workgroup's wavefronts meet: what the entries before it put into LDS is there for all
+constexpr int CL_CHAIN = 0xfc;                // an element-wise chain as a program: i0 commands of 16 bytes each in the entries behind this one
+constexpr int CL_PRELOAD = 0xfd;              // up to four vectors into LDS slots (p0..p3; i0, i2: their lengths, 16 bits each; i1: their slots): what a
+                                              // chain program works on
+constexpr int CL_NSLOT_MAX = 128, CL_SLOT_ELEMS = 256;   // LDS slots of a workgroup at most (as many as the device's LDS allows), floats in each
 constexpr int CL_NOP = 0xff;                  // an entry that only carries barriers (a workgroup with nothing to do in some levels)
 constexpr int CL_SPLIT = 0x200;               // a matrix command: its pieces are dealt round the wavefronts of all workgroups
 constexpr int CL_START_SHIFT = 12;            // 12 bits: where the command's work starts: a wavefront 0..15 of the workgroup or, for a split
@@ -42,10 +47,11 @@ constexpr int CL_WBLOCK = 4;                  // wavefronts of all workgroups ar
                                               // round the workgroups: the pieces of a 150-row product fall to 4 workgroups, not to 15
 constexpr long CL_SPIN_LIMIT = 40000000L;     // polls of a grid barrier before a workgroup gives up (far beyond any real wait)
 
+static bool g_slots = true;           // LH_CMDLIST_SLOTS=0 in the environment: chains read and write memory only
 static bool g_chains = true;          // LH_CMDLIST_CHAINS=0 in the environment: every dependent command opens a new level
 // A buffer as the device sees it: a directory (first entry and number of entries of each workgroup's list), the lists' commands
 // (64 bytes an entry; a command is copied into the list of every workgroup that has a part in it), then their op words.
-constexpr int CL_CAP = 4 * CL_BUF_CMDS;       // entries a buffer holds
+constexpr int CL_CAP = 6 * CL_BUF_CMDS;       // entries a buffer holds
 constexpr size_t CL_DIR_BYTES = CL_MAX_GROUPS * sizeof(uint2);
 constexpr size_t CL_BUF_BYTES = CL_DIR_BYTES + (sizeof(LhCmd) + sizeof(uint2)) * (size_t)(CL_CAP + CL_CHUNK);
 static_assert(CL_DIR_BYTES % 64 == 0, "the commands start on a 64-byte boundary");
@@ -57,10 +63,13 @@ struct Ring {
   unsigned long long* sync;          // device: [0] arrivals at grid barriers, [1] a workgroup gave up waiting
   unsigned long long sync_base;      // arrivals once everything launched so far has run
   int groups;                        // workgroups per launch
+  int nslot;                         // LDS slots of a workgroup for chain programs
   unsigned* host_flag; unsigned* host_flag_dev;       // pinned word a workgroup sets when its barrier wait ran out
 };
 static Ring g_ring = {};
 
+typedef __attribute__((address_space(1))) float gfloat;       // device (global) memory, as opposed to a generic address
+typedef __attribute__((address_space(1))) int gint;
 __device__ __forceinline__ float cl_bop(int op, float a, float b) {
   switch (op) { case LH_ADD: return a + b; case LH_SUB: return a - b; case LH_MUL: return a * b; default: return a / b; }
 }
@@ -104,8 +113,8 @@ __device__ __forceinline__ float cl_wave_max_all(float v) {
 // address computed per element (one workgroup's vector ALUs, not memory, bound these commands), constant column steps folded
 // into the instruction, and anything past the operand's last byte reads as zero or is not stored, so rows past the matrix
 // need no test.  The descriptor's base must be wave-uniform: the pointer comes out of LDS and is made so explicitly.
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t cl_rsrc(const void* p, int64_t bytes) {
-  const uint64_t a = (uint64_t)p;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t cl_rsrc(const gfloat* p, int64_t bytes) {
+  const uint64_t a = (uint64_t)(uintptr_t)p;
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
   return __builtin_amdgcn_make_buffer_rsrc((void*)(((uint64_t)hi << 32) | lo), 0, (int)bytes, 0x00020000);
 }
@@ -129,17 +138,25 @@ __device__ __forceinline__ float cl_wave_sum_dpp(float v) {
 // over 16 units takes one memory round trip): piece k goes to wavefront (start + k) mod GW, neighbouring wavefronts sit in
 // different workgroups, and the pieces of the commands of one level follow each other round the wavefronts, so a wavefront
 // rarely holds pieces of two of them and their memory round trips overlap instead of queueing.
-__device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int gw, const int GW) {
+__device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int gw, const int GW, float* S, uint64_t* SP) {
   constexpr int NW = CL_THREADS / 64;
   const int lane = threadIdx.x & 63, wave = gw, t = wave * 64 + lane;
   const int ST = GW * 64;                               // threads that share the command
-  float* p0 = (float*)c.p0; float* p1 = (float*)c.p1; float* p2 = (float*)c.p2; float* p3 = (float*)c.p3;
+  // Operands are device memory, and the pointers say so: an access through a generic pointer counts as an LDS operation too until it
+  // completes, so the wait for the next op word (an LDS read) would wait for every store of the command before it.
+  gfloat* p0 = (gfloat*)(uintptr_t)c.p0; gfloat* p1 = (gfloat*)(uintptr_t)c.p1; gfloat* p2 = (gfloat*)(uintptr_t)c.p2; gfloat* p3 = (gfloat*)(uintptr_t)c.p3;
   switch (opc) {
-    case CL_ZERO16: { uint4* p = (uint4*)c.p0; const int n = c.i0; for (int i = t; i < n; i += ST) p[i] = make_uint4(0, 0, 0, 0); break; }
+    case CL_ZERO16: {            // 16 bytes a thread
+      typedef __attribute__((ext_vector_type(4))) unsigned int vec4;
+      typedef __attribute__((address_space(1))) vec4 gvec4;
+      gvec4* p = (gvec4*)(uintptr_t)c.p0; const int n = c.i0; const vec4 z = {0u, 0u, 0u, 0u};
+      for (int i = t; i < n; i += ST) p[i] = z;
+      break;
+    }
     case CL_FILL: { const int n = c.i0; const float v = c.f0; for (int i = t; i < n; i += ST) p0[i] = v; break; }
     case CL_COPY: { const int n = c.i0; for (int i = t; i < n; i += ST) p0[i] = p1[i]; break; }
     case CL_GEAM: { const int n = c.i0; const float al = c.f0, be = c.f1; for (int i = t; i < n; i += ST) p0[i] = p1[i] * al + p2[i] * be; break; }
-    case CL_SCALAR: { const int n = c.i0, op = c.i1; const float s = c.f0; for (int i = t; i < n; i += ST) p0[i] = cl_bop(op, p1[i], s); break; }
+    case CL_SCALAR: { const int n = c.i0, op = c.i1; const float sc = c.f0; for (int i = t; i < n; i += ST) p0[i] = cl_bop(op, p1[i], sc); break; }
     case CL_BIN: { const int n = c.i0, op = c.i1; for (int i = t; i < n; i += ST) p0[i] = cl_bop(op, p1[i], p2[i]); break; }
     case CL_ACC: { const int n = c.i0; for (int i = t; i < n; i += ST) p0[i] = p0[i] + p1[i]; break; }
     case CL_ACCNEG: { const int n = c.i0; for (int i = t; i < n; i += ST) p0[i] = p0[i] + (0.0f - p1[i]); break; }
@@ -152,6 +169,60 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
       const bool need_g = !((op == LH_RELU || op == LH_HARDTANH) && inplace);
       for (int i = t; i < n; i += ST)
         p0[i] = cl_unary_grad(op, inplace, p0[i], need_x ? p1[i] : 0.f, need_y ? p2[i] : 0.f, need_g ? p3[i] : 0.f, lo, hi);
+      break;
+    }
+    case CL_PRELOAD: {           // element t of up to four vectors into their slots (all loads in flight together), and where the vectors live
+      const uint32_t n01 = (uint32_t)c.i0, n23 = (uint32_t)c.i2, sl = (uint32_t)c.i1;
+      const int n0 = n01 & 0xffff, n1 = n01 >> 16, n2 = n23 & 0xffff, n3 = n23 >> 16;
+      const float v0 = t < n0 ? p0[t] : 0.f, v1 = t < n1 ? p1[t] : 0.f, v2 = t < n2 ? p2[t] : 0.f, v3 = t < n3 ? p3[t] : 0.f;
+      if (t < n0) S[(sl & 0xff) * CL_SLOT_ELEMS + t] = v0;
+      if (t < n1) S[((sl >> 8) & 0xff) * CL_SLOT_ELEMS + t] = v1;
+      if (t < n2) S[((sl >> 16) & 0xff) * CL_SLOT_ELEMS + t] = v2;
+      if (t < n3) S[(sl >> 24) * CL_SLOT_ELEMS + t] = v3;
+      if (t == 0) {
+        if (n0) SP[sl & 0xff] = (uint64_t)(uintptr_t)c.p0;
+        if (n1) SP[(sl >> 8) & 0xff] = (uint64_t)(uintptr_t)c.p1;
+        if (n2) SP[(sl >> 16) & 0xff] = (uint64_t)(uintptr_t)c.p2;
+        if (n3) SP[sl >> 24] = (uint64_t)(uintptr_t)c.p3;
+      }
+      break;
+    }
+    case CL_SYNC: __syncthreads(); break;
+    case CL_CHAIN: {             // c.i0 packed commands in the entries behind this one (the same staged chunk): LDS to LDS, results also to memory
+      const int count = c.i0;
+      const uint4* prog = reinterpret_cast<const uint4*>(&c + 1);
+      uint4 ahead = prog[0];
+      for (int m = 0; m < count; m++) {
+        const uint32_t w0 = __builtin_amdgcn_readfirstlane(ahead.x), w1 = __builtin_amdgcn_readfirstlane(ahead.y);
+        const float f0 = __uint_as_float(__builtin_amdgcn_readfirstlane(ahead.z)), f1 = __uint_as_float(__builtin_amdgcn_readfirstlane(ahead.w));
+        ahead = prog[m + 1];                                   // the entry after the last packed command exists (the list's op words follow the commands)
+        const int mop = w0 & 0xff, n = (int)(w1 >> 16), sub = (int)(w1 >> 8) & 0x7f, inplace = (int)(w1 >> 15) & 1;
+        if (t >= n) continue;
+        float* d = S + ((w0 >> 8) & 0xff) * CL_SLOT_ELEMS + t;
+        const float* a = S + ((w0 >> 16) & 0xff) * CL_SLOT_ELEMS + t;
+        const float* b = S + (w0 >> 24) * CL_SLOT_ELEMS + t;
+        const float* g = S + (w1 & 0xff) * CL_SLOT_ELEMS + t;
+        float r;
+        switch (mop) {
+          case CL_FILL: r = f0; break;
+          case CL_COPY: r = *a; break;
+          case CL_GEAM: r = *a * f0 + *b * f1; break;
+          case CL_SCALAR: r = cl_bop(sub, *a, f0); break;
+          case CL_BIN: r = cl_bop(sub, *a, *b); break;
+          case CL_ACC: r = *d + *a; break;
+          case CL_ACCNEG: r = *d + (0.0f - *a); break;
+          case CL_ACCMUL: r = *d + *a * *b; break;
+          case CL_UNARY: r = cl_unary(sub, *a, f0, f1); break;
+          default: {             // CL_UNARY_GRAD: d = dx, a = x, b = y, g = dy
+            const bool rh = sub == LH_RELU || sub == LH_HARDTANH;
+            const bool need_x = rh ? !inplace : (sub == LH_LOG || sub == LH_SQUARE), need_y = rh ? inplace != 0 : !(sub == LH_LOG || sub == LH_SQUARE), need_g = !(rh && inplace);
+            r = cl_unary_grad(sub, inplace, *d, need_x ? *a : 0.f, need_y ? *b : 0.f, need_g ? *g : 0.f, f0, f1);
+            break;
+          }
+        }
+        *d = r;
+        ((gfloat*)(uintptr_t)SP[(w0 >> 8) & 0xff])[t] = r;
+      }
       break;
     }
     case CL_GEMV_N: {            // y[m] = alpha * A[m,n] x[n] + beta * y   (p0 = y, p1 = A, p2 = x; i2 = lda): a wavefront takes
@@ -267,14 +338,14 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
     }
     case CL_AXPY_DEV: {          // y += s[0] * x   (p0 = y, p1 = s, p2 = x)
       const int n = c.i0;
-      const float a = *(volatile float*)p1;                 // written by an earlier command: a vector load, not the scalar cache
+      const float a = *(volatile gfloat*)p1;                 // written by an earlier command: a vector load, not the scalar cache
       for (int i = t; i < n; i += ST) p0[i] = p0[i] + a * p2[i];
       break;
     }
     case CL_SOFTMAX: {           // rows of length cc, a wavefront per row   (p0 = y, p1 = x; i2 = log form)
       const int rows = c.i0, cc = c.i1, is_log = c.i2;
       for (int r = wave; r < rows; r += NW) {
-        const float* xp = p1 + (int64_t)r * cc; float* yp = p0 + (int64_t)r * cc;
+        const gfloat* xp = p1 + (int64_t)r * cc; gfloat* yp = p0 + (int64_t)r * cc;
         float mx = -3.402823466e+38f;
         for (int j = lane; j < cc; j += 64) mx = fmaxf(mx, xp[j]);
         mx = cl_wave_max_all(mx);
@@ -301,12 +372,12 @@ __device__ __forceinline__ void cl_run(const LhCmd& c, const int opc, const int 
       break;
     }
     case CL_NLL: {               // y[b] = -x[b*stride + target[b]]   (p0 = y, p1 = x, p2 = target)
-      const int batch = c.i0, stride = c.i1; const int* tg = (const int*)c.p2;
+      const int batch = c.i0, stride = c.i1; const gint* tg = (const gint*)(uintptr_t)c.p2;
       for (int b = t; b < batch; b += ST) p0[b] = -1.0f * p1[(int64_t)b * stride + tg[b]];
       break;
     }
     case CL_NLL_GRAD: {          // dx[b*stride + target[b]] += -dy[b]   (p0 = dx, p1 = dy, p2 = target)
-      const int batch = c.i0, stride = c.i1; const int* tg = (const int*)c.p2;
+      const int batch = c.i0, stride = c.i1; const gint* tg = (const gint*)(uintptr_t)c.p2;
       for (int b = t; b < batch; b += ST) p0[(int64_t)b * stride + tg[b]] += -1.0f * p1[b];
       break;
     }
@@ -368,6 +439,8 @@ __global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const uint2* dir, const 
                                                         unsigned long long sync_base, unsigned* host_flag, unsigned long long* trace) {
   __shared__ uint4 stage[CL_CHUNK * 4];                 // 256 commands of 64 bytes
   __shared__ uint2 sop[CL_CHUNK + 1];
+  extern __shared__ float slots[];                      // Ring::nslot slots of CL_SLOT_ELEMS floats
+  __shared__ uint64_t slot_ptr[CL_NSLOT_MAX];
   __shared__ int gave_up;
   constexpr int NW = CL_THREADS / 64;
   const int t = threadIdx.x, grp = blockIdx.x, ngrp = gridDim.x;
@@ -416,7 +489,7 @@ __global__ void __launch_bounds__(CL_THREADS) k_cmdlist(const uint2* dir, const 
         GW = NW;
       }
       if (gw >= pieces) continue;                       // no part of this command falls to this wavefront
-      cl_run(list[i], (int)(op & CL_OP_MASK), gw, GW);
+      cl_run(list[i], (int)(op & CL_OP_MASK), gw, GW, slots, slot_ptr);
     }
     __syncthreads();                                    // the staged commands are no longer read
   }
@@ -445,10 +518,23 @@ static bool ring_init() {
   int groups = 32;
   if (const char* e = getenv("LH_CMDLIST_GROUPS")) groups = atoi(e);
   if (const char* e = getenv("LH_CMDLIST_CHAINS")) g_chains = atoi(e) != 0;
+  if (const char* e = getenv("LH_CMDLIST_SLOTS")) g_slots = atoi(e) != 0;
   if (groups < 1) groups = 1;
   if (groups > CL_MAX_GROUPS) groups = CL_MAX_GROUPS;
   if (groups > g_num_cu / 4) groups = g_num_cu / 4 > 0 ? g_num_cu / 4 : 1;       // all workgroups of a launch must be resident together
   g_ring.groups = groups;
+  // LDS for the operand slots of chain programs: all the device gives a workgroup beyond the kernel's fixed 20 KB, 128 slots at most
+  g_ring.nslot = 44;
+  {
+    int lds = 0, dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && lds > 0) {
+      int want = (lds - 20 * 1024) / (CL_SLOT_ELEMS * 4);
+      if (want > CL_NSLOT_MAX) want = CL_NSLOT_MAX;
+      if (want > 44 && hipFuncSetAttribute(reinterpret_cast<const void*>(&k_cmdlist), hipFuncAttributeMaxDynamicSharedMemorySize, want * CL_SLOT_ELEMS * 4) == hipSuccess) g_ring.nslot = want;
+      else (void)hipGetLastError();
+    }
+    if (const char* e = getenv("LH_CMDLIST_NSLOT")) { const int v = atoi(e); if (v >= 0 && v <= g_ring.nslot) g_ring.nslot = v; }
+  }
   g_ring.cur = 0; g_ring.ready = true;
   return true;
 }
@@ -662,7 +748,9 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
 }
 }  // namespace
 
+static inline void memcpy_host(void* d, const void* s_, size_t nbytes) { __builtin_memcpy(d, s_, nbytes); }
 namespace lh {
+static long long g_stat_slot_chains = 0, g_stat_slots = 0, g_stat_chain_ptrs = 0;
 static unsigned long long g_tsc_push = 0, g_tsc_flush = 0, g_tsc_wait = 0, g_tsc_conf = 0, g_tsc_note = 0;      // host cycles spent recording (LH_CMDLIST_VERBOSE prints them)
 // Hands the recorded buffer to the device: commands in level order (recording order within a level), the first of each
 // level flagged for a barrier, each with the wavefront its elements start on.
@@ -691,12 +779,9 @@ void rec_flush() {
   for (int l = 0; l <= W.top; l++) { rot_of_level[l] = 0; owner_of_level[l] = 0; split_of_level[l] = 0; }
   static int chain_place[CL_BUF_CMDS + 1];
   for (int ch = 0; ch < W.nchains; ch++) chain_place[ch] = -1;
-  // Pass 1: where each command runs, and how long each workgroup's list gets.
+  // Pass 1: where each command runs.
   struct Place { uint32_t op, pieces; int g0, gn; };
   static Place place[CL_BUF_CMDS];
-  int entries[CL_MAX_GROUPS], passed[CL_MAX_GROUPS];
-  for (int g = 0; g < groups; g++) entries[g] = passed[g] = 0;
-  auto entries_for = [](int need) { return 1 + (need > 255 ? (need - 1) / 255 : 0); };      // an entry carries up to 255 barriers
   for (int k = 0; k < n; k++) {
     const int i = order[k], l = W.level[i];
     const LhCmd& c = W.cmd[i];
@@ -727,29 +812,166 @@ void rec_flush() {
       const int span = waves < all_w ? waves : all_w, b0 = at / CL_WBLOCK, b1 = (at + span - 1) / CL_WBLOCK;
       pl.g0 = b0 % groups; pl.gn = b1 - b0 + 1 < groups ? b1 - b0 + 1 : groups;
     } else { pl.g0 = owner; pl.gn = 1; }
-    for (int j = 0; j < pl.gn; j++) { const int g = (pl.g0 + j) % groups; entries[g] += entries_for(l - 1 - passed[g]); passed[g] = l - 1; }
   }
   const int barriers = W.top > 1 ? W.top - 1 : 0;
-  for (int g = 0; g < groups; g++) if (passed[g] < barriers) entries[g] += entries_for(barriers - passed[g]);
-  // Pass 2: the lists, one after the other.
+  // Chain programs.  The commands of an element-wise chain run one after the other on the same few wavefronts, and what one such
+  // command costs is not memory but the interpreter: some 280 dependent instructions of one wavefront, 0.7 us.  A chain of at least
+  // PROGRAM_MIN_CHAIN commands, all of kinds that write one result, none longer than an LDS slot, whose distinct operand addresses
+  // all get a slot of its workgroup (Ring::nslot per workgroup and level), becomes ONE entry of kind CL_CHAIN followed by its
+  // commands packed 16 bytes each (operation, slots, length, two scalars).  The workgroup loads every slotted vector, and notes its
+  // address, before its first entry of the level (entries of kind CL_PRELOAD on different wavefronts, then one CL_SYNC); the chain's
+  // wavefronts then run the packed commands from LDS to LDS, writing every result through to memory.
+  struct ChainProg { int count, nptr, head, owner, level, pieces, base, next, first_k, last_k; bool ok, programmed, emitted; };
+  struct ChainPtr { const void* p; int maxn, idx, next; };
+  static ChainProg cs[CL_BUF_CMDS + 1];
+  static ChainPtr cp[CL_BUF_CMDS * 4];
+  static uint32_t ptr_index[CL_BUF_CMDS];                      // per command (by position in `order`): the chain-local index of each pointer, a byte each
+  static int next_in_chain[CL_BUF_CMDS];
+  static uint8_t slots_used[CL_BUF_CMDS + 2][CL_MAX_GROUPS];
+  static int16_t bucket[CL_BUF_CMDS + 2][CL_MAX_GROUPS];       // the programmed chains of a (level, workgroup), linked through ChainProg::next
+  constexpr int PROGRAM_MIN_CHAIN = 6, SEGMENT = 128;          // commands of one CL_CHAIN entry at most (32 entries of payload behind it)
+  const bool use_programs = g_chains && g_slots;
+  for (int ch = 0; ch < W.nchains; ch++) { cs[ch].count = 0; cs[ch].programmed = false; cs[ch].emitted = false; }
+  if (use_programs) {
+    int ncp = 0;
+    for (int l = 0; l <= W.top; l++) for (int g = 0; g < groups; g++) { slots_used[l][g] = 0; bucket[l][g] = -1; }
+    for (int k = 0; k < n; k++) {
+      const int i = order[k], ch = W.chain[i];
+      if (ch < 0 || W.chain_class[ch] != 1) continue;
+      const LhCmd& c = W.cmd[i];
+      ChainProg& C = cs[ch];
+      if (C.count == 0) { C.nptr = 0; C.head = -1; C.owner = place[k].g0; C.level = W.level[i]; C.pieces = 1; C.ok = true; C.first_k = k; }
+      else next_in_chain[C.last_k] = k;
+      C.last_k = k; next_in_chain[k] = -1;
+      C.count++;
+      if (c.op == CL_ADAGRAD || c.op == CL_SGD || c.i0 > CL_SLOT_ELEMS) C.ok = false;
+      if (!C.ok) continue;
+      if ((int)place[k].pieces > C.pieces) C.pieces = (int)place[k].pieces;
+      const void* ptrs[4] = {c.p0, c.p1, c.p2, c.p3};
+      uint32_t word = 0;
+      for (int q = 0; q < 4; q++) {
+        uint32_t idx = 0xff;
+        if (ptrs[q]) {
+          int e = C.head;
+          while (e >= 0 && cp[e].p != ptrs[q]) e = cp[e].next;
+          if (e < 0 && C.nptr < r.nslot) { e = ncp++; cp[e].p = ptrs[q]; cp[e].maxn = 0; cp[e].idx = C.nptr++; cp[e].next = C.head; C.head = e; }
+          if (e < 0) C.ok = false;                              // more distinct operands than a workgroup has slots
+          else { if (c.i0 > cp[e].maxn) cp[e].maxn = c.i0; idx = (uint32_t)cp[e].idx; }
+        }
+        word |= idx << (8 * q);
+      }
+      ptr_index[k] = word;
+    }
+    for (int ch = 0; ch < W.nchains; ch++) {
+      ChainProg& C = cs[ch];
+      if (C.count < PROGRAM_MIN_CHAIN || !C.ok || W.chain_class[ch] != 1) continue;
+      uint8_t& used = slots_used[C.level][C.owner];
+      if (C.nptr > r.nslot - used) continue;                  // the workgroup's slots of this level are taken: the chain runs command by command
+      C.base = used; used = (uint8_t)(used + C.nptr);
+      C.programmed = true;
+      g_stat_slot_chains++; g_stat_slots += C.nptr; g_stat_chain_ptrs += C.count;
+      C.next = bucket[C.level][C.owner]; bucket[C.level][C.owner] = (int16_t)ch;
+    }
+  }
+  // Pass 2: the entries in the order they are made, each tagged with its workgroup; then every workgroup's entries are gathered
+  // into its list in the buffer.
+  struct Rec { LhCmd cmd; uint32_t op, pieces; int g; };
+  static Rec* recs = nullptr;
+  if (!recs) recs = new Rec[CL_CAP + CL_BUF_CMDS];
+  int nrec = 0;
+  int list_at[CL_MAX_GROUPS], list_n[CL_MAX_GROUPS], passed[CL_MAX_GROUPS], at_level[CL_MAX_GROUPS], total = 0;
+  auto put1 = [&](int g, uint32_t op, uint32_t pieces, const void* cmd64) {        // one entry on workgroup g's list
+    if (nrec < CL_CAP + CL_BUF_CMDS) { Rec& rc = recs[nrec]; rc.g = g; rc.op = op; rc.pieces = pieces; if (cmd64) memcpy_host(&rc.cmd, cmd64, sizeof(LhCmd)); }
+    nrec++;
+    list_n[g]++;
+  };
+  auto put = [&](int g, uint32_t op, uint32_t pieces, const void* cmd64, int l) {  // ... that belongs to level l: the barriers passed since come with it
+    int need = l - 1 - passed[g];
+    passed[g] = l - 1;
+    for (; need > 255; need -= 255) put1(g, (uint32_t)CL_NOP | (255u << CL_BARRIERS_SHIFT), 0u, nullptr);
+    put1(g, op | ((uint32_t)need << CL_BARRIERS_SHIFT), pieces, cmd64);
+  };
+  // the first entry of workgroup g at level l is about to be put: the level's preloads come before it
+  auto open_level = [&](int g, int l) {
+    at_level[g] = l;
+    if (!use_programs || bucket[l][g] < 0) return;
+    int rot = 0;
+    for (int ch = bucket[l][g]; ch >= 0; ch = cs[ch].next) {
+      const ChainProg& C = cs[ch];
+      LhCmd pc = LhCmd{}; int filled = 0;
+      for (int e = C.head; e >= 0; e = cp[e].next) {
+        const uint32_t nn = (uint32_t)cp[e].maxn, sl = (uint32_t)(C.base + cp[e].idx);
+        switch (filled) {
+          case 0: pc = LhCmd{}; pc.op = CL_PRELOAD; pc.p0 = (void*)cp[e].p; pc.i0 = (int32_t)nn; pc.i1 = (int32_t)sl; break;
+          case 1: pc.p1 = (void*)cp[e].p; pc.i0 = (int32_t)((uint32_t)pc.i0 | (nn << 16)); pc.i1 = (int32_t)((uint32_t)pc.i1 | (sl << 8)); break;
+          case 2: pc.p2 = (void*)cp[e].p; pc.i2 = (int32_t)nn; pc.i1 = (int32_t)((uint32_t)pc.i1 | (sl << 16)); break;
+          default: pc.p3 = (void*)cp[e].p; pc.i2 = (int32_t)((uint32_t)pc.i2 | (nn << 16)); pc.i1 = (int32_t)((uint32_t)pc.i1 | (sl << 24)); break;
+        }
+        if (++filled == 4 || cp[e].next < 0) {
+          put(g, (uint32_t)CL_PRELOAD | ((uint32_t)(rot & 15) << CL_START_SHIFT), (uint32_t)C.pieces, &pc, l);
+          rot += C.pieces; filled = 0;
+        }
+      }
+    }
+    LhCmd sync = LhCmd{}; sync.op = CL_SYNC;
+    put(g, (uint32_t)CL_SYNC, 0xffffu, &sync, l);
+  };
+  // a programmed chain, at the place of its first command: CL_CHAIN entries of up to SEGMENT commands, each followed by its packed commands
+  auto put_chain = [&](int g, int ch, int l, uint32_t place_op) {
+    ChainProg& C = cs[ch];
+    int k = C.first_k;
+    while (k >= 0) {
+      int seg = 0;
+      for (int kk = k; kk >= 0 && seg < SEGMENT; kk = next_in_chain[kk]) seg++;
+      const int payload = (seg + 3) / 4;
+      if (passed[g] < l - 1) put(g, (uint32_t)CL_NOP, 0u, nullptr, l);                   // the barriers before the chain, on an entry of their own
+      // the entry and its payload sit in one staged chunk of the list
+      while ((list_n[g] % CL_CHUNK) + 1 + payload > CL_CHUNK) put1(g, (uint32_t)CL_NOP, 0u, nullptr);
+      LhCmd head = LhCmd{}; head.op = CL_CHAIN; head.i0 = seg;
+      put1(g, (uint32_t)CL_CHAIN | (place_op & (0xfffu << CL_START_SHIFT)), (uint32_t)C.pieces, &head);
+      uint32_t pack[16]; int filled = 0;
+      for (int m = 0; m < seg; m++, k = next_in_chain[k]) {
+        const LhCmd& c = W.cmd[order[k]];
+        uint32_t sl[4];
+        for (int q = 0; q < 4; q++) { const uint32_t idx = (ptr_index[k] >> (8 * q)) & 0xffu; sl[q] = idx == 0xffu ? 0u : (uint32_t)C.base + idx; }
+        union { float f; uint32_t u; } f0, f1; f0.f = c.f0; f1.f = c.f1;
+        uint32_t* w = pack + 4 * filled;
+        w[0] = (uint32_t)c.op | (sl[0] << 8) | (sl[1] << 16) | (sl[2] << 24);
+        w[1] = sl[3] | (((uint32_t)c.i1 & 0x7fu) << 8) | ((c.i2 ? 1u : 0u) << 15) | ((uint32_t)c.i0 << 16);
+        w[2] = f0.u; w[3] = f1.u;
+        if (++filled == 4 || m + 1 == seg) { for (int z = 4 * filled; z < 16; z++) pack[z] = 0; put1(g, (uint32_t)CL_NOP, 0u, pack); filled = 0; }
+      }
+    }
+    C.emitted = true;
+  };
+  auto emit_all = [&]() {
+    for (int g = 0; g < groups; g++) { list_n[g] = 0; passed[g] = 0; at_level[g] = 0; }
+    for (int ch = 0; ch < W.nchains; ch++) cs[ch].emitted = false;
+    for (int k = 0; k < n; k++) {
+      const int i = order[k], l = W.level[i], ch = W.chain[i];
+      const Place& pl = place[k];
+      for (int j = 0; j < pl.gn; j++) {
+        const int g = (pl.g0 + j) % groups;
+        if (at_level[g] != l) open_level(g, l);
+        if (ch >= 0 && cs[ch].programmed) { if (!cs[ch].emitted) put_chain(g, ch, l, pl.op); }
+        else put(g, pl.op, pl.pieces, &W.cmd[i], l);
+      }
+    }
+    for (int g = 0; g < groups; g++) if (passed[g] < barriers) put(g, (uint32_t)CL_NOP, 0u, nullptr, barriers + 1);
+  };
+  emit_all();
+  for (int g = 0; g < groups; g++) { list_at[g] = total; total += list_n[g]; }
+  if (total > CL_CAP || nrec != total) { window_reset(W); LH_FAIL("command list: %d entries exceed a buffer (%d)", nrec, CL_CAP); return; }
   uint2* dir = reinterpret_cast<uint2*>(r.host[r.cur]);
   LhCmd* out = reinterpret_cast<LhCmd*>(r.host[r.cur] + CL_DIR_BYTES);
-  int first[CL_MAX_GROUPS], total = 0;
-  for (int g = 0; g < groups; g++) { first[g] = total; dir[g] = make_uint2((uint32_t)total, (uint32_t)entries[g]); total += entries[g]; passed[g] = 0; }
-  if (total > CL_CAP) { window_reset(W); LH_FAIL("command list: %d entries exceed a buffer (%d)", total, CL_CAP); return; }
   uint2* ops = reinterpret_cast<uint2*>(out + total);
-  auto put = [&](int g, uint32_t op, uint32_t pieces, const LhCmd* c, int need) {
-    for (; need > 255; need -= 255) { ops[first[g]] = make_uint2((uint32_t)CL_NOP | (255u << CL_BARRIERS_SHIFT), 0u); first[g]++; }
-    ops[first[g]] = make_uint2(op | ((uint32_t)need << CL_BARRIERS_SHIFT), pieces);
-    if (c) out[first[g]] = *c;
-    first[g]++;
-  };
-  for (int k = 0; k < n; k++) {
-    const int i = order[k], l = W.level[i];
-    const Place& pl = place[k];
-    for (int j = 0; j < pl.gn; j++) { const int g = (pl.g0 + j) % groups; put(g, pl.op, pl.pieces, &W.cmd[i], l - 1 - passed[g]); passed[g] = l - 1; }
+  for (int g = 0; g < groups; g++) { dir[g] = make_uint2((uint32_t)list_at[g], (uint32_t)list_n[g]); list_n[g] = 0; }
+  for (int q = 0; q < nrec; q++) {
+    const Rec& rc = recs[q];
+    const int at = list_at[rc.g] + list_n[rc.g]++;
+    ops[at] = make_uint2(rc.op, rc.pieces);
+    memcpy_host(&out[at], &rc.cmd, sizeof(LhCmd));
   }
-  for (int g = 0; g < groups; g++) if (passed[g] < barriers) put(g, (uint32_t)CL_NOP, 0u, nullptr, barriers - passed[g]);
   g_ring.levels += W.top;
   // LH_CMDLIST_TRACE=<launch>: workgroup 0 notes the time of every barrier of that launch and the next one; the host prints how long
   // each level took and what it held (a diagnostic: the launch is waited for)
@@ -771,7 +993,7 @@ void rec_flush() {
   ProfScope prof_(CAT_CMDLIST);
   hipError_t e = hipMemcpyAsync(r.mirror, r.host[r.cur], CL_DIR_BYTES + (sizeof(LhCmd) + sizeof(uint2)) * (size_t)total, hipMemcpyHostToDevice, g_stream_raw);
   if (e != hipSuccess) { LH_FAIL("command list copy: %s", hipGetErrorString(e)); return; }
-  hipLaunchKernelGGL(k_cmdlist, dim3(groups), dim3(CL_THREADS), 0, g_stream_raw, reinterpret_cast<const uint2*>(r.mirror),
+  hipLaunchKernelGGL(k_cmdlist, dim3(groups), dim3(CL_THREADS), (size_t)r.nslot * CL_SLOT_ELEMS * 4, g_stream_raw, reinterpret_cast<const uint2*>(r.mirror),
                      reinterpret_cast<const uint2*>(r.mirror + CL_DIR_BYTES + sizeof(LhCmd) * (size_t)total), reinterpret_cast<const LhCmd*>(r.mirror + CL_DIR_BYTES),
                      r.sync, r.sync_base, r.host_flag_dev, tracing ? trace_buf : nullptr);
   if (tracing) {
@@ -805,14 +1027,15 @@ bool rec_push(const LhCmd& c) {
   Extent x[4];
   const int k = cmd_extents(c, x);
   // the lists of how many workgroups the command goes on (an upper bound; the barrier-only entries are allowed for below)
-  int copies = 1;
+  int copies = cmd_lanewise(c) ? 3 : 1;             // an element-wise command may bring a CL_PRELOAD and a CL_SYNC entry with it
   if (cmd_splits(c)) {
     const int all_w = g_ring.groups * (CL_THREADS / 64), span = cmd_waves(c) < all_w ? cmd_waves(c) : all_w;
     copies = (span + CL_WBLOCK - 2) / CL_WBLOCK + 1;
     if (copies > g_ring.groups) copies = g_ring.groups;
   }
   for (int attempt = 0; attempt < 2; attempt++) {
-    if (W.n == CL_BUF_CMDS || W.entries + copies + g_ring.groups * 10 > CL_CAP) { rec_flush(); if (failed()) return false; }
+    // (a chain program is padded so that it does not straddle two staged chunks: up to 33 entries per 256, allowed for here)
+    if (W.n == CL_BUF_CMDS || W.entries + copies + g_ring.groups * 10 > CL_CAP - CL_BUF_CMDS) { rec_flush(); if (failed()) return false; }
     // cf: what the command must follow through operands that map onto wavefronts as the chain's do (all operands of an element-wise
     // command; what a matrix command writes, which cmd_extents lists first); cf_in: through what a matrix command reads
     Conflict cf, cf_in;
@@ -864,6 +1087,8 @@ void lh_cmdlist_end(void) {
   rec_flush();
   g_rec_on = 0;
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld commands in %lld levels, %lld launches\n", (long long)g_ring.recorded, (long long)g_ring.levels, (long long)g_ring.launches);
+  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %d operand slots per workgroup\n", g_ring.nslot);
+  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld chains run as programs, %lld operand slots, %lld commands in them\n", g_stat_slot_chains, g_stat_slots, g_stat_chain_ptrs);
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list host cycles: push %.1f M (flush inside %.1f M, of which waiting for a free buffer %.1f M), conflicts %.1f M, notes %.1f M\n", g_tsc_push * 1e-6, g_tsc_flush * 1e-6, g_tsc_wait * 1e-6, g_tsc_conf * 1e-6, g_tsc_note * 1e-6);
 }
 void lh_cmdlist_stats(int64_t* recorded, int64_t* launches) {

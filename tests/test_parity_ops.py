@@ -1045,8 +1045,66 @@ def test_command_list_reordering_keeps_every_dependence(on_hip):
     finally:
         be.batchSmallOps(False)
     assert all(np.isfinite(a).all() for a in direct)
+    # the matrix commands sum in another order than the stand-alone kernels (whose transposed product combines blocks with atomic
+    # adds, so its own result moves in the last bits from run to run), and 600 dependent operations carry that along: 1e-4, the
+    # tolerance for sums whose order is free; a command that ran before what it depends on is off by far more
     for i, (a, b_) in enumerate(zip(listed, direct)):
-        assert_close(a, b_, rtol=2e-5, what="buffer %d" % i)
+        assert_close(a, b_, rtol=1e-4, what="buffer %d" % i)
+
+
+def test_command_list_long_element_wise_chains_keep_their_operands_in_lds(on_hip):
+    """Chains of element-wise commands on the same vectors (each lane reads what it wrote itself) run inside one level; from four
+    commands on, the chain's operands are loaded into LDS slots before its first command and every result is written to the slot and
+    to memory.  Several independent chains of 60 commands over shared read-only inputs, in-place updates, operands of different
+    lengths at one address, more distinct operands than a workgroup has slots (the rest go through memory), gradient forms, and a
+    read of every buffer by a matrix command afterwards must give the bits of the same program issued one launch per operator."""
+    be = on_hip
+    lib = be.lib
+    vlen = 150
+
+    def program():
+        mark = be.getMallocAddr()
+        r = np.random.RandomState(3)
+        const = [be.fromHost((r.rand(vlen) + 0.5).astype(np.float32)) for _ in range(6)]        # read by every chain, written by none
+        outs = []
+        for chain in range(5):
+            n_own = 4 if chain < 4 else 48                                                        # the last chain has more operands than slots
+            own = [be.fromHost((r.rand(vlen) * 0.5 + 0.25).astype(np.float32)) for _ in range(n_own)]
+            ops = np.random.RandomState(100 + chain)
+            for step in range(60):
+                k = int(ops.randint(0, 8))
+                a, b_, c = (int(v) for v in ops.randint(0, n_own, 3))
+                u = const[int(ops.randint(0, len(const)))]
+                if k == 0: lib.lh_geam(own[a].ptr, 0.5, u.ptr, 0.25, own[c].ptr, vlen)
+                elif k == 1: lib.lh_unary(B.TANH, own[a].ptr, own[c].ptr, vlen, -1.0, 1.0)
+                elif k == 2: lib.lh_unary(B.SIGMOID, own[a].ptr, own[a].ptr, vlen, -1.0, 1.0)      # in place
+                elif k == 3: lib.lh_geam(own[a].ptr, 1.0, own[b_].ptr, -0.5, own[a].ptr, 40)        # a shorter range at the same address
+                elif k == 4: lib.lh_scalar_op(B.MUL, own[a].ptr, own[c].ptr, 0.75, vlen)
+                elif k == 5: lib.lh_unary_grad(B.TANH, u.ptr, own[a].ptr, own[b_].ptr, own[c].ptr, vlen, 0, -1.0, 1.0) if c not in (a, b_) else None
+                elif k == 6: lib.lh_fill(own[c].ptr, 0.125 * (step % 5), 100)
+                else: lib.lh_geam(own[a].ptr, 0.9, own[b_].ptr, 0.1, own[c].ptr, vlen)
+                if k == 5 and c not in (a, b_): lib.lh_unary(B.TANH, own[c].ptr, own[c].ptr, vlen, -1.0, 1.0)   # keeps the accumulator bounded
+            outs += own
+        # a matrix command over all results afterwards (another level: it must see what the chains wrote through to memory)
+        acc = be.mallocArray(vlen)
+        for v in outs[:8]: lib.lh_ger(1, vlen, const[0].ptr, v.ptr, acc.ptr)
+        from lantern_amd import _lib
+        _lib.check()
+        res = [be.toHost(v, vlen).copy() for v in outs] + [be.toHost(acc, vlen).copy()] + [be.toHost(v, vlen).copy() for v in const]
+        be.resetMallocAddr(mark)
+        return res
+
+    direct = program()
+    be.batchSmallOps(True)
+    try:
+        listed = program()
+    finally:
+        be.batchSmallOps(False)
+    assert all(np.isfinite(a).all() for a in direct)
+    n_chain_buffers = 4 * 4 + 48
+    for i, (a, b_) in enumerate(zip(listed, direct)):
+        if i == n_chain_buffers: assert_close(a, b_, rtol=2e-6, what="rank-1 updates over the chains' results")      # a + u * v may or may not be fused
+        else: assert np.array_equal(a, b_), "buffer %d differs by up to %g" % (i, np.abs(a - b_).max())
 
 
 # ---- residual join behind a batch norm: out = relu(bn(x) + shortcut) -----------------------------------
