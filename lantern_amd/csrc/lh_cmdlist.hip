@@ -12,8 +12,8 @@
 // than the highest level it depends on.  The buffer is executed level by level: commands of one level have no dependence on each
 // other and are spread over the workgroups and their wavefronts, so their round trips overlap; one barrier over all workgroups
 // per level makes a level's stores visible to the next.  Independent work of a program (the ten gate products of a tree node, the
-// two subtrees of a node) thus runs side by side without the program saying so.  Element-wise commands that depend only on each
-// other, lane by lane, share a level (a chain).  Each workgroup gets its own list of the commands it has a part in: the walk over
+// two subtrees of a node) thus runs side by side without the program saying so.  Commands that depend only on each other, lane by
+// lane (or row by row of what they write), share a level (a chain); long element-wise chains run as programs over LDS.  Each workgroup gets its own list of the commands it has a part in: the walk over
 // a list is scalar work, and a compute unit has one scalar unit for its 16 wavefronts.
 // The arithmetic of each command follows the stand-alone kernel of the same operation; no command uses atomics, so the result does
 // not depend on how many workgroups run it.
