@@ -61,7 +61,8 @@ def make_trainer(args, batch, cpu=False):
         from lantern_amd.apps.deepspeech2 import Trainer
         # learning rate 1e-5: the reference program's 3e-4 (DeepSpeech.scala:127) diverges within ten steps on random spectrograms
         return Trainer(batch=batch, freq=161, frames=args.frames, hidden=args.hidden, layers=3, label_len=50, lr=1e-5), batch, \
-            "DeepSpeech2-style step (configs[4]): batch %d, 1x161x%d, 3 bidirectional tanh RNN layers hidden %d, CTC over 29 symbols, Nesterov SGD lr 1e-5" % (batch, args.frames, args.hidden)
+            "DeepSpeech2-style step (configs[4]): batch %d, 1x161x%d, 3 bidirectional tanh RNN layers hidden %d with sequence-wise batch norm in front of layers 2 and 3 " \
+            "(the reference program builds them with useBatchNorm = false), CTC over 29 symbols, Nesterov SGD lr 1e-5" % (batch, args.frames, args.hidden)
     raise SystemExit("unknown workload %r" % w)
 
 
