@@ -39,16 +39,17 @@ __global__ void __launch_bounds__(TPB) k_lstm_fwd_point(float* __restrict__ act,
 }
 
 // act [B, 4H]: activations on entry, pre-activation gradients on exit.  dh_rec / dc hold what flows in from the step
-// processed before (null / ignored on the first processed step); dc is rewritten with the cell gradient passed on.
+// processed before (ignored on the first processed step); dh_rec is cleared, dc is rewritten with the cell gradient passed on.
 __global__ void __launch_bounds__(TPB) k_lstm_bwd_point(float* __restrict__ act, const float* __restrict__ c, const float* __restrict__ c_prev,
-                                                        const float* __restrict__ dy, const float* __restrict__ dh_rec, float* __restrict__ dc,
+                                                        const float* __restrict__ dy, float* __restrict__ dh_rec, float* __restrict__ dc,
                                                         int first, int B, int H, int ldh) {
   const int idx = blockIdx.x * TPB + threadIdx.x;
   if (idx >= B * H) return;
   const int b = idx / H, j = idx - b * H;
   float* a = act + (size_t)b * 4 * H + j;
   const float ig = a[0], fg = a[H], gg = a[2 * H], og = a[3 * H];
-  const float dh = dy[(size_t)b * ldh + j] + (dh_rec ? dh_rec[idx] : 0.f);
+  const float dh = dy[(size_t)b * ldh + j] + (first ? 0.f : dh_rec[idx]);
+  dh_rec[idx] = 0.f;                                             // the product that follows adds the next recurrent gradient into it
   const float tc = tanhf(c[idx]);
   const float dcc = dh * og * (1.f - tc * tc) + (first ? 0.f : dc[idx]);
   const float cp = c_prev ? c_prev[idx] : 0.f;
@@ -60,17 +61,21 @@ __global__ void __launch_bounds__(TPB) k_lstm_bwd_point(float* __restrict__ act,
 }
 
 // act [B, 3H]: input projection on entry, r, z, n on exit.  gh [B, 3H] = h_prev W_hh^T or null.  q [B, H] = W_hn h + b_hn.
-__global__ void __launch_bounds__(TPB) k_gru_fwd_point(float* __restrict__ act, const float* __restrict__ gh, const float* __restrict__ b_ih,
+// gh is cleared after it is read: the next step's product adds into it (a product with beta = 0 cut over K needs a pass of its own
+// that clears the result first, a launch per step).
+__global__ void __launch_bounds__(TPB) k_gru_fwd_point(float* __restrict__ act, float* __restrict__ gh, const float* __restrict__ b_ih,
                                                        const float* __restrict__ b_hh, const float* __restrict__ h_prev, int ldp, float* __restrict__ q,
                                                        float* __restrict__ h, int B, int H, int ldh) {
   const int idx = blockIdx.x * TPB + threadIdx.x;
   if (idx >= B * H) return;
   const int b = idx / H, j = idx - b * H;
   float* a = act + (size_t)b * 3 * H + j;
-  const float* g = gh ? gh + (size_t)b * 3 * H + j : nullptr;
-  const float r = sigm(a[0] + b_ih[j] + b_hh[j] + (g ? g[0] : 0.f));
-  const float z = sigm(a[H] + b_ih[H + j] + b_hh[H + j] + (g ? g[H] : 0.f));
-  const float qq = (g ? g[2 * H] : 0.f) + b_hh[2 * H + j];
+  float* g = gh + (size_t)b * 3 * H + j;
+  const float g0 = g[0], g1 = g[H], g2 = g[2 * H];               // zeros when there is no previous state
+  g[0] = 0.f; g[H] = 0.f; g[2 * H] = 0.f;
+  const float r = sigm(a[0] + b_ih[j] + b_hh[j] + g0);
+  const float z = sigm(a[H] + b_ih[H + j] + b_hh[H + j] + g1);
+  const float qq = g2 + b_hh[2 * H + j];
   const float n = tanhf(a[2 * H] + b_ih[2 * H + j] + r * qq);
   const float hp = h_prev ? h_prev[(size_t)b * ldp + j] : 0.f;      // ldp: row stride of h_prev (an initial state is [B, H])
   a[0] = r; a[H] = z; a[2 * H] = n;
@@ -140,18 +145,20 @@ void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const floa
   LH_REQUIRE(cx == nullptr || mode == 2, "lh_rnn_gated_fwd: only the LSTM has a cell state");
   LH_REQUIRE(x && w && y && reserve, "lh_rnn_gated_fwd: null operand");
   const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
-  const size_t gh_bytes = (size_t)D * B * G * sizeof(float);
+  const size_t per_dir = (size_t)B * G;
+  const size_t gh_bytes = (size_t)D * per_dir * sizeof(float);
   float* gh_all = (float*)lh_malloc_uninit(gh_bytes);
   if (gh_all == nullptr) return;
   // The two directions of a bidirectional layer share nothing but the input: the reverse one runs on the library's second
   // stream beside the forward one (in line when that stream is off, while a graph is recorded or in deterministic mode).
   auto run_direction = [&](int d) {
-    float* gh = gh_all + (size_t)d * B * G;
+    float* gh = gh_all + (size_t)d * per_dir;
     const float* Wih = w + d * dir_params(mode, I, H);
     const float* Whh = Wih + (size_t)G * I; const float* bih = Whh + (size_t)G * H; const float* bhh = bih + G;
     float* act = reserve + d * dir_reserve(mode, T, B, H);
     float* aux = act + (size_t)T * B * G;
     lh_sgemm(0, 1, T * B, G, I, 1.0f, x, I, Wih, I, 0.0f, act, G);          // input projection of every step
+    if (mode == 3) lh_fill(gh, 0.0f, (int64_t)B * G);
     for (int step = 0; step < T; step++) {
       const int t = d == 0 ? step : T - 1 - step, tp = d == 0 ? t - 1 : t + 1;
       float* h = y + (size_t)t * B * ldh + d * H;
@@ -159,14 +166,19 @@ void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const floa
       const float* hp = step == 0 ? (hx ? hx + (size_t)d * B * H : nullptr) : y + (size_t)tp * B * ldh + d * H;
       const int ldp = step == 0 ? H : ldh;
       const float* cp = step == 0 ? (cx ? cx + (size_t)d * B * H : nullptr) : aux + (size_t)tp * B * H;
-      if (hp) lh_sgemm(0, 1, B, G, H, 1.0f, hp, ldp, Whh, H, 0.0f, gh, G);
       float* a = act + (size_t)t * B * G;
-      if (mode == 2)
-        hipLaunchKernelGGL(k_lstm_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh,
+      // the hidden-side product ADDS into its target (beta = 1): a product cut over K with beta = 0 would first need a launch that
+      // clears it.  The LSTM adds straight into the step's input projection; the GRU keeps the hidden side apart (its n gate scales
+      // it by r) in gh, which the point kernel clears after reading.
+      if (mode == 2) {
+        if (hp) lh_sgemm(0, 1, B, G, H, 1.0f, hp, ldp, Whh, H, 1.0f, a, G);
+        hipLaunchKernelGGL(k_lstm_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, nullptr, bih, bhh,
                            cp, aux + (size_t)t * B * H, h, B, H, ldh);
-      else
-        hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, hp ? gh : nullptr, bih, bhh, hp, ldp,
+      } else {
+        if (hp) lh_sgemm(0, 1, B, G, H, 1.0f, hp, ldp, Whh, H, 1.0f, gh, G);
+        hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, gh, bih, bhh, hp, ldp,
                            aux + (size_t)t * B * H, h, B, H, ldh);
+      }
     }
   };
   const bool fork = D == 2 && g_stream_cur == g_stream_raw;
@@ -209,8 +221,8 @@ void lh_rnn_gated_bwd_init(int mode, const float* x, const float* hx, const floa
       const float* dyt = dy + (size_t)t * B * ldh + d * H;
       if (mode == 2) {
         hipLaunchKernelGGL(k_lstm_bwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, aux + (size_t)t * B * H,
-                           has_prev ? aux + (size_t)tp * B * H : c0, dyt, k == 0 ? nullptr : carry, dc, k == 0 ? 1 : 0, B, H, ldh);
-        if (has_prev) lh_sgemm(0, 0, B, H, G, 1.0f, a, G, Whh, H, 0.0f, carry, H);
+                           has_prev ? aux + (size_t)tp * B * H : c0, dyt, carry, dc, k == 0 ? 1 : 0, B, H, ldh);
+        if (has_prev) lh_sgemm(0, 0, B, H, G, 1.0f, a, G, Whh, H, 1.0f, carry, H);       // into the carry the point kernel has just cleared
       } else {
         float* g = dgh + (size_t)t * B * G;
         hipLaunchKernelGGL(k_gru_bwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, g, aux + (size_t)t * B * H,
