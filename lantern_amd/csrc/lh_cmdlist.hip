@@ -605,7 +605,7 @@ static int cmd_waves(const LhCmd& c) {
 // buffers share a block only when one lies inside the other's allocation: then the dependence is real or harmless);
 // larger ranges (matrices, zero fills) in a short table of distinct ranges.  A level is a uint16: 1 + highest level touched.
 constexpr uintptr_t SMALL_BYTES = 4096;
-constexpr int HASH_N = 65536, BIG_N = 96, PAGE_N = 16384, PAGE_SCAN_MAX = 512;
+constexpr int HASH_N = 8192, BIG_N = 96, PAGE_N = 16384, PAGE_SCAN_MAX = 512;
 // Chains.  An element-wise command gives element i of every operand to the same lane (thread i mod 1024 of the workgroup and
 // wavefront rotation it runs on).  If everything such a command must follow at the highest level L is ONE chain of element-wise
 // commands, through ranges that start at the very addresses this command's operands start at, then each lane only ever needs what
@@ -619,13 +619,17 @@ constexpr int HASH_N = 65536, BIG_N = 96, PAGE_N = 16384, PAGE_SCAN_MAX = 512;
 struct Window {
   LhCmd cmd[CL_BUF_CMDS]; uint16_t level[CL_BUF_CMDS]; int16_t chain[CL_BUF_CMDS]; uint8_t chain_class[CL_BUF_CMDS + 1]; int32_t chain_row[CL_BUF_CMDS + 1]; int n; int top, nchains;       // top: highest level handed out
   int entries;                                                                // upper bound of the entries the workgroups' lists will hold
-  struct Slot { uintptr_t key, wbase, rbase; uint32_t epoch; uint16_t w, r; int16_t wchain, rchain; } slot[HASH_N]; uint32_t epoch;
+  // per 256-byte block: the highest level that writes / reads it, by which chain, through a range starting where (16 bits of the
+  // start's float index tell two ranges over one block apart); four neighbouring blocks share a 64-byte bucket
+  struct Slot { uint16_t wbase, rbase, w, r; int16_t wchain, rchain; };
+  struct Bucket { uintptr_t key; uint32_t epoch; Slot sub[4]; uint32_t pad; } slot[HASH_N]; uint32_t epoch;
   struct Big { uintptr_t s, e; uint16_t w, r; int16_t wchain, rchain; } big[BIG_N]; int nbig; bool big_anywhere;
   // the distinct small ranges, each on the list of the one or two 4 KiB pages it touches: what a LARGE range is checked against
   struct Small { uintptr_t s, e, page0; uint16_t w, r; int next[2]; } small[CL_BUF_CMDS * 4]; int nsmall;
   struct Page { uintptr_t key; uint32_t epoch; int head; bool big; } page[PAGE_N];       // big: some large range touches the page
   uintptr_t small_lo, small_hi;                                               // bounding box of the small ranges
 };
+static_assert(sizeof(Window::Bucket) == 64, "a bucket of four blocks is one cache line");
 static Window* g_win = nullptr;
 
 static void window_reset(Window& W) {
@@ -633,14 +637,21 @@ static void window_reset(Window& W) {
   if (++W.epoch == 0) { for (int i = 0; i < HASH_N; i++) W.slot[i].epoch = 0; for (int i = 0; i < PAGE_N; i++) W.page[i].epoch = 0; W.epoch = 1; }
 }
 static inline Window::Slot* slot_of(Window& W, uintptr_t block, bool create) {
-  uint32_t h = (uint32_t)((block * 0x9E3779B97F4A7C15ull) >> 48) & (HASH_N - 1);
-  for (int probe = 0; probe < HASH_N; probe++, h = (h + 1) & (HASH_N - 1)) {
-    Window::Slot& sl = W.slot[h];
-    if (sl.epoch != W.epoch) { if (!create) return nullptr; sl.key = block; sl.epoch = W.epoch; sl.w = sl.r = 0; sl.wchain = sl.rchain = -1; sl.wbase = sl.rbase = 0; return &sl; }
-    if (sl.key == block) return &sl;
+  const uintptr_t four = block >> 2;
+  uint32_t h = (uint32_t)((four * 0x9E3779B97F4A7C15ull) >> 48) & (HASH_N - 1);
+  for (int probe = 0; probe < HASH_N / 2; probe++, h = (h + 1) & (HASH_N - 1)) {
+    Window::Bucket& bk = W.slot[h];
+    if (bk.epoch != W.epoch) {
+      if (!create) return nullptr;
+      bk.key = four; bk.epoch = W.epoch;
+      for (int q = 0; q < 4; q++) { Window::Slot& sl = bk.sub[q]; sl.w = sl.r = 0; sl.wchain = sl.rchain = -1; sl.wbase = sl.rbase = 0; }
+      return &bk.sub[block & 3];
+    }
+    if (bk.key == four) return &bk.sub[block & 3];
   }
   return nullptr;
 }
+static inline uint16_t base16(uintptr_t start) { return (uint16_t)(start >> 2); }
 static inline Window::Page* page_of(Window& W, uintptr_t pg, bool create) {
   uint32_t h = (uint32_t)((pg * 0x9E3779B97F4A7C15ull) >> 50) & (PAGE_N - 1);
   for (int probe = 0; probe < PAGE_N; probe++, h = (h + 1) & (PAGE_N - 1)) {
@@ -681,8 +692,8 @@ static void conflicts_of(Window& W, const Extent& x, Conflict& c) {
     for (uintptr_t blk = x.s >> 8; blk <= (x.e - 1) >> 8; blk++) {
       const Window::Slot* sl = slot_of(W, blk, false);
       if (!sl) continue;
-      c.see(sl->w, sl->wchain, sl->wbase == x.s);
-      if (x.w) c.see(sl->r, sl->rchain, sl->rbase == x.s);
+      c.see(sl->w, sl->wchain, sl->wbase == base16(x.s));
+      if (x.w) c.see(sl->r, sl->rchain, sl->rbase == base16(x.s));
     }
   } else if (x.s < W.small_hi && W.small_lo < x.e) {         // a large range over memory that small ranges of this window touch
     auto meet = [&](const Window::Small& m) { if (m.s < x.e && x.s < m.e) c.see(x.w ? (m.w > m.r ? m.w : m.r) : m.w, -1, false); };
@@ -702,11 +713,11 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
       Window::Slot* sl = slot_of(W, blk, true);
       if (!sl) return false;
       if (x.w) {
-        if (level > sl->w) { sl->w = (uint16_t)level; sl->wchain = (int16_t)chain; sl->wbase = x.s; }
-        else if (level == sl->w && (sl->wchain != chain || sl->wbase != x.s)) sl->wchain = -1;       // two chains (or two alignments) at one level
+        if (level > sl->w) { sl->w = (uint16_t)level; sl->wchain = (int16_t)chain; sl->wbase = base16(x.s); }
+        else if (level == sl->w && (sl->wchain != chain || sl->wbase != base16(x.s))) sl->wchain = -1;       // two chains (or two alignments) at one level
       } else {
-        if (level > sl->r) { sl->r = (uint16_t)level; sl->rchain = (int16_t)chain; sl->rbase = x.s; }
-        else if (level == sl->r && (sl->rchain != chain || sl->rbase != x.s)) sl->rchain = -1;
+        if (level > sl->r) { sl->r = (uint16_t)level; sl->rchain = (int16_t)chain; sl->rbase = base16(x.s); }
+        else if (level == sl->r && (sl->rchain != chain || sl->rbase != base16(x.s))) sl->rchain = -1;
       }
     }
     const uintptr_t pa = x.s >> 12, pb = (x.e - 1) >> 12;
@@ -751,7 +762,7 @@ static bool note_extent(Window& W, const Extent& x, int level, int chain) {
 static inline void memcpy_host(void* d, const void* s_, size_t nbytes) { __builtin_memcpy(d, s_, nbytes); }
 namespace lh {
 static long long g_stat_slot_chains = 0, g_stat_slots = 0, g_stat_chain_ptrs = 0;
-static unsigned long long g_tsc_push = 0, g_tsc_flush = 0, g_tsc_wait = 0, g_tsc_conf = 0, g_tsc_note = 0;      // host cycles spent recording (LH_CMDLIST_VERBOSE prints them)
+static unsigned long long g_tsc_push = 0, g_tsc_flush = 0, g_tsc_wait = 0;      // host cycles spent recording (LH_CMDLIST_VERBOSE prints them)
 // Hands the recorded buffer to the device: commands in level order (recording order within a level), the first of each
 // level flagged for a barrier, each with the wavefront its elements start on.
 void rec_flush() {
@@ -1040,17 +1051,13 @@ bool rec_push(const LhCmd& c) {
     // command; what a matrix command writes, which cmd_extents lists first); cf_in: through what a matrix command reads
     Conflict cf, cf_in;
     const int cls = cmd_class(c);
-    const unsigned long long q0 = __builtin_ia32_rdtsc();
     for (int i = 0; i < k; i++) conflicts_of(W, x[i], (cls >= 2 && i > 0) ? cf_in : cf);
-    g_tsc_conf += __builtin_ia32_rdtsc() - q0;
     int lv, chain;
     const int row = cls == 4 ? c.i1 : 0;             // rank-1 updates own rows: the same buffer cut into rows of another length is another mapping
     if (cls && g_chains && cf.one_chain && W.chain_class[cf.chain] == cls && W.chain_row[cf.chain] == row && cf_in.lv < cf.lv) { lv = cf.lv; chain = cf.chain; }      // joins the chain it follows
     else { lv = (cf.lv > cf_in.lv ? cf.lv : cf_in.lv) + 1; chain = -1; if (cls) { chain = W.nchains++; W.chain_class[chain] = (uint8_t)cls; W.chain_row[chain] = row; } }
     bool ok = true;
-    const unsigned long long q1 = __builtin_ia32_rdtsc();
     for (int i = 0; i < k && ok; i++) ok = note_extent(W, x[i], lv, (cls >= 2 && i > 0) ? -1 : chain);
-    g_tsc_note += __builtin_ia32_rdtsc() - q1;
     if (!ok) { rec_flush(); if (failed()) return false; continue; }       // a table is full: start a new buffer (which begins with a barrier)
     W.cmd[W.n] = c; W.level[W.n] = (uint16_t)lv; W.chain[W.n] = (int16_t)chain; W.n++;
     W.entries += copies;
@@ -1089,7 +1096,7 @@ void lh_cmdlist_end(void) {
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld commands in %lld levels, %lld launches\n", (long long)g_ring.recorded, (long long)g_ring.levels, (long long)g_ring.launches);
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %d operand slots per workgroup\n", g_ring.nslot);
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld chains run as programs, %lld operand slots, %lld commands in them\n", g_stat_slot_chains, g_stat_slots, g_stat_chain_ptrs);
-  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list host cycles: push %.1f M (flush inside %.1f M, of which waiting for a free buffer %.1f M), conflicts %.1f M, notes %.1f M\n", g_tsc_push * 1e-6, g_tsc_flush * 1e-6, g_tsc_wait * 1e-6, g_tsc_conf * 1e-6, g_tsc_note * 1e-6);
+  if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list host cycles: push %.1f M (flush inside %.1f M, of which waiting for a free buffer %.1f M)\n", g_tsc_push * 1e-6, g_tsc_flush * 1e-6, g_tsc_wait * 1e-6);
 }
 void lh_cmdlist_stats(int64_t* recorded, int64_t* launches) {
   if (recorded) *recorded = g_ring.recorded;
