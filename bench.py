@@ -176,7 +176,34 @@ def run_gpu(args):
         tr2, _, _ = make_trainer(args, args.batch)
         write_c_program_inputs(c_dir, tr2)
         tr2.close()
+    emitted = None
+    if args.c_host and args.workload != "treelstm":
+        # the step written out as straight-line C (what the reference's LMS back end emits), compiled, and timed after this process
+        # has released the device: the library without the Python mirror between two calls
+        import tempfile
+        from lantern_amd import emit_c
+        e_dir = tempfile.mkdtemp(prefix="lantern_emitted_")
+        text, data, tr3, _ = emit_c.record(lambda: make_trainer(args, args.batch)[0], be, desc, be.heap_bytes,
+                                           frame=(["lh_set_deterministic(1);"] if args.deterministic else []) + (["lh_set_side_stream(0);"] if args.no_side_stream else []))
+        open(os.path.join(e_dir, "step.c"), "w").write(text)
+        open(os.path.join(e_dir, "data.bin"), "wb").write(data)
+        emitted = (e_dir, text.count("\n"))
     be.cleanup()
+    if emitted is not None:
+        import subprocess, shutil
+        e_dir, lines = emitted
+        exe = os.path.join(e_dir, "step")
+        cc = subprocess.run(emit_c.compile_line(os.path.dirname(os.path.abspath(__file__)), os.path.join(e_dir, "step.c"), exe), capture_output=True, text=True)
+        if cc.returncode != 0:
+            sys.exit("bench.py: the emitted C program does not compile: " + cc.stderr[-2000:])
+        r = subprocess.run([exe, os.path.join(e_dir, "data.bin"), str(args.steps), str(args.warmup)], capture_output=True, text=True, timeout=900)
+        if r.returncode != 0 or not r.stdout.startswith("ms_per_step"):
+            sys.exit("bench.py: the emitted C program failed: " + r.stdout + r.stderr)
+        f = r.stdout.split()
+        emitted = {"ms_per_step": float(f[1]), "value": round(per_step / (float(f[1]) / 1000.0), 2), "first_loss": float(f[5]), "last_loss": float(f[7]), "lines_of_c": lines,
+                   "note": "the same step written out by lantern_amd/emit_c.py as a plain-C host program (one library call per operator, the loss read back with a wait every step), "
+                           "compiled with gcc and run on its own after this process released the device"}
+        shutil.rmtree(e_dir, ignore_errors=True)
     if c_dir is not None:
         import subprocess
         r = subprocess.run([TREE_C_PROGRAM, os.path.join(c_dir, "params.bin"), os.path.join(c_dir, "trees.txt"), os.path.join(c_dir, "out.bin"),
@@ -190,7 +217,7 @@ def run_gpu(args):
         if not args.keep_c_inputs:
             import shutil
             shutil.rmtree(c_dir, ignore_errors=True)
-    return {"c_host": c_host, "streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
+    return {"emitted": emitted, "c_host": c_host, "streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
             "per_step": per_step, "desc": desc}
 
 
@@ -243,6 +270,8 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--cpu-steps", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--c-host", action="store_true", help="also write the step out as a plain-C host program (lantern_amd/emit_c.py), compile and time it: "
+                    "the library without the Python mirror between two calls (fixed-shape workloads; needs gcc)")
     ap.add_argument("--keep-c-inputs", default=None, help="treelstm: write the C host program's input files (params.bin, trees.txt) into this directory and leave them there")
     ap.add_argument("--tree-file", default=None, help="treelstm: trees in the reference's array_tree.txt format instead of random ones (tests/golden/array_tree_first24.txt)")
     ap.add_argument("--no-side-stream", action="store_true", help="filter gradients in line on the main stream (kernel profiles: no two kernels overlap)")
@@ -275,7 +304,7 @@ def main():
         t = timed["cmdlist"][0] / 1000.0
         achieved = work.get("gemv_bytes", 0.0) / t / 1e9 if t > 0 else 0.0
         roof = {"bound": "hbm", "kernel": "k_cmdlist (%d interpreter launches/step running the gemv / rank-1 update / element-wise commands level by level "
-                                          "over 16 workgroups; bound by memory round trips and the barrier per level at these sizes; timed under the Python mirror)" % timed["cmdlist"][1],
+                                          "over the library's workgroups; bound by memory round trips and the barrier per level at these sizes; timed under the Python mirror)" % timed["cmdlist"][1],
                 "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": None,
                 "bytes_per_step": work.get("gemv_bytes", 0.0), "ms_per_step": round(timed["cmdlist"][0], 3)}
     else:
@@ -328,6 +357,8 @@ def main():
     if python_host is not None:
         out["config"]["host"] = "plain-C host program over the C-ABI (tests/host_c/treelstm_step.c): the reference's generated-code shape, command list on"
         out["python_mirror_host"] = python_host
+    if g.get("emitted"):
+        out["emitted_c_program"] = g["emitted"]
     if g["resident_sec"] is not None:
         out["resident_input"] = {"value": round(g["per_step"] * args.steps / g["resident_sec"], 2), "ms_per_step": round(1000.0 * g["resident_sec"] / args.steps, 3),
                                  "note": "the same steps with the batch resident on the device: no upload, no loss read-back"}

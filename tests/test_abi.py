@@ -187,3 +187,40 @@ def test_c_treelstm_command_list_gives_the_same_bits_on_any_number_of_workgroups
     assert results[0].size > len(trees) and np.isfinite(results[0].view(np.float32)).all()
     for r in results[1:]:
         assert np.array_equal(results[0], r)
+
+
+@pytest.mark.gpu
+def test_emitted_c_program_repeats_the_mirrors_training_steps(tmp_path, on_hip):
+    """lantern_amd/emit_c.py writes a program of the mirror out as straight-line C over the C-ABI (what the reference's LMS back end
+    emits: one library call per operator, shapes as literals, the step in a loop).  A small ResNet (bottleneck blocks, batch norm,
+    pooling, the classifier, momentum SGD: 32x32 images, batch 8) is recorded, compiled with gcc and run for five steps in a process
+    of its own; in deterministic mode its losses are, bit for bit, the losses of the mirror's own next five steps."""
+    import shutil
+    import numpy as np
+    from lantern_amd import emit_c
+    from lantern_amd.apps.resnet50 import ResNet50, Trainer
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    be = on_hip
+    be.setDeterministic(True)
+    try:
+        make = lambda: Trainer(ResNet50(num_classes=10, layers=(1, 1, 1, 1), imagenet_stem=False), 8, 32, 10, lr=0.01, momentum=0.9)
+        text, data, trainer, (first, second) = emit_c.record(make, be, "a small ResNet, batch 8", 1 << 30, frame=["lh_set_deterministic(1);"])
+        want = [second]
+        for _ in range(4):
+            want.append(float(trainer.step().toCPU()[0])); trainer.end_step()
+    finally:
+        be.setDeterministic(False)
+    assert text.count("lh_conv2d_fwd") >= 10 and "lh_multi_momentum" in text or "lh_momentum" in text
+    (tmp_path / "step.c").write_text(text)
+    (tmp_path / "data.bin").write_bytes(data)
+    exe = str(tmp_path / "step")
+    cc = subprocess.run(emit_c.compile_line(ROOT, str(tmp_path / "step.c"), exe), capture_output=True, text=True)
+    assert cc.returncode == 0 and "warning" not in cc.stderr, cc.stderr[-3000:]
+    deps = subprocess.run(["ldd", exe], capture_output=True, text=True).stdout
+    assert "liblantern_hip.so" in deps and "python" not in deps and "torch" not in deps, deps
+    out = subprocess.run([exe, str(tmp_path / "data.bin"), "5", "0", str(tmp_path / "losses.bin")], capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and out.stdout.startswith("ms_per_step"), out.stdout + out.stderr
+    got = np.fromfile(tmp_path / "losses.bin", np.float32)
+    assert got.size == 5 and first != second
+    assert np.array_equal(got, np.array(want, np.float32)), (got, want)
