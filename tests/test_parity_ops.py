@@ -909,10 +909,9 @@ def test_conv_with_batchnorm_statistics(pair, case, relu):
 
 
 # ---- command list: small operators recorded and run in order by one workgroup --------------------------
-def _small_op_program(be, rng_seed=50):
+def _small_op_program(be, rng_seed=50, n=150, m=37):
     """A chain of dependent small operators covering every recordable entry point; returns host copies of all results."""
     rng = np.random.RandomState(rng_seed)
-    n, m = 150, 37
     up = lambda a: be.fromHost(np.ascontiguousarray(a, np.float32))
     W = up(rng.randn(m, n) * 0.1); x = up(rng.randn(n)); bias = up(rng.randn(m)); gy = up(rng.randn(m))
     lib = be.lib
@@ -952,19 +951,22 @@ def _small_op_program(be, rng_seed=50):
     return [be.toHost(buf, cnt).copy() for buf, cnt in outs]
 
 
-def test_command_list_matches_one_launch_per_operator(on_hip):
+@pytest.mark.parametrize("n,m", [(150, 37), (1000, 64), (64, 300), (4100, 16)], ids=["150x37", "1000x64", "64x300", "4100x16"])
+def test_command_list_matches_one_launch_per_operator(on_hip, n, m):
     be = on_hip
-    direct = _small_op_program(be)
+    direct = _small_op_program(be, n=n, m=m)
     rec0, launches0 = be.cmdlistStats()
     be.batchSmallOps(True)
     try:
-        listed = _small_op_program(be)
+        listed = _small_op_program(be, n=n, m=m)
     finally:
         be.batchSmallOps(False)
     rec, launches = be.cmdlistStats()
     assert rec - rec0 >= 25 and 0 < launches - launches0 <= 30, (rec - rec0, launches - launches0)
+    # the products sum in another order than the stand-alone kernels: 2e-6 over 150 terms; over 1000 and more the differences reach
+    # 1e-6 of a product, and the gradients and the Adagrad step behind them (differences of near-equal terms) carry that to 1e-5
     for i, (a, b_) in enumerate(zip(listed, direct)):
-        assert_close(a, b_, rtol=2e-6, what="result %d" % i)
+        assert_close(a, b_, rtol=2e-6 if n <= 150 else 1e-4, what="result %d" % i)
 
 
 def test_command_list_keeps_program_order_around_other_kernels_and_wraps_its_buffers(on_hip):
@@ -995,15 +997,16 @@ def test_command_list_keeps_program_order_around_other_kernels_and_wraps_its_buf
     _lib.check()
 
 
-def test_command_list_reordering_keeps_every_dependence(on_hip):
+@pytest.mark.parametrize("n_vec,vlen,m", [(12, 150, 24), (10, 1000, 37), (8, 4500, 8), (12, 67, 67)],
+                         ids=["150x24", "1000x37", "4500x8_shared_by_all_workgroups", "67x67"])
+def test_command_list_reordering_keeps_every_dependence(on_hip, n_vec, vlen, m):
     """The command list runs independent commands of a buffer side by side and dependent ones in order.  A random program of
     several hundred small operations over a few buffers and their sub-ranges (reads after writes, writes after reads, writes
     after writes; vectors inside a matrix another command updates as a whole; a scalar one command leaves for the next) must
     give the bits of the same program issued one launch per operator, whose order is the program's."""
     be = on_hip
     lib = be.lib
-    rng = np.random.RandomState(77)
-    n_vec, vlen, m = 12, 150, 24
+    sub = min(64, vlen // 3)                    # length of the sub-range operations, which start a third into a vector
 
     def program():
         mark = be.getMallocAddr()
@@ -1027,7 +1030,7 @@ def test_command_list_reordering_keeps_every_dependence(on_hip):
                 lib.lh_dot_vv(vecs[a].ptr, vecs[b_].ptr, scal.ptr, vlen)
                 lib.lh_scalar_op(B.MUL, scal.ptr, scal.ptr, 1e-3, 1)
                 lib.lh_axpy_dev(vecs[c].ptr, scal.ptr, vecs[a].ptr, vlen) if a != c else None
-            else: lib.lh_geam(vecs[a].ptr, 1.0, vecs[b_].ptr + 4 * 50, -0.5, vecs[a].ptr, 64)                        # a[:64] -= b[50:114] / 2
+            else: lib.lh_geam(vecs[a].ptr, 1.0, vecs[b_].ptr + 4 * (vlen // 3), -0.5, vecs[a].ptr, sub)              # a[:sub] -= b[third : third + sub] / 2
             # keep the values bounded: the matrix is halved after an update, a vector that was added to goes through tanh (in place)
             if k == 3 and a != b_: lib.lh_scalar_op(B.MUL, mat.ptr, mat.ptr, 0.5, m * vlen)
             if k in (2, 8): lib.lh_unary(B.TANH, vecs[a].ptr, vecs[a].ptr, vlen, -1.0, 1.0)
@@ -1046,10 +1049,10 @@ def test_command_list_reordering_keeps_every_dependence(on_hip):
         be.batchSmallOps(False)
     assert all(np.isfinite(a).all() for a in direct)
     # the matrix commands sum in another order than the stand-alone kernels (whose transposed product combines blocks with atomic
-    # adds, so its own result moves in the last bits from run to run), and 600 dependent operations carry that along: 1e-4, the
-    # tolerance for sums whose order is free; a command that ran before what it depends on is off by far more
+    # adds, so its own result moves in the last bits from run to run), and 600 dependent operations carry that along and spread it
+    # (differences of 1e-5 to 5e-5 of a value are seen): 1e-3; a command that ran before what it depends on is off by 1e-2 and more
     for i, (a, b_) in enumerate(zip(listed, direct)):
-        assert_close(a, b_, rtol=1e-4, what="buffer %d" % i)
+        assert_close(a, b_, rtol=1e-3, what="buffer %d" % i)
 
 
 def test_command_list_long_element_wise_chains_keep_their_operands_in_lds(on_hip):
