@@ -166,7 +166,10 @@ def test_c_treelstm_program_tracks_the_oracle(tmp_path, cpu_backend, cmdlist):
 @pytest.mark.gpu
 def test_c_treelstm_command_list_gives_the_same_bits_on_any_number_of_workgroups(tmp_path, cpu_backend):
     """No command of the list combines partial results with atomic adds and every sum has a fixed order, so eight training steps
-    of the C program end in the same bits whether 1, 5 or 32 workgroups share the commands (LH_CMDLIST_GROUPS), and twice over."""
+    of the C program end in the same bits whether 1, 5 or 32 workgroups share the commands (LH_CMDLIST_GROUPS), twice over, and
+    also when element-wise chains run command by command instead of as programs over LDS (LH_CMDLIST_SLOTS=0) or when nothing is
+    chained at all and every dependent command opens a level (LH_CMDLIST_CHAINS=0): how the commands are scheduled is not
+    allowed to show in the result."""
     import numpy as np
     import lantern_amd as la
     from lantern_amd.apps.treelstm import Trainer, read_trees
@@ -178,10 +181,10 @@ def test_c_treelstm_command_list_gives_the_same_bits_on_any_number_of_workgroups
     write_treelstm_inputs(tmp_path, tr, tr.trees)
     tr.close(); cpu_backend.resetMallocAddr(mark)
     results = []
-    for groups in ("1", "5", "32", "32"):
+    for extra in ({"LH_CMDLIST_GROUPS": "1"}, {"LH_CMDLIST_GROUPS": "5"}, {}, {}, {"LH_CMDLIST_SLOTS": "0"}, {"LH_CMDLIST_CHAINS": "0"}):
         out_file = tmp_path / ("out_%d.bin" % len(results))
         out = subprocess.run([exe, str(tmp_path / "params.bin"), str(tmp_path / "trees.txt"), str(out_file), str(len(trees)), "0", "1"],
-                             capture_output=True, text=True, timeout=110, env=dict(os.environ, LH_CMDLIST_GROUPS=groups))
+                             capture_output=True, text=True, timeout=110, env=dict(os.environ, **extra))
         assert out.returncode == 0 and out.stdout.startswith("trees_per_s"), out.stdout + out.stderr
         results.append(np.fromfile(out_file, np.uint32))
     assert results[0].size > len(trees) and np.isfinite(results[0].view(np.float32)).all()
