@@ -144,8 +144,12 @@ void lh_graph_destroy(int graph);
  * them), a barrier over the workgroups between levels.  The barrier's wait is bounded: if a workgroup never arrives the
  * kernel ends, and the next call that touches the command list reports it.  Results equal those of the stand-alone kernels
  * up to summation order in the reductions; no command uses atomic adds and every sum has a fixed order, so two runs give the
- * same bits whatever the number of workgroups.  LH_CMDLIST_TRACE=<launch> prints, for that launch and the next, how long each
- * level took and what it held.  Generated code calls lh_cmdlist_begin() once after lh_setup(). */
+ * same bits whatever the number of workgroups.  Element-wise commands that depend only on each other lane by lane, and matrix
+ * commands that write the same rows, share a level (chains; LH_CMDLIST_CHAINS=0 turns them off); chains of six and more element-wise
+ * commands run as one entry over operands held in LDS (LH_CMDLIST_SLOTS=0 turns that off, LH_CMDLIST_NSLOT limits the slots).
+ * None of these switches changes a result.  LH_CMDLIST_TRACE=<launch> prints, for that launch and the next, how long each level
+ * took and what it held; LH_CMDLIST_VERBOSE=1 prints totals at lh_cmdlist_end.  Generated code calls lh_cmdlist_begin() once after
+ * lh_setup(). */
 void lh_cmdlist_begin(void);
 void lh_cmdlist_end(void);
 /* Commands recorded and interpreter launches since lh_setup (either pointer may be NULL). */
