@@ -99,9 +99,17 @@ struct LoadConvFwdTapB {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
   static constexpr bool SPLIT = true;
+  static constexpr bool STEP = true;
   const float* base; uint32_t nbytes;
   int C, H, W, sH, sW, pH, pW, HW;
   FastDiv dPQ, dQ, dC, dS;
+  // inside a tap the next slab is the same pixels, bk channel planes further on
+  __device__ __forceinline__ uint32_t step_bytes(int bk) const { return (uint32_t)(bk * HW) * 4u; }
+  __device__ __forceinline__ int run_slabs(int k, int bk) const {
+    uint32_t tap, ch;
+    dC.divmod(k, tap, ch);
+    return (C % bk) ? 1 : (C - (int)ch) / bk;
+  }
   struct State { int pix, h0, w0; bool valid; };
   __device__ __forceinline__ void init(State& s, int j, int ncols) const {
     s.valid = j < ncols;
@@ -131,9 +139,16 @@ struct LoadConvBwdDataTapB {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
   static constexpr bool SPLIT = true;
+  static constexpr bool STEP = true;
   const float* base; uint32_t nbytes;
   int K, P, Q, PQ, offH, offW;
   FastDiv dPIX, dWc, dK, dSc;       // class-grid pixels per sample, class-grid width, K, taps per row
+  __device__ __forceinline__ uint32_t step_bytes(int bk) const { return (uint32_t)(bk * PQ) * 4u; }
+  __device__ __forceinline__ int run_slabs(int k, int bk) const {
+    uint32_t tap, ko;
+    dK.divmod(k, tap, ko);
+    return (K % bk) ? 1 : (K - (int)ko) / bk;
+  }
   struct State { int nbase, hq, wq; bool valid; };
   __device__ __forceinline__ void init(State& s, int j, int ncols) const {
     s.valid = j < ncols;
@@ -232,6 +247,14 @@ struct EpiConvOut {
     c.off = (int)n * chan * PIX + (aH + eH * (int)u) * W + aW + eW * (int)v;
     return c;
   }
+  // lean stores: element (i, j) at lane_bytes(col(j)) + i * row_bytes() from `out` (the tensor is below 2 GiB); not with a bias
+  static constexpr bool LEAN = true;
+  __device__ __forceinline__ bool lean_ok(int M) const { return bias == nullptr && (M & 7) == 0; }
+  __device__ __forceinline__ float* lean_base() const { return out; }
+  __device__ __forceinline__ uint32_t lane_bytes(const Col& c) const { return (uint32_t)c.off * 4u; }
+  __device__ __forceinline__ uint32_t row_bytes() const { return (uint32_t)PIX * 4u; }
+  __device__ __forceinline__ uint32_t cell_row_bytes() const { return (uint32_t)W * 4u; }
+  __device__ __forceinline__ int lean_mode() const { return zfill2 ? 2 : (beta == 0.f ? 0 : 1); }
   // part: 0 = complete sum; 1 = first partial, 2 = later partial (atomic adds onto a prepared output)
   __device__ __forceinline__ void store(const Col& c, int i, int M, float v, int part) const {
     if (!c.valid || i >= M) return;

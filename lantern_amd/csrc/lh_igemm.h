@@ -64,7 +64,10 @@ struct LoadPlainK {
   static constexpr bool ALONG_K = true;
   static constexpr bool VEC4 = VEC;
   static constexpr bool SPLIT = false;
+  static constexpr bool STEP = true;
   const float* base; uint32_t nbytes; int ld;
+  __device__ __forceinline__ uint32_t step_bytes(int bk) const { return (uint32_t)bk * 4u; }
+  __device__ __forceinline__ int run_slabs(int, int) const { return 0x3fffffff; }
   struct State { uint32_t row; bool valid; };
   __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.row = (uint32_t)(s.valid ? col : 0) * (uint32_t)ld * 4u; }
   // byte offset of element k + e of the group starting at k (VEC: e == 0 stands for all four)
@@ -77,7 +80,10 @@ struct LoadPlainT {
   static constexpr bool ALONG_K = false;
   static constexpr bool VEC4 = false;
   static constexpr bool SPLIT = false;
+  static constexpr bool STEP = true;
   const float* base; uint32_t nbytes; int ld;
+  __device__ __forceinline__ uint32_t step_bytes(int bk) const { return (uint32_t)bk * (uint32_t)ld * 4u; }
+  __device__ __forceinline__ int run_slabs(int, int) const { return 0x3fffffff; }
   struct State { uint32_t col; bool valid; };
   __device__ __forceinline__ void init(State& s, int col, int ncols) const { s.valid = col < ncols; s.col = (uint32_t)(s.valid ? col : 0) * 4u; }
   __device__ __forceinline__ uint32_t off1(const State& s, int k, int kend, int e) const {
@@ -85,32 +91,45 @@ struct LoadPlainT {
   }
 };
 
+// A loader with STEP == true can also be advanced without recomputing anything per lane: inside a run of run_slabs(k, BK)
+// consecutive k-slabs (counting the one that starts at k) the per-lane offsets of a slab are those of the slab before it
+// plus the wave-uniform step_bytes(BK), which the kernel keeps in the scalar-offset operand of the loads.  (The range
+// check of a raw buffer load looks at the per-lane offset only, so LH_OOB lanes stay out of range under any scalar offset.)
+template <class L, class = void> struct LhCanStep { static constexpr bool value = false; };
+template <class L> struct LhCanStep<L, typename std::enable_if<L::STEP>::type> { static constexpr bool value = true; };
+
 // Offsets of one group of four k (one offset when the loader is VEC4).  A SPLIT loader gives one
 // per-lane byte offset for the group (o[0], LH_OOB when the group is out of range for this lane)
 // plus four wave-uniform byte offsets s[i] that go into the scalar-offset operand of the load.
-template <class L> struct LhOff { uint32_t o[4]; uint32_t s[4]; };
+template <class L> struct LhOff { uint32_t o[4]; };
+struct LhScal { uint32_t s[4]; };      // the wave-uniform parts of a SPLIT loader's group, kept apart from the per-lane ones so that they stay in scalar registers
 template <class L>
-__device__ __forceinline__ float4 lh_fetch4(__amdgpu_buffer_rsrc_t rsrc, const LhOff<L>& f) {
+// `xs`: wave-uniform bytes on top of every offset of the group (the slabs stepped over since the offsets were computed)
+__device__ __forceinline__ float4 lh_fetch4(__amdgpu_buffer_rsrc_t rsrc, const LhOff<L>& f, const LhScal& u, int xs = 0) {
   if (L::SPLIT) {
     float4 r;
-    r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[0], 0));
-    r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[1], 0));
-    r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[2], 0));
-    r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)f.s[3], 0));
+    r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[0] + xs, 0));
+    r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[1] + xs, 0));
+    r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[2] + xs, 0));
+    r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[3] + xs, 0));
     return r;
   }
   if (L::VEC4) {
     typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-    u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)f.o[0], 0, 0);
+    u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)f.o[0], xs, 0);
     return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
   }
   float4 r;
-  r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], 0, 0));
-  r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[1], 0, 0));
-  r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[2], 0, 0));
-  r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[3], 0, 0));
+  r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], xs, 0));
+  r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[1], xs, 0));
+  r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[2], xs, 0));
+  r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[3], xs, 0));
   return r;
 }
+
+// Does an epilogue offer lean stores (see the store section of igemm_block)?
+template <class E, class = void> struct LhHasLean { static constexpr bool value = false; };
+template <class E> struct LhHasLean<E, typename std::enable_if<E::LEAN>::type> { static constexpr bool value = true; };
 
 // ---- epilogue for row-major C ------------------------------------------------------------------
 // mode 0: C = alpha*acc + beta*C ; mode 1: atomicAdd(C, alpha*acc) (split-K)
@@ -132,16 +151,9 @@ struct EpiRowMajor {
   }
 };
 
-// Sum over the 32 lanes of each half of a wavefront (all 32 lanes get the total): DPP adds inside a
-// row of 16, one swizzle across the two rows.
-__device__ __forceinline__ float lh_half_sum32(float v) {
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
-  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // row_mirror
-  v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));                      // lane ^ 16
-  return v;
-}
+// bytes of LDS of one tile configuration: two stages of both operands, k-packed and padded
+template <int BM, int BN, int BK>
+constexpr size_t igemm_smem_bytes() { return (size_t)2 * (BK / 4) * ((BM + 8 / (BK / 4)) + (BN + 8 / (BK / 4))) * sizeof(float4); }
 
 // ---- the kernel ------------------------------------------------------------------------------------
 // The work of one block; `block` is its index within the launch (or within its group of a grouped launch).
@@ -167,6 +179,10 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   // is completed with atomic adds.
   long long u = 0, u_end = 1;
   if (SK) { u = gs.units * logical / gs.total; u_end = gs.units * (logical + 1) / gs.total; }
+  // STEPPED: both loaders can be advanced by a wave-uniform step, so inside a run of slabs the offsets of the next slab
+  // cost two scalar additions instead of a decode per element; a slab past the end of the reduction is switched off by a
+  // buffer descriptor of zero bytes (every lane out of range, the loads return 0 without touching memory).
+  constexpr bool STEPPED = LhCanStep<AL>::value && LhCanStep<BL>::value;
   const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc((void*)al.base, 0, (int)al.nbytes, LH_RSRC_FLAGS);
   const __amdgpu_buffer_rsrc_t rsB = __builtin_amdgcn_make_buffer_rsrc((void*)bl.base, 0, (int)bl.nbytes, LH_RSRC_FLAGS);
   const int t = threadIdx.x;
@@ -226,23 +242,55 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   float4 ra0[GA], rb0[GB], ra1[GA], rb1[GB];
   LhOff<AL> oa[GA];
   LhOff<BL> ob[GB];
+  LhScal ua[GA], ub[GB];
   // e-th offset of the slab starting at k0
   auto elem = [&](int e, int k0) {
     if (e < GA * EA) {
       const int g = e / EA, i = e % EA, k = k0 + 4 * a_kq[g];
-      if constexpr (AL::SPLIT) { if (i == 0) oa[g].o[0] = al.voff(sa[g], k, kend); oa[g].s[i] = al.soff(k, i); }
+      if constexpr (AL::SPLIT) { if (i == 0) oa[g].o[0] = al.voff(sa[g], k, kend); ua[g].s[i] = al.soff(k, i); }
       else oa[g].o[i] = al.off1(sa[g], k, kend, i);
     } else {
       const int f = e - GA * EA, g = f / EB, i = f % EB, k = k0 + 4 * b_kq[g];
-      if constexpr (BL::SPLIT) { if (i == 0) ob[g].o[0] = bl.voff(sb[g], k, kend); ob[g].s[i] = bl.soff(k, i); }
+      if constexpr (BL::SPLIT) { if (i == 0) ob[g].o[0] = bl.voff(sb[g], k, kend); ub[g].s[i] = bl.soff(k, i); }
       else ob[g].o[i] = bl.off1(sb[g], k, kend, i);
     }
   };
+  // State of the slab the next fetch loads (STEPPED): bytes stepped since (oa, ob) were computed; how many more slabs can
+  // be reached by stepping (whole slabs inside the reduction and inside the loaders' runs); the byte range of the buffer
+  // descriptors (0 switches the loads of a slab past the end of the reduction off).
+  int xsA = 0, xsB = 0, steps = 0, nrecA = (int)al.nbytes, nrecB = (int)bl.nbytes;
   auto fetch = [&](float4 (&ra)[GA], float4 (&rb)[GB]) {
+    if constexpr (STEPPED) {
+      const __amdgpu_buffer_rsrc_t ra_ = __builtin_amdgcn_make_buffer_rsrc((void*)al.base, 0, nrecA, LH_RSRC_FLAGS);
+      const __amdgpu_buffer_rsrc_t rb_ = __builtin_amdgcn_make_buffer_rsrc((void*)bl.base, 0, nrecB, LH_RSRC_FLAGS);
 #pragma unroll
-    for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(rsA, oa[g]);
+      for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(ra_, oa[g], ua[g], xsA);
 #pragma unroll
-    for (int g = 0; g < GB; g++) rb[g] = lh_fetch4<BL>(rsB, ob[g]);
+      for (int g = 0; g < GB; g++) rb[g] = lh_fetch4<BL>(rb_, ob[g], ub[g], xsB);
+    } else {
+#pragma unroll
+      for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(rsA, oa[g], ua[g]);
+#pragma unroll
+      for (int g = 0; g < GB; g++) rb[g] = lh_fetch4<BL>(rsB, ob[g], ub[g]);
+    }
+  };
+  // all offsets of the slab at kn from scratch
+  auto decode = [&](int kn) {
+    if constexpr (STEPPED) {
+      if (kn >= kend) { nrecA = 0; nrecB = 0; steps = 0; return; }
+#pragma unroll
+      for (int e = 0; e < NEL; e++) elem(e, kn);
+      xsA = 0; xsB = 0;
+      const int whole = (kend - kn) / BK;                       // whole slabs from kn on
+      steps = min(min(al.run_slabs(kn, BK), bl.run_slabs(kn, BK)), whole) - 1;
+    }
+  };
+  // (oa, ob, ...) describe the slab at kn - BK and are made to describe the slab at kn
+  auto advance = [&](int kn) {
+    if constexpr (STEPPED) {
+      if (__builtin_expect(steps > 0, 1)) { steps -= 1; xsA += (int)al.step_bytes(BK); xsB += (int)bl.step_bytes(BK); }
+      else decode(kn);
+    }
   };
   auto stash = [&](const float4 (&ra)[GA], const float4 (&rb)[GB], int stage) {
     const int o = stage * KQ;
@@ -259,14 +307,23 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   //   computed in small pieces placed between the MFMAs, so they issue while the matrix pipe is
   //   busy.  A global load therefore has a whole iteration plus the MFMA time of the next one to
   //   arrive.  Slabs past kend produce LH_OOB offsets (loads return 0) and LDS stages never read.
+  if constexpr (STEPPED) {
+    nrecA = (int)al.nbytes; nrecB = (int)bl.nbytes;
+    decode(kbeg);
+    fetch(ra0, rb0);
+    advance(kbeg + BK);
+    fetch(ra1, rb1);
+    advance(kbeg + 2 * BK);
+  } else {
 #pragma unroll
-  for (int e = 0; e < NEL; e++) elem(e, kbeg);
-  fetch(ra0, rb0);
+    for (int e = 0; e < NEL; e++) elem(e, kbeg);
+    fetch(ra0, rb0);
 #pragma unroll
-  for (int e = 0; e < NEL; e++) elem(e, kbeg + BK);
-  fetch(ra1, rb1);
+    for (int e = 0; e < NEL; e++) elem(e, kbeg + BK);
+    fetch(ra1, rb1);
 #pragma unroll
-  for (int e = 0; e < NEL; e++) elem(e, kbeg + 2 * BK);
+    for (int e = 0; e < NEL; e++) elem(e, kbeg + 2 * BK);
+  }
   stash(ra0, rb0, 0);
   __syncthreads();
 
@@ -303,6 +360,14 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
         const float bv = c == 0 ? b[cur][ni].x : c == 1 ? b[cur][ni].y : c == 2 ? b[cur][ni].z : b[cur][ni].w;
         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[mi][ni], 0, 0, 0);
         const int gm = pair * NM_PAIR + m;
+        if constexpr (STEPPED) {
+          if (gm == 1) {
+            __builtin_amdgcn_sched_barrier(0);
+            advance(k3);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          continue;
+        }
         const int e0 = (gm * NEL) / NM, e1 = ((gm + 1) * NEL) / NM;
         if (e1 > e0) {
           __builtin_amdgcn_sched_barrier(0);
@@ -331,25 +396,114 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   for (int ni = 0; ni < NI; ni++) cs[ni] = ep.col(n0 + wn * TN + ni * 32 + l32, gs.N);
   bool want_stats = false;
   if constexpr (EP::STATS && !SK) want_stats = ep.partial != nullptr;
+  // Lean stores (epilogues that offer them, complete sums only): the element of row i and column j lies at
+  // lane_bytes(j) + i * row_bytes(), so a store is one buffer instruction whose per-lane offset is fixed for the tile
+  // (LH_OOB for a column past the edge: the store is dropped) and whose row goes into the scalar offset; the two halves of
+  // a wavefront hold rows four apart, which the per-lane offset carries, and with M a multiple of 8 both are inside
+  // the matrix or both outside.  No address arithmetic per element is left in the vector unit.
+  bool lean = false;
+  if constexpr (LhHasLean<EP>::value) lean = part == 0 && ep.lean_ok(gs.M);
+  if constexpr (LhHasLean<EP>::value) {
+    if (lean) {
+      const __amdgpu_buffer_rsrc_t rsO = __builtin_amdgcn_make_buffer_rsrc((void*)ep.lean_base(), 0, (int)0x80000000u, LH_RSRC_FLAGS);
+      const uint32_t rb = ep.row_bytes();
+      uint32_t vo[NI];
 #pragma unroll
-  for (int mi = 0; mi < MI; mi++) {
-    const int ib = m0 + wm * TM + mi * 32 + 4 * half;
+      for (int ni = 0; ni < NI; ni++) vo[ni] = cs[ni].valid ? ep.lane_bytes(cs[ni]) + (uint32_t)(4 * half) * rb : LH_OOB;
+      const int mode = ep.lean_mode();             // 0: overwrite, 1: beta * old + value, 2: value and the three zeros of its 2 x 2 cell
+      auto pass = [&](auto MODE) {
+        constexpr int MD = decltype(MODE)::value;
 #pragma unroll
-    for (int v = 0; v < 16; v++) {
-      const int row = ib + 8 * (v / 4) + (v % 4);
-      float s1 = 0.f, s2 = 0.f;
+        for (int mi = 0; mi < MI; mi++) {
+          const int r0 = m0 + wm * TM + mi * 32;
+          // mode 1: all old values of the block are requested before the first of them is used (a store cannot be
+          // moved across a load by the compiler, so element by element every load would wait for a round trip of its own)
+          float old[MD == 1 ? 16 : 1][NI];
+          if constexpr (MD == 1) {
 #pragma unroll
-      for (int ni = 0; ni < NI; ni++) {
-        const float val = acc[mi][ni][v];
-        ep.store(cs[ni], row, gs.M, val, part);
-        if constexpr (EP::STATS && !SK) { const float x = cs[ni].valid ? val : 0.f; s1 += x; s2 = fmaf(x, x, s2); }
-      }
-      if constexpr (EP::STATS && !SK) {
-        if (want_stats) {
-          // sums of the accumulators: the host uses this path only for launches without a bias
-          s1 = lh_half_sum32(s1); s2 = lh_half_sum32(s2);
-          if (l32 == 0 && row < gs.M) { float2* p = reinterpret_cast<float2*>(ep.partial) + (size_t)row * ep.slotsTotal + (ep.slotBase + tn * 2 + wn); *p = make_float2(s1, s2); }
+            for (int v = 0; v < 16; v++) {
+              const int so = (int)((uint32_t)(r0 + 8 * (v / 4) + (v % 4)) * rb);
+              const bool in = r0 + 8 * (v / 4) < gs.M;
+#pragma unroll
+              for (int ni = 0; ni < NI; ni++)
+                old[v][ni] = in ? __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsO, (int)vo[ni], so, 0)) : 0.f;
+            }
+          }
+#pragma unroll
+          for (int v = 0; v < 16; v++) {
+            const int row = r0 + 8 * (v / 4) + (v % 4);        // of the lower half; the upper half is four rows further on
+            if (r0 + 8 * (v / 4) >= gs.M) continue;
+            const int so = (int)((uint32_t)row * rb);
+#pragma unroll
+            for (int ni = 0; ni < NI; ni++) {
+              float val = acc[mi][ni][v];
+              if constexpr (MD == 1) val = fmaf(ep.beta, old[v][ni], val);
+              if constexpr (MD == 2) {
+                typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+                u32x2 a2; a2.x = __float_as_uint(val); a2.y = 0u;
+                u32x2 z2; z2.x = 0u; z2.y = 0u;
+                __builtin_amdgcn_raw_buffer_store_b64(a2, rsO, (int)vo[ni], so, 0);
+                __builtin_amdgcn_raw_buffer_store_b64(z2, rsO, (int)vo[ni], so + (int)ep.cell_row_bytes(), 0);
+              } else {
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(val), rsO, (int)vo[ni], so, 0);
+              }
+            }
+          }
         }
+      };
+      if (mode == 0) pass(std::integral_constant<int, 0>());
+      else if (mode == 1) pass(std::integral_constant<int, 1>());
+      else pass(std::integral_constant<int, 2>());
+    }
+  }
+  if (!lean) {
+#pragma unroll
+    for (int mi = 0; mi < MI; mi++) {
+      const int ib = m0 + wm * TM + mi * 32 + 4 * half;
+#pragma unroll
+      for (int v = 0; v < 16; v++) {
+        const int row = ib + 8 * (v / 4) + (v % 4);
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++) ep.store(cs[ni], row, gs.M, acc[mi][ni][v], part);
+      }
+    }
+  }
+  if constexpr (EP::STATS && !SK) {
+    if (want_stats) {
+      // Row sums of the wavefront's TM x TN piece.  A lane holds 16 rows of one column, and a sum over columns done
+      // in registers costs five cross-lane steps per row; instead every 32 x 32 block goes through LDS once, transposed
+      // (the operand stages are free by now: the last barrier of the slab loop lies behind every read of them), so that
+      // lane l32 of each half reads row l32 of the block, 16 columns per half, and adds them up as it reads.
+      // Only this wavefront touches its region, whose LDS operations execute in program order.
+      // (sums of the accumulators: the host uses this path only for launches without a bias)
+      // Column c of the transposed block is kept rotated by 4c rows, which spreads both the 16-byte writes (lanes =
+      // columns) and the reads (lanes = rows) over all banks without padding.
+      constexpr int TLD = 32;
+      static_assert(4 * 32 * TLD * sizeof(float) <= igemm_smem_bytes<BM, BN, BK>(), "the transposed blocks of the four wavefronts fit the operand stages");
+      float* T = reinterpret_cast<float*>(lh_smem) + wave * (32 * TLD);
+#pragma unroll
+      for (int mi = 0; mi < MI; mi++) {
+        float r1 = 0.f, r2 = 0.f;
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++) {
+          const bool cv = cs[ni].valid;
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            float4 q;
+            q.x = cv ? acc[mi][ni][4 * g + 0] : 0.f; q.y = cv ? acc[mi][ni][4 * g + 1] : 0.f;
+            q.z = cv ? acc[mi][ni][4 * g + 2] : 0.f; q.w = cv ? acc[mi][ni][4 * g + 3] : 0.f;
+            *reinterpret_cast<float4*>(T + l32 * TLD + ((8 * g + 4 * half + 4 * l32) & 31)) = q;       // rows 8g + 4*half .. +3 of column l32
+          }
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+#pragma unroll
+          for (int c = 0; c < 16; c++) { const int cc = half * 16 + c; const float x = T[cc * TLD + ((l32 + 4 * cc) & 31)]; r1 += x; r2 = fmaf(x, x, r2); }
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+        }
+        r1 += __shfl_xor(r1, 32); r2 += __shfl_xor(r2, 32);
+        const int row = m0 + wm * TM + mi * 32 + l32;
+        if (half == 0 && row < gs.M) { float2* p = reinterpret_cast<float2*>(ep.partial) + (size_t)row * ep.slotsTotal + (ep.slotBase + tn * 2 + wn); *p = make_float2(r1, r2); }
       }
     }
   }
@@ -375,8 +529,6 @@ __global__ void __launch_bounds__(256) k_igemm_grouped(const IgemmGroups<AL, BL,
   igemm_block<BM, BN, BK, AL, BL, EP, false>(g.al[gi], g.bl[gi], g.ep[gi], g.gs[gi], b - g.first[gi]);
 }
 
-template <int BM, int BN, int BK>
-constexpr size_t igemm_smem_bytes() { return (size_t)2 * (BK / 4) * ((BM + 8 / (BK / 4)) + (BN + 8 / (BK / 4))) * sizeof(float4); }
 
 // Launch one tile configuration.
 //   splitK > 1 : the reduction is cut into splitK pieces per tile (needs an accumulating epilogue).
