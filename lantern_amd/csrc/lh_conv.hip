@@ -182,6 +182,14 @@ struct LoadConvBwdFilterA {
   const float* base; uint32_t nbytes;
   int K, PQ;
   FastDiv dPQ;
+  static constexpr bool STEP = true;
+  // a slab that lies inside one sample is followed, inside that sample, by the same offsets bk elements further on
+  __device__ __forceinline__ uint32_t step_bytes(int bk) const { return (uint32_t)bk * 4u; }
+  __device__ __forceinline__ int run_slabs(int k, int bk) const {
+    uint32_t n, pq;
+    dPQ.divmod(k, n, pq);
+    return (int)pq + bk > PQ ? 1 : (PQ - (int)pq) / bk;
+  }
   struct State { int rowoff; bool valid; };
   __device__ __forceinline__ void init(State& s, int i, int nrows) const { s.valid = i < nrows; s.rowoff = (s.valid ? i : 0) * PQ; }
   __device__ __forceinline__ uint32_t off1(const State& s, int kk, int kend, int e) const {

@@ -277,18 +277,23 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   // all offsets of the slab at kn from scratch
   auto decode = [&](int kn) {
     if constexpr (STEPPED) {
-      if (kn >= kend) { nrecA = 0; nrecB = 0; steps = 0; return; }
+      if (__builtin_amdgcn_readfirstlane((int)(kn >= kend))) { nrecA = 0; nrecB = 0; steps = 0; return; }
 #pragma unroll
       for (int e = 0; e < NEL; e++) elem(e, kn);
       xsA = 0; xsB = 0;
       const int whole = (kend - kn) / BK;                       // whole slabs from kn on
-      steps = min(min(al.run_slabs(kn, BK), bl.run_slabs(kn, BK)), whole) - 1;
+      steps = __builtin_amdgcn_readfirstlane(min(min(al.run_slabs(kn, BK), bl.run_slabs(kn, BK)), whole) - 1);
     }
   };
   // (oa, ob, ...) describe the slab at kn - BK and are made to describe the slab at kn
   auto advance = [&](int kn) {
     if constexpr (STEPPED) {
-      if (__builtin_expect(steps > 0, 1)) { steps -= 1; xsA += (int)al.step_bytes(BK); xsB += (int)bl.step_bytes(BK); }
+      // (the counters are the same in all lanes; saying so at every update keeps them, and the buffer descriptors and scalar
+      // offsets made from them, in scalar registers in every instantiation)
+      if (__builtin_expect(__builtin_amdgcn_readfirstlane(steps) > 0, 1)) {
+        steps = __builtin_amdgcn_readfirstlane(steps - 1);
+        xsA = __builtin_amdgcn_readfirstlane(xsA + (int)al.step_bytes(BK)); xsB = __builtin_amdgcn_readfirstlane(xsB + (int)bl.step_bytes(BK));
+      }
       else decode(kn);
     }
   };
@@ -396,7 +401,8 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   for (int ni = 0; ni < NI; ni++) cs[ni] = ep.col(n0 + wn * TN + ni * 32 + l32, gs.N);
   bool want_stats = false;
   if constexpr (EP::STATS && !SK) want_stats = ep.partial != nullptr;
-  // Lean stores (epilogues that offer them, complete sums only): the element of row i and column j lies at
+  // Lean stores (epilogues that offer them, complete sums only; partial sums added with buffer atomics, and the row-major
+  // epilogue of the filter gradient and sgemm, measured slower this way and stay on the general path): the element of row i and column j lies at
   // lane_bytes(j) + i * row_bytes(), so a store is one buffer instruction whose per-lane offset is fixed for the tile
   // (LH_OOB for a column past the edge: the store is dropped) and whose row goes into the scalar offset; the two halves of
   // a wavefront hold rows four apart, which the per-lane offset carries, and with M a multiple of 8 both are inside
