@@ -263,6 +263,7 @@ struct EpiConvOut {
   __device__ __forceinline__ uint32_t row_bytes() const { return (uint32_t)PIX * 4u; }
   __device__ __forceinline__ uint32_t cell_row_bytes() const { return (uint32_t)W * 4u; }
   __device__ __forceinline__ int lean_mode() const { return zfill2 ? 2 : (beta == 0.f ? 0 : 1); }
+  __device__ __forceinline__ float lean_scale() const { return 1.f; }
   // part: 0 = complete sum; 1 = first partial, 2 = later partial (atomic adds onto a prepared output)
   __device__ __forceinline__ void store(const Col& c, int i, int M, float v, int part) const {
     if (!c.valid || i >= M) return;

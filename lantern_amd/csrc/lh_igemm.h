@@ -141,6 +141,16 @@ struct EpiRowMajor {
   __device__ __forceinline__ void slice(int sp) { C += (long long)sp * sliceStride; }
   struct Col { int j; bool valid; };
   __device__ __forceinline__ Col col(int j, int N) const { Col c; c.j = j; c.valid = j < N; return c; }
+  // lean stores (see the store section of igemm_block): element (i, j) at j * 4 + i * ldc * 4 bytes from C, for matrices
+  // below 2 GiB; not for the atomic combination of partial sums, which measured slower through buffer atomics
+  static constexpr bool LEAN = true;
+  __device__ __forceinline__ bool lean_ok(int M) const { return !atomic && (M & 7) == 0 && (long long)M * ldc < 0x20000000LL; }
+  __device__ __forceinline__ float* lean_base() const { return C; }
+  __device__ __forceinline__ uint32_t lane_bytes(const Col& c) const { return (uint32_t)c.j * 4u; }
+  __device__ __forceinline__ uint32_t row_bytes() const { return (uint32_t)ldc * 4u; }
+  __device__ __forceinline__ uint32_t cell_row_bytes() const { return 0u; }
+  __device__ __forceinline__ int lean_mode() const { return beta == 0.f ? 0 : 1; }
+  __device__ __forceinline__ float lean_scale() const { return alpha; }
   // part: 0 = the whole reduction of this element is in v; 1 = first partial sum, 2 = a later one
   // (partials are combined with atomic adds onto an output the host has prepared)
   __device__ __forceinline__ void store(const Col& c, int i, int M, float v, int part) const {
@@ -401,8 +411,8 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   for (int ni = 0; ni < NI; ni++) cs[ni] = ep.col(n0 + wn * TN + ni * 32 + l32, gs.N);
   bool want_stats = false;
   if constexpr (EP::STATS && !SK) want_stats = ep.partial != nullptr;
-  // Lean stores (epilogues that offer them, complete sums only; partial sums added with buffer atomics, and the row-major
-  // epilogue of the filter gradient and sgemm, measured slower this way and stay on the general path): the element of row i and column j lies at
+  // Lean stores (epilogues that offer them, complete sums only; partial sums added with buffer atomics measured slower
+  // and stay on the general path): the element of row i and column j lies at
   // lane_bytes(j) + i * row_bytes(), so a store is one buffer instruction whose per-lane offset is fixed for the tile
   // (LH_OOB for a column past the edge: the store is dropped) and whose row goes into the scalar offset; the two halves of
   // a wavefront hold rows four apart, which the per-lane offset carries, and with M a multiple of 8 both are inside
@@ -417,6 +427,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
 #pragma unroll
       for (int ni = 0; ni < NI; ni++) vo[ni] = cs[ni].valid ? ep.lane_bytes(cs[ni]) + (uint32_t)(4 * half) * rb : LH_OOB;
       const int mode = ep.lean_mode();             // 0: overwrite, 1: beta * old + value, 2: value and the three zeros of its 2 x 2 cell
+      const float scale = ep.lean_scale();         // alpha of a gemm, 1 for a convolution
       auto pass = [&](auto MODE) {
         constexpr int MD = decltype(MODE)::value;
 #pragma unroll
@@ -442,7 +453,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
             const int so = (int)((uint32_t)row * rb);
 #pragma unroll
             for (int ni = 0; ni < NI; ni++) {
-              float val = acc[mi][ni][v];
+              float val = acc[mi][ni][v] * scale;
               if constexpr (MD == 1) val = fmaf(ep.beta, old[v][ni], val);
               if constexpr (MD == 2) {
                 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
