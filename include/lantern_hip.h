@@ -275,7 +275,9 @@ void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float*
  *   states and is all the backward pass needs besides x;  w = packed parameters, per direction
  *   W_ih[H,I], W_hh[H,H], b_ih[H], b_hh[H] (NNModule.scala:378-390), forward direction first.
  * lh_rnn_bwd: dx = beta_dx*dx + ... (dx may be NULL), dw += ...; takes T*B*D*H + D*H*H + ... floats of
- * scratch from the top of the arena and releases them before returning. */
+ * scratch from the top of the arena and releases them before returning.
+ * The recurrence runs one kernel per time step; for 16-byte aligned operands and 64 <= H <= 2048 that kernel uses the matrix
+ * instructions (LH_RNN_MFMA=0 in the environment keeps the vector form everywhere). */
 void lh_rnn_fwd(int mode, const float* x, const float* w, float* y, int T, int B, int I, int H, int bidir);
 void lh_rnn_bwd(int mode, const float* x, const float* y, const float* dy, const float* w, float* dx, float beta_dx, float* dw,
                 int T, int B, int I, int H, int bidir);
