@@ -9,6 +9,7 @@
 // directions in the same launch, each block producing 4-16 hidden units for the whole batch from
 // W_hh rows held in registers.  The output y doubles as the saved hidden states.
 #include "lh_common.h"
+#include "lh_rnn_tile.h"
 #include "../../include/lantern_hip.h"
 using namespace lh;
 
@@ -50,7 +51,6 @@ __device__ __forceinline__ void rnn_load_w(const float* __restrict__ W, int H, i
 //   pre(b, c)        called on a finishing lane before the sums: fetches what done() will need (so that those
 //                    loads are in flight during the arithmetic)
 //   done(b, c, s, f) called on the same lane with the finished sum of row b, weight row j0 + c
-struct RnnPre { float a, b, c; };
 constexpr int RED_LD = 65;
 template <int NK, int JC> struct RnnCfg { static constexpr int V = NK >= 32 ? 16 : 32; static constexpr int UBR = V / JC; };
 template <int NK, int JC, bool V4, class Pre, class Done>
@@ -148,86 +148,12 @@ __global__ void __launch_bounds__(TPB) k_rnn_bwd_step(BwdArgs a, int B, int H, i
       next[(int64_t)b * ld + i0 + c] = mode == 1 ? g * (1.0f - f.a * f.a) : (f.a > 0.f ? g : 0.f); });
 }
 
-// ---- the same step on the matrix pipes ------------------------------------------------------------------------
-// A block produces 16 hidden units for 16 * BT batch rows: BT 16 x 16 accumulator tiles of v_mfma_f32_16x16x4_f32 that share
-// the weight operand.  The reduction over k is cut NW ways: wavefront w takes the groups of 16 consecutive k numbered
-// w, w + NW, ...; inside a group lane l reads four consecutive k (one 16-byte load) of weight row j0 + l % 16 and of batch
-// row b0 + l % 16 (and b0 + 16 + l % 16), k = 16 * group + 4 * (l / 16) + (0..3), and component c of those loads feeds matrix
-// step c (which k a step contracts does not matter as long as both operands agree).  All loads of a wavefront are issued
-// before the first matrix instruction (NIT groups of 16-byte registers), so a step pays the memory latency once.
-// The partial tiles are added through LDS, and thread t finishes output t (and t + 256) of the block's.
-// Needs H % 4 == 0 and 16-byte aligned rows (the V4 condition of the kernels above).
-// Measured at T 185, B 32, H 800 (200 blocks with BT = 1): 5.0 us per step against 7.9 for the vector form; two batch tiles
-// per block (100 blocks) 7.2 us, eight wavefronts per block 5.1 us: BT = 1, NW = 4 is what gets launched.
-typedef float rnn_f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned rnn_u32x4 __attribute__((ext_vector_type(4)));
-constexpr int RNN_RSRC_FLAGS = 0x00020000;
-constexpr unsigned RNN_OOB = 0x80000000u;
-template <int NIT, int BT, int NW, class Pre, class Done>
-__device__ __forceinline__ void rnn_tile_mfma(const float* __restrict__ W, const float* __restrict__ in, int ld, bool use_in, int H, int B, int j0, int b0,
-                                              float* red, Pre pre, Done done) {
-  const int t = threadIdx.x, wave = t >> 6, lane = t & 63, r = lane & 15, kg = lane >> 4;
-  // the two outputs this thread finishes: index o = slot * 64 + lane' with slot = tile * 4 + v (accumulator register v of
-  // tile `tile`), lane' = 16 * (row / 4 within the tile) + unit
-  int ob[BT], oc[BT]; bool fin[BT]; RnnPre f[BT];
-#pragma unroll
-  for (int q = 0; q < BT; q++) {
-    const int o = (t & 255) + 256 * q, slot = o >> 6, ln = o & 63;
-    ob[q] = b0 + 16 * (slot >> 2) + 4 * (ln >> 4) + (slot & 3); oc[q] = ln & 15;
-    fin[q] = t < 256 && ob[q] < B && j0 + oc[q] < H;
-    f[q] = {0.f, 0.f, 0.f};
-    if (fin[q]) f[q] = pre(ob[q], oc[q]);
-  }
-  float tot[BT];
-#pragma unroll
-  for (int q = 0; q < BT; q++) tot[q] = 0.f;
-  if (use_in) {
-    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)W, 0, (int)((size_t)H * H * 4), RNN_RSRC_FLAGS);
-    const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, (int)(((size_t)(B - 1) * ld + H) * 4), RNN_RSRC_FLAGS);
-    const unsigned ow = j0 + r < H ? (unsigned)(j0 + r) * (unsigned)H * 4u : RNN_OOB;
-    const unsigned oh0 = b0 + r < B ? (unsigned)(b0 + r) * (unsigned)ld * 4u : RNN_OOB;
-    const unsigned oh1 = b0 + 16 + r < B ? (unsigned)(b0 + 16 + r) * (unsigned)ld * 4u : RNN_OOB;
-    rnn_u32x4 wv[NIT], h0[NIT], h1[NIT];
-#pragma unroll
-    for (int i = 0; i < NIT; i++) {
-      const int k = 16 * (wave + NW * i) + 4 * kg;
-      const bool in_k = k < H;                                   // H % 4 == 0: the group of four is inside the row or outside
-      wv[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, in_k ? (int)(ow + 4u * k) : (int)RNN_OOB, 0, 0);
-      h0[i] = __builtin_amdgcn_raw_buffer_load_b128(rh, in_k ? (int)(oh0 + 4u * k) : (int)RNN_OOB, 0, 0);
-      if (BT == 2) h1[i] = __builtin_amdgcn_raw_buffer_load_b128(rh, in_k ? (int)(oh1 + 4u * k) : (int)RNN_OOB, 0, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);             // every load is in flight before the first matrix instruction waits for one
-    rnn_f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < NIT; i++) {
-#pragma unroll
-      for (int c = 0; c < 4; c++) {
-        const float wc = __uint_as_float(wv[i][c]);
-        a0 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(h0[i][c]), wc, a0, 0, 0, 0);
-        if (BT == 2) a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(h1[i][c]), wc, a1, 0, 0, 0);
-      }
-    }
-    // D layout of a 16 x 16 tile: lane holds column (unit) lane % 16, rows (batch) 4 * (lane / 16) + v
-    float* my = red + wave * (256 * BT);
-#pragma unroll
-    for (int v = 0; v < 4; v++) { my[v * 64 + lane] = a0[v]; if (BT == 2) my[(4 + v) * 64 + lane] = a1[v]; }
-    __syncthreads();
-#pragma unroll
-    for (int q = 0; q < BT; q++) {
-      const int o = (t & 255) + 256 * q;
-#pragma unroll
-      for (int w = 0; w < NW; w++) tot[q] += red[w * (256 * BT) + o];
-    }
-  }
-#pragma unroll
-  for (int q = 0; q < BT; q++) if (fin[q]) done(ob[q], oc[q], tot[q], f[q]);
-}
 template <int NIT, int BT, int NW>
 __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(1, 2))) k_rnn_fwd_step_mfma(StepArgs a, int B, int H, int ld, int mode) {
   __shared__ float red[NW * 256 * BT];
   const int d = blockIdx.y, j0 = blockIdx.x * 16, b0 = blockIdx.z * (16 * BT);
   float* cur = a.cur[d]; const float* prev = a.prev[d]; const float* b1 = a.b1[d]; const float* b2 = a.b2[d];
-  rnn_tile_mfma<NIT, BT, NW>(a.W[d], prev, ld, prev != nullptr, H, B, j0, b0, red,
+  rnn_tile_mfma<NIT, BT, NW>(a.W[d], H, H, prev, ld, prev != nullptr, H, B, j0, b0, red,
     [&](int b, int c) { const int j = j0 + c; RnnPre f = {cur[(int64_t)b * ld + j], b1[j], b2[j]}; return f; },
     [&](int b, int c, float s, const RnnPre& f) { cur[(int64_t)b * ld + j0 + c] = act_fwd(mode, f.a + f.b + f.c + s); });
 }
@@ -236,7 +162,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(1,
   __shared__ float red[NW * 256 * BT];
   const int d = blockIdx.y, i0 = blockIdx.x * 16, b0 = blockIdx.z * (16 * BT);
   const float* cur = a.cur[d]; const float* dy = a.dy[d]; const float* hh = a.h[d]; float* next = a.next[d];
-  rnn_tile_mfma<NIT, BT, NW>(a.Wt[d], cur, ld, cur != nullptr, H, B, i0, b0, red,
+  rnn_tile_mfma<NIT, BT, NW>(a.Wt[d], H, H, cur, ld, cur != nullptr, H, B, i0, b0, red,
     [&](int b, int c) { const int64_t o = (int64_t)b * ld + i0 + c; RnnPre f = {hh[o], dy[o], 0.f}; return f; },
     [&](int b, int c, float s, const RnnPre& f) {
       const float g = f.b + s;
@@ -245,9 +171,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(1,
 // The matrix-pipe form runs for aligned operands (v4) and hidden sizes from 64 to 2048; LH_RNN_MFMA=0 in the environment
 // keeps every step on the vector form above.
 static bool rnn_use_mfma(bool v4, int H, int B, int ld) {
-  static int on = -1;
-  if (on < 0) { const char* e = getenv("LH_RNN_MFMA"); on = (e && e[0] == '0') ? 0 : 1; }
-  return on && v4 && H >= 64 && H <= 2048 && ((size_t)(B - 1) * ld + H) * 4 < 0x80000000ull && (size_t)H * H * 4 < 0x80000000ull;
+  return rnn_mfma_enabled() && v4 && H >= 64 && H <= 2048 && ((size_t)(B - 1) * ld + H) * 4 < 0x80000000ull && (size_t)H * H * 4 < 0x80000000ull;
 }
 
 // hidden sizes up to 64 * NK, JC weight rows per block (JC * NK <= 128 registers of weights).  v4: every row the
