@@ -144,6 +144,107 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(1,
     [&](int b, int c, float s, const RnnPre& f) { a.out[(int64_t)b * a.ldo + j0 + c] = f.a + s; });
 }
 static bool aligned16g(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// The LSTM's forward step in one launch: a block owns the four gates of four hidden units (column c of its tile stands for gate
+// c / 4 of unit u0 + c % 4, i.e. row (c / 4) * H + u0 + c % 4 of W_hh) for 16 batch rows; after the partial tiles are in LDS,
+// thread (batch row, unit) adds up the four gate sums and does what k_lstm_fwd_point does: activations into `act`, the new cell
+// and hidden state.  hp == nullptr: no previous state (the sums are zero).
+template <int NIT>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+k_lstm_fwd_step_mfma(const float* __restrict__ hp, int ldp, const float* __restrict__ Whh, float* __restrict__ act, const float* __restrict__ b_ih,
+                     const float* __restrict__ b_hh, const float* __restrict__ c_prev, float* __restrict__ c, float* __restrict__ h, int B, int H, int ldh) {
+  __shared__ float red[4 * 256];
+  const int t = threadIdx.x, u0 = blockIdx.x * 4, b0 = blockIdx.y * 16;
+  const int bl = t >> 2, u = t & 3, b = b0 + bl, j = u0 + u;
+  const bool fin = t < 64 && b < B && j < H;
+  float pa[4], pb[4], cp = 0.f;
+  if (fin) {
+    // what the output stage needs, requested before the products
+#pragma unroll
+    for (int g = 0; g < 4; g++) { pa[g] = act[(size_t)b * 4 * H + g * H + j]; pb[g] = b_ih[g * H + j]; }
+    cp = c_prev ? c_prev[(size_t)b * H + j] : 0.f;
+  }
+  if (hp) {
+    const int r = t & 15;
+    rnn_tile_partials<NIT, 1, 4>(Whh, H, (size_t)4 * H * H * 4, u0 + (r & 3) < H ? (r >> 2) * H + u0 + (r & 3) : -1, hp, ldp, H, B, b0, red);
+  }
+  if (!fin) return;
+  float p[4];
+#pragma unroll
+  for (int g = 0; g < 4; g++) {
+    float s = 0.f;
+    if (hp) { const int o = (bl & 3) * 64 + 16 * (bl >> 2) + 4 * g + u; s = (red[o] + red[256 + o]) + (red[512 + o] + red[768 + o]); }
+    p[g] = ((pa[g] + s) + pb[g]) + b_hh[g * H + j];
+  }
+  const float ig = sigm(p[0]), fg = sigm(p[1]), gg = tanhf(p[2]), og = sigm(p[3]);
+  const float cn = fg * cp + ig * gg;
+  float* a = act + (size_t)b * 4 * H + j;
+  a[0] = ig; a[H] = fg; a[2 * H] = gg; a[3 * H] = og;
+  c[(size_t)b * H + j] = cn;
+  h[(size_t)b * ldh + j] = og * tanhf(cn);
+}
+// The GRU's forward step the same way: three gates of four units are 12 of the tile's 16 columns (the last four stay idle);
+// the hidden-side sums are used where they are, so no buffer holds them between two launches.
+template <int NIT>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+k_gru_fwd_step_mfma(const float* __restrict__ hp, int ldp, const float* __restrict__ Whh, float* __restrict__ act, const float* __restrict__ b_ih,
+                    const float* __restrict__ b_hh, float* __restrict__ q, float* __restrict__ h, int B, int H, int ldh) {
+  __shared__ float red[4 * 256];
+  const int t = threadIdx.x, u0 = blockIdx.x * 4, b0 = blockIdx.y * 16;
+  const int bl = t >> 2, u = t & 3, b = b0 + bl, j = u0 + u;
+  const bool fin = t < 64 && b < B && j < H;
+  float pa[3], pb[3], hprev = 0.f;
+  if (fin) {
+#pragma unroll
+    for (int g = 0; g < 3; g++) { pa[g] = act[(size_t)b * 3 * H + g * H + j]; pb[g] = b_ih[g * H + j]; }
+    hprev = hp ? hp[(size_t)b * ldp + j] : 0.f;
+  }
+  if (hp) {
+    const int r = t & 15;
+    rnn_tile_partials<NIT, 1, 4>(Whh, H, (size_t)3 * H * H * 4, (r < 12 && u0 + (r & 3) < H) ? (r >> 2) * H + u0 + (r & 3) : -1, hp, ldp, H, B, b0, red);
+  }
+  if (!fin) return;
+  float gs[3];
+#pragma unroll
+  for (int g = 0; g < 3; g++) {
+    gs[g] = 0.f;
+    if (hp) { const int o = (bl & 3) * 64 + 16 * (bl >> 2) + 4 * g + u; gs[g] = (red[o] + red[256 + o]) + (red[512 + o] + red[768 + o]); }
+  }
+  const float r = sigm(pa[0] + pb[0] + b_hh[j] + gs[0]);
+  const float z = sigm(pa[1] + pb[1] + b_hh[H + j] + gs[1]);
+  const float qq = gs[2] + b_hh[2 * H + j];
+  const float n = tanhf(pa[2] + pb[2] + r * qq);
+  float* a = act + (size_t)b * 3 * H + j;
+  a[0] = r; a[H] = z; a[2 * H] = n;
+  q[(size_t)b * H + j] = qq;
+  h[(size_t)b * ldh + j] = (1.f - z) * n + z * hprev;
+}
+// true when the fused step ran; false: the caller runs the product and the element-wise kernel
+static bool gated_fused_ok(const float* hp, int ldp, const float* Whh, int ng, int B, int H) {
+  const int nit = (int)cdiv(cdiv(H, 16), 4);
+  return rnn_mfma_enabled() && (H & 3) == 0 && (ldp & 3) == 0 && (hp == nullptr || aligned16g(hp)) && aligned16g(Whh) && nit <= 16 &&
+         ((size_t)(B - 1) * ldp + H) * 4 < 0x80000000ull && (size_t)ng * H * H * 4 < 0x80000000ull;
+}
+static bool gru_fwd_step_fused(const float* hp, int ldp, const float* Whh, float* act, const float* b_ih, const float* b_hh, float* q, float* h,
+                               int B, int H, int ldh) {
+  if (!gated_fused_ok(hp, ldp, Whh, 3, B, H)) return false;
+  const int nit = (int)cdiv(cdiv(H, 16), 4);
+  const dim3 grid((unsigned)cdiv(H, 4), (unsigned)cdiv(B, 16));
+#define GOG(N) hipLaunchKernelGGL((k_gru_fwd_step_mfma<N>), grid, dim3(256), 0, g_stream, hp, ldp, Whh, act, b_ih, b_hh, q, h, B, H, ldh)
+  if (nit <= 4) GOG(4); else if (nit <= 8) GOG(8); else if (nit <= 13) GOG(13); else GOG(16);
+#undef GOG
+  return true;
+}
+static bool lstm_fwd_step_fused(const float* hp, int ldp, const float* Whh, float* act, const float* b_ih, const float* b_hh, const float* c_prev,
+                                float* c, float* h, int B, int H, int ldh) {
+  if (!gated_fused_ok(hp, ldp, Whh, 4, B, H)) return false;
+  const int nit = (int)cdiv(cdiv(H, 16), 4);
+  const dim3 grid((unsigned)cdiv(H, 4), (unsigned)cdiv(B, 16));
+#define GOL(N) hipLaunchKernelGGL((k_lstm_fwd_step_mfma<N>), grid, dim3(256), 0, g_stream, hp, ldp, Whh, act, b_ih, b_hh, c_prev, c, h, B, H, ldh)
+  if (nit <= 4) GOL(4); else if (nit <= 8) GOL(8); else if (nit <= 13) GOL(13); else GOL(16);
+#undef GOL
+  return true;
+}
 static void step_product_nt(const float* in, int ldi, const float* W, int ldw, float* out, int ldo, int B, int NJ, int K) {
   const int groups = (int)cdiv(K, 16), nw = groups > 64 ? 8 : 4, nit = (int)cdiv(groups, nw);
   const bool ok = rnn_mfma_enabled() && (K & 3) == 0 && (ldi & 3) == 0 && (ldw & 3) == 0 && aligned16g(in) && aligned16g(W) && nit <= 25 &&
@@ -205,13 +306,17 @@ void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const floa
       // clears it.  The LSTM adds straight into the step's input projection; the GRU keeps the hidden side apart (its n gate scales
       // it by r) in gh, which the point kernel clears after reading.
       if (mode == 2) {
-        if (hp) step_product_nt(hp, ldp, Whh, H, a, G, B, G, H);
-        hipLaunchKernelGGL(k_lstm_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, nullptr, bih, bhh,
-                           cp, aux + (size_t)t * B * H, h, B, H, ldh);
+        if (!lstm_fwd_step_fused(hp, ldp, Whh, a, bih, bhh, cp, aux + (size_t)t * B * H, h, B, H, ldh)) {
+          if (hp) step_product_nt(hp, ldp, Whh, H, a, G, B, G, H);
+          hipLaunchKernelGGL(k_lstm_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, nullptr, bih, bhh,
+                             cp, aux + (size_t)t * B * H, h, B, H, ldh);
+        }
       } else {
-        if (hp) step_product_nt(hp, ldp, Whh, H, gh, G, B, G, H);
-        hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, gh, bih, bhh, hp, ldp,
-                           aux + (size_t)t * B * H, h, B, H, ldh);
+        if (!gru_fwd_step_fused(hp, ldp, Whh, a, bih, bhh, aux + (size_t)t * B * H, h, B, H, ldh)) {
+          if (hp) step_product_nt(hp, ldp, Whh, H, gh, G, B, G, H);
+          hipLaunchKernelGGL(k_gru_fwd_point, dim3(point_grid(B, H)), dim3(TPB), 0, g_stream, a, gh, bih, bhh, hp, ldp,
+                             aux + (size_t)t * B * H, h, B, H, ldh);
+        }
       }
     }
   };
