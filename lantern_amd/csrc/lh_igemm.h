@@ -192,7 +192,9 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   // STEPPED: both loaders can be advanced by a wave-uniform step, so inside a run of slabs the offsets of the next slab
   // cost two scalar additions instead of a decode per element; a slab past the end of the reduction is switched off by a
   // buffer descriptor of zero bytes (every lane out of range, the loads return 0 without touching memory).
-  constexpr bool STEPPED = LhCanStep<AL>::value && LhCanStep<BL>::value;
+  // (Not on the 32-row tiles with a tap-major gather: they serve layers of at most 32 channels, where a filter tap is as deep
+  // as one 32-deep slab, every slab is decoded anyway and the interleaved decode below is the faster one.)
+  constexpr bool STEPPED = LhCanStep<AL>::value && LhCanStep<BL>::value && (BM >= 64 || !(AL::SPLIT || BL::SPLIT));
   const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc((void*)al.base, 0, (int)al.nbytes, LH_RSRC_FLAGS);
   const __amdgpu_buffer_rsrc_t rsB = __builtin_amdgcn_make_buffer_rsrc((void*)bl.base, 0, (int)bl.nbytes, LH_RSRC_FLAGS);
   const int t = threadIdx.x;
