@@ -740,7 +740,8 @@ def test_rnn_forward_and_backward(pair, case):
 
 
 @pytest.mark.parametrize("case", [(2, True, 7, 5, 20, 48), (3, True, 7, 5, 20, 48), (2, False, 1, 2, 5, 16), (3, False, 1, 2, 5, 16), (2, False, 9, 33, 7, 37),
-                                  (3, True, 4, 3, 33, 130), (2, True, 3, 4, 161, 96), (3, False, 12, 8, 64, 256)]
+                                  (3, True, 4, 3, 33, 130), (2, True, 3, 4, 161, 96), (3, False, 12, 8, 64, 256),
+                                  (2, True, 3, 32, 40, 800), (3, True, 3, 17, 24, 528), (2, False, 2, 20, 12, 1000)]
                          + _random_cases(108, 6, lambda r: (_ri(r, 2, 3), bool(r.rand() < 0.5), _ri(r, 1, 8), _ri(r, 1, 9), _ri(r, 1, 40), _pick(r, [5, 16, 37, 64, 130]))),
                          ids=lambda c: "mode%d_bi%d_T%d_B%d_I%d_H%d" % c)
 def test_gated_rnn_forward_and_backward(pair, case):
