@@ -435,8 +435,8 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
 #pragma unroll
         for (int mi = 0; mi < MI; mi++) {
           const int r0 = m0 + wm * TM + mi * 32;
-          // mode 1: all old values of the block are requested before the first of them is used (a store cannot be
-          // moved across a load by the compiler, so element by element every load would wait for a round trip of its own)
+          // mode 1: all old values of the block are requested before the first of them is used (the compiler cannot move
+          // a load across the store in front of it, so element by element every load would wait for a round trip of its own)
           float old[MD == 1 ? 16 : 1][NI];
           if constexpr (MD == 1) {
 #pragma unroll
