@@ -6,8 +6,9 @@
 //
 // The input projection of all time steps and the three weight/input gradients are large GEMMs
 // (lh_sgemm, MFMA).  Only the recurrence is sequential: one small kernel per time step, both
-// directions in the same launch, each block producing 4-16 hidden units for the whole batch from
-// W_hh rows held in registers.  The output y doubles as the saved hidden states.
+// directions in the same launch.  For aligned operands a block produces 16 hidden units for 16 batch rows
+// on the matrix pipes (lh_rnn_tile.h); otherwise 4-16 hidden units for the whole batch from W_hh rows held
+// in registers (the vector form).  The output y doubles as the saved hidden states.
 #include "lh_common.h"
 #include "lh_rnn_tile.h"
 #include "../../include/lantern_hip.h"

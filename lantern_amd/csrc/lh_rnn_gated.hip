@@ -7,8 +7,10 @@
 // b_hh[G] with G = 4H or 3H (NNModule.scala:378-390).
 //
 // Everything that is not sequential is one matrix product over all time steps (lh_sgemm on MFMA): the input projection,
-// both weight gradients, the input gradient.  A time step is one [B, H] x [H, G] product with the previous state and one
-// element-wise kernel over [B, H].  The forward pass leaves the gate activations and the cell state (GRU: W_hn h + b_hn)
+// both weight gradients, the input gradient.  A forward time step is one launch (the [B, H] x [H, G] product with the
+// previous state on 16 x 16 matrix tiles that hold all gates of four units, the gate arithmetic behind it); a backward
+// step, and a forward step on operands the tile kernel does not take, is a product plus one element-wise kernel over
+// [B, H].  The forward pass leaves the gate activations and the cell state (GRU: W_hn h + b_hn)
 // of every step in `reserve`; the backward pass turns the activations into pre-activation gradients in place.
 #include "lh_common.h"
 #include "lh_rnn_tile.h"
