@@ -177,3 +177,23 @@ def test_join_whose_shortcut_is_the_batchnorms_own_input(be):
     dxhat = dz * gam
     dh = (dxhat - dxhat.mean((0, 2, 3), keepdims=True) - xhat * (dxhat * xhat).mean((0, 2, 3), keepdims=True)) / np.sqrt(var + 1e-5) + dz
     np.testing.assert_allclose(fused[1], 1.5 * dh, rtol=2e-4, atol=2e-4)
+
+
+def test_relu_mask_recording_counts_flips(on_cpu):
+    """The tracking tests' relu-mask comparison (tests/test_training_parity.py): `_run(masks=)` records the sign pattern of every
+    non-negative tape value per step, `_mask_flips` counts where two runs differ.  Two runs of the same program on the oracle
+    record identical masks; one flipped bit in one tensor of one step is reported as exactly that."""
+    from tests.test_training_parity import _run, _mask_flips
+    from lantern_amd.apps.lenet import Trainer
+    mk = lambda: Trainer(batch=4, lr=0.0005)
+    m1, m2 = [], []
+    l1, _ = _run(mk, on_cpu, 2, masks=m1)
+    l2, _ = _run(mk, on_cpu, 2, masks=m2)
+    np.testing.assert_array_equal(l1, l2)
+    assert len(m1) == 2 and any(m is not None for m in m1[0]), "no relu output was recorded"
+    assert _mask_flips(m1, m2) == []
+    i = next(k for k, m in enumerate(m2[1]) if m is not None)
+    shape, bits = m2[1][i]
+    flipped = bits.copy(); flipped[0] ^= 0x80
+    m2[1][i] = (shape, flipped)
+    assert _mask_flips(m1, m2) == [(1, 1, 1)]
