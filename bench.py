@@ -79,6 +79,8 @@ def run_gpu(args):
         lib.lh_set_side_stream(0)
     if args.deterministic:
         be.setDeterministic(True)
+    if args.no_fusion:
+        lib.lh_set_fusion(0)
     streamed = bool(getattr(tr, "streamed", False))
     loss_first = None
     for i in range(args.warmup):
@@ -151,12 +153,17 @@ def run_gpu(args):
     if not getattr(tr, "batching", False):
         lib.lh_prof_enable(sum(1 << CATS.index(c) for c in hbm_cats))
         lib.lh_prof_collect(ms, calls, len(CATS))
+        wb = (C.c_double * len(CATS))()
+        lib.lh_work_collect(wb, len(CATS))          # reset: the library counts the algorithmic bytes of the kernels it chooses to run
         for _ in range(args.steps):
             tr.step()
             tr.end_step()
         be.sync()
         lib.lh_prof_collect(ms, calls, len(CATS))
+        lib.lh_work_collect(wb, len(CATS))
         timed_hbm = {c: (ms[CATS.index(c)] / args.steps, int(calls[CATS.index(c)]) // args.steps) for c in hbm_cats}
+        for c, key in (("bn_fwd", "bn_fwd_bytes"), ("bn_bwd", "bn_bwd_bytes"), ("elementwise", "elementwise_bytes")):
+            work[key] = wb[CATS.index(c)] / args.steps
     # a separate, untimed pass with every category instrumented (breakdown for the log)
     lib.lh_prof_enable((1 << CATS.index("cmdlist")) if getattr(tr, "batching", False) else (1 << len(CATS)) - 1)
     tr.step(); tr.end_step()
@@ -165,6 +172,21 @@ def run_gpu(args):
     lib.lh_prof_enable(0)
     loss_val = float(tr.step().toCPU()[0]); tr.end_step()
     peak_gb = lib.lh_heap_peak() / 2 ** 30
+    fstats = (C.c_int64 * 8)()
+    lib.lh_fusion_stats(fstats, 8)
+    unfused_sec = None
+    if args.workload == "resnet50" and not args.no_fusion and not args.graph:
+        # the same steps with the library running every call as issued (no chains fused, every lh_malloc cleared, every
+        # gradient accumulated, one optimizer launch per parameter): what the call sequence costs without the deferred work
+        lib.lh_set_fusion(0)
+        tr.step(); tr.end_step(); be.sync()
+        u0 = time.perf_counter()
+        for _ in range(args.steps):
+            tr.step()
+            tr.end_step()
+        be.sync()
+        unfused_sec = time.perf_counter() - u0
+        lib.lh_set_fusion(1)
     c_host = None
     c_dir = None
     if args.workload == "treelstm" and os.path.exists(TREE_C_PROGRAM):
@@ -219,7 +241,7 @@ def run_gpu(args):
         if not args.keep_c_inputs:
             import shutil
             shutil.rmtree(c_dir, ignore_errors=True)
-    return {"emitted": emitted, "c_host": c_host, "streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
+    return {"fusion_stats": [int(v) for v in fstats], "unfused_sec": unfused_sec, "emitted": emitted, "c_host": c_host, "streamed": streamed, "resident_sec": resident_sec, "timed_hbm": timed_hbm, "sec": t1 - t0, "issue_sec": (t_issued - t0) if t_issued is not None else None, "timed": timed, "work": work, "breakdown": breakdown, "loss": loss_val, "loss_first": loss_first, "arena_peak_gib": peak_gb,
             "per_step": per_step, "desc": desc}
 
 
@@ -279,6 +301,7 @@ def main():
     ap.add_argument("--no-side-stream", action="store_true", help="filter gradients in line on the main stream (kernel profiles: no two kernels overlap)")
     ap.add_argument("--resident", action="store_true", help="resnet50: keep one batch resident on the device (no per-step upload, no loss read-back)")
     ap.add_argument("--deterministic", action="store_true", help="fixed-order reductions and rule-chosen launch plans (lh_set_deterministic): what run-to-run bit equality costs")
+    ap.add_argument("--no-fusion", action="store_true", help="lh_set_fusion(0): every library call runs as issued (no chains fused, every block cleared when handed out)")
     ap.add_argument("--graph", action="store_true", help="time replays of the step recorded into a HIP graph (fixed-shape workloads)")
     ap.add_argument("--verbose", action="store_true")
     args = ap.parse_args()
@@ -350,6 +373,9 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": g["desc"], "global_batch": args.batch, "loss_first_step": round(g["loss_first"], 5) if g["loss_first"] is not None else None, "loss_after_run": round(g["loss"], 5), "arena_peak_gib": round(g["arena_peak_gib"], 2),
                    "launch": "hip graph replay" if args.graph else "one launch per kernel",
+                   "calls": "one library call per Backend trait method (conv2D_batch, batchNormTraining, relu in place, +, one momentum_update per parameter; "
+                            "every buffer from lh_malloc, every gradient accumulated): what scala/TensorDslHIP.scala emits; the library fuses the chains" +
+                            (" (fusion switched OFF for this run)" if args.no_fusion else ""),
                    "host_issue_ms_per_step": round(1000.0 * g["issue_sec"] / args.steps, 3) if g["issue_sec"] is not None else None,
                    "h2d": ("included: the batch (%.1f MB) is uploaded from pinned host memory for every step on a copy stream, beside the previous step; "
                            "the loss is read back every step without a wait" % (args.batch * 3 * args.hw * args.hw * 4 / 1e6)) if g["streamed"] else "not included: inputs resident on the device",
@@ -362,6 +388,13 @@ def main():
         out["python_mirror_host"] = python_host
     if g.get("emitted"):
         out["emitted_c_program"] = g["emitted"]
+    if g.get("unfused_sec"):
+        out["calls_run_as_issued"] = {"value": round(g["per_step"] * args.steps / g["unfused_sec"], 2), "ms_per_step": round(1000.0 * g["unfused_sec"] / args.steps, 3),
+                                      "note": "the same call sequence with lh_set_fusion(0): nothing fused, every lh_malloc cleared at once, gradients accumulated, 161 optimizer launches"}
+    fs = g.get("fusion_stats")
+    if fs:
+        out["config"]["library_fusion_totals"] = {"forward_chains": fs[0], "backward_chains": fs[1], "optimizer_calls_gathered": fs[2], "zero_fills_avoided": fs[3],
+                                                  "zero_fills_done": fs[4], "results_produced_on_demand": fs[5], "chains_ended_without_relu": fs[6]}
     if g["resident_sec"] is not None:
         out["resident_input"] = {"value": round(g["per_step"] * args.steps / g["resident_sec"], 2), "ms_per_step": round(1000.0 * g["resident_sec"] / args.steps, 3),
                                  "note": "the same steps with the batch resident on the device: no upload, no loss read-back"}

@@ -156,6 +156,37 @@ void lh_cmdlist_end(void);
 void lh_cmdlist_stats(int64_t* recorded, int64_t* launches);
 void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat);
 
+/* Fusion of adjacent calls (no counterpart in the reference, whose cuDNN backend runs every trait method as its own
+ * library call: CDN:833-880, 1025-1109, 1380-1429).  Lantern's generated code issues ONE call per method of the Backend
+ * trait: convBBP -> batchNorm -> relu(inPlace) arrive as lh_conv2d_fwd, lh_bn_train_fwd, lh_unary(LH_RELU, y, y)
+ * (ONNXLib.scala:847-872), the optimizer as one lh_momentum per parameter (NNModule.scala:296-303), and every buffer,
+ * gradients included, comes zero-filled from lh_malloc and is accumulated into (TD:1509-1514).  With fusion on (the
+ * default; LH_NO_FUSION=1 in the environment or lh_set_fusion(0) turn it off) the library puts work off until the next
+ * call shows what it is part of, so that such a program runs the kernels a hand-fused one would:
+ *   - lh_conv2d_fwd, lh_bn_train_fwd, a same-shape lh_bcast_op(LH_ADD), lh_unary_grad(LH_RELU, in place) and the same-shape
+ *     lh_bcast_op_grad(LH_ADD) behind it do not launch when called.  If the next call continues one of the chains
+ *       conv -> batch norm -> [+ shortcut] -> relu in place,     relu_grad -> [add_grad] -> batch-norm gradient
+ *     the chain runs as lh_conv2d_fwd_bn_apply / lh_bn_train_fwd_relu / lh_add_relu / lh_bn_bwd_relu / lh_bn_bwd_add_relu;
+ *     any other call (lh_malloc, lh_malloc_uninit and lh_mark excepted) first launches what is waiting, unfused.
+ *     Runs of lh_momentum / lh_sgd calls with equal hyper-parameters become one multi-tensor launch.
+ *   - a block of more than 1 MiB from lh_malloc is cleared when something first reads it; a call that overwrites it, or
+ *     would add into it with beta = 1, writes it without the clearing pass and without reading it; lh_rewind forgets it.
+ *   - what a fused chain does not store because programs do not read it (the batch norm's own output under a residual
+ *     join; the in-place masking of the gradient buffer by relu_grad) is produced when a call does read it.
+ * Results are those of the calls as issued (the fused kernels give the bits of the sequences they replace wherever two
+ * launches of the sequence itself agree bit for bit).  Every entry point of this header takes part; a pointer handed to
+ * anything else (another library, a kernel of the caller's) must be preceded by lh_sync() AND lh_flush_deferred().
+ * lh_fusion_stats: h_out[0..6] = forward chains fused, backward chains fused, optimizer calls gathered, zero fills avoided,
+ * zero fills done, results produced on demand, conv -> bn or bn -> + chains that ended without a relu. */
+void lh_set_fusion(int on);
+int lh_get_fusion(void);
+void lh_flush_deferred(void);               /* everything put off is enqueued now (nothing waits) */
+void lh_fusion_stats(int64_t* h_out, int n);
+/* Algorithmic bytes of the HBM-bound kernels launched since the last call, per LH_CAT_* category (a measurement aid for the
+ * benchmark: with fusion on, the caller no longer knows which kernels ran).  h_bytes[c] = bytes the kernels of category c
+ * must move at least (every operand read or written once per pass the kernel makes over it). */
+void lh_work_collect(double* h_bytes, int ncat);
+
 /* ---- fill / elementwise ------------------------------------------------ */
 void lh_fill(float* x, float v, int64_t n);                                    /* fill, fillInPlace: CUB:133-151 */
 void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, int64_t inner); /* fillWithBias: CPU:39-62 */

@@ -56,6 +56,11 @@ SIGNATURES = {
     "lh_cmdlist_end": (None, []),
     "lh_cmdlist_stats": (None, [C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "lh_prof_collect": (None, [P, P, I]),
+    "lh_set_fusion": (None, [I]),
+    "lh_get_fusion": (I, []),
+    "lh_flush_deferred": (None, []),
+    "lh_fusion_stats": (None, [P, I]),
+    "lh_work_collect": (None, [P, I]),
     "lh_fill": (None, [P, F, L]),
     "lh_fill_with_bias": (None, [P, P, L, L, L]),
     "lh_clip": (None, [P, F, L]),

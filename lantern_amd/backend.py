@@ -70,7 +70,7 @@ class Backend:
     """Operator API (TD:137-379).  Tensors are passed as objects with `.data` (Buf) and `.shape`."""
 
     name = "abstract"
-    ops_left = 0      # set by the tape before a convolution's backward: how many backward operators follow it
+    convs_open = 0    # kept by the tape: forward convolutions whose gradient call is still to come
 
     # -- memory ---------------------------------------------------------------------------
     def setup(self): raise NotImplementedError
@@ -82,7 +82,8 @@ class Backend:
     def getMallocAddr(self): raise NotImplementedError                      # TD:1782-1784 / CUB:18-20
     def resetMallocAddr(self, addr): raise NotImplementedError              # TD:1786-1789 / CUB:22-25
 
-    # -- fusable pairs: defaults are the unfused sequences of trait calls ------------------------------
+    # -- the library's fused entry points, callable directly (tests, hand-fused front ends); the defaults are the sequences
+    #    of trait calls they stand for.  The TensorR front end does not use them: it issues one trait call per operator. ----
     def batchNormTraining_into(self, x, scale, bias, rmean, rvar, y, sm, si, N, C, HW, relu, eps=1e-5, factor=0.1):
         """batchNormTraining writing into caller-provided y / saveMean / saveInvStd, optionally followed by relu(inPlace)."""
         yy, m, v = self.batchNormTraining(x, scale, bias, rmean, rvar, N, C, HW, eps, factor)
@@ -152,7 +153,7 @@ class BackendHIP(Backend):
         self.lib = None
         self.dropout_seed = 42
         self.side_order = int(os.environ.get("LH_SIDE_ORDER", "1"))
-        self.side_min_ops = int(os.environ.get("LH_SIDE_MIN_OPS", "6"))
+        self.side_min_convs = int(os.environ.get("LH_SIDE_MIN_CONVS", "2"))
         self.dropout_offset = 0
         self.work = {}            # algorithmic flop / bytes issued, by kind, while count_work is on (the benchmark's profiled pass)
         self.count_work = False
@@ -242,7 +243,7 @@ class BackendHIP(Backend):
     def fromHost(self, arr):
         arr = np.ascontiguousarray(arr)
         assert arr.dtype.itemsize == 4, "only 4-byte element types cross the boundary"
-        buf = self.mallocArray(arr.size, zero=False)
+        buf = self.mallocArray(arr.size)
         if arr.size:
             self.lib.lh_h2d(buf.ptr, arr.ctypes.data, arr.nbytes); _lib.check()
         return buf
@@ -283,7 +284,7 @@ class BackendHIP(Backend):
 
     def fillWithBias(self, dims, bias, dim):
         outer = int(np.prod(dims[:dim], dtype=np.int64)); c = dims[dim]; inner = int(np.prod(dims[dim + 1:], dtype=np.int64))
-        res = self.mallocArray(outer * c * inner, zero=False)
+        res = self.mallocArray(outer * c * inner)
         self.lib.lh_fill_with_bias(res.ptr, bias.ptr, outer, c, inner); _lib.check()
         return res
 
@@ -292,18 +293,18 @@ class BackendHIP(Backend):
 
     # -- dot family (TD:186-219; CUB:173-282) -----------------------------------------------
     def vectorVectorDot(self, x, y, n):
-        res = self.mallocArray(1, zero=False)
+        res = self.mallocArray(1)
         self.lib.lh_dot_vv(x.ptr, y.ptr, res.ptr, n); _lib.check()
         return res
 
     def matrixVectorDot(self, x, y, m, n):
-        res = self.mallocArray(m, zero=False)
+        res = self.mallocArray(m)
         self.lib.lh_sgemv(0, m, n, 1.0, x.ptr, n, y.ptr, 0.0, res.ptr); _lib.check()
         if self.count_work: self._count("gemv_flop", 2.0 * m * n); self._count("gemv_bytes", 4.0 * m * n)
         return res
 
     def matrixMatrixDot(self, x, y, m, k, n):
-        res = self.mallocArray(m * n, zero=False)
+        res = self.mallocArray(m * n)
         self.lib.lh_sgemm(0, 0, m, n, k, 1.0, x.ptr, k, y.ptr, n, 0.0, res.ptr, n); _lib.check()
         if self.count_work: self._count("gemm_flop", 2.0 * m * n * k)
         return res
@@ -329,7 +330,7 @@ class BackendHIP(Backend):
 
     # -- gemm (TD:279-280; CUB:589-688): result [d1,d3], contraction d2 --------------------------
     def gemm(self, x, tx, y, ty, alpha, d1, d2, d3):
-        res = self.mallocArray(d1 * d3, zero=False)
+        res = self.mallocArray(d1 * d3)
         self.lib.lh_sgemm(int(tx), int(ty), d1, d3, d2, alpha, x.ptr, d1 if tx else d2, y.ptr, d2 if ty else d3, 0.0, res.ptr, d3)
         _lib.check()
         if self.count_work: self._count("gemm_flop", 2.0 * d1 * d2 * d3)
@@ -356,7 +357,7 @@ class BackendHIP(Backend):
     # -- broadcast arithmetic (TD:222-270) ---------------------------------------------------------
     def bcast_op(self, op, a, ashape, b, bshape, oshape):
         n = int(np.prod(oshape, dtype=np.int64))
-        res = self.mallocArray(n, zero=False)
+        res = self.mallocArray(n)
         self.lib.lh_bcast_op(op, a.ptr, _ints(ashape), b.ptr, _ints(bshape), res.ptr, _ints(oshape), len(oshape)); _lib.check()
         return res
 
@@ -368,7 +369,7 @@ class BackendHIP(Backend):
         self.lib.lh_bcast_update(op, a.ptr, _ints(ashape), b.ptr, _ints(bshape), len(ashape)); _lib.check()
 
     def scalar_op(self, op, x, s, n, out=None):
-        res = out if out is not None else self.mallocArray(n, zero=False)
+        res = out if out is not None else self.mallocArray(n)
         self.lib.lh_scalar_op(op, x.ptr, res.ptr, s, n); _lib.check()
         return res
 
@@ -376,7 +377,7 @@ class BackendHIP(Backend):
         self.lib.lh_geam(x.ptr, alpha, y.ptr, beta, out.ptr, n); _lib.check()
 
     def trans(self, x, rows, cols):
-        res = self.mallocArray(rows * cols, zero=False)
+        res = self.mallocArray(rows * cols)
         self.lib.lh_trans(x.ptr, res.ptr, rows, cols); _lib.check()
         return res
 
@@ -384,7 +385,7 @@ class BackendHIP(Backend):
         self.lib.lh_trans_grad(xd.ptr, yd.ptr, rows, cols); _lib.check()
 
     def permute(self, x, dims, perm):
-        res = self.mallocArray(int(np.prod(dims, dtype=np.int64)), zero=False)
+        res = self.mallocArray(int(np.prod(dims, dtype=np.int64)))
         self.lib.lh_permute(x.ptr, res.ptr, _ints(dims), _ints(perm), len(dims)); _lib.check()
         return res
 
@@ -394,7 +395,7 @@ class BackendHIP(Backend):
     # -- conv / pool / bn ---------------------------------------------------------------------------
     def conv2D_batch(self, x, w, bias, N, C, H, W, K, R, S, sH, sW, pH, pW):
         P, Q = conv_size(H, R, sH, pH), conv_size(W, S, sW, pW)
-        y = self.mallocArray(N * K * P * Q, zero=False)
+        y = self.mallocArray(N * K * P * Q)
         self.lib.lh_conv2d_fwd(x.ptr, w.ptr, bias.ptr if bias is not None else 0, y.ptr, N, C, H, W, K, R, S, sH, sW, pH, pW); _lib.check()
         if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * P * Q)
         return y, None      # no im2col buffer is kept (BackendCudnn returns None too, CDN:859-866)
@@ -408,15 +409,15 @@ class BackendHIP(Backend):
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
         self.lib.lh_conv2d_fwd_bn_apply(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, scale.ptr, bbias.ptr, sm.ptr, si.ptr,
                                         rmean.ptr, rvar.ptr, eps, factor, 0, ybn.ptr, int(relu)); _lib.check()
-        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW); self._count("bn_fwd_bytes", 8.0 * N * K * HW)    # statistics from the conv epilogue: one read, one write
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def conv2D_batch_grad(self, x, xd, x_in, finput, w, wd, dy, bd, N, C, H, W, K, R, S, sH, sW, pH, pW, beta_dx=1.0):
         # The filter gradient is read by the optimizer only: it goes to the side stream, where it runs beside the
         # rest of the backward pass (x and dy stay untouched until the optimizer joins).  The input gradient, which
         # the next backward operator waits for, is issued first and stays on the main stream.
         so = self.side_order
-        if x_in or self.ops_left < self.side_min_ops:
-            so = 0      # (almost) nothing left to run beside it: the optimizer's join would only add the cross-stream hand-over
+        if x_in or self.convs_open < self.side_min_convs:
+            so = 0      # (almost) nothing left to run beside it (fewer than two convolution gradients follow): the optimizer's join would only add the cross-stream hand-over
         if so == 2:
             self.lib.lh_side_begin()
             self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
@@ -433,7 +434,7 @@ class BackendHIP(Backend):
 
     def maxPool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW, pad):
         P, Q = conv_size(H, kH, sH, pad), conv_size(W, kW, sW, pad)
-        y = self.mallocArray(N * C * P * Q, zero=False); idx = self.mallocArray(N * C * P * Q, zero=False)
+        y = self.mallocArray(N * C * P * Q); idx = self.mallocArray(N * C * P * Q)
         self.lib.lh_maxpool_fwd(x.ptr, y.ptr, idx.ptr, N, C, H, W, kH, kW, sH, sW, pad); _lib.check()
         return y, idx
 
@@ -448,7 +449,7 @@ class BackendHIP(Backend):
 
     def averagePool2D_batch(self, x, N, C, H, W, kH, kW, sH, sW, pH=0, pW=0):
         P, Q = conv_size(H, kH, sH, pH), conv_size(W, kW, sW, pW)
-        y = self.mallocArray(N * C * P * Q, zero=False)
+        y = self.mallocArray(N * C * P * Q)
         if pH or pW: self.lib.lh_avgpool_pad_fwd(x.ptr, y.ptr, N, C, H, W, kH, kW, sH, sW, pH, pW)
         else: self.lib.lh_avgpool_fwd(x.ptr, y.ptr, N, C, H, W, kH, kW, sH, sW)
         _lib.check()
@@ -460,29 +461,19 @@ class BackendHIP(Backend):
         _lib.check()
 
     def batchNormInference(self, x, scale, bias, rmean, rvar, N, C, HW, eps=1e-5):
-        y = self.mallocArray(N * C * HW, zero=False)
+        y = self.mallocArray(N * C * HW)
         self.lib.lh_bn_infer(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, N, C, HW, eps); _lib.check()
         return y
 
-    @staticmethod
-    def _bn_one_pass(N, C, HW):
-        """The library's rule for running a batch norm as one launch with a channel per block (lh_bn.hip: small_fits): the
-        channel's N*HW elements fit one block's registers and there are enough channels for the chip.  The tensor is then
-        read once, not twice (the byte counts below are what the kernels that run must move)."""
-        units = N * (HW // 4) if HW % 4 == 0 else N * HW
-        return units <= 16 * 256 and C >= 128
-
     def batchNormTraining(self, x, scale, bias, rmean, rvar, N, C, HW, eps=1e-5, factor=0.1):
-        y = self.mallocArray(N * C * HW, zero=False)
-        sm = self.mallocArray(C, zero=False); si = self.mallocArray(C, zero=False)
+        y = self.mallocArray(N * C * HW)
+        sm = self.mallocArray(C); si = self.mallocArray(C)
         self.lib.lh_bn_train_fwd(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
-        if self.count_work: self._count("bn_fwd_bytes", (8.0 if self._bn_one_pass(N, C, HW) else 12.0) * N * C * HW)       # x read for the statistics, read again, y written
         return y, sm, si
 
     def batchNormTraining_into(self, x, scale, bias, rmean, rvar, y, sm, si, N, C, HW, relu, eps=1e-5, factor=0.1):
         f = self.lib.lh_bn_train_fwd_relu if relu else self.lib.lh_bn_train_fwd
         f(x.ptr, scale.ptr, bias.ptr, rmean.ptr, rvar.ptr, y.ptr, sm.ptr, si.ptr, N, C, HW, eps, factor); _lib.check()
-        if self.count_work: self._count("bn_fwd_bytes", (8.0 if self._bn_one_pass(N, C, HW) else 12.0) * N * C * HW)
 
     def batchNorm_grad(self, x, xd, dy, scale, scaled, biasd, sm, si, N, C, HW, beta_dx=1.0, y_relu=None, bias=None):
         """y_relu: the layer's output went through a fused in-place relu; `bias` (the layer's beta) lets the
@@ -494,47 +485,35 @@ class BackendHIP(Backend):
         else:
             self.lib.lh_bn_bwd(x.ptr, dy.ptr, scale.ptr, sm.ptr, si.ptr, xdp, beta_dx, scaled.ptr, biasd.ptr, N, C, HW)
         _lib.check()
-        # x and dy read for the two sums, read again, dx written (and read first when it accumulates)
-        if self.count_work: self._count("bn_bwd_bytes", ((12.0 if self._bn_one_pass(N, C, HW) else 20.0) + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0)) * N * C * HW)
 
     def batchNormTraining_add_relu_into(self, x, scale, bias, rmean, rvar, shortcut, out, sm, si, N, C, HW, eps=1e-5, factor=0.1):
         self.lib.lh_bn_stats(x.ptr, sm.ptr, si.ptr, rmean.ptr, rvar.ptr, N, C, HW, eps, factor)
         self.lib.lh_bn_apply_add_relu(x.ptr, scale.ptr, bias.ptr, sm.ptr, si.ptr, shortcut.ptr, out.ptr, N, C, HW); _lib.check()
-        if self.count_work: self._count("bn_fwd_bytes", 16.0 * N * C * HW)       # statistics pass, then x and the shortcut read, out written
 
     def conv2D_batch_bn_add_relu_into(self, x, w, bias, yconv, dims, scale, bbias, rmean, rvar, shortcut, out, sm, si, eps=1e-5, factor=0.1):
         N, C, H, W, K, R, S, sH, sW, pH, pW = dims
         HW = conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW)
         self.lib.lh_conv2d_fwd_bn_apply(x.ptr, w.ptr, bias.ptr if bias is not None else 0, yconv.ptr, *dims, scale.ptr, bbias.ptr, sm.ptr, si.ptr,
                                         rmean.ptr, rvar.ptr, eps, factor, shortcut.ptr, out.ptr, 1); _lib.check()
-        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW); self._count("bn_fwd_bytes", 12.0 * N * K * HW)   # y and the shortcut read, out written
+        if self.count_work: self._count("conv_flop", 2.0 * N * K * C * R * S * HW)
 
     def batchNorm_add_relu_grad(self, x, xd, beta_dx, out, dout, scale, scaled, biasd, sm, si, sd, beta_sd, N, C, HW):
         self.lib.lh_bn_bwd_add_relu(x.ptr, out.ptr, dout.ptr, scale.ptr, sm.ptr, si.ptr, xd.ptr if xd is not None else 0, beta_dx,
                                     sd.ptr if sd is not None else 0, beta_sd, scaled.ptr, biasd.ptr, N, C, HW); _lib.check()
-        # pass 1 reads x, out, dout and writes the masked gradient (to the shortcut's buffer, or over dout); pass 2 reads x and the
-        # masked gradient and writes dx: 28 B per element, plus a read for each output that accumulates
-        if self.count_work:
-            if self._bn_one_pass(N, C, HW):      # x, out, dout read once; the shortcut's gradient and dx written (each read first when it accumulates)
-                self._count("bn_bwd_bytes", (16.0 + (4.0 if sd is not None else 0.0) + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0) + (4.0 if (sd is not None and beta_sd != 0.0) else 0.0)) * N * C * HW)
-            else:
-                self._count("bn_bwd_bytes", (28.0 + (4.0 if (xd is not None and beta_dx != 0.0) else 0.0) + (8.0 if (sd is not None and beta_sd != 0.0) else 0.0)) * N * C * HW)
 
     def add_into(self, a, b, out, n, relu):
         if relu: self.lib.lh_add_relu(a.ptr, b.ptr, out.ptr, n)
         else: self.lib.lh_geam(a.ptr, 1.0, b.ptr, 1.0, out.ptr, n)
         _lib.check()
-        if self.count_work: self._count("elementwise_bytes", 12.0 * n)
 
     def add_relu_grad(self, y, dy, ad, abeta, bd, bbeta, n):
         self.lib.lh_add_relu_grad(y.ptr, dy.ptr, ad.ptr if ad is not None else 0, abeta, bd.ptr if bd is not None else 0, bbeta, n); _lib.check()
-        if self.count_work: self._count("elementwise_bytes", (8.0 + (0 if ad is None else 4.0 + 4.0 * (abeta != 0.0)) + (0 if bd is None else 4.0 + 4.0 * (bbeta != 0.0))) * n)
 
     # -- dropout ------------------------------------------------------------------------------------
     def dropout(self, x, n, prob):
         if not (0.0 <= prob < 1.0):
             raise ValueError("dropout rate should be [0.0, 1), got %s" % prob)
-        y = self.mallocArray(n, zero=False); mask = self.mallocArray(n, zero=False)
+        y = self.mallocArray(n); mask = self.mallocArray(n)
         self.lib.lh_dropout_fwd(x.ptr, y.ptr, mask.ptr, n, prob, self.dropout_seed, self.dropout_offset); _lib.check()
         self.dropout_offset += n
         return y, mask
@@ -546,7 +525,7 @@ class BackendHIP(Backend):
         self.lib.lh_mask4d(x.ptr, lengths.ptr, n, c, d, t); _lib.check()
 
     def repeat0(self, x, rows, context, inner):
-        y = self.mallocArray((rows - context) * (context + 1) * inner, zero=False)
+        y = self.mallocArray((rows - context) * (context + 1) * inner)
         self.lib.lh_repeat0(x.ptr, y.ptr, rows, context, inner); _lib.check()
         return y
 
@@ -559,9 +538,9 @@ class BackendHIP(Backend):
         records = np.ascontiguousarray(records, dtype=np.uint8)
         n = int(records.shape[0])
         assert records.ndim == 2 and records.shape[1] == count + 1, "records must be [n, count + 1] bytes"
-        raw = self.mallocArray((records.nbytes + 3) // 4, zero=False)
-        x = self.mallocArray(n * count, zero=False)
-        y = self.mallocArray(n, zero=False)
+        raw = self.mallocArray((records.nbytes + 3) // 4)
+        x = self.mallocArray(n * count)
+        y = self.mallocArray(n)
         if n:
             self.lib.lh_h2d(raw.ptr, records.ctypes.data, records.nbytes); _lib.check()
             self.lib.lh_cifar_decode(raw.ptr, x.ptr, y.ptr, n, count); _lib.check()
@@ -569,7 +548,7 @@ class BackendHIP(Backend):
 
     # -- activations ---------------------------------------------------------------------------------
     def unary(self, op, x, n, inPlace=False, lo=-1.0, hi=1.0):
-        y = x if inPlace else self.mallocArray(n, zero=False)
+        y = x if inPlace else self.mallocArray(n)
         self.lib.lh_unary(op, x.ptr, y.ptr, n, lo, hi); _lib.check()
         return y
 
@@ -578,7 +557,7 @@ class BackendHIP(Backend):
 
     # -- softmax / loss --------------------------------------------------------------------------------
     def softmax(self, is_log, x, outer, c, inner):
-        y = self.mallocArray(outer * c * inner, zero=False)
+        y = self.mallocArray(outer * c * inner)
         self.lib.lh_softmax(int(is_log), x.ptr, y.ptr, outer, c, inner); _lib.check()
         return y
 
@@ -586,7 +565,7 @@ class BackendHIP(Backend):
         self.lib.lh_softmax_grad(int(is_log), y.ptr, dy.ptr, dx.ptr, outer, c, inner); _lib.check()
 
     def nllLoss(self, x, target, batch, stride):
-        y = self.mallocArray(batch, zero=False)
+        y = self.mallocArray(batch)
         self.lib.lh_nll(x.ptr, target.ptr, y.ptr, batch, stride); _lib.check()
         return y
 
@@ -595,12 +574,12 @@ class BackendHIP(Backend):
 
     # -- reductions -------------------------------------------------------------------------------------
     def sum(self, x, n):
-        y = self.mallocArray(1, zero=False)
+        y = self.mallocArray(1)
         self.lib.lh_sum_all(x.ptr, y.ptr, n); _lib.check()
         return y
 
     def mean(self, x, n):
-        y = self.mallocArray(1, zero=False)
+        y = self.mallocArray(1)
         self.lib.lh_mean_all(x.ptr, y.ptr, n); _lib.check()
         return y
 
@@ -608,7 +587,7 @@ class BackendHIP(Backend):
         self.lib.lh_add_scalar_from(dx.ptr, dy1.ptr, scale, n); _lib.check()
 
     def sum_dim(self, x, outer, dim, inner):
-        y = self.mallocArray(outer * inner, zero=False)
+        y = self.mallocArray(outer * inner)
         self.lib.lh_sum_dim(x.ptr, y.ptr, outer, dim, inner); _lib.check()
         return y
 
@@ -617,7 +596,7 @@ class BackendHIP(Backend):
 
     def concat(self, bufs, sizes, outer, inner):
         total = outer * inner * sum(sizes)
-        res = self.mallocArray(total, zero=False)
+        res = self.mallocArray(total)
         ptrs = (C.c_void_p * len(bufs))(*[b.ptr for b in bufs])
         self.lib.lh_concat(len(bufs), ptrs, _ints(sizes), res.ptr, outer, inner); _lib.check()
         return res
@@ -633,14 +612,14 @@ class BackendHIP(Backend):
     # -- recurrent layer, CTC (CDN:1638-1938) ------------------------------------------------------------
     def ctcLoss(self, probs, probs_d, input_lengths, labels, label_lengths, T, B, A):
         """probs [T,B,A] after softmax; lengths and labels are host int arrays; returns per-sample costs [B]."""
-        costs = self.mallocArray(B, zero=False)
+        costs = self.mallocArray(B)
         il = np.ascontiguousarray(input_lengths, np.int32); lb = np.ascontiguousarray(labels, np.int32); ll = np.ascontiguousarray(label_lengths, np.int32)
         self.lib.lh_ctc_loss(probs.ptr, probs_d.ptr if probs_d is not None else 0, lb.ctypes.data, ll.ctypes.data, il.ctypes.data, costs.ptr, T, B, A)
         _lib.check()
         return costs
 
     def rnn_forward(self, mode, x, w, T, B, I, H, bidir, hx=None):
-        y = self.mallocArray(T * B * H * (2 if bidir else 1), zero=False)
+        y = self.mallocArray(T * B * H * (2 if bidir else 1))
         self.lib.lh_rnn_fwd_init(mode, x.ptr, hx.ptr if hx is not None else 0, w.ptr, y.ptr, T, B, I, H, int(bidir)); _lib.check()
         if self.count_work: self._count("gemm_flop", 2.0 * T * B * H * I * (2 if bidir else 1)); self._count("rnn_flop", 2.0 * T * B * H * H * (2 if bidir else 1))
         return y
@@ -654,8 +633,8 @@ class BackendHIP(Backend):
     def rnn_gated_forward(self, mode, x, w, T, B, I, H, bidir, hx=None, cx=None):
         """LSTM (mode 2) / GRU (mode 3): returns (y, reserve); the reserve goes to rnn_gated_backward, once."""
         D = 2 if bidir else 1
-        y = self.mallocArray(T * B * H * D, zero=False)
-        reserve = self.mallocArray(self.lib.lh_rnn_gated_reserve_floats(mode, T, B, H, int(bidir)), zero=False)
+        y = self.mallocArray(T * B * H * D)
+        reserve = self.mallocArray(self.lib.lh_rnn_gated_reserve_floats(mode, T, B, H, int(bidir)))
         self.lib.lh_rnn_gated_fwd_init(mode, x.ptr, hx.ptr if hx is not None else 0, cx.ptr if cx is not None else 0, w.ptr, y.ptr, reserve.ptr,
                                        T, B, I, H, int(bidir)); _lib.check()
         G = (4 if mode == 2 else 3) * H

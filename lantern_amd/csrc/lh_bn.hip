@@ -645,6 +645,7 @@ void bn_finalize_conv_partials(const float* partial, int C, int ncols, int col1,
 void bn_apply_from_pieces(const float* y, const ConvPieces& pieces, const float* gamma, const float* beta, const float* shortcut, float* out, int relu,
                           int N, int C, int HW) {
   ProfScope prof_(CAT_BN_FWD);
+  work_add(CAT_BN_FWD, (shortcut ? 12.0 : 8.0) * N * C * (double)HW);      // y (and the shortcut) read, out written
   Plan p = make_plan(N, C, HW, (((uintptr_t)y | (uintptr_t)out | (uintptr_t)shortcut) & 15) == 0);
   dim3 grid(C, p.slices);
   const float* none = nullptr;
@@ -660,13 +661,37 @@ void bn_apply_from_pieces(const float* y, const ConvPieces& pieces, const float*
 }
 }  // namespace lh
 
+// What a batch-norm call reads and writes, stated to the deferred-work bookkeeping (lh_defer.hip); launches whatever is parked.
+static void bn_fwd_declare(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                           float* save_mean, float* save_invstd, int N, int C, int HW) {
+  if (!lazy::g_busy || lazy::g_replay) return;
+  const int64_t n = (int64_t)N * C * HW;
+  lazy::flush_parked();
+  lazy::rd_f(x, n); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rw_f(run_mean, C); lazy::rw_f(run_var, C);
+  if (y != x) lazy::wr_f(y, n);
+  lazy::wr_f(save_mean, C); lazy::wr_f(save_invstd, C);
+}
+// returns the beta to run with: 1 on a gradient buffer nobody has touched since lh_malloc becomes 0
+static float bn_bwd_declare(const float* x, const float* y, const float* dy, const float* gamma, const float* bias, const float* save_mean, const float* save_invstd,
+                            float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
+  if (!lazy::g_busy || lazy::g_replay) return beta_dx;
+  const int64_t n = (int64_t)N * C * HW;
+  lazy::flush_parked();
+  lazy::rd_f(x, n); lazy::rd_f(y, n); lazy::rd_f(dy, n); lazy::rd_f(gamma, C); lazy::rd_f(bias, C); lazy::rd_f(save_mean, C); lazy::rd_f(save_invstd, C);
+  if (dx && (beta_dx == 0.f || beta_dx == 1.f)) beta_dx = lazy::beta_f(dx, n, beta_dx);
+  lazy::rw_f(dgamma, C); lazy::rw_f(dbeta, C);
+  return beta_dx;
+}
+
 extern "C" {
 
 void lh_bn_stats(const float* x, float* save_mean, float* save_invstd, float* run_mean, float* run_var, int N, int C, int HW, float eps, float factor) {
-  ProfScope prof_(CAT_BN_FWD);
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_stats: empty shape [%d,%d,%d]", N, C, HW);
+  LZ_ENTER(); lazy::rd_f(x, (int64_t)N * C * HW); lazy::wr_f(save_mean, C); lazy::wr_f(save_invstd, C); lazy::rw_f(run_mean, C); lazy::rw_f(run_var, C);
+  ProfScope prof_(CAT_BN_FWD);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_stats: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   if (!get_partial()) return;
+  work_add(CAT_BN_FWD, 4.0 * N * C * (double)HW);
   Plan p = make_plan(N, C, HW, ((uintptr_t)x & 15) == 0);
   dim3 grid(C, p.slices);
   if (p.vec4) hipLaunchKernelGGL((k_bn_stats<true>), grid, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, HW, p.n_per);
@@ -678,8 +703,11 @@ void lh_bn_stats(const float* x, float* save_mean, float* save_invstd, float* ru
 
 void lh_bn_apply(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd, float* y,
                  int N, int C, int HW, int relu) {
-  ProfScope prof_(CAT_BN_FWD);
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_apply: empty shape [%d,%d,%d]", N, C, HW);
+  LZ_ENTER(); lazy::rd_f(x, (int64_t)N * C * HW); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rd_f(save_mean, C); lazy::rd_f(save_invstd, C);
+  if (y != x) lazy::wr_f(y, (int64_t)N * C * HW);
+  ProfScope prof_(CAT_BN_FWD);
+  work_add(CAT_BN_FWD, 8.0 * N * C * (double)HW);
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)y) & 15) == 0);
   dim3 grid(C, p.slices);
 #define GO(V, R) hipLaunchKernelGGL((k_bn_apply<V, R>), grid, dim3(TPB), 0, g_stream, x, y, gamma, beta, save_mean, save_invstd, N, C, HW, p.n_per)
@@ -691,9 +719,12 @@ void lh_bn_apply(const float* x, const float* gamma, const float* beta, const fl
 
 void lh_bn_infer(const float* x, const float* gamma, const float* beta, const float* run_mean, const float* run_var,
                  float* y, int N, int C, int HW, float eps) {
-  ProfScope prof_(CAT_BN_FWD);
   int64_t n = (int64_t)N * C * HW;
   if (n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(x, n); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rd_f(run_mean, C); lazy::rd_f(run_var, C);
+  if (y != x) lazy::wr_f(y, n);
+  ProfScope prof_(CAT_BN_FWD);
+  work_add(CAT_BN_FWD, 8.0 * (double)n);
   hipLaunchKernelGGL(k_bn_infer, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, gamma, beta, run_mean, run_var, C, HW, n, eps);
   LH_CHECK_LAUNCH();
 }
@@ -704,6 +735,7 @@ static void bn_train_fwd_impl(bool relu, const float* x, const float* gamma, con
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_train_fwd: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   if (!get_partial()) return;
   if (HW == 1 && !relu && C >= 32) {          // rows of channels: the column kernels
+    work_add(CAT_BN_FWD, 12.0 * N * (double)C);
     const Plan1 p1 = make_plan1(N, C);
     dim3 g1((unsigned)cdiv(C, C1), p1.slices);
     hipLaunchKernelGGL(k_bn1d_stats, g1, dim3(TPB), 0, g_stream, x, g_partial_ptr, N, C, p1.rows_per);
@@ -713,6 +745,7 @@ static void bn_train_fwd_impl(bool relu, const float* x, const float* gamma, con
     return;
   }
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)y) & 15) == 0);
+  work_add(CAT_BN_FWD, ((C >= 128 && small_fits(N, HW, p.vec4)) ? 8.0 : 12.0) * N * C * (double)HW);    // x read once (twice: statistics pass, then the apply pass), y written
   if (C >= 128 && small_fits(N, HW, p.vec4)) {          // a channel per block, one launch (given enough channels to occupy the chip)
 #define SMALL(V, R) hipLaunchKernelGGL((k_bn_small_fwd<V, R>), dim3(C), dim3(TPB), 0, g_stream, x, y, gamma, beta, run_mean, run_var, save_mean, save_invstd, N, C, HW, eps, factor)
     if (p.vec4) { if (relu) SMALL(true, true); else SMALL(true, false); }
@@ -743,6 +776,7 @@ static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, co
   LH_REQUIRE(beta_dx == 0.0f || beta_dx == 1.0f, "lh_bn_bwd: beta must be 0 or 1");
   if (!get_partial()) return;
   if (HW == 1 && relu == 0 && C >= 32) {
+    work_add(CAT_BN_BWD, (20.0 + (beta_dx != 0.0f ? 4.0 : 0.0)) * N * (double)C);
     const Plan1 p1 = make_plan1(N, C);
     dim3 g1((unsigned)cdiv(C, C1), p1.slices);
     hipLaunchKernelGGL(k_bn1d_bwd_stats, g1, dim3(TPB), 0, g_stream, x, dy, save_mean, save_invstd, g_partial_ptr, N, C, p1.rows_per);
@@ -753,6 +787,12 @@ static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, co
   }
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx | (uintptr_t)y_relu) & 15) == 0);
   const bool acc = beta_dx != 0.0f;
+  {
+    // x and dy (and y, when the relu mask is read from it) read once, or twice with the statistics pass; dx written, and read first when it accumulates
+    const bool one = C >= 128 && small_fits(N, HW, p.vec4);
+    const double per = (one ? 8.0 : 16.0) + (relu == 1 ? (one ? 4.0 : 8.0) : 0.0) + (dx ? 4.0 + (acc ? 4.0 : 0.0) : 0.0);
+    work_add(CAT_BN_BWD, per * N * C * (double)HW);
+  }
   if (C >= 128 && small_fits(N, HW, p.vec4)) {          // a channel per block, one launch
 #define SMALL(V, A, R) hipLaunchKernelGGL((k_bn_small_bwd<V, A, R>), dim3(C), dim3(TPB), 0, g_stream, x, y_relu, dy, gamma, bias, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW)
 #define SMALL_R(V, A) do { if (relu == 2) SMALL(V, A, 2); else if (relu == 1) SMALL(V, A, 1); else SMALL(V, A, 0); } while (0)
@@ -778,31 +818,47 @@ static void bn_bwd_impl(const float* x, const float* y_relu, const float* dy, co
 
 void lh_bn_train_fwd(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
                      float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
+  LZ_SCOPE();
+  // waits for the call behind it: relu in place or the residual join fuse with it; right behind a parked convolution the
+  // statistics come from that convolution's epilogue
+  if (lazy::park_bn_train_fwd(x, gamma, beta, run_mean, run_var, y, save_mean, save_invstd, N, C, HW, eps, factor)) return;
+  bn_fwd_declare(x, gamma, beta, run_mean, run_var, y, save_mean, save_invstd, N, C, HW);
   ProfScope prof_(CAT_BN_FWD);
   bn_train_fwd_impl(false, x, gamma, beta, run_mean, run_var, y, save_mean, save_invstd, N, C, HW, eps, factor);
 }
 void lh_bn_train_fwd_relu(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
                           float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor) {
+  LZ_SCOPE();
+  bn_fwd_declare(x, gamma, beta, run_mean, run_var, y, save_mean, save_invstd, N, C, HW);
   ProfScope prof_(CAT_BN_FWD);
   bn_train_fwd_impl(true, x, gamma, beta, run_mean, run_var, y, save_mean, save_invstd, N, C, HW, eps, factor);
 }
 void lh_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
+  LZ_SCOPE();
+  // right behind a parked relu_grad (and the gradient of a `+`): one fused backward instead of two or three passes
+  if (lazy::g_busy && !lazy::g_replay && lazy::take_bn_bwd(x, dy, gamma, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW)) return;
+  beta_dx = bn_bwd_declare(x, nullptr, dy, gamma, nullptr, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
   ProfScope prof_(CAT_BN_BWD);
   bn_bwd_impl(x, nullptr, dy, gamma, nullptr, 0, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
 }
 void lh_bn_bwd_relu(const float* x, const float* y, const float* dy, const float* gamma, const float* bias, const float* save_mean, const float* save_invstd,
                     float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW) {
-  ProfScope prof_(CAT_BN_BWD);
   LH_REQUIRE(y != nullptr || bias != nullptr, "lh_bn_bwd_relu: y or the layer's bias is required");
+  LZ_SCOPE();
+  beta_dx = bn_bwd_declare(x, bias ? nullptr : y, dy, gamma, bias, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
+  ProfScope prof_(CAT_BN_BWD);
   bn_bwd_impl(x, bias ? nullptr : y, dy, gamma, bias, bias ? 2 : 1, save_mean, save_invstd, dx, beta_dx, dgamma, dbeta, N, C, HW);
 }
 
 void lh_bn_apply_add_relu(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd,
                           const float* shortcut, float* out, int N, int C, int HW) {
-  ProfScope prof_(CAT_BN_FWD);
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_apply_add_relu: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(x && shortcut && out && gamma && beta && save_mean && save_invstd, "lh_bn_apply_add_relu: null operand");
+  LZ_ENTER(); lazy::rd_f(x, (int64_t)N * C * HW); lazy::rd_f(shortcut, (int64_t)N * C * HW); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rd_f(save_mean, C); lazy::rd_f(save_invstd, C);
+  if (out != x && out != shortcut) lazy::wr_f(out, (int64_t)N * C * HW);
+  ProfScope prof_(CAT_BN_FWD);
+  work_add(CAT_BN_FWD, 12.0 * N * C * (double)HW);
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)out | (uintptr_t)shortcut) & 15) == 0);
   dim3 grid(C, p.slices);
   if (p.vec4) hipLaunchKernelGGL((k_bn_apply_add_relu<true>), grid, dim3(TPB), 0, g_stream, x, shortcut, out, gamma, beta, save_mean, save_invstd, N, C, HW, p.n_per);
@@ -812,8 +868,17 @@ void lh_bn_apply_add_relu(const float* x, const float* gamma, const float* beta,
 
 void lh_bn_bwd_add_relu(const float* x, const float* out, float* dout, const float* gamma, const float* save_mean, const float* save_invstd,
                         float* dx, float beta_dx, float* ds, float beta_ds, float* dgamma, float* dbeta, int N, int C, int HW) {
-  ProfScope prof_(CAT_BN_BWD);
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_bwd_add_relu: empty shape [%d,%d,%d]", N, C, HW);
+  LZ_SCOPE();
+  if (lazy::g_busy && !lazy::g_replay) {
+    const int64_t n = (int64_t)N * C * HW;
+    lazy::flush_parked();
+    lazy::rd_f(x, n); lazy::rd_f(out, n); lazy::rw_f(dout, n); lazy::rd_f(gamma, C); lazy::rd_f(save_mean, C); lazy::rd_f(save_invstd, C);
+    if (dx && (beta_dx == 0.f || beta_dx == 1.f)) beta_dx = lazy::beta_f(dx, n, beta_dx);
+    if (ds && (beta_ds == 0.f || beta_ds == 1.f)) beta_ds = lazy::beta_f(ds, n, beta_ds);
+    lazy::rw_f(dgamma, C); lazy::rw_f(dbeta, C);
+  }
+  ProfScope prof_(CAT_BN_BWD);
   LH_REQUIRE(C <= MAX_PARTIALS, "lh_bn_bwd_add_relu: %d channels exceed the scratch (%d)", C, MAX_PARTIALS);
   LH_REQUIRE((beta_dx == 0.0f || beta_dx == 1.0f) && (beta_ds == 0.0f || beta_ds == 1.0f), "lh_bn_bwd_add_relu: beta must be 0 or 1");
   LH_REQUIRE(x && out && dout && gamma && save_mean && save_invstd, "lh_bn_bwd_add_relu: null operand");
@@ -821,6 +886,14 @@ void lh_bn_bwd_add_relu(const float* x, const float* out, float* dout, const flo
   LH_REQUIRE(dx == nullptr || dx != ds, "lh_bn_bwd_add_relu: dx and ds are the same buffer (a batch norm whose input is also the shortcut): the first pass would add into what the second overwrites; run lh_add_relu_grad and lh_bn_bwd instead");
   if (!get_partial()) return;
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)out | (uintptr_t)dout | (uintptr_t)dx | (uintptr_t)ds) & 15) == 0);
+  {
+    // one launch: x, out, dout read once; two passes: pass 1 reads x, out, dout and writes the masked gradient (to the shortcut's
+    // buffer, or over dout), pass 2 reads x and the masked gradient; dx and ds written, each read first when it accumulates
+    const bool one = C >= 128 && small_fits(N, HW, p.vec4);
+    const double per = one ? 12.0 + (ds ? 4.0 + (beta_ds != 0.0f ? 4.0 : 0.0) : 0.0) + (dx ? 4.0 + (beta_dx != 0.0f ? 4.0 : 0.0) : 0.0)
+                           : 24.0 + (ds && beta_ds != 0.0f ? 8.0 : 0.0) + (dx ? 4.0 + (beta_dx != 0.0f ? 4.0 : 0.0) : 0.0);
+    work_add(CAT_BN_BWD, per * N * C * (double)HW);
+  }
   if (C >= 128 && small_fits(N, HW, p.vec4)) {          // a channel per block, one launch; dout is left as it is
     const int dsm = ds == nullptr ? 0 : (beta_ds != 0.0f ? 2 : 1);
 #define SMALL(V, A, D) hipLaunchKernelGGL((k_bn_small_bwd_join<V, A, D>), dim3(C), dim3(TPB), 0, g_stream, x, out, (const float*)dout, ds, gamma, save_mean, save_invstd, dx, dgamma, dbeta, N, C, HW)

@@ -1086,6 +1086,7 @@ void lh_cmdlist_begin(void) {
   LH_REQUIRE(g_stream_raw != nullptr, "lh_cmdlist_begin before lh_setup");
   LH_REQUIRE(!g_capturing, "lh_cmdlist_begin: a graph is being recorded (the command buffers cannot be replayed)");
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_cmdlist_begin on the side stream");
+  { LZ_SCOPE(); lazy::flush_all(); }     // recorded commands do not pass through the deferred-work bookkeeping: it starts empty and stays empty while recording
   if (!ring_init()) return;
   if (g_win == nullptr) { g_win = new Window(); for (int i = 0; i < HASH_N; i++) g_win->slot[i].epoch = 0; for (int i = 0; i < PAGE_N; i++) g_win->page[i].epoch = 0; g_win->epoch = 0; window_reset(*g_win); }
   g_rec_on = 1;

@@ -20,7 +20,20 @@ void rec_flush();
 void cmdlist_release();           // frees the command buffers (lh_cleanup)
 bool multi_tensor_setup();        // the multi-tensor optimizers' device table: reserved by lh_setup, freed by lh_cleanup
 void multi_tensor_release();
-static inline hipStream_t ordered_stream() { if (g_rec_pending) rec_flush(); return g_stream_cur; }
+// Deferred work (lh_defer.hip): launches parked until the next call shows whether it fuses with them, zero fills of arena
+// blocks nobody has touched yet, and results of fused launches that the program could read but no kernel has written.
+// An entry point that states what it reads and writes (lazy::Scope + rd / wr / acc / rw below) is served exactly; any
+// other entry point reaches ordered_stream() at depth 0, which first brings everything deferred up to date.
+namespace lazy {
+extern bool g_busy;               // something is parked, pending or unwritten
+extern int g_depth;               // > 0 inside an entry point that declares its operands, and while deferred work is launched
+void flush_undeclared();
+}
+static inline hipStream_t ordered_stream() {
+  if (g_rec_pending) rec_flush();
+  if (lazy::g_busy && lazy::g_depth == 0) lazy::flush_undeclared();
+  return g_stream_cur;
+}
 #define g_stream (::lh::ordered_stream())     // every kernel is enqueued here
 extern int g_error_mode;         // 0 = print and exit, 1 = record and return
 extern int g_num_cu;             // compute units of the device in use
@@ -80,6 +93,11 @@ struct ProfScope {
   ~ProfScope() { if (on) prof_end(cat); }
 };
 
+// Algorithmic bytes of the HBM-bound kernels launched, per category (lh_work_collect): the kernels that run are chosen here
+// (fused or not, one pass or two), so the byte counts a roofline figure needs are kept here too.
+extern double g_work[CAT_COUNT];
+static inline void work_add(int cat, double bytes) { g_work[cat] += bytes; }
+
 // Category the matrix kernels launched below an entry point are timed under: the events then bracket the
 // k_igemm launch itself, not the small layout / fill kernels around it.
 extern int g_kernel_cat;
@@ -102,6 +120,58 @@ void bn_apply_from_pieces(const float* y, const ConvPieces& pieces, const float*
                           int N, int C, int HW);
 
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- deferred work: declarations an entry point makes about its operands (all sizes in bytes) -----------------------------
+namespace lazy {
+extern bool g_enabled;            // lh_set_fusion (LH_NO_FUSION in the environment): off = every call runs as issued, lh_malloc clears at once
+extern bool g_replay;             // deferred work is being launched: entry points run as called and declare nothing
+struct Scope { Scope() { g_depth++; } ~Scope() { g_depth--; } };
+static inline bool active() { return g_enabled && !g_replay; }
+void flush_parked();                               // launch what is parked (unfused)
+void flush_all();                                  // parked launches, pending zero fills and unwritten results: all brought up to date
+void rd(const void* p, size_t bytes);              // the range is about to be read
+void wr(const void* p, size_t bytes);              // the range is about to be overwritten as a whole
+bool acc(const void* p, size_t bytes);             // the range is about to be added into; true: it is a zero block nobody has cleared or touched, so overwrite it instead
+void rw(const void* p, size_t bytes);              // read and written in place
+static inline void rd_f(const void* p, int64_t n) { if (g_busy && p && n > 0) rd(p, (size_t)n * 4); }
+static inline void wr_f(const void* p, int64_t n) { if (g_busy && p && n > 0) wr(p, (size_t)n * 4); }
+static inline void rw_f(const void* p, int64_t n) { if (g_busy && p && n > 0) rw(p, (size_t)n * 4); }
+static inline bool acc_f(const void* p, int64_t n) { return g_busy && p && n > 0 ? acc(p, (size_t)n * 4) : false; }
+// accumulate with a beta the caller passed: 1 on a block nobody has touched becomes 0; 0 is a plain overwrite
+static inline float beta_f(const void* p, int64_t n, float beta) {
+  if (!g_busy || !p || n <= 0) return beta;
+  if (beta == 0.f) { wr(p, (size_t)n * 4); return 0.f; }
+  return acc(p, (size_t)n * 4) && beta == 1.f ? 0.f : beta;
+}
+// arena bookkeeping (lh_runtime.hip)
+void note_zero_block(void* p, size_t bytes);       // lh_malloc handed out [p, p + bytes) without clearing it
+void arena_released(char* from);                   // the arena above `from` is released (rewind, pop): nothing there can be read again
+bool defer_zero();                                 // lh_malloc may hand out large blocks uncleared now
+// parking; each returns true when the call has been taken over (parked or fused) and the entry point has nothing left to do
+bool park_conv_fwd(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
+bool park_bn_train_fwd(const float* x, const float* gamma, const float* beta, float* run_mean, float* run_var, float* y,
+                       float* save_mean, float* save_invstd, int N, int C, int HW, float eps, float factor);
+bool park_add(const float* a, const float* b, float* out, int64_t n);
+bool take_relu_inplace(float* y, int64_t n);
+bool park_relu_grad_inplace(const float* y, float* d, int64_t n);
+bool park_add_grad(float* ad, float* bd, const float* outd, int64_t n);
+bool take_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
+                 float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
+bool gather_update(int mode, float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n);
+void forget_forward_records();                     // parameters are about to change: what the backward pass would recompute from them is no longer valid
+void on_rewind(char* new_top);
+void reset();                                      // forget everything deferred without launching anything (lh_setup, lh_cleanup)
+}
+// An entry point that declares its operands opens with LZ_ENTER(): from here to its end nothing is brought up to date behind
+// its back, and whatever was parked (and is not continued by this call) is launched first.
+#define LZ_SCOPE() ::lh::lazy::Scope lz_scope_
+#define LZ_ENTER() ::lh::lazy::Scope lz_scope_; do { if (::lh::lazy::g_busy && !::lh::lazy::g_replay) ::lh::lazy::flush_parked(); } while (0)
+// kernels the deferred work needs from other files
+void mask_relu(float* dst, const float* src, const float* y, int64_t n);                     // dst = y > 0 ? src : 0
+void add_plain(const float* a, const float* b, float* out, int64_t n);
+void relu_grad_inplace_now(const float* y, float* d, int64_t n);
+void multi_update_now(int mode, int count, float* const* hx, float* const* hd, float* const* hv, const int64_t* hn, float lr, float mu, float clip, int nesterov);
+void zero_bytes_async(void* p, size_t bytes);      // bytes a multiple of 256
 
 // ---- command list: small operations recorded on the host and executed in order by one workgroup -------------
 // While recording is on (lh_cmdlist_begin), an entry point whose operands are small enough appends a command instead

@@ -613,8 +613,21 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
 
 extern "C" {
 
+// What a forward convolution reads and writes, stated to the deferred-work bookkeeping; launches whatever is parked.
+static void conv_fwd_declare(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
+  if (!lazy::g_busy || lazy::g_replay) return;
+  lazy::flush_parked();
+  ConvDims d;
+  if (!make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW)) return;
+  lazy::rd_f(x, (int64_t)N * C * H * W); lazy::rd_f(w, (int64_t)K * C * R * S); lazy::rd_f(bias, K); lazy::wr_f(y, (int64_t)N * K * d.P * d.Q);
+}
+
 void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
                    int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
+  LZ_SCOPE();
+  // waits for the call behind it: a batch norm of y takes its statistics from this launch's epilogue
+  if (lazy::park_conv_fwd(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW)) return;
+  conv_fwd_declare(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW);
   conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, nullptr);
 }
 
@@ -622,6 +635,9 @@ void lh_conv2d_fwd_bnstats(const float* x, const float* w, const float* bias, fl
                            int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW,
                            float* save_mean, float* save_invstd, float* run_mean, float* run_var, float eps, float factor) {
   LH_REQUIRE(save_mean && save_invstd, "lh_conv2d_fwd_bnstats: save_mean and save_invstd are required");
+  LZ_SCOPE();
+  conv_fwd_declare(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW);
+  lazy::wr_f(save_mean, K); lazy::wr_f(save_invstd, K); lazy::rw_f(run_mean, K); lazy::rw_f(run_var, K);
   BnStatsOut bn{save_mean, save_invstd, run_mean, run_var, eps, factor};
   conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, &bn);
 }
@@ -632,6 +648,16 @@ void lh_conv2d_fwd_bn_apply(const float* x, const float* w, const float* bias, f
                             float eps, float factor, const float* shortcut, float* out, int relu) {
   LH_REQUIRE(save_mean && save_invstd && gamma && beta && out, "lh_conv2d_fwd_bn_apply: gamma, beta, save_mean, save_invstd and out are required");
   LH_REQUIRE(shortcut == nullptr || relu, "lh_conv2d_fwd_bn_apply: the residual join is relu(bn(y) + shortcut)");
+  LZ_SCOPE();
+  conv_fwd_declare(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW);
+  if (lazy::g_busy && !lazy::g_replay) {
+    ConvDims dd;
+    if (make_dims(dd, N, C, H, W, K, R, S, sH, sW, pH, pW)) {
+      const int64_t no = (int64_t)N * K * dd.P * dd.Q;
+      lazy::rd_f(gamma, K); lazy::rd_f(beta, K); lazy::rd_f(shortcut, no); lazy::wr_f(save_mean, K); lazy::wr_f(save_invstd, K);
+      lazy::rw_f(run_mean, K); lazy::rw_f(run_var, K); lazy::wr_f(out, no);
+    }
+  }
   BnStatsOut bn{save_mean, save_invstd, run_mean, run_var, eps, factor};
   bn.gamma = gamma; bn.beta = beta; bn.shortcut = shortcut; bn.out = out; bn.relu = relu;
   conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, &bn);
@@ -648,6 +674,9 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_data: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_data: beta must be 0 or 1");
+  LZ_ENTER();
+  lazy::rd_f(dy, (int64_t)N * K * d.P * d.Q); lazy::rd_f(w, (int64_t)K * C * R * S);
+  beta = lazy::beta_f(dx, (int64_t)N * C * H * W, beta);       // a gradient buffer nobody has touched since lh_malloc is overwritten, not read
   const int RS = R * S, KRS = K * RS, HW = H * W, PQ = d.P * d.Q;
   const uint32_t dybytes = (uint32_t)((size_t)N * K * PQ * 4);
   bool ok = true;
@@ -801,6 +830,10 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_filter: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_filter: beta must be 0 or 1");
+  LZ_ENTER();
+  lazy::rd_f(x, (int64_t)N * C * H * W); lazy::rd_f(dy, (int64_t)N * K * d.P * d.Q);
+  beta = lazy::beta_f(dw, (int64_t)K * C * R * S, beta);
+  lazy::rw_f(db, K);
   // A filter gradient issued in line must not overtake one of the same filter that is still on the side stream.
   if (g_stream_cur == g_stream_raw) side_join();
   const int CRS = C * R * S, PQ = d.P * d.Q;

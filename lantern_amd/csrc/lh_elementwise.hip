@@ -68,6 +68,7 @@ __global__ void __launch_bounds__(TPB) k_add_relu_grad2(const float* __restrict_
 template <int NIN, class F>
 void ew(float* out, const float* a, const float* b, const float* c, int64_t n, F f) {
   if (n <= 0) return;
+  work_add(CAT_ELEMENTWISE, 4.0 * (NIN + 1) * (double)n);
   bool vec = al16(out) && al16(a) && (NIN < 2 || al16(b)) && (NIN < 3 || al16(c));
   int grid = stream_grid(n, TPB * 8);
   if (vec) hipLaunchKernelGGL((k_ew_vec<NIN, F>), dim3(grid), dim3(TPB), 0, g_stream, out, a, b, c, n, f);
@@ -130,7 +131,7 @@ __global__ void k_repeat0_grad(float* __restrict__ ind, const float* __restrict_
 
 extern "C" {
 
-void lh_fill(float* x, float v, int64_t n) { ProfScope prof_(CAT_FILL);
+void lh_fill(float* x, float v, int64_t n) { LZ_ENTER(); lazy::wr_f(x, n); ProfScope prof_(CAT_FILL);
   if (n > 0 && rec_ok(n)) { rec_cmd(CL_FILL, (int)n, 0, 0, v, 0.f, 0.f, 0.f, x, nullptr, nullptr, nullptr); return; }
   if (n <= 0) return;
   if (al16(x)) hipLaunchKernelGGL(k_fill, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, v, n);
@@ -141,11 +142,13 @@ void lh_fill(float* x, float v, int64_t n) { ProfScope prof_(CAT_FILL);
 void lh_fill_with_bias(float* y, const float* bias, int64_t outer, int64_t c, int64_t inner) {
   int64_t n = outer * c * inner;
   if (n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(bias, c); lazy::wr_f(y, n);
   hipLaunchKernelGGL(k_fill_bias, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, y, bias, c, inner, n);
   LH_CHECK_LAUNCH();
 }
 
 void lh_clip(float* x, float bound, int64_t n) {
+  LZ_ENTER(); lazy::rw_f(x, n);
   side_join();      // clips gradients, which may still be in flight on the side stream
   ew<1>(x, x, nullptr, nullptr, n, [bound] __device__(float v, float, float) { return v > bound ? bound : (v < -bound ? -bound : v); });
   LH_CHECK_LAUNCH();
@@ -162,6 +165,7 @@ __global__ void k_mask4d(float* x, const int* lengths, int64_t n, int cd, int t)
 void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t) {
   int64_t tot = (int64_t)n * c * d * t;
   if (tot <= 0) return;
+  LZ_ENTER(); lazy::rd_f(lengths, n); lazy::rw_f(x, tot);
   hipLaunchKernelGGL(k_mask4d, dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, x, lengths, tot, c * d, t);
   LH_CHECK_LAUNCH();
 }
@@ -169,12 +173,14 @@ void lh_mask4d(float* x, const int* lengths, int n, int c, int d, int t) {
 void lh_repeat0(const float* in, float* out, int rows, int context, int64_t inner) {
   if (rows < 1 || context < 0 || context >= rows || inner < 1) { LH_FAIL("lh_repeat0: rows %d, context %d, inner %lld", rows, context, (long long)inner); return; }
   const int64_t n_out = (int64_t)(rows - context) * (context + 1) * inner;
+  LZ_ENTER(); lazy::rd_f(in, (int64_t)rows * inner); lazy::wr_f(out, n_out);
   hipLaunchKernelGGL(k_repeat0, dim3(stream_grid(n_out, TPB * 4)), dim3(TPB), 0, g_stream, in, out, context + 1, inner, n_out);
   LH_CHECK_LAUNCH();
 }
 void lh_repeat0_grad(float* ind, const float* outd, int rows, int context, int64_t inner) {
   if (rows < 1 || context < 0 || context >= rows || inner < 1) { LH_FAIL("lh_repeat0_grad: rows %d, context %d, inner %lld", rows, context, (long long)inner); return; }
   const int64_t n_in = (int64_t)rows * inner;
+  LZ_ENTER(); lazy::rd_f(outd, (int64_t)(rows - context) * (context + 1) * inner); lazy::rw_f(ind, n_in);
   hipLaunchKernelGGL(k_repeat0_grad, dim3(stream_grid(n_in, TPB * 2)), dim3(TPB), 0, g_stream, ind, outd, context + 1, (int64_t)(rows - context), inner, n_in);
   LH_CHECK_LAUNCH();
 }
@@ -191,7 +197,12 @@ void lh_cifar_decode(const unsigned char* records, float* x, int* y, int n, int 
   LH_CHECK_LAUNCH();
 }
 
-void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) {
+  LZ_SCOPE();
+  // relu in place behind a parked batch norm, residual join or `+`: the chain runs as its fused kernel
+  if (op == LH_RELU && x == y && lazy::g_busy && !lazy::g_replay && lazy::take_relu_inplace(y, n)) return;
+  if (lazy::g_busy && !lazy::g_replay) { lazy::flush_parked(); if (x == y) lazy::rw_f(y, n); else { lazy::rd_f(x, n); lazy::wr_f(y, n); } }
+  ProfScope prof_(CAT_ELEMENTWISE);
   if (n > 0 && op >= LH_RELU && op <= LH_HARDTANH && rec_ok(n)) { rec_cmd(CL_UNARY, (int)n, op, 0, lo, hi, 0.f, 0.f, y, x, nullptr, nullptr); return; }
   switch (op) {
     case LH_RELU: ew<1>(y, x, nullptr, nullptr, n, [] __device__(float v, float, float) { return v < 0.f ? 0.f : v; }); break;
@@ -207,12 +218,27 @@ void lh_unary(int op, const float* x, float* y, int64_t n, float lo, float hi) {
   LH_CHECK_LAUNCH();
 }
 
-void lh_unary_grad(int op, const float* x, const float* y, const float* dy, float* dx, int64_t n, int inplace, float lo, float hi) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_unary_grad(int op, const float* x, const float* y, const float* dy, float* dx, int64_t n, int inplace, float lo, float hi) {
+  LZ_SCOPE();
+  // relu_grad in place waits for the call behind it: a batch-norm gradient (or `+`'s gradient, then a batch norm's) takes the mask along
+  if (op == LH_RELU && inplace && dy == dx && lazy::park_relu_grad_inplace(y, dx, n)) return;
+  bool fresh = false;
+  if (lazy::g_busy && !lazy::g_replay) {
+    lazy::flush_parked();
+    if (inplace) { lazy::rd_f(y, n); lazy::rw_f(dx, n); }
+    else {
+      if (op == LH_RELU || op == LH_HARDTANH || op == LH_LOG || op == LH_SQUARE) lazy::rd_f(x, n); else lazy::rd_f(y, n);
+      lazy::rd_f(dy, n);
+      if (op == LH_RELU) fresh = lazy::acc_f(dx, n); else lazy::rw_f(dx, n);
+    }
+  }
+  ProfScope prof_(CAT_ELEMENTWISE);
   if (n > 0 && op >= LH_RELU && op <= LH_HARDTANH && rec_ok(n)) { rec_cmd(CL_UNARY_GRAD, (int)n, op, inplace ? 1 : 0, lo, hi, 0.f, 0.f, dx, x, y, dy); return; }
   // out = dx; inputs (a, b, c) chosen per op.  All forms are dx (+)= g(x|y, dy).
   switch (op) {
     case LH_RELU:
       if (inplace) ew<2>(dx, dx, y, nullptr, n, [] __device__(float d, float yv, float) { return yv > 0.f ? d : 0.f; });
+      else if (fresh) ew<2>(dx, x, dy, nullptr, n, [] __device__(float xv, float g, float) { return 0.f + (xv < 0.f ? 0.f : g); });     // dx is an untouched zero block
       else ew<3>(dx, dx, x, dy, n, [] __device__(float d, float xv, float g) { return d + (xv < 0.f ? 0.f : g); });
       break;
     case LH_HARDTANH:
@@ -230,23 +256,32 @@ void lh_unary_grad(int op, const float* x, const float* y, const float* dy, floa
   LH_CHECK_LAUNCH();
 }
 
-void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) {
+  LZ_ENTER(); if (x == y) lazy::rw_f(y, n); else { lazy::rd_f(x, n); lazy::wr_f(y, n); }
+  ProfScope prof_(CAT_ELEMENTWISE);
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_scalar_op: unknown op %d", op);
   if (n > 0 && rec_ok(n)) { rec_cmd(CL_SCALAR, (int)n, op, 0, s, 0.f, 0.f, 0.f, y, x, nullptr, nullptr); return; }
   ew<1>(y, x, nullptr, nullptr, n, [op, s] __device__(float v, float, float) { return bop(op, v, s); });
   LH_CHECK_LAUNCH();
 }
 
-void lh_add_relu(const float* a, const float* b, float* out, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_add_relu(const float* a, const float* b, float* out, int64_t n) {
+  LZ_ENTER(); lazy::rd_f(a, n); lazy::rd_f(b, n); if (out != a && out != b) lazy::wr_f(out, n);
+  ProfScope prof_(CAT_ELEMENTWISE);
   ew<2>(out, a, b, nullptr, n, [] __device__(float x, float y, float) { float r = x + y; return r < 0.f ? 0.f : r; });
   LH_CHECK_LAUNCH();
 }
-void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, float* bd, float bbeta, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, float* bd, float bbeta, int64_t n) {
   // g = dy where y > 0 else 0 ; ad = abeta*ad + g ; bd = bbeta*bd + g   (either target may be NULL)
   if (n <= 0) return;
   LH_REQUIRE((abeta == 0.f || abeta == 1.f) && (bbeta == 0.f || bbeta == 1.f), "lh_add_relu_grad: beta must be 0 or 1");
+  LZ_ENTER(); lazy::rd_f(y, n); lazy::rd_f(dy, n);
+  if (ad) abeta = lazy::beta_f(ad, n, abeta);
+  if (bd && bd != ad) bbeta = lazy::beta_f(bd, n, bbeta);
+  ProfScope prof_(CAT_ELEMENTWISE);
   if (ad && bd && ad != bd && al16(y) && al16(dy) && al16(ad) && al16(bd)) {
     const int grid = stream_grid(n, TPB * 8);
+    work_add(CAT_ELEMENTWISE, (16.0 + (abeta != 0.f ? 4.0 : 0.0) + (bbeta != 0.f ? 4.0 : 0.0)) * (double)n);
 #define GO(A, B) hipLaunchKernelGGL((k_add_relu_grad2<A, B>), dim3(grid), dim3(TPB), 0, g_stream, y, dy, ad, bd, n)
     if (abeta != 0.f) { if (bbeta != 0.f) GO(true, true); else GO(true, false); }
     else { if (bbeta != 0.f) GO(false, true); else GO(false, false); }
@@ -265,7 +300,9 @@ void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, f
   LH_CHECK_LAUNCH();
 }
 
-void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) {
+  LZ_ENTER(); lazy::rd_f(x, n); lazy::rd_f(y, n); if (out != x && out != y) lazy::wr_f(out, n);
+  ProfScope prof_(CAT_ELEMENTWISE);
   if (n > 0 && rec_ok(n)) { rec_cmd(CL_GEAM, (int)n, 0, 0, alpha, beta, 0.f, 0.f, out, x, y, nullptr); return; }
   ew<2>(out, x, y, nullptr, n, [alpha, beta] __device__(float a, float b, float) { return a * alpha + b * beta; });
   LH_CHECK_LAUNCH();
@@ -390,11 +427,17 @@ void launch_reduce(int op, int which, float* small, const int* sdims4, const flo
 
 extern "C" {
 
-void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const int* bdims, float* out, const int* odims, int rank) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const int* bdims, float* out, const int* odims, int rank) {
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_op: unknown op %d", op);
   int64_t n = prod(odims, rank);
   if (n <= 0) return;
-  if (same_dims(adims, odims, rank) && same_dims(bdims, odims, rank)) {
+  LZ_SCOPE();
+  const bool same = same_dims(adims, odims, rank) && same_dims(bdims, odims, rank);
+  // a same-shape `+` waits for the call behind it: relu in place makes it one kernel, behind a parked batch norm the residual join
+  if (same && op == LH_ADD && !rec_ok(n) && lazy::park_add(a, b, out, n)) return;
+  if (lazy::g_busy && !lazy::g_replay) { lazy::flush_parked(); lazy::rd_f(a, prod(adims, rank)); lazy::rd_f(b, prod(bdims, rank)); lazy::wr_f(out, n); }
+  ProfScope prof_(CAT_ELEMENTWISE);
+  if (same) {
     if (rec_ok(n)) { rec_cmd(CL_BIN, (int)n, op, 0, 0.f, 0.f, 0.f, 0.f, out, a, b, nullptr); return; }
     ew<2>(out, a, b, nullptr, n, [op] __device__(float x, float y, float) { return bop(op, x, y); });
   } else {
@@ -407,7 +450,7 @@ void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const
 
 void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a_is_input,
                       const float* b, float* bd, const int* bdims, int b_is_input,
-                      const float* outd, const int* odims, int rank) { ProfScope prof_(CAT_ELEMENTWISE);
+                      const float* outd, const int* odims, int rank) {
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_op_grad: unknown op %d", op);
   int64_t n = prod(odims, rank);
   if (n <= 0) return;
@@ -416,6 +459,20 @@ void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a
   int pad = 4 - rank; int a4[4] = {1, 1, 1, 1}, b4[4] = {1, 1, 1, 1};
   for (int i = 0; i < rank; i++) { a4[pad + i] = adims[i]; b4[pad + i] = bdims[i]; }
   bool a_full = same_dims(adims, odims, rank), b_full = same_dims(bdims, odims, rank);
+  LZ_SCOPE();
+  // the gradient of a same-shape `+` right behind a parked relu_grad: both wait for a batch-norm gradient (the residual join's backward)
+  if (a_full && b_full && op == LH_ADD && lazy::g_busy && !lazy::g_replay && !rec_ok(n) &&
+      lazy::park_add_grad(a_is_input ? nullptr : ad, b_is_input ? nullptr : bd, outd, n)) return;
+  bool a_fresh = false, b_fresh = false;
+  if (lazy::g_busy && !lazy::g_replay) {
+    lazy::flush_parked();
+    lazy::rd_f(outd, n);
+    lazy::rd_f(a, prod(adims, rank)); lazy::rd_f(b, prod(bdims, rank));
+    const bool plain = a_full && b_full && (op == LH_ADD || op == LH_SUB);      // d += g / d -= g: an untouched zero block takes a copy
+    if (!a_is_input) { if (plain) a_fresh = lazy::acc_f(ad, n); else lazy::rw_f(ad, prod(adims, rank)); }
+    if (!b_is_input && !(bd == ad && !a_is_input)) { if (plain) b_fresh = lazy::acc_f(bd, n); else lazy::rw_f(bd, prod(bdims, rank)); }
+  }
+  ProfScope prof_(CAT_ELEMENTWISE);
   if (a_full && b_full && op != LH_DIV && rec_ok(n)) {       // same shapes: d += g, d += -g or d += g * other
     if (!a_is_input) rec_cmd(op == LH_MUL ? CL_ACCMUL : CL_ACC, (int)n, 0, 0, 0.f, 0.f, 0.f, 0.f, ad, outd, b, nullptr);
     if (!b_is_input) rec_cmd(op == LH_MUL ? CL_ACCMUL : (op == LH_SUB ? CL_ACCNEG : CL_ACC), (int)n, 0, 0, 0.f, 0.f, 0.f, 0.f, bd, outd, a, nullptr);
@@ -423,7 +480,8 @@ void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a
   }
   if (!a_is_input) {
     if (a_full) {
-      if (b_full && op == LH_ADD) ew<2>(ad, ad, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
+      if (b_full && (op == LH_ADD || op == LH_SUB) && a_fresh) ew<1>(ad, outd, nullptr, nullptr, n, [] __device__(float g, float, float) { return 0.f + g; });
+      else if (b_full && op == LH_ADD) ew<2>(ad, ad, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
       else if (b_full && op == LH_SUB) ew<2>(ad, ad, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
       else if (b_full && op == LH_MUL) ew<3>(ad, ad, outd, b, n, [] __device__(float d, float g, float bv) { return d + g * bv; });
       else hipLaunchKernelGGL(k_bcast_grad_full, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, op, 0, ad, a, b, outd, D, n);
@@ -433,7 +491,9 @@ void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a
   }
   if (!b_is_input) {
     if (b_full) {
-      if (a_full && op == LH_ADD) ew<2>(bd, bd, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
+      if (a_full && op == LH_ADD && b_fresh) ew<1>(bd, outd, nullptr, nullptr, n, [] __device__(float g, float, float) { return 0.f + g; });
+      else if (a_full && op == LH_SUB && b_fresh) ew<1>(bd, outd, nullptr, nullptr, n, [] __device__(float g, float, float) { return 0.f + (0.0f - g); });
+      else if (a_full && op == LH_ADD) ew<2>(bd, bd, outd, nullptr, n, [] __device__(float d, float g, float) { return d + g; });
       else if (a_full && op == LH_SUB) ew<2>(bd, bd, outd, nullptr, n, [] __device__(float d, float g, float) { return d + (0.0f - g); });
       else if (a_full && op == LH_MUL) ew<3>(bd, bd, outd, a, n, [] __device__(float d, float g, float av) { return d + g * av; });
       else hipLaunchKernelGGL(k_bcast_grad_full, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, op, 1, bd, a, b, outd, D, n);
@@ -446,9 +506,11 @@ void lh_bcast_op_grad(int op, const float* a, float* ad, const int* adims, int a
   LH_CHECK_LAUNCH();
 }
 
-void lh_bcast_update(int op, float* a, const int* adims, const float* b, const int* bdims, int rank) { ProfScope prof_(CAT_ELEMENTWISE);
+void lh_bcast_update(int op, float* a, const int* adims, const float* b, const int* bdims, int rank) {
   LH_REQUIRE(op >= LH_ADD && op <= LH_DIV, "lh_bcast_update: unknown op %d", op);
   LH_REQUIRE(rank >= 1 && rank <= 4, "lh_bcast_update: rank %d not in 1..4", rank);
+  LZ_ENTER(); lazy::rd_f(b, prod(bdims, rank)); lazy::rw_f(a, prod(adims, rank));
+  ProfScope prof_(CAT_ELEMENTWISE);
   int od[4];
   for (int i = 0; i < rank; i++) od[i] = adims[i] > bdims[i] ? adims[i] : bdims[i];
   int64_t n = prod(od, rank);
@@ -529,11 +591,13 @@ extern "C" {
 
 void lh_trans(const float* x, float* y, int rows, int cols) {
   if (rows <= 0 || cols <= 0) return;
+  LZ_ENTER(); lazy::rd_f(x, (int64_t)rows * cols); lazy::wr_f(y, (int64_t)rows * cols);
   hipLaunchKernelGGL((k_trans_tile<false>), dim3(cdiv(cols, 32), cdiv(rows, 32), 1), dim3(256), 0, g_stream, x, y, rows, cols, (int64_t)0);
   LH_CHECK_LAUNCH();
 }
 void lh_trans_grad(float* xd, const float* yd, int rows, int cols) {
   if (rows <= 0 || cols <= 0) return;
+  LZ_ENTER(); lazy::rd_f(yd, (int64_t)rows * cols); lazy::rw_f(xd, (int64_t)rows * cols);
   hipLaunchKernelGGL((k_trans_tile<true>), dim3(cdiv(cols, 32), cdiv(rows, 32), 1), dim3(256), 0, g_stream, yd, xd, rows, cols, (int64_t)0);
   LH_CHECK_LAUNCH();
 }
@@ -542,6 +606,7 @@ void lh_permute(const float* x, float* y, const int* dims, const int* perm, int 
   LH_REQUIRE(make_perm(P, dims, perm, rank), "lh_permute: bad rank/permutation");
   int64_t n = 1; for (int i = 0; i < rank; i++) n *= dims[i];
   if (n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(x, n); lazy::wr_f(y, n);
   hipLaunchKernelGGL((k_permute<false>), dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, P, n);
   LH_CHECK_LAUNCH();
 }
@@ -550,6 +615,7 @@ void lh_permute_grad(float* xd, const float* yd, const int* dims, const int* per
   LH_REQUIRE(make_perm(P, dims, perm, rank), "lh_permute_grad: bad rank/permutation");
   int64_t n = 1; for (int i = 0; i < rank; i++) n *= dims[i];
   if (n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(yd, n); lazy::rw_f(xd, n);
   hipLaunchKernelGGL((k_permute<true>), dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, yd, xd, P, n);
   LH_CHECK_LAUNCH();
 }
@@ -575,12 +641,16 @@ __global__ void __launch_bounds__(TPB) k_dropout(const float* x, float* y, float
 void lh_dropout_fwd(const float* x, float* y, float* mask, int64_t n, float p, uint64_t seed, uint64_t offset) {
   LH_REQUIRE(p >= 0.f && p < 1.f, "dropout rate should be [0.0, 1), got %f", p);
   if (n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(x, n); lazy::wr_f(y, n); lazy::wr_f(mask, n);
   hipLaunchKernelGGL(k_dropout, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, mask, n, p, 1.0f / (1.0f - p), seed, offset,
                      g_capturing ? (const unsigned long long*)g_capture_advance : (const unsigned long long*)nullptr);
   if (g_capturing) g_capture_drawn += (unsigned long long)n;
   LH_CHECK_LAUNCH();
 }
 void lh_dropout_bwd(const float* dy, const float* mask, float* dx, int64_t n) {
+  LZ_ENTER(); lazy::rd_f(dy, n); lazy::rd_f(mask, n);
+  if (lazy::acc_f(dx, n)) ew<2>(dx, mask, dy, nullptr, n, [] __device__(float m, float g, float) { return 0.f + m * g; });      // dx is an untouched zero block
+  else
   ew<3>(dx, dx, mask, dy, n, [] __device__(float d, float m, float g) { return d + m * g; });
   LH_CHECK_LAUNCH();
 }
@@ -602,6 +672,9 @@ __global__ void __launch_bounds__(TPB) k_concat(const float* __restrict__ src, f
 extern "C" {
 void lh_concat(int n, const float* const* h_in, const int* sizes, float* out, int outer, int inner) {
   int64_t row = 0; for (int t = 0; t < n; t++) row += (int64_t)sizes[t] * inner;
+  LZ_ENTER();
+  for (int t = 0; t < n; t++) lazy::rd_f(h_in[t], (int64_t)sizes[t] * inner * outer);
+  lazy::wr_f(out, row * outer);
   int64_t off = 0;
   for (int t = 0; t < n; t++) {
     int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
@@ -613,11 +686,13 @@ void lh_concat(int n, const float* const* h_in, const int* sizes, float* out, in
 void lh_concat_grad_beta(int n, float* const* h_ind, const float* h_beta, const int* sizes, const float* outd, int outer, int inner) {
   int64_t row = 0; for (int t = 0; t < n; t++) row += (int64_t)sizes[t] * inner;
   for (int t = 0; t < n && h_beta; t++) LH_REQUIRE(h_beta[t] == 0.f || h_beta[t] == 1.f, "lh_concat_grad_beta: beta must be 0 or 1");
+  LZ_ENTER(); lazy::rd_f(outd, row * outer);
   int64_t off = 0;
   for (int t = 0; t < n; t++) {
     int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
     if (tot > 0 && h_ind[t]) {
-      if (h_beta && h_beta[t] == 0.f) hipLaunchKernelGGL((k_concat<2>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
+      const float beta = lazy::beta_f(h_ind[t], tot, h_beta ? h_beta[t] : 1.f);
+      if (beta == 0.f) hipLaunchKernelGGL((k_concat<2>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
       else hipLaunchKernelGGL((k_concat<1>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
     }
     off += st;
@@ -734,7 +809,7 @@ __global__ void __launch_bounds__(MT_ARGS) k_mt_table_write(MtEntry* tab, const 
   if (i < n) tab[first + i] = a.e[i];
 }
 constexpr int MT_MAX_DEVICES = 16;
-struct MtStatic { MtEntry* ptr = nullptr; int count = 0; int64_t chunks = 0; uint64_t key = 0; };
+struct MtStatic { MtEntry* ptr = nullptr; };
 static MtStatic g_mt_static[MT_MAX_DEVICES];
 // The array's address on the current device (looked up once per device: every GPU holds its own copy).
 static MtStatic* mt_static_state() {
@@ -749,6 +824,35 @@ static MtStatic* mt_static_state() {
   }
   return st;
 }
+// The table is written on every call: a host-side note of what the array holds would be wrong as soon as a recorded graph
+// that contains table writes is replayed (it rewrites the array behind the note's back), and a call recorded into a graph
+// must carry its own writes.  At most count / 64 launches of one workgroup each.
+static void multi_update_static(int mode, int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
+                                float lr, float mu, float clip, int nesterov) {
+  if (count <= 0) return;
+  LH_REQUIRE(count <= MT_STATIC_MAX, "lh_multi_momentum_static: %d tensors, the fixed table holds at most %d (lh_multi_momentum has no such limit)", count, MT_STATIC_MAX);
+  LH_REQUIRE(h_x && h_d && h_n, "lh_multi_momentum_static: null pointer table");
+  int64_t chunks = 0;
+  for (int t = 0; t < count; t++) {
+    LH_REQUIRE(h_n[t] >= 0 && (h_n[t] == 0 || (h_x[t] && h_d[t] && (h_v == nullptr || h_v[t]))), "lh_multi_momentum_static: tensor %d has a null pointer or a negative size", t);
+    chunks += cdiv(h_n[t] > 0 ? h_n[t] : 1, MT_CHUNK);
+  }
+  LH_REQUIRE(chunks < 0x7fffffffLL, "lh_multi_momentum_static: %lld chunks of %d elements exceed one launch", (long long)chunks, MT_CHUNK);
+  MtStatic* st = mt_static_state();
+  if (st == nullptr) return;
+  int64_t c0 = 0;
+  for (int first = 0; first < count; first += MT_ARGS) {      // entries beyond `count` left by an earlier, larger call are never read
+    MtArgs a;
+    const int n = count - first < MT_ARGS ? count - first : MT_ARGS;
+    for (int i = 0; i < MT_ARGS; i++) {
+      if (i < n) { const int t = first + i; a.e[i] = {h_x[t], h_d[t], h_v ? h_v[t] : nullptr, h_n[t], c0}; c0 += cdiv(h_n[t] > 0 ? h_n[t] : 1, MT_CHUNK); }
+      else a.e[i] = {nullptr, nullptr, nullptr, 0, 0};
+    }
+    hipLaunchKernelGGL(k_mt_table_write, dim3(1), dim3(MT_ARGS), 0, g_stream, st->ptr, a, first, n);
+  }
+  hipLaunchKernelGGL(k_multi_update, dim3((unsigned)chunks), dim3(TPB), 0, g_stream, (const MtEntry*)st->ptr, count, mode, lr, mu, clip, nesterov);
+  LH_CHECK_LAUNCH();
+}
 }  // namespace
 
 namespace lh {
@@ -759,25 +863,51 @@ bool multi_tensor_setup() {
   return mt_static_state() != nullptr;                // the fixed table's address on this device
 }
 void multi_tensor_release() { if (g_mt.dev) (void)hipFree(g_mt.dev); g_mt = MtCache(); }
+// what lh_defer.hip launches for work it had put off
+void mask_relu(float* dst, const float* src, const float* y, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+  ew<2>(dst, src, y, nullptr, n, [] __device__(float d, float yv, float) { return yv > 0.f ? d : 0.f; });
+}
+void add_plain(const float* a, const float* b, float* out, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+  ew<2>(out, a, b, nullptr, n, [] __device__(float x, float y, float) { return x + y; });
+}
+void relu_grad_inplace_now(const float* y, float* d, int64_t n) { ProfScope prof_(CAT_ELEMENTWISE);
+  ew<2>(d, d, y, nullptr, n, [] __device__(float g, float yv, float) { return yv > 0.f ? g : 0.f; });
+}
+void multi_update_now(int mode, int count, float* const* hx, float* const* hd, float* const* hv, const int64_t* hn, float lr, float mu, float clip, int nesterov) {
+  ProfScope prof_(CAT_OPTIM);
+  // while a graph is recorded the table cannot be uploaded (a copy that waits): the kernel-written table serves
+  if (g_capturing && count <= MT_STATIC_MAX) multi_update_static(mode, count, hx, hd, hv, hn, lr, mu, clip, nesterov);
+  else multi_update(mode, count, hx, hd, hv, hn, lr, mu, clip, nesterov);
+}
 }  // namespace lh
 
 extern "C" {
-void lh_sgd(float* x, float* d, float lr, int64_t n) { ProfScope prof_(CAT_OPTIM);
+void lh_sgd(float* x, float* d, float lr, int64_t n) {
+  LZ_SCOPE();
   side_join();      // parameter gradients may still be in flight on the side stream
   if (n <= 0) return;
   LH_REQUIRE(al16(x) && al16(d), "lh_sgd: pointers must be 16-byte aligned");
+  if (lazy::gather_update(0, x, d, nullptr, lr, 0.f, 0.f, 0, n)) return;     // one launch for a run of these calls
+  if (lazy::g_busy && !lazy::g_replay) { lazy::flush_parked(); lazy::forget_forward_records(); lazy::rw_f(x, n); lazy::rw_f(d, n); }
+  ProfScope prof_(CAT_OPTIM);
   if (rec_ok(n)) { rec_cmd(CL_SGD, (int)n, 0, 0, lr, 0.f, 0.f, 0.f, x, d, nullptr, nullptr); return; }
   hipLaunchKernelGGL(k_sgd, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, lr, n);
   LH_CHECK_LAUNCH();
 }
-void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) { ProfScope prof_(CAT_OPTIM);
+void lh_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) {
+  LZ_SCOPE();
   side_join();      // parameter gradients may still be in flight on the side stream
   if (n <= 0) return;
   LH_REQUIRE(al16(x) && al16(d) && al16(v), "lh_momentum: pointers must be 16-byte aligned");
+  if (lazy::gather_update(1, x, d, v, lr, mu, clip, nesterov, n)) return;    // one launch for a run of these calls (NNModule.scala:296-303 issues one per parameter)
+  if (lazy::g_busy && !lazy::g_replay) { lazy::flush_parked(); lazy::forget_forward_records(); lazy::rw_f(x, n); lazy::rw_f(d, n); lazy::rw_f(v, n); }
+  ProfScope prof_(CAT_OPTIM);
   hipLaunchKernelGGL(k_momentum, dim3(stream_grid(n, TPB * 8)), dim3(TPB), 0, g_stream, x, d, v, lr, mu, clip, nesterov, n);
   LH_CHECK_LAUNCH();
 }
-void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) { ProfScope prof_(CAT_OPTIM);
+void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) {
+  LZ_ENTER(); lazy::forget_forward_records(); lazy::rw_f(x, n); lazy::rw_f(d, n); lazy::rw_f(m, n);
+  ProfScope prof_(CAT_OPTIM);
   side_join();      // parameter gradients may still be in flight on the side stream
   if (n <= 0) return;
   if (rec_ok(n)) { rec_cmd(CL_ADAGRAD, (int)n, 0, 0, lr, clip, 0.f, 0.f, x, d, m, nullptr); return; }
@@ -785,47 +915,27 @@ void lh_adagrad(float* x, float* d, float* m, float lr, float clip, int64_t n) {
   LH_CHECK_LAUNCH();
 }
 void lh_multi_momentum(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
-                       float lr, float mu, float clip, int nesterov) { ProfScope prof_(CAT_OPTIM);
+                       float lr, float mu, float clip, int nesterov) {
+  LZ_ENTER(); lazy::forget_forward_records();
+  for (int t = 0; t < count && lazy::g_busy; t++) { lazy::rw_f(h_x[t], h_n[t]); lazy::rw_f(h_d[t], h_n[t]); lazy::rw_f(h_v[t], h_n[t]); }
+  ProfScope prof_(CAT_OPTIM);
   side_join();      // parameter gradients may still be in flight on the side stream
   multi_update(1, count, h_x, h_d, h_v, h_n, lr, mu, clip, nesterov);
   if (!failed()) LH_CHECK_LAUNCH();
 }
 void lh_multi_momentum_static(int count, float* const* h_x, float* const* h_d, float* const* h_v, const int64_t* h_n,
-                              float lr, float mu, float clip, int nesterov) { ProfScope prof_(CAT_OPTIM);
+                              float lr, float mu, float clip, int nesterov) {
+  LZ_ENTER(); lazy::forget_forward_records();
+  for (int t = 0; t < count && lazy::g_busy && h_x && h_d && h_v && h_n; t++) { lazy::rw_f(h_x[t], h_n[t]); lazy::rw_f(h_d[t], h_n[t]); lazy::rw_f(h_v[t], h_n[t]); }
+  ProfScope prof_(CAT_OPTIM);
   side_join();      // parameter gradients may still be in flight on the side stream
-  if (count <= 0) return;
-  LH_REQUIRE(count <= MT_STATIC_MAX, "lh_multi_momentum_static: %d tensors, the fixed table holds at most %d (lh_multi_momentum has no such limit)", count, MT_STATIC_MAX);
-  LH_REQUIRE(h_x && h_d && h_v && h_n, "lh_multi_momentum_static: null pointer table");
-  int64_t chunks = 0;
-  for (int t = 0; t < count; t++) {
-    LH_REQUIRE(h_n[t] >= 0 && (h_n[t] == 0 || (h_x[t] && h_d[t] && h_v[t])), "lh_multi_momentum_static: tensor %d has a null pointer or a negative size", t);
-    chunks += cdiv(h_n[t] > 0 ? h_n[t] : 1, MT_CHUNK);
-  }
-  LH_REQUIRE(chunks < 0x7fffffffLL, "lh_multi_momentum_static: %lld chunks of %d elements exceed one launch", (long long)chunks, MT_CHUNK);
-  MtStatic* st = mt_static_state();
-  if (st == nullptr) return;
-  const uint64_t key = mt_key(1, count, h_x, h_d, h_v, h_n);
-  if (st->count != count || st->key != key) {
-    // (re)write the table: entries beyond `count` left by an earlier, larger call are never read
-    st->count = 0;
-    int64_t c0 = 0;
-    for (int first = 0; first < count; first += MT_ARGS) {
-      MtArgs a;
-      const int n = count - first < MT_ARGS ? count - first : MT_ARGS;
-      for (int i = 0; i < MT_ARGS; i++) {
-        if (i < n) { const int t = first + i; a.e[i] = {h_x[t], h_d[t], h_v[t], h_n[t], c0}; c0 += cdiv(h_n[t] > 0 ? h_n[t] : 1, MT_CHUNK); }
-        else a.e[i] = {nullptr, nullptr, nullptr, 0, 0};
-      }
-      hipLaunchKernelGGL(k_mt_table_write, dim3(1), dim3(MT_ARGS), 0, g_stream, st->ptr, a, first, n);
-    }
-    LH_CHECK_LAUNCH();
-    // A graph being recorded holds these writer launches; outside it the table would be stale, so it is not remembered.
-    if (!g_capturing) { st->count = count; st->key = key; st->chunks = chunks; }
-  }
-  hipLaunchKernelGGL(k_multi_update, dim3((unsigned)chunks), dim3(TPB), 0, g_stream, (const MtEntry*)st->ptr, count, 1, lr, mu, clip, nesterov);
-  LH_CHECK_LAUNCH();
+  LH_REQUIRE(count <= 0 || h_v != nullptr, "lh_multi_momentum_static: null pointer table");
+  multi_update_static(1, count, h_x, h_d, h_v, h_n, lr, mu, clip, nesterov);
 }
-void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr) { ProfScope prof_(CAT_OPTIM);
+void lh_multi_sgd(int count, float* const* h_x, float* const* h_d, const int64_t* h_n, float lr) {
+  LZ_ENTER(); lazy::forget_forward_records();
+  for (int t = 0; t < count && lazy::g_busy; t++) { lazy::rw_f(h_x[t], h_n[t]); lazy::rw_f(h_d[t], h_n[t]); }
+  ProfScope prof_(CAT_OPTIM);
   side_join();      // parameter gradients may still be in flight on the side stream
   multi_update(0, count, h_x, h_d, nullptr, h_n, lr, 0.f, 0.f, 0);
   if (!failed()) LH_CHECK_LAUNCH();

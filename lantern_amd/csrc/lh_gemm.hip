@@ -184,6 +184,12 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
   LH_REQUIRE(k >= 0, "lh_sgemm: negative k");
   LH_REQUIRE(lda >= (ta ? m : k) && ldb >= (tb ? k : n) && ldc >= n, "lh_sgemm: leading dimensions (%d,%d,%d) too small for m%d n%d k%d ta%d tb%d", lda, ldb, ldc, m, n, k, ta, tb);
   LH_REQUIRE(A && B && C, "lh_sgemm: null operand");
+  LZ_ENTER();
+  if (lazy::g_busy && !lazy::g_replay) {
+    lazy::rd_f(A, (int64_t)((ta ? k : m) - 1) * lda + (ta ? m : k)); lazy::rd_f(B, (int64_t)((tb ? n : k) - 1) * ldb + (tb ? k : n));
+    if (ldc == n && (beta == 0.f || beta == 1.f)) beta = lazy::beta_f(C, (int64_t)m * n, beta);     // a product added into a block nobody has touched overwrites it
+    else lazy::rw_f(C, (int64_t)(m - 1) * ldc + n);
+  }
   if ((int64_t)m * n * k >= (1 << 18) && m >= 16 && n >= 16) {
     const bool av = (lda % 4 == 0) && (((uintptr_t)A & 15) == 0) && (k % 4 == 0);
     const bool bv = (ldb % 4 == 0) && (((uintptr_t)B & 15) == 0) && (k % 4 == 0);
@@ -288,27 +294,31 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
 }
 extern "C" {
 void lh_sgemv(int trans, int m, int n, float alpha, const float* A, int lda, const float* x, float beta, float* y) {
-  ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(A, (int64_t)(m - 1) * lda + n); lazy::rd_f(x, trans ? m : n); lazy::rw_f(y, trans ? n : m);
+  ProfScope prof_(CAT_GEMM);
   if (rec_ok((int64_t)m * n, REC_MAX_MATRIX)) { rec_cmd(trans ? CL_GEMV_T : CL_GEMV_N, m, n, lda, alpha, beta, 0.f, 0.f, y, A, x, nullptr); return; }
   if (!trans) hipLaunchKernelGGL(k_sgemv_n, dim3(stream_grid((int64_t)m * 64, TPB)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
   else hipLaunchKernelGGL(k_sgemv_t, dim3((unsigned)cdiv(n, 32)), dim3(TPB), 0, g_stream, m, n, alpha, A, lda, x, beta, y);
   LH_CHECK_LAUNCH();
 }
 void lh_ger(int m, int n, const float* u, const float* v, float* A) {
-  ProfScope prof_(CAT_GEMM);
   if (m <= 0 || n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(u, m); lazy::rd_f(v, n); lazy::rw_f(A, (int64_t)m * n);
+  ProfScope prof_(CAT_GEMM);
   if (rec_ok((int64_t)m * n, REC_MAX_MATRIX)) { rec_cmd(CL_GER, m, n, 0, 0.f, 0.f, 0.f, 0.f, A, u, v, nullptr); return; }
   hipLaunchKernelGGL(k_ger, dim3(stream_grid((int64_t)m * n, TPB * 4)), dim3(TPB), 0, g_stream, m, n, u, v, A);
   LH_CHECK_LAUNCH();
 }
 void lh_dot_vv(const float* x, const float* y, float* out, int n) {
+  LZ_ENTER(); lazy::rd_f(x, n); lazy::rd_f(y, n); lazy::wr_f(out, 1);
   if (rec_ok(n)) { rec_cmd(CL_DOT, n, 0, 0, 0.f, 0.f, 0.f, 0.f, out, x, y, nullptr); return; }
   hipLaunchKernelGGL(k_dot, dim3(1), dim3(TPB), 0, g_stream, x, y, out, n);
   LH_CHECK_LAUNCH();
 }
 void lh_axpy_dev(float* y, const float* s, const float* x, int64_t n) {
   if (n <= 0) return;
+  LZ_ENTER(); lazy::rd_f(s, 1); lazy::rd_f(x, n); lazy::rw_f(y, n);
   if (rec_ok(n)) { rec_cmd(CL_AXPY_DEV, (int)n, 0, 0, 0.f, 0.f, 0.f, 0.f, y, s, x, nullptr); return; }
   hipLaunchKernelGGL(k_axpy_dev, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, y, s, x, n);
   LH_CHECK_LAUNCH();

@@ -263,6 +263,11 @@ __global__ void __launch_bounds__(256) k_avgpool_pad_bwd(const float* __restrict
 extern "C" {
 
 void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad) {
+  LZ_ENTER();
+  if (lazy::g_busy && kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pad >= 0 && H + 2 * pad >= kH && W + 2 * pad >= kW) {
+    const int64_t no = (int64_t)N * C * ((H + 2 * pad - kH) / sH + 1) * ((W + 2 * pad - kW) / sW + 1);
+    lazy::rd_f(x, (int64_t)N * C * H * W); lazy::wr_f(y, no); lazy::wr_f(argmax, no);
+  }
   ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pad >= 0, "lh_maxpool_fwd: kernel/stride must be >= 1 and pad >= 0");
   LH_REQUIRE(H + 2 * pad >= kH && W + 2 * pad >= kW, "Image too small for maxPool_k: %dx%d | (%d,%d)", H, W, kH, kW);
@@ -286,6 +291,7 @@ void lh_maxpool_fwd(const float* x, float* y, int* argmax, int N, int C, int H, 
   LH_CHECK_LAUNCH();
 }
 void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out) {
+  // the scatter form does not know how large dx is: everything deferred is brought up to date (ordered_stream() at depth 0)
   ProfScope prof_(CAT_POOL);
   if (n_out <= 0) return;
   hipLaunchKernelGGL(k_maxpool_bwd_atomic, dim3(stream_grid(n_out, TPB * 4)), dim3(TPB), 0, g_stream, dy, argmax, dx, n_out);
@@ -293,6 +299,12 @@ void lh_maxpool_bwd(const float* dy, const int* argmax, float* dx, int64_t n_out
 }
 void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float beta,
                           int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pad) {
+  LZ_ENTER();
+  if (lazy::g_busy && kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pad >= 0 && H + 2 * pad >= kH && W + 2 * pad >= kW && (beta == 0.f || beta == 1.f)) {
+    const int64_t no = (int64_t)N * C * ((H + 2 * pad - kH) / sH + 1) * ((W + 2 * pad - kW) / sW + 1);
+    lazy::rd_f(dy, no); lazy::rd_f(argmax, no);
+    beta = lazy::beta_f(dx, (int64_t)N * C * H * W, beta);
+  }
   ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pad >= 0, "lh_maxpool_bwd_dense: kernel/stride must be >= 1 and pad >= 0");
   LH_REQUIRE(H + 2 * pad >= kH && W + 2 * pad >= kW, "lh_maxpool_bwd_dense: image %dx%d too small for (%d,%d)", H, W, kH, kW);
@@ -320,6 +332,10 @@ void lh_maxpool_bwd_dense(const float* dy, const int* argmax, float* dx, float b
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {
+  LZ_ENTER();
+  if (lazy::g_busy && kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW) {
+    lazy::rd_f(x, (int64_t)N * C * H * W); lazy::wr_f(y, (int64_t)N * C * ((H - kH) / sH + 1) * ((W - kW) / sW + 1));
+  }
   ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW, "lh_avgpool_fwd: bad kernel/stride for %dx%d", H, W);
   int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
@@ -330,6 +346,10 @@ void lh_avgpool_fwd(const float* x, float* y, int N, int C, int H, int W, int kH
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW) {
+  LZ_ENTER();
+  if (lazy::g_busy && kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW) {
+    lazy::rd_f(dy, (int64_t)N * C * ((H - kH) / sH + 1) * ((W - kW) / sW + 1)); lazy::rw_f(dx, (int64_t)N * C * H * W);
+  }
   ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && H >= kH && W >= kW, "lh_avgpool_bwd: bad kernel/stride for %dx%d", H, W);
   int oH = (H - kH) / sH + 1, oW = (W - kW) / sW + 1;
@@ -341,6 +361,10 @@ void lh_avgpool_bwd(const float* dy, float* dx, int N, int C, int H, int W, int 
 }
 
 void lh_avgpool_pad_fwd(const float* x, float* y, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW) {
+  LZ_ENTER();
+  if (lazy::g_busy && kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pH >= 0 && pW >= 0 && H + 2 * pH >= kH && W + 2 * pW >= kW) {
+    lazy::rd_f(x, (int64_t)N * C * H * W); lazy::wr_f(y, (int64_t)N * C * ((H + 2 * pH - kH) / sH + 1) * ((W + 2 * pW - kW) / sW + 1));
+  }
   ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pH >= 0 && pW >= 0 && pH < kH && pW < kW, "lh_avgpool_pad_fwd: kernel (%d,%d) stride (%d,%d) pad (%d,%d)", kH, kW, sH, sW, pH, pW);
   LH_REQUIRE(H + 2 * pH >= kH && W + 2 * pW >= kW, "lh_avgpool_pad_fwd: image %dx%d too small for (%d,%d)", H, W, kH, kW);
@@ -351,6 +375,10 @@ void lh_avgpool_pad_fwd(const float* x, float* y, int N, int C, int H, int W, in
   LH_CHECK_LAUNCH();
 }
 void lh_avgpool_pad_bwd(const float* dy, float* dx, int N, int C, int H, int W, int kH, int kW, int sH, int sW, int pH, int pW) {
+  LZ_ENTER();
+  if (lazy::g_busy && kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pH >= 0 && pW >= 0 && H + 2 * pH >= kH && W + 2 * pW >= kW) {
+    lazy::rd_f(dy, (int64_t)N * C * ((H + 2 * pH - kH) / sH + 1) * ((W + 2 * pW - kW) / sW + 1)); lazy::rw_f(dx, (int64_t)N * C * H * W);
+  }
   ProfScope prof_(CAT_POOL);
   LH_REQUIRE(kH >= 1 && kW >= 1 && sH >= 1 && sW >= 1 && pH >= 0 && pW >= 0 && pH < kH && pW < kW, "lh_avgpool_pad_bwd: kernel (%d,%d) stride (%d,%d) pad (%d,%d)", kH, kW, sH, sW, pH, pW);
   LH_REQUIRE(H + 2 * pH >= kH && W + 2 * pW >= kW, "lh_avgpool_pad_bwd: image %dx%d too small for (%d,%d)", H, W, kH, kW);

@@ -173,18 +173,18 @@ __global__ void k_nll_grad(float* dx, const int* target, const float* dy, int ba
 
 extern "C" {
 
-void lh_sum_all(const float* x, float* out, int64_t n) { ProfScope prof_(CAT_REDUCE); sum_impl(x, out, n, 1.0f); if (!failed()) LH_CHECK_LAUNCH(); }
-void lh_mean_all(const float* x, float* out, int64_t n) { ProfScope prof_(CAT_REDUCE);
+void lh_sum_all(const float* x, float* out, int64_t n) { LZ_ENTER(); lazy::rd_f(x, n); lazy::wr_f(out, 1); ProfScope prof_(CAT_REDUCE); sum_impl(x, out, n, 1.0f); if (!failed()) LH_CHECK_LAUNCH(); }
+void lh_mean_all(const float* x, float* out, int64_t n) { LZ_ENTER(); lazy::rd_f(x, n); lazy::wr_f(out, 1); ProfScope prof_(CAT_REDUCE);
   LH_REQUIRE(n > 0, "lh_mean_all of an empty tensor");
   sum_impl(x, out, n, 1.0f / (float)n);
   if (!failed()) LH_CHECK_LAUNCH();
 }
-void lh_add_scalar_from(float* dx, const float* dy1, float scale, int64_t n) { ProfScope prof_(CAT_REDUCE);
+void lh_add_scalar_from(float* dx, const float* dy1, float scale, int64_t n) { LZ_ENTER(); lazy::rd_f(dy1, 1); lazy::rw_f(dx, n); ProfScope prof_(CAT_REDUCE);
   if (n <= 0) return;
   hipLaunchKernelGGL(k_add_scalar_from, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, dx, dy1, scale, n);
   LH_CHECK_LAUNCH();
 }
-void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner) { ProfScope prof_(CAT_REDUCE);
+void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner) { LZ_ENTER(); lazy::rd_f(x, (int64_t)outer * dim * inner); lazy::wr_f(y, (int64_t)outer * inner); ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * inner <= 0) return;
   if (inner == 1) hipLaunchKernelGGL(k_sum_rows, dim3(stream_grid((int64_t)outer * 64, TPB)), dim3(TPB), 0, g_stream, x, y, outer, dim);
   else if (!g_deterministic && (int64_t)outer * inner < 64 * (int64_t)g_num_cu && dim >= 512 && outer <= 65535) {      // slices add atomically
@@ -200,14 +200,14 @@ void lh_sum_dim(const float* x, float* y, int outer, int dim, int inner) { ProfS
   else hipLaunchKernelGGL(k_sum_dim_inner, dim3(stream_grid((int64_t)outer * inner, TPB)), dim3(TPB), 0, g_stream, x, y, outer, dim, inner);
   LH_CHECK_LAUNCH();
 }
-void lh_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner) { ProfScope prof_(CAT_REDUCE);
+void lh_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner) { LZ_ENTER(); lazy::rd_f(dy, (int64_t)outer * inner); lazy::rw_f(dx, (int64_t)outer * dim * inner); ProfScope prof_(CAT_REDUCE);
   int64_t n = (int64_t)outer * dim * inner;
   if (n <= 0) return;
   hipLaunchKernelGGL(k_sum_dim_grad, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, dx, dy, n, dim, inner);
   LH_CHECK_LAUNCH();
 }
 
-void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner) { ProfScope prof_(CAT_REDUCE);
+void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner) { LZ_ENTER(); lazy::rd_f(x, (int64_t)outer * c * inner); if (y != x) lazy::wr_f(y, (int64_t)outer * c * inner); ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * c * inner <= 0) return;
   if (inner == 1 && rec_ok((int64_t)outer * c)) { rec_cmd(CL_SOFTMAX, outer, c, is_log ? 1 : 0, 0.f, 0.f, 0.f, 0.f, y, x, nullptr, nullptr); return; }
   if (inner == 1) {
@@ -226,7 +226,7 @@ void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inne
   }
   LH_CHECK_LAUNCH();
 }
-void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int outer, int c, int inner) { ProfScope prof_(CAT_REDUCE);
+void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int outer, int c, int inner) { LZ_ENTER(); lazy::rd_f(y, (int64_t)outer * c * inner); lazy::rd_f(dy, (int64_t)outer * c * inner); lazy::rw_f(dx, (int64_t)outer * c * inner); ProfScope prof_(CAT_REDUCE);
   int64_t groups = (int64_t)outer * inner;
   if (groups * c <= 0) return;
   if (inner == 1 && rec_ok(groups * c)) { rec_cmd(CL_SOFTMAX_GRAD, outer, c, is_log ? 1 : 0, 0.f, 0.f, 0.f, 0.f, dx, y, dy, nullptr); return; }
@@ -235,13 +235,13 @@ void lh_softmax_grad(int is_log, const float* y, const float* dy, float* dx, int
   else hipLaunchKernelGGL((k_softmax_grad_wave<false>), dim3(grid), dim3(TPB), 0, g_stream, y, dy, dx, groups, c, inner);
   LH_CHECK_LAUNCH();
 }
-void lh_nll(const float* x, const int* target, float* y, int batch, int stride) { ProfScope prof_(CAT_REDUCE);
+void lh_nll(const float* x, const int* target, float* y, int batch, int stride) { LZ_ENTER(); lazy::rd_f(x, (int64_t)batch * stride); lazy::rd_f(target, batch); lazy::wr_f(y, batch); ProfScope prof_(CAT_REDUCE);
   if (batch <= 0) return;
   if (rec_ok(batch)) { rec_cmd(CL_NLL, batch, stride, 0, 0.f, 0.f, 0.f, 0.f, y, x, target, nullptr); return; }
   hipLaunchKernelGGL(k_nll, dim3(cdiv(batch, 64)), dim3(64), 0, g_stream, x, target, y, batch, stride);
   LH_CHECK_LAUNCH();
 }
-void lh_nll_grad(float* dx, const int* target, const float* dy, int batch, int stride) { ProfScope prof_(CAT_REDUCE);
+void lh_nll_grad(float* dx, const int* target, const float* dy, int batch, int stride) { LZ_ENTER(); lazy::rd_f(dy, batch); lazy::rd_f(target, batch); lazy::rw_f(dx, (int64_t)batch * stride); ProfScope prof_(CAT_REDUCE);
   if (batch <= 0) return;
   if (rec_ok(batch)) { rec_cmd(CL_NLL_GRAD, batch, stride, 0, 0.f, 0.f, 0.f, 0.f, dx, dy, target, nullptr); return; }
   hipLaunchKernelGGL(k_nll_grad, dim3(cdiv(batch, 64)), dim3(64), 0, g_stream, dx, target, dy, batch, stride);

@@ -22,6 +22,12 @@ void quiet_other_stream() {
   if (g_stream_cur == g_stream_raw) { if (g_side_dirty) (void)hipStreamSynchronize(g_side_stream); }
   else (void)hipStreamSynchronize(g_stream_raw);
 }
+void side_wait_for_main() {
+  if (!g_side_stream) return;
+  hipEvent_t ev = side_event();
+  LH_HIP(hipEventRecord(ev, g_stream_raw));
+  LH_HIP(hipStreamWaitEvent(g_side_stream, ev, 0));
+}
 void side_join() {
   if (!g_side_dirty) return;
   g_side_dirty = false;
@@ -60,6 +66,7 @@ bool failed() { return g_err[0] != 0; }
 
 // ---- event profiler ---------------------------------------------------------------------
 unsigned g_prof_mask = 0;
+double g_work[CAT_COUNT];
 int g_kernel_cat = CAT_GEMM;
 struct ProfRec { hipEvent_t a, b; int cat; };
 static std::vector<ProfRec> g_prof_recs;
@@ -72,14 +79,16 @@ static hipEvent_t prof_event() {
 }
 void prof_begin(int cat) {
   ProfRec r; r.a = prof_event(); r.b = nullptr; r.cat = cat;
-  if (r.a) (void)hipEventRecord(r.a, g_stream);
+  if (g_rec_pending) rec_flush();
+  if (r.a) (void)hipEventRecord(r.a, g_stream_cur);      // not ordered_stream(): timing a call must not bring deferred work forward
   g_prof_recs.push_back(r);
 }
 void prof_end(int cat) {
   for (size_t i = g_prof_recs.size(); i-- > 0;) {
     if (g_prof_recs[i].cat == cat && g_prof_recs[i].b == nullptr) {
       g_prof_recs[i].b = prof_event();
-      if (g_prof_recs[i].b) (void)hipEventRecord(g_prof_recs[i].b, g_stream);
+      if (g_rec_pending) rec_flush();
+      if (g_prof_recs[i].b) (void)hipEventRecord(g_prof_recs[i].b, g_stream_cur);
       return;
     }
   }
@@ -98,6 +107,7 @@ static void zero_async(void* p, size_t bytes) {  // bytes is a multiple of 256
   int grid = stream_grid((int64_t)n16, 256 * 4);
   hipLaunchKernelGGL(k_zero16, dim3(grid), dim3(256), 0, g_stream, (uint4*)p, n16);
 }
+void zero_bytes_async(void* p, size_t bytes) { ProfScope prof_(CAT_FILL); zero_async(p, bytes); }
 }  // namespace lh
 using namespace lh;
 
@@ -106,7 +116,7 @@ extern "C" {
 void lh_set_error_mode(int mode) { g_error_mode = mode; }
 void lh_set_tuning(int on) { g_tune_enabled = on != 0; }
 void lh_tune_counters(int64_t* measured, int64_t* remembered) { if (measured) *measured = g_plans_measured; if (remembered) *remembered = g_plans_remembered; }
-void lh_set_deterministic(int on) { side_join(); g_deterministic = on != 0; }
+void lh_set_deterministic(int on) { LZ_ENTER(); side_join(); g_deterministic = on != 0; }
 int lh_get_deterministic(void) { return g_deterministic ? 1 : 0; }
 const char* lh_last_error(void) { return g_err; }
 void lh_clear_error(void) { g_err[0] = 0; }
@@ -126,6 +136,7 @@ void lh_setup(size_t heap_bytes) {
   heap_bytes = (heap_bytes + 255) & ~(size_t)255;
   LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
   g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0; g_zero_end = 0;
+  lazy::reset();
   LH_HIP(hipMalloc((void**)&g_advance_pool, MAX_GRAPHS * sizeof(unsigned long long)));
   if (!multi_tensor_setup()) return;
 }
@@ -133,6 +144,7 @@ void lh_setup(size_t heap_bytes) {
 static void stage_release();
 static void copy_release();
 void lh_cleanup(void) {
+  lazy::reset();                 // whatever was deferred concerns memory that is about to go
   g_stream_cur = g_stream_raw;
   if (g_side_stream) { (void)hipStreamSynchronize(g_side_stream); (void)hipStreamDestroy(g_side_stream); for (auto& e : g_side_ev) (void)hipEventDestroy(e); }
   g_side_stream = nullptr; g_side_dirty = false;
@@ -152,6 +164,7 @@ void lh_cleanup(void) {
 
 void lh_sync(void) {
   LH_NOT_CAPTURING("lh_sync");
+  LZ_ENTER();                    // what is parked counts as enqueued; untouched zero blocks and unread results stay as they are
   side_join();
   lh_copy_join();
   LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH();
@@ -168,7 +181,11 @@ static void* bump(size_t bytes, bool zero) {
     return nullptr;
   }
   void* p = g_heap + g_top;
-  if (zero && g_top + need > g_zero_end) {
+  if (zero && need > ZERO_AHEAD && lazy::defer_zero()) {
+    // cleared when somebody reads it, never if its first user overwrites it
+    lazy::note_zero_block(p, need);
+  } else if (zero && g_top + need > g_zero_end) {
+    lazy::Scope lz_scope_;      // the fill below is ordered before anything that can touch the block: parked launches stay parked
     const size_t from = g_zero_end > g_top ? g_zero_end : g_top;
     size_t to = g_top + need;
     if (need < ZERO_AHEAD) to = g_top + ZERO_AHEAD < g_heap_bytes ? g_top + ZERO_AHEAD : g_heap_bytes;
@@ -186,12 +203,18 @@ void lh_free_top(size_t bytes) {
   size_t need = (bytes + 255) & ~(size_t)255;
   if (need == 0) need = 256;
   LH_REQUIRE(need <= g_top, "lh_free_top(%zu) below the arena base", bytes);
+  if (lazy::g_busy) {
+    if (lazy::g_depth == 0) { LZ_ENTER(); }       // a caller's pop (myGpuFree): nothing parked may still want the block
+    lazy::arena_released(g_heap + g_top - need);
+  }
   g_top -= need;
   g_zero_end = g_top;            // what was handed out above the new top may have been written
 }
 size_t lh_mark(void) { return g_top; }
 void lh_rewind(size_t mark) {
   LH_REQUIRE(mark <= g_top && (mark & 255) == 0, "lh_rewind(%zu): not a mark at or below the top (%zu)", mark, g_top);
+  LZ_SCOPE();
+  if (lazy::g_busy) lazy::on_rewind(g_heap + mark);     // zero fills and unread results of what is released are simply dropped
   side_join();      // what is handed out again must not be in use on the side stream
   g_top = mark;
   g_zero_end = mark;
@@ -226,8 +249,10 @@ static void stage_release() {
 
 void lh_h2d(void* dst, const void* h_src, size_t bytes) {
   LH_NOT_CAPTURING("lh_h2d");
+  LZ_ENTER();
   side_join();
   if (bytes == 0) return;
+  lazy::wr(dst, bytes);
   if (bytes <= STAGE_BYTES && stage_init()) {
     const int slot = (int)(g_stage_next++ % STAGE_SLOTS);
     if (g_stage_used[slot]) LH_HIP(hipEventSynchronize(g_stage_ev[slot]));       // long since complete unless 32 uploads are in flight
@@ -244,7 +269,10 @@ void lh_h2d(void* dst, const void* h_src, size_t bytes) {
 }
 void lh_d2h(void* h_dst, const void* src, size_t bytes) {
   LH_NOT_CAPTURING("lh_d2h");
+  LZ_ENTER();
+  lazy::rd(src, bytes);
   side_join();
+  lh_copy_join();    // an upload still on the copy stream may be what is read back
   LH_HIP(hipMemcpyAsync(h_dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
 }
@@ -277,6 +305,8 @@ void lh_h2d_async(void* dst, const void* h_src_pinned, size_t bytes) {
   LH_REQUIRE(g_stream_raw != nullptr, "lh_h2d_async before lh_setup");
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_h2d_async between lh_side_begin and lh_side_end");
   if (bytes == 0) return;
+  LZ_ENTER();
+  lazy::wr(dst, bytes);
   LH_REQUIRE(copy_init(), "lh_h2d_async: cannot create the copy stream");
   // after everything issued so far (the last reader of dst), beside everything issued from now on
   hipEvent_t ev = g_copy_ev[g_copy_ev_next++ % 4];
@@ -287,6 +317,7 @@ void lh_h2d_async(void* dst, const void* h_src_pinned, size_t bytes) {
 }
 void lh_copy_join(void) {
   if (!g_copy_dirty) return;
+  LH_NOT_CAPTURING("lh_copy_join with an upload pending");
   g_copy_dirty = false;
   hipEvent_t ev = g_copy_ev[g_copy_ev_next++ % 4];
   LH_HIP(hipEventRecord(ev, g_copy_stream));
@@ -295,10 +326,14 @@ void lh_copy_join(void) {
 void lh_d2h_async(void* h_dst_pinned, const void* src, size_t bytes) {
   LH_NOT_CAPTURING("lh_d2h_async");
   if (bytes == 0) return;
+  LZ_ENTER();
+  lazy::rd(src, bytes);
   LH_HIP(hipMemcpyAsync(h_dst_pinned, src, bytes, hipMemcpyDeviceToHost, g_stream));
 }
 
 void lh_d2d(void* dst, const void* src, size_t bytes) {
+  LZ_ENTER();
+  lazy::rd(src, bytes); lazy::wr(dst, bytes);
   if ((bytes & 3) == 0 && bytes > 0 && rec_ok((int64_t)(bytes / 4))) { rec_cmd(CL_COPY, (int)(bytes / 4), 0, 0, 0.f, 0.f, 0.f, 0.f, dst, src, nullptr, nullptr); return; }
   LH_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
 }
@@ -308,6 +343,7 @@ void lh_d2d(void* dst, const void* src, size_t bytes) {
 void lh_side_begin(void) {
   LH_REQUIRE(g_stream_raw != nullptr, "lh_side_begin before lh_setup");
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_side_begin: already on the side stream");
+  LZ_ENTER();                    // what is parked belongs in front of the fork
   // In line (no concurrency) when switched off, while kernels are timed one by one, or while the stream is recorded.
   if (!g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on || g_deterministic) return;
   hipEvent_t ev = side_event();
@@ -321,7 +357,9 @@ void lh_set_side_stream(int on) { g_side_enabled = on != 0; }
 int64_t lh_side_forks(void) { return g_side_forks; }
 
 void lh_capture_begin(void) {
+  { LZ_SCOPE(); lazy::flush_all(); }          // the recording starts from memory that is what the program thinks it is
   side_join();
+  lh_copy_join();
   LH_REQUIRE(g_stream_raw != nullptr, "lh_capture_begin before lh_setup");
   LH_REQUIRE(!g_capturing, "lh_capture_begin: already capturing");
   LH_REQUIRE(!g_rec_on, "lh_capture_begin: the command list is recording (its buffers cannot be replayed)");
@@ -336,6 +374,7 @@ void lh_capture_begin(void) {
 }
 int lh_capture_end(void) {
   if (!g_capturing) { LH_FAIL("lh_capture_end without lh_capture_begin"); return -1; }
+  { LZ_SCOPE(); lazy::flush_all(); }          // everything the recorded calls stand for is in the graph
   if (g_capture_drawn) hipLaunchKernelGGL(k_set_u64, dim3(1), dim3(1), 0, g_stream_raw, g_capture_advance, 1ull, g_capture_drawn);
   g_capturing = false;
   g_zero_end = g_top;       // fills recorded into the graph have not run
@@ -354,6 +393,7 @@ int lh_capture_end(void) {
   return (int)g_graphs.size() - 1;
 }
 void lh_graph_launch(int id) {
+  { LZ_SCOPE(); lazy::flush_all(); }
   LH_REQUIRE(id >= 0 && id < (int)g_graphs.size() && g_graphs[id] != nullptr, "lh_graph_launch: no graph %d", id);
   LH_HIP(hipGraphLaunch(g_graphs[id], g_stream));
 }
@@ -365,7 +405,11 @@ void lh_graph_destroy(int id) {
   g_graphs[id] = nullptr;
 }
 
-void lh_prof_enable(unsigned mask) { side_join(); g_prof_mask = mask; }
+void lh_work_collect(double* h_bytes, int ncat) {
+  for (int c = 0; c < ncat; c++) h_bytes[c] = c < CAT_COUNT ? g_work[c] : 0.0;
+  for (int c = 0; c < CAT_COUNT; c++) g_work[c] = 0.0;
+}
+void lh_prof_enable(unsigned mask) { LZ_ENTER(); side_join(); g_prof_mask = mask; }
 void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat) {
   for (int c = 0; c < ncat; c++) { h_ms[c] = 0.0; h_calls[c] = 0; }
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
@@ -383,7 +427,7 @@ void* lh_event_create(void) {
   if (hipEventCreate(&ev) != hipSuccess) { LH_FAIL("hipEventCreate failed"); return nullptr; }
   return (void*)ev;
 }
-void lh_event_record(void* ev) { LH_HIP(hipEventRecord((hipEvent_t)ev, g_stream)); }
+void lh_event_record(void* ev) { LZ_ENTER(); LH_HIP(hipEventRecord((hipEvent_t)ev, g_stream)); }
 float lh_event_elapsed_ms(void* start, void* stop) {
   float ms = -1.0f;
   if (g_capturing) { LH_FAIL("lh_event_elapsed_ms waits for the device, which a graph being recorded cannot do"); return ms; }

@@ -204,10 +204,11 @@ class Optim:
 
 
 class SGD(Optim):
-    """x = 1*x + (-lr)*d via geam, then clear_grad (NN:265-287; gradClip is ignored there too).
-    `fused=True` issues the same update for all tensors in one multi-tensor launch."""
+    """x = 1*x + (-lr)*d via geam, then clear_grad (NN:265-287; gradClip is ignored there too), as one backend call per
+    parameter (the HIP backend's `sgd_update`; its library gathers a run of them into one launch).
+    `fused=True` hands all tensors to the backend in one multi-tensor call instead."""
 
-    def __init__(self, module, learning_rate, gradClip=1.0, descent=True, fused=True):
+    def __init__(self, module, learning_rate, gradClip=1.0, descent=True, fused=False):
         super().__init__(module)
         self.lr = learning_rate if descent else -learning_rate
         self.fused = fused
@@ -222,9 +223,10 @@ class SGD(Optim):
 
 
 class SGD_Momentum(Optim):
-    """NN:296-303 + CPU:1232-1246: clip, v = mu*v + g, (nesterov), x -= lr*g, d = 0."""
+    """NN:296-303 + CPU:1232-1246: clip, v = mu*v + g, (nesterov), x -= lr*g, d = 0; one `momentum_update` per parameter,
+    as the reference's `step_func` issues them (`fused=True`: one multi-tensor backend call instead)."""
 
-    def __init__(self, module, learning_rate, momentum=0.9, gradClip=400.0, nesterov=False, descent=True, fused=True):
+    def __init__(self, module, learning_rate, momentum=0.9, gradClip=400.0, nesterov=False, descent=True, fused=False):
         super().__init__(module)
         assert descent
         self.lr, self.mu, self.clip, self.nesterov, self.fused = learning_rate, momentum, gradClip, nesterov, fused

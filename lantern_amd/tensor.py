@@ -5,6 +5,11 @@ Reference: src/main/scala/lantern/TensorDifferentiation.scala -- `Tensor` (386-1
 continuations (`shift`/`reset`): each TensorR op runs forward, calls the continuation, then runs
 its gradient code.  Here each op records its gradient code on a tape that `gradR*` replays in
 reverse, which issues the same backend calls in the same order.
+
+Every TensorR method below issues exactly the backend calls its Scala original stages, one per trait method, with every
+buffer from `mallocArray` (zero-filled) and every gradient accumulated: nothing is fused or reordered on this side.  What
+makes such a call sequence fast (conv -> batchNorm -> relu as one chain, gradients written instead of cleared and added,
+one launch for the optimizer) happens inside the backend's library.
 """
 import ctypes
 import math
@@ -27,52 +32,10 @@ def set_backend(b):
     return b
 
 
-# Peephole fusion.  An op whose result is very often consumed by an in-place relu (batchNorm, `+`)
-# does not launch at once: it parks itself here.  If the next op is that relu, one fused kernel
-# runs instead of two; any other op flushes the parked launch first, so program order on the
-# stream is unchanged (at most one launch is ever parked).
-_pending = None
-FUSE_CONV_BN = True       # batchNorm right behind a convolution takes its statistics from the convolution's epilogue
-FUSE_BN_ADD_RELU = True   # batchNorm -> + -> relu(inPlace), the residual join, runs as one pass forward and one fused backward
-
-
-class _Pending:
-    def __init__(self, owner, launch, kind="relu", launch_bn=None):
-        self.owner = owner          # the TensorR whose value is not computed yet
-        self.launch = launch        # launch(relu: bool)
-        self.kind = kind            # "relu": a following in-place relu can be fused in; "conv": a following batchNorm can
-        self.launch_bn = launch_bn  # kind "conv": launch_bn(scale, bias, rmean, rvar, ybn, sm, si, relu, shortcut=None)
-        self.bn = None              # a parked batchNorm describes itself here so that a following `+` can absorb it
-
-
-def _flush():
-    global _pending
-    if _pending is not None:
-        p, _pending = _pending, None
-        p.launch(False)
-
-
 def get_backend():
     if _backend is None:
         raise RuntimeError("no backend set: call set_backend(BackendHIP(...)) and backend.setup() first")
-    if _pending is not None:
-        _flush()
     return _backend
-
-
-def _park(owner, launch, kind="relu", launch_bn=None):
-    global _pending
-    _flush()
-    _pending = _Pending(owner, launch, kind, launch_bn)
-
-
-def _take_pending(owner, kind="relu"):
-    """The parked launch if it produces `owner` and is of `kind`, else None (and nothing is flushed)."""
-    global _pending
-    if _pending is not None and _pending.owner is owner and _pending.kind == kind:
-        p, _pending = _pending, None
-        return p
-    return None
 
 
 def _prod(dims):
@@ -446,38 +409,16 @@ def int_array(values):
 class TensorR:
     """A value with its gradient (TD:1146-1506).  `d` accumulates; inputs never receive one."""
 
-    def __init__(self, x, d=None, isInput=False, lazy_grad=False):
-        """`lazy_grad`: the gradient buffer of an intermediate value is created at its first use in
-        the backward pass.  The reference allocates it zero-filled at construction (TD:1509-1514)
-        and every gradient op accumulates; a first writer that can overwrite (beta = 0) makes the
-        zero fill and the read-modify-write unnecessary, with the same result."""
+    def __init__(self, x, d=None, isInput=False):
+        """The gradient is allocated zero-filled at construction; an input gets a 2-element dummy (TD:1509-1514)."""
         self.x = x
         self.isInput = isInput
-        self._d = d
-        if d is None and not lazy_grad:
-            self._d = Tensor.zeros(2) if isInput else Tensor.zeros_like(x)     # TD:1509-1514
-
-    @property
-    def d(self):
-        if self._d is None:
-            self._d = Tensor.zeros(2) if self.isInput else Tensor.zeros_like(self.x)
-        return self._d
-
-    @d.setter
-    def d(self, t):
-        self._d = t
-
-    def grad_target(self):
-        """(gradient buffer, beta) for an op that can either overwrite or accumulate."""
-        if self._d is None:
-            self._d = Tensor(get_backend().mallocArray(self.x.scalarCount, zero=False), self.x.shape)
-            return self._d.data, 0.0
-        return self._d.data, 1.0
+        self.d = d if d is not None else (Tensor.zeros(2) if isInput else Tensor.zeros_like(x))
 
     @staticmethod
     def _new(x):
-        """Result of an op: gradient created on demand."""
-        return TensorR(x, lazy_grad=True)
+        """Result of an op: `TensorR(x)`."""
+        return TensorR(x)
 
     def __call__(self, i): return TensorR(self.x(i), self.d(i))
 
@@ -507,26 +448,12 @@ class TensorR:
 
     # -- arithmetic --------------------------------------------------------------------------------
     def _bin(self, op, that):
-        if isinstance(that, TensorR) and op == B.ADD and self.x.shape == that.x.shape and self is not that:
-            return self._add_same_shape(that)      # before get_backend(): a parked batchNorm may be absorbed
         be = get_backend()
         if isinstance(that, TensorR):
             ya, a, b = self.x._bin(op, that.x)
             y = TensorR._new(ya)
-            def back():
-                full = a == ya.shape and b == ya.shape
-                if full and op == B.ADD and self is not that:
-                    # same-shape add: a fresh gradient buffer is written by a copy, not zero + accumulate
-                    for t in (self, that):
-                        if t.isInput: continue
-                        if t._d is None:
-                            buf, _ = t.grad_target()
-                            be.copyFloatArray(buf, y.d.data, ya.scalarCount)
-                        else:
-                            be.bcast_update(B.ADD, t.d.data, ya.shape, y.d.data, ya.shape)
-                    return
-                be.bcast_op_grad(op, self.x.data, self.d.data, a, self.isInput, that.x.data, that.d.data, b, that.isInput, y.d.data, ya.shape)
-            _tape.append(back)
+            # add_grad / minus_grad / mul_grad / div_grad (TD:1171-1206): both operands' gradients in one backend call
+            _tape.append(lambda: be.bcast_op_grad(op, self.x.data, self.d.data, a, self.isInput, that.x.data, that.d.data, b, that.isInput, y.d.data, ya.shape))
             return y
         s = float(that)
         y = TensorR._new(self.x._bin(op, s))
@@ -542,62 +469,6 @@ class TensorR:
     def __sub__(self, t): return self._bin(B.SUB, t)
     def __mul__(self, t): return self._bin(B.MUL, t)
     def __truediv__(self, t): return self._bin(B.DIV, t)
-
-    def _add_same_shape(self, that):
-        """`+` without broadcasting (TD:1171-1176, CPU:299-304), parked so that a following in-place
-        relu fuses with it (the residual join of ResNet)."""
-        global _pending
-        bnp = None                       # a parked batchNorm producing one of the operands: absorbed if a relu follows
-        if FUSE_BN_ADD_RELU and _pending is not None and _pending.bn is not None and (_pending.owner is self or _pending.owner is that):
-            bnp, _pending = _pending, None
-            if bnp.bn["xin"] is (that if bnp.owner is self else self):
-                # relu(bn(h) + h): the batch norm's input is also the shortcut, so both gradients of the fused backward would be
-                # one buffer (its first pass adds into what its second overwrites); this join runs unfused
-                bnp.launch(False)
-                bnp = None
-        be = get_backend()
-        n = self.x.scalarCount
-        ybuf = be.mallocArray(n, zero=False)
-        y = TensorR._new(Tensor(ybuf, self.x.shape))
-        st = {"relu": False, "joined": False}
-        other = None if bnp is None else (that if bnp.owner is self else self)
-
-        def launch(relu):
-            st["relu"] = relu
-            if bnp is not None and relu:
-                st["joined"] = True
-                bnp.launch(True, other.x.data, ybuf)
-                bnp.owner.x = None        # the batchNorm's own output is never materialised: a later read must fail, not see garbage
-                return
-            if bnp is not None:
-                bnp.launch(False)
-            _backend.add_into(self.x.data, that.x.data, ybuf, n, relu)
-        _park(y, launch)
-
-        def back():
-            if st["joined"]:
-                info = bnp.bn
-                xin = info["xin"]
-                xd, xbeta = (None, 1.0) if xin.isInput else xin.grad_target()
-                sd, sbeta = (None, 1.0) if other.isInput else other.grad_target()
-                be.batchNorm_add_relu_grad(xin.x.data, xd, xbeta, ybuf, y.d.data, info["scale"].x.data, info["scale"].d.data, info["bias"].d.data,
-                                           info["sm"], info["si"], sd, sbeta, info["N"], info["C"], info["HW"])
-                info["st"]["joined"] = True
-                return
-            if st["relu"]:
-                ad, ab = (None, 1.0) if self.isInput else self.grad_target()
-                bd, bb = (None, 1.0) if that.isInput else that.grad_target()
-                be.add_relu_grad(ybuf, y.d.data, ad, ab, bd, bb, n)
-                return
-            for t in (self, that):
-                if t.isInput: continue
-                if t._d is None:            # a fresh gradient buffer is written by a copy, not zero + accumulate
-                    buf, _ = t.grad_target()
-                    be.copyFloatArray(buf, y.d.data, n)
-                else:
-                    be.bcast_update(B.ADD, t.d.data, self.x.shape, y.d.data, self.x.shape)
-        _tape.append(back)
-        return y
 
     def dot(self, that):
         be = get_backend()
@@ -622,11 +493,7 @@ class TensorR:
         be = get_backend()
         d1, d2, d3 = Tensor._gemm_dims(self.x.shape, transX, that.x.shape, transY)
         y = TensorR._new(self.x.gemm(that.x, transX, transY, alpha))
-        def back():
-            xd, xbeta = (None, 1.0) if self.isInput else self.grad_target()
-            yd, ybeta = (None, 1.0) if that.isInput else that.grad_target()
-            be.gemm_grad(self.x.data, xd, self.isInput, transX, that.x.data, yd, that.isInput, transY, float(alpha), y.d.data, d1, d2, d3, xbeta, ybeta)
-        _tape.append(back)
+        _tape.append(lambda: be.gemm_grad(self.x.data, self.d.data, self.isInput, transX, that.x.data, that.d.data, that.isInput, transY, float(alpha), y.d.data, d1, d2, d3))
         return y
 
     def trans(self):
@@ -641,11 +508,6 @@ class TensorR:
 
     # -- activations ----------------------------------------------------------------------------------
     def _unary(self, op, inPlace=False, lo=-1.0, hi=1.0):
-        if inPlace and op == B.RELU:
-            p = _take_pending(self)
-            if p is not None:
-                p.launch(True)      # producer + relu in one kernel; its gradient closure applies the mask
-                return self
         be = get_backend()
         if inPlace:
             self.x._unary(op, True, lo, hi)
@@ -689,36 +551,13 @@ class TensorR:
 
     # -- bn / softmax / loss ----------------------------------------------------------------------------------
     def batchNorm(self, scale, bias, runningMean, runningVar):
-        conv = _take_pending(self, "conv") if FUSE_CONV_BN else None         # before get_backend(), which would flush it
+        """TD:1367-1372: batchNormTraining, then batchNorm_grad with the saved statistics."""
         be = get_backend()
         N, C, HW = self.x._bn_view()
-        n = self.x.scalarCount
-        ybuf = be.mallocArray(n, zero=False)
-        sm, si = be.mallocArray(C, zero=False), be.mallocArray(C, zero=False)
-        y = TensorR._new(Tensor(ybuf, self.x.shape))
-        st = {"relu": False}
-
-        def launch(relu, shortcut=None, out=None):
-            st["relu"] = relu
-            if shortcut is not None:          # absorbed by a following `+` and relu: out = relu(bn(x) + shortcut)
-                if conv is not None:
-                    conv.launch_bn(scale.x.data, bias.x.data, runningMean.data, runningVar.data, out, sm, si, True, shortcut)
-                else:
-                    _backend.batchNormTraining_add_relu_into(self.x.data, scale.x.data, bias.x.data, runningMean.data, runningVar.data, shortcut, out, sm, si, N, C, HW)
-            elif conv is not None:
-                conv.launch_bn(scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, relu)
-            else:
-                _backend.batchNormTraining_into(self.x.data, scale.x.data, bias.x.data, runningMean.data, runningVar.data, ybuf, sm, si, N, C, HW, relu)
-        _park(y, launch)
-        _pending.bn = {"xin": self, "scale": scale, "bias": bias, "sm": sm, "si": si, "N": N, "C": C, "HW": HW, "st": st}
-
-        def back():
-            if st.get("joined"):              # the residual join's backward has done this layer's part
-                return
-            xd, beta = (None, 1.0) if self.isInput else self.grad_target()
-            be.batchNorm_grad(self.x.data, xd, y.d.data, scale.x.data, scale.d.data, bias.d.data, sm, si, N, C, HW, beta,
-                              y_relu=ybuf if st["relu"] else None, bias=bias.x.data)
-        _tape.append(back)
+        yv, sm, si = self.x.batchNormTraining(scale.x, bias.x, runningMean, runningVar)
+        y = TensorR._new(yv)
+        _tape.append(lambda: be.batchNorm_grad(self.x.data, None if self.isInput else self.d.data, y.d.data, scale.x.data, scale.d.data, bias.d.data,
+                                               sm.data, si.data, N, C, HW))
         return y
 
     batchNorm1D = batchNorm
@@ -747,30 +586,18 @@ class TensorR:
     # -- conv / pool ----------------------------------------------------------------------------------------------
     def convBBP(self, kernel, bias, strides, pads):
         be = get_backend()
-        assert self.isInput or self._d is None or self._d.scalarCount == self.x.scalarCount, "For convBBP, THIS is either input or intermediate stage"
+        assert self.isInput or self.d.scalarCount == self.x.scalarCount, "For convBBP, THIS is either input or intermediate stage"
         assert self.x.rank == 4, "For convBBP, THIS is dim 4: batch, channel, row, col"
         assert kernel.x.rank == 4 and self.x.shape[1] == kernel.x.shape[1]
         N, C, H, W = self.x.shape; K, _, R, S = kernel.x.shape
         sH, sW = strides[0], strides[1]; pH, pW = Tensor._pads2(pads)
-        dims = (N, C, H, W, K, R, S, sH, sW, pH, pW)
-        kept = {"finput": None}
-        ybuf = be.mallocArray(N * K * conv_size(H, R, sH, pH) * conv_size(W, S, sW, pW), zero=False)
-        y = TensorR._new(Tensor(ybuf, (N, K, conv_size(H, R, sH, pH), conv_size(W, S, sW, pW))))
-        xbuf, wbuf, bbuf = self.x.data, kernel.x.data, (bias.x.data if bias is not None else None)
-        # parked: a batchNorm right behind the convolution takes its statistics from the convolution's epilogue
-        def launch(relu):
-            kept["finput"] = _backend.conv2D_batch_into(xbuf, wbuf, bbuf, ybuf, *dims)
-        def launch_bn(scale, bb, rm, rv, ybn, sm, si, relu, shortcut=None):
-            if shortcut is not None:
-                kept["finput"] = _backend.conv2D_batch_bn_add_relu_into(xbuf, wbuf, bbuf, ybuf, dims, scale, bb, rm, rv, shortcut, ybn, sm, si)
-            else:
-                kept["finput"] = _backend.conv2D_batch_bn_into(xbuf, wbuf, bbuf, ybuf, dims, scale, bb, rm, rv, ybn, sm, si, relu)
-        _park(y, launch, "conv", launch_bn)
+        yv, finput = self.x.conv2D_batch(kernel.x, bias.x if bias is not None else None, strides, pads)
+        y = TensorR._new(yv)
+        be.convs_open += 1                  # forward convolutions whose gradient is still to come (a backend may run filter gradients beside the ones that follow)
         def back():
-            xd, beta = (None, 1.0) if self.isInput else self.grad_target()
-            be.ops_left = len(_tape)        # backward operators still to come (a backend may run the filter gradient beside them)
-            be.conv2D_batch_grad(self.x.data, xd, self.isInput, kept["finput"], kernel.x.data, kernel.d.data, y.d.data,
-                                 bias.d.data if bias is not None else None, N, C, H, W, K, R, S, sH, sW, pH, pW, beta)
+            be.convs_open -= 1
+            be.conv2D_batch_grad(self.x.data, None if self.isInput else self.d.data, self.isInput, finput, kernel.x.data, kernel.d.data, y.d.data,
+                                 bias.d.data if bias is not None else None, N, C, H, W, K, R, S, sH, sW, pH, pW)
         _tape.append(back)
         return y
 
@@ -780,10 +607,7 @@ class TensorR:
         y = TensorR._new(yv)
         N, C, H, W = self.x.shape
         geom = (N, C, H, W, kernels[0], kernels[1], strides[0], strides[1], pads[0] if pads else 0)
-        def back():
-            xd, beta = self.grad_target()
-            be.maxPool2D_batch_grad(xd, y.d.data, idx, yv.scalarCount, geom, beta)
-        _tape.append(back)
+        _tape.append(lambda: be.maxPool2D_batch_grad(self.d.data, y.d.data, idx, yv.scalarCount, geom))
         return y
 
     def averagePoolBK(self, kernels, strides, pads=None):
@@ -810,11 +634,7 @@ class TensorR:
         y = TensorR._new(self.x.concat(dim, *[t.x for t in others]))
         outer, inner = _prod(self.x.shape[:dim]), _prod(self.x.shape[dim + 1:])
         sizes = [t.x.shape[dim] for t in ts]
-        def back():
-            # an input whose gradient nobody has written yet is overwritten (its buffer then needs no zero fill)
-            tg = [(None, 1.0) if t.isInput else t.grad_target() for t in ts]
-            be.concat_grad([b for b, _ in tg], sizes, y.d.data, outer, inner, [bt for _, bt in tg])
-        _tape.append(back)
+        _tape.append(lambda: be.concat_grad([None if t.isInput else t.d.data for t in ts], sizes, y.d.data, outer, inner))
         return y
 
     # -- recurrent layer, CTC ----------------------------------------------------------------------------
@@ -835,11 +655,11 @@ class TensorR:
             ybuf = be.rnn_forward(mode, self.x.data, w, T, Bn, I, hidden, bidirectional, hx=hx)
         y = TensorR._new(Tensor(ybuf, (T, Bn, D * hidden)))
         def back():
-            xd, beta = (None, 1.0) if self.isInput else self.grad_target()
+            xd = None if self.isInput else self.d.data
             if mode >= 2:
-                be.rnn_gated_backward(mode, self.x.data, ybuf, y.d.data, w, reserve, xd, dw, T, Bn, I, hidden, bidirectional, beta, hx=hx, cx=cx)
+                be.rnn_gated_backward(mode, self.x.data, ybuf, y.d.data, w, reserve, xd, dw, T, Bn, I, hidden, bidirectional, hx=hx, cx=cx)
             else:
-                be.rnn_backward(mode, self.x.data, ybuf, y.d.data, w, xd, dw, T, Bn, I, hidden, bidirectional, beta, hx=hx)
+                be.rnn_backward(mode, self.x.data, ybuf, y.d.data, w, xd, dw, T, Bn, I, hidden, bidirectional, hx=hx)
         _tape.append(back)
         return y
 

@@ -23,7 +23,7 @@ trait HipGenGPUOps extends CGenBase {
   import IR._
 
   override def emitNode(sym: Sym[Any], rhs: Def[Any]) = rhs match {
-    case a@GPUArrayNew(n) =>                                    // arena memory reads zero, as Tensor.zeros expects (TD:1075-1076)
+    case a@GPUArrayNew(n) =>                                    // arena memory reads zero, as Tensor.zeros expects (TD:1075-1076); large blocks are cleared only if something reads them before writing
       val dataType = remap(a.m)
       emitValDef(sym, "(" + dataType + "*)lh_malloc((size_t)" + quote(n) + " * sizeof(" + dataType + "))")
     case a@GPUArrayFromSeq(xs) =>
@@ -367,6 +367,7 @@ trait TensorDslHIP extends TensorDslCPU with GPUOps {
 
     // ---- convolution (CDN:833-880).  No descriptors, no per-site algorithm search in the emitted text: the library measures its
     //      launch plans on first use ------------------------------------------------------------------------------------------
+    var convsOpen = 0                                             // forward convolutions staged whose gradient call is still to come
     override def conv2D_batch(input: Tensor, kernel: Tensor, bias: Option[Tensor], strides: Seq[Int], pads: Seq[Int]): (Tensor, Option[Tensor], Int) = {
       assert(input.rank == 4, s"Convolution input must have rank 4, but got ${input.rank}")
       assert(kernel.rank == 4, s"Convolution kernel must have rank 4, but got ${kernel.rank}")
@@ -378,6 +379,7 @@ trait TensorDslHIP extends TensorDslCPU with GPUOps {
       val (sH, sW) = (strides(0), strides(1))
       val resShape = Seq(input.shape(0), kernel.shape(0), convSize(input.shape(2) + 2 * padH, kernel.shape(2), sH), convSize(input.shape(3) + 2 * padW, kernel.shape(3), sW))
       val res = Tensor(mallocArray[Float](resShape.product1), resShape: _*)
+      convsOpen += 1
       hip("lh_conv2d_fwd", input.data, kernel.data, bias.map(_.data: Any).getOrElse(nullFloats), res.data,
           input.shape(0), input.shape(1), input.shape(2), input.shape(3), kernel.shape(0), kernel.shape(2), kernel.shape(3), sH, sW, padH, padW)
       (res, None, 0)                                              // no im2col buffer, no algorithm counter (CDN:859-866 returns a counter)
@@ -390,11 +392,15 @@ trait TensorDslHIP extends TensorDslCPU with GPUOps {
       if (!input.isInput)                                         // CDN:873
         hip("lh_conv2d_bwd_data", res.d.data, filter.x.data, input.d.data, 1.0f, n, c, h, w, k, r, s, strides._1, strides._2, padding._1, padding._2)
       // Only the optimizer reads filter.d: the filter gradient runs on the library's side stream beside the rest of the backward
-      // pass (not for the network's first layer, where nothing is left to run beside it; the optimizer entry points join).
-      if (!input.isInput) hip("lh_side_begin")
+      // pass, unless fewer than two convolution gradients are still to come (with nothing left to run beside it the hand-over
+      // between the streams only delays the optimizer; the optimizer entry points join).  Gradient calls are staged in the reverse
+      // order of the forward calls, so the count of forward convolutions not yet matched is known here at staging time.
+      convsOpen -= 1
+      val fork = !input.isInput && convsOpen >= 2
+      if (fork) hip("lh_side_begin")
       hip("lh_conv2d_bwd_filter", input.x.data, res.d.data, filter.d.data, bias.map(_.d.data: Any).getOrElse(nullFloats), 1.0f,
           n, c, h, w, k, r, s, strides._1, strides._2, padding._1, padding._2)
-      if (!input.isInput) hip("lh_side_end")
+      if (fork) hip("lh_side_end")
     }
 
     // ---- pooling (CDN:882-982).  Max-pool keeps its argmax (global flat input index, first maximum wins: CPU:848-948), which the
@@ -666,35 +672,13 @@ trait TensorDslHIP extends TensorDslCPU with GPUOps {
                          dropout: Float = 0f, bidirectional: Boolean = false, reserve: Rep[Array[Float]], reserveSize: Rep[Int], counter: Int): Unit =
       rnnBackward(mode, input, hx, cx, w, output, numLayers, hiddenSize, dropout, bidirectional, reserve, reserveSize, counter)
 
-    // ---- fused forms with no counterpart in the trait; a front end that knows them emits one call for a sequence of trait calls ------
-    // conv -> batchNorm [-> relu(inPlace)] or conv -> batchNorm -> (+ shortcut) -> relu(inPlace): the convolution's store pass leaves
-    // the batch statistics, the normalisation reads the convolution's output once
-    def conv2D_batch_batchNorm(input: Tensor, kernel: Tensor, strides: Seq[Int], pads: Seq[Int], scale: Tensor, bias: Tensor, runningMean: Tensor, runningVar: Tensor,
-                               shortcut: Option[Tensor], relu: Boolean): (Tensor, Tensor, Tensor, Tensor) = {
-      val (padH, padW) = if (pads.size == 1) (pads(0), pads(0)) else if (pads.size == 2) (pads(0), pads(1)) else (pads(0), pads(2))
-      val resShape = Seq(input.shape(0), kernel.shape(0), convSize(input.shape(2) + 2 * padH, kernel.shape(2), strides(0)), convSize(input.shape(3) + 2 * padW, kernel.shape(3), strides(1)))
-      val conv = Tensor(mallocArray[Float](resShape.product1), resShape: _*); val out = Tensor(mallocArray[Float](resShape.product1), resShape: _*)
-      val saveMean = Tensor(mallocArray[Float](kernel.shape(0)), kernel.shape(0)); val saveInvStd = Tensor(mallocArray[Float](kernel.shape(0)), kernel.shape(0))
-      hip("lh_conv2d_fwd_bn_apply", input.data, kernel.data, nullFloats, conv.data, input.shape(0), input.shape(1), input.shape(2), input.shape(3),
-          kernel.shape(0), kernel.shape(2), kernel.shape(3), strides(0), strides(1), padH, padW, scale.data, bias.data, saveMean.data, saveInvStd.data,
-          runningMean.data, runningVar.data, 1e-5f, 0.1f, shortcut.map(_.data: Any).getOrElse(nullFloats), out.data, relu || shortcut.isDefined)
-      (out, conv, saveMean, saveInvStd)
-    }
+    // ---- no fused forms here.  The trait's one-call-per-method sequence is what this backend emits; the library recognises the
+    //      chains it can run as one kernel (conv -> batchNorm -> [+ shortcut] -> relu in place, their gradients in reverse, a run
+    //      of momentum_update / sgd_update calls) and overwrites gradient buffers nobody has touched since `mallocArray`
+    //      instead of clearing them and adding (lantern_hip.h, "Fusion of adjacent calls") -------------------------------------------
     // plain SGD in one pass (x -= lr*d; d = 0) instead of geam + clear_grad (NN:279-285); gradients are not clipped there either
     def sgd_update(tr: TensorR, learning_rate: Float, descent: Boolean): Unit =
       hip("lh_sgd", tr.x.data, tr.d.data, if (descent) learning_rate else -learning_rate, cast("int64_t", tr.x.scalarCount))
-    def sgd_update_all(trs: Seq[TensorR], learning_rate: Float, descent: Boolean): Unit = {
-      val counts = NewArray[Long](trs.size)
-      trs.zipWithIndex.foreach { case (tr, i) => counts(i) = tr.x.scalarCount.toLong }
-      hip("lh_multi_sgd", trs.size, hostPointers(trs.map(_.x.data)), hostPointers(trs.map(_.d.data)), counts, if (descent) learning_rate else -learning_rate)
-    }
-    // the whole model's momentum step in one launch (NN:296-303 loops over the parameters)
-    def momentum_update_all(trs: Seq[TensorR], ts: Seq[Tensor], learning_rate: Float, momentum: Float, gradClip: Float, nesterov: Boolean): Unit = {
-      val counts = NewArray[Long](trs.size)
-      trs.zipWithIndex.foreach { case (tr, i) => counts(i) = tr.x.scalarCount.toLong }
-      hip("lh_multi_momentum", trs.size, hostPointers(trs.map(_.x.data)), hostPointers(trs.map(_.d.data)), hostPointers(ts.map(_.data)), counts,
-          learning_rate, momentum, gradClip, nesterov)
-    }
   }
   object BackendHIP { def apply() = new BackendHIP }
   def BackendGPU: Backend = BackendHIP()                                                                           // as CUB:903-904

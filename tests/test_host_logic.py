@@ -1,5 +1,5 @@
-"""Host-side logic that needs no GPU: shape rules, the tape, lazy gradient buffers and the
-relu peephole (run on the CPU oracle backend)."""
+"""Host-side logic: shape rules, the tape, that the front end issues one backend call per trait method, and (on both backends)
+that the chains the library fuses give what the calls as issued give."""
 import numpy as np
 import pytest
 
@@ -46,7 +46,7 @@ def test_input_gets_no_gradient(on_cpu):  # TD:1510: inputs carry a 2-element du
     np.testing.assert_allclose(k.d.toCPU().ravel(), [4] * 9)
 
 
-def test_lazy_gradient_buffer_matches_eager(on_cpu):
+def test_gradient_through_add_relu_add(be):
     rng = np.random.RandomState(0)
     a, b = rng.randn(2, 3, 4, 4).astype(np.float32), rng.randn(2, 3, 4, 4).astype(np.float32)
 
@@ -60,51 +60,104 @@ def test_lazy_gradient_buffer_matches_eager(on_cpu):
     np.testing.assert_allclose(gy, mask * 1.0)
 
 
-def test_parked_launch_is_flushed_by_any_other_op(on_cpu):
-    """batchNorm parks its launch so a following in-place relu can fuse; anything else must see
-    the finished value."""
+class _Recorder:
+    """Stands in front of a backend and notes the name of every method the front end calls."""
+
+    def __init__(self, inner):
+        self._inner, self.calls = inner, []
+
+    def __getattr__(self, name):
+        v = getattr(self._inner, name)
+        if not callable(v):
+            return v
+        def call(*a, **k):
+            self.calls.append(name)
+            return v(*a, **k)
+        return call
+
+    def __setattr__(self, name, value):
+        if name in ("_inner", "calls"):
+            object.__setattr__(self, name, value)
+        else:
+            setattr(self._inner, name, value)
+
+
+def test_front_end_issues_one_backend_call_per_trait_method(on_cpu):
+    """The front end fuses nothing: conv -> batchNorm -> relu(inPlace) -> + -> relu(inPlace) reaches the backend as the calls
+    the reference stages for it (TD:1171-1176, 1324-1329, 1394-1410; relu in place: TD:1232-1238), gradients in reverse order,
+    and the optimizer as one momentum_update per parameter (NN:296-303)."""
+    from lantern_amd.nn import Module, Conv2D, BatchNorm2D, SGD_Momentum
     rng = np.random.RandomState(1)
-    x = TensorR(Tensor.fromNumpy(rng.randn(4, 2, 3, 3).astype(np.float32)))
-    g, b = TensorR(Tensor.ones(2)), TensorR(Tensor.zeros(2))
-    y = x.batchNorm(g, b, Tensor.zeros(2), Tensor.ones(2))
-    assert T._pending is not None and T._pending.owner is y
-    v = y.x.toCPU()                       # toCPU goes through get_backend(): flushes
-    assert T._pending is None
-    xs = x.x.toCPU()
-    ref = (xs - xs.mean(axis=(0, 2, 3), keepdims=True)) / np.sqrt(xs.var(axis=(0, 2, 3), keepdims=True) + 1e-5)
-    np.testing.assert_allclose(v, ref, rtol=1e-4, atol=1e-5)
-    y2 = x.batchNorm(g, b, Tensor.zeros(2), Tensor.ones(2)).relu(True)      # fused path
-    assert T._pending is None
-    np.testing.assert_allclose(y2.x.toCPU(), np.maximum(ref, 0), rtol=1e-4, atol=1e-5)
-    T._tape.clear()
+
+    class Net(Module):
+        def __init__(self):
+            super().__init__("net")
+            self.conv = self.add(Conv2D(3, 3, (3, 3), (1, 1), (1, 1), useBias=False, rng=rng))
+            self.bn = self.add(BatchNorm2D(3))
+
+        def __call__(self, x):
+            h = self.bn(self.conv(x)).relu(True)
+            return (self.bn(self.conv(h)) + h).relu(True)
+    net = Net()
+    opt = SGD_Momentum(net, 0.1, 0.9)
+    x = TensorR(Tensor.fromNumpy(rng.randn(2, 3, 4, 4).astype(np.float32)), isInput=True)
+    rec = _Recorder(on_cpu)
+    la.set_backend(rec)
+    try:
+        gradR_loss(lambda d: net(x).sum())(Tensor.zeros(1))
+        opt.step()
+    finally:
+        la.set_backend(on_cpu)
+    ops = [c for c in rec.calls if c not in ("mallocArray", "fillInPlace", "copyFloatArray")]
+    assert ops == ["conv2D_batch", "batchNormTraining", "unary",
+                   "conv2D_batch", "batchNormTraining", "bcast_op", "unary", "sum",
+                   "add_scalar_from", "unary_grad", "bcast_op_grad", "batchNorm_grad", "conv2D_batch_grad",
+                   "unary_grad", "batchNorm_grad", "conv2D_batch_grad",
+                   "momentum_update", "momentum_update", "momentum_update"], ops
 
 
-def test_fused_and_unfused_relu_gradients_agree(on_cpu):
+def _fusion(be, on):
+    """Switch the library's fusion of adjacent calls (the oracle has none to switch)."""
+    if be.name == "hip":
+        be.lib.lh_set_fusion(1 if on else 0)
+
+
+def test_fused_and_unfused_relu_gradients_agree(be):
+    """batchNorm -> relu(inPlace): the library runs the pair as one kernel (forward) and one fused backward; with a read of
+    the batch norm's output in between, or with fusion off, every call runs on its own.  Same values, same gradients."""
     rng = np.random.RandomState(2)
     xs = rng.randn(4, 3, 5, 5).astype(np.float32)
 
-    def run(fused):
-        x = TensorR(Tensor.fromNumpy(xs)); g = TensorR(Tensor.fromData((3,), 1.5, 0.5, 2.0)); b = TensorR(Tensor.fromData((3,), 0.1, -0.2, 0.0))
-        def f(d):
-            y = x.batchNorm(g, b, Tensor.zeros(3), Tensor.ones(3))
-            if not fused:
-                y.x.toCPU()                 # forces the unfused launch before relu
-            return (y.relu(True) * 2.0).sum()
-        gradR_loss(f)(Tensor.zeros(1))
-        return x.d.toCPU(), g.d.toCPU(), b.d.toCPU()
-    for u, v in zip(run(True), run(False)):
-        np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)
+    def run(fused, lib_fusion=True):
+        _fusion(be, lib_fusion)
+        try:
+            x = TensorR(Tensor.fromNumpy(xs)); g = TensorR(Tensor.fromData((3,), 1.5, 0.5, 2.0)); b = TensorR(Tensor.fromData((3,), 0.1, -0.2, 0.0))
+            def f(d):
+                y = x.batchNorm(g, b, Tensor.zeros(3), Tensor.ones(3))
+                if not fused:
+                    y.x.toCPU()                 # a read in between: the batch norm has to run before the relu is known
+                return (y.relu(True) * 2.0).sum()
+            gradR_loss(f)(Tensor.zeros(1))
+            return x.d.toCPU(), g.d.toCPU(), b.d.toCPU()
+        finally:
+            _fusion(be, True)
+    want = run(True)
+    for other in (run(False), run(True, lib_fusion=False)):
+        for u, v in zip(want, other):
+            np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)
 
 
 @pytest.mark.parametrize("bn_side", ["left", "right"])
-def test_residual_join_absorbs_the_batchnorm_and_matches_the_unfused_program(on_cpu, bn_side):
-    """conv -> batchNorm -> + shortcut -> relu(inPlace): with the join fused the batchNorm is absorbed by the `+`
-    (either operand) and its own output is never materialised; values and every gradient equal the unfused program."""
+def test_residual_join_matches_the_unfused_program(be, bn_side):
+    """conv -> batchNorm -> + shortcut -> relu(inPlace): the library runs the chain as one convolution launch and one
+    normalise-add-relu pass and never stores the batchNorm's own output; values and every gradient equal the program with
+    fusion off, and a later read of the batchNorm's output (and of the gradient buffers the fused backward left unmasked)
+    still gives what the calls as issued would have left there."""
     rng = np.random.RandomState(3)
     xs = rng.randn(2, 4, 6, 6).astype(np.float32); ws = (rng.randn(4, 4, 3, 3) * 0.2).astype(np.float32)
 
     def run(fused):
-        T.FUSE_BN_ADD_RELU = fused
+        _fusion(be, fused)
         try:
             x = TensorR(Tensor.fromNumpy(xs)); w = TensorR(Tensor.fromNumpy(ws))
             g = TensorR(Tensor.fromData((4,), 1.5, 0.5, 2.0, 1.0)); b = TensorR(Tensor.fromData((4,), 0.1, -0.2, 0.0, 0.3))
@@ -114,22 +167,23 @@ def test_residual_join_absorbs_the_batchnorm_and_matches_the_unfused_program(on_
                 y = h.convBBP(w, None, (1, 1), (1, 1)).batchNorm(g, b, Tensor.zeros(4), Tensor.ones(4))
                 kept["bn"] = y
                 z = (y + h) if bn_side == "left" else (h + y)
-                assert (T._pending is not None and T._pending.owner is z)
                 out = z.relu(True)
-                kept["out"] = out.x.toCPU().copy()
+                kept["z"] = out
                 return (out * out).sum()
             gradR_loss(f)(Tensor.zeros(1))
-            return kept, [kept["out"], x.d.toCPU(), w.d.toCPU(), g.d.toCPU(), b.d.toCPU()]
+            res = [kept["z"].x.toCPU(), x.d.toCPU(), w.d.toCPU(), g.d.toCPU(), b.d.toCPU()]
+            # read last: what the fused chain did not store (the batch norm's output, its gradient buffer = the masked gradient,
+            # and the join's gradient buffer masked in place by relu_grad)
+            res += [kept["bn"].x.toCPU(), kept["bn"].d.toCPU(), kept["z"].d.toCPU()]
+            return res
         finally:
-            T.FUSE_BN_ADD_RELU = True
-    kf, fused = run(True)
-    ku, plain = run(False)
-    assert kf["bn"].x is None and ku["bn"].x is not None          # absorbed: reading the batchNorm's output later fails loudly
+            _fusion(be, True)
+    fused, plain = run(True), run(False)
     for u, v in zip(fused, plain):
         np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)
 
 
-def test_batchnorm_followed_by_add_without_relu_runs_unfused(on_cpu):
+def test_batchnorm_followed_by_add_without_relu_runs_unfused(be):
     rng = np.random.RandomState(4)
     xs = rng.randn(3, 2, 4, 4).astype(np.float32)
     x = TensorR(Tensor.fromNumpy(xs)); g, b = TensorR(Tensor.ones(2)), TensorR(Tensor.zeros(2))
@@ -146,24 +200,24 @@ def test_batchnorm_followed_by_add_without_relu_runs_unfused(on_cpu):
 def test_join_whose_shortcut_is_the_batchnorms_own_input(be):
     """relu(bn(h) + h): the batch norm's input is also the shortcut, so the fused backward would be handed one buffer for both of
     its gradient outputs (its first pass adds the masked gradient into what its second pass overwrites, losing the shortcut's
-    share).  The mirror runs this join unfused; values and gradients equal the program with the fusion switched off."""
+    share).  The library runs this join unfused; values and gradients equal the program with the fusion switched off."""
     rng = np.random.RandomState(5)
     xs = rng.randn(4, 3, 5, 5).astype(np.float32)
 
     def run(fused):
-        T.FUSE_BN_ADD_RELU = fused
+        _fusion(be, fused)
         try:
             x = TensorR(Tensor.fromNumpy(xs)); g = TensorR(Tensor.fromData((3,), 1.5, 0.5, 2.0)); b = TensorR(Tensor.fromData((3,), 0.1, -0.2, 0.3))
             kept = {}
             def f(d):
                 h = x * 1.5
                 out = (h.batchNorm(g, b, Tensor.zeros(3), Tensor.ones(3)) + h).relu(True)
-                kept["out"] = out.x.toCPU().copy()
+                kept["out"] = out
                 return (out * out).sum()
             gradR_loss(f)(Tensor.zeros(1))
-            return [kept["out"], x.d.toCPU(), g.d.toCPU(), b.d.toCPU()]
+            return [kept["out"].x.toCPU(), x.d.toCPU(), g.d.toCPU(), b.d.toCPU()]
         finally:
-            T.FUSE_BN_ADD_RELU = True
+            _fusion(be, True)
     fused, plain = run(True), run(False)
     for u, v in zip(fused, plain):
         np.testing.assert_allclose(u, v, rtol=1e-5, atol=1e-6)

@@ -115,9 +115,12 @@ def test_literal_c_text_names_declared_functions():
 # Declared operators the Scala backend has no call for, with the reason.  Everything else it does not call must be runtime
 # plumbing (error mode, events, pinned memory, capture, tuning switches), which generated programs reach by name if at all.
 NOT_CALLED = {
-    # fused forms that the host-side tape chooses when it sees the pattern; the trait's one-op-per-method surface cannot express them
+    # fused forms: the backend emits the trait's one call per method, and the LIBRARY runs these when it recognises the chain
+    # (conv -> batchNorm -> [+] -> relu in place, their gradients, runs of optimizer calls); they stay callable for hand-written hosts
     "lh_add_relu", "lh_add_relu_grad", "lh_bn_apply", "lh_bn_apply_add_relu", "lh_bn_bwd_add_relu", "lh_bn_bwd_relu", "lh_bn_stats",
-    "lh_bn_train_fwd_relu", "lh_conv2d_fwd_bnstats", "lh_concat_grad_beta",
+    "lh_bn_train_fwd_relu", "lh_conv2d_fwd_bnstats", "lh_conv2d_fwd_bn_apply", "lh_concat_grad_beta", "lh_multi_momentum", "lh_multi_sgd",
+    # outputs the backend allocates come from lh_malloc (zero-filled, cleared on demand): the uncleared form is for hand-written hosts
+    # (the code generator still emits it for literal arrays it uploads at once)
     # superseded within the trait mapping: padded average pooling covers pad 0; the dense max-pool gradient replaces the scatter form
     "lh_avgpool_fwd", "lh_avgpool_bwd", "lh_maxpool_bwd",
     # the zero-state forms: the backend always calls the *_init forms, with NULL for a state it was not given
@@ -128,7 +131,7 @@ NOT_CALLED = {
     "lh_cifar_decode",
 }
 PLUMBING = re.compile(r"^lh_(set_|get_|last_error|clear_error|sync|heap_|free_top|host_|h2d_async|d2h_async|copy_join|capture_|graph_|tune_|"
-                      r"side_forks|side_join|event_|prof_|cmdlist_|multi_momentum_static)")
+                      r"side_forks|side_join|event_|prof_|cmdlist_|multi_momentum_static|flush_deferred|fusion_stats|work_collect)")
 
 
 def test_the_backend_uses_the_whole_operator_surface():
