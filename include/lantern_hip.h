@@ -142,7 +142,7 @@ void lh_graph_destroy(int graph);
  * level by level: commands that do not depend on each other side by side (element-wise commands dealt over 32 workgroups,
  * LH_CMDLIST_GROUPS in the environment overrides; the matrix commands cut by rows or columns over the wavefronts of all of
  * them), a barrier over the workgroups between levels.  The barrier's wait is bounded: if a workgroup never arrives the
- * kernel ends, and the next call that touches the command list reports it.  Results equal those of the stand-alone kernels
+ * kernel ends, and the next lh_sync, lh_d2h, hand-over of recorded commands or lh_cmdlist_end reports it.  Results equal those of the stand-alone kernels
  * up to summation order in the reductions; no command uses atomic adds and every sum has a fixed order, so two runs give the
  * same bits whatever the number of workgroups.  Element-wise commands that depend only on each other lane by lane, and matrix
  * commands that write the same rows, share a level (chains; LH_CMDLIST_CHAINS=0 turns them off); chains of six and more element-wise
@@ -152,6 +152,10 @@ void lh_graph_destroy(int graph);
  * lh_setup(). */
 void lh_cmdlist_begin(void);
 void lh_cmdlist_end(void);
+/* A test aid: sets, from the host, the flag a workgroup sets when its barrier wait runs out, so that the reporting and
+ * recovery path (the next lh_sync, lh_d2h, hand-over or lh_cmdlist_end reports "timed out" once and leaves the library
+ * usable) can be exercised without a kernel that gives up. */
+void lh_cmdlist_inject_timeout(void);
 /* Commands recorded and interpreter launches since lh_setup (either pointer may be NULL). */
 void lh_cmdlist_stats(int64_t* recorded, int64_t* launches);
 void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat);
@@ -383,7 +387,8 @@ void lh_conv2d_fwd_bn_apply(const float* x, const float* w, const float* bias, f
  * (from lh_conv2d_fwd_bnstats or lh_bn_stats), one pass.  Its backward, given dout = d loss / d out:
  *   g = dout where out > 0 else 0;   ds = beta_ds * ds + g;   dx = beta_dx * dx + batch-norm backward of g;
  *   dgamma += sum g * xhat;  dbeta += sum g.
- * When ds accumulates (beta_ds = 1) or is NULL, dout is overwritten with g.  dx may be NULL (no input gradient). */
+ * dout is unspecified after the call: some paths overwrite it with g (two passes with ds accumulating or NULL), the others
+ * leave it as it was.  dx may be NULL (no input gradient). */
 void lh_bn_apply_add_relu(const float* x, const float* gamma, const float* beta, const float* save_mean, const float* save_invstd,
                           const float* shortcut, float* out, int N, int C, int HW);
 void lh_bn_bwd_add_relu(const float* x, const float* out, float* dout, const float* gamma, const float* save_mean, const float* save_invstd,

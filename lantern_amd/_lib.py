@@ -54,6 +54,7 @@ SIGNATURES = {
     "lh_graph_destroy": (None, [I]),
     "lh_cmdlist_begin": (None, []),
     "lh_cmdlist_end": (None, []),
+    "lh_cmdlist_inject_timeout": (None, []),
     "lh_cmdlist_stats": (None, [C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
     "lh_prof_collect": (None, [P, P, I]),
     "lh_set_fusion": (None, [I]),

@@ -45,7 +45,7 @@ constexpr int CL_START_SHIFT = 12;            // 12 bits: where the command's wo
 constexpr int CL_BARRIERS_SHIFT = 24;         // 8 bits: barriers over all workgroups to pass before the entry (levels completed since the last one)
 constexpr int CL_WBLOCK = 4;                  // wavefronts of all workgroups are numbered in blocks of 4 of one workgroup, the blocks dealt
                                               // round the workgroups: the pieces of a 150-row product fall to 4 workgroups, not to 15
-constexpr long CL_SPIN_LIMIT = 40000000L;     // polls of a grid barrier before a workgroup gives up (far beyond any real wait)
+constexpr long CL_SPIN_LIMIT = 4000000L;      // polls of a grid barrier before a workgroup gives up: a few seconds, where a real wait is one level of commands (microseconds)
 
 static bool g_slots = true;           // LH_CMDLIST_SLOTS=0 in the environment: chains read and write memory only
 static bool g_chains = true;          // LH_CMDLIST_CHAINS=0 in the environment: every dependent command opens a new level
@@ -765,21 +765,28 @@ static long long g_stat_slot_chains = 0, g_stat_slots = 0, g_stat_chain_ptrs = 0
 static unsigned long long g_tsc_push = 0, g_tsc_flush = 0, g_tsc_wait = 0;      // host cycles spent recording (LH_CMDLIST_VERBOSE prints them)
 // Hands the recorded buffer to the device: commands in level order (recording order within a level), the first of each
 // level flagged for a barrier, each with the wavefront its elements start on.
+// An interpreter launch whose barrier wait ran out leaves a flag in pinned host memory.  Whoever looks next (the next
+// hand-over, lh_cmdlist_end, lh_sync, lh_d2h) reports it, with the barrier counters and the window put back so that the
+// library stays usable; the results of that buffer are incomplete.
+bool cmdlist_report_timeout() {
+  Ring& r = g_ring;
+  if (r.host_flag == nullptr || *(volatile unsigned*)r.host_flag == 0) return false;
+  (void)hipStreamSynchronize(g_stream_raw);
+  (void)hipMemset(r.sync, 0, 2 * sizeof(unsigned long long));
+  *r.host_flag = 0; r.sync_base = 0;
+  if (g_win) window_reset(*g_win);
+  g_rec_pending = 0;
+  LH_FAIL("command list: a barrier between workgroups timed out; the commands of that buffer did not all run");
+  return true;
+}
 void rec_flush() {
+  if (cmdlist_report_timeout()) return;
   if (g_rec_pending <= 0 || g_win == nullptr) return;
   const unsigned long long f0 = __builtin_ia32_rdtsc();
   Window& W = *g_win;
   const int n = W.n;
   g_rec_pending = 0;                                  // before any use of the stream below
   Ring& r = g_ring;
-  if (*(volatile unsigned*)r.host_flag != 0) {        // an earlier launch left its barrier: its results are incomplete
-    (void)hipStreamSynchronize(g_stream_raw);
-    (void)hipMemset(r.sync, 0, 2 * sizeof(unsigned long long));
-    *r.host_flag = 0; r.sync_base = 0;
-    window_reset(W);
-    LH_FAIL("command list: a barrier between workgroups timed out; the commands of that buffer did not all run");
-    return;
-  }
   const int groups = r.groups, all_w = groups * (CL_THREADS / 64);
   static int start[CL_BUF_CMDS + 2], order[CL_BUF_CMDS];
   for (int l = 0; l <= W.top + 1; l++) start[l] = 0;
@@ -1094,10 +1101,15 @@ void lh_cmdlist_begin(void) {
 void lh_cmdlist_end(void) {
   rec_flush();
   g_rec_on = 0;
+  (void)cmdlist_report_timeout();
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld commands in %lld levels, %lld launches\n", (long long)g_ring.recorded, (long long)g_ring.levels, (long long)g_ring.launches);
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %d operand slots per workgroup\n", g_ring.nslot);
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list: %lld chains run as programs, %lld operand slots, %lld commands in them\n", g_stat_slot_chains, g_stat_slots, g_stat_chain_ptrs);
   if (getenv("LH_CMDLIST_VERBOSE")) fprintf(stderr, "command list host cycles: push %.1f M (flush inside %.1f M, of which waiting for a free buffer %.1f M)\n", g_tsc_push * 1e-6, g_tsc_flush * 1e-6, g_tsc_wait * 1e-6);
+}
+void lh_cmdlist_inject_timeout(void) {
+  LH_REQUIRE(g_ring.host_flag != nullptr, "lh_cmdlist_inject_timeout before the first lh_cmdlist_begin");
+  *(volatile unsigned*)g_ring.host_flag = 1u;       // what a workgroup whose barrier wait ran out writes
 }
 void lh_cmdlist_stats(int64_t* recorded, int64_t* launches) {
   if (recorded) *recorded = g_ring.recorded;

@@ -18,6 +18,7 @@ void quiet_other_stream();        // host-side wait for the stream that is NOT c
 extern int g_rec_pending;
 void rec_flush();
 void cmdlist_release();           // frees the command buffers (lh_cleanup)
+bool cmdlist_report_timeout();    // true (and an error reported) if an interpreter launch gave up at a barrier since the last look
 bool multi_tensor_setup();        // the multi-tensor optimizers' device table: reserved by lh_setup, freed by lh_cleanup
 void multi_tensor_release();
 // Deferred work (lh_defer.hip): launches parked until the next call shows whether it fuses with them, zero fills of arena

@@ -168,6 +168,7 @@ void lh_sync(void) {
   side_join();
   lh_copy_join();
   LH_HIP(hipStreamSynchronize(g_stream)); LH_CHECK_LAUNCH();
+  (void)cmdlist_report_timeout();      // the wait is over: a barrier that gave up in a command-list launch is reported now, not at the next hand-over
 }
 
 static void* bump(size_t bytes, bool zero) {
@@ -275,6 +276,7 @@ void lh_d2h(void* h_dst, const void* src, size_t bytes) {
   lh_copy_join();    // an upload still on the copy stream may be what is read back
   LH_HIP(hipMemcpyAsync(h_dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
   LH_HIP(hipStreamSynchronize(g_stream));
+  (void)cmdlist_report_timeout();
 }
 // ---- transfers that do not stall the step: pinned host memory, a copy stream for uploads, read-backs without a wait ----
 static hipStream_t g_copy_stream = nullptr;

@@ -213,3 +213,111 @@ def test_onnx_built_networks_train_like_the_hand_built_applications(tmp_path, hi
     finally:
         be.setDeterministic(False)
         be.sync(); be.resetMallocAddr(mark)
+
+
+def _export(tmp_path, kind, N, cpu_backend, unit_variance=False):
+    """The hand-built application, initialised on the oracle backend, written out as an ONNX file; returns the path.
+    `unit_variance`: running variances of one instead of the initial zeros (NN:168-182), so that the inference function
+    (which divides by sqrt(runningVar + 1e-5)) gives values of ordinary size."""
+    from lantern_amd.nn import BatchNorm2D
+    la.set_backend(cpu_backend)
+    if kind == "resnet":
+        from lantern_amd.apps.resnet50 import ResNet50
+        model = ResNet50(num_classes=10, imagenet_stem=False, layers=(1, 1, 1, 1))
+    else:
+        from lantern_amd.apps.squeezenet import SqueezeNet
+        model = SqueezeNet(10)
+    if unit_variance:
+        todo = [model]
+        while todo:
+            m = todo.pop()
+            todo += list(m._children)
+            if isinstance(m, BatchNorm2D):
+                m.runningVar.fillInPlace(1.0)
+    b = GraphBuilder("input", [N, 3, 32, 32])
+    h = export_module_tree(b, kind, model, "input")
+    if kind == "resnet":
+        h = b.node("AveragePool", [h], ["avg"], kernel_shape=[2, 2], strides=[1, 1], pads=[0, 0, 0, 0])
+        h = b.node("Flatten", [h], ["flat"], axis=1)
+        h = b.node("Gemm", [h, b.init("fc.weight", model.fc_w.x.toCPU()), b.init("fc.bias", model.fc_b.x.toCPU())], ["out"], alpha=1.0, beta=1.0, transB=1)
+    else:
+        h = b.node("Reshape", [h, b.init("shape", np.array([N, -1], np.int64))], ["out"])
+    return b.save(str(tmp_path / (kind + ".onnx")), "out", [N, 10])
+
+
+class _OnnxTrainer:
+    """The reference's training loop over a model read from a file (resnet50FromOnnx.scala:150-191), in the shape the tracking
+    tests drive: step() returns the loss, end_step() rewinds the arena."""
+
+    def __init__(self, path, x, y, lr):
+        from lantern_amd.nn import SGD_Momentum
+        be = la.get_backend()
+        self.model = OnnxModel(path)
+        self.opt = SGD_Momentum(self.model, lr, 0.9)
+        self.x, self.target = Tensor.fromNumpy(x), int_array(y)
+        self.mark = be.getMallocAddr()
+
+    def step(self):
+        xin = TensorR(self.x, isInput=True)
+        loss = gradR_loss(lambda d: self.model(xin).logSoftmaxB(1).nllLossB(self.target).mean())(Tensor.zeros(1))
+        self.opt.step()
+        return loss
+
+    def end_step(self):
+        la.get_backend().resetMallocAddr(self.mark)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["resnet", "squeezenet"])
+def test_onnx_built_networks_track_the_oracle_on_the_device(tmp_path, hip_backend, cpu_backend, kind):
+    """The same readONNX program (training_func: ONNXLib.scala:833-1071) on the device and on the oracle backend, five steps
+    of momentum SGD: every loss and every parameter within the tracking bounds of tests/test_training_parity.py."""
+    from tests.test_training_parity import _compare
+    N = 8
+    rng = np.random.RandomState(3)
+    x = rng.randn(N, 3, 32, 32).astype(np.float32); y = rng.randint(0, 10, size=N).astype(np.int32)
+    path = _export(tmp_path, kind, N, cpu_backend)
+    _compare(lambda: _OnnxTrainer(path, x, y, 0.005), hip_backend, cpu_backend, steps=5, self_calibrate=True, flip_tol=2e-2)
+
+
+@pytest.mark.gpu
+def test_onnx_inference_func_on_the_device_against_the_oracle(tmp_path, hip_backend, cpu_backend):
+    """inference_func (ONNXLib.scala:597-830) on the device: batchNormInference, a max-pool and an average pool WITH pads,
+    a residual add, Flatten, Gemm with alpha / beta and softmax_batch, against the same program on the oracle backend; then the
+    ResNet and SqueezeNet files' inference functions."""
+    from tests.util import assert_close
+    rng = np.random.RandomState(7)
+    f32 = lambda a: np.asarray(a, np.float32)
+    b = GraphBuilder("x", [4, 3, 17, 17])
+    h = b.node("Conv", ["x", b.init("w1", f32(rng.randn(8, 3, 3, 3) * 0.3)), b.init("b1", f32(rng.randn(8) * 0.1))], ["c1"], kernel_shape=[3, 3], strides=[1, 1], pads=[1, 1, 1, 1])
+    h = b.node("BatchNormalization", [h, b.init("g", f32(rng.rand(8) + 0.5)), b.init("be", f32(rng.randn(8) * 0.1)), b.init("rm", f32(rng.randn(8) * 0.1)),
+                                      b.init("rv", f32(rng.rand(8) + 0.5))], ["bn"], epsilon=1e-5, momentum=0.9)
+    h = b.node("Relu", [h], ["r1"])
+    p = b.node("MaxPool", [h], ["mp"], kernel_shape=[3, 3], strides=[2, 2], pads=[1, 1, 1, 1])                    # 17 -> 9, real padding
+    m = b.node("Conv", [p, b.init("w2", f32(rng.randn(8, 8, 3, 3) * 0.2))], ["c2"], kernel_shape=[3, 3], strides=[1, 1], pads=[1, 1, 1, 1])
+    h = b.node("Relu", [b.node("Add", [m, p], ["a1"])], ["r2"])
+    h = b.node("AveragePool", [h], ["ap"], kernel_shape=[3, 3], strides=[2, 2], pads=[1, 1, 1, 1])              # 9 -> 5, divisor counts the image only
+    h = b.node("Flatten", [h], ["fl"], axis=1)
+    h = b.node("Gemm", [h, b.init("fw", f32(rng.randn(200, 6) * 0.1)), b.init("fb", f32(rng.randn(6) * 0.1))], ["gm"], alpha=0.5, beta=2.0)
+    h = b.node("Softmax", [h], ["sm"])
+    path = b.save(str(tmp_path / "infer.onnx"), "sm", [4, 6])
+    x = rng.randn(4, 3, 17, 17).astype(np.float32)
+
+    def infer(be, path, x):
+        la.set_backend(be)
+        mark = be.getMallocAddr()
+        try:
+            m = readONNX(path)
+            return m.inference_func(m.initializer_map_tensor())(Tensor.fromNumpy(x)).toCPU().copy()
+        finally:
+            be.resetMallocAddr(mark)
+    want, got = infer(cpu_backend, path, x), infer(hip_backend, path, x)
+    assert want.shape == (4, 6) and np.allclose(want.sum(1), 1.0, atol=1e-5)
+    assert_close(got, want, rtol=1e-4, what="inference_func: bn inference, padded pools, gemm alpha/beta, softmax")
+    # the two application networks as files: logits of the inference function (running statistics as initialised)
+    for kind in ("resnet", "squeezenet"):
+        path = _export(tmp_path, kind, 4, cpu_backend, unit_variance=True)
+        xs = rng.randn(4, 3, 32, 32).astype(np.float32)
+        want, got = infer(cpu_backend, path, xs), infer(hip_backend, path, xs)
+        assert np.isfinite(want).all() and np.abs(want).max() > 0
+        assert_close(got, want, rtol=1e-4, what="inference_func of the %s file" % kind)

@@ -975,6 +975,38 @@ def test_command_list_matches_one_launch_per_operator(on_hip, n, m):
         assert_close(a, b_, rtol=2e-6 if n <= 150 else 1e-4, what="result %d" % i)
 
 
+def test_command_list_reports_a_barrier_that_gave_up_and_stays_usable(on_hip):
+    """A workgroup whose barrier wait runs out sets a flag in pinned host memory and all workgroups leave.  The flag is set
+    from the host here (no kernel is made to give up): the next call that waits for the device reports it once, also when
+    nothing is pending, the barrier counters start over, and the same commands then run and give the right result."""
+    be = on_hip
+    lib = be.lib
+    one = be.fromHost(np.ones(64, np.float32))
+    be.batchSmallOps(True)
+    try:
+        acc = be.mallocArray(64)
+        for _ in range(5):
+            lib.lh_bcast_update(B.ADD, acc.ptr, B._ints((64,)), one.ptr, B._ints((64,)), 1)
+        be.sync()                                                               # handed over and finished: nothing pending now
+        lib.lh_cmdlist_inject_timeout()
+        with pytest.raises(LanternHipError, match="timed out"):
+            be.sync()                                                           # reported although no command is pending
+        be.sync()                                                               # once
+        lib.lh_cmdlist_inject_timeout()
+        with pytest.raises(LanternHipError, match="timed out"):
+            be.toHost(acc, 64)                                                  # a read-back reports it too
+        for _ in range(7):                                                      # the library is usable: levels and barriers start over
+            lib.lh_bcast_update(B.ADD, acc.ptr, B._ints((64,)), one.ptr, B._ints((64,)), 1)
+        assert (be.toHost(acc, 64) == 12.0).all()
+        lib.lh_cmdlist_inject_timeout()
+        lib.lh_cmdlist_end()                                                    # lh_cmdlist_end reports it as well
+        with pytest.raises(LanternHipError, match="timed out"):
+            la._lib.check()
+    finally:
+        be.batchSmallOps(False)
+    be.sync()
+
+
 def test_command_list_keeps_program_order_around_other_kernels_and_wraps_its_buffers(on_hip):
     """Recorded commands, kernels too large to record and copies interleave in program order; more commands than the
     pinned buffers hold in total go through without loss."""

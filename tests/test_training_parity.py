@@ -73,7 +73,7 @@ def _mask_flips(m_hip, m_ref):
     return out
 
 
-def _compare(make_trainer, hip_backend, cpu_backend, steps=10, tol=1e-3, per_tensor=1e-3, self_calibrate=False, flip_tol=None):
+def _compare(make_trainer, hip_backend, cpu_backend, steps=10, tol=1e-3, per_tensor=1e-3, self_calibrate=False, flip_tol=None, deterministic=True):
     """Tracking criteria (the north-star bar: loss and parameters after 10 steps within 1e-3 of the CPU reference).
     The device runs in deterministic mode (fixed-order reductions, rule-chosen launch plans), so the numbers below
     are the same in every run:
@@ -93,7 +93,9 @@ def _compare(make_trainer, hip_backend, cpu_backend, steps=10, tol=1e-3, per_ten
     then counts on one side only, and in a small batch that moves bias gradients (sums that nearly cancel) by
     several 1e-3 from the next step on.  With `flip_tol` the relu masks of both runs are recorded step by step and compared;
     if, and only if, they differ, the flips are printed and the steps after the first flip, and the parameters, are held to
-    `flip_tol` instead.  A run without a flip is held to `tol` throughout."""
+    `flip_tol` instead.  A run without a flip is held to `tol` throughout.
+    `deterministic=False`: the device runs as it is benchmarked (partial sums combined with atomic adds, launch plans chosen by
+    measurement, filter gradients on the side stream); the numbers then move in their last digits from run to run."""
     m_ref = [] if flip_tol is not None else None
     m_hip = [] if flip_tol is not None else None
     l_ref, p_ref = _run(make_trainer, cpu_backend, steps, masks=m_ref)
@@ -104,7 +106,7 @@ def _compare(make_trainer, hip_backend, cpu_backend, steps=10, tol=1e-3, per_ten
         print("oracle against itself after a one-ulp nudge: loss %.3g, parameters %.3g" % (
             float(np.max(np.abs(l_nudged - l_ref) / np.abs(l_ref))),
             _rel(np.concatenate([a.ravel() for _, a in p_nudged]), np.concatenate([b.ravel() for _, b in p_ref]))))
-    hip_backend.setDeterministic(True)
+    hip_backend.setDeterministic(deterministic)
     try:
         l_hip, p_hip = _run(make_trainer, hip_backend, steps, masks=m_hip)
     finally:
@@ -191,6 +193,32 @@ def test_resnet_bottlenecks_momentum_10_steps(hip_backend, cpu_backend):
     from lantern_amd.apps.resnet50 import ResNet50, Trainer
     _compare(lambda: Trainer(ResNet50(num_classes=10, imagenet_stem=False, layers=(1, 1, 1, 1)), 16, 32, 10, lr=0.001, momentum=0.9),
              hip_backend, cpu_backend, self_calibrate=True)
+
+
+def test_resnet_two_bottlenecks_per_stage_5_steps(hip_backend, cpu_backend):
+    """layers = (2, 2, 2, 2): every stage has a block WITHOUT a downsample branch behind its first one (the identity shortcut
+    of the residual join, a block input that collects two gradients), which one block per stage does not reach."""
+    from lantern_amd.apps.resnet50 import ResNet50, Trainer
+    # 2x2 maps in the last stage: batch norms over 64 values put relu inputs within rounding of zero from the first step on (a
+    # handful of mask flips against the oracle at step 0, thousands by step 4), hence flip_tol; measured: loss within 7e-4, parameters 5e-5
+    _compare(lambda: Trainer(ResNet50(num_classes=10, imagenet_stem=False, layers=(2, 2, 2, 2)), 16, 32, 10, lr=0.0005, momentum=0.9),
+             hip_backend, cpu_backend, steps=5, self_calibrate=True, flip_tol=2e-2)
+
+
+@pytest.mark.parametrize("net", ["squeezenet_b16", "resnet_1111"])
+def test_ten_steps_in_the_benchmarked_mode_track_the_oracle(hip_backend, cpu_backend, net):
+    """The configuration bench.py times (atomic combines, measured launch plans, filter gradients on the side stream), not
+    the deterministic mode of the other tests: ten steps against the oracle, loss and parameters within 2e-3 (the summation
+    order of the atomic combines differs from run to run, so the deviation printed here moves in its last digits)."""
+    if net == "squeezenet_b16":
+        from lantern_amd.apps.squeezenet import Trainer
+        mk = lambda: Trainer(batch=16, lr=0.001)
+    else:
+        from lantern_amd.apps.resnet50 import ResNet50, Trainer
+        mk = lambda: Trainer(ResNet50(num_classes=10, imagenet_stem=False, layers=(1, 1, 1, 1)), 16, 32, 10, lr=0.001, momentum=0.9)
+    forks0 = hip_backend.lib.lh_side_forks()
+    _compare(mk, hip_backend, cpu_backend, tol=2e-3, per_tensor=2e-3, self_calibrate=True, deterministic=False)
+    assert hip_backend.lib.lh_side_forks() > forks0, "the filter gradients were to run on the side stream"
 
 
 def test_resnet_imagenet_stem_3_steps(hip_backend, cpu_backend):

@@ -56,3 +56,50 @@ def test_static_table_rejects_more_tensors_than_it_holds(on_hip):
     be.lib.lh_multi_momentum_static(n, ptrs, ptrs, ptrs, ns, 0.1, 0.9, 1.0, 0)
     with pytest.raises(_lib.LanternHipError, match="at most 4096"):
         _lib.check()
+
+
+def test_static_table_update_recorded_into_a_graph_carries_its_own_table(on_hip):
+    """The table array is shared by every call on the GPU.  A call recorded into a graph records its table writes with it, and
+    an eager call never trusts what an earlier call left in the array: eager on set A, recording on set A, eager on set B,
+    a replay (set A again), eager on set A: every update lands on the tensors it was given, bit for bit what
+    lh_multi_momentum gives for the same sequence."""
+    be, lib = on_hip, on_hip.lib
+    rng = np.random.RandomState(9)
+    size_a, size_b = [300, 4096 * 3 + 5, 17, 70000], [5, 9000]
+    host = {k: [(rng.randn(n).astype(np.float32), rng.randn(n).astype(np.float32), rng.randn(n).astype(np.float32)) for n in sizes]
+            for k, sizes in (("a", size_a), ("b", size_b))}
+
+    def run(static):
+        bufs = {k: [(be.fromHost(x.copy()), be.fromHost(d.copy()), be.fromHost(v.copy()), x.size) for x, d, v in host[k]] for k in host}
+        tabs = {k: _tables(bufs[k]) for k in bufs}
+        entry = lib.lh_multi_momentum_static if static else lib.lh_multi_momentum
+        def call(k):
+            entry(*tabs[k], 0.1, 0.9, 2.0, 0); _lib.check()
+        def regrad(k, scale):
+            for (x, d, v), b in zip(host[k], bufs[k]):
+                be.upload(b[1], d * np.float32(scale))
+        call("a")                                   # eager, set A
+        regrad("a", 2.0)
+        graph = None
+        if static:
+            be.sync()
+            be.captureBegin()
+            call("a")                               # recorded, not run
+            graph = be.captureEnd()
+        call("b")                                   # eager, set B: the array now holds B's entries
+        if static:
+            be.graphLaunch(graph)                   # the replay writes A's entries itself
+        else:
+            call("a")
+        regrad("a", 3.0)
+        call("a")                                   # eager, set A again
+        be.sync()
+        out = {k: [tuple(be.toHost(b[j], b[3]) for j in range(3)) for b in bufs[k]] for k in bufs}
+        if graph is not None:
+            be.graphDestroy(graph)
+        return out
+    want, got = run(False), run(True)
+    for k in want:
+        for t, (w, g) in enumerate(zip(want[k], got[k])):
+            for name, a, b in zip(("x", "d", "v"), g, w):
+                np.testing.assert_array_equal(a, b, err_msg="set %s tensor %d %s" % (k, t, name))
