@@ -668,7 +668,7 @@ static void bn_fwd_declare(const float* x, const float* gamma, const float* beta
   const int64_t n = (int64_t)N * C * HW;
   lazy::flush_parked();
   lazy::rd_f(x, n); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rw_f(run_mean, C); lazy::rw_f(run_var, C);
-  if (y != x) lazy::wr_f(y, n);
+  lazy::out_f(y, n, y == x);
   lazy::wr_f(save_mean, C); lazy::wr_f(save_invstd, C);
 }
 // returns the beta to run with: 1 on a gradient buffer nobody has touched since lh_malloc becomes 0
@@ -705,7 +705,7 @@ void lh_bn_apply(const float* x, const float* gamma, const float* beta, const fl
                  int N, int C, int HW, int relu) {
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_apply: empty shape [%d,%d,%d]", N, C, HW);
   LZ_ENTER(); lazy::rd_f(x, (int64_t)N * C * HW); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rd_f(save_mean, C); lazy::rd_f(save_invstd, C);
-  if (y != x) lazy::wr_f(y, (int64_t)N * C * HW);
+  lazy::out_f(y, (int64_t)N * C * HW, y == x);
   ProfScope prof_(CAT_BN_FWD);
   work_add(CAT_BN_FWD, 8.0 * N * C * (double)HW);
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)y) & 15) == 0);
@@ -722,7 +722,7 @@ void lh_bn_infer(const float* x, const float* gamma, const float* beta, const fl
   int64_t n = (int64_t)N * C * HW;
   if (n <= 0) return;
   LZ_ENTER(); lazy::rd_f(x, n); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rd_f(run_mean, C); lazy::rd_f(run_var, C);
-  if (y != x) lazy::wr_f(y, n);
+  lazy::out_f(y, n, y == x);
   ProfScope prof_(CAT_BN_FWD);
   work_add(CAT_BN_FWD, 8.0 * (double)n);
   hipLaunchKernelGGL(k_bn_infer, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, x, y, gamma, beta, run_mean, run_var, C, HW, n, eps);
@@ -856,7 +856,7 @@ void lh_bn_apply_add_relu(const float* x, const float* gamma, const float* beta,
   LH_REQUIRE(N > 0 && C > 0 && HW > 0, "lh_bn_apply_add_relu: empty shape [%d,%d,%d]", N, C, HW);
   LH_REQUIRE(x && shortcut && out && gamma && beta && save_mean && save_invstd, "lh_bn_apply_add_relu: null operand");
   LZ_ENTER(); lazy::rd_f(x, (int64_t)N * C * HW); lazy::rd_f(shortcut, (int64_t)N * C * HW); lazy::rd_f(gamma, C); lazy::rd_f(beta, C); lazy::rd_f(save_mean, C); lazy::rd_f(save_invstd, C);
-  if (out != x && out != shortcut) lazy::wr_f(out, (int64_t)N * C * HW);
+  lazy::out_f(out, (int64_t)N * C * HW, out == x || out == shortcut);
   ProfScope prof_(CAT_BN_FWD);
   work_add(CAT_BN_FWD, 12.0 * N * C * (double)HW);
   Plan p = make_plan(N, C, HW, (((uintptr_t)x | (uintptr_t)out | (uintptr_t)shortcut) & 15) == 0);

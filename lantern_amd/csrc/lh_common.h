@@ -5,6 +5,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include "../../include/lantern_hip.h"
+#include "lh_cmd.h"
 
 namespace lh {
 
@@ -138,6 +139,9 @@ static inline void rd_f(const void* p, int64_t n) { if (g_busy && p && n > 0) rd
 static inline void wr_f(const void* p, int64_t n) { if (g_busy && p && n > 0) wr(p, (size_t)n * 4); }
 static inline void rw_f(const void* p, int64_t n) { if (g_busy && p && n > 0) rw(p, (size_t)n * 4); }
 static inline bool acc_f(const void* p, int64_t n) { return g_busy && p && n > 0 ? acc(p, (size_t)n * 4) : false; }
+// an output that may be one of the inputs (in-place forms): then it is read and written, and whatever was still to be produced
+// from its old contents is produced first
+static inline void out_f(const void* p, int64_t n, bool aliases_an_input) { if (aliases_an_input) rw_f(p, n); else wr_f(p, n); }
 // accumulate with a beta the caller passed: 1 on a block nobody has touched becomes 0; 0 is a plain overwrite
 static inline float beta_f(const void* p, int64_t n, float beta) {
   if (!g_busy || !p || n <= 0) return beta;
@@ -178,13 +182,6 @@ void zero_bytes_async(void* p, size_t bytes);      // bytes a multiple of 256
 // While recording is on (lh_cmdlist_begin), an entry point whose operands are small enough appends a command instead
 // of launching a kernel; a tree-structured model of 150-element vectors issues thousands of such operations per
 // step, and the host's launch rate is what bounds it.
-enum {
-  CL_ZERO16 = 0, CL_FILL, CL_COPY, CL_GEAM, CL_SCALAR, CL_BIN, CL_ACC, CL_ACCNEG, CL_ACCMUL, CL_UNARY, CL_UNARY_GRAD,
-  CL_GEMV_N, CL_GEMV_T, CL_GER, CL_DOT, CL_AXPY_DEV, CL_SOFTMAX, CL_SOFTMAX_GRAD, CL_NLL, CL_NLL_GRAD, CL_ADAGRAD, CL_SGD
-};
-struct LhCmd { int32_t op, i0, i1, i2; float f0, f1, f2, f3; void* p0; void* p1; void* p2; void* p3; };   // 64 bytes
-constexpr int64_t REC_MAX_ELEMS = 1 << 16;        // element-wise operands up to this many elements are recorded
-constexpr int64_t REC_MAX_MATRIX = 1 << 17;       // matrix-vector operands up to this many matrix elements
 extern int g_rec_on;
 bool rec_push(const LhCmd& c);                     // appends a command (launches a full buffer first); false on error
 static inline bool rec_ok(int64_t n, int64_t limit = REC_MAX_ELEMS) { return g_rec_on && n <= limit; }
@@ -208,7 +205,8 @@ static inline int stream_grid(int64_t n, int per_block) {
 
 }  // namespace lh
 
-// ---- device helpers -------------------------------------------------------
+// ---- device helpers (absent when a host compiler builds the host-side logic on its own for the sanitizer checks) ----
+#ifdef __HIPCC__
 __device__ __forceinline__ float lh_wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
@@ -248,3 +246,4 @@ __device__ __forceinline__ float lh_block_max(float v, float* smem) {
   __syncthreads();
   return smem[16];
 }
+#endif  // __HIPCC__

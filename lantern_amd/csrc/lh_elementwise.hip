@@ -266,7 +266,7 @@ void lh_scalar_op(int op, const float* x, float* y, float s, int64_t n) {
 }
 
 void lh_add_relu(const float* a, const float* b, float* out, int64_t n) {
-  LZ_ENTER(); lazy::rd_f(a, n); lazy::rd_f(b, n); if (out != a && out != b) lazy::wr_f(out, n);
+  LZ_ENTER(); lazy::rd_f(a, n); lazy::rd_f(b, n); lazy::out_f(out, n, out == a || out == b);
   ProfScope prof_(CAT_ELEMENTWISE);
   ew<2>(out, a, b, nullptr, n, [] __device__(float x, float y, float) { float r = x + y; return r < 0.f ? 0.f : r; });
   LH_CHECK_LAUNCH();
@@ -301,7 +301,7 @@ void lh_add_relu_grad(const float* y, const float* dy, float* ad, float abeta, f
 }
 
 void lh_geam(const float* x, float alpha, const float* y, float beta, float* out, int64_t n) {
-  LZ_ENTER(); lazy::rd_f(x, n); lazy::rd_f(y, n); if (out != x && out != y) lazy::wr_f(out, n);
+  LZ_ENTER(); lazy::rd_f(x, n); lazy::rd_f(y, n); lazy::out_f(out, n, out == x || out == y);
   ProfScope prof_(CAT_ELEMENTWISE);
   if (n > 0 && rec_ok(n)) { rec_cmd(CL_GEAM, (int)n, 0, 0, alpha, beta, 0.f, 0.f, out, x, y, nullptr); return; }
   ew<2>(out, x, y, nullptr, n, [alpha, beta] __device__(float a, float b, float) { return a * alpha + b * beta; });
@@ -435,7 +435,7 @@ void lh_bcast_op(int op, const float* a, const int* adims, const float* b, const
   const bool same = same_dims(adims, odims, rank) && same_dims(bdims, odims, rank);
   // a same-shape `+` waits for the call behind it: relu in place makes it one kernel, behind a parked batch norm the residual join
   if (same && op == LH_ADD && !rec_ok(n) && lazy::park_add(a, b, out, n)) return;
-  if (lazy::g_busy && !lazy::g_replay) { lazy::flush_parked(); lazy::rd_f(a, prod(adims, rank)); lazy::rd_f(b, prod(bdims, rank)); lazy::wr_f(out, n); }
+  if (lazy::g_busy && !lazy::g_replay) { lazy::flush_parked(); lazy::rd_f(a, prod(adims, rank)); lazy::rd_f(b, prod(bdims, rank)); lazy::out_f(out, n, out == a || out == b); }
   ProfScope prof_(CAT_ELEMENTWISE);
   if (same) {
     if (rec_ok(n)) { rec_cmd(CL_BIN, (int)n, op, 0, 0.f, 0.f, 0.f, 0.f, out, a, b, nullptr); return; }

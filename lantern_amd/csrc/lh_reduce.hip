@@ -207,7 +207,7 @@ void lh_sum_dim_grad(float* dx, const float* dy, int outer, int dim, int inner) 
   LH_CHECK_LAUNCH();
 }
 
-void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner) { LZ_ENTER(); lazy::rd_f(x, (int64_t)outer * c * inner); if (y != x) lazy::wr_f(y, (int64_t)outer * c * inner); ProfScope prof_(CAT_REDUCE);
+void lh_softmax(int is_log, const float* x, float* y, int outer, int c, int inner) { LZ_ENTER(); lazy::rd_f(x, (int64_t)outer * c * inner); lazy::out_f(y, (int64_t)outer * c * inner, y == x); ProfScope prof_(CAT_REDUCE);
   if ((int64_t)outer * c * inner <= 0) return;
   if (inner == 1 && rec_ok((int64_t)outer * c)) { rec_cmd(CL_SOFTMAX, outer, c, is_log ? 1 : 0, 0.f, 0.f, 0.f, 0.f, y, x, nullptr, nullptr); return; }
   if (inner == 1) {

@@ -389,3 +389,29 @@ def test_mean_clip_bias_fill_and_sgemv_literals():
     tv = np.array([1, -1], np.float32); zv = np.array([1, 1, 1], np.float32)
     lc.lc_sgemv(I(1), I(2), I(3), F(1.0), cptr(A), I(3), cptr(tv), F(1.0), cptr(zv))      # z += A^T t
     np.testing.assert_array_equal(zv, np.array([1 - 3, 1 - 3, 1 - 3], np.float32))
+
+
+@pytest.mark.parametrize("shape,context", [((7, 3, 5), 2), ((5, 4), 4), ((9,), 1), ((30, 2, 16), 20), ((4, 1, 1), 0)], ids=str)
+def test_repeat0_and_its_gradient_against_numpy(shape, context):
+    """repeat0 (TD:1446-1451; CDN:378-399): out[i0, i1] = in[i0 + i1] against numpy's sliding windows, bit for bit; the gradient
+    against the scatter the definition fixes (every window's slice added back onto the rows it was cut from, on top of what the
+    gradient buffer held), a literal case included."""
+    rng = np.random.RandomState(51)
+    x = rng.randn(*shape).astype(np.float32)
+    rows, inner = shape[0], int(np.prod(shape[1:]))
+    oshape = (rows - context, context + 1) + tuple(shape[1:])
+    y = np.full(oshape, -9, np.float32)
+    lc.lc_repeat0(cptr(x), cptr(y), I(rows), I(context), L(inner))
+    np.testing.assert_array_equal(y, np.stack([x[i:i + context + 1] for i in range(rows - context)]))
+    dy = rng.randn(*oshape).astype(np.float32)
+    dx = np.ones_like(x)
+    want = np.ones_like(x)
+    for i0 in range(rows - context):
+        for i1 in range(context + 1):
+            want[i0 + i1] += dy[i0, i1]
+    lc.lc_repeat0_grad(cptr(dx), cptr(dy), I(rows), I(context), L(inner))
+    np.testing.assert_allclose(dx, want, rtol=1e-6, atol=1e-6)
+    # by hand: rows 0..3, context 1 -> windows (0,1), (1,2), (2,3); ones as the windows' gradient: rows get 1, 2, 2, 1
+    d = np.zeros(4, np.float32); g = np.ones((3, 2), np.float32)
+    lc.lc_repeat0_grad(cptr(d), cptr(g), I(4), I(1), L(1))
+    np.testing.assert_array_equal(d, np.array([1, 2, 2, 1], np.float32))
