@@ -2,6 +2,7 @@
 // Reference behaviour being replaced: CUB:18-25, 113-131 (handles + arena + rewind),
 // API:453-473 (myGpuMalloc / myGpuFree), CUB:37-107 (toGPU / toCPU).
 #include "lh_common.h"
+#include "lh_arena.h"
 #include <stdarg.h>
 #include <string.h>
 #include <vector>
@@ -48,11 +49,8 @@ int g_error_mode = 0;
 int g_num_cu = 256;
 static char g_err[1024] = "";
 static char* g_heap = nullptr;
-static size_t g_heap_bytes = 0, g_top = 0, g_peak = 0;
-// [g_top, g_zero_end) is known to read zero (when g_zero_end > g_top): small zero-filled blocks are cleared a
-// window at a time, so a run of them costs one fill launch instead of one each.
-static size_t g_zero_end = 0;
-static const size_t ZERO_AHEAD = 1u << 20;
+static ArenaState g_arena;                     // bump pointer, peak, and the window above the top that is known to read zero (lh_arena.h)
+static const size_t ZERO_AHEAD = 1u << 20;     // small zero-filled blocks are cleared this much at a time; larger blocks may be cleared on demand
 
 bool fail(const char* file, int line, const char* fmt, ...) {
   char msg[768];
@@ -135,7 +133,7 @@ void lh_setup(size_t heap_bytes) {
   g_stream_cur = g_stream_raw; g_side_dirty = false;
   heap_bytes = (heap_bytes + 255) & ~(size_t)255;
   LH_HIP(hipMalloc((void**)&g_heap, heap_bytes));
-  g_heap_bytes = heap_bytes; g_top = 0; g_peak = 0; g_zero_end = 0;
+  g_arena = ArenaState(); g_arena.bytes = heap_bytes;
   lazy::reset();
   LH_HIP(hipMalloc((void**)&g_advance_pool, MAX_GRAPHS * sizeof(unsigned long long)));
   if (!multi_tensor_setup()) return;
@@ -159,7 +157,7 @@ void lh_cleanup(void) {
   g_advance_pool = nullptr; g_capture_advance = nullptr;
   if (g_heap) (void)hipFree(g_heap);
   if (g_stream_raw) (void)hipStreamDestroy(g_stream_raw);
-  g_heap = nullptr; g_stream_raw = nullptr; g_stream_cur = nullptr; g_heap_bytes = g_top = g_zero_end = 0;
+  g_heap = nullptr; g_stream_raw = nullptr; g_stream_cur = nullptr; g_arena = ArenaState();
 }
 
 void lh_sync(void) {
@@ -174,54 +172,43 @@ void lh_sync(void) {
 static void* bump(size_t bytes, bool zero) {
   if (!g_heap) { LH_FAIL("lh_malloc before lh_setup"); return nullptr; }
   if (zero && g_stream_cur != g_stream_raw) { LH_FAIL("lh_malloc between lh_side_begin and lh_side_end: zeroed memory is handed out in main-stream order only"); return nullptr; }
-  size_t need = (bytes + 255) & ~(size_t)255;
-  if (need == 0) need = 256;
-  if (g_top + need > g_heap_bytes) {
+  const ArenaGrant g = arena_bump(g_arena, bytes, zero, lazy::defer_zero(), ZERO_AHEAD);
+  if (!g.ok) {
     // API:462-464 aborts on overflow; here it takes the library's error path.
-    LH_FAIL("device arena exhausted: %zu used + %zu requested > %zu", g_top, need, g_heap_bytes);
+    LH_FAIL("device arena exhausted: %zu used + %zu requested > %zu", g_arena.top, g.need, g_arena.bytes);
     return nullptr;
   }
-  void* p = g_heap + g_top;
-  if (zero && need > ZERO_AHEAD && lazy::defer_zero()) {
-    // cleared when somebody reads it, never if its first user overwrites it
-    lazy::note_zero_block(p, need);
-  } else if (zero && g_top + need > g_zero_end) {
-    lazy::Scope lz_scope_;      // the fill below is ordered before anything that can touch the block: parked launches stay parked
-    const size_t from = g_zero_end > g_top ? g_zero_end : g_top;
-    size_t to = g_top + need;
-    if (need < ZERO_AHEAD) to = g_top + ZERO_AHEAD < g_heap_bytes ? g_top + ZERO_AHEAD : g_heap_bytes;
+  void* p = g_heap + g.offset;
+  if (g.lazy) {
+    lazy::note_zero_block(p, g.need);      // cleared when somebody reads it, never if its first user overwrites it
+  } else if (g.zero_to > g.zero_from) {
+    lazy::Scope lz_scope_;                 // the fill below is ordered before anything that can touch the block: parked launches stay parked
     ProfScope prof_(CAT_FILL);
-    zero_async(g_heap + from, to - from);
-    g_zero_end = to;
+    zero_async(g_heap + g.zero_from, g.zero_to - g.zero_from);
   }
-  g_top += need;
-  if (g_top > g_peak) g_peak = g_top;
   return p;
 }
 void* lh_malloc(size_t bytes) { return bump(bytes, true); }
 void* lh_malloc_uninit(size_t bytes) { return bump(bytes, false); }
 void lh_free_top(size_t bytes) {
-  size_t need = (bytes + 255) & ~(size_t)255;
-  if (need == 0) need = 256;
-  LH_REQUIRE(need <= g_top, "lh_free_top(%zu) below the arena base", bytes);
+  const size_t need = arena_round(bytes);
+  LH_REQUIRE(need <= g_arena.top, "lh_free_top(%zu) below the arena base", bytes);
   if (lazy::g_busy) {
     if (lazy::g_depth == 0) { LZ_ENTER(); }       // a caller's pop (myGpuFree): nothing parked may still want the block
-    lazy::arena_released(g_heap + g_top - need);
+    lazy::arena_released(g_heap + g_arena.top - need);
   }
-  g_top -= need;
-  g_zero_end = g_top;            // what was handed out above the new top may have been written
+  (void)arena_pop(g_arena, bytes);
 }
-size_t lh_mark(void) { return g_top; }
+size_t lh_mark(void) { return g_arena.top; }
 void lh_rewind(size_t mark) {
-  LH_REQUIRE(mark <= g_top && (mark & 255) == 0, "lh_rewind(%zu): not a mark at or below the top (%zu)", mark, g_top);
+  LH_REQUIRE(mark <= g_arena.top && (mark & 255) == 0, "lh_rewind(%zu): not a mark at or below the top (%zu)", mark, g_arena.top);
   LZ_SCOPE();
   if (lazy::g_busy) lazy::on_rewind(g_heap + mark);     // zero fills and unread results of what is released are simply dropped
   side_join();      // what is handed out again must not be in use on the side stream
-  g_top = mark;
-  g_zero_end = mark;
+  (void)arena_rewind(g_arena, mark);
 }
-size_t lh_heap_used(void) { return g_top; }
-size_t lh_heap_peak(void) { return g_peak; }
+size_t lh_heap_used(void) { return g_arena.top; }
+size_t lh_heap_peak(void) { return g_arena.peak; }
 
 // Small uploads (a tree's labels, a batch's targets) go through a ring of pinned staging slots and do not wait for the
 // device: the caller's buffer is free again when the call returns (it was copied into the slot), and the stream orders
@@ -372,14 +359,14 @@ void lh_capture_begin(void) {
   LH_CHECK_LAUNCH();
   LH_HIP(hipStreamBeginCapture(g_stream_raw, hipStreamCaptureModeThreadLocal));
   g_capturing = true;
-  g_zero_end = g_top;       // a zero fill done eagerly says nothing about replays: every block handed out while recording records its own fill
+  g_arena.zero_end = g_arena.top;       // a zero fill done eagerly says nothing about replays: every block handed out while recording records its own fill
 }
 int lh_capture_end(void) {
   if (!g_capturing) { LH_FAIL("lh_capture_end without lh_capture_begin"); return -1; }
   { LZ_SCOPE(); lazy::flush_all(); }          // everything the recorded calls stand for is in the graph
   if (g_capture_drawn) hipLaunchKernelGGL(k_set_u64, dim3(1), dim3(1), 0, g_stream_raw, g_capture_advance, 1ull, g_capture_drawn);
   g_capturing = false;
-  g_zero_end = g_top;       // fills recorded into the graph have not run
+  g_arena.zero_end = g_arena.top;       // fills recorded into the graph have not run
   hipGraph_t graph = nullptr;
   hipError_t e = hipStreamEndCapture(g_stream_raw, &graph);
   if (e != hipSuccess || graph == nullptr) {

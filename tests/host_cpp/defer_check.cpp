@@ -15,6 +15,7 @@
 #include <vector>
 
 #include "../../lantern_amd/csrc/lh_defer.hip"
+#include "../../lantern_amd/csrc/lh_arena.h"
 
 // ---- what the bookkeeping needs from the rest of the library ------------------------------------------------------------
 namespace lh {
@@ -50,23 +51,30 @@ void multi_update_now(int mode, int count, float* const* hx, float* const* hd, f
 }  // namespace lh
 using namespace lh;
 
-// ---- the simulated arena (the logic of lh_runtime.hip's bump allocator, with a lower threshold for "large") ---------------
-static char* g_heap; static size_t g_top = 0, g_heap_bytes = 0;
-static const size_t LAZY_MIN = 512;       // blocks of more than this many bytes are handed out uncleared when the bookkeeping is on
+// ---- the arena: the library's own bookkeeping (lh_arena.h) over host memory, acted on as lh_runtime.hip acts on it ----------
+static char* g_heap; static ArenaState g_arena;
+static const size_t ZERO_AHEAD = 512;     // the library uses 1 MiB; here two 256-byte blocks make a window and every activation (768 bytes) is "large"
 static void* sim_malloc(size_t bytes, bool zero) {
-  size_t need = (bytes + 255) & ~(size_t)255; if (need == 0) need = 256;
-  if (g_top + need > g_heap_bytes) { fprintf(stderr, "simulated arena exhausted\n"); exit(2); }
-  void* p = g_heap + g_top;
-  if (zero && need > LAZY_MIN && lazy::defer_zero()) lazy::note_zero_block(p, need);
-  else if (zero) { lazy::Scope s_; zero_bytes_async(p, need); }
-  g_top += need;
+  const ArenaGrant g = arena_bump(g_arena, bytes, zero, lazy::defer_zero(), ZERO_AHEAD);
+  if (!g.ok) { fprintf(stderr, "simulated arena exhausted\n"); exit(2); }
+  void* p = g_heap + g.offset;
+  if (g.lazy) lazy::note_zero_block(p, g.need);
+  else if (g.zero_to > g.zero_from) { lazy::Scope s_; zero_bytes_async(g_heap + g.zero_from, g.zero_to - g.zero_from); }
+  // the arena's own promise, checked where the simulation can see it at once: a block that was not put off reads zero now
+  if (zero && !g.lazy) for (size_t i = 0; i < g.need; i++) if (((char*)p)[i] != 0) { fprintf(stderr, "lh_malloc handed out a block of %zu bytes at offset %zu that does not read zero (byte %zu)\n", g.need, g.offset, i); exit(1); }
   return p;
 }
 static void sim_rewind(size_t mark) {
   lazy::Scope s_;
   if (lazy::g_busy) lazy::on_rewind(g_heap + mark);
-  memset(g_heap + mark, 0xCD, g_top - mark);          // what is handed out again is full of garbage
-  g_top = mark;
+  memset(g_heap + mark, 0xCD, g_arena.bytes - mark);  // what is handed out again is full of garbage (the zero window above the old top included)
+  if (!arena_rewind(g_arena, mark)) { fprintf(stderr, "bad mark\n"); exit(2); }
+}
+static void sim_pop(size_t bytes) {                   // lh_free_top: scratch taken from the top and given back
+  const size_t need = arena_round(bytes);
+  if (lazy::g_busy) { if (lazy::g_depth == 0) { LZ_ENTER(); } lazy::arena_released(g_heap + g_arena.top - need); }
+  memset(g_heap + g_arena.top - need, 0xCD, g_arena.bytes - (g_arena.top - need));
+  if (!arena_pop(g_arena, bytes)) { fprintf(stderr, "bad pop\n"); exit(2); }
 }
 
 // ---- simulated kernels: any deterministic functions will do, as long as a fused form computes what its parts compute ------
@@ -255,7 +263,7 @@ struct Layer { int kind; TR in, conv, bn, sc, out; float *w, *dw, *wv, *g, *dg, 
 static void run_program(uint64_t seed, bool enabled, std::vector<float>& trace, std::vector<char>& image, long long& kernels) {
   g_rng = seed;
   lazy::reset(); lazy::g_enabled = enabled; lazy::g_depth = 0;
-  memset(g_heap, 0xCD, g_heap_bytes); g_top = 0; g_kernels = 0;
+  memset(g_heap, 0xCD, g_arena.bytes); { const size_t b = g_arena.bytes; g_arena = ArenaState(); g_arena.bytes = b; } g_kernels = 0;
   auto vec = [&](int n, bool random) { float* p = (float*)sim_malloc(SZ(n), true); if (random) { std::vector<float> h(n); for (auto& v : h) v = rf(); lazy::Scope s_; lazy::wr(p, SZ(n)); memcpy(p, h.data(), SZ(n)); } return p; };
   auto tr = [&](float* x) { TR t; t.x = x; t.d = (float*)sim_malloc(SZ(NE), true); return t; };
   // parameters below the mark (gradients and momentum buffers start as untouched zero blocks of their own)
@@ -268,7 +276,7 @@ static void run_program(uint64_t seed, bool enabled, std::vector<float>& trace, 
   }
   float* input = vec(NE, true);
   float* big_d = (float*)sim_malloc(SZ(NE), true);       // a parameter-like large block: its first gradient overwrites it
-  const size_t mark = g_top;
+  const size_t mark = g_arena.top;
   const int steps = ri(1, 3);
   for (int step = 0; step < steps; step++) {
     // forward
@@ -318,7 +326,7 @@ static void run_program(uint64_t seed, bool enabled, std::vector<float>& trace, 
     const int extras = ri(0, 4);
     for (int e = 0; e < extras; e++) {
       Layer& l = L[ri(0, nlayers - 1)];
-      switch (ri(0, 8)) {
+      switch (ri(0, 9)) {
         case 7: t_geam(l.out.x, -1.f, l.out.x, 0.f, l.out.x, NE); t_d2h(trace, l.out.d, NE); break;       // in place over what a recipe still has to read (the relu mask)
         case 8: t_geam(l.out.d, 3.f, l.out.d, 0.f, l.out.d, NE); t_d2h(trace, l.bn.d, NE); break;         // in place over the gradient a recipe copies from
         case 0: t_d2h(trace, l.bn.x, NE); break;
@@ -327,21 +335,26 @@ static void run_program(uint64_t seed, bool enabled, std::vector<float>& trace, 
         case 3: t_undeclared(l.out.x, 7); break;
         case 4: t_fill(l.bn.d + 8, 2.5f, 16); break;
         case 5: { float* z = (float*)sim_malloc(SZ(NE), true); t_geam(z + 4, 1.f, l.out.x, 1.f, z + 4, 20); t_d2h(trace, z, NE); break; }
-        default: { float* z = (float*)sim_malloc(SZ(NE), true); t_d2h(trace, z + 10, 3); break; }
+        case 6: { float* z = (float*)sim_malloc(SZ(NE), true); t_d2h(trace, z + 10, 3); break; }
+        default: {      // scratch from the top, used and popped; then small zero blocks out of the same memory
+          float* sc = (float*)sim_malloc(SZ(NE), false); t_fill(sc, 9.f, NE); sim_pop(SZ(NE));
+          float* z1 = (float*)sim_malloc(SZ(5), true); float* z2 = (float*)sim_malloc(SZ(40), true); float* z3 = (float*)sim_malloc(SZ(NE), true);
+          t_d2h(trace, z1, 5); t_d2h(trace, z2, 40); t_geam(z3, 1.f, z2, 1.f, z3, 40); t_d2h(trace, z3 + 30, 20); break;
+        }
       }
     }
     if (step + 1 < steps || ri(0, 1)) sim_rewind(mark);
   }
   { lazy::Scope s_; lazy::flush_all(); }
-  image.assign(g_heap, g_heap + g_top);
+  image.assign(g_heap, g_heap + g_arena.top);
   kernels = g_kernels;
 }
 
 int main(int argc, char** argv) {
   const int programs = argc > 1 ? atoi(argv[1]) : 2000;
   const uint64_t seed0 = argc > 2 ? (uint64_t)atoll(argv[2]) : 1;
-  g_heap_bytes = 4u << 20;
-  g_heap = (char*)aligned_alloc(256, g_heap_bytes);
+  g_arena.bytes = 4u << 20;
+  g_heap = (char*)aligned_alloc(256, g_arena.bytes);
   long long k_on = 0, k_off = 0, fused = 0;
   for (int p = 0; p < programs; p++) {
     std::vector<float> t_off, t_on; std::vector<char> i_off, i_on; long long a = 0, b = 0;
