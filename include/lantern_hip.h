@@ -173,7 +173,7 @@ void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat);
  *     the chain runs as lh_conv2d_fwd_bn_apply / lh_bn_train_fwd_relu / lh_add_relu / lh_bn_bwd_relu / lh_bn_bwd_add_relu;
  *     any other call (lh_malloc, lh_malloc_uninit and lh_mark excepted) first launches what is waiting, unfused.
  *     Runs of lh_momentum / lh_sgd calls with equal hyper-parameters become one multi-tensor launch.
- *   - a block of more than 1 MiB from lh_malloc is cleared when something first reads it; a call that overwrites it, or
+ *   - a block of more than 16 KiB from lh_malloc is cleared when something first reads it; a call that overwrites it, or
  *     would add into it with beta = 1, writes it without the clearing pass and without reading it; lh_rewind forgets it.
  *   - what a fused chain does not store because programs do not read it (the batch norm's own output under a residual
  *     join; the in-place masking of the gradient buffer by relu_grad) is produced when a call does read it.

@@ -4,7 +4,7 @@
 // on the grants (it launches the fills), tests/host_cpp/defer_check.cpp uses the same code over host memory.
 //   - [top, zero_end) is known to read zero: small blocks are cleared a window of `zero_ahead` bytes at a time, so a run of
 //     them costs one fill, not one each; a pop or a rewind forgets the window (what lay above the new top may have been written);
-//   - a block of more than `zero_ahead` bytes is either cleared when handed out or, when the caller may put the clearing off
+//   - a block of more than `lazy_min` bytes is either cleared when handed out or, when the caller may put the clearing off
 //     (`may_defer`), handed out as it is and reported as `lazy` for the deferred-work bookkeeping to note.
 #pragma once
 #include <stddef.h>
@@ -18,12 +18,12 @@ struct ArenaGrant {
   size_t zero_from = 0, zero_to = 0;   // clear [zero_from, zero_to) now (empty when equal)
 };
 static inline size_t arena_round(size_t bytes) { size_t need = (bytes + 255) & ~(size_t)255; return need ? need : 256; }
-static inline ArenaGrant arena_bump(ArenaState& a, size_t bytes, bool zero, bool may_defer, size_t zero_ahead) {
+static inline ArenaGrant arena_bump(ArenaState& a, size_t bytes, bool zero, bool may_defer, size_t zero_ahead, size_t lazy_min) {
   ArenaGrant g;
   g.need = arena_round(bytes);
   if (g.need < bytes || a.top + g.need > a.bytes || a.top + g.need < a.top) return g;
   g.ok = true; g.offset = a.top;
-  if (zero && g.need > zero_ahead && may_defer) {
+  if (zero && g.need > lazy_min && may_defer) {
     g.lazy = true;
   } else if (zero && a.top + g.need > a.zero_end) {
     g.zero_from = a.zero_end > a.top ? a.zero_end : a.top;

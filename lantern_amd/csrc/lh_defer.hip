@@ -11,7 +11,7 @@
 //     point (lh_conv2d_fwd_bn_apply, lh_bn_train_fwd_relu, lh_add_relu, lh_bn_bwd_relu, lh_bn_bwd_add_relu); any other
 //     call first launches what is parked, unfused.  lh_malloc, lh_malloc_uninit and lh_mark do not count as calls here.
 //     Optimizer calls (lh_momentum, lh_sgd) with equal hyper-parameters are gathered into one multi-tensor launch.
-//  2. Zero fills on demand.  A block of more than 1 MiB from lh_malloc is not cleared when handed out; it is noted.  An
+//  2. Zero fills on demand.  A block of more than 16 KiB from lh_malloc is not cleared when handed out; it is noted.  An
 //     entry point that overwrites the block drops the note; one that would add into it (beta = 1) overwrites instead;
 //     anything that reads it gets it cleared first.  lh_rewind drops the notes of what it releases.
 //  3. Unwritten results.  A fused chain leaves out stores nobody normally reads: the batch norm's own output under a

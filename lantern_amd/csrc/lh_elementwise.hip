@@ -189,6 +189,7 @@ void lh_cifar_decode(const unsigned char* records, float* x, int* y, int n, int 
   if (n < 0 || count <= 0) { LH_FAIL("lh_cifar_decode: n %d, count %d", n, count); return; }
   if (n == 0) return;
   const int64_t tot = (int64_t)n * count;
+  LZ_ENTER(); lazy::rd(records, (size_t)n * ((size_t)count + 1)); lazy::wr_f(x, tot); lazy::wr_f(y, n);
   if (count % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
     hipLaunchKernelGGL(k_cifar_decode<4>, dim3(stream_grid(tot / 4, TPB)), dim3(TPB), 0, g_stream, records, x, y, tot / 4, count);
   } else {

@@ -398,6 +398,8 @@ void lh_rnn_fwd_init(int mode, const float* x, const float* hx, const float* w, 
   LH_REQUIRE(H <= 2048, "lh_rnn_fwd: hidden size %d above %d", H, 2048);
   LH_REQUIRE(x && w && y, "lh_rnn_fwd: null operand");
   const int D = bidir ? 2 : 1, ld = D * H;
+  LZ_ENTER();
+  lazy::rd_f(x, (int64_t)T * B * I); lazy::rd_f(w, (int64_t)D * dir_params(I, H)); lazy::rd_f(hx, (int64_t)D * B * H); lazy::wr_f(y, (int64_t)T * B * ld);
   for (int d = 0; d < D; d++) {          // input projection of every step straight into y
     const float* Wih = w + d * dir_params(I, H);
     lh_sgemm(0, 1, T * B, H, I, 1.0f, x, I, Wih, I, 0.0f, y + d * H, ld);
@@ -429,6 +431,10 @@ void lh_rnn_bwd_init(int mode, const float* x, const float* hx, const float* y, 
   LH_REQUIRE(beta_dx == 0.f || beta_dx == 1.f, "lh_rnn_bwd: beta must be 0 or 1");
   LH_REQUIRE(x && y && dy && w && dw, "lh_rnn_bwd: null operand");
   const int D = bidir ? 2 : 1, ld = D * H;
+  LZ_ENTER();
+  lazy::rd_f(x, (int64_t)T * B * I); lazy::rd_f(y, (int64_t)T * B * ld); lazy::rd_f(dy, (int64_t)T * B * ld); lazy::rd_f(w, (int64_t)D * dir_params(I, H));
+  lazy::rd_f(hx, (int64_t)D * B * H); lazy::rw_f(dw, (int64_t)D * dir_params(I, H));
+  if (dx) beta_dx = lazy::beta_f(dx, (int64_t)T * B * I, beta_dx);          // an input gradient nobody has touched since lh_malloc is overwritten
   // scratch from the top of the arena: dpre [T*B, D*H], W_hh^T per direction, column sums
   const size_t n_dpre = (size_t)T * B * ld, n_wt = (size_t)D * H * H, n_cs = (size_t)ld;
   const size_t bytes = (n_dpre + n_wt + n_cs) * sizeof(float);
@@ -483,6 +489,8 @@ void lh_ctc_loss(const float* probs, float* dprobs, const int* h_labels, const i
   LH_NOT_CAPTURING("lh_ctc_loss (it uploads its label and length arrays)");
   LH_REQUIRE(T >= 1 && B >= 1 && A >= 2, "lh_ctc_loss: bad shape T%d B%d A%d", T, B, A);
   LH_REQUIRE(probs && costs && h_labels && h_label_len && h_input_len, "lh_ctc_loss: null operand");
+  LZ_ENTER();
+  lazy::rd_f(probs, (int64_t)T * B * A); lazy::rw_f(dprobs, (int64_t)T * B * A); lazy::wr_f(costs, B);
   int total = 0, Lmax = 0;
   int* host = (int*)malloc(sizeof(int) * (size_t)(3 * B));
   if (!host) { LH_FAIL("lh_ctc_loss: out of host memory"); return; }

@@ -282,6 +282,9 @@ void lh_rnn_gated_fwd_init(int mode, const float* x, const float* hx, const floa
   LH_REQUIRE(cx == nullptr || mode == 2, "lh_rnn_gated_fwd: only the LSTM has a cell state");
   LH_REQUIRE(x && w && y && reserve, "lh_rnn_gated_fwd: null operand");
   const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
+  LZ_ENTER();
+  lazy::rd_f(x, (int64_t)T * B * I); lazy::rd_f(w, (int64_t)D * dir_params(mode, I, H)); lazy::rd_f(hx, (int64_t)D * B * H); lazy::rd_f(cx, (int64_t)D * B * H);
+  lazy::wr_f(y, (int64_t)T * B * ldh); lazy::wr_f(reserve, (int64_t)D * dir_reserve(mode, T, B, H));
   const size_t per_dir = (size_t)B * G;
   const size_t gh_bytes = (size_t)D * per_dir * sizeof(float);
   float* gh_all = (float*)lh_malloc_uninit(gh_bytes);
@@ -336,6 +339,11 @@ void lh_rnn_gated_bwd_init(int mode, const float* x, const float* hx, const floa
   LH_REQUIRE(beta_dx == 0.f || beta_dx == 1.f, "lh_rnn_gated_bwd: beta must be 0 or 1");
   LH_REQUIRE(x && y && dy && w && reserve && dw, "lh_rnn_gated_bwd: null operand");
   const int D = bidir ? 2 : 1, ldh = D * H, ng = gates_of(mode), G = ng * H;
+  LZ_ENTER();
+  lazy::rd_f(x, (int64_t)T * B * I); lazy::rd_f(y, (int64_t)T * B * ldh); lazy::rd_f(dy, (int64_t)T * B * ldh); lazy::rd_f(w, (int64_t)D * dir_params(mode, I, H));
+  lazy::rd_f(hx, (int64_t)D * B * H); lazy::rd_f(cx, (int64_t)D * B * H); lazy::rw_f(reserve, (int64_t)D * dir_reserve(mode, T, B, H));
+  lazy::rw_f(dw, (int64_t)D * dir_params(mode, I, H));
+  if (dx) beta_dx = lazy::beta_f(dx, (int64_t)T * B * I, beta_dx);
   // scratch from the top of the arena: recurrent gradient [B, H], cell gradient [B, H], column sums [2G],
   // and for the GRU the hidden-side pre-activation gradients of every step [T, B, G]
   const size_t n_bh = (size_t)B * H, n_dgh = mode == 3 ? (size_t)T * B * G : 0;

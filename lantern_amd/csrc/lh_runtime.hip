@@ -50,7 +50,8 @@ int g_num_cu = 256;
 static char g_err[1024] = "";
 static char* g_heap = nullptr;
 static ArenaState g_arena;                     // bump pointer, peak, and the window above the top that is known to read zero (lh_arena.h)
-static const size_t ZERO_AHEAD = 1u << 20;     // small zero-filled blocks are cleared this much at a time; larger blocks may be cleared on demand
+static const size_t ZERO_AHEAD = 1u << 20;     // small zero-filled blocks are cleared this much at a time
+static const size_t LAZY_MIN = 16u << 10;      // blocks of more than this may be cleared on demand instead (the networks on 32x32 images are made of blocks of 0.1 to 1 MiB)
 
 bool fail(const char* file, int line, const char* fmt, ...) {
   char msg[768];
@@ -172,7 +173,7 @@ void lh_sync(void) {
 static void* bump(size_t bytes, bool zero) {
   if (!g_heap) { LH_FAIL("lh_malloc before lh_setup"); return nullptr; }
   if (zero && g_stream_cur != g_stream_raw) { LH_FAIL("lh_malloc between lh_side_begin and lh_side_end: zeroed memory is handed out in main-stream order only"); return nullptr; }
-  const ArenaGrant g = arena_bump(g_arena, bytes, zero, lazy::defer_zero(), ZERO_AHEAD);
+  const ArenaGrant g = arena_bump(g_arena, bytes, zero, lazy::defer_zero(), ZERO_AHEAD, LAZY_MIN);
   if (!g.ok) {
     // API:462-464 aborts on overflow; here it takes the library's error path.
     LH_FAIL("device arena exhausted: %zu used + %zu requested > %zu", g_arena.top, g.need, g_arena.bytes);

@@ -53,9 +53,9 @@ using namespace lh;
 
 // ---- the arena: the library's own bookkeeping (lh_arena.h) over host memory, acted on as lh_runtime.hip acts on it ----------
 static char* g_heap; static ArenaState g_arena;
-static const size_t ZERO_AHEAD = 512;     // the library uses 1 MiB; here two 256-byte blocks make a window and every activation (768 bytes) is "large"
+static const size_t ZERO_AHEAD = 1024, LAZY_MIN = 512;     // the library uses 1 MiB and 16 KiB; here four 256-byte blocks make a window and every activation (768 bytes) is "large"
 static void* sim_malloc(size_t bytes, bool zero) {
-  const ArenaGrant g = arena_bump(g_arena, bytes, zero, lazy::defer_zero(), ZERO_AHEAD);
+  const ArenaGrant g = arena_bump(g_arena, bytes, zero, lazy::defer_zero(), ZERO_AHEAD, LAZY_MIN);
   if (!g.ok) { fprintf(stderr, "simulated arena exhausted\n"); exit(2); }
   void* p = g_heap + g.offset;
   if (g.lazy) lazy::note_zero_block(p, g.need);
