@@ -418,13 +418,16 @@ class BackendHIP(Backend):
         so = self.side_order
         if x_in or self.convs_open < self.side_min_convs:
             so = 0      # (almost) nothing left to run beside it (fewer than two convolution gradients follow): the optimizer's join would only add the cross-stream hand-over
-        if so == 2:
-            self.lib.lh_side_begin()
+        # With a bias the filter gradient goes first in any case: its bias sums are the first reader of dy, and a relu_grad(in place)
+        # issued just before is applied in that pass.
+        first = so == 2 or bd is not None
+        if first:
+            if so: self.lib.lh_side_begin()
             self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
-            self.lib.lh_side_end()
+            if so: self.lib.lh_side_end()
         if not x_in:
             self.lib.lh_conv2d_bwd_data(dy.ptr, w.ptr, xd.ptr, beta_dx, N, C, H, W, K, R, S, sH, sW, pH, pW)
-        if so != 2:
+        if not first:
             if so: self.lib.lh_side_begin()
             self.lib.lh_conv2d_bwd_filter(x.ptr, dy.ptr, wd.ptr, bd.ptr if bd is not None else 0, 1.0, N, C, H, W, K, R, S, sH, sW, pH, pW)
             if so: self.lib.lh_side_end()

@@ -160,6 +160,7 @@ bool park_add(const float* a, const float* b, float* out, int64_t n);
 bool take_relu_inplace(float* y, int64_t n);
 bool park_relu_grad_inplace(const float* y, float* d, int64_t n);
 bool park_add_grad(float* ad, float* bd, const float* outd, int64_t n);
+bool take_relu_grad_bias(const float* dy, float* db, int N, int K, int PQ);
 bool take_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                  float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
 bool gather_update(int mode, float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n);
@@ -175,6 +176,8 @@ void reset();                                      // forget everything deferred
 void mask_relu(float* dst, const float* src, const float* y, int64_t n);                     // dst = y > 0 ? src : 0
 void add_plain(const float* a, const float* b, float* out, int64_t n);
 void relu_grad_inplace_now(const float* y, float* d, int64_t n);
+void conv2d_fwd_relu_now(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW);
+void conv_bwd_bias_mask_now(const float* y, float* dy, float* db, int N, int K, int PQ);     // dy = y > 0 ? dy : 0 in place; db[k] += its sum over n, p, q
 void multi_update_now(int mode, int count, float* const* hx, float* const* hd, float* const* hv, const int64_t* hn, float lr, float mu, float clip, int nesterov);
 void zero_bytes_async(void* p, size_t bytes);      // bytes a multiple of 256
 

@@ -245,6 +245,7 @@ struct EpiConvOut {
   static constexpr bool STATS = false;
   static constexpr bool SLICED = false;
   float* out; const float* bias; int chan, PIX, W, eH, eW, aH, aW; float beta;
+  int relu = 0;             // complete sums are stored as max(v, 0); a launch that adds partial sums leaves that to a pass of its own (conv_fwd_impl)
   int zfill2 = 0;           // the grid is every second pixel of every second row of an image with even sides (a 1x1 filter, stride 2):
                             // the element is stored together with the three zeros of its 2x2 cell, so the output needs no clearing
   FastDiv dPIXc, dWc;
@@ -255,9 +256,16 @@ struct EpiConvOut {
     c.off = (int)n * chan * PIX + (aH + eH * (int)u) * W + aW + eW * (int)v;
     return c;
   }
-  // lean stores: element (i, j) at lane_bytes(col(j)) + i * row_bytes() from `out` (the tensor is below 2 GiB); not with a bias
+  // lean stores: element (i, j) at lane_bytes(col(j)) + i * row_bytes() from `out` (the tensor is below 2 GiB); the bias of
+  // the row and the clamp are applied to the value on its way (lean_fix)
   static constexpr bool LEAN = true;
-  __device__ __forceinline__ bool lean_ok(int M) const { return bias == nullptr && (M & 7) == 0; }
+  static constexpr bool LEAN_FIX = true;
+  __device__ __forceinline__ bool lean_ok(int M) const { return (M & 7) == 0; }
+  __device__ __forceinline__ float lean_fix(float v, int row) const {
+    if (bias) v += bias[row];
+    if (relu) v = v < 0.f ? 0.f : v;
+    return v;
+  }
   __device__ __forceinline__ float* lean_base() const { return out; }
   __device__ __forceinline__ uint32_t lane_bytes(const Col& c) const { return (uint32_t)c.off * 4u; }
   __device__ __forceinline__ uint32_t row_bytes() const { return (uint32_t)PIX * 4u; }
@@ -269,6 +277,7 @@ struct EpiConvOut {
     if (!c.valid || i >= M) return;
     float* p = out + c.off + i * PIX;
     if (bias && part < 2) v += bias[i];
+    if (relu && part == 0) v = v < 0.f ? 0.f : v;
     if (zfill2) {             // only set for overwriting, complete sums (host side)
       *reinterpret_cast<float2*>(p) = make_float2(v, 0.f);
       *reinterpret_cast<float2*>(p + W) = make_float2(0.f, 0.f);
@@ -314,21 +323,55 @@ __global__ void __launch_bounds__(TPB) k_filter_transpose(const float* __restric
     wt[i] = w[((int64_t)k * C + c) * RS + rs];
   }
 }
-// db[k] += sum over n, p, q of dy: block (k, slice of the batch); slices add their sums atomically
-__global__ void __launch_bounds__(TPB) k_conv_bwd_bias(const float* __restrict__ dy, float* db, int N, int K, int PQ, int n_per) {
+// db[k] += sum over n, p, q of dy: block (k, slice of the batch); slices add their sums atomically.
+// MASK: the gradient is one that relu_grad has yet to mask: dy = y > 0 ? dy : 0 is written back on the way.
+// VEC: P*Q is a multiple of 4 and the tensors are 16-byte aligned (every channel image then starts on a 16-byte boundary).
+// (sample, pixel) pairs are flattened over the threads: small maps (P*Q below the block size) keep every lane busy and the
+// loads of one thread do not wait for each other.  Both forms add the same terms in the same order.
+template <bool VEC, bool MASK>
+__global__ void __launch_bounds__(TPB) k_conv_bwd_bias(const float* __restrict__ y, float* dy, float* db, int N, int K, int PQ, int n_per) {
   __shared__ float sm[17];
   const int k = blockIdx.x, n0 = blockIdx.y * n_per, n1 = min(N, n0 + n_per);
-  // (sample, pixel) pairs flattened over the threads: small maps (PQ below the block size) keep every lane busy and
-  // the loads of one thread do not wait for each other
   float acc = 0.f;
-  const int total = (n1 - n0) * PQ;
+  if (VEC) {
+    const int PQ4 = PQ >> 2, total = (n1 - n0) * PQ4;
+#pragma unroll 2
+    for (int i = threadIdx.x; i < total; i += TPB) {
+      const int dn = i / PQ4, l = i - dn * PQ4;
+      const int64_t o = (((int64_t)(n0 + dn) * K + k) * PQ4 + l) * 4;
+      float4 g = *reinterpret_cast<const float4*>(dy + o);
+      if (MASK) {
+        const float4 a = *reinterpret_cast<const float4*>(y + o);
+        g.x = a.x > 0.f ? g.x : 0.f; g.y = a.y > 0.f ? g.y : 0.f; g.z = a.z > 0.f ? g.z : 0.f; g.w = a.w > 0.f ? g.w : 0.f;
+        *reinterpret_cast<float4*>(dy + o) = g;
+      }
+      acc += (g.x + g.y) + (g.z + g.w);
+    }
+  } else {
+    const int total = (n1 - n0) * PQ;
 #pragma unroll 4
-  for (int i = threadIdx.x; i < total; i += TPB) {
-    const int dn = i / PQ, l = i - dn * PQ;
-    acc += dy[((int64_t)(n0 + dn) * K + k) * PQ + l];
+    for (int i = threadIdx.x; i < total; i += TPB) {
+      const int dn = i / PQ, l = i - dn * PQ;
+      const int64_t o = ((int64_t)(n0 + dn) * K + k) * PQ + l;
+      float g = dy[o];
+      if (MASK) { g = y[o] > 0.f ? g : 0.f; dy[o] = g; }
+      acc += g;
+    }
   }
   acc = lh_block_sum(acc, sm);
   if (threadIdx.x == 0) atomicAdd(db + k, acc);
+}
+static void bias_grad_launch(const float* y, float* dy, float* db, int N, int K, int PQ) {
+  int bslices = g_deterministic ? 1 : (int)cdiv(4 * (int64_t)g_num_cu, K);     // slices of the batch add atomically: one slice when the order must be fixed
+  if (bslices > N) bslices = N;
+  if (bslices < 1) bslices = 1;
+  const int n_per = (int)cdiv(N, bslices);
+  const dim3 grid(K, (unsigned)cdiv(N, n_per));
+  const bool vec = PQ % 4 == 0 && (((uintptr_t)y | (uintptr_t)dy) & 15) == 0;
+  if (y && vec) hipLaunchKernelGGL((k_conv_bwd_bias<true, true>), grid, dim3(TPB), 0, g_stream, y, dy, db, N, K, PQ, n_per);
+  else if (y) hipLaunchKernelGGL((k_conv_bwd_bias<false, true>), grid, dim3(TPB), 0, g_stream, y, dy, db, N, K, PQ, n_per);
+  else if (vec) hipLaunchKernelGGL((k_conv_bwd_bias<true, false>), grid, dim3(TPB), 0, g_stream, y, dy, db, N, K, PQ, n_per);
+  else hipLaunchKernelGGL((k_conv_bwd_bias<false, false>), grid, dim3(TPB), 0, g_stream, y, dy, db, N, K, PQ, n_per);
 }
 
 #ifndef LH_CONV_BK
@@ -374,7 +417,9 @@ static bool launch_rounds(const AL& al, const BL& bl, const EP& ep, int M, int N
 // 128x128 / 64x128 tiles with two or three workers per CU.  8-9: stream-K over 64x64 tiles with four or eight workers per
 // CU, for products so small that even their 64x64 tiles leave most CUs with one block whose loads nothing hides.
 // 10: 32x128 tiles (32-deep slabs) for products of at most 32 rows, whose 64-row tiles would be half empty.
-constexpr int N_PLANS = 11;
+// 11-12: stream-K over 64x64 tiles with one worker per 32 or 8 slabs: a handful of tiles under a very long reduction (a filter
+// as large as the map: a fully connected layer), where a worker per CU would mean hundreds of atomic adds onto each element.
+constexpr int N_PLANS = 13;
 // LH_FORCE_M32 in the environment: products of at most 32 rows always take the 32-row tile (for tests of that tile; the
 // measured choice may well be another one).
 static inline bool force_m32() { return getenv("LH_FORCE_M32") != nullptr; }
@@ -384,12 +429,24 @@ static bool plan_valid(int plan, const EP& ep, int M, int K, bool can_zero) {
   if (plan == 10) return M <= 32;
   if ((plan == 1 || plan == 4 || plan == 6) && M <= 64) return false;
   if (plan >= 4 && plan <= 9) return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= 16;
+  if (plan >= 11) return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= 64;
   return true;
 }
+static bool g_launch_partial = false;     // the last launch_plan combined partial sums with atomic adds (stream-K): its epilogue saw incomplete sums
 template <class AL, class BL, class EP>
 static bool launch_plan(int plan, const AL& al, const BL& bl, const EP& ep, int M, int N, int K, float* zero_out, int64_t zero_n, bool prezeroed) {
+  g_launch_partial = false;
   if (plan == 10) return igemm_launch<32, 128, 32>(al, bl, ep, M, N, K, 1);
+  if (plan >= 11) {
+    g_launch_partial = true;
+    const int64_t units = cdiv(M, 64) * cdiv(N, 64) * cdiv(K, CONV_BK);
+    int64_t workers = cdiv(units, plan == 11 ? 32 : 8);
+    if (workers > 16 * (int64_t)g_num_cu) workers = 16 * (int64_t)g_num_cu;
+    if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
+    return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1, (int)workers);
+  }
   if (plan >= 4) {
+    g_launch_partial = true;
     const int workers = (plan >= 8 ? (plan == 8 ? 4 : 8) : (plan >= 6 ? 3 : 2)) * g_num_cu;
     if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
     if (plan >= 8) return igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
@@ -406,6 +463,7 @@ static bool launch_plan(int plan, const AL& al, const BL& bl, const EP& ep, int 
   // long reductions only: a worker's share must span many slabs for the per-segment set-up to pay off
   if (!g_deterministic && few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)workers && (ep.beta == 1.f || zero_out != nullptr || prezeroed)) {
     if (ep.beta == 0.f && !prezeroed) lh_fill(zero_out, 0.f, zero_n);
+    g_launch_partial = true;
     if (M > 64) return igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
     return igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, workers);
   }
@@ -502,13 +560,15 @@ struct BnStatsOut {
 
 // Forward convolution; with `bn` also the batch-norm statistics of its output channels.
 static void conv_fwd_impl(const float* x, const float* w, const float* bias, float* y,
-                          int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW, BnStatsOut* bn) {
+                          int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW, BnStatsOut* bn, int relu = 0) {
   KernelCat kc_(CAT_CONV_FWD);
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_fwd: bad shape N%d C%d H%d W%d K%d R%d S%d s(%d,%d) p(%d,%d)", N, C, H, W, K, R, S, sH, sW, pH, pW);
   const int RS = R * S, CRS = C * RS, PQ = d.P * d.Q;
   const uint32_t wbytes = (uint32_t)((size_t)K * CRS * 4), xbytes = (uint32_t)((size_t)N * C * H * W * 4);
   EpiConvOut ep = make_epi(y, bias, K, d.P, d.Q, 0.f);
+  ep.relu = (relu && bn == nullptr) ? 1 : 0;
+  g_launch_partial = false;
   bool ok;
   if (C % CONV_BK == 0 && ((uintptr_t)w & 15) == 0) {
     // tap-major reduction order; a 1x1 filter already has that layout
@@ -601,6 +661,10 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
   }
   if (!ok) return;
   LH_CHECK_LAUNCH();
+  if (ep.relu && g_launch_partial) {      // elements finished by atomic adds have not been clamped (the others have: clamping twice changes nothing)
+    lh_unary(LH_RELU, y, y, (int64_t)N * K * PQ, 0.f, 0.f);
+    return;
+  }
   // shapes whose launch leaves no statistics pieces: one extra pass over y
   if (bn && bn->out != nullptr && bn->shortcut == nullptr) {       // statistics pass + apply pass that combines the partial sums itself
     if (bn->relu) lh_bn_train_fwd_relu(y, bn->gamma, bn->beta, bn->run_mean, bn->run_var, bn->out, bn->save_mean, bn->save_invstd, N, K, PQ, bn->eps, bn->factor);
@@ -630,6 +694,20 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y,
   conv_fwd_declare(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW);
   conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, nullptr);
 }
+
+}  // extern "C"
+namespace lh {
+// relu(conv(x) + bias) written once: the clamp rides in the epilogue.  Called with the operands already stated.
+void conv_bwd_bias_mask_now(const float* y, float* dy, float* db, int N, int K, int PQ) {
+  KernelCat kc_(CAT_CONV_BWD_FILTER);
+  bias_grad_launch(y, dy, db, N, K, PQ);
+  LH_CHECK_LAUNCH();
+}
+void conv2d_fwd_relu_now(const float* x, const float* w, const float* bias, float* y, int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW) {
+  conv_fwd_impl(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW, nullptr, 1);
+}
+}  // namespace lh
+extern "C" {
 
 void lh_conv2d_fwd_bnstats(const float* x, const float* w, const float* bias, float* y,
                            int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW,
@@ -830,7 +908,10 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   ConvDims d;
   LH_REQUIRE(make_dims(d, N, C, H, W, K, R, S, sH, sW, pH, pW), "lh_conv2d_bwd_filter: bad shape");
   LH_REQUIRE(beta == 0.f || beta == 1.f, "lh_conv2d_bwd_filter: beta must be 0 or 1");
-  LZ_ENTER();
+  LZ_SCOPE();
+  // relu_grad(in place) on dy still parked: the bias gradient's pass over dy applies the mask as well
+  const bool bias_done = db && lazy::g_busy && !lazy::g_replay && lazy::take_relu_grad_bias(dy, db, N, K, d.P * d.Q);
+  if (lazy::g_busy && !lazy::g_replay) lazy::flush_parked();
   lazy::rd_f(x, (int64_t)N * C * H * W); lazy::rd_f(dy, (int64_t)N * K * d.P * d.Q);
   beta = lazy::beta_f(dw, (int64_t)K * C * R * S, beta);
   lazy::rw_f(db, K);
@@ -948,13 +1029,7 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     lh_free_top(partial_bytes);
   }
   if (!ok) return;
-  if (db) {
-    int bslices = g_deterministic ? 1 : (int)cdiv(2 * (int64_t)g_num_cu, K);     // slices of the batch add atomically: one slice when the order must be fixed
-    if (bslices > N) bslices = N;
-    if (bslices < 1) bslices = 1;
-    const int n_per = (int)cdiv(N, bslices);
-    hipLaunchKernelGGL(k_conv_bwd_bias, dim3(K, (unsigned)cdiv(N, n_per)), dim3(TPB), 0, g_stream, dy, db, N, K, PQ, n_per);
-  }
+  if (db && !bias_done) bias_grad_launch(nullptr, const_cast<float*>(dy), db, N, K, PQ);
   LH_CHECK_LAUNCH();
 }
 

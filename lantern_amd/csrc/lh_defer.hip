@@ -307,6 +307,14 @@ bool park_add(const float* a, const float* b, float* out, int64_t n) {
 }
 
 bool take_relu_inplace(float* y, int64_t n) {
+  if (g_p.kind == P_CONV && g_p.conv.y == y && (int64_t)g_p.conv.N * g_p.conv.K * g_p.conv.P * g_p.conv.Q == n) {
+    Parked p = std::move(g_p); g_p = Parked();
+    const ConvArgs& c = p.conv;
+    { Replay r_; conv2d_fwd_relu_now(c.x, c.w, c.bias, c.y, c.N, c.C, c.H, c.W, c.K, c.R, c.S, c.sH, c.sW, c.pH, c.pW); }
+    g_stat[ST_FUSED_FWD]++;
+    refresh_busy();
+    return true;
+  }
   if (g_p.kind == P_BN && !g_p.has_add && g_p.bn.y == y && g_p.bn.n == n) {
     Parked p = std::move(g_p); g_p = Parked();
     { Replay r_; launch_bn_chain(p, 1, nullptr, y); }
@@ -343,6 +351,19 @@ bool park_relu_grad_inplace(const float* y, float* d, int64_t n) {
   rd(y, (size_t)n * 4); rw(d, (size_t)n * 4);
   g_p.kind = P_RELU_GRAD; g_p.gy = y; g_p.gd = d; g_p.gn = n; g_p.ad = g_p.bd = nullptr;
   g_busy = true;
+  return true;
+}
+
+// A convolution's bias gradient asked for while relu_grad(in place) on the same output gradient is parked: one pass masks
+// the gradient and sums it per channel.
+bool take_relu_grad_bias(const float* dy, float* db, int N, int K, int PQ) {
+  if (g_p.kind != P_RELU_GRAD || (const float*)g_p.gd != dy || g_p.gn != (int64_t)N * K * PQ || !db) return false;
+  if (overlap((const char*)db, (size_t)K * 4, (const char*)g_p.gd, (size_t)g_p.gn * 4) || overlap((const char*)db, (size_t)K * 4, (const char*)g_p.gy, (size_t)g_p.gn * 4)) return false;
+  Parked p = std::move(g_p); g_p = Parked();
+  rw(db, (size_t)K * 4);
+  { Replay r_; conv_bwd_bias_mask_now(p.gy, p.gd, db, N, K, PQ); }
+  g_stat[ST_FUSED_BWD]++;
+  refresh_busy();
   return true;
 }
 

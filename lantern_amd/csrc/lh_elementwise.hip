@@ -657,19 +657,48 @@ void lh_dropout_bwd(const float* dy, const float* mask, float* dx, int64_t n) {
 }
 
 // ---------------------------------------------------------------- concat --------------
-// One launch per input tensor: rows of `st = sizes[t]*inner` floats are copied between a
-// packed source and a strided destination (or accumulated the other way for the gradient).
+// Up to four tensors per launch: a thread walks the strided side (the concatenated tensor), finds the tensor its position
+// belongs to, and copies from (or, for the gradient, adds or copies into) that tensor's packed rows of `st = sizes[t]*inner` floats.
 }  // extern "C"
-// GRAD: 0 = forward copy into the strided destination, 1 = gradient accumulated into the packed one, 2 = gradient overwriting it
-template <int GRAD>
-__global__ void __launch_bounds__(TPB) k_concat(const float* __restrict__ src, float* __restrict__ dst, int64_t st, int64_t row, int64_t off, int64_t n) {
+namespace {
+constexpr int CAT_MAX = 4;
+struct CatArgs { float* p[CAT_MAX]; int64_t st[CAT_MAX]; int64_t off[CAT_MAX]; int add[CAT_MAX]; int n; int64_t lo, width; };
+// GRAD: false = forward copy into the concatenated tensor, true = gradient into the packed ones (added where add[t], else overwriting)
+// T = float4: every row length, offset and pointer is a multiple of four floats; the lengths in CatArgs, row and total count float4s then.
+__device__ __forceinline__ float cat_add(float a, float b) { return a + b; }
+__device__ __forceinline__ float4 cat_add(float4 a, float4 b) { return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w); }
+template <bool GRAD, class T>
+__global__ void __launch_bounds__(TPB) k_concat(CatArgs a, float* cat_, int64_t row, int64_t total) {
+  T* cat = reinterpret_cast<T*>(cat_);
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, s = (int64_t)gridDim.x * TPB;
-  for (; i < n; i += s) {
-    int64_t h = i / st, l = i - h * st;
-    int64_t o = h * row + off + l;
-    if (GRAD == 1) dst[i] += src[o]; else if (GRAD == 2) dst[i] = src[o]; else dst[o] = src[i];
+  const bool narrow = total < 0x7fffffffLL && row < 0x7fffffffLL;      // 32-bit divisions where they suffice
+  for (; i < total; i += s) {
+    int64_t h, l;
+    if (narrow) { const uint32_t hh = (uint32_t)i / (uint32_t)a.width; h = hh; l = a.lo + ((uint32_t)i - hh * (uint32_t)a.width); }
+    else { h = i / a.width; l = a.lo + (i - h * a.width); }
+    int t = 0;
+#pragma unroll
+    for (int u = 1; u < CAT_MAX; u++) if (u < a.n && l >= a.off[u]) t = u;
+    T* q = reinterpret_cast<T*>(a.p[t]);
+    if (q == nullptr) continue;
+    const int64_t o = h * row + l, e = h * a.st[t] + (l - a.off[t]);
+    if (GRAD) q[e] = a.add[t] ? cat_add(q[e], cat[o]) : cat[o]; else cat[o] = q[e];
   }
 }
+// shrinks the lengths to float4 units when everything is a multiple of four floats and 16-byte aligned
+static bool cat_vectorize(CatArgs& a, const float* cat, int64_t& row, int64_t& tot) {
+  if ((row | a.lo | a.width) & 3 || ((uintptr_t)cat & 15)) return false;
+  for (int u = 0; u < a.n; u++) if ((a.st[u] | a.off[u]) & 3 || ((uintptr_t)a.p[u] & 15)) return false;
+  for (int u = 0; u < a.n; u++) { a.st[u] >>= 2; a.off[u] >>= 2; }
+  a.lo >>= 2; a.width >>= 2; row >>= 2; tot >>= 2;
+  return true;
+}
+template <bool GRAD>
+static void cat_launch(CatArgs a, float* cat, int64_t row, int64_t tot) {
+  if (cat_vectorize(a, cat, row, tot)) hipLaunchKernelGGL((k_concat<GRAD, float4>), dim3(stream_grid(tot, TPB * 2)), dim3(TPB), 0, g_stream, a, cat, row, tot);
+  else hipLaunchKernelGGL((k_concat<GRAD, float>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, a, cat, row, tot);
+}
+}  // namespace
 extern "C" {
 void lh_concat(int n, const float* const* h_in, const int* sizes, float* out, int outer, int inner) {
   int64_t row = 0; for (int t = 0; t < n; t++) row += (int64_t)sizes[t] * inner;
@@ -677,10 +706,12 @@ void lh_concat(int n, const float* const* h_in, const int* sizes, float* out, in
   for (int t = 0; t < n; t++) lazy::rd_f(h_in[t], (int64_t)sizes[t] * inner * outer);
   lazy::wr_f(out, row * outer);
   int64_t off = 0;
-  for (int t = 0; t < n; t++) {
-    int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
-    if (tot > 0) hipLaunchKernelGGL((k_concat<0>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, h_in[t], out, st, row, off, tot);
-    off += st;
+  for (int t0 = 0; t0 < n; t0 += CAT_MAX) {
+    CatArgs a{}; a.n = n - t0 < CAT_MAX ? n - t0 : CAT_MAX; a.lo = off;
+    for (int u = 0; u < a.n; u++) { a.p[u] = const_cast<float*>(h_in[t0 + u]); a.st[u] = (int64_t)sizes[t0 + u] * inner; a.off[u] = off; off += a.st[u]; }
+    a.width = off - a.lo;
+    const int64_t tot = a.width * outer;
+    if (tot > 0) cat_launch<false>(a, out, row, tot);
   }
   LH_CHECK_LAUNCH();
 }
@@ -689,14 +720,17 @@ void lh_concat_grad_beta(int n, float* const* h_ind, const float* h_beta, const 
   for (int t = 0; t < n && h_beta; t++) LH_REQUIRE(h_beta[t] == 0.f || h_beta[t] == 1.f, "lh_concat_grad_beta: beta must be 0 or 1");
   LZ_ENTER(); lazy::rd_f(outd, row * outer);
   int64_t off = 0;
-  for (int t = 0; t < n; t++) {
-    int64_t st = (int64_t)sizes[t] * inner, tot = st * outer;
-    if (tot > 0 && h_ind[t]) {
-      const float beta = lazy::beta_f(h_ind[t], tot, h_beta ? h_beta[t] : 1.f);
-      if (beta == 0.f) hipLaunchKernelGGL((k_concat<2>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
-      else hipLaunchKernelGGL((k_concat<1>), dim3(stream_grid(tot, TPB * 4)), dim3(TPB), 0, g_stream, outd, h_ind[t], st, row, off, tot);
+  for (int t0 = 0; t0 < n; t0 += CAT_MAX) {
+    CatArgs a{}; a.n = n - t0 < CAT_MAX ? n - t0 : CAT_MAX; a.lo = off;
+    bool any = false;
+    for (int u = 0; u < a.n; u++) {
+      const int t = t0 + u;
+      a.p[u] = h_ind[t]; a.st[u] = (int64_t)sizes[t] * inner; a.off[u] = off; off += a.st[u];
+      if (a.p[u] && a.st[u] > 0) { a.add[u] = lazy::beta_f(a.p[u], a.st[u] * outer, h_beta ? h_beta[t] : 1.f) != 0.f; any = true; }
     }
-    off += st;
+    a.width = off - a.lo;
+    const int64_t tot = a.width * outer;
+    if (tot > 0 && any) cat_launch<true>(a, const_cast<float*>(outd), row, tot);
   }
   LH_CHECK_LAUNCH();
 }

@@ -151,6 +151,8 @@ struct EpiRowMajor {
   __device__ __forceinline__ uint32_t cell_row_bytes() const { return 0u; }
   __device__ __forceinline__ int lean_mode() const { return beta == 0.f ? 0 : 1; }
   __device__ __forceinline__ float lean_scale() const { return alpha; }
+  static constexpr bool LEAN_FIX = false;         // nothing is added to or clamped in a stored element
+  __device__ __forceinline__ float lean_fix(float v, int) const { return v; }
   // part: 0 = the whole reduction of this element is in v; 1 = first partial sum, 2 = a later one
   // (partials are combined with atomic adds onto an output the host has prepared)
   __device__ __forceinline__ void store(const Col& c, int i, int M, float v, int part) const {
@@ -456,6 +458,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
 #pragma unroll
             for (int ni = 0; ni < NI; ni++) {
               float val = acc[mi][ni][v] * scale;
+              if constexpr (EP::LEAN_FIX) val = ep.lean_fix(val, row + 4 * half);
               if constexpr (MD == 1) val = fmaf(ep.beta, old[v][ni], val);
               if constexpr (MD == 2) {
                 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));

@@ -333,7 +333,7 @@ void lh_d2d(void* dst, const void* src, size_t bytes) {
 void lh_side_begin(void) {
   LH_REQUIRE(g_stream_raw != nullptr, "lh_side_begin before lh_setup");
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_side_begin: already on the side stream");
-  LZ_ENTER();                    // what is parked belongs in front of the fork
+  LZ_SCOPE();                    // what is parked stays parked: whoever launches it from the side stream does so on the main stream and lets the side stream wait
   // In line (no concurrency) when switched off, while kernels are timed one by one, or while the stream is recorded.
   if (!g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on || g_deterministic) return;
   hipEvent_t ev = side_event();

@@ -389,18 +389,24 @@ trait TensorDslHIP extends TensorDslCPU with GPUOps {
       assert(dilations == ((1, 1)), "dilated convolutions are not supported")
       val (n, c, h, w) = (input.x.shape(0), input.x.shape(1), input.x.shape(2), input.x.shape(3))
       val (k, r, s) = (filter.x.shape(0), filter.x.shape(2), filter.x.shape(3))
-      if (!input.isInput)                                         // CDN:873
-        hip("lh_conv2d_bwd_data", res.d.data, filter.x.data, input.d.data, 1.0f, n, c, h, w, k, r, s, strides._1, strides._2, padding._1, padding._2)
       // Only the optimizer reads filter.d: the filter gradient runs on the library's side stream beside the rest of the backward
       // pass, unless fewer than two convolution gradients are still to come (with nothing left to run beside it the hand-over
       // between the streams only delays the optimizer; the optimizer entry points join).  Gradient calls are staged in the reverse
       // order of the forward calls, so the count of forward convolutions not yet matched is known here at staging time.
       convsOpen -= 1
       val fork = !input.isInput && convsOpen >= 2
-      if (fork) hip("lh_side_begin")
-      hip("lh_conv2d_bwd_filter", input.x.data, res.d.data, filter.d.data, bias.map(_.d.data: Any).getOrElse(nullFloats), 1.0f,
-          n, c, h, w, k, r, s, strides._1, strides._2, padding._1, padding._2)
-      if (fork) hip("lh_side_end")
+      def filterGradient(): Unit = {
+        if (fork) hip("lh_side_begin")
+        hip("lh_conv2d_bwd_filter", input.x.data, res.d.data, filter.d.data, bias.map(_.d.data: Any).getOrElse(nullFloats), 1.0f,
+            n, c, h, w, k, r, s, strides._1, strides._2, padding._1, padding._2)
+        if (fork) hip("lh_side_end")
+      }
+      // With a bias the filter gradient is issued first: its bias sums are the first reader of res.d, and a relu_grad(inPlace)
+      // issued just before (conv -> relu networks) is applied in that pass instead of in one of its own.
+      if (bias.isDefined) filterGradient()
+      if (!input.isInput)                                         // CDN:873
+        hip("lh_conv2d_bwd_data", res.d.data, filter.x.data, input.d.data, 1.0f, n, c, h, w, k, r, s, strides._1, strides._2, padding._1, padding._2)
+      if (!bias.isDefined) filterGradient()
     }
 
     // ---- pooling (CDN:882-982).  Max-pool keeps its argmax (global flat input index, first maximum wins: CPU:848-948), which the

@@ -34,6 +34,10 @@ void zero_bytes_async(void* p, size_t bytes) { (void)ordered_stream(); memset(p,
 void mask_relu(float* dst, const float* src, const float* y, int64_t n) { (void)ordered_stream(); for (int64_t i = 0; i < n; i++) dst[i] = y[i] > 0.f ? src[i] : 0.f; g_kernels++; }
 void add_plain(const float* a, const float* b, float* out, int64_t n) { (void)ordered_stream(); for (int64_t i = 0; i < n; i++) out[i] = a[i] + b[i]; g_kernels++; }
 void relu_grad_inplace_now(const float* y, float* d, int64_t n) { (void)ordered_stream(); for (int64_t i = 0; i < n; i++) d[i] = y[i] > 0.f ? d[i] : 0.f; g_kernels++; }
+static void sim_conv_relu(const float* x, const float* w, const float* bias, float* y);
+void conv2d_fwd_relu_now(const float* x, const float* w, const float* bias, float* y, int, int, int, int, int, int, int, int, int, int, int) { (void)ordered_stream(); sim_conv_relu(x, w, bias, y); }
+static void sim_bias_grad(const float* y, float* dy, float* db);
+void conv_bwd_bias_mask_now(const float* y, float* dy, float* db, int, int, int) { (void)ordered_stream(); sim_bias_grad(y, dy, db); }
 static void k_update(int mode, float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) {
   for (int64_t i = 0; i < n; i++) {
     if (mode == 0) { x[i] = x[i] * 1.0f + d[i] * (-lr); d[i] = 0.f; continue; }
@@ -83,6 +87,11 @@ static inline int chan(int i) { return (i / HW_) % C_; }
 static void k_conv(const float* x, const float* w, const float* bias, float* y) { for (int i = 0; i < NE; i++) { float a = bias ? bias[chan(i)] : 0.f; for (int k = 0; k < 3; k++) a += x[(i + 7 * k) % NE] * w[(chan(i) + k) % 12]; y[i] = a; } g_kernels++; }
 static void k_conv_bwd_data(const float* dy, const float* w, float* dx, float beta) { for (int i = 0; i < NE; i++) { float a = 0.f; for (int k = 0; k < 3; k++) a += dy[(i + NE - 7 * k) % NE] * w[(chan((i + NE - 7 * k) % NE) + k) % 12]; dx[i] = (beta != 0.f ? dx[i] : 0.f) + a; } g_kernels++; }
 static void k_conv_bwd_filter(const float* x, const float* dy, float* dw, float beta) { for (int j = 0; j < 12; j++) { float a = 0.f; for (int i = 0; i < NE; i++) for (int k = 0; k < 3; k++) if ((chan(i) + k) % 12 == j) a += dy[i] * x[(i + 7 * k) % NE]; dw[j] = (beta != 0.f ? dw[j] : 0.f) + a; } g_kernels++; }
+namespace lh {
+static void sim_conv_relu(const float* x, const float* w, const float* bias, float* y) { k_conv(x, w, bias, y); for (int i = 0; i < NE; i++) y[i] = y[i] < 0.f ? 0.f : y[i]; }
+// bias gradient: channel sums of dy in element order; with y, dy is masked by y > 0 on the way (and written back)
+static void sim_bias_grad(const float* y, float* dy, float* db) { for (int i = 0; i < NE; i++) { if (y) dy[i] = y[i] > 0.f ? dy[i] : 0.f; db[chan(i)] += dy[i]; } g_kernels++; }
+}
 static void k_stats(const float* x, float* sm, float* si, float* rm, float* rv) {
   for (int c = 0; c < C_; c++) {
     double s = 0, q = 0; int cnt = 0;
@@ -237,6 +246,15 @@ static void t_conv_bwd(const float* x, const float* dy, const float* w, float* d
   { LZ_ENTER(); lazy::rd_f(dy, NE); lazy::rd_f(w, 12); float beta = lazy::beta_f(dx, NE, 1.f); (void)ordered_stream(); k_conv_bwd_data(dy, w, dx, beta); }
   { LZ_ENTER(); lazy::rd_f(x, NE); lazy::rd_f(dy, NE); float beta = lazy::beta_f(dw, 12, 1.f); (void)ordered_stream(); k_conv_bwd_filter(x, dy, dw, beta); }
 }
+// a convolution with a bias: the filter gradient (bias sums included) goes first, as the backends issue it
+static void t_conv_bwd_bias(const float* x, float* dy, const float* w, float* dx, float* dw, float* db) {
+  { LZ_SCOPE();
+    const bool done = lazy::g_busy && !lazy::g_replay && lazy::take_relu_grad_bias(dy, db, N_, C_, HW_);
+    if (lazy::g_busy && !lazy::g_replay) lazy::flush_parked();
+    lazy::rd_f(x, NE); lazy::rd_f(dy, NE); float beta = lazy::beta_f(dw, 12, 1.f); lazy::rw_f(db, C_);
+    (void)ordered_stream(); k_conv_bwd_filter(x, dy, dw, beta); if (!done) sim_bias_grad(nullptr, dy, db); }
+  if (dx) { LZ_ENTER(); lazy::rd_f(dy, NE); lazy::rd_f(w, 12); float beta = lazy::beta_f(dx, NE, 1.f); (void)ordered_stream(); k_conv_bwd_data(dy, w, dx, beta); }
+}
 static void t_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) {
   LZ_SCOPE();
   if (lazy::gather_update(1, x, d, v, lr, mu, clip, nesterov, n)) return;
@@ -258,7 +276,7 @@ static int ri(int lo, int hi) { return lo + (int)(rnd() % (uint32_t)(hi - lo + 1
 static float rf() { return (float)((int)(rnd() % 2001) - 1000) / 500.0f; }
 
 struct TR { float* x; float* d; };                 // a TensorR: value and gradient, both from the zero-filled arena
-struct Layer { int kind; TR in, conv, bn, sc, out; float *w, *dw, *wv, *g, *dg, *gv, *b, *db, *bv, *rm, *rv, *sm, *si; bool relu, join, has_conv; };
+struct Layer { int kind; TR in, conv, bn, sc, out; float *w, *dw, *wv, *g, *dg, *gv, *b, *db, *bv, *rm, *rv, *sm, *si; bool relu, join, has_conv, nobn; };
 
 static void run_program(uint64_t seed, bool enabled, std::vector<float>& trace, std::vector<char>& image, long long& kernels) {
   g_rng = seed;
@@ -283,6 +301,17 @@ static void run_program(uint64_t seed, bool enabled, std::vector<float>& trace, 
     TR h; h.x = input; h.d = nullptr;
     for (auto& l : L) {
       l.in = h; l.has_conv = ri(0, 4) != 0; l.join = ri(0, 2) == 0 && h.d != nullptr; l.relu = l.join || ri(0, 3) != 0;
+      l.nobn = ri(0, 3) == 0;
+      if (l.nobn) {                 // conv + bias -> relu in place, no batch norm (networks of that kind)
+        l.has_conv = true; l.join = false;
+        float* y = (float*)sim_malloc(SZ(NE), true); lh_conv2d_fwd(h.x, l.w, l.b, y, N_, C_, 1, HW_, C_, 1, 1, 1, 1, 0, 0); l.conv = tr(y);
+        if (ri(0, 9) == 0) t_d2h(trace, y, 5);
+        if (ri(0, 11) == 0) { float* tmp = (float*)sim_malloc(SZ(NE), true); t_geam(y, 1.f, y, 0.f, tmp, NE); }
+        if (l.relu) t_relu_inplace(y, NE);
+        l.bn = l.conv; l.out = l.conv; h = l.conv;
+        if (ri(0, 7) == 0) t_d2h(trace, y + ri(0, NE - 4), 4);
+        continue;
+      }
       const float* x = h.x;
       if (l.has_conv) { float* y = (float*)sim_malloc(SZ(NE), true); lh_conv2d_fwd(h.x, l.w, nullptr, y, N_, C_, 1, HW_, C_, 1, 1, 1, 1, 0, 0); l.conv = tr(y); x = y; }
       if (ri(0, 9) == 0) t_d2h(trace, x, 5);                                        // a read in between ends the chain
@@ -307,6 +336,7 @@ static void run_program(uint64_t seed, bool enabled, std::vector<float>& trace, 
       Layer& l = L[li];
       if (l.relu) t_relu_grad_inplace(l.out.x, l.out.d, NE);
       if (ri(0, 13) == 0) t_d2h(trace, l.out.d, 6);
+      if (l.nobn) { t_conv_bwd_bias(l.in.x, l.conv.d, l.w, l.in.d, l.dw, l.db); continue; }
       if (l.join) t_add_grad(l.bn.d, l.sc.d, l.out.d, NE);
       const TR& bx = l.has_conv ? l.conv : l.in;
       lh_bn_bwd(bx.x, l.bn.d, l.g, l.sm, l.si, bx.d, 1.0f, l.dg, l.db, N_, C_, HW_);

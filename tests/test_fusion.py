@@ -280,3 +280,98 @@ def test_parked_calls_run_in_program_order_around_other_calls(prog):
     np.testing.assert_array_equal(prog.down(cp, (NY,)), np.maximum(t_host.ravel(), 0))
     np.testing.assert_allclose(prog.down(t2, (NY,)), t_host.ravel(), rtol=1e-5, atol=1e-5)      # statistics from a pass of their own here
     _lib.check()
+
+
+def _trait_conv_bias_relu(pg, inp, geom, side=False):
+    """conv(+ bias) -> relu(inPlace) and its backward, one call per trait method: what a network without batch norms
+    (SqueezeNet's fire modules) issues.  The filter gradient goes first, as the backends issue it when there is a bias."""
+    lib = pg.lib
+    n, c, h, k, r, pad = geom
+    args = (n, c, h, h, k, r, r, 1, 1, pad, pad)
+    p = h + 2 * pad - r + 1
+    nx, ny = n * c * h * h, n * k * p * p
+    x, w, b = pg.up(inp["x"]), pg.up(inp["w"]), pg.up(inp["b"])
+    dw, db, dx = pg.malloc(k * c * r * r), pg.malloc(k), pg.malloc(nx)
+    y = pg.malloc(ny); lib.lh_conv2d_fwd(x, w, b, y, *args)
+    dy = pg.malloc(ny)
+    lib.lh_unary(RELU, y, y, ny, 0.0, 0.0)
+    _lib.check()
+    g = np.ascontiguousarray(inp["dout"]); lib.lh_h2d(dy, g.ctypes.data, g.nbytes)
+    lib.lh_unary_grad(RELU, y, y, dy, dy, ny, 1, 0.0, 0.0)
+    if side: lib.lh_side_begin()
+    lib.lh_conv2d_bwd_filter(x, dy, dw, db, 1.0, *args)
+    if side: lib.lh_side_end()
+    lib.lh_conv2d_bwd_data(dy, w, dx, 1.0, *args)
+    _lib.check()
+    return dict(y=pg.down(y, (ny,)), dy=pg.down(dy, (ny,)), dw=pg.down(dw, (k * c * r * r,)), db=pg.down(db, (k,)), dx=pg.down(dx, (nx,)))
+
+
+def _bias_inputs(seed, geom):
+    n, c, h, k, r, pad = geom
+    p = h + 2 * pad - r + 1
+    rng = np.random.RandomState(seed)
+    return dict(x=rng.randn(n, c, h, h).astype(np.float32), w=(rng.randn(k, c, r, r) / np.sqrt(c * r * r)).astype(np.float32),
+                b=(0.3 * rng.randn(k)).astype(np.float32), dout=rng.randn(n, k, p, p).astype(np.float32))
+
+
+@pytest.mark.parametrize("geom", [(8, 64, 28, 64, 3, 1), (64, 16, 16, 64, 1, 0), (4, 48, 9, 24, 3, 0)], ids=["3x3_28", "1x1_16", "ragged"])
+def test_conv_bias_relu_and_its_gradient_run_as_two_fewer_kernels_with_the_same_bits(prog, geom):
+    inp = _bias_inputs(41, geom)
+    s0 = _stats(prog.lib)
+    got = _trait_conv_bias_relu(prog, inp, geom)
+    s1 = _stats(prog.lib)
+    assert s1[0] - s0[0] == 1 and s1[1] - s0[1] == 1, "the clamp was to ride in the convolution's epilogue and the mask in the bias sums: %s" % (s1 - s0)
+    prog.lib.lh_set_fusion(0)
+    plain = _trait_conv_bias_relu(prog, inp, geom)
+    for k, v in plain.items():
+        np.testing.assert_array_equal(got[k], v, err_msg=k)
+    assert (got["y"] >= 0).all() and (got["y"] == 0).any()
+    np.testing.assert_array_equal(got["dy"], inp["dout"].ravel() * (got["y"] > 0))
+
+
+def test_conv_bias_relu_where_partial_sums_are_added_and_on_the_side_stream(on_hip):
+    """Default mode: a long reduction over few tiles runs with several blocks per tile adding their partial sums, so the
+    clamp cannot ride in the epilogue everywhere (it is applied by a pass behind the launch), and the filter gradient, bias
+    sums included, is issued on the side stream with the relu_grad still parked."""
+    pg = Prog(on_hip)
+    geom = (16, 1024, 16, 256, 3, 1)
+    inp = _bias_inputs(43, geom)
+    got = _trait_conv_bias_relu(pg, inp, geom, side=True)
+    on_hip.lib.lh_set_fusion(0)
+    try:
+        plain = _trait_conv_bias_relu(pg, inp, geom, side=True)
+    finally:
+        on_hip.lib.lh_set_fusion(1)
+    assert (got["y"] >= 0).all() and (got["y"] == 0).any()
+    for k, v in plain.items():
+        assert_close(got[k], v, rtol=2e-5, what=k)
+    # the mask is a function of y's sign, and a sum that lands within rounding of zero may fall on either side
+    agree = (got["y"] > 0) == (plain["y"] > 0)
+    assert agree.mean() > 0.9999
+
+
+def test_concat_of_more_tensors_than_one_launch_takes(prog):
+    lib = prog.lib
+    rng = np.random.RandomState(47)
+    outer, inner = 6, 35
+    sizes = [3, 1, 0, 7, 2, 5, 4]
+    parts = [rng.randn(outer, s, inner).astype(np.float32) for s in sizes]
+    ptrs = [prog.up(p) if p.size else 0 for p in parts]
+    row = sum(sizes)
+    out = prog.malloc(outer * row * inner)
+    lib.lh_concat(len(sizes), (C.c_void_p * len(sizes))(*ptrs), _ints(*sizes), out, outer, inner); _lib.check()
+    want = np.concatenate(parts, axis=1)
+    np.testing.assert_array_equal(prog.down(out, want.shape), want)
+    # gradient: accumulated into some, overwriting others, skipped for one
+    dout = rng.randn(*want.shape).astype(np.float32)
+    d_out = prog.up(dout)
+    init = [rng.randn(*p.shape).astype(np.float32) for p in parts]
+    dptrs = [prog.up(a) if a.size else 0 for a in init]
+    dptrs[3] = 0
+    betas = [1.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0]
+    lib.lh_concat_grad_beta(len(sizes), (C.c_void_p * len(sizes))(*dptrs), (F * len(sizes))(*betas), _ints(*sizes), d_out, outer, inner); _lib.check()
+    off = 0
+    for t, s in enumerate(sizes):
+        if s and dptrs[t]:
+            np.testing.assert_array_equal(prog.down(dptrs[t], init[t].shape), betas[t] * init[t] + dout[:, off:off + s, :], err_msg="tensor %d" % t)
+        off += s

@@ -142,6 +142,7 @@ TUNED_SHAPES = [
     (16, 32, 28, 28, 32, 3, 3, 1, 1, 1, 1),     # 32 channels in and out: the 32-row tiles compete in forward and input gradient (tap path)
     (50, 10, 12, 12, 20, 5, 5, 1, 1, 0, 0),     # LeNet's second convolution: 20- and 10-row products through the general loaders
     (8, 1, 41, 60, 32, 11, 5, 2, 2, 0, 0),      # one input channel, tall filter, stride 2 (DeepSpeech2's first layer in small)
+    (64, 512, 4, 4, 10, 4, 4, 1, 1, 0, 0),      # a filter as large as the map (SqueezeNet's classifier): one tile under an 8192-long reduction, the plans with one worker per few slabs compete
 ]
 
 

@@ -231,7 +231,7 @@ def test_resnet_imagenet_stem_3_steps(hip_backend, cpu_backend):
 def test_squeezenet_10_steps(hip_backend, cpu_backend):
     """All 26 biased convs, 8 concats, 3 max-pools, momentum SGD (the reference's configuration but batch 16)."""
     from lantern_amd.apps.squeezenet import Trainer
-    _compare(lambda: Trainer(batch=16, lr=0.001), hip_backend, cpu_backend)
+    _compare(lambda: Trainer(batch=16, lr=0.001), hip_backend, cpu_backend, flip_tol=5e-3)
 
 
 def test_squeezenet_avgpool_head_5_steps(hip_backend, cpu_backend):
