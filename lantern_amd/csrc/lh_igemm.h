@@ -613,8 +613,8 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
   return true;
 }
 
-// Times `launch` (a callable returning false on failure) on the library's stream: three repetitions, the first warms
-// the caches, the smaller of the other two counts.  Returns a negative number when a launch or the timer failed.
+// Times `launch` (a callable returning false on failure) on the library's stream: five repetitions, the first warms
+// the caches, the smallest of the other four counts (with two, which of two close plans won changed from run to run).  Returns a negative number when a launch or the timer failed.
 struct LaunchTimer {
   hipEvent_t e0 = nullptr, e1 = nullptr;
   bool ok;
@@ -623,7 +623,7 @@ struct LaunchTimer {
   template <class F>
   float ms(F launch) {
     float best = 3.0e38f;
-    for (int rep = 0; rep < 3; rep++) {
+    for (int rep = 0; rep < 5; rep++) {
       (void)hipEventRecord(e0, g_stream);
       if (!launch()) return -1.f;
       (void)hipEventRecord(e1, g_stream);
