@@ -13,6 +13,11 @@ extern hipStream_t g_stream_raw;  // the library's stream
 // Where entry points enqueue now: g_stream_raw, or the side stream between lh_side_begin and lh_side_end.
 extern hipStream_t g_stream_cur;
 void side_join();                 // the main stream waits for what the side stream was given (no-op when it is idle)
+void* side_scratch(size_t bytes); // a block for the kernels of the side stream (one user at a time, in that stream's order); nullptr after a reported failure
+// Scratch memory for a launch: the top of the arena on the main stream (stream order puts the next user of the same memory
+// behind this launch), the side stream's own block on the side stream.  One block per entry point at a time.
+void* scratch_take(size_t bytes, bool& side);
+void scratch_give(size_t bytes, bool side);
 void quiet_other_stream();        // host-side wait for the stream that is NOT current, so that a timing run has the device to itself
 // Small operations recorded by the command list (lh_cmdlist.hip) but not launched yet.  Anything that is about to use
 // the stream goes through `g_stream`, which launches the recorded commands first, so program order is kept.

@@ -942,14 +942,14 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   if (K <= 32 && force_m32()) { tp = TilePick{32, 128}; tiles = cdiv(K, 32) * cdiv(CRS, 128); split = clamp_split(cdiv(3 * (int64_t)g_num_cu, tiles)); tune_now = false; }
   // Deterministic mode: every slice of the reduction writes its own [K, CRS] block of scratch memory (no atomics), and a
   // second kernel adds the blocks onto beta*dw in slice order.
-  float* partial = nullptr; size_t partial_bytes = 0; int slices = 1;
+  float* partial = nullptr; size_t partial_bytes = 0; int slices = 1; bool on_side = false;
   if (g_deterministic && split > 1) {
     const int bk = tp.bm == 128 ? 16 : (tp.bm == 32 ? 32 : BWDF_BK);
     int64_t kper = cdiv(cdiv(red, split), bk) * bk; if (kper < bk) kper = bk;
     slices = (int)cdiv(red, kper);                                    // what igemm_launch will make of `split`
     if (slices > 1) {
       partial_bytes = (size_t)slices * K * CRS * sizeof(float);
-      partial = (float*)lh_malloc_uninit(partial_bytes);
+      partial = (float*)scratch_take(partial_bytes, on_side);
       if (partial == nullptr) return;
     }
   }
@@ -990,7 +990,8 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   };
   if (tune_now) {
     const size_t sbytes = (size_t)K * CRS * sizeof(float);
-    float* scratch = (float*)lh_malloc_uninit(sbytes);
+    bool tune_side = false;
+    float* scratch = (float*)scratch_take(sbytes, tune_side);
     LaunchTimer timer;
     if (scratch && timer.ok) {
       const double targets[] = {1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 5.0, 6.0};
@@ -1020,13 +1021,13 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
       g_bwdf_split[key] = best; g_plans_measured++;
       if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: tile %dx%d, %lld tiles, split %d (%.3f ms)\n", N, C, H, K, R, sH, tp.bm, tp.bn, (long long)tiles, split, best_ms);
     }
-    if (scratch) lh_free_top(sbytes);
+    if (scratch) scratch_give(sbytes, tune_side);
     if (failed()) return;
   }
   dispatch();
   if (partial) {
     if (ok) reduce_slices(dw, CRS, K, CRS, partial, slices, beta);
-    lh_free_top(partial_bytes);
+    scratch_give(partial_bytes, on_side);
   }
   if (!ok) return;
   if (db && !bias_done) bias_grad_launch(nullptr, const_cast<float*>(dy), db, N, K, PQ);

@@ -152,8 +152,33 @@ __global__ void __launch_bounds__(TPB) k_scale_rows(float* C, int ldc, int m, in
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
   for (; i < tot; i += st) { const int r = (int)(i / n), c = (int)(i - (int64_t)r * n); float* p = C + (int64_t)r * ldc + c; *p = beta == 0.f ? 0.f : beta * *p; }
 }
-// C = beta*C + sum of the slices' partial products, in slice order (the deterministic stand-in for atomic adds)
+// C = beta*C + sum of the slices' partial products, in slice order (the deterministic stand-in for atomic adds).
+// VEC: n and ldc are multiples of 4 and both pointers 16-byte aligned: four neighbours per lane, the loads of eight slices in flight.
+template <bool VEC>
 __global__ void __launch_bounds__(TPB) k_reduce_slices(float* C, int ldc, int m, int n, const float* __restrict__ partial, int slices, float beta) {
+  if (VEC) {
+    const int n4 = n >> 2;
+    const int64_t tot4 = (int64_t)m * n4;
+    const float4* __restrict__ P = reinterpret_cast<const float4*>(partial);
+    int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
+    for (; i < tot4; i += st) {
+      const int r = (int)(i / n4), c = (int)(i - (int64_t)r * n4);
+      float4* p = reinterpret_cast<float4*>(C + (int64_t)r * ldc) + c;
+      float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (beta != 0.f) { const float4 o = *p; acc = make_float4(beta * o.x, beta * o.y, beta * o.z, beta * o.w); }
+      int s = 0;
+      for (; s + 8 <= slices; s += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = P[(int64_t)(s + u) * tot4 + i];
+#pragma unroll
+        for (int u = 0; u < 8; u++) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
+      }
+      for (; s < slices; s++) { const float4 v = P[(int64_t)s * tot4 + i]; acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w; }
+      *p = acc;
+    }
+    return;
+  }
   const int64_t tot = (int64_t)m * n;
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
   for (; i < tot; i += st) {
@@ -173,7 +198,9 @@ static bool sgemm_mfma(const AL& al, const BL& bl, const EpiRowMajor& ep, int m,
 
 namespace lh {
 void reduce_slices(float* C, int ldc, int m, int n, const float* partial, int slices, float beta) {
-  hipLaunchKernelGGL(k_reduce_slices, dim3(stream_grid((int64_t)m * n, TPB * 2)), dim3(TPB), 0, g_stream, C, ldc, m, n, partial, slices, beta);
+  const bool vec = (n % 4 == 0) && (ldc % 4 == 0) && ((((uintptr_t)C | (uintptr_t)partial) & 15) == 0);
+  if (vec) hipLaunchKernelGGL((k_reduce_slices<true>), dim3(stream_grid((int64_t)m * (n / 4), TPB)), dim3(TPB), 0, g_stream, C, ldc, m, n, partial, slices, beta);
+  else hipLaunchKernelGGL((k_reduce_slices<false>), dim3(stream_grid((int64_t)m * n, TPB * 2)), dim3(TPB), 0, g_stream, C, ldc, m, n, partial, slices, beta);
 }
 }  // namespace lh
 
@@ -204,12 +231,12 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
     // one product under plan `pl` into Cout (row stride ldo) with the given beta
     auto run = [&](const SgemmPlan& pl, float* Cout, int ldo, float be) -> bool {
       EpiRowMajor e; e.C = Cout; e.ldc = ldo; e.alpha = alpha; e.beta = be; e.atomic = 0;
-      float* partial = nullptr; size_t pbytes = 0; int slices = 1;
+      float* partial = nullptr; size_t pbytes = 0; int slices = 1; bool pside = false;
       if (pl.split > 1 && g_deterministic) {            // slices into scratch blocks, added in order afterwards
         int64_t kper = cdiv(cdiv(k, pl.split), 16) * 16; if (kper < 16) kper = 16;
         slices = (int)cdiv(k, kper);
         pbytes = (size_t)slices * m * n * sizeof(float);
-        partial = (float*)lh_malloc_uninit(pbytes);
+        partial = (float*)scratch_take(pbytes, pside);
         if (partial == nullptr) return false;
         e.C = partial; e.ldc = n; e.beta = 0.f; e.sliceStride = (long long)m * n;
       } else if (pl.split > 1) {
@@ -224,7 +251,7 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
       else good = bv ? sgemm_mfma(at, bkv, e, m, n, k, pl) : sgemm_mfma(at, bks, e, m, n, k, pl);
       if (partial) {
         if (good) reduce_slices(Cout, ldo, m, n, partial, slices, be);
-        lh_free_top(pbytes);
+        scratch_give(pbytes, pside);
       }
       return good;
     };
@@ -237,7 +264,8 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
       if (it != chosen.end()) { pl = it->second; g_plans_remembered++; }
       else if (g_tune_measure) {
         const size_t sbytes = (size_t)m * n * sizeof(float);
-        float* scratch = (float*)lh_malloc_uninit(sbytes);
+        bool sside = false;
+        float* scratch = (float*)scratch_take(sbytes, sside);
         LaunchTimer timer;
         if (scratch && timer.ok) {
           const TilePick shapes[3] = {{128, 128}, {64, 128}, {64, 64}};
@@ -265,7 +293,7 @@ void lh_sgemm(int ta, int tb, int m, int n, int k, float alpha, const float* A, 
           if (best_ms >= 0.f && !failed()) { chosen[key] = best; pl = best; g_plans_measured++; }
           if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "sgemm ta%d tb%d %dx%dx%d: tile %dx%d, %d slice(s), %.3f ms\n", ta, tb, m, n, k, best.tp.bm, best.tp.bn, best.split, best_ms);
         }
-        if (scratch) lh_free_top(sbytes);
+        if (scratch) scratch_give(sbytes, sside);
         if (failed()) return;
       }
     }

@@ -29,6 +29,24 @@ void side_wait_for_main() {
   LH_HIP(hipEventRecord(ev, g_stream_raw));
   LH_HIP(hipStreamWaitEvent(g_side_stream, ev, 0));
 }
+// Scratch memory for kernels on the side stream.  Scratch from the top of the arena is safe on the main stream only (the stream
+// orders the next user of the same memory behind the kernel that was given it); the side stream's kernels run in their own
+// order among themselves, so they share one block of their own, which grows on demand.
+static char* g_side_scratch = nullptr; static size_t g_side_scratch_bytes = 0;
+void* side_scratch(size_t bytes) {
+  if (bytes <= g_side_scratch_bytes) return g_side_scratch;
+  if (hipDeviceSynchronize() != hipSuccess) { LH_FAIL("side scratch: the device did not come to rest"); return nullptr; }
+  if (g_side_scratch) (void)hipFree(g_side_scratch);
+  g_side_scratch = nullptr; g_side_scratch_bytes = 0;
+  const size_t want = ((bytes + (bytes >> 2)) + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+  void* p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess || p == nullptr) { LH_FAIL("side scratch: cannot allocate %zu bytes", want); return nullptr; }
+  g_side_scratch = (char*)p; g_side_scratch_bytes = want;
+  return p;
+}
+void* scratch_take(size_t bytes, bool& side) { side = g_stream_cur != g_stream_raw; return side ? side_scratch(bytes) : lh_malloc_uninit(bytes); }
+void scratch_give(size_t bytes, bool side) { if (!side) lh_free_top(bytes); }
+static void side_scratch_release() { if (g_side_scratch) (void)hipFree(g_side_scratch); g_side_scratch = nullptr; g_side_scratch_bytes = 0; }
 void side_join() {
   if (!g_side_dirty) return;
   g_side_dirty = false;
@@ -149,6 +167,7 @@ void lh_cleanup(void) {
   g_side_stream = nullptr; g_side_dirty = false;
   if (g_stream_raw) (void)hipStreamSynchronize(g_stream);
   cmdlist_release();
+  side_scratch_release();
   stage_release();
   copy_release();
   multi_tensor_release();
@@ -335,7 +354,9 @@ void lh_side_begin(void) {
   LH_REQUIRE(g_stream_cur == g_stream_raw, "lh_side_begin: already on the side stream");
   LZ_SCOPE();                    // what is parked stays parked: whoever launches it from the side stream does so on the main stream and lets the side stream wait
   // In line (no concurrency) when switched off, while kernels are timed one by one, or while the stream is recorded.
-  if (!g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on || g_deterministic) return;
+  // (Deterministic mode keeps the side stream: which stream a kernel runs on changes no sum's order; two filter gradients of
+  // one filter stay ordered by the joins, and the slices of a cut reduction are added up in slice order by a pass of their own.)
+  if (!g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on) return;
   hipEvent_t ev = side_event();
   LH_HIP(hipEventRecord(ev, g_stream));              // (flushes recorded commands first)
   LH_HIP(hipStreamWaitEvent(g_side_stream, ev, 0));
