@@ -423,13 +423,18 @@ constexpr int N_PLANS = 13;
 // LH_FORCE_M32 in the environment: products of at most 32 rows always take the 32-row tile (for tests of that tile; the
 // measured choice may well be another one).
 static inline bool force_m32() { return getenv("LH_FORCE_M32") != nullptr; }
+// LH_FORCE_PLAN=n in the environment: forward / input-gradient products take launch plan n where it is valid (for tests that
+// compare the plans' results with each other).
+static inline int force_plan() { const char* e = getenv("LH_FORCE_PLAN"); return e ? atoi(e) : -1; }
 template <class AL, class BL, class EP>
 static bool plan_valid(int plan, const EP& ep, int M, int K, bool can_zero) {
   if (plan == 0) return true;
   if (plan == 10) return M <= 32;
   if ((plan == 1 || plan == 4 || plan == 6) && M <= 64) return false;
-  if (plan >= 4 && plan <= 9) return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= 16;
-  if (plan >= 11) return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= 64;
+  if ((plan >= 4 && plan <= 9) || plan >= 11) {
+    if (g_deterministic) return false;        // partial sums meet in atomic adds, in whatever order the blocks arrive
+    return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= (plan >= 11 ? 64 : 16);
+  }
   return true;
 }
 static bool g_launch_partial = false;     // the last launch_plan combined partial sums with atomic adds (stream-K): its epilogue saw incomplete sums
@@ -485,8 +490,12 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
   static std::map<PlanKey, int> chosen;
   const bool can_zero = zero_out != nullptr || prezeroed;
   if (M <= 32 && force_m32()) return launch_plan(10, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
-  if (!g_tune_lookup || 2.0 * M * N * (double)K < g_tune_min_flop) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
-  const PlanKey key = {{M, N, K, ep.eH, ep.eW, ep.W, ep.PIX}};
+  const int forced = force_plan();
+  if (forced >= 0 && forced < N_PLANS && plan_valid<AL, BL, EP>(forced, ep, M, K, can_zero)) return launch_plan(forced, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  // Deterministic mode keeps the measured choice among the plans whose tiles are finished by one block each: they add the same
+  // terms in the same order whatever the tile shape, so which of them runs changes no bit (tests/test_parity_conv.py compares them).
+  if (!g_tune_enabled || 2.0 * M * N * (double)K < g_tune_min_flop) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  const PlanKey key = {{M, N, K, ep.eH | (g_deterministic ? 1 << 16 : 0), ep.eW, ep.W, ep.PIX}};
   auto it = chosen.find(key);
   if (it != chosen.end()) {
     g_plans_remembered++;
@@ -494,7 +503,7 @@ static bool launch_tiles(const AL& al, const BL& bl, const EP& ep, int M, int N,
     return launch_plan(plan, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   }
   // tuned only on a call that may be repeated: an overwriting epilogue onto an output this launch alone writes
-  if (!g_tune_measure || ep.beta != 0.f || prezeroed) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
+  if (g_capturing || ep.beta != 0.f || prezeroed) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   LaunchTimer timer;
   if (!timer.ok) return launch_plan(0, al, bl, ep, M, N, K, zero_out, zero_n, prezeroed);
   int best = 0; float best_ms = 3.0e38f, base_ms = 0.f;

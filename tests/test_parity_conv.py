@@ -231,3 +231,36 @@ def test_conv_deterministic_mode(on_hip, dims):
     finally:
         on_hip.setDeterministic(False)
     assert dev.lib.lh_get_deterministic() == 0
+
+
+@pytest.mark.parametrize("dims", [(8, 64, 28, 28, 128, 3, 3, 1, 1, 1, 1), (4, 256, 14, 14, 256, 1, 1, 1, 1, 0, 0), (6, 96, 15, 15, 160, 3, 3, 1, 1, 1, 1),
+                                  (16, 32, 28, 28, 32, 3, 3, 1, 1, 1, 1), (8, 128, 28, 28, 256, 1, 1, 2, 2, 0, 0)], ids=lambda d: "x".join(map(str, d)))
+def test_plain_tile_plans_give_the_same_bits(on_hip, dims, monkeypatch):
+    """The launch plans whose tiles are finished by one block each (128x128, 64x128, 64x64, 32x128) add the same terms in the
+    same order: forward output and input gradient are bit-identical whichever of them runs.  Deterministic mode relies on
+    that when it keeps the measured choice among them."""
+    dev = Dev(on_hip)
+    lib = on_hip.lib
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    rng = np.random.RandomState(91)
+    xd = dev.up(rng.randn(N, Cc, H, W).astype(np.float32))
+    wd = dev.up((rng.randn(K, Cc, R, S) / np.sqrt(Cc * R * S)).astype(np.float32))
+    dyd = dev.up(rng.randn(N, K, P, Q).astype(np.float32))
+    ny, nx = N * K * P * Q, N * Cc * H * W
+    lib.lh_set_deterministic(1)
+    try:
+        outs = {}
+        for plan in (3, 2, 1, 10):
+            monkeypatch.setenv("LH_FORCE_PLAN", str(plan))
+            y = dev.up(np.full(ny, 7.0, np.float32)); lib.lh_conv2d_fwd(xd.ptr, wd.ptr, 0, y.ptr, *dims)
+            dx = dev.up(np.full(nx, 7.0, np.float32)); lib.lh_conv2d_bwd_data(dyd.ptr, wd.ptr, dx.ptr, 0.0, *dims)
+            dev.check()
+            outs[plan] = (dev.down(y, (ny,)).copy(), dev.down(dx, (nx,)).copy())
+        for plan in (2, 1, 10):      # (a plan that does not fit the shape falls back to the rule's tile: equal all the same)
+            np.testing.assert_array_equal(outs[plan][0], outs[3][0], err_msg="forward, plan %d against plan 3" % plan)
+            np.testing.assert_array_equal(outs[plan][1], outs[3][1], err_msg="input gradient, plan %d against plan 3" % plan)
+        assert np.abs(outs[3][0]).max() > 0.1 and np.abs(outs[3][1]).max() > 0.1
+    finally:
+        monkeypatch.delenv("LH_FORCE_PLAN", raising=False)
+        lib.lh_set_deterministic(0)
