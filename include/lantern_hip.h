@@ -256,7 +256,8 @@ void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x,
  * whose result overwrites its output, the forward and input-gradient products (tile shape, stream-K workers; a few timed
  * repetitions of the launch itself).  Products below 1e7 flop (LH_TUNE_MIN_FLOP) keep the built-in rule.  Environment:
  * LH_NO_TUNE=1 keeps the built-in rules everywhere, LH_TUNE_VERBOSE=1 prints each choice to stderr, LH_FORCE_M32=1 (a test
- * switch) sends every product of at most 32 rows to the 32-row tile whatever was measured.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
+ * switch) sends every product of at most 32 rows to the 32-row tile whatever was measured, LH_FORCE_PLAN=n (a test switch) every forward /
+ * input-gradient product to launch plan n where the shape allows it.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
  * remembered and are used again after lh_set_tuning(1)). */
 void lh_set_tuning(int on);
 /* How many launch plans have been measured so far, and how many launches have used a remembered plan (either pointer may be
@@ -266,9 +267,11 @@ void lh_tune_counters(int64_t* measured, int64_t* remembered);
  * default, reductions that are cut across blocks (filter gradients, long matrix products with few tiles, stream-K tiles,
  * convolution bias gradients, sums over a long middle axis) combine their pieces with fp32 atomic adds, so two runs on the
  * same inputs differ in the last bits.  With lh_set_deterministic(1) (or LH_DETERMINISTIC=1 in the environment) every such
- * reduction writes its pieces to arena scratch and a second kernel adds them in a fixed order; stream-K and all measured
- * launch plans are off (the built-in rules decide tile shapes and slice counts, so nothing depends on a timing), and the side
- * stream runs in line.  Two runs of the same calls on the same inputs then give the same bits.  Outside the guarantee:
+ * reduction writes its pieces to scratch memory and a second kernel adds them in a fixed order; stream-K is off and every
+ * choice that changes the order of a sum follows a built-in rule, not a timing (slice counts and tiles of the filter gradients
+ * and of lh_sgemm, the tile of a forward launch that leaves batch-norm statistics).  The measured choice among the forward /
+ * input-gradient plans whose tiles are finished by one block each stays: they give the same bits whatever the tile shape.
+ * The side stream stays too.  Two runs of the same calls on the same inputs then give the same bits.  Outside the guarantee:
  * lh_maxpool_bwd (the scatter form: three or more overlapping windows add in any order; lh_maxpool_bwd_dense is exact)
  * and lh_ctc_loss (fp64 sums rounded to fp32 once). */
 void lh_set_deterministic(int on);
