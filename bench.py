@@ -394,7 +394,7 @@ def main():
     fs = g.get("fusion_stats")
     if fs:
         out["config"]["library_fusion_totals"] = {"forward_chains": fs[0], "backward_chains": fs[1], "optimizer_calls_gathered": fs[2], "zero_fills_avoided": fs[3],
-                                                  "zero_fills_done": fs[4], "results_produced_on_demand": fs[5], "chains_ended_without_relu": fs[6]}
+                                                  "zero_fills_done": fs[4], "results_produced_on_demand": fs[5], "chains_ended_without_relu": fs[6], "filter_copies_reused": fs[7]}
     if g["resident_sec"] is not None:
         out["resident_input"] = {"value": round(g["per_step"] * args.steps / g["resident_sec"], 2), "ms_per_step": round(1000.0 * g["resident_sec"] / args.steps, 3),
                                  "note": "the same steps with the batch resident on the device: no upload, no loss read-back"}

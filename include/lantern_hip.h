@@ -177,11 +177,16 @@ void lh_prof_collect(double* h_ms, int64_t* h_calls, int ncat);
  *     would add into it with beta = 1, writes it without the clearing pass and without reading it; lh_rewind forgets it.
  *   - what a fused chain does not store because programs do not read it (the batch norm's own output under a residual
  *     join; the in-place masking of the gradient buffer by relu_grad) is produced when a call does read it.
+ *   - the copies of a filter in the layouts the convolution kernels read (tap-major for the forward pass, transposed per
+ *     stride class for the input gradient) are kept, in device memory of their own outside the arena (at most 1 GiB together),
+ *     while nothing writes the filter: any call of this header that writes into the filter's range ends them, and so does a
+ *     rewind or pop that releases the filter; behind the gathered optimizer launch they are made again on the side stream.
  * Results are those of the calls as issued (the fused kernels give the bits of the sequences they replace wherever two
  * launches of the sequence itself agree bit for bit).  Every entry point of this header takes part; a pointer handed to
  * anything else (another library, a kernel of the caller's) must be preceded by lh_sync() AND lh_flush_deferred().
- * lh_fusion_stats: h_out[0..6] = forward chains fused, backward chains fused, optimizer calls gathered, zero fills avoided,
- * zero fills done, results produced on demand, conv -> bn or bn -> + chains that ended without a relu. */
+ * lh_fusion_stats: h_out[0..7] = forward chains fused, backward chains fused, optimizer calls gathered, zero fills avoided,
+ * zero fills done, results produced on demand, conv -> bn or bn -> + chains that ended without a relu, filter copies found
+ * kept by a convolution call. */
 void lh_set_fusion(int on);
 int lh_get_fusion(void);
 void lh_flush_deferred(void);               /* everything put off is enqueued now (nothing waits) */

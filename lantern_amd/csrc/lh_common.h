@@ -13,6 +13,11 @@ extern hipStream_t g_stream_raw;  // the library's stream
 // Where entry points enqueue now: g_stream_raw, or the side stream between lh_side_begin and lh_side_end.
 extern hipStream_t g_stream_cur;
 void side_join();                 // the main stream waits for what the side stream was given (no-op when it is idle)
+void* persistent_alloc(size_t bytes);      // device memory of its own, outside the arena (waits for the device); nullptr when there is none
+void persistent_free(void* p);
+bool side_work_begin();                    // library-internal fork: the side stream waits for the main stream and becomes current; false: not now
+void side_work_end();
+void build_filter_layout(int kind, const int* prm, const float* w, float* dst);      // lh_conv.hip: the copy kernel of a layout, on the current stream
 void* side_scratch(size_t bytes); // a block for the kernels of the side stream (one user at a time, in that stream's order); nullptr after a reported failure
 // Scratch memory for a launch: the top of the arena on the main stream (stream order puts the next user of the same memory
 // behind this launch), the side stream's own block on the side stream.  One block per entry point at a time.
@@ -31,6 +36,8 @@ void multi_tensor_release();
 // blocks nobody has touched yet, and results of fused launches that the program could read but no kernel has written.
 // An entry point that states what it reads and writes (lazy::Scope + rd / wr / acc / rw below) is served exactly; any
 // other entry point reaches ordered_stream() at depth 0, which first brings everything deferred up to date.
+constexpr int LAYOUT_PRM = 10;                       // parameters that name a filter layout (see lazy::layout_lookup)
+enum { LAYOUT_KRSC = 0, LAYOUT_CTK = 1, LAYOUT_CKRS = 2 };
 namespace lazy {
 extern bool g_busy;               // something is parked, pending or unwritten
 extern int g_depth;               // > 0 inside an entry point that declares its operands, and while deferred work is launched
@@ -169,6 +176,10 @@ bool take_relu_grad_bias(const float* dy, float* db, int N, int K, int PQ);
 bool take_bn_bwd(const float* x, const float* dy, const float* gamma, const float* save_mean, const float* save_invstd,
                  float* dx, float beta_dx, float* dgamma, float* dbeta, int N, int C, int HW);
 bool gather_update(int mode, float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n);
+// filter layouts (kept copies of a filter in the order a convolution kernel reads it; lh_defer.hip).  Returns the copy, or
+// nullptr when the caller has to use scratch memory as before; `build`: the copy has to be written first, by the caller, on
+// the current stream (build_filter_layout).
+float* layout_lookup(const float* w, size_t wbytes, int kind, const int* prm, size_t bytes, bool& build);
 void forget_forward_records();                     // parameters are about to change: what the backward pass would recompute from them is no longer valid
 void on_rewind(char* new_top);
 void reset();                                      // forget everything deferred without launching anything (lh_setup, lh_cleanup)

@@ -374,6 +374,39 @@ static void bias_grad_launch(const float* y, float* dy, float* db, int N, int K,
   else hipLaunchKernelGGL((k_conv_bwd_bias<false, false>), grid, dim3(TPB), 0, g_stream, y, dy, db, N, K, PQ, n_per);
 }
 
+}  // namespace
+namespace lh {
+// The copy kernel of a filter layout, on the current stream (prm as the convolution entry points fill it in).
+void build_filter_layout(int kind, const int* p, const float* w, float* dst) {
+  if (kind == LAYOUT_KRSC) {                 // {K, C, RS}
+    const int64_t n = (int64_t)p[0] * p[1] * p[2];
+    hipLaunchKernelGGL(k_filter_to_krsc, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, dst, p[1], p[2], n);
+  } else if (kind == LAYOUT_CTK) {           // {K, C, R, S, r0, s0, sH, sW, Rc, Sc}
+    const int64_t n = (int64_t)p[8] * p[9] * p[0] * p[1];
+    hipLaunchKernelGGL(k_filter_to_ctk, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, dst, p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], p[8], p[9], n);
+  } else {                                   // LAYOUT_CKRS {K, C, RS}
+    const int64_t n = (int64_t)p[0] * p[1] * p[2];
+    hipLaunchKernelGGL(k_filter_transpose, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, dst, p[0], p[1], p[2], n);
+  }
+}
+}  // namespace lh
+namespace {
+// The filter in the layout a launch reads: the library's kept copy (written now if it is stale), or, where none is kept,
+// scratch from the arena top that the caller pops behind the launch (stream order keeps that safe).
+struct FilterCopy { float* p = nullptr; size_t scratch = 0; };
+static bool filter_copy(FilterCopy& fc, const float* w, size_t wbytes, int kind, const int* prm, size_t bytes) {
+  bool build = false;
+  fc.scratch = 0;
+  fc.p = lazy::layout_lookup(w, wbytes, kind, prm, bytes, build);
+  if (fc.p == nullptr) {
+    fc.p = (float*)lh_malloc_uninit(bytes);
+    if (fc.p == nullptr) return false;
+    fc.scratch = bytes; build = true;
+  }
+  if (build) build_filter_layout(kind, prm, w, fc.p);
+  return true;
+}
+
 #ifndef LH_CONV_BK
 #define LH_CONV_BK 16
 #endif
@@ -584,12 +617,10 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
     const float* wk = w;
     size_t scratch = 0;
     if (RS > 1) {
-      scratch = wbytes;
-      float* wt = (float*)lh_malloc_uninit(scratch);   // released below: stream order keeps it safe
-      if (wt == nullptr) return;
-      int64_t n = (int64_t)K * CRS;
-      hipLaunchKernelGGL(k_filter_to_krsc, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, C, RS, n);
-      wk = wt;
+      const int prm[LAYOUT_PRM] = {K, C, RS};
+      FilterCopy fc;
+      if (!filter_copy(fc, w, wbytes, LAYOUT_KRSC, prm, wbytes)) return;
+      wk = fc.p; scratch = fc.scratch;
     }
     LoadPlainK<true> al; al.base = wk; al.nbytes = wbytes; al.ld = CRS;
     LoadConvFwdTapB bl; bl.base = x; bl.nbytes = xbytes; bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.HW = H * W;
@@ -793,20 +824,17 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
       if (fits && ng >= 2) {
         for (int i = 1; i < ng; i++) for (int j = i; j > 0 && cls[j].Kred > cls[j - 1].Kred; j--) { Cls t = cls[j]; cls[j] = cls[j - 1]; cls[j - 1] = t; }
         if (beta == 0.f && any_empty) lh_fill(dx, 0.f, (int64_t)N * C * HW);       // pixels no class reaches
-        size_t bytes = 0;
-        for (int i = 0; i < ng; i++) bytes += (((size_t)cls[i].Kred * C * sizeof(float)) + 255) & ~(size_t)255;
-        char* scratch = (char*)lh_malloc_uninit(bytes);
-        if (scratch == nullptr) return;
+        FilterCopy fcs[IGEMM_MAX_GROUPS];
+        auto release = [&]() { for (int i = ng - 1; i >= 0; i--) if (fcs[i].scratch) { lh_free_top(fcs[i].scratch); fcs[i].scratch = 0; } };
         LoadPlainK<true> al[IGEMM_MAX_GROUPS]; LoadConvBwdDataTapB bl[IGEMM_MAX_GROUPS]; EpiConvOut ep[IGEMM_MAX_GROUPS];
         int Ms[IGEMM_MAX_GROUPS], Ns[IGEMM_MAX_GROUPS], Ks[IGEMM_MAX_GROUPS];
-        size_t off = 0; int64_t ntot = 0; int kmax = 0;
+        int64_t ntot = 0; int kmax = 0;
         for (int i = 0; i < ng; i++) {
           const Cls& c = cls[i];
-          float* wt = (float*)(scratch + off);
           const size_t wbytes = (size_t)c.Kred * C * sizeof(float);
-          off += (wbytes + 255) & ~(size_t)255;
-          const int64_t n = (int64_t)c.Kred * C;
-          hipLaunchKernelGGL(k_filter_to_ctk, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, R, S, c.r0, c.s0, sH, sW, c.Rc, c.Sc, n);
+          const int prm[LAYOUT_PRM] = {K, C, R, S, c.r0, c.s0, sH, sW, c.Rc, c.Sc};
+          if (!filter_copy(fcs[i], w, (size_t)K * C * RS * sizeof(float), LAYOUT_CTK, prm, wbytes)) { release(); return; }
+          float* wt = fcs[i].p;
           al[i].base = wt; al[i].nbytes = (uint32_t)wbytes; al[i].ld = c.Kred;
           LoadConvBwdDataTapB& b = bl[i];
           b.base = dy; b.nbytes = dybytes; b.K = K; b.P = d.P; b.Q = d.Q; b.PQ = PQ;
@@ -841,7 +869,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
               if (tcand == 1 && C <= 64) continue;
               if (tcand == 4 && C > 32) continue;
               const float ms = timer.ms([&]() { return run(tcand); });
-              if (ms < 0.f || failed()) { lh_free_top(bytes); return; }
+              if (ms < 0.f || failed()) { release(); return; }
               if (ms < best_ms * 0.98f) { best_ms = ms; best = tcand; }
             }
             chosen[key] = best; tile = best; g_plans_measured++;
@@ -849,7 +877,7 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
           }
         }
         ok = run(tile);
-        lh_free_top(bytes);
+        release();
         if (!ok) return;
         LH_CHECK_LAUNCH();
         return;
@@ -880,13 +908,12 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
         ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred, zo, zn, pz);
       } else {
         size_t bytes = (size_t)Kred * C * sizeof(float);
-        float* wt = (float*)lh_malloc_uninit(bytes);     // released below: stream order keeps it safe
-        if (wt == nullptr) return;
-        int64_t n = (int64_t)Kred * C;
-        hipLaunchKernelGGL(k_filter_to_ctk, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, R, S, r0, s0, sH, sW, Rc, Sc, n);
-        LoadPlainK<true> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = Kred;
+        const int prm[LAYOUT_PRM] = {K, C, R, S, r0, s0, sH, sW, Rc, Sc};
+        FilterCopy fc;
+        if (!filter_copy(fc, w, (size_t)K * C * RS * sizeof(float), LAYOUT_CTK, prm, bytes)) return;
+        LoadPlainK<true> al; al.base = fc.p; al.nbytes = (uint32_t)bytes; al.ld = Kred;
         ok = launch_tiles(al, bl, ep, C, N * Hc * Wc, Kred, zo, zn, pz);
-        lh_free_top(bytes);
+        if (fc.scratch) lh_free_top(fc.scratch);
       }
     }
   } else {
@@ -898,13 +925,13 @@ void lh_conv2d_bwd_data(const float* dy, const float* w, float* dx, float beta,
       ok = launch_tiles(al, bl, ep, C, N * HW, KRS);
     } else {
       size_t bytes = (size_t)KRS * C * sizeof(float);
-      float* wt = (float*)lh_malloc_uninit(bytes);
-      if (wt == nullptr) return;
-      int64_t n = (int64_t)KRS * C;
-      hipLaunchKernelGGL(k_filter_transpose, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, wt, K, C, RS, n);
+      const int prm[LAYOUT_PRM] = {K, C, RS};
+      FilterCopy fc;
+      if (!filter_copy(fc, w, bytes, LAYOUT_CKRS, prm, bytes)) return;
+      float* wt = fc.p;
       if (KRS % 4 == 0) { LoadPlainK<true> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
       else { LoadPlainK<false> al; al.base = wt; al.nbytes = (uint32_t)bytes; al.ld = KRS; ok = launch_tiles(al, bl, ep, C, N * HW, KRS); }
-      lh_free_top(bytes);
+      if (fc.scratch) lh_free_top(fc.scratch);
     }
   }
   if (!ok) return;

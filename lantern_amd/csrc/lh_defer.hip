@@ -17,11 +17,15 @@
 //  3. Unwritten results.  A fused chain leaves out stores nobody normally reads: the batch norm's own output under a
 //     residual join, and the in-place masking of the gradient buffer by relu_grad.  Each is noted with the recipe that
 //     produces it; a later read of the range (or a write to what the recipe reads) runs the recipe first.
+//  4. Filter layouts.  The copies of a filter in the layouts the convolution kernels read are kept while nothing writes the
+//     filter, and made again beside the next step's first kernels after the optimizer launch that does (see below).
 //
 // Entry points that state their operands (lazy::Scope, rd / wr / acc / rw) are served exactly; every other entry point
 // reaches lh::ordered_stream() at depth 0, which brings all deferred work up to date before it enqueues anything.
-// Nothing here allocates device memory or waits for the device.
+// Apart from the memory of the filter copies (allocated when a filter is first seen, released with it), nothing here
+// allocates device memory or waits for the device.
 #include "lh_common.h"
+#include <string.h>
 #include <algorithm>
 #include <vector>
 
@@ -34,7 +38,7 @@ bool g_busy = false;
 int g_depth = 0;
 bool g_replay = false;
 static int64_t g_stat[8];        // fused chains, gathered updates, zero fills avoided / done, recipes run (lh_fusion_stats)
-enum { ST_FUSED_FWD, ST_FUSED_BWD, ST_GATHERED, ST_ZERO_SKIPPED, ST_ZERO_DONE, ST_RECIPES, ST_UNFUSED };
+enum { ST_FUSED_FWD, ST_FUSED_BWD, ST_GATHERED, ST_ZERO_SKIPPED, ST_ZERO_DONE, ST_RECIPES, ST_UNFUSED, ST_LAYOUTS };
 
 static inline size_t round256(size_t b) { b = (b + 255) & ~(size_t)255; return b ? b : 256; }
 static inline bool overlap(const char* a, size_t an, const char* b, size_t bn) { return a < b + bn && b < a + an; }
@@ -69,7 +73,8 @@ struct Parked {
 };
 static Parked g_p;
 
-static inline void refresh_busy() { g_busy = g_p.kind != P_NONE || !g_zero.empty() || !g_unwritten.empty(); }
+static int g_layouts_valid_count();
+static inline void refresh_busy() { g_busy = g_p.kind != P_NONE || !g_zero.empty() || !g_unwritten.empty() || g_layouts_valid_count() > 0; }
 static inline bool can_park() { return g_enabled && !g_replay && g_stream_cur == g_stream_raw && !g_rec_on; }
 
 // Launches made in a Replay's lifetime run as called (no parking, no declarations) and on the main stream; a side stream
@@ -82,6 +87,78 @@ struct Replay {
     if (saved_stream != g_stream_raw) side_wait_for_main();
   }
 };
+
+// ---- filter layouts ---------------------------------------------------------------------------------------------------
+// The convolution kernels read their filter in a layout of their own (tap-major for the forward pass, one transposed copy per
+// residue class for the input gradient): a copy kernel per layer and pass, 5-7 us each in the chain of a training step.  A copy
+// is kept in memory of its own for as long as nothing writes the filter: every stated write into the filter's range, every
+// call that states nothing, a rewind or pop that releases the filter, ends it.  After the gathered optimizer launch, which is
+// such a write, the copies that were in use are made again on the side stream, beside whatever the program does next; the
+// convolution that needs one waits for the side stream then (lh::side_join) instead of making it itself.
+struct Layout { const char* w; size_t wbytes; int kind; int prm[LAYOUT_PRM]; float* copy; size_t bytes; bool valid, used; };
+static std::vector<Layout> g_layouts;
+static int g_layouts_valid = 0;
+static size_t g_layout_bytes = 0;
+static bool g_layouts_on_side = false;                   // copies made on the side stream that the main stream has not waited for yet
+static const size_t LAYOUT_CAP = (size_t)1 << 30;        // all copies together; filters beyond that are copied per call as before
+
+static int g_layouts_valid_count() { return g_layouts_valid; }
+static inline void layout_set(Layout& l, bool v) { if (l.valid != v) { l.valid = v; g_layouts_valid += v ? 1 : -1; } }
+static void layouts_written(const char* lo, size_t nb) {
+  if (g_layouts_valid == 0) return;
+  for (auto& l : g_layouts) if (l.valid && overlap(lo, nb, l.w, l.wbytes)) layout_set(l, false);
+}
+static void layouts_all_stale() { if (g_layouts_valid) for (auto& l : g_layouts) layout_set(l, false); }
+static void layouts_released(const char* from) {
+  for (size_t i = 0; i < g_layouts.size();) {
+    if (g_layouts[i].w + g_layouts[i].wbytes > from) {
+      layout_set(g_layouts[i], false);
+      g_layout_bytes -= g_layouts[i].bytes;
+      persistent_free(g_layouts[i].copy);       // (waits for the device: only when a filter itself is released)
+      g_layouts.erase(g_layouts.begin() + i);
+    } else i++;
+  }
+}
+static void layouts_drop() { layouts_released(nullptr); }
+
+float* layout_lookup(const float* w, size_t wbytes, int kind, const int* prm, size_t bytes, bool& build) {
+  build = false;
+  if (!g_enabled || g_rec_on || g_capturing || g_prof_mask != 0 || g_stream_cur != g_stream_raw || w == nullptr) return nullptr;
+  for (auto& l : g_layouts) {
+    if (l.w != (const char*)w || l.kind != kind || l.bytes != bytes || memcmp(l.prm, prm, sizeof l.prm) != 0) continue;
+    l.used = true;
+    if (l.valid) {
+      if (g_layouts_on_side) { side_join(); g_layouts_on_side = false; }     // once per step: later lookups must not wait for the filter gradients that run there by then
+      g_stat[ST_LAYOUTS]++;
+      return l.copy;
+    }
+    // stale: the caller makes it again, in stream order in front of its use, and it holds until the filter is written again
+    layout_set(l, true); g_busy = true; build = true;
+    return l.copy;
+  }
+  if (g_layout_bytes + bytes > LAYOUT_CAP) return nullptr;
+  float* copy = (float*)persistent_alloc(bytes);
+  if (copy == nullptr) return nullptr;
+  Layout l{}; l.w = (const char*)w; l.wbytes = wbytes; l.kind = kind; memcpy(l.prm, prm, sizeof l.prm); l.copy = copy; l.bytes = bytes; l.valid = false; l.used = true;
+  g_layouts.push_back(l);
+  g_layout_bytes += bytes;
+  layout_set(g_layouts.back(), true); g_busy = true; build = true;
+  return copy;
+}
+// behind the optimizer launch: the copies the last step used, made again beside what comes next
+static void layouts_refresh() {
+  bool any = false;
+  for (auto& l : g_layouts) any = any || (l.used && !l.valid);
+  if (!any || !side_work_begin()) return;
+  for (auto& l : g_layouts) {
+    if (!l.used || l.valid) continue;
+    build_filter_layout(l.kind, l.prm, (const float*)l.w, l.copy);
+    layout_set(l, true);
+    l.used = false;
+  }
+  side_work_end();
+  g_layouts_on_side = true;
+}
 
 // ---- zero blocks ---------------------------------------------------------------------------------------------------
 void note_zero_block(void* p, size_t bytes) {
@@ -147,6 +224,7 @@ void rd(const void* p, size_t bytes) {
 void wr(const void* p, size_t bytes) {
   if (!g_busy || g_replay || p == nullptr || bytes == 0) return;
   const char* lo = (const char*)p;
+  layouts_written(lo, bytes);
   size_t a, b; zero_span(lo, lo + bytes, a, b);
   // blocks the write covers need no clearing; a block it only touches is cleared first
   while (a < b) {
@@ -159,6 +237,7 @@ void wr(const void* p, size_t bytes) {
 void rw(const void* p, size_t bytes) {
   if (!g_busy || g_replay || p == nullptr || bytes == 0) return;
   const char* lo = (const char*)p;
+  layouts_written(lo, bytes);
   size_t a, b; zero_span(lo, lo + bytes, a, b); clear_blocks(a, b);
   if (!g_unwritten.empty()) settle_unwritten(lo, bytes, 2);
   refresh_busy();
@@ -166,6 +245,7 @@ void rw(const void* p, size_t bytes) {
 bool acc(const void* p, size_t bytes) {
   if (!g_busy || g_replay || p == nullptr || bytes == 0) return false;
   const char* lo = (const char*)p;
+  layouts_written(lo, bytes);
   size_t a, b; zero_span(lo, lo + bytes, a, b);
   if (b == a + 1 && g_zero[a].p == lo && g_zero[a].bytes == round256(bytes)) {       // the whole block, still untouched: overwrite it
     g_zero.erase(g_zero.begin() + a);
@@ -235,6 +315,7 @@ void flush_parked() {
         break;
     }
   }
+  if (p.kind == P_UPDATE) layouts_refresh();
   if (p.kind == P_RELU_ADD_GRAD) note_mask(p.gd, p.gd, p.gy, p.gn);      // relu_grad(inPlace) leaves its gradient buffer masked; nobody has done that yet
   refresh_busy();
 }
@@ -249,7 +330,7 @@ void flush_all() {
   clear_blocks(0, g_zero.size());
   refresh_busy();
 }
-void flush_undeclared() { Scope s_; flush_all(); }
+void flush_undeclared() { Scope s_; flush_all(); layouts_all_stale(); refresh_busy(); }   // whoever states nothing may have written anything
 
 static bool conv_shape_ok(int N, int C, int H, int W, int K, int R, int S, int sH, int sW, int pH, int pW, int& P, int& Q) {
   if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || R <= 0 || S <= 0 || sH <= 0 || sW <= 0 || pH < 0 || pW < 0) return false;
@@ -426,9 +507,10 @@ bool gather_update(int mode, float* x, float* d, float* v, float lr, float mu, f
   return true;
 }
 void forget_forward_records() { g_records.clear(); }
-void reset() { g_p = Parked(); g_zero.clear(); g_unwritten.clear(); g_records.clear(); g_busy = false; g_replay = false; }
+void reset() { g_p = Parked(); g_zero.clear(); g_unwritten.clear(); g_records.clear(); layouts_drop(); g_busy = false; g_replay = false; }
 
 void arena_released(char* from) {
+  if (!g_layouts.empty()) layouts_released(from);
   while (!g_zero.empty() && g_zero.back().p >= from) g_zero.pop_back();
   for (size_t i = 0; i < g_unwritten.size();) {
     if (g_unwritten[i].dst >= from) g_unwritten.erase(g_unwritten.begin() + i); else i++;
@@ -467,11 +549,13 @@ extern "C" {
 void lh_set_fusion(int on) {
   lazy::Scope s_;
   lazy::flush_all();
+  lazy::layouts_all_stale();
+  lazy::refresh_busy();
   lazy::g_enabled = on != 0;
 }
 int lh_get_fusion(void) { return lazy::g_enabled ? 1 : 0; }
 void lh_flush_deferred(void) { lazy::Scope s_; lazy::flush_all(); }
 void lh_fusion_stats(int64_t* h_out, int n) {
-  for (int i = 0; i < n; i++) h_out[i] = i < 7 ? lazy::g_stat[i] : 0;
+  for (int i = 0; i < n; i++) h_out[i] = i < 8 ? lazy::g_stat[i] : 0;
 }
 }

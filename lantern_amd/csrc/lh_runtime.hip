@@ -44,6 +44,19 @@ void* side_scratch(size_t bytes) {
   g_side_scratch = (char*)p; g_side_scratch_bytes = want;
   return p;
 }
+void* persistent_alloc(size_t bytes) {
+  void* p = nullptr;
+  if (hipMalloc(&p, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+  return p;
+}
+void persistent_free(void* p) { if (p) (void)hipFree(p); }
+bool side_work_begin() {
+  if (!g_side_stream || !g_side_enabled || g_prof_mask != 0 || g_capturing || g_rec_on || g_stream_cur != g_stream_raw) return false;
+  side_wait_for_main();
+  g_stream_cur = g_side_stream; g_side_dirty = true;
+  return true;
+}
+void side_work_end() { g_stream_cur = g_stream_raw; }
 void* scratch_take(size_t bytes, bool& side) { side = g_stream_cur != g_stream_raw; return side ? side_scratch(bytes) : lh_malloc_uninit(bytes); }
 void scratch_give(size_t bytes, bool side) { if (!side) lh_free_top(bytes); }
 static void side_scratch_release() { if (g_side_scratch) (void)hipFree(g_side_scratch); g_side_scratch = nullptr; g_side_scratch_bytes = 0; }

@@ -29,6 +29,22 @@ void prof_end(int) {}
 bool fail(const char* file, int line, const char* fmt, ...) { fprintf(stderr, "%s:%d: %s\n", file, line, fmt); exit(2); }
 bool failed() { return false; }
 void side_wait_for_main() {}
+void side_join() {}
+bool g_capturing = false;
+static long long g_layout_builds = 0;
+void* persistent_alloc(size_t bytes) { return malloc(bytes); }
+void persistent_free(void* p) { free(p); }
+bool side_work_begin() { return true; }
+void side_work_end() {}
+// the simulated filter layout is a plain copy: a stale one still shows, because the values differ
+void build_filter_layout(int, const int*, const float* w, float* dst) { (void)ordered_stream(); memcpy(dst, w, 12 * sizeof(float)); g_layout_builds++; }
+static const float* sim_filter(const float* w) {
+  bool build = false; const int prm[LAYOUT_PRM] = {4, 3, 1};
+  float* c = lazy::layout_lookup(w, 12 * sizeof(float), LAYOUT_KRSC, prm, 12 * sizeof(float), build);
+  if (c == nullptr) return w;
+  if (build) build_filter_layout(LAYOUT_KRSC, prm, w, c);
+  return c;
+}
 static long long g_kernels = 0;           // simulated launches (the two modes differ in how many they need)
 void zero_bytes_async(void* p, size_t bytes) { (void)ordered_stream(); memset(p, 0, bytes); g_kernels++; }
 void mask_relu(float* dst, const float* src, const float* y, int64_t n) { (void)ordered_stream(); for (int64_t i = 0; i < n; i++) dst[i] = y[i] > 0.f ? src[i] : 0.f; g_kernels++; }
@@ -88,7 +104,7 @@ static void k_conv(const float* x, const float* w, const float* bias, float* y) 
 static void k_conv_bwd_data(const float* dy, const float* w, float* dx, float beta) { for (int i = 0; i < NE; i++) { float a = 0.f; for (int k = 0; k < 3; k++) a += dy[(i + NE - 7 * k) % NE] * w[(chan((i + NE - 7 * k) % NE) + k) % 12]; dx[i] = (beta != 0.f ? dx[i] : 0.f) + a; } g_kernels++; }
 static void k_conv_bwd_filter(const float* x, const float* dy, float* dw, float beta) { for (int j = 0; j < 12; j++) { float a = 0.f; for (int i = 0; i < NE; i++) for (int k = 0; k < 3; k++) if ((chan(i) + k) % 12 == j) a += dy[i] * x[(i + 7 * k) % NE]; dw[j] = (beta != 0.f ? dw[j] : 0.f) + a; } g_kernels++; }
 namespace lh {
-static void sim_conv_relu(const float* x, const float* w, const float* bias, float* y) { k_conv(x, w, bias, y); for (int i = 0; i < NE; i++) y[i] = y[i] < 0.f ? 0.f : y[i]; }
+static void sim_conv_relu(const float* x, const float* w, const float* bias, float* y) { k_conv(x, sim_filter(w), bias, y); for (int i = 0; i < NE; i++) y[i] = y[i] < 0.f ? 0.f : y[i]; }
 // bias gradient: channel sums of dy in element order; with y, dy is masked by y > 0 on the way (and written back)
 static void sim_bias_grad(const float* y, float* dy, float* db) { for (int i = 0; i < NE; i++) { if (y) dy[i] = y[i] > 0.f ? dy[i] : 0.f; db[chan(i)] += dy[i]; } g_kernels++; }
 }
@@ -126,7 +142,7 @@ void lh_conv2d_fwd(const float* x, const float* w, const float* bias, float* y, 
   LZ_SCOPE();
   if (lazy::park_conv_fwd(x, w, bias, y, N, C, H, W, K, R, S, sH, sW, pH, pW)) return;
   if (lazy::g_busy && !lazy::g_replay) { lazy::flush_parked(); lazy::rd(x, SZ(NE)); lazy::rd(w, SZ(12)); lazy::rd(bias, SZ(C_)); lazy::wr(y, SZ(NE)); }
-  (void)ordered_stream(); k_conv(x, w, bias, y);
+  (void)ordered_stream(); k_conv(x, sim_filter(w), bias, y);
 }
 void lh_bn_stats(const float* x, float* sm, float* si, float* rm, float* rv, int, int, int, float, float) {
   LZ_ENTER(); lazy::rd_f(x, NE); lazy::wr_f(sm, C_); lazy::wr_f(si, C_); lazy::rw_f(rm, C_); lazy::rw_f(rv, C_);
@@ -159,7 +175,7 @@ void lh_conv2d_fwd_bn_apply(const float* x, const float* w, const float* bias, f
     lazy::flush_parked(); lazy::rd_f(x, NE); lazy::rd_f(w, 12); lazy::rd_f(bias, C_); lazy::wr_f(y, NE); lazy::rd_f(g, C_); lazy::rd_f(b, C_); lazy::rd_f(sc, NE);
     lazy::wr_f(sm, C_); lazy::wr_f(si, C_); lazy::rw_f(rm, C_); lazy::rw_f(rv, C_); lazy::wr_f(out, NE);
   }
-  (void)ordered_stream(); k_conv(x, w, bias, y); k_stats(y, sm, si, rm, rv); k_apply(y, g, b, sm, si, sc, out, relu);
+  (void)ordered_stream(); k_conv(x, sim_filter(w), bias, y); k_stats(y, sm, si, rm, rv); k_apply(y, g, b, sm, si, sc, out, relu);
 }
 void lh_add_relu(const float* a, const float* b, float* out, int64_t n) {
   LZ_ENTER(); lazy::rd_f(a, n); lazy::rd_f(b, n); lazy::out_f(out, n, out == a || out == b);
@@ -243,7 +259,7 @@ static void t_add_grad(float* ad, float* bd, const float* outd, int64_t n) {    
   g_kernels++;
 }
 static void t_conv_bwd(const float* x, const float* dy, const float* w, float* dx, float* dw) {
-  { LZ_ENTER(); lazy::rd_f(dy, NE); lazy::rd_f(w, 12); float beta = lazy::beta_f(dx, NE, 1.f); (void)ordered_stream(); k_conv_bwd_data(dy, w, dx, beta); }
+  { LZ_ENTER(); lazy::rd_f(dy, NE); lazy::rd_f(w, 12); float beta = lazy::beta_f(dx, NE, 1.f); (void)ordered_stream(); k_conv_bwd_data(dy, sim_filter(w), dx, beta); }
   { LZ_ENTER(); lazy::rd_f(x, NE); lazy::rd_f(dy, NE); float beta = lazy::beta_f(dw, 12, 1.f); (void)ordered_stream(); k_conv_bwd_filter(x, dy, dw, beta); }
 }
 // a convolution with a bias: the filter gradient (bias sums included) goes first, as the backends issue it
@@ -253,7 +269,7 @@ static void t_conv_bwd_bias(const float* x, float* dy, const float* w, float* dx
     if (lazy::g_busy && !lazy::g_replay) lazy::flush_parked();
     lazy::rd_f(x, NE); lazy::rd_f(dy, NE); float beta = lazy::beta_f(dw, 12, 1.f); lazy::rw_f(db, C_);
     (void)ordered_stream(); k_conv_bwd_filter(x, dy, dw, beta); if (!done) sim_bias_grad(nullptr, dy, db); }
-  if (dx) { LZ_ENTER(); lazy::rd_f(dy, NE); lazy::rd_f(w, 12); float beta = lazy::beta_f(dx, NE, 1.f); (void)ordered_stream(); k_conv_bwd_data(dy, w, dx, beta); }
+  if (dx) { LZ_ENTER(); lazy::rd_f(dy, NE); lazy::rd_f(w, 12); float beta = lazy::beta_f(dx, NE, 1.f); (void)ordered_stream(); k_conv_bwd_data(dy, sim_filter(w), dx, beta); }
 }
 static void t_momentum(float* x, float* d, float* v, float lr, float mu, float clip, int nesterov, int64_t n) {
   LZ_SCOPE();
@@ -408,6 +424,8 @@ int main(int argc, char** argv) {
   }
   printf("defer_check: %d programs identical with and without deferred work; %lld chains fused; simulated launches %lld as issued, %lld with deferred work\n",
          programs, fused, k_off, k_on);
+  printf("filter copies: %lld made, %lld lookups served from a kept copy\n", g_layout_builds, (long long)lazy::g_stat[lazy::ST_LAYOUTS]);
+  lazy::reset();
   free(g_heap);
   return 0;
 }

@@ -375,3 +375,66 @@ def test_concat_of_more_tensors_than_one_launch_takes(prog):
         if s and dptrs[t]:
             np.testing.assert_array_equal(prog.down(dptrs[t], init[t].shape), betas[t] * init[t] + dout[:, off:off + s, :], err_msg="tensor %d" % t)
         off += s
+
+
+def test_kept_filter_copies_end_with_every_write_of_the_filter(prog):
+    """The convolution kernels read copies of the filter in layouts of their own; the library keeps a copy while nothing
+    writes the filter.  Every way of writing it (an upload, an operator in place, a fill, the gathered optimizer launch, a
+    rewind that hands its memory to another tensor) must end the copy: each time the convolution and its input gradient,
+    stride 1 and stride 2, are compared with what the library computes with nothing kept (lh_set_fusion(0))."""
+    lib = prog.lib
+    rng = np.random.RandomState(53)
+    n, c, h, k = 4, 32, 14, 48
+    x = prog.up(rng.randn(n, c, h, h).astype(np.float32))
+    w_host = (rng.randn(k, c, 3, 3) * 0.1).astype(np.float32)
+    mark0 = lib.lh_mark()
+    w = prog.up(w_host)
+    nw = w_host.size
+
+    def run(stride):
+        p = (h + 2 - 3) // stride + 1
+        args = (n, c, h, h, k, 3, 3, stride, stride, 1, 1)
+        y = prog.malloc(n * k * p * p); lib.lh_conv2d_fwd(x, w, 0, y, *args)
+        yh = prog.down(y, (n * k * p * p,))
+        dy = prog.up(np.cos(np.arange(n * k * p * p, dtype=np.float32)))
+        dx = prog.malloc(n * c * h * h); lib.lh_conv2d_bwd_data(dy, w, dx, 1.0, *args)
+        _lib.check()
+        return yh, prog.down(dx, (n * c * h * h,))
+
+    def check(what):
+        mark = lib.lh_mark()
+        got = [run(1), run(2)]
+        s0 = _stats(lib)[7]
+        again = [run(1), run(2)]                   # nothing written in between: served from the kept copies
+        assert _stats(lib)[7] - s0 >= 6, "forward (1 copy), stride-1 input gradient (1) and stride-2 input gradient (4 classes) were to find their copies: %s" % what
+        lib.lh_set_fusion(0)
+        want = [run(1), run(2)]
+        lib.lh_set_fusion(1)
+        for g, a, t in zip(got, again, want):
+            for u, v, z in zip(g, a, t):
+                np.testing.assert_array_equal(u, z, err_msg=what)
+                np.testing.assert_array_equal(v, z, err_msg=what + " (second time)")
+        lib.lh_rewind(mark)
+        return got[0][0]
+
+    y0 = check("first use")
+    w2 = (w_host * 1.5 + 0.01).astype(np.float32)
+    lib.lh_h2d(w, w2.ctypes.data, w2.nbytes)
+    y1 = check("after an upload")
+    assert np.abs(y1 - y0).max() > 1e-3
+    lib.lh_geam(w, F(0.5), w, F(0.0), w, nw)                     # in place
+    y2 = check("after an operator in place")
+    assert np.abs(y2 - y1).max() > 1e-3
+    lib.lh_fill(w + 4 * 100, F(0.25), 50)                        # part of it
+    y3 = check("after a fill over part of the filter")
+    assert np.abs(y3 - y2).max() > 1e-4
+    d = prog.up(rng.randn(nw).astype(np.float32)); v = prog.up(np.zeros(nw, np.float32))
+    lib.lh_momentum(w, d, v, 0.1, 0.9, 400.0, 0, nw)             # gathered, launched by the next call; copies made again behind it
+    y4 = check("after the optimizer")
+    assert np.abs(y4 - y3).max() > 1e-3
+    # the filter's memory handed to another tensor
+    lib.lh_rewind(mark0)
+    w_other = prog.up((rng.randn(k, c, 3, 3) * 0.1).astype(np.float32))
+    assert w_other == w
+    y5 = check("after a rewind that released the filter")
+    assert np.abs(y5 - y4).max() > 1e-3
