@@ -124,14 +124,13 @@ static void layouts_drop() { layouts_released(nullptr); }
 float* layout_lookup(const float* w, size_t wbytes, int kind, const int* prm, size_t bytes, bool& build) {
   build = false;
   if (!g_enabled || g_rec_on || g_capturing || g_prof_mask != 0 || g_stream_cur != g_stream_raw || w == nullptr) return nullptr;
+  // Copies made on the side stream since the last lookup: the main stream waits for them once, whether it is about to read one
+  // or to write one again (later lookups of the step must not wait for the filter gradients that run there by then).
+  if (g_layouts_on_side) { side_join(); g_layouts_on_side = false; }
   for (auto& l : g_layouts) {
     if (l.w != (const char*)w || l.kind != kind || l.bytes != bytes || memcmp(l.prm, prm, sizeof l.prm) != 0) continue;
     l.used = true;
-    if (l.valid) {
-      if (g_layouts_on_side) { side_join(); g_layouts_on_side = false; }     // once per step: later lookups must not wait for the filter gradients that run there by then
-      g_stat[ST_LAYOUTS]++;
-      return l.copy;
-    }
+    if (l.valid) { g_stat[ST_LAYOUTS]++; return l.copy; }
     // stale: the caller makes it again, in stream order in front of its use, and it holds until the filter is written again
     layout_set(l, true); g_busy = true; build = true;
     return l.copy;

@@ -417,7 +417,7 @@ int lh_capture_end(void) {
   return (int)g_graphs.size() - 1;
 }
 void lh_graph_launch(int id) {
-  { LZ_SCOPE(); lazy::flush_all(); }
+  lazy::flush_undeclared();         // a replay reads and writes whatever its recording did (parameters included): everything deferred is brought up to date, no kept copy survives
   LH_REQUIRE(id >= 0 && id < (int)g_graphs.size() && g_graphs[id] != nullptr, "lh_graph_launch: no graph %d", id);
   LH_HIP(hipGraphLaunch(g_graphs[id], g_stream));
 }
