@@ -438,3 +438,48 @@ def test_kept_filter_copies_end_with_every_write_of_the_filter(prog):
     assert w_other == w
     y5 = check("after a rewind that released the filter")
     assert np.abs(y5 - y4).max() > 1e-3
+
+
+def test_kept_filter_copies_end_with_a_graph_replay(on_hip):
+    """A recorded optimizer step replayed with lh_graph_launch changes the filter without any call that names it: the
+    convolution issued after the replay must read the new weights."""
+    pg = Prog(on_hip)
+    lib = on_hip.lib
+    rng = np.random.RandomState(59)
+    n, c, h, k = 4, 32, 14, 32
+    args = (n, c, h, h, k, 3, 3, 1, 1, 1, 1)
+    x = pg.up(rng.randn(n, c, h, h).astype(np.float32))
+    w = pg.up((rng.randn(k, c, 3, 3) * 0.1).astype(np.float32))
+    nw = k * c * 9
+    d = pg.up(rng.randn(nw).astype(np.float32)); v = pg.up(np.zeros(nw, np.float32))
+
+    def conv():
+        mark = lib.lh_mark()
+        y = pg.malloc(n * k * h * h); lib.lh_conv2d_fwd(x, w, 0, y, *args)
+        out = pg.down(y, (n * k * h * h,)); _lib.check()
+        lib.lh_rewind(mark)
+        return out
+    on_hip.setDeterministic(True)                           # (one launch plan, no atomics: the comparison below is bit for bit; the side stream stays on)
+    try:
+        _graph_replay_body(lib, conv, w, d, v, nw)
+    finally:
+        on_hip.setDeterministic(False)
+
+
+def _graph_replay_body(lib, conv, w, d, v, nw):
+    y0 = conv(); conv()                                     # the second call finds the kept copy
+    lib.lh_capture_begin()
+    lib.lh_momentum(w, d, v, 0.1, 0.9, 400.0, 0, nw)
+    gid = lib.lh_capture_end(); _lib.check()
+    for _ in range(2):
+        lib.lh_graph_launch(gid); _lib.check()
+        y1 = conv()
+        lib.lh_set_fusion(0)
+        try:
+            want = conv()
+        finally:
+            lib.lh_set_fusion(1)
+        np.testing.assert_array_equal(y1, want)
+        assert np.abs(y1 - y0).max() > 1e-3
+        y0 = y1
+    lib.lh_graph_destroy(gid); _lib.check()
