@@ -45,6 +45,13 @@ struct GemmShape {
   int streamk;                // != 0: `total` workers share tiles*slabsPerTile k-slabs evenly
   int slabsPerTile;
   long long units;            // tiles * slabsPerTile
+  // streamk == 2 (whole tiles and slices of the last ones: see igemm_launch_shared_tail): the first fixFull blocks compute
+  // one whole tile each; the tiles that are left are cut into fixCmax slices along the reduction (kPerSplit long), one block
+  // per slice.  A sliced tile is finished by the LAST of its slices to arrive: each stores its partial sums into fixWs
+  // (slot = slice), counts itself in fixCnt[tile], and the one that finds all others counted adds the partial sums up in
+  // slice order and runs the epilogue of a whole tile.  Nobody waits for anybody.
+  int fixFull, fixCmax, fixPer;       // fixPer: slices per XCD
+  float4* fixWs; int* fixCnt;
 };
 
 // ---- operand loaders ---------------------------------------------------------------------------
@@ -106,12 +113,15 @@ struct LhScal { uint32_t s[4]; };      // the wave-uniform parts of a SPLIT load
 template <class L>
 // `xs`: wave-uniform bytes on top of every offset of the group (the slabs stepped over since the offsets were computed)
 __device__ __forceinline__ float4 lh_fetch4(__amdgpu_buffer_rsrc_t rsrc, const LhOff<L>& f, const LhScal& u, int xs = 0) {
+  // (the scalar-offset operands are the same in all lanes by construction; said at the use, because inside the segment loop of
+  // the stream-K forms the compiler does not see it and wraps every load in a loop over the distinct values of a wavefront)
+  xs = __builtin_amdgcn_readfirstlane(xs);
   if (L::SPLIT) {
     float4 r;
-    r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[0] + xs, 0));
-    r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[1] + xs, 0));
-    r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[2] + xs, 0));
-    r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], (int)u.s[3] + xs, 0));
+    r.x = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], __builtin_amdgcn_readfirstlane((int)u.s[0]) + xs, 0));
+    r.y = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], __builtin_amdgcn_readfirstlane((int)u.s[1]) + xs, 0));
+    r.z = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], __builtin_amdgcn_readfirstlane((int)u.s[2]) + xs, 0));
+    r.w = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)f.o[0], __builtin_amdgcn_readfirstlane((int)u.s[3]) + xs, 0));
     return r;
   }
   if (L::VEC4) {
@@ -169,7 +179,7 @@ constexpr size_t igemm_smem_bytes() { return (size_t)2 * (BK / 4) * ((BM + 8 / (
 
 // ---- the kernel ------------------------------------------------------------------------------------
 // The work of one block; `block` is its index within the launch (or within its group of a grouped launch).
-template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
+template <int BM, int BN, int BK, class AL, class BL, class EP, int SK>      // SK: 0 one tile (or k-split of a tile) per block, 1 stream-K with atomic adds, 2 rounds + shared tail
 __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP& ep_in, const GemmShape& gs, const int block) {
   typename std::conditional<EP::SLICED, EP, const EP&>::type ep = ep_in;      // a sliced epilogue is a private copy that slice() moves
   constexpr int KQ = BK / 4, PAD = 8 / KQ, LDA = BM + PAD, LDB = BN + PAD;
@@ -184,13 +194,24 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   float4* As = lh_smem;
   float4* Bs = lh_smem + 2 * KQ * LDA;
 
-  const int logical = (block % 8) * gs.perXcd + block / 8;
+  int logical = (block % 8) * gs.perXcd + block / 8;
+  if (SK == 2) {
+    // every XCD gets an eighth of the whole tiles (consecutive ones: they share columns in its L2) and, behind them, an
+    // eighth of the slices, so that each compute unit is given its whole tiles first and its slices last
+    const int x = block % 8, li = block / 8, whole_per = gs.fixFull / 8;
+    if (li < whole_per) logical = x * whole_per + li;
+    else {
+      const int sl = x * gs.fixPer + (li - whole_per);
+      if (li - whole_per >= gs.fixPer || sl >= gs.total - gs.fixFull) return;
+      logical = gs.fixFull + sl;
+    }
+  }
   if (logical >= gs.total) return;
   // Work of this block: either one (tile, k-split) item, or -- stream-K -- an equal share of all
   // k-slabs of all tiles, walked tile by tile; a tile whose slabs are shared between two blocks
   // is completed with atomic adds.
   long long u = 0, u_end = 1;
-  if (SK) { u = gs.units * logical / gs.total; u_end = gs.units * (logical + 1) / gs.total; }
+  if (SK == 1) { u = gs.units * logical / gs.total; u_end = gs.units * (logical + 1) / gs.total; }
   // STEPPED: both loaders can be advanced by a wave-uniform step, so inside a run of slabs the offsets of the next slab
   // cost two scalar additions instead of a decode per element; a slab past the end of the reduction is switched off by a
   // buffer descriptor of zero bytes (every lane out of range, the loads return 0 without touching memory).
@@ -211,11 +232,24 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
     if (BL::ALONG_K) { b_kq[g] = t % KQ; b_col[g] = t / KQ + g * (256 / KQ); }
     else { b_col[g] = t % BN; b_kq[g] = __builtin_amdgcn_readfirstlane(t / BN) + g * (256 / BN); }
   }
-  const int lane = t & 63, wave = t >> 6, wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave, half = lane >> 5, l32 = lane & 31;
+  const int lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), wm = WM == 2 ? wave >> 1 : 0, wn = WM == 2 ? wave & 1 : wave, half = lane >> 5, l32 = lane & 31;
 
   while (u < u_end) {
   int tm, tn, kbeg, kend, part = 0;
-  if (SK) {
+  int fix_tile = 0, fix_n = 1, fix_slot = 0;       // SK == 2, part != 0: the sliced tile, its number of slices, this block's slice
+  if (SK == 2) {
+    int tile;
+    if (logical < gs.fixFull) { tile = logical; kbeg = 0; kend = gs.K; }
+    else {
+      const int i = logical - gs.fixFull;
+      fix_tile = i / gs.fixCmax; fix_slot = i - fix_tile * gs.fixCmax; fix_n = gs.fixCmax;
+      tile = gs.fixFull + fix_tile;
+      kbeg = fix_slot * gs.kPerSplit; kend = min(gs.K, kbeg + gs.kPerSplit);
+      part = 1;
+    }
+    tm = tile % gs.tilesM; tn = tile / gs.tilesM;
+    u = u_end;
+  } else if (SK) {
     const int tile = (int)(u / gs.slabsPerTile), s0 = (int)(u - (long long)tile * gs.slabsPerTile);
     const long long left = u_end - u;
     const int s1 = (int)(left < (long long)(gs.slabsPerTile - s0) ? s0 + left : gs.slabsPerTile);
@@ -232,6 +266,10 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
     kbeg = sp * gs.kPerSplit; kend = min(gs.K, kbeg + gs.kPerSplit);
     if constexpr (EP::SLICED) ep.slice(sp);
     u = u_end;
+  }
+  if (SK == 1) {       // the segment is the same for all lanes of the block
+    tm = __builtin_amdgcn_readfirstlane(tm); tn = __builtin_amdgcn_readfirstlane(tn);
+    kbeg = __builtin_amdgcn_readfirstlane(kbeg); kend = __builtin_amdgcn_readfirstlane(kend); part = __builtin_amdgcn_readfirstlane(part);
   }
   const int m0 = tm * BM, n0 = gs.colBase + tn * BN;
   typename AL::State sa[GA];
@@ -261,11 +299,11 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   auto elem = [&](int e, int k0) {
     if (e < GA * EA) {
       const int g = e / EA, i = e % EA, k = k0 + 4 * a_kq[g];
-      if constexpr (AL::SPLIT) { if (i == 0) oa[g].o[0] = al.voff(sa[g], k, kend); ua[g].s[i] = al.soff(k, i); }
+      if constexpr (AL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) oa[g].o[0] = al.voff(sa[g], ku, kend); ua[g].s[i] = al.soff(ku, i); }      // (a SPLIT loader's k is the same in all lanes: its groups run along the columns)
       else oa[g].o[i] = al.off1(sa[g], k, kend, i);
     } else {
       const int f = e - GA * EA, g = f / EB, i = f % EB, k = k0 + 4 * b_kq[g];
-      if constexpr (BL::SPLIT) { if (i == 0) ob[g].o[0] = bl.voff(sb[g], k, kend); ub[g].s[i] = bl.soff(k, i); }
+      if constexpr (BL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) ob[g].o[0] = bl.voff(sb[g], ku, kend); ub[g].s[i] = bl.soff(ku, i); }
       else ob[g].o[i] = bl.off1(sb[g], k, kend, i);
     }
   };
@@ -275,8 +313,10 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   int xsA = 0, xsB = 0, steps = 0, nrecA = (int)al.nbytes, nrecB = (int)bl.nbytes;
   auto fetch = [&](float4 (&ra)[GA], float4 (&rb)[GB]) {
     if constexpr (STEPPED) {
-      const __amdgpu_buffer_rsrc_t ra_ = __builtin_amdgcn_make_buffer_rsrc((void*)al.base, 0, nrecA, LH_RSRC_FLAGS);
-      const __amdgpu_buffer_rsrc_t rb_ = __builtin_amdgcn_make_buffer_rsrc((void*)bl.base, 0, nrecB, LH_RSRC_FLAGS);
+      // (the byte ranges are the same in all lanes; said here because inside the segment loop of the stream-K forms the
+      // compiler no longer sees it and wraps every load in a loop over the distinct descriptors of a wavefront)
+      const __amdgpu_buffer_rsrc_t ra_ = __builtin_amdgcn_make_buffer_rsrc((void*)al.base, 0, __builtin_amdgcn_readfirstlane(nrecA), LH_RSRC_FLAGS);
+      const __amdgpu_buffer_rsrc_t rb_ = __builtin_amdgcn_make_buffer_rsrc((void*)bl.base, 0, __builtin_amdgcn_readfirstlane(nrecB), LH_RSRC_FLAGS);
 #pragma unroll
       for (int g = 0; g < GA; g++) ra[g] = lh_fetch4<AL>(ra_, oa[g], ua[g], xsA);
 #pragma unroll
@@ -406,6 +446,64 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
     body(it + 1, 1, ra1, rb1, ra0, rb0);
   }
 
+  if constexpr (SK == 2) {
+    if (part) {
+      // The partial sums of this segment go to the workspace; the contributor that finds all the others counted adds them
+      // up, in slot order (its own included, so the result does not depend on who came last), and goes on as the owner of a
+      // whole tile.  Blocks on different XCDs do not share an L2, and a fence that writes a whole L2 back and invalidates it
+      // (what __threadfence() costs here: the launch took six times as long) is not needed for 16 KB: the partial sums are
+      // stored and loaded with the device-coherent cache policy (sc0 sc1: written through, read past the local L2), every
+      // wavefront waits for its stores to be acknowledged before the block counts itself, and the reads come after the count.
+      typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+      constexpr int Q = MI * NI * 4;          // 16-byte pieces per thread
+      constexpr int COHERENT = 17;            // cache policy bits of the buffer instructions: sc0 | sc1
+      const uint32_t slot_bytes = 256u * Q * 16u;
+      char* ws = reinterpret_cast<char*>(gs.fixWs) + (size_t)((size_t)fix_tile * gs.fixCmax) * slot_bytes;
+      {
+        const __amdgpu_buffer_rsrc_t rw_ = __builtin_amdgcn_make_buffer_rsrc((void*)(ws + (size_t)fix_slot * slot_bytes), 0, (int)slot_bytes, LH_RSRC_FLAGS);
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+          for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              u32x4 v4;
+              v4.x = __float_as_uint(acc[mi][ni][4 * q]); v4.y = __float_as_uint(acc[mi][ni][4 * q + 1]);
+              v4.z = __float_as_uint(acc[mi][ni][4 * q + 2]); v4.w = __float_as_uint(acc[mi][ni][4 * q + 3]);
+              __builtin_amdgcn_raw_buffer_store_b128(v4, rw_, (int)((t * Q + (mi * NI + ni) * 4 + q) * 16), 0, COHERENT);
+            }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      __shared__ int lh_fix_old;
+      if (t == 0) lh_fix_old = atomicAdd(gs.fixCnt + fix_tile, 1);
+      __syncthreads();
+      const int old = lh_fix_old;
+      if (old != fix_n - 1) continue;          // somebody else finishes this tile
+      if (t == 0) gs.fixCnt[fix_tile] = 0;     // left as found, for the next launch
+#pragma unroll
+      for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+          for (int v = 0; v < 16; v++) acc[mi][ni][v] = 0.f;
+      for (int sl = 0; sl < fix_n; sl++) {
+        const __amdgpu_buffer_rsrc_t rr_ = __builtin_amdgcn_make_buffer_rsrc((void*)(ws + (size_t)sl * slot_bytes), 0, (int)slot_bytes, LH_RSRC_FLAGS);
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+          for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(rr_, (int)((t * Q + (mi * NI + ni) * 4 + q) * 16), 0, COHERENT);
+              acc[mi][ni][4 * q] += __uint_as_float(w4.x); acc[mi][ni][4 * q + 1] += __uint_as_float(w4.y);
+              acc[mi][ni][4 * q + 2] += __uint_as_float(w4.z); acc[mi][ni][4 * q + 3] += __uint_as_float(w4.w);
+            }
+      }
+      part = 0;
+    }
+  }
+
   // D layout of a 32x32 block: column = lane % 32, row = 8*(v/4) + 4*(lane/32) + v%4
   // With EP::STATS the same pass also forms per-row sums of the finished tile (the batch-norm statistics of a
   // convolution's output rows = channels): every wavefront reduces its TM x TN piece over the columns and
@@ -414,7 +512,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
 #pragma unroll
   for (int ni = 0; ni < NI; ni++) cs[ni] = ep.col(n0 + wn * TN + ni * 32 + l32, gs.N);
   bool want_stats = false;
-  if constexpr (EP::STATS && !SK) want_stats = ep.partial != nullptr;
+  if constexpr (EP::STATS && SK != 1) want_stats = ep.partial != nullptr;
   // Lean stores (epilogues that offer them, complete sums only; partial sums added with buffer atomics measured slower
   // and stay on the general path): the element of row i and column j lies at
   // lane_bytes(j) + i * row_bytes(), so a store is one buffer instruction whose per-lane offset is fixed for the tile
@@ -490,7 +588,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
       }
     }
   }
-  if constexpr (EP::STATS && !SK) {
+  if constexpr (EP::STATS && SK != 1) {
     if (want_stats) {
       // Row sums of the wavefront's TM x TN piece.  A lane holds 16 rows of one column, and a sum over columns done
       // in registers costs five cross-lane steps per row; instead every 32 x 32 block goes through LDS once, transposed
@@ -532,7 +630,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   }  // segments
 }
 
-template <int BM, int BN, int BK, class AL, class BL, class EP, bool SK>
+template <int BM, int BN, int BK, class AL, class BL, class EP, int SK>
 __global__ void __launch_bounds__(256) k_igemm(const AL al, const BL bl, const EP ep, const GemmShape gs) {
   igemm_block<BM, BN, BK, AL, BL, EP, SK>(al, bl, ep, gs, (int)blockIdx.x);
 }
@@ -548,7 +646,7 @@ __global__ void __launch_bounds__(256) k_igemm_grouped(const IgemmGroups<AL, BL,
   int gi = 0;
 #pragma unroll
   for (int i = 1; i < IGEMM_MAX_GROUPS; i++) if (b >= g.first[i]) gi = i;
-  igemm_block<BM, BN, BK, AL, BL, EP, false>(g.al[gi], g.bl[gi], g.ep[gi], g.gs[gi], b - g.first[gi]);
+  igemm_block<BM, BN, BK, AL, BL, EP, 0>(g.al[gi], g.bl[gi], g.ep[gi], g.gs[gi], b - g.first[gi]);
 }
 
 
@@ -563,7 +661,7 @@ int igemm_blocks_per_cu() {
   static int occ = 0;
   if (occ == 0) {
     int v = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, k_igemm<BM, BN, BK, AL, BL, EP, false>, 256, igemm_smem_bytes<BM, BN, BK>()) != hipSuccess || v < 1) v = 2;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&v, k_igemm<BM, BN, BK, AL, BL, EP, 0>, 256, igemm_smem_bytes<BM, BN, BK>()) != hipSuccess || v < 1) v = 2;
     occ = v;
   }
   return occ;
@@ -596,11 +694,11 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
   if (gs.streamk) {
     if constexpr (smem <= 48 * 1024) {   // stream-K is instantiated for the forward / input-gradient tiles only
       ProfScope prof_(g_kernel_cat);
-      hipLaunchKernelGGL((k_igemm<BM, BN, BK, AL, BL, EP, true>), dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
+      hipLaunchKernelGGL((k_igemm<BM, BN, BK, AL, BL, EP, 1>), dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
       return true;
     } else { LH_FAIL("igemm: stream-K is not built for this tile"); return false; }
   }
-  auto kern = k_igemm<BM, BN, BK, AL, BL, EP, false>;
+  auto kern = k_igemm<BM, BN, BK, AL, BL, EP, 0>;
   static bool attr_done = false;
   if (smem > 48 * 1024 && !attr_done) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
@@ -611,6 +709,63 @@ bool igemm_launch(const AL& al, const BL& bl, const EP& ep, int M, int N, int K,
   ProfScope prof_(g_kernel_cat);
   hipLaunchKernelGGL(kern, dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
   return true;
+}
+
+// Whole tiles, and slices of the last ones (GemmShape::fixFull ...).  All tiles of these launches are resident at once, so a
+// compute unit's time is the number of tiles it was given: with 784 tiles on 256 units some unit has four and the rest wait
+// for it (3.06 on average: 76 %).  Here the multiple of the unit count that fits runs as whole tiles, one block each, and the
+// tiles that are left are cut along the reduction into 2, 4 or 8 slices, one block each, so that the last blocks placed are
+// small and land evenly.  The slices of a tile meet in a workspace; whichever arrives last adds them up in slice order and
+// runs the epilogue, so the output needs no clearing, the epilogue sees complete sums (bias, clamp, batch-norm statistics
+// work as on whole tiles) and the result does not depend on the order of arrival.  Main stream only: the counters and the
+// workspace (arena scratch) have one user at a time.
+constexpr int FIX_MAX_TILES = 4096;
+template <int BM, int BN, int BK, class AL, class BL, class EP>
+bool igemm_launch_shared_tail(const AL& al, const BL& bl, const EP& ep, int M, int N, int K, int col0 = 0, int col1 = -1) {
+  constexpr size_t smem = igemm_smem_bytes<BM, BN, BK>();
+  if constexpr (smem > 48 * 1024) { LH_FAIL("igemm: sliced tiles are not built for this tile shape"); return false; }
+  else {
+    if (col1 < 0 || col1 > N) col1 = N;
+    if (col0 >= col1) return true;
+    GemmShape gs{};
+    gs.M = M; gs.N = col1; gs.K = K; gs.colBase = col0;
+    gs.tilesM = (int)cdiv(M, BM); gs.tilesN = (int)cdiv(col1 - col0, BN);
+    gs.slabsPerTile = (int)cdiv(K > 0 ? K : 1, BK);
+    gs.units = (long long)gs.tilesM * gs.tilesN * gs.slabsPerTile;
+    gs.streamk = 2; gs.splitK = 1;
+    const int64_t tiles = (int64_t)gs.tilesM * gs.tilesN, cus = g_num_cu;
+    if (cus % 8 != 0) return igemm_launch<BM, BN, BK>(al, bl, ep, M, N, K, 1, 0, col0, col1);
+    const int64_t whole = tiles / cus * cus, tail = tiles - whole;
+    // slices per tile of the tail: the count whose last placement round is fullest (what is lost is the idle part of that
+    // round, in tiles per unit), at least four slabs per slice; ties go to the smaller count
+    int slices = 1; double best = 1e9;
+    for (int sc = 1; sc <= 8; sc *= 2) {
+      if (sc > 1 && gs.slabsPerTile / sc < 4) break;
+      const double lost = (double)cdiv(tail * sc, cus) / sc - (double)tail / cus;
+      if (lost < best - 1e-9) { best = lost; slices = sc; }
+    }
+    if (tail == 0 || slices == 1 || tail > FIX_MAX_TILES || tiles > 0x3fffffff || g_stream_cur != g_stream_raw)
+      return igemm_launch<BM, BN, BK>(al, bl, ep, M, N, K, 1, 0, col0, col1);
+    const int per = (int)cdiv(gs.slabsPerTile, slices);
+    gs.kPerSplit = per * BK;
+    gs.fixCmax = (int)cdiv(gs.slabsPerTile, per);
+    gs.fixFull = (int)whole;
+    const int64_t total = whole + tail * gs.fixCmax;
+    gs.total = (int)total;
+    gs.fixPer = (int)cdiv(tail * gs.fixCmax, 8);
+    gs.perXcd = (int)(whole / 8) + gs.fixPer;          // (the unit count is a multiple of 8, so are the whole tiles)
+    const size_t wsbytes = (size_t)tail * gs.fixCmax * BM * BN * sizeof(float);
+    gs.fixWs = (float4*)lh_malloc_uninit(wsbytes);
+    gs.fixCnt = fix_counters();
+    if (gs.fixWs == nullptr || gs.fixCnt == nullptr) return false;
+    if (getenv("LH_TAIL_VERBOSE")) fprintf(stderr, "sliced tail %dx%d: M%d N%d K%d: %lld whole tiles, %lld tiles in %d slices of %d slabs\n", BM, BN, M, col1 - col0, K, (long long)whole, (long long)tail, gs.fixCmax, per);
+    {
+      ProfScope prof_(g_kernel_cat);
+      hipLaunchKernelGGL((k_igemm<BM, BN, BK, AL, BL, EP, 2>), dim3(8 * gs.perXcd), dim3(256), smem, g_stream, al, bl, ep, gs);
+    }
+    lh_free_top(wsbytes);
+    return true;
+  }
 }
 
 // Times `launch` (a callable returning false on failure) on the library's stream: five repetitions, the first warms

@@ -44,6 +44,8 @@ void* side_scratch(size_t bytes) {
   g_side_scratch = (char*)p; g_side_scratch_bytes = want;
   return p;
 }
+static int* g_fix_cnt = nullptr;
+int* fix_counters() { return g_fix_cnt; }
 void* persistent_alloc(size_t bytes) {
   void* p = nullptr;
   if (hipMalloc(&p, bytes) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
@@ -168,6 +170,8 @@ void lh_setup(size_t heap_bytes) {
   g_arena = ArenaState(); g_arena.bytes = heap_bytes;
   lazy::reset();
   LH_HIP(hipMalloc((void**)&g_advance_pool, MAX_GRAPHS * sizeof(unsigned long long)));
+  LH_HIP(hipMalloc((void**)&g_fix_cnt, 4096 * sizeof(int)));          // FIX_MAX_TILES arrival counters (lh_igemm.h), zero between launches
+  LH_HIP(hipMemset(g_fix_cnt, 0, 4096 * sizeof(int)));
   if (!multi_tensor_setup()) return;
 }
 
@@ -188,6 +192,8 @@ void lh_cleanup(void) {
   g_graphs.clear(); g_capturing = false;
   if (g_advance_pool) (void)hipFree(g_advance_pool);
   g_advance_pool = nullptr; g_capture_advance = nullptr;
+  if (g_fix_cnt) (void)hipFree(g_fix_cnt);
+  g_fix_cnt = nullptr;
   if (g_heap) (void)hipFree(g_heap);
   if (g_stream_raw) (void)hipStreamDestroy(g_stream_raw);
   g_heap = nullptr; g_stream_raw = nullptr; g_stream_cur = nullptr; g_arena = ArenaState();

@@ -264,3 +264,85 @@ def test_plain_tile_plans_give_the_same_bits(on_hip, dims, monkeypatch):
     finally:
         monkeypatch.delenv("LH_FORCE_PLAN", raising=False)
         lib.lh_set_deterministic(0)
+
+
+SHARED_TAIL_SHAPES = [
+    (64, 256, 14, 14, 256, 1, 1, 1, 1, 0, 0),     # 784 tiles of 64x64: one round of whole tiles and a tail of 272 (on 256 compute units)
+    (16, 512, 7, 7, 512, 3, 3, 1, 1, 1, 1),       # fewer tiles than workers: every tile shared
+    (4, 256, 14, 14, 256, 3, 3, 1, 1, 1, 1),      # few tiles over a long reduction
+    (6, 96, 15, 15, 160, 3, 3, 1, 1, 1, 1),       # odd map: partial tiles in both directions
+    (64, 64, 28, 28, 128, 1, 1, 1, 1, 0, 0),      # short reduction (4 slabs): below the plans' floor, falls back to the rule
+    (8, 128, 28, 28, 256, 1, 1, 2, 2, 0, 0),      # stride 2: one class, 2x2 cells
+]
+
+
+@pytest.mark.parametrize("dims", SHARED_TAIL_SHAPES, ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("plan", [13, 14], ids=["tiles64x64", "tiles64x128"])
+def test_rounds_of_whole_tiles_and_a_shared_tail(on_hip, dims, plan, monkeypatch):
+    """The launch plans that cut the last round's tiles along the reduction over all compute units (the contributor that adds
+    the last piece finishes the tile): forward with bias and with the clamp, input gradient overwriting and accumulating,
+    against the whole-tile plan; two runs give the same bits (nothing is combined with atomic adds)."""
+    dev = Dev(on_hip)
+    lib = on_hip.lib
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    rng = np.random.RandomState(97)
+    xd = dev.up(rng.randn(N, Cc, H, W).astype(np.float32))
+    wd = dev.up((rng.randn(K, Cc, R, S) / np.sqrt(Cc * R * S)).astype(np.float32))
+    bd = dev.up(rng.randn(K).astype(np.float32))
+    dyd = dev.up(rng.randn(N, K, P, Q).astype(np.float32))
+    ny, nx = N * K * P * Q, N * Cc * H * W
+
+    def run(p):
+        monkeypatch.setenv("LH_FORCE_PLAN", str(p))
+        y = dev.up(np.full(ny, 7.0, np.float32)); lib.lh_conv2d_fwd(xd.ptr, wd.ptr, bd.ptr, y.ptr, *dims)
+        dx0 = dev.up(np.full(nx, 7.0, np.float32)); lib.lh_conv2d_bwd_data(dyd.ptr, wd.ptr, dx0.ptr, 0.0, *dims)
+        dx1 = dev.up(np.ones(nx, np.float32)); lib.lh_conv2d_bwd_data(dyd.ptr, wd.ptr, dx1.ptr, 1.0, *dims)
+        dev.check()
+        return [dev.down(y, (ny,)).copy(), dev.down(dx0, (nx,)).copy(), dev.down(dx1, (nx,)).copy() - 1.0]
+    try:
+        want = run(3)
+        got = run(plan)
+        again = run(plan)
+    finally:
+        monkeypatch.delenv("LH_FORCE_PLAN", raising=False)
+    for name, g, a, w_ in zip(("forward", "input gradient", "input gradient, accumulating"), got, again, want):
+        assert_close(g, w_, rtol=2e-5, what="%s, plan %d" % (name, plan))
+        if name != "input gradient, accumulating":
+            np.testing.assert_array_equal(g, a, err_msg="%s: two runs of plan %d" % (name, plan))
+    assert np.abs(want[0]).max() > 0.1 and np.abs(want[1]).max() > 0.1
+
+
+@pytest.mark.parametrize("dims", [(64, 256, 14, 14, 256, 1, 1, 1, 1, 0, 0), (16, 512, 7, 7, 512, 3, 3, 1, 1, 1, 1), (6, 96, 15, 15, 160, 3, 3, 1, 1, 1, 1)],
+                         ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("tile", [5, 6], ids=["tiles64x64", "tiles64x128"])
+def test_sliced_last_tiles_leave_the_same_batchnorm_statistics(on_hip, dims, tile, monkeypatch):
+    """The forward launch that leaves batch-norm statistics behind, with its last tiles cut along the reduction: the block that
+    finishes a sliced tile has the complete sums, so output and statistics are those of the whole-tile launch (to rounding:
+    the slices are added in slice order) and two runs agree bit for bit."""
+    dev = Dev(on_hip)
+    lib = on_hip.lib
+    N, Cc, H, W, K, R, S, sH, sW, pH, pW = dims
+    P, Q = (H + 2 * pH - R) // sH + 1, (W + 2 * pW - S) // sW + 1
+    rng = np.random.RandomState(101)
+    xd = dev.up(rng.randn(N, Cc, H, W).astype(np.float32))
+    wd = dev.up((rng.randn(K, Cc, R, S) / np.sqrt(Cc * R * S)).astype(np.float32))
+    ny = N * K * P * Q
+
+    def run(f):
+        monkeypatch.setenv("LH_FORCE_STATS_TILE", str(f))
+        y = dev.up(np.full(ny, 7.0, np.float32)); sm = dev.zeros(K); si = dev.zeros(K); rm = dev.zeros(K); rv = dev.up(np.ones(K, np.float32))
+        lib.lh_conv2d_fwd_bnstats(xd.ptr, wd.ptr, 0, y.ptr, *dims, sm.ptr, si.ptr, rm.ptr, rv.ptr, 1e-5, 0.1)
+        dev.check()
+        return [dev.down(y, (ny,)).copy(), dev.down(sm, (K,)).copy(), dev.down(si, (K,)).copy(), dev.down(rm, (K,)).copy(), dev.down(rv, (K,)).copy()]
+    try:
+        want = run(3)
+        got = run(tile)
+        again = run(tile)
+    finally:
+        monkeypatch.delenv("LH_FORCE_STATS_TILE", raising=False)
+    assert_close(got[0], want[0], rtol=2e-5, what="output")
+    for i, name in ((1, "mean"), (2, "1/std"), (3, "running mean"), (4, "running variance")):
+        np.testing.assert_allclose(got[i], want[i], rtol=2e-5, atol=2e-6, err_msg=name)
+    for g, a in zip(got, again):
+        np.testing.assert_array_equal(g, a)
