@@ -452,9 +452,9 @@ static bool launch_rounds(const AL& al, const BL& bl, const EP& ep, int M, int N
 // 10: 32x128 tiles (32-deep slabs) for products of at most 32 rows, whose 64-row tiles would be half empty.
 // 11-12: stream-K over 64x64 tiles with one worker per 32 or 8 slabs: a handful of tiles under a very long reduction (a filter
 // as large as the map: a fully connected layer), where a worker per CU would mean hundreds of atomic adds onto each element.
-// 13-14: rounds of whole 64x64 / 64x128 tiles, then a shared tail (igemm_launch_shared_tail): the last round's tiles are cut
-// along the reduction over all compute units and finished by whoever adds the last piece.
-constexpr int N_PLANS = 15;
+// 13-15: whole 64x64 / 64x128 / 128x128 tiles, the last ones (what is left over a multiple of the compute units) cut into
+// slices along the reduction and finished by whichever slice arrives last (igemm_launch_shared_tail).
+constexpr int N_PLANS = 16;
 // LH_FORCE_M32 in the environment: products of at most 32 rows always take the 32-row tile (for tests of that tile; the
 // measured choice may well be another one).
 static inline bool force_m32() { return getenv("LH_FORCE_M32") != nullptr; }
@@ -468,8 +468,8 @@ static bool plan_valid(int plan, const EP& ep, int M, int K, bool can_zero) {
   if (plan == 0) return true;
   if (plan == 10) return M <= 32;
   if ((plan == 1 || plan == 4 || plan == 6) && M <= 64) return false;
-  if (plan == 13 || plan == 14) return !g_deterministic && g_stream_cur == g_stream_raw && cdiv(K, CONV_BK) >= 8;   // (same bits in every run, but not those of the whole-tile plans)
-  if ((plan >= 4 && plan <= 9) || plan >= 11) {
+  if (plan >= 13 && plan <= 15) return !g_deterministic && g_stream_cur == g_stream_raw && cdiv(K, CONV_BK) >= 8 && (plan != 15 || M > 64);   // (same bits in every run, but not those of the whole-tile plans)
+  if ((plan >= 4 && plan <= 9) || plan == 11 || plan == 12) {
     if (g_deterministic) return false;        // partial sums meet in atomic adds, in whatever order the blocks arrive
     return (ep.beta == 1.f || can_zero) && cdiv(K, CONV_BK) >= (plan >= 11 ? 64 : 16);
   }
@@ -482,6 +482,7 @@ static bool launch_plan(int plan, const AL& al, const BL& bl, const EP& ep, int 
   if (plan == 10) return igemm_launch<32, 128, 32>(al, bl, ep, M, N, K, 1);
   if (plan == 13) return igemm_launch_shared_tail<64, 64, CONV_BK>(al, bl, ep, M, N, K);
   if (plan == 14) return igemm_launch_shared_tail<64, 128, CONV_BK>(al, bl, ep, M, N, K);
+  if (plan == 15) return igemm_launch_shared_tail<128, 128, CONV_BK>(al, bl, ep, M, N, K);
   if (plan >= 11) {
     g_launch_partial = true;
     const int64_t units = cdiv(M, 64) * cdiv(N, 64) * cdiv(K, CONV_BK);
@@ -565,14 +566,14 @@ struct StatLayout { int col1, g_main, slots_main, g_rem, slots_rem; int sliced =
 // The tile plan launch_tiles would choose, for a launch that also leaves statistics pieces.  Returns false (and
 // launches nothing) for shapes that take the stream-K path, whose tiles are finished by several blocks.
 template <class AL, class BL>
-static bool plan_tiles_stats(int M, int N, int K, StatLayout& L, int& bm, int& bn, int force = 0 /* 1-3: the tile of launch plan 1-3; 5, 6: 64x64 / 64x128 tiles with the last ones sliced */) {
+static bool plan_tiles_stats(int M, int N, int K, StatLayout& L, int& bm, int& bn, int force = 0 /* 1-3: the tile of launch plan 1-3; 5-7: 64x64 / 64x128 / 128x128 tiles with the last ones sliced */) {
   const int64_t t128 = cdiv(M, 128) * cdiv(N, 128), t64 = cdiv(M, 64) * cdiv(N, 128);
   const bool few = (M > 64 ? t128 : t64) < 6 * (int64_t)g_num_cu;
   const int64_t slabs = cdiv(K, CONV_BK);
   if (!g_deterministic && few && slabs >= 64 && slabs * (M > 64 ? t128 : t64) >= 48 * (int64_t)(2 * g_num_cu)) return false;
   TilePick tp = pick_tile_conv(M, N, K);
-  if (force == 1 && M > 64) tp = {128, 128}; else if (force == 2 || force == 6) tp = {64, 128}; else if (force == 3 || force == 5) tp = {64, 64};
-  L.sliced = (force == 5 || force == 6) && !g_deterministic && g_stream_cur == g_stream_raw && cdiv(K, CONV_BK) >= 8;
+  if ((force == 1 || force == 7) && M > 64) tp = {128, 128}; else if (force == 2 || force == 6) tp = {64, 128}; else if (force == 3 || force == 5) tp = {64, 64};
+  L.sliced = (force == 5 || force == 6 || (force == 7 && M > 64)) && !g_deterministic && g_stream_cur == g_stream_raw && cdiv(K, CONV_BK) >= 8;
   bm = tp.bm; bn = tp.bn;
   L.col1 = N; L.g_main = bn / 2; L.g_rem = 32; L.slots_rem = 0;
   if (bn == 128 && !L.sliced) {        // the surplus-tile split of launch_rounds
@@ -593,7 +594,7 @@ template <class AL, class BL>
 static bool launch_tiles_stats(const AL& al, const BL& bl, EpiConvOutStats ep, int M, int N, int K, const StatLayout& L, int bm, int bn) {
   ep.slotBase = 0;
   bool ok;
-  if (L.sliced) return bn == 128 ? igemm_launch_shared_tail<64, 128, CONV_BK>(al, bl, ep, M, N, K) : igemm_launch_shared_tail<64, 64, CONV_BK>(al, bl, ep, M, N, K);
+  if (L.sliced) return bm == 128 ? igemm_launch_shared_tail<128, 128, CONV_BK>(al, bl, ep, M, N, K) : (bn == 128 ? igemm_launch_shared_tail<64, 128, CONV_BK>(al, bl, ep, M, N, K) : igemm_launch_shared_tail<64, 64, CONV_BK>(al, bl, ep, M, N, K));
   if (bm == 128) ok = igemm_launch<128, 128, CONV_BK>(al, bl, ep, M, N, K, 1, 0, 0, L.col1);
   else if (bn == 128) ok = igemm_launch<64, 128, CONV_BK>(al, bl, ep, M, N, K, 1, 0, 0, L.col1);
   else ok = igemm_launch<64, 64, CONV_BK>(al, bl, ep, M, N, K, 1, 0, 0, L.col1);
@@ -642,7 +643,7 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
       const PlanKey key = {{K, N * PQ, CRS, H, W, sH, R}};
       const bool tunable = g_tune_lookup && 2.0 * K * CRS * (double)N * PQ >= g_tune_min_flop;
       int force = 0;
-      auto run = [&](int f) {           // 0: the rule's tile, 1-3: a forced tile, 4: unfused (any launch plan, then a pass over y), 5-6: 64x64 / 64x128 tiles, the last ones sliced
+      auto run = [&](int f) {           // 0: the rule's tile, 1-3: a forced tile, 4: unfused (any launch plan, then a pass over y), 5-7: 64x64 / 64x128 / 128x128 tiles, the last ones sliced
         if (f == 4) {
           if (!launch_tiles(al, bl, ep, K, N * PQ, CRS, y, (int64_t)N * K * PQ)) return false;
           lh_bn_stats(y, bn->save_mean, bn->save_invstd, nullptr, nullptr, N, K, PQ, bn->eps, bn->factor);
@@ -667,8 +668,8 @@ static void conv_fwd_impl(const float* x, const float* w, const float* bias, flo
           LaunchTimer timer;
           if (timer.ok) {
             float best_ms = 3.0e38f, base_ms = 0.f; int best = 0;
-            for (int f = 0; f <= 6; f++) {
-              if (f == 1 && K <= 64) continue;
+            for (int f = 0; f <= 7; f++) {
+              if ((f == 1 || f == 7) && K <= 64) continue;
               if (f >= 5 && (g_deterministic || CRS < 8 * CONV_BK)) continue;
               const float ms = timer.ms([&]() { return run(f); });
               if (ms < 0.f || failed()) return;

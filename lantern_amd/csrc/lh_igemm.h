@@ -738,6 +738,8 @@ bool igemm_launch_shared_tail(const AL& al, const BL& bl, const EP& ep, int M, i
     const int64_t whole = tiles / cus * cus, tail = tiles - whole;
     // slices per tile of the tail: the count whose last placement round is fullest (what is lost is the idle part of that
     // round, in tiles per unit), at least four slabs per slice; ties go to the smaller count
+    // (measured and dropped: preferring more slices at equal loss when there are fewer tiles than units, for the latency
+    // more blocks per unit hide: the CIFAR-shaped ResNet-50 step went from 4.18 to 4.33 ms)
     int slices = 1; double best = 1e9;
     for (int sc = 1; sc <= 8; sc *= 2) {
       if (sc > 1 && gs.slabsPerTile / sc < 4) break;

@@ -277,10 +277,10 @@ SHARED_TAIL_SHAPES = [
 
 
 @pytest.mark.parametrize("dims", SHARED_TAIL_SHAPES, ids=lambda d: "x".join(map(str, d)))
-@pytest.mark.parametrize("plan", [13, 14], ids=["tiles64x64", "tiles64x128"])
-def test_rounds_of_whole_tiles_and_a_shared_tail(on_hip, dims, plan, monkeypatch):
-    """The launch plans that cut the last round's tiles along the reduction over all compute units (the contributor that adds
-    the last piece finishes the tile): forward with bias and with the clamp, input gradient overwriting and accumulating,
+@pytest.mark.parametrize("plan", [13, 14, 15], ids=["tiles64x64", "tiles64x128", "tiles128x128"])
+def test_whole_tiles_and_slices_of_the_last_ones(on_hip, dims, plan, monkeypatch):
+    """The launch plans that cut the last tiles (what is left over a multiple of the compute units) into slices along the
+    reduction, one block each; the slice that arrives last adds them up and finishes the tile: forward with bias and with the clamp, input gradient overwriting and accumulating,
     against the whole-tile plan; two runs give the same bits (nothing is combined with atomic adds)."""
     dev = Dev(on_hip)
     lib = on_hip.lib
@@ -315,7 +315,7 @@ def test_rounds_of_whole_tiles_and_a_shared_tail(on_hip, dims, plan, monkeypatch
 
 @pytest.mark.parametrize("dims", [(64, 256, 14, 14, 256, 1, 1, 1, 1, 0, 0), (16, 512, 7, 7, 512, 3, 3, 1, 1, 1, 1), (6, 96, 15, 15, 160, 3, 3, 1, 1, 1, 1)],
                          ids=lambda d: "x".join(map(str, d)))
-@pytest.mark.parametrize("tile", [5, 6], ids=["tiles64x64", "tiles64x128"])
+@pytest.mark.parametrize("tile", [5, 6, 7], ids=["tiles64x64", "tiles64x128", "tiles128x128"])
 def test_sliced_last_tiles_leave_the_same_batchnorm_statistics(on_hip, dims, tile, monkeypatch):
     """The forward launch that leaves batch-norm statistics behind, with its last tiles cut along the reduction: the block that
     finishes a sliced tile has the complete sums, so output and statistics are those of the whole-tile launch (to rounding:
