@@ -99,6 +99,7 @@ struct Layout { const char* w; size_t wbytes; int kind; int prm[LAYOUT_PRM]; flo
 static std::vector<Layout> g_layouts;
 static int g_layouts_valid = 0;
 static size_t g_layout_bytes = 0;
+int g_layout_refresh_min = 8;                            // stale copies it takes for the side stream to be used (see layouts_refresh)
 static bool g_layouts_on_side = false;                   // copies made on the side stream that the main stream has not waited for yet
 static const size_t LAYOUT_CAP = (size_t)1 << 30;        // all copies together; filters beyond that are copied per call as before
 
@@ -146,9 +147,13 @@ float* layout_lookup(const float* w, size_t wbytes, int kind, const int* prm, si
 }
 // behind the optimizer launch: the copies the last step used, made again beside what comes next
 static void layouts_refresh() {
-  bool any = false;
-  for (auto& l : g_layouts) any = any || (l.used && !l.valid);
-  if (!any || !side_work_begin()) return;
+  // Only where it pays: handing work to the second stream and waiting for it once costs a few tens of microseconds of
+  // latency on both streams (LeNet's 0.26 ms step became 0.29 ms with its one copy made there, DeepSpeech2's 11.5 ms step
+  // 12.8: its 1110 back-to-back step kernels are dispatched more slowly while the second queue is in use), which a handful
+  // of 5 us copy kernels in the chain do not.  Networks with many filters to copy (8 or more) come out ahead.
+  int stale = 0;
+  for (auto& l : g_layouts) stale += (l.used && !l.valid) ? 1 : 0;
+  if (stale < g_layout_refresh_min || !side_work_begin()) return;
   for (auto& l : g_layouts) {
     if (!l.used || l.valid) continue;
     build_filter_layout(l.kind, l.prm, (const float*)l.w, l.copy);

@@ -400,6 +400,7 @@ int main(int argc, char** argv) {
   const int programs = argc > 1 ? atoi(argv[1]) : 2000;
   const uint64_t seed0 = argc > 2 ? (uint64_t)atoll(argv[2]) : 1;
   g_arena.bytes = 4u << 20;
+  lazy::g_layout_refresh_min = 1;           // (the library asks for eight stale copies before it uses the side stream; here every program has fewer)
   g_heap = (char*)aligned_alloc(256, g_arena.bytes);
   long long k_on = 0, k_off = 0, fused = 0;
   for (int p = 0; p < programs; p++) {
