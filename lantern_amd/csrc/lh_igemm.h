@@ -487,18 +487,32 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
         for (int ni = 0; ni < NI; ni++)
 #pragma unroll
           for (int v = 0; v < 16; v++) acc[mi][ni][v] = 0.f;
-      for (int sl = 0; sl < fix_n; sl++) {
-        const __amdgpu_buffer_rsrc_t rr_ = __builtin_amdgcn_make_buffer_rsrc((void*)(ws + (size_t)sl * slot_bytes), 0, (int)slot_bytes, LH_RSRC_FLAGS);
+      // the slices are added in slice order; the loads of up to four of them are in flight at once (each is a round trip to
+      // memory past the local L2, and nothing else is left to hide it behind)
+      constexpr int AHEAD = Q <= 4 ? 4 : (Q <= 8 ? 2 : 1);
+      for (int s0 = 0; s0 < fix_n; s0 += AHEAD) {
+        u32x4 w4[AHEAD][Q];
 #pragma unroll
-        for (int mi = 0; mi < MI; mi++)
+        for (int a = 0; a < AHEAD; a++) {
+          const int sl = s0 + a < fix_n ? s0 + a : fix_n - 1;          // (a repeat of the last slice is loaded and not added)
+          const __amdgpu_buffer_rsrc_t rr_ = __builtin_amdgcn_make_buffer_rsrc((void*)(ws + (size_t)sl * slot_bytes), 0, (int)slot_bytes, LH_RSRC_FLAGS);
 #pragma unroll
-          for (int ni = 0; ni < NI; ni++)
+          for (int j = 0; j < Q; j++) w4[a][j] = __builtin_amdgcn_raw_buffer_load_b128(rr_, (int)((t * Q + j) * 16), 0, COHERENT);
+        }
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-              const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(rr_, (int)((t * Q + (mi * NI + ni) * 4 + q) * 16), 0, COHERENT);
-              acc[mi][ni][4 * q] += __uint_as_float(w4.x); acc[mi][ni][4 * q + 1] += __uint_as_float(w4.y);
-              acc[mi][ni][4 * q + 2] += __uint_as_float(w4.z); acc[mi][ni][4 * q + 3] += __uint_as_float(w4.w);
-            }
+        for (int a = 0; a < AHEAD; a++) {
+          if (s0 + a >= fix_n) break;
+#pragma unroll
+          for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+            for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+              for (int q = 0; q < 4; q++) {
+                const u32x4 v4 = w4[a][(mi * NI + ni) * 4 + q];
+                acc[mi][ni][4 * q] += __uint_as_float(v4.x); acc[mi][ni][4 * q + 1] += __uint_as_float(v4.y);
+                acc[mi][ni][4 * q + 2] += __uint_as_float(v4.z); acc[mi][ni][4 * q + 3] += __uint_as_float(v4.w);
+              }
+        }
       }
       part = 0;
     }
