@@ -18,7 +18,7 @@ struct BwdfKey {
   int v[11];
   bool operator<(const BwdfKey& o) const { for (int i = 0; i < 11; i++) if (v[i] != o.v[i]) return v[i] < o.v[i]; return false; }
 };
-struct BwdfPlan { int bm, bn, split; };
+struct BwdfPlan { int bm, bn, split, twopass; };     // twopass: the slices go to scratch blocks and a second kernel adds them up (no atomic adds)
 static std::map<BwdfKey, BwdfPlan> g_bwdf_split;
 
 constexpr int TPB = 256;
@@ -979,31 +979,28 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   int split = clamp_split(cdiv(3 * (int64_t)g_num_cu, tiles));
   // How many slices pays best depends on how tiles x slices fall onto the resident block slots and on how short the
   // per-block reduction gets; it is measured once per shape (a few candidates on a scratch output) and remembered.
-  const BwdfKey key = {{N, C, H, W, K, R, S, sH, sW, pH, pW}};
+  const BwdfKey key = {{N, C, H, W, K, R, S, sH | (g_deterministic ? 1 << 16 : 0), sW, pH, pW}};     // deterministic mode measures among fewer forms
   const bool tunable = g_tune_lookup && max_split > 1 && 2.0 * K * CRS * (double)red >= g_tune_min_flop;
   bool tune_now = false;
+  // Slices are combined either with atomic adds onto dw (cleared first when beta = 0) or in two passes: every slice writes
+  // its own [K, CRS] block of scratch memory and a second kernel adds the blocks onto beta*dw in slice order.  Deterministic
+  // mode always takes the second; otherwise it is part of what is measured (large filters over small maps, where a block's
+  // reduction is short against the 64 KB of atomic adds it ends in, come out ahead with it).
+  bool twopass = g_deterministic;
   if (tunable) {
     auto it = g_bwdf_split.find(key);
-    if (it != g_bwdf_split.end()) { g_plans_remembered++; tp = TilePick{it->second.bm, it->second.bn}; tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn); split = clamp_split(it->second.split); }
+    if (it != g_bwdf_split.end()) { g_plans_remembered++; tp = TilePick{it->second.bm, it->second.bn}; tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn); split = clamp_split(it->second.split); twopass = it->second.twopass != 0; }
     else tune_now = g_tune_measure;
   }
   if (K <= 32 && force_m32()) { tp = TilePick{32, 128}; tiles = cdiv(K, 32) * cdiv(CRS, 128); split = clamp_split(cdiv(3 * (int64_t)g_num_cu, tiles)); tune_now = false; }
-  // Deterministic mode: every slice of the reduction writes its own [K, CRS] block of scratch memory (no atomics), and a
-  // second kernel adds the blocks onto beta*dw in slice order.
   float* partial = nullptr; size_t partial_bytes = 0; int slices = 1; bool on_side = false;
-  if (g_deterministic && split > 1) {
+  // what igemm_launch will make of `split` for the tile in tp
+  auto slices_of = [&](int sp) {
     const int bk = tp.bm == 128 ? 16 : (tp.bm == 32 ? 32 : BWDF_BK);
-    int64_t kper = cdiv(cdiv(red, split), bk) * bk; if (kper < bk) kper = bk;
-    slices = (int)cdiv(red, kper);                                    // what igemm_launch will make of `split`
-    if (slices > 1) {
-      partial_bytes = (size_t)slices * K * CRS * sizeof(float);
-      partial = (float*)scratch_take(partial_bytes, on_side);
-      if (partial == nullptr) return;
-    }
-  }
-  if (beta == 0.f && partial == nullptr) lh_fill(dw, 0.f, (int64_t)K * CRS);
+    int64_t kper = cdiv(cdiv(red, sp), bk) * bk; if (kper < bk) kper = bk;
+    return (int)cdiv(red, kper);
+  };
   EpiRowMajor ep; ep.C = dw; ep.ldc = CRS; ep.alpha = 1.f; ep.beta = 1.f; ep.atomic = split > 1 ? 1 : 0;
-  if (partial) { ep.C = partial; ep.sliceStride = (long long)K * CRS; ep.beta = 0.f; }
   bool ok = false;
   auto go = [&](auto al, auto bl) {
     al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
@@ -1036,47 +1033,80 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
     else if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<2>());
     else go(LoadConvBwdFilterA<false, true>(), LoadConvBwdFilterB<2>());
   };
+  // one launch of the plan in (tp, split) into `out` (accumulating), slices through `pbuf` when it is given
+  auto run_plan = [&](float* out, float* pbuf, float out_beta) {
+    const int sl = slices_of(split);
+    if (pbuf != nullptr && sl > 1) {
+      ep.C = pbuf; ep.sliceStride = (long long)K * CRS; ep.beta = 0.f;
+      dispatch();
+      if (ok) reduce_slices(out, CRS, K, CRS, pbuf, sl, out_beta);
+    } else {
+      ep.C = out; ep.sliceStride = 0; ep.beta = 1.f;
+      dispatch();
+    }
+  };
   if (tune_now) {
     const size_t sbytes = (size_t)K * CRS * sizeof(float);
+    const size_t pcap = (size_t)256 << 20;                    // two-pass candidates whose slices need more scratch than this are not tried
+    const double targets[] = {1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 5.0, 6.0};
+    const TilePick shapes[4] = {{128, 128}, {64, 128}, {64, 64}, {32, 128}};      // the last for layers of at most 32 output channels
+    // candidates first (the scratch for the two-pass ones is one block together with the output: the side stream has one block)
+    struct Cand { TilePick tp; int split; };
+    Cand cands[40]; int ncand = 0; size_t pmax = 0;
+    for (int sh = 0; sh < 4; sh++) {
+      if ((shapes[sh].bm == 128 && K < 128) || (shapes[sh].bn == 128 && CRS < 128) || (shapes[sh].bm == 32 && K > 32)) continue;
+      tp = shapes[sh];
+      tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
+      int cand[10]; int nc = 0;
+      auto add = [&](int v) { for (int i = 0; i < nc; i++) if (cand[i] == v) return; cand[nc++] = v; };
+      add(clamp_split((3 * (int64_t)g_num_cu) / tiles));
+      for (double t : targets) add(clamp_split((int64_t)(t * g_num_cu) / tiles));
+      for (int i = 0; i < nc && ncand < 40; i++) {
+        cands[ncand++] = Cand{tp, cand[i]};
+        const size_t pb = (size_t)slices_of(cand[i]) * sbytes;
+        if (slices_of(cand[i]) > 1 && pb <= pcap && pb > pmax) pmax = pb;
+      }
+    }
     bool tune_side = false;
-    float* scratch = (float*)scratch_take(sbytes, tune_side);
+    float* scratch = (float*)scratch_take(sbytes + pmax, tune_side);
     LaunchTimer timer;
     if (scratch && timer.ok) {
-      const double targets[] = {1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 5.0, 6.0};
-      const TilePick shapes[4] = {{128, 128}, {64, 128}, {64, 64}, {32, 128}};      // the last for layers of at most 32 output channels
-      float* const real_out = ep.C;
-      ep.C = scratch;
-      BwdfPlan best = {tp.bm, tp.bn, split}; float best_ms = 3.0e38f;
-      for (int sh = 0; sh < 4 && !failed(); sh++) {
-        if ((shapes[sh].bm == 128 && K < 128) || (shapes[sh].bn == 128 && CRS < 128) || (shapes[sh].bm == 32 && K > 32)) continue;
-        tp = shapes[sh];
+      float* const pbuf = scratch + (size_t)K * CRS;
+      BwdfPlan best = {tp.bm, tp.bn, split, 0}; float best_ms = 3.0e38f;
+      for (int ci = 0; ci < ncand && !failed(); ci++) {
+        tp = cands[ci].tp; split = cands[ci].split;
         tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
-        int cand[10]; int nc = 0;
-        auto add = [&](int v) { for (int i = 0; i < nc; i++) if (cand[i] == v) return; cand[nc++] = v; };
-        add(clamp_split((3 * (int64_t)g_num_cu) / tiles));
-        for (double t : targets) add(clamp_split((int64_t)(t * g_num_cu) / tiles));
-        for (int i = 0; i < nc && !failed(); i++) {
-          split = cand[i];
-          const float ms_min = timer.ms([&]() { dispatch(); return ok; });
-          if (ms_min < 0.f) break;
-          if (ms_min < best_ms) { best_ms = ms_min; best = BwdfPlan{tp.bm, tp.bn, cand[i]}; }
+        const int sl = slices_of(split);
+        if (!g_deterministic || sl == 1) {
+          const float ms_atomic = timer.ms([&]() { run_plan(scratch, nullptr, 1.f); return ok; });
+          if (ms_atomic < 0.f) break;
+          if (ms_atomic < best_ms) { best_ms = ms_atomic; best = BwdfPlan{tp.bm, tp.bn, split, 0}; }
+        }
+        if (sl > 1 && (size_t)sl * sbytes <= pmax) {
+          const float ms_two = timer.ms([&]() { run_plan(scratch, pbuf, 1.f); return ok; });
+          if (ms_two < 0.f) break;
+          if (ms_two < best_ms * 0.98f) { best_ms = ms_two; best = BwdfPlan{tp.bm, tp.bn, split, 1}; }
         }
       }
-      ep.C = real_out;
       tp = TilePick{best.bm, best.bn};
       tiles = cdiv(K, tp.bm) * cdiv(CRS, tp.bn);
-      split = best.split;
+      split = best.split; twopass = best.twopass != 0;
       g_bwdf_split[key] = best; g_plans_measured++;
-      if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: tile %dx%d, %lld tiles, split %d (%.3f ms)\n", N, C, H, K, R, sH, tp.bm, tp.bn, (long long)tiles, split, best_ms);
+      if (getenv("LH_TUNE_VERBOSE")) fprintf(stderr, "bwd_filter N%d C%d H%d K%d k%d s%d: tile %dx%d, %lld tiles, split %d%s (%.3f ms)\n", N, C, H, K, R, sH, tp.bm, tp.bn, (long long)tiles, split, twopass ? ", two passes" : "", best_ms);
     }
-    if (scratch) scratch_give(sbytes, tune_side);
+    if (scratch) scratch_give(sbytes + pmax, tune_side);
     if (failed()) return;
   }
-  dispatch();
-  if (partial) {
-    if (ok) reduce_slices(dw, CRS, K, CRS, partial, slices, beta);
-    scratch_give(partial_bytes, on_side);
+  slices = slices_of(split);
+  if (g_deterministic) twopass = true;
+  if (twopass && slices > 1) {
+    partial_bytes = (size_t)slices * K * CRS * sizeof(float);
+    partial = (float*)scratch_take(partial_bytes, on_side);
+    if (partial == nullptr) return;
   }
+  if (beta == 0.f && partial == nullptr) lh_fill(dw, 0.f, (int64_t)K * CRS);
+  run_plan(dw, partial, beta);
+  if (partial) scratch_give(partial_bytes, on_side);
   if (!ok) return;
   if (db && !bias_done) bias_grad_launch(nullptr, const_cast<float*>(dy), db, N, K, PQ);
   LH_CHECK_LAUNCH();
