@@ -18,6 +18,7 @@ void persistent_free(void* p);
 bool side_work_begin();                    // library-internal fork: the side stream waits for the main stream and becomes current; false: not now
 void side_work_end();
 void build_filter_layout(int kind, const int* prm, const float* w, float* dst);      // lh_conv.hip: the copy kernel of a layout, on the current stream
+void build_filter_layouts(int n, const int* kinds, const int* const* prms, const float* const* ws, float* const* dsts);      // the same for n layouts, batched into few launches
 int* fix_counters();                       // FIX_MAX_TILES zeroed ints in device memory (lh_setup): the arrival counters of igemm_launch_shared_tail, left zero by every launch
 void* side_scratch(size_t bytes); // a block for the kernels of the side stream (one user at a time, in that stream's order); nullptr after a reported failure
 // Scratch memory for a launch: the top of the arena on the main stream (stream order puts the next user of the same memory

@@ -298,6 +298,45 @@ static EpiConvOut make_epi(float* out, const float* bias, int chan, int Himg, in
   return ep;
 }
 
+// Several filter layouts in one launch (the copies of all of a network's filters, made again after an optimizer step: dozens of
+// tensors of a few KB to a few MB each, whose one-launch-per-copy form is bound by the launches).  Job j owns blocks
+// [start[j], start[j+1]); its parameters are those of build_filter_layout.
+constexpr int LAYOUT_BATCH = 40;
+struct LayoutJobs {
+  const float* w[LAYOUT_BATCH]; float* dst[LAYOUT_BATCH];
+  int kind[LAYOUT_BATCH]; int prm[LAYOUT_BATCH][LAYOUT_PRM];
+  int start[LAYOUT_BATCH + 1]; int njobs;
+};
+static_assert(sizeof(LayoutJobs) <= 4096, "kernel arguments are limited to 4 KB");
+__global__ void __launch_bounds__(TPB) k_filter_layouts(const LayoutJobs jobs) {
+  int j = 0;
+  while (j + 1 < jobs.njobs && (int)blockIdx.x >= jobs.start[j + 1]) j++;
+  const float* __restrict__ w = jobs.w[j]; float* __restrict__ wt = jobs.dst[j];
+  const int* p = jobs.prm[j];
+  const int kind = jobs.kind[j];
+  int64_t i = (int64_t)((int)blockIdx.x - jobs.start[j]) * TPB + threadIdx.x;
+  const int64_t st = (int64_t)(jobs.start[j + 1] - jobs.start[j]) * TPB;
+  if (kind == LAYOUT_KRSC) {
+    const int C = p[1], RS = p[2]; const int64_t n = (int64_t)p[0] * C * RS;
+    for (; i < n; i += st) {
+      int c = (int)(i % C); int64_t t = i / C; int rs = (int)(t % RS); int64_t k = t / RS;
+      wt[i] = w[(k * C + c) * RS + rs];
+    }
+  } else if (kind == LAYOUT_CTK) {
+    const int K = p[0], C = p[1], R = p[2], S = p[3], r0 = p[4], s0 = p[5], sH = p[6], sW = p[7], Rc = p[8], Sc = p[9];
+    const int64_t n = (int64_t)Rc * Sc * K * C;
+    for (; i < n; i += st) {
+      int k = (int)(i % K); int64_t t = i / K; int ts = (int)(t % Sc); t /= Sc; int tr = (int)(t % Rc); int c = (int)(t / Rc);
+      wt[i] = w[(((int64_t)k * C + c) * R + (r0 + sH * tr)) * S + (s0 + sW * ts)];
+    }
+  } else {
+    const int K = p[0], C = p[1], RS = p[2]; const int64_t n = (int64_t)K * C * RS;
+    for (; i < n; i += st) {
+      int rs = (int)(i % RS); int64_t t = i / RS; int k = (int)(t % K); int c = (int)(t / K);
+      wt[i] = w[((int64_t)k * C + c) * RS + rs];
+    }
+  }
+}
 // w[K][C][RS] -> wt[K][RS][C]   (forward, tap-major reduction order)
 __global__ void __launch_bounds__(TPB) k_filter_to_krsc(const float* __restrict__ w, float* __restrict__ wt, int C, int RS, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x, st = (int64_t)gridDim.x * TPB;
@@ -387,6 +426,23 @@ void build_filter_layout(int kind, const int* p, const float* w, float* dst) {
   } else {                                   // LAYOUT_CKRS {K, C, RS}
     const int64_t n = (int64_t)p[0] * p[1] * p[2];
     hipLaunchKernelGGL(k_filter_transpose, dim3(stream_grid(n, TPB * 4)), dim3(TPB), 0, g_stream, w, dst, p[0], p[1], p[2], n);
+  }
+}
+static int64_t layout_elems(int kind, const int* p) { return kind == LAYOUT_CTK ? (int64_t)p[8] * p[9] * p[0] * p[1] : (int64_t)p[0] * p[1] * p[2]; }
+// Several layouts at once, on the current stream: one launch per LAYOUT_BATCH of them.
+void build_filter_layouts(int n, const int* kinds, const int* const* prms, const float* const* ws, float* const* dsts) {
+  for (int first = 0; first < n; first += LAYOUT_BATCH) {
+    const int m = n - first < LAYOUT_BATCH ? n - first : LAYOUT_BATCH;
+    if (m == 1) { build_filter_layout(kinds[first], prms[first], ws[first], dsts[first]); continue; }
+    LayoutJobs jobs;
+    jobs.njobs = m; jobs.start[0] = 0;
+    for (int j = 0; j < m; j++) {
+      jobs.w[j] = ws[first + j]; jobs.dst[j] = dsts[first + j]; jobs.kind[j] = kinds[first + j];
+      for (int q = 0; q < LAYOUT_PRM; q++) jobs.prm[j][q] = prms[first + j][q];
+      jobs.start[j + 1] = jobs.start[j] + stream_grid(layout_elems(kinds[first + j], prms[first + j]), TPB * 4);
+    }
+    for (int j = m; j < LAYOUT_BATCH; j++) { jobs.w[j] = nullptr; jobs.dst[j] = nullptr; jobs.kind[j] = 0; for (int q = 0; q < LAYOUT_PRM; q++) jobs.prm[j][q] = 0; jobs.start[j + 1] = jobs.start[m]; }
+    hipLaunchKernelGGL(k_filter_layouts, dim3(jobs.start[m]), dim3(TPB), 0, g_stream, jobs);
   }
 }
 }  // namespace lh

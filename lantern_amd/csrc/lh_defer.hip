@@ -154,12 +154,14 @@ static void layouts_refresh() {
   int stale = 0;
   for (auto& l : g_layouts) stale += (l.used && !l.valid) ? 1 : 0;
   if (stale < g_layout_refresh_min || !side_work_begin()) return;
+  std::vector<int> kinds; std::vector<const int*> prms; std::vector<const float*> ws; std::vector<float*> dsts;
   for (auto& l : g_layouts) {
     if (!l.used || l.valid) continue;
-    build_filter_layout(l.kind, l.prm, (const float*)l.w, l.copy);
+    kinds.push_back(l.kind); prms.push_back(l.prm); ws.push_back((const float*)l.w); dsts.push_back(l.copy);
     layout_set(l, true);
     l.used = false;
   }
+  build_filter_layouts((int)kinds.size(), kinds.data(), prms.data(), ws.data(), dsts.data());
   side_work_end();
   g_layouts_on_side = true;
 }

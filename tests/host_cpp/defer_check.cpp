@@ -38,6 +38,7 @@ bool side_work_begin() { return true; }
 void side_work_end() {}
 // the simulated filter layout is a plain copy: a stale one still shows, because the values differ
 void build_filter_layout(int, const int*, const float* w, float* dst) { (void)ordered_stream(); memcpy(dst, w, 12 * sizeof(float)); g_layout_builds++; }
+void build_filter_layouts(int n, const int* kinds, const int* const* prms, const float* const* ws, float* const* dsts) { for (int i = 0; i < n; i++) build_filter_layout(kinds[i], prms[i], ws[i], dsts[i]); }
 static const float* sim_filter(const float* w) {
   bool build = false; const int prm[LAYOUT_PRM] = {4, 3, 1};
   float* c = lazy::layout_lookup(w, 12 * sizeof(float), LAYOUT_KRSC, prm, 12 * sizeof(float), build);
