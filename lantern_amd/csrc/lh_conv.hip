@@ -174,15 +174,21 @@ struct LoadConvBwdDataTapB {
 // VEC: PQ % 4 == 0 and dy 16-byte aligned (one 16-byte load per group of four reduction indices).
 // CARRY (PQ >= 4): the group's first index is decoded once and the other three follow by stepping with at most one carry
 // into the next sample, instead of one division each.
-template <bool VEC, bool CARRY = false>
+// PAD (maps whose P*Q is not a multiple of 4): the reduction runs over N * PQP indices, PQP = P*Q rounded up to a multiple of 4,
+// so that a group of four never crosses into the next sample and is one 16-byte load (4-byte aligned) again.  The indices
+// from P*Q to PQP - 1 of a sample stand for zeros: the last group of a sample, which has P*Q % 4 real elements, is loaded
+// from 4 - P*Q % 4 elements further down (inside the row) and moved up by the kernel (keep(), lh_keep_first), so nothing
+// outside the row is read.  dPQ divides by PQP; the other operand uses the same numbering.
+template <bool VEC, bool CARRY = false, bool PAD = false>
 struct LoadConvBwdFilterA {
   static constexpr bool ALONG_K = true;
-  static constexpr bool VEC4 = VEC;
+  static constexpr bool VEC4 = VEC || PAD;
   static constexpr bool SPLIT = false;
+  static constexpr bool MASKED = PAD;
   const float* base; uint32_t nbytes;
   int K, PQ;
   FastDiv dPQ;
-  static constexpr bool STEP = true;
+  static constexpr bool STEP = !PAD;
   // a slab that lies inside one sample is followed, inside that sample, by the same offsets bk elements further on
   __device__ __forceinline__ uint32_t step_bytes(int bk) const { return (uint32_t)bk * 4u; }
   __device__ __forceinline__ int run_slabs(int k, int bk) const {
@@ -192,6 +198,14 @@ struct LoadConvBwdFilterA {
   }
   struct State { int rowoff; bool valid; };
   __device__ __forceinline__ void init(State& s, int i, int nrows) const { s.valid = i < nrows; s.rowoff = (s.valid ? i : 0) * PQ; }
+  // PAD: the offset of the group's load and how many of its elements are real (the load starts 4 - keep elements early)
+  __device__ __forceinline__ uint32_t off_keep(const State& s, int kk, int kend, uint32_t& keep) const {
+    uint32_t n, pq;
+    dPQ.divmod(kk, n, pq);
+    const int left = PQ - (int)pq;
+    keep = (uint32_t)(left < 4 ? left : 4);
+    return (s.valid && kk < kend) ? (uint32_t)((int)n * K * PQ + s.rowoff + (int)pq - (4 - (int)keep)) * 4u : LH_OOB;
+  }
   __device__ __forceinline__ uint32_t off1(const State& s, int kk, int kend, int e) const {
     // VEC: the reduction length N*PQ is a multiple of 4 too, so the group at e == 0 is all in or all out
     uint32_t n, pq;
@@ -209,7 +223,8 @@ struct LoadConvBwdFilterA {
 // ---- B operand of the filter gradient: gather of x, reduction index (n, p, q) ------------------------------
 // column j = (c, r, s) fixed per thread.  MODE 1: Q % 4 == 0, the four reduction indices of a group share (n, p).
 // MODE 2 (Q >= 4): the group's first index is decoded once, the others step along the row with at most one carry
-// into the next row / sample.  MODE 0: one decode per index (maps narrower than 4).
+// into the next row / sample.  MODE 0: one decode per index (maps narrower than 4).  MODE 3: as MODE 2 over the padded
+// numbering of LoadConvBwdFilterA<.., PAD> (dPQ divides by PQP; a step past the last row is a padding index: zero).
 template <int MODE>
 struct LoadConvBwdFilterB {
   static constexpr bool ALONG_K = true;
@@ -229,12 +244,12 @@ struct LoadConvBwdFilterB {
     uint32_t n, pq, p, q;
     dPQ.divmod(MODE == 0 ? kk + e : kk, n, pq); dQ.divmod(pq, p, q);
     if (MODE != 0) q += (uint32_t)e;
-    if (MODE == 2 && q >= (uint32_t)Q) {
+    if ((MODE == 2 || MODE == 3) && q >= (uint32_t)Q) {
       q -= (uint32_t)Q; p += 1;
-      if (p >= (uint32_t)P) { p = 0; n += 1; }
+      if (MODE == 2 && p >= (uint32_t)P) { p = 0; n += 1; }
     }
     const int h = (int)p * sH + s.dh, w = (int)q * sW + s.dw;
-    const bool ok = s.valid && kk + e < kend && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
+    const bool ok = s.valid && kk + e < kend && (MODE != 3 || p < (uint32_t)P) && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
     return ok ? (uint32_t)((int)n * CHW + s.coff + h * W + w) * 4u : LH_OOB;
   }
 };
@@ -516,6 +531,8 @@ constexpr int N_PLANS = 16;
 static inline bool force_m32() { return getenv("LH_FORCE_M32") != nullptr; }
 // LH_FORCE_PLAN=n in the environment: forward / input-gradient products take launch plan n where it is valid (for tests that
 // compare the plans' results with each other).
+// LH_NO_PADDED_REDUCTION=1 (tests): the filter gradient over maps whose pixel count is not a multiple of 4 keeps to 4-byte loads
+static inline bool no_padded_reduction() { const char* e = getenv("LH_NO_PADDED_REDUCTION"); return e && e[0] == '1'; }
 static inline int force_plan() { const char* e = getenv("LH_FORCE_PLAN"); return e ? atoi(e) : -1; }
 // LH_FORCE_STATS_TILE=f: the same for the forward launches that leave batch-norm statistics behind (f as in conv_fwd_impl's `run`).
 static inline int force_stats_tile() { const char* e = getenv("LH_FORCE_STATS_TILE"); return e ? atoi(e) : -1; }
@@ -1022,7 +1039,12 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   // A filter gradient issued in line must not overtake one of the same filter that is still on the side stream.
   if (g_stream_cur == g_stream_raw) side_join();
   const int CRS = C * R * S, PQ = d.P * d.Q;
-  const int64_t red = (int64_t)N * PQ;
+  // Maps whose P*Q is not a multiple of 4 (7x7, 9x9, 81x185 ...): the reduction is numbered with every sample padded to a
+  // multiple of 4, which keeps dy (and x under a 1x1 filter) on 16-byte loads (LoadConvBwdFilterA<.., PAD>); for maps of
+  // 32 pixels and more, where the padding is at most a tenth of the reduction.
+  const int PQP = (PQ + 3) & ~3;
+  const bool padded = PQ % 4 != 0 && PQ >= 32 && d.Q >= 4 && !no_padded_reduction();
+  const int64_t red = (int64_t)N * (padded ? PQP : PQ);
   LH_REQUIRE(red < 0x7fffffffLL, "lh_conv2d_bwd_filter: reduction length too large");
   const bool avec = (PQ % 4 == 0) && (((uintptr_t)dy & 15) == 0);
   const bool rowvec = (d.Q % 4 == 0);
@@ -1059,9 +1081,9 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   EpiRowMajor ep; ep.C = dw; ep.ldc = CRS; ep.alpha = 1.f; ep.beta = 1.f; ep.atomic = split > 1 ? 1 : 0;
   bool ok = false;
   auto go = [&](auto al, auto bl) {
-    al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
+    al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(padded ? PQP : PQ);
     bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * H * W * 4); bl.C = C; bl.H = H; bl.W = W; bl.sH = sH; bl.sW = sW; bl.pH = pH; bl.pW = pW; bl.CHW = C * H * W;
-    bl.P = d.P; bl.Q = d.Q; bl.dPQ.init(PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
+    bl.P = d.P; bl.Q = d.Q; bl.dPQ.init(padded ? PQP : PQ); bl.dQ.init(d.Q); bl.dRS.init(R * S); bl.dS.init(S);
     if (tp.bm == 128) ok = igemm_launch<128, 128, 16>(al, bl, ep, K, CRS, (int)red, split);    // measured: the large tile prefers the short slab
     else if (tp.bm == 32) ok = igemm_launch<32, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
     else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
@@ -1069,8 +1091,8 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   };
   // 1x1, stride 1, no padding: the gather of x is a plain [C][N*PQ] matrix with the same layout as dy
   auto go_plain = [&](auto al, auto bl) {
-    al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(PQ);
-    bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * PQ * 4); bl.K = C; bl.PQ = PQ; bl.dPQ.init(PQ);
+    al.base = dy; al.nbytes = (uint32_t)((size_t)N * K * PQ * 4); al.K = K; al.PQ = PQ; al.dPQ.init(padded ? PQP : PQ);
+    bl.base = x; bl.nbytes = (uint32_t)((size_t)N * C * PQ * 4); bl.K = C; bl.PQ = PQ; bl.dPQ.init(padded ? PQP : PQ);
     if (tp.bm == 128) ok = igemm_launch<128, 128, 16>(al, bl, ep, K, CRS, (int)red, split);
     else if (tp.bm == 32) ok = igemm_launch<32, 128, 32>(al, bl, ep, K, CRS, (int)red, split);
     else if (tp.bn == 128) ok = igemm_launch<64, 128, BWDF_BK>(al, bl, ep, K, CRS, (int)red, split);
@@ -1081,7 +1103,9 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   const bool narrow = PQ < 4 || d.Q < 4;        // the stepping loaders assume at most one carry inside a group of four
   auto dispatch = [&]() {
     ep.atomic = (split > 1 && ep.sliceStride == 0) ? 1 : 0;
-    if (plain && avec && xvec) go_plain(LoadConvBwdFilterA<true>(), LoadConvBwdFilterA<true>());
+    if (padded && plain) go_plain(LoadConvBwdFilterA<false, false, true>(), LoadConvBwdFilterA<false, false, true>());
+    else if (padded) go(LoadConvBwdFilterA<false, false, true>(), LoadConvBwdFilterB<3>());
+    else if (plain && avec && xvec) go_plain(LoadConvBwdFilterA<true>(), LoadConvBwdFilterA<true>());
     else if (plain && !avec && !xvec && !narrow) go_plain(LoadConvBwdFilterA<false, true>(), LoadConvBwdFilterA<false, true>());
     else if (plain && !avec && !xvec) go_plain(LoadConvBwdFilterA<false>(), LoadConvBwdFilterA<false>());
     else if (narrow) { if (avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterB<0>()); else go(LoadConvBwdFilterA<false>(), LoadConvBwdFilterB<0>()); }

@@ -105,6 +105,19 @@ struct LoadPlainT {
 template <class L, class = void> struct LhCanStep { static constexpr bool value = false; };
 template <class L> struct LhCanStep<L, typename std::enable_if<L::STEP>::type> { static constexpr bool value = true; };
 
+// A MASKED loader (VEC4) loads a group whose first `keep` elements are real from 4 - keep elements before the group's
+// place: off_keep() gives offset and keep, and the loaded vector is moved up and filled with zeros before it goes to LDS.
+template <class L, class = void> struct LhMasked { static constexpr bool value = false; };
+template <class L> struct LhMasked<L, typename std::enable_if<L::MASKED>::type> { static constexpr bool value = true; };
+__device__ __forceinline__ float4 lh_keep_first(const float4 v, uint32_t keep) {
+  float4 r;
+  r.x = keep >= 4 ? v.x : (keep == 3 ? v.y : (keep == 2 ? v.z : v.w));
+  r.y = keep >= 4 ? v.y : (keep == 3 ? v.z : (keep == 2 ? v.w : 0.f));
+  r.z = keep >= 4 ? v.z : (keep == 3 ? v.w : 0.f);
+  r.w = keep >= 4 ? v.w : 0.f;
+  return r;
+}
+
 // Offsets of one group of four k (one offset when the loader is VEC4).  A SPLIT loader gives one
 // per-lane byte offset for the group (o[0], LH_OOB when the group is out of range for this lane)
 // plus four wave-uniform byte offsets s[i] that go into the scalar-offset operand of the load.
@@ -292,6 +305,7 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   constexpr int NEL = GA * EA + GB * EB;            // offsets to compute per slab and thread
   constexpr int NM_PAIR = 4 * MI * NI, NM = (KQ / 2) * NM_PAIR;
   float4 ra0[GA], rb0[GB], ra1[GA], rb1[GB];
+  uint32_t ka0[GA], kb0[GB], ka1[GA], kb1[GB];
   LhOff<AL> oa[GA];
   LhOff<BL> ob[GB];
   LhScal ua[GA], ub[GB];
@@ -300,10 +314,12 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
     if (e < GA * EA) {
       const int g = e / EA, i = e % EA, k = k0 + 4 * a_kq[g];
       if constexpr (AL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) oa[g].o[0] = al.voff(sa[g], ku, kend); ua[g].s[i] = al.soff(ku, i); }      // (a SPLIT loader's k is the same in all lanes: its groups run along the columns)
+      else if constexpr (LhMasked<AL>::value) oa[g].o[0] = al.off_keep(sa[g], k, kend, oa[g].o[1]);
       else oa[g].o[i] = al.off1(sa[g], k, kend, i);
     } else {
       const int f = e - GA * EA, g = f / EB, i = f % EB, k = k0 + 4 * b_kq[g];
       if constexpr (BL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) ob[g].o[0] = bl.voff(sb[g], ku, kend); ub[g].s[i] = bl.soff(ku, i); }
+      else if constexpr (LhMasked<BL>::value) ob[g].o[0] = bl.off_keep(sb[g], k, kend, ob[g].o[1]);
       else ob[g].o[i] = bl.off1(sb[g], k, kend, i);
     }
   };
@@ -311,7 +327,16 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   // be reached by stepping (whole slabs inside the reduction and inside the loaders' runs); the byte range of the buffer
   // descriptors (0 switches the loads of a slab past the end of the reduction off).
   int xsA = 0, xsB = 0, steps = 0, nrecA = (int)al.nbytes, nrecB = (int)bl.nbytes;
-  auto fetch = [&](float4 (&ra)[GA], float4 (&rb)[GB]) {
+  // (ka, kb: the keep counts of a MASKED loader's groups travel with the loaded registers until stash() applies them)
+  auto fetch = [&](float4 (&ra)[GA], float4 (&rb)[GB], uint32_t (&ka)[GA], uint32_t (&kb)[GB]) {
+    if constexpr (LhMasked<AL>::value) {
+#pragma unroll
+      for (int g = 0; g < GA; g++) ka[g] = oa[g].o[1];
+    }
+    if constexpr (LhMasked<BL>::value) {
+#pragma unroll
+      for (int g = 0; g < GB; g++) kb[g] = ob[g].o[1];
+    }
     if constexpr (STEPPED) {
       // (the byte ranges are the same in all lanes; said here because inside the segment loop of the stream-K forms the
       // compiler no longer sees it and wraps every load in a loop over the distinct descriptors of a wavefront)
@@ -351,12 +376,12 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
       else decode(kn);
     }
   };
-  auto stash = [&](const float4 (&ra)[GA], const float4 (&rb)[GB], int stage) {
+  auto stash = [&](const float4 (&ra)[GA], const float4 (&rb)[GB], const uint32_t (&ka)[GA], const uint32_t (&kb)[GB], int stage) {
     const int o = stage * KQ;
 #pragma unroll
-    for (int g = 0; g < GA; g++) As[(o + a_kq[g]) * LDA + a_col[g]] = ra[g];
+    for (int g = 0; g < GA; g++) As[(o + a_kq[g]) * LDA + a_col[g]] = LhMasked<AL>::value ? lh_keep_first(ra[g], ka[g]) : ra[g];
 #pragma unroll
-    for (int g = 0; g < GB; g++) Bs[(o + b_kq[g]) * LDB + b_col[g]] = rb[g];
+    for (int g = 0; g < GB; g++) Bs[(o + b_kq[g]) * LDB + b_col[g]] = LhMasked<BL>::value ? lh_keep_first(rb[g], kb[g]) : rb[g];
   };
 
   // Software pipeline over k-slabs (four slabs in flight):
@@ -369,28 +394,29 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   if constexpr (STEPPED) {
     nrecA = (int)al.nbytes; nrecB = (int)bl.nbytes;
     decode(kbeg);
-    fetch(ra0, rb0);
+    fetch(ra0, rb0, ka0, kb0);
     advance(kbeg + BK);
-    fetch(ra1, rb1);
+    fetch(ra1, rb1, ka1, kb1);
     advance(kbeg + 2 * BK);
   } else {
 #pragma unroll
     for (int e = 0; e < NEL; e++) elem(e, kbeg);
-    fetch(ra0, rb0);
+    fetch(ra0, rb0, ka0, kb0);
 #pragma unroll
     for (int e = 0; e < NEL; e++) elem(e, kbeg + BK);
-    fetch(ra1, rb1);
+    fetch(ra1, rb1, ka1, kb1);
 #pragma unroll
     for (int e = 0; e < NEL; e++) elem(e, kbeg + 2 * BK);
   }
-  stash(ra0, rb0, 0);
+  stash(ra0, rb0, ka0, kb0, 0);
   __syncthreads();
 
   // one iteration: compute slab `it` from LDS stage st, fetch slab it+2 into (rla, rlb), move slab
   // it+1 from (rsa, rsb) to LDS stage st^1
-  auto body = [&](int it, int st, float4 (&rla)[GA], float4 (&rlb)[GB], const float4 (&rsa)[GA], const float4 (&rsb)[GB]) {
+  auto body = [&](int it, int st, float4 (&rla)[GA], float4 (&rlb)[GB], uint32_t (&kla)[GA], uint32_t (&klb)[GB],
+                  const float4 (&rsa)[GA], const float4 (&rsb)[GB], const uint32_t (&ksa)[GA], const uint32_t (&ksb)[GB]) {
     const int k3 = kbeg + (it + 3) * BK;
-    fetch(rla, rlb);
+    fetch(rla, rlb, kla, klb);
     __builtin_amdgcn_sched_barrier(0);
     const float4* Asc = As + st * KQ * LDA + wm * TM + l32;
     const float4* Bsc = Bs + st * KQ * LDB + wn * TN + l32;
@@ -437,13 +463,13 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    stash(rsa, rsb, st ^ 1);
+    stash(rsa, rsb, ksa, ksb, st ^ 1);
     __syncthreads();
   };
   // the loop runs an even number of iterations: a trailing slab past kend is all zeros
   for (int it = 0; it < niter; it += 2) {
-    body(it, 0, ra0, rb0, ra1, rb1);
-    body(it + 1, 1, ra1, rb1, ra0, rb0);
+    body(it, 0, ra0, rb0, ka0, kb0, ra1, rb1, ka1, kb1);
+    body(it + 1, 1, ra1, rb1, ka1, kb1, ra0, rb0, ka0, kb0);
   }
 
   if constexpr (SK == 2) {

@@ -27,6 +27,10 @@ SHAPES = [
     (2, 96, 16, 16, 16, 1, 1, 1, 1, 0, 0),    # SqueezeNet squeeze (K = 16)
     (2, 512, 4, 4, 10, 4, 4, 1, 1, 0, 0),     # SqueezeNet head: 4x4 kernel onto 1x1
     (5, 256, 7, 7, 64, 1, 1, 1, 1, 0, 0),     # long reduction, 49-pixel maps
+    (3, 20, 9, 7, 24, 3, 3, 1, 1, 1, 1),      # 63-pixel maps: the last group of a sample has three real elements
+    (4, 64, 14, 14, 96, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2 onto 7x7 maps (gathered x, padded reduction numbering)
+    (2, 4, 21, 37, 32, 5, 3, 2, 1, 0, 1),     # 9x37 maps (333 pixels), 32 output channels: the 32-row tile
+    (3, 136, 7, 7, 130, 1, 1, 1, 1, 0, 0),    # 49-pixel maps, rows and columns just past one 128 tile
 ]
 
 
