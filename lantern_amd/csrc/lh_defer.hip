@@ -151,9 +151,12 @@ static void layouts_refresh() {
   // latency on both streams (LeNet's 0.26 ms step became 0.29 ms with its one copy made there, DeepSpeech2's 11.5 ms step
   // 12.8: its 1110 back-to-back step kernels are dispatched more slowly while the second queue is in use), which a handful
   // of 5 us copy kernels in the chain do not.  Networks with many filters to copy (8 or more) come out ahead.
+  // Fewer than that (or no second stream to use): two or more are still made in one launch, here on the main stream, instead of
+  // one launch each where they are next looked up.
   int stale = 0;
   for (auto& l : g_layouts) stale += (l.used && !l.valid) ? 1 : 0;
-  if (stale < g_layout_refresh_min || !side_work_begin()) return;
+  const bool side = stale >= g_layout_refresh_min && side_work_begin();
+  if (!side && (stale < 2 || g_rec_on || g_capturing || g_prof_mask != 0 || g_stream_cur != g_stream_raw)) return;
   std::vector<int> kinds; std::vector<const int*> prms; std::vector<const float*> ws; std::vector<float*> dsts;
   for (auto& l : g_layouts) {
     if (!l.used || l.valid) continue;
@@ -162,8 +165,7 @@ static void layouts_refresh() {
     l.used = false;
   }
   build_filter_layouts((int)kinds.size(), kinds.data(), prms.data(), ws.data(), dsts.data());
-  side_work_end();
-  g_layouts_on_side = true;
+  if (side) { side_work_end(); g_layouts_on_side = true; }
 }
 
 // ---- zero blocks ---------------------------------------------------------------------------------------------------
