@@ -316,7 +316,7 @@ static EpiConvOut make_epi(float* out, const float* bias, int chan, int Himg, in
 // Several filter layouts in one launch (the copies of all of a network's filters, made again after an optimizer step: dozens of
 // tensors of a few KB to a few MB each, whose one-launch-per-copy form is bound by the launches).  Job j owns blocks
 // [start[j], start[j+1]); its parameters are those of build_filter_layout.
-constexpr int LAYOUT_BATCH = 40;
+constexpr int LAYOUT_BATCH = 48;
 struct LayoutJobs {
   const float* w[LAYOUT_BATCH]; float* dst[LAYOUT_BATCH];
   int kind[LAYOUT_BATCH]; int prm[LAYOUT_BATCH][LAYOUT_PRM];
