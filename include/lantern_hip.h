@@ -257,12 +257,17 @@ void lh_axpy_dev(float* y, const float* h_or_d_scalar_on_device, const float* x,
 /* ---- conv2D_batch and its gradient (TD:292-296; CDN:515-880) ----------- */
 /* y[n,k,p,q] = bias[k] + sum_{c,r,s} x[n,c,p*sH-pH+r,q*sW-pW+s] * w[k,c,r,s]; bias may be NULL.
  * Launch plans are measured once per convolution shape on first use and remembered for the life of the process: the
- * filter gradient (tile shape and number of slices of its long reduction N*P*Q, timed on scratch memory) and, on calls
+ * filter gradient (tile shape, number of slices of its long reduction N*P*Q and how the slices are combined: atomic adds or a second
+ * summing kernel; timed on scratch memory) and, on calls
  * whose result overwrites its output, the forward and input-gradient products (tile shape, stream-K workers; a few timed
  * repetitions of the launch itself).  Products below 1e7 flop (LH_TUNE_MIN_FLOP) keep the built-in rule.  Environment:
  * LH_NO_TUNE=1 keeps the built-in rules everywhere, LH_TUNE_VERBOSE=1 prints each choice to stderr, LH_FORCE_M32=1 (a test
  * switch) sends every product of at most 32 rows to the 32-row tile whatever was measured, LH_FORCE_PLAN=n (a test switch) every forward /
- * input-gradient product to launch plan n where the shape allows it.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
+ * input-gradient product to launch plan n where the shape allows it, LH_FORCE_STATS_TILE=n (a test switch) every forward product that also leaves
+ * batch-norm statistics to tile plan n, LH_NO_PADDED_REDUCTION=1 (a test switch) the filter gradient over maps whose pixel count is not a multiple
+ * of 4 to 4-byte loads over the plain numbering of its reduction (by default samples are numbered with their pixel count rounded up to a multiple
+ * of 4, which keeps the loads 16 bytes wide; the sums then associate differently, within the usual rounding), LH_NO_SPLIT_GATHER=1 (a test switch)
+ * the filter gradient of unpadded filters with rows of 5 taps and more to the gather that decodes every element of x per lane.  lh_set_tuning(0) does the same as LH_NO_TUNE from inside the process (remembered plans stay
  * remembered and are used again after lh_set_tuning(1)). */
 void lh_set_tuning(int on);
 /* How many launch plans have been measured so far, and how many launches have used a remembered plan (either pointer may be

@@ -198,6 +198,7 @@ struct LoadConvBwdFilterA {
   }
   struct State { int rowoff; bool valid; };
   __device__ __forceinline__ void init(State& s, int i, int nrows) const { s.valid = i < nrows; s.rowoff = (s.valid ? i : 0) * PQ; }
+  static __device__ __forceinline__ float4 fix(const float4 v, uint32_t keep) { return lh_keep_first(v, keep); }
   // PAD: the offset of the group's load and how many of its elements are real (the load starts 4 - keep elements early)
   __device__ __forceinline__ uint32_t off_keep(const State& s, int kk, int kend, uint32_t& keep) const {
     uint32_t n, pq;
@@ -251,6 +252,64 @@ struct LoadConvBwdFilterB {
     const int h = (int)p * sH + s.dh, w = (int)q * sW + s.dw;
     const bool ok = s.valid && kk + e < kend && (MODE != 3 || p < (uint32_t)P) && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W;
     return ok ? (uint32_t)((int)n * CHW + s.coff + h * W + w) * 4u : LH_OOB;
+  }
+};
+
+// ---- B operand of the filter gradient, lanes along the columns: filters without padding whose rows are 5 taps and wider ----
+// Column j = (c, r, s) is fixed per lane and contributes c*H*W + r*W + s; the reduction index (n, p, q) is the same in all lanes
+// of a wavefront and contributes n*C*H*W + p*sH*W + q*sW, decoded on the scalar unit into the scalar-offset operand of the load:
+// no per-lane arithmetic per element at all (LoadConvBwdFilterB decodes and bounds-checks every element in vector registers,
+// which is what bounds the filter gradient of a 21x11 filter).  A wavefront's load covers 64 consecutive (c, r, s): runs of S
+// consecutive floats.  Without padding every tap of every output pixel lies inside the image, so there is nothing to check.
+// PADNUM: the padded numbering of LoadConvBwdFilterA<.., PAD> (dPQ divides by PQP; indices from P*Q on are zeros).
+// The elements of a group that lie past the end of the slice or are padding indices are cleared on the way to LDS (keep, fix);
+// their scalar offsets are 0, so what is loaded for them is inside the tensor.
+template <bool PADNUM>
+struct LoadConvBwdFilterSplitB {
+  static constexpr bool ALONG_K = false;
+  static constexpr bool VEC4 = false;
+  static constexpr bool SPLIT = true;
+  static constexpr bool STEP = false;
+  static constexpr bool MASKED = true;
+  const float* base; uint32_t nbytes;
+  int C, H, W, sH, sW, pH, pW, CHW, P, Q;
+  FastDiv dPQ, dQ, dRS, dS;
+  struct State { int off; bool valid; };
+  __device__ __forceinline__ void init(State& s, int j, int ncols) const {
+    s.valid = j < ncols;
+    uint32_t c, rs, r, ss;
+    dRS.divmod(s.valid ? j : 0, c, rs); dS.divmod(rs, r, ss);
+    s.off = (int)c * H * W + (int)r * W + (int)ss;
+  }
+  __device__ __forceinline__ uint32_t voff(const State& s, int k, int kend) const { return (s.valid && k < kend) ? (uint32_t)s.off * 4u : LH_OOB; }
+  __device__ __forceinline__ uint32_t keep(int k, int kend) const {
+    int left = kend - k;
+    if (PADNUM) { uint32_t n, pq; dPQ.divmod(k, n, pq); const int real = P * Q - (int)pq; left = left < real ? left : real; }
+    return (uint32_t)(left < 0 ? 0 : (left > 4 ? 4 : left));
+  }
+  // the four scalar offsets of the group at k (all scalar arithmetic): one decode, then steps along the row with the carries
+  __device__ __forceinline__ void soff4(int k, int kend, uint32_t (&so)[4]) const {
+    uint32_t n, pq, p, q;
+    dPQ.divmod(k, n, pq); dQ.divmod(pq, p, q);          // (with PADNUM a group starts on a real index: P*Q is not a multiple of 4)
+    int off = (int)n * CHW + (int)p * sH * W + (int)q * sW;
+    bool real = true;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      so[e] = (real && k + e < kend) ? (uint32_t)off * 4u : 0u;
+      q += 1; off += sW;
+      if ((int)q == Q) {
+        q = 0; p += 1; off += sH * W - Q * sW;
+        if ((int)p == P) {
+          if (PADNUM) real = false;                       // what is left of the group are padding indices
+          else { p = 0; n += 1; off = (int)n * CHW; }
+        }
+      }
+    }
+  }
+  static __device__ __forceinline__ float4 fix(const float4 v, uint32_t keep) {
+    float4 r;
+    r.x = keep > 0 ? v.x : 0.f; r.y = keep > 1 ? v.y : 0.f; r.z = keep > 2 ? v.z : 0.f; r.w = keep > 3 ? v.w : 0.f;
+    return r;
   }
 };
 
@@ -533,6 +592,8 @@ static inline bool force_m32() { return getenv("LH_FORCE_M32") != nullptr; }
 // compare the plans' results with each other).
 // LH_NO_PADDED_REDUCTION=1 (tests): the filter gradient over maps whose pixel count is not a multiple of 4 keeps to 4-byte loads
 static inline bool no_padded_reduction() { const char* e = getenv("LH_NO_PADDED_REDUCTION"); return e && e[0] == '1'; }
+// LH_NO_SPLIT_GATHER=1 (tests): the filter gradient of unpadded filters with wide rows keeps to the per-element gather of x
+static inline bool no_split_gather() { const char* e = getenv("LH_NO_SPLIT_GATHER"); return e && e[0] == '1'; }
 static inline int force_plan() { const char* e = getenv("LH_FORCE_PLAN"); return e ? atoi(e) : -1; }
 // LH_FORCE_STATS_TILE=f: the same for the forward launches that leave batch-norm statistics behind (f as in conv_fwd_impl's `run`).
 static inline int force_stats_tile() { const char* e = getenv("LH_FORCE_STATS_TILE"); return e ? atoi(e) : -1; }
@@ -1101,9 +1162,13 @@ void lh_conv2d_bwd_filter(const float* x, const float* dy, float* dw, float* db,
   const bool plain = R == 1 && S == 1 && sH == 1 && sW == 1 && pH == 0 && pW == 0;
   const bool xvec = (PQ % 4 == 0) && (((uintptr_t)x & 15) == 0);
   const bool narrow = PQ < 4 || d.Q < 4;        // the stepping loaders assume at most one carry inside a group of four
+  // filters without padding whose rows are 5 taps and wider: x is gathered with the lanes along (c, r, s) (LoadConvBwdFilterSplitB)
+  const bool wide_rows = pH == 0 && pW == 0 && S >= 5 && !no_split_gather();
   auto dispatch = [&]() {
     ep.atomic = (split > 1 && ep.sliceStride == 0) ? 1 : 0;
-    if (padded && plain) go_plain(LoadConvBwdFilterA<false, false, true>(), LoadConvBwdFilterA<false, false, true>());
+    if (wide_rows && padded) go(LoadConvBwdFilterA<false, false, true>(), LoadConvBwdFilterSplitB<true>());
+    else if (wide_rows && avec) go(LoadConvBwdFilterA<true>(), LoadConvBwdFilterSplitB<false>());
+    else if (padded && plain) go_plain(LoadConvBwdFilterA<false, false, true>(), LoadConvBwdFilterA<false, false, true>());
     else if (padded) go(LoadConvBwdFilterA<false, false, true>(), LoadConvBwdFilterB<3>());
     else if (plain && avec && xvec) go_plain(LoadConvBwdFilterA<true>(), LoadConvBwdFilterA<true>());
     else if (plain && !avec && !xvec && !narrow) go_plain(LoadConvBwdFilterA<false, true>(), LoadConvBwdFilterA<false, true>());

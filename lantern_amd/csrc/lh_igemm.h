@@ -105,8 +105,10 @@ struct LoadPlainT {
 template <class L, class = void> struct LhCanStep { static constexpr bool value = false; };
 template <class L> struct LhCanStep<L, typename std::enable_if<L::STEP>::type> { static constexpr bool value = true; };
 
-// A MASKED loader (VEC4) loads a group whose first `keep` elements are real from 4 - keep elements before the group's
-// place: off_keep() gives offset and keep, and the loaded vector is moved up and filled with zeros before it goes to LDS.
+// A MASKED loader says of every group how many of its elements are real (`keep`); the loaded vector passes through the loader's
+// fix(v, keep) before it goes to LDS.  VEC4 form (off_keep() gives offset and keep): the group is loaded from 4 - keep elements
+// before its place, fix() moves it up and fills with zeros (lh_keep_first).  SPLIT form (voff, keep, soff4): fix() clears the
+// elements from `keep` on.
 template <class L, class = void> struct LhMasked { static constexpr bool value = false; };
 template <class L> struct LhMasked<L, typename std::enable_if<L::MASKED>::type> { static constexpr bool value = true; };
 __device__ __forceinline__ float4 lh_keep_first(const float4 v, uint32_t keep) {
@@ -116,6 +118,12 @@ __device__ __forceinline__ float4 lh_keep_first(const float4 v, uint32_t keep) {
   r.z = keep >= 4 ? v.z : (keep == 3 ? v.w : 0.f);
   r.w = keep >= 4 ? v.w : 0.f;
   return r;
+}
+
+template <class L>
+__device__ __forceinline__ float4 lh_fix_group(const float4 v, uint32_t keep) {
+  if constexpr (LhMasked<L>::value) return L::fix(v, keep);
+  else return v;
 }
 
 // Offsets of one group of four k (one offset when the loader is VEC4).  A SPLIT loader gives one
@@ -313,12 +321,14 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   auto elem = [&](int e, int k0) {
     if (e < GA * EA) {
       const int g = e / EA, i = e % EA, k = k0 + 4 * a_kq[g];
-      if constexpr (AL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) oa[g].o[0] = al.voff(sa[g], ku, kend); ua[g].s[i] = al.soff(ku, i); }      // (a SPLIT loader's k is the same in all lanes: its groups run along the columns)
+      if constexpr (AL::SPLIT && LhMasked<AL>::value) { if (i == 0) { const int ku = __builtin_amdgcn_readfirstlane(k); oa[g].o[0] = al.voff(sa[g], ku, kend); oa[g].o[1] = al.keep(ku, kend); al.soff4(ku, kend, ua[g].s); } }
+      else if constexpr (AL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) oa[g].o[0] = al.voff(sa[g], ku, kend); ua[g].s[i] = al.soff(ku, i); }      // (a SPLIT loader's k is the same in all lanes: its groups run along the columns)
       else if constexpr (LhMasked<AL>::value) oa[g].o[0] = al.off_keep(sa[g], k, kend, oa[g].o[1]);
       else oa[g].o[i] = al.off1(sa[g], k, kend, i);
     } else {
       const int f = e - GA * EA, g = f / EB, i = f % EB, k = k0 + 4 * b_kq[g];
-      if constexpr (BL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) ob[g].o[0] = bl.voff(sb[g], ku, kend); ub[g].s[i] = bl.soff(ku, i); }
+      if constexpr (BL::SPLIT && LhMasked<BL>::value) { if (i == 0) { const int ku = __builtin_amdgcn_readfirstlane(k); ob[g].o[0] = bl.voff(sb[g], ku, kend); ob[g].o[1] = bl.keep(ku, kend); bl.soff4(ku, kend, ub[g].s); } }
+      else if constexpr (BL::SPLIT) { const int ku = __builtin_amdgcn_readfirstlane(k); if (i == 0) ob[g].o[0] = bl.voff(sb[g], ku, kend); ub[g].s[i] = bl.soff(ku, i); }
       else if constexpr (LhMasked<BL>::value) ob[g].o[0] = bl.off_keep(sb[g], k, kend, ob[g].o[1]);
       else ob[g].o[i] = bl.off1(sb[g], k, kend, i);
     }
@@ -379,9 +389,9 @@ __device__ __forceinline__ void igemm_block(const AL& al, const BL& bl, const EP
   auto stash = [&](const float4 (&ra)[GA], const float4 (&rb)[GB], const uint32_t (&ka)[GA], const uint32_t (&kb)[GB], int stage) {
     const int o = stage * KQ;
 #pragma unroll
-    for (int g = 0; g < GA; g++) As[(o + a_kq[g]) * LDA + a_col[g]] = LhMasked<AL>::value ? lh_keep_first(ra[g], ka[g]) : ra[g];
+    for (int g = 0; g < GA; g++) As[(o + a_kq[g]) * LDA + a_col[g]] = lh_fix_group<AL>(ra[g], ka[g]);
 #pragma unroll
-    for (int g = 0; g < GB; g++) Bs[(o + b_kq[g]) * LDB + b_col[g]] = LhMasked<BL>::value ? lh_keep_first(rb[g], kb[g]) : rb[g];
+    for (int g = 0; g < GB; g++) Bs[(o + b_kq[g]) * LDB + b_col[g]] = lh_fix_group<BL>(rb[g], kb[g]);
   };
 
   // Software pipeline over k-slabs (four slabs in flight):

@@ -31,6 +31,9 @@ SHAPES = [
     (4, 64, 14, 14, 96, 1, 1, 2, 2, 0, 0),    # 1x1 stride 2 onto 7x7 maps (gathered x, padded reduction numbering)
     (2, 4, 21, 37, 32, 5, 3, 2, 1, 0, 1),     # 9x37 maps (333 pixels), 32 output channels: the 32-row tile
     (3, 136, 7, 7, 130, 1, 1, 1, 1, 0, 0),    # 49-pixel maps, rows and columns just past one 128 tile
+    (2, 3, 13, 15, 12, 5, 5, 1, 1, 0, 0),     # no padding, 5-wide filter rows (x gathered with the lanes along (c, r, s)), 99-pixel maps
+    (2, 2, 31, 24, 32, 7, 6, 2, 1, 0, 0),     # the same with anisotropic stride, 247-pixel maps and the 32-row tile
+    (2, 6, 30, 24, 40, 9, 5, 2, 1, 0, 0),     # the same over maps of 220 pixels (a multiple of 4)
 ]
 
 
@@ -235,6 +238,24 @@ def test_conv_deterministic_mode(on_hip, dims):
     finally:
         on_hip.setDeterministic(False)
     assert dev.lib.lh_get_deterministic() == 0
+
+
+@pytest.mark.parametrize("dims", [(5, 256, 7, 7, 64, 1, 1, 1, 1, 0, 0), (4, 16, 7, 7, 24, 3, 3, 1, 1, 1, 1), (2, 4, 21, 37, 32, 5, 3, 2, 1, 0, 1)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_filter_gradient_without_the_padded_reduction(on_hip, dims, monkeypatch):
+    """Maps whose pixel count is not a multiple of 4: LH_NO_PADDED_REDUCTION=1 keeps the filter gradient on the 4-byte loads over the
+    plain numbering of the reduction; both forms (the default one runs in test_conv_fwd_bwd) match the oracle."""
+    monkeypatch.setenv("LH_NO_PADDED_REDUCTION", "1")
+    check_conv(Dev(on_hip), dims, bias=True)
+
+
+@pytest.mark.parametrize("dims", [(3, 10, 12, 12, 20, 5, 5, 1, 1, 0, 0), (2, 3, 13, 15, 12, 5, 5, 1, 1, 0, 0), (1, 1, 41, 30, 8, 11, 5, 2, 2, 0, 0)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_filter_gradient_of_unpadded_wide_filters_with_the_per_element_gather(on_hip, dims, monkeypatch):
+    """LH_NO_SPLIT_GATHER=1 keeps the filter gradient of unpadded filters with rows of 5 taps and more on the loader that decodes every
+    element of x per lane; both forms (the default one runs in test_conv_fwd_bwd) match the oracle."""
+    monkeypatch.setenv("LH_NO_SPLIT_GATHER", "1")
+    check_conv(Dev(on_hip), dims, bias=True)
 
 
 @pytest.mark.parametrize("dims", [(8, 64, 28, 28, 128, 3, 3, 1, 1, 1, 1), (4, 256, 14, 14, 256, 1, 1, 1, 1, 0, 0), (6, 96, 15, 15, 160, 3, 3, 1, 1, 1, 1),
