@@ -40,6 +40,36 @@ def test_random_conv_geometries(on_hip, group):
         on_hip.sync(); on_hip.resetMallocAddr(mark)
 
 
+def _conv_case_for_the_filter_gradient_loaders(rng, wide):
+    """Maps of up to 39 x 39 pixels (odd pixel counts of 32 and more take the padded numbering of the filter gradient's reduction);
+    wide: no padding and filter rows of 5 to 11 taps (x gathered with the lanes along the columns)."""
+    if wide:
+        R = int(rng.choice([1, 2, 3, 5, 9])); S = int(rng.choice([5, 6, 7, 11])); sH, sW = int(rng.choice([1, 2, 3])), int(rng.choice([1, 1, 2])); pH = pW = 0
+    else:
+        R = int(rng.choice([1, 3, 5])); S = int(rng.choice([1, 3, 5])); sH, sW = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
+        pH, pW = int(rng.randint(0, R)), int(rng.randint(0, S))
+    H = int(rng.randint(max(1, R - 2 * pH) + 3, 40)); W = int(rng.randint(max(1, S - 2 * pW) + 3, 40))
+    N = int(rng.choice([1, 2, 3, 5, 8, 16])); Cc = int(rng.choice([1, 2, 3, 4, 7, 16, 17, 32, 40, 64])); K = int(rng.choice([1, 5, 8, 16, 24, 32, 33, 64, 70, 130]))
+    return (N, Cc, H, W, K, R, S, sH, sW, pH, pW)
+
+
+@pytest.mark.parametrize("group", range(4))
+def test_random_conv_geometries_odd_maps_and_unpadded_wide_filters(on_hip, group):
+    dev = Dev(on_hip)
+    rng = np.random.RandomState(4000 + group)
+    for i in range(8):
+        dims = _conv_case_for_the_filter_gradient_loaders(rng, wide=bool(i & 1)); bias = bool(rng.rand() < 0.5)
+        det = group == 3                     # the last group in deterministic mode (slices of the reduction added up by a second kernel)
+        _say("conv (filter-gradient loaders) group %d case %d dims %s bias %s deterministic %s" % (group, i, dims, bias, det))
+        mark = on_hip.getMallocAddr()
+        if det: on_hip.setDeterministic(True)
+        try:
+            check_conv(dev, dims, bias)
+        finally:
+            if det: on_hip.setDeterministic(False)
+        on_hip.sync(); on_hip.resetMallocAddr(mark)
+
+
 @pytest.mark.parametrize("group", range(3))
 def test_random_conv_geometries_on_32_row_tiles(on_hip, group, monkeypatch):
     """The same sweep with at most 32 channels on either side and the library's test switch that sends every product of at
