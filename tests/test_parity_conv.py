@@ -150,6 +150,9 @@ TUNED_SHAPES = [
     (50, 10, 12, 12, 20, 5, 5, 1, 1, 0, 0),     # LeNet's second convolution: 20- and 10-row products through the general loaders
     (8, 1, 41, 60, 32, 11, 5, 2, 2, 0, 0),      # one input channel, tall filter, stride 2 (DeepSpeech2's first layer in small)
     (64, 512, 4, 4, 10, 4, 4, 1, 1, 0, 0),      # a filter as large as the map (SqueezeNet's classifier): one tile under an 8192-long reduction, the plans with one worker per few slabs compete
+    (32, 512, 7, 7, 512, 1, 1, 1, 1, 0, 0),     # 1x1 over 49-pixel maps: the filter gradient's padded numbering, slices by atomic adds or in two passes as measured
+    (16, 256, 7, 7, 256, 3, 3, 1, 1, 1, 1),     # 3x3 over 49-pixel maps
+    (4, 32, 33, 45, 32, 9, 5, 2, 1, 0, 0),      # DeepSpeech2's second layer in small: 13x41 maps (533 pixels), no padding, x gathered with the lanes along the columns
 ]
 
 
