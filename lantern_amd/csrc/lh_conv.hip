@@ -293,9 +293,9 @@ struct LoadConvBwdFilterSplitB {
     dPQ.divmod(k, n, pq); dQ.divmod(pq, p, q);          // (with PADNUM a group starts on a real index: P*Q is not a multiple of 4)
     int off = (int)n * CHW + (int)p * sH * W + (int)q * sW;
     bool real = true;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      so[e] = (real && k + e < kend) ? (uint32_t)off * 4u : 0u;
+    uint32_t r0, r1, r2, r3;
+    auto step = [&](uint32_t& out, int e) {
+      out = (real && k + e < kend) ? (uint32_t)off * 4u : 0u;
       q += 1; off += sW;
       if ((int)q == Q) {
         q = 0; p += 1; off += sH * W - Q * sW;
@@ -304,7 +304,9 @@ struct LoadConvBwdFilterSplitB {
           else { p = 0; n += 1; off = (int)n * CHW; }
         }
       }
-    }
+    };
+    step(r0, 0); step(r1, 1); step(r2, 2); step(r3, 3);
+    so[0] = r0; so[1] = r1; so[2] = r2; so[3] = r3;
   }
   static __device__ __forceinline__ float4 fix(const float4 v, uint32_t keep) {
     float4 r;
