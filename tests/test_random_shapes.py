@@ -111,3 +111,119 @@ def test_random_sgemm_shapes_with_row_strides(on_hip, group):
         assert_close(got[:, :n], ref[:, :n], what="sgemm values")
         np.testing.assert_array_equal(got[:, n:], Cm[:, n:], err_msg="columns beyond n were written")
         on_hip.sync(); on_hip.resetMallocAddr(mark)
+
+
+# ---- random networks: the library's deferred work against the same calls run as issued -------------------------------------------
+class _RandomNet:
+    """A stack of blocks drawn at random from what the five applications are made of: conv -> batchNorm -> relu(inPlace), conv with bias
+    -> relu(inPlace), a residual block (two such convolutions, the shortcut plain or projected, + and relu), a fire module (squeeze, two
+    expands, concat) and max-pooling; then a classifier convolution over what is left of the map.  Every tensor of a step is large
+    enough for its clearing to be put off."""
+
+    def __init__(self, rng, classes=7):
+        from lantern_amd.nn import Module, Conv2D, BatchNorm2D
+        self.m = Module("randomnet")
+        self.blocks = []
+        c, hw = 3, int(rng.choice([16, 24, 32]))
+        self.hw0 = hw
+        kinds = ["cbr", "cr", "res", "fire", "pool"]
+        for i in range(int(rng.randint(3, 7))):
+            kind = kinds[int(rng.randint(len(kinds)))] if i else "cbr"
+            if kind == "pool" and hw < 8: kind = "cr"
+            co = int(rng.choice([16, 24, 32, 48, 64]))
+            k = int(rng.choice([1, 3, 3, 5])); pad = (k // 2, k // 2)
+            stride = (2, 2) if (kind in ("cbr", "cr") and hw >= 16 and rng.rand() < 0.3) else (1, 1)
+            name = "b%d" % i
+            if kind == "cbr":
+                conv = self.m.add(Conv2D(c, co, (k, k), stride, pad, useBias=False, name=name + "conv", rng=rng)); bn = self.m.add(BatchNorm2D(co, name + "bn"))
+                self.blocks.append(("cbr", conv, bn)); c = co; hw = (hw + 2 * pad[0] - k) // stride[0] + 1
+            elif kind == "cr":
+                conv = self.m.add(Conv2D(c, co, (k, k), stride, pad, useBias=True, name=name + "conv", rng=rng))
+                self.blocks.append(("cr", conv)); c = co; hw = (hw + 2 * pad[0] - k) // stride[0] + 1
+            elif kind == "res":
+                mid = int(rng.choice([8, 16, 32]))
+                c1 = self.m.add(Conv2D(c, mid, (1, 1), useBias=False, name=name + "c1", rng=rng)); b1 = self.m.add(BatchNorm2D(mid, name + "b1"))
+                c2 = self.m.add(Conv2D(mid, co, (3, 3), (1, 1), (1, 1), useBias=False, name=name + "c2", rng=rng)); b2 = self.m.add(BatchNorm2D(co, name + "b2"))
+                proj = None
+                if co != c or rng.rand() < 0.3:
+                    proj = (self.m.add(Conv2D(c, co, (1, 1), useBias=False, name=name + "pc", rng=rng)), self.m.add(BatchNorm2D(co, name + "pb")))
+                self.blocks.append(("res", c1, b1, c2, b2, proj)); c = co
+            elif kind == "fire":
+                sq = int(rng.choice([8, 16])); e1, e3 = int(rng.choice([16, 32])), int(rng.choice([16, 32]))
+                s = self.m.add(Conv2D(c, sq, (1, 1), name=name + "s", rng=rng)); a = self.m.add(Conv2D(sq, e1, (1, 1), name=name + "e1", rng=rng))
+                b = self.m.add(Conv2D(sq, e3, (3, 3), (1, 1), (1, 1), name=name + "e3", rng=rng))
+                self.blocks.append(("fire", s, a, b)); c = e1 + e3
+            else:
+                self.blocks.append(("pool",)); hw = hw // 2
+        self.head = self.m.add(Conv2D(c, classes, (hw, hw), name="head", rng=rng))
+        self.classes = classes
+
+    def __call__(self, x):
+        h = x
+        for b in self.blocks:
+            if b[0] == "cbr": h = b[2](b[1](h)).relu(True)
+            elif b[0] == "cr": h = b[1](h).relu(True)
+            elif b[0] == "res":
+                o = b[2](b[1](h)).relu(True); o = b[4](b[3](o))
+                idt = h if b[5] is None else b[5][1](b[5][0](h))
+                h = (o + idt).relu(True)
+            elif b[0] == "fire":
+                s = b[1](h).relu(True); h = b[2](s).relu(True).concat(1, b[3](s).relu(True))
+            else: h = h.maxPoolBK((2, 2), (2, 2), None)
+        h = self.head(h)
+        return h.resize(h.x.shape[0], -1)
+
+
+def _random_net_steps(be, seed, steps, fusion):
+    """Losses and parameters after `steps` momentum steps of the network drawn from `seed` (deterministic mode set by the caller)."""
+    import lantern_amd as la
+    from lantern_amd.nn import SGD_Momentum
+    from lantern_amd.tensor import Tensor, TensorR, gradR_loss, int_array
+    la.set_backend(be)
+    if hasattr(be, "lib") and hasattr(be.lib, "lh_set_fusion"): be.lib.lh_set_fusion(1 if fusion else 0)
+    mark = be.getMallocAddr()
+    rng = np.random.RandomState(seed)
+    net = _RandomNet(rng)
+    opt = SGD_Momentum(net.m, 0.01, 0.9)
+    x = Tensor.fromNumpy(rng.standard_normal((8, 3, net.hw0, net.hw0)).astype(np.float32))
+    target = int_array(rng.randint(0, net.classes, size=8).astype(np.int32))
+    inner = be.getMallocAddr()
+    losses = []
+    for _ in range(steps):
+        xin = TensorR(x, isInput=True)
+        loss = gradR_loss(lambda dummy: net(xin).logSoftmaxB().nllLossB(target).mean())(Tensor.zeros(1))
+        opt.step()
+        losses.append(float(loss.toCPU()[0]))
+        be.resetMallocAddr(inner)
+    params = [(n, p.x.toCPU().copy()) for n, p in net.m.namedParameters()]
+    if hasattr(be, "sync"): be.sync()
+    be.resetMallocAddr(mark)
+    return np.array(losses), params, [b[0] for b in net.blocks]
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_networks_fused_and_as_issued_agree_and_track_the_oracle(hip_backend, cpu_backend, seed):
+    """Three momentum steps of a random stack of the applications' blocks, one library call per trait method: with the library's deferred work
+    (chains fused, clears put off, filter copies kept, the optimizer's calls gathered) and with every call run as issued the losses and
+    all parameters agree to rounding in deterministic mode, and track the oracle."""
+    be = hip_backend
+    be.setDeterministic(True)
+    try:
+        l1, p1, kinds = _random_net_steps(be, 500 + seed, 3, fusion=True)
+        _say("random network %d: blocks %s, losses %s" % (seed, kinds, l1))
+        l0, p0, _ = _random_net_steps(be, 500 + seed, 3, fusion=False)
+    finally:
+        be.lib.lh_set_fusion(1)
+        be.setDeterministic(False)
+    # (not the same bits: a fused convolution leaves the batch-norm statistics from its epilogue, tile by tile, the stand-alone pass sums
+    # the tensor in another order; a mistake in what is deferred shows as a wrong tensor, not as a last digit)
+    np.testing.assert_allclose(l1, l0, rtol=2e-5)
+    worst = 0.0
+    for (n, a), (_, b) in zip(p1, p0):
+        assert_close(a, b, rtol=2e-4, what="fused against as issued: " + n)
+        worst = max(worst, float(np.abs(a.astype(np.float64) - b).max() / (np.sqrt(np.mean(b.astype(np.float64) ** 2)) + 1e-30)))
+    _say("random network %d: largest parameter deviation between the two, relative to the tensor's rms: %.2e" % (seed, worst))
+    lc, pc, _ = _random_net_steps(cpu_backend, 500 + seed, 3, fusion=True)
+    np.testing.assert_allclose(l1, lc, rtol=1e-3)
+    for (n, a), (_, b) in zip(p1, pc):
+        assert_close(a, b, rtol=2e-3, what="against the oracle: " + n)
