@@ -228,3 +228,37 @@ def test_random_networks_fused_and_as_issued_give_the_same_bits_and_track_the_or
     np.testing.assert_allclose(l2, lc, rtol=1e-3, atol=1e-5)
     for (n, a), (_, b) in zip(p2, pc):
         assert_close(a, b, rtol=2e-3, what="against the oracle: " + n)
+
+
+class _RandomNetTrainer:
+    """The random network above behind the applications' trainer protocol (step, end_step, model)."""
+
+    def __init__(self, seed):
+        import lantern_amd as la
+        from lantern_amd.nn import SGD_Momentum
+        from lantern_amd.tensor import Tensor, int_array, get_backend
+        rng = np.random.RandomState(seed)
+        self.net = _RandomNet(rng); self.model = self.net.m
+        self.opt = SGD_Momentum(self.model, 0.01, 0.9)
+        self.x = Tensor.fromNumpy(rng.standard_normal((8, 3, self.net.hw0, self.net.hw0)).astype(np.float32))
+        self.target = int_array(rng.randint(0, self.net.classes, size=8).astype(np.int32))
+        self.mark = get_backend().getMallocAddr()
+
+    def step(self):
+        from lantern_amd.tensor import Tensor, TensorR, gradR_loss
+        xin = TensorR(self.x, isInput=True)
+        loss = gradR_loss(lambda dummy: self.net(xin).logSoftmaxB().nllLossB(self.target).mean())(Tensor.zeros(1))
+        self.opt.step()
+        return loss
+
+    def end_step(self):
+        from lantern_amd.tensor import get_backend
+        get_backend().resetMallocAddr(self.mark)
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_networks_graph_replays_give_the_eager_steps_bits(hip_backend, seed):
+    """The same random networks with the step recorded into a HIP graph after two eager steps: four replays, with eager work of the
+    program's own between them, give the losses and parameters of the same steps run eagerly, bit for bit in deterministic mode."""
+    from tests.test_training_parity import _graph_against_eager
+    _graph_against_eager(lambda: _RandomNetTrainer(700 + seed), hip_backend, eager_steps=2, replays=4, tol=0.0, per_tensor=1e-12, deterministic=True)
